@@ -1,0 +1,129 @@
+"""Builds the native parts of the docc `rocm` target, in-tree.
+
+Products (all under ``docc_amd/lib/``):
+
+* ``docc_rocm_<family>.hsaco``  gfx950 code objects, one per kernel family
+  (``hipcc --genco --offload-arch=gfx950``);
+* ``libdocc_rt_rocm.so``       the thin C-ABI runtime and the op launchers
+  (``include/docc_rocm_rt.h``, ``include/docc_rocm_ops.h``);
+* ``libdocc_rocm_target.so``   the library-node descriptors, dispatcher
+  registry, rocm plugin and host-code generator (``include/docc_rocm_target.h``).
+
+The reference drives its own compile steps with ``std::system`` from
+``python/bindings/py_structured_sdfg.cpp:355-560``; this module is the
+counterpart for the pre-built pieces and is what ``__graft_entry__.build()``
+calls.  Run ``python -m docc_amd.build`` to (re)build everything.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent.parent
+PKG = ROOT / "docc_amd"
+CSRC = PKG / "csrc"
+LIB = PKG / "lib"
+INCLUDE = ROOT / "include"
+ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+
+# kernel family -> source file; keep in step with kKernelImages in csrc/rt/runtime.cpp
+KERNEL_FAMILIES = {
+    "util": "util.hip",
+    "softmax": "softmax.hip",
+}
+
+# packed fp32 VALU ops are switched off for every device compile
+DEVICE_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or str(ROCM / "bin" / "hipcc")
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found; the rocm target needs the ROCm toolchain to build")
+    return exe
+
+
+def _run(cmd: list[str]) -> None:
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("build step failed:\n  " + " ".join(cmd) + "\n" + proc.stdout + proc.stderr)
+
+
+def _newer(target: Path, sources: list[Path]) -> bool:
+    if not target.exists():
+        return False
+    t = target.stat().st_mtime
+    return all(s.stat().st_mtime <= t for s in sources)
+
+
+def build_kernel_family(family: str, force: bool = True) -> Path:
+    src = CSRC / "kernels" / KERNEL_FAMILIES[family]
+    out = LIB / f"docc_rocm_{family}.hsaco"
+    deps = [src] + sorted((CSRC / "kernels").glob("*.h"))
+    if not force and _newer(out, deps):
+        return out
+    LIB.mkdir(parents=True, exist_ok=True)
+    _run([hipcc(), "--genco", *DEVICE_FLAGS, "-I", str(CSRC / "kernels"), str(src), "-o", str(out)])
+    return out
+
+
+def build_kernels(force: bool = True, jobs: int = 8) -> list[Path]:
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        return list(pool.map(lambda f: build_kernel_family(f, force), KERNEL_FAMILIES))
+
+
+def build_runtime(force: bool = True) -> Path:
+    srcs = sorted((CSRC / "rt").glob("*.cpp"))
+    deps = srcs + sorted((CSRC / "rt").glob("*.h")) + sorted(INCLUDE.glob("*.h"))
+    out = LIB / "libdocc_rt_rocm.so"
+    if not force and _newer(out, deps):
+        return out
+    LIB.mkdir(parents=True, exist_ok=True)
+    _run([
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__",
+        "-I", str(INCLUDE), "-I", str(CSRC / "rt"), "-I", str(ROCM / "include"),
+        *map(str, srcs), "-o", str(out),
+        "-L", str(ROCM / "lib"), "-lamdhip64", "-ldl", f"-Wl,-rpath,{ROCM / 'lib'}",
+    ])
+    return out
+
+
+def build_target(force: bool = True) -> Path | None:
+    srcs = sorted((CSRC / "target").glob("*.cpp"))
+    if not srcs:
+        return None
+    deps = srcs + sorted((CSRC / "target").glob("*.h")) + sorted(INCLUDE.glob("*.h"))
+    out = LIB / "libdocc_rocm_target.so"
+    if not force and _newer(out, deps):
+        return out
+    LIB.mkdir(parents=True, exist_ok=True)
+    _run([
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall",
+        "-I", str(INCLUDE), "-I", str(CSRC / "target"), *map(str, srcs), "-o", str(out),
+    ])
+    return out
+
+
+def build_all(force: bool = True) -> dict[str, list[str]]:
+    built = {"kernels": [str(p) for p in build_kernels(force)], "runtime": [str(build_runtime(force))]}
+    target = build_target(force)
+    if target:
+        built["target"] = [str(target)]
+    return built
+
+
+if __name__ == "__main__":
+    force = "--if-stale" not in sys.argv
+    for kind, paths in build_all(force).items():
+        for p in paths:
+            print(f"{kind}: {p}")

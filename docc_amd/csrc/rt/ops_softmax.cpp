@@ -1,0 +1,72 @@
+// Launchers for ml::Softmax and the utility kernels (see include/docc_rocm_ops.h).
+#include "docc_rocm_ops.h"
+#include "rt_state.h"
+
+using namespace docc::rt::rocm;
+
+extern "C" {
+
+int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols, const float* X, float* Y) {
+    if (rows < 0 || cols < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
+    if (rows == 0 || cols == 0) return 0;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
+    if (rows > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
+    hipStream_t s = (hipStream_t) stream;
+    const bool vec_ok = (cols % 4 == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
+    if (vec_ok && cols <= 4096) {
+        // one wavefront per row, 4 rows per 256-thread block
+        const char* name = cols <= 256    ? "docc_softmax_f32_wave_v1"
+                           : cols <= 512  ? "docc_softmax_f32_wave_v2"
+                           : cols <= 1024 ? "docc_softmax_f32_wave_v4"
+                           : cols <= 2048 ? "docc_softmax_f32_wave_v8"
+                                          : "docc_softmax_f32_wave_v16";
+        uint32_t grid = (uint32_t) ((rows + 3) / 4);
+        return launch(name, grid, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
+    }
+    if (vec_ok && cols <= 16384) {
+        const char* name = cols <= 8192 ? "docc_softmax_f32_block_v8" : "docc_softmax_f32_block_v16";
+        return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
+    }
+    return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+}
+
+static uint32_t grid_for(int64_t items) {
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    int64_t blocks = (items + 255) / 256;
+    int64_t cap = (int64_t) cus * 16;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return (uint32_t) blocks;
+}
+
+int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* src, void* dst) {
+    if (bytes < 0 || bytes % 16 != 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "copy_bytes: size must be a multiple of 16");
+    if (bytes == 0) return 0;
+    if (!src || !dst || (((uintptr_t) src | (uintptr_t) dst) % 16) != 0)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "copy_bytes: pointers must be 16-byte aligned");
+    int rc = ensure_device();
+    if (rc) return rc;
+    long n16 = bytes / 16;
+    return launch("docc_copy_b128", grid_for(n16), 1, 1, 256, 0, (hipStream_t) stream, src, dst, n16);
+}
+
+int docc_rocm_convert_f32_to_bf16(docc_rocm_stream_t stream, int64_t count, const float* src, uint16_t* dst) {
+    if (count < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "convert: negative count");
+    if (count == 0) return 0;
+    if (!src || !dst) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "convert: null pointer");
+    int rc = ensure_device();
+    if (rc) return rc;
+    return launch("docc_f32_to_bf16", grid_for(count), 1, 1, 256, 0, (hipStream_t) stream, src, dst, (long) count);
+}
+
+int docc_rocm_convert_bf16_to_f32(docc_rocm_stream_t stream, int64_t count, const uint16_t* src, float* dst) {
+    if (count < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "convert: negative count");
+    if (count == 0) return 0;
+    if (!src || !dst) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "convert: null pointer");
+    int rc = ensure_device();
+    if (rc) return rc;
+    return launch("docc_bf16_to_f32", grid_for(count), 1, 1, 256, 0, (hipStream_t) stream, src, dst, (long) count);
+}
+
+} // extern "C"

@@ -1,0 +1,308 @@
+// Thin C-ABI HIP runtime of the docc `rocm` target (see include/docc_rocm_rt.h).
+//
+// Structural counterpart of docc::rt::et::EtRuntimeWrapper (reference
+// targets/et/rt/src/runtime.cpp:55-176): a process-wide singleton per device
+// that owns the loaded kernel image, with the image located next to the
+// library unless an environment variable points elsewhere
+// (reference runtime.cpp:129-143).
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "rt_state.h"
+
+namespace docc::rt::rocm {
+
+namespace {
+
+thread_local std::string g_last_error;
+
+// One gfx950 code object per kernel family; all of them must be present.
+const char* const kKernelImages[] = {
+    "docc_rocm_util.hsaco",
+    "docc_rocm_softmax.hsaco",
+};
+
+struct DeviceState {
+    bool ready = false;
+    std::vector<hipModule_t> modules;
+    int compute_units = 0;
+    std::unordered_map<std::string, hipFunction_t> functions;
+};
+
+std::mutex g_mutex;
+std::vector<DeviceState> g_devices;
+
+std::string kernel_image_dir() {
+    const char* env = std::getenv("DOCC_ROCM_KERNEL_PATH");
+    std::string dir;
+    if (env && *env) {
+        dir = env;
+    } else {
+        Dl_info info;
+        if (dladdr((void*) &kernel_image_dir, &info) && info.dli_fname) {
+            dir = info.dli_fname;
+            auto pos = dir.find_last_of('/');
+            dir = (pos == std::string::npos) ? "." : dir.substr(0, pos);
+        } else {
+            dir = ".";
+        }
+    }
+    return dir;
+}
+
+} // namespace
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int check(hipError_t err, const char* what) {
+    if (err == hipSuccess) return 0;
+    return fail((int) err, "%s: %s (%s)", what, hipGetErrorString(err), hipGetErrorName(err));
+}
+
+int ensure_device() {
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return fail(DOCC_ROCM_ERR_NO_DEVICE, "no HIP device: %s", hipGetErrorString(err));
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if ((size_t) dev >= g_devices.size()) g_devices.resize(dev + 1);
+    DeviceState& st = g_devices[dev];
+    if (st.ready) return 0;
+    hipDeviceProp_t prop;
+    int rc = check(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+    if (rc) return rc;
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "device %d is %s; the rocm target is built for gfx950 only", dev,
+                    prop.gcnArchName);
+    st.compute_units = prop.multiProcessorCount;
+    std::string dir = kernel_image_dir();
+    std::vector<hipModule_t> modules;
+    for (const char* image : kKernelImages) {
+        std::string path = dir + "/" + image;
+        hipModule_t m;
+        err = hipModuleLoad(&m, path.c_str());
+        if (err != hipSuccess) {
+            for (hipModule_t loaded : modules) (void) hipModuleUnload(loaded);
+            return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "cannot load kernel image %s: %s", path.c_str(),
+                        hipGetErrorString(err));
+        }
+        modules.push_back(m);
+    }
+    st.modules = std::move(modules);
+    st.ready = true;
+    return 0;
+}
+
+int kernel(const char* name, hipFunction_t* fn) {
+    int rc = ensure_device();
+    if (rc) return rc;
+    int dev = 0;
+    (void) hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    DeviceState& st = g_devices[dev];
+    auto it = st.functions.find(name);
+    if (it != st.functions.end()) {
+        *fn = it->second;
+        return 0;
+    }
+    hipFunction_t f = nullptr;
+    hipError_t err = hipErrorNotFound;
+    for (hipModule_t m : st.modules) {
+        err = hipModuleGetFunction(&f, m, name);
+        if (err == hipSuccess) break;
+    }
+    // a miss in one image leaves HIP's per-thread "last error" set; clear it so
+    // that other users of the HIP runtime in this process do not pick it up
+    (void) hipGetLastError();
+    if (err != hipSuccess)
+        return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "kernel %s not in any kernel image: %s", name, hipGetErrorString(err));
+    st.functions.emplace(name, f);
+    *fn = f;
+    return 0;
+}
+
+int compute_units() {
+    int dev = 0;
+    (void) hipGetDevice(&dev);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if ((size_t) dev >= g_devices.size()) return 0;
+    return g_devices[dev].compute_units;
+}
+
+} // namespace docc::rt::rocm
+
+using namespace docc::rt::rocm;
+
+extern "C" {
+
+int docc_rocm_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int docc_rocm_init(int device) {
+    int n = docc_rocm_device_count();
+    if (n <= 0) return fail(DOCC_ROCM_ERR_NO_DEVICE, "no HIP device visible");
+    if (device < 0 || device >= n) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "device %d out of range [0,%d)", device, n);
+    int rc = check(hipSetDevice(device), "hipSetDevice");
+    if (rc) return rc;
+    return ensure_device();
+}
+
+int docc_rocm_device_info(char* arch, size_t arch_len, int* compute_units_out, int* clock_khz) {
+    int dev = 0;
+    int rc = check(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    hipDeviceProp_t prop;
+    rc = check(hipGetDeviceProperties(&prop, dev), "hipGetDeviceProperties");
+    if (rc) return rc;
+    if (arch && arch_len) {
+        std::strncpy(arch, prop.gcnArchName, arch_len - 1);
+        arch[arch_len - 1] = 0;
+    }
+    if (compute_units_out) *compute_units_out = prop.multiProcessorCount;
+    if (clock_khz) *clock_khz = prop.clockRate;
+    return 0;
+}
+
+int docc_rocm_module_load(const char* path, docc_rocm_module_t* module) {
+    if (!path || !module) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "module_load: null argument");
+    hipModule_t m;
+    hipError_t err = hipModuleLoad(&m, path);
+    if (err != hipSuccess) return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "cannot load %s: %s", path, hipGetErrorString(err));
+    *module = m;
+    return 0;
+}
+
+int docc_rocm_module_unload(docc_rocm_module_t module) {
+    return check(hipModuleUnload((hipModule_t) module), "hipModuleUnload");
+}
+
+int docc_rocm_module_get_function(docc_rocm_module_t module, const char* name, docc_rocm_function_t* function) {
+    if (!module || !name || !function) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "get_function: null argument");
+    hipFunction_t f;
+    hipError_t err = hipModuleGetFunction(&f, (hipModule_t) module, name);
+    if (err != hipSuccess) return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "kernel %s not found: %s", name, hipGetErrorString(err));
+    *function = f;
+    return 0;
+}
+
+int docc_rocm_malloc(void** dev_ptr, size_t bytes) {
+    if (!dev_ptr) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "malloc: null argument");
+    *dev_ptr = nullptr;
+    if (bytes == 0) return 0;
+    return check(hipMalloc(dev_ptr, bytes), "hipMalloc");
+}
+
+int docc_rocm_free(void* dev_ptr) {
+    if (!dev_ptr) return 0;
+    return check(hipFree(dev_ptr), "hipFree");
+}
+
+int docc_rocm_memset_async(void* dev_ptr, int value, size_t bytes, docc_rocm_stream_t stream) {
+    if (bytes == 0) return 0;
+    return check(hipMemsetAsync(dev_ptr, value, bytes, (hipStream_t) stream), "hipMemsetAsync");
+}
+
+int docc_rocm_host_malloc(void** host_ptr, size_t bytes) {
+    if (!host_ptr) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "host_malloc: null argument");
+    *host_ptr = nullptr;
+    if (bytes == 0) return 0;
+    return check(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault), "hipHostMalloc");
+}
+
+int docc_rocm_host_free(void* host_ptr) {
+    if (!host_ptr) return 0;
+    return check(hipHostFree(host_ptr), "hipHostFree");
+}
+
+int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes, docc_rocm_stream_t stream) {
+    if (bytes == 0) return 0;
+    return check(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t) stream), "hipMemcpyAsync(H2D)");
+}
+
+int docc_rocm_memcpy_d2h_async(void* dst_host, const void* src_dev, size_t bytes, docc_rocm_stream_t stream) {
+    if (bytes == 0) return 0;
+    return check(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t) stream), "hipMemcpyAsync(D2H)");
+}
+
+int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes, docc_rocm_stream_t stream) {
+    if (bytes == 0) return 0;
+    return check(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, (hipStream_t) stream), "hipMemcpyAsync(D2D)");
+}
+
+int docc_rocm_stream_create(docc_rocm_stream_t* stream) {
+    if (!stream) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "stream_create: null argument");
+    hipStream_t s;
+    int rc = check(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreate");
+    if (rc) return rc;
+    *stream = s;
+    return 0;
+}
+
+int docc_rocm_stream_destroy(docc_rocm_stream_t stream) {
+    if (!stream) return 0;
+    return check(hipStreamDestroy((hipStream_t) stream), "hipStreamDestroy");
+}
+
+int docc_rocm_stream_sync(docc_rocm_stream_t stream) {
+    return check(hipStreamSynchronize((hipStream_t) stream), "hipStreamSynchronize");
+}
+
+int docc_rocm_device_sync(void) { return check(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+
+int docc_rocm_launch(docc_rocm_function_t function, const uint32_t grid[3], const uint32_t block[3],
+                     uint32_t shared_bytes, docc_rocm_stream_t stream, void** args) {
+    if (!function || !grid || !block) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "launch: null argument");
+    if (grid[0] == 0 || grid[1] == 0 || grid[2] == 0) return 0;
+    uint64_t threads = (uint64_t) block[0] * block[1] * block[2];
+    if (threads == 0 || threads > 1024) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "launch: block of %llu threads", (unsigned long long) threads);
+    return check(hipModuleLaunchKernel((hipFunction_t) function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                       shared_bytes, (hipStream_t) stream, args, nullptr),
+                 "hipModuleLaunchKernel");
+}
+
+int docc_rocm_event_create(docc_rocm_event_t* event) {
+    if (!event) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "event_create: null argument");
+    hipEvent_t e;
+    int rc = check(hipEventCreate(&e), "hipEventCreate");
+    if (rc) return rc;
+    *event = e;
+    return 0;
+}
+
+int docc_rocm_event_destroy(docc_rocm_event_t event) {
+    if (!event) return 0;
+    return check(hipEventDestroy((hipEvent_t) event), "hipEventDestroy");
+}
+
+int docc_rocm_event_record(docc_rocm_event_t event, docc_rocm_stream_t stream) {
+    return check(hipEventRecord((hipEvent_t) event, (hipStream_t) stream), "hipEventRecord");
+}
+
+int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, float* ms) {
+    if (!ms) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "event_elapsed: null argument");
+    int rc = check(hipEventSynchronize((hipEvent_t) stop), "hipEventSynchronize");
+    if (rc) return rc;
+    return check(hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop), "hipEventElapsedTime");
+}
+
+const char* docc_rocm_last_error(void) { return g_last_error.c_str(); }
+
+const char* docc_rocm_version(void) { return "docc-rocm 0.1 (gfx950)"; }
+
+} // extern "C"

@@ -1,0 +1,210 @@
+"""ctypes binding of ``libdocc_rt_rocm.so`` (``include/docc_rocm_rt.h`` and
+``include/docc_rocm_ops.h``): the thin HIP runtime and the kernel launchers.
+
+There is no fallback: when the library or a GPU is missing, calls raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+LIB_DIR = Path(__file__).resolve().parent / "lib"
+LIB_PATH = LIB_DIR / "libdocc_rt_rocm.so"
+
+NO_TRANS = 111
+TRANS = 112
+
+
+class RocmRuntimeError(RuntimeError):
+    """A call into libdocc_rt_rocm.so returned a non-zero code."""
+
+    def __init__(self, fn: str, code: int, message: str):
+        super().__init__(f"{fn} failed with code {code}: {message}")
+        self.fn = fn
+        self.code = code
+
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+_f32 = ctypes.c_float
+_f64 = ctypes.c_double
+
+# name -> argtypes; every function returns int unless listed in _RESTYPE
+_SIGNATURES = {
+    "docc_rocm_init": [_int],
+    "docc_rocm_device_count": [],
+    "docc_rocm_device_info": [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(_int), ctypes.POINTER(_int)],
+    "docc_rocm_module_load": [ctypes.c_char_p, ctypes.POINTER(_vp)],
+    "docc_rocm_module_unload": [_vp],
+    "docc_rocm_module_get_function": [_vp, ctypes.c_char_p, ctypes.POINTER(_vp)],
+    "docc_rocm_malloc": [ctypes.POINTER(_vp), ctypes.c_size_t],
+    "docc_rocm_free": [_vp],
+    "docc_rocm_memset_async": [_vp, _int, ctypes.c_size_t, _vp],
+    "docc_rocm_host_malloc": [ctypes.POINTER(_vp), ctypes.c_size_t],
+    "docc_rocm_host_free": [_vp],
+    "docc_rocm_memcpy_h2d_async": [_vp, _vp, ctypes.c_size_t, _vp],
+    "docc_rocm_memcpy_d2h_async": [_vp, _vp, ctypes.c_size_t, _vp],
+    "docc_rocm_memcpy_d2d_async": [_vp, _vp, ctypes.c_size_t, _vp],
+    "docc_rocm_stream_create": [ctypes.POINTER(_vp)],
+    "docc_rocm_stream_destroy": [_vp],
+    "docc_rocm_stream_sync": [_vp],
+    "docc_rocm_device_sync": [],
+    "docc_rocm_launch": [_vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32), ctypes.c_uint32, _vp, ctypes.POINTER(_vp)],
+    "docc_rocm_event_create": [ctypes.POINTER(_vp)],
+    "docc_rocm_event_destroy": [_vp],
+    "docc_rocm_event_record": [_vp, _vp],
+    "docc_rocm_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(_f32)],
+    "docc_rocm_last_error": [],
+    "docc_rocm_version": [],
+    "docc_rocm_dgemm": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _vp, _i64, _f64, _vp, _i64],
+    "docc_rocm_sgemm": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64],
+    "docc_rocm_bf16gemm_f32": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64],
+    "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
+    "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
+    "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
+    "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
+    "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
+    "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
+}
+_RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p}
+
+#: every symbol the two public headers declare
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib: ctypes.CDLL | None = None
+
+
+def lib() -> ctypes.CDLL:
+    """Loads ``libdocc_rt_rocm.so`` (once). Raises when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RocmRuntimeError("load", -3, f"{LIB_PATH} is missing; run `python -m docc_amd.build`")
+        handle = ctypes.CDLL(str(LIB_PATH))
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _RESTYPE.get(name, _int)
+        _lib = handle
+    return _lib
+
+
+def last_error() -> str:
+    return (lib().docc_rocm_last_error() or b"").decode()
+
+
+def call(name: str, *args) -> None:
+    """Calls an int-returning entry point and raises on a non-zero code."""
+    rc = getattr(lib(), name)(*args)
+    if rc != 0:
+        raise RocmRuntimeError(name, rc, last_error())
+
+
+def version() -> str:
+    return lib().docc_rocm_version().decode()
+
+
+def device_count() -> int:
+    return int(lib().docc_rocm_device_count())
+
+
+def init(device: int = 0) -> None:
+    call("docc_rocm_init", device)
+
+
+def device_info() -> dict:
+    arch = ctypes.create_string_buffer(64)
+    cus = _int()
+    clk = _int()
+    call("docc_rocm_device_info", arch, 64, ctypes.byref(cus), ctypes.byref(clk))
+    return {"arch": arch.value.decode(), "compute_units": cus.value, "clock_khz": clk.value}
+
+
+def malloc(nbytes: int) -> int:
+    p = _vp()
+    call("docc_rocm_malloc", ctypes.byref(p), nbytes)
+    return p.value or 0
+
+
+def free(ptr: int) -> None:
+    call("docc_rocm_free", ptr)
+
+
+def memcpy_h2d(dst_dev: int, src_host: int, nbytes: int, stream: int = 0) -> None:
+    call("docc_rocm_memcpy_h2d_async", dst_dev, src_host, nbytes, stream)
+
+
+def memcpy_d2h(dst_host: int, src_dev: int, nbytes: int, stream: int = 0) -> None:
+    call("docc_rocm_memcpy_d2h_async", dst_host, src_dev, nbytes, stream)
+
+
+def stream_sync(stream: int = 0) -> None:
+    call("docc_rocm_stream_sync", stream)
+
+
+def device_sync() -> None:
+    call("docc_rocm_device_sync")
+
+
+class Event:
+    """HIP event recorded on an explicit stream."""
+
+    def __init__(self):
+        p = _vp()
+        call("docc_rocm_event_create", ctypes.byref(p))
+        self.handle = p.value
+
+    def record(self, stream: int = 0) -> None:
+        call("docc_rocm_event_record", self.handle, stream)
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = _f32()
+        call("docc_rocm_event_elapsed_ms", self.handle, stop.handle, ctypes.byref(ms))
+        return float(ms.value)
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().docc_rocm_event_destroy(self.handle)
+        except Exception:
+            pass
+
+
+# --- kernel launchers on raw device pointers -------------------------------
+
+def dgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, trans_a=NO_TRANS, trans_b=NO_TRANS, stream=0) -> None:
+    call("docc_rocm_dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
+
+
+def sgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, trans_a=NO_TRANS, trans_b=NO_TRANS, stream=0) -> None:
+    call("docc_rocm_sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
+
+
+def bf16gemm_f32(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, trans_a=NO_TRANS, trans_b=NO_TRANS, stream=0) -> None:
+    call("docc_rocm_bf16gemm_f32", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
+
+
+def softmax_f32(rows, cols, X, Y, stream=0) -> None:
+    call("docc_rocm_softmax_f32", stream, rows, cols, X, Y)
+
+
+def conv2d_f32(N, C, H, W, OC, KH, KW, stride, pad, dilation, X, Wt, bias, Y, stream=0) -> None:
+    call("docc_rocm_conv2d_f32", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pad[0], pad[1],
+         dilation[0], dilation[1], X, Wt, bias or None, Y)
+
+
+def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0) -> None:
+    call("docc_rocm_attention_bf16", stream, B, H, SQ, SKV, D, scale, Q, K, V, O, 1 if out_bf16 else 0)
+
+
+def copy_bytes(nbytes, src, dst, stream=0) -> None:
+    call("docc_rocm_copy_bytes", stream, nbytes, src, dst)
+
+
+def convert_f32_to_bf16(count, src, dst, stream=0) -> None:
+    call("docc_rocm_convert_f32_to_bf16", stream, count, src, dst)
+
+
+def convert_bf16_to_f32(count, src, dst, stream=0) -> None:
+    call("docc_rocm_convert_bf16_to_f32", stream, count, src, dst)

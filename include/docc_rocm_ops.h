@@ -1,0 +1,110 @@
+/*
+ * docc_rocm_ops.h - C-ABI launchers of the math library-node kernels of the
+ * docc `rocm` target (GEMM, Softmax, Conv, Attention) on gfx950.
+ *
+ * These are the calls the rocm library-node dispatchers print into generated
+ * host C++, in the place where the reference's dispatchers print
+ * `cblas_dgemm(...)` (sdfg/src/data_flow/library_nodes/math/blas/gemm_node.cpp:449-509)
+ * or `cublasDgemm(...)` (opt/src/targets/cuda/blas/gemm.cpp:131-185), and
+ * where the reference expands Softmax and Conv into host loop nests
+ * (sdfg/src/data_flow/library_nodes/math/tensor/reduce_ops/softmax_node.cpp:38-265,
+ *  sdfg/src/data_flow/library_nodes/math/tensor/conv_node.cpp:85-454).
+ *
+ * All pointers are DEVICE pointers (the WithTransfers dispatchers copy
+ * through docc_rocm_rt.h first). All matrices and tensors are dense,
+ * row-major / C-order, as the reference's frontends produce them. Each call
+ * enqueues its kernels on `stream` and returns without waiting. Return value:
+ * 0, a hipError_t, or a negative DOCC_ROCM_ERR_* code; message in
+ * docc_rocm_last_error().
+ *
+ * Library: libdocc_rt_rocm.so (same library as docc_rocm_rt.h).
+ */
+#ifndef DOCC_ROCM_OPS_H
+#define DOCC_ROCM_OPS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include "docc_rocm_rt.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* BLAS transpose codes as the reference's GEMMNode stores them
+ * (sdfg/include/sdfg/data_flow/library_nodes/math/blas/blas_node.h:49-126). */
+#define DOCC_ROCM_NO_TRANS 111
+#define DOCC_ROCM_TRANS 112
+
+/*
+ * C[m,n] = alpha * op(A)[m,k] * op(B)[k,n] + beta * C[m,n], row-major, with
+ * cblas semantics: when beta == 0, C is not read (it may hold NaNs).
+ * Replaces cblas_dgemm / cblas_sgemm as printed by GEMMNodeDispatcher_BLAS
+ * (reference gemm_node.cpp:474-505) and cublasDgemm / cublasSgemm
+ * (reference opt/src/targets/cuda/blas/gemm.cpp:131-185).
+ * Zero-sized m, n: nothing is done; k == 0: C = beta * C.
+ */
+int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                    double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta,
+                    double* C, int64_t ldc);
+int docc_rocm_sgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                    float alpha, const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C,
+                    int64_t ldc);
+
+/*
+ * bf16 inputs (raw bits, uint16_t, the type that crosses the reference's
+ * ctypes boundary for BFloat: python/docc/compiler/compiled_sdfg.py:16-31),
+ * fp32 accumulate and fp32 C. The reference's BLAS_Precision has no such
+ * mode (blas_node.h:49-55); this is the rocm target's added precision.
+ */
+int docc_rocm_bf16gemm_f32(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                           float alpha, const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                           float beta, float* C, int64_t ldc);
+
+/*
+ * Y[r, :] = softmax(X[r, :]) for r in [0, rows), fp32, both [rows, cols]
+ * contiguous. This is ml::Softmax over the last axis; any reduction over a
+ * trailing contiguous axis of an N-d tensor is this call with
+ * rows = product of the leading dims. Replaces the Max/Sub/Exp/Sum/Div
+ * loop nests of SoftmaxNode::expand (reference softmax_node.cpp:142-252).
+ * X == Y (in place) is allowed.
+ */
+int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols, const float* X, float* Y);
+
+/*
+ * ml::Conv, 2-d, NCHW fp32, group 1 (reference conv_node.h:9-22,48-217):
+ *   Y[n,oc,oh,ow] = bias[oc] + sum_{ic,kh,kw} X[n,ic,oh*sh-ph+kh*dh, ow*sw-pw+kw*dw] * W[oc,ic,kh,kw]
+ * with zero padding (taps outside the image contribute 0); bias may be NULL.
+ * Output size per the reference formula (conv_node.cpp:224-233):
+ *   OH = (H + 2*pad_h - dil_h*(KH-1) - 1) / stride_h + 1   (same for W).
+ */
+int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                         int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                         int64_t dil_h, int64_t dil_w, const float* X, const float* Wt, const float* bias,
+                         float* Y);
+
+/*
+ * ml::Attention (a node the rocm target adds; the reference has none):
+ *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
+ * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32
+ * scores, softmax and accumulation; non-causal. O is [B,H,SQ,D], fp32 when
+ * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 64.
+ */
+int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                             float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
+                             int out_bf16);
+
+/* fp32 -> bf16 (round to nearest even) and back, on the device; used by the
+ * WithTransfers dispatchers when a node's inputs arrive as fp32. */
+int docc_rocm_convert_f32_to_bf16(docc_rocm_stream_t stream, int64_t count, const float* src, uint16_t* dst);
+int docc_rocm_convert_bf16_to_f32(docc_rocm_stream_t stream, int64_t count, const uint16_t* src, float* dst);
+
+/* Plain device copy kernel of `bytes` bytes (multiple of 16): the known-size
+ * kernel against which rocprof's FETCH_SIZE / WRITE_SIZE counters are
+ * calibrated. */
+int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* src, void* dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOCC_ROCM_OPS_H */

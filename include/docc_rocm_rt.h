@@ -1,0 +1,115 @@
+/*
+ * docc_rocm_rt.h - thin C-ABI HIP runtime of the docc `rocm` target.
+ *
+ * This is the only door through which generated host C++ reaches the GPU:
+ * module load, device memory, asynchronous copies, kernel launch, stream
+ * synchronisation and an error string. It plays the role that
+ * docc::rt::et::EtRuntimeWrapper plays for the ET-SoC target
+ * (reference targets/et/rt/include/docc/rt/et/et.h:9-30, used by the
+ * dispatcher at targets/et/src/et/blas/gemm.cpp:137-204) and that the raw
+ * cudaMalloc/cudaMemcpy/cudaFree calls play for the CUDA target
+ * (reference opt/src/targets/cuda/cuda_data_offloading_node.cpp:139-173,
+ * opt/src/targets/cuda/blas/gemm.cpp:66-96).
+ *
+ * Conventions
+ *   - every function returns 0 on success and a non-zero HIP error code (or
+ *     a negative docc code, see below) on failure; the message is available
+ *     from docc_rocm_last_error() on the calling thread;
+ *   - plain pointers and sizes only; `stream` is a hipStream_t passed as
+ *     void* (NULL = the device's default stream);
+ *   - one process-wide state per device, created by docc_rocm_init() or
+ *     lazily by the first call; thread-safe.
+ *
+ * Library: libdocc_rt_rocm.so. The gfx950 code objects that hold the math
+ * kernels (docc_rocm_<family>.hsaco, one per kernel family) are looked up next
+ * to the library; the
+ * environment variable DOCC_ROCM_KERNEL_PATH overrides the directory, in the
+ * way DOCC_ET_KERNEL_PATH does for the ET target
+ * (reference targets/et/rt/src/runtime.cpp:129-143).
+ */
+#ifndef DOCC_ROCM_RT_H
+#define DOCC_ROCM_RT_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* negative codes are docc's own, positive ones are hipError_t values */
+#define DOCC_ROCM_OK 0
+#define DOCC_ROCM_ERR_INVALID_ARGUMENT (-1)
+#define DOCC_ROCM_ERR_UNSUPPORTED (-2)
+#define DOCC_ROCM_ERR_KERNEL_IMAGE (-3) /* code object missing or not loadable */
+#define DOCC_ROCM_ERR_NO_DEVICE (-4)
+
+typedef void* docc_rocm_module_t;   /* hipModule_t   */
+typedef void* docc_rocm_function_t; /* hipFunction_t */
+typedef void* docc_rocm_stream_t;   /* hipStream_t   */
+
+/* Selects `device` for the calling thread, creates its state and loads the
+ * math-kernel code object. Replaces EtRuntimeWrapper::get_instance() +
+ * get_device(idx) (reference et.h:16-20). Idempotent. */
+int docc_rocm_init(int device);
+
+/* Number of visible HIP devices, or 0. Does not create any state. */
+int docc_rocm_device_count(void);
+
+/* Name (gcnArchName) and compute-unit count of the current device. */
+int docc_rocm_device_info(char* arch, size_t arch_len, int* compute_units, int* clock_khz);
+
+/* Loads a gfx950 code object from a file. Replaces
+ * EtRuntimeWrapper::load_kernel_binary_blocking (reference et.h:22-23). */
+int docc_rocm_module_load(const char* path, docc_rocm_module_t* module);
+int docc_rocm_module_unload(docc_rocm_module_t module);
+int docc_rocm_module_get_function(docc_rocm_module_t module, const char* name, docc_rocm_function_t* function);
+
+/* Device memory. Replace cudaMalloc / cudaFree of the CUDA offloading node
+ * (reference cuda_data_offloading_node.cpp:150-170). */
+int docc_rocm_malloc(void** dev_ptr, size_t bytes);
+int docc_rocm_free(void* dev_ptr);
+int docc_rocm_memset_async(void* dev_ptr, int value, size_t bytes, docc_rocm_stream_t stream);
+
+/* Pinned host memory (hipHostMalloc) for callers that want truly
+ * asynchronous copies. */
+int docc_rocm_host_malloc(void** host_ptr, size_t bytes);
+int docc_rocm_host_free(void* host_ptr);
+
+/* Copies on a stream. Replace the blocking cudaMemcpy H2D/D2H of the CUDA
+ * offloading node (reference cuda_data_offloading_node.cpp:153-166); the
+ * caller orders them with docc_rocm_stream_sync. */
+int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes, docc_rocm_stream_t stream);
+int docc_rocm_memcpy_d2h_async(void* dst_host, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);
+int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);
+
+/* Streams (default priority only). */
+int docc_rocm_stream_create(docc_rocm_stream_t* stream);
+int docc_rocm_stream_destroy(docc_rocm_stream_t stream);
+int docc_rocm_stream_sync(docc_rocm_stream_t stream);
+int docc_rocm_device_sync(void);
+
+/* Launches `function` with an array of pointers to its arguments, as
+ * hipModuleLaunchKernel takes them. Replaces the `<<<grid, block>>>` launch
+ * the CUDA map dispatcher prints (reference
+ * opt/src/targets/cuda/codegen/cuda_map_dispatcher.cpp:236-262). */
+int docc_rocm_launch(docc_rocm_function_t function, const uint32_t grid[3], const uint32_t block[3],
+                     uint32_t shared_bytes, docc_rocm_stream_t stream, void** args);
+
+/* Events, for timing on the stream the kernels run on. */
+typedef void* docc_rocm_event_t;
+int docc_rocm_event_create(docc_rocm_event_t* event);
+int docc_rocm_event_destroy(docc_rocm_event_t event);
+int docc_rocm_event_record(docc_rocm_event_t event, docc_rocm_stream_t stream);
+int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, float* ms);
+
+/* Message of the last failure on this thread ("" if none). */
+const char* docc_rocm_last_error(void);
+
+/* Library version string, e.g. "docc-rocm 0.1 (gfx950)". */
+const char* docc_rocm_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOCC_ROCM_RT_H */

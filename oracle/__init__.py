@@ -1,0 +1,201 @@
+"""ctypes access to the CPU oracle (``oracle/docc_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()``
+and by the ``cpu_baseline`` leg of ``bench.py`` as the checker / the timed CPU
+baseline. The product (``docc_amd``) never imports this package.
+"""
+from __future__ import annotations
+
+import ctypes
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_DIR = Path(__file__).resolve().parent
+_LIB_PATH = _DIR / "libdocc_oracle.so"
+
+NO_TRANS = 111
+TRANS = 112
+
+
+def build(arch: str | None = None, out: str | None = None) -> Path:
+    """Compiles the oracle (``make -C oracle``); returns the library path."""
+    cmd = ["make", "-B", "-C", str(_DIR)]
+    if arch:
+        cmd.append(f"ARCH={arch}")
+    if out:
+        cmd.append(f"OUT={out}")
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("oracle build failed:\n" + proc.stdout + proc.stderr)
+    return Path(out) if out else _LIB_PATH
+
+
+_i64 = ctypes.c_int64
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+
+
+def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
+    lib.oracle_max_threads.restype = ctypes.c_int
+    lib.oracle_set_threads.argtypes = [ctypes.c_int]
+    lib.oracle_f32_to_bf16_array.argtypes = [_i64, _f32p, _u16p]
+    lib.oracle_bf16_to_f32_array.argtypes = [_i64, _u16p, _f32p]
+    for name, ptr, sc in (("f64", _f64p, ctypes.c_double), ("f32", _f32p, ctypes.c_float)):
+        getattr(lib, f"oracle_gemm_expanded_{name}").argtypes = [_i64, _i64, _i64, sc, ptr, _i64, ptr, _i64, sc, ptr, _i64]
+        getattr(lib, f"oracle_gemm_blas_{name}").argtypes = [ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, sc, ptr, _i64, ptr, _i64, sc, ptr, _i64]
+    lib.oracle_gemm_blas_f64_ld.argtypes = lib.oracle_gemm_blas_f64.argtypes
+    lib.oracle_gemm_blas_f32_acc64.argtypes = lib.oracle_gemm_blas_f32.argtypes
+    lib.oracle_gemm_bf16_f32.argtypes = [ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, ctypes.c_float, _u16p, _i64, _u16p, _i64, ctypes.c_float, _f32p, _i64]
+    for name in ("oracle_softmax_expanded_f32", "oracle_softmax_numpy_f32"):
+        getattr(lib, name).argtypes = [_i64, _i64, _f32p, _f32p]
+        getattr(lib, name).restype = ctypes.c_int
+    lib.oracle_conv_out_dim.argtypes = [_i64] * 6
+    lib.oracle_conv_out_dim.restype = _i64
+    lib.oracle_conv2d_f32.argtypes = [_i64] * 13 + [_f32p, _f32p, _f32p, _f32p]
+    lib.oracle_attention_bf16.argtypes = [_i64] * 5 + [ctypes.c_float, _u16p, _u16p, _u16p, _f32p]
+    lib.oracle_attention_bf16.restype = ctypes.c_int
+    return lib
+
+
+_lib: ctypes.CDLL | None = None
+
+
+def load(path: str | Path | None = None) -> ctypes.CDLL:
+    """Loads the oracle library, building it first when it does not exist."""
+    global _lib
+    if path is not None:
+        return _declare(ctypes.CDLL(str(path)))
+    if _lib is None:
+        if not _LIB_PATH.exists():
+            build()
+        _lib = _declare(ctypes.CDLL(str(_LIB_PATH)))
+    return _lib
+
+
+def _p(a: np.ndarray, ptr):
+    return a.ctypes.data_as(ptr)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def set_threads(n: int) -> None:
+    load().oracle_set_threads(int(n))
+
+
+def max_threads() -> int:
+    return int(load().oracle_max_threads())
+
+
+def f32_to_bf16(x) -> np.ndarray:
+    """fp32 array -> bf16 bits (uint16), round to nearest even."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    load().oracle_f32_to_bf16_array(x.size, _p(x, _f32p), _p(out, _u16p))
+    return out
+
+
+def bf16_to_f32(h) -> np.ndarray:
+    h = _c(h, np.uint16)
+    out = np.empty(h.shape, np.float32)
+    load().oracle_bf16_to_f32_array(h.size, _p(h, _u16p), _p(out, _f32p))
+    return out
+
+
+def _gemm_dims(A, B, trans_a, trans_b):
+    m, k = (A.shape[1], A.shape[0]) if trans_a == TRANS else A.shape
+    k2, n = (B.shape[1], B.shape[0]) if trans_b == TRANS else B.shape
+    if k != k2:
+        raise ValueError(f"inner dimensions differ: {k} vs {k2}")
+    return m, n, k
+
+
+def gemm(A, B, C=None, alpha=1.0, beta=0.0, trans_a=NO_TRANS, trans_b=NO_TRANS, variant="blas", lib=None) -> np.ndarray:
+    """C = alpha*op(A)*op(B) + beta*C on fp64 or fp32 arrays.
+
+    variant: "blas" (cblas semantics), "expanded" (the reference's loop nest,
+    NN only), "ld" (fp64 data, long-double accumulate) or "acc64" (fp32 data,
+    fp64 accumulate).
+    """
+    lib = lib or load()
+    dt = np.float64 if np.asarray(A).dtype == np.float64 else np.float32
+    A = _c(A, dt)
+    B = _c(B, dt)
+    m, n, k = _gemm_dims(A, B, trans_a, trans_b)
+    out = np.zeros((m, n), dt) if C is None else np.array(C, dtype=dt, order="C", copy=True)
+    ptr = _f64p if dt == np.float64 else _f32p
+    sfx = "f64" if dt == np.float64 else "f32"
+    lda, ldb, ldc = max(A.shape[1], 1), max(B.shape[1], 1), max(n, 1)
+    if variant == "expanded":
+        if trans_a != NO_TRANS or trans_b != NO_TRANS:
+            raise ValueError("the reference expands NoTrans/NoTrans only")
+        getattr(lib, f"oracle_gemm_expanded_{sfx}")(m, n, k, alpha, _p(A, ptr), lda, _p(B, ptr), ldb, beta, _p(out, ptr), ldc)
+        return out
+    name = {"blas": f"oracle_gemm_blas_{sfx}", "ld": "oracle_gemm_blas_f64_ld", "acc64": "oracle_gemm_blas_f32_acc64"}[variant]
+    getattr(lib, name)(trans_a, trans_b, m, n, k, alpha, _p(A, ptr), lda, _p(B, ptr), ldb, beta, _p(out, ptr), ldc)
+    return out
+
+
+def gemm_bf16(A_bits, B_bits, C=None, alpha=1.0, beta=0.0, trans_a=NO_TRANS, trans_b=NO_TRANS, lib=None) -> np.ndarray:
+    """bf16 bits in, fp32 accumulate and output."""
+    lib = lib or load()
+    A = _c(A_bits, np.uint16)
+    B = _c(B_bits, np.uint16)
+    m, n, k = _gemm_dims(A, B, trans_a, trans_b)
+    out = np.zeros((m, n), np.float32) if C is None else np.array(C, dtype=np.float32, order="C", copy=True)
+    lib.oracle_gemm_bf16_f32(trans_a, trans_b, m, n, k, alpha, _p(A, _u16p), max(A.shape[1], 1), _p(B, _u16p), max(B.shape[1], 1), beta, _p(out, _f32p), max(n, 1))
+    return out
+
+
+def softmax(X, variant="numpy", lib=None) -> np.ndarray:
+    """Row softmax over the last axis of an fp32 array of any rank."""
+    lib = lib or load()
+    X = _c(X, np.float32)
+    cols = X.shape[-1] if X.ndim else 1
+    rows = X.size // cols if cols else 0
+    out = np.empty_like(X)
+    fn = lib.oracle_softmax_numpy_f32 if variant == "numpy" else lib.oracle_softmax_expanded_f32
+    if fn(rows, cols, _p(X, _f32p), _p(out, _f32p)) != 0:
+        raise MemoryError("oracle softmax could not allocate its temporaries")
+    return out
+
+
+def conv_out_dim(d_in, pad, dilation, kernel, stride) -> int:
+    return int(load().oracle_conv_out_dim(d_in, pad, pad, dilation, kernel, stride))
+
+
+def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None) -> np.ndarray:
+    lib = lib or load()
+    X = _c(X, np.float32)
+    W = _c(W, np.float32)
+    N, C, H, Wd = X.shape
+    OC, C2, KH, KW = W.shape
+    if C2 != C:
+        raise ValueError("group != 1 is not supported")
+    OH = conv_out_dim(H, pad[0], dilation[0], KH, stride[0])
+    OW = conv_out_dim(Wd, pad[1], dilation[1], KW, stride[1])
+    Y = np.empty((N, OC, OH, OW), np.float32)
+    b = None if bias is None else _c(bias, np.float32)
+    lib.oracle_conv2d_f32(N, C, H, Wd, OC, KH, KW, stride[0], stride[1], pad[0], pad[1], dilation[0], dilation[1],
+                          _p(X, _f32p), _p(W, _f32p), _p(b, _f32p) if b is not None else None, _p(Y, _f32p))
+    return Y
+
+
+def attention(Q_bits, K_bits, V_bits, scale=None, lib=None) -> np.ndarray:
+    """bf16 bits [B,H,S,D] in, fp32 [B,H,SQ,D] out."""
+    lib = lib or load()
+    Q = _c(Q_bits, np.uint16)
+    K = _c(K_bits, np.uint16)
+    V = _c(V_bits, np.uint16)
+    B, H, SQ, D = Q.shape
+    SKV = K.shape[2]
+    if scale is None:
+        scale = 1.0 / float(np.sqrt(D))
+    O = np.empty((B, H, SQ, D), np.float32)
+    if lib.oracle_attention_bf16(B, H, SQ, SKV, D, scale, _p(Q, _u16p), _p(K, _u16p), _p(V, _u16p), _p(O, _f32p)) != 0:
+        raise MemoryError("oracle attention could not allocate its scratch row")
+    return O

@@ -1,0 +1,397 @@
+/*
+ * docc_oracle.c - CPU restatement of what docc's `openmp` target computes for
+ * the math library nodes GEMM, Softmax and Conv, plus closed-form references
+ * for the two node modes the rocm target adds (bf16 GEMM, Attention).
+ *
+ * THIS IS TEST INFRASTRUCTURE. It is the checker that the parity tests, the
+ * smoke test and the `cpu_baseline` leg of the benchmark compare against and
+ * time. Nothing in the product path may call it; the product path fails when
+ * its HIP library is missing instead of falling back to this file.
+ *
+ * Every function names the reference code it follows (paths relative to the
+ * reference tree). Loop structure mirrors the reference's expansions: Maps
+ * become `for` loops of which only the outermost carries
+ * `#pragma omp parallel for schedule(static)`, as OMPScheduler parallelises
+ * only the outermost Map (opt/src/passes/scheduler/omp_scheduler.cpp:9-20) and
+ * OMPMapDispatcher prints exactly that pragma
+ * (opt/src/targets/omp/codegen/omp_map_dispatcher.cpp:46-82); reductions are
+ * sequential `For` loops. Build with the reference JIT's flags
+ * (python/bindings/py_structured_sdfg.cpp:456,516):
+ *   gcc -O3 -march=native -mtune=native -funroll-loops -fopenmp -fPIC -shared
+ *
+ * How each function is pinned (see tests/test_oracle.py):
+ *   gemm_*      integer-valued known-answer products (exact in every
+ *               summation order), identity / permutation / rank-1 cases,
+ *               numpy.matmul, long-double accumulation bound;
+ *   softmax_*   scipy.special.softmax in fp64, row-sum / shift-invariance /
+ *               constant-row closed forms;
+ *   conv2d_f32  torch.nn.functional.conv2d in fp64, delta-kernel identity and
+ *               shift, all-ones tap counts at corner/edge/interior, bias-only;
+ *   attention   torch SDPA (math path) in fp64, equal-keys => mean of V,
+ *               key-permutation invariance;
+ *   bf16 conversion: exhaustive against torch's round-to-nearest-even.
+ * The reference holds no numeric golden vectors for any of these nodes (its
+ * tests recompute expectations with numpy/torch at run time), so the pins
+ * above are the mathematics and the library cross-checks.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORACLE_API __attribute__((visibility("default")))
+
+ORACLE_API int oracle_max_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+ORACLE_API void oracle_set_threads(int n) {
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+#else
+    (void) n;
+#endif
+}
+
+/* ------------------------------------------------------------------ bf16 */
+
+/* fp32 -> bf16 bits, round to nearest even; the value the reference's BFloat
+ * type (`__bf16`, sdfg/src/codegen/language_extensions/cpp_language_extension.cpp:9-52)
+ * takes on conversion from float. */
+ORACLE_API uint16_t oracle_f32_to_bf16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t) ((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t) (u >> 16);
+}
+
+ORACLE_API float oracle_bf16_to_f32(uint16_t h) {
+    uint32_t u = (uint32_t) h << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+ORACLE_API void oracle_f32_to_bf16_array(int64_t n, const float* src, uint16_t* dst) {
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_f32_to_bf16(src[i]);
+}
+
+ORACLE_API void oracle_bf16_to_f32_array(int64_t n, const uint16_t* src, float* dst) {
+    for (int64_t i = 0; i < n; i++) dst[i] = oracle_bf16_to_f32(src[i]);
+}
+
+/* ------------------------------------------------------------------ GEMM */
+
+/*
+ * GEMMNode::expand (sdfg/src/data_flow/library_nodes/math/blas/gemm_node.cpp:179-311),
+ * NoTrans/NoTrans only, as the reference expands it:
+ *   Map _i, Map _j: _sum = 0.0; For _k: _sum = A[lda*_i+_k] * B[ldb*_k+_j] + _sum;
+ *   C[ldc*_i+_j] = (_sum * alpha) + (C[ldc*_i+_j] * beta)
+ * The expansion reads C even when beta == 0.
+ */
+#define ORACLE_GEMM_EXPANDED(NAME, T)                                                                          \
+    ORACLE_API void NAME(int64_t m, int64_t n, int64_t k, T alpha, const T* A, int64_t lda, const T* B,        \
+                         int64_t ldb, T beta, T* C, int64_t ldc) {                                             \
+        _Pragma("omp parallel for schedule(static)") for (int64_t _i = 0; _i < m; _i++) {                      \
+            for (int64_t _j = 0; _j < n; _j++) {                                                               \
+                T _sum = (T) 0.0;                                                                              \
+                for (int64_t _k = 0; _k < k; _k++) _sum = A[lda * _i + _k] * B[ldb * _k + _j] + _sum;          \
+                T scaled_sum_temp = _sum * alpha;                                                              \
+                T scaled_input_temp = C[ldc * _i + _j] * beta;                                                 \
+                C[ldc * _i + _j] = scaled_sum_temp + scaled_input_temp;                                        \
+            }                                                                                                  \
+        }                                                                                                      \
+    }
+ORACLE_GEMM_EXPANDED(oracle_gemm_expanded_f64, double)
+ORACLE_GEMM_EXPANDED(oracle_gemm_expanded_f32, float)
+
+/*
+ * The call GEMMNodeDispatcher_BLAS prints (gemm_node.cpp:449-509):
+ *   cblas_?gemm(CblasRowMajor, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
+ * restated from the BLAS definition C = alpha*op(A)*op(B) + beta*C, where C
+ * is not read when beta == 0. trans codes are CBLAS's 111 (NoTrans) / 112
+ * (Trans), the values the node serialises (blas_node.h:49-126). The k-loop
+ * runs left to right in the element type.
+ */
+#define ORACLE_GEMM_BLAS(NAME, T, ACC)                                                                         \
+    ORACLE_API void NAME(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, T alpha, const T* A,       \
+                         int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc) {                    \
+        _Pragma("omp parallel for schedule(static)") for (int64_t i = 0; i < m; i++) {                         \
+            for (int64_t j = 0; j < n; j++) {                                                                  \
+                ACC sum = 0;                                                                                   \
+                for (int64_t p = 0; p < k; p++) {                                                              \
+                    ACC a = (trans_a == 112) ? A[lda * p + i] : A[lda * i + p];                                \
+                    ACC b = (trans_b == 112) ? B[ldb * j + p] : B[ldb * p + j];                                \
+                    sum += a * b;                                                                              \
+                }                                                                                              \
+                ACC r = (ACC) alpha * sum;                                                                     \
+                if (beta != (T) 0) r += (ACC) beta * (ACC) C[ldc * i + j];                                     \
+                C[ldc * i + j] = (T) r;                                                                        \
+            }                                                                                                  \
+        }                                                                                                      \
+    }
+ORACLE_GEMM_BLAS(oracle_gemm_blas_f64, double, double)
+ORACLE_GEMM_BLAS(oracle_gemm_blas_f32, float, float)
+/* long-double accumulation: the yardstick for the 1e-12 fp64 bound */
+ORACLE_GEMM_BLAS(oracle_gemm_blas_f64_ld, double, long double)
+/* fp32 data, fp64 accumulation: the yardstick for the fp32 bound */
+ORACLE_GEMM_BLAS(oracle_gemm_blas_f32_acc64, float, double)
+
+/*
+ * bf16 inputs (raw bits), fp32 accumulate and output. The reference has no
+ * such precision (BLAS_Precision is h,s,d,c,z: blas_node.h:49-55); this is the
+ * closed form C = alpha*A*B + beta*C evaluated in fp32 on the bf16 values,
+ * k left to right.
+ */
+ORACLE_API void oracle_gemm_bf16_f32(int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                                     const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, float beta,
+                                     float* C, int64_t ldc) {
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < m; i++) {
+        for (int64_t j = 0; j < n; j++) {
+            float sum = 0.f;
+            for (int64_t p = 0; p < k; p++) {
+                float a = oracle_bf16_to_f32((trans_a == 112) ? A[lda * p + i] : A[lda * i + p]);
+                float b = oracle_bf16_to_f32((trans_b == 112) ? B[ldb * j + p] : B[ldb * p + j]);
+                sum += a * b;
+            }
+            float r = alpha * sum;
+            if (beta != 0.f) r += beta * C[ldc * i + j];
+            C[ldc * i + j] = r;
+        }
+    }
+}
+
+/* --------------------------------------------------------------- Softmax */
+
+/*
+ * SoftmaxNode::expand over the last axis of X[rows, cols]
+ * (sdfg/src/data_flow/library_nodes/math/tensor/reduce_ops/softmax_node.cpp:112-252):
+ * six malloc'd temporaries, then Max(keepdims) -> Broadcast -> Sub -> Exp ->
+ * Sum(keepdims) -> Broadcast -> Div, each its own loop nest.
+ * Max: identity -INFINITY, fmaxf through memory (max_node.cpp:56-91);
+ * Sum: identity 0.0, left-to-right adds through memory (sum_node.cpp:20-57);
+ * the reduce nests follow ReduceNode::expand (reduce_node.cpp:188-333):
+ * an init nest, then Map over kept dims / For over reduced dims.
+ * The reference never frees the temporaries (no Free nodes); they are freed here.
+ * Returns 0, or -1 when a temporary cannot be allocated.
+ */
+ORACLE_API int oracle_softmax_expanded_f32(int64_t rows, int64_t cols, const float* X, float* Y) {
+    size_t full = (size_t) rows * (size_t) cols;
+    float* tmp_max = (float*) malloc(sizeof(float) * (size_t) (rows ? rows : 1));
+    float* tmp_max_bcast = (float*) malloc(sizeof(float) * (full ? full : 1));
+    float* tmp_sub = (float*) malloc(sizeof(float) * (full ? full : 1));
+    float* tmp_exp = (float*) malloc(sizeof(float) * (full ? full : 1));
+    float* tmp_sum = (float*) malloc(sizeof(float) * (size_t) (rows ? rows : 1));
+    float* tmp_sum_bcast = (float*) malloc(sizeof(float) * (full ? full : 1));
+    int rc = 0;
+    if (!tmp_max || !tmp_max_bcast || !tmp_sub || !tmp_exp || !tmp_sum || !tmp_sum_bcast) {
+        rc = -1;
+        goto done;
+    }
+    /* 1. Max */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++) tmp_max[i] = -INFINITY;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t k = 0; k < cols; k++) tmp_max[i] = fmaxf(X[i * cols + k], tmp_max[i]);
+    /* 1.5 Broadcast */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_max_bcast[i * cols + j] = tmp_max[i];
+    /* 2. Sub */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_sub[i * cols + j] = X[i * cols + j] - tmp_max_bcast[i * cols + j];
+    /* 3. Exp */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_exp[i * cols + j] = expf(tmp_sub[i * cols + j]);
+    /* 4. Sum */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++) tmp_sum[i] = 0.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t k = 0; k < cols; k++) tmp_sum[i] = tmp_exp[i * cols + k] + tmp_sum[i];
+    /* 4.5 Broadcast */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_sum_bcast[i * cols + j] = tmp_sum[i];
+    /* 5. Div */
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) Y[i * cols + j] = tmp_exp[i * cols + j] / tmp_sum_bcast[i * cols + j];
+done:
+    free(tmp_max);
+    free(tmp_max_bcast);
+    free(tmp_sub);
+    free(tmp_exp);
+    free(tmp_sum);
+    free(tmp_sum_bcast);
+    return rc;
+}
+
+/*
+ * The decomposed numpy form the reference's own softmax benchmark compiles
+ * (python/benchmarks/npbench/deep_learning/softmax/test_softmax.py:24-28):
+ *   tmp_max = max(x, -1, keepdims); tmp_out = exp(x - tmp_max);
+ *   tmp_sum = sum(tmp_out, -1, keepdims); return tmp_out / tmp_sum
+ * i.e. a Max-reduce nest, a Sub nest, an Exp nest, a Sum-reduce nest, a Div
+ * nest (broadcast operands are zero-stride views, python/docc/python/functions/numpy.py:1209-1233),
+ * and the copy into the caller's return buffer (python/docc/python/ast_parser.py:1186-1210).
+ * This is the form the `openmp` target can run for fp32 input and the one the
+ * CPU baseline times. Returns 0 or -1 (allocation failure).
+ */
+ORACLE_API int oracle_softmax_numpy_f32(int64_t rows, int64_t cols, const float* X, float* ret) {
+    size_t full = (size_t) rows * (size_t) cols;
+    float* tmp_max = (float*) malloc(sizeof(float) * (size_t) (rows ? rows : 1));
+    float* tmp_sub = (float*) malloc(sizeof(float) * (full ? full : 1));
+    float* tmp_out = (float*) malloc(sizeof(float) * (full ? full : 1));
+    float* tmp_sum = (float*) malloc(sizeof(float) * (size_t) (rows ? rows : 1));
+    float* result = (float*) malloc(sizeof(float) * (full ? full : 1));
+    int rc = 0;
+    if (!tmp_max || !tmp_sub || !tmp_out || !tmp_sum || !result) {
+        rc = -1;
+        goto done;
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++) tmp_max[i] = -INFINITY;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t k = 0; k < cols; k++) tmp_max[i] = fmaxf(X[i * cols + k], tmp_max[i]);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_sub[i * cols + j] = X[i * cols + j] - tmp_max[i];
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) tmp_out[i * cols + j] = expf(tmp_sub[i * cols + j]);
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++) tmp_sum[i] = 0.0f;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t k = 0; k < cols; k++) tmp_sum[i] = tmp_out[i * cols + k] + tmp_sum[i];
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) result[i * cols + j] = tmp_out[i * cols + j] / tmp_sum[i];
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++)
+        for (int64_t j = 0; j < cols; j++) ret[i * cols + j] = result[i * cols + j];
+done:
+    free(tmp_max);
+    free(tmp_sub);
+    free(tmp_out);
+    free(tmp_sum);
+    free(result);
+    return rc;
+}
+
+/* ------------------------------------------------------------------ Conv */
+
+/* Output extent, ConvNode::expand (sdfg/src/data_flow/library_nodes/math/tensor/conv_node.cpp:224-233):
+ * D_out = (D_in + pad_begin + pad_end - dilation*(kernel-1) - 1) / stride + 1 */
+ORACLE_API int64_t oracle_conv_out_dim(int64_t d_in, int64_t pad_begin, int64_t pad_end, int64_t dilation,
+                                       int64_t kernel, int64_t stride) {
+    int64_t num = d_in + pad_begin + pad_end - (dilation * (kernel - 1) + 1);
+    if (num < 0) return 0;
+    return num / stride + 1;
+}
+
+/*
+ * ConvNode::expand (conv_node.cpp:244-437), 2-d, group 1:
+ *   Map n, Map oc, Map od0, Map od1: accum = 0.0;
+ *     For ic, For k0, For k1:
+ *       accum = X[n, ic, od0*s0 - p0 + k0*d0, od1*s1 - p1 + k1*d1] * W[oc, ic, k0, k1] + accum
+ *   Y[n, oc, od0, od1] = accum + B[oc]      (or = accum without a bias edge)
+ * The reference indexes X without a bounds test, so with pad > 0 it reads out
+ * of bounds; the ONNX Conv definition its header cites (conv_node.h:9-22)
+ * pads with zeros, which is what the guard below does.
+ */
+ORACLE_API void oracle_conv2d_f32(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                  int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
+                                  int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y) {
+    int64_t OH = oracle_conv_out_dim(H, pad_h, pad_h, dil_h, KH, stride_h);
+    int64_t OW = oracle_conv_out_dim(W, pad_w, pad_w, dil_w, KW, stride_w);
+#pragma omp parallel for schedule(static)
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t oc = 0; oc < OC; oc++) {
+            for (int64_t od0 = 0; od0 < OH; od0++) {
+                for (int64_t od1 = 0; od1 < OW; od1++) {
+                    float accum = 0.0f;
+                    for (int64_t ic = 0; ic < C; ic++) {
+                        for (int64_t k0 = 0; k0 < KH; k0++) {
+                            for (int64_t k1 = 0; k1 < KW; k1++) {
+                                int64_t ih = od0 * stride_h - pad_h + k0 * dil_h;
+                                int64_t iw = od1 * stride_w - pad_w + k1 * dil_w;
+                                if (ih < 0 || ih >= H || iw < 0 || iw >= W) continue;
+                                accum = X[((n * C + ic) * H + ih) * W + iw] * Wt[((oc * C + ic) * KH + k0) * KW + k1] +
+                                        accum;
+                            }
+                        }
+                    }
+                    Y[((n * OC + oc) * OH + od0) * OW + od1] = bias ? accum + bias[oc] : accum;
+                }
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------- Attention */
+
+/*
+ * softmax(scale * Q K^T) V per (batch, head), non-causal, from bf16 inputs
+ * with fp32 scores, softmax and accumulation. The reference has no attention
+ * node and cannot express batched matmul (mlir/lib/Target/SDFG/LinalgToSDFGTranslator.cpp:517-523),
+ * so this is the closed form, written as the reference would compose it from
+ * its own pieces: MatMul (one GEMM per batch, matmul_node.cpp:366-499), scale,
+ * Softmax over the last axis (softmax_node.cpp:142-252), MatMul.
+ * O is fp32 [B,H,SQ,D]. Returns 0 or -1 (allocation failure).
+ */
+ORACLE_API int oracle_attention_bf16(int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, float scale,
+                                     const uint16_t* Q, const uint16_t* K, const uint16_t* V, float* O) {
+    int64_t BH = B * H;
+    int rc = 0;
+#pragma omp parallel for schedule(static)
+    for (int64_t bh = 0; bh < BH; bh++) {
+        float* s = (float*) malloc(sizeof(float) * (size_t) (SKV ? SKV : 1));
+        if (!s) {
+#pragma omp atomic write
+            rc = -1;
+            continue;
+        }
+        const uint16_t* q = Q + bh * SQ * D;
+        const uint16_t* kk = K + bh * SKV * D;
+        const uint16_t* v = V + bh * SKV * D;
+        float* o = O + bh * SQ * D;
+        for (int64_t i = 0; i < SQ; i++) {
+            float mx = -INFINITY;
+            for (int64_t j = 0; j < SKV; j++) {
+                float sum = 0.f;
+                for (int64_t d = 0; d < D; d++)
+                    sum = oracle_bf16_to_f32(q[i * D + d]) * oracle_bf16_to_f32(kk[j * D + d]) + sum;
+                s[j] = sum * scale;
+                mx = fmaxf(s[j], mx);
+            }
+            float den = 0.f;
+            for (int64_t j = 0; j < SKV; j++) {
+                s[j] = expf(s[j] - mx);
+                den = s[j] + den;
+            }
+            for (int64_t d = 0; d < D; d++) {
+                float acc = 0.f;
+                for (int64_t j = 0; j < SKV; j++) acc = (s[j] / den) * oracle_bf16_to_f32(v[j * D + d]) + acc;
+                o[i * D + d] = acc;
+            }
+        }
+        free(s);
+    }
+    return rc;
+}
