@@ -34,6 +34,8 @@ ROCM = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
 KERNEL_FAMILIES = {
     "util": "util.hip",
     "softmax": "softmax.hip",
+    "gemm_f32": "gemm_f32.hip",
+    "gemm_f64": "gemm_f64.hip",
 }
 
 # packed fp32 VALU ops are switched off for every device compile

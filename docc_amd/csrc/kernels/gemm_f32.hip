@@ -1,0 +1,15 @@
+// fp32 GEMM kernels (v_mfma_f32_32x32x2_f32), see gemm_mfma.h.
+#include "gemm_mfma.h"
+
+DOCC_GEMM_CONFIG(sgemm, float, 128, 128, 16, 2, 2)
+DOCC_GEMM_CONFIG(sgemm, float, 64, 64, 16, 2, 2)
+
+// C = beta * C (the k == 0 case); beta == 0 stores zeros without reading C.
+extern "C" __global__ __launch_bounds__(256) void docc_sgemm_scale_c(float* C, long M, long N, long ldc, float beta) {
+    const long total = M * N;
+    const long stride = (long) gridDim.x * 256;
+    for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        float* p = C + (i / N) * ldc + (i % N);
+        *p = (beta == 0.f) ? 0.f : beta * (*p);
+    }
+}

@@ -1,0 +1,289 @@
+// Tiled MFMA GEMM for fp32 and fp64 on gfx950:
+//   C[M,N] = alpha * op(A) * op(B) + beta * C,   row-major, any M, N, K.
+//
+// Replaces the cblas_?gemm call the reference prints for a GEMM node
+// (sdfg/src/data_flow/library_nodes/math/blas/gemm_node.cpp:474-505).
+//
+// Work decomposition
+//   - one work-group computes a BM x BN tile of C with WM x WN wavefronts,
+//     each wavefront a (BM/WM) x (BN/WN) sub-tile made of MT x MT MFMA tiles
+//     (v_mfma_f32_32x32x2_f32: MT = 32; v_mfma_f64_16x16x4_f64: MT = 16);
+//   - K is walked in steps of BK through two LDS buffers: while tile t is
+//     multiplied from one buffer, tile t+1 travels global -> registers and is
+//     stored into the other buffer, one barrier per step;
+//   - the MFMA k-index is permuted so that a lane reads VK consecutive k from
+//     LDS with one 128-bit load: lane group g = lane / MT owns
+//     k = kg*KG + g*VK + s (s < VK), and MFMA step s consumes register s of
+//     every lane. A and B use the same permutation, so the sum is unchanged;
+//   - tiles are numbered so that the work-groups that land on one XCD (ids
+//     congruent mod 8) cover a compact block of C and share A/B panels in
+//     that XCD's L2.
+#pragma once
+
+#include "common.h"
+
+namespace docc_k {
+
+template <typename T>
+struct Mfma;
+
+template <>
+struct Mfma<float> {
+    static constexpr int MT = 32;  // MFMA tile edge
+    static constexpr int G = 2;    // lane groups along k
+    static constexpr int VK = 4;   // consecutive k per lane per LDS read (16 bytes)
+    static constexpr int VEC = 4;  // elements per 128-bit global access
+    static constexpr int NACC = 16;
+    typedef f32x16 acc_t;
+    typedef f32x4 vec_t;
+    static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+    }
+    // row of accumulator register r inside the MT x MT tile (column is lane % MT)
+    static __device__ __forceinline__ int acc_row(int lane, int r) { return 8 * (r / 4) + (lane / 32) * 4 + (r % 4); }
+};
+
+typedef double f64x2 __attribute__((ext_vector_type(2)));
+
+template <>
+struct Mfma<double> {
+    static constexpr int MT = 16;
+    static constexpr int G = 4;
+    static constexpr int VK = 2;
+    static constexpr int VEC = 2;
+    static constexpr int NACC = 4;
+    typedef f64x4 acc_t;
+    typedef f64x2 vec_t;
+    static __device__ __forceinline__ acc_t mfma(double a, double b, acc_t c) {
+        return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int acc_row(int lane, int r) { return 4 * r + lane / 16; }
+};
+
+// Tile id -> tile coordinates: XCD-contiguous renumbering, then grouped
+// ordering (GROUP_M rows of tiles at a time) inside each XCD's range.
+__device__ __forceinline__ void gemm_tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int kXcd = 8;
+    constexpr int GROUP_M = 8;
+    const int total = tiles_m * tiles_n;
+    const int per = total / kXcd;
+    if (pid < per * kXcd) pid = (pid % kXcd) * per + pid / kXcd;
+    const int width = GROUP_M * tiles_n;
+    const int group = pid / width;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    tm = first_m + (pid % width) % gsize;
+    tn = (pid % width) / gsize;
+}
+
+// Global -> registers for a ROWS x COLS tile (COLS contiguous in memory) of a
+// row-major matrix with leading dimension ld; elements outside [rmax, cmax)
+// read as zero. NT threads, 128-bit accesses when ALIGNED.
+template <typename T, int ROWS, int COLS, int NT, bool ALIGNED>
+struct TileLoader {
+    typedef typename Mfma<T>::vec_t vec_t;
+    static constexpr int VEC = Mfma<T>::VEC;
+    static constexpr int VPR = COLS / VEC;            // vectors per tile row
+    static constexpr int NV = ROWS * VPR / NT;        // vectors per thread
+    static_assert(ROWS * VPR % NT == 0, "tile does not divide among the threads");
+
+    vec_t v[NV];
+
+    __device__ __forceinline__ void load(const T* __restrict__ base, long ld, long r0, long c0, long rmax, long cmax,
+                                         int tid) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = tid + i * NT;
+            const long r = r0 + idx / VPR;
+            const long c = c0 + (idx % VPR) * VEC;
+            vec_t val;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) val[e] = (T) 0;
+            if (r < rmax) {
+                const T* p = base + r * ld + c;
+                if (ALIGNED && c + VEC <= cmax) {
+                    val = *reinterpret_cast<const vec_t*>(p);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VEC; e++)
+                        if (c + e < cmax) val[e] = p[e];
+                }
+            }
+            v[i] = val;
+        }
+    }
+
+    // registers -> LDS tile with row stride LDS_LD elements
+    template <int LDS_LD>
+    __device__ __forceinline__ void store(T* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = tid + i * NT;
+            const int r = idx / VPR;
+            const int c = (idx % VPR) * VEC;
+            *reinterpret_cast<vec_t*>(lds + r * LDS_LD + c) = v[i];
+        }
+    }
+};
+
+// TA / TB: the operand is stored transposed in memory (A as [K,M], B as [N,K]).
+// "k-contiguous" operands (A when !TA, B when TB) live in LDS as [MN][BK+PADK];
+// "mn-contiguous" ones (A when TA, B when !TB) as [BK][MN+PADM].
+template <typename T, int BM, int BN, int BK, int WM, int WN, bool TA, bool TB, bool ALIGNED>
+struct GemmKernel {
+    typedef Mfma<T> X;
+    typedef typename X::acc_t acc_t;
+    typedef typename X::vec_t vec_t;
+    static constexpr int NT = 64 * WM * WN;
+    static constexpr int MT = X::MT;
+    static constexpr int VK = X::VK;
+    static constexpr int KG = X::G * VK;  // k consumed per LDS read round
+    static constexpr int WTM = BM / WM, WTN = BN / WN;
+    static constexpr int TM = WTM / MT, TN = WTN / MT;
+    static constexpr int PADK = 16 / sizeof(T);
+    static constexpr int PADM = 8;
+    static constexpr bool A_KC = !TA, B_KC = TB;
+    static constexpr int LDA_S = A_KC ? BK + PADK : BM + PADM;
+    static constexpr int LDB_S = B_KC ? BK + PADK : BN + PADM;
+    static constexpr int A_ELEMS = A_KC ? BM * LDA_S : BK * LDA_S;
+    static constexpr int B_ELEMS = B_KC ? BN * LDB_S : BK * LDB_S;
+    static constexpr int LDS_BYTES = 2 * (A_ELEMS + B_ELEMS) * (int) sizeof(T);
+    static_assert(BK % KG == 0, "BK must be a multiple of the k-group");
+    static_assert(WTM % MT == 0 && WTN % MT == 0, "wave tile must be a multiple of the MFMA tile");
+
+    typedef TileLoader<T, A_KC ? BM : BK, A_KC ? BK : BM, NT, ALIGNED> ALoader;
+    typedef TileLoader<T, B_KC ? BN : BK, B_KC ? BK : BN, NT, ALIGNED> BLoader;
+
+    static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
+                                               long M, long N, long K, long lda, long ldb, long ldc, T alpha,
+                                               T beta) {
+        // all LDS addressing is derived from this one array so that the
+        // compiler keeps it in the LDS address space (ds_* instructions)
+        extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
+        T* const lds = reinterpret_cast<T*>(docc_gemm_lds);
+        const int tid = threadIdx.x;
+        const int lane = tid & 63;
+        const int wave = tid >> 6;
+        const int wm = wave / WN, wn = wave % WN;
+        const int tiles_m = (int) ((M + BM - 1) / BM), tiles_n = (int) ((N + BN - 1) / BN);
+        int tm, tn;
+        gemm_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        const long m0 = (long) tm * BM, n0 = (long) tn * BN;
+
+        // LDS: A buffers at [0, 2*A_ELEMS), B buffers behind them
+        constexpr int B_BASE = 2 * A_ELEMS;
+
+        acc_t acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < X::NACC; r++) acc[i][j][r] = (T) 0;
+
+        ALoader la;
+        BLoader lb;
+        auto gload = [&](long k0) {
+            if (A_KC) la.load(A, lda, m0, k0, M, K, tid);
+            else la.load(A, lda, k0, m0, K, M, tid);
+            if (B_KC) lb.load(B, ldb, n0, k0, N, K, tid);
+            else lb.load(B, ldb, k0, n0, K, N, tid);
+        };
+
+        const int ktiles = (int) ((K + BK - 1) / BK);
+        gload(0);
+        la.template store<LDA_S>(lds, tid);
+        lb.template store<LDB_S>(lds + B_BASE, tid);
+        __syncthreads();
+
+        const int lrow = lane % MT;          // row (A) / column (B) inside an MFMA tile
+        const int lk = (lane / MT) * VK;     // this lane's first k inside a k-group
+
+        for (int kt = 0; kt < ktiles; kt++) {
+            const int cur = kt & 1;
+            if (kt + 1 < ktiles) gload((long) (kt + 1) * BK);
+            const T* as = lds + cur * A_ELEMS;
+            const T* bs = lds + B_BASE + cur * B_ELEMS;
+#pragma unroll
+            for (int kg = 0; kg < BK / KG; kg++) {
+                T a[TM][VK], b[TN][VK];
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const int row = wm * WTM + i * MT + lrow;
+                    if (A_KC) {
+                        vec_t t = *reinterpret_cast<const vec_t*>(as + row * LDA_S + kg * KG + lk);
+#pragma unroll
+                        for (int s = 0; s < VK; s++) a[i][s] = t[s];
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < VK; s++) a[i][s] = as[(kg * KG + lk + s) * LDA_S + row];
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    const int col = wn * WTN + j * MT + lrow;
+                    if (B_KC) {
+                        vec_t t = *reinterpret_cast<const vec_t*>(bs + col * LDB_S + kg * KG + lk);
+#pragma unroll
+                        for (int s = 0; s < VK; s++) b[j][s] = t[s];
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < VK; s++) b[j][s] = bs[(kg * KG + lk + s) * LDB_S + col];
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < VK; s++)
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++) acc[i][j] = X::mfma(a[i][s], b[j][s], acc[i][j]);
+            }
+            if (kt + 1 < ktiles) {
+                la.template store<LDA_S>(lds + (cur ^ 1) * A_ELEMS, tid);
+                lb.template store<LDB_S>(lds + B_BASE + (cur ^ 1) * B_ELEMS, tid);
+            }
+            __syncthreads();
+        }
+
+        // epilogue: C = alpha*acc + beta*C; C is not read when beta == 0
+        const bool use_c = (beta != (T) 0);
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const long col = n0 + wn * WTN + j * MT + lrow;
+#pragma unroll
+                for (int r = 0; r < X::NACC; r++) {
+                    const long row = m0 + wm * WTM + i * MT + X::acc_row(lane, r);
+                    if (row < M && col < N) {
+                        T* p = C + row * ldc + col;
+                        T val = alpha * acc[i][j][r];
+                        if (use_c) val += beta * (*p);
+                        *p = val;
+                    }
+                }
+            }
+        }
+    }
+};
+
+} // namespace docc_k
+
+// Defines the four transpose variants x {aligned, unaligned} of one tile
+// configuration as extern "C" kernels named
+//   docc_<prefix>_<BM>x<BN>x<BK>_<nn|nt|tn|tt>_<a|u>
+#define DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, TA, TB, TAG, AL, ALTAG)                                   \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_##PREFIX##_##BM##x##BN##x##BK##_##TAG##_##ALTAG( \
+        const T* A, const T* B, T* C, long M, long N, long K, long lda, long ldb, long ldc, T alpha, T beta) {  \
+        docc_k::GemmKernel<T, BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta); \
+    }
+
+#define DOCC_GEMM_CONFIG(PREFIX, T, BM, BN, BK, WM, WN)                    \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, false, false, nn, true, a)  \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, false, true, nt, true, a)   \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, true, false, tn, true, a)   \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, true, true, tt, true, a)    \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, false, false, nn, false, u) \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, false, true, nt, false, u)  \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, true, false, tn, false, u)  \
+    DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, true, true, tt, false, u)

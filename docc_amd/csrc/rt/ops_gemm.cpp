@@ -1,0 +1,83 @@
+// Launchers for the GEMM node kernels (see include/docc_rocm_ops.h).
+#include <cstdio>
+
+#include "docc_rocm_ops.h"
+#include "rt_state.h"
+
+using namespace docc::rt::rocm;
+
+namespace {
+
+struct TileConfig {
+    int bm, bn, bk, waves;
+};
+
+// LDS bytes of GemmKernel<T, BM, BN, BK, ...> (csrc/kernels/gemm_mfma.h)
+size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
+    const int padk = (int) (16 / elem), padm = 8;
+    const bool a_kc = !ta, b_kc = tb;
+    const int lda_s = a_kc ? c.bk + padk : c.bm + padm;
+    const int ldb_s = b_kc ? c.bk + padk : c.bn + padm;
+    const size_t a_elems = (size_t) (a_kc ? c.bm : c.bk) * lda_s;
+    const size_t b_elems = (size_t) (b_kc ? c.bn : c.bk) * ldb_s;
+    return 2 * (a_elems + b_elems) * elem;
+}
+
+template <typename T>
+int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n,
+                int64_t k, T alpha, const T* A, int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc,
+                const TileConfig& big, const TileConfig& small, int64_t big_min_tiles) {
+    if ((trans_a != DOCC_ROCM_NO_TRANS && trans_a != DOCC_ROCM_TRANS) ||
+        (trans_b != DOCC_ROCM_NO_TRANS && trans_b != DOCC_ROCM_TRANS))
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: transpose code must be 111 or 112", prefix);
+    if (m < 0 || n < 0 || k < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: negative dimension", prefix);
+    const bool ta = trans_a == DOCC_ROCM_TRANS, tb = trans_b == DOCC_ROCM_TRANS;
+    const int64_t a_cols = ta ? m : k, b_cols = tb ? k : n;
+    if (lda < (a_cols > 1 ? a_cols : 1) || ldb < (b_cols > 1 ? b_cols : 1) || ldc < (n > 1 ? n : 1))
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: leading dimension too small (lda=%lld ldb=%lld ldc=%lld)",
+                    prefix, (long long) lda, (long long) ldb, (long long) ldc);
+    if (m == 0 || n == 0) return 0;
+    if (!C || (k > 0 && (!A || !B))) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null pointer", prefix);
+    int rc = ensure_device();
+    if (rc) return rc;
+    hipStream_t s = (hipStream_t) stream;
+    char name[96];
+    if (k == 0) {
+        std::snprintf(name, sizeof(name), "docc_%s_scale_c", prefix);
+        int64_t blocks = (m * n + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        return launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
+    }
+    const int64_t big_tiles = ((m + big.bm - 1) / big.bm) * ((n + big.bn - 1) / big.bn);
+    const TileConfig& cfg = big_tiles >= big_min_tiles ? big : small;
+    const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
+    if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
+    const size_t vec = 16 / sizeof(T);
+    const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0);
+    std::snprintf(name, sizeof(name), "docc_%s_%dx%dx%d_%c%c_%c", prefix, cfg.bm, cfg.bn, cfg.bk, ta ? 't' : 'n',
+                  tb ? 't' : 'n', aligned ? 'a' : 'u');
+    const size_t lds = gemm_lds_bytes(cfg, ta, tb, sizeof(T));
+    return launch(name, (uint32_t) tiles, 1, 1, 64 * cfg.waves, (uint32_t) lds, s, A, B, C, (long) m, (long) n,
+                  (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta);
+}
+
+} // namespace
+
+extern "C" {
+
+int docc_rocm_sgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                    const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C, int64_t ldc) {
+    static const TileConfig big{128, 128, 16, 4}, small{64, 64, 16, 4};
+    return gemm_launch<float>("sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, big,
+                              small, 192);
+}
+
+int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                    double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta, double* C,
+                    int64_t ldc) {
+    static const TileConfig big{128, 128, 16, 4}, small{64, 64, 16, 4};
+    return gemm_launch<double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, big,
+                               small, 512);
+}
+
+} // extern "C"

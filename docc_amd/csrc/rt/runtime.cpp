@@ -26,6 +26,8 @@ thread_local std::string g_last_error;
 const char* const kKernelImages[] = {
     "docc_rocm_util.hsaco",
     "docc_rocm_softmax.hsaco",
+    "docc_rocm_gemm_f32.hsaco",
+    "docc_rocm_gemm_f64.hsaco",
 };
 
 struct DeviceState {

@@ -1,0 +1,170 @@
+"""GEMM node on the GPU against the CPU oracle, through the C-ABI
+(docc_rocm_dgemm / docc_rocm_sgemm).
+
+Tolerances (norm-wise relative error max|C - C_ref| / max|C_ref|):
+fp64 1e-12, fp32 1e-5. Integer-valued inputs are compared bit-exactly: every
+product and partial sum is exactly representable, so the result does not
+depend on summation order.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, host, rel_err_max
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.float64: 1e-12, np.float32: 1e-5}
+N, T = oracle.NO_TRANS, oracle.TRANS
+
+
+def run_gemm(rt, A, B, C=None, alpha=1.0, beta=0.0, ta=N, tb=N, lda=None, ldb=None, ldc=None, offset=0):
+    """Calls the C-ABI on device copies of A, B (2-d arrays as stored) and C."""
+    dt = A.dtype.type
+    m, k = (A.shape[1], A.shape[0]) if ta == T else A.shape
+    n = B.shape[0] if tb == T else B.shape[1]
+
+    def padded(M, ld):
+        # store M with leading dimension ld (>= cols), optionally shifted by `offset` elements
+        ld = ld or max(M.shape[1], 1)
+        buf = np.full(offset + max(M.shape[0], 1) * ld, np.nan, dt)
+        view = buf[offset:offset + M.shape[0] * ld].reshape(M.shape[0], ld)
+        view[:, :M.shape[1]] = M
+        return buf, ld
+
+    a_buf, lda = padded(A, lda)
+    b_buf, ldb = padded(B, ldb)
+    c_init = np.full((m, n), np.nan, dt) if C is None else C
+    c_buf, ldc = padded(c_init, ldc)
+    a, b, c = dev(a_buf), dev(b_buf), dev(c_buf)
+    es = a.element_size()
+    fn = rt.dgemm if dt == np.float64 else rt.sgemm
+    fn(m, n, k, alpha, a.data_ptr() + offset * es, lda, b.data_ptr() + offset * es, ldb, beta,
+       c.data_ptr() + offset * es, ldc, trans_a=ta, trans_b=tb)
+    torch.cuda.synchronize()
+    out = host(c)[offset:offset + m * ldc].reshape(m, ldc) if m else np.empty((0, ldc), dt)
+    if ldc > n and m:
+        assert np.isnan(out[:, n:]).all(), "kernel wrote into the padding of C"
+    return out[:, :n].copy()
+
+
+def int_matrix(rng, shape, dt, lim=8):
+    return rng.integers(-lim, lim + 1, shape).astype(dt)
+
+
+SHAPES = [(1, 1, 1), (17, 33, 65), (33, 17, 5), (64, 64, 64), (65, 63, 130), (128, 128, 16), (129, 257, 31),
+          (257, 129, 100), (1, 300, 7), (300, 1, 7), (40, 50, 1), (200, 136, 1024)]
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+@pytest.mark.parametrize("m,n,k", SHAPES)
+def test_gemm_integer_exact_nn(rt, dt, m, n, k):
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k)
+    A, B = int_matrix(rng, (m, k), dt), int_matrix(rng, (k, n), dt)
+    C = run_gemm(rt, A, B)
+    assert np.array_equal(C, oracle.gemm(A, B))
+    assert np.array_equal(C, (A.astype(np.float64) @ B.astype(np.float64)).astype(dt))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+@pytest.mark.parametrize("ta,tb", [(N, T), (T, N), (T, T)])
+@pytest.mark.parametrize("m,n,k", [(17, 33, 65), (130, 70, 40), (64, 128, 256), (5, 3, 2)])
+def test_gemm_integer_exact_transposed(rt, dt, ta, tb, m, n, k):
+    rng = np.random.default_rng(7 + m + n + k)
+    A = int_matrix(rng, (k, m) if ta == T else (m, k), dt)
+    B = int_matrix(rng, (n, k) if tb == T else (k, n), dt)
+    C = run_gemm(rt, A, B, ta=ta, tb=tb)
+    assert np.array_equal(C, oracle.gemm(A, B, trans_a=ta, trans_b=tb))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_gemm_alpha_beta_ld_and_alignment(rt, dt):
+    rng = np.random.default_rng(11)
+    m, n, k = 70, 45, 33
+    A, B, C0 = int_matrix(rng, (m, k), dt), int_matrix(rng, (k, n), dt), int_matrix(rng, (m, n), dt)
+    ref = oracle.gemm(A, B, C0, alpha=2.0, beta=-3.0)
+    # padded leading dimensions (aligned path)
+    assert np.array_equal(run_gemm(rt, A, B, C0, 2.0, -3.0, lda=40, ldb=48, ldc=52), ref)
+    # odd leading dimensions and a one-element pointer offset (unaligned path)
+    assert np.array_equal(run_gemm(rt, A, B, C0, 2.0, -3.0, lda=35, ldb=47, ldc=49, offset=1), ref)
+    # beta == 0: C is not read (it holds NaNs), as cblas specifies
+    out = run_gemm(rt, A, B, None, 1.0, 0.0)
+    assert np.isfinite(out).all() and np.array_equal(out, oracle.gemm(A, B))
+    # k == 0: C = beta * C
+    out = run_gemm(rt, np.zeros((m, 0), dt), np.zeros((0, n), dt), C0, 1.0, 2.0)
+    assert np.array_equal(out, 2 * C0)
+    out = run_gemm(rt, np.zeros((m, 0), dt), np.zeros((0, n), dt), None, 1.0, 0.0)
+    assert np.array_equal(out, np.zeros((m, n), dt))
+
+
+@pytest.mark.parametrize("dt", [np.float64, np.float32])
+def test_gemm_structured_cases(rt, dt):
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((100, 100)).astype(dt)
+    eye = np.eye(100, dtype=dt)
+    assert np.array_equal(run_gemm(rt, A, eye), A)
+    assert np.array_equal(run_gemm(rt, eye, A), A)
+    perm = eye[rng.permutation(100)]
+    assert np.array_equal(run_gemm(rt, perm, A), perm @ A)
+    # rank-1 outer product (m x 1 times 1 x n), the shape numpy.outer lowers to
+    u, v = rng.standard_normal((37, 1)).astype(dt), rng.standard_normal((1, 91)).astype(dt)
+    assert np.array_equal(run_gemm(rt, u, v), u @ v)
+    # A @ ones = row sums
+    ones = np.ones((100, 1), dtype=dt)
+    assert rel_err_max(run_gemm(rt, A, ones), A.astype(np.float64).sum(axis=1, keepdims=True)) <= TOL[dt]
+
+
+def test_gemm_errors(rt):
+    from docc_amd.runtime import RocmRuntimeError
+    a = torch.zeros(16, device="cuda")
+    with pytest.raises(RocmRuntimeError):
+        rt.sgemm(4, 4, 4, 1.0, a.data_ptr(), 2, a.data_ptr(), 4, 0.0, a.data_ptr(), 4)  # lda < k
+    with pytest.raises(RocmRuntimeError):
+        rt.sgemm(4, 4, 4, 1.0, a.data_ptr(), 4, a.data_ptr(), 4, 0.0, a.data_ptr(), 4, trans_a=7)
+    with pytest.raises(RocmRuntimeError):
+        rt.sgemm(-1, 4, 4, 1.0, a.data_ptr(), 4, a.data_ptr(), 4, 0.0, a.data_ptr(), 4)
+    rt.sgemm(0, 4, 4, 1.0, 0, 4, 0, 4, 0.0, 0, 4)  # empty: no-op
+
+
+def test_dgemm_config_1000(rt):
+    # benchmark configuration 1: uniform[0,1) 1000x1000 fp64, seed 0, vs a long-double accumulation
+    rng = np.random.default_rng(0)
+    A, B = rng.random((1000, 1000)), rng.random((1000, 1000))
+    C = run_gemm(rt, A, B)
+    ref = oracle.gemm(A, B, variant="ld")
+    assert rel_err_max(C, ref) <= 1e-12
+    # and against the form the reference's openmp target computes (cblas semantics, fp64 accumulate)
+    assert rel_err_max(C, oracle.gemm(A, B)) <= 1e-12
+
+
+def test_sgemm_random_medium(rt):
+    rng = np.random.default_rng(2)
+    A = (rng.standard_normal((300, 700)) / np.sqrt(700)).astype(np.float32)
+    B = (rng.standard_normal((700, 260)) / np.sqrt(700)).astype(np.float32)
+    C = run_gemm(rt, A, B)
+    assert rel_err_max(C, oracle.gemm(A, B, variant="acc64")) <= 1e-5
+    assert rel_err_max(C, oracle.gemm(A, B)) <= 1e-5
+
+
+def test_sgemm_config_4096(rt):
+    # benchmark configuration 3a: N(0,1)/sqrt(K), 4096^3 fp32, seed 2
+    rng = np.random.default_rng(2)
+    K = 4096
+    A = (rng.standard_normal((K, K)) / 64).astype(np.float32)
+    B = (rng.standard_normal((K, K)) / 64).astype(np.float32)
+    a, b = dev(A), dev(B)
+    c = torch.full((K, K), float("nan"), device="cuda")
+    rt.sgemm(K, K, K, 1.0, a.data_ptr(), K, b.data_ptr(), K, 0.0, c.data_ptr(), K)
+    torch.cuda.synchronize()
+    C = host(c)
+    assert np.isfinite(C).all()
+    # the oracle on a band of rows (the naive CPU loop nest is the slow side)
+    rows = np.r_[0:24, 2040:2064, 4072:4096]
+    ref = oracle.gemm(A[rows], B, variant="acc64")
+    assert rel_err_max(C[rows], ref) <= 1e-5
+    # size-independent property on the full result: C @ x == A @ (B @ x) for a probe vector, in fp64
+    x = rng.standard_normal(K)
+    lhs = C.astype(np.float64) @ x
+    rhs = A.astype(np.float64) @ (B.astype(np.float64) @ x)
+    assert np.abs(lhs - rhs).max() / np.abs(rhs).max() <= 1e-5
