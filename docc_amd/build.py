@@ -36,6 +36,7 @@ KERNEL_FAMILIES = {
     "softmax": "softmax.hip",
     "gemm_f32": "gemm_f32.hip",
     "gemm_f64": "gemm_f64.hip",
+    "gemm_bf16": "gemm_bf16.hip",
 }
 
 # packed fp32 VALU ops are switched off for every device compile

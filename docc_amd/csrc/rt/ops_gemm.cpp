@@ -1,5 +1,6 @@
 // Launchers for the GEMM node kernels (see include/docc_rocm_ops.h).
 #include <cstdio>
+#include <cstdlib>
 
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
@@ -14,7 +15,8 @@ struct TileConfig {
 
 // LDS bytes of GemmKernel<T, BM, BN, BK, ...> (csrc/kernels/gemm_mfma.h)
 size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
-    const int padk = (int) (16 / elem), padm = 8;
+    // fp32/fp64 pad mn-contiguous rows by 8 elements, bf16 (GemmBf16Kernel) by 16
+    const int padk = (int) (16 / elem), padm = elem == 2 ? 16 : 8;
     const bool a_kc = !ta, b_kc = tb;
     const int lda_s = a_kc ? c.bk + padk : c.bm + padm;
     const int ldb_s = b_kc ? c.bk + padk : c.bn + padm;
@@ -23,9 +25,10 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
     return 2 * (a_elems + b_elems) * elem;
 }
 
-template <typename T>
+// T: element type of A and B; S: type of C, alpha and beta
+template <typename T, typename S = T>
 int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n,
-                int64_t k, T alpha, const T* A, int64_t lda, const T* B, int64_t ldb, T beta, T* C, int64_t ldc,
+                int64_t k, S alpha, const T* A, int64_t lda, const T* B, int64_t ldb, S beta, S* C, int64_t ldc,
                 const TileConfig& big, const TileConfig& small, int64_t big_min_tiles) {
     if ((trans_a != DOCC_ROCM_NO_TRANS && trans_a != DOCC_ROCM_TRANS) ||
         (trans_b != DOCC_ROCM_NO_TRANS && trans_b != DOCC_ROCM_TRANS))
@@ -49,7 +52,12 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         return launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
     }
     const int64_t big_tiles = ((m + big.bm - 1) / big.bm) * ((n + big.bn - 1) / big.bn);
-    const TileConfig& cfg = big_tiles >= big_min_tiles ? big : small;
+    // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
+    const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
+    const bool use_big = force && force[0] == 'b'   ? true
+                         : force && force[0] == 's' ? false
+                                                    : big_tiles >= big_min_tiles;
+    const TileConfig& cfg = use_big ? big : small;
     const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     const size_t vec = 16 / sizeof(T);
@@ -78,6 +86,14 @@ int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t
     static const TileConfig big{128, 128, 16, 4}, small{64, 64, 16, 4};
     return gemm_launch<double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, big,
                                small, 512);
+}
+
+int docc_rocm_bf16gemm_f32(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                           float alpha, const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, float beta,
+                           float* C, int64_t ldc) {
+    static const TileConfig big{256, 256, 64, 4}, small{128, 128, 64, 4};
+    return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C,
+                                        ldc, big, small, 256);
 }
 
 } // extern "C"
