@@ -3,6 +3,5 @@
 #include "rt_state.h"
 using namespace docc::rt::rocm;
 extern "C" {
-int docc_rocm_conv2d_f32(docc_rocm_stream_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, int64_t, const float*, const float*, const float*, float*) { return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: not built"); }
 int docc_rocm_attention_bf16(docc_rocm_stream_t, int64_t, int64_t, int64_t, int64_t, int64_t, float, const uint16_t*, const uint16_t*, const uint16_t*, void*, int) { return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: not built"); }
 }

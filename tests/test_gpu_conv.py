@@ -1,0 +1,120 @@
+"""ml::Conv (2-d, NCHW, fp32) on the GPU against the CPU oracle, through
+docc_rocm_conv2d_f32. Tolerance 1e-5 norm-wise (max|y - y_ref| / max|y_ref|);
+integer-valued inputs are compared bit-exactly."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, host, rel_err_max
+
+pytestmark = pytest.mark.gpu
+
+
+def run_conv(rt, X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1)):
+    N, C, H, Wd = X.shape
+    OC, _, KH, KW = W.shape
+    OH = oracle.conv_out_dim(H, pad[0], dilation[0], KH, stride[0])
+    OW = oracle.conv_out_dim(Wd, pad[1], dilation[1], KW, stride[1])
+    x, w = dev(X), dev(W)
+    b = dev(bias) if bias is not None else None
+    y = torch.full((N, OC, OH, OW), float("nan"), device="cuda")
+    rt.conv2d_f32(N, C, H, Wd, OC, KH, KW, stride, pad, dilation, x.data_ptr(), w.data_ptr(),
+                  b.data_ptr() if b is not None else 0, y.data_ptr())
+    torch.cuda.synchronize()
+    return host(y)
+
+
+CASES = [
+    # N, C, H, W, OC, KH, KW, stride, pad, dil, bias
+    (2, 3, 7, 7, 4, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    (1, 2, 5, 5, 3, 3, 3, (1, 1), (0, 0), (1, 1), False),
+    (2, 5, 9, 11, 70, 3, 3, (1, 1), (1, 1), (1, 1), True),     # OC > one tile of 64
+    (3, 4, 12, 10, 8, 1, 1, (1, 1), (0, 0), (1, 1), True),     # 1x1
+    (2, 3, 13, 9, 5, 5, 3, (2, 1), (2, 1), (1, 1), True),      # rectangular kernel, mixed stride
+    (2, 3, 16, 16, 6, 3, 3, (2, 2), (1, 1), (2, 2), False),    # stride + dilation
+    (1, 7, 8, 8, 9, 7, 7, (1, 1), (3, 3), (1, 1), True),       # kernel ~ image
+    (4, 16, 20, 20, 32, 3, 3, (1, 1), (1, 1), (1, 1), True),
+    (1, 1, 4, 4, 1, 3, 3, (1, 1), (2, 2), (1, 1), False),      # pad larger than needed
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_integer_exact(rt, case):
+    N, C, H, W, OC, KH, KW, stride, pad, dil, use_bias = case
+    rng = np.random.default_rng(hash(case[:7]) & 0xffff)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, C, KH, KW)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    Y = run_conv(rt, X, Wt, b, stride, pad, dil)
+    ref = oracle.conv2d(X, Wt, b, stride, pad, dil)
+    assert Y.shape == ref.shape
+    assert np.array_equal(Y, ref)
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_conv_random_matches_oracle(rt, case):
+    N, C, H, W, OC, KH, KW, stride, pad, dil, use_bias = case
+    rng = np.random.default_rng(1 + (hash(case[:7]) & 0xffff))
+    X = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    Wt = (rng.standard_normal((OC, C, KH, KW)) * np.sqrt(2.0 / (C * KH * KW))).astype(np.float32)
+    b = (rng.standard_normal(OC) * 0.1).astype(np.float32) if use_bias else None
+    Y = run_conv(rt, X, Wt, b, stride, pad, dil)
+    assert rel_err_max(Y, oracle.conv2d(X, Wt, b, stride, pad, dil)) <= 1e-5
+
+
+def test_conv_closed_forms(rt):
+    rng = np.random.default_rng(0)
+    X = rng.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    # delta kernel per channel -> identity
+    Wt = np.zeros((3, 3, 3, 3), np.float32)
+    for c in range(3):
+        Wt[c, c, 1, 1] = 1.0
+    assert np.array_equal(run_conv(rt, X, Wt, None, pad=(1, 1)), X)
+    # shifted delta -> shift with a zero border
+    Wt[:] = 0
+    for c in range(3):
+        Wt[c, c, 0, 2] = 1.0  # reads X[h-1, w+1]
+    Y = run_conv(rt, X, Wt, None, pad=(1, 1))
+    exp = np.zeros_like(X)
+    exp[:, :, 1:, :-1] = X[:, :, :-1, 1:]
+    assert np.array_equal(Y, exp)
+    # all-ones input and weights: the output counts the taps inside the image (4 / 6 / 9 per channel)
+    C = 64
+    Y = run_conv(rt, np.ones((1, C, 6, 6), np.float32), np.ones((2, C, 3, 3), np.float32), None, pad=(1, 1))
+    assert Y[0, 0, 0, 0] == C * 4 and Y[0, 1, 0, 3] == C * 6 and Y[0, 0, 3, 3] == C * 9 and Y[0, 1, 5, 5] == C * 4
+    # zero weights: the output is the bias
+    b = np.arange(5, dtype=np.float32)
+    Y = run_conv(rt, X, np.zeros((5, 3, 3, 3), np.float32), b, pad=(1, 1))
+    assert np.array_equal(Y, np.broadcast_to(b[None, :, None, None], Y.shape))
+
+
+def test_conv_empty_and_errors(rt):
+    from docc_amd.runtime import RocmRuntimeError
+    rt.conv2d_f32(0, 3, 8, 8, 4, 3, 3, (1, 1), (1, 1), (1, 1), 0, 0, 0, 0)
+    rt.conv2d_f32(1, 3, 2, 2, 4, 3, 3, (1, 1), (0, 0), (1, 1), 0, 0, 0, 0)  # kernel larger than image: empty output
+    with pytest.raises(RocmRuntimeError):
+        rt.conv2d_f32(1, 3, 8, 8, 4, 3, 3, (0, 1), (1, 1), (1, 1), 0, 0, 0, 0)
+
+
+def test_conv_config_resnet_block(rt):
+    # benchmark configuration 5: N=32, 64 -> 64 channels, 56x56, 3x3, stride 1, pad 1, bias
+    g = torch.Generator().manual_seed(4)
+    X = torch.randn(32, 64, 56, 56, generator=g).numpy()
+    Wt = (torch.randn(64, 64, 3, 3, generator=g) * np.sqrt(2.0 / 576)).numpy()
+    b = (torch.randn(64, generator=g) * 0.1).numpy()
+    Y = run_conv(rt, X, Wt, b, pad=(1, 1))
+    assert np.isfinite(Y).all()
+    # oracle on two images (the first and the last)
+    sel = [0, 31]
+    assert rel_err_max(Y[sel], oracle.conv2d(X[sel], Wt, b, pad=(1, 1))) <= 1e-5
+    # full-size property: linearity in the input, conv(X) - conv(0) summed over everything
+    # equals sum_oc sum_ic sum_taps W * (sum of X over the window positions); checked through
+    # the channel-summed output against a conv of the channel structure done in fp64 on the CPU
+    tot = Y.astype(np.float64).sum(axis=(0, 2, 3)) - 32 * 56 * 56 * b.astype(np.float64)
+    Xs = X.astype(np.float64)
+    Xp = np.pad(Xs, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    # S[ic, kh, kw] = sum over n, oh, ow of X[n, ic, oh+kh-1, ow+kw-1]
+    S = np.array([[[Xp[:, ic, kh:kh + 56, kw:kw + 56].sum() for kw in range(3)] for kh in range(3)] for ic in range(64)])
+    exp = np.einsum("oikl,ikl->o", Wt.astype(np.float64), S)
+    assert np.abs(tot - exp).max() / np.abs(exp).max() <= 1e-4
