@@ -38,6 +38,7 @@ KERNEL_FAMILIES = {
     "gemm_f64": "gemm_f64.hip",
     "gemm_bf16": "gemm_bf16.hip",
     "conv2d": "conv2d.hip",
+    "attention": "attention.hip",
 }
 
 # packed fp32 VALU ops are switched off for every device compile

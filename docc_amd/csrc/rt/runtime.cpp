@@ -30,6 +30,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_gemm_f64.hsaco",
     "docc_rocm_gemm_bf16.hsaco",
     "docc_rocm_conv2d.hsaco",
+    "docc_rocm_attention.hsaco",
 };
 
 struct DeviceState {
