@@ -1,0 +1,272 @@
+#!/usr/bin/env python3
+"""Benchmark of the docc `rocm` target's library-node kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--only softmax,dgemm,...] [--no-cpu]
+
+Prints ONE JSON line. The headline (`value`, `roofline`, `cpu_baseline`) is the
+fp32 row softmax over [8192, 4096] (one step = one launch over one such
+tensor, inputs resident in HBM, rotating over four buffer pairs so that the
+256 MB Infinity Cache cannot serve the reads). The other benchmark
+configurations (fp64 GEMM 1000^3, fp32 and bf16 GEMM 4096^3, attention
+B8 H16 S2048 D64, conv2d N32 C64 56x56 3x3) are measured in the same run and
+reported under `kernels`, each with its own roofline fraction and CPU baseline.
+
+Kernel durations are taken with HIP events recorded on the stream the kernels
+are launched on (the null stream). The CPU baseline is the oracle - the C
+restatement of what the reference's `openmp` target emits - rebuilt with
+-march=native on this machine and run on the host cores, on a bounded sample
+where the full problem would take minutes.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import tempfile
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+METRIC = "GEMM/attn/conv TFLOP/s + softmax GB/s, % of roofline, vs openmp host target"
+
+# MI355X published peaks
+PEAK_HBM_GBS = 8000.0
+PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3, "bf16": 2516.6}
+
+# HBM bytes per softmax launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
+# same counters read for the 128 MiB copy kernel; see profiles/softmax_f32_8192x4096_pmc.txt.
+SOFTMAX_TRAFFIC_BYTES = None
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from docc_amd import runtime as rt
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    rt.init(0)
+    info = rt.device_info()
+    only = set(filter(None, args.only.split(",")))
+    want = lambda name: not only or name in only
+    stream = 0  # the null stream: torch allocates and we launch on it
+
+    def time_kernel(fn, iters, warm):
+        """Average launch duration in ms from HIP events around `iters` back-to-back launches."""
+        for i in range(warm):
+            fn(i)
+        rt.device_sync()
+        e0, e1 = rt.Event(), rt.Event()
+        e0.record(stream)
+        for i in range(iters):
+            fn(i)
+        e1.record(stream)
+        return e0.elapsed_ms(e1) / iters
+
+    # ---- CPU side -------------------------------------------------------------------
+    cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "1024")))
+    oracle_lib = None
+    if not args.no_cpu:
+        import oracle
+
+        try:  # the reference compiles its generated code with -march=native on the machine it runs on
+            native = Path(tempfile.gettempdir()) / f"libdocc_oracle_native_{os.getpid()}.so"
+            oracle.build(arch="native", out=str(native))
+            oracle_lib = oracle.load(native)
+            oracle_build = "gcc -O3 -march=native -funroll-loops -fopenmp"
+        except Exception:
+            oracle_lib = oracle.load()
+            oracle_build = "prebuilt x86-64-v3"
+        oracle_lib.oracle_set_threads(cores)
+
+    def cpu_time(fn, reps=3):
+        fn()  # cold run, as the reference's harness does (1 cold + timed runs)
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return statistics.median(ts)
+
+    kernels = {}
+    out = {}
+
+    # ---- headline: softmax [8192, 4096] fp32 --------------------------------------
+    if want("softmax"):
+        R, C = 8192, 4096
+        nbytes = 2 * R * C * 4
+        g = torch.Generator(device="cuda").manual_seed(1)
+        pairs = [(torch.randn(R, C, device="cuda", generator=g) * 8, torch.empty(R, C, device="cuda")) for _ in range(4)]
+        step = lambda i: rt.softmax_f32(R, C, pairs[i % 4][0].data_ptr(), pairs[i % 4][1].data_ptr(), stream)
+        for i in range(args.warmup):
+            step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(i)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        ms_per_step = wall * 1e3 / args.steps
+        kern_ms = time_kernel(step, args.steps, 5)
+        achieved = nbytes / kern_ms / 1e6
+        out.update(value=nbytes / (wall / args.steps) / 1e9, ms_per_step=ms_per_step)
+        out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                           "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": SOFTMAX_TRAFFIC_BYTES,
+                           "kernel": "docc_softmax_f32_wave_v16", "kernel_us": round(kern_ms * 1e3, 2),
+                           "algorithmic_bytes": nbytes}
+        # same number for a plain copy of the same bytes: the practical ceiling of this memory system
+        copy_ms = time_kernel(lambda i: rt.copy_bytes(R * C * 4, pairs[i % 4][0].data_ptr(), pairs[i % 4][1].data_ptr(), stream), 50, 5)
+        out["roofline"]["copy_kernel_GBps"] = round(nbytes / copy_ms / 1e6, 1)
+        if oracle_lib is not None:
+            X = pairs[0][0].cpu().numpy()
+            t = cpu_time(lambda: oracle.softmax(X, lib=oracle_lib))
+            out["cpu_baseline"] = {"value": round(nbytes / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                                   "sample": f"full [8192,4096] tensor, decomposed max/sub/exp/sum/div/copy form, median of 3 after 1 cold run; {oracle_build}"}
+        del pairs
+
+    def add_kernel(name, dtype, flops, ms, cpu=None, extra=None):
+        tf = flops / ms / 1e9
+        entry = {"tflops": round(tf, 2), "kernel_us": round(ms * 1e3, 2), "flop": flops,
+                 "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
+                              "frac": round(tf / PEAK_TFLOPS[dtype], 4)}, "dtype": dtype}
+        if cpu:
+            entry["cpu_baseline"] = cpu
+        if extra:
+            entry.update(extra)
+        kernels[name] = entry
+
+    # ---- config 1: fp64 GEMM 1000^3 ---------------------------------------------------
+    if want("dgemm"):
+        n = 1000
+        A = torch.rand(n, n, device="cuda", dtype=torch.float64)
+        B = torch.rand(n, n, device="cuda", dtype=torch.float64)
+        Cm = torch.empty(n, n, device="cuda", dtype=torch.float64)
+        ms = time_kernel(lambda i: rt.dgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 200, 10)
+        cpu = None
+        if oracle_lib is not None:
+            a, b = A.cpu().numpy(), B.cpu().numpy()
+            t = cpu_time(lambda: oracle.gemm(a, b, variant="expanded", lib=oracle_lib))
+            tb = cpu_time(lambda: a @ b)
+            cpu = {"value": round(2 * n**3 / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                   "sample": "full 1000^3, the reference's expanded loop nest (omp over i)",
+                   "host_blas_tflops": round(2 * n**3 / tb / 1e12, 4), "host_blas": "numpy/OpenBLAS dgemm (the call the reference's BLAS dispatcher emits)"}
+        add_kernel("dgemm_1000", "f64", 2 * n**3, ms, cpu)
+
+    # ---- config 3a: fp32 GEMM 4096^3 ----------------------------------------------------
+    if want("sgemm"):
+        n = 4096
+        A = torch.randn(n, n, device="cuda") / 64
+        B = torch.randn(n, n, device="cuda") / 64
+        Cm = torch.empty(n, n, device="cuda")
+        ms = time_kernel(lambda i: rt.sgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 20, 3)
+        cpu = None
+        if oracle_lib is not None:
+            rows = 128
+            a, b = A[:rows].cpu().numpy(), B.cpu().numpy()
+            t = cpu_time(lambda: oracle.gemm(a, b, variant="expanded", lib=oracle_lib), reps=1)
+            af = A.cpu().numpy()
+            tb = cpu_time(lambda: af @ b, reps=2)
+            cpu = {"value": round(2 * rows * n * n / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                   "sample": f"first {rows} rows of C ({rows}x4096x4096), the reference's expanded loop nest",
+                   "host_blas_tflops": round(2 * n**3 / tb / 1e12, 4), "host_blas": "numpy/OpenBLAS sgemm, full 4096^3"}
+        add_kernel("sgemm_4096", "f32", 2 * n**3, ms, cpu)
+        del A, B, Cm
+
+    # ---- config 3b: bf16 GEMM 4096^3, fp32 accumulate/output ------------------------------
+    if want("bgemm"):
+        n = 4096
+        A = (torch.randn(n, n, device="cuda") / 64).bfloat16()
+        B = (torch.randn(n, n, device="cuda") / 64).bfloat16()
+        Cm = torch.empty(n, n, device="cuda")
+        ms = time_kernel(lambda i: rt.bf16gemm_f32(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 50, 5)
+        cpu = None
+        if oracle_lib is not None:
+            rows = 128
+            a = A[:rows].cpu().view(torch.int16).numpy().view(np.uint16)
+            b = B.cpu().view(torch.int16).numpy().view(np.uint16)
+            t = cpu_time(lambda: oracle.gemm_bf16(a, b, lib=oracle_lib), reps=1)
+            cpu = {"value": round(2 * rows * n * n / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                   "sample": f"first {rows} rows of C, fp32 loop nest on the bf16 values (the reference has no bf16 GEMM)"}
+        add_kernel("bgemm_4096", "bf16", 2 * n**3, ms, cpu)
+        del A, B, Cm
+
+    # ---- config 4: attention B8 H16 S2048 D64 bf16 ----------------------------------------
+    if want("attention"):
+        Bn, H, S, D = 8, 16, 2048, 64
+        Q, K, V = (torch.randn(Bn, H, S, D, device="cuda").bfloat16() for _ in range(3))
+        O = torch.empty(Bn, H, S, D, device="cuda", dtype=torch.bfloat16)
+        ms = time_kernel(lambda i: rt.attention_bf16(Bn, H, S, S, D, 0.125, Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), out_bf16=True, stream=stream), 50, 5)
+        cpu = None
+        if oracle_lib is not None:
+            heads = max(cores, 1)
+            bits = lambda t: t.reshape(Bn * H, S, D)[:heads].reshape(1, heads, S, D).cpu().view(torch.int16).numpy().view(np.uint16)
+            q, k, v = bits(Q), bits(K), bits(V)
+            t = cpu_time(lambda: oracle.attention(q, k, v, 0.125, lib=oracle_lib), reps=1)
+            cpu = {"value": round(4 * heads * S * S * D / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                   "sample": f"{heads} of the 128 (batch, head) pairs, fp32 loop nests (the reference has no attention)"}
+        add_kernel("attention_b8h16s2048d64", "bf16", 4 * Bn * H * S * S * D, ms, cpu)
+        del Q, K, V, O
+
+    # ---- config 5: conv2d N32 C64->64 56x56 3x3 s1 p1 + bias ------------------------------
+    if want("conv"):
+        X = torch.randn(32, 64, 56, 56, device="cuda")
+        W = torch.randn(64, 64, 3, 3, device="cuda") * (2.0 / 576) ** 0.5
+        b = torch.randn(64, device="cuda") * 0.1
+        Y = torch.empty(32, 64, 56, 56, device="cuda")
+        ms = time_kernel(lambda i: rt.conv2d_f32(32, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), stream=stream), 100, 10)
+        flops = 2 * 32 * 64 * 56 * 56 * 64 * 9
+        cpu = None
+        if oracle_lib is not None:
+            x, w, bb = X.cpu().numpy(), W.cpu().numpy(), b.cpu().numpy()
+            t = cpu_time(lambda: oracle.conv2d(x, w, bb, pad=(1, 1), lib=oracle_lib), reps=1)
+            cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+                   "sample": "full problem, the reference's loop nest with a zero-padding guard (omp over n)"}
+        add_kernel("conv2d_n32c64hw56k3", "f32", flops, ms, cpu)
+
+    line = {
+        "metric": METRIC,
+        "value": round(out.get("value", 0.0), 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(out.get("ms_per_step", 0.0), 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "configs[1]: fp32 row softmax over axis -1 of an [8192, 4096] tensor, N(0,1)*8; one step = one launch, 268435456 algorithmic bytes",
+                   "device": info["arch"], "compute_units": info["compute_units"]},
+    }
+    if "roofline" in out:
+        line["roofline"] = out["roofline"]
+    if "cpu_baseline" in out:
+        line["cpu_baseline"] = out["cpu_baseline"]
+    line["kernels"] = kernels
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
