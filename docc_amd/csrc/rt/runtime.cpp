@@ -43,6 +43,10 @@ struct DeviceState {
 std::mutex g_mutex;
 std::vector<DeviceState> g_devices;
 
+std::mutex g_failure_mutex;
+int g_failure_code = 0;
+std::string g_failure_message;
+
 std::string kernel_image_dir() {
     const char* env = std::getenv("DOCC_ROCM_KERNEL_PATH");
     std::string dir;
@@ -304,6 +308,33 @@ int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, 
     int rc = check(hipEventSynchronize((hipEvent_t) stop), "hipEventSynchronize");
     if (rc) return rc;
     return check(hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop), "hipEventElapsedTime");
+}
+
+void docc_rocm_report_failure(const char* function, const char* call, int code) {
+    char buf[1024];
+    std::snprintf(buf, sizeof(buf), "%s: %s failed with code %d: %s", function ? function : "?", call ? call : "?", code,
+                  g_last_error.c_str());
+    if (std::getenv("DOCC_ROCM_DEBUG")) {
+        std::fprintf(stderr, "docc rocm: %s\n", buf);
+        std::exit(EXIT_FAILURE);
+    }
+    std::lock_guard<std::mutex> lock(g_failure_mutex);
+    if (g_failure_code == 0) {  // keep the first failure: later ones are usually consequences
+        g_failure_code = code;
+        g_failure_message = buf;
+    }
+}
+
+int docc_rocm_take_failure(char* message, size_t message_len) {
+    std::lock_guard<std::mutex> lock(g_failure_mutex);
+    const int code = g_failure_code;
+    if (message && message_len) {
+        std::strncpy(message, g_failure_message.c_str(), message_len - 1);
+        message[message_len - 1] = 0;
+    }
+    g_failure_code = 0;
+    g_failure_message.clear();
+    return code;
 }
 
 const char* docc_rocm_last_error(void) { return g_last_error.c_str(); }

@@ -1,0 +1,246 @@
+#include "codegen.h"
+
+#include <algorithm>
+#include <fstream>
+
+namespace sdfg::codegen {
+
+void PrettyPrinter::write(const std::string& s) {
+    for (char c : s) {
+        if (c == '\n') {
+            out_ << '\n';
+            at_line_start_ = true;
+            continue;
+        }
+        if (at_line_start_) {
+            out_ << std::string((size_t) indent_, ' ');
+            at_line_start_ = false;
+        }
+        out_ << c;
+    }
+}
+
+std::string CPPLanguageExtension::primitive_type(types::PrimitiveType t) const {
+    using P = types::PrimitiveType;
+    switch (t) {
+        case P::Void: return "void";
+        case P::Bool: return "bool";
+        case P::Int8: return "int8_t";
+        case P::Int16: return "int16_t";
+        case P::Int32: return "int32_t";
+        case P::Int64: return "int64_t";
+        case P::UInt8: return "uint8_t";
+        case P::UInt16: return "uint16_t";
+        case P::UInt32: return "uint32_t";
+        case P::UInt64: return "uint64_t";
+        case P::Half: return "_Float16";
+        case P::BFloat: return "__bf16";
+        case P::Float: return "float";
+        case P::Double: return "double";
+    }
+    return "void";
+}
+
+std::string CPPLanguageExtension::declaration(const std::string& name, const Container& c) const {
+    std::string s = primitive_type(c.element);
+    s += c.is_pointer ? " *" : " ";
+    return s + name;
+}
+
+CodeSnippet& CodeSnippetFactory::require(const std::string& name, const std::string& extension, bool as_file) {
+    auto it = snippets_.find(name);
+    if (it != snippets_.end()) {
+        if (it->second.extension() != extension)
+            throw std::runtime_error("Code snippet " + name + " already exists with extension " + it->second.extension());
+        return it->second;
+    }
+    return snippets_.emplace(name, CodeSnippet(extension, as_file)).first->second;
+}
+
+void LibraryNodeDispatcher::dispatch(PrettyPrinter& stream, PrettyPrinter& globals_stream,
+                                     CodeSnippetFactory& library_snippet_factory) {
+    stream << "{" << std::endl;
+    stream.setIndent(stream.indent() + 4);
+
+    // one local per input connector: container value or constant literal
+    for (auto& in : data_flow_graph_.inputs) {
+        if (in.is_constant) {
+            stream << language_extension_.primitive_type(in.type) << " " << in.connector << " = " << in.data << ";" << std::endl;
+        } else {
+            const Container& c = function_.container(in.data);
+            stream << language_extension_.declaration(in.connector, c) << " = " << in.data << ";" << std::endl;
+        }
+    }
+    // outputs that are not inputs as well get a local too
+    for (auto& out : data_flow_graph_.outputs) {
+        if (data_flow_graph_.input(out.connector)) continue;
+        const Container& c = function_.container(out.data);
+        stream << language_extension_.declaration(out.connector, c) << " = " << out.data << ";" << std::endl;
+    }
+    stream << std::endl;
+
+    this->dispatch_code(stream, globals_stream, library_snippet_factory);
+
+    stream << std::endl;
+    for (auto& out : data_flow_graph_.outputs) stream << out.data << " = " << out.connector << ";" << std::endl;
+
+    stream.setIndent(stream.indent() - 4);
+    stream << "}" << std::endl;
+}
+
+InstrumentationInfo LibraryNodeDispatcher::instrumentation_info() const {
+    InstrumentationInfo info;
+    info.region_name = node_.code();
+    info.target_type = "CPU";
+    const Expression flop = node_.flop();
+    if (!flop.empty()) info.metrics["flop"] = flop;
+    return info;
+}
+
+LibraryNodeDispatcherRegistry& LibraryNodeDispatcherRegistry::instance() {
+    static LibraryNodeDispatcherRegistry registry;
+    return registry;
+}
+
+void LibraryNodeDispatcherRegistry::register_library_node_dispatcher(const std::string& key, LibraryNodeDispatcherFn fn) {
+    std::lock_guard<std::mutex> lock(mutex_);
+    factories_.emplace(key, std::move(fn));
+}
+
+LibraryNodeDispatcherFn LibraryNodeDispatcherRegistry::get_library_node_dispatcher(const std::string& key) const {
+    auto it = factories_.find(key);
+    return it == factories_.end() ? nullptr : it->second;
+}
+
+std::vector<std::string> LibraryNodeDispatcherRegistry::keys() const {
+    std::lock_guard<std::mutex> lock(mutex_);
+    std::vector<std::string> out;
+    for (auto& kv : factories_) out.push_back(kv.first);
+    std::sort(out.begin(), out.end());
+    return out;
+}
+
+CPPCodeGenerator::CPPCodeGenerator(StructuredSDFG& sdfg, std::shared_ptr<CodeSnippetFactory> library_snippet_factory,
+                                   std::string externals_prefix)
+    : sdfg_(sdfg), library_snippet_factory_(library_snippet_factory ? std::move(library_snippet_factory)
+                                                                     : std::make_shared<CodeSnippetFactory>()),
+      externals_prefix_(std::move(externals_prefix)) {}
+
+std::string CPPCodeGenerator::function_definition() {
+    std::vector<std::string> args;
+    for (auto& name : sdfg_.arguments()) args.push_back(language_extension_.declaration(name, sdfg_.container(name)));
+    std::string arglist;
+    for (size_t i = 0; i < args.size(); i++) arglist += (i ? ", " : "") + args[i];
+    if (arglist.empty()) arglist = "void";
+    std::string ret = "void ";
+    if (!sdfg_.return_container().empty()) ret = language_extension_.declaration("", sdfg_.container(sdfg_.return_container()));
+    return "extern \"C\" " + ret + externals_prefix_ + sdfg_.name() + "(" + arglist + ")";
+}
+
+void CPPCodeGenerator::dispatch_includes() {
+    includes_stream_ << "#include <cmath>" << std::endl;
+    includes_stream_ << "#include <cstdio>" << std::endl;
+    includes_stream_ << "#include <cstdlib>" << std::endl;
+    includes_stream_ << "#include <cstring>" << std::endl;
+    includes_stream_ << "#include <cstdint>" << std::endl;
+}
+
+void CPPCodeGenerator::dispatch_schedule() {
+    main_stream_.setIndent(4);
+    // transients are declared at the top of the function (reference cpp_code_generator.cpp:156-224)
+    for (auto& kv : sdfg_.containers()) {
+        const Container& c = kv.second;
+        if (c.is_argument) continue;
+        main_stream_ << language_extension_.declaration(c.name, c);
+        if (c.is_pointer) main_stream_ << " = nullptr";
+        main_stream_ << ";" << std::endl;
+    }
+    // host transients are managed allocations of the function
+    for (auto& kv : sdfg_.containers()) {
+        const Container& c = kv.second;
+        if (c.is_argument || !c.transient || !c.is_pointer || c.storage != "CPU" || c.size_bytes.empty()) continue;
+        main_stream_ << c.name << " = (" << language_extension_.primitive_type(c.element) << " *) malloc(" << c.size_bytes
+                     << ");" << std::endl;
+    }
+    auto& registry = LibraryNodeDispatcherRegistry::instance();
+    for (auto& blk : sdfg_.blocks()) {
+        const std::string key = blk.node->code() + "::" + blk.node->implementation_type();
+        auto factory = registry.get_library_node_dispatcher(key);
+        if (!factory) throw std::runtime_error("No library node dispatcher found for library node code: " + key);
+        auto dispatcher = factory(language_extension_, sdfg_, blk, *blk.node);
+        dispatcher->dispatch(main_stream_, globals_stream_, *library_snippet_factory_);
+        instrumentation_.push_back(dispatcher->instrumentation_info());
+    }
+    for (auto& kv : sdfg_.containers()) {
+        const Container& c = kv.second;
+        if (c.is_argument || !c.transient || !c.is_pointer || c.storage != "CPU" || c.size_bytes.empty()) continue;
+        if (c.name == sdfg_.return_container()) continue;  // ownership passes to the caller
+        main_stream_ << "free(" << c.name << ");" << std::endl;
+    }
+    if (!sdfg_.return_container().empty()) main_stream_ << "return " << sdfg_.return_container() << ";" << std::endl;
+}
+
+bool CPPCodeGenerator::generate() {
+    dispatch_includes();
+    dispatch_schedule();
+    return true;
+}
+
+std::string CPPCodeGenerator::header_text() const {
+    return "#pragma once\n" + includes_stream_.str() + "\n" + classes_stream_.str() + "\n";
+}
+
+std::string CPPCodeGenerator::source_text(const std::string& header_name) {
+    std::ostringstream src;
+    src << "#include \"" << header_name << "\"\n";
+    // the same include may be requested by several dispatchers: keep the first of each line
+    {
+        std::istringstream lines(globals_stream_.str());
+        std::vector<std::string> seen;
+        std::string line;
+        while (std::getline(lines, line)) {
+            if (line.rfind("#include", 0) == 0) {
+                if (std::find(seen.begin(), seen.end(), line) != seen.end()) continue;
+                seen.push_back(line);
+            }
+            src << line << "\n";
+        }
+    }
+    src << "\n" << function_definition() << "\n{\n";
+    auto init_once = library_snippet_factory_->find(CODE_SNIPPET_INIT_ONCE);
+    if (init_once != library_snippet_factory_->snippets().end()) src << init_once->second.stream().str() << "\n";
+    src << main_stream_.str() << "\n";
+    auto deinit_once = library_snippet_factory_->find(CODE_SNIPPET_DEINIT_ONCE);
+    if (deinit_once != library_snippet_factory_->snippets().end()) src << deinit_once->second.stream().str() << "\n";
+    src << "}\n";
+    return src.str();
+}
+
+bool CPPCodeGenerator::as_source(const std::filesystem::path& header_path, const std::filesystem::path& source_path) {
+    std::ofstream header(header_path, std::ofstream::out | std::ofstream::trunc);
+    if (!header.is_open()) return false;
+    std::ofstream source(source_path, std::ofstream::out | std::ofstream::trunc);
+    if (!source.is_open()) return false;
+    header << header_text();
+    source << source_text(header_path.filename().string());
+    return true;
+}
+
+} // namespace sdfg::codegen
+
+namespace sdfg::passes {
+
+bool TargetMappingPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager) {
+    bool applied = false;
+    for (auto& blk : builder.subject().blocks()) {
+        for (const auto& mapper : target_mappers_) {
+            if (mapper->try_map(builder, analysis_manager, *blk.node)) {
+                applied = true;
+                break;  // the first mapper that accepts the node wins
+            }
+        }
+    }
+    return applied;
+}
+
+} // namespace sdfg::passes

@@ -1,0 +1,626 @@
+#include "rocm_target.h"
+
+#include <algorithm>
+#include <set>
+
+namespace sdfg::rocm {
+
+using codegen::CodeSnippetFactory;
+using codegen::InstrumentationInfo;
+using codegen::LanguageExtension;
+using codegen::LibraryNodeDispatcher;
+using codegen::PrettyPrinter;
+using data_flow::ConnectorBinding;
+using data_flow::LibraryNode;
+using structured_control_flow::Block;
+namespace blas = math::blas;
+namespace tensor = math::tensor;
+
+namespace {
+
+bool is_rocm_impl(const std::string& impl) {
+    return impl == ImplementationType_ROCMWithTransfers || impl == ImplementationType_ROCMWithoutTransfers;
+}
+
+bool is_math_node(const LibraryNode& node) {
+    const std::string& c = node.code();
+    return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
+           c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention;
+}
+
+// Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
+void emit_runtime_preamble(PrettyPrinter& globals, const Function& function) {
+    if (globals.str().find("#define DOCC_ROCM_CHECK") != std::string::npos) return;  // once per file
+    globals << "#include \"docc_rocm_rt.h\"" << std::endl;
+    globals << "#include \"docc_rocm_ops.h\"" << std::endl;
+    globals << "#ifndef DOCC_ROCM_CHECK" << std::endl;
+    globals << "#define DOCC_ROCM_ON_FAILURE " << (function.return_container().empty() ? "return" : "return nullptr") << std::endl;
+    globals << "#define DOCC_ROCM_CHECK(call) do { int __docc_rc = (call); if (__docc_rc != 0) { "
+               "docc_rocm_report_failure(__func__, #call, __docc_rc); DOCC_ROCM_ON_FAILURE; } } while (0)"
+            << std::endl;
+    globals << "#endif" << std::endl;
+}
+
+// ---- with-transfers scaffolding ---------------------------------------------------------
+
+struct DeviceOperand {
+    std::string connector;  // host-side local, e.g. "__A"
+    std::string device;     // device-side local, e.g. "d___A"
+    Expression bytes;
+    bool copy_in;
+    bool copy_out;
+};
+
+void emit_transfers_begin(PrettyPrinter& s, const std::vector<DeviceOperand>& ops) {
+    for (auto& op : ops) {
+        s << "void *" << op.device << " = nullptr;" << std::endl;
+        s << "const size_t " << op.device << "_bytes = (size_t) (" << op.bytes << ");" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_malloc(&" << op.device << ", " << op.device << "_bytes));" << std::endl;
+    }
+    for (auto& op : ops)
+        if (op.copy_in)
+            s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_h2d_async(" << op.device << ", " << op.connector << ", " << op.device
+              << "_bytes, nullptr));" << std::endl;
+}
+
+void emit_transfers_end(PrettyPrinter& s, const std::vector<DeviceOperand>& ops) {
+    for (auto& op : ops)
+        if (op.copy_out)
+            s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_d2h_async(" << op.connector << ", " << op.device << ", " << op.device
+              << "_bytes, nullptr));" << std::endl;
+    s << "DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
+    for (auto& op : ops) s << "DOCC_ROCM_CHECK(docc_rocm_free(" << op.device << "));" << std::endl;
+}
+
+Expression sum_bytes(const std::vector<DeviceOperand>& ops) {
+    Expression e;
+    for (auto& op : ops) {
+        if (op.copy_in) e += (e.empty() ? "" : " + ") + ("(" + op.bytes + ")");
+        if (op.copy_out) e += (e.empty() ? "" : " + ") + ("(" + op.bytes + ")");
+    }
+    return e.empty() ? "0" : e;
+}
+
+// Base for the math-node dispatchers: prints the launcher call on `args` (device pointers),
+// with or without the surrounding transfers.
+class RocmMathDispatcher : public LibraryNodeDispatcher {
+public:
+    RocmMathDispatcher(LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n, bool with_transfers)
+        : LibraryNodeDispatcher(le, f, b, n), with_transfers_(with_transfers) {}
+
+    void dispatch_code(PrettyPrinter& stream, PrettyPrinter& globals, CodeSnippetFactory&) override {
+        emit_runtime_preamble(globals, function_);
+        const std::string guard = guard_condition();
+        if (!guard.empty()) {
+            stream << "if (" << guard << ") {" << std::endl;
+            stream.setIndent(stream.indent() + 4);
+        }
+        std::vector<DeviceOperand> ops;
+        if (with_transfers_) {
+            ops = operands();
+            emit_transfers_begin(stream, ops);
+        }
+        auto name_of = [&](const std::string& connector) -> std::string {
+            if (!with_transfers_) return connector;
+            for (auto& op : ops)
+                if (op.connector == connector) return op.device;
+            return connector;
+        };
+        emit_launch(stream, name_of);
+        if (with_transfers_) emit_transfers_end(stream, ops);
+        if (!guard.empty()) {
+            stream.setIndent(stream.indent() - 4);
+            stream << "}" << std::endl;
+        }
+    }
+
+    InstrumentationInfo instrumentation_info() const override {
+        InstrumentationInfo info = LibraryNodeDispatcher::instrumentation_info();
+        info.target_type = "ROCM";
+        if (with_transfers_) info.metrics["pcie_bytes"] = sum_bytes(operands());
+        return info;
+    }
+
+protected:
+    virtual std::vector<DeviceOperand> operands() const = 0;
+    virtual void emit_launch(PrettyPrinter& stream, const std::function<std::string(const std::string&)>& name_of) = 0;
+    virtual std::string guard_condition() const { return ""; }
+
+    DeviceOperand operand(const std::string& connector, bool in, bool out) const {
+        return DeviceOperand{connector, "d_" + connector, node_.connector_bytes(connector), in, out};
+    }
+
+    bool with_transfers_;
+};
+
+// ---- GEMM ---------------------------------------------------------------------------------
+
+class GEMMNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    const blas::GEMMNode& gemm() const { return static_cast<const blas::GEMMNode&>(node_); }
+
+    std::vector<DeviceOperand> operands() const override {
+        // C travels to the device only when the node reads it (beta != 0)
+        const bool read_c = node_.reads("__C", data_flow_graph_.inputs);
+        return {operand("__A", true, false), operand("__B", true, false), operand("__C", read_c, true)};
+    }
+
+    std::string guard_condition() const override {
+        // same guard as the cuBLAS dispatcher (reference opt/src/targets/cuda/blas/gemm.cpp:17-26)
+        return "(" + gemm().m() + ") != 0 && (" + gemm().n() + ") != 0";
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& g = gemm();
+        std::string fn, in_t, out_t;
+        switch (g.precision()) {
+            case blas::d: fn = "docc_rocm_dgemm"; in_t = out_t = "double"; break;
+            case blas::s: fn = "docc_rocm_sgemm"; in_t = out_t = "float"; break;
+            case blas::b: fn = "docc_rocm_bf16gemm_f32"; in_t = "uint16_t"; out_t = "float"; break;
+            default: throw std::runtime_error("Invalid precision for ROCM GEMM node");
+        }
+        s << "DOCC_ROCM_CHECK(" << fn << "(nullptr, " << (int) g.trans_a() << ", " << (int) g.trans_b() << ", "
+          << language_extension_.expression(g.m()) << ", " << language_extension_.expression(g.n()) << ", "
+          << language_extension_.expression(g.k()) << ", __alpha, (const " << in_t << " *) " << name_of("__A") << ", "
+          << language_extension_.expression(g.lda()) << ", (const " << in_t << " *) " << name_of("__B") << ", "
+          << language_extension_.expression(g.ldb()) << ", __beta, (" << out_t << " *) " << name_of("__C") << ", "
+          << language_extension_.expression(g.ldc()) << "));" << std::endl;
+    }
+};
+
+// ---- MatMul (batched) -----------------------------------------------------------------------
+
+class MatMulNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    const tensor::MatMulNode& mm() const { return static_cast<const tensor::MatMulNode&>(node_); }
+
+    std::vector<DeviceOperand> operands() const override {
+        return {operand("A", true, false), operand("B", true, false), operand("Y", false, true)};
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        // one GEMM (alpha 1, beta 0) per batch entry, the shape of the reference's expansion
+        // (matmul_node.cpp:366-499)
+        const auto& n = mm();
+        std::string fn, in_t, out_t, one, zero;
+        switch (n.element()) {
+            case types::PrimitiveType::Double: fn = "docc_rocm_dgemm"; in_t = out_t = "double"; one = "1.0"; zero = "0.0"; break;
+            case types::PrimitiveType::Float: fn = "docc_rocm_sgemm"; in_t = out_t = "float"; one = "1.0f"; zero = "0.0f"; break;
+            case types::PrimitiveType::BFloat: fn = "docc_rocm_bf16gemm_f32"; in_t = "uint16_t"; out_t = "float"; one = "1.0f"; zero = "0.0f"; break;
+            default: throw std::runtime_error("Invalid element type for ROCM MatMul node");
+        }
+        s << "for (int64_t __b = 0; __b < (int64_t) (" << n.batch() << "); __b++) {" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "const " << in_t << " *__a_b = (const " << in_t << " *) " << name_of("A") << " + __b * (int64_t) ("
+          << symbolic::mul(n.m(), n.k()) << ");" << std::endl;
+        s << "const " << in_t << " *__b_b = (const " << in_t << " *) " << name_of("B");
+        if (n.b_is_batched()) s << " + __b * (int64_t) (" << symbolic::mul(n.k(), n.n()) << ")";
+        s << ";" << std::endl;
+        s << out_t << " *__y_b = (" << out_t << " *) " << name_of("Y") << " + __b * (int64_t) (" << symbolic::mul(n.m(), n.n())
+          << ");" << std::endl;
+        s << "DOCC_ROCM_CHECK(" << fn << "(nullptr, 111, 111, " << n.m() << ", " << n.n() << ", " << n.k() << ", " << one
+          << ", __a_b, " << n.k() << ", __b_b, " << n.n() << ", " << zero << ", __y_b, " << n.n() << "));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+};
+
+// ---- Softmax ------------------------------------------------------------------------------
+
+class SoftmaxNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::SoftmaxNode&>(node_);
+        s << "DOCC_ROCM_CHECK(docc_rocm_softmax_f32(nullptr, " << n.rows() << ", " << n.cols() << ", (const float *) "
+          << name_of("X") << ", (float *) " << name_of("Y") << "));" << std::endl;
+    }
+};
+
+// ---- Conv ---------------------------------------------------------------------------------
+
+class ConvNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    const tensor::ConvNode& conv() const { return static_cast<const tensor::ConvNode&>(node_); }
+
+    std::vector<DeviceOperand> operands() const override {
+        std::vector<DeviceOperand> ops{operand("X", true, false), operand("W", true, false)};
+        if (conv().has_bias()) ops.push_back(operand("B", true, false));
+        ops.push_back(operand("Y", false, true));
+        return ops;
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& c = conv();
+        auto get = [](const std::vector<Expression>& v, size_t i, const char* dflt) { return v.empty() ? Expression(dflt) : v[i]; };
+        s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32(nullptr, " << c.shape()[0] << ", " << c.shape()[1] << ", " << c.shape()[2]
+          << ", " << c.shape()[3] << ", " << c.output_channels() << ", " << c.kernel_shape()[0] << ", " << c.kernel_shape()[1]
+          << ", " << get(c.strides(), 0, "1") << ", " << get(c.strides(), 1, "1") << ", " << get(c.pads(), 0, "0") << ", "
+          << get(c.pads(), 1, "0") << ", " << get(c.dilations(), 0, "1") << ", " << get(c.dilations(), 1, "1")
+          << ", (const float *) " << name_of("X") << ", (const float *) " << name_of("W") << ", "
+          << (c.has_bias() ? "(const float *) " + name_of("B") : std::string("nullptr")) << ", (float *) " << name_of("Y")
+          << "));" << std::endl;
+    }
+};
+
+// ---- Attention ----------------------------------------------------------------------------
+
+class AttentionNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override {
+        return {operand("Q", true, false), operand("K", true, false), operand("V", true, false), operand("O", false, true)};
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& a = static_cast<const tensor::AttentionNode&>(node_);
+        const auto& q = a.shape_q();
+        s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16(nullptr, " << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv()
+          << ", " << q[3] << ", (float) (" << a.scale() << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) "
+          << name_of("K") << ", (const uint16_t *) " << name_of("V") << ", (void *) " << name_of("O") << ", "
+          << (a.output_element() == types::PrimitiveType::BFloat ? 1 : 0) << "));" << std::endl;
+    }
+};
+
+// ---- offloading node ------------------------------------------------------------------------
+
+class ROCMDataOffloadingNodeDispatcher : public LibraryNodeDispatcher {
+public:
+    using LibraryNodeDispatcher::LibraryNodeDispatcher;
+
+    void dispatch_code(PrettyPrinter& s, PrettyPrinter& globals, CodeSnippetFactory&) override {
+        emit_runtime_preamble(globals, function_);
+        const auto& n = static_cast<const ROCMDataOffloadingNode&>(node_);
+        const std::string size = language_extension_.expression(n.size());
+        // order as in the CUDA offloading dispatcher (reference cuda_data_offloading_node.cpp:139-173):
+        // allocate, copy, free; copies are followed by a stream wait because the node is blocking
+        if (n.is_alloc()) {
+            const std::string dst = n.is_h2d() ? "_dst" : "_ret";
+            s << "DOCC_ROCM_CHECK(docc_rocm_malloc((void **) &" << dst << ", (size_t) (" << size << ")));" << std::endl;
+        }
+        if (n.is_h2d()) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_h2d_async(_dst, _src, (size_t) (" << size << "), nullptr));" << std::endl;
+        } else if (n.is_d2h()) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_d2h_async(_dst, _src, (size_t) (" << size << "), nullptr));" << std::endl;
+            s << "DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
+        }
+        if (n.is_free()) {
+            const std::string ptr = n.is_d2h() ? "_src" : "_ptr";
+            s << "DOCC_ROCM_CHECK(docc_rocm_free(" << ptr << "));" << std::endl;
+        }
+    }
+
+    InstrumentationInfo instrumentation_info() const override {
+        const auto& n = static_cast<const ROCMDataOffloadingNode&>(node_);
+        InstrumentationInfo info;
+        info.region_name = n.toStr();
+        info.target_type = n.is_h2d() ? "H2D" : n.is_d2h() ? "D2H" : "ROCM";
+        if (n.is_h2d() || n.is_d2h()) info.metrics["pcie_bytes"] = n.size();
+        return info;
+    }
+};
+
+template <typename D>
+void register_math(codegen::LibraryNodeDispatcherRegistry& reg, const std::string& code) {
+    for (bool with : {true, false}) {
+        reg.register_library_node_dispatcher(
+            code + "::" + (with ? ImplementationType_ROCMWithTransfers : ImplementationType_ROCMWithoutTransfers),
+            [with](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
+                return std::make_unique<D>(le, f, b, n, with);
+            });
+    }
+}
+
+std::unique_ptr<LibraryNode> deserialize_attention(const json::Value& j) { return tensor::AttentionNode::from_json(j); }
+std::unique_ptr<LibraryNode> deserialize_offloading(const json::Value& j) { return ROCMDataOffloadingNode::from_json(j); }
+
+} // namespace
+
+void register_plugin(plugins::Context& context) {
+    auto& ser = context.library_node_serializer_registry;
+    ser.register_library_node_serializer(tensor::LibraryNodeType_Attention, &deserialize_attention);
+    ser.register_library_node_serializer(LibraryNodeType_ROCM_Offloading, &deserialize_offloading);
+
+    auto& reg = context.library_node_dispatcher_registry;
+    register_math<GEMMNodeDispatcher_ROCM>(reg, blas::LibraryNodeType_GEMM);
+    register_math<MatMulNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_MatMul);
+    register_math<SoftmaxNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Softmax);
+    register_math<ConvNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Conv);
+    register_math<AttentionNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Attention);
+    reg.register_library_node_dispatcher(
+        LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
+        [](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
+            return std::make_unique<ROCMDataOffloadingNodeDispatcher>(le, f, b, n);
+        });
+}
+
+void register_rocm_plugin() {
+    auto context = plugins::Context::global_context();
+    register_plugin(context);
+}
+
+const plugins::Plugin rocm_plugin = {"rocm", "0.1", "MI355X (gfx950) target for the math library nodes", &register_plugin};
+
+// ---------------------------------------------------------------------------------- mapper
+
+bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::AnalysisManager&, LibraryNode& node) const {
+    reason_.clear();
+    auto decline = [&](const std::string& why) {
+        reason_ = node.code() + ": " + why;
+        return false;
+    };
+    using P = types::PrimitiveType;
+    if (node.code() == blas::LibraryNodeType_GEMM) {
+        auto* g = dynamic_cast<blas::GEMMNode*>(&node);
+        if (!g) return decline("not a GEMM node object");
+        if (g->layout() != blas::RowMajor) return decline("only row-major layout is supported");
+        if (g->trans_a() == blas::ConjTrans || g->trans_b() == blas::ConjTrans) return decline("conjugate transpose is not supported");
+        if (g->precision() != blas::s && g->precision() != blas::d && g->precision() != blas::b)
+            return decline("precision must be s, d or b (bf16 with fp32 accumulate)");
+    } else if (node.code() == tensor::LibraryNodeType_MatMul) {
+        auto* m = dynamic_cast<tensor::MatMulNode*>(&node);
+        if (!m) return decline("not a MatMul node object");
+        if (m->element() != P::Float && m->element() != P::Double && m->element() != P::BFloat)
+            return decline("element type must be Float, Double or BFloat");
+    } else if (node.code() == tensor::LibraryNodeType_Softmax) {
+        auto* s = dynamic_cast<tensor::SoftmaxNode*>(&node);
+        if (!s) return decline("not a Softmax node object");
+        if (s->element() != P::Float) return decline("only Float is supported");
+        if (!s->last_axis_only()) return decline("only a reduction over the last axis is supported");
+    } else if (node.code() == tensor::LibraryNodeType_Conv) {
+        auto* c = dynamic_cast<tensor::ConvNode*>(&node);
+        if (!c) return decline("not a Conv node object");
+        if (c->element() != P::Float) return decline("only Float is supported");
+        if (c->kernel_shape().size() != 2) return decline("only 2-d convolution is supported");
+        int64_t group = 0;
+        if (!symbolic::is_integer(c->group(), &group) || group != 1) return decline("only group == 1 is supported");
+        if (!c->pads().empty() && (c->pads()[0] != c->pads()[2] || c->pads()[1] != c->pads()[3]))
+            return decline("padding must be symmetric (begin == end)");
+    } else if (node.code() == tensor::LibraryNodeType_Attention) {
+        auto* a = dynamic_cast<tensor::AttentionNode*>(&node);
+        if (!a) return decline("not an Attention node object");
+        if (a->element() != P::BFloat) return decline("inputs must be BFloat");
+        if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
+        int64_t d = 0;
+        if (!symbolic::is_integer(a->shape_q()[3], &d) || d != 64) return decline("head dimension must be 64");
+    } else {
+        return false;  // not a node of this target
+    }
+    node.implementation_type() = implementation_type_;
+    return true;
+}
+
+// ------------------------------------------------------------------------------ offloading
+
+namespace {
+
+ConnectorBinding make_binding(const std::string& connector, const std::string& data) {
+    ConnectorBinding b;
+    b.connector = connector;
+    b.data = data;
+    return b;
+}
+
+bool is_offloading(const Block& b) { return b.node->code() == LibraryNodeType_ROCM_Offloading; }
+
+const ROCMDataOffloadingNode& offloading(const Block& b) { return static_cast<const ROCMDataOffloadingNode&>(*b.node); }
+
+} // namespace
+
+bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
+    StructuredSDFG& sdfg = builder.subject();
+    bool applied = false;
+    // indices move while blocks are inserted: walk by position
+    for (size_t i = 0; i < sdfg.blocks().size(); i++) {
+        if (sdfg.blocks()[i].node->implementation_type() != ImplementationType_ROCMWithoutTransfers) continue;
+        if (is_offloading(sdfg.blocks()[i])) continue;
+        // already surrounded? (a device container is bound)
+        bool on_host = false;
+        for (auto& in : sdfg.blocks()[i].inputs)
+            if (!in.is_constant && sdfg.container(in.data).storage == "CPU" && sdfg.container(in.data).is_pointer) on_host = true;
+        for (auto& out : sdfg.blocks()[i].outputs)
+            if (sdfg.container(out.data).storage == "CPU") on_host = true;
+        if (!on_host) continue;
+
+        struct Plan {
+            std::string host, device;
+            Expression bytes;
+            bool read = false, written = false;
+        };
+        std::vector<Plan> plans;
+        auto plan_for = [&](const std::string& host) -> Plan& {
+            for (auto& p : plans)
+                if (p.host == host) return p;
+            plans.push_back(Plan{host, "__daisy_rocm_" + std::to_string(sdfg.blocks()[i].node->element_id()) + "_" + host, "", false, false});
+            return plans.back();
+        };
+        {
+            const Block& blk = sdfg.blocks()[i];
+            for (auto& in : blk.inputs) {
+                if (in.is_constant || !sdfg.container(in.data).is_pointer) continue;
+                Plan& p = plan_for(in.data);
+                p.bytes = blk.node->connector_bytes(in.connector);
+                if (blk.node->reads(in.connector, blk.inputs)) p.read = true;
+            }
+            for (auto& out : blk.outputs) {
+                Plan& p = plan_for(out.data);
+                p.bytes = blk.node->connector_bytes(out.connector);
+                p.written = true;
+            }
+        }
+        for (auto& p : plans) {
+            Container dev;
+            dev.name = p.device;
+            dev.is_pointer = true;
+            dev.element = sdfg.container(p.host).element;
+            dev.transient = true;
+            dev.storage = "ROCM_Generic";
+            sdfg.add_container(dev, false);
+        }
+        // rebind the node to the device containers
+        for (auto& in : sdfg.blocks()[i].inputs)
+            for (auto& p : plans)
+                if (!in.is_constant && in.data == p.host) in.data = p.device;
+        for (auto& out : sdfg.blocks()[i].outputs)
+            for (auto& p : plans)
+                if (out.data == p.host) out.data = p.device;
+        // before: ALLOC (+H2D when the node reads the operand)
+        size_t pos = i;
+        for (auto& p : plans) {
+            if (p.read) {
+                sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::H2D, BufferLifecycle::ALLOC),
+                               {make_binding("_src", p.host)}, {make_binding("_dst", p.device)}, pos++);
+            } else {
+                sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::NONE, BufferLifecycle::ALLOC),
+                               {}, {make_binding("_ret", p.device)}, pos++);
+            }
+        }
+        // the node now sits at `pos`; after it: D2H+FREE for what it wrote, FREE for the rest
+        size_t after = pos + 1;
+        for (auto& p : plans) {
+            if (p.written) {
+                sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::D2H, BufferLifecycle::FREE),
+                               {make_binding("_src", p.device)}, {make_binding("_dst", p.host)}, after++);
+            }
+        }
+        for (auto& p : plans) {
+            if (!p.written) {
+                sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::NONE, BufferLifecycle::FREE),
+                               {make_binding("_ptr", p.device)}, {}, after++);
+            }
+        }
+        i = after - 1;
+        applied = true;
+    }
+    return applied;
+}
+
+bool RocmDataTransferMinimizationPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
+    StructuredSDFG& sdfg = builder.subject();
+    auto& blocks = sdfg.blocks();
+    bool applied = false;
+
+    auto uses_host = [&](const Block& b, const std::string& host) {
+        for (auto& in : b.inputs)
+            if (!in.is_constant && in.data == host) return true;
+        for (auto& out : b.outputs)
+            if (out.data == host) return true;
+        return false;
+    };
+    auto needed_on_host = [&](const std::string& host, size_t from) {
+        const Container& c = sdfg.container(host);
+        if (c.is_argument || host == sdfg.return_container()) return true;
+        for (size_t j = from; j < blocks.size(); j++)
+            if (!is_offloading(blocks[j]) && uses_host(blocks[j], host)) return true;
+        return false;
+    };
+
+    bool changed = true;
+    while (changed) {
+        changed = false;
+        for (size_t i = 0; i < blocks.size() && !changed; i++) {
+            if (!is_offloading(blocks[i])) continue;
+            const auto& first = offloading(blocks[i]);
+            if (first.transfer_direction() == DataTransferDirection::NONE && first.is_free()) {
+                // a read-only operand freed here and uploaded again later from the same, unchanged
+                // host container: keep the first device copy alive instead
+                const std::string dev1 = blocks[i].inputs[0].data;
+                std::string host;
+                for (size_t k = 0; k < i; k++)
+                    if (is_offloading(blocks[k]) && offloading(blocks[k]).is_h2d() && blocks[k].outputs[0].data == dev1)
+                        host = blocks[k].inputs[0].data;
+                if (host.empty()) continue;
+                size_t j = i + 1;
+                while (j < blocks.size() && !uses_host(blocks[j], host)) j++;
+                if (j >= blocks.size() || !is_offloading(blocks[j])) continue;
+                const auto& again = offloading(blocks[j]);
+                if (!again.is_h2d() || !again.is_alloc() || again.size() != first.size() || again.device_id() != first.device_id()) continue;
+                const std::string dev2 = blocks[j].outputs[0].data;
+                blocks.erase(blocks.begin() + (long) j);
+                blocks.erase(blocks.begin() + (long) i);
+                for (size_t k = i; k < blocks.size(); k++) {
+                    for (auto& in : blocks[k].inputs)
+                        if (!in.is_constant && in.data == dev2) in.data = dev1;
+                    for (auto& out : blocks[k].outputs)
+                        if (out.data == dev2) out.data = dev1;
+                }
+                changed = applied = true;
+                continue;
+            }
+            if (!first.is_d2h() || !first.is_free()) continue;
+            const std::string host = blocks[i].outputs[0].data, dev1 = blocks[i].inputs[0].data;
+            // next block that touches the host container
+            size_t j = i + 1;
+            while (j < blocks.size() && !uses_host(blocks[j], host)) j++;
+            if (j >= blocks.size() || !is_offloading(blocks[j])) continue;
+            const auto& second = offloading(blocks[j]);
+            if (!second.is_h2d() || !second.is_alloc() || !first.redundant_with(second)) continue;
+            const std::string dev2 = blocks[j].outputs[0].data;
+            // the upload disappears; every later use of its device buffer refers to the first buffer
+            blocks.erase(blocks.begin() + (long) j);
+            for (size_t k = j; k < blocks.size(); k++) {
+                for (auto& in : blocks[k].inputs)
+                    if (!in.is_constant && in.data == dev2) in.data = dev1;
+                for (auto& out : blocks[k].outputs)
+                    if (out.data == dev2) out.data = dev1;
+            }
+            // the download stays only if the host still looks at the data, and no longer frees
+            if (needed_on_host(host, i + 1)) {
+                auto keep = std::make_unique<ROCMDataOffloadingNode>(first.size(), first.device_id(), DataTransferDirection::D2H,
+                                                                     BufferLifecycle::NO_CHANGE);
+                keep->set_element_id(blocks[i].node->element_id());
+                blocks[i].node = std::move(keep);
+            } else {
+                blocks.erase(blocks.begin() + (long) i);
+                // a host transient nobody touches any more needs no host memory
+                Container& c = sdfg.container(host);
+                bool any = false;
+                for (auto& b : blocks)
+                    if (uses_host(b, host)) any = true;
+                if (!any && c.transient) c.size_bytes.clear();
+            }
+            changed = applied = true;
+        }
+    }
+    return applied;
+}
+
+void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager,
+                            const std::string& category, const ScheduleOptions& options) {
+    (void) category;  // "desktop" / "server": one code path, kept for the interface
+    register_rocm_plugin();
+    if (options.offload != "function" && options.offload != "node" && options.offload != "none")
+        throw std::invalid_argument("rocm: option offload must be 'function', 'node' or 'none'");
+    const std::string impl = options.offload == "node" ? ImplementationType_ROCMWithTransfers : ImplementationType_ROCMWithoutTransfers;
+    auto mapper = std::make_shared<RocmLibNodeMapper>(impl);
+    for (auto& blk : builder.subject().blocks()) {
+        if (!is_math_node(*blk.node) || is_rocm_impl(blk.node->implementation_type())) continue;
+        if (!mapper->try_map(builder, analysis_manager, *blk.node) && options.require_all_mapped)
+            throw InvalidSDFGException("rocm target cannot map node " + mapper->last_decline_reason() +
+                                       " (this target has no CPU lowering)");
+    }
+    if (options.offload == "function") {
+        RocmOffloadTransform offload;
+        offload.run_pass(builder, analysis_manager);
+        RocmDataTransferMinimizationPass minimize;
+        minimize.run_pass(builder, analysis_manager);
+    }
+    analysis_manager.invalidate_all();
+}
+
+} // namespace sdfg::rocm

@@ -1,0 +1,73 @@
+// The `rocm` target: plugin registration, the library-node mapper, the
+// offloading transform with transfer minimisation, and the dispatchers that
+// print host C++ against the thin HIP runtime (include/docc_rocm_rt.h) and the
+// kernel launchers (include/docc_rocm_ops.h).
+//
+// Structure follows the two device targets of the reference:
+//   ET-SoC  targets/et/src/et/target.cpp:21-47 (register_plugin, scheduling passes),
+//           targets/et/src/et/et_lib_node_mapper.cpp:10-25 (TargetMapper::try_map),
+//           targets/et/src/et/blas/gemm.cpp:132-205 (WithTransfers dispatcher);
+//   CUDA    opt/include/sdfg/targets/cuda/plugin.h:20-105 (register_cuda_plugin),
+//           opt/src/targets/cuda/blas/gemm.cpp:33-185 (With/WithoutTransfers dispatchers),
+//           opt/src/targets/cuda/cuda_data_offloading_node.cpp:139-173 (transfer node dispatcher),
+//           opt/src/transformations/offloading/offload_transform.cpp:86-140 and
+//           opt/src/passes/offloading/data_transfer_minimization_pass.cpp (transfer elimination).
+#pragma once
+
+#include "codegen.h"
+
+namespace sdfg::rocm {
+
+// Registers (idempotently) the rocm serializers and dispatchers in the global registries.
+void register_rocm_plugin();
+void register_plugin(plugins::Context& context);
+extern const plugins::Plugin rocm_plugin;
+
+// Maps GEMM / ml::MatMul / ml::Softmax / ml::Conv / ml::Attention nodes whose dtype and layout the
+// kernels support to `implementation_type` (ROCMWithTransfers or ROCMWithoutTransfers);
+// declines (returns false, node untouched) otherwise and records why.
+class RocmLibNodeMapper : public plugins::TargetMapper {
+public:
+    explicit RocmLibNodeMapper(std::string implementation_type = ImplementationType_ROCMWithTransfers)
+        : implementation_type_(std::move(implementation_type)) {}
+    bool try_map(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager,
+                 data_flow::LibraryNode& node) const override;
+    // why the last declined node was declined ("" if none)
+    const std::string& last_decline_reason() const { return reason_; }
+
+private:
+    std::string implementation_type_;
+    mutable std::string reason_;
+};
+
+// Surrounds every ROCMWithoutTransfers node with offloading blocks (ALLOC[+H2D] before,
+// [D2H+]FREE after) on device containers `__daisy_rocm_<element id>_<container>`.
+class RocmOffloadTransform {
+public:
+    std::string name() { return "RocmOffloadTransform"; }
+    bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
+};
+
+// Removes D2H(+FREE) / H2D(+ALLOC) pairs on the same host container between consecutive
+// device nodes so that intermediates stay in HBM; drops the D2H altogether when the host
+// never looks at the container, and the host allocation of such transients with it.
+class RocmDataTransferMinimizationPass {
+public:
+    std::string name() { return "RocmDataTransferMinimization"; }
+    bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
+};
+
+struct ScheduleOptions {
+    // "function": nodes run WithoutTransfers between hoisted, minimised transfers (default)
+    // "node":     every node copies its operands itself (ROCMWithTransfers)
+    // "none":     the caller passes device pointers; no transfers are generated
+    std::string offload = "function";
+    // refuse to leave a math node unmapped (there is no CPU lowering in this target)
+    bool require_all_mapped = true;
+};
+
+// The scheduling entry of the target: mapping pass (+ offloading passes).
+void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager,
+                            const std::string& category, const ScheduleOptions& options);
+
+} // namespace sdfg::rocm

@@ -1,0 +1,427 @@
+// A descriptor-level carrier for the parts of docc's SDFG that the rocm target
+// needs: typed containers, an ordered argument list, a root sequence of
+// blocks each holding one library node with its connector bindings, and the
+// math library nodes GEMM / ml::MatMul / ml::Softmax / ml::Conv (fields, connector names
+// and JSON keys as in the reference) plus the ml::Attention node and the
+// ROCMOffloading transfer node that the rocm target adds.
+//
+// The reference's own IR (sdfg/include/sdfg/structured_sdfg.h, data_flow/*.h)
+// is a general graph with symbolic expressions (SymEngine); here symbolic
+// expressions are kept as C-expression strings over the function's integer
+// arguments, which is what they are printed as in generated code anyway.
+#pragma once
+
+#include <cstdint>
+#include <map>
+#include <memory>
+#include <optional>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "json.h"
+
+namespace sdfg {
+
+class InvalidSDFGException : public std::runtime_error {
+public:
+    using std::runtime_error::runtime_error;
+};
+
+namespace types {
+
+// reference: sdfg/include/sdfg/types/type.h (PrimitiveType)
+enum class PrimitiveType { Void, Bool, Int8, Int16, Int32, Int64, UInt8, UInt16, UInt32, UInt64, Half, BFloat, Float, Double };
+
+const char* primitive_type_to_string(PrimitiveType t);
+PrimitiveType primitive_type_from_string(const std::string& s);
+size_t primitive_type_size(PrimitiveType t);
+bool is_floating_point(PrimitiveType t);
+
+} // namespace types
+
+using Expression = std::string;  // C expression over int64 symbols, e.g. "_s0*_s1"
+
+namespace symbolic {
+Expression mul(const Expression& a, const Expression& b);
+Expression integer(int64_t v);
+bool is_integer(const Expression& e, int64_t* value = nullptr);
+} // namespace symbolic
+
+// Implementation types, following the "<LIB>With[out]Transfers" naming of the
+// reference (opt/include/sdfg/targets/cuda/cuda.h:20-26, targets/et/include/docc/target/et/target.h:10-11)
+inline const std::string ImplementationType_NONE = "NONE";
+inline const std::string ImplementationType_BLAS = "BLAS";
+inline const std::string ImplementationType_ROCMWithTransfers = "ROCMWithTransfers";
+inline const std::string ImplementationType_ROCMWithoutTransfers = "ROCMWithoutTransfers";
+
+struct Container {
+    std::string name;
+    bool is_pointer = false;
+    types::PrimitiveType element = types::PrimitiveType::Void;
+    bool is_argument = false;
+    bool transient = false;      // allocated and freed by the generated function
+    Expression size_bytes;       // transients: byte size
+    std::string storage = "CPU"; // "CPU" | "ROCM_Generic" (device memory, cf. NV_Generic in cuda_transform.h:21-37)
+};
+
+namespace data_flow {
+
+struct ConnectorBinding {
+    std::string connector;
+    bool is_constant = false;    // ConstantNode: `data` is the literal, printed verbatim
+    std::string data;            // container name or literal
+    types::PrimitiveType type = types::PrimitiveType::Void;  // constants only
+};
+
+// reference: sdfg/include/sdfg/data_flow/library_node.h:98-179
+class LibraryNode {
+public:
+    LibraryNode(std::string code, std::vector<std::string> outputs, std::vector<std::string> inputs, bool side_effect,
+                std::string implementation_type)
+        : code_(std::move(code)), outputs_(std::move(outputs)), inputs_(std::move(inputs)), side_effect_(side_effect),
+          implementation_type_(std::move(implementation_type)) {}
+    virtual ~LibraryNode() = default;
+
+    const std::string& code() const { return code_; }
+    const std::string& implementation_type() const { return implementation_type_; }
+    std::string& implementation_type() { return implementation_type_; }
+    bool side_effect() const { return side_effect_; }
+    const std::vector<std::string>& inputs() const { return inputs_; }
+    const std::vector<std::string>& outputs() const { return outputs_; }
+    size_t element_id() const { return element_id_; }
+    void set_element_id(size_t id) { element_id_ = id; }
+
+    virtual std::string toStr() const { return code_; }
+    virtual void validate() const {}
+    // floating point operations, as an expression, or "" when unknown
+    virtual Expression flop() const { return ""; }
+    // node payload (everything except the envelope keys)
+    virtual void to_json(json::Value& j) const = 0;
+
+    // Offloading support: byte extent of the memory behind a connector, and
+    // whether the node reads what is behind an input connector (GEMM does not
+    // read __C when beta is the constant 0).
+    virtual Expression connector_bytes(const std::string& connector) const = 0;
+    virtual bool reads(const std::string& connector, const std::vector<ConnectorBinding>& inputs) const { return true; }
+
+protected:
+    std::string code_;
+    std::vector<std::string> outputs_;
+    std::vector<std::string> inputs_;
+    bool side_effect_;
+    std::string implementation_type_;
+    size_t element_id_ = 0;
+};
+
+} // namespace data_flow
+
+namespace math::blas {
+
+// reference: sdfg/include/sdfg/data_flow/library_nodes/math/blas/blas_node.h:49-126
+enum BLAS_Precision : int { h = 'h', s = 's', d = 'd', c = 'c', z = 'z', b = 'b' /* bf16 in, fp32 accumulate/out: added by the rocm target */ };
+enum BLAS_Layout : int { RowMajor = 101, ColMajor = 102 };
+enum BLAS_Transpose : int { No = 111, Trans = 112, ConjTrans = 113 };
+
+types::PrimitiveType precision_input_type(BLAS_Precision p);
+types::PrimitiveType precision_output_type(BLAS_Precision p);
+
+inline const std::string LibraryNodeType_GEMM = "GEMM";
+
+// reference: sdfg/include/sdfg/data_flow/library_nodes/math/blas/gemm_node.h:14-112
+class GEMMNode : public data_flow::LibraryNode {
+public:
+    GEMMNode(std::string implementation_type, BLAS_Precision precision, BLAS_Layout layout, BLAS_Transpose trans_a,
+             BLAS_Transpose trans_b, Expression m, Expression n, Expression k, Expression lda, Expression ldb,
+             Expression ldc);
+
+    BLAS_Precision precision() const { return precision_; }
+    BLAS_Layout layout() const { return layout_; }
+    BLAS_Transpose trans_a() const { return trans_a_; }
+    BLAS_Transpose trans_b() const { return trans_b_; }
+    const Expression& m() const { return m_; }
+    const Expression& n() const { return n_; }
+    const Expression& k() const { return k_; }
+    const Expression& lda() const { return lda_; }
+    const Expression& ldb() const { return ldb_; }
+    const Expression& ldc() const { return ldc_; }
+    types::PrimitiveType scalar_primitive() const { return precision_input_type(precision_); }
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    bool reads(const std::string& connector, const std::vector<data_flow::ConnectorBinding>& inputs) const override;
+    static std::unique_ptr<GEMMNode> from_json(const json::Value& j);
+
+private:
+    BLAS_Precision precision_;
+    BLAS_Layout layout_;
+    BLAS_Transpose trans_a_, trans_b_;
+    Expression m_, n_, k_, lda_, ldb_, ldc_;
+};
+
+} // namespace math::blas
+
+namespace math::tensor {
+
+inline const std::string LibraryNodeType_Softmax = "ml::Softmax";
+inline const std::string LibraryNodeType_Conv = "ml::Conv";
+inline const std::string LibraryNodeType_MatMul = "ml::MatMul";
+inline const std::string LibraryNodeType_Attention = "ml::Attention";
+
+// reference: .../tensor/reduce_ops/softmax_node.h:9-49, reduce_node.h:194-245
+class SoftmaxNode : public data_flow::LibraryNode {
+public:
+    SoftmaxNode(std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> axes,
+                types::PrimitiveType element = types::PrimitiveType::Float);
+    const std::vector<Expression>& shape() const { return shape_; }
+    const std::vector<int64_t>& axes() const { return axes_; }
+    types::PrimitiveType element() const { return element_; }
+    Expression rows() const;  // product of all dims but the last
+    Expression cols() const;  // the last dim
+    bool last_axis_only() const;
+
+    void validate() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<SoftmaxNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    std::vector<int64_t> axes_;
+    types::PrimitiveType element_;
+};
+
+// reference: .../tensor/conv_node.h:48-217, conv_node.cpp:552-647
+class ConvNode : public data_flow::LibraryNode {
+public:
+    ConvNode(std::string implementation_type, std::vector<Expression> shape, std::vector<Expression> kernel_shape,
+             std::vector<Expression> strides, std::vector<Expression> pads, std::vector<Expression> dilations,
+             Expression output_channels, Expression group, bool has_bias,
+             types::PrimitiveType element = types::PrimitiveType::Float);
+    const std::vector<Expression>& shape() const { return shape_; }              // N, C, spatial...
+    const std::vector<Expression>& kernel_shape() const { return kernel_shape_; }
+    const std::vector<Expression>& strides() const { return strides_; }
+    const std::vector<Expression>& pads() const { return pads_; }                // begins..., ends...
+    const std::vector<Expression>& dilations() const { return dilations_; }
+    const Expression& output_channels() const { return output_channels_; }
+    const Expression& group() const { return group_; }
+    bool has_bias() const { return has_bias_; }
+    types::PrimitiveType element() const { return element_; }
+    // D_out per spatial dim (conv_node.cpp:224-233)
+    Expression output_dim(size_t i) const;
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ConvNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_, kernel_shape_, strides_, pads_, dilations_;
+    Expression output_channels_, group_;
+    bool has_bias_;
+    types::PrimitiveType element_;
+};
+
+// reference: .../tensor/matmul_node.h:49-193 (ONNX MatMul [...,M,K] @ [...,K,N]); contiguous operands only
+class MatMulNode : public data_flow::LibraryNode {
+public:
+    MatMulNode(std::string implementation_type, std::vector<Expression> shape_a, std::vector<Expression> shape_b,
+               types::PrimitiveType element);
+    const std::vector<Expression>& shape_a() const { return shape_a_; }
+    const std::vector<Expression>& shape_b() const { return shape_b_; }
+    types::PrimitiveType element() const { return element_; }
+    Expression batch() const;   // product of the leading dims of A ("1" when none); B must match or be 2-d
+    bool b_is_batched() const { return shape_b_.size() > 2; }
+    Expression m() const { return shape_a_[shape_a_.size() - 2]; }
+    Expression k() const { return shape_a_.back(); }
+    Expression n() const { return shape_b_.back(); }
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<MatMulNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_a_, shape_b_;
+    types::PrimitiveType element_;
+};
+
+// Added by the rocm target; the reference's node set has no attention
+// (sdfg/include/sdfg/data_flow/library_nodes/math/math.h:5-42).
+// O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D], non-causal.
+class AttentionNode : public data_flow::LibraryNode {
+public:
+    AttentionNode(std::string implementation_type, std::vector<Expression> shape_q, Expression seq_kv, std::string scale,
+                  types::PrimitiveType element, types::PrimitiveType output_element);
+    const std::vector<Expression>& shape_q() const { return shape_q_; }
+    const Expression& seq_kv() const { return seq_kv_; }
+    const std::string& scale() const { return scale_; }
+    types::PrimitiveType element() const { return element_; }
+    types::PrimitiveType output_element() const { return output_element_; }
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<AttentionNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_q_;
+    Expression seq_kv_;
+    std::string scale_;
+    types::PrimitiveType element_, output_element_;
+};
+
+} // namespace math::tensor
+
+namespace rocm {
+
+inline const std::string LibraryNodeType_ROCM_Offloading = "ROCMOffloading";
+
+// reference: opt/include/sdfg/targets/offloading/data_offloading_node.h:16-97
+enum class DataTransferDirection : int { D2H = -1, NONE = 0, H2D = 1 };
+enum class BufferLifecycle : int { FREE = -1, NO_CHANGE = 0, ALLOC = 1 };
+
+// Counterpart of CUDADataOffloadingNode (opt/src/targets/cuda/cuda_data_offloading_node.cpp:26-256):
+// connectors: H2D  in "_src" (host)   out "_dst" (device)
+//             D2H  in "_src" (device) out "_dst" (host)
+//             ALLOC only: out "_ret" (device);  FREE only: in "_ptr" (device)
+class ROCMDataOffloadingNode : public data_flow::LibraryNode {
+public:
+    ROCMDataOffloadingNode(Expression size, int device_id, DataTransferDirection direction, BufferLifecycle lifecycle);
+    const Expression& size() const { return size_; }
+    int device_id() const { return device_id_; }
+    DataTransferDirection transfer_direction() const { return direction_; }
+    BufferLifecycle buffer_lifecycle() const { return lifecycle_; }
+    bool is_h2d() const { return direction_ == DataTransferDirection::H2D; }
+    bool is_d2h() const { return direction_ == DataTransferDirection::D2H; }
+    bool is_alloc() const { return lifecycle_ == BufferLifecycle::ALLOC; }
+    bool is_free() const { return lifecycle_ == BufferLifecycle::FREE; }
+    bool blocking() const { return true; }
+    // true when `other` undoes or repeats this node on the same buffers (D2H followed by H2D ...)
+    bool redundant_with(const ROCMDataOffloadingNode& other) const;
+    bool equal_with(const ROCMDataOffloadingNode& other) const;
+
+    std::string toStr() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string&) const override { return size_; }
+    static std::unique_ptr<ROCMDataOffloadingNode> from_json(const json::Value& j);
+
+private:
+    Expression size_;
+    int device_id_;
+    DataTransferDirection direction_;
+    BufferLifecycle lifecycle_;
+};
+
+} // namespace rocm
+
+namespace structured_control_flow {
+
+// One block of the root sequence: a dataflow graph with exactly one library node.
+struct Block {
+    size_t element_id = 0;
+    std::unique_ptr<data_flow::LibraryNode> node;
+    std::vector<data_flow::ConnectorBinding> inputs;
+    std::vector<data_flow::ConnectorBinding> outputs;
+
+    const data_flow::ConnectorBinding* input(const std::string& connector) const;
+    const data_flow::ConnectorBinding* output(const std::string& connector) const;
+};
+
+} // namespace structured_control_flow
+
+// reference: sdfg/include/sdfg/function.h + structured_sdfg.h
+class StructuredSDFG {
+public:
+    explicit StructuredSDFG(std::string name) : name_(std::move(name)) {}
+
+    const std::string& name() const { return name_; }
+    const std::vector<std::string>& arguments() const { return arguments_; }
+    const std::map<std::string, Container>& containers() const { return containers_; }
+    std::vector<structured_control_flow::Block>& blocks() { return blocks_; }
+    const std::vector<structured_control_flow::Block>& blocks() const { return blocks_; }
+    bool exists(const std::string& name) const { return containers_.count(name) != 0; }
+    const Container& container(const std::string& name) const;
+    Container& container(const std::string& name);
+    // "" = void function; otherwise the function returns this pointer container (torch entry)
+    const std::string& return_container() const { return return_container_; }
+    void set_return_container(const std::string& name) { return_container_ = name; }
+
+    void add_container(Container c, bool is_argument);
+    structured_control_flow::Block& add_block(std::unique_ptr<data_flow::LibraryNode> node,
+                                              std::vector<data_flow::ConnectorBinding> inputs,
+                                              std::vector<data_flow::ConnectorBinding> outputs, size_t position = (size_t) -1);
+    size_t next_element_id() { return ++element_counter_; }
+
+    void add_metadata(const std::string& key, const std::string& value) { metadata_[key] = value; }
+    const std::string& metadata(const std::string& key) const;
+    const std::map<std::string, std::string>& metadata() const { return metadata_; }
+
+    // structure checks: containers exist, connectors complete, element types agree
+    void validate() const;
+
+    json::Value to_json() const;
+    static std::unique_ptr<StructuredSDFG> from_json(const json::Value& j);
+
+private:
+    std::string name_;
+    std::vector<std::string> arguments_;
+    std::map<std::string, Container> containers_;
+    std::vector<structured_control_flow::Block> blocks_;
+    std::map<std::string, std::string> metadata_;
+    std::string return_container_;
+    size_t element_counter_ = 0;
+};
+
+using Function = StructuredSDFG;
+
+namespace serializer {
+
+// reference: sdfg/include/sdfg/serializer/json_serializer.h (LibraryNodeSerializerRegistry)
+using LibraryNodeDeserializeFn = std::unique_ptr<data_flow::LibraryNode> (*)(const json::Value&);
+
+class LibraryNodeSerializerRegistry {
+public:
+    static LibraryNodeSerializerRegistry& instance();
+    // first registration wins, as in the reference's registries
+    void register_library_node_serializer(const std::string& code, LibraryNodeDeserializeFn fn);
+    LibraryNodeDeserializeFn get_library_node_serializer(const std::string& code) const;
+    size_t size() const;
+
+private:
+    LibraryNodeSerializerRegistry();
+    std::map<std::string, LibraryNodeDeserializeFn> fns_;
+};
+
+} // namespace serializer
+
+namespace builder {
+// Thin stand-in for builder::StructuredSDFGBuilder: the object passes mutate an SDFG through.
+class StructuredSDFGBuilder {
+public:
+    explicit StructuredSDFGBuilder(StructuredSDFG& sdfg) : sdfg_(sdfg) {}
+    StructuredSDFG& subject() { return sdfg_; }
+
+private:
+    StructuredSDFG& sdfg_;
+};
+} // namespace builder
+
+namespace analysis {
+class AnalysisManager {
+public:
+    explicit AnalysisManager(StructuredSDFG& sdfg) : sdfg_(sdfg) {}
+    StructuredSDFG& sdfg() { return sdfg_; }
+    void invalidate_all() {}
+
+private:
+    StructuredSDFG& sdfg_;
+};
+} // namespace analysis
+
+} // namespace sdfg

@@ -55,6 +55,8 @@ _SIGNATURES = {
     "docc_rocm_event_destroy": [_vp],
     "docc_rocm_event_record": [_vp, _vp],
     "docc_rocm_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(_f32)],
+    "docc_rocm_report_failure": [ctypes.c_char_p, ctypes.c_char_p, _int],
+    "docc_rocm_take_failure": [ctypes.c_char_p, ctypes.c_size_t],
     "docc_rocm_last_error": [],
     "docc_rocm_version": [],
     "docc_rocm_dgemm": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _vp, _i64, _f64, _vp, _i64],
@@ -67,7 +69,8 @@ _SIGNATURES = {
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
 }
-_RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p}
+_RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
+            "docc_rocm_report_failure": None}
 
 #: every symbol the two public headers declare
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -99,6 +102,13 @@ def call(name: str, *args) -> None:
     rc = getattr(lib(), name)(*args)
     if rc != 0:
         raise RocmRuntimeError(name, rc, last_error())
+
+
+def take_failure() -> tuple[int, str]:
+    """Collects (and clears) the failure reported by generated code, if any."""
+    buf = ctypes.create_string_buffer(1024)
+    code = lib().docc_rocm_take_failure(buf, 1024)
+    return int(code), buf.value.decode()
 
 
 def version() -> str:

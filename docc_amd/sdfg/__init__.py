@@ -1,0 +1,338 @@
+"""Python face of the SDFG carrier: `StructuredSDFG`, `StructuredSDFGBuilder`
+and the element types, over the C ABI of ``libdocc_rocm_target.so``
+(``include/docc_rocm_target.h``).
+
+It mirrors the part of the reference's ``docc.sdfg`` module that the hot path
+uses (python/bindings/bindings.cpp:136-480): ``StructuredSDFG.{parse, validate,
+expand, simplify, normalize, dump, schedule, _compile, metadata, loop_report,
+arguments, name}`` and ``StructuredSDFGBuilder.{add_container, add_gemm,
+add_reduce_op, add_conv, add_return}``. The SDFG itself lives as JSON text and
+is handed to the native library for every step that does real work.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+import json
+import os
+from pathlib import Path
+from typing import Any, Dict, List, Optional, Sequence
+
+_LIB_DIR = Path(__file__).resolve().parent.parent / "lib"
+_TARGET_LIB = _LIB_DIR / "libdocc_rocm_target.so"
+_INCLUDE_DIR = Path(__file__).resolve().parent.parent.parent / "include"
+
+_lib: Optional[ctypes.CDLL] = None
+
+#: every symbol include/docc_rocm_target.h declares
+EXPORTED_SYMBOLS = (
+    "docc_rocm_target_register", "docc_rocm_target_dispatcher_keys", "docc_rocm_target_validate",
+    "docc_rocm_target_schedule", "docc_rocm_target_generate", "docc_rocm_target_compile",
+    "docc_rocm_target_report", "docc_rocm_target_free", "docc_rocm_target_last_error",
+)
+
+
+class InvalidSDFGException(RuntimeError):
+    pass
+
+
+def _native() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not _TARGET_LIB.exists():
+            raise RuntimeError(f"{_TARGET_LIB} is missing; run `python -m docc_amd.build`")
+        lib = ctypes.CDLL(str(_TARGET_LIB))
+        cp = ctypes.c_char_p
+        lib.docc_rocm_target_register.restype = ctypes.c_int
+        for name, args in (("docc_rocm_target_dispatcher_keys", []), ("docc_rocm_target_validate", [cp]),
+                           ("docc_rocm_target_schedule", [cp, cp, cp]), ("docc_rocm_target_generate", [cp, cp]),
+                           ("docc_rocm_target_compile", [cp, cp, cp, cp]), ("docc_rocm_target_report", [cp])):
+            fn = getattr(lib, name)
+            fn.argtypes = args
+            fn.restype = ctypes.c_void_p  # kept as an address so that it can be freed
+        lib.docc_rocm_target_free.argtypes = [ctypes.c_void_p]
+        lib.docc_rocm_target_last_error.restype = cp
+        lib.docc_rocm_target_register()
+        _lib = lib
+    return _lib
+
+
+def _call(name: str, *args: Optional[str]) -> str:
+    lib = _native()
+    raw = getattr(lib, name)(*[a.encode() if a is not None else None for a in args])
+    if not raw:
+        msg = (lib.docc_rocm_target_last_error() or b"").decode()
+        raise InvalidSDFGException(msg or f"{name} failed")
+    try:
+        return ctypes.string_at(raw).decode()
+    finally:
+        lib.docc_rocm_target_free(raw)
+
+
+def registered_dispatchers() -> List[str]:
+    """The "<code>::<implementation type>" keys the code generator can dispatch."""
+    return json.loads(_call("docc_rocm_target_dispatcher_keys"))
+
+
+class PrimitiveType(enum.Enum):
+    Void = "Void"
+    Bool = "Bool"
+    Int8 = "Int8"
+    Int16 = "Int16"
+    Int32 = "Int32"
+    Int64 = "Int64"
+    UInt8 = "UInt8"
+    UInt16 = "UInt16"
+    UInt32 = "UInt32"
+    UInt64 = "UInt64"
+    Half = "Half"
+    BFloat = "BFloat"
+    Float = "Float"
+    Double = "Double"
+
+
+class Scalar:
+    def __init__(self, primitive_type: PrimitiveType):
+        self.primitive_type = primitive_type
+
+    def __repr__(self):
+        return f"Scalar({self.primitive_type.name})"
+
+
+class Pointer:
+    def __init__(self, pointee: Scalar):
+        self.pointee_type = pointee
+
+    @property
+    def primitive_type(self) -> PrimitiveType:
+        return self.pointee_type.primitive_type
+
+    def __repr__(self):
+        return f"Pointer({self.pointee_type!r})"
+
+
+# BLAS enums as the GEMM node serialises them (reference blas_node.h:49-126)
+BLAS_PRECISION = {PrimitiveType.Half: ord("h"), PrimitiveType.Float: ord("s"), PrimitiveType.Double: ord("d"),
+                  PrimitiveType.BFloat: ord("b")}
+ROW_MAJOR, COL_MAJOR = 101, 102
+NO_TRANS, TRANS = 111, 112
+
+
+def _expr(e: Any) -> str:
+    return str(int(e)) if isinstance(e, (int,)) or hasattr(e, "__index__") else str(e)
+
+
+class StructuredSDFG:
+    """An SDFG held as JSON; every operation goes through the native target library."""
+
+    def __init__(self, data: Dict[str, Any]):
+        self._data = data
+
+    # -- construction ---------------------------------------------------------
+    @staticmethod
+    def parse(text: str) -> "StructuredSDFG":
+        return StructuredSDFG(json.loads(_call("docc_rocm_target_validate", text)))
+
+    @staticmethod
+    def from_file(path: str) -> "StructuredSDFG":
+        return StructuredSDFG.parse(Path(path).read_text())
+
+    def to_json(self) -> str:
+        return json.dumps(self._data)
+
+    # -- inspection -----------------------------------------------------------
+    @property
+    def name(self) -> str:
+        return self._data["name"]
+
+    @property
+    def arguments(self) -> List[str]:
+        return list(self._data["arguments"])
+
+    @property
+    def containers(self) -> Dict[str, Any]:
+        return self._data["containers"]
+
+    @property
+    def return_container(self) -> str:
+        return self._data.get("return", "") or ""
+
+    def type(self, name: str):
+        c = self._data["containers"][name]
+        s = Scalar(PrimitiveType(c["element"]))
+        return Pointer(s) if c["type"] == "pointer" else s
+
+    def metadata(self, key: str) -> str:
+        return self._data.get("metadata", {})[key]
+
+    def add_metadata(self, key: str, value: str) -> None:
+        self._data.setdefault("metadata", {})[key] = str(value)
+
+    def library_nodes(self) -> List[Dict[str, Any]]:
+        return [c["dataflow"]["library_node"] for c in self._data["root"]["children"]]
+
+    def loop_report(self) -> Dict[str, int]:
+        """Counts per library-node code / implementation type and transfers (there are no loops in
+        these SDFGs); the analogue of the reference's loop_report (py_structured_sdfg.cpp:570-583)."""
+        return json.loads(_call("docc_rocm_target_report", self.to_json()))
+
+    # -- pipeline -------------------------------------------------------------
+    def validate(self) -> None:
+        self._data = json.loads(_call("docc_rocm_target_validate", self.to_json()))
+
+    def expand(self) -> None:
+        """Math library nodes are kept whole for the rocm target; nothing to expand. (The
+        reference expands them into loop nests for every target except the tensor targets,
+        python/docc/python/python_program.py:275-277.)"""
+
+    def simplify(self) -> None:
+        """No loop nests, so there is nothing to simplify."""
+
+    def normalize(self) -> None:
+        """No loop nests, so there is nothing to normalize."""
+
+    def dump(self, output_folder: str, suffix: str = "") -> None:
+        os.makedirs(output_folder, exist_ok=True)
+        name = self.name + (f".{suffix}" if suffix else "") + ".json"
+        Path(output_folder, name).write_text(json.dumps(self._data, indent=2))
+
+    def schedule(self, target: str, category: str = "server", remote_tuning: bool = False,
+                 options: Optional[Dict[str, Any]] = None) -> None:
+        if target in ("none", "sequential"):
+            return
+        if target != "rocm":
+            raise NotImplementedError(f"Target '{target}' is not supported: this package provides the 'rocm' target only")
+        opts = {k: v for k, v in (options or {}).items() if k in ("offload", "require_all_mapped")}
+        self._data = json.loads(_call("docc_rocm_target_schedule", self.to_json(), category, json.dumps(opts)))
+
+    def generate(self, output_folder: str) -> Dict[str, Any]:
+        """Writes <name>.h / <name>.cpp and returns the generator's report."""
+        return json.loads(_call("docc_rocm_target_generate", self.to_json(), output_folder))
+
+    def _compile(self, output_folder: str, target: str = "rocm", instrumentation_mode: str = "",
+                 capture_args: bool = False) -> str:
+        """Generates, compiles and links lib<name>.so; returns its path."""
+        return _call("docc_rocm_target_compile", self.to_json(), output_folder, str(_INCLUDE_DIR), str(_LIB_DIR))
+
+
+class StructuredSDFGBuilder:
+    """Builds the flat block sequence. Method names and argument meaning follow the reference's
+    PyStructuredSDFGBuilder (python/bindings/builder/py_structured_sdfg_builder.cpp:654-774 add_gemm,
+    :960-1013 add_conv, :1041-1088 add_reduce_op)."""
+
+    def __init__(self, name: str, return_type: Optional[Any] = None):
+        self._data: Dict[str, Any] = {"type": "structured_sdfg", "name": name, "arguments": [], "containers": {},
+                                      "return": "", "metadata": {}, "root": {"type": "sequence", "children": []}}
+        self._ids = 0
+
+    def exists(self, name: str) -> bool:
+        return name in self._data["containers"]
+
+    def find_new_name(self, prefix: str = "tmp_") -> str:
+        i = 0
+        while f"{prefix}{i}" in self._data["containers"]:
+            i += 1
+        return f"{prefix}{i}"
+
+    def add_container(self, name: str, type_: Any, is_argument: bool = False, transient_bytes: Optional[Any] = None,
+                      storage: str = "CPU") -> None:
+        if name in self._data["containers"]:
+            raise InvalidSDFGException(f"container '{name}' already exists")
+        entry = {"type": "pointer" if isinstance(type_, Pointer) else "scalar", "element": type_.primitive_type.value,
+                 "transient": transient_bytes is not None, "storage": storage}
+        if transient_bytes is not None:
+            entry["size"] = _expr(transient_bytes)
+        self._data["containers"][name] = entry
+        if is_argument:
+            self._data["arguments"].append(name)
+
+    def _element(self, name: str) -> PrimitiveType:
+        return PrimitiveType(self._data["containers"][name]["element"])
+
+    def _add_block(self, node: Dict[str, Any], inputs: Sequence[Dict[str, Any]], outputs: Sequence[Dict[str, Any]]) -> None:
+        self._ids += 2
+        node = {"type": "library_node", "element_id": self._ids, **node}
+        self._data["root"]["children"].append({"type": "block", "element_id": self._ids - 1, "dataflow": {
+            "library_node": node, "inputs": list(inputs), "outputs": list(outputs)}})
+
+    @staticmethod
+    def _operand(connector: str, value: Any, const_type: Optional[PrimitiveType] = None) -> Dict[str, Any]:
+        if const_type is not None:
+            return {"connector": connector, "constant": str(value), "type": const_type.value}
+        return {"connector": connector, "data": value}
+
+    def add_gemm(self, A: str, B: str, C: str, alpha: str, beta: str, m: Any, n: Any, k: Any, trans_a: bool = False,
+                 trans_b: bool = False, lda: Any = None, ldb: Any = None, ldc: Any = None) -> None:
+        """C = alpha * op(A) op(B) + beta * C, row-major. alpha/beta are literals ("1.0") or scalar
+        container names, as in the reference. The node is created with the BLAS implementation
+        type, like the reference's add_gemm; the precision follows A's element type, and bf16
+        operands select the added 'b' precision (fp32 accumulate, C must be Float)."""
+        elem = self._element(A)
+        if self._element(B) != elem:
+            raise InvalidSDFGException("GEMM: A and B must have the same element type")
+        if elem not in BLAS_PRECISION:
+            raise InvalidSDFGException(f"GEMM: unsupported element type {elem.name}")
+        out_elem = PrimitiveType.Float if elem == PrimitiveType.BFloat else elem
+        if self._element(C) != out_elem:
+            raise InvalidSDFGException(f"GEMM: C must be {out_elem.name} for {elem.name} operands")
+        lda = lda if lda is not None else (m if trans_a else k)
+        ldb = ldb if ldb is not None else (k if trans_b else n)
+        ldc = ldc if ldc is not None else n
+
+        def scalar(connector: str, v: str) -> Dict[str, Any]:
+            return self._operand(connector, v) if v in self._data["containers"] else self._operand(connector, v, out_elem)
+
+        self._add_block(
+            {"code": "GEMM", "implementation_type": "BLAS", "side_effect": False, "precision": BLAS_PRECISION[elem],
+             "layout": ROW_MAJOR, "trans_a": TRANS if trans_a else NO_TRANS, "trans_b": TRANS if trans_b else NO_TRANS,
+             "m": _expr(m), "n": _expr(n), "k": _expr(k), "lda": _expr(lda), "ldb": _expr(ldb), "ldc": _expr(ldc)},
+            [self._operand("__A", A), self._operand("__B", B), self._operand("__C", C), scalar("__alpha", alpha), scalar("__beta", beta)],
+            [self._operand("__C", C)])
+
+    def add_matmul(self, A: str, B: str, Y: str, shape_a: Sequence[Any], shape_b: Sequence[Any]) -> None:
+        """ml::MatMul, [..., M, K] @ [..., K, N] on contiguous operands."""
+        self._add_block({"code": "ml::MatMul", "implementation_type": "NONE", "side_effect": False,
+                         "shape_a": [_expr(s) for s in shape_a], "shape_b": [_expr(s) for s in shape_b],
+                         "element_type": self._element(A).value},
+                        [self._operand("A", A), self._operand("B", B)], [self._operand("Y", Y)])
+
+    def add_reduce_op(self, op: str, X: str, Y: str, shape: Sequence[Any], axes: Sequence[int], keepdims: bool = False) -> None:
+        if op != "softmax":
+            raise NotImplementedError(f"reduce op '{op}' is not part of the rocm target (softmax only)")
+        if keepdims:
+            raise InvalidSDFGException("Unsupported attribute on library node: softmax")
+        self._add_block({"code": "ml::Softmax", "implementation_type": "NONE", "side_effect": False,
+                         "shape": [_expr(s) for s in shape], "axes": [int(a) for a in axes], "keepdims": False,
+                         "element_type": self._element(X).value},
+                        [self._operand("X", X)], [self._operand("Y", Y)])
+
+    def add_conv(self, X: str, W: str, Y: str, shape: Sequence[Any], kernel_shape: Sequence[Any], strides: Sequence[Any],
+                 pads: Sequence[Any], dilations: Sequence[Any], output_channels: Any, group: Any = 1, B: Optional[str] = None) -> None:
+        """ml::Conv (ONNX semantics, zero padding); `pads` holds begins then ends."""
+        inputs = [self._operand("X", X), self._operand("W", W)]
+        if B is not None:
+            inputs.append(self._operand("B", B))
+        self._add_block({"code": "ml::Conv", "implementation_type": "NONE", "side_effect": False,
+                         "shape": [_expr(s) for s in shape], "kernel_shape": [_expr(s) for s in kernel_shape],
+                         "strides": [_expr(s) for s in strides], "pads": [_expr(s) for s in pads],
+                         "dilations": [_expr(s) for s in dilations], "output_channels": _expr(output_channels),
+                         "group": _expr(group), "has_bias": B is not None, "element_type": self._element(X).value},
+                        inputs, [self._operand("Y", Y)])
+
+    def add_attention(self, Q: str, K: str, V: str, O: str, shape_q: Sequence[Any], seq_kv: Any, scale: Any) -> None:
+        """ml::Attention: O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]."""
+        self._add_block({"code": "ml::Attention", "implementation_type": "NONE", "side_effect": False,
+                         "shape_q": [_expr(s) for s in shape_q], "seq_kv": _expr(seq_kv), "scale": repr(float(scale)),
+                         "element_type": self._element(Q).value, "output_type": self._element(O).value},
+                        [self._operand("Q", Q), self._operand("K", K), self._operand("V", V)], [self._operand("O", O)])
+
+    def add_return(self, container: str) -> None:
+        self._data["return"] = container
+
+    def add_metadata(self, key: str, value: str) -> None:
+        self._data["metadata"][key] = str(value)
+
+    def move(self) -> StructuredSDFG:
+        sdfg = StructuredSDFG(self._data)
+        sdfg.validate()
+        return sdfg

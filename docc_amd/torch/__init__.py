@@ -1,0 +1,539 @@
+"""`torch.compile(model, backend="docc")` and `compile_torch` for the `rocm` target.
+
+Same surface as the reference's `docc.torch` (mlir/docc/torch/__init__.py:15-441): `TorchProgram`,
+`compile_torch(model, example_input, target, category)`, the global `set_backend_options(target,
+category)` read by the backend, a backend registered under the name "docc" that returns a tuple of
+tensors to dynamo, and `metadata("return_shape")` on the SDFG.
+
+The reference goes FX -> torch-mlir -> linalg -> SDFG and supports only 2-d matmul and
+unpadded, bias-free convolution (mlir/lib/Target/SDFG/LinalgToSDFGTranslator.cpp:517-523,696-699);
+this front end lowers the FX graph directly and covers what the rocm kernels implement:
+
+    torch.matmul / @ / mm / bmm            -> GEMM (2-d, with transposed operands) or ml::MatMul (batched)
+    softmax(x, dim=-1) on fp32             -> ml::Softmax
+    F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
+    softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
+                                           -> ml::Attention (bf16, head dim 64)
+
+Tensors on a `cuda` device are passed to the generated function as device pointers (no
+transfers, the kernels run on the null stream in order with torch's default stream); CPU tensors
+are uploaded and downloaded by the generated code. Anything else raises NotImplementedError: this
+target has no CPU lowering to fall back to.
+"""
+from __future__ import annotations
+
+import ctypes
+import getpass
+import hashlib
+import math
+import operator
+import os
+import shutil
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+from docc_amd import runtime
+from docc_amd.compiler import CompiledSDFG, DoccProgram
+from docc_amd.python.target_registry import get_target_compile_fn, get_target_schedule_fn
+from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFG, StructuredSDFGBuilder
+
+import docc_amd.python  # noqa: F401  (registers the rocm target hooks)
+
+
+def _elem(dtype) -> PrimitiveType:
+    import torch
+
+    table = {torch.float32: PrimitiveType.Float, torch.float64: PrimitiveType.Double, torch.bfloat16: PrimitiveType.BFloat}
+    if dtype not in table:
+        raise NotImplementedError(f"tensor dtype {dtype} is not supported by the rocm target")
+    return table[dtype]
+
+
+class _T:
+    """A tensor held in an SDFG container."""
+
+    def __init__(self, name: str, shape: Sequence[int], dtype):
+        self.name, self.shape, self.dtype = name, [int(s) for s in shape], dtype
+
+
+class _Transposed:
+    def __init__(self, base: _T):
+        self.base = base
+
+
+class _Scores:
+    """scale * q @ k^T, kept symbolic until a softmax and a product with v complete the pattern."""
+
+    def __init__(self, q: _T, k: _T, scale: float = 1.0):
+        self.q, self.k, self.scale = q, k, scale
+
+
+class _Probs:
+    def __init__(self, scores: _Scores):
+        self.scores = scores
+
+
+class _FxLowering:
+    def __init__(self, gm, example_inputs: Sequence[Any], name: str):
+        import torch
+
+        self.torch = torch
+        self.gm = gm
+        self.builder = StructuredSDFGBuilder(name)
+        self.env: Dict[Any, Any] = {}
+        self.inputs: List[Tuple[str, Any]] = []      # (container, ("arg", index) | ("attr", qualified name))
+        self.outputs: List[Tuple[str, List[int], Any]] = []
+        self.example_inputs = list(example_inputs)
+        self._propagate_shapes()
+
+    # ---- shapes ---------------------------------------------------------------------
+    def _propagate_shapes(self):
+        torch = self.torch
+        if all("example_value" in n.meta or "tensor_meta" in n.meta for n in self.gm.graph.nodes if n.op not in ("output",)):
+            return
+        from torch._subclasses.fake_tensor import FakeTensorMode
+        from torch.fx.passes.shape_prop import ShapeProp
+
+        mode = FakeTensorMode(allow_non_fake_inputs=True)
+        fake = [mode.from_tensor(a) if isinstance(a, torch.Tensor) else a for a in self.example_inputs]
+        ShapeProp(self.gm, fake_mode=mode).propagate(*fake)
+
+    def meta(self, node):
+        v = node.meta.get("example_value")
+        if v is None:
+            v = node.meta.get("tensor_meta")
+        if v is None:
+            raise NotImplementedError(f"no shape information for FX node {node.name}")
+        return list(v.shape), v.dtype
+
+    # ---- containers ---------------------------------------------------------------------
+    def add_input(self, label: str, shape, dtype, source) -> _T:
+        name = self.builder.find_new_name(f"{label}_") if self.builder.exists(label) else label
+        self.builder.add_container(name, Pointer(Scalar(_elem(dtype))), True)
+        self.inputs.append((name, source))
+        return _T(name, shape, dtype)
+
+    def new_tensor(self, shape, dtype, dest: Optional[str]) -> _T:
+        if dest is not None:
+            if not self.builder.exists(dest):  # `_docc_ret_<i>`: an output pointer argument
+                self.builder.add_container(dest, Pointer(Scalar(_elem(dtype))), True)
+            return _T(dest, shape, dtype)
+        nbytes = int(math.prod(shape)) * self.torch.empty((), dtype=dtype).element_size()
+        name = self.builder.find_new_name("_tmp_")
+        self.builder.add_container(name, Pointer(Scalar(_elem(dtype))), False, transient_bytes=nbytes)
+        return _T(name, shape, dtype)
+
+    def fail(self, node, what: str):
+        raise NotImplementedError(f"FX node {node.name} ({node.target}): {what} is not supported by the rocm target")
+
+    # ---- operations -----------------------------------------------------------------------
+    def matmul(self, node, a, b, dest):
+        torch = self.torch
+        if isinstance(a, _Probs):
+            return self.attention(node, a.scores.q, a.scores.k, b, a.scores.scale, dest)
+        ta = tb = False
+        if isinstance(a, _Transposed):
+            ta, a = True, a.base
+        if isinstance(b, _Transposed):
+            tb, b = True, b.base
+        if not isinstance(a, _T) or not isinstance(b, _T):
+            self.fail(node, "a product of these operands")
+        if a.dtype != b.dtype:
+            self.fail(node, "a product of mixed dtypes")
+        if len(a.shape) > 2 and tb and not ta and a.dtype == torch.bfloat16 and len(b.shape) == len(a.shape):
+            return _Scores(a, b)  # q @ k^T: waits for its softmax
+        if a.dtype == torch.bfloat16:
+            self.fail(node, "a bf16 product outside the attention pattern (its result would have to be rounded back to bf16)")
+        if len(a.shape) == 2 and len(b.shape) == 2:
+            m, k = (a.shape[1], a.shape[0]) if ta else a.shape
+            k2, n = (b.shape[1], b.shape[0]) if tb else b.shape
+            if k != k2:
+                self.fail(node, f"inner dimensions {k} and {k2}")
+            out = self.new_tensor([m, n], a.dtype, dest)
+            one, zero = "1.0", "0.0"
+            self.builder.add_gemm(a.name, b.name, out.name, one, zero, m, n, k, ta, tb, a.shape[1], b.shape[1], n)
+            return out
+        if ta or tb:
+            self.fail(node, "a transposed operand in a batched product")
+        if len(b.shape) > 2 and b.shape[:-2] != a.shape[:-2]:
+            self.fail(node, "broadcasting batch dimensions")
+        out = self.new_tensor(a.shape[:-1] + [b.shape[-1]], a.dtype, dest)
+        self.builder.add_matmul(a.name, b.name, out.name, a.shape, b.shape)
+        return out
+
+    def attention(self, node, q: _T, k: _T, v, scale: float, dest):
+        torch = self.torch
+        if not isinstance(v, _T):
+            self.fail(node, "attention values of this form")
+        if len(q.shape) == 3:  # [B*H, S, D] given as 3-d: treat the leading dim as batch with one head
+            shape_q = [q.shape[0], 1, q.shape[1], q.shape[2]]
+        elif len(q.shape) == 4:
+            shape_q = list(q.shape)
+        else:
+            self.fail(node, "attention on tensors that are not 3-d or 4-d")
+        if q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
+            self.fail(node, "attention on tensors other than bfloat16")
+        if k.shape != v.shape or k.shape[:-2] != q.shape[:-2] or k.shape[-1] != q.shape[-1]:
+            self.fail(node, "attention with mismatched q/k/v shapes")
+        out = self.new_tensor(q.shape, q.dtype, dest)
+        self.builder.add_attention(q.name, k.name, v.name, out.name, shape_q, k.shape[-2], scale)
+        return out
+
+    def softmax(self, node, x, dim, dest):
+        if isinstance(x, _Scores):
+            if dim not in (-1, len(x.q.shape) - 1):
+                self.fail(node, "softmax of attention scores over an axis other than the last")
+            return _Probs(x)
+        if not isinstance(x, _T):
+            self.fail(node, "softmax of this value")
+        if dim not in (-1, len(x.shape) - 1):
+            self.fail(node, "softmax over an axis other than the last")
+        if x.dtype != self.torch.float32:
+            self.fail(node, "softmax on a dtype other than float32")
+        out = self.new_tensor(x.shape, x.dtype, dest)
+        self.builder.add_reduce_op("softmax", x.name, out.name, x.shape, [-1])
+        return out
+
+    def conv2d(self, node, x, w, bias, stride, padding, dilation, groups, dest):
+        pair = lambda v: [int(v), int(v)] if isinstance(v, int) else [int(e) for e in v]
+        if not isinstance(x, _T) or not isinstance(w, _T) or len(x.shape) != 4 or len(w.shape) != 4:
+            self.fail(node, "conv2d on these operands")
+        if groups != 1:
+            self.fail(node, "grouped convolution")
+        if isinstance(padding, str):
+            self.fail(node, "string padding modes")
+        if x.dtype != self.torch.float32:
+            self.fail(node, "conv2d on a dtype other than float32")
+        stride, padding, dilation = pair(stride), pair(padding), pair(dilation)
+        oh, ow = ((x.shape[2 + i] + 2 * padding[i] - dilation[i] * (w.shape[2 + i] - 1) - 1) // stride[i] + 1 for i in range(2))
+        out = self.new_tensor([x.shape[0], w.shape[0], oh, ow], x.dtype, dest)
+        self.builder.add_conv(x.name, w.name, out.name, x.shape, w.shape[2:], stride, padding + padding, dilation, w.shape[0], 1,
+                              bias.name if isinstance(bias, _T) else None)
+        return out
+
+    def scale(self, node, x, factor: float):
+        if isinstance(x, _Scores):
+            return _Scores(x.q, x.k, x.scale * factor)
+        self.fail(node, "scaling a tensor that is not an attention score matrix")
+
+    def transpose(self, node, x, d0: int, d1: int):
+        if not isinstance(x, _T):
+            self.fail(node, "transposing this value")
+        rank = len(x.shape)
+        if {d0 % rank, d1 % rank} != {rank - 2, rank - 1}:
+            self.fail(node, "a transpose other than of the last two dimensions")
+        return _Transposed(x)
+
+    # ---- graph walk -------------------------------------------------------------------------
+    def arg(self, a):
+        import torch.fx
+
+        if isinstance(a, torch.fx.Node):
+            return self.env[a]
+        return a
+
+    def lower(self) -> StructuredSDFG:
+        import torch
+        import torch.nn.functional as F
+
+        graph = self.gm.graph
+        output_node = next(n for n in graph.nodes if n.op == "output")
+        out_values = output_node.args[0]
+        out_list = list(out_values) if isinstance(out_values, (tuple, list)) else [out_values]
+        # the node that produces output i writes straight into `_docc_ret_<i>`
+        dest_of = {n: f"_docc_ret_{i}" for i, n in enumerate(out_list)}
+        arg_index = 0
+        for node in graph.nodes:
+            dest = dest_of.get(node)
+            if node.op == "placeholder":
+                shape, dtype = self.meta(node)
+                self.env[node] = self.add_input(node.name, shape, dtype, ("arg", arg_index))
+                arg_index += 1
+            elif node.op == "get_attr":
+                t = self.gm
+                for part in node.target.split("."):
+                    t = getattr(t, part)
+                self.env[node] = self.add_input(node.name, list(t.shape), t.dtype, ("attr", node.target))
+            elif node.op == "call_module":
+                mod = self.gm.get_submodule(node.target)
+                if not isinstance(mod, torch.nn.Conv2d):
+                    self.fail(node, f"module {type(mod).__name__}")
+                if mod.padding_mode != "zeros":
+                    self.fail(node, "non-zero padding modes")
+                w = self.add_input(f"{node.name}_weight", list(mod.weight.shape), mod.weight.dtype, ("attr", f"{node.target}.weight"))
+                b = None
+                if mod.bias is not None:
+                    b = self.add_input(f"{node.name}_bias", list(mod.bias.shape), mod.bias.dtype, ("attr", f"{node.target}.bias"))
+                self.env[node] = self.conv2d(node, self.arg(node.args[0]), w, b, mod.stride, mod.padding, mod.dilation, mod.groups, dest)
+            elif node.op in ("call_function", "call_method"):
+                self.env[node] = self.call(node, dest)
+            elif node.op == "output":
+                for i, n in enumerate(out_list):
+                    v = self.env[n]
+                    if not isinstance(v, _T) or v.name != f"_docc_ret_{i}":
+                        self.fail(n, "returning a value that no library node produces (inputs, views, partial patterns)")
+                    self.outputs.append((v.name, v.shape, v.dtype))
+        if not self.outputs:
+            raise NotImplementedError("the graph has no output produced by a library node")
+        self.builder.add_metadata("return_shape", "[" + ",".join(str(s) for s in self.outputs[0][1]) + "]")
+        return self._finish()
+
+    def _finish(self) -> StructuredSDFG:
+        # outputs are declared after the inputs: rebuild the argument order (inputs, then _docc_ret_<i>)
+        data = self.builder._data
+        outs = [name for name, _, _ in self.outputs]
+        data["arguments"] = [a for a in data["arguments"] if a not in outs] + outs
+        return self.builder.move()
+
+    def call(self, node, dest):
+        import torch
+        import torch.nn.functional as F
+
+        t = node.target
+        args = [self.arg(a) for a in node.args]
+        kwargs = {k: self.arg(v) for k, v in node.kwargs.items()}
+        method = t if node.op == "call_method" else None
+        # shape queries and arithmetic on plain Python numbers are folded while lowering
+        if t is getattr and isinstance(args[0], _T) and args[1] == "shape":
+            return tuple(args[0].shape)
+        if method == "size" and isinstance(args[0], _T):
+            return tuple(args[0].shape) if len(args) == 1 else args[0].shape[args[1]]
+        if method == "dim" and isinstance(args[0], _T):
+            return len(args[0].shape)
+        plain = lambda v: isinstance(v, (int, float, bool, str, type(None))) or (isinstance(v, (tuple, list)) and all(plain(e) for e in v))
+        if node.op == "call_function" and all(plain(a) for a in args) and all(plain(v) for v in kwargs.values()) and \
+                getattr(t, "__module__", "") in ("math", "_operator", "operator", "builtins"):
+            return t(*args, **kwargs)
+        if t in (torch.matmul, operator.matmul, torch.mm, torch.bmm) or method in ("matmul", "mm", "bmm"):
+            return self.matmul(node, args[0], args[1], dest)
+        if t is torch.transpose or method == "transpose":
+            return self.transpose(node, args[0], args[1], args[2])
+        if method == "permute" or t is torch.permute:
+            dims = list(args[1]) if isinstance(args[1], (tuple, list)) else list(args[1:])
+            rank = len(dims)
+            if dims[:-2] == list(range(rank - 2)) and dims[-2:] == [rank - 1, rank - 2]:
+                return self.transpose(node, args[0], -2, -1)
+            self.fail(node, "this permutation")
+        if t is getattr and args[1] in ("mT", "T"):
+            if args[1] == "T" and isinstance(args[0], _T) and len(args[0].shape) != 2:
+                self.fail(node, ".T on a tensor that is not 2-d")
+            return self.transpose(node, args[0], -2, -1)
+        if method in ("t",) or t is torch.t:
+            return self.transpose(node, args[0], 0, 1)
+        if t in (operator.truediv, torch.div) or method == "div":
+            if isinstance(args[1], (int, float)):
+                return self.scale(node, args[0], 1.0 / float(args[1]))
+        if t in (operator.mul, torch.mul) or method == "mul":
+            for x, c in ((args[0], args[1]), (args[1], args[0])):
+                if isinstance(c, (int, float)):
+                    return self.scale(node, x, float(c))
+        if t in (torch.softmax, F.softmax) or method == "softmax":
+            dim = kwargs.get("dim", args[1] if len(args) > 1 else None)
+            if dim is None:
+                self.fail(node, "softmax without an explicit dim")
+            return self.softmax(node, args[0], int(dim), dest)
+        if t in (F.conv2d, torch.conv2d):
+            names = ["input", "weight", "bias", "stride", "padding", "dilation", "groups"]
+            defaults = {"bias": None, "stride": 1, "padding": 0, "dilation": 1, "groups": 1}
+            bound = {**defaults, **dict(zip(names, args)), **kwargs}
+            return self.conv2d(node, bound["input"], bound["weight"], bound["bias"], bound["stride"], bound["padding"],
+                               bound["dilation"], bound["groups"], dest)
+        if t is F.scaled_dot_product_attention:
+            names = ["query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale"]
+            bound = {"attn_mask": None, "dropout_p": 0.0, "is_causal": False, "scale": None, **dict(zip(names, args)), **kwargs}
+            if bound["attn_mask"] is not None or bound["dropout_p"] not in (0, 0.0) or bound["is_causal"]:
+                self.fail(node, "masked, causal or dropout attention")
+            q = bound["query"]
+            if not isinstance(q, _T):
+                self.fail(node, "attention on this query")
+            scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
+            return self.attention(node, q, bound["key"], bound["value"], float(scale), dest)
+        if method == "contiguous" or t is torch.Tensor.contiguous:
+            return args[0]
+        self.fail(node, "this operation")
+
+
+class _CompiledTorch:
+    """Calls the generated function on torch tensors (device or host pointers)."""
+
+    def __init__(self, lib_path: str, sdfg: StructuredSDFG, inputs, outputs, gm, on_device: bool):
+        runtime.lib()
+        self.lib_path, self.sdfg = lib_path, sdfg
+        self.lib = ctypes.CDLL(lib_path)
+        self.func = getattr(self.lib, sdfg.name)
+        self.func.argtypes = [ctypes.c_void_p] * len(sdfg.arguments)
+        self.func.restype = None
+        self.inputs, self.outputs, self.gm, self.on_device = inputs, outputs, gm, on_device
+
+    def __call__(self, *args):
+        import torch
+
+        device = torch.device("cuda", torch.cuda.current_device()) if self.on_device else torch.device("cpu")
+        keep, ptrs = [], []
+        for name, (kind, ref) in self.inputs:
+            if kind == "arg":
+                t = args[ref]
+            else:
+                t = self.gm
+                for part in ref.split("."):
+                    t = getattr(t, part)
+            t = t.detach()
+            if t.device.type != device.type:
+                raise ValueError(f"input '{name}' is on {t.device}, the program was compiled for {device.type} tensors")
+            t = t.contiguous()
+            keep.append(t)
+            ptrs.append(t.data_ptr())
+        outs = [torch.empty(shape, dtype=dtype, device=device) for _, shape, dtype in self.outputs]
+        if self.on_device:
+            runtime.init(device.index or 0)
+            current = torch.cuda.current_stream()
+            if current != torch.cuda.default_stream():
+                current.synchronize()  # the kernels run on the null stream
+        self.func(*ptrs, *[o.data_ptr() for o in outs])
+        code, message = runtime.take_failure()
+        if code != 0:
+            raise runtime.RocmRuntimeError(self.sdfg.name, code, message)
+        if self.on_device and torch.cuda.current_stream() != torch.cuda.default_stream():
+            torch.cuda.default_stream().synchronize()
+        return outs[0] if len(outs) == 1 else tuple(outs)
+
+
+class TorchProgram(DoccProgram):
+    def __init__(self, model, example_input: Any = None, target: str = "none", category: str = "server",
+                 remote_tuning: bool = False, instrumentation_mode: Optional[str] = None, capture_args: Optional[bool] = None,
+                 name: Optional[str] = None):
+        if name is None:
+            name = model.__class__.__name__ if hasattr(model, "__class__") else "torch_model"
+        super().__init__(name=name, target=target, category=category, remote_tuning=remote_tuning,
+                         instrumentation_mode=instrumentation_mode, capture_args=capture_args)
+        self.model = model
+        self.example_input = example_input
+        self._sdfg: Optional[StructuredSDFG] = None
+        self._compiled: Optional[_CompiledTorch] = None
+        self._input_info: list = []
+        self._output_info: list = []
+        self._gm = None
+
+    def _examples(self, args: Sequence[Any]) -> List[Any]:
+        if args:
+            return list(args)
+        if self.example_input is None:
+            raise ValueError("TorchProgram needs an example input to compile")
+        return list(self.example_input) if isinstance(self.example_input, (tuple, list)) else [self.example_input]
+
+    def _graph_module(self):
+        import torch.fx
+
+        if self._gm is None:
+            self._gm = self.model if isinstance(self.model, torch.fx.GraphModule) else torch.fx.symbolic_trace(self.model)
+        return self._gm
+
+    def _get_cache_key(self, *args: Any) -> str:
+        import torch
+
+        parts = []
+        for a in self._examples(args):
+            parts.append(f"{tuple(a.shape)}:{a.dtype}:{a.device.type}" if isinstance(a, torch.Tensor) else f"scalar({type(a).__name__})")
+        return "|".join(parts)
+
+    def _lower(self, examples):
+        lowering = _FxLowering(self._graph_module(), examples, f"__docc_{self.name}")
+        sdfg = lowering.lower()
+        return sdfg, lowering
+
+    def to_sdfg(self, *args: Any) -> StructuredSDFG:
+        return self._lower(self._examples(args))[0]
+
+    def compile(self, *args: Any, output_folder: Optional[str] = None) -> _CompiledTorch:
+        import torch
+
+        examples = self._examples(args)
+        key = self._get_cache_key(*examples)
+        if output_folder is None and key in self.cache:
+            return self.cache[key]
+        on_device = any(isinstance(a, torch.Tensor) and a.device.type == "cuda" for a in examples)
+        sdfg, lowering = self._lower(examples)
+        self._sdfg = sdfg
+        folder = output_folder
+        if folder is None:
+            stable_id = hashlib.sha256(f"{self.name}|{self.target}|{self.category}|{key}".encode()).hexdigest()[:16]
+            base = os.environ.get("DOCC_TMP") or f"/tmp/{os.getenv('USER') or getpass.getuser()}/DOCC"
+            folder = f"{base}/{self.name}-{stable_id}"
+        if os.path.exists(folder):
+            shutil.rmtree(folder)
+        sdfg.validate()
+        sdfg.expand()
+        sdfg.simplify()
+        if self.target != "none":
+            sdfg.normalize()
+        sdfg.dump(folder)
+        options = {"offload": "none" if on_device else "function"}
+        if self.target != "none":
+            schedule_fn = get_target_schedule_fn(self.target)
+            if schedule_fn is not None:
+                schedule_fn(sdfg, self.category, options)
+            else:
+                sdfg.schedule(self.target, self.category, self.remote_tuning)
+        self.last_sdfg = sdfg
+        sdfg.dump(folder, "post_sched")
+        compile_fn = get_target_compile_fn(self.target)
+        if compile_fn is not None:
+            lib_path = compile_fn(sdfg, folder, self.instrumentation_mode or "", bool(self.capture_args), options)
+        else:
+            lib_path = sdfg._compile(output_folder=folder, target=self.target, instrumentation_mode=self.instrumentation_mode or "",
+                                     capture_args=bool(self.capture_args))
+        compiled = _CompiledTorch(lib_path, sdfg, lowering.inputs, lowering.outputs, self._graph_module(), on_device)
+        self._output_info = [{"shape": tuple(shape)} for _, shape, _ in lowering.outputs]
+        if output_folder is None:
+            self.cache[key] = compiled
+        self._compiled = compiled
+        return compiled
+
+    def __call__(self, *args: Any) -> Any:
+        compiled = self.compile(*args)
+        return self._convert_outputs(compiled(*self._convert_inputs(args)), args)
+
+    def _convert_inputs(self, args: tuple) -> tuple:
+        return args
+
+    def _convert_outputs(self, result: Any, original_args: tuple) -> Any:
+        return result
+
+
+def compile_torch(model, example_input, target: str = "none", category: str = "server") -> TorchProgram:
+    return TorchProgram(model, example_input=example_input, target=target, category=category)
+
+
+_backend_options = {"target": "none", "category": "server"}
+
+
+def set_backend_options(target: str = "none", category: str = "server"):
+    """Global options read by the "docc" torch.compile backend; call before torch.compile."""
+    _backend_options["target"] = target
+    _backend_options["category"] = category
+
+
+def _docc_backend(gm, example_inputs):
+    """Called by torch.compile(backend="docc") with the FX graph dynamo captured."""
+    example_input = example_inputs[0] if len(example_inputs) == 1 else tuple(example_inputs)
+    program = TorchProgram(gm, example_input=example_input, target=_backend_options["target"],
+                           category=_backend_options["category"])
+
+    def compiled_fn(*args):
+        result = program(*args)
+        return result if isinstance(result, (tuple, list)) else (result,)
+
+    return compiled_fn
+
+
+def _register_backend():
+    try:
+        import torch._dynamo
+
+        torch._dynamo.register_backend(name="docc")(_docc_backend)
+    except ImportError:  # torch without dynamo
+        pass
+    except Exception:  # already registered (module imported twice)
+        pass
+
+
+_register_backend()

@@ -103,6 +103,19 @@ int docc_rocm_event_destroy(docc_rocm_event_t event);
 int docc_rocm_event_record(docc_rocm_event_t event, docc_rocm_stream_t stream);
 int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, float* ms);
 
+/*
+ * Failure channel of generated code. The generated `extern "C"` functions have
+ * no error return (reference calling convention: sdfg/src/codegen/code_generators/cpp_code_generator.cpp:8-24),
+ * so a failing runtime call is reported here and the generated function
+ * returns early. With DOCC_ROCM_DEBUG set in the environment the report is
+ * printed and the process exits, which is what the reference's CUDA target
+ * does under DOCC_CUDA_DEBUG (opt/src/targets/cuda/cuda.cpp:62-91); otherwise
+ * the failure is kept until the caller collects it with
+ * docc_rocm_take_failure (returns the code, 0 if none, and clears it).
+ */
+void docc_rocm_report_failure(const char* function, const char* call, int code);
+int docc_rocm_take_failure(char* message, size_t message_len);
+
 /* Message of the last failure on this thread ("" if none). */
 const char* docc_rocm_last_error(void);
 

@@ -1,0 +1,65 @@
+/*
+ * docc_rocm_target.h - C ABI of the `rocm` target library (libdocc_rocm_target.so):
+ * SDFG (de)serialisation, scheduling for the rocm target, host-code generation
+ * and the compile/link driver.
+ *
+ * It exposes, over plain strings, the steps the reference's Python driver
+ * performs on a `StructuredSDFG` through its pybind11 module
+ * (python/bindings/py_structured_sdfg.cpp:124-560: validate, schedule(target),
+ * _compile; python/bindings/bindings.cpp:136-160,483-487) and is what a
+ * `register_target_overrides("rocm", schedule_fn, compile_fn)` hook
+ * (python/docc/python/target_registry.py:4-42) calls into.
+ *
+ * SDFGs travel as JSON text. Functions returning `char*` return a
+ * malloc'ed NUL-terminated string that the caller releases with
+ * docc_rocm_target_free, or NULL on failure with the message available from
+ * docc_rocm_target_last_error() on the calling thread.
+ */
+#ifndef DOCC_ROCM_TARGET_H
+#define DOCC_ROCM_TARGET_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Registers the rocm plugin's serializers and dispatchers (idempotent). Counterpart of
+ * register_cuda_plugin() (reference opt/include/sdfg/targets/cuda/plugin.h:20-105) being called
+ * from the module initialiser (python/bindings/bindings.cpp:51-60). Returns 0. */
+int docc_rocm_target_register(void);
+
+/* JSON array of the registered "<code>::<implementation type>" dispatcher keys. */
+char* docc_rocm_target_dispatcher_keys(void);
+
+/* Parses and validates an SDFG; returns its canonical JSON. Counterpart of
+ * StructuredSDFG.parse + validate (reference bindings.cpp:136-160). */
+char* docc_rocm_target_validate(const char* sdfg_json);
+
+/* Runs the rocm scheduling passes (node mapping, offloading, transfer minimisation) and
+ * returns the scheduled SDFG. `options_json` may be NULL or an object with
+ * "offload": "function" | "node" | "none" and "require_all_mapped": bool.
+ * Counterpart of PyStructuredSDFG::schedule (reference py_structured_sdfg.cpp:320-347). */
+char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, const char* options_json);
+
+/* Generates <output_dir>/<name>.h and <name>.cpp and returns a JSON report:
+ * {"header": path, "source": path, "function": definition, "instrumentation": [...]}.
+ * Counterpart of CPPCodeGenerator::generate + as_source (reference py_structured_sdfg.cpp:355-420). */
+char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir);
+
+/* generate + compile + link into <output_dir>/lib<name>.so against `runtime_lib_dir`/libdocc_rt_rocm.so
+ * with headers from `include_dir`; returns the library path. The compiler is
+ * $DOCC_CXX, else ROCm's clang++, invoked through std::system like the reference's JIT step
+ * (py_structured_sdfg.cpp:456,485,516-551: -c -fPIC -O3 -march=native -mtune=native -funroll-loops, then -shared). */
+char* docc_rocm_target_compile(const char* sdfg_json, const char* output_dir, const char* include_dir,
+                               const char* runtime_lib_dir);
+
+/* JSON object counting the library nodes per "<code>::<implementation type>" plus transfers,
+ * the analogue of loop_report() (reference py_structured_sdfg.cpp:570-583). */
+char* docc_rocm_target_report(const char* sdfg_json);
+
+void docc_rocm_target_free(char* text);
+const char* docc_rocm_target_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DOCC_ROCM_TARGET_H */

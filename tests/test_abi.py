@@ -1,0 +1,78 @@
+"""The C-ABI libraries load on a machine without a GPU and export every symbol the public
+headers declare; no compute entry point is called here."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+INCLUDE = ROOT / "include"
+
+
+def declared_functions(header: Path):
+    text = re.sub(r"/\*.*?\*/", "", header.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(docc_rocm_\w+)\s*\(", text)))
+
+
+def test_runtime_library_exports_every_declared_symbol():
+    from docc_amd import runtime
+
+    lib = ctypes.CDLL(str(runtime.LIB_PATH))
+    declared = declared_functions(INCLUDE / "docc_rocm_rt.h") + declared_functions(INCLUDE / "docc_rocm_ops.h")
+    assert len(declared) >= 35
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
+    # and the Python binding covers exactly the declared set
+    assert sorted(runtime.EXPORTED_SYMBOLS) == sorted(declared)
+
+
+def test_target_library_exports_every_declared_symbol():
+    import docc_amd.sdfg as sdfg
+
+    lib = ctypes.CDLL(str(sdfg._TARGET_LIB))
+    declared = declared_functions(INCLUDE / "docc_rocm_target.h")
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/ but not exported"
+    assert sorted(sdfg.EXPORTED_SYMBOLS) == sorted(declared)
+
+
+def test_kernel_images_are_built():
+    from docc_amd import build, runtime
+
+    for family in build.KERNEL_FAMILIES:
+        assert (runtime.LIB_DIR / f"docc_rocm_{family}.hsaco").exists(), family
+    # the runtime's image list and the build's family list name the same files
+    src = (ROOT / "docc_amd" / "csrc" / "rt" / "runtime.cpp").read_text()
+    listed = set(re.findall(r'"docc_rocm_(\w+)\.hsaco"', src))
+    assert listed == set(build.KERNEL_FAMILIES)
+
+
+def test_runtime_reports_errors_without_a_gpu_or_with_bad_arguments():
+    import torch
+
+    from docc_amd import runtime
+
+    assert runtime.version().startswith("docc-rocm")
+    assert runtime.take_failure() == (0, "")
+    if torch.cuda.is_available():
+        pytest.skip("error paths below are for a machine without a GPU")
+    assert runtime.device_count() == 0
+    with pytest.raises(runtime.RocmRuntimeError) as e:
+        runtime.init(0)
+    assert e.value.code == -4 and "no HIP device" in str(e.value)
+    # argument validation comes before any device work
+    with pytest.raises(runtime.RocmRuntimeError) as e:
+        runtime.sgemm(4, 4, 4, 1.0, 1, 2, 1, 4, 0.0, 1, 4)
+    assert e.value.code == -1
+    with pytest.raises(runtime.RocmRuntimeError):
+        runtime.attention_bf16(1, 1, 8, 8, 128, 0.1, 16, 16, 16, 16)
+    # there is no CPU fallback: a well-formed call fails loudly when no device is present
+    with pytest.raises(runtime.RocmRuntimeError):
+        runtime.softmax_f32(4, 4, 16, 16)
+    # the failure channel of generated code keeps the first report
+    runtime.lib().docc_rocm_report_failure(b"f", b"docc_rocm_malloc(...)", 2)
+    runtime.lib().docc_rocm_report_failure(b"g", b"later", 3)
+    code, message = runtime.take_failure()
+    assert code == 2 and "docc_rocm_malloc" in message
+    assert runtime.take_failure() == (0, "")

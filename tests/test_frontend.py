@@ -1,0 +1,246 @@
+"""`@native` and the torch front end up to (not including) execution: lowering to library nodes,
+argument order of the generated function, the compile cache rule, target-registry hooks. Modelled
+on the reference's python/tests/python/program/test_caching.py:6-57 and
+python/tests/python/targets/test_overrides.py:9-72."""
+import math
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+import docc_amd.torch as docc_torch
+from docc_amd.python import (conv2d, native, register_target, register_target_overrides, softmax, unregister_target)
+
+
+@pytest.fixture(autouse=True)
+def tmp_docc(tmp_path, monkeypatch):
+    monkeypatch.setenv("DOCC_TMP", str(tmp_path / "docc"))
+
+
+def test_matmul_lowers_to_one_gemm_with_reference_argument_order():
+    @native(target="rocm")
+    def matmul_op(a, b):
+        return a @ b
+
+    a = np.random.rand(10, 10)
+    sdfg = matmul_op.to_sdfg(a, a)
+    # user parameters, then one shape symbol (all dims equal), then the output pointer
+    assert sdfg.arguments == ["a", "b", "_s0", "_docc_ret_0"]
+    assert sdfg.name == "matmul_op_sdfg"
+    (node,) = sdfg.library_nodes()
+    assert node["code"] == "GEMM" and node["precision"] == ord("d") and node["m"] == node["n"] == node["k"] == "_s0"
+    sdfg = matmul_op.to_sdfg(np.zeros((5, 7), np.float32), np.zeros((7, 3), np.float32))
+    assert sdfg.arguments == ["a", "b", "_s0", "_s1", "_s2", "_docc_ret_0"]
+    node = sdfg.library_nodes()[0]
+    assert (node["precision"], node["m"], node["n"], node["k"], node["lda"], node["ldb"], node["ldc"]) == (ord("s"), "_s0", "_s2", "_s1", "_s1", "_s2", "_s2")
+
+
+def test_other_matmul_spellings_and_polybench_gemm():
+    @native
+    def np_matmul(a, b):
+        return np.matmul(a, b)
+
+    @native
+    def dot_t(a, b):
+        return np.dot(a, b.T)
+
+    @native
+    def gemm(alpha, beta, C, A, B):
+        C[:] = alpha * A @ B + beta * C
+
+    @native
+    def into_arg(A, B, C):
+        C = A @ B
+
+    a = np.zeros((6, 6))
+    assert np_matmul.to_sdfg(a, a).library_nodes()[0]["code"] == "GEMM"
+    assert dot_t.to_sdfg(a, a).library_nodes()[0]["trans_b"] == 112
+    sdfg = gemm.to_sdfg(1.5, 1.2, a, a, a)
+    assert sdfg.arguments == ["alpha", "beta", "C", "A", "B", "_s0"]     # in place: no return buffer
+    df = sdfg._data["root"]["children"][0]["dataflow"]
+    binds = {b["connector"]: b.get("data") for b in df["inputs"]}
+    assert binds == {"__A": "A", "__B": "B", "__C": "C", "__alpha": "alpha", "__beta": "beta"}
+    assert len(sdfg.library_nodes()) == 1                                  # exactly one GEMM node, no loops
+    assert into_arg.to_sdfg(a, a, a).arguments == ["A", "B", "C", "_s0"]
+
+
+def test_softmax_forms_and_conv():
+    @native
+    def sp(x):
+        return scipy.special.softmax(x, axis=-1)
+
+    @native
+    def decomposed(x):
+        tmp_max = np.max(x, axis=-1, keepdims=True)
+        tmp_out = np.exp(x - tmp_max)
+        tmp_sum = np.sum(tmp_out, axis=-1, keepdims=True)
+        return tmp_out / tmp_sum
+
+    @native
+    def conv(x, w, b):
+        return conv2d(x, w, b, stride=1, padding=1)
+
+    x = np.zeros((4, 3, 8, 8), np.float32)
+    for prog in (sp, decomposed):
+        (node,) = prog.to_sdfg(x).library_nodes()
+        assert node["code"] == "ml::Softmax" and node["axes"] == [-1] and node["shape"] == ["_s0", "_s1", "_s2", "_s2"]
+    (node,) = conv.to_sdfg(x, np.zeros((5, 3, 3, 3), np.float32), np.zeros(5, np.float32)).library_nodes()
+    assert node["code"] == "ml::Conv" and node["pads"] == ["1", "1", "1", "1"] and node["has_bias"] is True
+    # the marker functions compute the same thing in plain numpy
+    y = np.random.rand(3, 7).astype(np.float32)
+    assert np.allclose(softmax(y), scipy.special.softmax(y, axis=-1))
+    xs, ws = np.random.rand(1, 2, 5, 5), np.random.rand(3, 2, 3, 3)
+    ref = torch.nn.functional.conv2d(torch.from_numpy(xs), torch.from_numpy(ws), padding=1).numpy()
+    assert np.allclose(conv2d(xs, ws, padding=1), ref)
+
+
+def test_unsupported_code_is_rejected_not_run_on_the_cpu():
+    @native
+    def loop(a, b):
+        for i in range(a.shape[0]):
+            b[i] = a[i]
+
+    @native
+    def add(a, b):
+        return a + b
+
+    a = np.zeros(4)
+    with pytest.raises(NotImplementedError, match="rocm target"):
+        loop.to_sdfg(a, a)
+    with pytest.raises(NotImplementedError):
+        add.to_sdfg(a, a)
+
+
+def test_compile_cache_follows_shape_structure():
+    @native
+    def mm(a, b):
+        return a @ b
+
+    c1 = mm.compile(np.random.rand(16, 16), np.random.rand(16, 16))
+    c2 = mm.compile(np.random.rand(32, 32), np.random.rand(32, 32))   # same structure, other values
+    assert c1 is c2
+    c3 = mm.compile(np.random.rand(16, 8), np.random.rand(8, 16))     # different structure
+    assert c3 is not c1 and c3.sdfg.arguments == ["a", "b", "_s0", "_s1", "_docc_ret_0"]
+    c4 = mm.compile(np.zeros((16, 16), np.float32), np.zeros((16, 16), np.float32))   # different dtype
+    assert c4 is not c1
+    assert c1.get_return_shape(np.zeros((5, 5)), np.zeros((5, 5))) == (5, 5)
+
+
+def test_target_overrides_are_consulted(capsys):
+    calls = []
+
+    def schedule(sdfg, category, options):
+        calls.append(("schedule", category, sorted(options)))
+        sdfg.schedule("rocm", category, False, {"offload": "node"})
+
+    def schedule_legacy(sdfg, category):
+        calls.append(("legacy", category))
+        sdfg.schedule("rocm", category, False)
+
+    def compile_(sdfg, out_dir, inst_mode, capture, options):
+        calls.append(("compile", inst_mode, capture))
+        return sdfg._compile(out_dir, "rocm", inst_mode, capture)
+
+    register_target_overrides("special", schedule, compile_)
+    register_target("special_legacy", schedule_legacy)
+    try:
+        @native(target="special", category="desktop")
+        def f(a, b):
+            return a @ b
+
+        @native(target="special_legacy")
+        def g(a, b):
+            return a @ b
+
+        a = np.zeros((4, 4), np.float32)
+        f.compile(a, a)
+        g.compile(a, a)
+        out = capsys.readouterr().out
+        assert "is not supported" not in out
+        assert calls == [("schedule", "desktop", ["remote_tuning"]), ("compile", "", False), ("legacy", "server")]
+        assert f.last_sdfg.library_nodes()[0]["implementation_type"] == "ROCMWithTransfers"
+    finally:
+        unregister_target("special")
+        unregister_target("special_legacy")
+
+    @native(target="openmp")
+    def h(a, b):
+        return a @ b
+
+    with pytest.raises(NotImplementedError):
+        h.compile(np.zeros((4, 4)), np.zeros((4, 4)))
+    assert "Target 'openmp' is not supported" in capsys.readouterr().out
+
+
+class Attn(torch.nn.Module):
+    def forward(self, q, k, v):
+        s = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(q.shape[-1])
+        return torch.matmul(torch.softmax(s, dim=-1), v)
+
+
+def test_torch_lowering_recognises_attention_conv_and_matmul():
+    q = torch.randn(2, 4, 128, 64).bfloat16()
+    sdfg = docc_torch.TorchProgram(Attn(), (q, q, q), target="rocm").to_sdfg()
+    assert sdfg.name == "__docc_Attn" and sdfg.arguments == ["q", "k", "v", "_docc_ret_0"]
+    (node,) = sdfg.library_nodes()
+    assert node["code"] == "ml::Attention" and float(node["scale"]) == 0.125 and node["shape_q"] == ["2", "4", "128", "64"]
+    assert sdfg.metadata("return_shape") == "[2,4,128,64]"
+
+    class Sdpa(torch.nn.Module):
+        def forward(self, q, k, v):
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v)
+
+    assert docc_torch.TorchProgram(Sdpa(), (q, q, q), target="rocm").to_sdfg().library_nodes()[0]["code"] == "ml::Attention"
+
+    class Conv(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.conv = torch.nn.Conv2d(8, 16, 3, padding=1)
+
+        def forward(self, x):
+            return self.conv(x)
+
+    sdfg = docc_torch.compile_torch(Conv(), torch.randn(2, 8, 14, 14), target="rocm").to_sdfg()
+    assert sdfg.arguments == ["x", "conv_weight", "conv_bias", "_docc_ret_0"]
+    assert sdfg.library_nodes()[0]["pads"] == ["1", "1", "1", "1"]
+
+    class MM(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.softmax(a @ b.t(), dim=-1)
+
+    sdfg = docc_torch.TorchProgram(MM(), (torch.randn(8, 6), torch.randn(5, 6)), target="rocm").to_sdfg()
+    assert [n["code"] for n in sdfg.library_nodes()] == ["GEMM", "ml::Softmax"] and sdfg.library_nodes()[0]["trans_b"] == 112
+
+    class Unsupported(torch.nn.Module):
+        def forward(self, a):
+            return torch.relu(a)
+
+    with pytest.raises(NotImplementedError):
+        docc_torch.TorchProgram(Unsupported(), torch.randn(4), target="rocm").to_sdfg()
+
+
+def test_torch_backend_is_registered_and_reads_global_options():
+    import torch._dynamo
+
+    assert "docc" in torch._dynamo.list_backends(None)
+    docc_torch.set_backend_options(target="rocm", category="server")
+    assert docc_torch._backend_options == {"target": "rocm", "category": "server"}
+    captured = {}
+
+    def schedule(sdfg, category, options):
+        captured["options"] = options
+        sdfg.schedule("rocm", category, False, options)
+
+    register_target_overrides("probe", schedule, None)
+    try:
+        docc_torch.set_backend_options(target="probe")
+        program = docc_torch.TorchProgram(Attn(), None, target="probe")
+        q = torch.randn(1, 1, 64, 64).bfloat16()
+        compiled = program.compile(q, q, q)
+        assert captured["options"] == {"offload": "function"}      # CPU tensors: the generated code moves the data
+        assert program.last_sdfg.loop_report()["H2D"] == 3 and program.last_sdfg.loop_report()["D2H"] == 1
+        assert program.compile(q, q, q) is compiled                 # cached per shapes/dtypes/device
+    finally:
+        unregister_target("probe")
+        docc_torch.set_backend_options(target="rocm")

@@ -1,0 +1,170 @@
+"""End to end on the GPU through the reference's entry points: `@native(target="rocm")` and
+`torch.compile(model, backend="docc")`, compared with the CPU oracle. These tests read like the
+reference's own (python/tests/python/functions/numpy/test_linalg.py:5-24,
+python/benchmarks/npbench/polybench/test_gemm.py:23-89, .../deep_learning/softmax/test_softmax.py:24-84,
+mlir/integration/torch/test_matmul.py, test_conv2d.py) with the target switched to rocm.
+
+Tolerances (norm-wise relative error): fp64 1e-12, fp32 1e-5, bf16 2e-2."""
+import math
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+import docc_amd.torch as docc_torch
+import oracle
+from docc_amd.python import conv2d, native
+from gpu_util import rel_err_max
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(autouse=True)
+def tmp_docc(tmp_path, monkeypatch):
+    monkeypatch.setenv("DOCC_TMP", str(tmp_path / "docc"))
+    docc_torch.set_backend_options(target="rocm", category="server")
+
+
+def bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def test_native_matmul_config_1():
+    @native(target="rocm")
+    def matmul(A, B):
+        return A @ B
+
+    rng = np.random.default_rng(0)
+    A, B = rng.random((1000, 1000)), rng.random((1000, 1000))
+    C = matmul(A, B)
+    assert C.dtype == np.float64 and C.shape == (1000, 1000) and C.flags.c_contiguous
+    assert rel_err_max(C, oracle.gemm(A, B, variant="ld")) <= 1e-12
+    # second call: cached program, other values and size
+    A2, B2 = rng.random((37, 37)), rng.random((37, 37))
+    assert rel_err_max(matmul(A2, B2), oracle.gemm(A2, B2, variant="ld")) <= 1e-12
+    assert len(matmul.cache) == 1
+
+
+@pytest.mark.parametrize("offload", ["function", "node"])
+def test_native_polybench_gemm(offload):
+    @native(target="rocm", offload=offload)
+    def gemm(alpha, beta, C, A, B):
+        C[:] = alpha * A @ B + beta * C
+
+    rng = np.random.default_rng(42)
+    NI, NJ, NK = 100, 110, 120     # non-square, like the reference benchmark's S size scaled down
+    A, B, C = rng.random((NI, NK)), rng.random((NK, NJ)), rng.random((NI, NJ))
+    ref = oracle.gemm(A, B, C, alpha=1.5, beta=1.2)
+    gemm(1.5, 1.2, C, A, B)
+    assert rel_err_max(C, ref) <= 1e-12
+    report = gemm.last_sdfg.loop_report()
+    assert report["GEMM"] == 1     # exactly one GEMM node, as the reference's harness expects on every target
+
+
+def test_native_softmax_like_the_reference_benchmark():
+    @native(target="rocm")
+    def softmax(x):
+        tmp_max = np.max(x, axis=-1, keepdims=True)
+        tmp_out = np.exp(x - tmp_max)
+        tmp_sum = np.sum(tmp_out, axis=-1, keepdims=True)
+        return tmp_out / tmp_sum
+
+    rng = np.random.default_rng(42)
+    x = rng.random((16, 16, 128, 128), dtype=np.float32)      # size "S" of the reference benchmark
+    y = softmax(x)
+    assert y.dtype == np.float32 and y.shape == x.shape
+    assert rel_err_max(y, oracle.softmax(x)) <= 1e-5
+    np.testing.assert_allclose(y, scipy.special.softmax(x.astype(np.float64), axis=-1), rtol=1e-5, atol=1e-8)
+
+
+def test_native_chain_keeps_the_intermediate_on_the_device():
+    @native(target="rocm")
+    def chain(a, b, x):
+        t = a @ b
+        return scipy.special.softmax(t @ x, axis=-1)
+
+    rng = np.random.default_rng(3)
+    a, b, x = (rng.standard_normal((96, 96)).astype(np.float32) * 0.2 for _ in range(3))
+    y = chain(a, b, x)
+    ref = oracle.softmax(oracle.gemm(oracle.gemm(a, b), x))
+    assert rel_err_max(y, ref) <= 1e-4    # two chained fp32 products feed an exponential
+    r = chain.last_sdfg.loop_report()
+    assert r["H2D"] == 3 and r["D2H"] == 1
+
+
+def test_native_conv():
+    @native(target="rocm")
+    def conv(x, w, b):
+        return conv2d(x, w, b, stride=1, padding=1)
+
+    g = np.load(__import__("pathlib").Path(__file__).parent / "golden" / "conv_2x3x7x7_k3_p1_bias_f32.npz")
+    y = conv(g["X"], g["W"], g["b"])
+    assert y.shape == (2, 4, 7, 7)
+    assert rel_err_max(y, g["Y"]) <= 1e-5
+    assert rel_err_max(y, oracle.conv2d(g["X"], g["W"], g["b"], pad=(1, 1))) <= 1e-5
+
+
+class Attn(torch.nn.Module):
+    def forward(self, q, k, v):
+        s = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(q.shape[-1])
+        return torch.matmul(torch.softmax(s, dim=-1), v)
+
+
+def test_torch_compile_attention_config_4():
+    torch.manual_seed(3)
+    Q, K, V = (torch.randn(8, 16, 2048, 64).bfloat16() for _ in range(3))
+    model = torch.compile(Attn(), backend="docc")
+    out = model(Q.cuda(), K.cuda(), V.cuda())
+    assert out.device.type == "cuda" and out.dtype == torch.bfloat16 and out.shape == (8, 16, 2048, 64)
+    O = out.float().cpu().numpy()
+    assert np.isfinite(O).all()
+    for (b, h) in [(0, 0), (5, 9)]:
+        ref = oracle.attention(bits(Q[b:b + 1, h:h + 1, 512:576]), bits(K[b:b + 1, h:h + 1]), bits(V[b:b + 1, h:h + 1]))
+        assert rel_err_max(O[b, h, 512:576], ref[0, 0]) <= 2e-2
+
+
+def test_torch_compile_attention_cpu_tensors_and_golden():
+    g = np.load(__import__("pathlib").Path(__file__).parent / "golden" / "attn_1x2x96x64_bf16.npz")
+    to_t = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    model = torch.compile(Attn(), backend="docc")
+    out = model(to_t(g["Q"]), to_t(g["K"]), to_t(g["V"]))      # CPU tensors: generated code does the transfers
+    assert out.device.type == "cpu"
+    assert rel_err_max(out.float().numpy(), g["O"]) <= 2e-2
+
+
+def test_torch_compile_conv_config_5():
+    torch.manual_seed(4)
+    conv = torch.nn.Conv2d(64, 64, 3, stride=1, padding=1, bias=True)
+    torch.nn.init.kaiming_normal_(conv.weight)
+    with torch.no_grad():
+        conv.bias.copy_(torch.randn(64) * 0.1)
+    X = torch.randn(32, 64, 56, 56)
+    program = docc_torch.compile_torch(conv.cuda(), X.cuda(), target="rocm")
+    Y = program(X.cuda())
+    assert Y.shape == (32, 64, 56, 56) and Y.device.type == "cuda"
+    ref = oracle.conv2d(X[:2].numpy(), conv.weight.detach().cpu().numpy(), conv.bias.detach().cpu().numpy(), pad=(1, 1))
+    assert rel_err_max(Y[:2].cpu().numpy(), ref) <= 1e-5
+
+
+def test_torch_backend_matmul_softmax_fp32():
+    class MM(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.softmax(a @ b, dim=-1)
+
+    torch.manual_seed(815)      # the seed of the reference's torch integration tests
+    a, b = torch.randn(64, 48), torch.randn(48, 80)
+    model = torch.compile(MM(), backend="docc")
+    res = model(a.cuda(), b.cuda())
+    assert isinstance(res, torch.Tensor)
+    ref = oracle.softmax(oracle.gemm(a.numpy(), b.numpy()))
+    assert rel_err_max(res.cpu().numpy(), ref) <= 1e-5
+
+    class BMM(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.matmul(a, b)
+
+    a3, b3 = torch.randn(4, 20, 30, dtype=torch.float64), torch.randn(4, 30, 10, dtype=torch.float64)
+    out = docc_torch.compile_torch(BMM(), (a3, b3), target="rocm")(a3, b3)   # batched: ml::MatMul
+    refs = np.stack([oracle.gemm(a3[i].numpy(), b3[i].numpy(), variant="ld") for i in range(4)])
+    assert rel_err_max(out.numpy(), refs) <= 1e-12

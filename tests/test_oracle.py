@@ -1,0 +1,173 @@
+"""Pins the CPU oracle (oracle/docc_oracle.c) without the reference, which holds no numeric
+fixtures for these nodes: committed golden vectors (closed forms evaluated in float64 by
+tests/golden/make_golden.py), library cross-checks (numpy.matmul, scipy.special.softmax, torch
+conv2d / scaled_dot_product_attention in float64) and closed-form cases chosen so that a dropped
+term, a wrong index or a transposed operand fails at least one of them."""
+from pathlib import Path
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+import oracle
+
+GOLDEN = Path(__file__).resolve().parent / "golden"
+N, T = oracle.NO_TRANS, oracle.TRANS
+
+
+def rel(y, ref):
+    return float(np.abs(np.asarray(y, np.float64) - ref).max() / np.abs(ref).max())
+
+
+# ---- GEMM -----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("tag", ["f64", "f32"])
+def test_gemm_golden(tag):
+    g = np.load(GOLDEN / f"gemm_int_17x33x65_{tag}.npz")
+    for variant in ("blas", "expanded"):
+        assert np.array_equal(oracle.gemm(g["A"], g["B"], variant=variant), g["C"])
+        assert np.array_equal(oracle.gemm(g["A"], g["B"], g["C0"], alpha=2.0, beta=-3.0, variant=variant), g["C_alpha2_beta_m3"])
+    # transposed storage gives the same product
+    assert np.array_equal(oracle.gemm(g["A"].T.copy(), g["B"], trans_a=T), g["C"])
+    assert np.array_equal(oracle.gemm(g["A"], g["B"].T.copy(), trans_b=T), g["C"])
+    assert np.array_equal(oracle.gemm(g["A"].T.copy(), g["B"].T.copy(), trans_a=T, trans_b=T), g["C"])
+
+
+def test_gemm_bf16_golden():
+    g = np.load(GOLDEN / "gemm_int_17x33x65_bf16.npz")
+    assert np.array_equal(oracle.gemm_bf16(g["A"], g["B"]), g["C"])
+    assert np.array_equal(oracle.gemm_bf16(g["A"].T.copy(), g["B"].T.copy(), trans_a=T, trans_b=T), g["C"])
+
+
+def test_gemm_against_numpy_and_structure():
+    rng = np.random.default_rng(0)
+    A, B = rng.random((37, 91)), rng.random((91, 23))
+    ref = A @ B
+    assert rel(oracle.gemm(A, B), ref) <= 1e-14
+    assert rel(oracle.gemm(A, B, variant="ld"), ref) <= 1e-14
+    Af, Bf = A.astype(np.float32), B.astype(np.float32)
+    assert rel(oracle.gemm(Af, Bf), Af.astype(np.float64) @ Bf.astype(np.float64)) <= 1e-5
+    assert rel(oracle.gemm(Af, Bf, variant="acc64"), Af.astype(np.float64) @ Bf.astype(np.float64)) <= 1e-7
+    # non-commutativity: a transposed-operand mistake cannot pass
+    assert rel(oracle.gemm(A, B), (B.T @ A.T).T) <= 1e-14
+    eye = np.eye(23)
+    assert np.array_equal(oracle.gemm(B, eye), B)
+    # rank-1 outer product and row sums
+    u, v = rng.random((9, 1)), rng.random((1, 13))
+    assert np.array_equal(oracle.gemm(u, v), u * v)
+    assert rel(oracle.gemm(A, np.ones((91, 1))), A.sum(axis=1, keepdims=True)) <= 1e-14
+
+
+def test_gemm_beta_semantics():
+    rng = np.random.default_rng(1)
+    A, B = rng.random((5, 6)), rng.random((6, 4))
+    nan = np.full((5, 4), np.nan)
+    # cblas semantics: beta == 0 does not read C; the reference's expansion multiplies it (NaN * 0 = NaN)
+    assert np.isfinite(oracle.gemm(A, B, nan, beta=0.0, variant="blas")).all()
+    assert np.isnan(oracle.gemm(A, B, nan, beta=0.0, variant="expanded")).all()
+    # k == 0: C = beta * C
+    C0 = rng.random((5, 4))
+    assert np.allclose(oracle.gemm(np.zeros((5, 0)), np.zeros((0, 4)), C0, beta=2.0), 2 * C0)
+
+
+def test_bf16_conversion_matches_torch_exhaustively_on_a_sweep():
+    # every bf16 value and the float32 values half-way and just around them
+    hi = np.arange(0, 1 << 16, dtype=np.uint32) << 16
+    for lo in (0x0000, 0x7FFF, 0x8000, 0x8001, 0xFFFF):
+        bits = (hi | lo).astype(np.uint32)
+        x = bits.view(np.float32)
+        keep = ~np.isnan(x)
+        want = torch.from_numpy(x[keep]).bfloat16().view(torch.int16).numpy().view(np.uint16)
+        assert np.array_equal(oracle.f32_to_bf16(x[keep]), want)
+    b = np.arange(0, 1 << 16, dtype=np.uint16)
+    back = oracle.bf16_to_f32(b)
+    assert np.array_equal(back.view(np.uint32), b.astype(np.uint32) << 16)
+
+
+# ---- softmax --------------------------------------------------------------------------
+
+@pytest.mark.parametrize("variant", ["numpy", "expanded"])
+def test_softmax_golden_and_scipy(variant):
+    g = np.load(GOLDEN / "softmax_8x257_f32.npz")
+    Y = oracle.softmax(g["X"], variant=variant)
+    assert rel(Y, g["Y"]) <= 1e-6
+    rng = np.random.default_rng(5)
+    X = (rng.standard_normal((3, 5, 64)) * 8).astype(np.float32)
+    assert rel(oracle.softmax(X, variant=variant), scipy.special.softmax(X.astype(np.float64), axis=-1)) <= 1e-6
+
+
+def test_softmax_closed_forms():
+    X = np.full((3, 10), 2.5, np.float32)
+    assert np.allclose(oracle.softmax(X), 0.1, rtol=1e-6)
+    rng = np.random.default_rng(2)
+    X = (rng.standard_normal((4, 33)) * 8).astype(np.float32)
+    Y = oracle.softmax(X)
+    assert np.allclose(Y.sum(axis=-1), 1.0, atol=1e-6)
+    assert np.array_equal(Y.argmax(axis=-1), X.argmax(axis=-1))
+    assert np.allclose(oracle.softmax(X + np.float32(16.0)), Y, rtol=1e-4, atol=1e-12)
+    big = np.array([[1000.0, 0.0, -1000.0]], np.float32)   # max subtraction: no overflow
+    assert np.array_equal(oracle.softmax(big), np.array([[1.0, 0.0, 0.0]], np.float32))
+    assert oracle.softmax(np.zeros((0, 7), np.float32)).shape == (0, 7)
+
+
+# ---- conv -----------------------------------------------------------------------------
+
+def test_conv_golden():
+    g = np.load(GOLDEN / "conv_2x3x7x7_k3_p1_bias_f32.npz")
+    assert rel(oracle.conv2d(g["X"], g["W"], g["b"], pad=(1, 1)), g["Y"]) <= 1e-6
+
+
+@pytest.mark.parametrize("stride,pad,dil", [((1, 1), (0, 0), (1, 1)), ((2, 1), (1, 2), (1, 1)), ((1, 1), (2, 2), (2, 2)), ((3, 2), (0, 1), (1, 2))])
+def test_conv_against_torch(stride, pad, dil):
+    g = torch.Generator().manual_seed(7)
+    x, w, b = torch.randn(2, 3, 11, 9, generator=g), torch.randn(5, 3, 3, 2, generator=g), torch.randn(5, generator=g)
+    ref = torch.nn.functional.conv2d(x.double(), w.double(), b.double(), stride=stride, padding=pad, dilation=dil).numpy()
+    Y = oracle.conv2d(x.numpy(), w.numpy(), b.numpy(), stride, pad, dil)
+    assert Y.shape == ref.shape
+    assert rel(Y, ref) <= 1e-6
+    assert rel(oracle.conv2d(x.numpy(), w.numpy(), None, stride, pad, dil), ref - b.double().numpy()[None, :, None, None]) <= 1e-6
+
+
+def test_conv_closed_forms():
+    # all-ones input and kernel: the output counts the taps inside the image (zero padding)
+    Y = oracle.conv2d(np.ones((1, 2, 5, 5), np.float32), np.ones((1, 2, 3, 3), np.float32), pad=(1, 1))
+    assert Y[0, 0, 0, 0] == 8 and Y[0, 0, 0, 2] == 12 and Y[0, 0, 2, 2] == 18
+    # a delta kernel shifts the image
+    X = np.arange(2 * 1 * 4 * 4, dtype=np.float32).reshape(2, 1, 4, 4)
+    W = np.zeros((1, 1, 3, 3), np.float32)
+    W[0, 0, 1, 1] = 1
+    assert np.array_equal(oracle.conv2d(X, W, pad=(1, 1)), X)
+    W[:] = 0
+    W[0, 0, 2, 1] = 1   # reads X[h+1, w]
+    exp = np.zeros_like(X)
+    exp[:, :, :-1, :] = X[:, :, 1:, :]
+    assert np.array_equal(oracle.conv2d(X, W, pad=(1, 1)), exp)
+    # output extent formula of the reference (conv_node.cpp:224-233)
+    assert oracle.conv_out_dim(56, 1, 1, 3, 1) == 56 and oracle.conv_out_dim(7, 0, 2, 3, 2) == 2 and oracle.conv_out_dim(2, 0, 1, 3, 1) == 0
+
+
+# ---- attention ------------------------------------------------------------------------
+
+def test_attention_golden_and_torch():
+    g = np.load(GOLDEN / "attn_1x2x96x64_bf16.npz")
+    assert rel(oracle.attention(g["Q"], g["K"], g["V"], 0.125), g["O"]) <= 1e-5
+    gen = torch.Generator().manual_seed(11)
+    q, k, v = (torch.randn(2, 2, 40, 64, generator=gen).bfloat16() for _ in range(3))
+    bits = lambda t: t.view(torch.int16).numpy().view(np.uint16)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double()).numpy()
+    assert rel(oracle.attention(bits(q), bits(k), bits(v)), ref) <= 1e-5
+
+
+def test_attention_closed_forms():
+    gen = torch.Generator().manual_seed(12)
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    q, v = torch.randn(1, 1, 9, 64, generator=gen).bfloat16(), torch.randn(1, 1, 20, 64, generator=gen).bfloat16()
+    k = torch.randn(1, 1, 1, 64, generator=gen).bfloat16().expand(1, 1, 20, 64)
+    O = oracle.attention(bits(q), bits(k), bits(v))
+    assert rel(O, np.broadcast_to(v.double().mean(dim=2, keepdim=True).numpy(), O.shape)) <= 1e-5
+    k = torch.randn(1, 1, 20, 64, generator=gen).bfloat16()
+    perm = torch.randperm(20, generator=gen)
+    a = oracle.attention(bits(q), bits(k), bits(v))
+    b = oracle.attention(bits(q), bits(k[:, :, perm]), bits(v[:, :, perm]))
+    assert rel(a, b.astype(np.float64)) <= 1e-5

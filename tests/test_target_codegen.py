@@ -1,0 +1,235 @@
+"""The rocm target's C++ side, driven through its C ABI: SDFG (de)serialisation with the
+reference's node payload keys, the "<code>::<implementation type>" dispatcher registry, the node
+mapper, the offloading transform with transfer minimisation, and the emitted host C++ (checked
+as text, the way the reference tests its dispatchers: opt/tests/cuda/cuda_library_nodes_test.cpp:513-651)."""
+import ctypes
+import json
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from docc_amd import runtime
+from docc_amd.sdfg import (InvalidSDFGException, Pointer, PrimitiveType, Scalar, StructuredSDFG, StructuredSDFGBuilder,
+                           registered_dispatchers)
+
+F64, F32, BF16, I64 = (Pointer(Scalar(PrimitiveType.Double)), Pointer(Scalar(PrimitiveType.Float)),
+                       Pointer(Scalar(PrimitiveType.BFloat)), Scalar(PrimitiveType.Int64))
+
+
+def gemm_sdfg(ptr=F64, name="matmul_sdfg"):
+    b = StructuredSDFGBuilder(name)
+    b.add_container("A", ptr, True)
+    b.add_container("B", ptr, True)
+    b.add_container("_s0", I64, True)
+    b.add_container("_docc_ret_0", F32 if ptr is BF16 else ptr, True)
+    b.add_gemm("A", "B", "_docc_ret_0", "1.0", "0.0", "_s0", "_s0", "_s0")
+    return b.move()
+
+
+def source_of(sdfg, tmp_path):
+    report = sdfg.generate(str(tmp_path))
+    return Path(report["source"]).read_text(), report
+
+
+def test_registry_holds_every_rocm_key():
+    keys = registered_dispatchers()
+    for code in ("GEMM", "ml::MatMul", "ml::Softmax", "ml::Conv", "ml::Attention"):
+        assert f"{code}::ROCMWithTransfers" in keys and f"{code}::ROCMWithoutTransfers" in keys
+    assert "ROCMOffloading::NONE" in keys
+
+
+def test_gemm_node_json_uses_the_reference_keys():
+    node = gemm_sdfg().library_nodes()[0]
+    # keys of GEMMNodeSerializer (reference gemm_node.cpp:387-405) inside the library_node envelope
+    for key in ("type", "element_id", "code", "implementation_type", "precision", "layout", "trans_a", "trans_b",
+                "m", "n", "k", "lda", "ldb", "ldc"):
+        assert key in node
+    assert node["code"] == "GEMM" and node["implementation_type"] == "BLAS"
+    assert node["precision"] == ord("d") and node["layout"] == 101 and node["trans_a"] == 111 and node["trans_b"] == 111
+    # a round trip through the native parser keeps everything
+    again = StructuredSDFG.parse(gemm_sdfg().to_json())
+    assert again.library_nodes()[0] == node and again.arguments == ["A", "B", "_s0", "_docc_ret_0"]
+
+
+def test_validation_errors():
+    b = StructuredSDFGBuilder("bad")
+    b.add_container("A", F64, True)
+    with pytest.raises(InvalidSDFGException):
+        b.add_container("A", F64, True)
+    data = json.loads(gemm_sdfg().to_json())
+    data["root"]["children"][0]["dataflow"]["inputs"][0]["data"] = "nope"
+    with pytest.raises(InvalidSDFGException, match="unknown container"):
+        StructuredSDFG.parse(json.dumps(data))
+    data = json.loads(gemm_sdfg().to_json())
+    data["root"]["children"][0]["dataflow"]["library_node"]["code"] = "Mystery"
+    with pytest.raises(InvalidSDFGException, match="No library node serializer"):
+        StructuredSDFG.parse(json.dumps(data))
+    data = json.loads(gemm_sdfg().to_json())
+    del data["root"]["children"][0]["dataflow"]["inputs"][4]
+    with pytest.raises(InvalidSDFGException, match="__beta"):
+        StructuredSDFG.parse(json.dumps(data))
+
+
+def test_unscheduled_node_has_no_dispatcher(tmp_path):
+    # the BLAS implementation type belongs to the reference's CPU path, which this target does not carry
+    with pytest.raises(InvalidSDFGException, match="No library node dispatcher found for library node code: GEMM::BLAS"):
+        gemm_sdfg().generate(str(tmp_path))
+
+
+def test_mapper_sets_implementation_types_and_declines_what_the_kernels_lack():
+    s = gemm_sdfg()
+    s.schedule("rocm", options={"offload": "node"})
+    assert s.library_nodes()[0]["implementation_type"] == "ROCMWithTransfers"
+    s = gemm_sdfg()
+    s.schedule("rocm", options={"offload": "none"})
+    assert s.library_nodes()[0]["implementation_type"] == "ROCMWithoutTransfers"
+    assert s.loop_report()["H2D"] == 0
+    # column-major GEMM is declined; with no CPU lowering that is an error, not a silent fallback
+    data = json.loads(gemm_sdfg().to_json())
+    data["root"]["children"][0]["dataflow"]["library_node"]["layout"] = 102
+    with pytest.raises(InvalidSDFGException, match="row-major"):
+        StructuredSDFG.parse(json.dumps(data)).schedule("rocm")
+    s = StructuredSDFG.parse(json.dumps(data))
+    s.schedule("rocm", options={"require_all_mapped": False})
+    assert s.library_nodes()[0]["implementation_type"] == "BLAS"
+    # softmax over a leading axis, grouped conv, head dim != 64
+    b = StructuredSDFGBuilder("s")
+    b.add_container("X", F32, True)
+    b.add_container("Y", F32, True)
+    b.add_reduce_op("softmax", "X", "Y", [4, 8], [0])
+    with pytest.raises(InvalidSDFGException, match="last axis"):
+        b.move().schedule("rocm")
+    b = StructuredSDFGBuilder("c")
+    for n in ("X", "W", "Y"):
+        b.add_container(n, F32, True)
+    b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 4, group=2)
+    with pytest.raises(InvalidSDFGException, match="group"):
+        b.move().schedule("rocm")
+    b = StructuredSDFGBuilder("a")
+    for n in ("Q", "K", "V", "O"):
+        b.add_container(n, BF16, True)
+    b.add_attention("Q", "K", "V", "O", [1, 2, 16, 128], 16, 0.1)
+    with pytest.raises(InvalidSDFGException, match="head dimension"):
+        b.move().schedule("rocm")
+    with pytest.raises(NotImplementedError):
+        gemm_sdfg().schedule("openmp")
+
+
+def test_with_transfers_dispatcher_text(tmp_path):
+    s = gemm_sdfg()
+    s.schedule("rocm", options={"offload": "node"})
+    src, report = source_of(s, tmp_path)
+    assert report["function"] == 'extern "C" void matmul_sdfg(double *A, double *B, int64_t _s0, double *_docc_ret_0)'
+    flat = re.sub(r"\s+", " ", src)
+    # connector locals, constants printed verbatim, write-back (reference block_dispatcher.cpp:333-438)
+    for piece in ("double *__A = A;", "double *__B = B;", "double *__C = _docc_ret_0;", "double __alpha = 1.0;",
+                  "double __beta = 0.0;", "_docc_ret_0 = __C;"):
+        assert piece in flat
+    # alloc x3, upload of A and B only (beta == 0: C is not read), launch, download, sync, free x3
+    assert flat.count("docc_rocm_malloc(") == 3 and flat.count("docc_rocm_free(") == 3
+    assert flat.count("docc_rocm_memcpy_h2d_async(") == 2 and flat.count("docc_rocm_memcpy_d2h_async(") == 1
+    assert "docc_rocm_dgemm(nullptr, 111, 111, _s0, _s0, _s0, __alpha, (const double *) d___A, _s0, (const double *) d___B, _s0, __beta, (double *) d___C, _s0)" in flat
+    assert flat.index("docc_rocm_memcpy_h2d_async") < flat.index("docc_rocm_dgemm") < flat.index("docc_rocm_memcpy_d2h_async") < flat.index("docc_rocm_stream_sync")
+    assert "if ((_s0) != 0 && (_s0) != 0)" in flat            # zero-size guard, as the cuBLAS dispatcher has
+    assert '#include "docc_rocm_rt.h"' in src and src.count("#define DOCC_ROCM_CHECK") == 1
+    metrics = report["instrumentation"][0]
+    assert metrics["target_type"] == "ROCM" and "flop" in metrics["metrics"] and "pcie_bytes" in metrics["metrics"]
+
+
+def test_beta_nonzero_uploads_c(tmp_path):
+    b = StructuredSDFGBuilder("gemm_acc")
+    for n in ("A", "B", "C"):
+        b.add_container(n, F32, True)
+    b.add_gemm("A", "B", "C", "1.5", "1.2", 8, 8, 8)
+    s = b.move()
+    s.schedule("rocm", options={"offload": "node"})
+    src, _ = source_of(s, tmp_path)
+    assert src.count("docc_rocm_memcpy_h2d_async(") == 3 and "docc_rocm_sgemm(" in src and "float __alpha = 1.5;" in src
+
+
+def test_bf16_gemm_text(tmp_path):
+    s = gemm_sdfg(BF16, "bf")
+    s.schedule("rocm", options={"offload": "none"})
+    src, report = source_of(s, tmp_path)
+    assert report["function"] == 'extern "C" void bf(__bf16 *A, __bf16 *B, int64_t _s0, float *_docc_ret_0)'
+    assert "docc_rocm_bf16gemm_f32(nullptr, 111, 111, _s0, _s0, _s0, __alpha, (const uint16_t *) __A" in src
+    assert "float __alpha = 1.0;" in src and "docc_rocm_malloc" not in src
+
+
+def chain_sdfg():
+    """T = A @ B; Y = softmax(T): the intermediate T is a transient."""
+    b = StructuredSDFGBuilder("chain")
+    b.add_container("A", F32, True)
+    b.add_container("B", F32, True)
+    b.add_container("Y", F32, True)
+    b.add_container("T", F32, False, transient_bytes=64 * 64 * 4)
+    b.add_gemm("A", "B", "T", "1.0", "0.0", 64, 64, 64)
+    b.add_reduce_op("softmax", "T", "Y", [64, 64], [-1])
+    return b.move()
+
+
+def test_offloading_keeps_intermediates_on_the_device(tmp_path):
+    s = chain_sdfg()
+    s.schedule("rocm")                     # default: function-level offloading
+    report = s.loop_report()
+    assert report["GEMM::ROCMWithoutTransfers"] == 1 and report["ml::Softmax::ROCMWithoutTransfers"] == 1
+    assert report["H2D"] == 2 and report["D2H"] == 1          # A, B up; Y down; T never crosses PCIe
+    assert "size" not in s.containers["T"]                     # and needs no host memory any more
+    codes = [(n["code"], n.get("transfer_direction"), n.get("buffer_lifecycle")) for n in s.library_nodes()]
+    assert codes.index(("GEMM", None, None)) < codes.index(("ml::Softmax", None, None))
+    src, _ = source_of(s, tmp_path)
+    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")  # no host allocation left
+    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(") == 4
+    # without minimisation (per-node transfers) T would cross twice
+    s2 = chain_sdfg()
+    s2.schedule("rocm", options={"offload": "node"})
+    assert s2.loop_report()["H2D"] == 0 and "ROCMOffloading" not in s2.loop_report()
+    src2, _ = source_of(s2, tmp_path / "node")
+    assert src2.count("docc_rocm_memcpy_h2d_async(") == 3 and src2.count("docc_rocm_memcpy_d2h_async(") == 2
+
+
+def test_offloading_reuses_a_read_only_operand(tmp_path):
+    b = StructuredSDFGBuilder("reuse")
+    for n in ("A", "B", "C", "D"):
+        b.add_container(n, F64, True)
+    b.add_gemm("A", "B", "C", "1.0", "0.0", 16, 16, 16)
+    b.add_gemm("C", "B", "D", "1.0", "0.0", 16, 16, 16)
+    s = b.move()
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 2          # A and B once each; C stays on the device
+    assert r["D2H"] == 2          # C and D are arguments: both come back
+    offload = [n for n in s.library_nodes() if n["code"] == "ROCMOffloading"]
+    # payload keys of the reference's offloading node (cuda_data_offloading_node.cpp:198-256)
+    assert all({"size", "device_id", "transfer_direction", "buffer_lifecycle"} <= set(n) for n in offload)
+    d2h_only = [n for n in offload if n["transfer_direction"] == -1 and n["buffer_lifecycle"] == 0]
+    assert len(d2h_only) == 1     # C's download no longer frees: the second GEMM still reads the device copy
+
+
+def test_generated_function_honours_the_calling_convention(tmp_path):
+    """Compiles an emitted function and calls it through ctypes the way CompiledSDFG does. Without a
+    GPU the first runtime call fails; the function must return early and report through the failure
+    channel instead of touching its arguments or aborting."""
+    import torch
+
+    s = gemm_sdfg()
+    s.schedule("rocm", options={"offload": "node"})
+    lib_path = s._compile(str(tmp_path))
+    assert Path(lib_path).name == "libmatmul_sdfg.so"
+    runtime.lib()
+    lib = ctypes.CDLL(lib_path)
+    fn = lib.matmul_sdfg
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    fn.restype = None
+    A, B = np.ones((4, 4)), np.ones((4, 4))
+    out = np.full((4, 4), -1.0)
+    # zero-sized problem: the guard skips every device call, on any machine
+    fn(A.ctypes.data, B.ctypes.data, 0, out.ctypes.data)
+    assert runtime.take_failure() == (0, "") and (out == -1.0).all()
+    if not torch.cuda.is_available():
+        fn(A.ctypes.data, B.ctypes.data, 4, out.ctypes.data)
+        code, message = runtime.take_failure()
+        assert code != 0 and "matmul_sdfg" in message and "docc_rocm_malloc" in message
+        assert (out == -1.0).all()
