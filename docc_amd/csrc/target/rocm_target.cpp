@@ -614,6 +614,42 @@ void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::A
             throw InvalidSDFGException("rocm target cannot map node " + mapper->last_decline_reason() +
                                        " (this target has no CPU lowering)");
     }
+    if (options.offload == "none") {
+        // the caller's pointers are device pointers, so every array the nodes touch lives in HBM:
+        // arguments are relabelled, transients are allocated and freed on the device around their uses
+        // (a host malloc'ed transient handed to a kernel would fault)
+        StructuredSDFG& sdfg = builder.subject();
+        std::vector<std::string> transients;
+        for (auto& kv : sdfg.containers()) {
+            if (!kv.second.is_pointer) continue;
+            Container& c = sdfg.container(kv.first);
+            c.storage = "ROCM_Generic";
+            if (c.transient && !c.is_argument && !c.size_bytes.empty()) transients.push_back(kv.first);
+        }
+        for (auto& name : transients) {
+            auto touches = [&](const Block& b) {
+                for (auto& in : b.inputs)
+                    if (!in.is_constant && in.data == name) return true;
+                for (auto& out : b.outputs)
+                    if (out.data == name) return true;
+                return false;
+            };
+            size_t first = (size_t) -1, last = 0;
+            for (size_t i = 0; i < sdfg.blocks().size(); i++)
+                if (touches(sdfg.blocks()[i])) {
+                    if (first == (size_t) -1) first = i;
+                    last = i;
+                }
+            Container& c = sdfg.container(name);
+            const Expression bytes = c.size_bytes;
+            c.size_bytes.clear();  // no host allocation
+            if (first == (size_t) -1) continue;
+            sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(bytes, 0, DataTransferDirection::NONE, BufferLifecycle::FREE),
+                           {make_binding("_ptr", name)}, {}, last + 1);
+            sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(bytes, 0, DataTransferDirection::NONE, BufferLifecycle::ALLOC),
+                           {}, {make_binding("_ret", name)}, first);
+        }
+    }
     if (options.offload == "function") {
         RocmOffloadTransform offload;
         offload.run_pass(builder, analysis_manager);

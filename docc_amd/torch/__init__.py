@@ -90,6 +90,8 @@ class _FxLowering:
         torch = self.torch
         if all("example_value" in n.meta or "tensor_meta" in n.meta for n in self.gm.graph.nodes if n.op not in ("output",)):
             return
+        if any(not isinstance(a, (torch.Tensor, int, float, bool)) for a in self.example_inputs):
+            return  # symbolic inputs: dynamo has already annotated the graph
         from torch._subclasses.fake_tensor import FakeTensorMode
         from torch.fx.passes.shape_prop import ShapeProp
 
@@ -103,7 +105,8 @@ class _FxLowering:
             v = node.meta.get("tensor_meta")
         if v is None:
             raise NotImplementedError(f"no shape information for FX node {node.name}")
-        return list(v.shape), v.dtype
+        # symbolic sizes (dynamo's automatic dynamic shapes) are specialised to their current value
+        return [int(d) for d in v.shape], v.dtype
 
     # ---- containers ---------------------------------------------------------------------
     def add_input(self, label: str, shape, dtype, source) -> _T:
@@ -245,8 +248,12 @@ class _FxLowering:
         for node in graph.nodes:
             dest = dest_of.get(node)
             if node.op == "placeholder":
-                shape, dtype = self.meta(node)
-                self.env[node] = self.add_input(node.name, shape, dtype, ("arg", arg_index))
+                example = node.meta.get("example_value", self.example_inputs[arg_index] if arg_index < len(self.example_inputs) else None)
+                if example is not None and not isinstance(example, torch.Tensor):
+                    self.env[node] = int(example) if isinstance(example, (int, torch.SymInt)) else example  # a size passed as an input
+                else:
+                    shape, dtype = self.meta(node)
+                    self.env[node] = self.add_input(node.name, shape, dtype, ("arg", arg_index))
                 arg_index += 1
             elif node.op == "get_attr":
                 t = self.gm

@@ -233,3 +233,18 @@ def test_generated_function_honours_the_calling_convention(tmp_path):
         code, message = runtime.take_failure()
         assert code != 0 and "matmul_sdfg" in message and "docc_rocm_malloc" in message
         assert (out == -1.0).all()
+
+
+def test_device_pointer_mode_allocates_transients_on_the_device(tmp_path):
+    """offload == "none": the caller passes device pointers, so an intermediate must be a device
+    allocation too - a host malloc'ed buffer handed to a kernel faults the GPU."""
+    s = chain_sdfg()
+    s.schedule("rocm", options={"offload": "none"})
+    r = s.loop_report()
+    assert r["H2D"] == 0 and r["D2H"] == 0 and r["ROCMOffloading"] == 2       # ALLOC and FREE of T
+    assert s.containers["T"]["storage"] == "ROCM_Generic" and "size" not in s.containers["T"]
+    src, _ = source_of(s, tmp_path)
+    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")
+    flat = re.sub(r"\s+", " ", src)
+    assert flat.index("docc_rocm_malloc(") < flat.index("docc_rocm_sgemm(") < flat.index("docc_rocm_softmax_f32(") < flat.index("docc_rocm_free(")
+    assert src.count("docc_rocm_malloc(") == 1 and src.count("docc_rocm_free(") == 1
