@@ -77,11 +77,20 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     float m_run = -__builtin_huge_valf();   // running max of scale*log2e*score
     float l_part = 0.f;                     // this lane's part of the running sum (its 32 keys per block)
 
-    typedef TileLoader<uint16_t, kBlockKV, kHeadDim, 256, true> KVLoader;
+    // K and V blocks: 64 keys x 64 d, walked along the keys; keys past the end read as zero
+    typedef TileLoader<uint16_t, kBlockKV, kHeadDim, 256, true, false> KVLoader;
     KVLoader lk, lv;
     const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
-    lk.load(Kh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
-    lv.load(Vh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
+    const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
+    lk.init(Kh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
+    lv.init(Vh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
+    if (full_blocks > 0) {
+        lk.load_full();
+        lv.load_full();
+    } else {
+        lk.load_tail(keys_left, tid);
+        lv.load_tail(keys_left, tid);
+    }
     lk.template store<kLdK>(lds, tid);
     lv.template store<kLdV>(lds + V_BASE, tid);
     __syncthreads();
@@ -94,9 +103,16 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
     for (int kb = 0; kb < nblocks; kb++) {
         const int cur = kb & 1;
-        if (kb + 1 < nblocks) {
-            lk.load(Kh, kHeadDim, (long) (kb + 1) * kBlockKV, 0, SKV, kHeadDim, tid);
-            lv.load(Vh, kHeadDim, (long) (kb + 1) * kBlockKV, 0, SKV, kHeadDim, tid);
+        if (kb + 1 < full_blocks) {
+            lk.advance();
+            lv.advance();
+            lk.load_full();
+            lv.load_full();
+        } else if (kb + 1 < nblocks) {
+            lk.advance();
+            lv.advance();
+            lk.load_tail(keys_left, tid);
+            lv.load_tail(keys_left, tid);
         }
         const uint16_t* ks_ = lds + cur * kKElems;
         const uint16_t* vs_ = lds + V_BASE + cur * kVElems;

@@ -42,7 +42,7 @@ struct ConvGatherKernel {
     static_assert(BK * BN % NT == 0 && BK % KG == 0, "tile shape");
     static constexpr int KSTEP = NT / BN;    // k distance between a thread's consecutive elements
 
-    typedef TileLoader<float, BM, BK, NT, ALIGNED> ALoader;
+    typedef TileLoader<float, BM, BK, NT, ALIGNED, true> ALoader;
 
     static __device__ __forceinline__ void run(const ConvParams& p) {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_conv_lds[];
@@ -95,20 +95,27 @@ struct ConvGatherKernel {
 
         ALoader la;
         float bv[NB];
-        auto gload = [&](int kt) {
-            la.load(p.Wt, K, m0, (long) kt * BK, p.OC, K, tid);
+        unsigned bok = 0;  // bit i: gathered element i is a real input pixel (not padding)
+        la.init(p.Wt, K, m0, 0, p.OC, K, tid);
+        const int full = K / BK, kleft = K - full * BK;
+        auto gload = [&](int kt) {   // called for kt = 0, 1, 2, ... in order
+            if (kt > 0) la.advance();
+            if (kt < full) la.load_full();
+            else la.load_tail(kleft, tid);
             const int4* tab = reinterpret_cast<const int4*>(ktab) + (kt & 1) * BK;
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const int4 e = tab[kk0 + i * KSTEP];
                 const int ih = ih0 + e.y, iw = iw0 + e.z;
                 const bool ok = col_ok && e.w && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-                bv[i] = ok ? xbase[e.x] : 0.f;
+                // branch-free: padding taps read the tensor origin and are zeroed in bstore()
+                bv[i] = *(ok ? xbase + e.x : p.X);
+                bok = ok ? (bok | (1u << i)) : (bok & ~(1u << i));
             }
         };
         auto bstore = [&](float* bs) {
 #pragma unroll
-            for (int i = 0; i < NB; i++) bs[(kk0 + i * KSTEP) * LDB_S + tid % BN] = bv[i];
+            for (int i = 0; i < NB; i++) bs[(kk0 + i * KSTEP) * LDB_S + tid % BN] = ((bok >> i) & 1u) ? bv[i] : 0.f;
         };
 
         const int ktiles = (K + BK - 1) / BK;

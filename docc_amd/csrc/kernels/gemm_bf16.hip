@@ -44,8 +44,8 @@ struct GemmBf16Kernel {
     static constexpr int B_ELEMS = (B_KC ? BN : BK) * LDB_S;
     static_assert(BK % KS == 0, "BK must be a multiple of 16");
 
-    typedef TileLoader<uint16_t, A_KC ? BM : BK, A_KC ? BK : BM, NT, ALIGNED> ALoader;
-    typedef TileLoader<uint16_t, B_KC ? BN : BK, B_KC ? BK : BN, NT, ALIGNED> BLoader;
+    typedef TileLoader<uint16_t, A_KC ? BM : BK, A_KC ? BK : BM, NT, ALIGNED, A_KC> ALoader;
+    typedef TileLoader<uint16_t, B_KC ? BN : BK, B_KC ? BK : BN, NT, ALIGNED, B_KC> BLoader;
 
     // eight k-values (k0 .. k0+15 split over the two lane halves) of row/column `idx0 + lane % 32`
     template <bool KC, int LD>
@@ -92,22 +92,12 @@ struct GemmBf16Kernel {
 
         ALoader la;
         BLoader lb;
-        auto gload = [&](long k0) {
-            if (A_KC) la.load(A, lda, m0, k0, M, K, tid);
-            else la.load(A, lda, k0, m0, K, M, tid);
-            if (B_KC) lb.load(B, ldb, n0, k0, N, K, tid);
-            else lb.load(B, ldb, k0, n0, K, N, tid);
-        };
+        if (A_KC) la.init(A, lda, m0, 0, M, K, tid);
+        else la.init(A, lda, 0, m0, K, M, tid);
+        if (B_KC) lb.init(B, ldb, n0, 0, N, K, tid);
+        else lb.init(B, ldb, 0, n0, K, N, tid);
 
-        const int ktiles = (int) ((K + BK - 1) / BK);
-        gload(0);
-        la.template store<LDA_S>(lds, tid);
-        lb.template store<LDB_S>(lds + B_BASE, tid);
-        __syncthreads();
-
-        for (int kt = 0; kt < ktiles; kt++) {
-            const int cur = kt & 1;
-            if (kt + 1 < ktiles) gload((long) (kt + 1) * BK);
+        auto compute = [&](int cur) {
             const uint16_t* as = lds + cur * A_ELEMS;
             const uint16_t* bs = lds + B_BASE + cur * B_ELEMS;
 #pragma unroll
@@ -123,12 +113,47 @@ struct GemmBf16Kernel {
                     for (int j = 0; j < TN; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
             }
-            if (kt + 1 < ktiles) {
-                la.template store<LDA_S>(lds + (cur ^ 1) * A_ELEMS, tid);
-                lb.template store<LDB_S>(lds + B_BASE + (cur ^ 1) * B_ELEMS, tid);
-            }
+        };
+        auto stage = [&](int buf) {
+            la.template store<LDA_S>(lds + buf * A_ELEMS, tid);
+            lb.template store<LDB_S>(lds + B_BASE + buf * B_ELEMS, tid);
+        };
+
+        const int full = (int) (K / BK);
+        const int kleft = (int) (K - (long) full * BK);
+        if (full > 0) {
+            la.load_full();
+            lb.load_full();
+        } else {
+            la.load_tail(kleft, tid);
+            lb.load_tail(kleft, tid);
+        }
+        stage(0);
+        __syncthreads();
+        int kt = 0;
+        for (; kt + 1 < full; kt++) {
+            la.advance();
+            lb.advance();
+            la.load_full();
+            lb.load_full();
+            compute(kt & 1);
+            // keep the stores of step kt+1 (which wait for its loads) behind the MFMAs of step kt:
+            // without this fence the scheduler hoists them and the load latency is exposed
+            __builtin_amdgcn_sched_barrier(0);
+            stage((kt + 1) & 1);
             __syncthreads();
         }
+        if (full > 0 && kleft > 0) {
+            la.advance();
+            lb.advance();
+            la.load_tail(kleft, tid);
+            lb.load_tail(kleft, tid);
+            compute(kt & 1);
+            stage((kt + 1) & 1);
+            __syncthreads();
+            kt++;
+        }
+        compute(kt & 1);
 
         const bool use_c = (beta != 0.f);
         const int lrow = lane & 31;

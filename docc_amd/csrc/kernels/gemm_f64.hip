@@ -3,6 +3,8 @@
 
 DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 16, 2, 2)
 DOCC_GEMM_CONFIG(dgemm, double, 128, 128, 16, 2, 2)
+DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 32, 2, 2)
+DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 64, 2, 2)
 
 extern "C" __global__ __launch_bounds__(256) void docc_dgemm_scale_c(double* C, long M, long N, long ldc, double beta) {
     const long total = M * N;

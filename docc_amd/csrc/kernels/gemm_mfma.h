@@ -76,40 +76,85 @@ __device__ __forceinline__ void gemm_tile_coords(int pid, int tiles_m, int tiles
     tn = (pid % width) / gsize;
 }
 
-// Global -> registers for a ROWS x COLS tile (COLS contiguous in memory) of a
-// row-major matrix with leading dimension ld; elements outside [rmax, cmax)
-// read as zero. NT threads, 128-bit accesses when ALIGNED.
-template <typename T, int ROWS, int COLS, int NT, bool ALIGNED>
+// Global -> registers -> LDS for a ROWS x COLS tile (COLS contiguous in memory) of a row-major
+// operand, walked along K. K runs along the columns for a k-contiguous operand
+// (K_ALONG_COLS) and along the rows otherwise; the other coordinate is the operand's m or n
+// index.
+//
+// Loads are unconditional in the steady state: the m/n coordinate of every vector is clamped
+// into the matrix when the loader is set up (rows or columns beyond the edge hold copies of
+// valid data; the outputs they feed are never stored), each vector keeps one pointer that
+// advances by a constant per K-step, and only the last, partial K-step masks (to zero, because
+// that data does feed valid outputs). No branch and no select stands between a load and the
+// MFMAs of the current step, so the loads stay in flight while the step is multiplied.
+// ALIGNED promises 16-byte aligned rows and contiguous extents that are multiples of VEC.
+template <typename T, int ROWS, int COLS, int NT, bool ALIGNED, bool K_ALONG_COLS>
 struct TileLoader {
     typedef typename Mfma<T>::vec_t vec_t;
     static constexpr int VEC = Mfma<T>::VEC;
     static constexpr int VPR = COLS / VEC;            // vectors per tile row
     static constexpr int NV = ROWS * VPR / NT;        // vectors per thread
+    static constexpr int BK = K_ALONG_COLS ? COLS : ROWS;
     static_assert(ROWS * VPR % NT == 0, "tile does not divide among the threads");
 
+    const T* p[NV];   // address of vector i in the current K-step
+    int lim[NV];      // unaligned, K along rows: last valid element offset of the vector (may be negative)
     vec_t v[NV];
+    long kstep;
 
-    __device__ __forceinline__ void load(const T* __restrict__ base, long ld, long r0, long c0, long rmax, long cmax,
+    // (r0, c0): tile origin at K = 0; rmax / cmax: matrix extents
+    __device__ __forceinline__ void init(const T* __restrict__ base, long ld, long r0, long c0, long rmax, long cmax,
                                          int tid) {
+        kstep = K_ALONG_COLS ? (long) COLS : (long) ROWS * ld;
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int idx = tid + i * NT;
-            const long r = r0 + idx / VPR;
-            const long c = c0 + (idx % VPR) * VEC;
-            vec_t val;
-#pragma unroll
-            for (int e = 0; e < VEC; e++) val[e] = (T) 0;
-            if (r < rmax) {
-                const T* p = base + r * ld + c;
-                if (ALIGNED && c + VEC <= cmax) {
-                    val = *reinterpret_cast<const vec_t*>(p);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < VEC; e++)
-                        if (c + e < cmax) val[e] = p[e];
-                }
+            long r = r0 + idx / VPR;
+            long c = c0 + (idx % VPR) * VEC;
+            lim[i] = VEC - 1;
+            if (K_ALONG_COLS) {
+                r = r < rmax ? r : rmax - 1;               // clamp the m/n index
+            } else if (ALIGNED) {
+                c = c + VEC <= cmax ? c : cmax - VEC;      // whole vectors: clamp the vector start
+            } else {
+                lim[i] = (int) (cmax - 1 - c);             // per element: offsets beyond lim are clamped to it
             }
-            v[i] = val;
+            p[i] = base + r * ld + c;
+        }
+    }
+
+    __device__ __forceinline__ void advance() {
+#pragma unroll
+        for (int i = 0; i < NV; i++) p[i] += kstep;
+    }
+
+    // a K-step that lies entirely inside [0, K)
+    __device__ __forceinline__ void load_full() {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            if (ALIGNED) {
+                v[i] = *reinterpret_cast<const vec_t*>(p[i]);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) v[i][e] = p[i][(!K_ALONG_COLS && e > lim[i]) ? lim[i] : e];
+            }
+        }
+    }
+
+    // the last K-step when only `kleft` < BK values of k remain: the rest reads as zero
+    __device__ __forceinline__ void load_tail(int kleft, int tid) {
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int idx = tid + i * NT;
+            const int lr = idx / VPR, lc = (idx % VPR) * VEC;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const bool ok = K_ALONG_COLS ? (lc + e < kleft) : (lr < kleft);
+                const int off = (!K_ALONG_COLS && !ALIGNED && e > lim[i]) ? lim[i] : e;
+                // outside: read this thread's own first element of the first K-step instead (a valid address)
+                const T raw = ok ? p[i][off] : (T) 0;
+                v[i][e] = raw;
+            }
         }
     }
 
@@ -119,9 +164,7 @@ struct TileLoader {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int idx = tid + i * NT;
-            const int r = idx / VPR;
-            const int c = (idx % VPR) * VEC;
-            *reinterpret_cast<vec_t*>(lds + r * LDS_LD + c) = v[i];
+            *reinterpret_cast<vec_t*>(lds + (idx / VPR) * LDS_LD + (idx % VPR) * VEC) = v[i];
         }
     }
 };
@@ -151,8 +194,8 @@ struct GemmKernel {
     static_assert(BK % KG == 0, "BK must be a multiple of the k-group");
     static_assert(WTM % MT == 0 && WTN % MT == 0, "wave tile must be a multiple of the MFMA tile");
 
-    typedef TileLoader<T, A_KC ? BM : BK, A_KC ? BK : BM, NT, ALIGNED> ALoader;
-    typedef TileLoader<T, B_KC ? BN : BK, B_KC ? BK : BN, NT, ALIGNED> BLoader;
+    typedef TileLoader<T, A_KC ? BM : BK, A_KC ? BK : BM, NT, ALIGNED, A_KC> ALoader;
+    typedef TileLoader<T, B_KC ? BN : BK, B_KC ? BK : BN, NT, ALIGNED, B_KC> BLoader;
 
     static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                long M, long N, long K, long lda, long ldb, long ldc, T alpha,
@@ -183,25 +226,15 @@ struct GemmKernel {
 
         ALoader la;
         BLoader lb;
-        auto gload = [&](long k0) {
-            if (A_KC) la.load(A, lda, m0, k0, M, K, tid);
-            else la.load(A, lda, k0, m0, K, M, tid);
-            if (B_KC) lb.load(B, ldb, n0, k0, N, K, tid);
-            else lb.load(B, ldb, k0, n0, K, N, tid);
-        };
-
-        const int ktiles = (int) ((K + BK - 1) / BK);
-        gload(0);
-        la.template store<LDA_S>(lds, tid);
-        lb.template store<LDB_S>(lds + B_BASE, tid);
-        __syncthreads();
+        if (A_KC) la.init(A, lda, m0, 0, M, K, tid);
+        else la.init(A, lda, 0, m0, K, M, tid);
+        if (B_KC) lb.init(B, ldb, n0, 0, N, K, tid);
+        else lb.init(B, ldb, 0, n0, K, N, tid);
 
         const int lrow = lane % MT;          // row (A) / column (B) inside an MFMA tile
         const int lk = (lane / MT) * VK;     // this lane's first k inside a k-group
 
-        for (int kt = 0; kt < ktiles; kt++) {
-            const int cur = kt & 1;
-            if (kt + 1 < ktiles) gload((long) (kt + 1) * BK);
+        auto compute = [&](int cur) {
             const T* as = lds + cur * A_ELEMS;
             const T* bs = lds + B_BASE + cur * B_ELEMS;
 #pragma unroll
@@ -238,12 +271,48 @@ struct GemmKernel {
 #pragma unroll
                         for (int j = 0; j < TN; j++) acc[i][j] = X::mfma(a[i][s], b[j][s], acc[i][j]);
             }
-            if (kt + 1 < ktiles) {
-                la.template store<LDA_S>(lds + (cur ^ 1) * A_ELEMS, tid);
-                lb.template store<LDB_S>(lds + B_BASE + (cur ^ 1) * B_ELEMS, tid);
-            }
+        };
+        auto stage = [&](int buf) {
+            la.template store<LDA_S>(lds + buf * A_ELEMS, tid);
+            lb.template store<LDB_S>(lds + B_BASE + buf * B_ELEMS, tid);
+        };
+
+        // K-steps 0 .. full-1 lie inside K, an optional last one is partial
+        const int full = (int) (K / BK);
+        const int kleft = (int) (K - (long) full * BK);
+        if (full > 0) {
+            la.load_full();
+            lb.load_full();
+        } else {
+            la.load_tail(kleft, tid);
+            lb.load_tail(kleft, tid);
+        }
+        stage(0);
+        __syncthreads();
+        int kt = 0;
+        for (; kt + 1 < full; kt++) {   // steady state: step kt+1 travels while step kt is multiplied
+            la.advance();
+            lb.advance();
+            la.load_full();
+            lb.load_full();
+            compute(kt & 1);
+            // keep the stores of step kt+1 (which wait for its loads) behind the MFMAs of step kt:
+            // without this fence the scheduler hoists them and the load latency is exposed
+            __builtin_amdgcn_sched_barrier(0);
+            stage((kt + 1) & 1);
             __syncthreads();
         }
+        if (full > 0 && kleft > 0) {
+            la.advance();
+            lb.advance();
+            la.load_tail(kleft, tid);
+            lb.load_tail(kleft, tid);
+            compute(kt & 1);
+            stage((kt + 1) & 1);
+            __syncthreads();
+            kt++;
+        }
+        compute(kt & 1);
 
         // epilogue: C = alpha*acc + beta*C; C is not read when beta == 0
         const bool use_c = (beta != (T) 0);

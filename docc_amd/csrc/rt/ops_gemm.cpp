@@ -57,11 +57,20 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     const bool use_big = force && force[0] == 'b'   ? true
                          : force && force[0] == 's' ? false
                                                     : big_tiles >= big_min_tiles;
-    const TileConfig& cfg = use_big ? big : small;
+    TileConfig cfg = use_big ? big : small;
+    // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES selects a built configuration directly (tuning)
+    if (const char* c = std::getenv("DOCC_ROCM_GEMM_CFG")) {
+        TileConfig t{};
+        if (std::sscanf(c, "%dx%dx%dx%d", &t.bm, &t.bn, &t.bk, &t.waves) == 4 && t.bm > 0 && t.bn > 0 && t.bk > 0 && t.waves > 0) cfg = t;
+    }
     const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     const size_t vec = 16 / sizeof(T);
-    const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0);
+    // the aligned kernels read whole 128-bit vectors: pointers, leading dimensions and the
+    // contiguous extents of both operands must be multiples of the vector length
+    const int64_t a_contig = ta ? m : k, b_contig = tb ? k : n;
+    const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0) &&
+                         (a_contig % (int64_t) vec == 0) && (b_contig % (int64_t) vec == 0);
     std::snprintf(name, sizeof(name), "docc_%s_%dx%dx%d_%c%c_%c", prefix, cfg.bm, cfg.bn, cfg.bk, ta ? 't' : 'n',
                   tb ? 't' : 'n', aligned ? 'a' : 'u');
     const size_t lds = gemm_lds_bytes(cfg, ta, tb, sizeof(T));
