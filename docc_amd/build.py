@@ -37,8 +37,23 @@ KERNEL_FAMILIES = {
     "gemm_f32": "gemm_f32.hip",
     "gemm_f64": "gemm_f64.hip",
     "gemm_bf16": "gemm_bf16.hip",
+    "gemm_bf16_async": "gemm_bf16_async.hip",
+    "gemm_bf16_async_big": "gemm_bf16_async_big.hip",
     "conv2d": "conv2d.hip",
     "attention": "attention.hip",
+}
+
+# Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary
+# VGPRs: without it the compiler parks loop-carried accumulators in VGPRs and copies them to and
+# from AGPRs around the MFMAs of every K-step (64 extra VALU instructions per step for a
+# 32-register accumulator). Families whose accumulators alone need more than 256 registers
+# (the 256x256 bf16 tile) cannot use it.
+FAMILY_FLAGS = {
+    "gemm_f64": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_f32": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_bf16_async": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "conv2d": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 # packed fp32 VALU ops are switched off for every device compile
@@ -78,7 +93,7 @@ def build_kernel_family(family: str, force: bool = True) -> Path:
     if not force and _newer(out, deps):
         return out
     LIB.mkdir(parents=True, exist_ok=True)
-    _run([hipcc(), "--genco", *DEVICE_FLAGS, "-I", str(CSRC / "kernels"), str(src), "-o", str(out)])
+    _run([hipcc(), "--genco", *DEVICE_FLAGS, *FAMILY_FLAGS.get(family, []), "-I", str(CSRC / "kernels"), str(src), "-o", str(out)])
     return out
 
 

@@ -1,0 +1,322 @@
+// Tiled MFMA GEMM with an asynchronous, multi-stage global -> LDS pipeline (gfx950):
+//   C[M,N] = alpha * op(A) * op(B) + beta * C,  row-major, A/B fp64, fp32 or bf16 (fp32 C for bf16).
+//
+// Same tiling as gemm_mfma.h; what differs is how operand tiles reach LDS:
+//   - every 16-byte granule of a tile travels with one `global_load_lds_dwordx4`: the data goes
+//     from memory straight into LDS, no registers and no LDS store instruction in between;
+//     a wave-instruction fills 64 consecutive granules (1 KiB);
+//   - S stages of LDS are kept: while step kt is multiplied, the loads of steps kt+1 .. kt+S-1
+//     are in flight, so an L2 miss has S-1 steps to come back. One `s_waitcnt vmcnt(n)` and one
+//     `s_barrier` per step; n leaves the newer steps' loads outstanding;
+//   - because the LDS position of a granule is fixed by the lane that loads it, rows cannot be
+//     padded; bank conflicts are avoided by XOR-swizzling the granule index with the row
+//     (the lane simply fetches the global granule that belongs in its slot);
+//   - the partial last K-step (and nothing else) goes through registers, masked to zero.
+// Requires 16-byte aligned operands with contiguous extents that are multiples of the vector
+// length (the launcher sends everything else to the gemm_mfma.h kernels).
+#pragma once
+
+#include "gemm_mfma.h"
+
+namespace docc_k {
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* global_ptr_t;
+typedef uint16_t u16x8a __attribute__((ext_vector_type(8)));
+typedef short s16x4a __attribute__((ext_vector_type(4)));
+typedef short s16x8a __attribute__((ext_vector_type(8)));
+
+template <typename T>
+struct AsyncTraits;
+template <>
+struct AsyncTraits<float> {
+    static constexpr int VEC = 4, MT = 32, G = 2, KG = 8, NACC = 16;   // KG: k consumed per fetch round
+    typedef f32x4 vec_t;
+    typedef f32x16 acc_t;
+    typedef float out_t;
+    static __device__ __forceinline__ int swz_mn(int k) { return ((k >> 2) & 1) << 3; }
+};
+template <>
+struct AsyncTraits<double> {
+    static constexpr int VEC = 2, MT = 16, G = 4, KG = 8, NACC = 4;
+    typedef f64x2 vec_t;
+    typedef f64x4 acc_t;
+    typedef double out_t;
+    static __device__ __forceinline__ int swz_mn(int k) { return ((k >> 1) & 1) << 3; }
+};
+template <>
+struct AsyncTraits<uint16_t> {   // bf16 bits
+    static constexpr int VEC = 8, MT = 32, G = 2, KG = 16, NACC = 16;
+    typedef u16x8a vec_t;
+    typedef f32x16 acc_t;
+    typedef float out_t;
+    static __device__ __forceinline__ int swz_mn(int k) { return (k & 3) << 2; }
+};
+
+// One operand tile of ROWS x COLS elements (COLS contiguous) in an LDS stage.
+template <typename T, int ROWS, int COLS, int NT, bool K_ALONG_COLS>
+struct AsyncTile {
+    typedef AsyncTraits<T> X;
+    typedef typename X::vec_t vec_t;
+    static constexpr int VEC = X::VEC;
+    static constexpr int VPR = COLS / VEC;          // granules per row
+    static constexpr int NG = ROWS * VPR;           // granules per tile
+    static constexpr int NW = NT / 64;
+    static constexpr int NV = NG / NT;              // granules per thread
+    static constexpr int ELEMS = ROWS * COLS;
+    static constexpr int BK = K_ALONG_COLS ? COLS : ROWS;
+    static_assert(NG % NT == 0, "tile does not divide among the threads");
+    static_assert(K_ALONG_COLS ? (VPR == 16 || VPR == 8 || VPR == 4) : (VPR >= 16), "row length not covered by the swizzles");
+
+    // granule-index swizzle of a row
+    static __device__ __forceinline__ int swz(int row) {
+        // 16 consecutive rows read the same k-granule at once: spread them over the 16 slots of 256 bytes
+        if (K_ALONG_COLS) return VPR == 16 ? (row & 15) : VPR == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+        return X::swz_mn(row);
+    }
+    // element offset (inside a stage) of the granule that holds columns cv*VEC .. of `row`
+    static __device__ __forceinline__ int granule_offset(int row, int cv) { return (row * VPR + (cv ^ swz(row))) * VEC; }
+
+    const T* p[NV];
+    long kstep;
+
+    __device__ __forceinline__ void init(const T* __restrict__ base, long ld, long r0, long c0, long rmax, long cmax, int tid) {
+        kstep = K_ALONG_COLS ? (long) COLS : (long) ROWS * ld;
+        const int wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int g = (i * NW + wave) * 64 + lane;   // the LDS slot this lane fills
+            const int row = g / VPR, cv = (g % VPR) ^ swz(row);
+            long r = r0 + row, c = c0 + (long) cv * VEC;
+            if (K_ALONG_COLS) r = r < rmax ? r : rmax - 1;
+            else c = c + VEC <= cmax ? c : cmax - VEC;
+            p[i] = base + r * ld + c;
+        }
+    }
+
+    __device__ __forceinline__ void advance() {
+#pragma unroll
+        for (int i = 0; i < NV; i++) p[i] += kstep;
+    }
+
+    // asynchronous copy of the current K-step into `stage`
+    __device__ __forceinline__ void issue(T* stage, int tid) const {
+        const int wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < NV; i++)
+            __builtin_amdgcn_global_load_lds((global_ptr_t) p[i], (lds_ptr_t) (stage + (i * NW + wave) * 64 * VEC), 16, 0, 0);
+    }
+
+    // the partial last K-step through registers: k >= kleft reads as zero
+    __device__ __forceinline__ void copy_tail(T* stage, int kleft, int tid) const {
+        const int wave = tid >> 6, lane = tid & 63;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            const int g = (i * NW + wave) * 64 + lane;
+            const int row = g / VPR, cv = (g % VPR) ^ swz(row);
+            vec_t v;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const bool ok = K_ALONG_COLS ? (cv * VEC + e < kleft) : (row < kleft);
+                v[e] = ok ? p[i][e] : (T) 0;
+            }
+            *reinterpret_cast<vec_t*>(stage + g * VEC) = v;
+        }
+    }
+};
+
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool TA, bool TB>
+struct AsyncGemmKernel {
+    typedef AsyncTraits<T> X;
+    typedef typename X::acc_t acc_t;
+    typedef typename X::vec_t vec_t;
+    typedef typename X::out_t out_t;
+    static constexpr int NT = 64 * WM * WN;
+    static constexpr int MT = X::MT, VEC = X::VEC, KG = X::KG;
+    static constexpr int WTM = BM / WM, WTN = BN / WN;
+    static constexpr int TM = WTM / MT, TN = WTN / MT;
+    static constexpr bool A_KC = !TA, B_KC = TB;
+    typedef AsyncTile<T, A_KC ? BM : BK, A_KC ? BK : BM, NT, A_KC> ATile;
+    typedef AsyncTile<T, B_KC ? BN : BK, B_KC ? BK : BN, NT, B_KC> BTile;
+    static constexpr int STAGE_ELEMS = ATile::ELEMS + BTile::ELEMS;
+    static constexpr int LDS_BYTES = STAGES * STAGE_ELEMS * (int) sizeof(T);
+    static constexpr int LOADS_PER_STEP = ATile::NV + BTile::NV;
+    static_assert(BK % KG == 0, "BK must be a multiple of the k-group");
+    static_assert(STAGES >= 2 && (STAGES - 1) * LOADS_PER_STEP < 64, "vmcnt holds at most 63 outstanding loads");
+
+    static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, out_t* __restrict__ C,
+                                               long M, long N, long K, long lda, long ldb, long ldc, out_t alpha,
+                                               out_t beta) {
+        extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
+        T* const lds = reinterpret_cast<T*>(docc_gemm_lds);
+
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int wm = wave / WN, wn = wave % WN;
+        const int tiles_m = (int) ((M + BM - 1) / BM), tiles_n = (int) ((N + BN - 1) / BN);
+        int tm, tn;
+        gemm_tile_coords(blockIdx.x, tiles_m, tiles_n, tm, tn);
+        const long m0 = (long) tm * BM, n0 = (long) tn * BN;
+
+        acc_t acc[TM][TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < X::NACC; r++) acc[i][j][r] = 0;
+
+        ATile ta;
+        BTile tb;
+        if (A_KC) ta.init(A, lda, m0, 0, M, K, tid);
+        else ta.init(A, lda, 0, m0, K, M, tid);
+        if (B_KC) tb.init(B, ldb, n0, 0, N, K, tid);
+        else tb.init(B, ldb, 0, n0, K, N, tid);
+
+        const int lidx = lane % MT;     // row of A / column of B inside an MFMA tile
+        const int lg = lane / MT;       // k-group of this lane
+
+        // ---- the multiply of one staged K-step ---------------------------------------------
+        auto compute = [&](const T* stage) {
+            const T* as = stage;
+            const T* bs = stage + ATile::ELEMS;
+            if constexpr (sizeof(T) == 2) {
+                // bf16: one MFMA consumes 16 k; lane (idx, g) supplies k = 8g .. 8g+7
+#pragma unroll
+                for (int ks = 0; ks < BK / 16; ks++) {
+                    bf16x8 a[TM], b[TN];
+                    auto fetch = [&](auto tile_tag, const T* base, int idx0, bool kc) -> bf16x8 {
+                        typedef decltype(tile_tag) Tile;
+                        if (kc) {
+                            const int row = idx0 + lidx;
+                            const u16x8a v = *reinterpret_cast<const u16x8a*>(base + Tile::granule_offset(row, ks * 2 + lg));
+                            return __builtin_bit_cast(bf16x8, v);
+                        }
+                        // transposed read: 16-lane group = 4 k-rows x 16 columns, see gemm_bf16.hip
+                        const int s = lane & 15, grp = lane >> 4;
+                        const int krow = ks * 16 + 8 * (grp >> 1) + (s >> 2);
+                        const int col = idx0 + 16 * (grp & 1) + 4 * (s & 3);
+                        typedef __attribute__((address_space(3))) s16x4a lds_s16x4;
+                        const T* plo = base + Tile::granule_offset(krow, col / 8) + (col & 7);
+                        const T* phi = base + Tile::granule_offset(krow + 4, col / 8) + (col & 7);
+                        const s16x4a lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
+                        const s16x4a hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
+                        const s16x8a v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                        return __builtin_bit_cast(bf16x8, v);
+                    };
+#pragma unroll
+                    for (int i = 0; i < TM; i++) a[i] = fetch(ATile{}, as, wm * WTM + i * MT, A_KC);
+#pragma unroll
+                    for (int j = 0; j < TN; j++) b[j] = fetch(BTile{}, bs, wn * WTN + j * MT, B_KC);
+#pragma unroll
+                    for (int i = 0; i < TM; i++)
+#pragma unroll
+                        for (int j = 0; j < TN; j++)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+                }
+            } else {
+                // fp32 / fp64: lane group g owns k = kg*KG + g*VK .. +VK-1 (VK = VEC: one granule)
+                constexpr int VK = VEC;
+#pragma unroll
+                for (int kg = 0; kg < BK / KG; kg++) {
+                    T a[TM][VK], b[TN][VK];
+                    auto fetch = [&](auto tile_tag, const T* base, int idx0, bool kc, T* out) {
+                        typedef decltype(tile_tag) Tile;
+                        if (kc) {
+                            const vec_t v = *reinterpret_cast<const vec_t*>(base + Tile::granule_offset(idx0 + lidx, kg * X::G + lg));
+#pragma unroll
+                            for (int s = 0; s < VK; s++) out[s] = v[s];
+                        } else {
+                            const int col = idx0 + lidx;
+#pragma unroll
+                            for (int s = 0; s < VK; s++)
+                                out[s] = base[Tile::granule_offset(kg * KG + lg * VK + s, col / VEC) + col % VEC];
+                        }
+                    };
+#pragma unroll
+                    for (int i = 0; i < TM; i++) fetch(ATile{}, as, wm * WTM + i * MT, A_KC, a[i]);
+#pragma unroll
+                    for (int j = 0; j < TN; j++) fetch(BTile{}, bs, wn * WTN + j * MT, B_KC, b[j]);
+#pragma unroll
+                    for (int s = 0; s < VK; s++)
+#pragma unroll
+                        for (int i = 0; i < TM; i++)
+#pragma unroll
+                            for (int j = 0; j < TN; j++) acc[i][j] = Mfma<T>::mfma(a[i][s], b[j][s], acc[i][j]);
+                }
+            }
+        };
+
+        // ---- pipeline --------------------------------------------------------------------------
+        const int full = (int) (K / BK);
+        const int kleft = (int) (K - (long) full * BK);
+        const int ksteps = full + (kleft > 0 ? 1 : 0);
+        auto stage_of = [&](int kt) { return lds + (kt % STAGES) * STAGE_ELEMS; };
+        auto fill = [&](int kt) {   // starts the copy of step kt (called for kt = 0, 1, 2, ... in order)
+            if (kt > 0) {
+                ta.advance();
+                tb.advance();
+            }
+            T* st = stage_of(kt);
+            if (kt < full) {
+                ta.issue(st, tid);
+                tb.issue(st + ATile::ELEMS, tid);
+            } else {
+                ta.copy_tail(st, kleft, tid);
+                tb.copy_tail(st + ATile::ELEMS, kleft, tid);
+            }
+        };
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; s++)
+            if (s < ksteps) fill(s);
+
+        for (int kt = 0; kt < ksteps; kt++) {
+            // step kt has landed once at most the loads of the STAGES-2 newer full steps are outstanding;
+            // near the end fewer newer steps exist, so everything is awaited
+            if (kt + STAGES - 2 < full) {
+                asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * LOADS_PER_STEP) : "memory");
+            } else {
+                asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();   // all waves' parts of step kt are in LDS; step kt-1 is fully consumed
+            asm volatile("" ::: "memory");
+            if (kt + STAGES - 1 < ksteps) fill(kt + STAGES - 1);   // into the stage step kt-1 occupied
+            compute(stage_of(kt));
+        }
+
+        // ---- epilogue ------------------------------------------------------------------------------
+        const bool use_c = (beta != (out_t) 0);
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const long col = n0 + wn * WTN + j * MT + lidx;
+#pragma unroll
+                for (int r = 0; r < X::NACC; r++) {
+                    const int rr = (sizeof(T) == 8) ? Mfma<double>::acc_row(lane, r) : Mfma<float>::acc_row(lane, r);
+                    const long row = m0 + wm * WTM + i * MT + rr;
+                    if (row < M && col < N) {
+                        out_t* p = C + row * ldc + col;
+                        out_t val = alpha * acc[i][j][r];
+                        if (use_c) val += beta * (*p);
+                        *p = val;
+                    }
+                }
+            }
+        }
+    }
+};
+
+} // namespace docc_k
+
+// extern "C" kernels docc_<prefix>a_<BM>x<BN>x<BK>s<STAGES>_<nn|nt|tn|tt>
+#define DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, TA, TB, TAG)                                          \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_##PREFIX##a_##BM##x##BN##x##BK##s##ST##_##TAG(  \
+        const T* A, const T* B, OT* C, long M, long N, long K, long lda, long ldb, long ldc, OT alpha, OT beta) {   \
+        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta); \
+    }
+
+#define DOCC_AGEMM_CONFIG(PREFIX, T, OT, BM, BN, BK, WM, WN, ST)            \
+    DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, false, false, nn)   \
+    DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, false, true, nt)    \
+    DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, true, false, tn)    \
+    DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, true, true, tt)

@@ -1,10 +1,17 @@
 // fp64 GEMM kernels (v_mfma_f64_16x16x4_f64), see gemm_mfma.h.
-#include "gemm_mfma.h"
+#include "gemm_async.h"
 
 DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 16, 2, 2)
 DOCC_GEMM_CONFIG(dgemm, double, 128, 128, 16, 2, 2)
-DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 32, 2, 2)
-DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 64, 2, 2)
+
+// asynchronous multi-stage pipeline (aligned operands)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 2)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 4)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 6)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 128, 128, 16, 2, 2, 3)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 16, 2, 2, 4)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 32, 2, 2, 3)
+DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 32, 2, 2, 3)
 
 extern "C" __global__ __launch_bounds__(256) void docc_dgemm_scale_c(double* C, long M, long N, long ldc, double beta) {
     const long total = M * N;

@@ -11,6 +11,7 @@ namespace {
 
 struct TileConfig {
     int bm, bn, bk, waves;
+    int stages;  // > 0: asynchronous multi-stage kernel (gemm_async.h), aligned operands only
 };
 
 // LDS bytes of GemmKernel<T, BM, BN, BK, ...> (csrc/kernels/gemm_mfma.h)
@@ -29,7 +30,7 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
 template <typename T, typename S = T>
 int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n,
                 int64_t k, S alpha, const T* A, int64_t lda, const T* B, int64_t ldb, S beta, S* C, int64_t ldc,
-                const TileConfig& big, const TileConfig& small, int64_t big_min_tiles) {
+                TileConfig (*pick)(int64_t m, int64_t n, bool aligned, int force)) {
     if ((trans_a != DOCC_ROCM_NO_TRANS && trans_a != DOCC_ROCM_TRANS) ||
         (trans_b != DOCC_ROCM_NO_TRANS && trans_b != DOCC_ROCM_TRANS))
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: transpose code must be 111 or 112", prefix);
@@ -51,29 +52,34 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         if (blocks > 4096) blocks = 4096;
         return launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
     }
-    const int64_t big_tiles = ((m + big.bm - 1) / big.bm) * ((n + big.bn - 1) / big.bn);
-    // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
-    const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
-    const bool use_big = force && force[0] == 'b'   ? true
-                         : force && force[0] == 's' ? false
-                                                    : big_tiles >= big_min_tiles;
-    TileConfig cfg = use_big ? big : small;
-    // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES selects a built configuration directly (tuning)
-    if (const char* c = std::getenv("DOCC_ROCM_GEMM_CFG")) {
-        TileConfig t{};
-        if (std::sscanf(c, "%dx%dx%dx%d", &t.bm, &t.bn, &t.bk, &t.waves) == 4 && t.bm > 0 && t.bn > 0 && t.bk > 0 && t.waves > 0) cfg = t;
-    }
-    const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
-    if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     const size_t vec = 16 / sizeof(T);
     // the aligned kernels read whole 128-bit vectors: pointers, leading dimensions and the
     // contiguous extents of both operands must be multiples of the vector length
     const int64_t a_contig = ta ? m : k, b_contig = tb ? k : n;
     const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0) &&
                          (a_contig % (int64_t) vec == 0) && (b_contig % (int64_t) vec == 0);
-    std::snprintf(name, sizeof(name), "docc_%s_%dx%dx%d_%c%c_%c", prefix, cfg.bm, cfg.bn, cfg.bk, ta ? 't' : 'n',
-                  tb ? 't' : 'n', aligned ? 'a' : 'u');
-    const size_t lds = gemm_lds_bytes(cfg, ta, tb, sizeof(T));
+    // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
+    const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
+    TileConfig cfg = pick(m, n, aligned, force && force[0] == 'b' ? 1 : force && force[0] == 's' ? -1 : 0);
+    // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES[xSTAGES] selects a built configuration directly (tuning)
+    if (const char* c = std::getenv("DOCC_ROCM_GEMM_CFG")) {
+        TileConfig t{};
+        const int got = std::sscanf(c, "%dx%dx%dx%dx%d", &t.bm, &t.bn, &t.bk, &t.waves, &t.stages);
+        if (got >= 4 && t.bm > 0 && t.bn > 0 && t.bk > 0 && t.waves > 0) cfg = t;
+    }
+    if (cfg.stages > 0 && !aligned) cfg = pick(m, n, false, 0);   // the asynchronous kernels need aligned operands
+    const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
+    if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
+    size_t lds;
+    if (cfg.stages > 0) {
+        std::snprintf(name, sizeof(name), "docc_%sa_%dx%dx%ds%d_%c%c", prefix, cfg.bm, cfg.bn, cfg.bk, cfg.stages,
+                      ta ? 't' : 'n', tb ? 't' : 'n');
+        lds = (size_t) cfg.stages * ((size_t) cfg.bm * cfg.bk + (size_t) cfg.bk * cfg.bn) * sizeof(T);
+    } else {
+        std::snprintf(name, sizeof(name), "docc_%s_%dx%dx%d_%c%c_%c", prefix, cfg.bm, cfg.bn, cfg.bk, ta ? 't' : 'n',
+                      tb ? 't' : 'n', aligned ? 'a' : 'u');
+        lds = gemm_lds_bytes(cfg, ta, tb, sizeof(T));
+    }
     return launch(name, (uint32_t) tiles, 1, 1, 64 * cfg.waves, (uint32_t) lds, s, A, B, C, (long) m, (long) n,
                   (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta);
 }
@@ -82,27 +88,49 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
 
 extern "C" {
 
+// Tile selection. `force`: +1 largest tile, -1 smallest tile, 0 by problem size. Asynchronous
+// (staged) configurations need aligned operands; the others handle everything.
+static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); }
+
+static TileConfig pick_sgemm(int64_t m, int64_t n, bool, int force) {
+    const TileConfig big{128, 128, 16, 4, 0}, small{64, 64, 16, 4, 0};
+    if (force) return force > 0 ? big : small;
+    return tiles_of(m, n, 128, 128) >= 4096 ? big : small;
+}
+
+static TileConfig pick_dgemm(int64_t m, int64_t n, bool aligned, int force) {
+    const TileConfig big{128, 128, 16, 4, 3}, mid{64, 64, 16, 4, 4}, small{64, 32, 16, 4, 4};
+    const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
+    if (!aligned) return force > 0 ? plain_big : plain_small;
+    if (force) return force > 0 ? big : small;
+    const int64_t t = tiles_of(m, n, 64, 64);
+    return t >= 2048 ? big : t > 512 ? mid : small;   // few tiles: halve them so that two work-groups share a CU
+}
+
+static TileConfig pick_bgemm(int64_t m, int64_t n, bool aligned, int force) {
+    const TileConfig big{256, 256, 64, 4, 2}, small{128, 128, 32, 4, 4};
+    const TileConfig plain_big{256, 256, 64, 4, 0}, plain_small{128, 128, 64, 4, 0};
+    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 256, 256) >= 256 ? plain_big : plain_small);
+    if (force) return force > 0 ? big : small;
+    return tiles_of(m, n, 256, 256) >= 192 ? big : small;
+}
+
 int docc_rocm_sgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
                     const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C, int64_t ldc) {
-    static const TileConfig big{128, 128, 16, 4}, small{64, 64, 16, 4};
-    return gemm_launch<float>("sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, big,
-                              small, 192);
+    return gemm_launch<float>("sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, pick_sgemm);
 }
 
 int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                     double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta, double* C,
                     int64_t ldc) {
-    static const TileConfig big{128, 128, 16, 4}, small{64, 64, 16, 4};
-    return gemm_launch<double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, big,
-                               small, 512);
+    return gemm_launch<double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, pick_dgemm);
 }
 
 int docc_rocm_bf16gemm_f32(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                            float alpha, const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, float beta,
                            float* C, int64_t ldc) {
-    static const TileConfig big{256, 256, 64, 4}, small{128, 128, 64, 4};
-    return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C,
-                                        ldc, big, small, 256);
+    return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+                                        pick_bgemm);
 }
 
 } // extern "C"

@@ -29,6 +29,8 @@ const char* const kKernelImages[] = {
     "docc_rocm_gemm_f32.hsaco",
     "docc_rocm_gemm_f64.hsaco",
     "docc_rocm_gemm_bf16.hsaco",
+    "docc_rocm_gemm_bf16_async.hsaco",
+    "docc_rocm_gemm_bf16_async_big.hsaco",
     "docc_rocm_conv2d.hsaco",
     "docc_rocm_attention.hsaco",
 };
