@@ -192,3 +192,183 @@ struct ConvGatherKernel {
 
 DOCC_CONV_GATHER(64, 128, 16, 2, 2, true, a)
 DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
+
+// ---------------------------------------------------------------------------------------------
+// Stride-1, dilation-1 convolution with LDS-staged input halos.
+//
+// One work-group computes 64 output channels x a strip of TH full output rows of one image
+// (TH*OW <= 448 pixels = 14 MFMA column tiles). Wave w takes output-channel tile (w & 1) and
+// pixel tiles 7*(w >> 1) .. +6, so the four waves hold the whole strip in 7 accumulators each.
+// K = C*KH*KW is walked in chunks of 8 input channels. Per chunk the work-group stages
+//   - the input patch [8][TH+KH-1][OW+KW-1] (halo rows and columns included, zeros where the
+//     patch leaves the image): every input pixel is read from memory once per strip instead
+//     of KH*KW times, and
+//   - the weight slab [64][8*KH*KW] (contiguous in memory),
+// into one of two LDS buffers while the previous chunk is multiplied. The B operand of the
+// MFMA is read straight from the patch: element (k = (ic,kh,kw), pixel (r,c)) sits at
+// ic*PS + (r+kh)*WP + (c+kw). The k-order of the MFMA inside a chunk is tap-major: k-group t is
+// filter tap t, and its eight k-values are the eight channels (lane half g, register s ->
+// channel 4g+s). The patch address is then a wave-uniform term (tap offset + s*PS) plus a
+// per-lane term (pixel offset + 4g*PS): im2col costs one add per LDS read. The weight slab is
+// stored tap-major to match ([oc][tap][channel]), so a lane fetches its four channels with one
+// 128-bit read.
+namespace docc_k {
+
+template <int KH, int KW>
+struct ConvHaloKernel {
+    static constexpr int KHW = KH * KW;
+    static constexpr int CI = 8;                 // input channels per chunk
+    static constexpr int KC = CI * KHW;          // k per chunk (a multiple of 8)
+    static constexpr int NKG = KC / 8;           // k-groups per chunk
+    static constexpr int TN = 7;                 // MFMA column tiles per wave
+    static constexpr int BN = 2 * TN * 32;       // pixels per work-group (448)
+    static constexpr int LDA_S = KC + 4;
+    static constexpr int A_ELEMS = 64 * LDA_S;
+    static constexpr int NL = 24;                // patch elements per thread per chunk (upper bound)
+    static constexpr int NWV = (64 * KC / 4 + 255) / 256;   // weight float4s per thread per chunk
+
+    static __device__ __forceinline__ void run(const ConvParams& p, int TH) {
+        extern __shared__ __attribute__((aligned(16))) unsigned char docc_conv_lds[];
+        float* const lds = reinterpret_cast<float*>(docc_conv_lds);
+        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int l32 = lane & 31, g = lane >> 5;
+        const int ocw = wave & 1, pg = wave >> 1;
+
+        const int WP = p.OW + KW - 1, PR = TH + KH - 1, PS = PR * WP;
+        const int stage_elems = A_ELEMS + CI * PS;     // [weights | patch]
+        const int strips = (p.OH + TH - 1) / TH;
+        const int n = blockIdx.x / strips, oh0 = (blockIdx.x % strips) * TH;
+        const int oc0 = blockIdx.y * 64;
+        const int npix = TH * p.OW;                    // pixels of a full strip
+
+        // per-lane patch offsets for the 7 column tiles of this wave: pixel (r, c) of the strip, plus
+        // the channel block of this lane half
+        int pix4[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            int q = pg * (TN * 32) + j * 32 + l32;
+            q = q < npix ? q : 0;
+            pix4[j] = (q / p.OW) * WP + (q % p.OW) + 4 * g * PS;
+        }
+
+        // patch elements this thread moves per chunk: offset inside one image's channel chunk, or -1 (zero)
+        int poff[NL];
+        const int pelems = CI * PS;
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+            const int e = tid + i * 256;
+            int off = -1;
+            if (e < pelems) {
+                const int ic = e / PS, rem = e % PS;
+                const int ih = oh0 - p.pad_h + rem / WP, iw = rem % WP - p.pad_w;
+                if (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) off = (ic * p.H + ih) * p.W + iw;
+            }
+            poff[i] = off;
+        }
+        const float* xn = p.X + (long) n * p.C * p.H * p.W;
+        const int K = p.C * KHW;
+        // weight slab: row (oc) and float4 column of each of this thread's vectors
+        const float* wptr[NWV];
+        int wrow[NWV], wcol[NWV];
+#pragma unroll
+        for (int i = 0; i < NWV; i++) {
+            const int idx = tid + i * 256;
+            const int row = idx / (KC / 4), cv = idx % (KC / 4);
+            const int oc = oc0 + row < p.OC ? oc0 + row : p.OC - 1;
+            wptr[i] = p.Wt + (long) oc * K + cv * 4;
+            wrow[i] = idx < 64 * (KC / 4) ? row : -1;
+            wcol[i] = cv * 4;
+        }
+
+        f32x16 acc[TN];
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
+
+        float pv[NL];
+        f32x4 wv[NWV];
+        auto gload = [&](int ch) {
+            const float* xc = xn + (long) ch * CI * p.H * p.W;
+#pragma unroll
+            for (int i = 0; i < NL; i++) pv[i] = xc[poff[i] < 0 ? 0 : poff[i]];
+#pragma unroll
+            for (int i = 0; i < NWV; i++) wv[i] = *reinterpret_cast<const f32x4*>(wptr[i] + ch * KC);
+        };
+        auto stage = [&](int buf) {
+            float* as = lds + buf * stage_elems;
+            float* ps = as + A_ELEMS;
+#pragma unroll
+            for (int i = 0; i < NL; i++)
+                if (tid + i * 256 < pelems) ps[tid + i * 256] = poff[i] < 0 ? 0.f : pv[i];
+            // weights arrive as [oc][channel][tap] and are stored as [oc][tap][channel]
+#pragma unroll
+            for (int i = 0; i < NWV; i++) {
+                if (wrow[i] < 0) continue;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int k = wcol[i] + e;
+                    as[wrow[i] * LDA_S + (k % KHW) * CI + k / KHW] = wv[i][e];
+                }
+            }
+        };
+        auto compute = [&](int buf) {
+            const int abase = buf * stage_elems;            // wave-uniform, changes every chunk
+            const int pbase = abase + A_ELEMS;
+            const float* arow = lds + abase + (ocw * 32 + l32) * LDA_S + 4 * g;
+#pragma unroll
+            for (int t = 0; t < KHW; t++) {
+                const f32x4 a = *reinterpret_cast<const f32x4*>(arow + t * CI);
+                float b[TN][4];
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    const int u = pbase + s * PS + (t / KW) * WP + (t % KW);   // wave-uniform
+#pragma unroll
+                    for (int j = 0; j < TN; j++) b[j][s] = lds[u + pix4[j]];
+                }
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int s = 0; s < 4; s++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[j][s], acc[j], 0, 0, 0);
+            }
+        };
+
+        const int nch = p.C / CI;
+        gload(0);
+        stage(0);
+        __syncthreads();
+        int ch = 0;
+        for (; ch + 1 < nch; ch++) {
+            gload(ch + 1);
+            compute(ch & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            stage((ch + 1) & 1);
+            __syncthreads();
+        }
+        compute(ch & 1);
+
+        // epilogue: rows of the accumulator = output channels, columns = pixels of the strip
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int q = pg * (TN * 32) + j * 32 + l32;
+            const int oh = oh0 + q / p.OW, ow = q % p.OW;
+            if (q >= npix || oh >= p.OH) continue;
+            float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
+                if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = acc[j][r] + (p.bias ? p.bias[oc] : 0.f);
+            }
+        }
+    }
+};
+
+} // namespace docc_k
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1>::run(p, TH);
+}

@@ -1,4 +1,6 @@
 // Launcher for ml::Conv (see include/docc_rocm_ops.h).
+#include <cstdlib>
+
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
 
@@ -43,6 +45,22 @@ extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_
 
     ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
                  (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w};
+    // Stride-1, dilation-1 3x3 and 1x1 convolutions take the LDS-halo kernel: 64 output channels x a
+    // strip of TH full output rows (at most 448 pixels) per work-group, 8 input channels per chunk.
+    const bool halo_shape = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 &&
+                            ((KH == 3 && KW == 3) || (KH == 1 && KW == 1)) && C % 8 == 0 && C > 0 && OW <= 448 &&
+                            ((uintptr_t) Wt % 16 == 0) && ((C * KH * KW) % 4 == 0);
+    if (halo_shape && !std::getenv("DOCC_ROCM_CONV_GATHER")) {
+        int64_t TH = 448 / OW;
+        if (TH > OH) TH = OH;
+        const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch floats per input channel
+        const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * PS;      // weights + patch, floats
+        const int64_t strips = (OH + TH - 1) / TH;
+        if (8 * PS <= 24 * 256 && 2 * stage * 4 <= 160 * 1024 && N * strips < lim && (OC + 63) / 64 <= 65535) {
+            return launch(KH == 3 ? "docc_conv2d_f32_halo_3x3" : "docc_conv2d_f32_halo_1x1", (uint32_t) (N * strips),
+                          (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (2 * stage * 4), (hipStream_t) stream, p, (int) TH);
+        }
+    }
     constexpr int BM = 64, BN = 128, BK = 16;
     const int64_t tiles = ((OC + BM - 1) / BM) * ((N * OH * OW + BN - 1) / BN);
     if (tiles >= lim) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: too many tiles");

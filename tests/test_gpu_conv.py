@@ -36,6 +36,12 @@ CASES = [
     (1, 7, 8, 8, 9, 7, 7, (1, 1), (3, 3), (1, 1), True),       # kernel ~ image
     (4, 16, 20, 20, 32, 3, 3, (1, 1), (1, 1), (1, 1), True),
     (1, 1, 4, 4, 1, 3, 3, (1, 1), (2, 2), (1, 1), False),      # pad larger than needed
+    # stride-1 3x3 / 1x1 with C % 8 == 0: the LDS-halo kernel
+    (2, 8, 9, 11, 70, 3, 3, (1, 1), (1, 1), (1, 1), True),     # OC > 64 and not a multiple of 32, odd image
+    (3, 16, 30, 30, 40, 3, 3, (1, 1), (0, 0), (1, 1), False),   # no padding, several strips per image (OH % TH != 0)
+    (1, 24, 5, 100, 64, 3, 3, (1, 1), (2, 1), (1, 1), True),    # wide rows: 4 rows per strip, asymmetric pad sizes
+    (2, 32, 12, 12, 16, 1, 1, (1, 1), (0, 0), (1, 1), True),    # 1x1
+    (1, 8, 3, 448, 8, 3, 3, (1, 1), (1, 1), (1, 1), False),     # one row per strip
 ]
 
 
