@@ -16,6 +16,7 @@
 // for the next K-step is rebuilt in LDS by BK threads per step, so no thread
 // divides in the inner loop.
 #include "gemm_mfma.h"
+#include <type_traits>
 
 namespace docc_k {
 
@@ -200,31 +201,27 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 // (TH*OW <= 448 pixels = 14 MFMA column tiles). Wave w takes output-channel tile (w & 1) and
 // pixel tiles 7*(w >> 1) .. +6, so the four waves hold the whole strip in 7 accumulators each.
 // K = C*KH*KW is walked in chunks of 8 input channels. Per chunk the work-group stages
-//   - the input patch [8][TH+KH-1][OW+KW-1] (halo rows and columns included, zeros where the
-//     patch leaves the image): every input pixel is read from memory once per strip instead
-//     of KH*KW times, and
-//   - the weight slab [64][8*KH*KW] (contiguous in memory),
-// into one of two LDS buffers while the previous chunk is multiplied. The B operand of the
-// MFMA is read straight from the patch: element (k = (ic,kh,kw), pixel (r,c)) sits at
-// ic*PS + (r+kh)*WP + (c+kw). The k-order of the MFMA inside a chunk is tap-major: k-group t is
-// filter tap t, and its eight k-values are the eight channels (lane half g, register s ->
-// channel 4g+s). The patch address is then a wave-uniform term (tap offset + s*PS) plus a
-// per-lane term (pixel offset + 4g*PS): im2col costs one add per LDS read. The weight slab is
-// stored tap-major to match ([oc][tap][channel]), so a lane fetches its four channels with one
-// 128-bit read.
+//   - the input patch [TH+KH-1][OW+KW-1][8] (halo rows and columns included, zeros where the
+//     patch leaves the image, the eight channels of a pixel adjacent): every input pixel is read
+//     from memory once per strip instead of KH*KW times, and
+//   - the weight slab [64][8*KH*KW] (contiguous in memory), stored tap-major ([oc][tap][channel]),
+// into one of two LDS buffers while the previous chunk is multiplied. The k-order of the MFMA
+// inside a chunk is tap-major: k-group t is filter tap t, and its eight k-values are the eight
+// channels (lane half g, register s -> channel 4g+s). Both operands of the four MFMAs of a tap
+// are then one 128-bit LDS read per lane: the weights at [oc][t][4g..4g+3], the pixels at
+// [(r+kh)*WP + (c+kw)][4g..4g+3], whose address is a wave-uniform tap term plus a per-lane pixel
+// term: im2col costs one add per read.
 namespace docc_k {
 
 template <int KH, int KW>
 struct ConvHaloKernel {
     static constexpr int KHW = KH * KW;
     static constexpr int CI = 8;                 // input channels per chunk
-    static constexpr int KC = CI * KHW;          // k per chunk (a multiple of 8)
-    static constexpr int NKG = KC / 8;           // k-groups per chunk
+    static constexpr int KC = CI * KHW;          // k per chunk
     static constexpr int TN = 7;                 // MFMA column tiles per wave
-    static constexpr int BN = 2 * TN * 32;       // pixels per work-group (448)
     static constexpr int LDA_S = KC + 4;
     static constexpr int A_ELEMS = 64 * LDA_S;
-    static constexpr int NL = 24;                // patch elements per thread per chunk (upper bound)
+    static constexpr int NR = 3;                 // patch pixels per thread per chunk (upper bound)
     static constexpr int NWV = (64 * KC / 4 + 255) / 256;   // weight float4s per thread per chunk
 
     static __device__ __forceinline__ void run(const ConvParams& p, int TH) {
@@ -235,49 +232,51 @@ struct ConvHaloKernel {
         const int ocw = wave & 1, pg = wave >> 1;
 
         const int WP = p.OW + KW - 1, PR = TH + KH - 1, PS = PR * WP;
-        const int stage_elems = A_ELEMS + CI * PS;     // [weights | patch]
+        const int stage_elems = A_ELEMS + (PS + 1) * CI;    // [weights | patch | one spare pixel]
         const int strips = (p.OH + TH - 1) / TH;
         const int n = blockIdx.x / strips, oh0 = (blockIdx.x % strips) * TH;
         const int oc0 = blockIdx.y * 64;
         const int npix = TH * p.OW;                    // pixels of a full strip
 
-        // per-lane patch offsets for the 7 column tiles of this wave: pixel (r, c) of the strip, plus
-        // the channel block of this lane half
-        int pix4[TN];
+        // per-lane patch offsets (floats) of the 7 column tiles of this wave: pixel (r, c) of the
+        // strip and the channel half of this lane
+        int boff[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             int q = pg * (TN * 32) + j * 32 + l32;
             q = q < npix ? q : 0;
-            pix4[j] = (q / p.OW) * WP + (q % p.OW) + 4 * g * PS;
+            boff[j] = ((q / p.OW) * WP + (q % p.OW)) * CI + 4 * g;
         }
 
-        // patch elements this thread moves per chunk: offset inside one image's channel chunk, or -1 (zero)
-        int poff[NL];
-        const int pelems = CI * PS;
+        // patch pixels this thread moves per chunk: byte offset inside one channel plane (0 when the
+        // value is a zero of the padding), validity, and the LDS pixel slot (the spare one for
+        // threads beyond the patch)
+        unsigned goff[NR];
+        int slot[NR];
+        bool inside[NR];
 #pragma unroll
-        for (int i = 0; i < NL; i++) {
-            const int e = tid + i * 256;
-            int off = -1;
-            if (e < pelems) {
-                const int ic = e / PS, rem = e % PS;
-                const int ih = oh0 - p.pad_h + rem / WP, iw = rem % WP - p.pad_w;
-                if (ih >= 0 && ih < p.H && iw >= 0 && iw < p.W) off = (ic * p.H + ih) * p.W + iw;
-            }
-            poff[i] = off;
+        for (int r = 0; r < NR; r++) {
+            const int e = tid + r * 256;
+            const int ih = oh0 - p.pad_h + e / WP, iw = e % WP - p.pad_w;
+            inside[r] = e < PS && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            goff[r] = inside[r] ? 4u * (unsigned) (ih * p.W + iw) : 0u;
+            slot[r] = (e < PS ? e : PS) * CI;
         }
-        const float* xn = p.X + (long) n * p.C * p.H * p.W;
+        const long HW = (long) p.H * p.W;
+        const char* xn = reinterpret_cast<const char*>(p.X + (long) n * p.C * HW);
         const int K = p.C * KHW;
-        // weight slab: row (oc) and float4 column of each of this thread's vectors
-        const float* wptr[NWV];
-        int wrow[NWV], wcol[NWV];
+        // weight slab: memory holds [oc][channel][tap], LDS wants [oc][tap][channel]. Each of this
+        // thread's vectors is four channels of one (oc, tap): four loads KHW floats apart, one
+        // 128-bit LDS write (surplus threads aim at the spare pixel).
+        unsigned woff[NWV];
+        int wdst[NWV];
 #pragma unroll
         for (int i = 0; i < NWV; i++) {
             const int idx = tid + i * 256;
-            const int row = idx / (KC / 4), cv = idx % (KC / 4);
+            const int row = idx / (KC / 4), rem = idx % (KC / 4);     // rem = 2*tap + channel half
             const int oc = oc0 + row < p.OC ? oc0 + row : p.OC - 1;
-            wptr[i] = p.Wt + (long) oc * K + cv * 4;
-            wrow[i] = idx < 64 * (KC / 4) ? row : -1;
-            wcol[i] = cv * 4;
+            woff[i] = 4u * (unsigned) (oc * K + (rem & 1) * 4 * KHW + (rem >> 1));
+            wdst[i] = idx < 64 * (KC / 4) ? row * LDA_S + rem * 4 : A_ELEMS + PS * CI;
         }
 
         f32x16 acc[TN];
@@ -286,78 +285,173 @@ struct ConvHaloKernel {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[j][r] = 0.f;
 
-        float pv[NL];
+        // loads of one chunk: a wave-uniform base per channel plane plus the lane's 32-bit offset
+        float pv[NR][CI];
         f32x4 wv[NWV];
-        auto gload = [&](int ch) {
-            const float* xc = xn + (long) ch * CI * p.H * p.W;
+        // the staging work of one chunk in NSL slices: patch pixel i, or weight vector i - NR
+        constexpr int NSL = NR + NWV;
+        auto gload_slice = [&](int i, int ch) {
+            if (i < NR) {
+                const char* xc = xn + (long) ch * CI * HW * 4;
 #pragma unroll
-            for (int i = 0; i < NL; i++) pv[i] = xc[poff[i] < 0 ? 0 : poff[i]];
+                for (int c = 0; c < CI; c++) pv[i][c] = *reinterpret_cast<const float*>(xc + (long) c * HW * 4 + goff[i]);
+            } else {
+                const char* wc = reinterpret_cast<const char*>(p.Wt + ch * KC);
 #pragma unroll
-            for (int i = 0; i < NWV; i++) wv[i] = *reinterpret_cast<const f32x4*>(wptr[i] + ch * KC);
-        };
-        auto stage = [&](int buf) {
-            float* as = lds + buf * stage_elems;
-            float* ps = as + A_ELEMS;
-#pragma unroll
-            for (int i = 0; i < NL; i++)
-                if (tid + i * 256 < pelems) ps[tid + i * 256] = poff[i] < 0 ? 0.f : pv[i];
-            // weights arrive as [oc][channel][tap] and are stored as [oc][tap][channel]
-#pragma unroll
-            for (int i = 0; i < NWV; i++) {
-                if (wrow[i] < 0) continue;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int k = wcol[i] + e;
-                    as[wrow[i] * LDA_S + (k % KHW) * CI + k / KHW] = wv[i][e];
-                }
+                for (int e = 0; e < 4; e++) wv[i - NR][e] = *reinterpret_cast<const float*>(wc + woff[i - NR] + e * KHW * 4);
             }
         };
-        auto compute = [&](int buf) {
-            const int abase = buf * stage_elems;            // wave-uniform, changes every chunk
-            const int pbase = abase + A_ELEMS;
-            const float* arow = lds + abase + (ocw * 32 + l32) * LDA_S + 4 * g;
+        auto gload = [&](int ch) {
+#pragma unroll
+            for (int i = 0; i < NSL; i++) gload_slice(i, ch);
+        };
+        auto stage_slice = [&](int i, int base) {
+            float* as = lds + base;
+            if (i < NR) {
+                float* ps = as + A_ELEMS + slot[i];
+                f32x4 lo, hi;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    lo[c] = inside[i] ? pv[i][c] : 0.f;
+                    hi[c] = inside[i] ? pv[i][4 + c] : 0.f;
+                }
+                *reinterpret_cast<f32x4*>(ps) = lo;
+                *reinterpret_cast<f32x4*>(ps + 4) = hi;
+            } else {
+                *reinterpret_cast<f32x4*>(as + wdst[i - NR]) = wv[i - NR];
+            }
+        };
+
+        // The chunks form one stream of taps over a ring of three LDS buffers. While chunk ch is
+        // multiplied out of buffer cur, chunk ch+1 (its loads were issued a chunk earlier) is written
+        // into buffer nxt in slices spread over the taps T0..TB, each slice followed by the loads
+        // that refill its registers with chunk ch+2 (a burst of all loads at once would back up the
+        // address path and stall the wave), and the work-group meets at its one barrier per chunk. The last tap of the chunk already prefetches the first
+        // operands of the next one, so the matrix pipe never waits for the barrier and an LDS round
+        // trip in a row. Three buffers because a wave that has passed the barrier of chunk ch writes
+        // buffer (ch+2)%3 while a slower wave may still read (ch)%3 and everyone reads (ch+1)%3 next.
+        constexpr int T0 = 0;
+        constexpr int TB = KHW > 1 ? KHW - 2 : 0;
+        f32x4 a[2], b[2][TN];
+        auto fetch = [&](int base, int t, int to) {
+            const float* arow = lds + base + (ocw * 32 + l32) * LDA_S + 4 * g + t * CI;
+            a[to] = *reinterpret_cast<const f32x4*>(arow);
+            const float* bt = lds + base + A_ELEMS + ((t / KW) * WP + (t % KW)) * CI;     // wave-uniform
+#pragma unroll
+            for (int j = 0; j < TN; j++) b[to][j] = *reinterpret_cast<const f32x4*>(bt + boff[j]);
+        };
+        // par: parity of the chunk's first tap in the tap stream (operand registers alternate per tap).
+        // Each tap is one scheduling region: its 28 MFMAs, the LDS reads of the next tap's operands,
+        // and the staging slices that fall on it with their refill loads. The group barriers at the
+        // end of the region lay these out as "one MFMA, then one LDS read or one LDS write and one
+        // load" so that the matrix pipe is fed while the other pipes work.
+        float bias_r[16];
+        auto step = [&](auto par_c, auto has_next_c, int cur, int nxt, int after) {
+            constexpr int PAR = decltype(par_c)::value;
+            constexpr bool NEXT = decltype(has_next_c)::value;
+            if constexpr (!NEXT) {
+                // bias of this lane's 16 accumulator rows, fetched under the last chunk
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
+                    bias_r[r] = p.bias ? p.bias[oc < p.OC ? oc : p.OC - 1] : 0.f;
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int t = 0; t < KHW; t++) {
-                const f32x4 a = *reinterpret_cast<const f32x4*>(arow + t * CI);
-                float b[TN][4];
+                const int so = (t + PAR) & 1;
+                const bool reads = t + 1 < KHW || (NEXT && KHW > 1);
+                if (t + 1 < KHW) fetch(cur, t + 1, so ^ 1);
+                else if (NEXT && KHW > 1) fetch(nxt, 0, so ^ 1);      // the barrier of this chunk is behind us
 #pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    const int u = pbase + s * PS + (t / KW) * WP + (t % KW);   // wave-uniform
+                for (int s = 0; s < 4; s++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++) b[j][s] = lds[u + pix4[j]];
+                    for (int j = 0; j < TN; j++)
+                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[so][s], b[so][j][s], acc[j], 0, 0, 0);
+                int writes = 0, loads = 0;
+                if constexpr (NEXT) {
+                    const int i0 = t < T0 ? 0 : NSL * (t - T0) / (TB + 1 - T0);
+                    const int i1 = t < T0 ? 0 : (t > TB ? NSL : NSL * (t + 1 - T0) / (TB + 1 - T0));
+#pragma unroll
+                    for (int i = i0; i < i1; i++) {
+                        stage_slice(i, nxt);
+                        gload_slice(i, after);
+                        writes += i < NR ? 2 : 1;
+                        loads += i < NR ? CI : 4;
+                    }
                 }
 #pragma unroll
-                for (int j = 0; j < TN; j++)
-#pragma unroll
-                    for (int s = 0; s < 4; s++) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[j][s], acc[j], 0, 0, 0);
+                for (int i = 0; i < 4 * TN; i++) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // MFMA
+                    if (reads && i < TN + 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS read
+                    if (i >= TN + 1 && i - (TN + 1) < writes) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS write
+                    if (i >= TN + 1 && ((i - (TN + 1)) & 1) == 0 && (i - (TN + 1)) / 2 < loads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // load
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (NEXT) {
+                    if (t == TB) __syncthreads();
+                }
             }
+            if constexpr (NEXT && KHW == 1) fetch(nxt, 0, (PAR + 1) & 1);
         };
 
         const int nch = p.C / CI;
         gload(0);
-        stage(0);
+#pragma unroll
+        for (int i = 0; i < NSL; i++) stage_slice(i, 0);
+        if (nch > 1) gload(1);
         __syncthreads();
+        fetch(0, 0, 0);
+        // ring positions as LDS float offsets
+        int cur = 0, nxt = stage_elems;
+        auto advance = [&]() {
+            cur = nxt;
+            nxt = nxt + stage_elems;
+            if (nxt == 3 * stage_elems) nxt = 0;
+        };
+        constexpr int P1 = KHW & 1;      // parity of the second chunk of a pair
         int ch = 0;
-        for (; ch + 1 < nch; ch++) {
-            gload(ch + 1);
-            compute(ch & 1);
-            __builtin_amdgcn_sched_barrier(0);
-            stage((ch + 1) & 1);
-            __syncthreads();
+        for (; ch + 2 < nch; ch += 2) {
+            step(std::integral_constant<int, 0>{}, std::true_type{}, cur, nxt, ch + 2);
+            advance();
+            step(std::integral_constant<int, P1>{}, std::true_type{}, cur, nxt, ch + 3 < nch ? ch + 3 : nch - 1);
+            advance();
         }
-        compute(ch & 1);
+        if (ch + 2 == nch) {
+            step(std::integral_constant<int, 0>{}, std::true_type{}, cur, nxt, nch - 1);
+            advance();
+            step(std::integral_constant<int, P1>{}, std::false_type{}, cur, nxt, 0);
+        } else {
+            step(std::integral_constant<int, 0>{}, std::false_type{}, cur, nxt, 0);
+        }
 
-        // epilogue: rows of the accumulator = output channels, columns = pixels of the strip
+        // epilogue: rows of the accumulator = output channels, columns = pixels of the strip. A tile
+        // that lies wholly inside the output (the usual case) is stored by straight-line code; one
+        // branch per element costs more in instruction fetch than the stores themselves.
+        const bool whole = oc0 + 64 <= p.OC && oh0 + TH <= p.OH && (pg + 1) * (TN * 32) <= npix;
+        if (whole) {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int q = pg * (TN * 32) + j * 32 + l32;
-            const int oh = oh0 + q / p.OW, ow = q % p.OW;
-            if (q >= npix || oh >= p.OH) continue;
-            float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+            for (int j = 0; j < TN; j++) {
+                const int q = pg * (TN * 32) + j * 32 + l32;
+                float* ybase = p.Y + ((long) n * p.OC * p.OH + oh0 + q / p.OW) * p.OW + q % p.OW +
+                               (long) (oc0 + ocw * 32 + 4 * g) * p.OH * p.OW;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
-                if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = acc[j][r] + (p.bias ? p.bias[oc] : 0.f);
+                for (int r = 0; r < 16; r++)
+                    ybase[(long) (8 * (r / 4) + r % 4) * p.OH * p.OW] = acc[j][r] + bias_r[r];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                const int q = pg * (TN * 32) + j * 32 + l32;
+                const int oh = oh0 + q / p.OW, ow = q % p.OW;
+                if (q >= npix || oh >= p.OH) continue;
+                float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
+                    if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = acc[j][r] + bias_r[r];
+                }
             }
         }
     }

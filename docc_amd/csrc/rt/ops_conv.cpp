@@ -53,12 +53,12 @@ extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_
     if (halo_shape && !std::getenv("DOCC_ROCM_CONV_GATHER")) {
         int64_t TH = 448 / OW;
         if (TH > OH) TH = OH;
-        const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch floats per input channel
-        const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * PS;      // weights + patch, floats
+        const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch pixels
+        const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
-        if (8 * PS <= 24 * 256 && 2 * stage * 4 <= 160 * 1024 && N * strips < lim && (OC + 63) / 64 <= 65535) {
+        if (PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
             return launch(KH == 3 ? "docc_conv2d_f32_halo_3x3" : "docc_conv2d_f32_halo_1x1", (uint32_t) (N * strips),
-                          (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (2 * stage * 4), (hipStream_t) stream, p, (int) TH);
+                          (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
         }
     }
     constexpr int BM = 64, BN = 128, BK = 16;
