@@ -17,6 +17,7 @@
 #pragma once
 
 #include "gemm_mfma.h"
+#include <type_traits>
 
 namespace docc_k {
 
@@ -77,12 +78,18 @@ struct AsyncTile {
     // element offset (inside a stage) of the granule that holds columns cv*VEC .. of `row`
     static __device__ __forceinline__ int granule_offset(int row, int cv) { return (row * VPR + (cv ^ swz(row))) * VEC; }
 
-    const T* p[NV];
-    long kstep;
+    const char* base;      // wave-uniform: origin of the tile of the current K-step
+    unsigned off[NV];      // this lane's granules: byte offsets from the origin
+    long kstep_bytes;
 
-    __device__ __forceinline__ void init(const T* __restrict__ base, long ld, long r0, long c0, long rmax, long cmax, int tid) {
-        kstep = K_ALONG_COLS ? (long) COLS : (long) ROWS * ld;
+    // The tile covers rows r0.. and columns c0.. of an rmax x cmax operand; out-of-range rows (columns
+    // of a k-major tile) are clamped to the edge - their products land in rows/columns of C that are
+    // never stored. The host guarantees that ROWS*ld*sizeof(T) fits the 32-bit offsets.
+    __device__ __forceinline__ void init(const T* __restrict__ mat, long ld, long r0, long c0, long rmax, long cmax, int tid) {
+        kstep_bytes = (K_ALONG_COLS ? (long) COLS : (long) ROWS * ld) * (long) sizeof(T);
         const int wave = tid >> 6, lane = tid & 63;
+        const long cbase = K_ALONG_COLS ? c0 : (c0 + VEC <= cmax ? c0 : cmax - VEC);
+        base = reinterpret_cast<const char*>(mat + r0 * ld + cbase);
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int g = (i * NW + wave) * 64 + lane;   // the LDS slot this lane fills
@@ -90,21 +97,19 @@ struct AsyncTile {
             long r = r0 + row, c = c0 + (long) cv * VEC;
             if (K_ALONG_COLS) r = r < rmax ? r : rmax - 1;
             else c = c + VEC <= cmax ? c : cmax - VEC;
-            p[i] = base + r * ld + c;
+            off[i] = (unsigned) (((r - r0) * ld + (c - cbase)) * (long) sizeof(T));
         }
     }
 
-    __device__ __forceinline__ void advance() {
-#pragma unroll
-        for (int i = 0; i < NV; i++) p[i] += kstep;
-    }
+    __device__ __forceinline__ void advance() { base += kstep_bytes; }
 
-    // asynchronous copy of the current K-step into `stage`
-    __device__ __forceinline__ void issue(T* stage, int tid) const {
-        const int wave = tid >> 6;
+    // asynchronous copy of granule i of the current K-step into `stage` (wave: wave-uniform index)
+    __device__ __forceinline__ void issue_one(T* stage, int i, int wave) const {
+        __builtin_amdgcn_global_load_lds((global_ptr_t) (base + off[i]), (lds_ptr_t) (stage + (i * NW + wave) * 64 * VEC), 16, 0, 0);
+    }
+    __device__ __forceinline__ void issue(T* stage, int wave) const {
 #pragma unroll
-        for (int i = 0; i < NV; i++)
-            __builtin_amdgcn_global_load_lds((global_ptr_t) p[i], (lds_ptr_t) (stage + (i * NW + wave) * 64 * VEC), 16, 0, 0);
+        for (int i = 0; i < NV; i++) issue_one(stage, i, wave);
     }
 
     // the partial last K-step through registers: k >= kleft reads as zero
@@ -118,7 +123,7 @@ struct AsyncTile {
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
                 const bool ok = K_ALONG_COLS ? (cv * VEC + e < kleft) : (row < kleft);
-                v[e] = ok ? p[i][e] : (T) 0;
+                v[e] = ok ? reinterpret_cast<const T*>(base + off[i])[e] : (T) 0;
             }
             *reinterpret_cast<vec_t*>(stage + g * VEC) = v;
         }
@@ -150,7 +155,7 @@ struct AsyncGemmKernel {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
         T* const lds = reinterpret_cast<T*>(docc_gemm_lds);
 
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int wm = wave / WN, wn = wave % WN;
         const int tiles_m = (int) ((M + BM - 1) / BM), tiles_n = (int) ((N + BN - 1) / BN);
         int tm, tn;
@@ -175,78 +180,83 @@ struct AsyncGemmKernel {
         const int lidx = lane % MT;     // row of A / column of B inside an MFMA tile
         const int lg = lane / MT;       // k-group of this lane
 
-        // ---- the multiply of one staged K-step ---------------------------------------------
-        auto compute = [&](const T* stage) {
-            const T* as = stage;
-            const T* bs = stage + ATile::ELEMS;
+        // ---- operands of one inner step (16 k for bf16, KG k otherwise) in two register sets --------
+        constexpr int VK = VEC;
+        constexpr int NKI = (sizeof(T) == 2) ? BK / 16 : BK / KG;     // inner steps per staged K-step
+        static_assert(NKI % 2 == 0, "operand register sets alternate per inner step");
+        bf16x8 ah[2][TM], bh[2][TN];             // bf16
+        T a[2][TM][VK], b[2][TN][VK];            // fp32 / fp64
+        // piece idx of a fetch: operand tile idx of A (idx < TM) or tile idx - TM of B
+        constexpr int NPIECE = TM + TN;
+        auto fetch_piece = [&](const T* stage, int ki, int to, int idx) {
+            const bool is_a = idx < TM;
+            const int t = is_a ? idx : idx - TM;
+            const T* base = is_a ? stage : stage + ATile::ELEMS;
+            const int idx0 = is_a ? wm * WTM + t * MT : wn * WTN + t * MT;
+            const bool kc = is_a ? A_KC : B_KC;
+            auto goff = [&](int row, int cv) { return is_a ? ATile::granule_offset(row, cv) : BTile::granule_offset(row, cv); };
             if constexpr (sizeof(T) == 2) {
                 // bf16: one MFMA consumes 16 k; lane (idx, g) supplies k = 8g .. 8g+7
-#pragma unroll
-                for (int ks = 0; ks < BK / 16; ks++) {
-                    bf16x8 a[TM], b[TN];
-                    auto fetch = [&](auto tile_tag, const T* base, int idx0, bool kc) -> bf16x8 {
-                        typedef decltype(tile_tag) Tile;
-                        if (kc) {
-                            const int row = idx0 + lidx;
-                            const u16x8a v = *reinterpret_cast<const u16x8a*>(base + Tile::granule_offset(row, ks * 2 + lg));
-                            return __builtin_bit_cast(bf16x8, v);
-                        }
-                        // transposed read: 16-lane group = 4 k-rows x 16 columns, see gemm_bf16.hip
-                        const int s = lane & 15, grp = lane >> 4;
-                        const int krow = ks * 16 + 8 * (grp >> 1) + (s >> 2);
-                        const int col = idx0 + 16 * (grp & 1) + 4 * (s & 3);
-                        typedef __attribute__((address_space(3))) s16x4a lds_s16x4;
-                        const T* plo = base + Tile::granule_offset(krow, col / 8) + (col & 7);
-                        const T* phi = base + Tile::granule_offset(krow + 4, col / 8) + (col & 7);
-                        const s16x4a lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
-                        const s16x4a hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
-                        const s16x8a v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        return __builtin_bit_cast(bf16x8, v);
-                    };
-#pragma unroll
-                    for (int i = 0; i < TM; i++) a[i] = fetch(ATile{}, as, wm * WTM + i * MT, A_KC);
-#pragma unroll
-                    for (int j = 0; j < TN; j++) b[j] = fetch(BTile{}, bs, wn * WTN + j * MT, B_KC);
-#pragma unroll
-                    for (int i = 0; i < TM; i++)
-#pragma unroll
-                        for (int j = 0; j < TN; j++)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+                bf16x8 r;
+                if (kc) {
+                    const u16x8a v = *reinterpret_cast<const u16x8a*>(base + goff(idx0 + lidx, ki * 2 + lg));
+                    r = __builtin_bit_cast(bf16x8, v);
+                } else {
+                    // transposed read: 16-lane group = 4 k-rows x 16 columns, see gemm_bf16.hip
+                    const int s = lane & 15, grp = lane >> 4;
+                    const int krow = ki * 16 + 8 * (grp >> 1) + (s >> 2);
+                    const int col = idx0 + 16 * (grp & 1) + 4 * (s & 3);
+                    typedef __attribute__((address_space(3))) s16x4a lds_s16x4;
+                    const T* plo = base + goff(krow, col / 8) + (col & 7);
+                    const T* phi = base + goff(krow + 4, col / 8) + (col & 7);
+                    const s16x4a lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
+                    const s16x4a hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
+                    const s16x8a v = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    r = __builtin_bit_cast(bf16x8, v);
                 }
+                if (is_a) ah[to][t] = r;
+                else bh[to][t] = r;
             } else {
-                // fp32 / fp64: lane group g owns k = kg*KG + g*VK .. +VK-1 (VK = VEC: one granule)
-                constexpr int VK = VEC;
+                // fp32 / fp64: lane group g owns k = ki*KG + g*VK .. +VK-1 (VK = VEC: one granule)
+                T* out = is_a ? a[to][t] : b[to][t];
+                if (kc) {
+                    const vec_t v = *reinterpret_cast<const vec_t*>(base + goff(idx0 + lidx, ki * X::G + lg));
 #pragma unroll
-                for (int kg = 0; kg < BK / KG; kg++) {
-                    T a[TM][VK], b[TN][VK];
-                    auto fetch = [&](auto tile_tag, const T* base, int idx0, bool kc, T* out) {
-                        typedef decltype(tile_tag) Tile;
-                        if (kc) {
-                            const vec_t v = *reinterpret_cast<const vec_t*>(base + Tile::granule_offset(idx0 + lidx, kg * X::G + lg));
+                    for (int s = 0; s < VK; s++) out[s] = v[s];
+                } else {
+                    const int col = idx0 + lidx;
 #pragma unroll
-                            for (int s = 0; s < VK; s++) out[s] = v[s];
-                        } else {
-                            const int col = idx0 + lidx;
+                    for (int s = 0; s < VK; s++) out[s] = base[goff(ki * KG + lg * VK + s, col / VEC) + col % VEC];
+                }
+            }
+        };
+        auto fetch = [&](const T* stage, int ki, int to) {
 #pragma unroll
-                            for (int s = 0; s < VK; s++)
-                                out[s] = base[Tile::granule_offset(kg * KG + lg * VK + s, col / VEC) + col % VEC];
-                        }
-                    };
+            for (int idx = 0; idx < NPIECE; idx++) fetch_piece(stage, ki, to, idx);
+        };
+        // MFMAs lo .. hi-1 of the NM of one inner step (order: k-slice, tile row, tile column)
+        constexpr int NM = (sizeof(T) == 2 ? 1 : VK) * TM * TN;
+        auto mma = [&](int from, int lo, int hi) {
 #pragma unroll
-                    for (int i = 0; i < TM; i++) fetch(ATile{}, as, wm * WTM + i * MT, A_KC, a[i]);
-#pragma unroll
-                    for (int j = 0; j < TN; j++) fetch(BTile{}, bs, wn * WTN + j * MT, B_KC, b[j]);
-#pragma unroll
-                    for (int s = 0; s < VK; s++)
-#pragma unroll
-                        for (int i = 0; i < TM; i++)
-#pragma unroll
-                            for (int j = 0; j < TN; j++) acc[i][j] = Mfma<T>::mfma(a[i][s], b[j][s], acc[i][j]);
+            for (int m = lo; m < (hi < NM ? hi : NM); m++) {
+                const int s = m / (TM * TN), i = (m / TN) % TM, j = m % TN;
+                if constexpr (sizeof(T) == 2) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ah[from][i], bh[from][j], acc[i][j], 0, 0, 0);
+                } else {
+                    acc[i][j] = Mfma<T>::mfma(a[from][i][s], b[from][j][s], acc[i][j]);
                 }
             }
         };
 
         // ---- pipeline --------------------------------------------------------------------------
+        // The K-steps are copied STAGES ahead into a ring of LDS stages; the operands of an inner
+        // step are read from LDS one inner step ahead into the other register set. The last inner
+        // step of K-step kt therefore already needs K-step kt+1: that is where the wave waits for
+        // its own copies of kt+1, meets the others at the barrier (after which nobody reads stage kt
+        // any more: its last operands are in registers), refills stage kt with step kt+STAGES and
+        // reads the first operands of kt+1. Each of these blocks is issued behind one MFMA of the
+        // current inner step (fences keep them there), so the matrix pipe has work while the other
+        // pipes are fed and the LDS round trip passes under the remaining MFMAs.
         const int full = (int) (K / BK);
         const int kleft = (int) (K - (long) full * BK);
         const int ksteps = full + (kleft > 0 ? 1 : 0);
@@ -258,51 +268,99 @@ struct AsyncGemmKernel {
             }
             T* st = stage_of(kt);
             if (kt < full) {
-                ta.issue(st, tid);
-                tb.issue(st + ATile::ELEMS, tid);
+                ta.issue(st, wave);
+                tb.issue(st + ATile::ELEMS, wave);
             } else {
                 ta.copy_tail(st, kleft, tid);
                 tb.copy_tail(st + ATile::ELEMS, kleft, tid);
             }
         };
-#pragma unroll
-        for (int s = 0; s < STAGES - 1; s++)
-            if (s < ksteps) fill(s);
-
-        for (int kt = 0; kt < ksteps; kt++) {
-            // step kt has landed once at most the loads of the STAGES-2 newer full steps are outstanding;
-            // near the end fewer newer steps exist, so everything is awaited
+        // step kt has landed once at most the loads of the STAGES-2 newer full steps are outstanding;
+        // near the end fewer newer steps exist, so everything is awaited
+        auto arrive = [&](int kt) {
             if (kt + STAGES - 2 < full) {
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * LOADS_PER_STEP) : "memory");
             } else {
                 asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
             }
-            __builtin_amdgcn_s_barrier();   // all waves' parts of step kt are in LDS; step kt-1 is fully consumed
+            __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (kt + STAGES - 1 < ksteps) fill(kt + STAGES - 1);   // into the stage step kt-1 occupied
-            compute(stage_of(kt));
-        }
+        };
+#pragma unroll
+        for (int s = 0; s < STAGES - 1; s++)
+            if (s < ksteps) fill(s);
+        arrive(0);
+        if (STAGES - 1 < ksteps) fill(STAGES - 1);
+        fetch(stage_of(0), 0, 0);
+
+        // the last K-step has no successor: it is peeled so that the loop body is free of branches
+        // around MFMAs (they would make the compiler copy accumulators between the paths)
+        // One inner step: its NM MFMAs, each followed (and fenced, so that it stays there) by its
+        // share of the other pipes' work - a lump of LDS reads or copies between two MFMAs would
+        // leave the matrix pipe idle while the lump is issued.
+        //   inner steps but the last: the LDS reads of the next inner step's operands;
+        //   last inner step, after its first MFMA: wait + barrier (see above), then the copies that
+        //   refill stage kt and the LDS reads of step kt+1's first operands.
+        // mode 0: steady state (the refill is a full asynchronous step, nothing in the body branches);
+        // mode 1: near the end (the refill may be the K tail or absent); mode 2: the last step
+        auto kstep = [&](int kt, auto mode_c) {
+            constexpr int MODE = decltype(mode_c)::value;
+            constexpr bool NEXT = MODE != 2;
+            const T* st = stage_of(kt);
+#pragma unroll
+            for (int ki = 0; ki < NKI; ki++) {
+                if (ki + 1 < NKI) {
+#pragma unroll
+                    for (int n = 0; n < NM; n++) {
+                        mma(ki & 1, n, n + 1);
+#pragma unroll
+                        for (int q = n * NPIECE / NM; q < (n + 1) * NPIECE / NM; q++) fetch_piece(st, ki + 1, (ki + 1) & 1, q);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else if (NEXT) {
+                    mma(ki & 1, 0, 1);
+                    __builtin_amdgcn_sched_barrier(0);
+                    T* dst = lds + (kt % STAGES) * STAGE_ELEMS;     // stage kt, free after the barrier
+                    if (MODE == 0) {
+                        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * LOADS_PER_STEP) : "memory");
+                        __builtin_amdgcn_s_barrier();
+                        asm volatile("" ::: "memory");
+                        ta.advance();
+                        tb.advance();
+                    } else {
+                        arrive(kt + 1);
+                        if (kt + STAGES < ksteps) fill(kt + STAGES);
+                    }
+                    const T* nst = stage_of(kt + 1);
+#pragma unroll
+                    for (int n = 1; n < NM; n++) {
+                        mma(ki & 1, n, n + 1);
+                        if (MODE == 0) {
+#pragma unroll
+                            for (int q = (n - 1) * LOADS_PER_STEP / (NM - 1); q < n * LOADS_PER_STEP / (NM - 1); q++) {
+                                if (q < ATile::NV) ta.issue_one(dst, q, wave);
+                                else tb.issue_one(dst + ATile::ELEMS, q - ATile::NV, wave);
+                            }
+                        }
+#pragma unroll
+                        for (int q = (n - 1) * NPIECE / (NM - 1); q < n * NPIECE / (NM - 1); q++) fetch_piece(nst, 0, 0, q);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
+                    mma(ki & 1, 0, NM);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        int kt = 0;
+        for (; kt + STAGES < full; kt++) kstep(kt, std::integral_constant<int, 0>{});
+        for (; kt + 1 < ksteps; kt++) kstep(kt, std::integral_constant<int, 1>{});
+        kstep(kt, std::integral_constant<int, 2>{});
 
         // ---- epilogue ------------------------------------------------------------------------------
-        const bool use_c = (beta != (out_t) 0);
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const long col = n0 + wn * WTN + j * MT + lidx;
-#pragma unroll
-                for (int r = 0; r < X::NACC; r++) {
-                    const int rr = (sizeof(T) == 8) ? Mfma<double>::acc_row(lane, r) : Mfma<float>::acc_row(lane, r);
-                    const long row = m0 + wm * WTM + i * MT + rr;
-                    if (row < M && col < N) {
-                        out_t* p = C + row * ldc + col;
-                        out_t val = alpha * acc[i][j][r];
-                        if (use_c) val += beta * (*p);
-                        *p = val;
-                    }
-                }
-            }
-        }
+        gemm_store_wave<TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lidx, alpha, beta, acc, [&](int r) {
+            return (sizeof(T) == 8) ? Mfma<double>::acc_row(lane, r) : Mfma<float>::acc_row(lane, r);
+        });
     }
 };
 

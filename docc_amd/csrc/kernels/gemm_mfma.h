@@ -60,6 +60,60 @@ struct Mfma<double> {
     static __device__ __forceinline__ int acc_row(int lane, int r) { return 4 * r + lane / 16; }
 };
 
+// Epilogue of one wave: C = alpha*acc + beta*C over its TM x TN accumulator tiles (C is not read
+// when beta == 0). (row0, col0) is the wave tile's origin in C, lcol = lane % MT the lane's column,
+// acc_row(r) the row of accumulator register r inside a tile for this lane. A wave tile that lies
+// wholly inside C - all but the last row and column of tiles - is stored by straight-line code:
+// with one bounds branch per element the instruction fetch of the cold, branchy epilogue costs
+// more than the stores themselves.
+template <int TM, int TN, int MT, int NACC, typename OT, typename AccT, typename RowFn>
+__device__ __forceinline__ void gemm_store_wave(OT* C, long ldc, long M, long N, long row0, long col0, int lcol,
+                                                OT alpha, OT beta, AccT (&acc)[TM][TN], RowFn acc_row) {
+    const bool use_c = (beta != (OT) 0);
+    if (row0 + TM * MT <= M && col0 + TN * MT <= N) {
+        OT* base = C + (row0 + acc_row(0)) * ldc + col0 + lcol;
+        if (!use_c) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < NACC; r++)
+                        base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT] = alpha * acc[i][j][r];
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    OT old[NACC];
+#pragma unroll
+                    for (int r = 0; r < NACC; r++) old[r] = base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT];
+#pragma unroll
+                    for (int r = 0; r < NACC; r++)
+                        base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT] = alpha * acc[i][j][r] + beta * old[r];
+                }
+        }
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const long col = col0 + j * MT + lcol;
+#pragma unroll
+            for (int r = 0; r < NACC; r++) {
+                const long row = row0 + i * MT + acc_row(r);
+                if (row < M && col < N) {
+                    OT* p = C + row * ldc + col;
+                    OT val = alpha * acc[i][j][r];
+                    if (use_c) val += beta * (*p);
+                    *p = val;
+                }
+            }
+        }
+    }
+}
+
 // Tile id -> tile coordinates: XCD-contiguous renumbering, then grouped
 // ordering (GROUP_M rows of tiles at a time) inside each XCD's range.
 __device__ __forceinline__ void gemm_tile_coords(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
@@ -314,25 +368,8 @@ struct GemmKernel {
         }
         compute(kt & 1);
 
-        // epilogue: C = alpha*acc + beta*C; C is not read when beta == 0
-        const bool use_c = (beta != (T) 0);
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const long col = n0 + wn * WTN + j * MT + lrow;
-#pragma unroll
-                for (int r = 0; r < X::NACC; r++) {
-                    const long row = m0 + wm * WTM + i * MT + X::acc_row(lane, r);
-                    if (row < M && col < N) {
-                        T* p = C + row * ldc + col;
-                        T val = alpha * acc[i][j][r];
-                        if (use_c) val += beta * (*p);
-                        *p = val;
-                    }
-                }
-            }
-        }
+        gemm_store_wave<TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lrow, alpha, beta, acc,
+                                             [&](int r) { return X::acc_row(lane, r); });
     }
 };
 
