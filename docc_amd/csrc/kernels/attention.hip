@@ -22,7 +22,16 @@
 //                                                from the S^T accumulator registers as they
 //                                                are (the k-order of the MFMA is permuted to
 //                                                the accumulator's row order on both operands).
+//
+// The softmax arithmetic, not the MFMAs, is the longer half of a block (32 scores per lane:
+// exp2, scale, max, sum, pack), so it is kept to the minimum: v_max3 for the maximum, one
+// v_permlane32_swap for the exchange, v_cvt_pk_bf16_f32 for the packing, the row sum taken
+// from the packed values with v_dot2c_f32_bf16 (it then sums exactly what the second product
+// multiplies), and the rescale of the output skipped while no lane's maximum moves. The scores
+// of block i+1 are issued to the matrix pipe before the softmax of block i starts, and K/V
+// blocks arrive in a ring of LDS stages by asynchronous global->LDS copies.
 #include "gemm_mfma.h"
+#include <type_traits>
 
 namespace docc_k {
 
@@ -30,6 +39,9 @@ typedef uint16_t u16x8_t __attribute__((ext_vector_type(8)));
 typedef uint16_t u16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) void* attn_lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* attn_global_ptr_t;
 
 template <>
 struct Mfma<uint16_t> {
@@ -38,11 +50,28 @@ struct Mfma<uint16_t> {
 };
 
 constexpr int kHeadDim = 64;
-constexpr int kBlockQ = 128;   // queries per work-group
-constexpr int kBlockKV = 64;   // keys per step
-constexpr int kLdK = kHeadDim + 8;    // K tile [key][d], padded
-constexpr int kLdV = kHeadDim + 16;   // V tile [key][d], padded for the transposed reads
-constexpr int kKElems = kBlockKV * kLdK, kVElems = kBlockKV * kLdV;
+constexpr int kBlockQ = 128;     // queries per work-group
+constexpr int kBlockKV = 64;     // keys per step
+constexpr int kAttnStages = 2;   // LDS ring depth: block kb+1 is copied while block kb is worked on
+constexpr int kTileElems = kBlockKV * kHeadDim;          // one K or V block, unpadded, 16-byte granules swizzled
+constexpr int kStageElems = 2 * kTileElems;              // [K | V]
+
+// granule (8 bf16) index inside a row of 8 granules, swizzled so that the reads below are conflict-free:
+// K: a 128-bit read touches 16 consecutive rows at one granule column; V: a transposed 64-bit read
+// touches 4 consecutive rows x 4 granule columns
+__device__ __forceinline__ int attn_k_off(int row, int cv) { return (row * 8 + (cv ^ ((row >> 1) & 7))) * 8; }
+__device__ __forceinline__ int attn_v_off(int row, int cv) { return (row * 8 + (cv ^ (((row >> 1) & 1) << 2))) * 8; }
+
+// x of lanes 0..31 (which = 0) or of lanes 32..63 (which = 1), seen from both halves of the wave:
+// v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second.
+// The second operand goes through an empty asm so that the compiler cannot treat the two results
+// of a swap of equal inputs as equal.
+__device__ __forceinline__ float half_swap(float x, int which) {
+    unsigned a = __builtin_bit_cast(unsigned, x), b = a;
+    asm volatile("" : "+v"(b));
+    const auto sw = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    return __builtin_bit_cast(float, which ? sw[1] : sw[0]);
+}
 
 template <bool OUT_BF16>
 __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
@@ -50,14 +79,13 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
                                                   int SKV, float scale_log2e) {
     extern __shared__ __attribute__((aligned(16))) unsigned char docc_attn_lds[];
     uint16_t* const lds = reinterpret_cast<uint16_t*>(docc_attn_lds);
-    constexpr int V_BASE = 2 * kKElems;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qj = lane & 31, g = lane >> 5;
     const long bh = blockIdx.y;
     const uint16_t* Qh = Q + bh * (long) SQ * kHeadDim;
-    const uint16_t* Kh = K + bh * (long) SKV * kHeadDim;
-    const uint16_t* Vh = V + bh * (long) SKV * kHeadDim;
+    const char* Kh = reinterpret_cast<const char*>(K + bh * (long) SKV * kHeadDim);
+    const char* Vh = reinterpret_cast<const char*>(V + bh * (long) SKV * kHeadDim);
     const int q = blockIdx.x * kBlockQ + wave * 32 + qj;   // this lane's query
 
     // Q^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q
@@ -69,6 +97,52 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         bq[ks] = __builtin_bit_cast(bf16x8, v);
     }
 
+    const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
+    const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
+
+    // K/V copies: a block is 512 granules of 16 bytes per tensor, two per thread. LDS slot s (in copy
+    // order: lane-contiguous) holds row s/8, granule column (s%8) ^ swizzle(row).
+    unsigned koff[2], voff[2];     // byte offsets of this lane's granules inside a full block
+    int krow[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int s = (i * 4 + wave) * 64 + lane;
+        const int row = s >> 3, cs = s & 7;
+        krow[i] = row;
+        koff[i] = (unsigned) ((row * 8 + (cs ^ ((row >> 1) & 7))) * 16);
+        voff[i] = (unsigned) ((row * 8 + (cs ^ (((row >> 1) & 1) << 2))) * 16);
+    }
+    auto issue = [&](int kb) {   // starts the copy of block kb into its stage
+        uint16_t* st = lds + (kb % kAttnStages) * kStageElems;
+        const char* kp = Kh + (long) kb * (kTileElems * 2);
+        const char* vp = Vh + (long) kb * (kTileElems * 2);
+        const bool partial = kb >= full_blocks;     // rows past the end copy the last key (scores masked, V zeroed below)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            unsigned ko = koff[i], vo = voff[i];
+            if (partial && krow[i] >= keys_left) {
+                ko -= (unsigned) ((krow[i] - (keys_left - 1)) * 128);
+                vo -= (unsigned) ((krow[i] - (keys_left - 1)) * 128);
+            }
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + ko), (attn_lds_ptr_t) (st + (i * 4 + wave) * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + vo), (attn_lds_ptr_t) (st + kTileElems + (i * 4 + wave) * 512), 16, 0, 0);
+        }
+    };
+    // block kb has landed in every wave's view; rows of a partial last V block are cleared so that
+    // 0 * (copied value) cannot produce a NaN
+    auto arrive = [&](int kb, int newer_blocks) {
+        (void) newer_blocks;
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (kb >= full_blocks) {
+            uint16_t* vt = lds + (kb % kAttnStages) * kStageElems + kTileElems;
+            const u16x8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int s = keys_left * 8 + tid; s < 512; s += 256) *reinterpret_cast<u16x8_t*>(vt + s * 8) = z;
+            __syncthreads();
+        }
+    };
+
     f32x16 ot[2];   // O^T tiles: d = 32*dt + acc_row(lane, r), column = this lane's query
 #pragma unroll
     for (int dt = 0; dt < 2; dt++)
@@ -77,58 +151,39 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     float m_run = -__builtin_huge_valf();   // running max of scale*log2e*score
     float l_part = 0.f;                     // this lane's part of the running sum (its 32 keys per block)
 
-    // K and V blocks: 64 keys x 64 d, walked along the keys; keys past the end read as zero
-    typedef TileLoader<uint16_t, kBlockKV, kHeadDim, 256, true, false> KVLoader;
-    KVLoader lk, lv;
-    const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
-    const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
-    lk.init(Kh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
-    lv.init(Vh, kHeadDim, 0, 0, SKV, kHeadDim, tid);
-    if (full_blocks > 0) {
-        lk.load_full();
-        lv.load_full();
-    } else {
-        lk.load_tail(keys_left, tid);
-        lv.load_tail(keys_left, tid);
-    }
-    lk.template store<kLdK>(lds, tid);
-    lv.template store<kLdV>(lds + V_BASE, tid);
-    __syncthreads();
-
     // lane roles for the transposed V reads (see gemm_bf16.hip)
     const int ts = lane & 15, tgrp = lane >> 4;
     const int tr_row = 4 * (tgrp >> 1) + (ts >> 2);            // + 16*(u%2) + 32*t (+8 for the high half)
     const int tr_col = 16 * (tgrp & 1) + 4 * (ts & 3);         // + 32*dt
     typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
 
-    for (int kb = 0; kb < nblocks; kb++) {
-        const int cur = kb & 1;
-        if (kb + 1 < full_blocks) {
-            lk.advance();
-            lv.advance();
-            lk.load_full();
-            lv.load_full();
-        } else if (kb + 1 < nblocks) {
-            lk.advance();
-            lv.advance();
-            lk.load_tail(keys_left, tid);
-            lv.load_tail(keys_left, tid);
-        }
-        const uint16_t* ks_ = lds + cur * kKElems;
-        const uint16_t* vs_ = lds + V_BASE + cur * kVElems;
+    f32x16 st[2];
 
-        // scores, transposed: st[t][r] = <K[32t + acc_row(r)], Q[q]>
-        f32x16 st[2];
+    // scores, transposed: s[t][r] = <K[32t + acc_row(r)], Q[q]> for the block in `stage`
+    auto scores = [&](int kb, f32x16 (&s)[2]) {
+        const uint16_t* ks_ = lds + (kb % kAttnStages) * kStageElems;
 #pragma unroll
         for (int t = 0; t < 2; t++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) st[t][r] = 0.f;
+            for (int r = 0; r < 16; r++) s[t][r] = 0.f;
 #pragma unroll
             for (int ks = 0; ks < 4; ks++) {
-                const u16x8_t kv = *reinterpret_cast<const u16x8_t*>(ks_ + (32 * t + qj) * kLdK + 16 * ks + 8 * g);
-                st[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv), bq[ks], st[t], 0, 0, 0);
+                const u16x8_t kv = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off(32 * t + qj, 2 * ks + g));
+                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv), bq[ks], s[t], 0, 0, 0);
             }
         }
+    };
+
+    // one block: scores -> softmax -> O^T += V^T P^T. The kernel is sized for four waves per SIMD
+    // (128 registers, 32 KB of LDS per work-group): a wave issues a vector instruction only every
+    // other slot, so the softmax arithmetic of one wave needs the other waves' MFMAs and arithmetic
+    // to fill the pipes; the same waves hide the latency of the copies, which run one block ahead.
+    auto block = [&](int kb, f32x16 (&s)[2]) {
+        // block kb must have landed; after the barrier every wave is done with block kb-1, whose
+        // stage takes block kb+1
+        arrive(kb, 0);
+        if (kb + 1 < nblocks) issue(kb + 1);
+        scores(kb, s);
         // keys past the end (last block only) score -inf
         if ((kb + 1) * kBlockKV > SKV) {
 #pragma unroll
@@ -136,59 +191,71 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int key = kb * kBlockKV + 32 * t + Mfma<float>::acc_row(lane, r);
-                    if (key >= SKV) st[t][r] = -__builtin_huge_valf();
+                    if (key >= SKV) s[t][r] = -__builtin_huge_valf();
                 }
         }
         // online softmax over this lane's 32 keys and its partner's (lane ^ 32) 32 keys
-        float mx = st[0][0];
+        float mx = s[0][0];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, st[t][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+        mx = fmaxf(half_swap(mx, 0), half_swap(mx, 1));
         const float m_new = fmaxf(m_run, mx * scale_log2e);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // first block: exp2(-inf) = 0
         m_run = m_new;
+        // p = exp2(scale*s - m), packed to bf16 pairs in accumulator order; the row sum is taken from
+        // the packed values
+        bf16x2_t pk[2][8];
+        bf16x2_t ones;
+        ones[0] = (__bf16) 1.0f;
+        ones[1] = (__bf16) 1.0f;
         float psum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(st[t][r], scale_log2e, -m_new));
-                st[t][r] = p;
-                psum += p;
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale_log2e, -m_new));
+                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], scale_log2e, -m_new));
+                bf16x2_t pp;
+                pp[0] = (__bf16) p0;
+                pp[1] = (__bf16) p1;
+                pk[t][r / 2] = pp;
+                psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
             }
         l_part = __builtin_fmaf(l_part, alpha, psum);
+        // the output is rescaled only when some lane's maximum moved (rare after the first blocks)
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+            for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
+                for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
+        }
 
         // O^T += V^T P^T, 16 keys per MFMA; key order inside a step follows the accumulator rows
+        const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            bf16x8 pb;
-#pragma unroll
-            for (int e = 0; e < 8; e++) pb[e] = (__bf16) st[u >> 1][8 * (u & 1) + e];
+            struct Pack { bf16x2_t v[4]; } pack = {{pk[u >> 1][4 * (u & 1)], pk[u >> 1][4 * (u & 1) + 1], pk[u >> 1][4 * (u & 1) + 2], pk[u >> 1][4 * (u & 1) + 3]}};
+            const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
             const int row = 32 * (u >> 1) + 16 * (u & 1) + tr_row;
 #pragma unroll
             for (int dt = 0; dt < 2; dt++) {
-                const uint16_t* vp = vs_ + row * kLdV + 32 * dt + tr_col;
-                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) vp);
-                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) (vp + 8 * kLdV));
+                const int col = 32 * dt + tr_col;
+                const uint16_t* plo = vs_ + attn_v_off(row, col >> 3) + (col & 7);
+                const uint16_t* phi = vs_ + attn_v_off(row + 8, col >> 3) + (col & 7);
+                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
+                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
                 const s16x8_t va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
                 ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va), pb, ot[dt], 0, 0, 0);
             }
         }
+    };
 
-        if (kb + 1 < nblocks) {
-            lk.template store<kLdK>(lds + (cur ^ 1) * kKElems, tid);
-            lv.template store<kLdV>(lds + V_BASE + (cur ^ 1) * kVElems, tid);
-        }
-        __syncthreads();
-    }
+    issue(0);
+    for (int kb = 0; kb < nblocks; kb++) block(kb, st);
 
-    const float l = l_part + __shfl_xor(l_part, 32, 64);
+    const float l = half_swap(l_part, 0) + half_swap(l_part, 1);
     const float inv = 1.0f / l;
     if (q < SQ) {
 #pragma unroll
@@ -215,13 +282,13 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
 } // namespace docc_k
 
-extern "C" __global__ __launch_bounds__(256) void docc_attention_bf16_d64_f32out(const uint16_t* Q, const uint16_t* K,
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void docc_attention_bf16_d64_f32out(const uint16_t* Q, const uint16_t* K,
                                                                                  const uint16_t* V, void* O, int SQ,
                                                                                  int SKV, float scale_log2e) {
     docc_k::attention_fwd_d64<false>(Q, K, V, O, SQ, SKV, scale_log2e);
 }
 
-extern "C" __global__ __launch_bounds__(256) void docc_attention_bf16_d64_bf16out(const uint16_t* Q, const uint16_t* K,
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void docc_attention_bf16_d64_bf16out(const uint16_t* Q, const uint16_t* K,
                                                                                   const uint16_t* V, void* O, int SQ,
                                                                                   int SKV, float scale_log2e) {
     docc_k::attention_fwd_d64<true>(Q, K, V, O, SQ, SKV, scale_log2e);
