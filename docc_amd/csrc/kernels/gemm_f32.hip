@@ -1,8 +1,15 @@
-// fp32 GEMM kernels (v_mfma_f32_32x32x2_f32), see gemm_mfma.h.
-#include "gemm_mfma.h"
+// fp32 GEMM kernels (v_mfma_f32_32x32x2_f32), see gemm_mfma.h and gemm_async.h.
+#include "gemm_async.h"
 
 DOCC_GEMM_CONFIG(sgemm, float, 128, 128, 16, 2, 2)
 DOCC_GEMM_CONFIG(sgemm, float, 64, 64, 16, 2, 2)
+
+// asynchronous multi-stage variants (aligned operands)
+DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 128, 16, 2, 2, 3)
+DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 128, 32, 2, 2, 3)
+DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 256, 16, 2, 2, 3)
+DOCC_AGEMM_CONFIG(sgemm, float, float, 64, 64, 16, 2, 2, 4)
+DOCC_AGEMM_CONFIG(sgemm, float, float, 64, 64, 32, 2, 2, 3)
 
 // C = beta * C (the k == 0 case); beta == 0 stores zeros without reading C.
 extern "C" __global__ __launch_bounds__(256) void docc_sgemm_scale_c(float* C, long M, long N, long ldc, float beta) {

@@ -67,7 +67,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         const int got = std::sscanf(c, "%dx%dx%dx%dx%d", &t.bm, &t.bn, &t.bk, &t.waves, &t.stages);
         if (got >= 4 && t.bm > 0 && t.bn > 0 && t.bk > 0 && t.waves > 0) cfg = t;
     }
-    if (cfg.stages > 0 && !aligned) cfg = pick(m, n, false, 0);   // the asynchronous kernels need aligned operands
+    // the asynchronous kernels need aligned operands and address a tile with 32-bit byte offsets
+    const int64_t max_edge = cfg.bm > cfg.bn ? (cfg.bm > cfg.bk ? cfg.bm : cfg.bk) : (cfg.bn > cfg.bk ? cfg.bn : cfg.bk);
+    const bool offsets_fit = max_edge * (lda > ldb ? lda : ldb) * (int64_t) sizeof(T) < (int64_t(1) << 32);
+    if (cfg.stages > 0 && !(aligned && offsets_fit)) cfg = pick(m, n, false, 0);
     const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     size_t lds;
@@ -92,10 +95,13 @@ extern "C" {
 // (staged) configurations need aligned operands; the others handle everything.
 static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); }
 
-static TileConfig pick_sgemm(int64_t m, int64_t n, bool, int force) {
-    const TileConfig big{128, 128, 16, 4, 0}, small{64, 64, 16, 4, 0};
-    if (force) return force > 0 ? big : small;
-    return tiles_of(m, n, 128, 128) >= 4096 ? big : small;
+static TileConfig pick_sgemm(int64_t m, int64_t n, bool aligned, int force) {
+    const TileConfig wide{128, 256, 16, 4, 3}, big{128, 128, 16, 4, 3}, small{64, 64, 16, 4, 4};
+    const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
+    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128) >= 256 ? plain_big : plain_small);
+    if (force) return force > 0 ? wide : small;
+    // the largest tile that still gives every CU a work-group
+    return tiles_of(m, n, 128, 256) >= 256 ? wide : tiles_of(m, n, 128, 128) >= 256 ? big : small;
 }
 
 static TileConfig pick_dgemm(int64_t m, int64_t n, bool aligned, int force) {

@@ -168,3 +168,30 @@ def test_sgemm_config_4096(rt):
     lhs = C.astype(np.float64) @ x
     rhs = A.astype(np.float64) @ (B.astype(np.float64) @ x)
     assert np.abs(lhs - rhs).max() / np.abs(rhs).max() <= 1e-5
+
+
+# every built tile configuration, selected through DOCC_ROCM_GEMM_CFG (BMxBNxBKxWAVES[xSTAGES]; a
+# trailing stage count picks the asynchronous multi-stage kernel), on shapes with ragged edges,
+# a K tail and all four transpose combinations
+F64_CFGS = ["64x64x16x4", "128x128x16x4", "64x64x16x4x2", "64x64x16x4x4", "64x64x16x4x6", "128x128x16x4x3",
+            "64x32x16x4x4", "64x32x32x4x3", "64x64x32x4x3"]
+F32_CFGS = ["64x64x16x4", "128x128x16x4", "128x128x16x4x3", "128x128x32x4x3", "128x256x16x4x3", "64x64x16x4x4",
+            "64x64x32x4x3"]
+
+
+@pytest.mark.parametrize("dt,cfg", [(np.float64, c) for c in F64_CFGS] + [(np.float32, c) for c in F32_CFGS])
+def test_gemm_every_tile_configuration(rt, dt, cfg):
+    import os
+    rng = np.random.default_rng(sum(cfg.encode()))
+    os.environ["DOCC_ROCM_GEMM_CFG"] = cfg
+    try:
+        for (m, n, k) in [(300, 260, 200), (129, 520, 72), (64, 64, 16), (4, 8, 1000)]:
+            for ta in (N, T):
+                for tb in (N, T):
+                    A = int_matrix(rng, (k, m) if ta == T else (m, k), dt, lim=4)
+                    B = int_matrix(rng, (n, k) if tb == T else (k, n), dt, lim=4)
+                    C0 = int_matrix(rng, (m, n), dt, lim=4)
+                    out = run_gemm(rt, A, B, C0, 2.0, -1.0, ta=ta, tb=tb)
+                    assert np.array_equal(out, oracle.gemm(A, B, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb)), (cfg, m, n, k, ta, tb)
+    finally:
+        os.environ.pop("DOCC_ROCM_GEMM_CFG", None)

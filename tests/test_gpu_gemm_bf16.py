@@ -105,3 +105,28 @@ def test_device_bf16_conversion_matches_oracle(rt):
     bits = host(dst, np.uint16)
     assert np.array_equal(bits, oracle.f32_to_bf16(x))
     assert np.array_equal(host(back), oracle.bf16_to_f32(bits))
+
+
+# every built tile configuration (DOCC_ROCM_GEMM_CFG = BMxBNxBKxWAVES[xSTAGES]; a stage count picks the
+# asynchronous kernel), ragged edges, a K tail, all transposes
+BF16_CFGS = ["128x128x64x4", "256x256x64x4", "128x128x64x4x3", "128x128x64x4x4", "128x128x32x4x4", "128x256x64x4x3",
+             "256x256x64x4x2", "256x256x32x4x4"]
+
+
+@pytest.mark.parametrize("cfg", BF16_CFGS)
+def test_bgemm_every_tile_configuration(rt, cfg):
+    rng = np.random.default_rng(sum(cfg.encode()))
+    os.environ["DOCC_ROCM_GEMM_CFG"] = cfg
+    try:
+        for (m, n, k) in [(304, 264, 200), (136, 520, 72), (8, 16, 1000)]:
+            for ta in (N, T):
+                for tb in (N, T):
+                    A = rng.integers(-4, 5, (k, m) if ta == T else (m, k)).astype(np.float32)
+                    B = rng.integers(-4, 5, (n, k) if tb == T else (k, n)).astype(np.float32)
+                    C0 = rng.integers(-4, 5, (m, n)).astype(np.float32)
+                    Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+                    out = run_bgemm(rt, Ab, Bb, C0, alpha=2.0, beta=-1.0, ta=ta, tb=tb)
+                    ref = oracle.gemm_bf16(Ab, Bb, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb)
+                    assert np.array_equal(out, ref), (cfg, m, n, k, ta, tb)
+    finally:
+        os.environ.pop("DOCC_ROCM_GEMM_CFG", None)
