@@ -73,9 +73,15 @@ def main():
     stream = 0  # the null stream: torch allocates and we launch on it
 
     def time_kernel(fn, iters, warm):
-        """Average launch duration in ms from HIP events around `iters` back-to-back launches."""
-        for i in range(warm):
+        """Average launch duration in ms from HIP events around `iters` back-to-back launches, after
+        `warm` launches and at least a quarter of a second of them (the clocks ramp up from idle)."""
+        t_warm = time.perf_counter()
+        i = 0
+        while i < warm or time.perf_counter() - t_warm < 0.25:
             fn(i)
+            i += 1
+            if i % 16 == 0:
+                rt.device_sync()
         rt.device_sync()
         e0, e1 = rt.Event(), rt.Event()
         e0.record(stream)
@@ -145,11 +151,37 @@ def main():
                                    "sample": f"full [8192,4096] tensor, decomposed max/sub/exp/sum/div/copy form, median of 3 after 1 cold run; {oracle_build}"}
         del pairs
 
+    # What the power limit leaves of the nominal MFMA peak on this device: a bare loop of MFMAs on
+    # N(0,1) operands (the multipliers toggle as in a real GEMM), one and two waves per SIMD, best of
+    # the two. Reported beside the nominal peak; `frac` stays relative to the nominal peak.
+    ceiling_cache = {}
+
+    def mfma_ceiling(dtype):
+        if dtype in ceiling_cache:
+            return ceiling_cache[dtype]
+        prec = {"f64": 64, "f32": 32, "bf16": 16}[dtype]
+        ops = torch.randn(4096, device="cuda")
+        sink = torch.empty(2 * 256 * max(info["compute_units"], 1), device="cuda")
+        iters = 4000
+        best = 0.0
+        for waves in (1, 2):
+            flop = [0.0]
+
+            def probe(i, waves=waves):
+                flop[0] = rt.mfma_probe(prec, waves, iters, ops.data_ptr(), sink.data_ptr(), stream)
+
+            ms = time_kernel(probe, 5, 2)
+            best = max(best, flop[0] / ms / 1e9)
+        ceiling_cache[dtype] = round(best, 1)
+        return ceiling_cache[dtype]
+
     def add_kernel(name, dtype, flops, ms, cpu=None, extra=None):
         tf = flops / ms / 1e9
+        ceiling = mfma_ceiling(dtype)
         entry = {"tflops": round(tf, 2), "kernel_us": round(ms * 1e3, 2), "flop": flops,
                  "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
-                              "frac": round(tf / PEAK_TFLOPS[dtype], 4)}, "dtype": dtype}
+                              "frac": round(tf / PEAK_TFLOPS[dtype], 4), "mfma_loop_random_operands": ceiling,
+                              "frac_of_mfma_loop": round(tf / ceiling, 4) if ceiling else None}, "dtype": dtype}
         if cpu:
             entry["cpu_baseline"] = cpu
         if extra:

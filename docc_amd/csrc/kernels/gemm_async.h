@@ -303,6 +303,11 @@ struct AsyncGemmKernel {
         //   refill stage kt and the LDS reads of step kt+1's first operands.
         // mode 0: steady state (the refill is a full asynchronous step, nothing in the body branches);
         // mode 1: near the end (the refill may be the K tail or absent); mode 2: the last step
+        // shares per MFMA slot, dealt from the first slot on so that the last LDS read is issued well
+        // before the inner step ends (its latency would otherwise be waited for at the next step)
+        constexpr int PPM = (NPIECE + NM - 1) / NM;                   // pieces per MFMA, inner steps but the last
+        constexpr int PPL = (NPIECE + NM - 2) / (NM - 1);             // pieces per MFMA, last inner step
+        constexpr int LPM = (LOADS_PER_STEP + NM - 2) / (NM - 1);     // copies per MFMA, last inner step
         auto kstep = [&](int kt, auto mode_c) {
             constexpr int MODE = decltype(mode_c)::value;
             constexpr bool NEXT = MODE != 2;
@@ -314,7 +319,7 @@ struct AsyncGemmKernel {
                     for (int n = 0; n < NM; n++) {
                         mma(ki & 1, n, n + 1);
 #pragma unroll
-                        for (int q = n * NPIECE / NM; q < (n + 1) * NPIECE / NM; q++) fetch_piece(st, ki + 1, (ki + 1) & 1, q);
+                        for (int q = n * PPM; q < (n + 1) * PPM && q < NPIECE; q++) fetch_piece(st, ki + 1, (ki + 1) & 1, q);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 } else if (NEXT) {
@@ -337,13 +342,13 @@ struct AsyncGemmKernel {
                         mma(ki & 1, n, n + 1);
                         if (MODE == 0) {
 #pragma unroll
-                            for (int q = (n - 1) * LOADS_PER_STEP / (NM - 1); q < n * LOADS_PER_STEP / (NM - 1); q++) {
+                            for (int q = (n - 1) * LPM; q < n * LPM && q < LOADS_PER_STEP; q++) {
                                 if (q < ATile::NV) ta.issue_one(dst, q, wave);
                                 else tb.issue_one(dst + ATile::ELEMS, q - ATile::NV, wave);
                             }
                         }
 #pragma unroll
-                        for (int q = (n - 1) * NPIECE / (NM - 1); q < n * NPIECE / (NM - 1); q++) fetch_piece(nst, 0, 0, q);
+                        for (int q = (n - 1) * PPL; q < n * PPL && q < NPIECE; q++) fetch_piece(nst, 0, 0, q);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 } else {

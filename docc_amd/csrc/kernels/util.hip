@@ -1,4 +1,4 @@
-// Small utility kernels: calibration copy and fp32 <-> bf16 conversion.
+// Small utility kernels: calibration copy, MFMA rate probes and fp32 <-> bf16 conversion.
 #include "common.h"
 
 using namespace docc_k;
@@ -24,4 +24,73 @@ extern "C" __global__ __launch_bounds__(256) void docc_bf16_to_f32(const uint16_
     long i = (long) blockIdx.x * 256 + threadIdx.x;
     const long stride = (long) gridDim.x * 256;
     for (; i < n; i += stride) dst[i] = bf16_bits_to_f32(src[i]);
+}
+
+// MFMA rate probes: `iters` rounds of 32 back-to-back MFMAs per wave on operands taken from
+// `operands` (4096 floats; random values make the multipliers toggle as they do in a real GEMM,
+// zeros do not), four accumulators, eight operand register sets in rotation. They measure what the
+// power limit leaves of the nominal matrix peak on the device at hand - the ceiling a GEMM-shaped
+// kernel can reach with that data. One wave per SIMD per work-group; launch 2 per CU for two.
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+typedef double probe_f64x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+
+extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f64(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
+    probe_f64x4 acc[4];
+    for (int i = 0; i < 4; i++) acc[i] = {0, 0, 0, 0};
+    double a[8], b[8];
+    for (int i = 0; i < 8; i++) {
+        a[i] = operands[(threadIdx.x * 8 + i) & 4095];
+        b[i] = operands[(threadIdx.x * 8 + i + 2048) & 4095];
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+    }
+    double r = 0;
+    for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][3];
+    sink[blockIdx.x * 256 + threadIdx.x] = (float) r;
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f32(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
+    probe_f32x16 acc[4];
+    for (int i = 0; i < 4; i++)
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    float a[8], b[8];
+    for (int i = 0; i < 8; i++) {
+        a[i] = operands[(threadIdx.x * 8 + i) & 4095];
+        b[i] = operands[(threadIdx.x * 8 + i + 2048) & 4095];
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+    }
+    float r = 0;
+    for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][15];
+    sink[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_bf16(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
+    probe_f32x16 acc[4];
+    for (int i = 0; i < 4; i++)
+        for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    probe_bf16x8 a[8], b[8];
+    for (int i = 0; i < 8; i++)
+        for (int e = 0; e < 8; e++) {
+            a[i][e] = (__bf16) operands[(threadIdx.x * 64 + i * 8 + e) & 4095];
+            b[i][e] = (__bf16) operands[(threadIdx.x * 64 + i * 8 + e + 1777) & 4095];
+        }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+    }
+    float r = 0;
+    for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][15];
+    sink[blockIdx.x * 256 + threadIdx.x] = r;
 }

@@ -68,6 +68,7 @@ _SIGNATURES = {
     "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
+    "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
             "docc_rocm_report_failure": None}
@@ -210,6 +211,13 @@ def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0
 
 def copy_bytes(nbytes, src, dst, stream=0) -> None:
     call("docc_rocm_copy_bytes", stream, nbytes, src, dst)
+
+
+def mfma_probe(precision, waves_per_simd, iters, operands, sink, stream=0) -> float:
+    """Launches the MFMA rate probe; returns the floating-point operations of the launch."""
+    flop = ctypes.c_double(0.0)
+    call("docc_rocm_mfma_probe", stream, precision, waves_per_simd, iters, operands, sink, ctypes.addressof(flop))
+    return flop.value
 
 
 def convert_f32_to_bf16(count, src, dst, stream=0) -> None:

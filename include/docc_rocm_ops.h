@@ -104,6 +104,16 @@ int docc_rocm_convert_bf16_to_f32(docc_rocm_stream_t stream, int64_t count, cons
  * calibrated. */
 int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* src, void* dst);
 
+/* Measurement aid, no counterpart in the reference: `iters` rounds of 32 back-to-back
+ * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16) on
+ * every SIMD, `waves_per_simd` (1 or 2) waves each, operands taken from `operands`
+ * (4096 floats on the device). `sink` receives 256 floats per work-group (CUs *
+ * waves_per_simd groups); *flop (host, optional) the floating-point operations of
+ * the launch. Timed with events it gives the matrix rate the power limit allows for
+ * that operand data: the practical ceiling beside the nominal peak. */
+int docc_rocm_mfma_probe(docc_rocm_stream_t stream, int precision, int waves_per_simd, int iters, const float* operands,
+                         float* sink, double* flop);
+
 #ifdef __cplusplus
 }
 #endif
