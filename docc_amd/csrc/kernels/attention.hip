@@ -25,7 +25,7 @@
 //
 // The softmax arithmetic, not the MFMAs, is the longer half of a block (32 scores per lane:
 // exp2, scale, max, sum, pack), so it is kept to the minimum: v_max3 for the maximum, one
-// v_permlane32_swap for the exchange, v_cvt_pk_bf16_f32 for the packing, the row sum taken
+// v_permlane32_swap for the exchange, one v_perm_b32 per pair for the packing, the row sum taken
 // from the packed values with v_dot2c_f32_bf16 (it then sums exactly what the second product
 // multiplies), and the rescale of the output skipped while no lane's maximum moves. The scores
 // of block i+1 are issued to the matrix pipe before the softmax of block i starts, and K/V
@@ -82,11 +82,17 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qj = lane & 31, g = lane >> 5;
-    const long bh = blockIdx.y;
+    // work-group -> (head, query block): consecutive work-group ids go round the 8 XCDs, so the id is
+    // renumbered to give each XCD whole heads - the 16 query blocks of a head then share one L2
+    const int nqb = gridDim.x, total = gridDim.x * gridDim.y;
+    int lid = blockIdx.y * gridDim.x + blockIdx.x;
+    if (total % 8 == 0) lid = (lid % 8) * (total / 8) + lid / 8;
+    const long bh = lid / nqb;
+    const int qblk = lid % nqb;
     const uint16_t* Qh = Q + bh * (long) SQ * kHeadDim;
     const char* Kh = reinterpret_cast<const char*>(K + bh * (long) SKV * kHeadDim);
     const char* Vh = reinterpret_cast<const char*>(V + bh * (long) SKV * kHeadDim);
-    const int q = blockIdx.x * kBlockQ + wave * 32 + qj;   // this lane's query
+    const int q = qblk * kBlockQ + wave * 32 + qj;   // this lane's query
 
     // Q^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q
     bf16x8 bq[4];
@@ -217,9 +223,9 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
             for (int r = 0; r < 16; r += 2) {
                 const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale_log2e, -m_new));
                 const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], scale_log2e, -m_new));
-                bf16x2_t pp;
-                pp[0] = (__bf16) p0;
-                pp[1] = (__bf16) p1;
+                // bf16 by truncation (one v_perm_b32; the rounding convert runs at half rate): the row
+                // sum below is taken from the same truncated values, so the bias cancels in O = PV / sum
+                const bf16x2_t pp = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, p1), __builtin_bit_cast(unsigned, p0), 0x07060302u));
                 pk[t][r / 2] = pp;
                 psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
             }
