@@ -23,13 +23,21 @@
 //                                                are (the k-order of the MFMA is permuted to
 //                                                the accumulator's row order on both operands).
 //
-// The softmax arithmetic, not the MFMAs, is the longer half of a block (32 scores per lane:
-// exp2, scale, max, sum, pack), so it is kept to the minimum: v_max3 for the maximum, one
-// v_permlane32_swap for the exchange, one v_perm_b32 per pair for the packing, the row sum taken
-// from the packed values with v_dot2c_f32_bf16 (it then sums exactly what the second product
-// multiplies), and the rescale of the output skipped while no lane's maximum moves. The scores
-// of block i+1 are issued to the matrix pipe before the softmax of block i starts, and K/V
-// blocks arrive in a ring of LDS stages by asynchronous global->LDS copies.
+// The softmax arithmetic, not the MFMAs, is the longer half of a block (32 scores per lane), so
+// it is cut to exp2, pack and sum:
+//   - scale*log2(e) is folded into Q once (Q' = bf16(Q * scale * log2e)), so the score product
+//     already yields log2-domain scores;
+//   - the reference point m of the online softmax rides in the MFMA's C operand: S' = K Q'^T - m,
+//     p = exp2(S') with no subtraction pass;
+//   - m does not have to be the exact running maximum: softmax is shift invariant and fp32/bf16
+//     keep their relative precision at any magnitude, so m stays what the first block set until a
+//     block's row sum shows growth beyond 2^40 (or inf) - only then the block takes the slow path
+//     (true block maximum, rescale of the output and the sum, recomputed p). The usual block has no
+//     max pass and no rescale;
+//   - p is packed to bf16 by one v_perm_b32 per pair (truncation) and the row sum is taken from the
+//     packed values with v_dot2c_f32_bf16: it sums exactly what the second product multiplies, so
+//     the truncation bias cancels in O = PV / sum.
+// K/V blocks arrive in a ring of LDS stages by asynchronous global->LDS copies.
 #include "gemm_mfma.h"
 #include <type_traits>
 
@@ -94,12 +102,14 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const char* Vh = reinterpret_cast<const char*>(V + bh * (long) SKV * kHeadDim);
     const int q = qblk * kBlockQ + wave * 32 + qj;   // this lane's query
 
-    // Q^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q
+    // Q'^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q, times scale*log2e
     bf16x8 bq[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) {
         u16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (q < SQ) v = *reinterpret_cast<const u16x8_t*>(Qh + (long) q * kHeadDim + 16 * ks + 8 * g);
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = f32_to_bf16_rne(bf16_bits_to_f32(v[e]) * scale_log2e);
         bq[ks] = __builtin_bit_cast(bf16x8, v);
     }
 
@@ -154,7 +164,10 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     for (int dt = 0; dt < 2; dt++)
 #pragma unroll
         for (int r = 0; r < 16; r++) ot[dt][r] = 0.f;
-    float m_run = -__builtin_huge_valf();   // running max of scale*log2e*score
+    float m_run = 0.f;                      // reference point of the exponentials (log2 domain)
+    f32x16 negm;                            // -m_run in every register: the C operand of the score MFMAs
+#pragma unroll
+    for (int r = 0; r < 16; r++) negm[r] = 0.f;
     float l_part = 0.f;                     // this lane's part of the running sum (its 32 keys per block)
 
     // lane roles for the transposed V reads (see gemm_bf16.hip)
@@ -165,26 +178,46 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
     f32x16 st[2];
 
-    // scores, transposed: s[t][r] = <K[32t + acc_row(r)], Q[q]> for the block in `stage`
+    // scores relative to the reference point, transposed: s[t][r] = <K[32t + acc_row(r)], Q'[q]> - m_run
     auto scores = [&](int kb, f32x16 (&s)[2]) {
         const uint16_t* ks_ = lds + (kb % kAttnStages) * kStageElems;
 #pragma unroll
         for (int t = 0; t < 2; t++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) s[t][r] = 0.f;
-#pragma unroll
             for (int ks = 0; ks < 4; ks++) {
                 const u16x8_t kv = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off(32 * t + qj, 2 * ks + g));
-                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv), bq[ks], s[t], 0, 0, 0);
+                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv), bq[ks], ks == 0 ? negm : s[t], 0, 0, 0);
             }
         }
     };
 
-    // one block: scores -> softmax -> O^T += V^T P^T. The kernel is sized for four waves per SIMD
-    // (128 registers, 32 KB of LDS per work-group): a wave issues a vector instruction only every
-    // other slot, so the softmax arithmetic of one wave needs the other waves' MFMAs and arithmetic
-    // to fill the pipes; the same waves hide the latency of the copies, which run one block ahead.
-    auto block = [&](int kb, f32x16 (&s)[2]) {
+    bf16x2_t pk[2][8];
+    // p = exp2(s), packed to bf16 pairs in accumulator order; returns this lane's row sum of the packed values
+    auto exponentials = [&](f32x16 (&s)[2]) {
+        bf16x2_t ones;
+        ones[0] = (__bf16) 1.0f;
+        ones[1] = (__bf16) 1.0f;
+        float psum = 0.f;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(s[t][r]);
+                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
+                const bf16x2_t pp = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, p1), __builtin_bit_cast(unsigned, p0), 0x07060302u));
+                pk[t][r / 2] = pp;
+                psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
+            }
+        return psum;
+    };
+
+    // one block: scores -> exponentials -> O^T += V^T P^T. Sized for three to four waves per SIMD: a
+    // wave issues an instruction only every 4-5 cycles, so the arithmetic of one wave needs the other
+    // waves' MFMAs and arithmetic to fill the pipes; the same waves hide the latency of the copies,
+    // which run one block ahead.
+    auto block = [&](int kb, auto first_c) {
+        constexpr bool FIRST = decltype(first_c)::value;
+        f32x16 (&s)[2] = st;
         // block kb must have landed; after the barrier every wave is done with block kb-1, whose
         // stage takes block kb+1
         arrive(kb, 0);
@@ -200,43 +233,40 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
                     if (key >= SKV) s[t][r] = -__builtin_huge_valf();
                 }
         }
-        // online softmax over this lane's 32 keys and its partner's (lane ^ 32) 32 keys
-        float mx = s[0][0];
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-        mx = fmaxf(half_swap(mx, 0), half_swap(mx, 1));
-        const float m_new = fmaxf(m_run, mx * scale_log2e);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // first block: exp2(-inf) = 0
-        m_run = m_new;
-        // p = exp2(scale*s - m), packed to bf16 pairs in accumulator order; the row sum is taken from
-        // the packed values
-        bf16x2_t pk[2][8];
-        bf16x2_t ones;
-        ones[0] = (__bf16) 1.0f;
-        ones[1] = (__bf16) 1.0f;
         float psum = 0.f;
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], scale_log2e, -m_new));
-                const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], scale_log2e, -m_new));
-                // bf16 by truncation (one v_perm_b32; the rounding convert runs at half rate): the row
-                // sum below is taken from the same truncated values, so the bias cancels in O = PV / sum
-                const bf16x2_t pp = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, p1), __builtin_bit_cast(unsigned, p0), 0x07060302u));
-                pk[t][r / 2] = pp;
-                psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
-            }
-        l_part = __builtin_fmaf(l_part, alpha, psum);
-        // the output is rescaled only when some lane's maximum moved (rare after the first blocks)
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-            for (int dt = 0; dt < 2; dt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
+        bool slow = FIRST;
+        if (!FIRST) {
+            psum = exponentials(s);
+            // growth of the maximum beyond 2^40 over the reference point (or an overflow) shows in the sum
+            slow = __builtin_amdgcn_ballot_w64(!(psum < 0x1p40f)) != 0;
         }
+        if (slow) {
+            // move the reference point to the true maximum of what this lane pair has seen
+            float mx = s[0][0];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+            mx = fmaxf(half_swap(mx, 0), half_swap(mx, 1));
+            const float d = FIRST ? mx : fmaxf(mx, 0.f);             // s is relative to m_run (0 in the first block)
+            const float alpha = FIRST ? 0.f : __builtin_amdgcn_exp2f(-d);
+            m_run += d;
+#pragma unroll
+            for (int r = 0; r < 16; r++) negm[r] = -m_run;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) s[t][r] -= d;
+            if (!FIRST) {
+                l_part *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
+            }
+            psum = exponentials(s);
+        }
+        l_part += psum;
 
         // O^T += V^T P^T, 16 keys per MFMA; key order inside a step follows the accumulator rows
         const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
@@ -259,7 +289,8 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     };
 
     issue(0);
-    for (int kb = 0; kb < nblocks; kb++) block(kb, st);
+    block(0, std::true_type{});
+    for (int kb = 1; kb < nblocks; kb++) block(kb, std::false_type{});
 
     const float l = half_swap(l_part, 0) + half_swap(l_part, 1);
     const float inv = 1.0f / l;
@@ -288,13 +319,13 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
 } // namespace docc_k
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void docc_attention_bf16_d64_f32out(const uint16_t* Q, const uint16_t* K,
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void docc_attention_bf16_d64_f32out(const uint16_t* Q, const uint16_t* K,
                                                                                  const uint16_t* V, void* O, int SQ,
                                                                                  int SKV, float scale_log2e) {
     docc_k::attention_fwd_d64<false>(Q, K, V, O, SQ, SKV, scale_log2e);
 }
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4))) void docc_attention_bf16_d64_bf16out(const uint16_t* Q, const uint16_t* K,
+extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void docc_attention_bf16_d64_bf16out(const uint16_t* Q, const uint16_t* K,
                                                                                   const uint16_t* V, void* O, int SQ,
                                                                                   int SKV, float scale_log2e) {
     docc_k::attention_fwd_d64<true>(Q, K, V, O, SQ, SKV, scale_log2e);
