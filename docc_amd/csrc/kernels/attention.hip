@@ -60,7 +60,7 @@ struct Mfma<uint16_t> {
 constexpr int kHeadDim = 64;
 constexpr int kBlockQ = 128;     // queries per work-group
 constexpr int kBlockKV = 64;     // keys per step
-constexpr int kAttnStages = 2;   // LDS ring depth: block kb+1 is copied while block kb is worked on
+constexpr int kAttnStages = 3;   // LDS ring depth: blocks kb+1 and kb+2 are in flight while block kb is worked on
 constexpr int kTileElems = kBlockKV * kHeadDim;          // one K or V block, unpadded, 16-byte granules swizzled
 constexpr int kStageElems = 2 * kTileElems;              // [K | V]
 
@@ -147,8 +147,9 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     // block kb has landed in every wave's view; rows of a partial last V block are cleared so that
     // 0 * (copied value) cannot produce a NaN
     auto arrive = [&](int kb, int newer_blocks) {
-        (void) newer_blocks;
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        // each block is four copies per lane; one newer block may still be in flight
+        if (newer_blocks > 0) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (kb >= full_blocks) {
@@ -181,14 +182,18 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     // scores relative to the reference point, transposed: s[t][r] = <K[32t + acc_row(r)], Q'[q]> - m_run
     auto scores = [&](int kb, f32x16 (&s)[2]) {
         const uint16_t* ks_ = lds + (kb % kAttnStages) * kStageElems;
+        // all eight K operands are requested before the first MFMA: one LDS round trip, not eight
+        u16x8_t kv[2][4];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
+        for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) {
-                const u16x8_t kv = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off(32 * t + qj, 2 * ks + g));
-                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv), bq[ks], ks == 0 ? negm : s[t], 0, 0, 0);
-            }
-        }
+            for (int ks = 0; ks < 4; ks++) kv[t][ks] = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off(32 * t + qj, 2 * ks + g));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv[t][ks]), bq[ks], ks == 0 ? negm : s[t], 0, 0, 0);
     };
 
     bf16x2_t pk[2][8];
@@ -219,9 +224,9 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         constexpr bool FIRST = decltype(first_c)::value;
         f32x16 (&s)[2] = st;
         // block kb must have landed; after the barrier every wave is done with block kb-1, whose
-        // stage takes block kb+1
-        arrive(kb, 0);
-        if (kb + 1 < nblocks) issue(kb + 1);
+        // stage takes block kb+2
+        arrive(kb, kb + 1 < nblocks ? 1 : 0);
+        if (kb + 2 < nblocks) issue(kb + 2);
         scores(kb, s);
         // keys past the end (last block only) score -inf
         if ((kb + 1) * kBlockKV > SKV) {
@@ -233,6 +238,7 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
                     if (key >= SKV) s[t][r] = -__builtin_huge_valf();
                 }
         }
+        const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
         float psum = 0.f;
         bool slow = FIRST;
         if (!FIRST) {
@@ -268,27 +274,41 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         }
         l_part += psum;
 
-        // O^T += V^T P^T, 16 keys per MFMA; key order inside a step follows the accumulator rows
-        const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
+        // O^T += V^T P^T, 16 keys per MFMA; key order inside a step follows the accumulator rows.
+        // The V operands of two MFMA pairs are requested together (they do not depend on P).
+        auto pv_half = [&](int h) {
+            s16x8_t va[2][2];
 #pragma unroll
-        for (int u = 0; u < 4; u++) {
-            struct Pack { bf16x2_t v[4]; } pack = {{pk[u >> 1][4 * (u & 1)], pk[u >> 1][4 * (u & 1) + 1], pk[u >> 1][4 * (u & 1) + 2], pk[u >> 1][4 * (u & 1) + 3]}};
-            const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
-            const int row = 32 * (u >> 1) + 16 * (u & 1) + tr_row;
+            for (int uu = 0; uu < 2; uu++) {
+                const int u = 2 * h + uu;
+                const int row = 32 * (u >> 1) + 16 * (u & 1) + tr_row;
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) {
-                const int col = 32 * dt + tr_col;
-                const uint16_t* plo = vs_ + attn_v_off(row, col >> 3) + (col & 7);
-                const uint16_t* phi = vs_ + attn_v_off(row + 8, col >> 3) + (col & 7);
-                const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
-                const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
-                const s16x8_t va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va), pb, ot[dt], 0, 0, 0);
+                for (int dt = 0; dt < 2; dt++) {
+                    const int col = 32 * dt + tr_col;
+                    const uint16_t* plo = vs_ + attn_v_off(row, col >> 3) + (col & 7);
+                    const uint16_t* phi = vs_ + attn_v_off(row + 8, col >> 3) + (col & 7);
+                    const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
+                    const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
+                    va[uu][dt] = s16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                }
             }
-        }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int uu = 0; uu < 2; uu++) {
+                const int u = 2 * h + uu;
+                struct Pack { bf16x2_t v[4]; } pack = {{pk[u >> 1][4 * (u & 1)], pk[u >> 1][4 * (u & 1) + 1], pk[u >> 1][4 * (u & 1) + 2], pk[u >> 1][4 * (u & 1) + 3]}};
+                const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
+#pragma unroll
+                for (int dt = 0; dt < 2; dt++)
+                    ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[uu][dt]), pb, ot[dt], 0, 0, 0);
+            }
+        };
+        pv_half(0);
+        pv_half(1);
     };
 
     issue(0);
+    if (nblocks > 1) issue(1);
     block(0, std::true_type{});
     for (int kb = 1; kb < nblocks; kb++) block(kb, std::false_type{});
 

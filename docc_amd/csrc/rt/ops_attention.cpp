@@ -21,8 +21,8 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
         return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: batch*heads must be <= 65535 and sequences < 2^31");
     int rc = ensure_device();
     if (rc) return rc;
-    // LDS: ring of 2 stages x (K block [64][64] + V block [64][64]) bf16
-    const uint32_t lds = 2 * (2 * 64 * 64) * 2;
+    // LDS: ring of 3 stages x (K block [64][64] + V block [64][64]) bf16
+    const uint32_t lds = 3 * (2 * 64 * 64) * 2;
     const float scale_log2e = scale * 1.4426950408889634f;
     return launch(out_bf16 ? "docc_attention_bf16_d64_bf16out" : "docc_attention_bf16_d64_f32out",
                   (uint32_t) ((SQ + 127) / 128), (uint32_t) (B * H), 1, 256, lds, (hipStream_t) stream, Q, K, V, O,
