@@ -41,6 +41,7 @@ KERNEL_FAMILIES = {
     "gemm_bf16_async_big": "gemm_bf16_async_big.hip",
     "conv2d": "conv2d.hip",
     "attention": "attention.hip",
+    "elementwise": "elementwise.hip",
 }
 
 # Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary

@@ -1,0 +1,171 @@
+// Elementwise tensor nodes and ml::Broadcast, fp32 and fp64, for gfx950.
+//
+// Replace the Maps that ElementWiseUnaryNode / ElementWiseBinaryNode::expand produce (reference
+// sdfg/include/sdfg/data_flow/library_nodes/math/tensor/elementwise_node.h: Y[i] = f(X[i]) or
+// f(A[i], B[i]) over the linearised shape) and BroadcastNode::expand (broadcast_node.h:13-43).
+// Operation semantics follow the reference's expansions:
+//   ReLU     fmax(x, 0.0)            elementwise_ops/relu_node.cpp:40-43
+//   Sigmoid  1.0 / (1.0 + exp(-x))   elementwise_ops/sigmoid_node.cpp:46-70
+//   Maximum / Minimum  fmax / fmin   elementwise_ops/maximum_node.cpp:64, minimum_node.cpp
+//   Abs, Exp, Sqrt, Tanh, Erf        the libm function of the element type (cmath_node.h)
+//   Add, Sub, Mul, Div               the IEEE operation
+//
+// HBM-bound: 8 (unary) or 12 (binary) bytes per fp32 element. One 128-bit access per operand
+// and lane, grid-stride over the vectors, scalar tail; unaligned operands take the scalar path.
+#include "common.h"
+
+namespace docc_k {
+
+enum UnaryOp : int { kAbs = 0, kExp = 1, kReLU = 2, kSigmoid = 3, kSqrt = 4, kTanh = 5, kErf = 6 };
+enum BinaryOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMaximum = 4, kMinimum = 5 };
+
+template <int OP>
+__device__ __forceinline__ float unary(float x) {
+    if (OP == kAbs) return fabsf(x);
+    if (OP == kExp) return expf(x);
+    if (OP == kReLU) return fmaxf(x, 0.0f);
+    if (OP == kSigmoid) return 1.0f / (1.0f + expf(-x));
+    if (OP == kSqrt) return sqrtf(x);
+    if (OP == kTanh) return tanhf(x);
+    return erff(x);
+}
+template <int OP>
+__device__ __forceinline__ double unary(double x) {
+    if (OP == kAbs) return fabs(x);
+    if (OP == kExp) return exp(x);
+    if (OP == kReLU) return fmax(x, 0.0);
+    if (OP == kSigmoid) return 1.0 / (1.0 + exp(-x));
+    if (OP == kSqrt) return sqrt(x);
+    if (OP == kTanh) return tanh(x);
+    return erf(x);
+}
+template <int OP>
+__device__ __forceinline__ float binary(float a, float b) {
+    if (OP == kAdd) return a + b;
+    if (OP == kSub) return a - b;
+    if (OP == kMul) return a * b;
+    if (OP == kDiv) return a / b;
+    if (OP == kMaximum) return fmaxf(a, b);
+    return fminf(a, b);
+}
+template <int OP>
+__device__ __forceinline__ double binary(double a, double b) {
+    if (OP == kAdd) return a + b;
+    if (OP == kSub) return a - b;
+    if (OP == kMul) return a * b;
+    if (OP == kDiv) return a / b;
+    if (OP == kMaximum) return fmax(a, b);
+    return fmin(a, b);
+}
+
+template <typename T>
+struct Vec128;
+template <>
+struct Vec128<float> {
+    typedef float type __attribute__((ext_vector_type(4)));
+    static constexpr int N = 4;
+};
+template <>
+struct Vec128<double> {
+    typedef double type __attribute__((ext_vector_type(2)));
+    static constexpr int N = 2;
+};
+
+// nvec: number of whole 128-bit vectors to process vectorised (0 when an operand is unaligned)
+template <typename T, int OP>
+__device__ __forceinline__ void unary_kernel(const T* X, T* Y, long n, long nvec) {
+    typedef typename Vec128<T>::type V;
+    constexpr int N = Vec128<T>::N;
+    const long stride = (long) gridDim.x * blockDim.x;
+    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = tid; i < nvec; i += stride) {
+        V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(X) + i);
+#pragma unroll
+        for (int e = 0; e < N; e++) v[e] = unary<OP>(v[e]);
+        __builtin_nontemporal_store(v, reinterpret_cast<V*>(Y) + i);
+    }
+    for (long i = nvec * N + tid; i < n; i += stride) Y[i] = unary<OP>(X[i]);
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void binary_kernel(const T* A, const T* B, T* Y, long n,
+                                              long nvec) {
+    typedef typename Vec128<T>::type V;
+    constexpr int N = Vec128<T>::N;
+    const long stride = (long) gridDim.x * blockDim.x;
+    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = tid; i < nvec; i += stride) {
+        const V a = __builtin_nontemporal_load(reinterpret_cast<const V*>(A) + i);
+        const V b = __builtin_nontemporal_load(reinterpret_cast<const V*>(B) + i);
+        V y;
+#pragma unroll
+        for (int e = 0; e < N; e++) y[e] = binary<OP>(a[e], b[e]);
+        __builtin_nontemporal_store(y, reinterpret_cast<V*>(Y) + i);
+    }
+    for (long i = nvec * N + tid; i < n; i += stride) Y[i] = binary<OP>(A[i], B[i]);
+}
+
+// ml::Broadcast: Y[o] = X[offset(o)], numpy rules (an input dimension of extent 1 repeats)
+struct BroadcastParams {
+    int rank;
+    long n;                 // elements of the output
+    long out_dims[6];
+    long in_strides[6];     // in elements; 0 for a broadcast dimension
+};
+
+template <typename T>
+__device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const BroadcastParams& p) {
+    const long stride = (long) gridDim.x * blockDim.x;
+    for (long o = (long) blockIdx.x * blockDim.x + threadIdx.x; o < p.n; o += stride) {
+        long rem = o, off = 0;
+#pragma unroll
+        for (int d = 5; d >= 0; d--) {
+            if (d < p.rank) {
+                const long c = rem % p.out_dims[d];
+                rem /= p.out_dims[d];
+                off += c * p.in_strides[d];
+            }
+        }
+        Y[o] = X[off];
+    }
+}
+
+} // namespace docc_k
+
+#define DOCC_EW_UNARY(NAME, OP)                                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f32(const float* X, float* Y, long n, long nvec) {       \
+        docc_k::unary_kernel<float, docc_k::OP>(X, Y, n, nvec);                                                              \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f64(const double* X, double* Y, long n, long nvec) {     \
+        docc_k::unary_kernel<double, docc_k::OP>(X, Y, n, nvec);                                                             \
+    }
+#define DOCC_EW_BINARY(NAME, OP)                                                                                             \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f32(const float* A, const float* B, float* Y, long n,    \
+                                                                           long nvec) {                                      \
+        docc_k::binary_kernel<float, docc_k::OP>(A, B, Y, n, nvec);                                                          \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f64(const double* A, const double* B, double* Y, long n, \
+                                                                           long nvec) {                                      \
+        docc_k::binary_kernel<double, docc_k::OP>(A, B, Y, n, nvec);                                                         \
+    }
+
+DOCC_EW_UNARY(abs, kAbs)
+DOCC_EW_UNARY(exp, kExp)
+DOCC_EW_UNARY(relu, kReLU)
+DOCC_EW_UNARY(sigmoid, kSigmoid)
+DOCC_EW_UNARY(sqrt, kSqrt)
+DOCC_EW_UNARY(tanh, kTanh)
+DOCC_EW_UNARY(erf, kErf)
+DOCC_EW_BINARY(add, kAdd)
+DOCC_EW_BINARY(sub, kSub)
+DOCC_EW_BINARY(mul, kMul)
+DOCC_EW_BINARY(div, kDiv)
+DOCC_EW_BINARY(maximum, kMaximum)
+DOCC_EW_BINARY(minimum, kMinimum)
+
+extern "C" __global__ __launch_bounds__(256) void docc_broadcast_f32(const float* X, float* Y, docc_k::BroadcastParams p) {
+    docc_k::broadcast_kernel<float>(X, Y, p);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_broadcast_f64(const double* X, double* Y, docc_k::BroadcastParams p) {
+    docc_k::broadcast_kernel<double>(X, Y, p);
+}

@@ -33,6 +33,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_gemm_bf16_async_big.hsaco",
     "docc_rocm_conv2d.hsaco",
     "docc_rocm_attention.hsaco",
+    "docc_rocm_elementwise.hsaco",
 };
 
 struct DeviceState {

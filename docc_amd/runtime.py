@@ -67,6 +67,9 @@ _SIGNATURES = {
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
     "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
+    "docc_rocm_elementwise_unary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp],
+    "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
+    "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
@@ -211,6 +214,26 @@ def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0
 
 def copy_bytes(nbytes, src, dst, stream=0) -> None:
     call("docc_rocm_copy_bytes", stream, nbytes, src, dst)
+
+
+UNARY_OPS = {"abs": 0, "exp": 1, "relu": 2, "sigmoid": 3, "sqrt": 4, "tanh": 5, "erf": 6}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+
+
+def elementwise_unary(op, precision, n, X, Y, stream=0) -> None:
+    call("docc_rocm_elementwise_unary", stream, UNARY_OPS[op] if isinstance(op, str) else op, precision, n, X, Y)
+
+
+def elementwise_binary(op, precision, n, A, B, Y, stream=0) -> None:
+    call("docc_rocm_elementwise_binary", stream, BINARY_OPS[op] if isinstance(op, str) else op, precision, n, A, B, Y)
+
+
+def broadcast(precision, in_shape, out_shape, X, Y, stream=0) -> None:
+    rank = len(out_shape)
+    in_shape = (1,) * (rank - len(in_shape)) + tuple(in_shape)   # numpy rule: missing leading dimensions are 1
+    ins = (ctypes.c_int64 * rank)(*in_shape)
+    outs = (ctypes.c_int64 * rank)(*out_shape)
+    call("docc_rocm_broadcast", stream, precision, rank, ctypes.addressof(ins), ctypes.addressof(outs), X, Y)
 
 
 def mfma_probe(precision, waves_per_simd, iters, operands, sink, stream=0) -> float:

@@ -104,6 +104,34 @@ int docc_rocm_convert_bf16_to_f32(docc_rocm_stream_t stream, int64_t count, cons
  * calibrated. */
 int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* src, void* dst);
 
+/* Elementwise tensor nodes (reference sdfg/include/sdfg/data_flow/library_nodes/math/tensor/
+ * elementwise_node.h: ElementWiseUnaryNode Y[i] = f(X[i]), ElementWiseBinaryNode
+ * Y[i] = f(A[i], B[i]) over the linearised shape; replaces the Maps their expand()
+ * emits). `precision` 32 (float) or 64 (double); `n` elements; in place (Y == X or
+ * Y == A) is allowed. Operation codes: */
+#define DOCC_ROCM_UNARY_ABS 0      /* ml::Abs      fabs        */
+#define DOCC_ROCM_UNARY_EXP 1      /* ml::Exp      exp         */
+#define DOCC_ROCM_UNARY_RELU 2     /* ml::ReLU     fmax(x, 0)  (elementwise_ops/relu_node.cpp:40-43) */
+#define DOCC_ROCM_UNARY_SIGMOID 3  /* ml::Sigmoid  1/(1+exp(-x)) (sigmoid_node.cpp:46-70) */
+#define DOCC_ROCM_UNARY_SQRT 4     /* ml::Sqrt     sqrt        */
+#define DOCC_ROCM_UNARY_TANH 5     /* ml::Tanh     tanh        */
+#define DOCC_ROCM_UNARY_ERF 6      /* ml::Erf      erf         */
+#define DOCC_ROCM_BINARY_ADD 0     /* ml::Add */
+#define DOCC_ROCM_BINARY_SUB 1     /* ml::Sub */
+#define DOCC_ROCM_BINARY_MUL 2     /* ml::Mul */
+#define DOCC_ROCM_BINARY_DIV 3     /* ml::Div */
+#define DOCC_ROCM_BINARY_MAXIMUM 4 /* ml::Maximum  fmax (maximum_node.cpp:64) */
+#define DOCC_ROCM_BINARY_MINIMUM 5 /* ml::Minimum  fmin */
+int docc_rocm_elementwise_unary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y);
+int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A, const void* B,
+                                 void* Y);
+
+/* ml::Broadcast (reference .../tensor/broadcast_node.h:13-43): Y of shape out_shape is X
+ * of shape in_shape repeated along every dimension where in_shape is 1 (numpy rules,
+ * equal ranks, rank 1..6). Shapes are host arrays of `rank` extents. */
+int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, const int64_t* in_shape, const int64_t* out_shape,
+                        const void* X, void* Y);
+
 /* Measurement aid, no counterpart in the reference: `iters` rounds of 32 back-to-back
  * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16) on
  * every SIMD, `waves_per_simd` (1 or 2) waves each, operands taken from `operands`

@@ -57,6 +57,11 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.oracle_conv2d_f32.argtypes = [_i64] * 13 + [_f32p, _f32p, _f32p, _f32p]
     lib.oracle_attention_bf16.argtypes = [_i64] * 5 + [ctypes.c_float, _u16p, _u16p, _u16p, _f32p]
     lib.oracle_attention_bf16.restype = ctypes.c_int
+    lib.oracle_elementwise_unary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p]
+    lib.oracle_elementwise_unary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p]
+    lib.oracle_elementwise_binary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p, _f32p]
+    lib.oracle_elementwise_binary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p, _f64p]
+    lib.oracle_broadcast.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), ctypes.c_void_p, ctypes.c_void_p]
     return lib
 
 
@@ -199,3 +204,50 @@ def attention(Q_bits, K_bits, V_bits, scale=None, lib=None) -> np.ndarray:
     if lib.oracle_attention_bf16(B, H, SQ, SKV, D, scale, _p(Q, _u16p), _p(K, _u16p), _p(V, _u16p), _p(O, _f32p)) != 0:
         raise MemoryError("oracle attention could not allocate its scratch row")
     return O
+
+
+UNARY_OPS = {"abs": 0, "exp": 1, "relu": 2, "sigmoid": 3, "sqrt": 4, "tanh": 5, "erf": 6}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+
+
+def elementwise_unary(op: str, X, lib=None) -> np.ndarray:
+    """Y[i] = f(X[i]) for fp32 or fp64 X of any shape."""
+    lib = lib or load()
+    dt = np.float64 if np.asarray(X).dtype == np.float64 else np.float32
+    X = _c(X, dt)
+    out = np.empty_like(X)
+    ptr = _f64p if dt == np.float64 else _f32p
+    fn = lib.oracle_elementwise_unary_f64 if dt == np.float64 else lib.oracle_elementwise_unary_f32
+    if fn(UNARY_OPS[op], X.size, _p(X, ptr), _p(out, ptr)) != 0:
+        raise ValueError(f"unknown unary operation {op}")
+    return out
+
+
+def elementwise_binary(op: str, A, B, lib=None) -> np.ndarray:
+    """Y[i] = f(A[i], B[i]) for equally shaped fp32 or fp64 operands."""
+    lib = lib or load()
+    dt = np.float64 if np.asarray(A).dtype == np.float64 else np.float32
+    A, B = _c(A, dt), _c(B, dt)
+    if A.shape != B.shape:
+        raise ValueError("elementwise operands must have the same shape (broadcast first)")
+    out = np.empty_like(A)
+    ptr = _f64p if dt == np.float64 else _f32p
+    fn = lib.oracle_elementwise_binary_f64 if dt == np.float64 else lib.oracle_elementwise_binary_f32
+    if fn(BINARY_OPS[op], A.size, _p(A, ptr), _p(B, ptr), _p(out, ptr)) != 0:
+        raise ValueError(f"unknown binary operation {op}")
+    return out
+
+
+def broadcast(X, out_shape, lib=None) -> np.ndarray:
+    """ml::Broadcast: X (rank padded on the left with 1s) repeated to out_shape."""
+    lib = lib or load()
+    X = np.ascontiguousarray(X)
+    out_shape = tuple(int(d) for d in out_shape)
+    in_shape = (1,) * (len(out_shape) - X.ndim) + X.shape
+    out = np.empty(out_shape, X.dtype)
+    ins = (_i64 * len(out_shape))(*in_shape)
+    outs = (_i64 * len(out_shape))(*out_shape)
+    rc = lib.oracle_broadcast(X.dtype.itemsize, len(out_shape), ins, outs, X.ctypes.data, out.ctypes.data)
+    if rc != 0:
+        raise ValueError(f"cannot broadcast {X.shape} to {out_shape}")
+    return out

@@ -29,7 +29,11 @@
  *               shift, all-ones tap counts at corner/edge/interior, bias-only;
  *   attention   torch SDPA (math path) in fp64, equal-keys => mean of V,
  *               key-permutation invariance;
- *   bf16 conversion: exhaustive against torch's round-to-nearest-even.
+ *   bf16 conversion: exhaustive against torch's round-to-nearest-even;
+ *   elementwise_*  numpy's ufuncs (bit-exact for the IEEE operations and the
+ *               selections, <= 2 ulp for exp/tanh/erf/sigmoid), closed forms
+ *               (relu of negatives is +0, sigmoid(0) = 1/2, tanh odd, x/x = 1);
+ *   broadcast   numpy.broadcast_to.
  * The reference holds no numeric golden vectors for any of these nodes (its
  * tests recompute expectations with numpy/torch at run time), so the pins
  * above are the mathematics and the library cross-checks.
@@ -394,4 +398,106 @@ ORACLE_API int oracle_attention_bf16(int64_t B, int64_t H, int64_t SQ, int64_t S
         free(s);
     }
     return rc;
+}
+
+
+/* ------------------------------------------------------------------------------------------
+ * Elementwise tensor nodes: Y[i] = f(X[i]) / f(A[i], B[i]) over the linearised shape
+ * (sdfg/include/sdfg/data_flow/library_nodes/math/tensor/elementwise_node.h; expansions in
+ * sdfg/src/data_flow/library_nodes/math/tensor/elementwise_ops/: relu_node.cpp:40-43 fmax(x, 0.0),
+ * sigmoid_node.cpp:46-70 neg -> exp -> add 1.0 -> 1.0 / x, maximum_node.cpp:64 fmax, minimum_node.cpp
+ * fmin, abs/exp/sqrt/tanh/erf the libm call of the element type, add/sub/mul/div one tasklet).
+ * One Map over the elements: omp parallel for. Operation codes as in include/docc_rocm_ops.h. */
+#define ORACLE_UNARY_BODY(T, SUF)                                                          \
+    switch (op) {                                                                          \
+        case 0: y = fabs##SUF(x); break;                                                   \
+        case 1: y = exp##SUF(x); break;                                                    \
+        case 2: y = fmax##SUF(x, (T) 0.0); break;                                          \
+        case 3: { T t = -x; t = exp##SUF(t); t = t + (T) 1.0; y = (T) 1.0 / t; break; }    \
+        case 4: y = sqrt##SUF(x); break;                                                   \
+        case 5: y = tanh##SUF(x); break;                                                   \
+        default: y = erf##SUF(x); break;                                                   \
+    }
+#define ORACLE_BINARY_BODY(T, SUF)                                                         \
+    switch (op) {                                                                          \
+        case 0: y = a + b; break;                                                          \
+        case 1: y = a - b; break;                                                          \
+        case 2: y = a * b; break;                                                          \
+        case 3: y = a / b; break;                                                          \
+        case 4: y = fmax##SUF(a, b); break;                                                \
+        default: y = fmin##SUF(a, b); break;                                               \
+    }
+
+ORACLE_API int oracle_elementwise_unary_f32(int op, int64_t n, const float* X, float* Y) {
+    if (op < 0 || op > 6) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const float x = X[i];
+        float y;
+        ORACLE_UNARY_BODY(float, f)
+        Y[i] = y;
+    }
+    return 0;
+}
+
+ORACLE_API int oracle_elementwise_unary_f64(int op, int64_t n, const double* X, double* Y) {
+    if (op < 0 || op > 6) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const double x = X[i];
+        double y;
+        ORACLE_UNARY_BODY(double, )
+        Y[i] = y;
+    }
+    return 0;
+}
+
+ORACLE_API int oracle_elementwise_binary_f32(int op, int64_t n, const float* A, const float* B, float* Y) {
+    if (op < 0 || op > 5) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const float a = A[i], b = B[i];
+        float y;
+        ORACLE_BINARY_BODY(float, f)
+        Y[i] = y;
+    }
+    return 0;
+}
+
+ORACLE_API int oracle_elementwise_binary_f64(int op, int64_t n, const double* A, const double* B, double* Y) {
+    if (op < 0 || op > 5) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const double a = A[i], b = B[i];
+        double y;
+        ORACLE_BINARY_BODY(double, )
+        Y[i] = y;
+    }
+    return 0;
+}
+
+/* ml::Broadcast (sdfg/include/sdfg/data_flow/library_nodes/math/tensor/broadcast_node.h:13-43): the
+ * output of shape out_shape reads the input at the same coordinates, with coordinate 0 along every
+ * dimension whose input extent is 1. `esize` bytes per element, equal ranks. */
+ORACLE_API int oracle_broadcast(int esize, int rank, const int64_t* in_shape, const int64_t* out_shape, const void* X, void* Y) {
+    if (rank < 1 || rank > 8) return 1;
+    int64_t in_stride[8], n = 1, stride = 1;
+    for (int d = rank - 1; d >= 0; d--) {
+        if (in_shape[d] != out_shape[d] && in_shape[d] != 1) return 2;
+        in_stride[d] = in_shape[d] == 1 ? 0 : stride;
+        stride *= in_shape[d];
+        n *= out_shape[d];
+    }
+    const char* x = (const char*) X;
+    char* y = (char*) Y;
+#pragma omp parallel for schedule(static)
+    for (int64_t o = 0; o < n; o++) {
+        int64_t rem = o, off = 0;
+        for (int d = rank - 1; d >= 0; d--) {
+            off += (rem % out_shape[d]) * in_stride[d];
+            rem /= out_shape[d];
+        }
+        memcpy(y + o * esize, x + off * esize, (size_t) esize);
+    }
+    return 0;
 }

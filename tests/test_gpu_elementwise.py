@@ -1,0 +1,128 @@
+"""Elementwise tensor nodes and ml::Broadcast on the GPU against the CPU oracle, through
+docc_rocm_elementwise_unary / _binary / docc_rocm_broadcast.
+
+Bars: bit-exact for the IEEE operations and the selections (add, sub, mul, div, maximum, minimum,
+abs, relu, sqrt, broadcast); exp / tanh / sigmoid / erf within 4 units in the last place of the
+oracle's libm result (1e-6 relative in fp32, 1e-15 in fp64)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+EXACT_UNARY = ["abs", "relu", "sqrt"]
+LIBM_UNARY = ["exp", "tanh", "sigmoid", "erf"]
+BINARY = ["add", "sub", "mul", "div", "maximum", "minimum"]
+SIZES = [0, 1, 3, 4, 255, 1000, 4099, 1 << 20]
+
+
+def prec(dt):
+    return 64 if dt == np.float64 else 32
+
+
+def run_unary(rt, op, x, offset=0, in_place=False):
+    buf = dev(np.concatenate([np.zeros(offset, x.dtype), x.ravel()]))
+    out = buf if in_place else torch.full_like(buf, float("nan"))
+    es = buf.element_size()
+    rt.elementwise_unary(op, prec(x.dtype), x.size, buf.data_ptr() + offset * es, out.data_ptr() + offset * es)
+    torch.cuda.synchronize()
+    return host(out)[offset:].reshape(x.shape)
+
+
+def run_binary(rt, op, a, b, offset=0):
+    da = dev(np.concatenate([np.zeros(offset, a.dtype), a.ravel()]))
+    db = dev(np.concatenate([np.zeros(offset, a.dtype), b.ravel()]))
+    out = torch.full_like(da, float("nan"))
+    es = da.element_size()
+    rt.elementwise_binary(op, prec(a.dtype), a.size, da.data_ptr() + offset * es, db.data_ptr() + offset * es, out.data_ptr() + offset * es)
+    torch.cuda.synchronize()
+    return host(out)[offset:].reshape(a.shape)
+
+
+def ulps(y, ref):
+    spacing = np.spacing(np.abs(ref))
+    finite = np.isfinite(ref)
+    assert np.array_equal(np.isfinite(y), finite)
+    return float((np.abs(y[finite].astype(np.float64) - ref[finite].astype(np.float64)) / spacing[finite]).max()) if finite.any() else 0.0
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("n", SIZES)
+def test_binary_bit_exact(rt, dt, n):
+    rng = np.random.default_rng(n + 1)
+    a = (rng.standard_normal(n) * 10).astype(dt)
+    b = (rng.standard_normal(n) * 10).astype(dt)
+    if n > 100:
+        b[::97] = 0.0
+        a[::193] = np.nan
+        a[5], b[5] = np.inf, -np.inf
+    for op in BINARY:
+        for offset in (0, 1):   # offset 1: operands not 16-byte aligned -> scalar path
+            assert np.array_equal(run_binary(rt, op, a, b, offset), oracle.elementwise_binary(op, a, b), equal_nan=True), (op, offset)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("n", SIZES)
+def test_unary(rt, dt, n):
+    rng = np.random.default_rng(n + 7)
+    x = (rng.standard_normal(n) * 4).astype(dt)
+    if n > 100:
+        x[3], x[4], x[6] = np.inf, -np.inf, np.nan
+    for op in EXACT_UNARY:
+        arg = np.abs(x) if op == "sqrt" else x
+        for offset in (0, 1):
+            assert np.array_equal(run_unary(rt, op, arg, offset), oracle.elementwise_unary(op, arg), equal_nan=True), (op, offset)
+    for op in LIBM_UNARY:
+        ref = oracle.elementwise_unary(op, x)
+        got = run_unary(rt, op, x)
+        nan = np.isnan(ref)
+        assert np.array_equal(np.isnan(got), nan)
+        assert ulps(got[~nan], ref[~nan]) <= 4, op
+    # in place
+    assert np.array_equal(run_unary(rt, "relu", x, in_place=True), oracle.elementwise_unary("relu", x), equal_nan=True)
+
+
+def test_large_shape_and_closed_forms(rt):
+    # the benchmark shape of the softmax configuration, as an elementwise problem
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((8192, 4096)).astype(np.float32)
+    b = rng.standard_normal((8192, 4096)).astype(np.float32)
+    y = run_binary(rt, "add", a, b)
+    assert np.array_equal(y, a + b)
+    r = run_unary(rt, "relu", a)
+    assert (r >= 0).all() and np.array_equal(r, np.maximum(a, 0))
+    assert np.array_equal(run_binary(rt, "sub", a, a), np.zeros_like(a))
+    assert np.array_equal(run_binary(rt, "div", a, a), np.ones_like(a))
+    s = run_unary(rt, "sigmoid", np.zeros(1000, np.float32))
+    assert np.array_equal(s, np.full(1000, 0.5, np.float32))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("in_shape,out_shape", [((3,), (2, 3)), ((4, 1), (4, 5)), ((1, 3, 1, 2), (2, 3, 4, 2)), ((1,), (7,)),
+                                                ((2, 3), (2, 3)), ((1, 64, 1, 1), (8, 64, 14, 14)), ((1, 4096), (512, 4096)),
+                                                ((1, 1, 1, 1, 1, 5), (2, 3, 2, 3, 2, 5))])
+def test_broadcast(rt, dt, in_shape, out_shape):
+    rng = np.random.default_rng(len(out_shape))
+    x = rng.standard_normal(in_shape).astype(dt)
+    dx = dev(x)
+    out = torch.full(out_shape, float("nan"), device="cuda", dtype=torch.float64 if dt == np.float64 else torch.float32)
+    rt.broadcast(prec(dt), in_shape, out_shape, dx.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out), oracle.broadcast(x, out_shape))
+    assert np.array_equal(host(out), np.broadcast_to(x, out_shape))
+
+
+def test_errors(rt):
+    from docc_amd.runtime import RocmRuntimeError
+    a = torch.zeros(16, device="cuda")
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_unary(99, 32, 16, a.data_ptr(), a.data_ptr())
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_binary("add", 16, 16, a.data_ptr(), a.data_ptr(), a.data_ptr())     # precision 16
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_unary("exp", 32, 16, 0, a.data_ptr())
+    with pytest.raises(RocmRuntimeError):
+        rt.broadcast(32, (2, 3), (2, 4), a.data_ptr(), a.data_ptr())
+    rt.elementwise_unary("exp", 32, 0, 0, 0)   # empty: no-op

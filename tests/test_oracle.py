@@ -171,3 +171,81 @@ def test_attention_closed_forms():
     a = oracle.attention(bits(q), bits(k), bits(v))
     b = oracle.attention(bits(q), bits(k[:, :, perm]), bits(v[:, :, perm]))
     assert rel(a, b.astype(np.float64)) <= 1e-5
+
+
+# ---- elementwise nodes and broadcast ------------------------------------------------------
+
+def ulp_diff(y, ref):
+    """Largest distance in units in the last place of `ref`'s type."""
+    ref = np.asarray(ref)
+    y = np.asarray(y, ref.dtype)
+    spacing = np.spacing(np.abs(ref).astype(ref.dtype))
+    finite = np.isfinite(ref)
+    assert np.array_equal(np.isfinite(y), finite)
+    return float((np.abs(y[finite].astype(np.float64) - ref[finite].astype(np.float64)) / spacing[finite]).max()) if finite.any() else 0.0
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_elementwise_binary_matches_ieee(dt):
+    rng = np.random.default_rng(3)
+    a = (rng.standard_normal(1001) * 10).astype(dt)
+    b = (rng.standard_normal(1001) * 10).astype(dt)
+    b[::97] = 0.0                      # division by zero -> inf / nan as IEEE says
+    a[::193] = np.nan                  # fmax / fmin return the other operand for one NaN
+    with np.errstate(all="ignore"):
+        assert np.array_equal(oracle.elementwise_binary("add", a, b), a + b, equal_nan=True)
+        assert np.array_equal(oracle.elementwise_binary("sub", a, b), a - b, equal_nan=True)
+        assert np.array_equal(oracle.elementwise_binary("mul", a, b), a * b, equal_nan=True)
+        assert np.array_equal(oracle.elementwise_binary("div", a, b), a / b, equal_nan=True)
+    assert np.array_equal(oracle.elementwise_binary("maximum", a, b), np.fmax(a, b), equal_nan=True)
+    assert np.array_equal(oracle.elementwise_binary("minimum", a, b), np.fmin(a, b), equal_nan=True)
+    # not commutative operations in the right order
+    assert oracle.elementwise_binary("sub", np.array([5], dt), np.array([3], dt))[0] == 2
+    assert oracle.elementwise_binary("div", np.array([6], dt), np.array([3], dt))[0] == 2
+    with pytest.raises(ValueError):
+        oracle.elementwise_binary("add", np.zeros((2, 3), dt), np.zeros((3, 2), dt))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_elementwise_unary_closed_forms_and_numpy(dt):
+    rng = np.random.default_rng(4)
+    x = (rng.standard_normal(2001) * 4).astype(dt)
+    # exact operations
+    assert np.array_equal(oracle.elementwise_unary("abs", x), np.abs(x))
+    relu = oracle.elementwise_unary("relu", x)
+    assert np.array_equal(relu, np.fmax(x, dt(0)))
+    assert (relu >= 0).all() and np.array_equal(relu[x > 0], x[x > 0])
+    assert oracle.elementwise_unary("relu", np.array([np.nan], dt))[0] == 0          # fmax(NaN, 0) = 0
+    sq = oracle.elementwise_unary("sqrt", np.abs(x))
+    assert np.array_equal(sq, np.sqrt(np.abs(x)))                                    # correctly rounded in both
+    # transcendental ones: numpy evaluated in float64 (longdouble for fp64) and rounded is the yardstick
+    wide = np.longdouble if dt == np.float64 else np.float64
+    xw = x.astype(wide)
+    import scipy.special as sp
+    cases = {"exp": np.exp(xw), "tanh": np.tanh(xw), "sigmoid": 1 / (1 + np.exp(-xw)),
+             "erf": sp.erf(x.astype(np.float64)).astype(wide)}
+    for op, ref in cases.items():
+        assert ulp_diff(oracle.elementwise_unary(op, x), ref.astype(dt)) <= (4 if op == "sigmoid" else 2), op
+    # closed forms
+    z = np.zeros(3, dt)
+    assert np.array_equal(oracle.elementwise_unary("exp", z), np.ones(3, dt))
+    assert np.array_equal(oracle.elementwise_unary("sigmoid", z), np.full(3, 0.5, dt))
+    assert np.array_equal(oracle.elementwise_unary("tanh", -x), -oracle.elementwise_unary("tanh", x))
+    assert np.array_equal(oracle.elementwise_unary("erf", -x), -oracle.elementwise_unary("erf", x))
+    big = np.array([1000.0, -1000.0], dt)
+    assert np.array_equal(oracle.elementwise_unary("sigmoid", big), np.array([1.0, 0.0], dt))
+    assert np.array_equal(oracle.elementwise_unary("tanh", big), np.array([1.0, -1.0], dt))
+    # shape is kept
+    assert oracle.elementwise_unary("exp", np.zeros((2, 3, 4), dt)).shape == (2, 3, 4)
+
+
+def test_broadcast_matches_numpy():
+    rng = np.random.default_rng(5)
+    for in_shape, out_shape in [((3,), (2, 3)), ((4, 1), (4, 5)), ((1, 3, 1, 2), (2, 3, 4, 2)), ((1,), (7,)), ((2, 3), (2, 3)),
+                                ((64,), (2, 64, 1, 1))[:0] or ((1, 64, 1, 1), (2, 64, 3, 3))]:
+        x = rng.standard_normal(in_shape).astype(np.float32)
+        assert np.array_equal(oracle.broadcast(x, out_shape), np.broadcast_to(x, out_shape))
+        xd = rng.standard_normal(in_shape)
+        assert np.array_equal(oracle.broadcast(xd, out_shape), np.broadcast_to(xd, out_shape))
+    with pytest.raises(ValueError):
+        oracle.broadcast(np.zeros((2, 3), np.float32), (2, 4))
