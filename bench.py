@@ -47,7 +47,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv")
+    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
     return ap.parse_args()
 
@@ -275,6 +275,29 @@ def main():
             cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": "full problem, the reference's loop nest with a zero-padding guard (omp over n)"}
         add_kernel("conv2d_n32c64hw56k3", "f32", flops, ms, cpu)
+
+    # ---- elementwise tensor nodes on the softmax tensor's shape (HBM-bound) --------------------
+    if want("elementwise"):
+        n = 8192 * 4096
+        a, b2, y = (torch.randn(n, device="cuda") for _ in range(3))
+        cases = {"add_f32": (12 * n, lambda i: rt.elementwise_binary("add", 32, n, a.data_ptr(), b2.data_ptr(), y.data_ptr(), stream)),
+                 "relu_f32": (8 * n, lambda i: rt.elementwise_unary("relu", 32, n, a.data_ptr(), y.data_ptr(), stream)),
+                 "sigmoid_f32": (8 * n, lambda i: rt.elementwise_unary("sigmoid", 32, n, a.data_ptr(), y.data_ptr(), stream)),
+                 "broadcast_row_f32": (4 * n + 4 * 4096, lambda i: rt.broadcast(32, (1, 4096), (8192, 4096), a.data_ptr(), y.data_ptr(), stream))}
+        for name, (nbytes_e, fn) in cases.items():
+            ms = time_kernel(fn, 50, 5)
+            gbs = nbytes_e / ms / 1e6
+            kernels[f"elementwise_{name}_8192x4096"] = {
+                "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
+                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(gbs / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_e}}
+        if oracle_lib is not None:
+            ah, bh = a.cpu().numpy(), b2.cpu().numpy()
+            t = cpu_time(lambda: oracle.elementwise_binary("add", ah, bh, lib=oracle_lib))
+            kernels["elementwise_add_f32_8192x4096"]["cpu_baseline"] = {
+                "value": round(12 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
+                "sample": "full tensor, the Map the reference's ElementWiseBinaryNode expands to (omp parallel for)"}
+        del a, b2, y
 
     line = {
         "metric": METRIC,

@@ -105,28 +105,65 @@ __device__ __forceinline__ void binary_kernel(const T* A, const T* B, T* Y, long
     for (long i = nvec * N + tid; i < n; i += stride) Y[i] = binary<OP>(A[i], B[i]);
 }
 
-// ml::Broadcast: Y[o] = X[offset(o)], numpy rules (an input dimension of extent 1 repeats)
+// One operand is a scalar (the reference binds a constant or scalar container to "A" or "B",
+// python/bindings/builder/py_structured_sdfg_builder.cpp:894-908): Y[i] = f(A[i], b), or
+// f(b, A[i]) when LEFT.
+template <typename T, int OP, bool LEFT>
+__device__ __forceinline__ void binary_scalar_kernel(const T* A, T b, T* Y, long n, long nvec) {
+    typedef typename Vec128<T>::type V;
+    constexpr int N = Vec128<T>::N;
+    const long stride = (long) gridDim.x * blockDim.x;
+    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = tid; i < nvec; i += stride) {
+        V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(A) + i);
+#pragma unroll
+        for (int e = 0; e < N; e++) v[e] = LEFT ? binary<OP>(b, v[e]) : binary<OP>(v[e], b);
+        __builtin_nontemporal_store(v, reinterpret_cast<V*>(Y) + i);
+    }
+    for (long i = nvec * N + tid; i < n; i += stride) Y[i] = LEFT ? binary<OP>(b, A[i]) : binary<OP>(A[i], b);
+}
+
+// ml::Broadcast: Y[o] = X[offset(o)], numpy rules (an input dimension of extent 1 repeats).
+// The launcher collapses the shape first (extent-1 output dimensions dropped, neighbours that
+// are both repeated or both contiguous merged), so that `rank` is 1..3 for the usual cases.
+// Write-bound: 4 or 8 bytes per output element; the input is re-read from cache.
 struct BroadcastParams {
     int rank;
     long n;                 // elements of the output
     long out_dims[6];
-    long in_strides[6];     // in elements; 0 for a broadcast dimension
+    long in_strides[6];     // in elements; 0 for a repeated dimension
 };
 
-template <typename T>
+// VEC consecutive outputs of the innermost dimension per lane and step (its extent is a
+// multiple of VEC), one 128-bit store; I: index type (32-bit when the output fits)
+template <typename T, int VEC, typename I>
 __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const BroadcastParams& p) {
-    const long stride = (long) gridDim.x * blockDim.x;
-    for (long o = (long) blockIdx.x * blockDim.x + threadIdx.x; o < p.n; o += stride) {
-        long rem = o, off = 0;
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    const I stride = (I) gridDim.x * blockDim.x;
+    const I nv = (I) (p.n / VEC);
+    const int last = p.rank - 1;
+    const I inner = (I) p.out_dims[last] / VEC;
+    const bool inner_repeats = p.in_strides[last] == 0;
+    for (I v = (I) blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += stride) {
+        I rem = v / inner;
+        long off = inner_repeats ? 0 : (long) (v % inner) * VEC;
 #pragma unroll
-        for (int d = 5; d >= 0; d--) {
-            if (d < p.rank) {
-                const long c = rem % p.out_dims[d];
-                rem /= p.out_dims[d];
-                off += c * p.in_strides[d];
+        for (int d = 4; d >= 0; d--) {
+            if (d < last) {
+                const I e = (I) p.out_dims[d];
+                off += (long) (rem % e) * p.in_strides[d];
+                rem /= e;
             }
         }
-        Y[o] = X[off];
+        V y;
+        if (inner_repeats) {
+            const T x = X[off];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) y[e] = x;
+        } else {
+            y = *reinterpret_cast<const V*>(X + off);
+        }
+        __builtin_nontemporal_store(y, reinterpret_cast<V*>(Y) + v);
     }
 }
 
@@ -139,6 +176,15 @@ __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const Broadca
     extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f64(const double* X, double* Y, long n, long nvec) {     \
         docc_k::unary_kernel<double, docc_k::OP>(X, Y, n, nvec);                                                             \
     }
+#define DOCC_EW_BINARY_SCALAR(NAME, OP, SIDE, LEFT)                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_##SIDE##_f32(const float* A, float b, float* Y, long n,  \
+                                                                                    long nvec) {                             \
+        docc_k::binary_scalar_kernel<float, docc_k::OP, LEFT>(A, b, Y, n, nvec);                                             \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_##SIDE##_f64(const double* A, double b, double* Y,       \
+                                                                                    long n, long nvec) {                     \
+        docc_k::binary_scalar_kernel<double, docc_k::OP, LEFT>(A, b, Y, n, nvec);                                            \
+    }
 #define DOCC_EW_BINARY(NAME, OP)                                                                                             \
     extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f32(const float* A, const float* B, float* Y, long n,    \
                                                                            long nvec) {                                      \
@@ -147,7 +193,9 @@ __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const Broadca
     extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f64(const double* A, const double* B, double* Y, long n, \
                                                                            long nvec) {                                      \
         docc_k::binary_kernel<double, docc_k::OP>(A, B, Y, n, nvec);                                                         \
-    }
+    }                                                                                                                        \
+    DOCC_EW_BINARY_SCALAR(NAME, OP, sr, false)                                                                               \
+    DOCC_EW_BINARY_SCALAR(NAME, OP, sl, true)
 
 DOCC_EW_UNARY(abs, kAbs)
 DOCC_EW_UNARY(exp, kExp)
@@ -163,9 +211,16 @@ DOCC_EW_BINARY(div, kDiv)
 DOCC_EW_BINARY(maximum, kMaximum)
 DOCC_EW_BINARY(minimum, kMinimum)
 
-extern "C" __global__ __launch_bounds__(256) void docc_broadcast_f32(const float* X, float* Y, docc_k::BroadcastParams p) {
-    docc_k::broadcast_kernel<float>(X, Y, p);
-}
-extern "C" __global__ __launch_bounds__(256) void docc_broadcast_f64(const double* X, double* Y, docc_k::BroadcastParams p) {
-    docc_k::broadcast_kernel<double>(X, Y, p);
-}
+#define DOCC_BROADCAST(NAME, T, VEC, I)                                                                                     \
+    extern "C" __global__ __launch_bounds__(256) void docc_broadcast_##NAME(const T* X, T* Y, docc_k::BroadcastParams p) {     \
+        docc_k::broadcast_kernel<T, VEC, I>(X, Y, p);                                                                       \
+    }
+// <type>_v<lanes>_i<index bits>
+DOCC_BROADCAST(f32_v4_i32, float, 4, unsigned)
+DOCC_BROADCAST(f32_v1_i32, float, 1, unsigned)
+DOCC_BROADCAST(f32_v4_i64, float, 4, long)
+DOCC_BROADCAST(f32_v1_i64, float, 1, long)
+DOCC_BROADCAST(f64_v2_i32, double, 2, unsigned)
+DOCC_BROADCAST(f64_v1_i32, double, 1, unsigned)
+DOCC_BROADCAST(f64_v2_i64, double, 2, long)
+DOCC_BROADCAST(f64_v1_i64, double, 1, long)

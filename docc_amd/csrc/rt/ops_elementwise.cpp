@@ -70,28 +70,72 @@ extern "C" int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, i
                   nvec);
 }
 
+extern "C" int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A,
+                                                   double scalar, int scalar_is_lhs, void* Y) {
+    if (op < 0 || op >= (int) (sizeof(kBinaryNames) / sizeof(kBinaryNames[0])))
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_binary_scalar: unknown operation %d", op);
+    if (int rc = check_precision("elementwise_binary_scalar", precision)) return rc;
+    if (n < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_binary_scalar: negative count");
+    if (n == 0) return 0;
+    if (!A || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_binary_scalar: null pointer");
+    if (int rc = ensure_device()) return rc;
+    const int per_vec = precision == 32 ? 4 : 2;
+    const bool aligned = (((uintptr_t) A | (uintptr_t) Y) % 16) == 0;
+    const long nvec = aligned ? (long) (n / per_vec) : 0;
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_ew_%s_%s_f%d", kBinaryNames[op], scalar_is_lhs ? "sl" : "sr", precision);
+    const uint32_t grid = grid_for(aligned ? (n + per_vec - 1) / per_vec : n);
+    if (precision == 32) return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, A, (float) scalar, Y, (long) n, nvec);
+    return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, A, scalar, Y, (long) n, nvec);
+}
+
 extern "C" int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, const int64_t* in_shape,
                                    const int64_t* out_shape, const void* X, void* Y) {
     if (int rc = check_precision("broadcast", precision)) return rc;
     if (rank < 1 || rank > 6) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "broadcast: rank %d (1..6 are built)", rank);
     if (!in_shape || !out_shape) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "broadcast: null shape");
-    BroadcastParams p{};
-    p.rank = rank;
-    p.n = 1;
-    long stride = 1;
+    long dims[6], strides[6];
+    long n = 1, stride = 1;
     for (int d = rank - 1; d >= 0; d--) {
         if (in_shape[d] < 0 || out_shape[d] < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "broadcast: negative extent");
         if (in_shape[d] != out_shape[d] && in_shape[d] != 1)
             return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "broadcast: dimension %d has extent %lld, cannot become %lld", d,
                         (long long) in_shape[d], (long long) out_shape[d]);
-        p.out_dims[d] = (long) out_shape[d];
-        p.in_strides[d] = in_shape[d] == 1 ? 0 : stride;
+        dims[d] = (long) out_shape[d];
+        strides[d] = in_shape[d] == 1 ? 0 : stride;
         stride *= (long) in_shape[d];
-        p.n *= (long) out_shape[d];
+        n *= (long) out_shape[d];
     }
-    if (p.n == 0) return 0;
+    if (n == 0) return 0;
     if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "broadcast: null pointer");
     if (int rc = ensure_device()) return rc;
-    return launch(precision == 32 ? "docc_broadcast_f32" : "docc_broadcast_f64", grid_for(p.n), 1, 1, 256, 0, (hipStream_t) stream, X, Y,
-                  p);
+    // collapse: drop extent-1 dimensions, merge neighbours that are both repeated or contiguous
+    BroadcastParams p{};
+    p.n = n;
+    int r = 0;
+    for (int d = 0; d < rank; d++) {
+        if (dims[d] == 1) continue;
+        if (r > 0 && ((p.in_strides[r - 1] == 0 && strides[d] == 0) ||
+                      (strides[d] != 0 && p.in_strides[r - 1] == strides[d] * dims[d]))) {
+            p.out_dims[r - 1] *= dims[d];
+            p.in_strides[r - 1] = strides[d];
+        } else {
+            p.out_dims[r] = dims[d];
+            p.in_strides[r] = strides[d];
+            r++;
+        }
+    }
+    if (r == 0) {  // a single element
+        p.out_dims[0] = 1;
+        p.in_strides[0] = 0;
+        r = 1;
+    }
+    p.rank = r;
+    const int per_vec = precision == 32 ? 4 : 2;
+    const bool vec = p.out_dims[r - 1] % per_vec == 0 && (uintptr_t) Y % 16 == 0 &&
+                     (p.in_strides[r - 1] == 0 || (uintptr_t) X % 16 == 0);
+    const int lanes = vec ? per_vec : 1;
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_broadcast_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
+    return launch(name, grid_for(n / lanes), 1, 1, 256, 0, (hipStream_t) stream, X, Y, p);
 }

@@ -22,10 +22,19 @@ bool is_rocm_impl(const std::string& impl) {
     return impl == ImplementationType_ROCMWithTransfers || impl == ImplementationType_ROCMWithoutTransfers;
 }
 
+bool is_elementwise_code(const std::string& c) {
+    for (auto& u : tensor::UnaryNodeCodes)
+        if (u == c) return true;
+    for (auto& b : tensor::BinaryNodeCodes)
+        if (b == c) return true;
+    return false;
+}
+
 bool is_math_node(const LibraryNode& node) {
     const std::string& c = node.code();
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
-           c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention;
+           c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
+           is_elementwise_code(c);
 }
 
 // Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
@@ -181,7 +190,7 @@ protected:
     const tensor::MatMulNode& mm() const { return static_cast<const tensor::MatMulNode&>(node_); }
 
     std::vector<DeviceOperand> operands() const override {
-        return {operand("A", true, false), operand("B", true, false), operand("Y", false, true)};
+        return {operand("A", true, false), operand("B", true, false), operand("C", false, true)};
     }
 
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
@@ -315,6 +324,78 @@ public:
     }
 };
 
+// ---- Elementwise / Broadcast ----------------------------------------------------------------
+// Counterpart of what CUDAMapDispatcher prints for the Maps these nodes expand to (reference
+// opt/src/targets/cuda/...): here one launcher call per node.
+
+class ElementWiseNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    // a constant or a scalar container bound to "A" or "B" (the reference's builder binds
+    // either, python/bindings/builder/py_structured_sdfg_builder.cpp:894-908)
+    bool is_scalar(const std::string& connector) const {
+        const auto* in = data_flow_graph_.input(connector);
+        return in && (in->is_constant || !function_.container(in->data).is_pointer);
+    }
+
+    std::vector<DeviceOperand> operands() const override {
+        const auto& n = static_cast<const tensor::ElementWiseNode&>(node_);
+        if (!n.is_binary()) return {operand("X", true, false), operand("Y", false, true)};
+        std::vector<DeviceOperand> ops;
+        if (!is_scalar("A")) ops.push_back(operand("A", true, false));
+        if (!is_scalar("B")) ops.push_back(operand("B", true, false));
+        ops.push_back(operand("C", false, true));
+        return ops;
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::ElementWiseNode&>(node_);
+        const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
+        if (!n.is_binary()) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_elementwise_unary(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision
+              << ", " << n.count() << ", " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+            return;
+        }
+        const bool sa = is_scalar("A"), sb = is_scalar("B");
+        if (sa && sb) throw InvalidSDFGException(n.code() + ": both operands are scalars");
+        if (sa || sb)
+            s << "DOCC_ROCM_CHECK(docc_rocm_elementwise_binary_scalar(nullptr, " << n.operation() << " /* " << n.code() << " */, "
+              << precision << ", " << n.count() << ", " << name_of(sa ? "B" : "A") << ", (double) " << (sa ? "A" : "B") << ", "
+              << (sa ? 1 : 0) << ", " << name_of("C") << "));" << std::endl;
+        else
+            s << "DOCC_ROCM_CHECK(docc_rocm_elementwise_binary(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision
+              << ", " << n.count() << ", " << name_of("A") << ", " << name_of("B") << ", " << name_of("C") << "));" << std::endl;
+    }
+};
+
+class BroadcastNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::BroadcastNode&>(node_);
+        const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        auto list = [&](const char* name, const std::vector<Expression>& shape) {
+            s << "const int64_t " << name << "[] = {";
+            for (size_t i = 0; i < shape.size(); i++) s << (i ? ", " : "") << "(int64_t) (" << shape[i] << ")";
+            s << "};" << std::endl;
+        };
+        list("__docc_in_shape", n.input_shape());
+        list("__docc_out_shape", n.output_shape());
+        s << "DOCC_ROCM_CHECK(docc_rocm_broadcast(nullptr, " << precision << ", " << n.output_shape().size()
+          << ", __docc_in_shape, __docc_out_shape, " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+};
+
 template <typename D>
 void register_math(codegen::LibraryNodeDispatcherRegistry& reg, const std::string& code) {
     for (bool with : {true, false}) {
@@ -342,6 +423,9 @@ void register_plugin(plugins::Context& context) {
     register_math<SoftmaxNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Softmax);
     register_math<ConvNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Conv);
     register_math<AttentionNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Attention);
+    for (auto& code : tensor::UnaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
+    for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
+    register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
     reg.register_library_node_dispatcher(
         LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
         [](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
@@ -398,6 +482,15 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
         int64_t d = 0;
         if (!symbolic::is_integer(a->shape_q()[3], &d) || d != 64) return decline("head dimension must be 64");
+    } else if (is_elementwise_code(node.code())) {
+        auto* e = dynamic_cast<tensor::ElementWiseNode*>(&node);
+        if (!e) return decline("not an elementwise node object");
+        if (e->element() != P::Float && e->element() != P::Double) return decline("element type must be Float or Double");
+    } else if (node.code() == tensor::LibraryNodeType_Broadcast) {
+        auto* b = dynamic_cast<tensor::BroadcastNode*>(&node);
+        if (!b) return decline("not a Broadcast node object");
+        if (b->element() != P::Float && b->element() != P::Double) return decline("element type must be Float or Double");
+        if (b->output_shape().size() > 6) return decline("rank above 6 is not supported");
     } else {
         return false;  // not a node of this target
     }

@@ -401,6 +401,80 @@ Expression AttentionNode::connector_bytes(const std::string& connector) const {
     return bytes_of(symbolic::mul(symbolic::mul(bh, seq_kv_), shape_q_[3]), element_);
 }
 
+// ---- elementwise / broadcast ----
+
+static bool is_in(const std::vector<std::string>& v, const std::string& s) {
+    for (auto& e : v)
+        if (e == s) return true;
+    return false;
+}
+
+ElementWiseNode::ElementWiseNode(std::string code, std::string implementation_type, std::vector<Expression> shape,
+                                 types::PrimitiveType element)
+    : LibraryNode(code, is_in(BinaryNodeCodes, code) ? std::vector<std::string>{"C"} : std::vector<std::string>{"Y"},
+                  is_in(BinaryNodeCodes, code) ? std::vector<std::string>{"A", "B"} : std::vector<std::string>{"X"}, false,
+                  std::move(implementation_type)),
+      shape_(std::move(shape)), element_(element) {}
+
+int ElementWiseNode::operation() const {
+    const auto& codes = is_binary() ? BinaryNodeCodes : UnaryNodeCodes;
+    for (size_t i = 0; i < codes.size(); i++)
+        if (codes[i] == code_) return (int) i;
+    return -1;
+}
+
+Expression ElementWiseNode::count() const { return product(shape_, 0, shape_.size()); }
+
+void ElementWiseNode::validate() const {
+    if (operation() < 0) throw InvalidSDFGException(code_ + ": not an elementwise node code");
+    if (shape_.empty()) throw InvalidSDFGException(code_ + ": empty shape");
+}
+
+void ElementWiseNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<ElementWiseNode> ElementWiseNode::from_json(const Value& j) {
+    const Value* et = j.find("element_type");
+    return std::make_unique<ElementWiseNode>(j.at("code").as_string(), impl_of(j), exprs_from_json(j.at("shape")),
+                                             et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression ElementWiseNode::connector_bytes(const std::string&) const { return bytes_of(count(), element_); }
+
+BroadcastNode::BroadcastNode(std::string implementation_type, std::vector<Expression> input_shape,
+                             std::vector<Expression> output_shape, types::PrimitiveType element)
+    : LibraryNode(LibraryNodeType_Broadcast, {"Y"}, {"X"}, false, std::move(implementation_type)),
+      input_shape_(std::move(input_shape)), output_shape_(std::move(output_shape)), element_(element) {}
+
+void BroadcastNode::validate() const {
+    if (output_shape_.empty()) throw InvalidSDFGException("Broadcast: empty output shape");
+    if (input_shape_.size() != output_shape_.size()) throw InvalidSDFGException("Broadcast: input and output ranks differ");
+    for (size_t d = 0; d < input_shape_.size(); d++) {
+        int64_t a = 0, b = 0;
+        if (symbolic::is_integer(input_shape_[d], &a) && symbolic::is_integer(output_shape_[d], &b) && a != b && a != 1)
+            throw InvalidSDFGException("Broadcast: dimension " + std::to_string(d) + " cannot be broadcast");
+    }
+}
+
+void BroadcastNode::to_json(Value& j) const {
+    j.set("input_shape", exprs_to_json(input_shape_));
+    j.set("output_shape", exprs_to_json(output_shape_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<BroadcastNode> BroadcastNode::from_json(const Value& j) {
+    const Value* et = j.find("element_type");
+    return std::make_unique<BroadcastNode>(impl_of(j), exprs_from_json(j.at("input_shape")), exprs_from_json(j.at("output_shape")),
+                                           et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression BroadcastNode::connector_bytes(const std::string& connector) const {
+    const auto& shape = connector == "X" ? input_shape_ : output_shape_;
+    return bytes_of(product(shape, 0, shape.size()), element_);
+}
+
 } // namespace math::tensor
 
 // ------------------------------------------------------------- offloading
@@ -694,6 +768,9 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     fns_[math::tensor::LibraryNodeType_Softmax] = &deserialize<math::tensor::SoftmaxNode>;
     fns_[math::tensor::LibraryNodeType_Conv] = &deserialize<math::tensor::ConvNode>;
     fns_[math::tensor::LibraryNodeType_MatMul] = &deserialize<math::tensor::MatMulNode>;
+    for (auto& code : math::tensor::UnaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
+    for (auto& code : math::tensor::BinaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
+    fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
 }
 
 LibraryNodeSerializerRegistry& LibraryNodeSerializerRegistry::instance() {

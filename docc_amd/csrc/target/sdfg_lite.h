@@ -276,6 +276,53 @@ private:
     types::PrimitiveType element_, output_element_;
 };
 
+// Elementwise tensor nodes: Y[i] = f(X[i]) or f(A[i], B[i]) over the linearised shape.
+// reference: .../tensor/elementwise_node.cpp:20 (ElementWiseUnaryNode "X" -> "Y"), :176
+// (ElementWiseBinaryNode "A","B" -> "C"), JSON keys code + shape; elementwise_ops/*.h for the codes.
+inline const std::vector<std::string> UnaryNodeCodes = {"ml::Abs", "ml::Exp", "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf"};
+inline const std::vector<std::string> BinaryNodeCodes = {"ml::Add", "ml::Sub", "ml::Mul", "ml::Div", "ml::Maximum", "ml::Minimum"};
+inline const std::string LibraryNodeType_Broadcast = "ml::Broadcast";
+
+class ElementWiseNode : public data_flow::LibraryNode {
+public:
+    ElementWiseNode(std::string code, std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element);
+    const std::vector<Expression>& shape() const { return shape_; }
+    types::PrimitiveType element() const { return element_; }
+    bool is_binary() const { return inputs_.size() == 2; }
+    // position of the code in UnaryNodeCodes / BinaryNodeCodes = the runtime's operation code
+    int operation() const;
+    Expression count() const;
+
+    void validate() const override;
+    Expression flop() const override { return count(); }
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ElementWiseNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    types::PrimitiveType element_;
+};
+
+// reference: .../tensor/broadcast_node.h:13-80 ("X" -> "Y", JSON keys input_shape, output_shape)
+class BroadcastNode : public data_flow::LibraryNode {
+public:
+    BroadcastNode(std::string implementation_type, std::vector<Expression> input_shape, std::vector<Expression> output_shape,
+                  types::PrimitiveType element);
+    const std::vector<Expression>& input_shape() const { return input_shape_; }
+    const std::vector<Expression>& output_shape() const { return output_shape_; }
+    types::PrimitiveType element() const { return element_; }
+
+    void validate() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<BroadcastNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> input_shape_, output_shape_;
+    types::PrimitiveType element_;
+};
+
 } // namespace math::tensor
 
 namespace rocm {

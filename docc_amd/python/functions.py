@@ -31,3 +31,19 @@ def conv2d(x, w, bias=None, stride=1, padding=0, dilation=1):
     if bias is not None:
         y += np.asarray(bias).reshape(1, -1, 1, 1)
     return y
+
+
+def relu(x):
+    """max(x, 0) elementwise (the ml::ReLU node)."""
+    return np.maximum(x, 0)
+
+
+def sigmoid(x):
+    """1 / (1 + exp(-x)) elementwise (the ml::Sigmoid node)."""
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+def erf(x):
+    """The error function elementwise (the ml::Erf node)."""
+    from scipy.special import erf as _erf
+    return _erf(x)

@@ -20,6 +20,11 @@ NotImplementedError (there is no CPU lowering behind it):
     the decomposed form  m = np.max(x, axis=-1, keepdims=True); e = np.exp(x - m);
                          s = np.sum(e, axis=-1, keepdims=True); e / s
     conv2d(x, w, bias, stride=, padding=, dilation=)
+    x + y, x - y, x * y, x / y, np.maximum(x, y), np.minimum(x, y) on float arrays whose shapes
+        broadcast by numpy's rules (the smaller operand goes through ml::Broadcast), or on an
+        array and a scalar (literal or scalar argument)
+    np.abs, np.exp, np.sqrt, np.tanh, scipy.special.erf / expit, relu(x), sigmoid(x),
+        np.maximum(x, 0)  (ReLU)
 """
 from __future__ import annotations
 
@@ -231,6 +236,97 @@ class _Lowering(ast.NodeVisitor):
                         w.shape[0], 1, bias.name if bias is not None else None)
         return out
 
+    def broadcast_shape(self, node: ast.AST, a: Sequence[str], b: Sequence[str]) -> List[str]:
+        rank = max(len(a), len(b))
+        a, b = ["1"] * (rank - len(a)) + list(a), ["1"] * (rank - len(b)) + list(b)
+        out = []
+        for x, y in zip(a, b):
+            if x != y and x != "1" and y != "1":
+                raise ValueError(f"{self.func.__name__}: operands could not be broadcast together ({a} vs {b})")
+            out.append(y if x == "1" else x)
+        return out
+
+    def expanded(self, x: _Array, shape: List[str]) -> _Array:
+        """`x` repeated to `shape` through ml::Broadcast (a no-op when the shapes agree)."""
+        if x.shape == shape:
+            return x
+        padded = ["1"] * (len(shape) - len(x.shape)) + x.shape
+        if len(shape) > 6:
+            raise NotImplementedError(f"{self.func.__name__}: broadcast of rank {len(shape)} (up to 6 are built)")
+        out = self.new_array(shape, x.elem, None)
+        self.b.add_broadcast(x.name, out.name, padded, shape)
+        return out
+
+    def array_of(self, node: ast.AST, v: Any) -> Any:
+        """Materialises `scalar * array` as an array; other values pass through."""
+        if isinstance(v, _Lazy) and v.kind == "scaled":
+            return self.elementwise(node, "mul", v.base, v.scalar, None)
+        return v
+
+    def elementwise(self, node: ast.AST, op: str, a: Any, b: Any, dest: Optional[str]) -> _Array:
+        a, b = self.array_of(node, a), self.array_of(node, b)
+        arrays = [v for v in (a, b) if isinstance(v, _Array)]
+        if not arrays or not all(isinstance(v, (_Array, _ScalarValue)) for v in (a, b)):
+            self.fail(node, f"elementwise '{op}' of these operands")
+        elem = arrays[0].elem
+        if elem not in _SIZES or any(v.elem != elem for v in arrays):
+            self.fail(node, f"elementwise '{op}' of non-float or mixed element types")
+        if len(arrays) == 1:
+            shape = arrays[0].shape
+            out = self.new_array(shape, elem, dest)
+            self.b.add_elementwise_op(op, a.name if isinstance(a, _Array) else a.text, b.name if isinstance(b, _Array) else b.text,
+                                      out.name, shape)
+            return out
+        shape = self.broadcast_shape(node, a.shape, b.shape)
+        a, b = self.expanded(a, shape), self.expanded(b, shape)
+        out = self.new_array(shape, elem, dest)
+        self.b.add_elementwise_op(op, a.name, b.name, out.name, shape)
+        return out
+
+    def unary(self, node: ast.AST, op: str, x: Any, dest: Optional[str]) -> _Array:
+        x = self.array_of(node, x)
+        if not isinstance(x, _Array) or x.elem not in _SIZES:
+            self.fail(node, f"'{op}' of a value that is not a float array")
+        out = self.new_array(x.shape, x.elem, dest)
+        self.b.add_elementwise_unary_op(op, x.name, out.name, x.shape)
+        return out
+
+    def is_product(self, n: ast.AST) -> bool:
+        """`A @ B` or `scalar * (A @ B)`, syntactically."""
+        if isinstance(n, ast.BinOp) and isinstance(n.op, ast.MatMult):
+            return True
+        if isinstance(n, ast.BinOp) and isinstance(n.op, ast.Mult):
+            return any(self.scalar_of(s) is not None and isinstance(o, ast.BinOp) and isinstance(o.op, ast.MatMult)
+                       for s, o in ((n.left, n.right), (n.right, n.left)))
+        return False
+
+    def gemm_accumulate(self, node: ast.BinOp, dest: Optional[str]) -> Optional[_Array]:
+        """`alpha * A @ B + beta * C` written into C: one GEMM in place. Only when the statement
+        names C as its destination; any other sum is an elementwise node."""
+        if dest is None:
+            return None
+        for prod, acc in ((node.left, node.right), (node.right, node.left)):
+            if not self.is_product(prod) or self.is_product(acc):
+                continue
+            beta, cnode = "1.0", acc
+            if isinstance(acc, ast.BinOp) and isinstance(acc.op, ast.Mult):
+                for sn, on in ((acc.left, acc.right), (acc.right, acc.left)):
+                    s = self.scalar_of(sn)
+                    if s is not None and isinstance(on, ast.Name):
+                        beta, cnode = s.text, on
+                        break
+            if not (isinstance(cnode, ast.Name) and isinstance(self.env.get(cnode.id), _Array) and self.env[cnode.id].name == dest):
+                continue
+            alpha, pnode = "1.0", prod
+            if isinstance(pnode.op, ast.Mult):
+                for sn, on in ((pnode.left, pnode.right), (pnode.right, pnode.left)):
+                    s = self.scalar_of(sn)
+                    if s is not None and isinstance(on, ast.BinOp) and isinstance(on.op, ast.MatMult):
+                        alpha, pnode = s.text, on
+                        break
+            return self.matmul(node, self.ev(pnode.left), self.ev(pnode.right), dest, alpha=alpha, beta=beta)
+        return None
+
     # ---- expressions -------------------------------------------------------------
     def ev(self, node: ast.AST, dest: Optional[str] = None) -> Any:
         if isinstance(node, ast.Name):
@@ -263,40 +359,24 @@ class _Lowering(ast.NodeVisitor):
                     return self.matmul(node, self.ev(other.left), self.ev(other.right), dest, alpha=s.text)
                 v = self.ev(other)
                 if isinstance(v, _Array):
-                    return _Lazy("scaled", v, s)
-            self.fail(node, "this multiplication")
+                    # a factor of a product to come (alpha * A @ B parses as (alpha * A) @ B); it
+                    # becomes an ml::Mul node when used as an array instead
+                    return _Lazy("scaled", v, s) if dest is None else self.elementwise(node, "mul", v, s, dest)
+                self.fail(node, "this multiplication")
+            return self.elementwise(node, "mul", self.ev(node.left), self.ev(node.right), dest)
         if isinstance(node.op, ast.Add):
-            # alpha * A @ B + beta * C  (either order), in place on C
-            for prod, acc in ((node.left, node.right), (node.right, node.left)):
-                c = self.ev(acc) if not (isinstance(acc, ast.BinOp) and isinstance(acc.op, ast.MatMult)) else None
-                beta = "1.0"
-                if isinstance(c, _Lazy) and c.kind == "scaled":
-                    beta, c = c.scalar.text, c.base
-                if not isinstance(c, _Array):
-                    continue
-                if dest is not None and dest != c.name:
-                    self.fail(node, "alpha*A@B + beta*C into a buffer other than C")
-                alpha, pnode = "1.0", prod
-                if isinstance(pnode, ast.BinOp) and isinstance(pnode.op, ast.Mult):
-                    for sn, on in ((pnode.left, pnode.right), (pnode.right, pnode.left)):
-                        s = self.scalar_of(sn)
-                        if s is not None and isinstance(on, ast.BinOp) and isinstance(on.op, ast.MatMult):
-                            alpha, pnode = s.text, on
-                            break
-                if not (isinstance(pnode, ast.BinOp) and isinstance(pnode.op, ast.MatMult)):
-                    continue
-                return self.matmul(node, self.ev(pnode.left), self.ev(pnode.right), c.name, alpha=alpha, beta=beta)
-            self.fail(node, "this addition")
+            r = self.gemm_accumulate(node, dest)
+            return r if r is not None else self.elementwise(node, "add", self.ev(node.left), self.ev(node.right), dest)
         if isinstance(node.op, ast.Sub):
             x, m = self.ev(node.left), self.ev(node.right)
             if isinstance(x, _Array) and isinstance(m, _Lazy) and m.kind == "max_keep" and m.base.name == x.name:
                 return _Lazy("sub_max", x)
-            self.fail(node, "this subtraction")
+            return self.elementwise(node, "sub", x, m, dest)
         if isinstance(node.op, ast.Div):
             e, s = self.ev(node.left), self.ev(node.right)
             if isinstance(e, _Lazy) and e.kind == "exp_sub" and isinstance(s, _Lazy) and s.kind == "sum_keep" and s.base.name == e.base.name:
                 return self.softmax(node, e.base, -1, dest)
-            self.fail(node, "this division")
+            return self.elementwise(node, "div", e, s, dest)
         self.fail(node, f"operator {type(node.op).__name__}")
 
     def call(self, node: ast.Call, dest: Optional[str]) -> Any:
@@ -313,7 +393,7 @@ class _Lowering(ast.NodeVisitor):
             import scipy.special as _sp
             scipy_softmax = _sp.softmax
         except Exception:  # scipy is optional
-            scipy_softmax = None
+            _sp = scipy_softmax = None
         if fn is not None and fn in (scipy_softmax, _functions.softmax):
             return self.softmax(node, self.ev(node.args[0]), self.kw(node, "axis", 1, -1 if fn is _functions.softmax else None) or -1, dest)
         if fn is _functions.conv2d:
@@ -327,6 +407,26 @@ class _Lowering(ast.NodeVisitor):
             v = self.ev(node.args[0])
             if isinstance(v, _Lazy) and v.kind == "sub_max":
                 return _Lazy("exp_sub", v.base)
+            return self.unary(node, "exp", v, dest)
+        unary_fns = {np.abs: "abs", np.absolute: "abs", np.fabs: "abs", np.sqrt: "sqrt", np.tanh: "tanh",
+                     _functions.relu: "relu", _functions.sigmoid: "sigmoid", _functions.erf: "erf"}
+        if _sp is not None:
+            unary_fns.update({_sp.erf: "erf", _sp.expit: "sigmoid"})
+        if fn is not None and len(node.args) == 1 and not node.keywords:
+            for f, op in unary_fns.items():
+                if fn is f:
+                    return self.unary(node, op, self.ev(node.args[0]), dest)
+        binary_fns = {np.maximum: "max", np.minimum: "min", np.add: "add", np.subtract: "sub", np.multiply: "mul",
+                      np.divide: "div", np.true_divide: "div"}
+        if fn is not None and len(node.args) == 2 and not node.keywords:
+            for f, op in binary_fns.items():
+                if fn is f:
+                    a, b = self.ev(node.args[0]), self.ev(node.args[1])
+                    if op == "max":  # np.maximum(x, 0): the ReLU node
+                        for x, z in ((a, b), (b, a)):
+                            if isinstance(z, _ScalarValue) and z.text in ("0.0", "-0.0") and isinstance(x, (_Array, _Lazy)):
+                                return self.unary(node, "relu", x, dest)
+                    return self.elementwise(node, op, a, b, dest)
         if fn is np.sum:
             v = self.ev(node.args[0])
             if isinstance(v, _Lazy) and v.kind == "exp_sub" and axis_last(v.base):

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
     "docc_rocm_elementwise_unary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp],
     "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
+    "docc_rocm_elementwise_binary_scalar": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, ctypes.c_double, ctypes.c_int, _vp],
     "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
@@ -226,6 +227,12 @@ def elementwise_unary(op, precision, n, X, Y, stream=0) -> None:
 
 def elementwise_binary(op, precision, n, A, B, Y, stream=0) -> None:
     call("docc_rocm_elementwise_binary", stream, BINARY_OPS[op] if isinstance(op, str) else op, precision, n, A, B, Y)
+
+
+def elementwise_binary_scalar(op, precision, n, A, scalar, Y, scalar_is_lhs=False, stream=0) -> None:
+    """Y = f(A, scalar), or f(scalar, A) when scalar_is_lhs."""
+    call("docc_rocm_elementwise_binary_scalar", stream, BINARY_OPS[op] if isinstance(op, str) else op, precision, n, A,
+         float(scalar), int(bool(scalar_is_lhs)), Y)
 
 
 def broadcast(precision, in_shape, out_shape, X, Y, stream=0) -> None:

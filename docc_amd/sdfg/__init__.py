@@ -319,6 +319,45 @@ class StructuredSDFGBuilder:
                          "group": _expr(group), "has_bias": B is not None, "element_type": self._element(X).value},
                         inputs, [self._operand("Y", Y)])
 
+    #: elementwise tensor node codes (reference .../tensor/elementwise_ops/*.h)
+    UNARY_CODES = {"abs": "ml::Abs", "exp": "ml::Exp", "relu": "ml::ReLU", "sigmoid": "ml::Sigmoid", "sqrt": "ml::Sqrt",
+                   "tanh": "ml::Tanh", "erf": "ml::Erf"}
+    BINARY_CODES = {"add": "ml::Add", "sub": "ml::Sub", "mul": "ml::Mul", "div": "ml::Div", "max": "ml::Maximum",
+                    "min": "ml::Minimum", "maximum": "ml::Maximum", "minimum": "ml::Minimum"}
+
+    def add_elementwise_op(self, op: str, A: str, B: str, C: str, shape: Sequence[Any]) -> None:
+        """Binary elementwise node "A","B" -> "C" over equally shaped operands (reference add_elementwise_op,
+        python/bindings/builder/py_structured_sdfg_builder.cpp:839-908: op names add, sub, mul, div, min, max).
+        As there, an operand that names no container is bound as a constant of the result's element type;
+        a scalar container is passed by value."""
+        if op not in self.BINARY_CODES:
+            raise NotImplementedError(f"elementwise op '{op}' is not part of the rocm target")
+        elem = self._element(C)
+
+        def bind(connector: str, v: Any) -> Dict[str, Any]:
+            return self._operand(connector, v) if v in self._data["containers"] else self._operand(connector, v, elem)
+
+        self._add_block({"code": self.BINARY_CODES[op], "implementation_type": "NONE", "side_effect": False,
+                         "shape": [_expr(s) for s in shape], "element_type": elem.value},
+                        [bind("A", A), bind("B", B)], [self._operand("C", C)])
+
+    def add_elementwise_unary_op(self, op: str, X: str, Y: str, shape: Sequence[Any]) -> None:
+        """Unary elementwise node "X" -> "Y" (reference add_elementwise_unary_op, same file :910-952)."""
+        if op not in self.UNARY_CODES:
+            raise NotImplementedError(f"elementwise op '{op}' is not part of the rocm target")
+        self._add_block({"code": self.UNARY_CODES[op], "implementation_type": "NONE", "side_effect": False,
+                         "shape": [_expr(s) for s in shape], "element_type": self._element(X).value},
+                        [self._operand("X", X)], [self._operand("Y", Y)])
+
+    def add_broadcast(self, X: str, Y: str, input_shape: Sequence[Any], output_shape: Sequence[Any]) -> None:
+        """ml::Broadcast (reference .../tensor/broadcast_node.h): equal ranks, extent-1 dimensions repeat."""
+        if len(input_shape) != len(output_shape):
+            raise InvalidSDFGException("ml::Broadcast: input and output ranks differ")
+        self._add_block({"code": "ml::Broadcast", "implementation_type": "NONE", "side_effect": False,
+                         "input_shape": [_expr(s) for s in input_shape], "output_shape": [_expr(s) for s in output_shape],
+                         "element_type": self._element(X).value},
+                        [self._operand("X", X)], [self._operand("Y", Y)])
+
     def add_attention(self, Q: str, K: str, V: str, O: str, shape_q: Sequence[Any], seq_kv: Any, scale: Any) -> None:
         """ml::Attention: O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]."""
         self._add_block({"code": "ml::Attention", "implementation_type": "NONE", "side_effect": False,

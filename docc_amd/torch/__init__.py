@@ -14,6 +14,11 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
                                            -> ml::Attention (bf16, head dim 64)
+    + - * / torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
+                                           -> ml::Add .. ml::Minimum, with ml::Broadcast where shapes differ
+    relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh)
+                                           -> ml::ReLU .. ml::Erf
+    F.linear / nn.Linear                   -> GEMM with the weight transposed, bias through Broadcast + Add
 
 Tensors on a `cuda` device are passed to the generated function as device pointers (no
 transfers, the kernels run on the null stream in order with torch's default stream); CPU tensors
@@ -213,10 +218,63 @@ class _FxLowering:
                               bias.name if isinstance(bias, _T) else None)
         return out
 
-    def scale(self, node, x, factor: float):
+    def scale(self, node, x, factor: float, dest=None):
         if isinstance(x, _Scores):
             return _Scores(x.q, x.k, x.scale * factor)
-        self.fail(node, "scaling a tensor that is not an attention score matrix")
+        return self.elementwise(node, "mul", x, float(factor), dest)
+
+    def expanded(self, node, x: _T, shape: List[int]) -> _T:
+        """`x` repeated to `shape` through ml::Broadcast (a no-op when the shapes agree)."""
+        if x.shape == shape:
+            return x
+        if len(shape) > 6:
+            self.fail(node, "a broadcast of rank above 6")
+        out = self.new_tensor(shape, x.dtype, None)
+        self.builder.add_broadcast(x.name, out.name, [1] * (len(shape) - len(x.shape)) + x.shape, shape)
+        return out
+
+    def elementwise(self, node, op: str, a, b, dest):
+        torch = self.torch
+        tensors = [v for v in (a, b) if isinstance(v, _T)]
+        if not tensors or not all(isinstance(v, (_T, int, float)) and not isinstance(v, bool) for v in (a, b)):
+            self.fail(node, f"elementwise {op} of these operands")
+        dtype = tensors[0].dtype
+        if dtype not in (torch.float32, torch.float64) or any(v.dtype != dtype for v in tensors):
+            self.fail(node, f"elementwise {op} on dtypes other than one of float32 / float64")
+        if len(tensors) == 2:
+            try:
+                shape = list(torch.broadcast_shapes(tuple(a.shape), tuple(b.shape)))
+            except RuntimeError:
+                self.fail(node, f"shapes {a.shape} and {b.shape}, which do not broadcast,")
+            a, b = self.expanded(node, a, shape), self.expanded(node, b, shape)
+        else:
+            shape = tensors[0].shape
+        out = self.new_tensor(shape, dtype, dest)
+        name = lambda v: v.name if isinstance(v, _T) else repr(float(v))
+        self.builder.add_elementwise_op(op, name(a), name(b), out.name, shape)
+        return out
+
+    def unary(self, node, op: str, x, dest):
+        if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
+            self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
+        out = self.new_tensor(x.shape, x.dtype, dest)
+        self.builder.add_elementwise_unary_op(op, x.name, out.name, x.shape)
+        return out
+
+    def linear(self, node, x, w, bias, dest):
+        """x [..., K] times w[N, K] transposed, plus bias [N]: one GEMM over the flattened rows."""
+        if not isinstance(x, _T) or not isinstance(w, _T) or len(w.shape) != 2 or len(x.shape) < 1 or x.shape[-1] != w.shape[1]:
+            self.fail(node, "linear on these operands")
+        if x.dtype != w.dtype or x.dtype not in (self.torch.float32, self.torch.float64):
+            self.fail(node, "linear on dtypes other than float32 / float64")
+        n, k = w.shape
+        m = int(math.prod(x.shape[:-1]))
+        shape = x.shape[:-1] + [n]
+        out = self.new_tensor(shape, x.dtype, dest if bias is None else None)
+        self.builder.add_gemm(x.name, w.name, out.name, "1.0", "0.0", m, n, k, False, True, k, k, n)
+        if bias is None:
+            return out
+        return self.elementwise(node, "add", out, bias, dest)
 
     def transpose(self, node, x, d0: int, d1: int):
         if not isinstance(x, _T):
@@ -262,6 +320,17 @@ class _FxLowering:
                 self.env[node] = self.add_input(node.name, list(t.shape), t.dtype, ("attr", node.target))
             elif node.op == "call_module":
                 mod = self.gm.get_submodule(node.target)
+                activations = {torch.nn.ReLU: "relu", torch.nn.Sigmoid: "sigmoid", torch.nn.Tanh: "tanh"}
+                if type(mod) in activations:
+                    self.env[node] = self.unary(node, activations[type(mod)], self.arg(node.args[0]), dest)
+                    continue
+                if isinstance(mod, torch.nn.Linear):
+                    w = self.add_input(f"{node.name}_weight", list(mod.weight.shape), mod.weight.dtype, ("attr", f"{node.target}.weight"))
+                    b = None
+                    if mod.bias is not None:
+                        b = self.add_input(f"{node.name}_bias", list(mod.bias.shape), mod.bias.dtype, ("attr", f"{node.target}.bias"))
+                    self.env[node] = self.linear(node, self.arg(node.args[0]), w, b, dest)
+                    continue
                 if not isinstance(mod, torch.nn.Conv2d):
                     self.fail(node, f"module {type(mod).__name__}")
                 if mod.padding_mode != "zeros":
@@ -326,13 +395,38 @@ class _FxLowering:
             return self.transpose(node, args[0], -2, -1)
         if method in ("t",) or t is torch.t:
             return self.transpose(node, args[0], 0, 1)
-        if t in (operator.truediv, torch.div) or method == "div":
-            if isinstance(args[1], (int, float)):
+        if t in (operator.truediv, torch.div, torch.true_divide) or method in ("div", "true_divide"):
+            if kwargs.get("rounding_mode") is not None:
+                self.fail(node, "division with a rounding mode")
+            if isinstance(args[1], (int, float)) and isinstance(args[0], _Scores):
                 return self.scale(node, args[0], 1.0 / float(args[1]))
-        if t in (operator.mul, torch.mul) or method == "mul":
+            return self.elementwise(node, "div", args[0], args[1], dest)
+        if t in (operator.mul, torch.mul, torch.multiply) or method in ("mul", "multiply"):
             for x, c in ((args[0], args[1]), (args[1], args[0])):
-                if isinstance(c, (int, float)):
+                if isinstance(c, (int, float)) and isinstance(x, _Scores):
                     return self.scale(node, x, float(c))
+            return self.elementwise(node, "mul", args[0], args[1], dest)
+        if t in (operator.add, torch.add) or method == "add":
+            if kwargs.get("alpha", 1) != 1:
+                self.fail(node, "add with alpha")
+            return self.elementwise(node, "add", args[0], args[1], dest)
+        if t in (operator.sub, torch.sub, torch.subtract) or method in ("sub", "subtract"):
+            if kwargs.get("alpha", 1) != 1:
+                self.fail(node, "sub with alpha")
+            return self.elementwise(node, "sub", args[0], args[1], dest)
+        if t in (torch.maximum, torch.minimum) or method in ("maximum", "minimum"):
+            return self.elementwise(node, "max" if (t is torch.maximum or method == "maximum") else "min", args[0], args[1], dest)
+        unary_fns = {"relu": (torch.relu, F.relu), "sigmoid": (torch.sigmoid, F.sigmoid), "tanh": (torch.tanh, F.tanh),
+                     "exp": (torch.exp,), "abs": (torch.abs, torch.absolute), "sqrt": (torch.sqrt,),
+                     "erf": (torch.erf, torch.special.erf)}
+        for op, fns in unary_fns.items():
+            if any(t is f for f in fns) or method == op:
+                if kwargs.get("inplace"):
+                    self.fail(node, "an in-place activation")
+                return self.unary(node, op, args[0], dest)
+        if t is F.linear:
+            bias = args[2] if len(args) > 2 else kwargs.get("bias")
+            return self.linear(node, args[0], args[1], bias, dest)
         if t in (torch.softmax, F.softmax) or method == "softmax":
             dim = kwargs.get("dim", args[1] if len(args) > 1 else None)
             if dim is None:

@@ -125,6 +125,12 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
 int docc_rocm_elementwise_unary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y);
 int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A, const void* B,
                                  void* Y);
+/* One operand is a scalar: the reference binds a constant or a scalar container to "A" or
+ * "B" of the binary node (python/bindings/builder/py_structured_sdfg_builder.cpp:894-908).
+ * Y[i] = f(A[i], scalar), or f(scalar, A[i]) when scalar_is_lhs != 0; the scalar is
+ * rounded to float for precision 32. */
+int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A, double scalar,
+                                        int scalar_is_lhs, void* Y);
 
 /* ml::Broadcast (reference .../tensor/broadcast_node.h:13-43): Y of shape out_shape is X
  * of shape in_shape repeated along every dimension where in_shape is 1 (numpy rules,

@@ -10,7 +10,8 @@ import scipy.special
 import torch
 
 import docc_amd.torch as docc_torch
-from docc_amd.python import (conv2d, native, register_target, register_target_overrides, softmax, unregister_target)
+from docc_amd.python import (conv2d, erf, native, register_target, register_target_overrides, relu, sigmoid, softmax,
+                             unregister_target)
 
 
 @pytest.fixture(autouse=True)
@@ -55,6 +56,10 @@ def test_other_matmul_spellings_and_polybench_gemm():
 
     a = np.zeros((6, 6))
     assert np_matmul.to_sdfg(a, a).library_nodes()[0]["code"] == "GEMM"
+    batched = np_matmul.to_sdfg(np.zeros((4, 5, 6), np.float32), np.zeros((4, 6, 3), np.float32))
+    (node,) = batched.library_nodes()
+    assert node["code"] == "ml::MatMul" and node["shape_a"] == ["_s0", "_s1", "_s2"] and node["shape_b"] == ["_s0", "_s2", "_s3"]
+    assert batched._data["root"]["children"][0]["dataflow"]["outputs"] == [{"connector": "Y", "data": "_docc_ret_0"}]
     assert dot_t.to_sdfg(a, a).library_nodes()[0]["trans_b"] == 112
     sdfg = gemm.to_sdfg(1.5, 1.2, a, a, a)
     assert sdfg.arguments == ["alpha", "beta", "C", "A", "B", "_s0"]     # in place: no return buffer
@@ -102,6 +107,10 @@ def test_unsupported_code_is_rejected_not_run_on_the_cpu():
             b[i] = a[i]
 
     @native
+    def power(a, b):
+        return a ** b
+
+    @native
     def add(a, b):
         return a + b
 
@@ -109,7 +118,60 @@ def test_unsupported_code_is_rejected_not_run_on_the_cpu():
     with pytest.raises(NotImplementedError, match="rocm target"):
         loop.to_sdfg(a, a)
     with pytest.raises(NotImplementedError):
-        add.to_sdfg(a, a)
+        power.to_sdfg(a, a)
+    with pytest.raises(NotImplementedError):          # integer arrays have no elementwise kernels
+        add.to_sdfg(np.zeros(4, np.int64), np.zeros(4, np.int64))
+    with pytest.raises(ValueError, match="broadcast"):
+        add.to_sdfg(np.zeros((4, 3)), np.zeros((4, 2)))
+
+
+def test_elementwise_expressions_lower_to_tensor_nodes():
+    @native
+    def dense(x, w, b):
+        return relu(x @ w + b)
+
+    @native
+    def mixed(x, y, s):
+        return np.tanh(x * y - 0.5) / (s * y)
+
+    @native
+    def clip(x, y):
+        return np.minimum(np.maximum(x, 0), np.abs(y))
+
+    @native
+    def in_place(x, y):
+        y[:] = np.exp(x) + y
+
+    x, w, b = np.zeros((8, 5), np.float32), np.zeros((5, 3), np.float32), np.zeros(3, np.float32)
+    sdfg = dense.to_sdfg(x, w, b)
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes == ["GEMM", "ml::Broadcast", "ml::Add", "ml::ReLU"]
+    bc = sdfg.library_nodes()[1]
+    assert bc["input_shape"] == ["1", "_s2"] and bc["output_shape"] == ["_s0", "_s2"]
+    blocks = [c["dataflow"] for c in sdfg._data["root"]["children"]]
+    assert {i["connector"] for i in blocks[2]["inputs"]} == {"A", "B"} and blocks[2]["outputs"][0]["connector"] == "C"
+    assert blocks[3]["inputs"][0]["connector"] == "X" and blocks[3]["outputs"][0] == {"connector": "Y", "data": "_docc_ret_0"}
+    # intermediates are transients of the generated function, only the result is an argument
+    assert sdfg.arguments == ["x", "w", "b", "_s0", "_s1", "_s2", "_docc_ret_0"]
+
+    z = np.zeros((4, 6))
+    sdfg = mixed.to_sdfg(z, z, 2.0)
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Mul", "ml::Sub", "ml::Tanh", "ml::Mul", "ml::Div"]
+    blocks = [c["dataflow"] for c in sdfg._data["root"]["children"]]
+    sub_b = next(i for i in blocks[1]["inputs"] if i["connector"] == "B")
+    assert sub_b == {"connector": "B", "constant": "0.5", "type": "Double"}
+    mul_s = {i["connector"]: i for i in blocks[3]["inputs"]}
+    assert mul_s["B"] == {"connector": "B", "data": "s"} and mul_s["A"]["data"] == "y"   # scalar argument by value
+    assert all(n["element_type"] == "Double" for n in sdfg.library_nodes())
+
+    assert [n["code"] for n in clip.to_sdfg(z, z).library_nodes()] == ["ml::ReLU", "ml::Abs", "ml::Minimum"]
+    sdfg = in_place.to_sdfg(z, z)
+    assert sdfg.arguments == ["x", "y", "_s0", "_s1"]
+    assert sdfg._data["root"]["children"][1]["dataflow"]["outputs"][0]["data"] == "y"
+    # the marker functions are plain numpy outside @native
+    v = np.linspace(-3, 3, 7)
+    assert np.allclose(relu(v), np.maximum(v, 0)) and np.allclose(sigmoid(v), scipy.special.expit(v))
+    assert np.allclose(erf(v), scipy.special.erf(v))
 
 
 def test_compile_cache_follows_shape_structure():
@@ -214,10 +276,50 @@ def test_torch_lowering_recognises_attention_conv_and_matmul():
 
     class Unsupported(torch.nn.Module):
         def forward(self, a):
-            return torch.relu(a)
+            return torch.cumsum(a, 0)
 
     with pytest.raises(NotImplementedError):
         docc_torch.TorchProgram(Unsupported(), torch.randn(4), target="rocm").to_sdfg()
+
+
+def test_torch_lowering_of_elementwise_operations_and_linear():
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = torch.nn.Linear(12, 20)
+            self.act = torch.nn.ReLU()
+            self.fc2 = torch.nn.Linear(20, 6, bias=False)
+
+        def forward(self, x):
+            return torch.tanh(self.fc2(self.act(self.fc1(x)))) * 0.5
+
+    x = torch.randn(4, 7, 12)
+    sdfg = docc_torch.TorchProgram(Mlp(), (x,), target="rocm").to_sdfg()
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes == ["GEMM", "ml::Broadcast", "ml::Add", "ml::ReLU", "GEMM", "ml::Tanh", "ml::Mul"]
+    g = sdfg.library_nodes()[0]
+    assert (g["m"], g["n"], g["k"], g["trans_b"], g["ldb"]) == ("28", "20", "12", 112, "12")    # rows flattened, weight [N, K] transposed
+    assert sdfg.library_nodes()[1]["input_shape"] == ["1", "1", "20"] and sdfg.metadata("return_shape") == "[4,7,6]"
+    last = sdfg._data["root"]["children"][-1]["dataflow"]
+    assert {"connector": "B", "constant": "0.5", "type": "Float"} in last["inputs"] and last["outputs"][0]["data"] == "_docc_ret_0"
+
+    class Arith(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.maximum(a - b, b / 3) + torch.sigmoid(a).exp() * torch.sqrt(b.abs())
+
+    sdfg = docc_torch.TorchProgram(Arith(), (torch.randn(5, 3, dtype=torch.float64), torch.randn(3, dtype=torch.float64)),
+                                   target="rocm").to_sdfg()
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes == ["ml::Broadcast", "ml::Sub", "ml::Div", "ml::Broadcast", "ml::Maximum", "ml::Sigmoid", "ml::Exp", "ml::Abs",
+                     "ml::Sqrt", "ml::Broadcast", "ml::Mul", "ml::Add"]
+    assert all(n["element_type"] == "Double" for n in sdfg.library_nodes())
+
+    class Ints(torch.nn.Module):
+        def forward(self, a):
+            return a + a
+
+    with pytest.raises(NotImplementedError):
+        docc_torch.TorchProgram(Ints(), torch.ones(4, dtype=torch.int32), target="rocm").to_sdfg()
 
 
 def test_torch_backend_is_registered_and_reads_global_options():

@@ -1,5 +1,5 @@
 """Elementwise tensor nodes and ml::Broadcast on the GPU against the CPU oracle, through
-docc_rocm_elementwise_unary / _binary / docc_rocm_broadcast.
+docc_rocm_elementwise_unary / _binary / _binary_scalar / docc_rocm_broadcast.
 
 Bars: bit-exact for the IEEE operations and the selections (add, sub, mul, div, maximum, minimum,
 abs, relu, sqrt, broadcast); exp / tanh / sigmoid / erf within 4 units in the last place of the
@@ -82,6 +82,27 @@ def test_unary(rt, dt, n):
         assert ulps(got[~nan], ref[~nan]) <= 4, op
     # in place
     assert np.array_equal(run_unary(rt, "relu", x, in_place=True), oracle.elementwise_unary("relu", x), equal_nan=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [1, 5, 1000, 4099])
+def test_binary_with_a_scalar_operand_bit_exact(rt, dt, n):
+    rng = np.random.default_rng(n + 3)
+    a = (rng.standard_normal(n) * 10).astype(dt)
+    if n > 100:
+        a[7], a[8], a[9] = np.nan, np.inf, 0.0
+    for scalar in (2.5, -0.1, 0.0):      # -0.1 is rounded to the element type first, as the array operand would be
+        full = np.full(n, scalar, dt)
+        for op in BINARY:
+            for offset in (0, 1):
+                for lhs in (False, True):
+                    da = dev(np.concatenate([np.zeros(offset, dt), a]))
+                    out = torch.full_like(da, float("nan"))
+                    es = da.element_size()
+                    rt.elementwise_binary_scalar(op, prec(dt), n, da.data_ptr() + offset * es, scalar, out.data_ptr() + offset * es, lhs)
+                    torch.cuda.synchronize()
+                    ref = oracle.elementwise_binary(op, full, a) if lhs else oracle.elementwise_binary(op, a, full)
+                    assert np.array_equal(host(out)[offset:], ref, equal_nan=True), (op, scalar, offset, lhs)
 
 
 def test_large_shape_and_closed_forms(rt):

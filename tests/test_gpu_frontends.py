@@ -14,7 +14,7 @@ import torch
 
 import docc_amd.torch as docc_torch
 import oracle
-from docc_amd.python import conv2d, native
+from docc_amd.python import conv2d, native, relu, sigmoid
 from gpu_util import rel_err_max
 
 pytestmark = pytest.mark.gpu
@@ -168,3 +168,64 @@ def test_torch_backend_matmul_softmax_fp32():
     out = docc_torch.compile_torch(BMM(), (a3, b3), target="rocm")(a3, b3)   # batched: ml::MatMul
     refs = np.stack([oracle.gemm(a3[i].numpy(), b3[i].numpy(), variant="ld") for i in range(4)])
     assert rel_err_max(out.numpy(), refs) <= 1e-12
+
+
+def test_native_dense_layer_stays_on_the_device():
+    """relu(x @ w + b): GEMM, Broadcast, Add and ReLU nodes; only the arguments cross PCIe."""
+    @native(target="rocm")
+    def dense(x, w, b):
+        return relu(x @ w + b)
+
+    rng = np.random.default_rng(11)
+    x, w, b = rng.standard_normal((200, 96)).astype(np.float32), rng.standard_normal((96, 130)).astype(np.float32), \
+        rng.standard_normal(130).astype(np.float32)
+    y = dense(x, w, b)
+    t = oracle.gemm(x, w)
+    ref = oracle.elementwise_unary("relu", oracle.elementwise_binary("add", t, oracle.broadcast(b, t.shape)))
+    assert y.shape == (200, 130) and rel_err_max(y, ref) <= 1e-5 and (y >= 0).all()
+    r = dense.last_sdfg.loop_report()
+    assert r["H2D"] == 3 and r["D2H"] == 1
+    assert [r[k] for k in ("GEMM", "ml::Broadcast", "ml::Add", "ml::ReLU")] == [1, 1, 1, 1]
+
+
+def test_native_elementwise_expression_fp64():
+    @native(target="rocm")
+    def expr(x, y, s):
+        return np.tanh(x * y - 0.5) / (s * np.abs(y) + 1.0) + np.minimum(sigmoid(x), 2.0 - np.sqrt(np.abs(y)))
+
+    rng = np.random.default_rng(5)
+    x, y = rng.standard_normal((37, 53)), rng.standard_normal((37, 53))
+    got = expr(x, y, 0.75)
+    ref = np.tanh(x * y - 0.5) / (0.75 * np.abs(y) + 1.0) + np.minimum(1.0 / (1.0 + np.exp(-x)), 2.0 - np.sqrt(np.abs(y)))
+    assert got.dtype == np.float64 and rel_err_max(got, ref) <= 1e-12
+    # in place into an argument, scalar on the left of a subtraction
+    @native(target="rocm")
+    def update(x, y):
+        y[:] = 1.0 - np.exp(x) * y
+
+    y2 = y.copy()
+    update(x, y2)
+    assert rel_err_max(y2, 1.0 - np.exp(x) * y) <= 1e-12
+
+
+def test_torch_compile_mlp_fp32():
+    class Mlp(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc1 = torch.nn.Linear(64, 128)
+            self.fc2 = torch.nn.Linear(128, 32)
+
+        def forward(self, x):
+            return torch.sigmoid(self.fc2(torch.relu(self.fc1(x)))) - 0.5
+
+    torch.manual_seed(0)
+    model = Mlp().cuda()
+    x = torch.randn(16, 10, 64, device="cuda")
+    program = docc_torch.compile_torch(model, x, target="rocm")
+    y = program(x)
+    assert y.is_cuda and y.shape == (16, 10, 32)
+    with torch.no_grad():
+        ref = model.double()(x.double())
+    assert rel_err_max(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+    r = program.last_sdfg.loop_report()
+    assert r["GEMM"] == 2 and r["H2D"] == 0 and r["D2H"] == 0      # device tensors: no transfers at all

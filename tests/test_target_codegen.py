@@ -35,7 +35,9 @@ def source_of(sdfg, tmp_path):
 
 def test_registry_holds_every_rocm_key():
     keys = registered_dispatchers()
-    for code in ("GEMM", "ml::MatMul", "ml::Softmax", "ml::Conv", "ml::Attention"):
+    for code in ("GEMM", "ml::MatMul", "ml::Softmax", "ml::Conv", "ml::Attention", "ml::Broadcast", "ml::Abs", "ml::Exp",
+                 "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf", "ml::Add", "ml::Sub", "ml::Mul", "ml::Div",
+                 "ml::Maximum", "ml::Minimum"):
         assert f"{code}::ROCMWithTransfers" in keys and f"{code}::ROCMWithoutTransfers" in keys
     assert "ROCMOffloading::NONE" in keys
 
@@ -248,3 +250,73 @@ def test_device_pointer_mode_allocates_transients_on_the_device(tmp_path):
     flat = re.sub(r"\s+", " ", src)
     assert flat.index("docc_rocm_malloc(") < flat.index("docc_rocm_sgemm(") < flat.index("docc_rocm_softmax_f32(") < flat.index("docc_rocm_free(")
     assert src.count("docc_rocm_malloc(") == 1 and src.count("docc_rocm_free(") == 1
+
+
+def dense_sdfg():
+    """Y = relu(X @ W + bias) * 0.5: GEMM, Broadcast of the bias row, Add, ReLU, Mul by a constant."""
+    b = StructuredSDFGBuilder("dense")
+    for n in ("X", "W", "bias", "Y"):
+        b.add_container(n, F32, True)
+    for n in ("T0", "T1", "T2", "T3"):
+        b.add_container(n, F32, False, transient_bytes=32 * 16 * 4)
+    b.add_gemm("X", "W", "T0", "1.0", "0.0", 32, 16, 8)
+    b.add_broadcast("bias", "T1", [1, 16], [32, 16])
+    b.add_elementwise_op("add", "T0", "T1", "T2", [32, 16])
+    b.add_elementwise_unary_op("relu", "T2", "T3", [32, 16])
+    b.add_elementwise_op("mul", "T3", "0.5", "Y", [32, 16])
+    return b.move()
+
+
+def test_elementwise_nodes_round_trip_and_dispatch(tmp_path):
+    s = dense_sdfg()
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["GEMM", "ml::Broadcast", "ml::Add", "ml::ReLU", "ml::Mul"]
+    # payload keys of the reference's serializers: shape (elementwise_node.cpp), input_shape / output_shape (broadcast_node.cpp)
+    assert nodes[2]["shape"] == ["32", "16"] and nodes[1]["input_shape"] == ["1", "16"] and nodes[1]["output_shape"] == ["32", "16"]
+    assert StructuredSDFG.parse(s.to_json()).library_nodes() == nodes
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 3 and r["D2H"] == 1          # X, W, bias up; Y down; T0..T3 stay in device memory
+    for t in ("T0", "T1", "T2", "T3"):
+        assert "size" not in s.containers[t]
+    src, _ = source_of(s, tmp_path)
+    flat = re.sub(r"\s+", " ", src)
+    assert "docc_rocm_broadcast(nullptr, 32, 2, __docc_in_shape, __docc_out_shape, X, Y)" in flat
+    assert "const int64_t __docc_in_shape[] = {(int64_t) (1), (int64_t) (16)};" in flat
+    assert "docc_rocm_elementwise_binary(nullptr, 0 /* ml::Add */, 32, 512, A, B, C)" in flat
+    assert "docc_rocm_elementwise_unary(nullptr, 2 /* ml::ReLU */, 32, 512, X, Y)" in flat
+    # the constant operand is passed by value, the array one as the only pointer
+    assert "float B = 0.5;" in flat
+    assert "docc_rocm_elementwise_binary_scalar(nullptr, 2 /* ml::Mul */, 32, 512, A, (double) B, 0, C)" in flat
+    order = [flat.index(k) for k in ("docc_rocm_sgemm(", "docc_rocm_broadcast(", "docc_rocm_elementwise_binary(",
+                                     "docc_rocm_elementwise_unary(", "docc_rocm_elementwise_binary_scalar(")]
+    assert order == sorted(order)
+
+
+def test_elementwise_with_transfers_and_scalar_on_the_left(tmp_path):
+    b = StructuredSDFGBuilder("rsub")
+    b.add_container("x", F64, True)
+    b.add_container("s", Scalar(PrimitiveType.Double), True)
+    b.add_container("y", F64, True)
+    b.add_elementwise_op("sub", "s", "x", "y", ["_n"])
+    b.add_container("_n", I64, True)
+    s = b.move()
+    s.schedule("rocm", options={"offload": "node"})
+    src, report = source_of(s, tmp_path)
+    flat = re.sub(r"\s+", " ", src)
+    assert "docc_rocm_elementwise_binary_scalar(nullptr, 1 /* ml::Sub */, 64, _n, d_B, (double) A, 1, d_C)" in flat
+    assert flat.count("docc_rocm_malloc(") == 2 and flat.count("docc_rocm_memcpy_h2d_async(") == 1   # the scalar is not an operand buffer
+    assert flat.count("docc_rocm_memcpy_d2h_async(") == 1
+    # what the kernels lack is declined, not run elsewhere
+    b = StructuredSDFGBuilder("ints")
+    for n in ("a", "c"):
+        b.add_container(n, Pointer(Scalar(PrimitiveType.Int32)), True)
+    b.add_elementwise_unary_op("abs", "a", "c", [8])
+    with pytest.raises(InvalidSDFGException, match="Float or Double"):
+        b.move().schedule("rocm")
+    b = StructuredSDFGBuilder("bc")
+    for n in ("a", "c"):
+        b.add_container(n, F32, True)
+    with pytest.raises(InvalidSDFGException, match="cannot be broadcast"):
+        b.add_broadcast("a", "c", [3, 4], [5, 4])
+        b.move().validate()
