@@ -119,6 +119,22 @@ def build_runtime(force: bool = True) -> Path:
     return out
 
 
+def build_rtl(force: bool = True) -> Path:
+    """libdocc_rtl_rocm.so: the `__daisy_instrumentation_*` runtime with the ROCm event set
+    (needs libdocc_rt_rocm.so, built first)."""
+    srcs = sorted((CSRC / "rtl").glob("*.cpp"))
+    deps = srcs + sorted(INCLUDE.glob("*.h"))
+    out = LIB / "libdocc_rtl_rocm.so"
+    if not force and _newer(out, deps):
+        return out
+    LIB.mkdir(parents=True, exist_ok=True)
+    _run([
+        "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", str(INCLUDE), *map(str, srcs), "-o", str(out),
+        "-L", str(LIB), "-ldocc_rt_rocm", "-ldl", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{ROCM / 'lib'}",
+    ])
+    return out
+
+
 def build_target(force: bool = True) -> Path | None:
     srcs = sorted((CSRC / "target").glob("*.cpp"))
     if not srcs:
@@ -137,6 +153,7 @@ def build_target(force: bool = True) -> Path | None:
 
 def build_all(force: bool = True) -> dict[str, list[str]]:
     built = {"kernels": [str(p) for p in build_kernels(force)], "runtime": [str(build_runtime(force))]}
+    built["rtl"] = [str(build_rtl(force))]
     target = build_target(force)
     if target:
         built["target"] = [str(target)]

@@ -89,12 +89,107 @@ void LibraryNodeDispatcher::dispatch(PrettyPrinter& stream, PrettyPrinter& globa
 }
 
 InstrumentationInfo LibraryNodeDispatcher::instrumentation_info() const {
+    // reference block_dispatcher.cpp:440-442: element id, "unknown", SEQUENTIAL
     InstrumentationInfo info;
+    info.element_id = node_.element_id();
     info.region_name = node_.code();
-    info.target_type = "CPU";
     const Expression flop = node_.flop();
     if (!flop.empty()) info.metrics["flop"] = flop;
     return info;
+}
+
+// ------------------------------------------------------------------ instrumentation plan
+
+namespace {
+std::string c_string(const std::string& s) {
+    std::string out = "\"";
+    for (char c : s) {
+        if (c == '"' || c == '\\') out += '\\';
+        if (c == '\n') {
+            out += "\\n";
+            continue;
+        }
+        out += c;
+    }
+    return out + "\"";
+}
+
+std::string metadata_or_empty(const StructuredSDFG& sdfg, const char* key) {
+    auto it = sdfg.metadata().find(key);
+    return it == sdfg.metadata().end() ? "" : it->second;
+}
+} // namespace
+
+void InstrumentationPlan::begin_instrumentation(const structured_control_flow::Block& block, PrettyPrinter& stream,
+                                                const InstrumentationInfo& info) const {
+    const std::string stem = sdfg_.name() + "_" + std::to_string(block.node->element_id());
+    const std::string md = stem + "_md", id = stem + "_id";
+    const auto& dbg = block.debug_info;
+    stream << "__daisy_metadata_t " << md << ";" << std::endl;
+    stream << md << ".file_name = " << c_string(dbg.filename) << ";" << std::endl;
+    stream << md << ".function_name = " << c_string(dbg.function) << ";" << std::endl;
+    stream << md << ".line_begin = " << dbg.start_line << ";" << std::endl;
+    stream << md << ".line_end = " << dbg.end_line << ";" << std::endl;
+    stream << md << ".column_begin = " << dbg.start_column << ";" << std::endl;
+    stream << md << ".column_end = " << dbg.end_column << ";" << std::endl;
+    stream << md << ".sdfg_name = " << c_string(sdfg_.name()) << ";" << std::endl;
+    stream << md << ".sdfg_file = " << c_string(metadata_or_empty(sdfg_, "sdfg_file")) << ";" << std::endl;
+    stream << md << ".arg_capture_path = " << c_string(metadata_or_empty(sdfg_, "arg_capture_path")) << ";" << std::endl;
+    stream << md << ".features_file = " << c_string(metadata_or_empty(sdfg_, "features_file")) << ";" << std::endl;
+    stream << md << ".opt_report_file = " << c_string(metadata_or_empty(sdfg_, "opt_report_file")) << ";" << std::endl;
+    stream << md << ".element_id = " << info.element_id << ";" << std::endl;
+    stream << md << ".element_type = " << c_string(info.element_type) << ";" << std::endl;
+    stream << md << ".target_type = " << c_string(info.target_type) << ";" << std::endl;
+    const LoopInfo& li = info.loop_info;
+    stream << md << ".loopnest_index = " << li.loopnest_index << ";" << std::endl;
+    stream << md << ".num_loops = " << li.num_loops << ";" << std::endl;
+    stream << md << ".num_maps = " << li.num_maps << ";" << std::endl;
+    stream << md << ".num_fors = " << li.num_fors << ";" << std::endl;
+    stream << md << ".num_whiles = " << li.num_whiles << ";" << std::endl;
+    stream << md << ".max_depth = " << li.max_depth << ";" << std::endl;
+    stream << md << ".is_perfectly_nested = " << (li.is_perfectly_nested ? "1" : "0") << ";" << std::endl;
+    stream << md << ".is_perfectly_parallel = " << (li.is_perfectly_parallel ? "1" : "0") << ";" << std::endl;
+    stream << md << ".is_elementwise = " << (li.is_elementwise ? "1" : "0") << ";" << std::endl;
+    stream << md << ".has_side_effects = " << (li.has_side_effects ? "1" : "0") << ";" << std::endl;
+    stream << md << ".region_uuid = " << c_string(stem) << ";" << std::endl;
+    const char* set = "__DAISY_EVENT_SET_NONE";
+    switch (nodes_.at(block.node->element_id())) {
+        case InstrumentationEventType::CPU: set = "__DAISY_EVENT_SET_CPU"; break;
+        case InstrumentationEventType::ROCM: set = "__DAISY_EVENT_SET_ROCM"; break;
+        case InstrumentationEventType::NONE: break;
+    }
+    stream << "long long " << id << " = __daisy_instrumentation_init(&" << md << ", " << set << ");" << std::endl;
+    stream << "__daisy_instrumentation_enter(" << id << ");" << std::endl;
+}
+
+void InstrumentationPlan::end_instrumentation(const structured_control_flow::Block& block, PrettyPrinter& stream,
+                                              const InstrumentationInfo& info) const {
+    const std::string id = sdfg_.name() + "_" + std::to_string(block.node->element_id()) + "_id";
+    stream << "__daisy_instrumentation_exit(" << id << ");" << std::endl;
+    for (auto& entry : info.metrics)
+        stream << "__daisy_instrumentation_metric(" << id << ", \"" << entry.first << "\", " << entry.second << ");" << std::endl;
+    stream << "__daisy_instrumentation_finalize(" << id << ");" << std::endl;
+}
+
+std::unique_ptr<InstrumentationPlan> InstrumentationPlan::none(const StructuredSDFG& sdfg) {
+    return std::make_unique<InstrumentationPlan>(sdfg, std::map<size_t, InstrumentationEventType>{});
+}
+
+std::unique_ptr<InstrumentationPlan> InstrumentationPlan::outermost_loops_plan(const StructuredSDFG& sdfg) {
+    std::map<size_t, InstrumentationEventType> nodes;
+    for (auto& blk : sdfg.blocks()) {
+        const std::string& impl = blk.node->implementation_type();
+        const auto* offloading = dynamic_cast<const rocm::ROCMDataOffloadingNode*>(blk.node.get());
+        const bool transfer = offloading && (offloading->is_h2d() || offloading->is_d2h());
+        if ((!offloading && impl.rfind("ROCM", 0) == 0) || transfer) nodes[blk.node->element_id()] = InstrumentationEventType::ROCM;
+    }
+    return std::make_unique<InstrumentationPlan>(sdfg, std::move(nodes));
+}
+
+std::unique_ptr<InstrumentationPlan> InstrumentationPlan::from_mode(const StructuredSDFG& sdfg, const std::string& mode) {
+    if (mode.empty()) return none(sdfg);
+    if (mode == "ols") return outermost_loops_plan(sdfg);
+    throw std::runtime_error("Unsupported instrumentation plan: " + mode);
 }
 
 LibraryNodeDispatcherRegistry& LibraryNodeDispatcherRegistry::instance() {
@@ -121,10 +216,10 @@ std::vector<std::string> LibraryNodeDispatcherRegistry::keys() const {
 }
 
 CPPCodeGenerator::CPPCodeGenerator(StructuredSDFG& sdfg, std::shared_ptr<CodeSnippetFactory> library_snippet_factory,
-                                   std::string externals_prefix)
+                                   std::string externals_prefix, const InstrumentationPlan* instrumentation_plan)
     : sdfg_(sdfg), library_snippet_factory_(library_snippet_factory ? std::move(library_snippet_factory)
                                                                      : std::make_shared<CodeSnippetFactory>()),
-      externals_prefix_(std::move(externals_prefix)) {}
+      externals_prefix_(std::move(externals_prefix)), instrumentation_plan_(instrumentation_plan) {}
 
 std::string CPPCodeGenerator::function_definition() {
     std::vector<std::string> args;
@@ -143,6 +238,8 @@ void CPPCodeGenerator::dispatch_includes() {
     includes_stream_ << "#include <cstdlib>" << std::endl;
     includes_stream_ << "#include <cstring>" << std::endl;
     includes_stream_ << "#include <cstdint>" << std::endl;
+    // the reference includes <daisy_rtl/daisy_rtl.h> here; this header declares the same protocol
+    if (instrumentation_plan_ && !instrumentation_plan_->empty()) includes_stream_ << "#include \"docc_rocm_rtl.h\"" << std::endl;
 }
 
 void CPPCodeGenerator::dispatch_schedule() {
@@ -168,8 +265,13 @@ void CPPCodeGenerator::dispatch_schedule() {
         auto factory = registry.get_library_node_dispatcher(key);
         if (!factory) throw std::runtime_error("No library node dispatcher found for library node code: " + key);
         auto dispatcher = factory(language_extension_, sdfg_, blk, *blk.node);
+        // brackets as in the reference's DataFlowDispatcher::dispatch_library_node (block_dispatcher.cpp:305-319)
+        const bool instrument = instrumentation_plan_ && instrumentation_plan_->should_instrument(*blk.node);
+        const InstrumentationInfo info = dispatcher->instrumentation_info();
+        if (instrument) instrumentation_plan_->begin_instrumentation(blk, main_stream_, info);
         dispatcher->dispatch(main_stream_, globals_stream_, *library_snippet_factory_);
-        instrumentation_.push_back(dispatcher->instrumentation_info());
+        if (instrument) instrumentation_plan_->end_instrumentation(blk, main_stream_, info);
+        instrumentation_.push_back(info);
     }
     for (auto& kv : sdfg_.containers()) {
         const Container& c = kv.second;

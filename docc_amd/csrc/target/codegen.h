@@ -107,10 +107,59 @@ private:
     std::map<std::string, CodeSnippet> snippets_;
 };
 
+// reference: sdfg/include/sdfg/analysis/loop_analysis.h:25-42 (defaults of a non-loop element)
+struct LoopInfo {
+    int loopnest_index = -1;
+    size_t num_loops = 0, num_maps = 0, num_fors = 0, num_whiles = 0, max_depth = 0;
+    bool is_perfectly_nested = false, is_perfectly_parallel = false, is_elementwise = false, has_side_effects = false;
+};
+
+// reference: sdfg/include/sdfg/codegen/instrumentation/instrumentation_info.h:15-59
+inline const std::string ElementType_H2DTransfer = "h2d_transfer";
+inline const std::string ElementType_D2HTransfer = "d2h_transfer";
+inline const std::string ElementType_Math = "math";
+inline const std::string ElementType_Unknown = "unknown";
+inline const std::string TargetType_SEQUENTIAL = "SEQUENTIAL";
+inline const std::string TargetType_ROCM = "ROCM";
+
 struct InstrumentationInfo {
-    std::string region_name;
-    std::string target_type;                        // "CPU" | "ROCM"
+    size_t element_id = 0;
+    std::string element_type = ElementType_Unknown;
+    std::string target_type = TargetType_SEQUENTIAL;
+    LoopInfo loop_info;
     std::map<std::string, Expression> metrics;      // e.g. "flop", "pcie_bytes"
+    std::string region_name;                        // the node's code, for the generator's report
+};
+
+enum class InstrumentationEventType { CPU, ROCM, NONE };
+
+// Which elements are bracketed by the `__daisy_instrumentation_*` calls, and the text of the
+// brackets (reference sdfg/src/codegen/instrumentation/instrumentation_plan.cpp:22-141: one
+// `__daisy_metadata_t <sdfg>_<id>_md`, `long long <sdfg>_<id>_id = __daisy_instrumentation_init`,
+// enter / exit, one `__daisy_instrumentation_metric` per metric, finalize).
+class InstrumentationPlan {
+public:
+    InstrumentationPlan(const StructuredSDFG& sdfg, std::map<size_t, InstrumentationEventType> nodes)
+        : sdfg_(sdfg), nodes_(std::move(nodes)) {}
+
+    bool should_instrument(const data_flow::LibraryNode& node) const { return nodes_.count(node.element_id()) != 0; }
+    bool empty() const { return nodes_.empty(); }
+    size_t size() const { return nodes_.size(); }
+    void begin_instrumentation(const structured_control_flow::Block& block, PrettyPrinter& stream, const InstrumentationInfo& info) const;
+    void end_instrumentation(const structured_control_flow::Block& block, PrettyPrinter& stream, const InstrumentationInfo& info) const;
+
+    static std::unique_ptr<InstrumentationPlan> none(const StructuredSDFG& sdfg);
+    // The reference's "ols" mode brackets the outermost loops. The rocm target's library nodes
+    // stand where the outermost loop of their expansion would be, so they are the regions here:
+    // every node whose implementation type is a rocm one, and every transfer.
+    static std::unique_ptr<InstrumentationPlan> outermost_loops_plan(const StructuredSDFG& sdfg);
+    // "" -> none, "ols" -> outermost_loops_plan, anything else throws
+    // "Unsupported instrumentation plan: <mode>" (reference python/bindings/py_structured_sdfg.cpp:376-383)
+    static std::unique_ptr<InstrumentationPlan> from_mode(const StructuredSDFG& sdfg, const std::string& mode);
+
+private:
+    const StructuredSDFG& sdfg_;
+    std::map<size_t, InstrumentationEventType> nodes_;
 };
 
 class LibraryNodeDispatcher {
@@ -155,7 +204,7 @@ private:
 class CPPCodeGenerator {
 public:
     CPPCodeGenerator(StructuredSDFG& sdfg, std::shared_ptr<CodeSnippetFactory> library_snippet_factory = nullptr,
-                     std::string externals_prefix = "");
+                     std::string externals_prefix = "", const InstrumentationPlan* instrumentation_plan = nullptr);
 
     // Walks the root sequence and fills the streams. Throws std::runtime_error
     // "No library node dispatcher found for library node code: <key>" when a key is missing
@@ -178,6 +227,7 @@ private:
     CPPLanguageExtension language_extension_;
     std::shared_ptr<CodeSnippetFactory> library_snippet_factory_;
     std::string externals_prefix_;
+    const InstrumentationPlan* instrumentation_plan_;
     PrettyPrinter includes_stream_, classes_stream_, globals_stream_, main_stream_;
     std::vector<InstrumentationInfo> instrumentation_;
 };

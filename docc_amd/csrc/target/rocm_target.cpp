@@ -125,7 +125,8 @@ public:
 
     InstrumentationInfo instrumentation_info() const override {
         InstrumentationInfo info = LibraryNodeDispatcher::instrumentation_info();
-        info.target_type = "ROCM";
+        info.element_type = codegen::ElementType_Math;
+        info.target_type = codegen::TargetType_ROCM;
         if (with_transfers_) info.metrics["pcie_bytes"] = sum_bytes(operands());
         return info;
     }
@@ -316,10 +317,14 @@ public:
 
     InstrumentationInfo instrumentation_info() const override {
         const auto& n = static_cast<const ROCMDataOffloadingNode&>(node_);
-        InstrumentationInfo info;
+        // as the CUDA transfer node reports itself (reference cuda_data_offloading_node.cpp:175-196)
+        InstrumentationInfo info = LibraryNodeDispatcher::instrumentation_info();
         info.region_name = n.toStr();
-        info.target_type = n.is_h2d() ? "H2D" : n.is_d2h() ? "D2H" : "ROCM";
-        if (n.is_h2d() || n.is_d2h()) info.metrics["pcie_bytes"] = n.size();
+        info.target_type = codegen::TargetType_ROCM;
+        if (n.is_h2d() || n.is_d2h()) {
+            info.element_type = n.is_h2d() ? codegen::ElementType_H2DTransfer : codegen::ElementType_D2HTransfer;
+            info.metrics["pcie_bytes"] = n.size();
+        }
         return info;
     }
 };
@@ -572,15 +577,17 @@ bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, ana
         for (auto& out : sdfg.blocks()[i].outputs)
             for (auto& p : plans)
                 if (out.data == p.host) out.data = p.device;
+        // the transfers of a node carry its source position
+        const structured_control_flow::DebugInfo dbg = sdfg.blocks()[i].debug_info;
         // before: ALLOC (+H2D when the node reads the operand)
         size_t pos = i;
         for (auto& p : plans) {
             if (p.read) {
                 sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::H2D, BufferLifecycle::ALLOC),
-                               {make_binding("_src", p.host)}, {make_binding("_dst", p.device)}, pos++);
+                               {make_binding("_src", p.host)}, {make_binding("_dst", p.device)}, pos++).debug_info = dbg;
             } else {
                 sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::NONE, BufferLifecycle::ALLOC),
-                               {}, {make_binding("_ret", p.device)}, pos++);
+                               {}, {make_binding("_ret", p.device)}, pos++).debug_info = dbg;
             }
         }
         // the node now sits at `pos`; after it: D2H+FREE for what it wrote, FREE for the rest
@@ -588,13 +595,13 @@ bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, ana
         for (auto& p : plans) {
             if (p.written) {
                 sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::D2H, BufferLifecycle::FREE),
-                               {make_binding("_src", p.device)}, {make_binding("_dst", p.host)}, after++);
+                               {make_binding("_src", p.device)}, {make_binding("_dst", p.host)}, after++).debug_info = dbg;
             }
         }
         for (auto& p : plans) {
             if (!p.written) {
                 sdfg.add_block(std::make_unique<ROCMDataOffloadingNode>(p.bytes, 0, DataTransferDirection::NONE, BufferLifecycle::FREE),
-                               {make_binding("_ptr", p.device)}, {}, after++);
+                               {make_binding("_ptr", p.device)}, {}, after++).debug_info = dbg;
             }
         }
         i = after - 1;

@@ -688,6 +688,17 @@ json::Value StructuredSDFG::to_json() const {
         Value b;
         b.set("type", "block");
         b.set("element_id", blk.element_id);
+        if (blk.debug_info.has) {
+            Value d;
+            d.set("has", true);
+            d.set("filename", blk.debug_info.filename);
+            d.set("function", blk.debug_info.function);
+            d.set("start_line", (int64_t) blk.debug_info.start_line);
+            d.set("start_column", (int64_t) blk.debug_info.start_column);
+            d.set("end_line", (int64_t) blk.debug_info.end_line);
+            d.set("end_column", (int64_t) blk.debug_info.end_column);
+            b.set("debug_info", std::move(d));
+        }
         b.set("dataflow", std::move(df));
         children.push_back(std::move(b));
     }
@@ -745,7 +756,19 @@ std::unique_ptr<StructuredSDFG> StructuredSDFG::from_json(const json::Value& j) 
             }
             return out;
         };
-        sdfg->add_block(std::move(node), bindings(df.at("inputs")), bindings(df.at("outputs")));
+        auto& blk = sdfg->add_block(std::move(node), bindings(df.at("inputs")), bindings(df.at("outputs")));
+        if (const Value* d = child.find("debug_info")) {
+            const Value* has = d->find("has");
+            if (has && has->as_bool()) {
+                blk.debug_info.has = true;
+                blk.debug_info.filename = d->at("filename").as_string();
+                blk.debug_info.function = d->at("function").as_string();
+                blk.debug_info.start_line = (long) d->at("start_line").as_int();
+                blk.debug_info.start_column = (long) d->at("start_column").as_int();
+                blk.debug_info.end_line = (long) d->at("end_line").as_int();
+                blk.debug_info.end_column = (long) d->at("end_column").as_int();
+            }
+        }
     }
     return sdfg;
 }

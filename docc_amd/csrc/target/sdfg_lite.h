@@ -369,9 +369,19 @@ private:
 
 namespace structured_control_flow {
 
+// Source position of an element (reference sdfg/include/sdfg/element.h DebugInfo; JSON keys of
+// json_serializer.cpp debug_info_to_json: has, filename, function, start_line, start_column,
+// end_line, end_column).
+struct DebugInfo {
+    bool has = false;
+    std::string filename, function;
+    long start_line = 0, start_column = 0, end_line = 0, end_column = 0;
+};
+
 // One block of the root sequence: a dataflow graph with exactly one library node.
 struct Block {
     size_t element_id = 0;
+    DebugInfo debug_info;
     std::unique_ptr<data_flow::LibraryNode> node;
     std::vector<data_flow::ConnectorBinding> inputs;
     std::vector<data_flow::ConnectorBinding> outputs;

@@ -55,12 +55,14 @@ struct Generated {
     std::vector<std::filesystem::path> snippet_files;
 };
 
-Generated generate(StructuredSDFG& sdfg, const char* output_dir) {
+Generated generate(StructuredSDFG& sdfg, const char* output_dir, const char* instrumentation_mode, bool* instrumented = nullptr) {
     if (!output_dir || !*output_dir) throw std::invalid_argument("no output directory");
     std::filesystem::path dir(output_dir);
     std::filesystem::create_directories(dir);
     auto snippets = std::make_shared<codegen::CodeSnippetFactory>(dir);
-    codegen::CPPCodeGenerator gen(sdfg, snippets);
+    auto plan = codegen::InstrumentationPlan::from_mode(sdfg, instrumentation_mode ? instrumentation_mode : "");
+    if (instrumented) *instrumented = !plan->empty();
+    codegen::CPPCodeGenerator gen(sdfg, snippets, "", plan.get());
     gen.generate();
     Generated g;
     g.header = dir / (sdfg.name() + ".h");
@@ -119,10 +121,10 @@ char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, con
     });
 }
 
-char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir) {
+char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir, const char* instrumentation_mode) {
     return guarded([&] {
         auto sdfg = parse(sdfg_json);
-        Generated g = generate(*sdfg, output_dir);
+        Generated g = generate(*sdfg, output_dir, instrumentation_mode);
         json::Value report;
         report.set("header", g.header.string());
         report.set("source", g.source.string());
@@ -131,6 +133,8 @@ char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir) {
         for (auto& info : g.instrumentation) {
             json::Value r;
             r.set("region", info.region_name);
+            r.set("element_id", info.element_id);
+            r.set("element_type", info.element_type);
             r.set("target_type", info.target_type);
             json::Value metrics{json::Object{}};
             for (auto& kv : info.metrics) metrics.set(kv.first, kv.second);
@@ -143,11 +147,12 @@ char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir) {
 }
 
 char* docc_rocm_target_compile(const char* sdfg_json, const char* output_dir, const char* include_dir,
-                               const char* runtime_lib_dir) {
+                               const char* runtime_lib_dir, const char* instrumentation_mode) {
     return guarded([&] {
         if (!include_dir || !runtime_lib_dir) throw std::invalid_argument("include and runtime library directories are required");
         auto sdfg = parse(sdfg_json);
-        Generated g = generate(*sdfg, output_dir);
+        bool instrumented = false;
+        Generated g = generate(*sdfg, output_dir, instrumentation_mode, &instrumented);
         const std::filesystem::path dir(output_dir);
         const std::string cxx = host_compiler();
         // compile, then link: two compiler processes, as the reference's JIT does
@@ -158,7 +163,7 @@ char* docc_rocm_target_compile(const char* sdfg_json, const char* output_dir, co
         if (std::system(compile.c_str()) != 0) throw std::runtime_error("Compilation failed: " + compile);
         const std::filesystem::path lib = dir / ("lib" + sdfg->name() + ".so");
         std::string link = cxx + " -shared " + quote(object.string()) + " -o " + quote(lib.string()) + " -L" + quote(runtime_lib_dir) +
-                           " -ldocc_rt_rocm -Wl,-rpath," + quote(runtime_lib_dir) + " -lm -lstdc++ >> " + quote(log.string()) + " 2>&1";
+                           (instrumented ? " -ldocc_rtl_rocm" : "") + " -ldocc_rt_rocm -Wl,-rpath," + quote(runtime_lib_dir) + " -lm -lstdc++ >> " + quote(log.string()) + " 2>&1";
         if (std::system(link.c_str()) != 0) throw std::runtime_error("Linking failed: " + link);
         return lib.string();
     });

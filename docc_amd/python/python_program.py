@@ -497,8 +497,17 @@ class _Lowering(ast.NodeVisitor):
         self.fail(node, f"statement {type(node).__name__}")
 
     def visit_FunctionDef(self, node: ast.FunctionDef):
+        try:
+            filename = inspect.getsourcefile(self.func) or ""
+            first = inspect.getsourcelines(self.func)[1]
+        except (OSError, TypeError):
+            filename, first = "", 1
         for stmt in node.body:
+            # the nodes a statement lowers to carry its source range (lines of the file, not of the snippet)
+            self.b.set_debug_info(filename, self.func.__name__, first + stmt.lineno - 1, stmt.col_offset + 1,
+                                  first + (stmt.end_lineno or stmt.lineno) - 1, (stmt.end_col_offset or stmt.col_offset) + 1)
             self.visit(stmt)
+        self.b.set_debug_info()
 
     def visit_arguments(self, node):
         return

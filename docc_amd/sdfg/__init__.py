@@ -45,8 +45,8 @@ def _native() -> ctypes.CDLL:
         cp = ctypes.c_char_p
         lib.docc_rocm_target_register.restype = ctypes.c_int
         for name, args in (("docc_rocm_target_dispatcher_keys", []), ("docc_rocm_target_validate", [cp]),
-                           ("docc_rocm_target_schedule", [cp, cp, cp]), ("docc_rocm_target_generate", [cp, cp]),
-                           ("docc_rocm_target_compile", [cp, cp, cp, cp]), ("docc_rocm_target_report", [cp])):
+                           ("docc_rocm_target_schedule", [cp, cp, cp]), ("docc_rocm_target_generate", [cp, cp, cp]),
+                           ("docc_rocm_target_compile", [cp, cp, cp, cp, cp]), ("docc_rocm_target_report", [cp])):
             fn = getattr(lib, name)
             fn.argtypes = args
             fn.restype = ctypes.c_void_p  # kept as an address so that it can be freed
@@ -192,9 +192,17 @@ class StructuredSDFG:
         """No loop nests, so there is nothing to normalize."""
 
     def dump(self, output_folder: str, suffix: str = "") -> None:
+        """Writes <name>[.<suffix>].json and records the file names in the SDFG's metadata, as the
+        reference's dump does (python/bindings/py_structured_sdfg.cpp:263-292); instrumented code
+        carries them into every trace event."""
         os.makedirs(output_folder, exist_ok=True)
-        name = self.name + (f".{suffix}" if suffix else "") + ".json"
-        Path(output_folder, name).write_text(json.dumps(self._data, indent=2))
+        stem = self.name + (f".{suffix}" if suffix else "")
+        meta = self._data.setdefault("metadata", {})
+        meta["sdfg_file"] = str(Path(output_folder, stem + ".json"))
+        meta["arg_capture_path"] = str(Path(output_folder, "arg_captures" + (f".{suffix}" if suffix else "")))
+        meta["features_file"] = str(Path(output_folder, stem + ".npz"))
+        meta["opt_report_file"] = str(Path(output_folder, stem + ".opt_report.json"))
+        Path(output_folder, stem + ".json").write_text(json.dumps(self._data, indent=2))
 
     def schedule(self, target: str, category: str = "server", remote_tuning: bool = False,
                  options: Optional[Dict[str, Any]] = None) -> None:
@@ -205,14 +213,19 @@ class StructuredSDFG:
         opts = {k: v for k, v in (options or {}).items() if k in ("offload", "require_all_mapped")}
         self._data = json.loads(_call("docc_rocm_target_schedule", self.to_json(), category, json.dumps(opts)))
 
-    def generate(self, output_folder: str) -> Dict[str, Any]:
+    def generate(self, output_folder: str, instrumentation_mode: str = "") -> Dict[str, Any]:
         """Writes <name>.h / <name>.cpp and returns the generator's report."""
-        return json.loads(_call("docc_rocm_target_generate", self.to_json(), output_folder))
+        return json.loads(_call("docc_rocm_target_generate", self.to_json(), output_folder, instrumentation_mode or ""))
 
     def _compile(self, output_folder: str, target: str = "rocm", instrumentation_mode: str = "",
                  capture_args: bool = False) -> str:
-        """Generates, compiles and links lib<name>.so; returns its path."""
-        return _call("docc_rocm_target_compile", self.to_json(), output_folder, str(_INCLUDE_DIR), str(_LIB_DIR))
+        """Generates, compiles and links lib<name>.so; returns its path. `instrumentation_mode`
+        "" or "ols" (reference py_structured_sdfg.cpp:376-383); argument capture is not part of
+        this target."""
+        if capture_args:
+            raise NotImplementedError("argument capture (capture_args=True) is not part of the rocm target")
+        return _call("docc_rocm_target_compile", self.to_json(), output_folder, str(_INCLUDE_DIR), str(_LIB_DIR),
+                     instrumentation_mode or "")
 
 
 class StructuredSDFGBuilder:
@@ -249,11 +262,23 @@ class StructuredSDFGBuilder:
     def _element(self, name: str) -> PrimitiveType:
         return PrimitiveType(self._data["containers"][name]["element"])
 
+    def set_debug_info(self, filename: str = "", function: str = "", start_line: int = 0, start_column: int = 0,
+                       end_line: int = 0, end_column: int = 0) -> None:
+        """Source position attached to the blocks added from now on (the reference passes a
+        DebugInfo to every add_* call; its JSON keys are those of debug_info_to_json,
+        sdfg/src/serializer/json_serializer.cpp). An empty filename clears it."""
+        self._debug_info = None if not filename else {
+            "has": True, "filename": filename, "function": function, "start_line": int(start_line),
+            "start_column": int(start_column), "end_line": int(end_line), "end_column": int(end_column)}
+
     def _add_block(self, node: Dict[str, Any], inputs: Sequence[Dict[str, Any]], outputs: Sequence[Dict[str, Any]]) -> None:
         self._ids += 2
         node = {"type": "library_node", "element_id": self._ids, **node}
-        self._data["root"]["children"].append({"type": "block", "element_id": self._ids - 1, "dataflow": {
-            "library_node": node, "inputs": list(inputs), "outputs": list(outputs)}})
+        block = {"type": "block", "element_id": self._ids - 1, "dataflow": {
+            "library_node": node, "inputs": list(inputs), "outputs": list(outputs)}}
+        if getattr(self, "_debug_info", None):
+            block["debug_info"] = dict(self._debug_info)
+        self._data["root"]["children"].append(block)
 
     @staticmethod
     def _operand(connector: str, value: Any, const_type: Optional[PrimitiveType] = None) -> Dict[str, Any]:

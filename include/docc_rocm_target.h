@@ -42,15 +42,19 @@ char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, con
 
 /* Generates <output_dir>/<name>.h and <name>.cpp and returns a JSON report:
  * {"header": path, "source": path, "function": definition, "instrumentation": [...]}.
+ * `instrumentation_mode`: NULL or "" for none, "ols" to bracket every rocm node and transfer with
+ * the `__daisy_instrumentation_*` calls (include/docc_rocm_rtl.h); any other value is the error
+ * "Unsupported instrumentation plan: <mode>".
  * Counterpart of CPPCodeGenerator::generate + as_source (reference py_structured_sdfg.cpp:355-420). */
-char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir);
+char* docc_rocm_target_generate(const char* sdfg_json, const char* output_dir, const char* instrumentation_mode);
 
 /* generate + compile + link into <output_dir>/lib<name>.so against `runtime_lib_dir`/libdocc_rt_rocm.so
  * with headers from `include_dir`; returns the library path. The compiler is
  * $DOCC_CXX, else ROCm's clang++, invoked through std::system like the reference's JIT step
- * (py_structured_sdfg.cpp:456,485,516-551: -c -fPIC -O3 -march=native -mtune=native -funroll-loops, then -shared). */
+ * (py_structured_sdfg.cpp:456,485,516-551: -c -fPIC -O3 -march=native -mtune=native -funroll-loops, then -shared).
+ * An instrumented library also links `runtime_lib_dir`/libdocc_rtl_rocm.so. */
 char* docc_rocm_target_compile(const char* sdfg_json, const char* output_dir, const char* include_dir,
-                               const char* runtime_lib_dir);
+                               const char* runtime_lib_dir, const char* instrumentation_mode);
 
 /* JSON object counting the library nodes per "<code>::<implementation type>" plus transfers,
  * the analogue of loop_report() (reference py_structured_sdfg.cpp:570-583). */

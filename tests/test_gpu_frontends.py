@@ -229,3 +229,37 @@ def test_torch_compile_mlp_fp32():
     assert rel_err_max(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
     r = program.last_sdfg.loop_report()
     assert r["GEMM"] == 2 and r["H2D"] == 0 and r["D2H"] == 0      # device tensors: no transfers at all
+
+
+@pytest.mark.parametrize("mode", ["", "aggregate"])
+def test_instrumented_program_writes_a_trace_with_device_times(tmp_path, mode):
+    """`instrumentation_mode="ols"`: every rocm node and transfer is a region timed with HIP events;
+    the trace is written when the process ends."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    out = tmp_path / "trace.json"
+    env = dict(os.environ, __DAISY_INSTRUMENTATION_FILE=str(out), __DAISY_INSTRUMENTATION_MODE=mode, DOCC_TMP=str(tmp_path / "docc"),
+               PYTHONPATH=str(Path(__file__).resolve().parent.parent))
+    r = subprocess.run([sys.executable, "-m", "docc_amd.examples.dense_instrumented"], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    events = json.loads(out.read_text())["traceEvents"]
+    kinds = {}
+    for e in events:
+        kinds.setdefault(e["args"]["docc"]["element_type"], []).append(e)
+    runs = 1 if mode == "aggregate" else 3
+    assert len(kinds["math"]) == 4 * runs             # GEMM, Broadcast, Add, ReLU
+    assert len(kinds["h2d_transfer"]) == 3 * runs and len(kinds["d2h_transfer"]) == 1 * runs
+    assert all(e["args"]["target_type"] == "ROCM" and e["args"]["function"] == "dense" and e["dur"] > 0 for e in events)
+    flop = [e["args"]["metrics"].get("static:::flop") for e in kinds["math"]]
+    expect = 2.0 * 512 * 384 * 256 + 2.0 * 512 * 384     # multiply-adds plus the alpha/beta epilogue, as the reference counts
+    assert any((f["mean"] if isinstance(f, dict) else f) == expect for f in flop if f is not None)
+    pcie = sorted((e["args"]["metrics"]["static:::pcie_bytes"]["mean"] if mode == "aggregate" else e["args"]["metrics"]["static:::pcie_bytes"])
+                  for e in kinds["h2d_transfer"])[-1]
+    assert pcie == 512 * 256 * 4
+    # a GEMM of this size takes well under 10 ms on the device; a region's time is a device time, not the process's
+    gemm = [e for e in kinds["math"] if e["name"].startswith("dense") and (e["args"]["metrics"].get("static:::flop") is not None)]
+    assert gemm and min(e["dur"] / (3 if mode == "aggregate" else 1) for e in gemm) < 10000
