@@ -1,0 +1,518 @@
+// Conversion between the reference's SDFG wire format and the block list of this target.
+//
+// The reference writes an SDFG as (sdfg/src/serializer/json_serializer.cpp:56-353)
+//   { name, element_counter, type, return_type, structures[], containers{name: <type>}, arguments[],
+//     externals[], metadata{}, root: <sequence> }
+//   <sequence> = { type "sequence", children[], transitions[] }, children: block | for | map | while |
+//                if_else | return | break | continue | sequence
+//   block.dataflow = { nodes[], edges[] }; nodes: access_node {data} | constant_node {data, data_type} |
+//                    tasklet | library_node {code, implementation_type, ...payload};
+//                    edges: {src, dst, src_conn, dst_conn, subset[], base_type}
+//   <type> = { type: scalar | pointer | array | structure | function | tensor | reference,
+//              primitive_type (enum value), pointee_type / element_type, storage_type {value, allocation,
+//              deallocation, allocation_size?}, ... }
+// What the rocm target can take from it is a root sequence of blocks that hold one library node
+// each (with its access and constant nodes), allocation and release of temporaries (Malloc / Free
+// nodes, managed storage) and a final return; loop nests, tasklets and branches have no lowering
+// here and are refused with the element that stopped the import.
+#include <algorithm>
+#include <cctype>
+#include <map>
+#include <set>
+
+#include "rocm_target.h"
+#include "sdfg_lite.h"
+
+namespace sdfg::serializer {
+
+using json::Array;
+using json::Object;
+using json::Value;
+
+namespace {
+
+// enum PrimitiveType of the reference (sdfg/include/sdfg/types/type.h:35-55), by value
+const char* const kReferencePrimitive[] = {"Void",  "Bool",   "Int8",   "Int16",   "Int32", "Int64",  "Int128", "UInt8",
+                                           "UInt16", "UInt32", "UInt64", "UInt128", "Half",  "BFloat", "Float",  "Double"};
+
+types::PrimitiveType primitive_of(const Value& v, const std::string& where) {
+    const int64_t i = v.as_int();
+    if (i < 0 || i >= (int64_t) (sizeof(kReferencePrimitive) / sizeof(kReferencePrimitive[0])) || i == 6 || i == 11)
+        throw InvalidSDFGException(where + ": primitive type " + std::to_string(i) + " is not supported");
+    return types::primitive_type_from_string(kReferencePrimitive[i]);
+}
+
+int64_t reference_primitive(types::PrimitiveType t) {
+    const std::string name = types::primitive_type_to_string(t);
+    for (size_t i = 0; i < sizeof(kReferencePrimitive) / sizeof(kReferencePrimitive[0]); i++)
+        if (name == kReferencePrimitive[i]) return (int64_t) i;
+    return 0;
+}
+
+// element type behind a scalar, pointer, array or tensor type
+types::PrimitiveType element_of(const Value& type, const std::string& where) {
+    const std::string kind = type.at("type").as_string();
+    if (kind == "scalar") return primitive_of(type.at("primitive_type"), where);
+    if (kind == "pointer") {
+        const Value* pointee = type.find("pointee_type");
+        if (!pointee) throw InvalidSDFGException(where + ": opaque pointer");
+        return element_of(*pointee, where);
+    }
+    if (kind == "array" || kind == "tensor") return element_of(type.at("element_type"), where);
+    throw InvalidSDFGException(where + ": " + kind + " types are not supported by the rocm target");
+}
+
+// Expressions arrive in SymEngine's spelling; the only construct of it that is not C is the power
+// operator. `base**n` (n a small non-negative integer) becomes a product.
+std::string c_expression(std::string e) {
+    for (size_t at = e.find("**"); at != std::string::npos; at = e.find("**")) {
+        size_t begin = at;
+        if (begin > 0 && e[begin - 1] == ')') {
+            int depth = 0;
+            while (begin > 0) {
+                begin--;
+                if (e[begin] == ')') depth++;
+                if (e[begin] == '(' && --depth == 0) break;
+            }
+            if (depth != 0) throw InvalidSDFGException("unbalanced expression '" + e + "'");
+        } else {
+            while (begin > 0 && (std::isalnum((unsigned char) e[begin - 1]) || e[begin - 1] == '_' || e[begin - 1] == '.')) begin--;
+        }
+        size_t end = at + 2;
+        while (end < e.size() && std::isdigit((unsigned char) e[end])) end++;
+        if (begin == at || end == at + 2 || end - (at + 2) > 2)
+            throw InvalidSDFGException("power in '" + e + "' is not a small integer power of a term");
+        const std::string base = e.substr(begin, at - begin);
+        const int n = std::stoi(e.substr(at + 2, end - (at + 2)));
+        std::string product = n == 0 ? "1" : "(" + base;
+        for (int i = 1; i < n; i++) product += "*" + base;
+        if (n > 0) product += ")";
+        e = e.substr(0, begin) + product + e.substr(end);
+    }
+    return e;
+}
+
+// the same rewrite on every string inside a node payload
+Value c_expressions(const Value& v) {
+    if (v.is_string()) return Value(c_expression(v.as_string()));
+    if (v.is_array()) {
+        Array a;
+        for (auto& e : v.as_array()) a.push_back(c_expressions(e));
+        return Value(std::move(a));
+    }
+    if (v.is_object()) {
+        Object o;
+        for (auto& kv : v.as_object()) o.emplace_back(kv.first, c_expressions(kv.second));
+        return Value(std::move(o));
+    }
+    return v;
+}
+
+std::string describe(const Value& element) {
+    std::string s = element.at("type").as_string();
+    if (const Value* id = element.find("element_id")) s += " (element " + std::to_string(id->as_int()) + ")";
+    return s;
+}
+
+Value debug_info_of(const Value& element) {
+    const Value* d = element.find("debug_info");
+    if (d && d->is_object()) {
+        const Value* has = d->find("has");
+        if (has && has->is_bool() && has->as_bool()) return *d;
+    }
+    return Value();
+}
+
+struct Import {
+    const Value& src;
+    Value out;
+    Object containers;   // lite container entries, by name
+    std::set<std::string> transient_done;
+
+    explicit Import(const Value& j) : src(j) {}
+
+    Value& container(const std::string& name) {
+        for (auto& kv : containers)
+            if (kv.first == name) return kv.second;
+        throw InvalidSDFGException("container '" + name + "' does not exist");
+    }
+
+    void import_containers() {
+        for (auto& kv : src.at("containers").as_object()) {
+            const Value& t = kv.second;
+            const std::string kind = t.at("type").as_string();
+            const std::string where = "container '" + kv.first + "'";
+            Value c;
+            if (kind == "scalar") {
+                c.set("type", "scalar");
+            } else if (kind == "pointer") {
+                c.set("type", "pointer");
+            } else {
+                throw InvalidSDFGException(where + ": " + kind + " types are not supported by the rocm target");
+            }
+            c.set("element", types::primitive_type_to_string(element_of(t, where)));
+            bool transient = false;
+            std::string storage = "CPU";
+            if (const Value* st = t.find("storage_type")) {
+                const std::string v = st->at("value").as_string();
+                if (v == "ROCM_Generic")
+                    storage = v;
+                else if (v.rfind("CPU", 0) != 0)
+                    throw InvalidSDFGException(where + ": storage " + v + " belongs to another target");
+                // managed allocation: the generated function owns the buffer (reference type.h:67-79)
+                const Value* alloc = st->find("allocation");
+                const Value* size = st->find("allocation_size");
+                if (alloc && alloc->as_int() == 1 && size) {
+                    transient = true;
+                    c.set("size", c_expression(size->as_expression()));
+                }
+            }
+            c.set("transient", transient);
+            c.set("storage", storage);
+            containers.emplace_back(kv.first, std::move(c));
+        }
+    }
+
+    // a block of the reference -> nullopt (nothing to do) or one lite block
+    bool import_block(const Value& block, Array& children) {
+        const Value& df = block.at("dataflow");
+        const Array& nodes = df.at("nodes").as_array();
+        if (nodes.empty()) return false;   // e.g. the empty view block add_gemm leaves behind
+        std::map<int64_t, const Value*> by_id;
+        const Value* lib = nullptr;
+        for (auto& n : nodes) {
+            by_id[n.at("element_id").as_int()] = &n;
+            const std::string kind = n.at("type").as_string();
+            if (kind == "tasklet")
+                throw InvalidSDFGException(describe(n) + " in " + describe(block) + ": tasklets are not lowered by the rocm target");
+            if (kind == "library_node") {
+                if (lib) throw InvalidSDFGException(describe(block) + ": more than one library node in a block");
+                lib = &n;
+            }
+        }
+        if (!lib) return false;   // access nodes only: no computation
+        const int64_t lib_id = lib->at("element_id").as_int();
+        const std::string code = lib->at("code").as_string();
+
+        auto node_of = [&](const Value& edge, const char* end) -> const Value& {
+            auto it = by_id.find(edge.at(end).as_int());
+            if (it == by_id.end()) throw InvalidSDFGException(describe(block) + ": edge refers to an unknown node");
+            return *it->second;
+        };
+
+        Array inputs, outputs;
+        const Value* out_type = nullptr;
+        bool has_bias_edge = false;
+        for (auto& e : df.at("edges").as_array()) {
+            const bool into = e.at("dst").as_int() == lib_id, from = e.at("src").as_int() == lib_id;
+            if (!into && !from) throw InvalidSDFGException(describe(block) + ": data movement beside the library node");
+            for (auto& s : e.at("subset").as_array())
+                if (s.as_expression() != "0")
+                    throw InvalidSDFGException(describe(block) + ": a subset on an operand of " + code + " (views are not supported)");
+            Value b;
+            if (into) {
+                const Value& n = node_of(e, "src");
+                b.set("connector", e.at("dst_conn").as_string());
+                if (n.at("type").as_string() == "constant_node") {
+                    b.set("constant", c_expression(n.at("data").as_expression()));
+                    b.set("type", types::primitive_type_to_string(element_of(n.at("data_type"), describe(n))));
+                } else {
+                    b.set("data", n.at("data").as_string());
+                }
+                if (e.at("dst_conn").as_string() == "B") has_bias_edge = true;
+                inputs.push_back(std::move(b));
+            } else {
+                const Value& n = node_of(e, "dst");
+                b.set("connector", e.at("src_conn").as_string());
+                b.set("data", n.at("data").as_string());
+                out_type = &e.at("base_type");
+                outputs.push_back(std::move(b));
+            }
+        }
+
+        // allocation and release of a temporary: the container becomes a transient of the function
+        if (code == "Malloc") {
+            if (outputs.size() != 1) throw InvalidSDFGException(describe(*lib) + ": Malloc without a target");
+            Value& c = container(outputs[0].at("data").as_string());
+            c.set("transient", true);
+            c.set("size", c_expression(lib->at("size").as_expression()));
+            return false;
+        }
+        if (code == "Free") return false;
+
+        Value node{Object{}};
+        for (auto& kv : lib->as_object())
+            if (kv.first != "debug_info") node.set(kv.first, c_expressions(kv.second));
+        node.set("side_effect", false);
+        // what the reference keeps in the memlet types, the block list keeps on the node
+        if (code != "GEMM" && !node.contains("element_type")) {
+            if (!out_type) throw InvalidSDFGException(describe(*lib) + ": no output edge");
+            node.set("element_type", types::primitive_type_to_string(element_of(*out_type, describe(*lib))));
+        }
+        if (code == "ml::Conv" && !node.contains("has_bias")) node.set("has_bias", has_bias_edge);
+        if (code == "ml::MatMul") {
+            for (const char* key : {"offset_a", "offset_b"})
+                if (const Value* o = node.find(key))
+                    if (o->as_expression() != "0") throw InvalidSDFGException(describe(*lib) + ": ml::MatMul with an operand offset");
+            for (const char* key : {"strides_a", "strides_b"})
+                if (const Value* s = node.find(key))
+                    if (!s->as_array().empty() && s->as_array().back().as_expression() != "1")
+                        throw InvalidSDFGException(describe(*lib) + ": ml::MatMul on a non-contiguous operand");
+        }
+
+        Value flow;
+        flow.set("library_node", std::move(node));
+        flow.set("inputs", Value(std::move(inputs)));
+        flow.set("outputs", Value(std::move(outputs)));
+        Value b;
+        b.set("type", "block");
+        b.set("element_id", block.at("element_id").as_int());
+        Value dbg = debug_info_of(*lib);
+        if (dbg.is_null()) dbg = debug_info_of(block);
+        if (!dbg.is_null()) b.set("debug_info", std::move(dbg));
+        b.set("dataflow", std::move(flow));
+        children.push_back(std::move(b));
+        return true;
+    }
+
+    void import_sequence(const Value& seq, Array& children, std::string& returned) {
+        if (const Value* transitions = seq.find("transitions"))
+            for (auto& t : transitions->as_array())
+                if (!t.at("assignments").as_array().empty())
+                    throw InvalidSDFGException(describe(t) + ": symbol assignments between blocks are not lowered by the rocm target");
+        for (auto& child : seq.at("children").as_array()) {
+            const std::string kind = child.at("type").as_string();
+            if (!returned.empty())
+                throw InvalidSDFGException(describe(child) + ": code after the return");
+            if (kind == "block") {
+                import_block(child, children);
+            } else if (kind == "sequence") {
+                import_sequence(child, children, returned);
+            } else if (kind == "return") {
+                const std::string data = child.at("data").as_string();
+                if (child.contains("data_type")) throw InvalidSDFGException(describe(child) + ": returning a constant");
+                returned = data.empty() ? "\x01" : data;
+            } else {
+                throw InvalidSDFGException(describe(child) + ": control flow other than a sequence of library-node blocks is not "
+                                           "lowered by the rocm target");
+            }
+        }
+    }
+
+    Value run() {
+        for (const char* key : {"name", "containers", "arguments", "root"})
+            if (!src.contains(key)) throw InvalidSDFGException(std::string("not an SDFG: no \"") + key + "\"");
+        if (const Value* t = src.find("type"))
+            if (t->is_string() && t->as_string() != "CPU")
+                throw InvalidSDFGException("function type " + t->as_string() + " belongs to another target");
+        if (const Value* ex = src.find("externals"))
+            if (!ex->as_array().empty()) throw InvalidSDFGException("externals are not supported by the rocm target");
+        import_containers();
+        Array children;
+        std::string returned;
+        import_sequence(src.at("root"), children, returned);
+        out.set("type", "structured_sdfg");
+        out.set("name", src.at("name").as_string());
+        out.set("arguments", src.at("arguments"));
+        out.set("containers", Value(std::move(containers)));
+        out.set("return", returned == "\x01" ? std::string() : returned);
+        Value meta{Object{}};
+        if (const Value* m = src.find("metadata"))
+            for (auto& kv : m->as_object()) meta.set(kv.first, kv.second);
+        out.set("metadata", std::move(meta));
+        Value root;
+        root.set("type", "sequence");
+        root.set("children", Value(std::move(children)));
+        out.set("root", std::move(root));
+        return out;
+    }
+};
+
+// ---- export ---------------------------------------------------------------------------
+
+Value empty_debug_info() {
+    Value d;
+    d.set("has", false);
+    d.set("filename", "");
+    d.set("function", "");
+    d.set("start_line", 0);
+    d.set("start_column", 0);
+    d.set("end_line", 0);
+    d.set("end_column", 0);
+    return d;
+}
+
+Value storage_json(const Container& c) {
+    Value s;
+    s.set("value", c.storage == "CPU" ? (c.transient && c.is_pointer ? "CPU_Heap" : "CPU_Stack") : c.storage);
+    const bool managed = c.transient && c.is_pointer && !c.size_bytes.empty();
+    s.set("allocation", managed ? 1 : 0);
+    s.set("deallocation", managed ? 1 : 0);
+    if (managed) s.set("allocation_size", c.size_bytes);
+    return s;
+}
+
+Value plain_storage() {
+    Value s;
+    s.set("value", "CPU_Stack");
+    s.set("allocation", 0);
+    s.set("deallocation", 0);
+    return s;
+}
+
+Value scalar_json(types::PrimitiveType t, Value storage) {
+    Value j;
+    j.set("type", "scalar");
+    j.set("primitive_type", reference_primitive(t));
+    j.set("storage_type", std::move(storage));
+    j.set("initializer", "");
+    j.set("alignment", 0);
+    return j;
+}
+
+Value type_json(const Container& c) {
+    if (!c.is_pointer) return scalar_json(c.element, storage_json(c));
+    Value j;
+    j.set("type", "pointer");
+    j.set("pointee_type", scalar_json(c.element, plain_storage()));
+    j.set("storage_type", storage_json(c));
+    j.set("initializer", "");
+    j.set("alignment", 0);
+    return j;
+}
+
+} // namespace
+
+// the reference's serializer always writes "element_counter"; the block list never does
+bool is_reference_format(const Value& j) { return j.is_object() && j.contains("element_counter"); }
+
+Value import_reference_json(const Value& j) { return Import(j).run(); }
+
+Value export_reference_json(const StructuredSDFG& sdfg) {
+    size_t counter = 0;
+    auto next = [&] { return (int64_t) ++counter; };
+    Value j;
+    j.set("name", sdfg.name());
+    j.set("type", "CPU");
+    Container nothing;
+    nothing.element = types::PrimitiveType::Void;
+    j.set("return_type", sdfg.return_container().empty() ? type_json(nothing) : type_json(sdfg.container(sdfg.return_container())));
+    j.set("structures", Value(Array{}));
+    Value containers{Object{}};
+    for (auto& kv : sdfg.containers()) containers.set(kv.first, type_json(kv.second));
+    j.set("containers", std::move(containers));
+    Array args;
+    for (auto& a : sdfg.arguments()) args.emplace_back(a);
+    j.set("arguments", Value(std::move(args)));
+    j.set("externals", Value(Array{}));
+    Value meta{Object{}};
+    for (auto& kv : sdfg.metadata()) meta.set(kv.first, kv.second);
+    j.set("metadata", std::move(meta));
+
+    auto debug_json = [](const structured_control_flow::DebugInfo& d) {
+        if (!d.has) return empty_debug_info();
+        Value v;
+        v.set("has", true);
+        v.set("filename", d.filename);
+        v.set("function", d.function);
+        v.set("start_line", (int64_t) d.start_line);
+        v.set("start_column", (int64_t) d.start_column);
+        v.set("end_line", (int64_t) d.end_line);
+        v.set("end_column", (int64_t) d.end_column);
+        return v;
+    };
+    auto transition = [&] {
+        Value t;
+        t.set("type", "transition");
+        t.set("element_id", next());
+        t.set("debug_info", empty_debug_info());
+        t.set("assignments", Value(Array{}));
+        return t;
+    };
+
+    Value root;
+    root.set("type", "sequence");
+    root.set("element_id", next());
+    root.set("debug_info", empty_debug_info());
+    Array children, transitions;
+    for (auto& blk : sdfg.blocks()) {
+        Value b;
+        b.set("type", "block");
+        b.set("element_id", next());
+        b.set("debug_info", debug_json(blk.debug_info));
+        Array nodes, edges;
+        Value lib;
+        const int64_t lib_id = next();
+        lib.set("element_id", lib_id);
+        lib.set("debug_info", debug_json(blk.debug_info));
+        lib.set("type", "library_node");
+        lib.set("implementation_type", blk.node->implementation_type());
+        lib.set("code", blk.node->code());
+        blk.node->to_json(lib);
+        nodes.push_back(std::move(lib));
+        auto edge = [&](int64_t src, const std::string& src_conn, int64_t dst, const std::string& dst_conn, Value base_type) {
+            Value e;
+            e.set("element_id", next());
+            e.set("debug_info", empty_debug_info());
+            e.set("src", src);
+            e.set("dst", dst);
+            e.set("src_conn", src_conn);
+            e.set("dst_conn", dst_conn);
+            e.set("subset", Value(Array{}));
+            e.set("base_type", std::move(base_type));
+            edges.push_back(std::move(e));
+        };
+        for (auto& in : blk.inputs) {
+            Value n;
+            const int64_t id = next();
+            n.set("element_id", id);
+            n.set("debug_info", empty_debug_info());
+            if (in.is_constant) {
+                n.set("type", "constant_node");
+                n.set("data", in.data);
+                n.set("data_type", scalar_json(in.type, plain_storage()));
+                nodes.push_back(std::move(n));
+                edge(id, "void", lib_id, in.connector, scalar_json(in.type, plain_storage()));
+            } else {
+                n.set("type", "access_node");
+                n.set("data", in.data);
+                nodes.push_back(std::move(n));
+                edge(id, "void", lib_id, in.connector, type_json(sdfg.container(in.data)));
+            }
+        }
+        for (auto& out : blk.outputs) {
+            Value n;
+            const int64_t id = next();
+            n.set("element_id", id);
+            n.set("debug_info", empty_debug_info());
+            n.set("type", "access_node");
+            n.set("data", out.data);
+            nodes.push_back(std::move(n));
+            edge(lib_id, out.connector, id, "void", type_json(sdfg.container(out.data)));
+        }
+        Value df;
+        df.set("type", "dataflow");
+        df.set("nodes", Value(std::move(nodes)));
+        df.set("edges", Value(std::move(edges)));
+        b.set("dataflow", std::move(df));
+        children.push_back(std::move(b));
+        transitions.push_back(transition());
+    }
+    {
+        // the reference's front end closes every function with a return node
+        Value r;
+        r.set("type", "return");
+        r.set("element_id", next());
+        r.set("data", sdfg.return_container());
+        r.set("debug_info", empty_debug_info());
+        children.push_back(std::move(r));
+        transitions.push_back(transition());
+    }
+    root.set("children", Value(std::move(children)));
+    root.set("transitions", Value(std::move(transitions)));
+    j.set("root", std::move(root));
+    j.set("element_counter", (int64_t) counter);
+    return j;
+}
+
+} // namespace sdfg::serializer

@@ -439,6 +439,13 @@ using Function = StructuredSDFG;
 
 namespace serializer {
 
+// The reference's own wire format (sdfg/src/serializer/json_serializer.cpp:56-353), see interchange.cpp.
+bool is_reference_format(const json::Value& j);
+// -> the block-list JSON that StructuredSDFG::from_json reads; throws InvalidSDFGException naming the
+// element that has no lowering on the rocm target
+json::Value import_reference_json(const json::Value& j);
+json::Value export_reference_json(const StructuredSDFG& sdfg);
+
 // reference: sdfg/include/sdfg/serializer/json_serializer.h (LibraryNodeSerializerRegistry)
 using LibraryNodeDeserializeFn = std::unique_ptr<data_flow::LibraryNode> (*)(const json::Value&);
 

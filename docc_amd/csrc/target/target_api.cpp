@@ -34,7 +34,10 @@ char* guarded(F&& fn) {
 std::unique_ptr<StructuredSDFG> parse(const char* text) {
     if (!text) throw std::invalid_argument("null SDFG text");
     rocm::register_rocm_plugin();
-    auto sdfg = StructuredSDFG::from_json(json::Value::parse(text));
+    json::Value j = json::Value::parse(text);
+    // SDFGs written by the reference's own serializer are accepted wherever an SDFG is
+    if (serializer::is_reference_format(j)) j = serializer::import_reference_json(j);
+    auto sdfg = StructuredSDFG::from_json(j);
     sdfg->validate();
     return sdfg;
 }
@@ -102,6 +105,22 @@ char* docc_rocm_target_dispatcher_keys(void) {
 
 char* docc_rocm_target_validate(const char* sdfg_json) {
     return guarded([&] { return parse(sdfg_json)->to_json().dump(2); });
+}
+
+char* docc_rocm_target_import(const char* docc_json) {
+    return guarded([&] {
+        if (!docc_json) throw std::invalid_argument("null SDFG text");
+        rocm::register_rocm_plugin();
+        json::Value j = json::Value::parse(docc_json);
+        if (!serializer::is_reference_format(j)) throw InvalidSDFGException("not in docc's SDFG JSON format (no \"element_counter\")");
+        auto sdfg = StructuredSDFG::from_json(serializer::import_reference_json(j));
+        sdfg->validate();
+        return sdfg->to_json().dump(2);
+    });
+}
+
+char* docc_rocm_target_export(const char* sdfg_json) {
+    return guarded([&] { return serializer::export_reference_json(*parse(sdfg_json)).dump(2); });
 }
 
 char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, const char* options_json) {

@@ -29,6 +29,7 @@ EXPORTED_SYMBOLS = (
     "docc_rocm_target_register", "docc_rocm_target_dispatcher_keys", "docc_rocm_target_validate",
     "docc_rocm_target_schedule", "docc_rocm_target_generate", "docc_rocm_target_compile",
     "docc_rocm_target_report", "docc_rocm_target_free", "docc_rocm_target_last_error",
+    "docc_rocm_target_import", "docc_rocm_target_export",
 )
 
 
@@ -45,7 +46,8 @@ def _native() -> ctypes.CDLL:
         cp = ctypes.c_char_p
         lib.docc_rocm_target_register.restype = ctypes.c_int
         for name, args in (("docc_rocm_target_dispatcher_keys", []), ("docc_rocm_target_validate", [cp]),
-                           ("docc_rocm_target_schedule", [cp, cp, cp]), ("docc_rocm_target_generate", [cp, cp, cp]),
+                           ("docc_rocm_target_schedule", [cp, cp, cp]),
+                           ("docc_rocm_target_import", [cp]), ("docc_rocm_target_export", [cp]), ("docc_rocm_target_generate", [cp, cp, cp]),
                            ("docc_rocm_target_compile", [cp, cp, cp, cp, cp]), ("docc_rocm_target_report", [cp])):
             fn = getattr(lib, name)
             fn.argtypes = args
@@ -131,7 +133,19 @@ class StructuredSDFG:
     # -- construction ---------------------------------------------------------
     @staticmethod
     def parse(text: str) -> "StructuredSDFG":
+        """Parses and validates an SDFG, in this package's JSON format or in the one docc's own
+        serializer writes (StructuredSDFG.dump of a docc install)."""
         return StructuredSDFG(json.loads(_call("docc_rocm_target_validate", text)))
+
+    @staticmethod
+    def from_docc_json(text: str) -> "StructuredSDFG":
+        """Imports an SDFG written by docc (reference sdfg/src/serializer/json_serializer.cpp:56-353).
+        Raises InvalidSDFGException naming the first element the rocm target has no lowering for."""
+        return StructuredSDFG(json.loads(_call("docc_rocm_target_import", text)))
+
+    def to_docc_json(self) -> str:
+        """This SDFG in docc's JSON format."""
+        return _call("docc_rocm_target_export", self.to_json())
 
     @staticmethod
     def from_file(path: str) -> "StructuredSDFG":

@@ -34,6 +34,19 @@ char* docc_rocm_target_dispatcher_keys(void);
  * StructuredSDFG.parse + validate (reference bindings.cpp:136-160). */
 char* docc_rocm_target_validate(const char* sdfg_json);
 
+/* Reads an SDFG in docc's own JSON format - what StructuredSDFG.dump / JSONSerializer::serialize
+ * write (reference sdfg/src/serializer/json_serializer.cpp:56-353, python/bindings/py_structured_sdfg.cpp:263-292) -
+ * and returns it in this library's format. Accepted: a root sequence of blocks with one library node
+ * each (GEMM and the ml:: nodes of this target, with their access and constant nodes), Malloc / Free
+ * nodes and managed storage for temporaries, a final return. Anything else (loop nests, tasklets,
+ * branches, views) is an error that names the element. Every other entry point of this header accepts
+ * both formats. */
+char* docc_rocm_target_import(const char* docc_json);
+
+/* The reverse: an SDFG of this library in docc's JSON format (blocks with library / access /
+ * constant nodes and edges, transitions, a closing return node, element ids renumbered). */
+char* docc_rocm_target_export(const char* sdfg_json);
+
 /* Runs the rocm scheduling passes (node mapping, offloading, transfer minimisation) and
  * returns the scheduled SDFG. `options_json` may be NULL or an object with
  * "offload": "function" | "node" | "none" and "require_all_mapped": bool.

@@ -263,3 +263,28 @@ def test_instrumented_program_writes_a_trace_with_device_times(tmp_path, mode):
     # a GEMM of this size takes well under 10 ms on the device; a region's time is a device time, not the process's
     gemm = [e for e in kinds["math"] if e["name"].startswith("dense") and (e["args"]["metrics"].get("static:::flop") is not None)]
     assert gemm and min(e["dur"] / (3 if mode == "aggregate" else 1) for e in gemm) < 10000
+
+
+def test_program_in_docc_json_format_runs(tmp_path):
+    """An SDFG in the layout docc's serializer writes (two chained GEMMs with a Malloc'ed temporary) is
+    imported, scheduled, compiled and run: C = 1.5 * (A @ B) @ B + 0.5 * C."""
+    import ctypes
+    import json
+
+    from docc_amd import runtime
+    from docc_amd.sdfg import StructuredSDFG
+    from test_interchange import gemm_program
+
+    s = StructuredSDFG.parse(json.dumps(gemm_program()))
+    s.schedule("rocm")
+    lib = ctypes.CDLL(s._compile(str(tmp_path)))
+    fn = lib.two_mm_sdfg
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    fn.restype = None
+    rng = np.random.default_rng(2)
+    n = 150
+    A, B, C = rng.random((n, n)), rng.random((n, n)), rng.random((n, n))
+    ref = oracle.gemm(oracle.gemm(A, B), B, C, alpha=1.5, beta=0.5)
+    fn(A.ctypes.data, B.ctypes.data, C.ctypes.data, n)
+    assert runtime.take_failure() == (0, "")
+    assert rel_err_max(C, ref) <= 1e-12

@@ -1,0 +1,216 @@
+"""SDFG JSON interchange with docc's own serializer (reference sdfg/src/serializer/json_serializer.cpp:56-353).
+
+`tests/golden/docc_tiled_matmul_sdfg.json` is a data file of the reference (examples/input/transfertuning/
+matmul_sdfg.json, minified): a tiled matmul loop nest written by docc's serializer. It pins the envelope,
+the type encoding (primitive type numbers, pointer -> array -> scalar) and the dataflow node / edge layout.
+The library-node programs below are written by hand in the same layout, following what
+PyStructuredSDFGBuilder::add_gemm builds (python/bindings/builder/py_structured_sdfg_builder.cpp:654-774: an
+empty view block, one access node per edge, C bound as input and output, constants for alpha / beta) and
+the node serializers (gemm_node.cpp:387-405, malloc.cpp:43-53)."""
+import copy
+import json
+import re
+from pathlib import Path
+
+import pytest
+
+from docc_amd.sdfg import InvalidSDFGException, Pointer, PrimitiveType, Scalar, StructuredSDFG, StructuredSDFGBuilder
+
+GOLDEN = Path(__file__).parent / "golden" / "docc_tiled_matmul_sdfg.json"
+NO_DEBUG = {"has": False, "filename": "", "function": "", "start_line": 0, "start_column": 0, "end_line": 0, "end_column": 0}
+STACK = {"value": "CPU_Stack", "allocation": 0, "deallocation": 0}
+FLOAT, DOUBLE, INT64 = 14, 15, 5
+
+
+def scalar(prim):
+    return {"type": "scalar", "primitive_type": prim, "storage_type": STACK, "initializer": "", "alignment": 0}
+
+
+def pointer(prim):
+    return {"type": "pointer", "pointee_type": scalar(prim), "storage_type": STACK, "initializer": "", "alignment": 0}
+
+
+class Ids:
+    def __init__(self):
+        self.n = 0
+
+    def __call__(self):
+        self.n += 1
+        return self.n
+
+
+def docc_block(ids, lib, inputs, outputs, containers, debug=None):
+    """One block as docc serialises it: the library node, one access / constant node per edge."""
+    lib = {"element_id": ids(), "debug_info": debug or NO_DEBUG, "type": "library_node", **lib}
+    nodes, edges = [lib], []
+    for conn, value in inputs:
+        nid = ids()
+        if isinstance(value, tuple):      # (literal, primitive type): a constant node
+            nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "constant_node", "data": value[0], "data_type": scalar(value[1])})
+            base = scalar(value[1])
+        else:
+            nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "access_node", "data": value})
+            base = containers[value]
+        edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": nid, "dst": lib["element_id"], "src_conn": "void",
+                      "dst_conn": conn, "subset": [], "base_type": base})
+    for conn, name in outputs:
+        nid = ids()
+        nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "access_node", "data": name})
+        edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": lib["element_id"], "dst": nid, "src_conn": conn,
+                      "dst_conn": "void", "subset": [], "base_type": containers[name]})
+    return {"type": "block", "element_id": ids(), "debug_info": debug or NO_DEBUG,
+            "dataflow": {"type": "dataflow", "nodes": nodes, "edges": edges}}
+
+
+def docc_sdfg(name, containers, arguments, children, ids):
+    transitions = [{"type": "transition", "element_id": ids(), "debug_info": NO_DEBUG, "assignments": []} for _ in children]
+    return {"name": name, "element_counter": ids.n + 1, "type": "CPU", "return_type": scalar(0), "structures": [],
+            "containers": containers, "arguments": arguments, "externals": [], "metadata": {"sdfg_file": "/tmp/x.json"},
+            "root": {"type": "sequence", "element_id": ids(), "debug_info": NO_DEBUG, "children": children, "transitions": transitions}}
+
+
+def gemm_program():
+    """T = A @ B (temporary from Malloc), C = 1.5 * T @ B + 0.5 * C, Free(T), return."""
+    ids = Ids()
+    containers = {n: pointer(DOUBLE) for n in ("A", "B", "C", "_tmp_0")}
+    containers["_s0"] = scalar(INT64)
+    gemm = {"implementation_type": "BLAS", "code": "GEMM", "precision": ord("d"), "layout": 101, "trans_a": 111, "trans_b": 111,
+            "m": "_s0", "n": "_s0", "k": "_s0", "lda": "_s0", "ldb": "_s0", "ldc": "_s0"}
+    dbg = {"has": True, "filename": "/home/u/prog.py", "function": "two_mm", "start_line": 7, "start_column": 4, "end_line": 7, "end_column": 20}
+    children = [
+        docc_block(ids, {"implementation_type": "NONE", "code": "Malloc", "size": "8*_s0**2"}, [], [("_ret", "_tmp_0")], containers),
+        {"type": "block", "element_id": ids(), "debug_info": NO_DEBUG, "dataflow": {"type": "dataflow", "nodes": [], "edges": []}},
+        docc_block(ids, gemm, [("__A", "A"), ("__B", "B"), ("__C", "_tmp_0"), ("__alpha", ("1.0", DOUBLE)), ("__beta", ("0.0", DOUBLE))],
+                   [("__C", "_tmp_0")], containers, dbg),
+        docc_block(ids, gemm, [("__A", "_tmp_0"), ("__B", "B"), ("__C", "C"), ("__alpha", ("1.5", DOUBLE)), ("__beta", ("0.5", DOUBLE))],
+                   [("__C", "C")], containers),
+        docc_block(ids, {"implementation_type": "NONE", "code": "Free"}, [("_ptr", "_tmp_0")], [("_ptr", "_tmp_0")], containers),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    return docc_sdfg("two_mm_sdfg", containers, ["A", "B", "C", "_s0"], children, ids)
+
+
+def test_reference_data_file_pins_the_envelope_and_type_encoding():
+    data = json.loads(GOLDEN.read_text())
+    # a loop nest has no lowering on this target: the import stops at the first map and says so
+    with pytest.raises(InvalidSDFGException, match=r"map \(element \d+\): control flow other than a sequence of library-node blocks"):
+        StructuredSDFG.from_docc_json(json.dumps(data))
+    # its declarations alone import: arrays behind pointers decay to their element type, type numbers as in docc's enum
+    head = dict(data, root={"type": "sequence", "element_id": 1, "debug_info": NO_DEBUG, "children": [], "transitions": []})
+    s = StructuredSDFG.from_docc_json(json.dumps(head))
+    assert s.name == "sdfg_test" and s.arguments == ["A", "B", "C", "K", "N", "M"]
+    assert s.containers["A"] == {"type": "pointer", "element": "Float", "transient": False, "storage": "CPU"}
+    assert s.containers["i"]["type"] == "scalar" and s.containers["i"]["element"] == "UInt64" and s.containers["K"]["element"] == "UInt64"
+    # a tasklet block on its own is refused with its element named
+    def first_block(n):
+        if n.get("type") == "block":
+            return n
+        for c in n.get("children", []):
+            r = first_block(c)
+            if r:
+                return r
+        return first_block(n["root"]) if "root" in n and n["type"] != "sequence" else None
+    blk = first_block(data["root"])
+    only = dict(data, root={"type": "sequence", "element_id": 1, "debug_info": NO_DEBUG, "children": [blk],
+                            "transitions": [{"type": "transition", "element_id": 2, "debug_info": NO_DEBUG, "assignments": []}]})
+    with pytest.raises(InvalidSDFGException, match=r"tasklet \(element \d+\) in block"):
+        StructuredSDFG.from_docc_json(json.dumps(only))
+
+
+def test_gemm_program_written_like_docc_imports_schedules_and_generates(tmp_path):
+    text = json.dumps(gemm_program())
+    s = StructuredSDFG.from_docc_json(text)
+    assert s.arguments == ["A", "B", "C", "_s0"] and s.metadata("sdfg_file") == "/tmp/x.json"
+    assert s.containers["_tmp_0"] == {"type": "pointer", "element": "Double", "transient": True, "storage": "CPU", "size": "8*(_s0*_s0)"}     # SymEngine's power spelled as C
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["GEMM", "GEMM"]          # Malloc / Free became the transient, the view block vanished
+    assert nodes[0]["implementation_type"] == "BLAS" and nodes[0]["precision"] == ord("d") and nodes[0]["lda"] == "_s0"
+    first = s._data["root"]["children"][0]
+    binds = {b["connector"]: b.get("data", b.get("constant")) for b in first["dataflow"]["inputs"]}
+    assert binds == {"__A": "A", "__B": "B", "__C": "_tmp_0", "__alpha": "1.0", "__beta": "0.0"}
+    assert first["dataflow"]["outputs"] == [{"connector": "__C", "data": "_tmp_0"}]
+    assert first["debug_info"]["function"] == "two_mm" and first["debug_info"]["start_line"] == 7
+    # every entry point takes the docc format directly
+    assert StructuredSDFG.parse(text).library_nodes() == nodes
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 3 and r["D2H"] == 1            # A, B, C up (beta != 0 reads C); C down; the temporary never leaves the device
+    src = Path(s.generate(str(tmp_path))["source"]).read_text()
+    assert src.count("docc_rocm_dgemm(") == 2 and 'extern "C" void two_mm_sdfg(double *A, double *B, double *C, int64_t _s0)' in src
+
+
+def test_import_refuses_what_it_cannot_lower():
+    base = gemm_program()
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][2]["dataflow"]["edges"][0]["subset"] = ["_s0"]
+    with pytest.raises(InvalidSDFGException, match="subset on an operand of GEMM"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    bad = copy.deepcopy(base)
+    bad["root"]["transitions"][0]["assignments"] = [{"symbol": "i", "expression": "0"}]
+    with pytest.raises(InvalidSDFGException, match="symbol assignments"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    bad = copy.deepcopy(base)
+    bad["containers"]["A"]["storage_type"] = {"value": "NV_Generic", "allocation": 0, "deallocation": 0}
+    with pytest.raises(InvalidSDFGException, match="NV_Generic belongs to another target"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][2]["dataflow"]["nodes"][0]["code"] = "Memcpy"
+    with pytest.raises(InvalidSDFGException, match="No library node serializer found for Memcpy"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["dataflow"]["nodes"][0]["size"] = "8*_s0**_s0"
+    with pytest.raises(InvalidSDFGException, match="not a small integer power"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["dataflow"]["nodes"][0]["size"] = "8*(1 + _s0)**3"
+    assert StructuredSDFG.from_docc_json(json.dumps(bad)).containers["_tmp_0"]["size"] == "8*((1 + _s0)*(1 + _s0)*(1 + _s0))"
+    bad = copy.deepcopy(base)
+    bad["root"]["children"].append({"type": "break", "element_id": 999, "debug_info": NO_DEBUG})
+    with pytest.raises(InvalidSDFGException, match="code after the return"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    with pytest.raises(InvalidSDFGException, match="element_counter"):
+        StructuredSDFG.from_docc_json(StructuredSDFGBuilder("x").move().to_json())
+
+
+def test_export_writes_docc_layout_and_round_trips():
+    F32 = Pointer(Scalar(PrimitiveType.Float))
+    b = StructuredSDFGBuilder("dense")
+    for n in ("X", "W", "bias", "Y"):
+        b.add_container(n, F32, True)
+    for n in ("T0", "T1", "T2"):
+        b.add_container(n, F32, False, transient_bytes=32 * 16 * 4)
+    b.set_debug_info("/src/m.py", "dense", 3, 5, 3, 30)
+    b.add_gemm("X", "W", "T0", "1.0", "0.0", 32, 16, 8)
+    b.add_broadcast("bias", "T1", [1, 16], [32, 16])
+    b.add_elementwise_op("add", "T0", "T1", "T2", [32, 16])
+    b.add_reduce_op("softmax", "T2", "T0", [32, 16], [-1])
+    b.add_elementwise_op("mul", "T0", "0.5", "Y", [32, 16])
+    s = b.move()
+    d = json.loads(s.to_docc_json())
+    # the keys JSONSerializer::serialize writes, in a shape its deserialize accepts
+    assert set(d) == {"name", "element_counter", "type", "return_type", "structures", "containers", "arguments", "externals", "metadata", "root"}
+    assert d["type"] == "CPU" and d["return_type"]["primitive_type"] == 0 and d["arguments"] == ["X", "W", "bias", "Y"]
+    assert d["containers"]["X"]["pointee_type"]["primitive_type"] == FLOAT
+    t0 = d["containers"]["T0"]["storage_type"]
+    assert t0 == {"value": "CPU_Heap", "allocation": 1, "deallocation": 1, "allocation_size": "2048"}
+    root = d["root"]
+    assert root["type"] == "sequence" and len(root["children"]) == len(root["transitions"]) == 6 and root["children"][-1]["type"] == "return"
+    ids = re.findall(r'"element_id": (\d+)', json.dumps(d))
+    assert len(ids) == len(set(ids)) and max(map(int, ids)) == d["element_counter"]
+    blk = root["children"][0]
+    assert set(blk) == {"type", "element_id", "debug_info", "dataflow"} and blk["debug_info"]["start_line"] == 3
+    kinds = [n["type"] for n in blk["dataflow"]["nodes"]]
+    assert kinds == ["library_node", "access_node", "access_node", "access_node", "constant_node", "constant_node", "access_node"]
+    lib = blk["dataflow"]["nodes"][0]
+    assert lib["code"] == "GEMM" and lib["implementation_type"] == "BLAS" and lib["precision"] == ord("s") and lib["m"] == "32"
+    edge = blk["dataflow"]["edges"][0]
+    assert set(edge) == {"element_id", "debug_info", "src", "dst", "src_conn", "dst_conn", "subset", "base_type"}
+    assert edge["dst"] == lib["element_id"] and edge["dst_conn"] == "__A" and edge["src_conn"] == "void" and edge["subset"] == []
+    # and back
+    again = StructuredSDFG.from_docc_json(json.dumps(d))
+    strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]
+    assert strip(again.library_nodes()) == strip(s.library_nodes())
+    assert again.containers == s.containers and again.arguments == s.arguments
+    for a, b2 in zip(again._data["root"]["children"], s._data["root"]["children"]):
+        assert a["dataflow"]["inputs"] == b2["dataflow"]["inputs"] and a["dataflow"]["outputs"] == b2["dataflow"]["outputs"]
+        assert a.get("debug_info") == b2.get("debug_info")
