@@ -283,7 +283,10 @@ def main():
         cases = {"add_f32": (12 * n, lambda i: rt.elementwise_binary("add", 32, n, a.data_ptr(), b2.data_ptr(), y.data_ptr(), stream)),
                  "relu_f32": (8 * n, lambda i: rt.elementwise_unary("relu", 32, n, a.data_ptr(), y.data_ptr(), stream)),
                  "sigmoid_f32": (8 * n, lambda i: rt.elementwise_unary("sigmoid", 32, n, a.data_ptr(), y.data_ptr(), stream)),
-                 "broadcast_row_f32": (4 * n + 4 * 4096, lambda i: rt.broadcast(32, (1, 4096), (8192, 4096), a.data_ptr(), y.data_ptr(), stream))}
+                 "broadcast_row_f32": (4 * n + 4 * 4096, lambda i: rt.broadcast(32, (1, 4096), (8192, 4096), a.data_ptr(), y.data_ptr(), stream)),
+                 # relu(a + bias row): what the fusion pass makes of Broadcast + Add + ReLU (28 B/element as three nodes)
+                 "fused_bias_relu_f32": (8 * n + 4 * 4096, lambda i: rt.elementwise_fused(32, (8192, 4096), "add", a.data_ptr(), (8192, 4096),
+                                                                                        b2.data_ptr(), (4096,), ["relu"], y.data_ptr(), stream))}
         for name, (nbytes_e, fn) in cases.items():
             ms = time_kernel(fn, 50, 5)
             gbs = nbytes_e / ms / 1e6

@@ -167,6 +167,106 @@ __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const Broadca
     }
 }
 
+// Fused chain: Y = post_k(...post_1(f(A', B'))), where A' and B' are A and B repeated to the
+// output shape by numpy's rules (or a scalar), f one of the binary operations (or absent: the
+// chain starts from A'), and post_i unary operations. It stands for a Broadcast node folded into
+// its consumer and for unary nodes folded into their producer: one pass over memory instead of
+// one per node. The operation codes are uniform over the launch, so the switches below are
+// scalar branches.
+struct FusedParams {
+    long n;                 // elements of the output
+    int rank;               // collapsed by the launcher
+    long dims[6];
+    long a_strides[6];      // in elements, 0 where the operand repeats
+    long b_strides[6];
+    int binary;             // BinaryOp or -1
+    int a_scalar, b_scalar; // operand is the scalar below instead of an array
+    double scalar_a, scalar_b;
+    int npost;
+    int post[4];            // UnaryOp codes
+};
+
+template <typename T>
+__device__ __forceinline__ T fused_unary(int op, T x) {
+    switch (op) {
+        case kAbs: return unary<kAbs>(x);
+        case kExp: return unary<kExp>(x);
+        case kReLU: return unary<kReLU>(x);
+        case kSigmoid: return unary<kSigmoid>(x);
+        case kSqrt: return unary<kSqrt>(x);
+        case kTanh: return unary<kTanh>(x);
+        default: return unary<kErf>(x);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ T fused_binary(int op, T a, T b) {
+    switch (op) {
+        case kAdd: return binary<kAdd>(a, b);
+        case kSub: return binary<kSub>(a, b);
+        case kMul: return binary<kMul>(a, b);
+        case kDiv: return binary<kDiv>(a, b);
+        case kMaximum: return binary<kMaximum>(a, b);
+        default: return binary<kMinimum>(a, b);
+    }
+}
+
+template <typename T, int VEC, typename I>
+__device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const FusedParams& p) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    const I stride = (I) gridDim.x * blockDim.x;
+    const I nv = (I) (p.n / VEC);
+    const int last = p.rank - 1;
+    const I inner = (I) p.dims[last] / VEC;
+    const bool a_inner = !p.a_scalar && p.a_strides[last] != 0, b_inner = !p.b_scalar && p.b_strides[last] != 0;
+    const bool has_b = p.binary >= 0;
+    for (I v = (I) blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += stride) {
+        I rem = v / inner;
+        const long in = (long) (v % inner) * VEC;
+        long oa = a_inner ? in : 0, ob = b_inner ? in : 0;
+#pragma unroll
+        for (int d = 4; d >= 0; d--) {
+            if (d < last) {
+                const I e = (I) p.dims[d];
+                const long c = (long) (rem % e);
+                rem /= e;
+                oa += c * p.a_strides[d];
+                ob += c * p.b_strides[d];
+            }
+        }
+        V a, b;
+        if (p.a_scalar) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = (T) p.scalar_a;
+        } else if (a_inner) {
+            a = __builtin_nontemporal_load(reinterpret_cast<const V*>(A + oa));
+        } else {
+            const T x = A[oa];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = x;
+        }
+        if (has_b) {
+            if (p.b_scalar) {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) b[e] = (T) p.scalar_b;
+            } else if (b_inner) {
+                b = __builtin_nontemporal_load(reinterpret_cast<const V*>(B + ob));
+            } else {
+                const T x = B[ob];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) b[e] = x;
+            }
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = fused_binary<T>(p.binary, a[e], b[e]);
+        }
+        for (int k = 0; k < p.npost; k++) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = fused_unary<T>(p.post[k], a[e]);
+        }
+        __builtin_nontemporal_store(a, reinterpret_cast<V*>(Y) + v);
+    }
+}
+
 } // namespace docc_k
 
 #define DOCC_EW_UNARY(NAME, OP)                                                                                              \
@@ -224,3 +324,17 @@ DOCC_BROADCAST(f64_v2_i32, double, 2, unsigned)
 DOCC_BROADCAST(f64_v1_i32, double, 1, unsigned)
 DOCC_BROADCAST(f64_v2_i64, double, 2, long)
 DOCC_BROADCAST(f64_v1_i64, double, 1, long)
+
+#define DOCC_EW_FUSED(NAME, T, VEC, I)                                                                                      \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_##NAME(const T* A, const T* B, T* Y,                       \
+                                                                           docc_k::FusedParams p) {                         \
+        docc_k::fused_kernel<T, VEC, I>(A, B, Y, p);                                                                        \
+    }
+DOCC_EW_FUSED(f32_v4_i32, float, 4, unsigned)
+DOCC_EW_FUSED(f32_v1_i32, float, 1, unsigned)
+DOCC_EW_FUSED(f32_v4_i64, float, 4, long)
+DOCC_EW_FUSED(f32_v1_i64, float, 1, long)
+DOCC_EW_FUSED(f64_v2_i32, double, 2, unsigned)
+DOCC_EW_FUSED(f64_v1_i32, double, 1, unsigned)
+DOCC_EW_FUSED(f64_v2_i64, double, 2, long)
+DOCC_EW_FUSED(f64_v1_i64, double, 1, long)

@@ -29,6 +29,33 @@ struct BroadcastParams {
     long in_strides[6];
 };
 
+// mirrors docc_k::FusedParams (csrc/kernels/elementwise.hip)
+struct FusedParams {
+    long n;
+    int rank;
+    long dims[6];
+    long a_strides[6];
+    long b_strides[6];
+    int binary;
+    int a_scalar, b_scalar;
+    double scalar_a, scalar_b;
+    int npost;
+    int post[4];
+};
+
+// element strides of an operand of shape `in` (extent 1 repeats) inside the output shape
+int operand_strides(const char* what, int rank, const int64_t* in, const int64_t* out, long* strides) {
+    long stride = 1;
+    for (int d = rank - 1; d >= 0; d--) {
+        if (in[d] != out[d] && in[d] != 1)
+            return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: dimension %d has extent %lld, cannot become %lld", what, d,
+                        (long long) in[d], (long long) out[d]);
+        strides[d] = in[d] == 1 ? 0 : stride;
+        stride *= (long) in[d];
+    }
+    return 0;
+}
+
 int check_precision(const char* what, int precision) {
     if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: precision must be 32 or 64", what);
     return 0;
@@ -138,4 +165,75 @@ extern "C" int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int
     char name[64];
     std::snprintf(name, sizeof(name), "docc_broadcast_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
     return launch(name, grid_for(n / lanes), 1, 1, 256, 0, (hipStream_t) stream, X, Y, p);
+}
+
+extern "C" int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precision, int rank, const int64_t* shape, int binary_op,
+                                           const int64_t* a_shape, const void* A, double a_scalar, const int64_t* b_shape,
+                                           const void* B, double b_scalar, int n_post, const int* post_ops, void* Y) {
+    const char* what = "elementwise_fused";
+    if (int rc = check_precision(what, precision)) return rc;
+    if (rank < 1 || rank > 6) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: rank %d (1..6 are built)", what, rank);
+    if (!shape) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null shape", what);
+    const int n_binary = (int) (sizeof(kBinaryNames) / sizeof(kBinaryNames[0])), n_unary = (int) (sizeof(kUnaryNames) / sizeof(kUnaryNames[0]));
+    if (binary_op < -1 || binary_op >= n_binary) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: unknown binary operation %d", what, binary_op);
+    if (n_post < 0 || n_post > 4) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: %d unary operations (up to 4)", what, n_post);
+    if (n_post > 0 && !post_ops) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null operation list", what);
+    FusedParams p{};
+    for (int k = 0; k < n_post; k++) {
+        if (post_ops[k] < 0 || post_ops[k] >= n_unary) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: unknown unary operation %d", what, post_ops[k]);
+        p.post[k] = post_ops[k];
+    }
+    p.npost = n_post;
+    p.binary = binary_op;
+    const bool has_b = binary_op >= 0;
+    p.a_scalar = a_shape == nullptr;
+    p.b_scalar = has_b && b_shape == nullptr;
+    p.scalar_a = a_scalar;
+    p.scalar_b = b_scalar;
+    if (p.a_scalar && (!has_b || p.b_scalar)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: no array operand", what);
+    long dims[6], sa[6] = {0}, sb[6] = {0};
+    long n = 1;
+    for (int d = 0; d < rank; d++) {
+        if (shape[d] < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: negative extent", what);
+        dims[d] = (long) shape[d];
+        n *= dims[d];
+    }
+    if (!p.a_scalar)
+        if (int rc = operand_strides(what, rank, a_shape, shape, sa)) return rc;
+    if (has_b && !p.b_scalar)
+        if (int rc = operand_strides(what, rank, b_shape, shape, sb)) return rc;
+    if (n == 0) return 0;
+    if (!Y || (!p.a_scalar && !A) || (has_b && !p.b_scalar && !B)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null pointer", what);
+    if (int rc = ensure_device()) return rc;
+    // collapse: drop extent-1 dimensions; merge neighbours that are contiguous (or repeated) in both operands
+    int r = 0;
+    for (int d = 0; d < rank; d++) {
+        if (dims[d] == 1) continue;
+        if (r > 0 && p.a_strides[r - 1] == sa[d] * dims[d] && p.b_strides[r - 1] == sb[d] * dims[d]) {
+            p.dims[r - 1] *= dims[d];
+            p.a_strides[r - 1] = sa[d];
+            p.b_strides[r - 1] = sb[d];
+        } else {
+            p.dims[r] = dims[d];
+            p.a_strides[r] = sa[d];
+            p.b_strides[r] = sb[d];
+            r++;
+        }
+    }
+    if (r == 0) {
+        p.dims[0] = 1;
+        r = 1;
+    }
+    p.rank = r;
+    p.n = n;
+    const int per_vec = precision == 32 ? 4 : 2;
+    auto vector_ok = [&](bool scalar, const void* ptr, long inner_stride) {
+        return scalar || inner_stride == 0 || (inner_stride == 1 && (uintptr_t) ptr % 16 == 0);
+    };
+    const bool vec = p.dims[r - 1] % per_vec == 0 && (uintptr_t) Y % 16 == 0 && vector_ok(p.a_scalar, A, p.a_strides[r - 1]) &&
+                     (!has_b || vector_ok(p.b_scalar, B, p.b_strides[r - 1]));
+    const int lanes = vec ? per_vec : 1;
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_ew_fused_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
+    return launch(name, grid_for(n / lanes), 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, p);
 }

@@ -401,6 +401,69 @@ protected:
     }
 };
 
+// ---- fused elementwise chain ---------------------------------------------------------------
+
+class FusedElementWiseDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    const ROCMFusedElementWiseNode& fused() const { return static_cast<const ROCMFusedElementWiseNode&>(node_); }
+
+    std::vector<DeviceOperand> operands() const override {
+        std::vector<DeviceOperand> ops;
+        if (!fused().a_shape().empty()) ops.push_back(operand("A", true, false));
+        if (fused().has_b() && !fused().b_shape().empty()) ops.push_back(operand("B", true, false));
+        ops.push_back(operand("Y", false, true));
+        return ops;
+    }
+
+    static int index_of(const std::vector<std::string>& codes, const std::string& code) {
+        for (size_t i = 0; i < codes.size(); i++)
+            if (codes[i] == code) return (int) i;
+        return -1;
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = fused();
+        const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        auto list = [&](const char* name, const std::vector<Expression>& shape) {
+            s << "const int64_t " << name << "[] = {";
+            for (size_t i = 0; i < shape.size(); i++) s << (i ? ", " : "") << "(int64_t) (" << shape[i] << ")";
+            s << "};" << std::endl;
+        };
+        list("__docc_shape", n.shape());
+        const bool a_array = !n.a_shape().empty(), b_array = n.has_b() && !n.b_shape().empty();
+        if (a_array) list("__docc_a_shape", n.a_shape());
+        if (b_array) list("__docc_b_shape", n.b_shape());
+        s << "const int __docc_post[] = {";
+        for (size_t i = 0; i < n.post().size(); i++)
+            s << (i ? ", " : "") << index_of(tensor::UnaryNodeCodes, n.post()[i]) << " /* " << n.post()[i] << " */";
+        if (n.post().empty()) s << "0";
+        s << "};" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_elementwise_fused(nullptr, " << precision << ", " << n.shape().size() << ", __docc_shape, ";
+        if (n.has_b())
+            s << index_of(tensor::BinaryNodeCodes, n.binary()) << " /* " << n.binary() << " */, ";
+        else
+            s << "-1, ";
+        if (a_array)
+            s << "__docc_a_shape, " << name_of("A") << ", 0.0, ";
+        else
+            s << "nullptr, nullptr, (double) A, ";
+        if (b_array)
+            s << "__docc_b_shape, " << name_of("B") << ", 0.0, ";
+        else if (n.has_b())
+            s << "nullptr, nullptr, (double) B, ";
+        else
+            s << "nullptr, nullptr, 0.0, ";
+        s << n.post().size() << ", __docc_post, " << name_of("Y") << "));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+};
+
 template <typename D>
 void register_math(codegen::LibraryNodeDispatcherRegistry& reg, const std::string& code) {
     for (bool with : {true, false}) {
@@ -431,6 +494,7 @@ void register_plugin(plugins::Context& context) {
     for (auto& code : tensor::UnaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
+    register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
     reg.register_library_node_dispatcher(
         LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
         [](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
@@ -501,6 +565,159 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
     }
     node.implementation_type() = implementation_type_;
     return true;
+}
+
+// ---------------------------------------------------------------------------------- fusion
+
+namespace {
+
+bool is_rocm_type(const std::string& impl) {
+    return impl == ImplementationType_ROCMWithTransfers || impl == ImplementationType_ROCMWithoutTransfers;
+}
+
+struct Uses {
+    std::vector<size_t> readers, writers;
+};
+
+Uses uses_of(const StructuredSDFG& sdfg, const std::string& name) {
+    Uses u;
+    for (size_t i = 0; i < sdfg.blocks().size(); i++) {
+        const Block& b = sdfg.blocks()[i];
+        for (auto& in : b.inputs)
+            if (!in.is_constant && in.data == name) u.readers.push_back(i);
+        for (auto& out : b.outputs)
+            if (out.data == name) u.writers.push_back(i);
+    }
+    return u;
+}
+
+// an intermediate that exists only to carry a value from block `producer` to block `consumer`
+bool is_private_link(const StructuredSDFG& sdfg, const std::string& name, size_t producer, size_t consumer) {
+    const Container& c = sdfg.container(name);
+    if (c.is_argument || !c.transient || name == sdfg.return_container()) return false;
+    const Uses u = uses_of(sdfg, name);
+    return u.writers.size() == 1 && u.writers[0] == producer && u.readers.size() == 1 && u.readers[0] == consumer && producer < consumer;
+}
+
+// nothing between the two blocks (exclusive) writes `name`
+bool unwritten_between(const StructuredSDFG& sdfg, const std::string& name, size_t from, size_t to) {
+    for (size_t i = from + 1; i < to; i++)
+        for (auto& out : sdfg.blocks()[i].outputs)
+            if (out.data == name) return false;
+    return true;
+}
+
+// nothing between the two blocks (exclusive) reads or writes `name`
+bool untouched_between(const StructuredSDFG& sdfg, const std::string& name, size_t from, size_t to) {
+    for (size_t i = from + 1; i < to; i++) {
+        for (auto& in : sdfg.blocks()[i].inputs)
+            if (!in.is_constant && in.data == name) return false;
+        for (auto& out : sdfg.blocks()[i].outputs)
+            if (out.data == name) return false;
+    }
+    return true;
+}
+
+std::vector<Expression> ones(size_t rank) { return std::vector<Expression>(rank, "1"); }
+
+// Rewrites an elementwise node as the equivalent fused node (no-op for one that already is).
+void make_fused(StructuredSDFG& sdfg, size_t i) {
+    Block& blk = sdfg.blocks()[i];
+    auto* e = dynamic_cast<tensor::ElementWiseNode*>(blk.node.get());
+    if (!e) return;
+    const bool binary = e->is_binary();
+    auto shape_of = [&](const char* connector) -> std::vector<Expression> {
+        const ConnectorBinding* in = blk.input(connector);
+        const bool scalar = in->is_constant || !sdfg.container(in->data).is_pointer;
+        return scalar ? std::vector<Expression>{} : e->shape();
+    };
+    auto node = std::make_unique<ROCMFusedElementWiseNode>(
+        e->implementation_type(), e->shape(), e->element(), binary ? e->code() : "", shape_of(binary ? "A" : "X"),
+        binary ? shape_of("B") : std::vector<Expression>{}, binary ? std::vector<std::string>{} : std::vector<std::string>{e->code()});
+    node->set_element_id(e->element_id());
+    for (auto& in : blk.inputs)
+        if (in.connector == "X") in.connector = "A";
+    for (auto& out : blk.outputs) out.connector = "Y";
+    blk.node = std::move(node);
+}
+
+} // namespace
+
+bool RocmElementwiseFusionPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
+    StructuredSDFG& sdfg = builder.subject();
+    auto& blocks = sdfg.blocks();
+    bool applied = false;
+    bool changed = true;
+    while (changed) {
+        changed = false;
+        // (1) a Broadcast whose result feeds exactly one operand of one later binary node: the node
+        //     reads the small operand itself
+        for (size_t i = 0; i < blocks.size() && !changed; i++) {
+            auto* bc = dynamic_cast<tensor::BroadcastNode*>(blocks[i].node.get());
+            if (!bc || !is_rocm_type(bc->implementation_type())) continue;
+            const std::string link = blocks[i].outputs[0].data, source = blocks[i].inputs[0].data;
+            const Uses u = uses_of(sdfg, link);
+            if (u.readers.size() != 1) continue;
+            const size_t j = u.readers[0];
+            if (!is_private_link(sdfg, link, i, j) || !unwritten_between(sdfg, source, i, j)) continue;
+            auto* consumer = blocks[j].node.get();
+            const bool plain = dynamic_cast<tensor::ElementWiseNode*>(consumer) && static_cast<tensor::ElementWiseNode*>(consumer)->is_binary();
+            auto* fused = dynamic_cast<ROCMFusedElementWiseNode*>(consumer);
+            if (!(plain || (fused && fused->has_b())) || consumer->implementation_type() != bc->implementation_type()) continue;
+            // the consumer must not write the small operand it is about to read in a different order
+            if (blocks[j].outputs[0].data == source) continue;
+            if (plain) make_fused(sdfg, j);
+            auto* f = static_cast<ROCMFusedElementWiseNode*>(blocks[j].node.get());
+            if (f->shape() != bc->output_shape()) continue;
+            const char* connector = blocks[j].input("A")->data == link && !blocks[j].input("A")->is_constant ? "A" : "B";
+            auto node = std::make_unique<ROCMFusedElementWiseNode>(
+                f->implementation_type(), f->shape(), f->element(), f->binary(),
+                std::string(connector) == "A" ? bc->input_shape() : f->a_shape(),
+                std::string(connector) == "B" ? bc->input_shape() : f->b_shape(), f->post());
+            node->set_element_id(f->element_id());
+            blocks[j].node = std::move(node);
+            for (auto& in : blocks[j].inputs)
+                if (in.connector == connector) in.data = source;
+            blocks.erase(blocks.begin() + (long) i);
+            sdfg.remove_container(link);
+            changed = applied = true;
+        }
+        // (2) a unary node on a value that only it reads: an epilogue of the elementwise node that made the value
+        for (size_t j = 0; j < blocks.size() && !changed; j++) {
+            auto* un = dynamic_cast<tensor::ElementWiseNode*>(blocks[j].node.get());
+            if (!un || un->is_binary() || !is_rocm_type(un->implementation_type())) continue;
+            const ConnectorBinding* x = blocks[j].input("X");
+            if (!x || x->is_constant) continue;
+            const std::string link = x->data, result = blocks[j].outputs[0].data;
+            const Uses u = uses_of(sdfg, link);
+            if (u.writers.size() != 1) continue;
+            const size_t i = u.writers[0];
+            if (!is_private_link(sdfg, link, i, j)) continue;
+            auto* producer = blocks[i].node.get();
+            const bool plain = dynamic_cast<tensor::ElementWiseNode*>(producer) != nullptr;
+            auto* fused = dynamic_cast<ROCMFusedElementWiseNode*>(producer);
+            if (!(plain || fused) || producer->implementation_type() != un->implementation_type()) continue;
+            // the result is now written where the producer stands: nothing in between may look at it,
+            // and the producer must not read it through a repeated (out-of-order) operand
+            if (!untouched_between(sdfg, result, i, j)) continue;
+            if (plain) make_fused(sdfg, i);
+            auto* f = static_cast<ROCMFusedElementWiseNode*>(blocks[i].node.get());
+            if (f->post().size() >= 4 || f->shape() != un->shape()) continue;
+            bool aliased_repeat = false;
+            for (auto& in : blocks[i].inputs)
+                if (!in.is_constant && in.data == result) {
+                    const auto& s = in.connector == "A" ? f->a_shape() : f->b_shape();
+                    if (s != f->shape()) aliased_repeat = true;
+                }
+            if (aliased_repeat) continue;
+            f->post().push_back(un->code());
+            blocks[i].outputs[0].data = result;
+            blocks.erase(blocks.begin() + (long) j);
+            sdfg.remove_container(link);
+            changed = applied = true;
+        }
+    }
+    return applied;
 }
 
 // ------------------------------------------------------------------------------ offloading
@@ -713,6 +930,10 @@ void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::A
         if (!mapper->try_map(builder, analysis_manager, *blk.node) && options.require_all_mapped)
             throw InvalidSDFGException("rocm target cannot map node " + mapper->last_decline_reason() +
                                        " (this target has no CPU lowering)");
+    }
+    if (options.fuse_elementwise) {
+        RocmElementwiseFusionPass fusion;
+        fusion.run_pass(builder, analysis_manager);
     }
     if (options.offload == "none") {
         // the caller's pointers are device pointers, so every array the nodes touch lives in HBM:

@@ -57,6 +57,16 @@ public:
     bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
 };
 
+// Folds a Broadcast node into the binary elementwise node that consumes it and unary elementwise
+// nodes into the elementwise node that produces their operand (ROCMFusedElementWise, one kernel
+// per chain), when the value in between is a transient nothing else looks at. Counterpart of
+// the reference's MapFusion over the expanded Maps (python/bindings/py_structured_sdfg.cpp:258-260).
+class RocmElementwiseFusionPass {
+public:
+    std::string name() { return "RocmElementwiseFusion"; }
+    bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
+};
+
 struct ScheduleOptions {
     // "function": nodes run WithoutTransfers between hoisted, minimised transfers (default)
     // "node":     every node copies its operands itself (ROCMWithTransfers)
@@ -64,6 +74,8 @@ struct ScheduleOptions {
     std::string offload = "function";
     // refuse to leave a math node unmapped (there is no CPU lowering in this target)
     bool require_all_mapped = true;
+    // run RocmElementwiseFusionPass after the mapping
+    bool fuse_elementwise = true;
 };
 
 // The scheduling entry of the target: mapping pass (+ offloading passes).

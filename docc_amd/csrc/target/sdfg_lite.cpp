@@ -494,6 +494,62 @@ std::vector<std::string> offload_outputs(DataTransferDirection d, BufferLifecycl
 }
 } // namespace
 
+ROCMFusedElementWiseNode::ROCMFusedElementWiseNode(std::string implementation_type, std::vector<Expression> shape,
+                                                   types::PrimitiveType element, std::string binary, std::vector<Expression> a_shape,
+                                                   std::vector<Expression> b_shape, std::vector<std::string> post)
+    : LibraryNode(LibraryNodeType_ROCM_FusedElementWise, {"Y"},
+                  binary.empty() ? std::vector<std::string>{"A"} : std::vector<std::string>{"A", "B"}, false, std::move(implementation_type)),
+      shape_(std::move(shape)), element_(element), binary_(std::move(binary)), a_shape_(std::move(a_shape)),
+      b_shape_(std::move(b_shape)), post_(std::move(post)) {}
+
+void ROCMFusedElementWiseNode::validate() const {
+    using namespace math::tensor;
+    auto known = [](const std::vector<std::string>& codes, const std::string& c) { return std::find(codes.begin(), codes.end(), c) != codes.end(); };
+    if (shape_.empty() || shape_.size() > 6) throw InvalidSDFGException(code_ + ": rank must be 1..6");
+    if (!binary_.empty() && !known(BinaryNodeCodes, binary_)) throw InvalidSDFGException(code_ + ": unknown binary operation " + binary_);
+    if (post_.size() > 4) throw InvalidSDFGException(code_ + ": more than four unary operations");
+    for (auto& p : post_)
+        if (!known(UnaryNodeCodes, p)) throw InvalidSDFGException(code_ + ": unknown unary operation " + p);
+    for (auto* operand : {&a_shape_, &b_shape_}) {
+        if (operand->empty()) continue;   // scalar
+        if (operand->size() != shape_.size()) throw InvalidSDFGException(code_ + ": operand rank differs from the output rank");
+        for (size_t d = 0; d < shape_.size(); d++)
+            if ((*operand)[d] != shape_[d] && (*operand)[d] != "1")
+                throw InvalidSDFGException(code_ + ": dimension " + std::to_string(d) + " cannot be broadcast");
+    }
+    if (a_shape_.empty() && (binary_.empty() || b_shape_.empty())) throw InvalidSDFGException(code_ + ": no array operand");
+}
+
+Expression ROCMFusedElementWiseNode::flop() const {
+    const size_t ops = (binary_.empty() ? 0 : 1) + post_.size();
+    return symbolic::mul(std::to_string(ops ? ops : 1), product(shape_, 0, shape_.size()));
+}
+
+void ROCMFusedElementWiseNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+    j.set("binary", binary_);
+    j.set("a_shape", exprs_to_json(a_shape_));
+    j.set("b_shape", exprs_to_json(b_shape_));
+    Array post;
+    for (auto& p : post_) post.emplace_back(p);
+    j.set("post", Value(std::move(post)));
+}
+
+std::unique_ptr<ROCMFusedElementWiseNode> ROCMFusedElementWiseNode::from_json(const Value& j) {
+    std::vector<std::string> post;
+    for (auto& p : j.at("post").as_array()) post.push_back(p.as_string());
+    return std::make_unique<ROCMFusedElementWiseNode>(impl_of(j), exprs_from_json(j.at("shape")),
+                                                      types::primitive_type_from_string(j.at("element_type").as_string()),
+                                                      j.at("binary").as_string(), exprs_from_json(j.at("a_shape")),
+                                                      exprs_from_json(j.at("b_shape")), std::move(post));
+}
+
+Expression ROCMFusedElementWiseNode::connector_bytes(const std::string& connector) const {
+    const std::vector<Expression>& s = connector == "A" ? a_shape_ : connector == "B" ? b_shape_ : shape_;
+    return bytes_of(s.empty() ? Expression("1") : product(s, 0, s.size()), element_);
+}
+
 ROCMDataOffloadingNode::ROCMDataOffloadingNode(Expression size, int device_id, DataTransferDirection direction,
                                                BufferLifecycle lifecycle)
     : LibraryNode(LibraryNodeType_ROCM_Offloading, offload_outputs(direction, lifecycle), offload_inputs(direction, lifecycle),
@@ -579,6 +635,18 @@ void StructuredSDFG::add_container(Container c, bool is_argument) {
     c.is_argument = is_argument;
     if (is_argument) arguments_.push_back(c.name);
     containers_.emplace(c.name, std::move(c));
+}
+
+void StructuredSDFG::remove_container(const std::string& name) {
+    const Container& c = container(name);
+    if (c.is_argument || name == return_container_) throw InvalidSDFGException("container '" + name + "' is part of the signature");
+    for (auto& blk : blocks_) {
+        for (auto& in : blk.inputs)
+            if (!in.is_constant && in.data == name) throw InvalidSDFGException("container '" + name + "' is still in use");
+        for (auto& out : blk.outputs)
+            if (out.data == name) throw InvalidSDFGException("container '" + name + "' is still in use");
+    }
+    containers_.erase(name);
 }
 
 structured_control_flow::Block& StructuredSDFG::add_block(std::unique_ptr<data_flow::LibraryNode> node,
@@ -794,6 +862,7 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     for (auto& code : math::tensor::UnaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     for (auto& code : math::tensor::BinaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
+    fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
 }
 
 LibraryNodeSerializerRegistry& LibraryNodeSerializerRegistry::instance() {

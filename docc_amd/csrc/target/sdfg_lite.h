@@ -365,6 +365,42 @@ private:
     BufferLifecycle lifecycle_;
 };
 
+// A chain of elementwise nodes run as one kernel: Y = post_k(...post_1(binary(A', B'))), A' and
+// B' the operands repeated to `shape` (or scalars). Written only by the target's fusion pass, in
+// place of a Broadcast node folded into its consumer and of unary nodes folded into their
+// producer; the reference fuses the expanded Maps instead (py_structured_sdfg.cpp:258-260).
+// connectors: in "A" [, "B"], out "Y". JSON keys: shape, element_type, binary ("" = none),
+// a_shape / b_shape ([] = scalar operand), post.
+inline const std::string LibraryNodeType_ROCM_FusedElementWise = "ROCMFusedElementWise";
+
+class ROCMFusedElementWiseNode : public data_flow::LibraryNode {
+public:
+    ROCMFusedElementWiseNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element,
+                             std::string binary, std::vector<Expression> a_shape, std::vector<Expression> b_shape,
+                             std::vector<std::string> post);
+    const std::vector<Expression>& shape() const { return shape_; }
+    types::PrimitiveType element() const { return element_; }
+    const std::string& binary() const { return binary_; }
+    const std::vector<Expression>& a_shape() const { return a_shape_; }
+    const std::vector<Expression>& b_shape() const { return b_shape_; }
+    const std::vector<std::string>& post() const { return post_; }
+    std::vector<std::string>& post() { return post_; }
+    bool has_b() const { return !binary_.empty(); }
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ROCMFusedElementWiseNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    types::PrimitiveType element_;
+    std::string binary_;
+    std::vector<Expression> a_shape_, b_shape_;
+    std::vector<std::string> post_;
+};
+
 } // namespace rocm
 
 namespace structured_control_flow {
@@ -410,6 +446,8 @@ public:
     void set_return_container(const std::string& name) { return_container_ = name; }
 
     void add_container(Container c, bool is_argument);
+    // a transient that no block refers to any more
+    void remove_container(const std::string& name);
     structured_control_flow::Block& add_block(std::unique_ptr<data_flow::LibraryNode> node,
                                               std::vector<data_flow::ConnectorBinding> inputs,
                                               std::vector<data_flow::ConnectorBinding> outputs, size_t position = (size_t) -1);

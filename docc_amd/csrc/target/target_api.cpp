@@ -131,6 +131,7 @@ char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, con
             json::Value o = json::Value::parse(options_json);
             if (const json::Value* v = o.find("offload")) options.offload = v->as_string();
             if (const json::Value* v = o.find("require_all_mapped")) options.require_all_mapped = v->as_bool();
+            if (const json::Value* v = o.find("fuse")) options.fuse_elementwise = v->as_bool();
         }
         builder::StructuredSDFGBuilder builder(*sdfg);
         analysis::AnalysisManager analysis_manager(*sdfg);

@@ -71,6 +71,8 @@ _SIGNATURES = {
     "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
     "docc_rocm_elementwise_binary_scalar": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, ctypes.c_double, ctypes.c_int, _vp],
     "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
+    "docc_rocm_elementwise_fused": [_vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_double, _vp, _vp,
+                                    ctypes.c_double, ctypes.c_int, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
@@ -241,6 +243,29 @@ def broadcast(precision, in_shape, out_shape, X, Y, stream=0) -> None:
     ins = (ctypes.c_int64 * rank)(*in_shape)
     outs = (ctypes.c_int64 * rank)(*out_shape)
     call("docc_rocm_broadcast", stream, precision, rank, ctypes.addressof(ins), ctypes.addressof(outs), X, Y)
+
+
+def elementwise_fused(precision, shape, binary, a, a_shape, b, b_shape, post, Y, stream=0) -> None:
+    """Y = post_k(...post_1(binary(a, b))) over `shape`. `a` / `b`: a device address with its shape
+    (left-padded to the output rank) or a Python number with shape None; `binary` None starts the
+    chain from `a`; `post`: names of unary operations."""
+    rank = len(shape)
+    dims = (ctypes.c_int64 * rank)(*shape)
+
+    def operand(value, value_shape):
+        if value_shape is None:
+            return None, 0, float(value)
+        padded = (1,) * (rank - len(value_shape)) + tuple(value_shape)
+        arr = (ctypes.c_int64 * rank)(*padded)
+        return arr, value, 0.0
+
+    a_arr, a_ptr, a_val = operand(a, a_shape)
+    b_arr, b_ptr, b_val = operand(b, b_shape) if binary is not None else (None, 0, 0.0)
+    ops = (ctypes.c_int * max(len(post), 1))(*[UNARY_OPS[o] if isinstance(o, str) else o for o in post])
+    code = -1 if binary is None else (BINARY_OPS[binary] if isinstance(binary, str) else binary)
+    call("docc_rocm_elementwise_fused", stream, precision, rank, ctypes.addressof(dims), code,
+         ctypes.addressof(a_arr) if a_arr is not None else None, a_ptr, a_val,
+         ctypes.addressof(b_arr) if b_arr is not None else None, b_ptr, b_val, len(post), ctypes.addressof(ops), Y)
 
 
 def mfma_probe(precision, waves_per_simd, iters, operands, sink, stream=0) -> float:

@@ -138,6 +138,19 @@ int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, int op, int p
 int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, const int64_t* in_shape, const int64_t* out_shape,
                         const void* X, void* Y);
 
+/* A chain of elementwise nodes in one pass: Y = post_k(...post_1(f(A', B'))). A' and B' are
+ * the operands repeated to `shape` by numpy's rules (`a_shape` / `b_shape`: `rank` extents, each
+ * equal to the output's or 1), or the scalar `a_scalar` / `b_scalar` when the shape pointer is
+ * NULL; `binary_op` is a DOCC_ROCM_BINARY_* code or -1 (the chain then starts from A' and B is
+ * ignored); `post_ops` holds `n_post` (0..4) DOCC_ROCM_UNARY_* codes applied in order. This is
+ * what the target's fusion pass emits for a Broadcast node folded into its consumer and unary
+ * nodes folded into their producer (the reference reaches the same through MapFusion over the
+ * expanded Maps, python/bindings/py_structured_sdfg.cpp:258-260). Each step rounds to the
+ * element type as the separate nodes would. */
+int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precision, int rank, const int64_t* shape, int binary_op,
+                                const int64_t* a_shape, const void* A, double a_scalar, const int64_t* b_shape, const void* B,
+                                double b_scalar, int n_post, const int* post_ops, void* Y);
+
 /* Measurement aid, no counterpart in the reference: `iters` rounds of 32 back-to-back
  * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16) on
  * every SIMD, `waves_per_simd` (1 or 2) waves each, operands taken from `operands`

@@ -147,3 +147,62 @@ def test_errors(rt):
     with pytest.raises(RocmRuntimeError):
         rt.broadcast(32, (2, 3), (2, 4), a.data_ptr(), a.data_ptr())
     rt.elementwise_unary("exp", 32, 0, 0, 0)   # empty: no-op
+
+
+FUSED_CASES = [
+    # out shape, a shape (None: scalar), b shape, binary, post
+    ((200, 130), (200, 130), (130,), "add", ["relu"]),                   # bias + activation after a product
+    ((64, 96), (64, 1), (64, 96), "sub", ["abs", "sqrt"]),               # column operand on the left
+    ((4, 8, 14, 14), (4, 8, 14, 14), (1, 8, 1, 1), "mul", []),           # NCHW channel scale
+    ((37, 53), (37, 53), None, "maximum", ["relu", "abs"]),              # scalar on the right
+    ((37, 53), None, (37, 53), "div", []),                               # scalar on the left
+    ((1000,), (1000,), None, None, ["abs", "sqrt", "relu"]),             # unary chain only
+    ((3, 5, 7), (3, 1, 7), (1, 5, 1), "minimum", ["abs"]),               # both operands repeat
+    ((2, 3, 2, 3, 2, 4), (2, 3, 2, 3, 2, 4), (4,), "add", ["relu"]),     # rank 6
+    ((8192, 4096), (8192, 4096), (4096,), "add", ["relu"]),              # the softmax tensor's shape
+]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("case", FUSED_CASES, ids=[str(i) for i in range(len(FUSED_CASES))])
+def test_fused_chain_equals_the_separate_nodes_bit_for_bit(rt, dt, case):
+    """docc_rocm_elementwise_fused against the oracle's Broadcast -> binary -> unary... chain. Only
+    operations whose result is exactly rounded are used here, so the bar is bit-exact."""
+    shape, a_shape, b_shape, binary, post = case
+    rng = np.random.default_rng(len(shape) * 7 + len(post))
+    make = lambda s: (rng.standard_normal(s) * 4).astype(dt)
+    a = make(a_shape) if a_shape is not None else 1.75
+    b = make(b_shape) if b_shape is not None else -0.3
+    if binary == "div" and b_shape is not None:
+        b[b == 0] = 1
+    full = lambda v, s: oracle.broadcast(v, shape) if s is not None else np.full(shape, v, dt)
+    ref = full(a, a_shape)
+    if binary is not None:
+        ref = oracle.elementwise_binary(binary, ref, full(b, b_shape))
+    for op in post:
+        ref = oracle.elementwise_unary(op, ref)
+    da = dev(a) if a_shape is not None else None
+    db = dev(b) if (b_shape is not None and binary is not None) else None
+    out = torch.full(shape, float("nan"), device="cuda", dtype=torch.float64 if dt == np.float64 else torch.float32)
+    rt.elementwise_fused(prec(dt), shape, binary, da.data_ptr() if da is not None else a, a_shape,
+                         db.data_ptr() if db is not None else b, b_shape if binary is not None else None, post, out.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(out), ref, equal_nan=True)
+
+
+def test_fused_chain_with_libm_operations_and_unaligned_operands(rt):
+    rng = np.random.default_rng(9)
+    x, bias = rng.standard_normal((65, 33)).astype(np.float32), rng.standard_normal(33).astype(np.float32)
+    ref = oracle.elementwise_unary("tanh", oracle.elementwise_unary("sigmoid", oracle.elementwise_binary("add", x, oracle.broadcast(bias, x.shape))))
+    dx, dbias = dev(x), dev(np.concatenate([np.zeros(1, np.float32), bias]))      # bias off a 16-byte boundary, odd inner extent
+    out = torch.full(x.shape, float("nan"), device="cuda")
+    rt.elementwise_fused(32, x.shape, "add", dx.data_ptr(), x.shape, dbias.data_ptr() + 4, bias.shape, ["sigmoid", "tanh"], out.data_ptr())
+    torch.cuda.synchronize()
+    assert ulps(host(out), ref) <= 8
+    from docc_amd.runtime import RocmRuntimeError
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_fused(32, (4, 4), "add", dx.data_ptr(), (4, 3), dx.data_ptr(), (4, 4), [], out.data_ptr())     # 3 cannot become 4
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_fused(32, (4, 4), None, 1.0, None, 0, None, ["relu"], out.data_ptr())                           # no array operand
+    with pytest.raises(RocmRuntimeError):
+        rt.elementwise_fused(32, (4, 4), None, dx.data_ptr(), (4, 4), 0, None, ["relu"] * 5, out.data_ptr())           # five unary operations

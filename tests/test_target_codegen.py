@@ -274,7 +274,7 @@ def test_elementwise_nodes_round_trip_and_dispatch(tmp_path):
     # payload keys of the reference's serializers: shape (elementwise_node.cpp), input_shape / output_shape (broadcast_node.cpp)
     assert nodes[2]["shape"] == ["32", "16"] and nodes[1]["input_shape"] == ["1", "16"] and nodes[1]["output_shape"] == ["32", "16"]
     assert StructuredSDFG.parse(s.to_json()).library_nodes() == nodes
-    s.schedule("rocm")
+    s.schedule("rocm", options={"fuse": False})      # one launcher call per node
     r = s.loop_report()
     assert r["H2D"] == 3 and r["D2H"] == 1          # X, W, bias up; Y down; T0..T3 stay in device memory
     for t in ("T0", "T1", "T2", "T3"):
@@ -320,3 +320,56 @@ def test_elementwise_with_transfers_and_scalar_on_the_left(tmp_path):
     with pytest.raises(InvalidSDFGException, match="cannot be broadcast"):
         b.add_broadcast("a", "c", [3, 4], [5, 4])
         b.move().validate()
+
+
+def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
+    """relu(X @ W + bias) * 0.5: the Broadcast moves into the Add, the ReLU into the Add; the multiplication by
+    a constant is a binary node of its own and stays. GEMM + two elementwise launches instead of five."""
+    s = dense_sdfg()
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["GEMM"] == 1 and r["ROCMFusedElementWise"] == 1 and r["ml::Mul"] == 1
+    assert "ml::Broadcast" not in r and "ml::Add" not in r and "ml::ReLU" not in r
+    assert r["H2D"] == 3 and r["D2H"] == 1
+    assert set(s.containers) >= {"T0", "T3"} and "T1" not in s.containers and "T2" not in s.containers
+    fused = next(n for n in s.library_nodes() if n["code"] == "ROCMFusedElementWise")
+    assert fused["binary"] == "ml::Add" and fused["a_shape"] == ["32", "16"] and fused["b_shape"] == ["1", "16"]
+    assert fused["post"] == ["ml::ReLU"] and fused["implementation_type"] == "ROCMWithoutTransfers"
+    strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]       # ids are renumbered by a parse
+    assert strip(StructuredSDFG.parse(s.to_json()).library_nodes()) == strip(s.library_nodes())    # the fused node serialises
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path)[0])
+    assert "const int64_t __docc_b_shape[] = {(int64_t) (1), (int64_t) (16)};" in flat
+    assert "const int __docc_post[] = {2 /* ml::ReLU */};" in flat
+    assert ("docc_rocm_elementwise_fused(nullptr, 32, 2, __docc_shape, 0 /* ml::Add */, __docc_a_shape, A, 0.0, __docc_b_shape, B, 0.0, "
+            "1, __docc_post, Y)") in flat
+    assert flat.count("docc_rocm_malloc(") == 6      # X W bias on the device, T0, T3, Y: two intermediates fewer
+
+    # unary chains fold too, up to four operations; a value that something else reads is not folded away
+    b = StructuredSDFGBuilder("chain")
+    for n in ("X", "Y", "Z"):
+        b.add_container(n, F64, True)
+    for n in ("T0", "T1", "T2"):
+        b.add_container(n, F64, False, transient_bytes=800)
+    b.add_elementwise_unary_op("abs", "X", "T0", [100])
+    b.add_elementwise_unary_op("sqrt", "T0", "T1", [100])
+    b.add_elementwise_unary_op("tanh", "T1", "T2", [100])
+    b.add_elementwise_op("sub", "T2", "T1", "Y", [100])        # T1 has a second reader
+    b.add_elementwise_unary_op("exp", "Y", "Z", [100])         # Y is an argument: stays
+    s = b.move()
+    s.schedule("rocm")
+    nodes = [(n["code"], n.get("post"), n.get("binary")) for n in s.library_nodes() if not n["code"].startswith("ROCMOff")]
+    assert nodes == [("ROCMFusedElementWise", ["ml::Abs", "ml::Sqrt"], ""), ("ml::Tanh", None, None), ("ml::Sub", None, None),
+                     ("ml::Exp", None, None)]
+
+    # per-node transfers keep working on the fused node, scalars are passed by value
+    b = StructuredSDFGBuilder("scalar")
+    b.add_container("x", F32, True)
+    b.add_container("y", F32, True)
+    b.add_container("t", F32, False, transient_bytes=40)
+    b.add_elementwise_op("max", "x", "0.25", "t", [10])
+    b.add_elementwise_unary_op("sigmoid", "t", "y", [10])
+    s = b.move()
+    s.schedule("rocm", options={"offload": "node"})
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "scalar")[0])
+    assert "docc_rocm_elementwise_fused(nullptr, 32, 1, __docc_shape, 4 /* ml::Maximum */, __docc_a_shape, d_A, 0.0, nullptr, nullptr, (double) B, 1, __docc_post, d_Y)" in flat
+    assert flat.count("docc_rocm_memcpy_h2d_async(") == 1 and flat.count("docc_rocm_memcpy_d2h_async(") == 1
