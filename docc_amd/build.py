@@ -39,6 +39,11 @@ KERNEL_FAMILIES = {
     "gemm_bf16": "gemm_bf16.hip",
     "gemm_bf16_async": "gemm_bf16_async.hip",
     "gemm_bf16_async_big": "gemm_bf16_async_big.hip",
+    "gemm_f32_epilogue": "gemm_f32_epilogue.hip",
+    "gemm_f64_epilogue": "gemm_f64_epilogue.hip",
+    "gemm_bf16_epilogue": "gemm_bf16_epilogue.hip",
+    "gemm_bf16_async_epilogue": "gemm_bf16_async_epilogue.hip",
+    "gemm_bf16_async_big_epilogue": "gemm_bf16_async_big_epilogue.hip",
     "conv2d": "conv2d.hip",
     "attention": "attention.hip",
     "elementwise": "elementwise.hip",
@@ -53,6 +58,9 @@ FAMILY_FLAGS = {
     "gemm_f64": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "gemm_f32": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "gemm_bf16_async": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_f64_epilogue": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_f32_epilogue": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_bf16_async_epilogue": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "conv2d": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
@@ -90,7 +98,7 @@ def _newer(target: Path, sources: list[Path]) -> bool:
 def build_kernel_family(family: str, force: bool = True) -> Path:
     src = CSRC / "kernels" / KERNEL_FAMILIES[family]
     out = LIB / f"docc_rocm_{family}.hsaco"
-    deps = [src] + sorted((CSRC / "kernels").glob("*.h"))
+    deps = [src] + sorted((CSRC / "kernels").glob("*.h")) + sorted((CSRC / "kernels").glob("gemm*.hip"))
     if not force and _newer(out, deps):
         return out
     LIB.mkdir(parents=True, exist_ok=True)

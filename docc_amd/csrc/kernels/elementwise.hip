@@ -3,60 +3,13 @@
 // Replace the Maps that ElementWiseUnaryNode / ElementWiseBinaryNode::expand produce (reference
 // sdfg/include/sdfg/data_flow/library_nodes/math/tensor/elementwise_node.h: Y[i] = f(X[i]) or
 // f(A[i], B[i]) over the linearised shape) and BroadcastNode::expand (broadcast_node.h:13-43).
-// Operation semantics follow the reference's expansions:
-//   ReLU     fmax(x, 0.0)            elementwise_ops/relu_node.cpp:40-43
-//   Sigmoid  1.0 / (1.0 + exp(-x))   elementwise_ops/sigmoid_node.cpp:46-70
-//   Maximum / Minimum  fmax / fmin   elementwise_ops/maximum_node.cpp:64, minimum_node.cpp
-//   Abs, Exp, Sqrt, Tanh, Erf        the libm function of the element type (cmath_node.h)
-//   Add, Sub, Mul, Div               the IEEE operation
+// Operation semantics: elementwise_ops.h.
 //
 // HBM-bound: 8 (unary) or 12 (binary) bytes per fp32 element. One 128-bit access per operand
 // and lane, grid-stride over the vectors, scalar tail; unaligned operands take the scalar path.
-#include "common.h"
+#include "elementwise_ops.h"
 
 namespace docc_k {
-
-enum UnaryOp : int { kAbs = 0, kExp = 1, kReLU = 2, kSigmoid = 3, kSqrt = 4, kTanh = 5, kErf = 6 };
-enum BinaryOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMaximum = 4, kMinimum = 5 };
-
-template <int OP>
-__device__ __forceinline__ float unary(float x) {
-    if (OP == kAbs) return fabsf(x);
-    if (OP == kExp) return expf(x);
-    if (OP == kReLU) return fmaxf(x, 0.0f);
-    if (OP == kSigmoid) return 1.0f / (1.0f + expf(-x));
-    if (OP == kSqrt) return sqrtf(x);
-    if (OP == kTanh) return tanhf(x);
-    return erff(x);
-}
-template <int OP>
-__device__ __forceinline__ double unary(double x) {
-    if (OP == kAbs) return fabs(x);
-    if (OP == kExp) return exp(x);
-    if (OP == kReLU) return fmax(x, 0.0);
-    if (OP == kSigmoid) return 1.0 / (1.0 + exp(-x));
-    if (OP == kSqrt) return sqrt(x);
-    if (OP == kTanh) return tanh(x);
-    return erf(x);
-}
-template <int OP>
-__device__ __forceinline__ float binary(float a, float b) {
-    if (OP == kAdd) return a + b;
-    if (OP == kSub) return a - b;
-    if (OP == kMul) return a * b;
-    if (OP == kDiv) return a / b;
-    if (OP == kMaximum) return fmaxf(a, b);
-    return fminf(a, b);
-}
-template <int OP>
-__device__ __forceinline__ double binary(double a, double b) {
-    if (OP == kAdd) return a + b;
-    if (OP == kSub) return a - b;
-    if (OP == kMul) return a * b;
-    if (OP == kDiv) return a / b;
-    if (OP == kMaximum) return fmax(a, b);
-    return fmin(a, b);
-}
 
 template <typename T>
 struct Vec128;
@@ -186,31 +139,6 @@ struct FusedParams {
     int post[4];            // UnaryOp codes
 };
 
-template <typename T>
-__device__ __forceinline__ T fused_unary(int op, T x) {
-    switch (op) {
-        case kAbs: return unary<kAbs>(x);
-        case kExp: return unary<kExp>(x);
-        case kReLU: return unary<kReLU>(x);
-        case kSigmoid: return unary<kSigmoid>(x);
-        case kSqrt: return unary<kSqrt>(x);
-        case kTanh: return unary<kTanh>(x);
-        default: return unary<kErf>(x);
-    }
-}
-
-template <typename T>
-__device__ __forceinline__ T fused_binary(int op, T a, T b) {
-    switch (op) {
-        case kAdd: return binary<kAdd>(a, b);
-        case kSub: return binary<kSub>(a, b);
-        case kMul: return binary<kMul>(a, b);
-        case kDiv: return binary<kDiv>(a, b);
-        case kMaximum: return binary<kMaximum>(a, b);
-        default: return binary<kMinimum>(a, b);
-    }
-}
-
 template <typename T, int VEC, typename I>
 __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const FusedParams& p) {
     typedef T V __attribute__((ext_vector_type(VEC)));
@@ -257,11 +185,11 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
                 for (int e = 0; e < VEC; e++) b[e] = x;
             }
 #pragma unroll
-            for (int e = 0; e < VEC; e++) a[e] = fused_binary<T>(p.binary, a[e], b[e]);
+            for (int e = 0; e < VEC; e++) a[e] = apply_binary<T>(p.binary, a[e], b[e]);
         }
         for (int k = 0; k < p.npost; k++) {
 #pragma unroll
-            for (int e = 0; e < VEC; e++) a[e] = fused_unary<T>(p.post[k], a[e]);
+            for (int e = 0; e < VEC; e++) a[e] = apply_unary<T>(p.post[k], a[e]);
         }
         __builtin_nontemporal_store(a, reinterpret_cast<V*>(Y) + v);
     }

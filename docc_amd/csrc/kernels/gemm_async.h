@@ -151,7 +151,7 @@ struct AsyncGemmKernel {
 
     static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, out_t* __restrict__ C,
                                                long M, long N, long K, long lda, long ldb, long ldc, out_t alpha,
-                                               out_t beta) {
+                                               out_t beta, const out_t* bias, int act) {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
         T* const lds = reinterpret_cast<T*>(docc_gemm_lds);
 
@@ -363,7 +363,7 @@ struct AsyncGemmKernel {
         kstep(kt, std::integral_constant<int, 2>{});
 
         // ---- epilogue ------------------------------------------------------------------------------
-        gemm_store_wave<TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lidx, alpha, beta, acc, [&](int r) {
+        gemm_store_wave<kGemmEpilogue, TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lidx, alpha, beta, bias, act, acc, [&](int r) {
             return (sizeof(T) == 8) ? Mfma<double>::acc_row(lane, r) : Mfma<float>::acc_row(lane, r);
         });
     }
@@ -373,9 +373,10 @@ struct AsyncGemmKernel {
 
 // extern "C" kernels docc_<prefix>a_<BM>x<BN>x<BK>s<STAGES>_<nn|nt|tn|tt>
 #define DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, TA, TB, TAG)                                          \
-    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_##PREFIX##a_##BM##x##BN##x##BK##s##ST##_##TAG(  \
-        const T* A, const T* B, OT* C, long M, long N, long K, long lda, long ldb, long ldc, OT alpha, OT beta) {   \
-        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta); \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_##PREFIX##a_##BM##x##BN##x##BK##s##ST##_##TAG)(  \
+        const T* A, const T* B, OT* C, long M, long N, long K, long lda, long ldb, long ldc, OT alpha, OT beta,    \
+        const OT* bias, int act) {                                                                                 \
+        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
     }
 
 #define DOCC_AGEMM_CONFIG(PREFIX, T, OT, BM, BN, BK, WM, WN, ST)            \

@@ -68,7 +68,7 @@ struct GemmBf16Kernel {
 
     static __device__ __forceinline__ void run(const uint16_t* __restrict__ A, const uint16_t* __restrict__ B,
                                                float* __restrict__ C, long M, long N, long K, long lda, long ldb,
-                                               long ldc, float alpha, float beta) {
+                                               long ldc, float alpha, float beta, const float* bias, int act) {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
         uint16_t* const lds = reinterpret_cast<uint16_t*>(docc_gemm_lds);
         constexpr int B_BASE = 2 * A_ELEMS;
@@ -155,35 +155,18 @@ struct GemmBf16Kernel {
         }
         compute(kt & 1);
 
-        const bool use_c = (beta != 0.f);
-        const int lrow = lane & 31;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const long col = n0 + wn * WTN + j * MT + lrow;
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const long row = m0 + wm * WTM + i * MT + Mfma<float>::acc_row(lane, r);
-                    if (row < M && col < N) {
-                        float* p = C + row * ldc + col;
-                        float val = alpha * acc[i][j][r];
-                        if (use_c) val += beta * (*p);
-                        *p = val;
-                    }
-                }
-            }
-        }
+        gemm_store_wave<kGemmEpilogue, TM, TN, MT, 16>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lane & 31, alpha, beta, bias, act, acc,
+                                        [&](int r) { return Mfma<float>::acc_row(lane, r); });
     }
 };
 
 } // namespace docc_k
 
 #define DOCC_BGEMM_ONE(BM, BN, BK, WM, WN, TA, TB, TAG, AL, ALTAG)                                                  \
-    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_bgemm_##BM##x##BN##x##BK##_##TAG##_##ALTAG(      \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_bgemm_##BM##x##BN##x##BK##_##TAG##_##ALTAG)(      \
         const uint16_t* A, const uint16_t* B, float* C, long M, long N, long K, long lda, long ldb, long ldc,       \
-        float alpha, float beta) {                                                                                  \
-        docc_k::GemmBf16Kernel<BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta);  \
+        float alpha, float beta, const float* bias, int act) {                                                      \
+        docc_k::GemmBf16Kernel<BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
     }
 
 #define DOCC_BGEMM_CONFIG(BM, BN, BK, WM, WN)                    \
@@ -199,6 +182,7 @@ struct GemmBf16Kernel {
 DOCC_BGEMM_CONFIG(128, 128, 64, 2, 2)
 DOCC_BGEMM_CONFIG(256, 256, 64, 2, 2)
 
+#ifndef DOCC_GEMM_EPILOGUE
 extern "C" __global__ __launch_bounds__(256) void docc_bgemm_scale_c(float* C, long M, long N, long ldc, float beta) {
     const long total = M * N;
     const long stride = (long) gridDim.x * 256;
@@ -207,3 +191,4 @@ extern "C" __global__ __launch_bounds__(256) void docc_bgemm_scale_c(float* C, l
         *p = (beta == 0.f) ? 0.f : beta * (*p);
     }
 }
+#endif

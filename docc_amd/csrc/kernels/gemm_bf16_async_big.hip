@@ -3,4 +3,6 @@
 #include "gemm_async.h"
 
 DOCC_AGEMM_CONFIG(bgemm, uint16_t, float, 256, 256, 64, 2, 2, 2)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(bgemm, uint16_t, float, 256, 256, 32, 2, 2, 4)
+#endif

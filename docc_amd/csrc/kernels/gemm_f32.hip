@@ -6,11 +6,16 @@ DOCC_GEMM_CONFIG(sgemm, float, 64, 64, 16, 2, 2)
 
 // asynchronous multi-stage variants (aligned operands)
 DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 128, 16, 2, 2, 3)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 128, 32, 2, 2, 3)
+#endif
 DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 256, 16, 2, 2, 3)
 DOCC_AGEMM_CONFIG(sgemm, float, float, 64, 64, 16, 2, 2, 4)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(sgemm, float, float, 64, 64, 32, 2, 2, 3)
+#endif
 
+#ifndef DOCC_GEMM_EPILOGUE
 // C = beta * C (the k == 0 case); beta == 0 stores zeros without reading C.
 extern "C" __global__ __launch_bounds__(256) void docc_sgemm_scale_c(float* C, long M, long N, long ldc, float beta) {
     const long total = M * N;
@@ -20,3 +25,4 @@ extern "C" __global__ __launch_bounds__(256) void docc_sgemm_scale_c(float* C, l
         *p = (beta == 0.f) ? 0.f : beta * (*p);
     }
 }
+#endif

@@ -5,14 +5,21 @@ DOCC_GEMM_CONFIG(dgemm, double, 64, 64, 16, 2, 2)
 DOCC_GEMM_CONFIG(dgemm, double, 128, 128, 16, 2, 2)
 
 // asynchronous multi-stage pipeline (aligned operands)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 2)
+#endif
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 4)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 16, 2, 2, 6)
+#endif
 DOCC_AGEMM_CONFIG(dgemm, double, double, 128, 128, 16, 2, 2, 3)
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 16, 2, 2, 4)
+#ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 32, 2, 2, 3)
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 32, 2, 2, 3)
+#endif
 
+#ifndef DOCC_GEMM_EPILOGUE
 extern "C" __global__ __launch_bounds__(256) void docc_dgemm_scale_c(double* C, long M, long N, long ldc, double beta) {
     const long total = M * N;
     const long stride = (long) gridDim.x * 256;
@@ -21,3 +28,4 @@ extern "C" __global__ __launch_bounds__(256) void docc_dgemm_scale_c(double* C, 
         *p = (beta == 0.0) ? 0.0 : beta * (*p);
     }
 }
+#endif

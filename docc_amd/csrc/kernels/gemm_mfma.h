@@ -20,9 +20,23 @@
 //     that XCD's L2.
 #pragma once
 
-#include "common.h"
+#include "elementwise_ops.h"
+
+// A translation unit compiled with DOCC_GEMM_EPILOGUE holds the epilogue variants of its kernels:
+// same tiles, names with the suffix "_e", C = act(alpha A B + beta C + bias) in the store.
+#ifdef DOCC_GEMM_EPILOGUE
+#define DOCC_GEMM_NAME(base) base##_e
+#else
+#define DOCC_GEMM_NAME(base) base
+#endif
 
 namespace docc_k {
+
+#ifdef DOCC_GEMM_EPILOGUE
+constexpr bool kGemmEpilogue = true;
+#else
+constexpr bool kGemmEpilogue = false;
+#endif
 
 template <typename T>
 struct Mfma;
@@ -66,11 +80,68 @@ struct Mfma<double> {
 // wholly inside C - all but the last row and column of tiles - is stored by straight-line code:
 // with one bounds branch per element the instruction fetch of the cold, branchy epilogue costs
 // more than the stores themselves.
-template <int TM, int TN, int MT, int NACC, typename OT, typename AccT, typename RowFn>
-__device__ __forceinline__ void gemm_store_wave(OT* C, long ldc, long M, long N, long row0, long col0, int lcol,
-                                                OT alpha, OT beta, AccT (&acc)[TM][TN], RowFn acc_row) {
+// alpha * acc + beta * old with one fixed contraction (the product alpha * acc rounded, then one fused
+// multiply-add), so that interior tiles, edge tiles and the fused epilogue all round alike
+__device__ __forceinline__ float gemm_axpby(float alpha, float acc, float beta, float old) {
+    return __builtin_fmaf(beta, old, alpha * acc);
+}
+__device__ __forceinline__ double gemm_axpby(double alpha, double acc, double beta, double old) {
+    return __builtin_fma(beta, old, alpha * acc);
+}
+
+// Epilogue of a fused chain: C = act(alpha * A B + beta * C + bias[col]), ACT a compile-time
+// UnaryOp or -1. Every step rounds as the separate nodes would (the sum is kept from contracting
+// with the product before it).
+template <int ACT, int TM, int TN, int MT, int NACC, typename OT, typename AccT, typename RowFn>
+__device__ __forceinline__ void gemm_store_wave_epilogue(OT* C, long ldc, long M, long N, long row0, long col0, int lcol, OT alpha,
+                                                         OT beta, const OT* bias, AccT (&acc)[TM][TN], RowFn acc_row) {
     const bool use_c = (beta != (OT) 0);
-    if (row0 + TM * MT <= M && col0 + TN * MT <= N) {
+    const bool whole = row0 + TM * MT <= M && col0 + TN * MT <= N;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const long col = col0 + j * MT + lcol;
+        const bool col_ok = whole || col < N;
+        const OT b = (bias != nullptr && col_ok) ? bias[col] : (OT) 0;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int r = 0; r < NACC; r++) {
+                const long row = row0 + i * MT + acc_row(r);
+                if (whole || (row < M && col_ok)) {
+                    OT* p = C + row * ldc + col;
+                    OT val = use_c ? gemm_axpby(alpha, (OT) acc[i][j][r], beta, *p) : alpha * acc[i][j][r];
+                    if (bias != nullptr) {
+                        asm volatile("" : "+v"(val));
+                        val += b;
+                    }
+                    if (ACT >= 0) val = unary<ACT>(val);
+                    *p = val;
+                }
+            }
+    }
+}
+
+// EPI: the kernel is one of the epilogue variants (built apart from the plain kernels, whose
+// register allocation must not carry the activation code); bias / act are ignored otherwise.
+template <bool EPI, int TM, int TN, int MT, int NACC, typename OT, typename AccT, typename RowFn>
+__device__ __forceinline__ void gemm_store_wave(OT* C, long ldc, long M, long N, long row0, long col0, int lcol,
+                                                OT alpha, OT beta, const OT* bias, int act, AccT (&acc)[TM][TN], RowFn acc_row) {
+    if constexpr (EPI) {
+#define DOCC_EPILOGUE_CASE(ACT) \
+    gemm_store_wave_epilogue<ACT, TM, TN, MT, NACC>(C, ldc, M, N, row0, col0, lcol, alpha, beta, bias, acc, acc_row)
+        // only the activations that cost one instruction are built into the store: each case is a fully
+        // unrolled copy of the epilogue; the others run as an elementwise kernel after the GEMM
+        switch (act) {
+            case kAbs: DOCC_EPILOGUE_CASE(kAbs); break;
+            case kReLU: DOCC_EPILOGUE_CASE(kReLU); break;
+            default: DOCC_EPILOGUE_CASE(-1); break;
+        }
+#undef DOCC_EPILOGUE_CASE
+        return;
+    }
+    const bool use_c = (beta != (OT) 0);
+    const bool whole = row0 + TM * MT <= M && col0 + TN * MT <= N;
+    if (whole) {
         OT* base = C + (row0 + acc_row(0)) * ldc + col0 + lcol;
         if (!use_c) {
 #pragma unroll
@@ -90,7 +161,7 @@ __device__ __forceinline__ void gemm_store_wave(OT* C, long ldc, long M, long N,
                     for (int r = 0; r < NACC; r++) old[r] = base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT];
 #pragma unroll
                     for (int r = 0; r < NACC; r++)
-                        base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT] = alpha * acc[i][j][r] + beta * old[r];
+                        base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT] = gemm_axpby(alpha, (OT) acc[i][j][r], beta, old[r]);
                 }
         }
         return;
@@ -105,9 +176,7 @@ __device__ __forceinline__ void gemm_store_wave(OT* C, long ldc, long M, long N,
                 const long row = row0 + i * MT + acc_row(r);
                 if (row < M && col < N) {
                     OT* p = C + row * ldc + col;
-                    OT val = alpha * acc[i][j][r];
-                    if (use_c) val += beta * (*p);
-                    *p = val;
+                    *p = use_c ? gemm_axpby(alpha, (OT) acc[i][j][r], beta, *p) : alpha * acc[i][j][r];
                 }
             }
         }
@@ -253,7 +322,7 @@ struct GemmKernel {
 
     static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ C,
                                                long M, long N, long K, long lda, long ldb, long ldc, T alpha,
-                                               T beta) {
+                                               T beta, const T* bias, int act) {
         // all LDS addressing is derived from this one array so that the
         // compiler keeps it in the LDS address space (ds_* instructions)
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_gemm_lds[];
@@ -368,7 +437,7 @@ struct GemmKernel {
         }
         compute(kt & 1);
 
-        gemm_store_wave<TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lrow, alpha, beta, acc,
+        gemm_store_wave<kGemmEpilogue, TM, TN, MT, X::NACC>(C, ldc, M, N, m0 + wm * WTM, n0 + wn * WTN, lrow, alpha, beta, bias, act, acc,
                                              [&](int r) { return X::acc_row(lane, r); });
     }
 };
@@ -379,9 +448,10 @@ struct GemmKernel {
 // configuration as extern "C" kernels named
 //   docc_<prefix>_<BM>x<BN>x<BK>_<nn|nt|tn|tt>_<a|u>
 #define DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, TA, TB, TAG, AL, ALTAG)                                   \
-    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_##PREFIX##_##BM##x##BN##x##BK##_##TAG##_##ALTAG( \
-        const T* A, const T* B, T* C, long M, long N, long K, long lda, long ldb, long ldc, T alpha, T beta) {  \
-        docc_k::GemmKernel<T, BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta); \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_##PREFIX##_##BM##x##BN##x##BK##_##TAG##_##ALTAG)( \
+        const T* A, const T* B, T* C, long M, long N, long K, long lda, long ldb, long ldc, T alpha, T beta,    \
+        const T* bias, int act) {                                                                              \
+        docc_k::GemmKernel<T, BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
     }
 
 #define DOCC_GEMM_CONFIG(PREFIX, T, BM, BN, BK, WM, WN)                    \

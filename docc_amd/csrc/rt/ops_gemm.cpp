@@ -1,6 +1,7 @@
 // Launchers for the GEMM node kernels (see include/docc_rocm_ops.h).
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
@@ -30,7 +31,7 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
 template <typename T, typename S = T>
 int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n,
                 int64_t k, S alpha, const T* A, int64_t lda, const T* B, int64_t ldb, S beta, S* C, int64_t ldc,
-                TileConfig (*pick)(int64_t m, int64_t n, bool aligned, int force)) {
+                TileConfig (*pick)(int64_t m, int64_t n, bool aligned, int force), const S* bias = nullptr, int activation = -1) {
     if ((trans_a != DOCC_ROCM_NO_TRANS && trans_a != DOCC_ROCM_TRANS) ||
         (trans_b != DOCC_ROCM_NO_TRANS && trans_b != DOCC_ROCM_TRANS))
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: transpose code must be 111 or 112", prefix);
@@ -40,6 +41,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     if (lda < (a_cols > 1 ? a_cols : 1) || ldb < (b_cols > 1 ? b_cols : 1) || ldc < (n > 1 ? n : 1))
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: leading dimension too small (lda=%lld ldb=%lld ldc=%lld)",
                     prefix, (long long) lda, (long long) ldb, (long long) ldc);
+    if (activation < -1 || activation > DOCC_ROCM_UNARY_ERF)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: unknown activation %d", prefix, activation);
+    if (activation >= 0 && activation != DOCC_ROCM_UNARY_RELU && activation != DOCC_ROCM_UNARY_ABS)
+        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: only ReLU and Abs are built into the GEMM store (activation %d)", prefix, activation);
     if (m == 0 || n == 0) return 0;
     if (!C || (k > 0 && (!A || !B))) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null pointer", prefix);
     int rc = ensure_device();
@@ -50,7 +55,14 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         std::snprintf(name, sizeof(name), "docc_%s_scale_c", prefix);
         int64_t blocks = (m * n + 255) / 256;
         if (blocks > 4096) blocks = 4096;
-        return launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
+        rc = launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
+        if (rc || (!bias && activation < 0)) return rc;
+        // the epilogue of an empty product: C = act(beta * C + bias), through the elementwise kernel
+        if (ldc != n) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 with an epilogue needs ldc == n", prefix);
+        const int64_t shape[2] = {m, n}, row[2] = {1, n};
+        const int post[1] = {activation};
+        return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
+                                           bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
     }
     const size_t vec = 16 / sizeof(T);
     // the aligned kernels read whole 128-bit vectors: pointers, leading dimensions and the
@@ -83,8 +95,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                       tb ? 't' : 'n', aligned ? 'a' : 'u');
         lds = gemm_lds_bytes(cfg, ta, tb, sizeof(T));
     }
+    // the variants with bias / activation in the store carry the suffix "_e"
+    if (bias || activation >= 0) std::strncat(name, "_e", sizeof(name) - std::strlen(name) - 1);
     return launch(name, (uint32_t) tiles, 1, 1, 64 * cfg.waves, (uint32_t) lds, s, A, B, C, (long) m, (long) n,
-                  (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta);
+                  (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta, bias, activation);
 }
 
 } // namespace
@@ -137,6 +151,27 @@ int docc_rocm_bf16gemm_f32(docc_rocm_stream_t stream, int trans_a, int trans_b, 
                            float* C, int64_t ldc) {
     return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
                                         pick_bgemm);
+}
+
+int docc_rocm_sgemm_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                             const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C, int64_t ldc,
+                             const float* bias, int activation) {
+    return gemm_launch<float>("sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, pick_sgemm, bias,
+                              activation);
+}
+
+int docc_rocm_dgemm_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                             double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta, double* C,
+                             int64_t ldc, const double* bias, int activation) {
+    return gemm_launch<double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, pick_dgemm, bias,
+                               activation);
+}
+
+int docc_rocm_bf16gemm_f32_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                                    float alpha, const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, float beta,
+                                    float* C, int64_t ldc, const float* bias, int activation) {
+    return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+                                        pick_bgemm, bias, activation);
 }
 
 } // extern "C"

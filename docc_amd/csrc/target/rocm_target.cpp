@@ -155,7 +155,10 @@ protected:
     std::vector<DeviceOperand> operands() const override {
         // C travels to the device only when the node reads it (beta != 0)
         const bool read_c = node_.reads("__C", data_flow_graph_.inputs);
-        return {operand("__A", true, false), operand("__B", true, false), operand("__C", read_c, true)};
+        std::vector<DeviceOperand> ops{operand("__A", true, false), operand("__B", true, false)};
+        if (gemm().epilogue_bias()) ops.push_back(operand("__bias", true, false));
+        ops.push_back(operand("__C", read_c, true));
+        return ops;
     }
 
     std::string guard_condition() const override {
@@ -172,12 +175,26 @@ protected:
             case blas::b: fn = "docc_rocm_bf16gemm_f32"; in_t = "uint16_t"; out_t = "float"; break;
             default: throw std::runtime_error("Invalid precision for ROCM GEMM node");
         }
+        if (g.has_epilogue()) fn += "_epilogue";
         s << "DOCC_ROCM_CHECK(" << fn << "(nullptr, " << (int) g.trans_a() << ", " << (int) g.trans_b() << ", "
           << language_extension_.expression(g.m()) << ", " << language_extension_.expression(g.n()) << ", "
           << language_extension_.expression(g.k()) << ", __alpha, (const " << in_t << " *) " << name_of("__A") << ", "
           << language_extension_.expression(g.lda()) << ", (const " << in_t << " *) " << name_of("__B") << ", "
           << language_extension_.expression(g.ldb()) << ", __beta, (" << out_t << " *) " << name_of("__C") << ", "
-          << language_extension_.expression(g.ldc()) << "));" << std::endl;
+          << language_extension_.expression(g.ldc());
+        if (g.has_epilogue()) {
+            // C = act(alpha A B + beta C + bias[column]) in the store of the GEMM
+            int act = -1;
+            for (size_t i = 0; i < tensor::UnaryNodeCodes.size(); i++)
+                if (tensor::UnaryNodeCodes[i] == g.epilogue_activation()) act = (int) i;
+            if (g.epilogue_bias())
+                s << ", (const " << out_t << " *) " << name_of("__bias");
+            else
+                s << ", nullptr";
+            s << ", " << act;
+            if (act >= 0) s << " /* " << g.epilogue_activation() << " */";
+        }
+        s << "));" << std::endl;
     }
 };
 
@@ -571,6 +588,13 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
 
 namespace {
 
+ConnectorBinding make_binding(const std::string& connector, const std::string& data) {
+    ConnectorBinding b;
+    b.connector = connector;
+    b.data = data;
+    return b;
+}
+
 bool is_rocm_type(const std::string& impl) {
     return impl == ImplementationType_ROCMWithTransfers || impl == ImplementationType_ROCMWithoutTransfers;
 }
@@ -617,8 +641,6 @@ bool untouched_between(const StructuredSDFG& sdfg, const std::string& name, size
     }
     return true;
 }
-
-std::vector<Expression> ones(size_t rank) { return std::vector<Expression>(rank, "1"); }
 
 // Rewrites an elementwise node as the equivalent fused node (no-op for one that already is).
 void make_fused(StructuredSDFG& sdfg, size_t i) {
@@ -716,6 +738,91 @@ bool RocmElementwiseFusionPass::run_pass(builder::StructuredSDFGBuilder& builder
             sdfg.remove_container(link);
             changed = applied = true;
         }
+        // (3) the elementwise node behind a GEMM: the bias row and a one-instruction activation move into
+        //     the GEMM's store; what is left of the chain (other activations) stays an elementwise node
+        for (size_t i = 0; i < blocks.size() && !changed; i++) {
+            auto* gemm = dynamic_cast<blas::GEMMNode*>(blocks[i].node.get());
+            if (!gemm || !is_rocm_type(gemm->implementation_type()) || gemm->has_epilogue()) continue;
+            if (gemm->ldc() != gemm->n()) continue;   // the chain sees C as a dense [m, n] array
+            const std::string link = blocks[i].outputs[0].data;
+            const Container& lc = sdfg.container(link);
+            if (lc.is_argument || !lc.transient || link == sdfg.return_container()) continue;
+            const Uses u = uses_of(sdfg, link);
+            // the GEMM's own "__C" binding counts as a reader only if beta may be non-zero
+            const bool reads_c = gemm->reads("__C", blocks[i].inputs);
+            std::vector<size_t> readers;
+            for (size_t r : u.readers)
+                if (r != i || reads_c) readers.push_back(r);
+            if (u.writers.size() != 1 || readers.size() != 1 || readers[0] <= i) continue;
+            const size_t j = readers[0];
+            if (dynamic_cast<tensor::ElementWiseNode*>(blocks[j].node.get())) {
+                if (blocks[j].node->implementation_type() != gemm->implementation_type()) continue;
+                make_fused(sdfg, j);
+            }
+            auto* f = dynamic_cast<ROCMFusedElementWiseNode*>(blocks[j].node.get());
+            if (!f || f->implementation_type() != gemm->implementation_type()) continue;
+            if (f->element() != blas::precision_output_type(gemm->precision())) continue;
+            // [.., n] with the leading extents multiplying to m
+            const auto& shape = f->shape();
+            if (shape.empty() || shape.back() != gemm->n()) continue;
+            Expression lead = "1";
+            for (size_t d = 0; d + 1 < shape.size(); d++) lead = symbolic::mul(lead, shape[d]);
+            if (lead != gemm->m()) continue;
+            auto is_row = [&](const std::vector<Expression>& s) {
+                if (s.size() != shape.size() || s.back() != gemm->n()) return false;
+                for (size_t d = 0; d + 1 < s.size(); d++)
+                    if (s[d] != "1") return false;
+                return true;
+            };
+            const ConnectorBinding* a = blocks[j].input("A");
+            const ConnectorBinding* b = f->has_b() ? blocks[j].input("B") : nullptr;
+            const bool a_is_link = a && !a->is_constant && a->data == link && f->a_shape() == shape;
+            const bool b_is_link = b && !b->is_constant && b->data == link && f->b_shape() == shape;
+            std::string bias;
+            if (f->has_b()) {
+                if (f->binary() != "ml::Add" || a_is_link == b_is_link) continue;
+                const ConnectorBinding* other = a_is_link ? b : a;
+                if (other->is_constant || !sdfg.container(other->data).is_pointer || !is_row(a_is_link ? f->b_shape() : f->a_shape())) continue;
+                if (shape.size() > 1 && gemm->m() == "1") continue;   // a [1, n] operand is ambiguous with the full shape
+                bias = other->data;
+                if (!unwritten_between(sdfg, bias, i, j)) continue;
+            } else if (!a_is_link) {
+                continue;
+            }
+            std::vector<std::string> post = f->post();
+            std::string activation;
+            if (!post.empty() && (post[0] == "ml::ReLU" || post[0] == "ml::Abs")) {
+                activation = post[0];
+                post.erase(post.begin());
+            }
+            if (bias.empty() && activation.empty()) continue;
+            const std::string result = blocks[j].outputs[0].data;
+            if (post.empty()) {
+                // the whole chain is in the store: the GEMM writes the chain's result
+                if (!untouched_between(sdfg, result, i, j) || result == bias) continue;
+                bool operand_is_result = false;
+                for (auto& in : blocks[i].inputs)
+                    if (!in.is_constant && in.data == result) operand_is_result = true;
+                if (operand_is_result) continue;   // A or B would be overwritten while it is read
+                gemm->set_epilogue(!bias.empty(), activation);
+                for (auto& in : blocks[i].inputs)
+                    if (in.connector == "__C") in.data = result;
+                blocks[i].outputs[0].data = result;
+                if (!bias.empty()) blocks[i].inputs.push_back(make_binding("__bias", bias));
+                blocks.erase(blocks.begin() + (long) j);
+                sdfg.remove_container(link);
+            } else {
+                gemm->set_epilogue(!bias.empty(), activation);
+                if (!bias.empty()) blocks[i].inputs.push_back(make_binding("__bias", bias));
+                auto rest = std::make_unique<ROCMFusedElementWiseNode>(f->implementation_type(), shape, f->element(), "", shape,
+                                                                       std::vector<Expression>{}, post);
+                rest->set_element_id(f->element_id());
+                std::vector<ConnectorBinding> inputs{make_binding("A", link)};
+                blocks[j].inputs = std::move(inputs);
+                blocks[j].node = std::move(rest);
+            }
+            changed = applied = true;
+        }
     }
     return applied;
 }
@@ -723,13 +830,6 @@ bool RocmElementwiseFusionPass::run_pass(builder::StructuredSDFGBuilder& builder
 // ------------------------------------------------------------------------------ offloading
 
 namespace {
-
-ConnectorBinding make_binding(const std::string& connector, const std::string& data) {
-    ConnectorBinding b;
-    b.connector = connector;
-    b.data = data;
-    return b;
-}
 
 bool is_offloading(const Block& b) { return b.node->code() == LibraryNodeType_ROCM_Offloading; }
 

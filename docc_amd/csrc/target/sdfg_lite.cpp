@@ -144,6 +144,13 @@ GEMMNode::GEMMNode(std::string implementation_type, BLAS_Precision precision, BL
       precision_(precision), layout_(layout), trans_a_(trans_a), trans_b_(trans_b), m_(std::move(m)), n_(std::move(n)),
       k_(std::move(k)), lda_(std::move(lda)), ldb_(std::move(ldb)), ldc_(std::move(ldc)) {}
 
+void GEMMNode::set_epilogue(bool bias, std::string activation) {
+    if (bias && !epilogue_bias_) inputs_.push_back("__bias");
+    if (!bias && epilogue_bias_) inputs_.erase(std::remove(inputs_.begin(), inputs_.end(), std::string("__bias")), inputs_.end());
+    epilogue_bias_ = bias;
+    epilogue_activation_ = std::move(activation);
+}
+
 void GEMMNode::validate() const {
     if (precision_ != h && precision_ != s && precision_ != d && precision_ != b)
         throw InvalidSDFGException("GEMM: unsupported precision");
@@ -152,6 +159,8 @@ void GEMMNode::validate() const {
         if (t != No && t != Trans && t != ConjTrans) throw InvalidSDFGException("GEMM: bad transpose code");
     for (auto* e : {&m_, &n_, &k_, &lda_, &ldb_, &ldc_})
         if (e->empty()) throw InvalidSDFGException("GEMM: empty dimension expression");
+    if (!epilogue_activation_.empty() && epilogue_activation_ != "ml::ReLU" && epilogue_activation_ != "ml::Abs")
+        throw InvalidSDFGException("GEMM: only ml::ReLU and ml::Abs can be part of the store, not " + epilogue_activation_);
 }
 
 Expression GEMMNode::flop() const {
@@ -171,14 +180,22 @@ void GEMMNode::to_json(Value& j) const {
     j.set("lda", lda_);
     j.set("ldb", ldb_);
     j.set("ldc", ldc_);
+    if (has_epilogue()) {
+        j.set("epilogue_bias", epilogue_bias_);
+        j.set("epilogue_activation", epilogue_activation_);
+    }
 }
 
 std::unique_ptr<GEMMNode> GEMMNode::from_json(const Value& j) {
-    return std::make_unique<GEMMNode>(impl_of(j), (BLAS_Precision) j.at("precision").as_int(),
-                                      (BLAS_Layout) j.at("layout").as_int(), (BLAS_Transpose) j.at("trans_a").as_int(),
-                                      (BLAS_Transpose) j.at("trans_b").as_int(), j.at("m").as_expression(),
-                                      j.at("n").as_expression(), j.at("k").as_expression(), j.at("lda").as_expression(),
-                                      j.at("ldb").as_expression(), j.at("ldc").as_expression());
+    auto node = std::make_unique<GEMMNode>(impl_of(j), (BLAS_Precision) j.at("precision").as_int(),
+                                           (BLAS_Layout) j.at("layout").as_int(), (BLAS_Transpose) j.at("trans_a").as_int(),
+                                           (BLAS_Transpose) j.at("trans_b").as_int(), j.at("m").as_expression(),
+                                           j.at("n").as_expression(), j.at("k").as_expression(), j.at("lda").as_expression(),
+                                           j.at("ldb").as_expression(), j.at("ldc").as_expression());
+    const Value* eb = j.find("epilogue_bias");
+    const Value* ea = j.find("epilogue_activation");
+    if (eb || ea) node->set_epilogue(eb && eb->as_bool(), ea ? ea->as_string() : "");
+    return node;
 }
 
 Expression GEMMNode::connector_bytes(const std::string& connector) const {
@@ -186,6 +203,7 @@ Expression GEMMNode::connector_bytes(const std::string& connector) const {
     if (connector == "__A") return bytes_of(symbolic::mul(trans_a_ == No ? m_ : k_, lda_), precision_input_type(precision_));
     if (connector == "__B") return bytes_of(symbolic::mul(trans_b_ == No ? k_ : n_, ldb_), precision_input_type(precision_));
     if (connector == "__C") return bytes_of(symbolic::mul(m_, ldc_), precision_output_type(precision_));
+    if (connector == "__bias") return bytes_of(n_, precision_output_type(precision_));
     return "0";
 }
 

@@ -147,6 +147,15 @@ public:
     const Expression& ldc() const { return ldc_; }
     types::PrimitiveType scalar_primitive() const { return precision_input_type(precision_); }
 
+    // Set by the rocm target's fusion pass only (the reference's node has neither): the rest of a dense
+    // layer in the store, C = act(alpha A B + beta C + bias[column]). `bias` adds the input connector
+    // "__bias" (n values of C's type); `activation` is an elementwise node code or "". JSON keys
+    // "epilogue_bias" / "epilogue_activation", written only when set.
+    void set_epilogue(bool bias, std::string activation);
+    bool epilogue_bias() const { return epilogue_bias_; }
+    const std::string& epilogue_activation() const { return epilogue_activation_; }
+    bool has_epilogue() const { return epilogue_bias_ || !epilogue_activation_.empty(); }
+
     void validate() const override;
     Expression flop() const override;
     void to_json(json::Value& j) const override;
@@ -159,6 +168,8 @@ private:
     BLAS_Layout layout_;
     BLAS_Transpose trans_a_, trans_b_;
     Expression m_, n_, k_, lda_, ldb_, ldc_;
+    bool epilogue_bias_ = false;
+    std::string epilogue_activation_;
 };
 
 } // namespace math::blas

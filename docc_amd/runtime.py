@@ -62,6 +62,9 @@ _SIGNATURES = {
     "docc_rocm_dgemm": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _vp, _i64, _f64, _vp, _i64],
     "docc_rocm_sgemm": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64],
     "docc_rocm_bf16gemm_f32": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64],
+    "docc_rocm_dgemm_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _vp, _i64, _f64, _vp, _i64, _vp, _int],
+    "docc_rocm_sgemm_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64, _vp, _int],
+    "docc_rocm_bf16gemm_f32_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64, _vp, _int],
     "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
@@ -200,6 +203,15 @@ def sgemm(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, trans_a=NO_TRANS, trans_
 
 def bf16gemm_f32(m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, trans_a=NO_TRANS, trans_b=NO_TRANS, stream=0) -> None:
     call("docc_rocm_bf16gemm_f32", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
+
+
+def gemm_epilogue(kind, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias=None, activation=None, trans_a=NO_TRANS,
+                  trans_b=NO_TRANS, stream=0) -> None:
+    """C = act(alpha * op(A) op(B) + beta * C + bias[column]); kind "d", "s" or "b" (bf16 inputs),
+    bias a device address or None, activation the name of a unary operation or None."""
+    fn = {"d": "docc_rocm_dgemm_epilogue", "s": "docc_rocm_sgemm_epilogue", "b": "docc_rocm_bf16gemm_f32_epilogue"}[kind]
+    act = -1 if activation is None else (UNARY_OPS[activation] if isinstance(activation, str) else activation)
+    call(fn, stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias or None, act)
 
 
 def softmax_f32(rows, cols, X, Y, stream=0) -> None:

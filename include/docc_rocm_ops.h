@@ -62,6 +62,27 @@ int docc_rocm_bf16gemm_f32(docc_rocm_stream_t stream, int trans_a, int trans_b, 
                            float beta, float* C, int64_t ldc);
 
 /*
+ * GEMM with the rest of a dense layer in its epilogue:
+ *     C = act(alpha * op(A) op(B) + beta * C + bias[column])
+ * `bias`: n values or NULL; `activation`: DOCC_ROCM_UNARY_RELU, DOCC_ROCM_UNARY_ABS (below) or -1
+ * (the other unary operations are not built into the store: DOCC_ROCM_ERR_UNSUPPORTED). The sum is
+ * rounded after each step, as the GEMM node followed by ml::Add (of the bias row, through
+ * ml::Broadcast) and the unary node would round it; this is what the target's fusion pass emits
+ * for that chain, so that C is written once instead of being re-read by every node. The
+ * reference has no such form: its cuBLAS dispatcher calls plain gemm
+ * (opt/src/targets/cuda/blas/gemm.cpp:66-96) and the epilogue stays a Map.
+ */
+int docc_rocm_dgemm_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                             double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta,
+                             double* C, int64_t ldc, const double* bias, int activation);
+int docc_rocm_sgemm_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                             float alpha, const float* A, int64_t lda, const float* B, int64_t ldb, float beta, float* C,
+                             int64_t ldc, const float* bias, int activation);
+int docc_rocm_bf16gemm_f32_epilogue(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                                    float alpha, const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb,
+                                    float beta, float* C, int64_t ldc, const float* bias, int activation);
+
+/*
  * Y[r, :] = softmax(X[r, :]) for r in [0, rows), fp32, both [rows, cols]
  * contiguous. This is ml::Softmax over the last axis; any reduction over a
  * trailing contiguous axis of an N-d tensor is this call with

@@ -75,11 +75,11 @@ def test_brackets_in_the_generated_code(tmp_path):
         assert piece in flat, piece
     # init < enter < launch < exit < metric < finalize
     order = [flat.index(k) for k in (f"__daisy_instrumentation_init(&{stem}_md", f"__daisy_instrumentation_enter({stem}_id)",
-                                     "docc_rocm_sgemm(", f"__daisy_instrumentation_exit({stem}_id)",
+                                     "docc_rocm_sgemm_epilogue(", f"__daisy_instrumentation_exit({stem}_id)",
                                      f"__daisy_instrumentation_metric({stem}_id", f"__daisy_instrumentation_finalize({stem}_id)")]
     assert order == sorted(order)
     # math nodes and transfers are regions; allocations and frees are not
-    assert flat.count("__daisy_instrumentation_enter(") == 2 + 2 + 1      # GEMM, ReLU; A, B up; C down
+    assert flat.count("__daisy_instrumentation_enter(") == 1 + 2 + 1      # the GEMM with the ReLU in its store; A, B up; C down
     with pytest.raises(InvalidSDFGException, match="Unsupported instrumentation plan: loops"):
         s.generate(str(tmp_path / "bad"), "loops")
     with pytest.raises(NotImplementedError, match="capture"):

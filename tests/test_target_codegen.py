@@ -323,26 +323,76 @@ def test_elementwise_with_transfers_and_scalar_on_the_left(tmp_path):
 
 
 def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
-    """relu(X @ W + bias) * 0.5: the Broadcast moves into the Add, the ReLU into the Add; the multiplication by
-    a constant is a binary node of its own and stays. GEMM + two elementwise launches instead of five."""
+    """relu(X @ W + bias) * 0.5: the Broadcast moves into the Add, the ReLU into the Add, and the whole chain into
+    the store of the GEMM; the multiplication by a constant is a binary node of its own and stays. Two
+    launches instead of five, the intermediates gone."""
     s = dense_sdfg()
     s.schedule("rocm")
     r = s.loop_report()
-    assert r["GEMM"] == 1 and r["ROCMFusedElementWise"] == 1 and r["ml::Mul"] == 1
-    assert "ml::Broadcast" not in r and "ml::Add" not in r and "ml::ReLU" not in r
+    assert r["GEMM"] == 1 and r["ml::Mul"] == 1
+    for gone in ("ml::Broadcast", "ml::Add", "ml::ReLU", "ROCMFusedElementWise"):
+        assert gone not in r
     assert r["H2D"] == 3 and r["D2H"] == 1
-    assert set(s.containers) >= {"T0", "T3"} and "T1" not in s.containers and "T2" not in s.containers
+    assert "T3" in s.containers and not {"T0", "T1", "T2"} & set(s.containers)
+    gemm = next(n for n in s.library_nodes() if n["code"] == "GEMM")
+    assert gemm["epilogue_bias"] is True and gemm["epilogue_activation"] == "ml::ReLU" and gemm["implementation_type"] == "ROCMWithoutTransfers"
+    strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]       # ids are renumbered by a parse
+    assert strip(StructuredSDFG.parse(s.to_json()).library_nodes()) == strip(s.library_nodes())    # the epilogue fields serialise
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path)[0])
+    assert ("docc_rocm_sgemm_epilogue(nullptr, 111, 111, 32, 16, 8, __alpha, (const float *) __A, 8, (const float *) __B, 16, __beta, "
+            "(float *) __C, 16, (const float *) __bias, 2 /* ml::ReLU */)") in flat
+    assert "float *__bias = __daisy_rocm_" in flat
+    assert flat.count("docc_rocm_malloc(") == 5      # X W bias on the device, T3, Y
+
+    # without the GEMM in front the chain is one elementwise launch
+    b = StructuredSDFGBuilder("ew")
+    for n in ("A", "bias", "Y"):
+        b.add_container(n, F32, True)
+    for n in ("T1", "T2"):
+        b.add_container(n, F32, False, transient_bytes=32 * 16 * 4)
+    b.add_broadcast("bias", "T1", [1, 16], [32, 16])
+    b.add_elementwise_op("add", "A", "T1", "T2", [32, 16])
+    b.add_elementwise_unary_op("relu", "T2", "Y", [32, 16])
+    s = b.move()
+    s.schedule("rocm")
     fused = next(n for n in s.library_nodes() if n["code"] == "ROCMFusedElementWise")
     assert fused["binary"] == "ml::Add" and fused["a_shape"] == ["32", "16"] and fused["b_shape"] == ["1", "16"]
     assert fused["post"] == ["ml::ReLU"] and fused["implementation_type"] == "ROCMWithoutTransfers"
-    strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]       # ids are renumbered by a parse
-    assert strip(StructuredSDFG.parse(s.to_json()).library_nodes()) == strip(s.library_nodes())    # the fused node serialises
-    flat = re.sub(r"\s+", " ", source_of(s, tmp_path)[0])
+    assert strip(StructuredSDFG.parse(s.to_json()).library_nodes()) == strip(s.library_nodes())
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "ew")[0])
     assert "const int64_t __docc_b_shape[] = {(int64_t) (1), (int64_t) (16)};" in flat
     assert "const int __docc_post[] = {2 /* ml::ReLU */};" in flat
     assert ("docc_rocm_elementwise_fused(nullptr, 32, 2, __docc_shape, 0 /* ml::Add */, __docc_a_shape, A, 0.0, __docc_b_shape, B, 0.0, "
             "1, __docc_post, Y)") in flat
-    assert flat.count("docc_rocm_malloc(") == 6      # X W bias on the device, T0, T3, Y: two intermediates fewer
+
+    # an activation that is not one instruction stays behind the GEMM; the bias still moves into the store
+    b = StructuredSDFGBuilder("tanh_layer")
+    for n in ("X", "W", "bias", "Y"):
+        b.add_container(n, F64, True)
+    for n in ("T0", "T1", "T2"):
+        b.add_container(n, F64, False, transient_bytes=32 * 16 * 8)
+    b.add_gemm("X", "W", "T0", "1.0", "0.0", 32, 16, 8)
+    b.add_broadcast("bias", "T1", [1, 16], [32, 16])
+    b.add_elementwise_op("add", "T1", "T0", "T2", [32, 16])      # bias on the left
+    b.add_elementwise_unary_op("tanh", "T2", "Y", [32, 16])
+    s = b.move()
+    s.schedule("rocm")
+    nodes = [n for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert [n["code"] for n in nodes] == ["GEMM", "ROCMFusedElementWise"]
+    assert nodes[0]["epilogue_bias"] is True and nodes[0]["epilogue_activation"] == ""
+    assert nodes[1]["binary"] == "" and nodes[1]["post"] == ["ml::Tanh"]
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "tanh")[0])
+    assert "(const double *) __bias, -1)" in flat and "docc_rocm_dgemm_epilogue(" in flat
+
+    # beta != 0 makes the GEMM a reader of its own output: the chain is left alone; so is a C with a padded leading dimension
+    b = StructuredSDFGBuilder("acc")
+    for n in ("X", "W", "T0", "Y"):
+        b.add_container(n, F32, True)
+    b.add_gemm("X", "W", "T0", "1.0", "1.0", 32, 16, 8)
+    b.add_elementwise_unary_op("relu", "T0", "Y", [32, 16])
+    s = b.move()
+    s.schedule("rocm")
+    assert "epilogue_activation" not in next(n for n in s.library_nodes() if n["code"] == "GEMM")
 
     # unary chains fold too, up to four operations; a value that something else reads is not folded away
     b = StructuredSDFGBuilder("chain")
