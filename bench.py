@@ -223,7 +223,12 @@ def main():
                    "sample": f"first {rows} rows of C ({rows}x4096x4096), the reference's expanded loop nest",
                    "host_blas_tflops": round(2 * n**3 / tb / 1e12, 4), "host_blas": "numpy/OpenBLAS sgemm, full 4096^3"}
         add_kernel("sgemm_4096", "f32", 2 * n**3, ms, cpu)
-        del A, B, Cm
+        # the same product with bias row + ReLU in its store (what the fusion pass makes of a dense layer)
+        bias = torch.randn(n, device="cuda")
+        ms_e = time_kernel(lambda i: rt.gemm_epilogue("s", n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n,
+                                                      bias.data_ptr(), "relu", stream=stream), 20, 3)
+        add_kernel("sgemm_4096_bias_relu", "f32", 2 * n**3, ms_e)
+        del A, B, Cm, bias
 
     # ---- config 3b: bf16 GEMM 4096^3, fp32 accumulate/output ------------------------------
     if want("bgemm"):

@@ -97,16 +97,30 @@ __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const Broadca
     const int last = p.rank - 1;
     const I inner = (I) p.out_dims[last] / VEC;
     const bool inner_repeats = p.in_strides[last] == 0;
-    for (I v = (I) blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += stride) {
-        I rem = v / inner;
-        long off = inner_repeats ? 0 : (long) (v % inner) * VEC;
+    // position of the lane's vector as (row, column) of the innermost dimension, advanced without divisions
+    I v = (I) blockIdx.x * blockDim.x + threadIdx.x;
+    I col = v % inner, row = v / inner;
+    const I step_col = stride % inner, step_row = stride / inner;
+    for (; v < nv; v += stride) {
+        long off = inner_repeats ? 0 : (long) col * VEC;
+        if (p.rank == 2) {
+            off += (long) row * p.in_strides[0];
+        } else if (p.rank > 2) {
+            I rem = row;
 #pragma unroll
-        for (int d = 4; d >= 0; d--) {
-            if (d < last) {
-                const I e = (I) p.out_dims[d];
-                off += (long) (rem % e) * p.in_strides[d];
-                rem /= e;
+            for (int d = 4; d >= 0; d--) {
+                if (d < last) {
+                    const I e = (I) p.out_dims[d];
+                    off += (long) (rem % e) * p.in_strides[d];
+                    rem /= e;
+                }
             }
+        }
+        col += step_col;
+        row += step_row;
+        if (col >= inner) {
+            col -= inner;
+            row++;
         }
         V y;
         if (inner_repeats) {
@@ -134,6 +148,7 @@ struct FusedParams {
     long b_strides[6];
     int binary;             // BinaryOp or -1
     int a_scalar, b_scalar; // operand is the scalar below instead of an array
+    int a_reused, b_reused; // operand repeats along some dimension: keep it in the caches
     double scalar_a, scalar_b;
     int npost;
     int post[4];            // UnaryOp codes
@@ -148,26 +163,40 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
     const I inner = (I) p.dims[last] / VEC;
     const bool a_inner = !p.a_scalar && p.a_strides[last] != 0, b_inner = !p.b_scalar && p.b_strides[last] != 0;
     const bool has_b = p.binary >= 0;
-    for (I v = (I) blockIdx.x * blockDim.x + threadIdx.x; v < nv; v += stride) {
-        I rem = v / inner;
-        const long in = (long) (v % inner) * VEC;
+    I v = (I) blockIdx.x * blockDim.x + threadIdx.x;
+    I col = v % inner, row = v / inner;
+    const I step_col = stride % inner, step_row = stride / inner;
+    for (; v < nv; v += stride) {
+        const long in = (long) col * VEC;
         long oa = a_inner ? in : 0, ob = b_inner ? in : 0;
+        if (p.rank == 2) {
+            oa += (long) row * p.a_strides[0];
+            ob += (long) row * p.b_strides[0];
+        } else if (p.rank > 2) {
+            I rem = row;
 #pragma unroll
-        for (int d = 4; d >= 0; d--) {
-            if (d < last) {
-                const I e = (I) p.dims[d];
-                const long c = (long) (rem % e);
-                rem /= e;
-                oa += c * p.a_strides[d];
-                ob += c * p.b_strides[d];
+            for (int d = 4; d >= 0; d--) {
+                if (d < last) {
+                    const I e = (I) p.dims[d];
+                    const long c = (long) (rem % e);
+                    rem /= e;
+                    oa += c * p.a_strides[d];
+                    ob += c * p.b_strides[d];
+                }
             }
+        }
+        col += step_col;
+        row += step_row;
+        if (col >= inner) {
+            col -= inner;
+            row++;
         }
         V a, b;
         if (p.a_scalar) {
 #pragma unroll
             for (int e = 0; e < VEC; e++) a[e] = (T) p.scalar_a;
         } else if (a_inner) {
-            a = __builtin_nontemporal_load(reinterpret_cast<const V*>(A + oa));
+            a = p.a_reused ? *reinterpret_cast<const V*>(A + oa) : __builtin_nontemporal_load(reinterpret_cast<const V*>(A + oa));
         } else {
             const T x = A[oa];
 #pragma unroll
@@ -178,7 +207,7 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
 #pragma unroll
                 for (int e = 0; e < VEC; e++) b[e] = (T) p.scalar_b;
             } else if (b_inner) {
-                b = __builtin_nontemporal_load(reinterpret_cast<const V*>(B + ob));
+                b = p.b_reused ? *reinterpret_cast<const V*>(B + ob) : __builtin_nontemporal_load(reinterpret_cast<const V*>(B + ob));
             } else {
                 const T x = B[ob];
 #pragma unroll

@@ -38,6 +38,7 @@ struct FusedParams {
     long b_strides[6];
     int binary;
     int a_scalar, b_scalar;
+    int a_reused, b_reused;
     double scalar_a, scalar_b;
     int npost;
     int post[4];
@@ -226,6 +227,10 @@ extern "C" int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precis
     }
     p.rank = r;
     p.n = n;
+    for (int d = 0; d < r; d++) {
+        if (p.a_strides[d] == 0) p.a_reused = 1;
+        if (p.b_strides[d] == 0) p.b_reused = 1;
+    }
     const int per_vec = precision == 32 ? 4 : 2;
     auto vector_ok = [&](bool scalar, const void* ptr, long inner_stride) {
         return scalar || inner_stride == 0 || (inner_stride == 1 && (uintptr_t) ptr % 16 == 0);
