@@ -49,6 +49,7 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the PCIe-inclusive calls through @native")
     return ap.parse_args()
 
 
@@ -307,6 +308,43 @@ def main():
                 "sample": "full tensor, the Map the reference's ElementWiseBinaryNode expands to (omp parallel for)"}
         del a, b2, y
 
+    # ---- PCIe-inclusive: host arrays in, host array out, through @native (never the reported `value`) ----
+    end_to_end = {}
+    if not args.no_e2e and (want("softmax") or want("dgemm")):
+        import scipy.special
+
+        from docc_amd.python import native
+
+        os.environ.setdefault("DOCC_TMP", str(Path(tempfile.gettempdir()) / f"docc_bench_{os.getpid()}"))
+
+        @native(target="rocm")
+        def softmax_native(x):
+            return scipy.special.softmax(x, axis=-1)
+
+        @native(target="rocm")
+        def matmul_native(a, b):
+            return a @ b
+
+        def host_time(fn, reps=5):
+            fn()  # JIT compilation and the first launch
+            ts = []
+            for _ in range(reps):
+                t0 = time.perf_counter()
+                fn()
+                ts.append(time.perf_counter() - t0)
+            return statistics.median(ts)
+
+        if want("softmax"):
+            xh = (np.random.default_rng(1).standard_normal((8192, 4096)) * 8).astype(np.float32)
+            t = host_time(lambda: softmax_native(xh))
+            end_to_end["softmax_f32_8192x4096"] = {"ms": round(t * 1e3, 2), "GBps": round(2 * xh.nbytes / t / 1e9, 1),
+                                                   "moved_over_pcie_bytes": 2 * xh.nbytes}
+        if want("dgemm"):
+            rng = np.random.default_rng(0)
+            ah, bh = rng.random((1000, 1000)), rng.random((1000, 1000))
+            t = host_time(lambda: matmul_native(ah, bh))
+            end_to_end["dgemm_1000"] = {"ms": round(t * 1e3, 2), "tflops": round(2e9 / t / 1e12, 3), "moved_over_pcie_bytes": 3 * ah.nbytes}
+
     line = {
         "metric": METRIC,
         "value": round(out.get("value", 0.0), 1),
@@ -328,6 +366,8 @@ def main():
     if "cpu_baseline" in out:
         line["cpu_baseline"] = out["cpu_baseline"]
     line["kernels"] = kernels
+    if end_to_end:
+        line["end_to_end_through_native"] = end_to_end
     print(json.dumps(line))
 
 
