@@ -300,6 +300,15 @@ def main():
                 "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
                 "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(gbs / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_e}}
+        # reduce nodes on the same tensor: over the rows' extent (one wavefront per row) and over the rows (one lane per column)
+        for name, (outer, extent, inner) in {"sum_rows_f32": (8192, 4096, 1), "max_columns_f32": (1, 8192, 4096)}.items():
+            op = name.split("_")[0]
+            ms = time_kernel(lambda i: rt.reduce(op, 32, outer, extent, inner, a.data_ptr(), y.data_ptr(), stream), 50, 5)
+            nbytes_r = 4 * n + 4 * outer * inner
+            kernels[f"reduce_{name}_8192x4096"] = {
+                "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
+                "roofline": {"bound": "hbm", "achieved": round(nbytes_r / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                             "frac": round(nbytes_r / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_r}}
         if oracle_lib is not None:
             ah, bh = a.cpu().numpy(), b2.cpu().numpy()
             t = cpu_time(lambda: oracle.elementwise_binary("add", ah, bh, lib=oracle_lib))

@@ -47,6 +47,7 @@ KERNEL_FAMILIES = {
     "conv2d": "conv2d.hip",
     "attention": "attention.hip",
     "elementwise": "elementwise.hip",
+    "reduce": "reduce.hip",
 }
 
 # Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary

@@ -1,0 +1,206 @@
+// Reduce tensor nodes (ml::Sum, ml::Max, ml::Min, ml::Mean) over a block of adjacent axes, fp32
+// and fp64, for gfx950.
+//
+// The reference expands a ReduceNode into an initialisation nest and a nest that accumulates
+// through memory, left to right (sdfg/src/data_flow/library_nodes/math/tensor/reduce_node.cpp:
+// 188-333; identities and combiners: sum_node.cpp:20-57 `0` and `+`, max_node.cpp:56-91
+// `-INFINITY` and fmax, min_node.cpp `INFINITY` and fmin; Mean is Sum followed by a division by
+// the number of reduced elements, mean_node.cpp). Here the input is seen as [outer, reduce, inner]:
+//   inner == 1  one wavefront per output element: 128-bit loads strided over the wave, a tree
+//               over the lanes at the end (HBM-bound: one read of X)
+//   inner  > 1  one lane per output element, walking the reduced extent with stride `inner`, so
+//               that neighbouring lanes read neighbouring addresses; when there are too few
+//               output elements to fill the device the reduced extent is cut into slices, one
+//               work-group row per slice, whose partial results go through a scratch array in
+//               device memory and are combined, in slice order, by a second launch
+// Sums are therefore added in another order than the reference's loop: equal to it within the
+// usual bound (reduce * epsilon * sum|x|), exactly equal for Max and Min.
+#include "common.h"
+
+namespace docc_k {
+
+enum ReduceOp : int { kSum = 0, kMax = 1, kMin = 2, kMean = 3 };
+
+template <int OP, typename T>
+__device__ __forceinline__ T reduce_identity() {
+    if (OP == kMax) return -__builtin_huge_val();
+    if (OP == kMin) return __builtin_huge_val();
+    return (T) 0;
+}
+
+template <int OP>
+__device__ __forceinline__ float combine(float a, float b) {
+    if (OP == kMax) return fmaxf(a, b);
+    if (OP == kMin) return fminf(a, b);
+    return a + b;
+}
+template <int OP>
+__device__ __forceinline__ double combine(double a, double b) {
+    if (OP == kMax) return fmax(a, b);
+    if (OP == kMin) return fmin(a, b);
+    return a + b;
+}
+
+template <int OP, typename T>
+__device__ __forceinline__ T wave_combine(T v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = combine<OP>(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Y[row] = reduce over X[row, 0..R); nvec = R / VEC when rows are 16-byte aligned, else 0
+template <typename T, int OP, int VEC>
+__device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, long nvec) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    const int lane = threadIdx.x & 63;
+    const long waves = (long) gridDim.x * (blockDim.x >> 6);
+    for (long row = (long) blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const T* x = X + row * R;
+        T acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = reduce_identity<OP, T>();
+        for (long i = lane; i < nvec; i += kWave) {
+            const V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(x) + i);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc[e] = combine<OP>(acc[e], v[e]);
+        }
+        T a = acc[0];
+#pragma unroll
+        for (int e = 1; e < VEC; e++) a = combine<OP>(a, acc[e]);
+        for (long i = nvec * VEC + lane; i < R; i += kWave) a = combine<OP>(a, x[i]);
+        a = wave_combine<OP>(a);
+        if (lane == 0) Y[row] = OP == kMean ? a / (T) R : a;
+    }
+}
+
+// Y[o, i] = reduce over r of X[o, r, i]
+template <typename T, int OP>
+__device__ __forceinline__ void column_reduce(const T* X, T* Y, long outer, long R, long inner) {
+    const long total = outer * inner;
+    const long stride = (long) gridDim.x * blockDim.x;
+    for (long idx = (long) blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+        const long o = idx / inner, i = idx % inner;
+        const T* x = X + o * R * inner + i;
+        T a0 = reduce_identity<OP, T>(), a1 = a0, a2 = a0, a3 = a0;
+        long r = 0;
+        for (; r + 4 <= R; r += 4) {   // four independent chains keep the loads in flight
+            a0 = combine<OP>(a0, x[(r + 0) * inner]);
+            a1 = combine<OP>(a1, x[(r + 1) * inner]);
+            a2 = combine<OP>(a2, x[(r + 2) * inner]);
+            a3 = combine<OP>(a3, x[(r + 3) * inner]);
+        }
+        for (; r < R; r++) a0 = combine<OP>(a0, x[r * inner]);
+        const T a = combine<OP>(combine<OP>(a0, a1), combine<OP>(a2, a3));
+        Y[idx] = OP == kMean ? a / (T) R : a;
+    }
+}
+
+// Partial results of the sliced column reduction: [slice][outer * inner] elements. Every call
+// that slices writes the part it reads back, so nothing has to be cleared; calls that overlap
+// on one device (different streams) would share it and must not.
+constexpr long kReduceScratchBytes = 8L << 20;
+__device__ __attribute__((aligned(256))) unsigned char docc_reduce_scratch[kReduceScratchBytes];
+
+// P[s, o, i] = reduce over the rows of slice s of X[o, r, i]; grid.y = number of slices. Each lane
+// owns VEC neighbouring columns (inner % VEC == 0, X 16-byte aligned when VEC > 1): one 128-bit load
+// per row.
+template <typename T, int OP, int VEC>
+__device__ __forceinline__ void column_reduce_partial(const T* X, long outer, long R, long inner, long chunk) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    T* P = reinterpret_cast<T*>(docc_reduce_scratch);
+    const long total = outer * inner;
+    const long idx = ((long) blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    if (idx >= total) return;
+    const long r0 = (long) blockIdx.y * chunk, r1 = min(R, r0 + chunk);
+    const long o = idx / inner, i = idx % inner;
+    const T* x = X + o * R * inner + i;
+    V a0, a1;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) a0[e] = a1[e] = reduce_identity<OP, T>();
+    long r = r0;
+    for (; r + 2 <= r1; r += 2) {   // two independent chains keep the loads in flight
+        const V v0 = __builtin_nontemporal_load(reinterpret_cast<const V*>(x + (r + 0) * inner));
+        const V v1 = __builtin_nontemporal_load(reinterpret_cast<const V*>(x + (r + 1) * inner));
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            a0[e] = combine<OP>(a0[e], v0[e]);
+            a1[e] = combine<OP>(a1[e], v1[e]);
+        }
+    }
+    for (; r < r1; r++) {
+        const V v0 = *reinterpret_cast<const V*>(x + r * inner);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) a0[e] = combine<OP>(a0[e], v0[e]);
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; e++) a0[e] = combine<OP>(a0[e], a1[e]);
+    *reinterpret_cast<V*>(P + (long) blockIdx.y * total + idx) = a0;
+}
+
+// Y[idx] = combine over the slices of P[s, idx]. A work-group takes 16 neighbouring output
+// elements; 16 lanes per element each combine every 16th slice, then one lane combines the 16
+// partial values in order (the order of the additions is fixed by the launch geometry alone).
+template <typename T, int OP>
+__device__ __forceinline__ void column_reduce_final(T* Y, long total, long R, long slices) {
+    __shared__ T part[16][17];
+    const T* P = reinterpret_cast<const T*>(docc_reduce_scratch);
+    const int col = threadIdx.x & 15, lane_s = threadIdx.x >> 4;
+    const long idx = (long) blockIdx.x * 16 + col;
+    T a = reduce_identity<OP, T>();
+    if (idx < total)
+        for (long s = lane_s; s < slices; s += 16) a = combine<OP>(a, P[s * total + idx]);
+    part[lane_s][col] = a;
+    __syncthreads();
+    if (lane_s == 0 && idx < total) {
+        T r = part[0][col];
+#pragma unroll
+        for (int k = 1; k < 16; k++) r = combine<OP>(r, part[k][col]);
+        Y[idx] = OP == kMean ? r / (T) R : r;
+    }
+}
+
+} // namespace docc_k
+
+#define DOCC_REDUCE(NAME, OP)                                                                                                  \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_row_##NAME##_f32(const float* X, float* Y, long rows, long R,   \
+                                                                                   long nvec) {                                \
+        docc_k::row_reduce<float, docc_k::OP, 4>(X, Y, rows, R, nvec);                                                         \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_row_##NAME##_f64(const double* X, double* Y, long rows, long R, \
+                                                                                   long nvec) {                                \
+        docc_k::row_reduce<double, docc_k::OP, 2>(X, Y, rows, R, nvec);                                                        \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_col_##NAME##_f32(const float* X, float* Y, long outer, long R,  \
+                                                                                   long inner) {                               \
+        docc_k::column_reduce<float, docc_k::OP>(X, Y, outer, R, inner);                                                       \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_col_##NAME##_f64(const double* X, double* Y, long outer,        \
+                                                                                   long R, long inner) {                       \
+        docc_k::column_reduce<double, docc_k::OP>(X, Y, outer, R, inner);                                                      \
+    }
+
+#define DOCC_REDUCE_SLICED(NAME, OP, SFX, T)                                                                                   \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colp_##NAME##_##SFX(const T* X, long outer, long R, long inner, \
+                                                                                      long chunk) {                            \
+        docc_k::column_reduce_partial<T, docc_k::OP, 1>(X, outer, R, inner, chunk);                                            \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colpv_##NAME##_##SFX(const T* X, long outer, long R,            \
+                                                                                       long inner, long chunk) {               \
+        docc_k::column_reduce_partial<T, docc_k::OP, 16 / sizeof(T)>(X, outer, R, inner, chunk);                               \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colf_##NAME##_##SFX(T* Y, long total, long R, long slices) {    \
+        docc_k::column_reduce_final<T, docc_k::OP>(Y, total, R, slices);                                                       \
+    }
+
+DOCC_REDUCE(sum, kSum)
+DOCC_REDUCE(max, kMax)
+DOCC_REDUCE(min, kMin)
+DOCC_REDUCE(mean, kMean)
+DOCC_REDUCE_SLICED(sum, kSum, f32, float)
+DOCC_REDUCE_SLICED(sum, kSum, f64, double)
+DOCC_REDUCE_SLICED(max, kMax, f32, float)
+DOCC_REDUCE_SLICED(max, kMax, f64, double)
+DOCC_REDUCE_SLICED(min, kMin, f32, float)
+DOCC_REDUCE_SLICED(min, kMin, f64, double)
+DOCC_REDUCE_SLICED(mean, kMean, f32, float)
+DOCC_REDUCE_SLICED(mean, kMean, f64, double)

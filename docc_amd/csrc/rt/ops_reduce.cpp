@@ -1,0 +1,63 @@
+// Launcher for the reduce tensor nodes (see include/docc_rocm_ops.h).
+#include <cstdio>
+
+#include "docc_rocm_ops.h"
+#include "rt_state.h"
+
+using namespace docc::rt::rocm;
+
+extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision, int64_t outer, int64_t reduce, int64_t inner,
+                                const void* X, void* Y) {
+    static const char* const names[] = {"sum", "max", "min", "mean"};
+    if (op < 0 || op > DOCC_ROCM_REDUCE_MEAN) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "reduce: unknown operation %d", op);
+    if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "reduce: precision must be 32 or 64");
+    if (outer < 0 || reduce < 0 || inner < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "reduce: negative extent");
+    if (outer == 0 || inner == 0) return 0;
+    if (reduce == 0 && (op == DOCC_ROCM_REDUCE_MEAN))
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "reduce: mean over an empty extent");
+    if (!Y || (reduce > 0 && !X)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "reduce: null pointer");
+    if (int rc = ensure_device()) return rc;
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    char name[64];
+    if (inner == 1) {
+        const int per_vec = precision == 32 ? 4 : 2;
+        const size_t elem = precision / 8;
+        // every row starts on a 16-byte boundary
+        const bool aligned = (uintptr_t) X % 16 == 0 && (reduce * elem) % 16 == 0;
+        const long nvec = aligned ? (long) (reduce / per_vec) : 0;
+        int64_t blocks = (outer + 3) / 4;   // four wavefronts per work-group, one row each
+        if (blocks > (int64_t) cus * 16) blocks = (int64_t) cus * 16;
+        std::snprintf(name, sizeof(name), "docc_reduce_row_%s_f%d", names[op], precision);
+        return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) outer, (long) reduce, nvec);
+    }
+    const int64_t total = outer * inner;
+    int64_t blocks = (total + 255) / 256;
+    // Too few output elements to fill the device: cut the reduced extent into slices. Their partial
+    // results go through the kernels' 8 MiB scratch array (docc_reduce_scratch in reduce.hip).
+    if (blocks < (int64_t) cus * 2 && reduce >= 64) {
+        const int per_vec = 128 / precision;
+        const bool vec = inner % per_vec == 0 && (uintptr_t) X % 16 == 0;
+        const int64_t pblocks = vec ? (total / per_vec + 255) / 256 : blocks;
+        const int64_t scratch_elems = (int64_t(8) << 20) / (precision / 8);
+        int64_t slices = ((int64_t) cus * 8 + pblocks - 1) / pblocks;
+        if (slices > reduce / 16) slices = reduce / 16;
+        if (slices > scratch_elems / total) slices = scratch_elems / total;
+        if (slices > 256) slices = 256;
+        if (slices > 1) {
+            const int64_t chunk = (reduce + slices - 1) / slices;
+            slices = (reduce + chunk - 1) / chunk;
+            std::snprintf(name, sizeof(name), "docc_reduce_colp%s_%s_f%d", vec ? "v" : "", names[op], precision);
+            // the partial pass of a mean adds; the division happens once, in the final pass
+            if (int rc = launch(name, (uint32_t) pblocks, (uint32_t) slices, 1, 256, 0, (hipStream_t) stream, X, (long) outer,
+                                (long) reduce, (long) inner, (long) chunk))
+                return rc;
+            std::snprintf(name, sizeof(name), "docc_reduce_colf_%s_f%d", names[op], precision);
+            return launch(name, (uint32_t) ((total + 15) / 16), 1, 1, 256, 0, (hipStream_t) stream, Y, (long) total, (long) reduce,
+                          (long) slices);
+        }
+    }
+    if (blocks > (int64_t) cus * 16) blocks = (int64_t) cus * 16;
+    std::snprintf(name, sizeof(name), "docc_reduce_col_%s_f%d", names[op], precision);
+    return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) outer, (long) reduce, (long) inner);
+}

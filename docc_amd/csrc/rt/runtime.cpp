@@ -39,6 +39,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_conv2d.hsaco",
     "docc_rocm_attention.hsaco",
     "docc_rocm_elementwise.hsaco",
+    "docc_rocm_reduce.hsaco",
 };
 
 struct DeviceState {

@@ -34,7 +34,7 @@ bool is_math_node(const LibraryNode& node) {
     const std::string& c = node.code();
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
            c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
-           is_elementwise_code(c);
+           is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
 }
 
 // Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
@@ -418,6 +418,23 @@ protected:
     }
 };
 
+// ---- Reduce --------------------------------------------------------------------------------
+
+class ReduceNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::ReduceNode&>(node_);
+        const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
+        s << "DOCC_ROCM_CHECK(docc_rocm_reduce(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision << ", "
+          << n.outer() << ", " << n.extent() << ", " << n.inner() << ", " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+    }
+};
+
 // ---- fused elementwise chain ---------------------------------------------------------------
 
 class FusedElementWiseDispatcher_ROCM : public RocmMathDispatcher {
@@ -511,6 +528,7 @@ void register_plugin(plugins::Context& context) {
     for (auto& code : tensor::UnaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
+    for (auto& code : tensor::ReduceNodeCodes) register_math<ReduceNodeDispatcher_ROCM>(reg, code);
     register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
     reg.register_library_node_dispatcher(
         LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
@@ -572,6 +590,9 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         auto* e = dynamic_cast<tensor::ElementWiseNode*>(&node);
         if (!e) return decline("not an elementwise node object");
         if (e->element() != P::Float && e->element() != P::Double) return decline("element type must be Float or Double");
+    } else if (auto* r = dynamic_cast<tensor::ReduceNode*>(&node)) {
+        if (r->element() != P::Float && r->element() != P::Double) return decline("element type must be Float or Double");
+        if (!r->adjacent_axes()) return decline("the reduced axes must be adjacent (one block)");
     } else if (node.code() == tensor::LibraryNodeType_Broadcast) {
         auto* b = dynamic_cast<tensor::BroadcastNode*>(&node);
         if (!b) return decline("not a Broadcast node object");

@@ -421,6 +421,77 @@ Expression AttentionNode::connector_bytes(const std::string& connector) const {
 
 // ---- elementwise / broadcast ----
 
+ReduceNode::ReduceNode(std::string code, std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> axes,
+                       bool keepdims, types::PrimitiveType element)
+    : LibraryNode(std::move(code), {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)),
+      axes_(std::move(axes)), keepdims_(keepdims), element_(element) {}
+
+int ReduceNode::operation() const {
+    for (size_t i = 0; i < ReduceNodeCodes.size(); i++)
+        if (ReduceNodeCodes[i] == code_) return (int) i;
+    return -1;
+}
+
+std::vector<int64_t> ReduceNode::sorted_axes() const {
+    std::vector<int64_t> a = axes_;
+    const int64_t rank = (int64_t) shape_.size();
+    for (auto& v : a)
+        if (v < 0) v += rank;
+    std::sort(a.begin(), a.end());
+    a.erase(std::unique(a.begin(), a.end()), a.end());
+    return a;
+}
+
+bool ReduceNode::adjacent_axes() const {
+    const auto a = sorted_axes();
+    return !a.empty() && a.back() - a.front() + 1 == (int64_t) a.size();
+}
+
+Expression ReduceNode::outer() const { return product(shape_, 0, (size_t) sorted_axes().front()); }
+Expression ReduceNode::extent() const { return product(shape_, (size_t) sorted_axes().front(), (size_t) sorted_axes().back() + 1); }
+Expression ReduceNode::inner() const { return product(shape_, (size_t) sorted_axes().back() + 1, shape_.size()); }
+Expression ReduceNode::product_all() const { return product(shape_, 0, shape_.size()); }
+
+void ReduceNode::validate() const {
+    if (operation() < 0) throw InvalidSDFGException(code_ + ": not a reduce node code");
+    if (shape_.empty()) throw InvalidSDFGException(code_ + ": empty shape");
+    if (axes_.empty()) throw InvalidSDFGException(code_ + ": no reduction axis");
+    const int64_t rank = (int64_t) shape_.size();
+    for (auto a : axes_)
+        if (a < -rank || a >= rank)   // message of the reference's expansion (mean_node.cpp)
+            throw InvalidSDFGException("Library Node: Axis value out of bounds. Axis: " + std::to_string(a) +
+                                       " Shape size: " + std::to_string(rank));
+}
+
+void ReduceNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    Array ax;
+    for (auto a : axes_) ax.emplace_back(a);
+    j.set("axes", Value(std::move(ax)));
+    j.set("keepdims", keepdims_);
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<ReduceNode> ReduceNode::from_json(const Value& j) {
+    std::vector<int64_t> axes;
+    for (auto& a : j.at("axes").as_array()) axes.push_back(a.as_int());
+    const Value* kd = j.find("keepdims");
+    const Value* et = j.find("element_type");
+    return std::make_unique<ReduceNode>(j.at("code").as_string(), impl_of(j), exprs_from_json(j.at("shape")), std::move(axes),
+                                        kd && kd->is_bool() && kd->as_bool(),
+                                        et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression ReduceNode::connector_bytes(const std::string& connector) const {
+    if (connector == "X") return bytes_of(product_all(), element_);
+    // the output holds every extent that is not reduced
+    Expression kept = "1";
+    const auto axes = sorted_axes();
+    for (size_t d = 0; d < shape_.size(); d++)
+        if (std::find(axes.begin(), axes.end(), (int64_t) d) == axes.end()) kept = symbolic::mul(kept, shape_[d]);
+    return bytes_of(kept, element_);
+}
+
 static bool is_in(const std::vector<std::string>& v, const std::string& s) {
     for (auto& e : v)
         if (e == s) return true;
@@ -880,6 +951,7 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     for (auto& code : math::tensor::UnaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     for (auto& code : math::tensor::BinaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
+    for (auto& code : math::tensor::ReduceNodeCodes) fns_[code] = &deserialize<math::tensor::ReduceNode>;
     fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
 }
 

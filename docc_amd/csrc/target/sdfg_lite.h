@@ -287,6 +287,43 @@ private:
     types::PrimitiveType element_, output_element_;
 };
 
+// Reduce nodes over a set of axes, "X" -> "Y" (reference .../tensor/reduce_node.h, reduce_ops/
+// {sum,max,min,mean}_node.h; JSON keys shape, axes, keepdims as in reduce_node.h:194-245). Y has
+// the reduced axes removed, or kept with extent 1 when keepdims is set.
+inline const std::vector<std::string> ReduceNodeCodes = {"ml::Sum", "ml::Max", "ml::Min", "ml::Mean"};
+
+class ReduceNode : public data_flow::LibraryNode {
+public:
+    ReduceNode(std::string code, std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> axes,
+               bool keepdims, types::PrimitiveType element);
+    const std::vector<Expression>& shape() const { return shape_; }
+    const std::vector<int64_t>& axes() const { return axes_; }
+    bool keepdims() const { return keepdims_; }
+    types::PrimitiveType element() const { return element_; }
+    // position of the code in ReduceNodeCodes = the runtime's operation code
+    int operation() const;
+    // the axes, normalised and sorted; `adjacent` tells whether they form one block
+    std::vector<int64_t> sorted_axes() const;
+    bool adjacent_axes() const;
+    // [outer, reduce, inner] view of the input for a block of adjacent axes
+    Expression outer() const;
+    Expression extent() const;
+    Expression inner() const;
+
+    void validate() const override;
+    Expression flop() const override { return product_all(); }
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ReduceNode> from_json(const json::Value& j);
+
+private:
+    Expression product_all() const;
+    std::vector<Expression> shape_;
+    std::vector<int64_t> axes_;
+    bool keepdims_;
+    types::PrimitiveType element_;
+};
+
 // Elementwise tensor nodes: Y[i] = f(X[i]) or f(A[i], B[i]) over the linearised shape.
 // reference: .../tensor/elementwise_node.cpp:20 (ElementWiseUnaryNode "X" -> "Y"), :176
 // (ElementWiseBinaryNode "A","B" -> "C"), JSON keys code + shape; elementwise_ops/*.h for the codes.

@@ -25,6 +25,8 @@ NotImplementedError (there is no CPU lowering behind it):
         array and a scalar (literal or scalar argument)
     np.abs, np.exp, np.sqrt, np.tanh, scipy.special.erf / expit, relu(x), sigmoid(x),
         np.maximum(x, 0)  (ReLU)
+    np.sum / np.max / np.min / np.mean (and the array methods) over one axis or a block of
+        adjacent axes, with keepdims
 """
 from __future__ import annotations
 
@@ -86,8 +88,10 @@ class _Lazy:
     """A value that only exists as part of a larger pattern (scaled or transposed operands, the
     pieces of the decomposed softmax)."""
 
-    def __init__(self, kind: str, base: Any, scalar: Any = None):
+    def __init__(self, kind: str, base: Any, scalar: Any = None, src: Any = None):
         self.kind, self.base, self.scalar = kind, base, scalar
+        self.src = src          # the pattern piece this one was built from
+        self.array = None       # set once the value had to exist on its own
 
 
 class _ScalarValue:
@@ -178,6 +182,7 @@ class _Lowering(ast.NodeVisitor):
             ta, left = True, left.base
         if isinstance(right, _Lazy) and right.kind == "transposed":
             tb, right = True, right.base
+        left, right = self.array_of(node, left), self.array_of(node, right)
         if not isinstance(left, _Array) or not isinstance(right, _Array):
             self.fail(node, "a matrix product of non-array operands")
         if left.elem != right.elem:
@@ -257,11 +262,43 @@ class _Lowering(ast.NodeVisitor):
         self.b.add_broadcast(x.name, out.name, padded, shape)
         return out
 
-    def array_of(self, node: ast.AST, v: Any) -> Any:
-        """Materialises `scalar * array` as an array; other values pass through."""
-        if isinstance(v, _Lazy) and v.kind == "scaled":
-            return self.elementwise(node, "mul", v.base, v.scalar, None)
-        return v
+    def array_of(self, node: ast.AST, v: Any, dest: Optional[str] = None) -> Any:
+        """A pattern piece that turns out to be used on its own becomes the node(s) it stands for;
+        other values pass through."""
+        if not isinstance(v, _Lazy) or v.kind == "transposed":
+            return v
+        if v.array is not None:
+            return v.array
+        if v.kind == "scaled":
+            arr = self.elementwise(node, "mul", v.base, v.scalar, dest)
+        elif v.kind == "max_keep":
+            arr = self.reduce(node, "max", v.base, -1, True, dest)
+        elif v.kind == "sub_max":
+            arr = self.elementwise(node, "sub", v.base, self.array_of(node, v.src), dest)
+        elif v.kind == "exp_sub":
+            arr = self.unary(node, "exp", self.array_of(node, v.src), dest)
+        elif v.kind == "sum_keep":
+            arr = self.reduce(node, "sum", self.array_of(node, v.src), -1, True, dest)
+        else:
+            return v
+        v.array = arr
+        return arr
+
+    def reduce(self, node: ast.AST, op: str, x: Any, axis: Any, keepdims: bool, dest: Optional[str]) -> _Array:
+        x = self.array_of(node, x)
+        if not isinstance(x, _Array) or x.elem not in _SIZES:
+            self.fail(node, f"'{op}' reduction of a value that is not a float array")
+        rank = len(x.shape)
+        axes = list(range(rank)) if axis is None else ([axis] if isinstance(axis, int) else list(axis))
+        if any(not isinstance(a, int) or a < -rank or a >= rank for a in axes):
+            raise ValueError(f"{self.func.__name__}: axis {axis} is out of bounds for an array of rank {rank}")
+        axes = sorted({a % rank for a in axes})
+        if axes != list(range(axes[0], axes[-1] + 1)):
+            self.fail(node, "a reduction over axes that are not adjacent")
+        shape = [("1" if d in axes else s) for d, s in enumerate(x.shape) if keepdims or d not in axes]
+        out = self.new_array(shape, x.elem, dest)
+        self.b.add_reduce_op(op, x.name, out.name, x.shape, axes, keepdims)
+        return out
 
     def elementwise(self, node: ast.AST, op: str, a: Any, b: Any, dest: Optional[str]) -> _Array:
         a, b = self.array_of(node, a), self.array_of(node, b)
@@ -370,7 +407,7 @@ class _Lowering(ast.NodeVisitor):
         if isinstance(node.op, ast.Sub):
             x, m = self.ev(node.left), self.ev(node.right)
             if isinstance(x, _Array) and isinstance(m, _Lazy) and m.kind == "max_keep" and m.base.name == x.name:
-                return _Lazy("sub_max", x)
+                return _Lazy("sub_max", x, src=m)
             return self.elementwise(node, "sub", x, m, dest)
         if isinstance(node.op, ast.Div):
             e, s = self.ev(node.left), self.ev(node.right)
@@ -401,12 +438,12 @@ class _Lowering(ast.NodeVisitor):
         axis_last = lambda x: self.kw(node, "axis", 1, None) in (-1, len(x.shape) - 1) and self.kw(node, "keepdims", None, False) is True
         if fn in (np.max, np.amax):
             x = self.ev(node.args[0])
-            if isinstance(x, _Array) and axis_last(x):
+            if isinstance(x, _Array) and axis_last(x) and dest is None:
                 return _Lazy("max_keep", x)
         if fn is np.exp:
             v = self.ev(node.args[0])
             if isinstance(v, _Lazy) and v.kind == "sub_max":
-                return _Lazy("exp_sub", v.base)
+                return _Lazy("exp_sub", v.base, src=v)
             return self.unary(node, "exp", v, dest)
         unary_fns = {np.abs: "abs", np.absolute: "abs", np.fabs: "abs", np.sqrt: "sqrt", np.tanh: "tanh",
                      _functions.relu: "relu", _functions.sigmoid: "sigmoid", _functions.erf: "erf"}
@@ -427,15 +464,24 @@ class _Lowering(ast.NodeVisitor):
                             if isinstance(z, _ScalarValue) and z.text in ("0.0", "-0.0") and isinstance(x, (_Array, _Lazy)):
                                 return self.unary(node, "relu", x, dest)
                     return self.elementwise(node, op, a, b, dest)
+        reductions = {np.sum: "sum", np.max: "max", np.amax: "max", np.min: "min", np.amin: "min", np.mean: "mean"}
         if fn is np.sum:
             v = self.ev(node.args[0])
             if isinstance(v, _Lazy) and v.kind == "exp_sub" and axis_last(v.base):
-                return _Lazy("sum_keep", v.base)
+                return _Lazy("sum_keep", v.base, src=v)
+        for f, op in reductions.items():
+            if fn is f and node.args:
+                return self.reduce(node, op, self.ev(node.args[0]), self.kw(node, "axis", 1, None), bool(self.kw(node, "keepdims", None, False)), dest)
+        # the same as methods of an array: x.sum(axis=..), x.max(..), x.min(..), x.mean(..)
+        if fn is None and isinstance(node.func, ast.Attribute) and node.func.attr in ("sum", "max", "min", "mean"):
+            base = self.ev(node.func.value)
+            if isinstance(base, (_Array, _Lazy)):
+                return self.reduce(node, node.func.attr, base, self.kw(node, "axis", 0, None), bool(self.kw(node, "keepdims", None, False)), dest)
         self.fail(node, f"call to {ast.unparse(node.func)}")
 
     # ---- statements --------------------------------------------------------------
     def materialise(self, node: ast.AST, value_node: ast.AST, dest: Optional[str]) -> _Array:
-        v = self.ev(value_node, dest)
+        v = self.array_of(node, self.ev(value_node, dest), dest)
         if not isinstance(v, _Array):
             self.fail(node, "a statement whose value is not an array produced by a library node")
         if dest is not None and v.name != dest:
@@ -477,7 +523,7 @@ class _Lowering(ast.NodeVisitor):
             # into a probe, so lower once to learn the shape, into the final buffer
             name = f"_docc_ret_{len(self.outputs)}"
             before = len(self.b._data["root"]["children"])
-            result = self.ev(v, name)
+            result = self.array_of(node, self.ev(v, name), name)
             if not isinstance(result, _Array) or result.name != name or len(self.b._data["root"]["children"]) == before:
                 self.fail(node, "returning a value that is not produced by a library node")
             self.outputs.append(name)

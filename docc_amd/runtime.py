@@ -74,6 +74,7 @@ _SIGNATURES = {
     "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
     "docc_rocm_elementwise_binary_scalar": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, ctypes.c_double, ctypes.c_int, _vp],
     "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
+    "docc_rocm_reduce": [_vp, ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_elementwise_fused": [_vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_double, _vp, _vp,
                                     ctypes.c_double, ctypes.c_int, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
@@ -255,6 +256,14 @@ def broadcast(precision, in_shape, out_shape, X, Y, stream=0) -> None:
     ins = (ctypes.c_int64 * rank)(*in_shape)
     outs = (ctypes.c_int64 * rank)(*out_shape)
     call("docc_rocm_broadcast", stream, precision, rank, ctypes.addressof(ins), ctypes.addressof(outs), X, Y)
+
+
+REDUCE_OPS = {"sum": 0, "max": 1, "min": 2, "mean": 3}
+
+
+def reduce(op, precision, outer, extent, inner, X, Y, stream=0) -> None:
+    """Y[o, i] = op over r of X[o, r, i] for X seen as [outer, extent, inner]."""
+    call("docc_rocm_reduce", stream, REDUCE_OPS[op] if isinstance(op, str) else op, precision, outer, extent, inner, X, Y)
 
 
 def elementwise_fused(precision, shape, binary, a, a_shape, b, b_shape, post, Y, stream=0) -> None:

@@ -335,9 +335,20 @@ class StructuredSDFGBuilder:
                          "element_type": self._element(A).value},
                         [self._operand("A", A), self._operand("B", B)], [self._operand("Y", Y)])
 
+    #: reduce node codes (reference .../tensor/reduce_ops/*.h); "std" is not part of the rocm target
+    REDUCE_CODES = {"sum": "ml::Sum", "max": "ml::Max", "min": "ml::Min", "mean": "ml::Mean"}
+
     def add_reduce_op(self, op: str, X: str, Y: str, shape: Sequence[Any], axes: Sequence[int], keepdims: bool = False) -> None:
+        """Reduce node "X" -> "Y" over `axes` of an input of `shape` (reference add_reduce_op,
+        python/bindings/builder/py_structured_sdfg_builder.cpp:1041-1088: sum, max, min, mean, std, softmax)."""
+        if op in self.REDUCE_CODES:
+            self._add_block({"code": self.REDUCE_CODES[op], "implementation_type": "NONE", "side_effect": False,
+                             "shape": [_expr(s) for s in shape], "axes": [int(a) for a in axes], "keepdims": bool(keepdims),
+                             "element_type": self._element(X).value},
+                            [self._operand("X", X)], [self._operand("Y", Y)])
+            return
         if op != "softmax":
-            raise NotImplementedError(f"reduce op '{op}' is not part of the rocm target (softmax only)")
+            raise NotImplementedError(f"reduce op '{op}' is not part of the rocm target")
         if keepdims:
             raise InvalidSDFGException("Unsupported attribute on library node: softmax")
         self._add_block({"code": "ml::Softmax", "implementation_type": "NONE", "side_effect": False,

@@ -19,6 +19,7 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh)
                                            -> ml::ReLU .. ml::Erf
     F.linear / nn.Linear                   -> GEMM with the weight transposed, bias through Broadcast + Add
+    sum / mean / amax / amin over one dim or a block of adjacent dims (keepdim) -> ml::Sum .. ml::Min
 
 Tensors on a `cuda` device are passed to the generated function as device pointers (no
 transfers, the kernels run on the null stream in order with torch's default stream); CPU tensors
@@ -261,6 +262,19 @@ class _FxLowering:
         self.builder.add_elementwise_unary_op(op, x.name, out.name, x.shape)
         return out
 
+    def reduce(self, node, op: str, x, dim, keepdim: bool, dest):
+        if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
+            self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
+        rank = len(x.shape)
+        dims = list(range(rank)) if dim is None or dim == [] or dim == () else ([dim] if isinstance(dim, int) else list(dim))
+        dims = sorted({int(d) % rank for d in dims})
+        if dims != list(range(dims[0], dims[-1] + 1)):
+            self.fail(node, "a reduction over dims that are not adjacent")
+        shape = [(1 if d in dims else s) for d, s in enumerate(x.shape) if keepdim or d not in dims]
+        out = self.new_tensor(shape, x.dtype, dest)
+        self.builder.add_reduce_op(op, x.name, out.name, x.shape, dims, keepdim)
+        return out
+
     def linear(self, node, x, w, bias, dest):
         """x [..., K] times w[N, K] transposed, plus bias [N]: one GEMM over the flattened rows."""
         if not isinstance(x, _T) or not isinstance(w, _T) or len(w.shape) != 2 or len(x.shape) < 1 or x.shape[-1] != w.shape[1]:
@@ -424,6 +438,14 @@ class _FxLowering:
                 if kwargs.get("inplace"):
                     self.fail(node, "an in-place activation")
                 return self.unary(node, op, args[0], dest)
+        reductions = {"sum": (torch.sum,), "mean": (torch.mean,), "amax": (torch.amax,), "amin": (torch.amin,)}
+        for name, fns in reductions.items():
+            if any(t is f for f in fns) or method == name:
+                if kwargs.get("dtype") is not None:
+                    self.fail(node, "a reduction with a dtype conversion")
+                dim = kwargs.get("dim", kwargs.get("axis", args[1] if len(args) > 1 else None))
+                keepdim = bool(kwargs.get("keepdim", kwargs.get("keepdims", args[2] if len(args) > 2 else False)))
+                return self.reduce(node, {"amax": "max", "amin": "min"}.get(name, name), args[0], dim, keepdim, dest)
         if t is F.linear:
             bias = args[2] if len(args) > 2 else kwargs.get("bias")
             return self.linear(node, args[0], args[1], bias, dest)

@@ -159,6 +159,23 @@ int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, int op, int p
 int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, const int64_t* in_shape, const int64_t* out_shape,
                         const void* X, void* Y);
 
+/* Reduce tensor nodes ml::Sum / ml::Max / ml::Min / ml::Mean over a block of adjacent axes
+ * (reference sdfg/include/sdfg/data_flow/library_nodes/math/tensor/reduce_node.h and
+ * reduce_ops/{sum,max,min,mean}_node.h; replaces the loop nests ReduceNode::expand emits,
+ * reduce_node.cpp:188-333). X is seen as [outer, reduce, inner] (contiguous), Y as
+ * [outer, inner]: Y[o, i] = op over r of X[o, r, i]; keepdims only changes the shape the caller
+ * attaches to Y. Max / Min use fmax / fmin like the reference (a NaN is ignored unless the
+ * whole extent is NaN); an empty extent gives the identity (0, -inf, +inf). A reduction with
+ * inner > 1 and few output elements is sliced along the reduced extent; the slices' partial
+ * results pass through an 8 MiB array in device memory that belongs to the kernels' code object
+ * and is shared by every such call on the device: do not overlap them on different streams. */
+#define DOCC_ROCM_REDUCE_SUM 0
+#define DOCC_ROCM_REDUCE_MAX 1
+#define DOCC_ROCM_REDUCE_MIN 2
+#define DOCC_ROCM_REDUCE_MEAN 3
+int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision, int64_t outer, int64_t reduce, int64_t inner,
+                     const void* X, void* Y);
+
 /* A chain of elementwise nodes in one pass: Y = post_k(...post_1(f(A', B'))). A' and B' are
  * the operands repeated to `shape` by numpy's rules (`a_shape` / `b_shape`: `rank` extents, each
  * equal to the output's or 1), or the scalar `a_scalar` / `b_scalar` when the shape pointer is

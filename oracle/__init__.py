@@ -62,6 +62,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.oracle_elementwise_binary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p, _f32p]
     lib.oracle_elementwise_binary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p, _f64p]
     lib.oracle_broadcast.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), ctypes.c_void_p, ctypes.c_void_p]
+    lib.oracle_reduce_f32.argtypes = [ctypes.c_int, _i64, _i64, _i64, _f32p, _f32p]
+    lib.oracle_reduce_f64.argtypes = [ctypes.c_int, _i64, _i64, _i64, _f64p, _f64p]
     return lib
 
 
@@ -251,3 +253,28 @@ def broadcast(X, out_shape, lib=None) -> np.ndarray:
     if rc != 0:
         raise ValueError(f"cannot broadcast {X.shape} to {out_shape}")
     return out
+
+
+REDUCE_OPS = {"sum": 0, "max": 1, "min": 2, "mean": 3}
+
+
+def reduce(op: str, X, axes, keepdims: bool = False, lib=None) -> np.ndarray:
+    """ml::Sum / ml::Max / ml::Min / ml::Mean of an fp32 or fp64 array over a block of adjacent axes,
+    accumulated left to right like the reference's expansion."""
+    lib = lib or load()
+    dt = np.float64 if np.asarray(X).dtype == np.float64 else np.float32
+    X = _c(X, dt)
+    rank = X.ndim
+    axes = sorted(a % rank for a in ([axes] if np.isscalar(axes) else axes))
+    if axes != list(range(axes[0], axes[-1] + 1)):
+        raise ValueError("the reduced axes must be adjacent")
+    outer = int(np.prod(X.shape[:axes[0]], dtype=np.int64))
+    extent = int(np.prod(X.shape[axes[0]:axes[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(X.shape[axes[-1] + 1:], dtype=np.int64))
+    out = np.empty((outer, inner), dt)
+    ptr = _f64p if dt == np.float64 else _f32p
+    fn = lib.oracle_reduce_f64 if dt == np.float64 else lib.oracle_reduce_f32
+    if fn(REDUCE_OPS[op], outer, extent, inner, _p(X, ptr), _p(out, ptr)) != 0:
+        raise ValueError(f"reduce '{op}' over an extent of {extent}")
+    kept = [1 if d in axes else s for d, s in enumerate(X.shape)] if keepdims else [s for d, s in enumerate(X.shape) if d not in axes]
+    return out.reshape(kept)

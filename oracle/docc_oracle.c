@@ -501,3 +501,29 @@ ORACLE_API int oracle_broadcast(int esize, int rank, const int64_t* in_shape, co
     }
     return 0;
 }
+
+/* Reduce nodes ml::Sum / ml::Max / ml::Min / ml::Mean over a block of adjacent axes, X seen as
+ * [outer, reduce, inner]. Restates ReduceNode::expand (reduce_node.cpp:188-333): Y is first set to the
+ * identity (sum_node.cpp:20-57 "0", max_node.cpp:56-67 "-INFINITY", min_node.cpp "INFINITY"), then
+ * accumulated through memory along the reduced extent, left to right: Y = X + Y, Y = fmax(X, Y)
+ * (max_node.cpp:73-91), Y = fmin(X, Y). Mean is the Sum node followed by a Div by the number of reduced
+ * elements (mean_node.cpp). op: 0 sum, 1 max, 2 min, 3 mean. */
+#define ORACLE_REDUCE(NAME, T, FMAX, FMIN, NEG_INF, POS_INF)                                                  \
+    ORACLE_API int NAME(int op, int64_t outer, int64_t reduce, int64_t inner, const T* X, T* Y) {              \
+        if (op < 0 || op > 3) return 1;                                                                       \
+        if (op == 3 && reduce == 0) return 2;                                                                 \
+        _Pragma("omp parallel for schedule(static)") for (int64_t o = 0; o < outer; o++) {                    \
+            for (int64_t i = 0; i < inner; i++) Y[o * inner + i] = op == 1 ? NEG_INF : op == 2 ? POS_INF : (T) 0; \
+            for (int64_t r = 0; r < reduce; r++)                                                              \
+                for (int64_t i = 0; i < inner; i++) {                                                         \
+                    const T x = X[(o * reduce + r) * inner + i];                                              \
+                    T* y = &Y[o * inner + i];                                                                 \
+                    *y = op == 1 ? FMAX(x, *y) : op == 2 ? FMIN(x, *y) : x + *y;                              \
+                }                                                                                             \
+            if (op == 3)                                                                                      \
+                for (int64_t i = 0; i < inner; i++) Y[o * inner + i] = Y[o * inner + i] / (T) reduce;         \
+        }                                                                                                     \
+        return 0;                                                                                             \
+    }
+ORACLE_REDUCE(oracle_reduce_f32, float, fmaxf, fminf, -INFINITY, INFINITY)
+ORACLE_REDUCE(oracle_reduce_f64, double, fmax, fmin, -INFINITY, INFINITY)

@@ -314,6 +314,21 @@ def test_torch_lowering_of_elementwise_operations_and_linear():
                      "ml::Sqrt", "ml::Broadcast", "ml::Mul", "ml::Add"]
     assert all(n["element_type"] == "Double" for n in sdfg.library_nodes())
 
+    class Norm(torch.nn.Module):
+        def forward(self, x):
+            return x - x.mean(dim=-1, keepdim=True)
+
+    sdfg = docc_torch.TorchProgram(Norm(), (torch.randn(4, 5, 6),), target="rocm").to_sdfg()
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Mean", "ml::Broadcast", "ml::Sub"]
+    assert sdfg.library_nodes()[0]["axes"] == [2] and sdfg.library_nodes()[0]["keepdims"] is True
+
+    class Pool(torch.nn.Module):
+        def forward(self, x):
+            return torch.sum(x, (2, 3)), x.amax(dim=1)
+
+    sdfg = docc_torch.TorchProgram(Pool(), (torch.randn(2, 3, 4, 5),), target="rocm").to_sdfg()
+    assert [(n["code"], n["axes"]) for n in sdfg.library_nodes()] == [("ml::Sum", [2, 3]), ("ml::Max", [1])]
+
     class Ints(torch.nn.Module):
         def forward(self, a):
             return a + a
@@ -346,3 +361,44 @@ def test_torch_backend_is_registered_and_reads_global_options():
     finally:
         unregister_target("probe")
         docc_torch.set_backend_options(target="rocm")
+
+
+def test_reductions_and_softmax_pieces_used_on_their_own():
+    @native
+    def stats(x):
+        return np.sum(x, axis=1), x.max(axis=(1, 2), keepdims=True), np.mean(x), np.min(x, axis=0)
+
+    @native
+    def normalise(x):
+        m = np.max(x, axis=-1, keepdims=True)
+        e = np.exp(x - m)
+        return e / np.sum(e, axis=-1, keepdims=True), m          # the softmax node, and the maximum as a value of its own
+
+    @native
+    def centred(x):
+        return x - np.mean(x, axis=0, keepdims=True)
+
+    x = np.zeros((4, 5, 6), np.float32)
+    sdfg = stats.to_sdfg(x)
+    nodes = sdfg.library_nodes()
+    assert [(n["code"], n["axes"], n["keepdims"]) for n in nodes] == [("ml::Sum", [1], False), ("ml::Max", [1, 2], True),
+                                                                      ("ml::Mean", [0, 1, 2], False), ("ml::Min", [0], False)]
+    assert all(n["shape"] == ["_s0", "_s1", "_s2"] and n["element_type"] == "Float" for n in nodes)
+    assert sdfg.arguments == ["x", "_s0", "_s1", "_s2", "_docc_ret_0", "_docc_ret_1", "_docc_ret_2", "_docc_ret_3"]
+    assert [n["code"] for n in normalise.to_sdfg(x).library_nodes()] == ["ml::Softmax", "ml::Max"]
+    sdfg = centred.to_sdfg(np.zeros((7, 3)))
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Mean", "ml::Broadcast", "ml::Sub"]
+    assert sdfg.library_nodes()[1]["input_shape"] == ["1", "_s1"]
+
+    @native
+    def scattered(x):
+        return np.sum(x, axis=(0, 2))
+
+    with pytest.raises(NotImplementedError, match="not adjacent"):
+        scattered.to_sdfg(x)
+    with pytest.raises(ValueError, match="out of bounds"):
+        native(_bad_axis).to_sdfg(x)
+
+
+def _bad_axis(x):
+    return np.sum(x, axis=5)

@@ -299,3 +299,47 @@ def test_program_in_docc_json_format_runs(tmp_path):
     fn(A.ctypes.data, B.ctypes.data, C.ctypes.data, n)
     assert runtime.take_failure() == (0, "")
     assert rel_err_max(C, ref) <= 1e-12
+
+
+def test_native_reductions_and_layer_statistics():
+    """np.sum / max / min / mean over rows, columns and blocks of axes; the softmax pieces as values of their own."""
+    @native(target="rocm")
+    def stats(x):
+        return np.sum(x, axis=1), x.max(axis=(1, 2), keepdims=True), np.mean(x), np.min(x, axis=0)
+
+    @native(target="rocm")
+    def centred(x):
+        return x - np.mean(x, axis=0, keepdims=True)
+
+    @native(target="rocm")
+    def normalise(x):
+        m = np.max(x, axis=-1, keepdims=True)
+        e = np.exp(x - m)
+        return e / np.sum(e, axis=-1, keepdims=True), m
+
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((12, 50, 36)).astype(np.float32)
+    s, mx, mean, mn = stats(x)
+    assert s.shape == (12, 36) and mx.shape == (12, 1, 1) and np.shape(mean) == () and mn.shape == (50, 36)
+    np.testing.assert_allclose(s, x.astype(np.float64).sum(axis=1), rtol=1e-5, atol=1e-5)
+    assert np.array_equal(mx, x.max(axis=(1, 2), keepdims=True)) and np.array_equal(mn, x.min(axis=0))
+    np.testing.assert_allclose(mean, x.astype(np.float64).mean(), rtol=1e-5, atol=1e-6)
+    assert stats.last_sdfg.loop_report()["H2D"] == 1           # x goes to the device once for the four nodes
+
+    y = rng.standard_normal((300, 40))
+    np.testing.assert_allclose(centred(y), y - y.mean(axis=0, keepdims=True), rtol=1e-12, atol=1e-12)
+    p, m = normalise(x)
+    assert rel_err_max(p, oracle.softmax(x)) <= 1e-5 and np.array_equal(m, x.max(axis=-1, keepdims=True))
+
+
+def test_torch_reductions_fp32():
+    class Pool(torch.nn.Module):
+        def forward(self, x):
+            return torch.mean(x, dim=(2, 3)), x.amax(dim=1, keepdim=True)
+
+    x = torch.randn(8, 16, 14, 14, device="cuda")
+    program = docc_torch.compile_torch(Pool(), x, target="rocm")
+    avg, mx = program(x)
+    assert avg.is_cuda and avg.shape == (8, 16) and mx.shape == (8, 1, 14, 14)
+    assert torch.allclose(avg, x.double().mean(dim=(2, 3)).float(), rtol=1e-5, atol=1e-6)
+    assert torch.equal(mx, x.amax(dim=1, keepdim=True))

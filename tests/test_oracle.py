@@ -249,3 +249,38 @@ def test_broadcast_matches_numpy():
         assert np.array_equal(oracle.broadcast(xd, out_shape), np.broadcast_to(xd, out_shape))
     with pytest.raises(ValueError):
         oracle.broadcast(np.zeros((2, 3), np.float32), (2, 4))
+
+
+def test_reduce_nodes_against_numpy_and_closed_forms():
+    """oracle.reduce (ml::Sum / Max / Min / Mean) pinned by numpy's reductions in float64, by integer-valued
+    inputs (every partial sum exact, so the order of the additions cannot matter) and by the identities of
+    an empty extent; Max / Min must be exactly numpy's reductions, and fmax / fmin where a NaN is present."""
+    rng = np.random.default_rng(12)
+    for dt in (np.float32, np.float64):
+        x = rng.standard_normal((5, 7, 3, 4)).astype(dt)
+        for axes in ((3,), (0,), (1, 2), (0, 1, 2, 3), (-1,), (2, 3)):
+            for keep in (False, True):
+                ax = tuple(a % 4 for a in axes)
+                tol = 1e-5 if dt == np.float32 else 1e-13
+                np.testing.assert_allclose(oracle.reduce("sum", x, axes, keep), x.astype(np.float64).sum(axis=ax, keepdims=keep), rtol=tol, atol=tol)
+                np.testing.assert_allclose(oracle.reduce("mean", x, axes, keep), x.astype(np.float64).mean(axis=ax, keepdims=keep), rtol=tol, atol=tol)
+                assert np.array_equal(oracle.reduce("max", x, axes, keep), x.max(axis=ax, keepdims=keep))
+                assert np.array_equal(oracle.reduce("min", x, axes, keep), x.min(axis=ax, keepdims=keep))
+                assert oracle.reduce("sum", x, axes, keep).dtype == dt
+        ints = rng.integers(-8, 9, (6, 50, 3)).astype(dt)
+        assert np.array_equal(oracle.reduce("sum", ints, (1,)), ints.sum(axis=1))                  # exact in any order
+        assert np.array_equal(oracle.reduce("mean", np.full((4, 8), 3.0, dt), (1,)), np.full(4, 3.0, dt))
+        # fmax / fmin skip a NaN; a row of nothing but NaN keeps the identity the reference starts from
+        y = np.array([[1.0, np.nan, 3.0], [np.nan, np.nan, np.nan], [-np.inf, 2.0, np.inf]], dt)
+        assert np.array_equal(oracle.reduce("max", y, (1,)), np.array([3.0, -np.inf, np.inf], dt))
+        assert np.array_equal(oracle.reduce("min", y, (1,)), np.array([1.0, np.inf, -np.inf], dt))
+        assert np.array_equal(oracle.reduce("max", y[[0, 2]], (1,)), np.fmax.reduce(y[[0, 2]], axis=1))
+        # an empty extent leaves the identity
+        e = np.zeros((3, 0, 2), dt)
+        assert np.array_equal(oracle.reduce("sum", e, (1,)), np.zeros((3, 2), dt))
+        assert np.array_equal(oracle.reduce("max", e, (1,)), np.full((3, 2), -np.inf, dt))
+        assert np.array_equal(oracle.reduce("min", e, (1,)), np.full((3, 2), np.inf, dt))
+    with pytest.raises(ValueError):
+        oracle.reduce("sum", np.zeros((2, 3, 4)), (0, 2))        # not a block of adjacent axes
+    with pytest.raises(ValueError):
+        oracle.reduce("mean", np.zeros((2, 0)), (1,))

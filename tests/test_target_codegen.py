@@ -37,7 +37,7 @@ def test_registry_holds_every_rocm_key():
     keys = registered_dispatchers()
     for code in ("GEMM", "ml::MatMul", "ml::Softmax", "ml::Conv", "ml::Attention", "ml::Broadcast", "ml::Abs", "ml::Exp",
                  "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf", "ml::Add", "ml::Sub", "ml::Mul", "ml::Div",
-                 "ml::Maximum", "ml::Minimum"):
+                 "ml::Maximum", "ml::Minimum", "ml::Sum", "ml::Max", "ml::Min", "ml::Mean", "ROCMFusedElementWise"):
         assert f"{code}::ROCMWithTransfers" in keys and f"{code}::ROCMWithoutTransfers" in keys
     assert "ROCMOffloading::NONE" in keys
 
@@ -423,3 +423,39 @@ def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
     flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "scalar")[0])
     assert "docc_rocm_elementwise_fused(nullptr, 32, 1, __docc_shape, 4 /* ml::Maximum */, __docc_a_shape, d_A, 0.0, nullptr, nullptr, (double) B, 1, __docc_post, d_Y)" in flat
     assert flat.count("docc_rocm_memcpy_h2d_async(") == 1 and flat.count("docc_rocm_memcpy_d2h_async(") == 1
+
+
+def test_reduce_nodes_dispatch_and_decline(tmp_path):
+    b = StructuredSDFGBuilder("red")
+    for n in ("X", "S", "M"):
+        b.add_container(n, F32, True)
+    b.add_container("_n", I64, True)
+    b.add_reduce_op("sum", "X", "S", ["_n", 64, 56, 56], [2, 3])            # [_n, 64, 56*56] -> [_n, 64]
+    b.add_reduce_op("max", "X", "M", ["_n", 64, 56, 56], [-3], keepdims=True)   # over the channels: inner extent 56*56
+    s = b.move()
+    nodes = s.library_nodes()
+    # payload keys of the reference's reduce serializer (reduce_node.h:194-245)
+    assert nodes[0]["code"] == "ml::Sum" and nodes[0]["axes"] == [2, 3] and nodes[0]["keepdims"] is False
+    assert nodes[1]["code"] == "ml::Max" and nodes[1]["axes"] == [-3] and nodes[1]["keepdims"] is True
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["ml::Sum::ROCMWithoutTransfers"] == 1 and r["H2D"] == 1 and r["D2H"] == 2     # X goes up once for both nodes
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path)[0])
+    assert "docc_rocm_reduce(nullptr, 0 /* ml::Sum */, 32, _n*64, 3136, 1, X, Y)" in flat
+    assert "docc_rocm_reduce(nullptr, 1 /* ml::Max */, 32, _n, 64, 3136, X, Y)" in flat
+    assert "(size_t) (_n*64*4)" in flat.replace("(_n*64)*4", "_n*64*4")                      # Y of the sum: the kept extents
+    # what the kernels do not cover is declined by the mapper, with the reason
+    b = StructuredSDFGBuilder("scattered")
+    for n in ("X", "Y"):
+        b.add_container(n, F64, True)
+    b.add_reduce_op("mean", "X", "Y", [4, 5, 6], [0, 2])
+    with pytest.raises(InvalidSDFGException, match="adjacent"):
+        b.move().schedule("rocm")
+    with pytest.raises(NotImplementedError, match="std"):
+        StructuredSDFGBuilder("s").add_reduce_op("std", "X", "Y", [4], [0])
+    b = StructuredSDFGBuilder("axis")
+    for n in ("X", "Y"):
+        b.add_container(n, F64, True)
+    b.add_reduce_op("sum", "X", "Y", [4, 5], [2])
+    with pytest.raises(InvalidSDFGException, match="Axis value out of bounds"):
+        b.move().validate()
