@@ -6,11 +6,12 @@
 // temporaries) by one kernel that reads X once and writes Y once.
 //
 // HBM-bound: algorithmic traffic is 8 bytes per element. Three shapes:
-//   wave-per-row  (cols <= 4096, cols % 4 == 0): a 64-lane wavefront holds the
-//       whole row in registers (NV float4 per lane, 128-bit coalesced loads),
+//   wave-per-row  (cols <= 1024, cols % 4 == 0; built up to 4096): a 64-lane wavefront
+//       holds the whole row in registers (NV float4 per lane, 128-bit coalesced loads),
 //       reduces max and sum with wave shuffles only - no LDS, no barrier;
 //   block-per-row (cols <= 16384, cols % 4 == 0): 256 threads hold the row,
-//       partial results cross the four waves through LDS;
+//       partial results cross the four waves through LDS; ahead of the wavefront
+//       per row from 2048 columns on (more rows in flight per register);
 //   streaming     (any cols): per-lane online max/sum over the row, then a
 //       second read (served by L2 / Infinity Cache) to write the result.
 #include "common.h"
@@ -152,6 +153,9 @@ DOCC_SOFTMAX_WAVE(16)
                                                                                    long rows, int cols) {  \
         softmax_block_kernel<NV>(X, Y, rows, cols);                                                        \
     }
+DOCC_SOFTMAX_BLOCK(1)
+DOCC_SOFTMAX_BLOCK(2)
+DOCC_SOFTMAX_BLOCK(4)
 DOCC_SOFTMAX_BLOCK(8)
 DOCC_SOFTMAX_BLOCK(16)
 

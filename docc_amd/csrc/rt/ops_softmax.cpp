@@ -1,4 +1,6 @@
 // Launchers for ml::Softmax and the utility kernels (see include/docc_rocm_ops.h).
+#include <cstdlib>
+
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
 
@@ -13,7 +15,12 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
     if (rows > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
     hipStream_t s = (hipStream_t) stream;
     const bool vec_ok = (cols % 4 == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
-    if (vec_ok && cols <= 4096) {
+    // Up to 1024 columns one wavefront per row moves the most bytes (6.1-6.4 TB/s measured against 2.6-5.6
+    // for a work-group per row); from 2048 columns on the work-group per row is ahead (6.1-6.3 against
+    // 5.8-6.0 TB/s). DOCC_ROCM_SOFTMAX=wave|block overrides the choice where both exist (tuning).
+    const char* force = std::getenv("DOCC_ROCM_SOFTMAX");
+    const bool wave = force && force[0] == 'w' ? true : force && force[0] == 'b' ? false : cols <= 1024;
+    if (vec_ok && cols <= 4096 && wave) {
         // one wavefront per row, 4 rows per 256-thread block
         const char* name = cols <= 256    ? "docc_softmax_f32_wave_v1"
                            : cols <= 512  ? "docc_softmax_f32_wave_v2"
@@ -24,7 +31,11 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
         return launch(name, grid, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     }
     if (vec_ok && cols <= 16384) {
-        const char* name = cols <= 8192 ? "docc_softmax_f32_block_v8" : "docc_softmax_f32_block_v16";
+        const char* name = cols <= 1024   ? "docc_softmax_f32_block_v1"
+                           : cols <= 2048 ? "docc_softmax_f32_block_v2"
+                           : cols <= 4096 ? "docc_softmax_f32_block_v4"
+                           : cols <= 8192 ? "docc_softmax_f32_block_v8"
+                                          : "docc_softmax_f32_block_v16";
         return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     }
     return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
