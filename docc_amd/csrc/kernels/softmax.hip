@@ -11,7 +11,8 @@
 //       reduces max and sum with wave shuffles only - no LDS, no barrier;
 //   block-per-row (cols <= 16384, cols % 4 == 0): 256 threads hold the row,
 //       partial results cross the four waves through LDS; ahead of the wavefront
-//       per row from 2048 columns on (more rows in flight per register);
+//       per row from 2048 columns on (more rows in flight per register); rows of
+//       2049..4096 columns use 512 threads (two vectors per lane), the others 256;
 //   streaming     (any cols): per-lane online max/sum over the row, then a
 //       second read (served by L2 / Infinity Cache) to write the result.
 #include "common.h"
@@ -72,30 +73,37 @@ __device__ __forceinline__ void softmax_wave_kernel(const float* X, float* Y, lo
     softmax_row_wave<NV>(X + row * (long) cols, Y + row * (long) cols, cols, lane);
 }
 
-// block reductions across the 4 waves of a 256-thread block
+// block reductions across the NW waves of a work-group
+template <int NW = 4>
 __device__ __forceinline__ float block_max(float v, float* lds) {
     v = wave_max(v);
     const int w = threadIdx.x / kWave;
     if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
     __syncthreads();
-    float r = fmaxf(fmaxf(lds[0], lds[1]), fmaxf(lds[2], lds[3]));
+    float r = lds[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r = fmaxf(r, lds[i]);
     __syncthreads();
     return r;
 }
 
+template <int NW = 4>
 __device__ __forceinline__ float block_sum(float v, float* lds) {
     v = wave_sum(v);
     const int w = threadIdx.x / kWave;
     if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
     __syncthreads();
-    float r = (lds[0] + lds[1]) + (lds[2] + lds[3]);
+    float r = lds[0];
+#pragma unroll
+    for (int i = 1; i < NW; i++) r += lds[i];
     __syncthreads();
     return r;
 }
 
-template <int NV>
+template <int NV, int NW = 4>
 __device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, long rows, int cols) {
-    __shared__ float lds[4];
+    constexpr int NT = NW * kWave;
+    __shared__ float lds[NW];
     const long row = blockIdx.x;
     const int nvec = cols >> 2;
     const f32x4* xv = reinterpret_cast<const f32x4*>(X + row * (long) cols);
@@ -103,7 +111,7 @@ __device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, l
     f32x4 v[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        int c = threadIdx.x + i * 256;
+        int c = threadIdx.x + i * NT;
         if (c < nvec) {
             v[i] = __builtin_nontemporal_load(xv + c);
         } else {
@@ -113,7 +121,7 @@ __device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, l
     float m = kNegInf;
 #pragma unroll
     for (int i = 0; i < NV; i++) m = fmaxf(fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)), m);
-    m = block_max(m, lds);
+    m = block_max<NW>(m, lds);
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
@@ -123,11 +131,11 @@ __device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, l
         v[i].w = exp_neg(v[i].w - m);
         s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
     }
-    s = block_sum(s, lds);
+    s = block_sum<NW>(s, lds);
     const float inv = 1.0f / s;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        int c = threadIdx.x + i * 256;
+        int c = threadIdx.x + i * NT;
         if (c < nvec) {
             f32x4 o = v[i] * inv;
             __builtin_nontemporal_store(o, yv + c);
@@ -153,6 +161,13 @@ DOCC_SOFTMAX_WAVE(16)
                                                                                    long rows, int cols) {  \
         softmax_block_kernel<NV>(X, Y, rows, cols);                                                        \
     }
+// eight wavefronts per row
+#define DOCC_SOFTMAX_BLOCK8(NV)                                                                             \
+    extern "C" __global__ __launch_bounds__(512) void docc_softmax_f32_block8_v##NV(const float* X, float* Y, \
+                                                                                    long rows, int cols) {  \
+        softmax_block_kernel<NV, 8>(X, Y, rows, cols);                                                      \
+    }
+DOCC_SOFTMAX_BLOCK8(2)
 DOCC_SOFTMAX_BLOCK(1)
 DOCC_SOFTMAX_BLOCK(2)
 DOCC_SOFTMAX_BLOCK(4)

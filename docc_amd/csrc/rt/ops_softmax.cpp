@@ -17,7 +17,7 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
     const bool vec_ok = (cols % 4 == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
     // Up to 1024 columns one wavefront per row moves the most bytes (6.1-6.4 TB/s measured against 2.6-5.6
     // for a work-group per row); from 2048 columns on the work-group per row is ahead (6.1-6.3 against
-    // 5.8-6.0 TB/s). DOCC_ROCM_SOFTMAX=wave|block overrides the choice where both exist (tuning).
+    // 5.8-6.0 TB/s). DOCC_ROCM_SOFTMAX=wave|block overrides the choice (tuning; block = four wavefronts per row).
     const char* force = std::getenv("DOCC_ROCM_SOFTMAX");
     const bool wave = force && force[0] == 'w' ? true : force && force[0] == 'b' ? false : cols <= 1024;
     if (vec_ok && cols <= 4096 && wave) {
@@ -30,6 +30,9 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
         uint32_t grid = (uint32_t) ((rows + 3) / 4);
         return launch(name, grid, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     }
+    if (vec_ok && cols > 2048 && cols <= 4096 && !(force && force[0] == 'b'))
+        // eight wavefronts per row, two vectors per lane: 6.24 TB/s against 6.09 with four wavefronts at 4096 columns
+        return launch("docc_softmax_f32_block8_v2", (uint32_t) rows, 1, 1, 512, 0, s, X, Y, (long) rows, (int) cols);
     if (vec_ok && cols <= 16384) {
         const char* name = cols <= 1024   ? "docc_softmax_f32_block_v1"
                            : cols <= 2048 ? "docc_softmax_f32_block_v2"

@@ -25,8 +25,8 @@ def run_softmax(rt, X: np.ndarray) -> np.ndarray:
 
 @pytest.mark.parametrize(
     "rows,cols",
-    [(1, 1), (3, 4), (8, 257), (5, 7), (64, 256), (33, 260), (17, 1024), (9, 2048), (16, 4096), (7, 4100),
-     (5, 8192), (3, 16384), (2, 16388), (2, 40000), (1000, 12), (4, 3)],
+    [(1, 1), (3, 4), (8, 257), (5, 7), (64, 256), (33, 260), (17, 1024), (6, 1028), (9, 2048), (9, 2052), (11, 3000),
+     (5, 4092), (16, 4096), (7, 4100), (5, 8192), (3, 16384), (2, 16388), (2, 40000), (1000, 12), (4, 3)],
 )
 def test_softmax_matches_oracle(rt, rows, cols):
     rng = np.random.default_rng(rows * 100003 + cols)
@@ -36,6 +36,19 @@ def test_softmax_matches_oracle(rt, rows, cols):
     assert rel_err_max(Y, ref) <= TOL_F32
     # element-wise as well: 2e-6 relative plus an absolute floor for denormal outputs
     np.testing.assert_allclose(Y, ref, rtol=2e-5, atol=1e-30)
+    np.testing.assert_allclose(Y.sum(axis=-1), 1.0, rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("force", ["wave", "block"])
+@pytest.mark.parametrize("cols", [512, 1024, 2048, 3000, 4096])
+def test_softmax_every_built_variant(rt, monkeypatch, force, cols):
+    """The wavefront-per-row and work-group-per-row kernels are both built up to 4096 columns; the launcher
+    picks by width. Forcing either must give the same result."""
+    monkeypatch.setenv("DOCC_ROCM_SOFTMAX", force)
+    rng = np.random.default_rng(cols)
+    X = (rng.standard_normal((37, cols)) * 8).astype(np.float32)
+    Y = run_softmax(rt, X)
+    assert rel_err_max(Y, oracle.softmax(X)) <= TOL_F32
     np.testing.assert_allclose(Y.sum(axis=-1), 1.0, rtol=0, atol=1e-5)
 
 
