@@ -375,8 +375,10 @@ struct AsyncGemmKernel {
 #define DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, TA, TB, TAG)                                          \
     extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_##PREFIX##a_##BM##x##BN##x##BK##s##ST##_##TAG)(  \
         const T* A, const T* B, OT* C, long M, long N, long K, long lda, long ldb, long ldc, OT alpha, OT beta,    \
-        const OT* bias, int act) {                                                                                 \
-        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
+        const OT* bias, int act, long batch_a, long batch_b, long batch_c) {                                       \
+        const long z = blockIdx.y;                                                                                 \
+        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A + z * batch_a, B + z * batch_b, C + z * batch_c, M, N, \
+                                                                        K, lda, ldb, ldc, alpha, beta, bias, act); \
     }
 
 #define DOCC_AGEMM_CONFIG(PREFIX, T, OT, BM, BN, BK, WM, WN, ST)            \

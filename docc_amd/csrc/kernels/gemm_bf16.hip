@@ -165,8 +165,10 @@ struct GemmBf16Kernel {
 #define DOCC_BGEMM_ONE(BM, BN, BK, WM, WN, TA, TB, TAG, AL, ALTAG)                                                  \
     extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_bgemm_##BM##x##BN##x##BK##_##TAG##_##ALTAG)(      \
         const uint16_t* A, const uint16_t* B, float* C, long M, long N, long K, long lda, long ldb, long ldc,       \
-        float alpha, float beta, const float* bias, int act) {                                                      \
-        docc_k::GemmBf16Kernel<BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
+        float alpha, float beta, const float* bias, int act, long batch_a, long batch_b, long batch_c) {            \
+        const long z = blockIdx.y;                                                                                  \
+        docc_k::GemmBf16Kernel<BM, BN, BK, WM, WN, TA, TB, AL>::run(A + z * batch_a, B + z * batch_b, C + z * batch_c, M, N, K, \
+                                                                    lda, ldb, ldc, alpha, beta, bias, act);         \
     }
 
 #define DOCC_BGEMM_CONFIG(BM, BN, BK, WM, WN)                    \

@@ -450,8 +450,11 @@ struct GemmKernel {
 #define DOCC_GEMM_ONE(PREFIX, T, BM, BN, BK, WM, WN, TA, TB, TAG, AL, ALTAG)                                   \
     extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_##PREFIX##_##BM##x##BN##x##BK##_##TAG##_##ALTAG)( \
         const T* A, const T* B, T* C, long M, long N, long K, long lda, long ldb, long ldc, T alpha, T beta,    \
-        const T* bias, int act) {                                                                              \
-        docc_k::GemmKernel<T, BM, BN, BK, WM, WN, TA, TB, AL>::run(A, B, C, M, N, K, lda, ldb, ldc, alpha, beta, bias, act); \
+        const T* bias, int act, long batch_a, long batch_b, long batch_c) {                                    \
+        /* blockIdx.y = entry of the batch; the strides are in elements, 0 for a shared operand */             \
+        const long z = blockIdx.y;                                                                             \
+        docc_k::GemmKernel<T, BM, BN, BK, WM, WN, TA, TB, AL>::run(A + z * batch_a, B + z * batch_b, C + z * batch_c, M, N, K, \
+                                                                   lda, ldb, ldc, alpha, beta, bias, act);     \
     }
 
 #define DOCC_GEMM_CONFIG(PREFIX, T, BM, BN, BK, WM, WN)                    \

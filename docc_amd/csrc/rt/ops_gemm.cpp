@@ -31,7 +31,8 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
 template <typename T, typename S = T>
 int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n,
                 int64_t k, S alpha, const T* A, int64_t lda, const T* B, int64_t ldb, S beta, S* C, int64_t ldc,
-                TileConfig (*pick)(int64_t m, int64_t n, bool aligned, int force), const S* bias = nullptr, int activation = -1) {
+                TileConfig (*pick)(int64_t m, int64_t n, int64_t batch, bool aligned, int force), const S* bias = nullptr,
+                int activation = -1, int64_t batch = 1, int64_t batch_a = 0, int64_t batch_b = 0, int64_t batch_c = 0) {
     if ((trans_a != DOCC_ROCM_NO_TRANS && trans_a != DOCC_ROCM_TRANS) ||
         (trans_b != DOCC_ROCM_NO_TRANS && trans_b != DOCC_ROCM_TRANS))
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: transpose code must be 111 or 112", prefix);
@@ -45,7 +46,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: unknown activation %d", prefix, activation);
     if (activation >= 0 && activation != DOCC_ROCM_UNARY_RELU && activation != DOCC_ROCM_UNARY_ABS)
         return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: only ReLU and Abs are built into the GEMM store (activation %d)", prefix, activation);
-    if (m == 0 || n == 0) return 0;
+    if (batch < 0 || batch > 65535) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: batch must be 0..65535", prefix);
+    if (batch_a < 0 || batch_b < 0 || batch_c < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: negative batch stride", prefix);
+    if (m == 0 || n == 0 || batch == 0) return 0;
+    if (batch > 1 && batch_c < (m - 1) * ldc + n) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: the C matrices of the batch overlap", prefix);
     if (!C || (k > 0 && (!A || !B))) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: null pointer", prefix);
     int rc = ensure_device();
     if (rc) return rc;
@@ -55,8 +59,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         std::snprintf(name, sizeof(name), "docc_%s_scale_c", prefix);
         int64_t blocks = (m * n + 255) / 256;
         if (blocks > 4096) blocks = 4096;
-        rc = launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C, (long) m, (long) n, (long) ldc, beta);
+        for (int64_t z = 0; z < batch && rc == 0; z++)   // an empty product: one small launch per entry
+            rc = launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C + z * batch_c, (long) m, (long) n, (long) ldc, beta);
         if (rc || (!bias && activation < 0)) return rc;
+        if (batch > 1) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 with an epilogue and a batch", prefix);
         // the epilogue of an empty product: C = act(beta * C + bias), through the elementwise kernel
         if (ldc != n) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 with an epilogue needs ldc == n", prefix);
         const int64_t shape[2] = {m, n}, row[2] = {1, n};
@@ -69,10 +75,11 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // contiguous extents of both operands must be multiples of the vector length
     const int64_t a_contig = ta ? m : k, b_contig = tb ? k : n;
     const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0) &&
-                         (a_contig % (int64_t) vec == 0) && (b_contig % (int64_t) vec == 0);
+                         (a_contig % (int64_t) vec == 0) && (b_contig % (int64_t) vec == 0) &&
+                         (batch == 1 || (batch_a % (int64_t) vec == 0 && batch_b % (int64_t) vec == 0));
     // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
     const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
-    TileConfig cfg = pick(m, n, aligned, force && force[0] == 'b' ? 1 : force && force[0] == 's' ? -1 : 0);
+    TileConfig cfg = pick(m, n, batch, aligned, force && force[0] == 'b' ? 1 : force && force[0] == 's' ? -1 : 0);
     // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES[xSTAGES] selects a built configuration directly (tuning)
     if (const char* c = std::getenv("DOCC_ROCM_GEMM_CFG")) {
         TileConfig t{};
@@ -82,7 +89,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // the asynchronous kernels need aligned operands and address a tile with 32-bit byte offsets
     const int64_t max_edge = cfg.bm > cfg.bn ? (cfg.bm > cfg.bk ? cfg.bm : cfg.bk) : (cfg.bn > cfg.bk ? cfg.bn : cfg.bk);
     const bool offsets_fit = max_edge * (lda > ldb ? lda : ldb) * (int64_t) sizeof(T) < (int64_t(1) << 32);
-    if (cfg.stages > 0 && !(aligned && offsets_fit)) cfg = pick(m, n, false, 0);
+    if (cfg.stages > 0 && !(aligned && offsets_fit)) cfg = pick(m, n, batch, false, 0);
     const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     size_t lds;
@@ -97,42 +104,62 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     }
     // the variants with bias / activation in the store carry the suffix "_e"
     if (bias || activation >= 0) std::strncat(name, "_e", sizeof(name) - std::strlen(name) - 1);
-    return launch(name, (uint32_t) tiles, 1, 1, 64 * cfg.waves, (uint32_t) lds, s, A, B, C, (long) m, (long) n,
-                  (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta, bias, activation);
+    return launch(name, (uint32_t) tiles, (uint32_t) batch, 1, 64 * cfg.waves, (uint32_t) lds, s, A, B, C, (long) m, (long) n,
+                  (long) k, (long) lda, (long) ldb, (long) ldc, alpha, beta, bias, activation, (long) batch_a, (long) batch_b,
+                  (long) batch_c);
 }
 
 } // namespace
+
+// A batch of equally shaped products in launches of at most 65535 entries (the limit of gridDim.y).
+template <typename T, typename S>
+static int gemm_batched(const char* prefix, docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                        S alpha, const T* A, int64_t lda, int64_t stride_a, const T* B, int64_t ldb, int64_t stride_b, S beta, S* C,
+                        int64_t ldc, int64_t stride_c, int64_t batch,
+                        TileConfig (*pick)(int64_t m, int64_t n, int64_t batch, bool aligned, int force)) {
+    if (batch < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: negative batch", prefix);
+    const int64_t kMaxGridY = 65535;
+    for (int64_t b0 = 0; b0 < batch; b0 += kMaxGridY) {
+        const int64_t nb = batch - b0 < kMaxGridY ? batch - b0 : kMaxGridY;
+        const int rc = gemm_launch<T, S>(prefix, stream, trans_a, trans_b, m, n, k, alpha, A ? A + b0 * stride_a : A, lda,
+                                         B ? B + b0 * stride_b : B, ldb, beta, C ? C + b0 * stride_c : C, ldc, pick, nullptr, -1, nb,
+                                         stride_a, stride_b, stride_c);
+        if (rc) return rc;
+    }
+    return 0;
+}
 
 extern "C" {
 
 // Tile selection. `force`: +1 largest tile, -1 smallest tile, 0 by problem size. Asynchronous
 // (staged) configurations need aligned operands; the others handle everything.
-static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn); }
+// tiles of one matrix times the number of matrices: what there is to spread over the compute units
+static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn, int64_t batch = 1) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; }
 
-static TileConfig pick_sgemm(int64_t m, int64_t n, bool aligned, int force) {
+static TileConfig pick_sgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
     const TileConfig wide{128, 256, 16, 4, 3}, big{128, 128, 16, 4, 3}, small{64, 64, 16, 4, 4};
     const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
-    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128) >= 256 ? plain_big : plain_small);
+    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128, batch) >= 256 ? plain_big : plain_small);
     if (force) return force > 0 ? wide : small;
     // the largest tile that still gives every CU a work-group
-    return tiles_of(m, n, 128, 256) >= 256 ? wide : tiles_of(m, n, 128, 128) >= 256 ? big : small;
+    return tiles_of(m, n, 128, 256, batch) >= 256 ? wide : tiles_of(m, n, 128, 128, batch) >= 256 ? big : small;
 }
 
-static TileConfig pick_dgemm(int64_t m, int64_t n, bool aligned, int force) {
+static TileConfig pick_dgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
     const TileConfig big{128, 128, 16, 4, 3}, mid{64, 64, 16, 4, 4}, small{64, 32, 16, 4, 4};
     const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
     if (!aligned) return force > 0 ? plain_big : plain_small;
     if (force) return force > 0 ? big : small;
-    const int64_t t = tiles_of(m, n, 64, 64);
+    const int64_t t = tiles_of(m, n, 64, 64, batch);
     return t >= 2048 ? big : t > 512 ? mid : small;   // few tiles: halve them so that two work-groups share a CU
 }
 
-static TileConfig pick_bgemm(int64_t m, int64_t n, bool aligned, int force) {
+static TileConfig pick_bgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
     const TileConfig big{256, 256, 64, 4, 2}, small{128, 128, 32, 4, 4};
     const TileConfig plain_big{256, 256, 64, 4, 0}, plain_small{128, 128, 64, 4, 0};
-    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 256, 256) >= 256 ? plain_big : plain_small);
+    if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 256, 256, batch) >= 256 ? plain_big : plain_small);
     if (force) return force > 0 ? big : small;
-    return tiles_of(m, n, 256, 256) >= 192 ? big : small;
+    return tiles_of(m, n, 256, 256, batch) >= 192 ? big : small;
 }
 
 int docc_rocm_sgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
@@ -172,6 +199,27 @@ int docc_rocm_bf16gemm_f32_epilogue(docc_rocm_stream_t stream, int trans_a, int 
                                     float* C, int64_t ldc, const float* bias, int activation) {
     return gemm_launch<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
                                         pick_bgemm, bias, activation);
+}
+
+int docc_rocm_sgemm_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                            const float* A, int64_t lda, int64_t stride_a, const float* B, int64_t ldb, int64_t stride_b, float beta,
+                            float* C, int64_t ldc, int64_t stride_c, int64_t batch) {
+    return gemm_batched<float, float>("sgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C,
+                                      ldc, stride_c, batch, pick_sgemm);
+}
+
+int docc_rocm_dgemm_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, double alpha,
+                            const double* A, int64_t lda, int64_t stride_a, const double* B, int64_t ldb, int64_t stride_b,
+                            double beta, double* C, int64_t ldc, int64_t stride_c, int64_t batch) {
+    return gemm_batched<double, double>("dgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta,
+                                        C, ldc, stride_c, batch, pick_dgemm);
+}
+
+int docc_rocm_bf16gemm_f32_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k, float alpha,
+                                   const uint16_t* A, int64_t lda, int64_t stride_a, const uint16_t* B, int64_t ldb,
+                                   int64_t stride_b, float beta, float* C, int64_t ldc, int64_t stride_c, int64_t batch) {
+    return gemm_batched<uint16_t, float>("bgemm", stream, trans_a, trans_b, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta,
+                                         C, ldc, stride_c, batch, pick_bgemm);
 }
 
 } // extern "C"

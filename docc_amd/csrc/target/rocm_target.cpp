@@ -212,8 +212,8 @@ protected:
     }
 
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
-        // one GEMM (alpha 1, beta 0) per batch entry, the shape of the reference's expansion
-        // (matmul_node.cpp:366-499)
+        // the batch of GEMMs (alpha 1, beta 0) that the reference's expansion loops over
+        // (matmul_node.cpp:366-499), as one launch
         const auto& n = mm();
         std::string fn, in_t, out_t, one, zero;
         switch (n.element()) {
@@ -222,19 +222,12 @@ protected:
             case types::PrimitiveType::BFloat: fn = "docc_rocm_bf16gemm_f32"; in_t = "uint16_t"; out_t = "float"; one = "1.0f"; zero = "0.0f"; break;
             default: throw std::runtime_error("Invalid element type for ROCM MatMul node");
         }
-        s << "for (int64_t __b = 0; __b < (int64_t) (" << n.batch() << "); __b++) {" << std::endl;
-        s.setIndent(s.indent() + 4);
-        s << "const " << in_t << " *__a_b = (const " << in_t << " *) " << name_of("A") << " + __b * (int64_t) ("
-          << symbolic::mul(n.m(), n.k()) << ");" << std::endl;
-        s << "const " << in_t << " *__b_b = (const " << in_t << " *) " << name_of("B");
-        if (n.b_is_batched()) s << " + __b * (int64_t) (" << symbolic::mul(n.k(), n.n()) << ")";
-        s << ";" << std::endl;
-        s << out_t << " *__y_b = (" << out_t << " *) " << name_of("Y") << " + __b * (int64_t) (" << symbolic::mul(n.m(), n.n())
-          << ");" << std::endl;
-        s << "DOCC_ROCM_CHECK(" << fn << "(nullptr, 111, 111, " << n.m() << ", " << n.n() << ", " << n.k() << ", " << one
-          << ", __a_b, " << n.k() << ", __b_b, " << n.n() << ", " << zero << ", __y_b, " << n.n() << "));" << std::endl;
-        s.setIndent(s.indent() - 4);
-        s << "}" << std::endl;
+        const Expression stride_b = n.b_is_batched() ? symbolic::mul(n.k(), n.n()) : Expression("0");
+        s << "DOCC_ROCM_CHECK(" << fn << "_batched(nullptr, 111, 111, " << n.m() << ", " << n.n() << ", " << n.k() << ", " << one
+          << ", (const " << in_t << " *) " << name_of("A") << ", " << n.k() << ", (int64_t) (" << symbolic::mul(n.m(), n.k())
+          << "), (const " << in_t << " *) " << name_of("B") << ", " << n.n() << ", (int64_t) (" << stride_b << "), " << zero
+          << ", (" << out_t << " *) " << name_of("Y") << ", " << n.n() << ", (int64_t) (" << symbolic::mul(n.m(), n.n())
+          << "), (int64_t) (" << n.batch() << ")));" << std::endl;
     }
 };
 

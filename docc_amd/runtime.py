@@ -65,6 +65,9 @@ _SIGNATURES = {
     "docc_rocm_dgemm_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _vp, _i64, _f64, _vp, _i64, _vp, _int],
     "docc_rocm_sgemm_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64, _vp, _int],
     "docc_rocm_bf16gemm_f32_epilogue": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _vp, _i64, _f32, _vp, _i64, _vp, _int],
+    "docc_rocm_dgemm_batched": [_vp, _int, _int, _i64, _i64, _i64, _f64, _vp, _i64, _i64, _vp, _i64, _i64, _f64, _vp, _i64, _i64, _i64],
+    "docc_rocm_sgemm_batched": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _i64, _vp, _i64, _i64, _f32, _vp, _i64, _i64, _i64],
+    "docc_rocm_bf16gemm_f32_batched": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _i64, _vp, _i64, _i64, _f32, _vp, _i64, _i64, _i64],
     "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
@@ -213,6 +216,14 @@ def gemm_epilogue(kind, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias=None,
     fn = {"d": "docc_rocm_dgemm_epilogue", "s": "docc_rocm_sgemm_epilogue", "b": "docc_rocm_bf16gemm_f32_epilogue"}[kind]
     act = -1 if activation is None else (UNARY_OPS[activation] if isinstance(activation, str) else activation)
     call(fn, stream, trans_a, trans_b, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, bias or None, act)
+
+
+def gemm_batched(kind, batch, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, trans_a=NO_TRANS,
+                 trans_b=NO_TRANS, stream=0) -> None:
+    """C[z] = alpha * op(A[z]) op(B[z]) + beta * C[z] for z < batch in one launch; strides in elements, 0 shares
+    an input across the batch; kind "d", "s" or "b" (bf16 inputs)."""
+    fn = {"d": "docc_rocm_dgemm_batched", "s": "docc_rocm_sgemm_batched", "b": "docc_rocm_bf16gemm_f32_batched"}[kind]
+    call(fn, stream, trans_a, trans_b, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, batch)
 
 
 def softmax_f32(rows, cols, X, Y, stream=0) -> None:

@@ -83,6 +83,26 @@ int docc_rocm_bf16gemm_f32_epilogue(docc_rocm_stream_t stream, int trans_a, int 
                                     float beta, float* C, int64_t ldc, const float* bias, int activation);
 
 /*
+ * A batch of `batch` equally shaped products in one launch: entry z uses
+ * A + z*stride_a, B + z*stride_b, C + z*stride_c (strides in elements; 0
+ * shares an input across the batch, the C matrices must not overlap).
+ * Replaces the loop of GEMM nodes that the reference's ml::MatMul expands
+ * to, one per batch entry (sdfg/src/data_flow/library_nodes/math/tensor/
+ * matmul_node.cpp:366-499); the reference's cuBLAS dispatcher has no batched
+ * form (opt/src/targets/cuda/blas/gemm.cpp:66-96).
+ */
+int docc_rocm_dgemm_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                            double alpha, const double* A, int64_t lda, int64_t stride_a, const double* B, int64_t ldb,
+                            int64_t stride_b, double beta, double* C, int64_t ldc, int64_t stride_c, int64_t batch);
+int docc_rocm_sgemm_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                            float alpha, const float* A, int64_t lda, int64_t stride_a, const float* B, int64_t ldb,
+                            int64_t stride_b, float beta, float* C, int64_t ldc, int64_t stride_c, int64_t batch);
+int docc_rocm_bf16gemm_f32_batched(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
+                                   float alpha, const uint16_t* A, int64_t lda, int64_t stride_a, const uint16_t* B,
+                                   int64_t ldb, int64_t stride_b, float beta, float* C, int64_t ldc, int64_t stride_c,
+                                   int64_t batch);
+
+/*
  * Y[r, :] = softmax(X[r, :]) for r in [0, rows), fp32, both [rows, cols]
  * contiguous. This is ml::Softmax over the last axis; any reduction over a
  * trailing contiguous axis of an N-d tensor is this call with

@@ -160,6 +160,21 @@ def test_bf16_gemm_text(tmp_path):
     assert "float __alpha = 1.0;" in src and "docc_rocm_malloc" not in src
 
 
+def test_matmul_node_is_one_batched_launch(tmp_path):
+    """[6, 32, 16] @ [16, 24]: B is shared (stride 0); with a batched B its stride is k*n."""
+    for shape_b, stride_b in (([16, 24], "0"), ([6, 16, 24], "384")):
+        b = StructuredSDFGBuilder("bmm")
+        for n in ("A", "B", "Y"):
+            b.add_container(n, F32, True)
+        b.add_matmul("A", "B", "Y", [6, 32, 16], shape_b)
+        s = b.move()
+        s.schedule("rocm", options={"offload": "none"})
+        src, _ = source_of(s, tmp_path)
+        assert ("docc_rocm_sgemm_batched(nullptr, 111, 111, 32, 24, 16, 1.0f, (const float *) A, 16, (int64_t) (512), "
+                f"(const float *) B, 24, (int64_t) ({stride_b}), 0.0f, (float *) Y, 24, (int64_t) (768), (int64_t) (6)));") in src
+        assert "for (int64_t __b" not in src
+
+
 def chain_sdfg():
     """T = A @ B; Y = softmax(T): the intermediate T is a transient."""
     b = StructuredSDFGBuilder("chain")
