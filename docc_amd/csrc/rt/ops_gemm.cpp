@@ -137,7 +137,7 @@ extern "C" {
 static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn, int64_t batch = 1) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; }
 
 static TileConfig pick_sgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
-    const TileConfig wide{128, 256, 16, 4, 3}, big{128, 128, 16, 4, 3}, small{64, 64, 16, 4, 4};
+    const TileConfig wide{128, 256, 32, 4, 2}, big{128, 128, 32, 4, 3}, small{64, 64, 16, 4, 4};
     const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
     if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128, batch) >= 256 ? plain_big : plain_small);
     if (force) return force > 0 ? wide : small;
