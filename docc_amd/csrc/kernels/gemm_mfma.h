@@ -97,25 +97,48 @@ __device__ __forceinline__ void gemm_store_wave_epilogue(OT* C, long ldc, long M
                                                          OT beta, const OT* bias, AccT (&acc)[TM][TN], RowFn acc_row) {
     const bool use_c = (beta != (OT) 0);
     const bool whole = row0 + TM * MT <= M && col0 + TN * MT <= N;
+    // the bias values of this lane's columns; without a bias -0.0, whose addition changes no value
+    OT b[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const long col = col0 + j * MT + lcol;
-        const bool col_ok = whole || col < N;
-        const OT b = (bias != nullptr && col_ok) ? bias[col] : (OT) 0;
+        b[j] = (bias != nullptr && (whole || col < N)) ? bias[col] : (OT) -0.0;
+    }
+    auto finish = [&](OT val, int j) {
+        asm volatile("" : "+v"(val));   // the product is rounded before the bias is added, as by the separate nodes
+        val += b[j];
+        if (ACT >= 0) val = unary<ACT>(val);
+        return val;
+    };
+    if (whole) {   // interior tile: one base address, constant offsets, no bounds tests
+        OT* base = C + (row0 + acc_row(0)) * ldc + col0 + lcol;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                OT old[NACC];
+                if (use_c) {
+#pragma unroll
+                    for (int r = 0; r < NACC; r++) old[r] = base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT];
+                }
+#pragma unroll
+                for (int r = 0; r < NACC; r++)
+                    base[(long) (i * MT + acc_row(r) - acc_row(0)) * ldc + j * MT] =
+                        finish(use_c ? gemm_axpby(alpha, (OT) acc[i][j][r], beta, old[r]) : alpha * acc[i][j][r], j);
+            }
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const long col = col0 + j * MT + lcol;
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int r = 0; r < NACC; r++) {
                 const long row = row0 + i * MT + acc_row(r);
-                if (whole || (row < M && col_ok)) {
+                if (row < M && col < N) {
                     OT* p = C + row * ldc + col;
-                    OT val = use_c ? gemm_axpby(alpha, (OT) acc[i][j][r], beta, *p) : alpha * acc[i][j][r];
-                    if (bias != nullptr) {
-                        asm volatile("" : "+v"(val));
-                        val += b;
-                    }
-                    if (ACT >= 0) val = unary<ACT>(val);
-                    *p = val;
+                    *p = finish(use_c ? gemm_axpby(alpha, (OT) acc[i][j][r], beta, *p) : alpha * acc[i][j][r], j);
                 }
             }
     }
