@@ -1,4 +1,5 @@
-// Row softmax over the last axis, fp32, for gfx950.
+// Softmax for gfx950: the fp32 row kernels (reduction over the last axis) and, below them, the
+// general forms: fp64, and a reduction over inner axes ([outer, reduce, inner] view).
 //
 // Replaces the seven loop nests SoftmaxNode::expand produces (reference
 // sdfg/src/data_flow/library_nodes/math/tensor/reduce_ops/softmax_node.cpp:142-252:
@@ -190,7 +191,7 @@ extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_stream(const 
         if (v > m) {
             s = s * exp_neg(m - v) + 1.0f; // m == -inf: s is 0 and exp(-inf) is 0
             m = v;
-        } else {
+        } else if (v != kNegInf) {   // -inf weighs nothing (and -inf - -inf must not reach the exponential); NaN poisons s
             s += exp_neg(v - m);
         }
     }
@@ -198,6 +199,146 @@ extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_stream(const 
     // a thread that saw no element has m = -inf, s = 0: contributes 0
     float contrib = (m == kNegInf) ? 0.f : s * exp_neg(m - gm);
     float gs = block_sum(contrib, lds);
+    gs += gm - gm;   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
     const float inv = 1.0f / gs;
     for (long c = threadIdx.x; c < cols; c += 256) y[c] = exp_neg(x[c] - gm) * inv;
 }
+
+// ------------------------------------------------------------------------------------------
+// General forms: the reference's node reduces over any set of axes and takes its element type
+// from its memlets (softmax_node.cpp:38-110). A block of adjacent axes is the middle extent of an
+// [outer, reduce, inner] view of the contiguous input.
+
+namespace {
+
+template <typename T> struct SoftmaxMath;
+template <> struct SoftmaxMath<float> {
+    static __device__ __forceinline__ float neg_inf() { return kNegInf; }
+    static __device__ __forceinline__ float exp_le0(float t) { return exp_neg(t); }
+    static __device__ __forceinline__ float max(float a, float b) { return fmaxf(a, b); }
+};
+template <> struct SoftmaxMath<double> {
+    static __device__ __forceinline__ double neg_inf() { return -__builtin_huge_val(); }
+    static __device__ __forceinline__ double exp_le0(double t) { return exp(t); }
+    static __device__ __forceinline__ double max(double a, double b) { return fmax(a, b); }
+};
+
+// running (maximum, sum of exp(x - maximum)) of the elements seen so far; (-inf, 0) for none
+template <typename T>
+__device__ __forceinline__ void online_step(T v, T& m, T& s) {
+    using M = SoftmaxMath<T>;
+    if (v > m) {
+        s = s * M::exp_le0(m - v) + (T) 1;   // m == -inf: s is 0 and exp(-inf) is 0
+        m = v;
+    } else if (v != M::neg_inf()) {   // -inf weighs nothing (and -inf - -inf must not reach the exponential); NaN poisons s
+        s += M::exp_le0(v - m);
+    }
+}
+
+// merges the pairs of the NP threads that share a column; lm / ls hold one pair per thread
+template <typename T>
+__device__ __forceinline__ void merge_pairs(const T* lm, const T* ls, int first, int step, int count, T& gm, T& gs) {
+    using M = SoftmaxMath<T>;
+    gm = M::neg_inf();
+    for (int i = 0; i < count; i++) gm = M::max(gm, lm[first + i * step]);
+    gs = (T) 0;
+    for (int i = 0; i < count; i++) {
+        const T m = lm[first + i * step];
+        if (m != M::neg_inf()) gs += ls[first + i * step] * M::exp_le0(m - gm);
+    }
+    gs += gm - gm;   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
+}
+
+// inner == 1, any type: one 256-thread block per row, two reads of the row.
+template <typename T>
+__device__ __forceinline__ void softmax_row_stream(const T* X, T* Y, long cols) {
+    using M = SoftmaxMath<T>;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const long row = blockIdx.x;
+    const T* x = X + row * cols;
+    T* y = Y + row * cols;
+    T m = M::neg_inf(), s = (T) 0;
+    for (long c = threadIdx.x; c < cols; c += 256) online_step(x[c], m, s);
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    // tree over the 256 pairs
+    for (int half = 128; half > 0; half >>= 1) {
+        if ((int) threadIdx.x < half) {
+            const T m2 = lm[threadIdx.x + half], s2 = ls[threadIdx.x + half];
+            const T m1 = lm[threadIdx.x], s1 = ls[threadIdx.x];
+            const T g = M::max(m1, m2);
+            T acc = (T) 0;
+            if (m1 != M::neg_inf()) acc += s1 * M::exp_le0(m1 - g);
+            if (m2 != M::neg_inf()) acc += s2 * M::exp_le0(m2 - g);
+            lm[threadIdx.x] = g;
+            ls[threadIdx.x] = acc;
+        }
+        __syncthreads();
+    }
+    const T gm = lm[0];
+    const T gs = ls[0] + (gm - gm);   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
+    for (long c = threadIdx.x; c < cols; c += 256) y[c] = M::exp_le0(x[c] - gm) / gs;
+}
+
+// inner > 1: a block owns 64 adjacent inner positions of one outer index (lane = inner position, so
+// that every access of a wave is one contiguous segment) and its four waves split the reduced extent.
+template <typename T>
+__device__ __forceinline__ void softmax_strided_tile(const T* X, T* Y, long reduce, long inner, long tiles) {
+    using M = SoftmaxMath<T>;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const long o = blockIdx.x / tiles;
+    const long col = (blockIdx.x % tiles) * 64 + (threadIdx.x & 63);
+    const int part = threadIdx.x >> 6;
+    const bool live = col < inner;
+    const T* x = X + o * reduce * inner + col;
+    T* y = Y + o * reduce * inner + col;
+    T m = M::neg_inf(), s = (T) 0;
+    if (live)
+        for (long r = part; r < reduce; r += 4) online_step(x[r * inner], m, s);
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    T gm, gs;
+    merge_pairs(lm, ls, (int) (threadIdx.x & 63), 64, 4, gm, gs);
+    if (live)
+        for (long r = part; r < reduce; r += 4) y[r * inner] = M::exp_le0(x[r * inner] - gm) / gs;
+}
+
+// inner a power of two up to 32: a block owns one outer index, whose [reduce, inner] slab is contiguous;
+// thread t walks the slab with stride 256 and therefore stays in column t % inner.
+template <typename T>
+__device__ __forceinline__ void softmax_strided_slab(const T* X, T* Y, long reduce, int inner) {
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    using M = SoftmaxMath<T>;
+    const long n = reduce * inner;
+    const T* x = X + (long) blockIdx.x * n;
+    T* y = Y + (long) blockIdx.x * n;
+    T m = M::neg_inf(), s = (T) 0;
+    for (long i = threadIdx.x; i < n; i += 256) online_step(x[i], m, s);
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    T gm, gs;
+    merge_pairs(lm, ls, (int) (threadIdx.x & (inner - 1)), inner, 256 / inner, gm, gs);
+    for (long i = threadIdx.x; i < n; i += 256) y[i] = M::exp_le0(x[i] - gm) / gs;
+}
+
+} // namespace
+
+extern "C" __global__ __launch_bounds__(256) void docc_softmax_f64_stream(const double* X, double* Y, long rows, long cols) {
+    softmax_row_stream<double>(X, Y, cols);
+}
+#define DOCC_SOFTMAX_STRIDED(T, SUFFIX)                                                                                     \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_tile(const T* X, T* Y, long reduce, long inner, \
+                                                                                  long tiles) {                             \
+        softmax_strided_tile<T>(X, Y, reduce, inner, tiles);                                                                \
+    }                                                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_slab(const T* X, T* Y, long reduce, int inner) { \
+        softmax_strided_slab<T>(X, Y, reduce, inner);                                                                       \
+    }
+DOCC_SOFTMAX_STRIDED(float, f32)
+DOCC_SOFTMAX_STRIDED(double, f64)

@@ -1,4 +1,5 @@
 // Launchers for ml::Softmax and the utility kernels (see include/docc_rocm_ops.h).
+#include <cstdio>
 #include <cstdlib>
 
 #include "docc_rocm_ops.h"
@@ -42,6 +43,31 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
         return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     }
     return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+}
+
+int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y) {
+    if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: precision must be 32 or 64");
+    if (outer < 0 || reduce < 0 || inner < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
+    if (outer == 0 || reduce == 0 || inner == 0) return 0;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
+    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
+    hipStream_t s = (hipStream_t) stream;
+    const char* t = precision == 32 ? "f32" : "f64";
+    char name[64];
+    if (inner == 1) {
+        if (outer > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
+        return launch("docc_softmax_f64_stream", (uint32_t) outer, 1, 1, 256, 0, s, X, Y, (long) outer, (long) reduce);
+    }
+    if (inner <= 32 && (inner & (inner - 1)) == 0) {
+        // a few inner positions: one work-group per outer index walks its contiguous slab
+        if (outer > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 outer indices");
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_slab", t);
+        return launch(name, (uint32_t) outer, 1, 1, 256, 0, s, X, Y, (long) reduce, (int) inner);
+    }
+    const int64_t tiles = (inner + 63) / 64;
+    if (tiles > 0x7fffffffLL / outer) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 work-groups");
+    std::snprintf(name, sizeof(name), "docc_softmax_%s_tile", t);
+    return launch(name, (uint32_t) (outer * tiles), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles);
 }
 
 static uint32_t grid_for(int64_t items) {

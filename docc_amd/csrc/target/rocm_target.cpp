@@ -242,8 +242,15 @@ protected:
 
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
         const auto& n = static_cast<const tensor::SoftmaxNode&>(node_);
-        s << "DOCC_ROCM_CHECK(docc_rocm_softmax_f32(nullptr, " << n.rows() << ", " << n.cols() << ", (const float *) "
-          << name_of("X") << ", (float *) " << name_of("Y") << "));" << std::endl;
+        if (n.last_axis_only() && n.element() == types::PrimitiveType::Float) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_softmax_f32(nullptr, " << n.rows() << ", " << n.cols() << ", (const float *) "
+              << name_of("X") << ", (float *) " << name_of("Y") << "));" << std::endl;
+            return;
+        }
+        // a block of adjacent axes: the middle extent of an [outer, extent, inner] view
+        s << "DOCC_ROCM_CHECK(docc_rocm_softmax(nullptr, " << (n.element() == types::PrimitiveType::Double ? 64 : 32) << ", "
+          << n.outer() << ", " << n.extent() << ", " << n.inner() << ", (const void *) " << name_of("X") << ", (void *) "
+          << name_of("Y") << "));" << std::endl;
     }
 };
 
@@ -561,8 +568,8 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
     } else if (node.code() == tensor::LibraryNodeType_Softmax) {
         auto* s = dynamic_cast<tensor::SoftmaxNode*>(&node);
         if (!s) return decline("not a Softmax node object");
-        if (s->element() != P::Float) return decline("only Float is supported");
-        if (!s->last_axis_only()) return decline("only a reduction over the last axis is supported");
+        if (s->element() != P::Float && s->element() != P::Double) return decline("element type must be Float or Double");
+        if (!s->adjacent_axes()) return decline("the reduced axes must be adjacent (one block)");
     } else if (node.code() == tensor::LibraryNodeType_Conv) {
         auto* c = dynamic_cast<tensor::ConvNode*>(&node);
         if (!c) return decline("not a Conv node object");

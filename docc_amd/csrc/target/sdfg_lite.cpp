@@ -234,6 +234,25 @@ bool SoftmaxNode::last_axis_only() const {
     return axes_[0] == -1 || axes_[0] == rank - 1;
 }
 
+std::vector<int64_t> SoftmaxNode::sorted_axes() const {
+    std::vector<int64_t> a = axes_;
+    const int64_t rank = (int64_t) shape_.size();
+    for (auto& v : a)
+        if (v < 0) v += rank;
+    std::sort(a.begin(), a.end());
+    a.erase(std::unique(a.begin(), a.end()), a.end());
+    return a;
+}
+
+bool SoftmaxNode::adjacent_axes() const {
+    const auto a = sorted_axes();
+    return !a.empty() && a.back() - a.front() + 1 == (int64_t) a.size();
+}
+
+Expression SoftmaxNode::outer() const { return product(shape_, 0, (size_t) sorted_axes().front()); }
+Expression SoftmaxNode::extent() const { return product(shape_, (size_t) sorted_axes().front(), (size_t) sorted_axes().back() + 1); }
+Expression SoftmaxNode::inner() const { return product(shape_, (size_t) sorted_axes().back() + 1, shape_.size()); }
+
 void SoftmaxNode::validate() const {
     if (shape_.empty()) throw InvalidSDFGException("Softmax: empty shape");
     if (axes_.empty()) throw InvalidSDFGException("Softmax: no reduction axis");

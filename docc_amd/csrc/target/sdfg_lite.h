@@ -192,6 +192,13 @@ public:
     Expression rows() const;  // product of all dims but the last
     Expression cols() const;  // the last dim
     bool last_axis_only() const;
+    // the axes, normalised and sorted; `adjacent` tells whether they form one block, which is the
+    // middle extent of an [outer, extent, inner] view of the input
+    std::vector<int64_t> sorted_axes() const;
+    bool adjacent_axes() const;
+    Expression outer() const;
+    Expression extent() const;
+    Expression inner() const;
 
     void validate() const override;
     void to_json(json::Value& j) const override;

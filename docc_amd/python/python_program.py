@@ -205,15 +205,21 @@ class _Lowering(ast.NodeVisitor):
         self.b.add_matmul(left.name, right.name, out.name, left.shape, right.shape)
         return out
 
-    def softmax(self, node: ast.AST, x: Any, axis: int, dest: Optional[str]) -> _Array:
+    def softmax(self, node: ast.AST, x: Any, axis: Any, dest: Optional[str]) -> _Array:
+        """`axis`: an int, a tuple of ints, or None for all axes (scipy's default)."""
         if not isinstance(x, _Array):
             self.fail(node, "softmax of a non-array")
-        if axis not in (-1, len(x.shape) - 1):
-            self.fail(node, "softmax over an axis other than the last")
-        if x.elem != PrimitiveType.Float:
-            self.fail(node, "softmax of a non-float32 array")
+        rank = len(x.shape)
+        axes = list(range(rank)) if axis is None else [axis] if isinstance(axis, int) else list(axis)
+        if not axes or any(not isinstance(a, int) or a < -rank or a >= rank for a in axes):
+            self.fail(node, "softmax axis out of range")
+        normal = sorted({a % rank for a in axes})
+        if normal[-1] - normal[0] + 1 != len(normal):
+            self.fail(node, "softmax over axes that are not adjacent")
+        if x.elem not in (PrimitiveType.Float, PrimitiveType.Double):
+            self.fail(node, "softmax of an array that is neither float32 nor float64")
         out = self.new_array(x.shape, x.elem, dest)
-        self.b.add_reduce_op("softmax", x.name, out.name, x.shape, [axis])
+        self.b.add_reduce_op("softmax", x.name, out.name, x.shape, axes)
         return out
 
     def conv(self, node: ast.Call, dest: Optional[str]) -> _Array:
@@ -432,7 +438,7 @@ class _Lowering(ast.NodeVisitor):
         except Exception:  # scipy is optional
             _sp = scipy_softmax = None
         if fn is not None and fn in (scipy_softmax, _functions.softmax):
-            return self.softmax(node, self.ev(node.args[0]), self.kw(node, "axis", 1, -1 if fn is _functions.softmax else None) or -1, dest)
+            return self.softmax(node, self.ev(node.args[0]), self.kw(node, "axis", 1, -1 if fn is _functions.softmax else None), dest)
         if fn is _functions.conv2d:
             return self.conv(node, dest)
         axis_last = lambda x: self.kw(node, "axis", 1, None) in (-1, len(x.shape) - 1) and self.kw(node, "keepdims", None, False) is True

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "docc_rocm_sgemm_batched": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _i64, _vp, _i64, _i64, _f32, _vp, _i64, _i64, _i64],
     "docc_rocm_bf16gemm_f32_batched": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _i64, _vp, _i64, _i64, _f32, _vp, _i64, _i64, _i64],
     "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
+    "docc_rocm_softmax": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
     "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
@@ -224,6 +225,11 @@ def gemm_batched(kind, batch, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b
     an input across the batch; kind "d", "s" or "b" (bf16 inputs)."""
     fn = {"d": "docc_rocm_dgemm_batched", "s": "docc_rocm_sgemm_batched", "b": "docc_rocm_bf16gemm_f32_batched"}[kind]
     call(fn, stream, trans_a, trans_b, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, batch)
+
+
+def softmax(precision, outer, reduce, inner, X, Y, stream=0) -> None:
+    """Softmax over the middle extent of an [outer, reduce, inner] view; precision 32 or 64."""
+    call("docc_rocm_softmax", stream, precision, outer, reduce, inner, X, Y)
 
 
 def softmax_f32(rows, cols, X, Y, stream=0) -> None:

@@ -194,12 +194,12 @@ class _FxLowering:
             return _Probs(x)
         if not isinstance(x, _T):
             self.fail(node, "softmax of this value")
-        if dim not in (-1, len(x.shape) - 1):
-            self.fail(node, "softmax over an axis other than the last")
-        if x.dtype != self.torch.float32:
-            self.fail(node, "softmax on a dtype other than float32")
+        if not -len(x.shape) <= dim < len(x.shape):
+            self.fail(node, "softmax dim out of range")
+        if x.dtype not in (self.torch.float32, self.torch.float64):
+            self.fail(node, "softmax on a dtype other than float32 / float64")
         out = self.new_tensor(x.shape, x.dtype, dest)
-        self.builder.add_reduce_op("softmax", x.name, out.name, x.shape, [-1])
+        self.builder.add_reduce_op("softmax", x.name, out.name, x.shape, [dim])
         return out
 
     def conv2d(self, node, x, w, bias, stride, padding, dilation, groups, dest):

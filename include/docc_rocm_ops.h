@@ -113,6 +113,17 @@ int docc_rocm_bf16gemm_f32_batched(docc_rocm_stream_t stream, int trans_a, int t
 int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols, const float* X, float* Y);
 
 /*
+ * ml::Softmax in general: X and Y are contiguous and viewed as [outer, reduce, inner], the
+ * softmax runs over the middle extent (a block of adjacent axes of the node; the product of
+ * the axes before it is `outer`, of those after it `inner`); precision 32 (float) or 64
+ * (double). The reference's node takes any axes and its element type from its memlets
+ * (softmax_node.cpp:38-110). inner == 1 with precision 32 is docc_rocm_softmax_f32; the other
+ * forms read X twice (running maximum and sum, then the results).
+ */
+int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner,
+                      const void* X, void* Y);
+
+/*
  * ml::Conv, 2-d, NCHW fp32, group 1 (reference conv_node.h:9-22,48-217):
  *   Y[n,oc,oh,ow] = bias[oc] + sum_{ic,kh,kw} X[n,ic,oh*sh-ph+kh*dh, ow*sw-pw+kw*dw] * W[oc,ic,kh,kw]
  * with zero padding (taps outside the image contribute 0); bias may be NULL.

@@ -52,6 +52,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     for name in ("oracle_softmax_expanded_f32", "oracle_softmax_numpy_f32"):
         getattr(lib, name).argtypes = [_i64, _i64, _f32p, _f32p]
         getattr(lib, name).restype = ctypes.c_int
+    lib.oracle_softmax_expanded_f64.argtypes = [_i64, _i64, _f64p, _f64p]
+    lib.oracle_softmax_expanded_f64.restype = ctypes.c_int
     lib.oracle_conv_out_dim.argtypes = [_i64] * 6
     lib.oracle_conv_out_dim.restype = _i64
     lib.oracle_conv2d_f32.argtypes = [_i64] * 13 + [_f32p, _f32p, _f32p, _f32p]
@@ -169,6 +171,29 @@ def softmax(X, variant="numpy", lib=None) -> np.ndarray:
     if fn(rows, cols, _p(X, _f32p), _p(out, _f32p)) != 0:
         raise MemoryError("oracle softmax could not allocate its temporaries")
     return out
+
+
+def softmax_axes(X, axes=(-1,), lib=None) -> np.ndarray:
+    """Softmax over any set of axes of an fp32 or fp64 array, the way the node's expansion computes it
+    (reference softmax_node.cpp:38-265): the reduced axes are moved to the end in ascending order, which is
+    the order the reduce nests visit them in, and the row form runs on that view."""
+    lib = lib or load()
+    X = np.asarray(X)
+    dt = np.float64 if X.dtype == np.float64 else np.float32
+    axes = sorted({a % X.ndim for a in axes})
+    kept = [d for d in range(X.ndim) if d not in axes]
+    perm = kept + axes
+    Xt = _c(np.transpose(X, perm), dt)
+    cols = int(np.prod([X.shape[a] for a in axes])) if axes else 1
+    rows = Xt.size // cols if cols else 0
+    out = np.empty_like(Xt)
+    if dt == np.float64:
+        rc = lib.oracle_softmax_expanded_f64(rows, cols, _p(Xt, _f64p), _p(out, _f64p))
+    else:
+        rc = lib.oracle_softmax_expanded_f32(rows, cols, _p(Xt, _f32p), _p(out, _f32p))
+    if rc != 0:
+        raise MemoryError("oracle softmax could not allocate its temporaries")
+    return np.ascontiguousarray(np.transpose(out, np.argsort(perm)))
 
 
 def conv_out_dim(d_in, pad, dilation, kernel, stride) -> int:

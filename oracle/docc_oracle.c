@@ -245,6 +245,41 @@ done:
 }
 
 /*
+ * The same expansion for fp64 elements (the element type of the node is that of its
+ * memlets, softmax_node.cpp:89-90; Max uses fmax, Exp uses exp: max_node.cpp:56-67,
+ * cmath_node.h:364-365). The two broadcast temporaries are read in place of the
+ * reduced ones; the arithmetic and its order are those of the seven nests above.
+ * Reductions over other axes than the last are this function on the input with the
+ * reduced axes moved to the end, in ascending order: the reduce nests visit the reduced
+ * dimensions in that order (reduce_node.cpp:188-333).
+ */
+ORACLE_API int oracle_softmax_expanded_f64(int64_t rows, int64_t cols, const double* X, double* Y) {
+    size_t full = (size_t) rows * (size_t) cols;
+    double* tmp_max = (double*) malloc(sizeof(double) * (size_t) (rows ? rows : 1));
+    double* tmp_exp = (double*) malloc(sizeof(double) * (full ? full : 1));
+    double* tmp_sum = (double*) malloc(sizeof(double) * (size_t) (rows ? rows : 1));
+    int rc = 0;
+    if (!tmp_max || !tmp_exp || !tmp_sum) {
+        rc = -1;
+        goto done;
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < rows; i++) {
+        tmp_max[i] = -INFINITY;
+        for (int64_t k = 0; k < cols; k++) tmp_max[i] = fmax(X[i * cols + k], tmp_max[i]);
+        for (int64_t j = 0; j < cols; j++) tmp_exp[i * cols + j] = exp(X[i * cols + j] - tmp_max[i]);
+        tmp_sum[i] = 0.0;
+        for (int64_t k = 0; k < cols; k++) tmp_sum[i] = tmp_exp[i * cols + k] + tmp_sum[i];
+        for (int64_t j = 0; j < cols; j++) Y[i * cols + j] = tmp_exp[i * cols + j] / tmp_sum[i];
+    }
+done:
+    free(tmp_max);
+    free(tmp_exp);
+    free(tmp_sum);
+    return rc;
+}
+
+/*
  * The decomposed numpy form the reference's own softmax benchmark compiles
  * (python/benchmarks/npbench/deep_learning/softmax/test_softmax.py:24-28):
  *   tmp_max = max(x, -1, keepdims); tmp_out = exp(x - tmp_max);

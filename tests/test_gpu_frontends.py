@@ -343,3 +343,36 @@ def test_torch_reductions_fp32():
     assert avg.is_cuda and avg.shape == (8, 16) and mx.shape == (8, 1, 14, 14)
     assert torch.allclose(avg, x.double().mean(dim=(2, 3)).float(), rtol=1e-5, atol=1e-6)
     assert torch.equal(mx, x.amax(dim=1, keepdim=True))
+
+
+def test_softmax_over_other_axes_and_fp64_through_both_front_ends():
+    """scipy.special.softmax with an axis argument (an inner axis, a block of axes, all axes by default) on fp32
+    and fp64, and torch.softmax over a leading dim."""
+    @native(target="rocm")
+    def over_axis_1(x):
+        return scipy.special.softmax(x, axis=1)
+
+    @native(target="rocm")
+    def over_block(x):
+        return scipy.special.softmax(x, axis=(0, 1))
+
+    @native(target="rocm")
+    def over_all(x):
+        return scipy.special.softmax(x)
+
+    rng = np.random.default_rng(8)
+    for dt, tol in ((np.float32, 1e-5), (np.float64, 1e-12)):
+        x = (rng.standard_normal((6, 40, 24)) * 4).astype(dt)
+        for fn, axes in ((over_axis_1, (1,)), (over_block, (0, 1)), (over_all, (0, 1, 2))):
+            y = fn(x)
+            assert y.dtype == dt and y.shape == x.shape
+            assert rel_err_max(y, oracle.softmax_axes(x, axes)) <= tol
+            np.testing.assert_allclose(y, scipy.special.softmax(x.astype(np.float64), axis=axes), rtol=20 * tol, atol=1e-30)
+
+    class S(torch.nn.Module):
+        def forward(self, a):
+            return torch.softmax(a, dim=0)
+
+    a = torch.randn(33, 70, dtype=torch.float64)
+    out = docc_torch.compile_torch(S(), (a,), target="rocm")(a)
+    assert rel_err_max(out.numpy(), oracle.softmax_axes(a.numpy(), (0,))) <= 1e-12

@@ -104,3 +104,72 @@ def test_softmax_full_config(rt):
     # oracle on a slice of rows (the oracle is the slow side)
     sel = np.r_[0:64, 4000:4064, 8128:8192]
     assert rel_err_max(Y[sel], oracle.softmax(X[sel])) <= TOL_F32
+
+
+# ---- the general entry point: fp64, and reductions over inner axes ------------------------------------
+
+GENERAL = [  # shape, axes
+    ((5, 7), (0,)), ((64, 300), (0,)), ((3, 1000, 8), (1,)), ((4, 257, 16), (1,)), ((2, 50, 33), (1,)), ((6, 31, 64), (1,)),
+    ((2, 9, 200), (0, 1)), ((3, 4, 5, 6), (1, 2)), ((7, 129), (-1,)), ((1, 5000), (-1,)), ((4, 6, 2), (1,)), ((1, 4096, 1), (1,)),
+    ((3, 3, 3), (0, 1, 2)), ((2, 2048, 4), (-2,)), ((5, 1, 70), (1,)),
+]
+
+
+@pytest.mark.parametrize("dt,tol", [(np.float32, TOL_F32), (np.float64, 1e-12)], ids=["f32", "f64"])
+@pytest.mark.parametrize("shape,axes", GENERAL, ids=["x".join(map(str, s)) + "_ax" + "".join(str(a % len(s)) for a in ax) for s, ax in GENERAL])
+def test_softmax_general_matches_oracle(rt, dt, tol, shape, axes):
+    rng = np.random.default_rng(sum(shape) * 31 + len(axes))
+    X = (rng.standard_normal(shape) * 8).astype(dt)
+    norm = sorted(a % len(shape) for a in axes)
+    outer = int(np.prod(shape[:norm[0]], dtype=np.int64))
+    reduce_ = int(np.prod(shape[norm[0]:norm[-1] + 1], dtype=np.int64))
+    inner = int(np.prod(shape[norm[-1] + 1:], dtype=np.int64))
+    x = dev(X)
+    y = torch.empty_like(x)
+    rt.softmax(64 if dt == np.float64 else 32, outer, reduce_, inner, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    Y = host(y)
+    ref = oracle.softmax_axes(X, axes)
+    assert rel_err_max(Y, ref) <= tol
+    np.testing.assert_allclose(Y, ref, rtol=20 * tol, atol=1e-300 if dt == np.float64 else 1e-30)
+    np.testing.assert_allclose(Y.sum(axis=tuple(norm)), 1.0, rtol=0, atol=max(tol, 1e-14) * 4)
+
+
+def test_softmax_general_edge_values_and_empty(rt):
+    """Infinite and NaN entries poison their own column only, the way the node's Sub / Exp / Sum / Div steps
+    would; an empty extent launches nothing."""
+    X = np.zeros((3, 6, 5), np.float64)
+    X[0, 2, 1] = np.inf          # inf - inf = NaN in the Sub step: the whole column becomes NaN
+    X[1, 0, 3] = np.nan
+    X[2, :, 4] = -np.inf         # max = -inf: NaN as well
+    X[2, 1, 0] = -np.inf         # one -inf among finite values: weight 0
+    x = dev(X)
+    y = torch.empty_like(x)
+    rt.softmax(64, 3, 6, 5, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    Y = host(y)
+    with np.errstate(invalid="ignore"):
+        ref = oracle.softmax_axes(X, (1,))
+    assert np.array_equal(np.isnan(Y), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    np.testing.assert_allclose(Y[ok], ref[ok], rtol=1e-14)
+    assert Y[2, 1, 0] == 0.0 and np.isnan(Y[0, :, 1]).all() and np.isnan(Y[2, :, 4]).all()
+    # the same for the fp32 row kernels
+    Xr = np.zeros((4, 300), np.float32)
+    Xr[0, 7] = np.inf
+    Xr[1, 9] = np.nan
+    Xr[2, :] = -np.inf
+    for cols in (300, 40004):     # block kernel, streaming kernel
+        Xc = np.zeros((4, cols), np.float32)
+        Xc[:, :300] = Xr
+        Xc[2, :] = -np.inf
+        Yr = run_softmax(rt, Xc)
+        assert np.isnan(Yr[:3]).all() and np.allclose(Yr[3], 1.0 / cols)
+    z = torch.zeros(8, device="cuda")
+    rt.softmax(32, 0, 4, 2, z.data_ptr(), z.data_ptr())
+    rt.softmax(64, 2, 0, 2, z.data_ptr(), z.data_ptr())
+    torch.cuda.synchronize()
+    assert host(z).sum() == 0
+    from docc_amd.runtime import RocmRuntimeError
+    with pytest.raises(RocmRuntimeError, match="precision"):
+        rt.softmax(16, 1, 4, 2, z.data_ptr(), z.data_ptr())

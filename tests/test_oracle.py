@@ -111,6 +111,21 @@ def test_softmax_closed_forms():
     assert oracle.softmax(np.zeros((0, 7), np.float32)).shape == (0, 7)
 
 
+@pytest.mark.parametrize("dt,tol", [(np.float32, 1e-6), (np.float64, 1e-15)])
+@pytest.mark.parametrize("axes", [(-1,), (0,), (1,), (1, 2), (0, 1, 2), (0, 2)])
+def test_softmax_over_any_axes_against_scipy(dt, tol, axes):
+    """The library cross-check (scipy in fp64), sums of one over the reduced axes, and for the last axis the
+    row form itself: a transposition slip or a wrong inverse permutation fails the first two."""
+    rng = np.random.default_rng(11 + len(axes))
+    X = (rng.standard_normal((5, 7, 6)) * 6).astype(dt)
+    Y = oracle.softmax_axes(X, axes)
+    assert Y.dtype == dt and Y.shape == X.shape
+    assert rel(Y, scipy.special.softmax(X.astype(np.float64), axis=axes)) <= tol
+    assert np.allclose(Y.sum(axis=axes), 1.0, atol=10 * tol * X.size)
+    if axes == (-1,) and dt == np.float32:
+        assert np.array_equal(Y, oracle.softmax(X, variant="expanded"))
+
+
 # ---- conv -----------------------------------------------------------------------------
 
 def test_conv_golden():

@@ -96,12 +96,12 @@ def test_mapper_sets_implementation_types_and_declines_what_the_kernels_lack():
     s = StructuredSDFG.parse(json.dumps(data))
     s.schedule("rocm", options={"require_all_mapped": False})
     assert s.library_nodes()[0]["implementation_type"] == "BLAS"
-    # softmax over a leading axis, grouped conv, head dim != 64
+    # softmax over scattered axes, grouped conv, head dim != 64
     b = StructuredSDFGBuilder("s")
     b.add_container("X", F32, True)
     b.add_container("Y", F32, True)
-    b.add_reduce_op("softmax", "X", "Y", [4, 8], [0])
-    with pytest.raises(InvalidSDFGException, match="last axis"):
+    b.add_reduce_op("softmax", "X", "Y", [4, 8, 3], [0, 2])
+    with pytest.raises(InvalidSDFGException, match="adjacent"):
         b.move().schedule("rocm")
     b = StructuredSDFGBuilder("c")
     for n in ("X", "W", "Y"):
@@ -158,6 +158,25 @@ def test_bf16_gemm_text(tmp_path):
     assert report["function"] == 'extern "C" void bf(__bf16 *A, __bf16 *B, int64_t _s0, float *_docc_ret_0)'
     assert "docc_rocm_bf16gemm_f32(nullptr, 111, 111, _s0, _s0, _s0, __alpha, (const uint16_t *) __A" in src
     assert "float __alpha = 1.0;" in src and "docc_rocm_malloc" not in src
+
+
+def test_softmax_over_inner_axes_and_fp64(tmp_path):
+    """A block of adjacent axes is the middle extent of an [outer, extent, inner] view; the last axis of an
+    fp32 tensor keeps its own entry point."""
+    cases = [(F32, [4, 8, 6], [1], "docc_rocm_softmax(nullptr, 32, 4, 8, 6, (const void *) X, (void *) Y)"),
+             (F32, [4, 8, 6], [0, 1], "docc_rocm_softmax(nullptr, 32, 1, 32, 6, (const void *) X, (void *) Y)"),
+             (F64, [4, 8, 6], [-1], "docc_rocm_softmax(nullptr, 64, 32, 6, 1, (const void *) X, (void *) Y)"),
+             (F64, [4, 8, 6], [-2, 2], "docc_rocm_softmax(nullptr, 64, 4, 48, 1, (const void *) X, (void *) Y)"),
+             (F32, [4, 8, 6], [2], "docc_rocm_softmax_f32(nullptr, 32, 6, (const float *) X, (float *) Y)")]
+    for ptr, shape, axes, text in cases:
+        b = StructuredSDFGBuilder("sm")
+        b.add_container("X", ptr, True)
+        b.add_container("Y", ptr, True)
+        b.add_reduce_op("softmax", "X", "Y", shape, axes)
+        s = b.move()
+        s.schedule("rocm", options={"offload": "none"})
+        src, _ = source_of(s, tmp_path)
+        assert text in src, (axes, src)
 
 
 def test_matmul_node_is_one_batched_launch(tmp_path):
