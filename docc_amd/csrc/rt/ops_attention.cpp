@@ -28,3 +28,75 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
                   (uint32_t) ((SQ + 127) / 128), (uint32_t) (B * H), 1, 256, lds, (hipStream_t) stream, Q, K, V, O,
                   (int) SQ, (int) SKV, scale_log2e);
 }
+
+// ---- any head dimension, through a caller-provided workspace -----------------------------------
+
+namespace {
+
+// bytes of scores (fp32) + probabilities (bf16) + an fp32 result per (batch, head) pair
+int64_t attention_bytes_per_head(int64_t SQ, int64_t SKV, int64_t D, int out_bf16) {
+    const int64_t scores = (SQ * SKV * 4 + 255) / 256 * 256, probs = (SQ * SKV * 2 + 255) / 256 * 256;
+    const int64_t out32 = out_bf16 ? (SQ * D * 4 + 255) / 256 * 256 : 0;
+    return scores + probs + out32;
+}
+
+constexpr int64_t kAttentionWorkspaceCap = int64_t(2) << 30;   // heads are processed in chunks that fit this
+
+int64_t attention_heads_per_chunk(int64_t BH, int64_t per_head) {
+    int64_t n = per_head > 0 ? kAttentionWorkspaceCap / per_head : BH;
+    if (n < 1) n = 1;
+    return n < BH ? n : BH;
+}
+
+} // namespace
+
+extern "C" int64_t docc_rocm_attention_bf16_workspace_bytes(int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, int out_bf16) {
+    if (B <= 0 || H <= 0 || SQ <= 0 || SKV <= 0 || D <= 0) return 0;
+    if (D == 64) return 0;   // the fused kernel keeps scores and probabilities in registers
+    const int64_t per_head = attention_bytes_per_head(SQ, SKV, D, out_bf16);
+    return attention_heads_per_chunk(B * H, per_head) * per_head;
+}
+
+extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                                           float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
+                                           int out_bf16, void* workspace, int64_t workspace_bytes) {
+    if (D == 64) return docc_rocm_attention_bf16(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16);
+    if (B < 0 || H < 0 || SQ < 0 || SKV < 0 || D < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: negative shape");
+    if (B == 0 || H == 0 || SQ == 0) return 0;
+    if (SKV == 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: no keys (softmax over an empty axis)");
+    if (D == 0) return 0;
+    if (!Q || !K || !V || !O) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: null pointer");
+    if (!(scale > 0.f) || !std::isfinite(scale)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: scale must be positive and finite");
+    const int64_t need = docc_rocm_attention_bf16_workspace_bytes(B, H, SQ, SKV, D, out_bf16);
+    if (!workspace || workspace_bytes < need || ((uintptr_t) workspace % 256) != 0)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: head dim %lld needs a 256-byte aligned workspace of %lld bytes",
+                    (long long) D, (long long) need);
+    // S = scale * Q K^T (batched bf16 GEMM, fp32 out), P = softmax rows of S, rounded to bf16, O = P V
+    const int64_t BH = B * H, per_head = attention_bytes_per_head(SQ, SKV, D, out_bf16);
+    const int64_t chunk = attention_heads_per_chunk(BH, per_head);
+    const int64_t scores_bytes = (SQ * SKV * 4 + 255) / 256 * 256, probs_bytes = (SQ * SKV * 2 + 255) / 256 * 256;
+    char* ws = (char*) workspace;
+    float* S = (float*) ws;
+    uint16_t* P = (uint16_t*) (ws + chunk * scores_bytes);
+    float* O32 = (float*) (ws + chunk * (scores_bytes + probs_bytes));
+    // inside the chunk the matrices are packed (strides in elements, not the rounded byte sizes)
+    for (int64_t h0 = 0; h0 < BH; h0 += chunk) {
+        const int64_t nh = BH - h0 < chunk ? BH - h0 : chunk;
+        int rc = docc_rocm_bf16gemm_f32_batched(stream, DOCC_ROCM_NO_TRANS, DOCC_ROCM_TRANS, SQ, SKV, D, scale, Q + h0 * SQ * D, D,
+                                                SQ * D, K + h0 * SKV * D, D, SKV * D, 0.f, S, SKV, SQ * SKV, nh);
+        if (rc) return rc;
+        rc = docc_rocm_softmax_f32(stream, nh * SQ, SKV, S, S);
+        if (rc) return rc;
+        rc = docc_rocm_convert_f32_to_bf16(stream, nh * SQ * SKV, S, P);
+        if (rc) return rc;
+        float* out = out_bf16 ? O32 : (float*) O + h0 * SQ * D;
+        rc = docc_rocm_bf16gemm_f32_batched(stream, DOCC_ROCM_NO_TRANS, DOCC_ROCM_NO_TRANS, SQ, D, SKV, 1.f, P, SKV, SQ * SKV,
+                                            V + h0 * SKV * D, D, SKV * D, 0.f, out, D, SQ * D, nh);
+        if (rc) return rc;
+        if (out_bf16) {
+            rc = docc_rocm_convert_f32_to_bf16(stream, nh * SQ * D, O32, (uint16_t*) O + h0 * SQ * D);
+            if (rc) return rc;
+        }
+    }
+    return 0;
+}

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <set>
+#include <sstream>
 
 namespace sdfg::rocm {
 
@@ -297,10 +298,33 @@ protected:
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
         const auto& a = static_cast<const tensor::AttentionNode&>(node_);
         const auto& q = a.shape_q();
-        s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16(nullptr, " << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv()
-          << ", " << q[3] << ", (float) (" << a.scale() << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) "
-          << name_of("K") << ", (const uint16_t *) " << name_of("V") << ", (void *) " << name_of("O") << ", "
-          << (a.output_element() == types::PrimitiveType::BFloat ? 1 : 0) << "));" << std::endl;
+        const int out_bf16 = a.output_element() == types::PrimitiveType::BFloat ? 1 : 0;
+        int64_t d = 0;
+        if (symbolic::is_integer(q[3], &d) && d == 64) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16(nullptr, " << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv()
+              << ", " << q[3] << ", (float) (" << a.scale() << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) "
+              << name_of("K") << ", (const uint16_t *) " << name_of("V") << ", (void *) " << name_of("O") << ", " << out_bf16
+              << "));" << std::endl;
+            return;
+        }
+        // another head dimension (or one known at run time only): scores and probabilities live in a
+        // workspace that this node allocates around its launches
+        std::ostringstream dims;
+        dims << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv() << ", " << q[3];
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "const int64_t __ws_bytes = docc_rocm_attention_bf16_workspace_bytes(" << dims.str() << ", " << out_bf16 << ");" << std::endl;
+        s << "void *__ws = nullptr;" << std::endl;
+        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc(&__ws, (size_t) __ws_bytes));" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16_ws(nullptr, " << dims.str() << ", (float) (" << a.scale()
+          << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) " << name_of("K") << ", (const uint16_t *) "
+          << name_of("V") << ", (void *) " << name_of("O") << ", " << out_bf16 << ", __ws, __ws_bytes));" << std::endl;
+        s << "if (__ws) {" << std::endl;
+        s << "    DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
+        s << "    DOCC_ROCM_CHECK(docc_rocm_free(__ws));" << std::endl;
+        s << "}" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
     }
 };
 
@@ -584,8 +608,7 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!a) return decline("not an Attention node object");
         if (a->element() != P::BFloat) return decline("inputs must be BFloat");
         if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
-        int64_t d = 0;
-        if (!symbolic::is_integer(a->shape_q()[3], &d) || d != 64) return decline("head dimension must be 64");
+        // head dimension 64 runs the fused kernel, any other the GEMM / softmax / GEMM sequence
     } else if (is_elementwise_code(node.code())) {
         auto* e = dynamic_cast<tensor::ElementWiseNode*>(&node);
         if (!e) return decline("not an elementwise node object");

@@ -72,6 +72,8 @@ _SIGNATURES = {
     "docc_rocm_softmax": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
+    "docc_rocm_attention_bf16_workspace_bytes": [_i64] * 5 + [_int],
+    "docc_rocm_attention_bf16_ws": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int, _vp, _i64],
     "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
     "docc_rocm_elementwise_unary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp],
@@ -85,7 +87,7 @@ _SIGNATURES = {
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
-            "docc_rocm_report_failure": None}
+            "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64}
 
 #: every symbol the two public headers declare
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -243,6 +245,16 @@ def conv2d_f32(N, C, H, W, OC, KH, KW, stride, pad, dilation, X, Wt, bias, Y, st
 
 def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0) -> None:
     call("docc_rocm_attention_bf16", stream, B, H, SQ, SKV, D, scale, Q, K, V, O, 1 if out_bf16 else 0)
+
+
+def attention_bf16_workspace_bytes(B, H, SQ, SKV, D, out_bf16=False) -> int:
+    return int(lib().docc_rocm_attention_bf16_workspace_bytes(B, H, SQ, SKV, D, 1 if out_bf16 else 0))
+
+
+def attention_bf16_ws(B, H, SQ, SKV, D, scale, Q, K, V, O, workspace, workspace_bytes, out_bf16=False, stream=0) -> None:
+    """Attention for any head dimension; `workspace` is device memory of attention_bf16_workspace_bytes(...) bytes."""
+    call("docc_rocm_attention_bf16_ws", stream, B, H, SQ, SKV, D, scale, Q, K, V, O, 1 if out_bf16 else 0, workspace or None,
+         workspace_bytes)
 
 
 def copy_bytes(nbytes, src, dst, stream=0) -> None:

@@ -140,11 +140,25 @@ int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_
  *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
  * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32
  * scores, softmax and accumulation; non-causal. O is [B,H,SQ,D], fp32 when
- * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 64.
+ * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 64
+ * (docc_rocm_attention_bf16_ws takes any D).
  */
 int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
                              float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
                              int out_bf16);
+
+/*
+ * The same node for any head dimension D, with device memory of the caller for the scores:
+ * D == 64 runs the kernel above and needs none; otherwise S = scale * Q K^T (batched bf16
+ * GEMM, fp32 out), a row softmax, the probabilities rounded to bf16 and O = P V run as
+ * separate kernels over chunks of (batch, head) pairs that keep the workspace under 2 GiB.
+ * `workspace` must be 256-byte aligned and hold what _workspace_bytes returns for the
+ * same arguments (0 when no workspace is needed). Calls on one stream may share a workspace.
+ */
+int64_t docc_rocm_attention_bf16_workspace_bytes(int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, int out_bf16);
+int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                                float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
+                                int out_bf16, void* workspace, int64_t workspace_bytes);
 
 /* fp32 -> bf16 (round to nearest even) and back, on the device; used by the
  * WithTransfers dispatchers when a node's inputs arrive as fp32. */

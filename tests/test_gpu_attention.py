@@ -92,3 +92,59 @@ def test_attention_config_b8_h16_s2048(rt):
     vmin = V.float().amin(dim=2, keepdim=True).numpy()
     vmax = V.float().amax(dim=2, keepdim=True).numpy()
     assert (O >= vmin - 0.02).all() and (O <= vmax + 0.02).all()
+
+
+# ---- any head dimension, through docc_rocm_attention_bf16_ws ---------------------------------------
+
+def run_attention_ws(rt, Qb, Kb, Vb, scale=None, out_bf16=False, slack=0):
+    B, H, SQ, D = Qb.shape
+    SKV = Kb.shape[2]
+    scale = scale if scale is not None else 1.0 / np.sqrt(D)
+    q, k, v = dev(Qb), dev(Kb), dev(Vb)
+    o = torch.full((B, H, SQ, D), float("nan"), device="cuda", dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    need = rt.attention_bf16_workspace_bytes(B, H, SQ, SKV, D, out_bf16)
+    ws = torch.empty(max(need + slack, 256), dtype=torch.uint8, device="cuda")
+    assert ws.data_ptr() % 256 == 0
+    rt.attention_bf16_ws(B, H, SQ, SKV, D, scale, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr(), need,
+                         out_bf16=out_bf16)
+    torch.cuda.synchronize()
+    return o.float().cpu().numpy(), need
+
+
+@pytest.mark.parametrize("B,H,SQ,SKV,D", [(1, 2, 96, 96, 128), (2, 3, 128, 64, 32), (1, 2, 130, 200, 128), (1, 1, 33, 65, 80),
+                                          (1, 1, 1, 1, 8), (2, 2, 256, 512, 128), (1, 1, 7, 1000, 16), (1, 2, 50, 70, 7),
+                                          (1, 2, 96, 96, 64)])
+@pytest.mark.parametrize("out_bf16", [False, True])
+def test_attention_any_head_dimension_matches_oracle(rt, B, H, SQ, SKV, D, out_bf16):
+    g = torch.Generator().manual_seed(B * 7 + H * 5 + SQ * 3 + SKV + D)
+    Q, K, V = (torch.randn(B, H, s, D, generator=g).bfloat16() for s in (SQ, SKV, SKV))
+    O, need = run_attention_ws(rt, bits(Q), bits(K), bits(V), out_bf16=out_bf16)
+    assert (need == 0) == (D == 64)        # head dim 64 runs the fused kernel and needs no workspace
+    ref = oracle.attention(bits(Q), bits(K), bits(V))
+    assert np.isfinite(O).all()
+    assert rel_err_max(O, ref) <= TOL_BF16
+
+
+def test_attention_workspace_is_checked_and_chunked(rt):
+    from docc_amd.runtime import RocmRuntimeError
+    t = torch.zeros(1 << 16, dtype=torch.bfloat16, device="cuda")
+    p = t.data_ptr()
+    need = rt.attention_bf16_workspace_bytes(1, 1, 8, 8, 128)
+    assert need >= 8 * 8 * 6
+    with pytest.raises(RocmRuntimeError, match="workspace"):
+        rt.attention_bf16_ws(1, 1, 8, 8, 128, 0.1, p, p, p, p, 0, 0)
+    with pytest.raises(RocmRuntimeError, match="workspace"):
+        rt.attention_bf16_ws(1, 1, 8, 8, 128, 0.1, p, p, p, p, p, need - 1)
+    # more (batch, head) pairs than one 2 GiB chunk of scores holds: 40 x 4096 x 4096 x 6 B = 3.75 GiB
+    B, H, S, D = 1, 40, 4096, 32
+    need = rt.attention_bf16_workspace_bytes(B, H, S, S, D)
+    assert need <= 2 << 30 and need < H * S * S * 6
+    g = torch.Generator(device="cuda").manual_seed(9)
+    Q, K, V = (torch.randn(B, H, S, D, device="cuda", generator=g).bfloat16() for _ in range(3))
+    o = torch.empty(B, H, S, D, device="cuda")
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    rt.attention_bf16_ws(B, H, S, S, D, D ** -0.5, Q.data_ptr(), K.data_ptr(), V.data_ptr(), o.data_ptr(), ws.data_ptr(), need)
+    torch.cuda.synchronize()
+    for h in (0, 21, 39):       # heads of the first and of the second chunk
+        ref = oracle.attention(bits(Q[:, h:h + 1, :256].cpu()), bits(K[:, h:h + 1].cpu()), bits(V[:, h:h + 1].cpu()))
+        assert rel_err_max(o[:, h:h + 1, :256].cpu().numpy(), ref) <= TOL_BF16

@@ -376,3 +376,14 @@ def test_softmax_over_other_axes_and_fp64_through_both_front_ends():
     a = torch.randn(33, 70, dtype=torch.float64)
     out = docc_torch.compile_torch(S(), (a,), target="rocm")(a)
     assert rel_err_max(out.numpy(), oracle.softmax_axes(a.numpy(), (0,))) <= 1e-12
+
+
+def test_torch_attention_with_head_dimension_128():
+    """Another head dimension than 64: the node brings a workspace for its scores (GEMM, softmax, GEMM)."""
+    torch.manual_seed(5)
+    Q, K, V = (torch.randn(2, 3, 200, 128).bfloat16() for _ in range(3))
+    for dev_in in ("cuda", "cpu"):
+        program = docc_torch.compile_torch(Attn(), tuple(t.to(dev_in) for t in (Q, K, V)), target="rocm")
+        out = program(*(t.to(dev_in) for t in (Q, K, V)))
+        assert out.device.type == dev_in and out.dtype == torch.bfloat16 and out.shape == (2, 3, 200, 128)
+        assert rel_err_max(out.float().cpu().numpy(), oracle.attention(bits(Q), bits(K), bits(V))) <= 2e-2

@@ -110,10 +110,11 @@ def test_mapper_sets_implementation_types_and_declines_what_the_kernels_lack():
     with pytest.raises(InvalidSDFGException, match="group"):
         b.move().schedule("rocm")
     b = StructuredSDFGBuilder("a")
-    for n in ("Q", "K", "V", "O"):
-        b.add_container(n, BF16, True)
-    b.add_attention("Q", "K", "V", "O", [1, 2, 16, 128], 16, 0.1)
-    with pytest.raises(InvalidSDFGException, match="head dimension"):
+    for n in ("Q", "K", "V"):
+        b.add_container(n, F32, True)
+    b.add_container("O", F32, True)
+    b.add_attention("Q", "K", "V", "O", [1, 2, 16, 64], 16, 0.1)
+    with pytest.raises(InvalidSDFGException, match="BFloat"):
         b.move().schedule("rocm")
     with pytest.raises(NotImplementedError):
         gemm_sdfg().schedule("openmp")
@@ -177,6 +178,23 @@ def test_softmax_over_inner_axes_and_fp64(tmp_path):
         s.schedule("rocm", options={"offload": "none"})
         src, _ = source_of(s, tmp_path)
         assert text in src, (axes, src)
+
+
+def test_attention_with_another_head_dimension_brings_its_workspace(tmp_path):
+    for d, fused in ((64, True), (128, False)):
+        b = StructuredSDFGBuilder("att")
+        for n in ("Q", "K", "V", "O"):
+            b.add_container(n, BF16, True)
+        b.add_attention("Q", "K", "V", "O", [2, 4, 256, d], 192, 0.125)
+        s = b.move()
+        s.schedule("rocm", options={"offload": "none"})
+        src, _ = source_of(s, tmp_path)
+        if fused:
+            assert "docc_rocm_attention_bf16(nullptr, 2, 4, 256, 192, 64, (float) (0.125)," in src and "_ws" not in src
+        else:
+            assert "docc_rocm_attention_bf16_workspace_bytes(2, 4, 256, 192, 128, 1);" in src
+            assert "docc_rocm_attention_bf16_ws(nullptr, 2, 4, 256, 192, 128, (float) (0.125), (const uint16_t *) Q" in src
+            assert src.index("docc_rocm_malloc(&__ws") < src.index("docc_rocm_attention_bf16_ws(") < src.index("docc_rocm_free(__ws)")
 
 
 def test_matmul_node_is_one_batched_launch(tmp_path):
