@@ -267,6 +267,7 @@ DOCC_EW_BINARY(mul, kMul)
 DOCC_EW_BINARY(div, kDiv)
 DOCC_EW_BINARY(maximum, kMaximum)
 DOCC_EW_BINARY(minimum, kMinimum)
+DOCC_EW_BINARY(pow, kPow)
 
 #define DOCC_BROADCAST(NAME, T, VEC, I)                                                                                     \
     extern "C" __global__ __launch_bounds__(256) void docc_broadcast_##NAME(const T* X, T* Y, docc_k::BroadcastParams p) {     \

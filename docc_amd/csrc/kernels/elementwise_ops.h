@@ -5,6 +5,7 @@
 //   Maximum / Minimum  fmax / fmin   elementwise_ops/maximum_node.cpp:64, minimum_node.cpp
 //   Abs, Exp, Sqrt, Tanh, Erf        the libm function of the element type (cmath_node.h)
 //   Add, Sub, Mul, Div               the IEEE operation
+//   Pow      pow(a, b)               elementwise_ops/pow_node.cpp:52-54 (CMathFunction::pow)
 #pragma once
 
 #include "common.h"
@@ -12,7 +13,7 @@
 namespace docc_k {
 
 enum UnaryOp : int { kAbs = 0, kExp = 1, kReLU = 2, kSigmoid = 3, kSqrt = 4, kTanh = 5, kErf = 6 };
-enum BinaryOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMaximum = 4, kMinimum = 5 };
+enum BinaryOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMaximum = 4, kMinimum = 5, kPow = 6 };
 
 template <int OP>
 __device__ __forceinline__ float unary(float x) {
@@ -41,6 +42,7 @@ __device__ __forceinline__ float binary(float a, float b) {
     if (OP == kMul) return a * b;
     if (OP == kDiv) return a / b;
     if (OP == kMaximum) return fmaxf(a, b);
+    if (OP == kPow) return powf(a, b);
     return fminf(a, b);
 }
 template <int OP>
@@ -50,6 +52,7 @@ __device__ __forceinline__ double binary(double a, double b) {
     if (OP == kMul) return a * b;
     if (OP == kDiv) return a / b;
     if (OP == kMaximum) return fmax(a, b);
+    if (OP == kPow) return pow(a, b);
     return fmin(a, b);
 }
 
@@ -75,6 +78,7 @@ __device__ __forceinline__ T apply_binary(int op, T a, T b) {
         case kMul: return binary<kMul>(a, b);
         case kDiv: return binary<kDiv>(a, b);
         case kMaximum: return binary<kMaximum>(a, b);
+        case kPow: return binary<kPow>(a, b);
         default: return binary<kMinimum>(a, b);
     }
 }

@@ -10,7 +10,7 @@ using namespace docc::rt::rocm;
 namespace {
 
 const char* const kUnaryNames[] = {"abs", "exp", "relu", "sigmoid", "sqrt", "tanh", "erf"};
-const char* const kBinaryNames[] = {"add", "sub", "mul", "div", "maximum", "minimum"};
+const char* const kBinaryNames[] = {"add", "sub", "mul", "div", "maximum", "minimum", "pow"};
 
 // Work-groups for `items` lane-items, at most `per_cu` per compute unit (the kernels stride over the
 // rest). Measured on [8192, 4096] fp32: kernels that only move data are fastest with one vector per lane
@@ -110,7 +110,7 @@ extern "C" int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, i
     const long nvec = aligned ? (long) (n / per_vec) : 0;
     char name[64];
     std::snprintf(name, sizeof(name), "docc_ew_%s_f%d", kBinaryNames[op], precision);
-    return launch(name, grid_for(aligned ? (n + per_vec - 1) / per_vec : n, kGridStreaming), 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, (long) n,
+    return launch(name, grid_for(aligned ? (n + per_vec - 1) / per_vec : n, op == DOCC_ROCM_BINARY_POW ? kGridTranscendental : kGridStreaming), 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, (long) n,
                   nvec);
 }
 
@@ -128,7 +128,7 @@ extern "C" int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, in
     const long nvec = aligned ? (long) (n / per_vec) : 0;
     char name[64];
     std::snprintf(name, sizeof(name), "docc_ew_%s_%s_f%d", kBinaryNames[op], scalar_is_lhs ? "sl" : "sr", precision);
-    const uint32_t grid = grid_for(aligned ? (n + per_vec - 1) / per_vec : n, kGridStreaming);
+    const uint32_t grid = grid_for(aligned ? (n + per_vec - 1) / per_vec : n, op == DOCC_ROCM_BINARY_POW ? kGridTranscendental : kGridStreaming);
     if (precision == 32) return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, A, (float) scalar, Y, (long) n, nvec);
     return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, A, scalar, Y, (long) n, nvec);
 }

@@ -335,7 +335,7 @@ private:
 // reference: .../tensor/elementwise_node.cpp:20 (ElementWiseUnaryNode "X" -> "Y"), :176
 // (ElementWiseBinaryNode "A","B" -> "C"), JSON keys code + shape; elementwise_ops/*.h for the codes.
 inline const std::vector<std::string> UnaryNodeCodes = {"ml::Abs", "ml::Exp", "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf"};
-inline const std::vector<std::string> BinaryNodeCodes = {"ml::Add", "ml::Sub", "ml::Mul", "ml::Div", "ml::Maximum", "ml::Minimum"};
+inline const std::vector<std::string> BinaryNodeCodes = {"ml::Add", "ml::Sub", "ml::Mul", "ml::Div", "ml::Maximum", "ml::Minimum", "ml::Pow"};
 inline const std::string LibraryNodeType_Broadcast = "ml::Broadcast";
 
 class ElementWiseNode : public data_flow::LibraryNode {

@@ -20,7 +20,7 @@ NotImplementedError (there is no CPU lowering behind it):
     the decomposed form  m = np.max(x, axis=-1, keepdims=True); e = np.exp(x - m);
                          s = np.sum(e, axis=-1, keepdims=True); e / s
     conv2d(x, w, bias, stride=, padding=, dilation=)
-    x + y, x - y, x * y, x / y, np.maximum(x, y), np.minimum(x, y) on float arrays whose shapes
+    x + y, x - y, x * y, x / y, x ** y, np.maximum(x, y), np.minimum(x, y) on float arrays whose shapes
         broadcast by numpy's rules (the smaller operand goes through ml::Broadcast), or on an
         array and a scalar (literal or scalar argument)
     np.abs, np.exp, np.sqrt, np.tanh, scipy.special.erf / expit, relu(x), sigmoid(x),
@@ -420,6 +420,8 @@ class _Lowering(ast.NodeVisitor):
             if isinstance(e, _Lazy) and e.kind == "exp_sub" and isinstance(s, _Lazy) and s.kind == "sum_keep" and s.base.name == e.base.name:
                 return self.softmax(node, e.base, -1, dest)
             return self.elementwise(node, "div", e, s, dest)
+        if isinstance(node.op, ast.Pow):
+            return self.elementwise(node, "pow", self.ev(node.left), self.ev(node.right), dest)
         self.fail(node, f"operator {type(node.op).__name__}")
 
     def call(self, node: ast.Call, dest: Optional[str]) -> Any:
@@ -460,7 +462,7 @@ class _Lowering(ast.NodeVisitor):
                 if fn is f:
                     return self.unary(node, op, self.ev(node.args[0]), dest)
         binary_fns = {np.maximum: "max", np.minimum: "min", np.add: "add", np.subtract: "sub", np.multiply: "mul",
-                      np.divide: "div", np.true_divide: "div"}
+                      np.divide: "div", np.true_divide: "div", np.power: "pow"}
         if fn is not None and len(node.args) == 2 and not node.keywords:
             for f, op in binary_fns.items():
                 if fn is f:

@@ -262,7 +262,7 @@ def copy_bytes(nbytes, src, dst, stream=0) -> None:
 
 
 UNARY_OPS = {"abs": 0, "exp": 1, "relu": 2, "sigmoid": 3, "sqrt": 4, "tanh": 5, "erf": 6}
-BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5, "pow": 6}
 
 
 def elementwise_unary(op, precision, n, X, Y, stream=0) -> None:

@@ -373,11 +373,11 @@ class StructuredSDFGBuilder:
     UNARY_CODES = {"abs": "ml::Abs", "exp": "ml::Exp", "relu": "ml::ReLU", "sigmoid": "ml::Sigmoid", "sqrt": "ml::Sqrt",
                    "tanh": "ml::Tanh", "erf": "ml::Erf"}
     BINARY_CODES = {"add": "ml::Add", "sub": "ml::Sub", "mul": "ml::Mul", "div": "ml::Div", "max": "ml::Maximum",
-                    "min": "ml::Minimum", "maximum": "ml::Maximum", "minimum": "ml::Minimum"}
+                    "min": "ml::Minimum", "maximum": "ml::Maximum", "minimum": "ml::Minimum", "pow": "ml::Pow"}
 
     def add_elementwise_op(self, op: str, A: str, B: str, C: str, shape: Sequence[Any]) -> None:
         """Binary elementwise node "A","B" -> "C" over equally shaped operands (reference add_elementwise_op,
-        python/bindings/builder/py_structured_sdfg_builder.cpp:839-908: op names add, sub, mul, div, min, max).
+        python/bindings/builder/py_structured_sdfg_builder.cpp:839-908: op names add, sub, mul, div, pow, min, max).
         As there, an operand that names no container is bound as a constant of the result's element type;
         a scalar container is passed by value."""
         if op not in self.BINARY_CODES:

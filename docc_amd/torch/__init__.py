@@ -14,7 +14,7 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
                                            -> ml::Attention (bf16, head dim 64)
-    + - * / torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
+    + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
                                            -> ml::Add .. ml::Minimum, with ml::Broadcast where shapes differ
     relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh)
                                            -> ml::ReLU .. ml::Erf
@@ -428,6 +428,8 @@ class _FxLowering:
             if kwargs.get("alpha", 1) != 1:
                 self.fail(node, "sub with alpha")
             return self.elementwise(node, "sub", args[0], args[1], dest)
+        if t in (operator.pow, torch.pow) or method == "pow":
+            return self.elementwise(node, "pow", args[0], args[1], dest)
         if t in (torch.maximum, torch.minimum) or method in ("maximum", "minimum"):
             return self.elementwise(node, "max" if (t is torch.maximum or method == "maximum") else "min", args[0], args[1], dest)
         unary_fns = {"relu": (torch.relu, F.relu), "sigmoid": (torch.sigmoid, F.sigmoid), "tanh": (torch.tanh, F.tanh),

@@ -188,6 +188,7 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
 #define DOCC_ROCM_BINARY_DIV 3     /* ml::Div */
 #define DOCC_ROCM_BINARY_MAXIMUM 4 /* ml::Maximum  fmax (maximum_node.cpp:64) */
 #define DOCC_ROCM_BINARY_MINIMUM 5 /* ml::Minimum  fmin */
+#define DOCC_ROCM_BINARY_POW 6     /* ml::Pow      pow(a, b) (pow_node.cpp:52-54) */
 int docc_rocm_elementwise_unary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y);
 int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A, const void* B,
                                  void* Y);

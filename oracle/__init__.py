@@ -234,7 +234,7 @@ def attention(Q_bits, K_bits, V_bits, scale=None, lib=None) -> np.ndarray:
 
 
 UNARY_OPS = {"abs": 0, "exp": 1, "relu": 2, "sigmoid": 3, "sqrt": 4, "tanh": 5, "erf": 6}
-BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "maximum": 4, "minimum": 5, "pow": 6}
 
 
 def elementwise_unary(op: str, X, lib=None) -> np.ndarray:

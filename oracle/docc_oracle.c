@@ -460,6 +460,7 @@ ORACLE_API int oracle_attention_bf16(int64_t B, int64_t H, int64_t SQ, int64_t S
         case 2: y = a * b; break;                                                          \
         case 3: y = a / b; break;                                                          \
         case 4: y = fmax##SUF(a, b); break;                                                \
+        case 6: y = pow##SUF(a, b); break; /* pow_node.cpp:52-54: CMathFunction::pow */     \
         default: y = fmin##SUF(a, b); break;                                               \
     }
 
@@ -488,7 +489,7 @@ ORACLE_API int oracle_elementwise_unary_f64(int op, int64_t n, const double* X, 
 }
 
 ORACLE_API int oracle_elementwise_binary_f32(int op, int64_t n, const float* A, const float* B, float* Y) {
-    if (op < 0 || op > 5) return 1;
+    if (op < 0 || op > 6) return 1;
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; i++) {
         const float a = A[i], b = B[i];
@@ -500,7 +501,7 @@ ORACLE_API int oracle_elementwise_binary_f32(int op, int64_t n, const float* A, 
 }
 
 ORACLE_API int oracle_elementwise_binary_f64(int op, int64_t n, const double* A, const double* B, double* Y) {
-    if (op < 0 || op > 5) return 1;
+    if (op < 0 || op > 6) return 1;
 #pragma omp parallel for schedule(static)
     for (int64_t i = 0; i < n; i++) {
         const double a = A[i], b = B[i];

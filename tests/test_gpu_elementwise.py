@@ -64,6 +64,30 @@ def test_binary_bit_exact(rt, dt, n):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_pow_within_libm_accuracy(rt, dt):
+    """ml::Pow: the array, scalar-exponent (x ** 2, x ** 0.5) and scalar-base forms; exact on the IEEE special
+    cases, within 4 ulp of the oracle's libm elsewhere."""
+    rng = np.random.default_rng(12)
+    a = (np.abs(rng.standard_normal(5000)) * 3 + 0.05).astype(dt)
+    b = (rng.standard_normal(5000) * 3).astype(dt)
+    for offset in (0, 1):
+        assert ulps(run_binary(rt, "pow", a, b, offset), oracle.elementwise_binary("pow", a, b)) <= 4
+    base = np.array([2, 3, 0.5, -2, -2, 0, 7, np.inf, 1, -3, 0, -0.0], dt)
+    expo = np.array([10, 2, 2, 3, 0.5, 0, 0, -1, np.nan, 2, -1, -3], dt)
+    with np.errstate(all="ignore"):
+        assert np.array_equal(run_binary(rt, "pow", base, expo), oracle.elementwise_binary("pow", base, expo), equal_nan=True)
+    for scalar, lhs in ((2.0, False), (0.5, False), (3.0, False), (-1.0, False), (2.0, True), (10.0, True)):
+        x = (a if not lhs else b)
+        dx = dev(x)
+        out = torch.full_like(dx, float("nan"))
+        rt.elementwise_binary_scalar("pow", prec(dt), x.size, dx.data_ptr(), scalar, out.data_ptr(), lhs)
+        torch.cuda.synchronize()
+        full = np.full(x.size, scalar, dt)
+        ref = oracle.elementwise_binary("pow", full, x) if lhs else oracle.elementwise_binary("pow", x, full)
+        assert ulps(host(out), ref) <= 4, (scalar, lhs)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
 @pytest.mark.parametrize("n", SIZES)
 def test_unary(rt, dt, n):
     rng = np.random.default_rng(n + 7)

@@ -387,3 +387,25 @@ def test_torch_attention_with_head_dimension_128():
         out = program(*(t.to(dev_in) for t in (Q, K, V)))
         assert out.device.type == dev_in and out.dtype == torch.bfloat16 and out.shape == (2, 3, 200, 128)
         assert rel_err_max(out.float().cpu().numpy(), oracle.attention(bits(Q), bits(K), bits(V))) <= 2e-2
+
+
+def test_power_operator_through_both_front_ends():
+    """x ** 2, x ** y and np.power lower to ml::Pow (array or scalar operand); torch.pow likewise."""
+    @native(target="rocm")
+    def norms(x, y):
+        return np.sqrt(x ** 2 + np.power(y, 2.0)) ** (y / 4)
+
+    rng = np.random.default_rng(21)
+    x, y = rng.standard_normal((64, 50)), rng.standard_normal((64, 50))
+    got = norms(x, y)
+    ref = np.sqrt(x ** 2 + y ** 2) ** (y / 4)
+    np.testing.assert_allclose(got, ref, rtol=1e-13)
+    assert [n["code"] for n in norms.last_sdfg.library_nodes()].count("ml::Pow") == 3
+
+    class P(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.pow(a.abs(), b) + a ** 2
+
+    a, b = torch.randn(40, 30), torch.randn(40, 30)
+    out = docc_torch.compile_torch(P(), (a, b), target="rocm")(a, b)
+    np.testing.assert_allclose(out.numpy(), (a.abs() ** b + a ** 2).numpy(), rtol=2e-6)

@@ -214,6 +214,12 @@ def test_elementwise_binary_matches_ieee(dt):
         assert np.array_equal(oracle.elementwise_binary("div", a, b), a / b, equal_nan=True)
     assert np.array_equal(oracle.elementwise_binary("maximum", a, b), np.fmax(a, b), equal_nan=True)
     assert np.array_equal(oracle.elementwise_binary("minimum", a, b), np.fmin(a, b), equal_nan=True)
+    # pow: exact cases (order of the operands, the IEEE special values), and numpy's pow within 1 ulp elsewhere
+    base, expo = np.array([2, 3, 0.5, -2, -2, 0, 7, np.inf, 1], dt), np.array([10, 2, 2, 3, 0.5, 0, 0, -1, np.nan], dt)
+    with np.errstate(all="ignore"):
+        assert np.array_equal(oracle.elementwise_binary("pow", base, expo), np.array([1024, 9, 0.25, -8, np.nan, 1, 1, 0, 1], dt), equal_nan=True)
+        p, q = np.abs(a[:500]) + dt(0.1), b[:500] / dt(4)
+        assert ulp_diff(oracle.elementwise_binary("pow", p, q), np.power(p.astype(np.float64), q.astype(np.float64)).astype(dt)) <= 1
     # not commutative operations in the right order
     assert oracle.elementwise_binary("sub", np.array([5], dt), np.array([3], dt))[0] == 2
     assert oracle.elementwise_binary("div", np.array([6], dt), np.array([3], dt))[0] == 2
