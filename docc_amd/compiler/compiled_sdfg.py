@@ -91,7 +91,7 @@ class CompiledSDFG:
         for name in self.output_args:
             elem = PrimitiveType(self.sdfg.containers[name]["element"])
             shape = tuple(int(eval(e, {"__builtins__": {}}, syms)) for e in self.output_shapes[name])
-            buf = np.empty(shape, dtype=_NUMPY[elem])
+            buf = runtime.result_array(shape, _NUMPY[elem])
             outputs[name] = buf
             by_name[name] = buf.ctypes.data
         call_args = [syms[n] if n in syms else by_name[n] for n in self.arg_names]

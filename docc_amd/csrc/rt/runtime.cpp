@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <unordered_map>
 #include <vector>
@@ -51,6 +52,27 @@ struct DeviceState {
 
 std::mutex g_mutex;
 std::vector<DeviceState> g_devices;
+
+// Device blocks that docc_rocm_free keeps for the next docc_rocm_malloc of the same (rounded) size: generated
+// code allocates and frees the same buffers on every call of a compiled function, and hipMalloc / hipFree
+// cost more than a small kernel. Keyed by (device, bytes); `live` remembers the size of what is handed out.
+struct BlockCache {
+    std::mutex mutex;
+    std::multimap<std::pair<int, size_t>, void*> free_blocks;
+    std::unordered_map<void*, std::pair<int, size_t>> live;
+    size_t cached_bytes = 0;
+    size_t limit = 0;   // bytes the cache may hold; 0 switches it off
+};
+
+BlockCache& block_cache() {
+    static BlockCache* cache = [] {
+        auto* c = new BlockCache();   // never destroyed: blocks may be freed during process exit
+        c->limit = size_t(4) << 30;
+        if (const char* e = std::getenv("DOCC_ROCM_POOL_BYTES")) c->limit = (size_t) std::strtoull(e, nullptr, 10);
+        return c;
+    }();
+    return *cache;
+}
 
 std::mutex g_failure_mutex;
 int g_failure_code = 0;
@@ -223,12 +245,98 @@ int docc_rocm_malloc(void** dev_ptr, size_t bytes) {
     if (!dev_ptr) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "malloc: null argument");
     *dev_ptr = nullptr;
     if (bytes == 0) return 0;
-    return check(hipMalloc(dev_ptr, bytes), "hipMalloc");
+    BlockCache& c = block_cache();
+    if (c.limit == 0) return check(hipMalloc(dev_ptr, bytes), "hipMalloc");
+    const size_t rounded = (bytes + 255) & ~size_t(255);
+    int dev = 0;
+    int rc = check(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    {
+        std::lock_guard<std::mutex> lock(c.mutex);
+        auto it = c.free_blocks.find({dev, rounded});
+        if (it != c.free_blocks.end()) {
+            *dev_ptr = it->second;
+            c.cached_bytes -= rounded;
+            c.free_blocks.erase(it);
+            c.live[*dev_ptr] = {dev, rounded};
+            return 0;
+        }
+    }
+    hipError_t e = hipMalloc(dev_ptr, rounded);
+    if (e == hipErrorOutOfMemory) {   // give the cached blocks back and try once more
+        (void) hipGetLastError();
+        docc_rocm_pool_trim();
+        e = hipMalloc(dev_ptr, rounded);
+    }
+    rc = check(e, "hipMalloc");
+    if (rc) return rc;
+    std::lock_guard<std::mutex> lock(c.mutex);
+    c.live[*dev_ptr] = {dev, rounded};
+    return 0;
 }
 
 int docc_rocm_free(void* dev_ptr) {
     if (!dev_ptr) return 0;
-    return check(hipFree(dev_ptr), "hipFree");
+    BlockCache& c = block_cache();
+    std::pair<int, size_t> key{0, 0};
+    bool keep = false;
+    {
+        std::lock_guard<std::mutex> lock(c.mutex);
+        auto it = c.live.find(dev_ptr);
+        if (it != c.live.end()) {
+            key = it->second;
+            c.live.erase(it);
+            keep = c.limit > 0 && key.second <= c.limit - (c.cached_bytes < c.limit ? c.cached_bytes : c.limit);
+        }
+    }
+    if (!keep) return check(hipFree(dev_ptr), "hipFree");
+    // hipFree waits for the device before it releases memory; a block that stays allocated must do the same
+    // before another caller can get it
+    int rc = check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    if (rc) {
+        (void) hipFree(dev_ptr);
+        return rc;
+    }
+    std::lock_guard<std::mutex> lock(c.mutex);
+    c.free_blocks.insert({key, dev_ptr});
+    c.cached_bytes += key.second;
+    return 0;
+}
+
+int docc_rocm_pool_trim(void) {
+    BlockCache& c = block_cache();
+    std::multimap<std::pair<int, size_t>, void*> blocks;
+    {
+        std::lock_guard<std::mutex> lock(c.mutex);
+        blocks.swap(c.free_blocks);
+        c.cached_bytes = 0;
+    }
+    int rc = 0;
+    for (auto& b : blocks) {
+        const int r = check(hipFree(b.second), "hipFree");
+        if (r && !rc) rc = r;
+    }
+    return rc;
+}
+
+int docc_rocm_pool_stats(size_t* cached_bytes, size_t* cached_blocks, size_t* limit_bytes) {
+    BlockCache& c = block_cache();
+    std::lock_guard<std::mutex> lock(c.mutex);
+    if (cached_bytes) *cached_bytes = c.cached_bytes;
+    if (cached_blocks) *cached_blocks = c.free_blocks.size();
+    if (limit_bytes) *limit_bytes = c.limit;
+    return 0;
+}
+
+int docc_rocm_pool_set_limit(size_t limit_bytes) {
+    BlockCache& c = block_cache();
+    {
+        std::lock_guard<std::mutex> lock(c.mutex);
+        c.limit = limit_bytes;
+    }
+    size_t cached = 0;
+    docc_rocm_pool_stats(&cached, nullptr, nullptr);
+    return cached > limit_bytes ? docc_rocm_pool_trim() : 0;
 }
 
 int docc_rocm_memset_async(void* dev_ptr, int value, size_t bytes, docc_rocm_stream_t stream) {

@@ -507,7 +507,11 @@ class _CompiledTorch:
             t = t.contiguous()
             keep.append(t)
             ptrs.append(t.data_ptr())
-        outs = [torch.empty(shape, dtype=dtype, device=device) for _, shape, dtype in self.outputs]
+        # results for CPU callers of 1 MiB and more are pinned (torch caches such blocks): the device-to-host copy runs
+        # at link speed instead of through the driver's staging of pageable memory
+        pin = lambda shape, dtype: (not self.on_device and torch.cuda.is_available() and
+                                    math.prod(shape) * torch.empty((), dtype=dtype).element_size() >= (1 << 20))
+        outs = [torch.empty(shape, dtype=dtype, device=device, pin_memory=pin(shape, dtype)) for _, shape, dtype in self.outputs]
         if self.on_device:
             runtime.init(device.index or 0)
             current = torch.cuda.current_stream()

@@ -69,6 +69,14 @@ int docc_rocm_module_get_function(docc_rocm_module_t module, const char* name, d
  * (reference cuda_data_offloading_node.cpp:150-170). */
 int docc_rocm_malloc(void** dev_ptr, size_t bytes);
 int docc_rocm_free(void* dev_ptr);
+/* docc_rocm_free waits for the device (as hipFree does) and keeps the block for the next
+ * docc_rocm_malloc of the same size, rounded up to 256 bytes: a compiled function allocates the
+ * same buffers on every call. The cache holds at most DOCC_ROCM_POOL_BYTES bytes (default 4 GiB,
+ * 0 = every call goes to hipMalloc / hipFree) and is emptied when hipMalloc runs out of memory.
+ * No counterpart in the reference, whose CUDA nodes call cudaMalloc / cudaFree each time. */
+int docc_rocm_pool_trim(void);
+int docc_rocm_pool_stats(size_t* cached_bytes, size_t* cached_blocks, size_t* limit_bytes);
+int docc_rocm_pool_set_limit(size_t limit_bytes);
 int docc_rocm_memset_async(void* dev_ptr, int value, size_t bytes, docc_rocm_stream_t stream);
 
 /* Pinned host memory (hipHostMalloc) for callers that want truly

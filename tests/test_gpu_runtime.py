@@ -1,0 +1,99 @@
+"""The thin HIP runtime on a device: memory, copies and the device block cache behind
+docc_rocm_malloc / docc_rocm_free (include/docc_rocm_rt.h)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_copies_round_trip(rt):
+    x = np.arange(100000, dtype=np.float64)
+    y = np.zeros_like(x)
+    p = rt.malloc(x.nbytes)
+    rt.memcpy_h2d(p, x.ctypes.data, x.nbytes)
+    rt.memcpy_d2h(y.ctypes.data, p, x.nbytes)
+    rt.stream_sync()
+    rt.free(p)
+    assert np.array_equal(x, y)
+
+
+def test_free_keeps_blocks_for_the_next_malloc_of_that_size(rt):
+    rt.pool_trim()
+    _, _, limit = rt.pool_stats()
+    try:
+        rt.pool_set_limit(1 << 30)
+        a = rt.malloc(1000)               # rounded up to 1024
+        b = rt.malloc(5 << 20)
+        rt.free(a)
+        rt.free(b)
+        assert rt.pool_stats()[:2] == (1024 + (5 << 20), 2)
+        assert rt.malloc(1024) == a       # same rounded size: the cached block
+        assert rt.malloc(5 << 20) == b
+        c = rt.malloc(5 << 20)            # the cache is empty for this size: a new block
+        assert c not in (a, b) and rt.pool_stats()[:2] == (0, 0)
+        for p in (a, b, c):
+            rt.free(p)
+        assert rt.pool_stats()[1] == 3
+        # a block larger than what the cache may still hold goes back to the driver
+        rt.pool_set_limit(8 << 20)        # shrinking trims
+        assert rt.pool_stats()[:2] == (0, 0)
+        big = rt.malloc(16 << 20)
+        rt.free(big)
+        assert rt.pool_stats()[:2] == (0, 0)
+        # limit 0: no caching at all
+        rt.pool_set_limit(0)
+        p = rt.malloc(4096)
+        rt.free(p)
+        assert rt.pool_stats()[:2] == (0, 0)
+    finally:
+        rt.pool_set_limit(limit)
+
+
+def test_cached_blocks_hold_no_stale_work(rt):
+    """free() waits for the device before it keeps a block, so the next owner cannot race with a kernel of the last."""
+    import torch
+    n = 1 << 22
+    src = torch.arange(n, dtype=torch.float32, device="cuda")
+    p = rt.malloc(n * 4)
+    rt.elementwise_unary("abs", 32, n, src.data_ptr(), p)     # enqueued, not awaited
+    rt.free(p)
+    q = rt.malloc(n * 4)
+    assert q == p
+    out = np.empty(n, np.float32)
+    rt.memcpy_d2h(out.ctypes.data, q, n * 4)
+    rt.stream_sync()
+    rt.free(q)
+    assert np.array_equal(out, np.arange(n, dtype=np.float32))
+
+
+def test_result_arrays_are_pinned_and_reused(rt):
+    import gc
+    rt.pinned_trim()
+    small = rt.result_array((10, 10), np.float32)
+    assert small.base is None                                    # below 1 MiB: ordinary memory
+    a = rt.result_array((512, 1024), np.float64)                 # 4 MiB
+    assert a.shape == (512, 1024) and a.dtype == np.float64 and a.flags.c_contiguous and a.flags.writeable
+    a[:] = 3.0
+    addr = a.ctypes.data
+    # a device copy lands in it
+    p = rt.malloc(a.nbytes)
+    src = np.arange(a.size, dtype=np.float64).reshape(a.shape)
+    rt.memcpy_h2d(p, src.ctypes.data, a.nbytes)
+    rt.memcpy_d2h(a.ctypes.data, p, a.nbytes)
+    rt.stream_sync()
+    rt.free(p)
+    assert np.array_equal(a, src)
+    view = a[5:7]
+    del a
+    gc.collect()
+    b = rt.result_array((512, 1024), np.float64)
+    assert b.ctypes.data != addr                                  # a view still holds the first block
+    del view
+    gc.collect()
+    c = rt.result_array((1024, 512), np.float64)
+    assert c.ctypes.data == addr                                  # released with its last view, reused for the same size
+    del b, c
+    gc.collect()
+    rt.pinned_trim()
