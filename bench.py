@@ -309,6 +309,13 @@ def main():
                 "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
                 "roofline": {"bound": "hbm", "achieved": round(nbytes_r / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": round(nbytes_r / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_r}}
+        # ml::Transpose of the same tensor (64 x 64 tiles through LDS) and of a [64, 128, 64, 64] tensor with its two
+        # middle axes swapped (rows of 64 elements move as they are)
+        for name, shape, perm in (("transpose_f32_8192x4096", (8192, 4096), (1, 0)), ("transpose_f32_64x128x64x64_0213", (64, 128, 64, 64), (0, 2, 1, 3))):
+            ms = time_kernel(lambda i: rt.transpose(4, shape, perm, a.data_ptr(), y.data_ptr(), stream), 50, 5)
+            kernels[name] = {"kernel_us": round(ms * 1e3, 2), "dtype": "b32",
+                             "roofline": {"bound": "hbm", "achieved": round(8 * n / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                          "frac": round(8 * n / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": 8 * n}}
         if oracle_lib is not None:
             ah, bh = a.cpu().numpy(), b2.cpu().numpy()
             t = cpu_time(lambda: oracle.elementwise_binary("add", ah, bh, lib=oracle_lib))

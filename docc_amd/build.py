@@ -48,6 +48,7 @@ KERNEL_FAMILIES = {
     "attention": "attention.hip",
     "elementwise": "elementwise.hip",
     "reduce": "reduce.hip",
+    "transpose": "transpose.hip",
 }
 
 # Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary

@@ -41,6 +41,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_attention.hsaco",
     "docc_rocm_elementwise.hsaco",
     "docc_rocm_reduce.hsaco",
+    "docc_rocm_transpose.hsaco",
 };
 
 struct DeviceState {

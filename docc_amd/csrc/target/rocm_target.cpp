@@ -35,7 +35,7 @@ bool is_math_node(const LibraryNode& node) {
     const std::string& c = node.code();
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
            c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
-           is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
+           c == tensor::LibraryNodeType_Transpose || is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
 }
 
 // Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
@@ -442,6 +442,32 @@ protected:
     }
 };
 
+// ---- Transpose -----------------------------------------------------------------------------
+
+class TransposeNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::TransposeNode&>(node_);
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "const int64_t __docc_shape[] = {";
+        for (size_t i = 0; i < n.shape().size(); i++) s << (i ? ", " : "") << "(int64_t) (" << n.shape()[i] << ")";
+        s << "};" << std::endl;
+        s << "const int64_t __docc_perm[] = {";
+        for (size_t i = 0; i < n.perm().size(); i++) s << (i ? ", " : "") << n.perm()[i];
+        s << "};" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_transpose(nullptr, " << types::primitive_type_size(n.element()) << ", " << n.shape().size()
+          << ", __docc_shape, __docc_perm, " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+};
+
 // ---- Reduce --------------------------------------------------------------------------------
 
 class ReduceNodeDispatcher_ROCM : public RocmMathDispatcher {
@@ -552,6 +578,7 @@ void register_plugin(plugins::Context& context) {
     for (auto& code : tensor::UnaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
+    register_math<TransposeNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Transpose);
     for (auto& code : tensor::ReduceNodeCodes) register_math<ReduceNodeDispatcher_ROCM>(reg, code);
     register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
     reg.register_library_node_dispatcher(
@@ -621,6 +648,12 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!b) return decline("not a Broadcast node object");
         if (b->element() != P::Float && b->element() != P::Double) return decline("element type must be Float or Double");
         if (b->output_shape().size() > 6) return decline("rank above 6 is not supported");
+    } else if (node.code() == tensor::LibraryNodeType_Transpose) {
+        auto* t = dynamic_cast<tensor::TransposeNode*>(&node);
+        if (!t) return decline("not a Transpose node object");
+        const size_t bytes = types::primitive_type_size(t->element());
+        if (bytes != 1 && bytes != 2 && bytes != 4 && bytes != 8) return decline("element size must be 1, 2, 4 or 8 bytes");
+        if (t->shape().size() > 6 || t->shape().empty()) return decline("rank must be 1..6");
     } else {
         return false;  // not a node of this target
     }

@@ -583,6 +583,42 @@ Expression BroadcastNode::connector_bytes(const std::string& connector) const {
     return bytes_of(product(shape, 0, shape.size()), element_);
 }
 
+TransposeNode::TransposeNode(std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> perm,
+                             types::PrimitiveType element)
+    : LibraryNode(LibraryNodeType_Transpose, {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)),
+      perm_(std::move(perm)), element_(element) {
+    if (perm_.empty())   // default permutation: reverse (transpose_node.cpp:27-31)
+        for (size_t i = 0; i < shape_.size(); i++) perm_.push_back((int64_t) (shape_.size() - 1 - i));
+}
+
+void TransposeNode::validate() const {
+    if (perm_.size() != shape_.size()) throw InvalidSDFGException("Permutation rank must match shape rank");
+    std::vector<bool> seen(shape_.size(), false);
+    for (auto p : perm_) {
+        if (p < 0 || p >= (int64_t) shape_.size() || seen[(size_t) p]) throw InvalidSDFGException("Transpose: perm is not a permutation of the axes");
+        seen[(size_t) p] = true;
+    }
+}
+
+void TransposeNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    Array pm;
+    for (auto p : perm_) pm.emplace_back(p);
+    j.set("perm", Value(std::move(pm)));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<TransposeNode> TransposeNode::from_json(const Value& j) {
+    std::vector<int64_t> perm;
+    if (const Value* pm = j.find("perm"))
+        for (auto& p : pm->as_array()) perm.push_back(p.as_int());
+    const Value* et = j.find("element_type");
+    return std::make_unique<TransposeNode>(impl_of(j), exprs_from_json(j.at("shape")), std::move(perm),
+                                           et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression TransposeNode::connector_bytes(const std::string&) const { return bytes_of(product(shape_, 0, shape_.size()), element_); }
+
 } // namespace math::tensor
 
 // ------------------------------------------------------------- offloading
@@ -970,6 +1006,7 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     for (auto& code : math::tensor::UnaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     for (auto& code : math::tensor::BinaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
+    fns_[math::tensor::LibraryNodeType_Transpose] = &deserialize<math::tensor::TransposeNode>;
     for (auto& code : math::tensor::ReduceNodeCodes) fns_[code] = &deserialize<math::tensor::ReduceNode>;
     fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
 }

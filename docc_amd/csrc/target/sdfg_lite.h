@@ -337,6 +337,7 @@ private:
 inline const std::vector<std::string> UnaryNodeCodes = {"ml::Abs", "ml::Exp", "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf"};
 inline const std::vector<std::string> BinaryNodeCodes = {"ml::Add", "ml::Sub", "ml::Mul", "ml::Div", "ml::Maximum", "ml::Minimum", "ml::Pow"};
 inline const std::string LibraryNodeType_Broadcast = "ml::Broadcast";
+inline const std::string LibraryNodeType_Transpose = "ml::Transpose";
 
 class ElementWiseNode : public data_flow::LibraryNode {
 public:
@@ -375,6 +376,26 @@ public:
 
 private:
     std::vector<Expression> input_shape_, output_shape_;
+    types::PrimitiveType element_;
+};
+
+// reference: .../tensor/transpose_node.h:14-60 (connectors "X" -> "Y", JSON keys "shape" and "perm";
+// an empty permutation reverses the axes, transpose_node.cpp:27-31)
+class TransposeNode : public data_flow::LibraryNode {
+public:
+    TransposeNode(std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> perm, types::PrimitiveType element);
+    const std::vector<Expression>& shape() const { return shape_; }   // of the input
+    const std::vector<int64_t>& perm() const { return perm_; }        // output axis i is input axis perm[i]
+    types::PrimitiveType element() const { return element_; }
+
+    void validate() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<TransposeNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    std::vector<int64_t> perm_;
     types::PrimitiveType element_;
 };
 

@@ -271,11 +271,13 @@ class _Lowering(ast.NodeVisitor):
     def array_of(self, node: ast.AST, v: Any, dest: Optional[str] = None) -> Any:
         """A pattern piece that turns out to be used on its own becomes the node(s) it stands for;
         other values pass through."""
-        if not isinstance(v, _Lazy) or v.kind == "transposed":
+        if not isinstance(v, _Lazy):
             return v
         if v.array is not None:
             return v.array
-        if v.kind == "scaled":
+        if v.kind == "transposed":   # of a matrix, and not an operand of a product: the ml::Transpose node
+            arr = self.transpose(node, v.base, None, dest)
+        elif v.kind == "scaled":
             arr = self.elementwise(node, "mul", v.base, v.scalar, dest)
         elif v.kind == "max_keep":
             arr = self.reduce(node, "max", v.base, -1, True, dest)
@@ -289,6 +291,21 @@ class _Lowering(ast.NodeVisitor):
             return v
         v.array = arr
         return arr
+
+    def transpose(self, node: ast.AST, x: Any, axes: Any, dest: Optional[str]) -> _Array:
+        """np.transpose(x, axes): ml::Transpose; `axes` None reverses the axes."""
+        x = self.array_of(node, x)
+        if not isinstance(x, _Array) or x.elem not in _SIZES:
+            self.fail(node, "transposing a value that is not a float array")
+        rank = len(x.shape)
+        perm = list(range(rank))[::-1] if axes is None else [int(a) % rank for a in axes]
+        if sorted(perm) != list(range(rank)):
+            raise ValueError(f"{self.func.__name__}: axes don't match array")
+        if rank > 6:
+            raise NotImplementedError(f"{self.func.__name__}: transpose of rank {rank} (up to 6 are built)")
+        out = self.new_array([x.shape[p] for p in perm], x.elem, dest)
+        self.b.add_transpose(x.name, out.name, x.shape, perm)
+        return out
 
     def reduce(self, node: ast.AST, op: str, x: Any, axis: Any, keepdims: bool, dest: Optional[str]) -> _Array:
         x = self.array_of(node, x)
@@ -382,8 +399,11 @@ class _Lowering(ast.NodeVisitor):
         if isinstance(node, ast.Attribute) and node.attr in ("T", "mT"):
             base = self.ev(node.value)
             if isinstance(base, _Array) and len(base.shape) == 2:
-                return _Lazy("transposed", base)
-            self.fail(node, "transposing this value")
+                return _Lazy("transposed", base)   # a GEMM flag when it feeds a product, else a node
+            if node.attr == "mT":
+                rank = len(base.shape) if isinstance(base, _Array) else 0
+                return self.transpose(node, base, list(range(rank - 2)) + [rank - 1, rank - 2] if rank >= 2 else None, dest)
+            return self.transpose(node, base, None, dest)
         if isinstance(node, ast.BinOp):
             return self.binop(node, dest)
         if isinstance(node, ast.Call):
@@ -430,10 +450,26 @@ class _Lowering(ast.NodeVisitor):
             return self.matmul(node, self.ev(node.func.value), self.ev(node.args[0]), dest)
         if fn in (np.matmul, np.dot):
             return self.matmul(node, self.ev(node.args[0]), self.ev(node.args[1]), dest)
-        if fn is np.transpose and len(node.args) == 1:
-            base = self.ev(node.args[0])
-            if isinstance(base, _Array) and len(base.shape) == 2:
+        if fn is np.transpose or (fn is None and isinstance(node.func, ast.Attribute) and node.func.attr == "transpose"):
+            method = fn is None
+            base = self.ev(node.func.value if method else node.args[0])
+            rest = node.args if method else node.args[1:]
+            axes = self.kw(node, "axes", None, None)
+            if rest:
+                axes = [ast.literal_eval(a) for a in rest] if len(rest) > 1 else ast.literal_eval(rest[0])
+                if isinstance(axes, int):
+                    axes = [axes]
+            if axes is None and isinstance(base, _Array) and len(base.shape) == 2:
                 return _Lazy("transposed", base)
+            return self.transpose(node, base, axes, dest)
+        if fn is np.swapaxes and len(node.args) == 3:
+            base = self.array_of(node, self.ev(node.args[0]))
+            if not isinstance(base, _Array):
+                self.fail(node, "swapaxes of a value that is not an array")
+            perm = list(range(len(base.shape)))
+            i, j = (ast.literal_eval(a) % len(perm) for a in node.args[1:])
+            perm[i], perm[j] = perm[j], perm[i]
+            return self.transpose(node, base, perm, dest)
         try:
             import scipy.special as _sp
             scipy_softmax = _sp.softmax
@@ -532,6 +568,10 @@ class _Lowering(ast.NodeVisitor):
             name = f"_docc_ret_{len(self.outputs)}"
             before = len(self.b._data["root"]["children"])
             result = self.array_of(node, self.ev(v, name), name)
+            if isinstance(result, _Array) and result.name != name and result.elem in _SIZES and 1 <= len(result.shape) <= 6:
+                # a value that already has a home (a variable, an argument): the copy into the return buffer that the
+                # reference's front end emits as a loop (ast_parser.py:1186-1210) is a Transpose with the identity order
+                result = self.transpose(node, result, list(range(len(result.shape))), name)
             if not isinstance(result, _Array) or result.name != name or len(self.b._data["root"]["children"]) == before:
                 self.fail(node, "returning a value that is not produced by a library node")
             self.outputs.append(name)

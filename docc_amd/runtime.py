@@ -84,6 +84,7 @@ _SIGNATURES = {
     "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
     "docc_rocm_elementwise_binary_scalar": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, ctypes.c_double, ctypes.c_int, _vp],
     "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
+    "docc_rocm_transpose": [_vp, _int, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp, _vp],
     "docc_rocm_reduce": [_vp, ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_elementwise_fused": [_vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_double, _vp, _vp,
                                     ctypes.c_double, ctypes.c_int, _vp, _vp],
@@ -336,6 +337,12 @@ def elementwise_fused(precision, shape, binary, a, a_shape, b, b_shape, post, Y,
     call("docc_rocm_elementwise_fused", stream, precision, rank, ctypes.addressof(dims), code,
          ctypes.addressof(a_arr) if a_arr is not None else None, a_ptr, a_val,
          ctypes.addressof(b_arr) if b_arr is not None else None, b_ptr, b_val, len(post), ctypes.addressof(ops), Y)
+
+
+def transpose(element_bytes, shape, perm, X, Y, stream=0) -> None:
+    """Y = X with its axes permuted: Y.shape[i] = shape[perm[i]]."""
+    rank = len(shape)
+    call("docc_rocm_transpose", stream, element_bytes, rank, (_i64 * max(rank, 1))(*shape), (_i64 * max(rank, 1))(*perm), X, Y)
 
 
 def mfma_probe(precision, waves_per_simd, iters, operands, sink, stream=0) -> float:

@@ -408,6 +408,16 @@ class StructuredSDFGBuilder:
                          "element_type": self._element(X).value},
                         [self._operand("X", X)], [self._operand("Y", Y)])
 
+    def add_transpose(self, X: str, Y: str, shape: Sequence[Any], perm: Optional[Sequence[int]] = None) -> None:
+        """ml::Transpose (reference .../tensor/transpose_node.h): Y.shape[i] = shape[perm[i]]; no perm reverses the axes."""
+        rank = len(shape)
+        perm = [int(p) % rank if rank else int(p) for p in perm] if perm is not None else list(range(rank))[::-1]
+        if sorted(perm) != list(range(rank)):
+            raise InvalidSDFGException("ml::Transpose: perm is not a permutation of the axes")
+        self._add_block({"code": "ml::Transpose", "implementation_type": "NONE", "side_effect": False,
+                         "shape": [_expr(s) for s in shape], "perm": perm, "element_type": self._element(X).value},
+                        [self._operand("X", X)], [self._operand("Y", Y)])
+
     def add_attention(self, Q: str, K: str, V: str, O: str, shape_q: Sequence[Any], seq_kv: Any, scale: Any) -> None:
         """ml::Attention: O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]."""
         self._add_block({"code": "ml::Attention", "implementation_type": "NONE", "side_effect": False,

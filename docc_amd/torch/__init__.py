@@ -192,6 +192,7 @@ class _FxLowering:
             if dim not in (-1, len(x.q.shape) - 1):
                 self.fail(node, "softmax of attention scores over an axis other than the last")
             return _Probs(x)
+        x = self.tensor(node, x)
         if not isinstance(x, _T):
             self.fail(node, "softmax of this value")
         if not -len(x.shape) <= dim < len(x.shape):
@@ -236,6 +237,7 @@ class _FxLowering:
 
     def elementwise(self, node, op: str, a, b, dest):
         torch = self.torch
+        a, b = self.tensor(node, a), self.tensor(node, b)
         tensors = [v for v in (a, b) if isinstance(v, _T)]
         if not tensors or not all(isinstance(v, (_T, int, float)) and not isinstance(v, bool) for v in (a, b)):
             self.fail(node, f"elementwise {op} of these operands")
@@ -256,6 +258,7 @@ class _FxLowering:
         return out
 
     def unary(self, node, op: str, x, dest):
+        x = self.tensor(node, x)
         if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
         out = self.new_tensor(x.shape, x.dtype, dest)
@@ -263,6 +266,7 @@ class _FxLowering:
         return out
 
     def reduce(self, node, op: str, x, dim, keepdim: bool, dest):
+        x = self.tensor(node, x)
         if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
         rank = len(x.shape)
@@ -290,13 +294,38 @@ class _FxLowering:
             return out
         return self.elementwise(node, "add", out, bias, dest)
 
-    def transpose(self, node, x, d0: int, d1: int):
+    def transpose(self, node, x, d0: int, d1: int, dest=None):
+        x = self.tensor(node, x)
         if not isinstance(x, _T):
             self.fail(node, "transposing this value")
         rank = len(x.shape)
-        if {d0 % rank, d1 % rank} != {rank - 2, rank - 1}:
-            self.fail(node, "a transpose other than of the last two dimensions")
-        return _Transposed(x)
+        if {d0 % rank, d1 % rank} == {rank - 2, rank - 1} and dest is None:
+            return _Transposed(x)   # a GEMM flag when it feeds a product; ml::Transpose when used as a tensor
+        dims = list(range(rank))
+        dims[d0 % rank], dims[d1 % rank] = dims[d1 % rank], dims[d0 % rank]
+        return self.permute(node, x, dims, dest)
+
+    def permute(self, node, x, dims, dest=None):
+        """ml::Transpose: the result is a contiguous tensor with the permuted shape."""
+        x = self.tensor(node, x)
+        if not isinstance(x, _T):
+            self.fail(node, "permuting this value")
+        rank = len(x.shape)
+        dims = [int(d) % rank for d in dims]
+        if sorted(dims) != list(range(rank)):
+            self.fail(node, "a permutation that does not name every dim once")
+        if rank > 6:
+            self.fail(node, "a permutation of rank above 6")
+        out = self.new_tensor([x.shape[d] for d in dims], x.dtype, dest)
+        self.builder.add_transpose(x.name, out.name, x.shape, dims)
+        return out
+
+    def tensor(self, node, v, dest=None):
+        """A transposed view that is used as a tensor of its own (not as an operand of a product) is materialised."""
+        if isinstance(v, _Transposed):
+            rank = len(v.base.shape)
+            return self.permute(node, v.base, list(range(rank - 2)) + [rank - 1, rank - 2], dest)
+        return v
 
     # ---- graph walk -------------------------------------------------------------------------
     def arg(self, a):
@@ -359,6 +388,12 @@ class _FxLowering:
             elif node.op == "output":
                 for i, n in enumerate(out_list):
                     v = self.env[n]
+                    if isinstance(v, _Transposed):
+                        v = self.tensor(n, v, f"_docc_ret_{i}")
+                    elif isinstance(v, _T) and v.name != f"_docc_ret_{i}" and 1 <= len(v.shape) <= 6:
+                        # a value that lives elsewhere (an input, the operand of a view): copied into the result
+                        # by a Transpose with the identity order
+                        v = self.permute(n, v, list(range(len(v.shape))), f"_docc_ret_{i}")
                     if not isinstance(v, _T) or v.name != f"_docc_ret_{i}":
                         self.fail(n, "returning a value that no library node produces (inputs, views, partial patterns)")
                     self.outputs.append((v.name, v.shape, v.dtype))
@@ -396,19 +431,19 @@ class _FxLowering:
         if t in (torch.matmul, operator.matmul, torch.mm, torch.bmm) or method in ("matmul", "mm", "bmm"):
             return self.matmul(node, args[0], args[1], dest)
         if t is torch.transpose or method == "transpose":
-            return self.transpose(node, args[0], args[1], args[2])
+            return self.transpose(node, args[0], args[1], args[2], dest)
         if method == "permute" or t is torch.permute:
             dims = list(args[1]) if isinstance(args[1], (tuple, list)) else list(args[1:])
             rank = len(dims)
-            if dims[:-2] == list(range(rank - 2)) and dims[-2:] == [rank - 1, rank - 2]:
-                return self.transpose(node, args[0], -2, -1)
-            self.fail(node, "this permutation")
+            if rank >= 2 and dims[:-2] == list(range(rank - 2)) and dims[-2:] == [rank - 1, rank - 2]:
+                return self.transpose(node, args[0], -2, -1, dest)
+            return self.permute(node, args[0], dims, dest)
         if t is getattr and args[1] in ("mT", "T"):
             if args[1] == "T" and isinstance(args[0], _T) and len(args[0].shape) != 2:
                 self.fail(node, ".T on a tensor that is not 2-d")
-            return self.transpose(node, args[0], -2, -1)
+            return self.transpose(node, args[0], -2, -1, dest)
         if method in ("t",) or t is torch.t:
-            return self.transpose(node, args[0], 0, 1)
+            return self.transpose(node, args[0], 0, 1, dest)
         if t in (operator.truediv, torch.div, torch.true_divide) or method in ("div", "true_divide"):
             if kwargs.get("rounding_mode") is not None:
                 self.fail(node, "division with a rounding mode")
@@ -473,7 +508,7 @@ class _FxLowering:
             scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
             return self.attention(node, q, bound["key"], bound["value"], float(scale), dest)
         if method == "contiguous" or t is torch.Tensor.contiguous:
-            return args[0]
+            return self.tensor(node, args[0], dest)   # a transposed view becomes the tensor it stands for
         self.fail(node, "this operation")
 
 

@@ -205,6 +205,15 @@ int docc_rocm_elementwise_binary_scalar(docc_rocm_stream_t stream, int op, int p
 int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, const int64_t* in_shape, const int64_t* out_shape,
                         const void* X, void* Y);
 
+/*
+ * ml::Transpose: Y = X with its axes permuted, Y.shape[i] = shape[perm[i]] (the ONNX meaning the
+ * reference's node has: transpose_node.h:14-60, JSON keys "shape" and "perm"); both contiguous,
+ * rank <= 6, elements of 1, 2, 4 or 8 bytes (the node moves bits, integer types included), X and Y
+ * distinct. Replaces the loop nest of TransposeNode::expand (transpose_node.cpp).
+ */
+int docc_rocm_transpose(docc_rocm_stream_t stream, int element_bytes, int rank, const int64_t* shape, const int64_t* perm,
+                        const void* X, void* Y);
+
 /* Reduce tensor nodes ml::Sum / ml::Max / ml::Min / ml::Mean over a block of adjacent axes
  * (reference sdfg/include/sdfg/data_flow/library_nodes/math/tensor/reduce_node.h and
  * reduce_ops/{sum,max,min,mean}_node.h; replaces the loop nests ReduceNode::expand emits,

@@ -64,6 +64,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.oracle_elementwise_binary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p, _f32p]
     lib.oracle_elementwise_binary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p, _f64p]
     lib.oracle_broadcast.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), ctypes.c_void_p, ctypes.c_void_p]
+    lib.oracle_transpose.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), ctypes.c_void_p, ctypes.c_void_p]
     lib.oracle_reduce_f32.argtypes = [ctypes.c_int, _i64, _i64, _i64, _f32p, _f32p]
     lib.oracle_reduce_f64.argtypes = [ctypes.c_int, _i64, _i64, _i64, _f64p, _f64p]
     return lib
@@ -303,3 +304,17 @@ def reduce(op: str, X, axes, keepdims: bool = False, lib=None) -> np.ndarray:
         raise ValueError(f"reduce '{op}' over an extent of {extent}")
     kept = [1 if d in axes else s for d, s in enumerate(X.shape)] if keepdims else [s for d, s in enumerate(X.shape) if d not in axes]
     return out.reshape(kept)
+
+
+def transpose(X, perm=None, lib=None) -> np.ndarray:
+    """X with its axes permuted, out.shape[i] = X.shape[perm[i]] (reversed axes when perm is None), any dtype."""
+    lib = lib or load()
+    X = np.ascontiguousarray(X)
+    perm = list(range(X.ndim))[::-1] if perm is None else [int(p) % X.ndim for p in perm]
+    out = np.empty([X.shape[p] for p in perm], X.dtype)
+    rank = X.ndim
+    shape = (_i64 * max(rank, 1))(*X.shape)
+    pm = (_i64 * max(rank, 1))(*perm)
+    if lib.oracle_transpose(X.dtype.itemsize, rank, shape, pm, X.ctypes.data, out.ctypes.data) != 0:
+        raise ValueError("invalid permutation or rank above 8")
+    return out

@@ -563,3 +563,44 @@ ORACLE_API int oracle_broadcast(int esize, int rank, const int64_t* in_shape, co
     }
 ORACLE_REDUCE(oracle_reduce_f32, float, fmaxf, fminf, -INFINITY, INFINITY)
 ORACLE_REDUCE(oracle_reduce_f64, double, fmax, fmin, -INFINITY, INFINITY)
+
+
+/* ------------------------------------------------------------- Transpose */
+
+/*
+ * TransposeNode::expand (sdfg/src/data_flow/library_nodes/math/tensor/transpose_node.cpp:97-176):
+ * one Map per input axis around an assign tasklet, Y[i_perm[0], i_perm[1], ...] = X[i_0, i_1, ...]
+ * with Y's shape[i] = shape[perm[i]]. The node moves elements of any type (integers included,
+ * transpose_node.h:47), hence bytes here. Returns 0, or 1 for a rank above 8 or an invalid perm.
+ */
+ORACLE_API int oracle_transpose(int element_bytes, int rank, const int64_t* shape, const int64_t* perm, const void* X, void* Y) {
+    if (rank < 0 || rank > 8 || element_bytes <= 0) return 1;
+    int64_t out_shape[8], out_stride[8], n = 1;
+    int seen[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = 0; i < rank; i++) {
+        if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) return 1;
+        seen[perm[i]] = 1;
+        out_shape[i] = shape[perm[i]];
+        n *= shape[i];
+    }
+    int64_t s = 1;
+    for (int i = rank - 1; i >= 0; i--) {
+        out_stride[i] = s;
+        s *= out_shape[i];
+    }
+    /* stride in Y of a step along input axis a: a sits at output position p with perm[p] == a */
+    int64_t y_stride_of_input_axis[8];
+    for (int p = 0; p < rank; p++) y_stride_of_input_axis[perm[p]] = out_stride[p];
+    const char* x = (const char*) X;
+    char* y = (char*) Y;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        int64_t rem = i, off = 0;
+        for (int a = rank - 1; a >= 0; a--) {
+            off += (rem % shape[a]) * y_stride_of_input_axis[a];
+            rem /= shape[a];
+        }
+        memcpy(y + off * element_bytes, x + i * element_bytes, (size_t) element_bytes);
+    }
+    return 0;
+}

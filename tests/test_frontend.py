@@ -407,3 +407,43 @@ def test_reductions_and_softmax_pieces_used_on_their_own():
 
 def _bad_axis(x):
     return np.sum(x, axis=5)
+
+
+def test_transposes_lower_to_a_gemm_flag_or_a_transpose_node():
+    @native
+    def gram(a):
+        return a.T @ a                        # operand of a product: the flag of the GEMM, no node
+
+    @native
+    def flipped(a, b):
+        return a.T + b                        # used as an array: ml::Transpose
+
+    @native
+    def permuted(x):
+        return np.transpose(x, (2, 0, 1)) * 2.0
+
+    @native
+    def reversed_axes(x):
+        return np.exp(x.T)                    # rank 3: axes reversed
+
+    @native
+    def swapped(x):
+        return np.swapaxes(x, 0, 1)
+
+    a = np.zeros((6, 4))
+    g = gram.to_sdfg(a).library_nodes()
+    assert [n["code"] for n in g] == ["GEMM"] and g[0]["trans_a"] == 112 and g[0]["trans_b"] == 111
+    f = flipped.to_sdfg(a, np.zeros((4, 6))).library_nodes()
+    assert [n["code"] for n in f] == ["ml::Transpose", "ml::Add"] and f[0]["perm"] == [1, 0]
+    x = np.zeros((3, 4, 5), np.float32)
+    p = permuted.to_sdfg(x).library_nodes()
+    assert [n["code"] for n in p] == ["ml::Transpose", "ml::Mul"] and p[0]["perm"] == [2, 0, 1]
+    assert reversed_axes.to_sdfg(x).library_nodes()[0]["perm"] == [2, 1, 0]
+    s = swapped.to_sdfg(x)
+    assert s.library_nodes()[0]["perm"] == [1, 0, 2]
+    @native
+    def repeated_axis(x):
+        return np.transpose(x, (0, 0, 1))
+
+    with pytest.raises(ValueError, match="axes"):
+        repeated_axis.to_sdfg(x)

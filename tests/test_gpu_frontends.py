@@ -409,3 +409,25 @@ def test_power_operator_through_both_front_ends():
     a, b = torch.randn(40, 30), torch.randn(40, 30)
     out = docc_torch.compile_torch(P(), (a, b), target="rocm")(a, b)
     np.testing.assert_allclose(out.numpy(), (a.abs() ** b + a ** 2).numpy(), rtol=2e-6)
+
+
+def test_transposes_through_both_front_ends():
+    @native(target="rocm")
+    def mix(a, b, x):
+        g = a.T @ a                                  # GEMM flag
+        return np.transpose(x, (2, 0, 1)) * 2.0, a.T + b, g
+
+    rng = np.random.default_rng(31)
+    a, b, x = rng.standard_normal((60, 40)), rng.standard_normal((40, 60)), rng.standard_normal((5, 6, 7))
+    p, s, g = mix(a, b, x)
+    assert np.array_equal(p, np.transpose(x, (2, 0, 1)) * 2.0) and np.array_equal(s, a.T + b)
+    assert rel_err_max(g, oracle.gemm(np.ascontiguousarray(a.T), a, variant="ld")) <= 1e-12
+
+    class P(torch.nn.Module):
+        def forward(self, t, u):
+            return (t.permute(0, 2, 1, 3) + 1.0, torch.relu(u.transpose(0, 1)), t.transpose(1, 2).contiguous())
+
+    t, u = torch.randn(2, 3, 4, 5), torch.randn(30, 20, dtype=torch.float64)
+    o1, o2, o3 = docc_torch.compile_torch(P(), (t, u), target="rocm")(t, u)
+    assert torch.equal(o1, t.permute(0, 2, 1, 3) + 1.0) and torch.equal(o2, torch.relu(u.transpose(0, 1)))
+    assert torch.equal(o3, t.transpose(1, 2).contiguous())

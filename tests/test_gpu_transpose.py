@@ -1,0 +1,78 @@
+"""ml::Transpose on the GPU against the CPU oracle, through docc_rocm_transpose. The node moves bits:
+bit-exact for every element size (1, 2, 4, 8 bytes), rank up to six."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from gpu_util import dev, host
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = {1: np.uint8, 2: np.int16, 4: np.float32, 8: np.float64}
+
+
+def run_transpose(rt, X, perm):
+    x = dev(X)
+    out_shape = [X.shape[p] for p in perm]
+    y = torch.full(out_shape, 7, dtype=x.dtype, device="cuda") if X.size else torch.empty(out_shape, dtype=x.dtype, device="cuda")
+    rt.transpose(X.dtype.itemsize, X.shape, perm, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    return host(y)
+
+
+def values(shape, dt, seed):
+    rng = np.random.default_rng(seed)
+    n = int(np.prod(shape, dtype=np.int64))
+    if np.issubdtype(dt, np.floating):
+        return rng.standard_normal(n).astype(dt).reshape(shape)
+    return rng.integers(0, 200, n).astype(dt).reshape(shape)
+
+
+@pytest.mark.parametrize("bytes_", [1, 2, 4, 8])
+def test_every_permutation_of_small_tensors(rt, bytes_):
+    dt = DTYPES[bytes_]
+    for shape in ((3, 5), (4, 3, 5), (2, 3, 4, 5), (70, 3, 66)):
+        X = values(shape, dt, sum(shape))
+        for perm in itertools.permutations(range(len(shape))):
+            got = run_transpose(rt, X, perm)
+            assert np.array_equal(got, oracle.transpose(X, perm)), (shape, perm)
+            assert np.array_equal(got, np.transpose(X, perm))
+
+
+CASES = [  # shape, perm: tiles with ragged edges, merged axes, unit axes, rank 6, the attention and NCHW <-> NHWC forms
+    ((1000, 1000), (1, 0)), ((129, 257), (1, 0)), ((64, 64), (1, 0)), ((1, 300), (1, 0)), ((300, 1), (1, 0)),
+    ((8, 16, 200, 64), (0, 2, 1, 3)), ((8, 16, 200, 64), (0, 1, 3, 2)), ((32, 64, 14, 14), (0, 2, 3, 1)), ((32, 14, 14, 64), (0, 3, 1, 2)),
+    ((2, 3, 4, 5, 6, 7), (5, 3, 1, 0, 2, 4)), ((2, 3, 4, 5, 6, 7), (0, 1, 2, 3, 4, 5)), ((2, 1, 3, 1, 5), (4, 3, 2, 1, 0)),
+    ((5, 6, 7), (1, 0, 2)), ((0, 5), (1, 0)), ((7,), (0,)), ((3, 4, 65, 2), (2, 0, 1, 3)),
+]
+
+
+@pytest.mark.parametrize("shape,perm", CASES, ids=["x".join(map(str, s)) + "_" + "".join(map(str, p)) for s, p in CASES])
+def test_transpose_shapes(rt, shape, perm):
+    for dt in (np.float32, np.float64, np.int16):
+        X = values(shape, dt, len(shape) + sum(perm))
+        assert np.array_equal(run_transpose(rt, X, perm), oracle.transpose(X, perm)), dt
+
+
+def test_transpose_involution_at_full_size_and_errors(rt):
+    """[8192, 4096] fp32: transposing twice gives the input back; row sums become column sums."""
+    g = torch.Generator(device="cuda").manual_seed(4)
+    x = torch.randn(8192, 4096, device="cuda", generator=g)
+    y, z = torch.empty(4096, 8192, device="cuda"), torch.empty(8192, 4096, device="cuda")
+    rt.transpose(4, (8192, 4096), (1, 0), x.data_ptr(), y.data_ptr())
+    rt.transpose(4, (4096, 8192), (1, 0), y.data_ptr(), z.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(x, z) and torch.equal(y[17], x[:, 17]) and torch.equal(y[:, 8000], x[8000])
+    from docc_amd.runtime import RocmRuntimeError
+    p = x.data_ptr()
+    with pytest.raises(RocmRuntimeError, match="permutation"):
+        rt.transpose(4, (4, 4), (0, 0), p, y.data_ptr())
+    with pytest.raises(RocmRuntimeError, match="in place"):
+        rt.transpose(4, (4, 4), (1, 0), p, p)
+    with pytest.raises(RocmRuntimeError, match="element size"):
+        rt.transpose(3, (4, 4), (1, 0), p, y.data_ptr())
+    with pytest.raises(RocmRuntimeError, match="rank"):
+        rt.transpose(4, (2,) * 7, tuple(range(7)), p, y.data_ptr())

@@ -197,6 +197,35 @@ def test_attention_with_another_head_dimension_brings_its_workspace(tmp_path):
             assert src.index("docc_rocm_malloc(&__ws") < src.index("docc_rocm_attention_bf16_ws(") < src.index("docc_rocm_free(__ws)")
 
 
+def test_transpose_node_round_trips_and_dispatches(tmp_path):
+    b = StructuredSDFGBuilder("tr")
+    b.add_container("X", F32, True)
+    b.add_container("Y", F32, True)
+    b.add_container("_s0", I64, True)
+    b.add_transpose("X", "Y", ["_s0", 3, 5], [2, 0, 1])
+    s = b.move()
+    node = s.library_nodes()[0]
+    assert node["code"] == "ml::Transpose" and node["perm"] == [2, 0, 1] and node["shape"] == ["_s0", "3", "5"]
+    again = StructuredSDFG.parse(s.to_json()).library_nodes()[0]
+    assert {k: v for k, v in again.items() if k != "element_id"} == {k: v for k, v in node.items() if k != "element_id"}
+    s.schedule("rocm", options={"offload": "node"})
+    src, _ = source_of(s, tmp_path)
+    assert "const int64_t __docc_shape[] = {(int64_t) (_s0), (int64_t) (3), (int64_t) (5)};" in src
+    assert "const int64_t __docc_perm[] = {2, 0, 1};" in src
+    assert "docc_rocm_transpose(nullptr, 4, 3, __docc_shape, __docc_perm, d_X, d_Y)" in src
+    # no permutation: the axes are reversed, as in the reference's constructor
+    b = StructuredSDFGBuilder("tr2")
+    b.add_container("X", F64, True)
+    b.add_container("Y", F64, True)
+    b.add_transpose("X", "Y", [2, 3, 4])
+    assert b.move().library_nodes()[0]["perm"] == [2, 1, 0]
+    with pytest.raises(InvalidSDFGException, match="permutation"):
+        b = StructuredSDFGBuilder("bad")
+        b.add_container("X", F32, True)
+        b.add_container("Y", F32, True)
+        b.add_transpose("X", "Y", [2, 3], [0, 0])
+
+
 def test_matmul_node_is_one_batched_launch(tmp_path):
     """[6, 32, 16] @ [16, 24]: B is shared (stride 0); with a batched B its stride is k*n."""
     for shape_b, stride_b in (([16, 24], "0"), ([6, 16, 24], "384")):
