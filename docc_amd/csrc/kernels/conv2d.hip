@@ -466,3 +466,24 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3(docc_
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_k::ConvParams p, int TH) {
     docc_k::ConvHaloKernel<1, 1>::run(p, TH);
 }
+
+// Explicit im2col for the layers the two kernels above serve badly (small images, many channels): the
+// columns of images n0 .. n0+nn-1 as one row-major matrix col[K = C*KH*KW][nn * OH*OW], zero where a tap
+// leaves the image, so that the convolution is one GEMM  W[OC][K] x col  into [OC][nn * OH*OW].
+// Thread = one column (image, pixel), blockIdx.y walks the K rows: writes are contiguous, reads follow ow.
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_im2col_f32(docc_k::ConvParams p, int n0, int nn, float* col) {
+    const int P = p.OH * p.OW, K = p.C * p.KH * p.KW;
+    const long cols = (long) nn * P;
+    const long j = (long) blockIdx.x * 256 + threadIdx.x;
+    if (j >= cols) return;
+    const int n = n0 + (int) (j / P), pix = (int) (j % P);
+    const int oh = pix / p.OW, ow = pix % p.OW;
+    const int ih0 = oh * p.stride_h - p.pad_h, iw0 = ow * p.stride_w - p.pad_w;
+    const float* x = p.X + (long) n * p.C * p.H * p.W;
+    for (int kk = blockIdx.y; kk < K; kk += gridDim.y) {
+        const int c = kk / (p.KH * p.KW), t = kk % (p.KH * p.KW);
+        const int ih = ih0 + (t / p.KW) * p.dil_h, iw = iw0 + (t % p.KW) * p.dil_w;
+        const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+        col[(long) kk * cols + j] = inside ? x[((long) c * p.H + ih) * p.W + iw] : 0.f;
+    }
+}

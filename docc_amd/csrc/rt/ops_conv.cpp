@@ -26,10 +26,91 @@ int64_t out_dim(int64_t d_in, int64_t pad, int64_t dil, int64_t kernel, int64_t 
 
 } // namespace
 
-extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
-                                    int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h,
-                                    int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
-                                    const float* bias, float* Y) {
+namespace {
+
+constexpr int64_t kConvWorkspaceCap = int64_t(2) << 30;   // images are processed in chunks that fit this
+
+// Rough times (us) of the three ways to run a layer, from what the kernels were measured to sustain. The halo
+// kernel computes 64 channels x 448 pixels per work-group whatever the strip really holds, one work-group per CU
+// at a time, at about 490 GFLOP/s per CU. The gather kernel sustains about 55 TFLOP/s when its 64 x 128 tiles
+// fill the CUs evenly. The GEMM on a column matrix runs at about 75 TFLOP/s on these shapes; the columns are
+// written and read once at about 5 TB/s, and the extra launches (columns, bias, transpose) cost about 15 us.
+double halo_time_us(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t K, int cus) {
+    int64_t TH = 448 / OW;
+    if (TH > OH) TH = OH;
+    if (TH < 1) TH = 1;
+    const int64_t groups = N * ((OH + TH - 1) / TH) * ((OC + 63) / 64);
+    const int64_t rounds = (groups + cus - 1) / cus;
+    return (double) rounds * (2.0 * 64 * 448 * (double) K) / 490e3;
+}
+
+double gather_time_us(int64_t N, int64_t OC, int64_t P, int64_t K, int cus) {
+    const int64_t tiles = ((OC + 63) / 64) * ((N * P + 127) / 128);
+    const int64_t rounds = (tiles + cus - 1) / cus;
+    return (double) rounds * cus * (2.0 * 64 * 128 * (double) K) / 55e6;
+}
+
+double gemm_time_us(int64_t N, int64_t OC, int64_t P, int64_t K, bool needs_columns) {
+    const double padded_oc = (double) ((OC + 63) / 64 * 64);
+    return 2.0 * padded_oc * (double) K * (double) N * (double) P / 75e6 +
+           (needs_columns ? 2.0 * 4.0 * (double) N * (double) K * (double) P / 5e6 + 15.0 : 5.0);
+}
+
+// bytes of columns + GEMM result per image
+int64_t conv_bytes_per_image(int64_t OC, int64_t K, int64_t P) { return (K * P * 4 + 255) / 256 * 256 + (OC * P * 4 + 255) / 256 * 256; }
+
+enum class ConvPath { Halo, Gather, Gemm1x1, GemmColumns };
+
+// shapes the LDS-halo kernel is built for (the launcher also wants 16-byte aligned weights)
+bool halo_shape_ok(int64_t C, int64_t KH, int64_t KW, int64_t OW, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w) {
+    return stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && ((KH == 3 && KW == 3) || (KH == 1 && KW == 1)) && C % 8 == 0 &&
+           C > 0 && OW <= 448 && (C * KH * KW) % 4 == 0;
+}
+
+ConvPath choose_path(int64_t N, int64_t C, int64_t OC, int64_t KH, int64_t KW, int64_t OH, int64_t OW, int64_t stride_h, int64_t stride_w,
+                     int64_t pad_h, int64_t pad_w, bool halo_ok, bool have_workspace) {
+    const char* force = std::getenv("DOCC_ROCM_CONV");   // halo | gather | gemm (tuning and tests)
+    const bool pointwise = KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0;
+    const ConvPath gemm = pointwise ? ConvPath::Gemm1x1 : ConvPath::GemmColumns;
+    const bool gemm_ok = pointwise || have_workspace;
+    if (force && force[0] == 'h' && halo_ok) return ConvPath::Halo;
+    if (force && force[0] == 'g' && force[1] == 'a') return ConvPath::Gather;
+    if (force && force[0] == 'g' && force[1] == 'e' && gemm_ok) return gemm;
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    const int64_t K = C * KH * KW, P = OH * OW;
+    // the aligned GEMM kernels want rows of the weight and column matrices that are multiples of 16 bytes
+    const bool gemm_fast = gemm_ok && K % 4 == 0 && (pointwise ? P % 4 == 0 : true);
+    // 1x1 layers move more bytes than they compute, which the models above do not see: measured, the batched GEMM
+    // wins from 128 input channels on (C 256 -> 64 on 56 x 56: 50 against 65 us; C 64 -> 256: 99 against 74)
+    if (pointwise) return gemm_fast && C >= 128 ? gemm : halo_ok ? ConvPath::Halo : ConvPath::Gather;
+    const double direct = halo_ok ? halo_time_us(N, OC, OH, OW, K, cus) : gather_time_us(N, OC, P, K, cus);
+    if (gemm_fast && gemm_time_us(N, OC, P, K, true) < 0.75 * direct) return gemm;
+    return halo_ok ? ConvPath::Halo : ConvPath::Gather;
+}
+
+} // namespace
+
+extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                                        int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
+                                                        int64_t dil_w) {
+    if (N <= 0 || C <= 0 || OC <= 0 || KH <= 0 || KW <= 0 || stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0) return 0;
+    const int64_t OH = out_dim(H, pad_h, dil_h, KH, stride_h), OW = out_dim(W, pad_w, dil_w, KW, stride_w);
+    if (OH <= 0 || OW <= 0) return 0;
+    if (KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0) return 0;   // the input is the column matrix
+    // nothing either when one of the direct kernels would be chosen anyway (operands assumed aligned)
+    const bool halo_ok = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w);
+    if (choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, pad_h, pad_w, halo_ok, true) != ConvPath::GemmColumns) return 0;
+    const int64_t per_image = conv_bytes_per_image(OC, C * KH * KW, OH * OW);
+    int64_t images = kConvWorkspaceCap / per_image;
+    if (images < 1) images = 1;
+    if (images > N) images = N;
+    return images * per_image;
+}
+
+static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                      int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X,
+                      const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
     if (N < 0 || C < 0 || H < 0 || W < 0 || OC < 0 || KH <= 0 || KW <= 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
     if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0)
@@ -47,10 +128,54 @@ extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_
                  (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w};
     // Stride-1, dilation-1 3x3 and 1x1 convolutions take the LDS-halo kernel: 64 output channels x a
     // strip of TH full output rows (at most 448 pixels) per work-group, 8 input channels per chunk.
-    const bool halo_shape = stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 &&
-                            ((KH == 3 && KW == 3) || (KH == 1 && KW == 1)) && C % 8 == 0 && C > 0 && OW <= 448 &&
-                            ((uintptr_t) Wt % 16 == 0) && ((C * KH * KW) % 4 == 0);
-    if (halo_shape && !std::getenv("DOCC_ROCM_CONV_GATHER")) {
+    const bool halo_shape = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w) && ((uintptr_t) Wt % 16 == 0);
+    const int64_t need = docc_rocm_conv2d_f32_workspace_bytes(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w);
+    const bool have_workspace = workspace && workspace_bytes >= need && need > 0 && ((uintptr_t) workspace % 256) == 0;
+    const ConvPath path = C == 0 ? ConvPath::Gather
+                                 : choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, pad_h, pad_w, halo_shape, have_workspace);
+    if (path == ConvPath::Gemm1x1) {
+        // Y[n] (OC x P) = W (OC x C) X[n] (C x P): one batched GEMM on the tensors as they lie; the bias is
+        // written first and accumulated onto
+        const int64_t P = OH * OW;
+        if (bias) {
+            const int64_t in_shape[3] = {1, OC, 1}, out_shape[3] = {N, OC, P};
+            rc = docc_rocm_broadcast(stream, 32, 3, in_shape, out_shape, bias, Y);
+            if (rc) return rc;
+        }
+        return docc_rocm_sgemm_batched(stream, DOCC_ROCM_NO_TRANS, DOCC_ROCM_NO_TRANS, OC, P, C, 1.f, Wt, C, 0, X, P, C * P, bias ? 1.f : 0.f,
+                                       Y, P, OC * P, N);
+    }
+    if (path == ConvPath::GemmColumns) {
+        const int64_t P = OH * OW, K = C * KH * KW;
+        const int64_t per_image = conv_bytes_per_image(OC, K, P);
+        int64_t chunk = workspace_bytes / per_image;
+        if (chunk > N) chunk = N;
+        float* col = (float*) workspace;
+        float* result = (float*) ((char*) workspace + chunk * ((K * P * 4 + 255) / 256 * 256));
+        for (int64_t n0 = 0; n0 < N; n0 += chunk) {
+            const int64_t nn = N - n0 < chunk ? N - n0 : chunk;
+            const int64_t cols = nn * P;
+            rc = launch("docc_conv2d_im2col_f32", (uint32_t) ((cols + 255) / 256), (uint32_t) (K < 65535 ? K : 65535), 1, 256, 0,
+                        (hipStream_t) stream, p, (int) n0, (int) nn, col);
+            if (rc) return rc;
+            // one image: the GEMM result is the output itself; more: [OC][nn][P], moved to [nn][OC][P] afterwards
+            float* out = nn == 1 ? Y + n0 * OC * P : result;
+            if (bias) {
+                const int64_t in_shape[2] = {OC, 1}, out_shape[2] = {OC, cols};
+                rc = docc_rocm_broadcast(stream, 32, 2, in_shape, out_shape, bias, out);
+                if (rc) return rc;
+            }
+            rc = docc_rocm_sgemm(stream, DOCC_ROCM_NO_TRANS, DOCC_ROCM_NO_TRANS, OC, cols, K, 1.f, Wt, K, col, cols, bias ? 1.f : 0.f, out, cols);
+            if (rc) return rc;
+            if (nn > 1) {
+                const int64_t shape[3] = {OC, nn, P}, perm[3] = {1, 0, 2};
+                rc = docc_rocm_transpose(stream, 4, 3, shape, perm, result, Y + n0 * OC * P);
+                if (rc) return rc;
+            }
+        }
+        return 0;
+    }
+    if (path == ConvPath::Halo) {
         int64_t TH = 448 / OW;
         if (TH > OH) TH = OH;
         const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch pixels
@@ -70,4 +195,19 @@ extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_
     const uint32_t lds = 2 * (BM * (BK + 4) + BK * (BN + 8)) * 4 + 2 * BK * 16;
     return launch(aligned ? "docc_conv2d_f32_gather_64x128_a" : "docc_conv2d_f32_gather_64x128_u", (uint32_t) tiles, 1,
                   1, 256, lds, (hipStream_t) stream, p);
+}
+
+extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                                    int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h,
+                                    int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
+                                    const float* bias, float* Y) {
+    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, nullptr, 0);
+}
+
+extern "C" int docc_rocm_conv2d_f32_ws(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                                       int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h,
+                                       int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
+                                       const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
+    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, workspace,
+                      workspace_bytes);
 }

@@ -141,8 +141,18 @@ static TileConfig pick_sgemm(int64_t m, int64_t n, int64_t batch, bool aligned, 
     const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
     if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128, batch) >= 256 ? plain_big : plain_small);
     if (force) return force > 0 ? wide : small;
-    // the largest tile that still gives every CU a work-group
-    return tiles_of(m, n, 128, 256, batch) >= 256 ? wide : tiles_of(m, n, 128, 128, batch) >= 256 ? big : small;
+    // Score = share of a tile's area that is real output x share of the CUs that get a work-group x what the
+    // tile sustains relative to the widest (141 / 138 / about 105 TFLOP/s on large problems): a 64-row product
+    // wastes half of a 128-row tile, a 1000^2 one leaves most CUs idle with the large tiles.
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    auto score = [&](const TileConfig& c, double rel) {
+        const double padded = (double) ((m + c.bm - 1) / c.bm * c.bm) * (double) ((n + c.bn - 1) / c.bn * c.bn);
+        const double fill = (double) tiles_of(m, n, c.bm, c.bn, batch) / cus;
+        return rel * ((double) m * (double) n / padded) * (fill < 1.0 ? fill : 1.0);
+    };
+    const double sw = score(wide, 1.0), sb = score(big, 0.97), ss = score(small, 0.75);
+    return sw >= sb && sw >= ss ? wide : sb >= ss ? big : small;
 }
 
 static TileConfig pick_dgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {

@@ -274,13 +274,28 @@ protected:
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
         const auto& c = conv();
         auto get = [](const std::vector<Expression>& v, size_t i, const char* dflt) { return v.empty() ? Expression(dflt) : v[i]; };
-        s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32(nullptr, " << c.shape()[0] << ", " << c.shape()[1] << ", " << c.shape()[2]
-          << ", " << c.shape()[3] << ", " << c.output_channels() << ", " << c.kernel_shape()[0] << ", " << c.kernel_shape()[1]
-          << ", " << get(c.strides(), 0, "1") << ", " << get(c.strides(), 1, "1") << ", " << get(c.pads(), 0, "0") << ", "
-          << get(c.pads(), 1, "0") << ", " << get(c.dilations(), 0, "1") << ", " << get(c.dilations(), 1, "1")
-          << ", (const float *) " << name_of("X") << ", (const float *) " << name_of("W") << ", "
+        std::ostringstream dims;
+        dims << c.shape()[0] << ", " << c.shape()[1] << ", " << c.shape()[2] << ", " << c.shape()[3] << ", " << c.output_channels() << ", "
+             << c.kernel_shape()[0] << ", " << c.kernel_shape()[1] << ", " << get(c.strides(), 0, "1") << ", " << get(c.strides(), 1, "1")
+             << ", " << get(c.pads(), 0, "0") << ", " << get(c.pads(), 1, "0") << ", " << get(c.dilations(), 0, "1") << ", "
+             << get(c.dilations(), 1, "1");
+        // layers that run as im2col + GEMM take their column matrix from a workspace that lives around the node;
+        // for the others the size is 0 and nothing is allocated
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "const int64_t __ws_bytes = docc_rocm_conv2d_f32_workspace_bytes(" << dims.str() << ");" << std::endl;
+        s << "void *__ws = nullptr;" << std::endl;
+        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc(&__ws, (size_t) __ws_bytes));" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32_ws(nullptr, " << dims.str() << ", (const float *) " << name_of("X")
+          << ", (const float *) " << name_of("W") << ", "
           << (c.has_bias() ? "(const float *) " + name_of("B") : std::string("nullptr")) << ", (float *) " << name_of("Y")
-          << "));" << std::endl;
+          << ", __ws, __ws_bytes));" << std::endl;
+        s << "if (__ws) {" << std::endl;
+        s << "    DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
+        s << "    DOCC_ROCM_CHECK(docc_rocm_free(__ws));" << std::endl;
+        s << "}" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
     }
 };
 

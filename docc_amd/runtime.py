@@ -75,6 +75,8 @@ _SIGNATURES = {
     "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
     "docc_rocm_softmax": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
+    "docc_rocm_conv2d_f32_workspace_bytes": [_i64] * 13,
+    "docc_rocm_conv2d_f32_ws": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp, _vp, _i64],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
     "docc_rocm_attention_bf16_workspace_bytes": [_i64] * 5 + [_int],
     "docc_rocm_attention_bf16_ws": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int, _vp, _i64],
@@ -92,7 +94,8 @@ _SIGNATURES = {
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
-            "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64}
+            "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64,
+            "docc_rocm_conv2d_f32_workspace_bytes": _i64}
 
 #: every symbol the two public headers declare
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -262,6 +265,16 @@ def softmax_f32(rows, cols, X, Y, stream=0) -> None:
 def conv2d_f32(N, C, H, W, OC, KH, KW, stride, pad, dilation, X, Wt, bias, Y, stream=0) -> None:
     call("docc_rocm_conv2d_f32", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pad[0], pad[1],
          dilation[0], dilation[1], X, Wt, bias or None, Y)
+
+
+def conv2d_f32_workspace_bytes(N, C, H, W, OC, KH, KW, stride, pad, dilation) -> int:
+    return int(lib().docc_rocm_conv2d_f32_workspace_bytes(N, C, H, W, OC, KH, KW, stride[0], stride[1], pad[0], pad[1], dilation[0], dilation[1]))
+
+
+def conv2d_f32_ws(N, C, H, W, OC, KH, KW, stride, pad, dilation, X, Wt, bias, Y, workspace, workspace_bytes, stream=0) -> None:
+    """conv2d_f32 with device memory for a column matrix (conv2d_f32_workspace_bytes(...) bytes, 0 = none needed)."""
+    call("docc_rocm_conv2d_f32_ws", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pad[0], pad[1],
+         dilation[0], dilation[1], X, Wt, bias or None, Y, workspace or None, workspace_bytes)
 
 
 def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0) -> None:

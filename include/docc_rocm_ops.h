@@ -136,6 +136,24 @@ int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_
                          float* Y);
 
 /*
+ * The same node with device memory of the caller for a column matrix. Layers that the direct
+ * kernels serve badly (small images with many channels, strides, large filters) run as an explicit
+ * im2col followed by one GEMM  W[OC][C*KH*KW] x columns  over chunks of images that keep the
+ * workspace under 2 GiB, and a Transpose of the result into [N][OC][OH*OW]; 1x1 stride-1 layers
+ * without padding are a batched GEMM on the tensors as they lie and need no workspace. The
+ * choice is made from the shape; _workspace_bytes returns 0 where a direct kernel is chosen.
+ * `workspace`: 256-byte aligned, at least _workspace_bytes(...) bytes; with less (or NULL) the call
+ * behaves like docc_rocm_conv2d_f32.
+ */
+int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                             int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
+                                             int64_t dil_w);
+int docc_rocm_conv2d_f32_ws(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                            int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                            int64_t dil_h, int64_t dil_w, const float* X, const float* Wt, const float* bias,
+                            float* Y, void* workspace, int64_t workspace_bytes);
+
+/*
  * ml::Attention (a node the rocm target adds; the reference has none):
  *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
  * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32
