@@ -196,8 +196,8 @@ extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_stream(const 
         }
     }
     float gm = block_max(m, lds);
-    // a thread that saw no element has m = -inf, s = 0: contributes 0
-    float contrib = (m == kNegInf) ? 0.f : s * exp_neg(m - gm);
+    // a thread that saw no element has m = -inf, s = 0: contributes 0 (a NaN sum counts even then)
+    float contrib = (m == kNegInf && s == s) ? 0.f : s * exp_neg(m - gm);
     float gs = block_sum(contrib, lds);
     gs += gm - gm;   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
     const float inv = 1.0f / gs;
@@ -235,6 +235,14 @@ __device__ __forceinline__ void online_step(T v, T& m, T& s) {
     }
 }
 
+// what a (maximum m, sum s) pair adds to a sum taken relative to g >= m: nothing when no element was seen
+// (m = -inf, s = 0), but a NaN sum counts even then (a NaN element does not move the maximum)
+template <typename T>
+__device__ __forceinline__ T pair_weight(T m, T s, T g) {
+    using M = SoftmaxMath<T>;
+    return (m == M::neg_inf() && s == s) ? (T) 0 : s * M::exp_le0(m - g);
+}
+
 // merges the pairs of the NP threads that share a column; lm / ls hold one pair per thread
 template <typename T>
 __device__ __forceinline__ void merge_pairs(const T* lm, const T* ls, int first, int step, int count, T& gm, T& gs) {
@@ -242,10 +250,7 @@ __device__ __forceinline__ void merge_pairs(const T* lm, const T* ls, int first,
     gm = M::neg_inf();
     for (int i = 0; i < count; i++) gm = M::max(gm, lm[first + i * step]);
     gs = (T) 0;
-    for (int i = 0; i < count; i++) {
-        const T m = lm[first + i * step];
-        if (m != M::neg_inf()) gs += ls[first + i * step] * M::exp_le0(m - gm);
-    }
+    for (int i = 0; i < count; i++) gs += pair_weight(lm[first + i * step], ls[first + i * step], gm);
     gs += gm - gm;   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
 }
 
@@ -269,11 +274,8 @@ __device__ __forceinline__ void softmax_row_stream(const T* X, T* Y, long cols) 
             const T m2 = lm[threadIdx.x + half], s2 = ls[threadIdx.x + half];
             const T m1 = lm[threadIdx.x], s1 = ls[threadIdx.x];
             const T g = M::max(m1, m2);
-            T acc = (T) 0;
-            if (m1 != M::neg_inf()) acc += s1 * M::exp_le0(m1 - g);
-            if (m2 != M::neg_inf()) acc += s2 * M::exp_le0(m2 - g);
             lm[threadIdx.x] = g;
-            ls[threadIdx.x] = acc;
+            ls[threadIdx.x] = pair_weight(m1, s1, g) + pair_weight(m2, s2, g);
         }
         __syncthreads();
     }
@@ -327,7 +329,104 @@ __device__ __forceinline__ void softmax_strided_slab(const T* X, T* Y, long redu
     for (long i = threadIdx.x; i < n; i += 256) y[i] = M::exp_le0(x[i] - gm) / gs;
 }
 
+// Few columns and a long reduced extent leave the tile kernel with a handful of work-groups that each walk
+// the whole extent twice. The sliced pair spreads the rows as well: work-group (outer index, slice of rows,
+// 64-column tile) first leaves its running (maximum, sum) pairs in the scratch array below, then - in a second
+// launch - every work-group merges the pairs of all slices of its columns and writes the results of its own
+// slice. The scratch array is shared by every such call on the device.
+constexpr long kSoftmaxScratchBytes = 8l << 20;
+__device__ __attribute__((aligned(256))) unsigned char docc_softmax_scratch[kSoftmaxScratchBytes];
+
+struct SlicedWork {
+    long o, col, r0, r1;   // outer index, this lane's column, rows [r0, r1) of the slice
+    long slice;
+    bool live;
+};
+
+__device__ __forceinline__ SlicedWork sliced_work(long reduce, long inner, long tiles, int slices) {
+    SlicedWork w;
+    long b = blockIdx.x;
+    const long tile = b % tiles;
+    b /= tiles;
+    w.slice = b % slices;
+    w.o = b / slices;
+    w.col = tile * 64 + (threadIdx.x & 63);
+    const long per = (reduce + slices - 1) / slices;
+    w.r0 = w.slice * per;
+    w.r1 = w.r0 + per < reduce ? w.r0 + per : reduce;
+    w.live = w.col < inner;
+    return w;
+}
+
+template <typename T>
+__device__ __forceinline__ void softmax_sliced_partial(const T* X, long reduce, long inner, long tiles, int slices) {
+    using M = SoftmaxMath<T>;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const SlicedWork w = sliced_work(reduce, inner, tiles, slices);
+    const int part = threadIdx.x >> 6;
+    const T* x = X + w.o * reduce * inner + w.col;
+    T m = M::neg_inf(), s = (T) 0;
+    if (w.live)
+        for (long r = w.r0 + part; r < w.r1; r += 4) online_step(x[r * inner], m, s);
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    if (part == 0 && w.live) {
+        // the pair of the slice, without the NaN marker for infinite maxima: that is applied once, at the end
+        T gm = M::neg_inf();
+        for (int i = 0; i < 4; i++) gm = M::max(gm, lm[(threadIdx.x & 63) + 64 * i]);
+        T gs = (T) 0;
+        for (int i = 0; i < 4; i++) gs += pair_weight(lm[(threadIdx.x & 63) + 64 * i], ls[(threadIdx.x & 63) + 64 * i], gm);
+        T* P = reinterpret_cast<T*>(docc_softmax_scratch);
+        const long at = ((w.o * slices + w.slice) * inner + w.col) * 2;
+        P[at] = gm;
+        P[at + 1] = gs;
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void softmax_sliced_finish(const T* X, T* Y, long reduce, long inner, long tiles, int slices) {
+    using M = SoftmaxMath<T>;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const SlicedWork w = sliced_work(reduce, inner, tiles, slices);
+    const int part = threadIdx.x >> 6;
+    const T* P = reinterpret_cast<const T*>(docc_softmax_scratch);
+    // the four waves share the slices of this column
+    T m = M::neg_inf(), s = (T) 0;
+    if (w.live)
+        for (int sl = part; sl < slices; sl += 4) {
+            const long at = ((w.o * slices + sl) * inner + w.col) * 2;
+            const T pm = P[at], ps = P[at + 1];
+            const T g = M::max(m, pm);
+            s = pair_weight(m, s, g) + pair_weight(pm, ps, g);
+            m = g;
+        }
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    T gm, gs;
+    merge_pairs(lm, ls, (int) (threadIdx.x & 63), 64, 4, gm, gs);
+    if (!w.live) return;
+    const T* x = X + w.o * reduce * inner + w.col;
+    T* y = Y + w.o * reduce * inner + w.col;
+    for (long r = w.r0 + part; r < w.r1; r += 4) y[r * inner] = M::exp_le0(x[r * inner] - gm) / gs;
+}
+
 } // namespace
+
+#define DOCC_SOFTMAX_SLICED(T, SUFFIX)                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_partial(const T* X, long reduce, long inner, \
+                                                                                            long tiles, int slices) {       \
+        softmax_sliced_partial<T>(X, reduce, inner, tiles, slices);                                                           \
+    }                                                                                                                         \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_finish(const T* X, T* Y, long reduce,       \
+                                                                                           long inner, long tiles, int slices) { \
+        softmax_sliced_finish<T>(X, Y, reduce, inner, tiles, slices);                                                         \
+    }
+DOCC_SOFTMAX_SLICED(float, f32)
+DOCC_SOFTMAX_SLICED(double, f64)
 
 extern "C" __global__ __launch_bounds__(256) void docc_softmax_f64_stream(const double* X, double* Y, long rows, long cols) {
     softmax_row_stream<double>(X, Y, cols);

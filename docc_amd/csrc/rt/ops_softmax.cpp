@@ -66,6 +66,25 @@ int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, i
     }
     const int64_t tiles = (inner + 63) / 64;
     if (tiles > 0x7fffffffLL / outer) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 work-groups");
+    // Few (outer index, column tile) pairs and many rows: slice the rows as well, so that about four work-groups
+    // per CU share the tensor; the pairs of the slices go through the kernels' 8 MiB scratch array.
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    const int64_t groups = outer * tiles;
+    if (groups < 2 * (int64_t) cus && reduce >= 256) {
+        int64_t slices = (4 * (int64_t) cus + groups - 1) / groups;
+        if (slices > reduce / 64) slices = reduce / 64;
+        const int64_t pair_bytes = 2 * (precision / 8);
+        const int64_t fit = (int64_t(8) << 20) / (outer * inner * pair_bytes);
+        if (slices > fit) slices = fit;
+        if (slices >= 2) {
+            std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_partial", t);
+            int rc = launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, X, (long) reduce, (long) inner, (long) tiles, (int) slices);
+            if (rc) return rc;
+            std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_finish", t);
+            return launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles, (int) slices);
+        }
+    }
     std::snprintf(name, sizeof(name), "docc_softmax_%s_tile", t);
     return launch(name, (uint32_t) (outer * tiles), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles);
 }

@@ -118,7 +118,10 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
  * the axes before it is `outer`, of those after it `inner`); precision 32 (float) or 64
  * (double). The reference's node takes any axes and its element type from its memlets
  * (softmax_node.cpp:38-110). inner == 1 with precision 32 is docc_rocm_softmax_f32; the other
- * forms read X twice (running maximum and sum, then the results).
+ * forms read X twice (running maximum and sum, then the results). With few columns and a long
+ * reduced extent the intermediate (maximum, sum) pairs of row slices pass through an 8 MiB scratch
+ * array in the kernel image, shared by every such call on the device: do not overlap them on
+ * different streams.
  */
 int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner,
                       const void* X, void* Y);

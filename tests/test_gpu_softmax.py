@@ -112,6 +112,8 @@ GENERAL = [  # shape, axes
     ((5, 7), (0,)), ((64, 300), (0,)), ((3, 1000, 8), (1,)), ((4, 257, 16), (1,)), ((2, 50, 33), (1,)), ((6, 31, 64), (1,)),
     ((2, 9, 200), (0, 1)), ((3, 4, 5, 6), (1, 2)), ((7, 129), (-1,)), ((1, 5000), (-1,)), ((4, 6, 2), (1,)), ((1, 4096, 1), (1,)),
     ((3, 3, 3), (0, 1, 2)), ((2, 2048, 4), (-2,)), ((5, 1, 70), (1,)),
+    # few columns, long extents: the rows are sliced over work-groups as well
+    ((1000, 300), (0,)), ((3, 700, 130), (1,)), ((2, 4096, 65), (1,)), ((1, 257, 64), (1,)), ((5000, 40), (0,)),
 ]
 
 
@@ -165,6 +167,23 @@ def test_softmax_general_edge_values_and_empty(rt):
         Xc[2, :] = -np.inf
         Yr = run_softmax(rt, Xc)
         assert np.isnan(Yr[:3]).all() and np.allclose(Yr[3], 1.0 / cols)
+    # sliced path: a NaN that is the only element one thread sees besides -inf, an infinite value in one slice
+    for dt in (np.float32, np.float64):
+        Xs = np.zeros((1, 1024, 70), dt)
+        Xs[0, :, 5] = -np.inf
+        Xs[0, 517, 5] = np.nan
+        Xs[0, 900, 9] = np.inf
+        Xs[0, 3, 11] = -np.inf
+        xs = dev(Xs)
+        ys = torch.empty_like(xs)
+        rt.softmax(64 if dt == np.float64 else 32, 1, 1024, 70, xs.data_ptr(), ys.data_ptr())
+        torch.cuda.synchronize()
+        Ys = host(ys)
+        with np.errstate(invalid="ignore"):
+            refs = oracle.softmax_axes(Xs, (1,))
+        assert np.array_equal(np.isnan(Ys), np.isnan(refs))
+        assert np.isnan(Ys[0, :, 5]).all() and np.isnan(Ys[0, :, 9]).all() and Ys[0, 3, 11] == 0
+        np.testing.assert_allclose(Ys[~np.isnan(refs)], refs[~np.isnan(refs)], rtol=1e-5 if dt == np.float32 else 1e-13)
     z = torch.zeros(8, device="cuda")
     rt.softmax(32, 0, 4, 2, z.data_ptr(), z.data_ptr())
     rt.softmax(64, 2, 0, 2, z.data_ptr(), z.data_ptr())
