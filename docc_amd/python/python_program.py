@@ -508,7 +508,9 @@ class _Lowering(ast.NodeVisitor):
                             if isinstance(z, _ScalarValue) and z.text in ("0.0", "-0.0") and isinstance(x, (_Array, _Lazy)):
                                 return self.unary(node, "relu", x, dest)
                     return self.elementwise(node, op, a, b, dest)
-        reductions = {np.sum: "sum", np.max: "max", np.amax: "max", np.min: "min", np.amin: "min", np.mean: "mean"}
+        reductions = {np.sum: "sum", np.max: "max", np.amax: "max", np.min: "min", np.amin: "min", np.mean: "mean", np.std: "std"}
+        if (fn is np.std or (fn is None and isinstance(node.func, ast.Attribute) and node.func.attr == "std")) and self.kw(node, "ddof", None, 0) != 0:
+            self.fail(node, "a standard deviation with ddof != 0")
         if fn is np.sum:
             v = self.ev(node.args[0])
             if isinstance(v, _Lazy) and v.kind == "exp_sub" and axis_last(v.base):
@@ -517,7 +519,7 @@ class _Lowering(ast.NodeVisitor):
             if fn is f and node.args:
                 return self.reduce(node, op, self.ev(node.args[0]), self.kw(node, "axis", 1, None), bool(self.kw(node, "keepdims", None, False)), dest)
         # the same as methods of an array: x.sum(axis=..), x.max(..), x.min(..), x.mean(..)
-        if fn is None and isinstance(node.func, ast.Attribute) and node.func.attr in ("sum", "max", "min", "mean"):
+        if fn is None and isinstance(node.func, ast.Attribute) and node.func.attr in ("sum", "max", "min", "mean", "std"):
             base = self.ev(node.func.value)
             if isinstance(base, (_Array, _Lazy)):
                 return self.reduce(node, node.func.attr, base, self.kw(node, "axis", 0, None), bool(self.kw(node, "keepdims", None, False)), dest)

@@ -347,6 +347,9 @@ class StructuredSDFGBuilder:
                              "element_type": self._element(X).value},
                             [self._operand("X", X)], [self._operand("Y", Y)])
             return
+        if op == "std":
+            self._add_std(X, Y, shape, axes, keepdims)
+            return
         if op != "softmax":
             raise NotImplementedError(f"reduce op '{op}' is not part of the rocm target")
         if keepdims:
@@ -355,6 +358,34 @@ class StructuredSDFGBuilder:
                          "shape": [_expr(s) for s in shape], "axes": [int(a) for a in axes], "keepdims": False,
                          "element_type": self._element(X).value},
                         [self._operand("X", X)], [self._operand("Y", Y)])
+
+    def _add_std(self, X: str, Y: str, shape: Sequence[Any], axes: Sequence[int], keepdims: bool) -> None:
+        """The node chain StdNode::expand leaves behind (reference .../reduce_ops/std_node.cpp: X*X, Mean of it,
+        Mean(X), its square, their difference, Sqrt), built directly: the population standard deviation
+        sqrt(mean(x^2) - mean(x)^2) with the reference's rounding at every step; temporaries are transients."""
+        elem = self._element(X)
+        rank = len(shape)
+        norm = sorted({int(a) % rank for a in axes})
+        out_shape = [("1" if d in norm else _expr(s)) for d, s in enumerate(shape) if keepdims or d not in norm] or ["1"]
+        size = {PrimitiveType.Float: 4, PrimitiveType.Double: 8}.get(elem)
+        if size is None:
+            raise InvalidSDFGException("ml::Std: element type must be Float or Double")
+
+        def temp(dims):
+            nbytes = str(size)
+            for d in dims:
+                nbytes = f"({_expr(d)})*{nbytes}"
+            name = self.find_new_name("_std_tmp_")
+            self.add_container(name, Pointer(Scalar(elem)), False, transient_bytes=nbytes)
+            return name
+
+        x2, mean_x2, mean_x = temp(shape), temp(out_shape), temp(out_shape)
+        self.add_elementwise_op("mul", X, X, x2, shape)
+        self.add_reduce_op("mean", x2, mean_x2, shape, axes, keepdims)
+        self.add_reduce_op("mean", X, mean_x, shape, axes, keepdims)
+        self.add_elementwise_op("mul", mean_x, mean_x, mean_x, out_shape)
+        self.add_elementwise_op("sub", mean_x2, mean_x, mean_x2, out_shape)
+        self.add_elementwise_unary_op("sqrt", mean_x2, Y, out_shape)
 
     def add_conv(self, X: str, W: str, Y: str, shape: Sequence[Any], kernel_shape: Sequence[Any], strides: Sequence[Any],
                  pads: Sequence[Any], dilations: Sequence[Any], output_channels: Any, group: Any = 1, B: Optional[str] = None) -> None:

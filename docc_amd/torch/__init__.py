@@ -483,6 +483,15 @@ class _FxLowering:
                 dim = kwargs.get("dim", kwargs.get("axis", args[1] if len(args) > 1 else None))
                 keepdim = bool(kwargs.get("keepdim", kwargs.get("keepdims", args[2] if len(args) > 2 else False)))
                 return self.reduce(node, {"amax": "max", "amin": "min"}.get(name, name), args[0], dim, keepdim, dest)
+        if t is torch.std or method == "std":
+            # the node computes the population value sqrt(mean(x^2) - mean(x)^2): torch's default divides by n - 1
+            correction = kwargs.get("correction", None)
+            if correction is None:
+                correction = 1 if kwargs.get("unbiased", True) else 0
+            if correction != 0:
+                self.fail(node, "a standard deviation with a correction other than 0 (pass correction=0)")
+            dim = kwargs.get("dim", args[1] if len(args) > 1 else None)
+            return self.reduce(node, "std", args[0], dim, bool(kwargs.get("keepdim", False)), dest)
         if t is F.linear:
             bias = args[2] if len(args) > 2 else kwargs.get("bias")
             return self.linear(node, args[0], args[1], bias, dest)

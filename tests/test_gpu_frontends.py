@@ -271,9 +271,10 @@ def test_instrumented_program_writes_a_trace_with_device_times(tmp_path, mode):
     pcie = sorted((e["args"]["metrics"]["static:::pcie_bytes"]["mean"] if mode == "aggregate" else e["args"]["metrics"]["static:::pcie_bytes"])
                   for e in kinds["h2d_transfer"])[-1]
     assert pcie == 512 * 256 * 4
-    # a GEMM of this size takes well under 10 ms on the device; a region's time is a device time, not the process's
+    # even with the first launch uploading its code object a GEMM of this size stays well under 50 ms on the device;
+    # a region's time is a device time, not the process's (compilation alone takes seconds)
     gemm = [e for e in kinds["math"] if e["name"].startswith("dense") and (e["args"]["metrics"].get("static:::flop") is not None)]
-    assert gemm and min(e["dur"] / (3 if mode == "aggregate" else 1) for e in gemm) < 10000
+    assert gemm and min(e["dur"] / (3 if mode == "aggregate" else 1) for e in gemm) < 50000
 
 
 def test_program_in_docc_json_format_runs(tmp_path):
@@ -431,3 +432,32 @@ def test_transposes_through_both_front_ends():
     o1, o2, o3 = docc_torch.compile_torch(P(), (t, u), target="rocm")(t, u)
     assert torch.equal(o1, t.permute(0, 2, 1, 3) + 1.0) and torch.equal(o2, torch.relu(u.transpose(0, 1)))
     assert torch.equal(o3, t.transpose(1, 2).contiguous())
+
+
+def test_standard_deviation_is_the_reference_node_chain():
+    """np.std / torch.std(correction=0): Mul, Mean, Mean, Mul, Sub, Sqrt, the chain StdNode::expand builds
+    (population value, sqrt(mean(x^2) - mean(x)^2))."""
+    @native(target="rocm")
+    def spread(x):
+        return np.std(x, axis=1), x.std(axis=(0, 1), keepdims=True)
+
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((40, 300, 6)) * 3 + 1.5
+    a, b = spread(x)
+    codes = [n["code"] for n in spread.last_sdfg.library_nodes() if n["code"].startswith("ml::")]
+    assert codes[:6] == ["ml::Mul", "ml::Mean", "ml::Mean", "ml::Mul", "ml::Sub", "ml::Sqrt"]
+    np.testing.assert_allclose(a, np.std(x, axis=1), rtol=1e-10)
+    np.testing.assert_allclose(b, np.std(x, axis=(0, 1), keepdims=True), rtol=1e-10)
+    # the same steps on the CPU oracle, bit for bit
+    m2 = oracle.reduce("mean", oracle.elementwise_binary("mul", x, x), (1,))
+    m1 = oracle.reduce("mean", x, (1,))
+    want = oracle.elementwise_unary("sqrt", oracle.elementwise_binary("sub", m2, oracle.elementwise_binary("mul", m1, m1)))
+    np.testing.assert_allclose(a, want, rtol=1e-12)
+
+    class S(torch.nn.Module):
+        def forward(self, t):
+            return torch.std(t, dim=-1, correction=0)
+
+    t = torch.randn(64, 500)
+    out = docc_torch.compile_torch(S(), (t,), target="rocm")(t)
+    np.testing.assert_allclose(out.numpy(), t.std(dim=-1, correction=0).numpy(), rtol=2e-4)

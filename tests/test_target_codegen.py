@@ -532,8 +532,16 @@ def test_reduce_nodes_dispatch_and_decline(tmp_path):
     b.add_reduce_op("mean", "X", "Y", [4, 5, 6], [0, 2])
     with pytest.raises(InvalidSDFGException, match="adjacent"):
         b.move().schedule("rocm")
-    with pytest.raises(NotImplementedError, match="std"):
-        StructuredSDFGBuilder("s").add_reduce_op("std", "X", "Y", [4], [0])
+    # std is the chain of nodes the reference's StdNode expands to
+    b = StructuredSDFGBuilder("s")
+    for n in ("X", "Y"):
+        b.add_container(n, F32, True)
+    b.add_reduce_op("std", "X", "Y", [4, 9], [1])
+    s = b.move()
+    assert [n["code"] for n in s.library_nodes()] == ["ml::Mul", "ml::Mean", "ml::Mean", "ml::Mul", "ml::Sub", "ml::Sqrt"]
+    assert sorted(k for k, c in s.containers.items() if c["transient"]) == ["_std_tmp_0", "_std_tmp_1", "_std_tmp_2"]
+    with pytest.raises(NotImplementedError, match="var"):
+        StructuredSDFGBuilder("s").add_reduce_op("var", "X", "Y", [4], [0])
     b = StructuredSDFGBuilder("axis")
     for n in ("X", "Y"):
         b.add_container(n, F64, True)
