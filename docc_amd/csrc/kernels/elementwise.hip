@@ -296,3 +296,45 @@ DOCC_EW_FUSED(f64_v2_i32, double, 2, unsigned)
 DOCC_EW_FUSED(f64_v1_i32, double, 1, unsigned)
 DOCC_EW_FUSED(f64_v2_i64, double, 2, long)
 DOCC_EW_FUSED(f64_v1_i64, double, 1, long)
+
+
+// ---- ml::Cast ---------------------------------------------------------------------------------
+// Y[i] = (D) X[i], the conversion an assign tasklet between differently typed memlets compiles to
+// (reference elementwise_ops/cast_node.cpp:39-40): round to nearest even between floating types,
+// truncation towards zero from a floating type to an integer. bf16 travels as raw 16-bit words.
+namespace docc_k {
+
+struct Bf16Bits { unsigned short bits; };
+
+template <typename S> __device__ __forceinline__ auto cast_load(const S* p, long i) { return p[i]; }
+template <> __device__ __forceinline__ auto cast_load<Bf16Bits>(const Bf16Bits* p, long i) { return bf16_bits_to_f32(p[i].bits); }
+
+template <typename D, typename V> __device__ __forceinline__ void cast_store(D* p, long i, V v) { p[i] = (D) v; }
+template <> __device__ __forceinline__ void cast_store<Bf16Bits, float>(Bf16Bits* p, long i, float v) { p[i].bits = f32_to_bf16_rne(v); }
+
+template <typename S, typename D>
+__device__ __forceinline__ void cast_kernel(const S* X, D* Y, long n) {
+    const long stride = (long) gridDim.x * 256;
+    for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < n; i += stride) cast_store<D>(Y, i, cast_load<S>(X, i));
+}
+
+} // namespace docc_k
+
+#define DOCC_CAST(SN, S, DN, D)                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_cast_##SN##_##DN(const S* X, D* Y, long n) {                    \
+        docc_k::cast_kernel<S, D>(X, Y, n);                                                                              \
+    }
+DOCC_CAST(f32, float, f64, double)
+DOCC_CAST(f64, double, f32, float)
+DOCC_CAST(f32, float, bf16, docc_k::Bf16Bits)
+DOCC_CAST(bf16, docc_k::Bf16Bits, f32, float)
+DOCC_CAST(f32, float, f16, _Float16)
+DOCC_CAST(f16, _Float16, f32, float)
+DOCC_CAST(i32, int, f32, float)
+DOCC_CAST(i32, int, f64, double)
+DOCC_CAST(i64, long, f32, float)
+DOCC_CAST(i64, long, f64, double)
+DOCC_CAST(f32, float, i32, int)
+DOCC_CAST(f64, double, i32, int)
+DOCC_CAST(f32, float, i64, long)
+DOCC_CAST(f64, double, i64, long)

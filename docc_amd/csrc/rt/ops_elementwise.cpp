@@ -258,3 +258,30 @@ extern "C" int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precis
     std::snprintf(name, sizeof(name), "docc_ew_fused_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
     return launch(name, grid_for(n / lanes, kGridFused), 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, p);
 }
+
+extern "C" int docc_rocm_cast(docc_rocm_stream_t stream, int src_type, int dst_type, int64_t n, const void* X, void* Y) {
+    static const char* const kTypeNames[] = {"f16", "bf16", "f32", "f64", "i32", "i64"};
+    static const int kSize[] = {2, 2, 4, 8, 4, 8};
+    if (src_type < 0 || src_type > DOCC_ROCM_TYPE_I64 || dst_type < 0 || dst_type > DOCC_ROCM_TYPE_I64)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "cast: unknown type code");
+    if (n < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "cast: negative count");
+    if (n == 0) return 0;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "cast: null pointer");
+    if (src_type == dst_type) {
+        if (X == Y) return 0;
+        return check(hipMemcpyAsync(Y, X, (size_t) n * kSize[src_type], hipMemcpyDeviceToDevice, (hipStream_t) stream), "hipMemcpyAsync");
+    }
+    // built: fp32 <-> fp64 / bf16 / fp16, int32 / int64 <-> fp32 / fp64
+    const bool f = src_type == DOCC_ROCM_TYPE_F32 || src_type == DOCC_ROCM_TYPE_F64, g = dst_type == DOCC_ROCM_TYPE_F32 || dst_type == DOCC_ROCM_TYPE_F64;
+    const bool s16 = src_type <= DOCC_ROCM_TYPE_BF16, d16 = dst_type <= DOCC_ROCM_TYPE_BF16;
+    const bool si = src_type >= DOCC_ROCM_TYPE_I32, di = dst_type >= DOCC_ROCM_TYPE_I32;
+    const bool built = (f && g) || (s16 && dst_type == DOCC_ROCM_TYPE_F32) || (d16 && src_type == DOCC_ROCM_TYPE_F32) || (si && g) || (f && di);
+    if (!built)
+        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "cast: %s -> %s is not built (16-bit types convert through f32, integers to and from f32 / f64)",
+                    kTypeNames[src_type], kTypeNames[dst_type]);
+    int rc = ensure_device();
+    if (rc) return rc;
+    char name[48];
+    std::snprintf(name, sizeof(name), "docc_cast_%s_%s", kTypeNames[src_type], kTypeNames[dst_type]);
+    return launch(name, grid_for(n, kGridStreaming), 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) n);
+}

@@ -202,6 +202,7 @@ struct Import {
 
         Array inputs, outputs;
         const Value* out_type = nullptr;
+        const Value* in_type = nullptr;
         bool has_bias_edge = false;
         for (auto& e : df.at("edges").as_array()) {
             const bool into = e.at("dst").as_int() == lib_id, from = e.at("src").as_int() == lib_id;
@@ -219,6 +220,7 @@ struct Import {
                 } else {
                     b.set("data", n.at("data").as_string());
                 }
+                if (!in_type) in_type = &e.at("base_type");
                 if (e.at("dst_conn").as_string() == "B") has_bias_edge = true;
                 inputs.push_back(std::move(b));
             } else {
@@ -245,6 +247,12 @@ struct Import {
             if (kv.first != "debug_info") node.set(kv.first, c_expressions(kv.second));
         node.set("side_effect", false);
         // what the reference keeps in the memlet types, the block list keeps on the node
+        if (code == "ml::Cast") {   // "target_type" is the enum value there, the name here; the element type is the input's
+            if (!in_type) throw InvalidSDFGException(describe(*lib) + ": no input edge");
+            const Value* tt = node.find("target_type");
+            if (tt && tt->is_number()) node.set("target_type", types::primitive_type_to_string(primitive_of(*tt, describe(*lib))));
+            if (!node.contains("element_type")) node.set("element_type", types::primitive_type_to_string(element_of(*in_type, describe(*lib))));
+        }
         if (code != "GEMM" && !node.contains("element_type")) {
             if (!out_type) throw InvalidSDFGException(describe(*lib) + ": no output edge");
             node.set("element_type", types::primitive_type_to_string(element_of(*out_type, describe(*lib))));
@@ -449,6 +457,9 @@ Value export_reference_json(const StructuredSDFG& sdfg) {
         lib.set("implementation_type", blk.node->implementation_type());
         lib.set("code", blk.node->code());
         blk.node->to_json(lib);
+        if (blk.node->code() == "ml::Cast")
+            if (const Value* tt = lib.find("target_type"))
+                if (tt->is_string()) lib.set("target_type", reference_primitive(types::primitive_type_from_string(tt->as_string())));
         nodes.push_back(std::move(lib));
         auto edge = [&](int64_t src, const std::string& src_conn, int64_t dst, const std::string& dst_conn, Value base_type) {
             Value e;

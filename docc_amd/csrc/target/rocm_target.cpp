@@ -35,7 +35,7 @@ bool is_math_node(const LibraryNode& node) {
     const std::string& c = node.code();
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
            c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
-           c == tensor::LibraryNodeType_Transpose || is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
+           c == tensor::LibraryNodeType_Transpose || c == tensor::LibraryNodeType_Cast || is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
 }
 
 // Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
@@ -457,6 +457,43 @@ protected:
     }
 };
 
+// ---- Cast ----------------------------------------------------------------------------------
+
+// runtime type code (DOCC_ROCM_TYPE_*) of an element type, or -1
+int cast_type_code(types::PrimitiveType t) {
+    switch (t) {
+        case types::PrimitiveType::Half: return 0;
+        case types::PrimitiveType::BFloat: return 1;
+        case types::PrimitiveType::Float: return 2;
+        case types::PrimitiveType::Double: return 3;
+        case types::PrimitiveType::Int32: return 4;
+        case types::PrimitiveType::Int64: return 5;
+        default: return -1;
+    }
+}
+
+bool cast_is_built(int s, int d) {
+    if (s < 0 || d < 0) return false;
+    if (s == d) return true;
+    const bool f = s == 2 || s == 3, g = d == 2 || d == 3;
+    return (f && g) || (s <= 1 && d == 2) || (d <= 1 && s == 2) || (s >= 4 && g) || (f && d >= 4);
+}
+
+class CastNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::CastNode&>(node_);
+        s << "DOCC_ROCM_CHECK(docc_rocm_cast(nullptr, " << cast_type_code(n.element()) << " /* " << types::primitive_type_to_string(n.element())
+          << " */, " << cast_type_code(n.target_type()) << " /* " << types::primitive_type_to_string(n.target_type()) << " */, " << n.count()
+          << ", " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+    }
+};
+
 // ---- Transpose -----------------------------------------------------------------------------
 
 class TransposeNodeDispatcher_ROCM : public RocmMathDispatcher {
@@ -594,6 +631,7 @@ void register_plugin(plugins::Context& context) {
     for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
     register_math<TransposeNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Transpose);
+    register_math<CastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Cast);
     for (auto& code : tensor::ReduceNodeCodes) register_math<ReduceNodeDispatcher_ROCM>(reg, code);
     register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
     reg.register_library_node_dispatcher(
@@ -663,6 +701,12 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!b) return decline("not a Broadcast node object");
         if (b->element() != P::Float && b->element() != P::Double) return decline("element type must be Float or Double");
         if (b->output_shape().size() > 6) return decline("rank above 6 is not supported");
+    } else if (node.code() == tensor::LibraryNodeType_Cast) {
+        auto* c = dynamic_cast<tensor::CastNode*>(&node);
+        if (!c) return decline("not a Cast node object");
+        if (!cast_is_built(cast_type_code(c->element()), cast_type_code(c->target_type())))
+            return decline(std::string("conversion ") + types::primitive_type_to_string(c->element()) + " -> " +
+                           types::primitive_type_to_string(c->target_type()) + " is not built");
     } else if (node.code() == tensor::LibraryNodeType_Transpose) {
         auto* t = dynamic_cast<tensor::TransposeNode*>(&node);
         if (!t) return decline("not a Transpose node object");

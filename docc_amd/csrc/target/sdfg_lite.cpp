@@ -583,6 +583,31 @@ Expression BroadcastNode::connector_bytes(const std::string& connector) const {
     return bytes_of(product(shape, 0, shape.size()), element_);
 }
 
+CastNode::CastNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element, types::PrimitiveType target)
+    : LibraryNode(LibraryNodeType_Cast, {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)), element_(element),
+      target_(target) {}
+
+Expression CastNode::count() const { return shape_.empty() ? Expression("1") : product(shape_, 0, shape_.size()); }
+
+void CastNode::validate() const {
+    if (element_ == types::PrimitiveType::Void || target_ == types::PrimitiveType::Void) throw InvalidSDFGException("Cast: void element type");
+}
+
+void CastNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    j.set("target_type", types::primitive_type_to_string(target_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<CastNode> CastNode::from_json(const Value& j) {
+    const Value* et = j.find("element_type");
+    return std::make_unique<CastNode>(impl_of(j), exprs_from_json(j.at("shape")),
+                                      et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float,
+                                      types::primitive_type_from_string(j.at("target_type").as_string()));
+}
+
+Expression CastNode::connector_bytes(const std::string& connector) const { return bytes_of(count(), connector == "X" ? element_ : target_); }
+
 TransposeNode::TransposeNode(std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> perm,
                              types::PrimitiveType element)
     : LibraryNode(LibraryNodeType_Transpose, {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)),
@@ -1007,6 +1032,7 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     for (auto& code : math::tensor::BinaryNodeCodes) fns_[code] = &deserialize<math::tensor::ElementWiseNode>;
     fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
     fns_[math::tensor::LibraryNodeType_Transpose] = &deserialize<math::tensor::TransposeNode>;
+    fns_[math::tensor::LibraryNodeType_Cast] = &deserialize<math::tensor::CastNode>;
     for (auto& code : math::tensor::ReduceNodeCodes) fns_[code] = &deserialize<math::tensor::ReduceNode>;
     fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
 }

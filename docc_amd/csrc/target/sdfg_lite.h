@@ -338,6 +338,7 @@ inline const std::vector<std::string> UnaryNodeCodes = {"ml::Abs", "ml::Exp", "m
 inline const std::vector<std::string> BinaryNodeCodes = {"ml::Add", "ml::Sub", "ml::Mul", "ml::Div", "ml::Maximum", "ml::Minimum", "ml::Pow"};
 inline const std::string LibraryNodeType_Broadcast = "ml::Broadcast";
 inline const std::string LibraryNodeType_Transpose = "ml::Transpose";
+inline const std::string LibraryNodeType_Cast = "ml::Cast";
 
 class ElementWiseNode : public data_flow::LibraryNode {
 public:
@@ -377,6 +378,26 @@ public:
 private:
     std::vector<Expression> input_shape_, output_shape_;
     types::PrimitiveType element_;
+};
+
+// reference: .../tensor/elementwise_ops/cast_node.h:13-60 (connectors "X" -> "Y", JSON keys "shape" and
+// "target_type"; the input's element type comes from its memlet there and is kept on the node here)
+class CastNode : public data_flow::LibraryNode {
+public:
+    CastNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element, types::PrimitiveType target);
+    const std::vector<Expression>& shape() const { return shape_; }
+    types::PrimitiveType element() const { return element_; }
+    types::PrimitiveType target_type() const { return target_; }
+    Expression count() const;
+
+    void validate() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<CastNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    types::PrimitiveType element_, target_;
 };
 
 // reference: .../tensor/transpose_node.h:14-60 (connectors "X" -> "Y", JSON keys "shape" and "perm";

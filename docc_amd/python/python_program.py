@@ -462,6 +462,18 @@ class _Lowering(ast.NodeVisitor):
             if axes is None and isinstance(base, _Array) and len(base.shape) == 2:
                 return _Lazy("transposed", base)
             return self.transpose(node, base, axes, dest)
+        if fn is None and isinstance(node.func, ast.Attribute) and node.func.attr == "astype" and node.args:
+            base = self.array_of(node, self.ev(node.func.value))
+            target = {np.float32: PrimitiveType.Float, np.float64: PrimitiveType.Double}.get(self.resolve(node.args[0]))
+            if target is None and isinstance(node.args[0], ast.Constant):
+                target = {"float32": PrimitiveType.Float, "float64": PrimitiveType.Double}.get(node.args[0].value)
+            if not isinstance(base, _Array) or target is None:
+                self.fail(node, "astype to a type other than float32 / float64")
+            if base.elem not in (PrimitiveType.Float, PrimitiveType.Double, PrimitiveType.Int32, PrimitiveType.Int64):
+                self.fail(node, "astype of an array that is not float32, float64, int32 or int64")
+            out = self.new_array(base.shape, target, dest)
+            self.b.add_cast_op(base.name, out.name, base.shape)   # the same type copies
+            return out
         if fn is np.swapaxes and len(node.args) == 3:
             base = self.array_of(node, self.ev(node.args[0]))
             if not isinstance(base, _Array):

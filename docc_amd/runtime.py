@@ -86,6 +86,7 @@ _SIGNATURES = {
     "docc_rocm_elementwise_binary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp, _vp],
     "docc_rocm_elementwise_binary_scalar": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, ctypes.c_double, ctypes.c_int, _vp],
     "docc_rocm_broadcast": [_vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp],
+    "docc_rocm_cast": [_vp, _int, _int, _i64, _vp, _vp],
     "docc_rocm_transpose": [_vp, _int, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp, _vp],
     "docc_rocm_reduce": [_vp, ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_elementwise_fused": [_vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_double, _vp, _vp,
@@ -350,6 +351,15 @@ def elementwise_fused(precision, shape, binary, a, a_shape, b, b_shape, post, Y,
     call("docc_rocm_elementwise_fused", stream, precision, rank, ctypes.addressof(dims), code,
          ctypes.addressof(a_arr) if a_arr is not None else None, a_ptr, a_val,
          ctypes.addressof(b_arr) if b_arr is not None else None, b_ptr, b_val, len(post), ctypes.addressof(ops), Y)
+
+
+CAST_TYPES = {"f16": 0, "bf16": 1, "f32": 2, "f64": 3, "i32": 4, "i64": 5}
+
+
+def cast(src_type, dst_type, n, X, Y, stream=0) -> None:
+    """Y[i] = (dst_type) X[i]; types by name (CAST_TYPES) or code."""
+    code = lambda t: CAST_TYPES[t] if isinstance(t, str) else t
+    call("docc_rocm_cast", stream, code(src_type), code(dst_type), n, X, Y)
 
 
 def transpose(element_bytes, shape, perm, X, Y, stream=0) -> None:

@@ -439,6 +439,13 @@ class StructuredSDFGBuilder:
                          "element_type": self._element(X).value},
                         [self._operand("X", X)], [self._operand("Y", Y)])
 
+    def add_cast_op(self, X: str, Y: str, shape: Sequence[Any]) -> None:
+        """ml::Cast "X" -> "Y": Y[i] = (type of Y) X[i] (reference add_cast_op,
+        python/bindings/builder/py_structured_sdfg_builder.cpp:1015-1038; the target type is that of Y's container)."""
+        self._add_block({"code": "ml::Cast", "implementation_type": "NONE", "side_effect": False, "shape": [_expr(s) for s in shape],
+                         "target_type": self._element(Y).value, "element_type": self._element(X).value},
+                        [self._operand("X", X)], [self._operand("Y", Y)])
+
     def add_transpose(self, X: str, Y: str, shape: Sequence[Any], perm: Optional[Sequence[int]] = None) -> None:
         """ml::Transpose (reference .../tensor/transpose_node.h): Y.shape[i] = shape[perm[i]]; no perm reverses the axes."""
         rank = len(shape)

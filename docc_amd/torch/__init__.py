@@ -48,7 +48,8 @@ import docc_amd.python  # noqa: F401  (registers the rocm target hooks)
 def _elem(dtype) -> PrimitiveType:
     import torch
 
-    table = {torch.float32: PrimitiveType.Float, torch.float64: PrimitiveType.Double, torch.bfloat16: PrimitiveType.BFloat}
+    table = {torch.float32: PrimitiveType.Float, torch.float64: PrimitiveType.Double, torch.bfloat16: PrimitiveType.BFloat,
+             torch.float16: PrimitiveType.Half, torch.int32: PrimitiveType.Int32, torch.int64: PrimitiveType.Int64}
     if dtype not in table:
         raise NotImplementedError(f"tensor dtype {dtype} is not supported by the rocm target")
     return table[dtype]
@@ -320,6 +321,23 @@ class _FxLowering:
         self.builder.add_transpose(x.name, out.name, x.shape, dims)
         return out
 
+    def cast(self, node, x, dtype, dest=None):
+        """ml::Cast; the same dtype passes the tensor on."""
+        x = self.tensor(node, x)
+        if not isinstance(x, _T):
+            self.fail(node, "converting this value")
+        if x.dtype == dtype:
+            return x
+        code = {self.torch.float16: 0, self.torch.bfloat16: 1, self.torch.float32: 2, self.torch.float64: 3, self.torch.int32: 4,
+                self.torch.int64: 5}
+        s, d = code.get(x.dtype, -1), code.get(dtype, -1)
+        f, g = s in (2, 3), d in (2, 3)
+        if s < 0 or d < 0 or not ((f and g) or (s <= 1 and d == 2) or (d <= 1 and s == 2) or (s >= 4 and g) or (f and d >= 4)):
+            self.fail(node, f"a conversion from {x.dtype} to {dtype} (16-bit types convert through float32, integers to and from float32 / float64)")
+        out = self.new_tensor(x.shape, dtype, dest)
+        self.builder.add_cast_op(x.name, out.name, x.shape)
+        return out
+
     def tensor(self, node, v, dest=None):
         """A transposed view that is used as a tensor of its own (not as an operand of a product) is materialised."""
         if isinstance(v, _Transposed):
@@ -516,6 +534,14 @@ class _FxLowering:
                 self.fail(node, "attention on this query")
             scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
             return self.attention(node, q, bound["key"], bound["value"], float(scale), dest)
+        casts = {"float": torch.float32, "double": torch.float64, "bfloat16": torch.bfloat16, "half": torch.float16, "int": torch.int32,
+                 "long": torch.int64}
+        if method in casts and len(args) == 1:
+            return self.cast(node, args[0], casts[method], dest)
+        if method in ("to", "type") and (len(args) > 1 or "dtype" in kwargs):
+            dtype = kwargs.get("dtype", args[1] if len(args) > 1 else None)
+            if isinstance(dtype, torch.dtype):
+                return self.cast(node, args[0], dtype, dest)
         if method == "contiguous" or t is torch.Tensor.contiguous:
             return self.tensor(node, args[0], dest)   # a transposed view becomes the tensor it stands for
         self.fail(node, "this operation")

@@ -235,6 +235,20 @@ int docc_rocm_broadcast(docc_rocm_stream_t stream, int precision, int rank, cons
 int docc_rocm_transpose(docc_rocm_stream_t stream, int element_bytes, int rank, const int64_t* shape, const int64_t* perm,
                         const void* X, void* Y);
 
+/*
+ * ml::Cast: Y[i] = (D) X[i] for n contiguous elements, the conversion of an assign tasklet between
+ * memlets of different types (reference elementwise_ops/cast_node.cpp:39-40, node keys "shape" and
+ * "target_type"): round to nearest even between floating types, truncation towards zero to an
+ * integer. Built: fp32 <-> fp64, bf16, fp16; int32 / int64 <-> fp32 / fp64; equal types copy.
+ */
+#define DOCC_ROCM_TYPE_F16 0
+#define DOCC_ROCM_TYPE_BF16 1 /* raw 16-bit words */
+#define DOCC_ROCM_TYPE_F32 2
+#define DOCC_ROCM_TYPE_F64 3
+#define DOCC_ROCM_TYPE_I32 4
+#define DOCC_ROCM_TYPE_I64 5
+int docc_rocm_cast(docc_rocm_stream_t stream, int src_type, int dst_type, int64_t n, const void* X, void* Y);
+
 /* Reduce tensor nodes ml::Sum / ml::Max / ml::Min / ml::Mean over a block of adjacent axes
  * (reference sdfg/include/sdfg/data_flow/library_nodes/math/tensor/reduce_node.h and
  * reduce_ops/{sum,max,min,mean}_node.h; replaces the loop nests ReduceNode::expand emits,

@@ -318,3 +318,19 @@ def transpose(X, perm=None, lib=None) -> np.ndarray:
     if lib.oracle_transpose(X.dtype.itemsize, rank, shape, pm, X.ctypes.data, out.ctypes.data) != 0:
         raise ValueError("invalid permutation or rank above 8")
     return out
+
+
+def cast(X, dtype) -> np.ndarray:
+    """ml::Cast: the conversion an assign between differently typed memlets compiles to (reference
+    elementwise_ops/cast_node.cpp:39-40) - round to nearest even between floating types, truncation towards
+    zero to an integer, which is what numpy's astype does for these types. `dtype` "bf16" gives the raw
+    16-bit words (from fp32, through the C routine that test_oracle checks against torch); a uint16 input
+    with dtype float32 is read as bf16 words."""
+    X = np.ascontiguousarray(X)
+    if isinstance(dtype, str) and dtype == "bf16":
+        return f32_to_bf16(X.astype(np.float32, copy=False)) if X.dtype != np.uint16 else X.copy()
+    dtype = np.dtype(dtype)
+    if X.dtype == np.uint16:
+        return bf16_to_f32(X).astype(dtype, copy=False)
+    with np.errstate(all="ignore"):
+        return X.astype(dtype)

@@ -230,3 +230,55 @@ def test_fused_chain_with_libm_operations_and_unaligned_operands(rt):
         rt.elementwise_fused(32, (4, 4), None, 1.0, None, 0, None, ["relu"], out.data_ptr())                           # no array operand
     with pytest.raises(RocmRuntimeError):
         rt.elementwise_fused(32, (4, 4), None, dx.data_ptr(), (4, 4), 0, None, ["relu"] * 5, out.data_ptr())           # five unary operations
+
+
+CASTS = [("f32", "f64"), ("f64", "f32"), ("f32", "bf16"), ("bf16", "f32"), ("f32", "f16"), ("f16", "f32"), ("i32", "f32"), ("i32", "f64"),
+         ("i64", "f32"), ("i64", "f64"), ("f32", "i32"), ("f64", "i32"), ("f32", "i64"), ("f64", "i64"), ("f32", "f32")]
+NP_OF = {"f16": np.float16, "bf16": np.uint16, "f32": np.float32, "f64": np.float64, "i32": np.int32, "i64": np.int64}
+
+
+@pytest.mark.parametrize("src,dst", CASTS, ids=[f"{s}_to_{d}" for s, d in CASTS])
+def test_cast_bit_exact(rt, src, dst):
+    """ml::Cast: round to nearest even between floating types (ties, subnormals, overflow to inf, NaN), truncation
+    towards zero to integers, exact or rounded integer -> floating."""
+    rng = np.random.default_rng(len(src) * 7 + len(dst))
+    n = 10007
+    if src.startswith("i"):
+        x = rng.integers(-2 ** 30, 2 ** 30, n).astype(NP_OF[src])
+        x[:6] = [0, 1, -1, 16777217, -16777219, 2 ** 30 + 1]          # 2^24 + 1: rounds in fp32
+        if src == "i64":
+            x[6:9] = [2 ** 53 + 1, -(2 ** 62) - 1, 2 ** 40 + 3]
+    elif src == "bf16":
+        x = oracle.f32_to_bf16((rng.standard_normal(n) * 100).astype(np.float32))
+        x[:4] = [0x7f80, 0xff80, 0x7fc0, 0x0001]                       # inf, -inf, NaN, smallest subnormal
+    else:
+        x = (rng.standard_normal(n) * 1000).astype(NP_OF[src])
+        x[:10] = [0.0, -0.0, 1.5, 2049.0, 2051.0, 1e-40, 65520.0, 3.0e38, 1.0000000596046448, -7.99]
+        if dst.startswith("i"):
+            x = np.clip(x, -2.0e9, 2.0e9).astype(NP_OF[src])         # out-of-range conversions are undefined in C
+        else:
+            x[10:13] = [np.inf, -np.inf, np.nan]
+    dx = dev(x)
+    out = torch.empty(n, dtype={"f16": torch.float16, "bf16": torch.int16, "f32": torch.float32, "f64": torch.float64,
+                                "i32": torch.int32, "i64": torch.int64}[dst], device="cuda")
+    rt.cast(src, dst, n, dx.data_ptr(), out.data_ptr())
+    torch.cuda.synchronize()
+    got = host(out)
+    want = oracle.cast(x, "bf16" if dst == "bf16" else NP_OF[dst])
+    if dst == "bf16":
+        got = got.view(np.uint16)
+        nan = (want & 0x7fff) > 0x7f80
+        assert np.array_equal(((got & 0x7fff) > 0x7f80), nan) and np.array_equal(got[~nan], want[~nan])
+    else:
+        assert np.array_equal(got, want, equal_nan=True)
+    if (src, dst) == ("f32", "f16"):
+        assert np.isinf(got[6]) and got[3] == 2048.0 and got[4] == 2052.0 and got[2] == 1.5      # 65520 overflows; ties go to even
+
+
+def test_cast_rejects_what_is_not_built(rt):
+    from docc_amd.runtime import RocmRuntimeError
+    x = torch.zeros(64, device="cuda")
+    with pytest.raises(RocmRuntimeError, match="not built"):
+        rt.cast("f64", "bf16", 8, x.data_ptr(), x.data_ptr())
+    with pytest.raises(RocmRuntimeError, match="unknown type"):
+        rt.cast(9, 2, 8, x.data_ptr(), x.data_ptr())

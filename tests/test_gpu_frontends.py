@@ -461,3 +461,29 @@ def test_standard_deviation_is_the_reference_node_chain():
     t = torch.randn(64, 500)
     out = docc_torch.compile_torch(S(), (t,), target="rocm")(t)
     np.testing.assert_allclose(out.numpy(), t.std(dim=-1, correction=0).numpy(), rtol=2e-4)
+
+
+def test_casts_through_both_front_ends():
+    @native(target="rocm")
+    def widen(x, k):
+        return np.sqrt(x.astype(np.float64)) + k.astype(np.float64)
+
+    rng = np.random.default_rng(5)
+    x = np.abs(rng.standard_normal((30, 50))).astype(np.float32)
+    k = rng.integers(-5, 5, (30, 50))
+    got = widen(x, k)
+    assert got.dtype == np.float64
+    np.testing.assert_array_equal(got, np.sqrt(x.astype(np.float64)) + k.astype(np.float64))
+    assert [n["code"] for n in widen.last_sdfg.library_nodes() if n["code"].startswith("ml::")] == ["ml::Cast", "ml::Sqrt", "ml::Cast", "ml::Add"]
+
+    class Mixed(torch.nn.Module):
+        def forward(self, q, k, v):
+            s = torch.matmul(q.bfloat16(), k.bfloat16().transpose(-2, -1)) / 8.0
+            return torch.matmul(torch.softmax(s, dim=-1), v.bfloat16()).float()
+
+    torch.manual_seed(9)
+    q, k, v = (torch.randn(1, 2, 96, 64) for _ in range(3))
+    out = docc_torch.compile_torch(Mixed(), (q, k, v), target="rocm")(q, k, v)
+    assert out.dtype == torch.float32
+    ref = oracle.attention(bits(q.bfloat16()), bits(k.bfloat16()), bits(v.bfloat16()))
+    assert rel_err_max(out.numpy(), ref) <= 2e-2

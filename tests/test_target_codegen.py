@@ -226,6 +226,26 @@ def test_transpose_node_round_trips_and_dispatches(tmp_path):
         b.add_transpose("X", "Y", [2, 3], [0, 0])
 
 
+def test_cast_node_dispatches_and_declines(tmp_path):
+    b = StructuredSDFGBuilder("cast")
+    b.add_container("X", F32, True)
+    b.add_container("Y", BF16, True)
+    b.add_container("_s0", I64, True)
+    b.add_cast_op("X", "Y", ["_s0", 8])
+    s = b.move()
+    node = s.library_nodes()[0]
+    assert node["code"] == "ml::Cast" and node["target_type"] == "BFloat" and node["element_type"] == "Float"
+    s.schedule("rocm", options={"offload": "none"})
+    src, _ = source_of(s, tmp_path)
+    assert "docc_rocm_cast(nullptr, 2 /* Float */, 1 /* BFloat */, _s0*8, X, Y)" in src
+    b = StructuredSDFGBuilder("cast2")
+    b.add_container("X", F64, True)
+    b.add_container("Y", BF16, True)
+    b.add_cast_op("X", "Y", [4])
+    with pytest.raises(InvalidSDFGException, match="Double -> BFloat is not built"):
+        b.move().schedule("rocm")
+
+
 def test_matmul_node_is_one_batched_launch(tmp_path):
     """[6, 32, 16] @ [16, 24]: B is shared (stride 0); with a batched B its stride is k*n."""
     for shape_b, stride_b in (([16, 24], "0"), ([6, 16, 24], "384")):
