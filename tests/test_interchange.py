@@ -214,3 +214,26 @@ def test_export_writes_docc_layout_and_round_trips():
     for a, b2 in zip(again._data["root"]["children"], s._data["root"]["children"]):
         assert a["dataflow"]["inputs"] == b2["dataflow"]["inputs"] and a["dataflow"]["outputs"] == b2["dataflow"]["outputs"]
         assert a.get("debug_info") == b2.get("debug_info")
+
+
+def test_cast_and_transpose_nodes_cross_the_formats():
+    """ml::Cast carries its target type as the reference's enum value there (cast_node.cpp serializer) and takes the
+    input's element type from the input memlet; ml::Transpose carries shape and perm."""
+    b = StructuredSDFGBuilder("ct")
+    b.add_container("X", Pointer(Scalar(PrimitiveType.Float)), True)
+    b.add_container("H", Pointer(Scalar(PrimitiveType.BFloat)), False, transient_bytes=6 * 4 * 2)
+    b.add_container("Y", Pointer(Scalar(PrimitiveType.BFloat)), True)
+    b.add_cast_op("X", "H", [6, 4])
+    b.add_transpose("H", "Y", [6, 4], [1, 0])
+    s = b.move()
+    d = json.loads(s.to_docc_json())
+    cast, tr = (c["dataflow"]["nodes"][0] for c in d["root"]["children"][:2])
+    assert cast["code"] == "ml::Cast" and cast["target_type"] == 13 and cast["shape"] == ["6", "4"]      # BFloat in the reference's enum
+    assert tr["code"] == "ml::Transpose" and tr["perm"] == [1, 0]
+    # a dump as the reference writes it has no element_type key on the nodes
+    for n in (cast, tr):
+        n.pop("element_type", None)
+    again = StructuredSDFG.from_docc_json(json.dumps(d))
+    strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]
+    assert strip(again.library_nodes()) == strip(s.library_nodes())
+    assert again.library_nodes()[0]["element_type"] == "Float" and again.library_nodes()[0]["target_type"] == "BFloat"
