@@ -253,7 +253,8 @@ def test_cast_bit_exact(rt, src, dst):
         x[:4] = [0x7f80, 0xff80, 0x7fc0, 0x0001]                       # inf, -inf, NaN, smallest subnormal
     else:
         x = (rng.standard_normal(n) * 1000).astype(NP_OF[src])
-        x[:10] = [0.0, -0.0, 1.5, 2049.0, 2051.0, 1e-40, 65520.0, 3.0e38, 1.0000000596046448, -7.99]
+        with np.errstate(over="ignore"):      # 3e38 is inf in fp16
+            x[:10] = [0.0, -0.0, 1.5, 2049.0, 2051.0, 1e-40, 65520.0, 3.0e38, 1.0000000596046448, -7.99]
         if dst.startswith("i"):
             x = np.clip(x, -2.0e9, 2.0e9).astype(NP_OF[src])         # out-of-range conversions are undefined in C
         else:
@@ -282,3 +283,50 @@ def test_cast_rejects_what_is_not_built(rt):
         rt.cast("f64", "bf16", 8, x.data_ptr(), x.data_ptr())
     with pytest.raises(RocmRuntimeError, match="unknown type"):
         rt.cast(9, 2, 8, x.data_ptr(), x.data_ptr())
+
+
+def test_more_than_2_to_the_31_elements(rt):
+    """The kernels switch to 64-bit indices past 2^31 elements: unary, binary with a scalar, fused chain with a
+    repeated row, broadcast, transpose (rows and tiles) and cast on a tensor of 2^31 + 8192 fp32 elements (8.6 GB),
+    checked on the device at the start, around the 2^31 boundary and at the end."""
+    cols = 4096
+    rows = (1 << 31) // cols + 2
+    n = rows * cols
+    assert n > (1 << 31)
+    x = torch.empty(n, device="cuda")
+    x.copy_(torch.arange(n, device="cuda", dtype=torch.float32) % 1021 - 510.0)      # exact small integers, both signs
+    y = torch.empty(n, device="cuda")
+    windows = [slice(0, 5000), slice((1 << 31) - 5000, (1 << 31) + 5000), slice(n - 5000, n)]
+
+    def same(got, want):
+        for w in windows:
+            assert torch.equal(got[w], want[w])
+
+    rt.elementwise_unary("relu", 32, n, x.data_ptr(), y.data_ptr())
+    same(y, torch.relu(x))
+    rt.elementwise_binary_scalar("mul", 32, n, x.data_ptr(), 2.0, y.data_ptr())
+    for w in windows:
+        assert torch.equal(y[w], x[w] * 2.0)
+    row = torch.arange(cols, device="cuda", dtype=torch.float32)
+    rt.elementwise_fused(32, (rows, cols), "add", x.data_ptr(), (rows, cols), row.data_ptr(), (cols,), ["abs"], y.data_ptr())
+    for w in windows:
+        idx = torch.arange(w.start, w.stop, device="cuda")
+        assert torch.equal(y[w], (x[w] + row[idx % cols]).abs())
+    rt.broadcast(32, (1, cols), (rows, cols), row.data_ptr(), y.data_ptr())
+    for w in windows:
+        idx = torch.arange(w.start, w.stop, device="cuda")
+        assert torch.equal(y[w], row[idx % cols])
+    # transpose [rows, cols] -> [cols, rows] (tiles), and [rows / 2, 2, cols] -> [2, rows / 2, cols] (rows kernel)
+    rt.transpose(4, (rows, cols), (1, 0), x.data_ptr(), y.data_ptr())
+    yt = y.view(cols, rows)
+    for c, r0 in ((0, 0), (17, rows - 300), (cols - 1, rows // 2), (cols - 1, rows - 64)):
+        assert torch.equal(yt[c, r0:r0 + 64], x.view(rows, cols)[r0:r0 + 64, c])
+    rt.transpose(4, (rows // 2, 2, cols), (1, 0, 2), x.data_ptr(), y.data_ptr())
+    y3, x3 = y.view(2, rows // 2, cols), x.view(rows // 2, 2, cols)
+    for h, r in ((0, 0), (1, rows // 2 - 1), (1, 5), (0, rows // 4)):
+        assert torch.equal(y3[h, r], x3[r, h])
+    del y
+    z = torch.empty(n, device="cuda", dtype=torch.float64)
+    rt.cast("f32", "f64", n, x.data_ptr(), z.data_ptr())
+    for w in windows:
+        assert torch.equal(z[w], x[w].double())

@@ -192,3 +192,32 @@ def test_softmax_general_edge_values_and_empty(rt):
     from docc_amd.runtime import RocmRuntimeError
     with pytest.raises(RocmRuntimeError, match="precision"):
         rt.softmax(16, 1, 4, 2, z.data_ptr(), z.data_ptr())
+
+
+def test_softmax_and_reductions_past_2_to_the_31_elements(rt):
+    """[524290, 4096] fp32 (2^31 + 8192 elements): row offsets need 64 bits. Rows at the start, around the 2^31
+    boundary and at the end against the oracle; row sums and a reduction over the rows on the device."""
+    cols = 4096
+    rows = (1 << 31) // cols + 2
+    g = torch.Generator(device="cuda").manual_seed(6)
+    x = torch.empty(rows, cols, device="cuda")
+    x.normal_(0, 4, generator=g)
+    y = torch.empty_like(x)
+    rt.softmax_f32(rows, cols, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    for r0 in (0, rows // 2 - 2, rows - 3):
+        assert rel_err_max(host(y[r0:r0 + 3]), oracle.softmax(host(x[r0:r0 + 3]))) <= TOL_F32
+    sums = torch.empty(rows, device="cuda")
+    rt.reduce("sum", 32, rows, cols, 1, y.data_ptr(), sums.data_ptr())
+    torch.cuda.synchronize()
+    assert float((sums - 1).abs().max()) <= 1e-5
+    # over the rows (one result per column): the sliced column kernels walk 2^31 elements
+    colmax = torch.empty(cols, device="cuda")
+    rt.reduce("max", 32, 1, rows, cols, x.data_ptr(), colmax.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(colmax, x.max(dim=0).values)
+    # softmax over the rows of the last 300000 x 4096 block viewed as [1, 300000, 4096] would not add coverage of
+    # the index width; the general entry point is exercised past 2^31 through its row form instead
+    rt.softmax(32, rows, cols, 1, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    assert rel_err_max(host(y[rows - 2:]), oracle.softmax(host(x[rows - 2:]))) <= TOL_F32
