@@ -195,3 +195,42 @@ def test_gemm_every_tile_configuration(rt, dt, cfg):
                     assert np.array_equal(out, oracle.gemm(A, B, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb)), (cfg, m, n, k, ta, tb)
     finally:
         os.environ.pop("DOCC_ROCM_GEMM_CFG", None)
+
+
+def test_gemm_with_leading_dimensions_and_batch_strides_past_32_bit_offsets(rt):
+    """A with a row stride of 2^23 + 8 floats: a 128-row tile spans more than 2^32 bytes, which the asynchronous
+    kernels' 32-bit tile offsets cannot address - the launcher must take the register-path kernels. And a batch
+    whose stride is past 2^31 elements."""
+    import torch
+    m, n, k = 300, 256, 64
+    lda = (1 << 23) + 8
+    g = torch.Generator(device="cuda").manual_seed(12)
+    a_buf = torch.zeros(m * lda, device="cuda")
+    a = a_buf.view(m, lda)[:, :k]
+    a.copy_(torch.randint(-4, 5, (m, k), device="cuda", generator=g).float())
+    b = torch.randint(-4, 5, (k, n), device="cuda", generator=g).float()
+    c = torch.full((m, n), float("nan"), device="cuda")
+    rt.sgemm(m, n, k, 1.0, a_buf.data_ptr(), lda, b.data_ptr(), n, 0.0, c.data_ptr(), n)
+    torch.cuda.synchronize()
+    want = oracle.gemm(a.cpu().numpy(), b.cpu().numpy())
+    assert np.array_equal(c.cpu().numpy(), want)            # integer-valued: exact
+    # transposed: A^T stored [k, m] with the same stride
+    at_buf = torch.zeros(k * lda, device="cuda")
+    at = at_buf.view(k, lda)[:, :m]
+    at.copy_(a.t())
+    c.fill_(float("nan"))
+    rt.sgemm(m, n, k, 1.0, at_buf.data_ptr(), lda, b.data_ptr(), n, 0.0, c.data_ptr(), n, trans_a=T)
+    torch.cuda.synchronize()
+    assert np.array_equal(c.cpu().numpy(), want)
+    del a_buf, at_buf
+    # batch of 3 with A matrices 2^31 + 64 elements apart
+    stride_a = (1 << 31) + 64
+    a3 = torch.zeros(2 * stride_a + m * k, device="cuda")
+    mats = [torch.randint(-4, 5, (m, k), device="cuda", generator=g).float() for _ in range(3)]
+    for z, mat in enumerate(mats):
+        a3[z * stride_a:z * stride_a + m * k].copy_(mat.reshape(-1))
+    c3 = torch.full((3, m, n), float("nan"), device="cuda")
+    rt.gemm_batched("s", 3, m, n, k, 1.0, a3.data_ptr(), k, stride_a, b.data_ptr(), n, 0, 0.0, c3.data_ptr(), n, m * n)
+    torch.cuda.synchronize()
+    for z in range(3):
+        assert np.array_equal(c3[z].cpu().numpy(), oracle.gemm(mats[z].cpu().numpy(), b.cpu().numpy())), z
