@@ -17,16 +17,22 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
     if (!(scale > 0.f) || !std::isfinite(scale)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: scale must be positive and finite");
     if ((((uintptr_t) Q | (uintptr_t) K | (uintptr_t) V | (uintptr_t) O) % 16) != 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: pointers must be 16-byte aligned");
-    if (B * H > 65535 || SQ > 0x7fffffffLL - 128 || SKV > 0x7fffffffLL - 64)
-        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: batch*heads must be <= 65535 and sequences < 2^31");
+    if (SQ > 0x7fffffffLL - 128 || SKV > 0x7fffffffLL - 64) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: sequences must be < 2^31");
     int rc = ensure_device();
     if (rc) return rc;
     // LDS: ring of 3 stages x (K block [64][64] + V block [64][64]) bf16
     const uint32_t lds = 3 * (2 * 64 * 64) * 2;
     const float scale_log2e = scale * 1.4426950408889634f;
-    return launch(out_bf16 ? "docc_attention_bf16_d64_bf16out" : "docc_attention_bf16_d64_f32out",
-                  (uint32_t) ((SQ + 127) / 128), (uint32_t) (B * H), 1, 256, lds, (hipStream_t) stream, Q, K, V, O,
-                  (int) SQ, (int) SKV, scale_log2e);
+    // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
+    const int64_t BH = B * H, out_bytes = out_bf16 ? 2 : 4;
+    for (int64_t h0 = 0; h0 < BH; h0 += 65535) {
+        const int64_t nh = BH - h0 < 65535 ? BH - h0 : 65535;
+        rc = launch(out_bf16 ? "docc_attention_bf16_d64_bf16out" : "docc_attention_bf16_d64_f32out", (uint32_t) ((SQ + 127) / 128),
+                    (uint32_t) nh, 1, 256, lds, (hipStream_t) stream, Q + h0 * SQ * 64, K + h0 * SKV * 64, V + h0 * SKV * 64,
+                    (void*) ((char*) O + h0 * SQ * 64 * out_bytes), (int) SQ, (int) SKV, scale_log2e);
+        if (rc) return rc;
+    }
+    return 0;
 }
 
 // ---- any head dimension, through a caller-provided workspace -----------------------------------

@@ -148,3 +148,18 @@ def test_attention_workspace_is_checked_and_chunked(rt):
     for h in (0, 21, 39):       # heads of the first and of the second chunk
         ref = oracle.attention(bits(Q[:, h:h + 1, :256].cpu()), bits(K[:, h:h + 1].cpu()), bits(V[:, h:h + 1].cpu()))
         assert rel_err_max(o[:, h:h + 1, :256].cpu().numpy(), ref) <= TOL_BF16
+
+
+def test_attention_more_pairs_than_one_grid_holds(rt):
+    """70 000 (batch, head) pairs: the launcher splits them over launches of at most 65 535."""
+    B, H, S = 7, 10000, 16
+    g = torch.Generator(device="cuda").manual_seed(2)
+    Q, K, V = (torch.randn(B, H, S, 64, device="cuda", generator=g).bfloat16() for _ in range(3))
+    o = torch.full((B, H, S, 64), float("nan"), device="cuda")
+    rt.attention_bf16(B, H, S, S, 64, 0.125, Q.data_ptr(), K.data_ptr(), V.data_ptr(), o.data_ptr())
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(o).all())
+    flat = lambda t: t.reshape(1, B * H, S, 64)
+    for p in (0, 65534, 65535, 69999):
+        ref = oracle.attention(bits(flat(Q)[:, p:p + 1].cpu()), bits(flat(K)[:, p:p + 1].cpu()), bits(flat(V)[:, p:p + 1].cpu()))
+        assert rel_err_max(flat(o)[:, p:p + 1].cpu().numpy(), ref) <= TOL_BF16, p
