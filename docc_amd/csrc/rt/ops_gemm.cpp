@@ -55,16 +55,16 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     if (rc) return rc;
     hipStream_t s = (hipStream_t) stream;
     char name[96];
-    if (k == 0) {
+    if (k == 0 || alpha == (S) 0) {   // an empty product, or one BLAS does not reference ("when ALPHA is zero ...")
         std::snprintf(name, sizeof(name), "docc_%s_scale_c", prefix);
         int64_t blocks = (m * n + 255) / 256;
         if (blocks > 4096) blocks = 4096;
         for (int64_t z = 0; z < batch && rc == 0; z++)   // an empty product: one small launch per entry
             rc = launch(name, (uint32_t) blocks, 1, 1, 256, 0, s, C + z * batch_c, (long) m, (long) n, (long) ldc, beta);
         if (rc || (!bias && activation < 0)) return rc;
-        if (batch > 1) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 with an epilogue and a batch", prefix);
+        if (batch > 1) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 or alpha == 0 with an epilogue and a batch", prefix);
         // the epilogue of an empty product: C = act(beta * C + bias), through the elementwise kernel
-        if (ldc != n) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 with an epilogue needs ldc == n", prefix);
+        if (ldc != n) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: k == 0 or alpha == 0 with an epilogue needs ldc == n", prefix);
         const int64_t shape[2] = {m, n}, row[2] = {1, n};
         const int post[1] = {activation};
         return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,

@@ -38,7 +38,8 @@ extern "C" {
 
 /*
  * C[m,n] = alpha * op(A)[m,k] * op(B)[k,n] + beta * C[m,n], row-major, with
- * cblas semantics: when beta == 0, C is not read (it may hold NaNs).
+ * cblas semantics: when beta == 0, C is not read (it may hold NaNs); when alpha == 0,
+ * A and B are not referenced (C = beta * C).
  * Replaces cblas_dgemm / cblas_sgemm as printed by GEMMNodeDispatcher_BLAS
  * (reference gemm_node.cpp:474-505) and cublasDgemm / cublasSgemm
  * (reference opt/src/targets/cuda/blas/gemm.cpp:131-185).

@@ -122,7 +122,9 @@ ORACLE_GEMM_EXPANDED(oracle_gemm_expanded_f32, float)
  * The call GEMMNodeDispatcher_BLAS prints (gemm_node.cpp:449-509):
  *   cblas_?gemm(CblasRowMajor, transA, transB, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc)
  * restated from the BLAS definition C = alpha*op(A)*op(B) + beta*C, where C
- * is not read when beta == 0. trans codes are CBLAS's 111 (NoTrans) / 112
+ * is not read when beta == 0 and A, B are not referenced when alpha == 0 (the
+ * BLAS definition of ?GEMM: "when ALPHA is zero then A and B are not referenced",
+ * so NaNs in them do not reach C). trans codes are CBLAS's 111 (NoTrans) / 112
  * (Trans), the values the node serialises (blas_node.h:49-126). The k-loop
  * runs left to right in the element type.
  */
@@ -132,7 +134,7 @@ ORACLE_GEMM_EXPANDED(oracle_gemm_expanded_f32, float)
         _Pragma("omp parallel for schedule(static)") for (int64_t i = 0; i < m; i++) {                         \
             for (int64_t j = 0; j < n; j++) {                                                                  \
                 ACC sum = 0;                                                                                   \
-                for (int64_t p = 0; p < k; p++) {                                                              \
+                for (int64_t p = 0; p < (alpha == (T) 0 ? 0 : k); p++) {                                       \
                     ACC a = (trans_a == 112) ? A[lda * p + i] : A[lda * i + p];                                \
                     ACC b = (trans_b == 112) ? B[ldb * j + p] : B[ldb * p + j];                                \
                     sum += a * b;                                                                              \

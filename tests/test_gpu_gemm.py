@@ -234,3 +234,29 @@ def test_gemm_with_leading_dimensions_and_batch_strides_past_32_bit_offsets(rt):
     torch.cuda.synchronize()
     for z in range(3):
         assert np.array_equal(c3[z].cpu().numpy(), oracle.gemm(mats[z].cpu().numpy(), b.cpu().numpy())), z
+
+
+@pytest.mark.parametrize("kind", ["d", "s", "b"])
+def test_gemm_alpha_zero_does_not_reference_a_and_b(rt, kind):
+    """The BLAS definition: with alpha == 0 the product is not formed, so NaNs in A or B stay out of C = beta * C
+    (and beta == 0 stores zeros over a NaN-filled C)."""
+    import torch
+    m, n, k = 70, 90, 40
+    dt = torch.float64 if kind == "d" else torch.float32
+    a = torch.full((m, k), float("nan"), device="cuda", dtype=dt)
+    b = torch.full((k, n), float("nan"), device="cuda", dtype=dt)
+    if kind == "b":
+        a, b = a.bfloat16(), b.bfloat16()
+    c0 = torch.arange(m * n, device="cuda", dtype=dt).reshape(m, n) / 7
+    fn = {"d": rt.dgemm, "s": rt.sgemm, "b": rt.bf16gemm_f32}[kind]
+    c = c0.clone()
+    fn(m, n, k, 0.0, a.data_ptr(), k, b.data_ptr(), n, -1.5, c.data_ptr(), n)
+    torch.cuda.synchronize()
+    assert torch.equal(c, c0 * -1.5)
+    c = torch.full((m, n), float("nan"), device="cuda", dtype=dt)
+    fn(m, n, k, 0.0, a.data_ptr(), k, b.data_ptr(), n, 0.0, c.data_ptr(), n)
+    torch.cuda.synchronize()
+    assert torch.equal(c, torch.zeros_like(c))
+    want = oracle.gemm(np.full((m, k), np.nan, np.float64 if kind == "d" else np.float32), np.full((k, n), np.nan, np.float64 if kind == "d" else np.float32),
+                       c0.cpu().numpy(), alpha=0.0, beta=-1.5)
+    assert np.array_equal(want, (c0 * -1.5).cpu().numpy())

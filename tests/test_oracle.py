@@ -69,6 +69,12 @@ def test_gemm_beta_semantics():
     # k == 0: C = beta * C
     C0 = rng.random((5, 4))
     assert np.allclose(oracle.gemm(np.zeros((5, 0)), np.zeros((0, 4)), C0, beta=2.0), 2 * C0)
+    # alpha == 0: A and B are not referenced (the BLAS definition), so their NaNs stay out of C
+    An = A.copy()
+    An[2, 3] = np.nan
+    assert np.array_equal(oracle.gemm(An, B, C0, alpha=0.0, beta=2.0, variant="blas"), 2 * C0)
+    assert np.array_equal(oracle.gemm(An, B, nan, alpha=0.0, beta=0.0, variant="blas"), np.zeros((5, 4)))
+    assert np.isnan(oracle.gemm(An, B, C0, alpha=1e-300, beta=2.0, variant="blas")[2]).all()
 
 
 def test_bf16_conversion_matches_torch_exhaustively_on_a_sweep():
