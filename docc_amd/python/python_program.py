@@ -195,6 +195,26 @@ class _Lowering(ast.NodeVisitor):
             out = self.new_array([m, n], left.elem, dest)
             self.b.add_gemm(left.name, right.name, out.name, alpha, beta, m, n, k, ta, tb, left.shape[1], right.shape[1], n)
             return out
+        # vectors, numpy's rules: matrix @ vector and vector @ matrix are GEMMs with one column / one row, the result
+        # loses that axis; vector @ vector is the sum of the products
+        if len(left.shape) == 2 and len(right.shape) == 1 and not tb:
+            m, k = (left.shape[1], left.shape[0]) if ta else left.shape
+            if k != right.shape[0]:
+                raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({k} vs {right.shape[0]})")
+            out = self.new_array([m], left.elem, dest)
+            self.b.add_gemm(left.name, right.name, out.name, alpha, beta, m, "1", k, ta, False, left.shape[1], "1", "1")
+            return out
+        if len(left.shape) == 1 and len(right.shape) == 2 and not ta:
+            k2, n = (right.shape[1], right.shape[0]) if tb else right.shape
+            if left.shape[0] != k2:
+                raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({left.shape[0]} vs {k2})")
+            out = self.new_array([n], left.elem, dest)
+            self.b.add_gemm(left.name, right.name, out.name, alpha, beta, "1", n, left.shape[0], False, tb, left.shape[0], right.shape[1], n)
+            return out
+        if len(left.shape) == 1 and len(right.shape) == 1 and not (ta or tb) and alpha == "1.0" and beta == "0.0":
+            if left.shape[0] != right.shape[0]:
+                raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({left.shape[0]} vs {right.shape[0]})")
+            return self.reduce(node, "sum", self.elementwise(node, "mul", left, right, None), None, False, dest)
         if ta or tb or alpha != "1.0" or beta != "0.0":
             self.fail(node, "a scaled or transposed batched product")
         if len(left.shape) < 2 or len(right.shape) < 2 or (len(right.shape) > 2 and right.shape[:-2] != left.shape[:-2]):

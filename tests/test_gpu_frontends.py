@@ -487,3 +487,18 @@ def test_casts_through_both_front_ends():
     assert out.dtype == torch.float32
     ref = oracle.attention(bits(q.bfloat16()), bits(k.bfloat16()), bits(v.bfloat16()))
     assert rel_err_max(out.numpy(), ref) <= 2e-2
+
+
+def test_products_with_vectors_follow_numpy():
+    @native(target="rocm")
+    def products(a, x, y):
+        return a @ x, y @ a, x @ x, a.T @ y
+
+    rng = np.random.default_rng(2)
+    a, x, y = rng.standard_normal((300, 200)), rng.standard_normal(200), rng.standard_normal(300)
+    ax, ya, xx, aty = products(a, x, y)
+    assert ax.shape == (300,) and ya.shape == (200,) and aty.shape == (200,) and np.ndim(xx) == 0
+    assert rel_err_max(ax, a @ x) <= 1e-12 and rel_err_max(ya, y @ a) <= 1e-12 and rel_err_max(aty, a.T @ y) <= 1e-12      # the fp64 GEMM bar
+    np.testing.assert_allclose(xx, x @ x, rtol=1e-13)
+    codes = [n["code"] for n in products.last_sdfg.library_nodes() if not n["code"].startswith("ROCM")]
+    assert codes == ["GEMM", "GEMM", "ml::Mul", "ml::Sum", "GEMM"]
