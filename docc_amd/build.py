@@ -49,6 +49,7 @@ KERNEL_FAMILIES = {
     "elementwise": "elementwise.hip",
     "reduce": "reduce.hip",
     "transpose": "transpose.hip",
+    "gemv": "gemv.hip",
 }
 
 # Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary

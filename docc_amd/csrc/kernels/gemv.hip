@@ -1,0 +1,135 @@
+// Matrix-vector forms of the GEMM node for gfx950: a product with one output column or one output row moves
+// the matrix once and computes two flops per element, so it is HBM-bound (4 or 8 bytes per element) and the
+// MFMA tiles of the GEMM kernels - built for 64 and more columns - would idle. Two kernels cover the four
+// cases (C = alpha * op(A) op(B) + beta * C with n == 1 or m == 1, either operand transposed or not):
+//   rows   y[i] = alpha * <M[i, :], x> + beta * y[i]      the matrix's rows are contiguous: one wavefront per row,
+//          128-bit loads, the vector comes from the caches;
+//   cols   y[j] = alpha * sum_p x[p] * M[p, j] + beta * y[j]   a lane owns columns (contiguous across lanes), the
+//          rows are cut into slices over work-groups whose partial sums meet in a scratch array; a second
+//          launch adds them in slice order, so the result does not depend on scheduling.
+// fp32 sums in fp32, fp64 in fp64 (cblas_?gemm semantics, reference gemm_node.cpp:474-505); when beta == 0, y
+// is not read.
+#include "common.h"
+
+namespace docc_k {
+
+constexpr long kGemvScratchBytes = 8l << 20;
+__device__ __attribute__((aligned(256))) unsigned char docc_gemv_scratch[kGemvScratchBytes];
+
+template <typename T>
+__device__ __forceinline__ T gemv_wave_sum(T v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// VEC elements per load when the launcher found rows and vector aligned, else 1
+template <typename T, int VEC>
+__device__ __forceinline__ void gemv_rows(const T* __restrict__ M, long ld, const T* __restrict__ x, long incx, T* __restrict__ y, long incy,
+                                          long rows, long k, T alpha, T beta) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    const int lane = threadIdx.x & 63;
+    const long row = (long) blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* m = M + row * ld;
+    T acc = (T) 0;
+    if (VEC > 1) {
+        const long nv = k / VEC;
+        const V* mv = reinterpret_cast<const V*>(m);
+        const V* xv = reinterpret_cast<const V*>(x);
+        for (long c = lane; c < nv; c += 64) {
+            const V a = __builtin_nontemporal_load(mv + c);
+            const V b = xv[c];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) acc += a[e] * b[e];
+        }
+        for (long c = nv * VEC + lane; c < k; c += 64) acc += m[c] * x[c];
+    } else {
+        for (long c = lane; c < k; c += 64) acc += m[c] * x[c * incx];
+    }
+    acc = gemv_wave_sum(acc);
+    if (lane == 0) {
+        T* out = y + row * incy;
+        *out = beta == (T) 0 ? alpha * acc : __builtin_fma(beta, *out, alpha * acc);
+    }
+}
+
+// partial sums of rows [slice * chunk, ...) for VEC columns per lane; P[slice][col]
+template <typename T, int VEC>
+__device__ __forceinline__ void gemv_cols_partial(const T* __restrict__ M, long ld, const T* __restrict__ x, long incx, long rows, long cols,
+                                                  long chunk) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    T* P = reinterpret_cast<T*>(docc_gemv_scratch);
+    const long col = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (col >= cols) return;
+    const long r0 = (long) blockIdx.y * chunk;
+    const long r1 = r0 + chunk < rows ? r0 + chunk : rows;
+    T acc[VEC], acc1[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[e] = acc1[e] = (T) 0;
+    long r = r0;
+    if (VEC > 1) {
+        for (; r + 2 <= r1; r += 2) {   // two independent chains keep the loads in flight
+            const V a0 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + r * ld + col));
+            const V a1 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + (r + 1) * ld + col));
+            const T w0 = x[r * incx], w1 = x[(r + 1) * incx];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                acc[e] += w0 * a0[e];
+                acc1[e] += w1 * a1[e];
+            }
+        }
+    }
+    for (; r < r1; r++) {
+        const T w = x[r * incx];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] += w * M[r * ld + col + e];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; e++) P[(long) blockIdx.y * cols + col + e] = acc[e] + acc1[e];
+}
+
+template <typename T>
+__device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, long cols, int slices, T alpha, T beta) {
+    // a work-group takes 16 neighbouring columns; 16 lanes per column each add every 16th slice, then one lane
+    // adds the 16 sums in order: the order of the additions is fixed by the launch geometry alone
+    __shared__ T part[16][17];
+    const T* P = reinterpret_cast<const T*>(docc_gemv_scratch);
+    const int c = threadIdx.x & 15, g = threadIdx.x >> 4;
+    const long col = (long) blockIdx.x * 16 + c;
+    T acc = (T) 0;
+    if (col < cols)
+        for (long s = g; s < slices; s += 16) acc += P[s * cols + col];
+    part[g][c] = acc;
+    __syncthreads();
+    if (g == 0 && col < cols) {
+        T r = part[0][c];
+#pragma unroll
+        for (int i = 1; i < 16; i++) r += part[i][c];
+        T* out = y + col * incy;
+        *out = beta == (T) 0 ? alpha * r : __builtin_fma(beta, *out, alpha * r);
+    }
+}
+
+} // namespace docc_k
+
+#define DOCC_GEMV(NAME, T, VEC)                                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_rows_##NAME##_v##VEC(const T* M, long ld, const T* x, long incx, T* y,   \
+                                                                                     long incy, long rows, long k, T alpha, T beta) { \
+        docc_k::gemv_rows<T, VEC>(M, ld, x, incx, y, incy, rows, k, alpha, beta);                                                      \
+    }                                                                                                                                 \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colp_##NAME##_v##VEC(const T* M, long ld, const T* x, long incx,        \
+                                                                                     long rows, long cols, long chunk) {              \
+        docc_k::gemv_cols_partial<T, VEC>(M, ld, x, incx, rows, cols, chunk);                                                          \
+    }
+DOCC_GEMV(f32, float, 4)
+DOCC_GEMV(f32, float, 1)
+DOCC_GEMV(f64, double, 2)
+DOCC_GEMV(f64, double, 1)
+
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f32(float* y, long incy, long cols, int slices, float alpha, float beta) {
+    docc_k::gemv_cols_final<float>(y, incy, cols, slices, alpha, beta);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f64(double* y, long incy, long cols, int slices, double alpha, double beta) {
+    docc_k::gemv_cols_final<double>(y, incy, cols, slices, alpha, beta);
+}

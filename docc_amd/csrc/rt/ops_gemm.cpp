@@ -1,5 +1,6 @@
 // Launchers for the GEMM node kernels (see include/docc_rocm_ops.h).
 #include <cstdio>
+#include <type_traits>
 #include <cstdlib>
 #include <cstring>
 
@@ -25,6 +26,62 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
     const size_t a_elems = (size_t) (a_kc ? c.bm : c.bk) * lda_s;
     const size_t b_elems = (size_t) (b_kc ? c.bn : c.bk) * ldb_s;
     return 2 * (a_elems + b_elems) * elem;
+}
+
+// One output column or one output row: the matrix-vector kernels (csrc/kernels/gemv.hip). Returns 1 when the
+// shape is not one of theirs (the caller goes on to the tiled kernels), 0 or an error code otherwise.
+template <typename S>
+int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, int64_t n, int64_t k, S alpha, const S* A, int64_t lda,
+                const S* B, int64_t ldb, S beta, S* C, int64_t ldc) {
+    if (std::getenv("DOCC_ROCM_GEMV_OFF")) return 1;   // tuning and tests: always the tiled kernels
+    const S *M, *x;
+    int64_t ld, incx, incy, rows, cols;
+    bool by_rows;
+    if (n == 1) {          // y = op(A) b: A as stored is [m][k] (rows form) or [k][m] (columns form)
+        M = A, ld = lda, x = B, incx = tb ? 1 : ldb, incy = ldc;
+        by_rows = !ta;
+        rows = ta ? k : m, cols = ta ? m : k;
+    } else if (m == 1) {   // y = a op(B): B as stored is [n][k] (rows form) or [k][n] (columns form)
+        M = B, ld = ldb, x = A, incx = ta ? lda : 1, incy = 1;
+        by_rows = tb;
+        rows = tb ? n : k, cols = tb ? k : n;
+    } else {
+        return 1;
+    }
+    const int bits = (int) sizeof(S) * 8, vec = 16 / (int) sizeof(S);
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    char name[64];
+    if (by_rows) {
+        // one wavefront per row: worth it from a few rows per SIMD on
+        if (rows < 4 * (int64_t) cus) return 1;
+        if ((rows + 3) / 4 > 0x7fffffffLL) return 1;
+        const bool aligned = incx == 1 && ((uintptr_t) M | (uintptr_t) x) % 16 == 0 && ld % vec == 0;
+        std::snprintf(name, sizeof(name), "docc_gemv_rows_f%d_v%d", bits, aligned ? vec : 1);
+        return launch(name, (uint32_t) ((rows + 3) / 4), 1, 1, 256, 0, s, M, (long) ld, x, (long) incx, C, (long) incy, (long) rows,
+                      (long) cols, alpha, beta);
+    }
+    // columns form: lanes own columns, the rows are sliced so that about eight work-groups per CU share the matrix;
+    // the slices' sums meet in the kernels' 8 MiB scratch array
+    if (cols < 256 || rows < 64) return 1;
+    const bool aligned = (uintptr_t) M % 16 == 0 && ld % vec == 0 && cols % vec == 0;
+    const int lanes = aligned ? vec : 1;
+    const int64_t col_blocks = (cols / lanes + 255) / 256;
+    int64_t slices = (8 * (int64_t) cus + col_blocks - 1) / col_blocks;
+    if (slices > rows / 16) slices = rows / 16;
+    const int64_t fit = (int64_t(8) << 20) / ((int64_t) sizeof(S) * cols);
+    if (slices > fit) slices = fit;
+    if (slices > 256) slices = 256;
+    if (slices < 1) return 1;
+    const int64_t chunk = (rows + slices - 1) / slices;
+    slices = (rows + chunk - 1) / chunk;
+    if (col_blocks > 0x7fffffffLL || slices > 65535) return 1;
+    std::snprintf(name, sizeof(name), "docc_gemv_colp_f%d_v%d", bits, lanes);
+    int rc = launch(name, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, M, (long) ld, x, (long) incx, (long) rows, (long) cols,
+                    (long) chunk);
+    if (rc) return rc;
+    std::snprintf(name, sizeof(name), "docc_gemv_colf_f%d", bits);
+    return launch(name, (uint32_t) ((cols + 15) / 16), 1, 1, 256, 0, s, C, (long) incy, (long) cols, (int) slices, alpha, beta);
 }
 
 // T: element type of A and B; S: type of C, alpha and beta
@@ -69,6 +126,12 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         const int post[1] = {activation};
         return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
                                            bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
+    }
+    if constexpr (std::is_same<T, S>::value) {
+        if ((m == 1 || n == 1) && batch == 1 && !bias && activation < 0) {
+            rc = gemv_launch<S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+            if (rc != 1) return rc;
+        }
     }
     const size_t vec = 16 / sizeof(T);
     // the aligned kernels read whole 128-bit vectors: pointers, leading dimensions and the

@@ -42,6 +42,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_elementwise.hsaco",
     "docc_rocm_reduce.hsaco",
     "docc_rocm_transpose.hsaco",
+    "docc_rocm_gemv.hsaco",
 };
 
 struct DeviceState {

@@ -260,3 +260,35 @@ def test_gemm_alpha_zero_does_not_reference_a_and_b(rt, kind):
     want = oracle.gemm(np.full((m, k), np.nan, np.float64 if kind == "d" else np.float32), np.full((k, n), np.nan, np.float64 if kind == "d" else np.float32),
                        c0.cpu().numpy(), alpha=0.0, beta=-1.5)
     assert np.array_equal(want, (c0 * -1.5).cpu().numpy())
+
+
+GEMV_CASES = [  # m, n, k, ta, tb: one output column or row, each operand layout; sizes that take the matrix-vector kernels
+    (3000, 1, 700, N, N), (3000, 1, 701, N, T), (2048, 1, 1024, T, N), (1500, 1, 333, T, T),
+    (1, 3000, 700, N, N), (1, 2048, 1024, N, T), (1, 1501, 333, T, N), (1, 4096, 96, T, T),
+    (5000, 1, 8, N, N), (1, 300, 5000, N, N),
+]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("case", GEMV_CASES, ids=[f"{c[0]}x{c[1]}x{c[2]}" + "nt"[c[3] == T] + "nt"[c[4] == T] for c in GEMV_CASES])
+def test_gemm_with_one_column_or_one_row(rt, monkeypatch, dt, case):
+    """The matrix-vector kernels behind the GEMM entry points: integer-valued operands give the oracle's integers
+    (any summation order), random ones stay within the GEMM bars; the tiled kernels (DOCC_ROCM_GEMV_OFF) agree."""
+    m, n, k, ta, tb = case
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    A = int_matrix(rng, (k, m) if ta == T else (m, k), dt, lim=4)
+    B = int_matrix(rng, (n, k) if tb == T else (k, n), dt, lim=4)
+    C0 = int_matrix(rng, (m, n), dt, lim=4)
+    for alpha, beta in ((1.0, 0.0), (2.0, -1.0)):
+        want = oracle.gemm(A, B, C0, alpha=alpha, beta=beta, trans_a=ta, trans_b=tb)
+        assert np.array_equal(run_gemm(rt, A, B, C0, alpha, beta, ta=ta, tb=tb), want), (alpha, beta)
+    # padded leading dimensions and unaligned operands take the scalar variants
+    padded = run_gemm(rt, A, B, C0, 2.0, -1.0, ta=ta, tb=tb, lda=A.shape[1] + 3, ldb=B.shape[1] + 5, ldc=n + 2, offset=1)
+    assert np.array_equal(padded, oracle.gemm(A, B, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb))
+    Ar, Br = rng.standard_normal(A.shape).astype(dt), rng.standard_normal(B.shape).astype(dt)
+    got = run_gemm(rt, Ar, Br, C0, 1.5, 0.5, ta=ta, tb=tb)
+    ref = oracle.gemm(Ar, Br, C0, alpha=1.5, beta=0.5, trans_a=ta, trans_b=tb, variant="ld" if dt == np.float64 else "acc64")
+    assert rel_err_max(got, ref) <= (1e-12 if dt == np.float64 else 1e-5)
+    monkeypatch.setenv("DOCC_ROCM_GEMV_OFF", "1")
+    tiled = run_gemm(rt, Ar, Br, C0, 1.5, 0.5, ta=ta, tb=tb)
+    assert rel_err_max(tiled, ref) <= (1e-12 if dt == np.float64 else 1e-5)
