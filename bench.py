@@ -230,6 +230,17 @@ def main():
                                                       bias.data_ptr(), "relu", stream=stream), 20, 3)
         add_kernel("sgemm_4096_bias_relu", "f32", 2 * n**3, ms_e)
         del A, B, Cm, bias
+        # one output column / one output row: the matrix-vector kernels, HBM-bound (the matrix moves once)
+        nv = 8192
+        Mx, xv, yv = torch.randn(nv, nv, device="cuda"), torch.randn(nv, device="cuda"), torch.empty(nv, device="cuda")
+        for name, call in (("sgemv_8192x8192_rows", lambda i: rt.sgemm(nv, 1, nv, 1.0, Mx.data_ptr(), nv, xv.data_ptr(), 1, 0.0, yv.data_ptr(), 1, stream=stream)),
+                           ("sgemv_8192x8192_columns", lambda i: rt.sgemm(1, nv, nv, 1.0, xv.data_ptr(), nv, Mx.data_ptr(), nv, 0.0, yv.data_ptr(), nv, stream=stream))):
+            ms_v = time_kernel(call, 50, 5)
+            nbytes_v = 4 * (nv * nv + 2 * nv)
+            kernels[name] = {"kernel_us": round(ms_v * 1e3, 2), "dtype": "f32",
+                             "roofline": {"bound": "hbm", "achieved": round(nbytes_v / ms_v / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                          "frac": round(nbytes_v / ms_v / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_v}}
+        del Mx, xv, yv
 
     # ---- config 3b: bf16 GEMM 4096^3, fp32 accumulate/output ------------------------------
     if want("bgemm"):
