@@ -7,8 +7,8 @@
 //   cols   y[j] = alpha * sum_p x[p] * M[p, j] + beta * y[j]   a lane owns columns (contiguous across lanes), the
 //          rows are cut into slices over work-groups whose partial sums meet in a scratch array; a second
 //          launch adds them in slice order, so the result does not depend on scheduling.
-// fp32 sums in fp32, fp64 in fp64 (cblas_?gemm semantics, reference gemm_node.cpp:474-505); when beta == 0, y
-// is not read.
+// fp32 sums in fp32, fp64 in fp64 (cblas_?gemm semantics, reference gemm_node.cpp:474-505), bf16 operands (raw
+// 16-bit words) in fp32 with an fp32 result, like the bf16 GEMM; when beta == 0, y is not read.
 #include "common.h"
 
 namespace docc_k {
@@ -23,15 +23,20 @@ __device__ __forceinline__ T gemv_wave_sum(T v) {
     return v;
 }
 
+// element as stored -> the type the sums run in
+template <typename T, typename In> __device__ __forceinline__ T gemv_value(In v) { return (T) v; }
+template <> __device__ __forceinline__ float gemv_value<float, unsigned short>(unsigned short v) { return bf16_bits_to_f32(v); }
+
+// In: element type of the matrix and the vector, T: type of the sums and of y.
 // VEC elements per load when the launcher found rows and vector aligned, else 1
-template <typename T, int VEC>
-__device__ __forceinline__ void gemv_rows(const T* __restrict__ M, long ld, const T* __restrict__ x, long incx, T* __restrict__ y, long incy,
+template <typename In, typename T, int VEC>
+__device__ __forceinline__ void gemv_rows(const In* __restrict__ M, long ld, const In* __restrict__ x, long incx, T* __restrict__ y, long incy,
                                           long rows, long k, T alpha, T beta) {
-    typedef T V __attribute__((ext_vector_type(VEC)));
+    typedef In V __attribute__((ext_vector_type(VEC)));
     const int lane = threadIdx.x & 63;
     const long row = (long) blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= rows) return;
-    const T* m = M + row * ld;
+    const In* m = M + row * ld;
     T acc = (T) 0;
     if (VEC > 1) {
         const long nv = k / VEC;
@@ -41,11 +46,11 @@ __device__ __forceinline__ void gemv_rows(const T* __restrict__ M, long ld, cons
             const V a = __builtin_nontemporal_load(mv + c);
             const V b = xv[c];
 #pragma unroll
-            for (int e = 0; e < VEC; e++) acc += a[e] * b[e];
+            for (int e = 0; e < VEC; e++) acc += gemv_value<T, In>(a[e]) * gemv_value<T, In>(b[e]);
         }
-        for (long c = nv * VEC + lane; c < k; c += 64) acc += m[c] * x[c];
+        for (long c = nv * VEC + lane; c < k; c += 64) acc += gemv_value<T, In>(m[c]) * gemv_value<T, In>(x[c]);
     } else {
-        for (long c = lane; c < k; c += 64) acc += m[c] * x[c * incx];
+        for (long c = lane; c < k; c += 64) acc += gemv_value<T, In>(m[c]) * gemv_value<T, In>(x[c * incx]);
     }
     acc = gemv_wave_sum(acc);
     if (lane == 0) {
@@ -55,10 +60,10 @@ __device__ __forceinline__ void gemv_rows(const T* __restrict__ M, long ld, cons
 }
 
 // partial sums of rows [slice * chunk, ...) for VEC columns per lane; P[slice][col]
-template <typename T, int VEC>
-__device__ __forceinline__ void gemv_cols_partial(const T* __restrict__ M, long ld, const T* __restrict__ x, long incx, long rows, long cols,
+template <typename In, typename T, int VEC>
+__device__ __forceinline__ void gemv_cols_partial(const In* __restrict__ M, long ld, const In* __restrict__ x, long incx, long rows, long cols,
                                                   long chunk) {
-    typedef T V __attribute__((ext_vector_type(VEC)));
+    typedef In V __attribute__((ext_vector_type(VEC)));
     T* P = reinterpret_cast<T*>(docc_gemv_scratch);
     const long col = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
     if (col >= cols) return;
@@ -72,18 +77,18 @@ __device__ __forceinline__ void gemv_cols_partial(const T* __restrict__ M, long 
         for (; r + 2 <= r1; r += 2) {   // two independent chains keep the loads in flight
             const V a0 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + r * ld + col));
             const V a1 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + (r + 1) * ld + col));
-            const T w0 = x[r * incx], w1 = x[(r + 1) * incx];
+            const T w0 = gemv_value<T, In>(x[r * incx]), w1 = gemv_value<T, In>(x[(r + 1) * incx]);
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
-                acc[e] += w0 * a0[e];
-                acc1[e] += w1 * a1[e];
+                acc[e] += w0 * gemv_value<T, In>(a0[e]);
+                acc1[e] += w1 * gemv_value<T, In>(a1[e]);
             }
         }
     }
     for (; r < r1; r++) {
-        const T w = x[r * incx];
+        const T w = gemv_value<T, In>(x[r * incx]);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) acc[e] += w * M[r * ld + col + e];
+        for (int e = 0; e < VEC; e++) acc[e] += w * gemv_value<T, In>(M[r * ld + col + e]);
     }
 #pragma unroll
     for (int e = 0; e < VEC; e++) P[(long) blockIdx.y * cols + col + e] = acc[e] + acc1[e];
@@ -113,19 +118,21 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
 
 } // namespace docc_k
 
-#define DOCC_GEMV(NAME, T, VEC)                                                                                                       \
-    extern "C" __global__ __launch_bounds__(256) void docc_gemv_rows_##NAME##_v##VEC(const T* M, long ld, const T* x, long incx, T* y,   \
+#define DOCC_GEMV(NAME, In, T, VEC)                                                                                                   \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_rows_##NAME##_v##VEC(const In* M, long ld, const In* x, long incx, T* y, \
                                                                                      long incy, long rows, long k, T alpha, T beta) { \
-        docc_k::gemv_rows<T, VEC>(M, ld, x, incx, y, incy, rows, k, alpha, beta);                                                      \
+        docc_k::gemv_rows<In, T, VEC>(M, ld, x, incx, y, incy, rows, k, alpha, beta);                                                  \
     }                                                                                                                                 \
-    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colp_##NAME##_v##VEC(const T* M, long ld, const T* x, long incx,        \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colp_##NAME##_v##VEC(const In* M, long ld, const In* x, long incx,      \
                                                                                      long rows, long cols, long chunk) {              \
-        docc_k::gemv_cols_partial<T, VEC>(M, ld, x, incx, rows, cols, chunk);                                                          \
+        docc_k::gemv_cols_partial<In, T, VEC>(M, ld, x, incx, rows, cols, chunk);                                                      \
     }
-DOCC_GEMV(f32, float, 4)
-DOCC_GEMV(f32, float, 1)
-DOCC_GEMV(f64, double, 2)
-DOCC_GEMV(f64, double, 1)
+DOCC_GEMV(f32, float, float, 4)
+DOCC_GEMV(f32, float, float, 1)
+DOCC_GEMV(f64, double, double, 2)
+DOCC_GEMV(f64, double, double, 1)
+DOCC_GEMV(bf16, unsigned short, float, 8)
+DOCC_GEMV(bf16, unsigned short, float, 1)
 
 extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f32(float* y, long incy, long cols, int slices, float alpha, float beta) {
     docc_k::gemv_cols_final<float>(y, incy, cols, slices, alpha, beta);

@@ -30,11 +30,11 @@ size_t gemm_lds_bytes(const TileConfig& c, bool ta, bool tb, size_t elem) {
 
 // One output column or one output row: the matrix-vector kernels (csrc/kernels/gemv.hip). Returns 1 when the
 // shape is not one of theirs (the caller goes on to the tiled kernels), 0 or an error code otherwise.
-template <typename S>
-int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, int64_t n, int64_t k, S alpha, const S* A, int64_t lda,
-                const S* B, int64_t ldb, S beta, S* C, int64_t ldc) {
+template <typename T, typename S>
+int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, int64_t n, int64_t k, S alpha, const T* A, int64_t lda,
+                const T* B, int64_t ldb, S beta, S* C, int64_t ldc) {
     if (std::getenv("DOCC_ROCM_GEMV_OFF")) return 1;   // tuning and tests: always the tiled kernels
-    const S *M, *x;
+    const T *M, *x;
     int64_t ld, incx, incy, rows, cols;
     bool by_rows;
     if (n == 1) {          // y = op(A) b: A as stored is [m][k] (rows form) or [k][m] (columns form)
@@ -48,7 +48,9 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
     } else {
         return 1;
     }
-    const int bits = (int) sizeof(S) * 8, vec = 16 / (int) sizeof(S);
+    const int vec = 16 / (int) sizeof(T);
+    const char* type = sizeof(T) == 2 ? "bf16" : sizeof(T) == 4 ? "f32" : "f64";   // elements of the matrix
+    const int bits = (int) sizeof(S) * 8;                                        // of the sums and of y
     int cus = compute_units();
     if (cus <= 0) cus = 256;
     char name[64];
@@ -57,7 +59,7 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         if (rows < 4 * (int64_t) cus) return 1;
         if ((rows + 3) / 4 > 0x7fffffffLL) return 1;
         const bool aligned = incx == 1 && ((uintptr_t) M | (uintptr_t) x) % 16 == 0 && ld % vec == 0;
-        std::snprintf(name, sizeof(name), "docc_gemv_rows_f%d_v%d", bits, aligned ? vec : 1);
+        std::snprintf(name, sizeof(name), "docc_gemv_rows_%s_v%d", type, aligned ? vec : 1);
         return launch(name, (uint32_t) ((rows + 3) / 4), 1, 1, 256, 0, s, M, (long) ld, x, (long) incx, C, (long) incy, (long) rows,
                       (long) cols, alpha, beta);
     }
@@ -76,7 +78,7 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
     const int64_t chunk = (rows + slices - 1) / slices;
     slices = (rows + chunk - 1) / chunk;
     if (col_blocks > 0x7fffffffLL || slices > 65535) return 1;
-    std::snprintf(name, sizeof(name), "docc_gemv_colp_f%d_v%d", bits, lanes);
+    std::snprintf(name, sizeof(name), "docc_gemv_colp_%s_v%d", type, lanes);
     int rc = launch(name, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, M, (long) ld, x, (long) incx, (long) rows, (long) cols,
                     (long) chunk);
     if (rc) return rc;
@@ -127,11 +129,9 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
                                            bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
     }
-    if constexpr (std::is_same<T, S>::value) {
-        if ((m == 1 || n == 1) && batch == 1 && !bias && activation < 0) {
-            rc = gemv_launch<S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
-            if (rc != 1) return rc;
-        }
+    if ((m == 1 || n == 1) && batch == 1 && !bias && activation < 0) {
+        rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        if (rc != 1) return rc;
     }
     const size_t vec = 16 / sizeof(T);
     // the aligned kernels read whole 128-bit vectors: pointers, leading dimensions and the

@@ -43,8 +43,8 @@ extern "C" {
  * Replaces cblas_dgemm / cblas_sgemm as printed by GEMMNodeDispatcher_BLAS
  * (reference gemm_node.cpp:474-505) and cublasDgemm / cublasSgemm
  * (reference opt/src/targets/cuda/blas/gemm.cpp:131-185).
- * Zero-sized m, n: nothing is done; k == 0: C = beta * C. fp32 / fp64 products with one output
- * column or row run as matrix-vector kernels (HBM-bound); their partial sums may pass through a
+ * Zero-sized m, n: nothing is done; k == 0: C = beta * C. Products with one output
+ * column or row (bf16 ones too) run as matrix-vector kernels (HBM-bound); their partial sums may pass through a
  * scratch array in the kernel image: do not overlap such calls on different streams.
  */
 int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,

@@ -130,3 +130,27 @@ def test_bgemm_every_tile_configuration(rt, cfg):
                     assert np.array_equal(out, ref), (cfg, m, n, k, ta, tb)
     finally:
         os.environ.pop("DOCC_ROCM_GEMM_CFG", None)
+
+
+BGEMV_CASES = [(3000, 1, 704, N, N), (3000, 1, 701, N, T), (2048, 1, 1024, T, N), (1504, 1, 333, T, T),
+               (1, 3000, 700, N, N), (1, 2048, 1024, N, T), (1, 1501, 333, T, N), (1, 4096, 96, T, T)]
+
+
+@pytest.mark.parametrize("case", BGEMV_CASES, ids=[f"{c[0]}x{c[1]}x{c[2]}" + "nt"[c[3] == T] + "nt"[c[4] == T] for c in BGEMV_CASES])
+def test_bgemm_with_one_column_or_one_row(rt, monkeypatch, case):
+    """bf16 products with one output column or row take the matrix-vector kernels (a decoder's x W): integer
+    values give the oracle's integers, random ones stay within the bf16 bar, the tiled kernels agree."""
+    m, n, k, ta, tb = case
+    rng = np.random.default_rng(m + 31 * n + 977 * k)
+    A = rng.integers(-8, 9, (k, m) if ta == T else (m, k)).astype(np.float32)
+    B = rng.integers(-8, 9, (n, k) if tb == T else (k, n)).astype(np.float32)
+    C0 = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+    for alpha, beta in ((1.0, 0.0), (2.0, -1.0)):
+        got = run_bgemm(rt, Ab, Bb, C0, alpha, beta, ta=ta, tb=tb)
+        assert np.array_equal(got, oracle.gemm_bf16(Ab, Bb, C0, alpha=alpha, beta=beta, trans_a=ta, trans_b=tb)), (alpha, beta)
+    Ar, Br = oracle.f32_to_bf16(rng.standard_normal(A.shape).astype(np.float32)), oracle.f32_to_bf16(rng.standard_normal(B.shape).astype(np.float32))
+    ref = oracle.gemm_bf16(Ar, Br, trans_a=ta, trans_b=tb)
+    assert rel_err_max(run_bgemm(rt, Ar, Br, ta=ta, tb=tb), ref) <= 1e-5      # fp32 sums of exact products: far inside 2e-2
+    monkeypatch.setenv("DOCC_ROCM_GEMV_OFF", "1")
+    assert rel_err_max(run_bgemm(rt, Ar, Br, ta=ta, tb=tb), ref) <= 1e-5
