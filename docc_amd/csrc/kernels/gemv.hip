@@ -59,6 +59,68 @@ __device__ __forceinline__ void gemv_rows(const In* __restrict__ M, long ld, con
     }
 }
 
+// A few vectors at once (a small batch against a weight matrix whose rows are contiguous, y = x W^T):
+// y[row * sy_row + v * sy_vec] = alpha * <M[row, :], X[v, :]> + beta * y[..] for v < nv <= NV. The matrix still
+// moves once; the vectors (nv * k elements) come from the caches.
+template <typename In, typename T, int VEC, int NV>
+__device__ __forceinline__ void gemv_rows_multi(const In* __restrict__ M, long ld, const In* __restrict__ X, long ldx, int nv, T* __restrict__ y,
+                                                long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {
+    typedef In V __attribute__((ext_vector_type(VEC)));
+    constexpr int RW = 4;   // matrix rows per wavefront: a piece of the vectors is loaded once for four rows
+    const int lane = threadIdx.x & 63;
+    const long row0 = ((long) blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
+    if (row0 >= rows) return;
+    const In* m[RW];
+#pragma unroll
+    for (int r = 0; r < RW; r++) m[r] = M + (row0 + r < rows ? row0 + r : rows - 1) * ld;   // rows past the end repeat the last one
+    T acc[RW][NV];
+#pragma unroll
+    for (int r = 0; r < RW; r++)
+#pragma unroll
+        for (int v = 0; v < NV; v++) acc[r][v] = (T) 0;
+    const long nvec = VEC > 1 ? k / VEC : 0;
+    for (long c = lane; c < nvec; c += 64) {
+        V a[RW];
+#pragma unroll
+        for (int r = 0; r < RW; r++) a[r] = __builtin_nontemporal_load(reinterpret_cast<const V*>(m[r]) + c);
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            if (v < nv) {
+                const V b = reinterpret_cast<const V*>(X + v * ldx)[c];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
+                    const T bv = gemv_value<T, In>(b[e]);
+#pragma unroll
+                    for (int r = 0; r < RW; r++) acc[r][v] += gemv_value<T, In>(a[r][e]) * bv;
+                }
+            }
+        }
+    }
+    for (long c = nvec * VEC + lane; c < k; c += 64) {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            if (v < nv) {
+                const T bv = gemv_value<T, In>(X[v * ldx + c]);
+#pragma unroll
+                for (int r = 0; r < RW; r++) acc[r][v] += gemv_value<T, In>(m[r][c]) * bv;
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < RW; r++) {
+#pragma unroll
+        for (int v = 0; v < NV; v++) {
+            if (v < nv) {
+                const T sum = gemv_wave_sum(acc[r][v]);
+                if (lane == 0 && row0 + r < rows) {
+                    T* out = y + (row0 + r) * sy_row + v * sy_vec;
+                    *out = beta == (T) 0 ? alpha * sum : __builtin_fma(beta, *out, alpha * sum);
+                }
+            }
+        }
+    }
+}
+
 // partial sums of rows [slice * chunk, ...) for VEC columns per lane; P[slice][col]
 template <typename In, typename T, int VEC>
 __device__ __forceinline__ void gemv_cols_partial(const In* __restrict__ M, long ld, const In* __restrict__ x, long incx, long rows, long cols,
@@ -127,6 +189,20 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
                                                                                      long rows, long cols, long chunk) {              \
         docc_k::gemv_cols_partial<In, T, VEC>(M, ld, x, incx, rows, cols, chunk);                                                      \
     }
+#define DOCC_GEMV_MULTI(NAME, In, T, VEC, NV)                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_rowsm_##NAME##_v##VEC##_n##NV(                                          \
+        const In* M, long ld, const In* X, long ldx, int nv, T* y, long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {     \
+        docc_k::gemv_rows_multi<In, T, VEC, NV>(M, ld, X, ldx, nv, y, sy_row, sy_vec, rows, k, alpha, beta);                            \
+    }
+#define DOCC_GEMV_MULTI_ALL(NAME, In, T, VEC) \
+    DOCC_GEMV_MULTI(NAME, In, T, VEC, 2) DOCC_GEMV_MULTI(NAME, In, T, VEC, 4) DOCC_GEMV_MULTI(NAME, In, T, VEC, 8)
+DOCC_GEMV_MULTI_ALL(f32, float, float, 4)
+DOCC_GEMV_MULTI_ALL(f32, float, float, 1)
+DOCC_GEMV_MULTI_ALL(f64, double, double, 2)
+DOCC_GEMV_MULTI_ALL(f64, double, double, 1)
+DOCC_GEMV_MULTI_ALL(bf16, unsigned short, float, 8)
+DOCC_GEMV_MULTI_ALL(bf16, unsigned short, float, 1)
+
 DOCC_GEMV(f32, float, float, 4)
 DOCC_GEMV(f32, float, float, 1)
 DOCC_GEMV(f64, double, double, 2)

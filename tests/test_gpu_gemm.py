@@ -266,6 +266,8 @@ GEMV_CASES = [  # m, n, k, ta, tb: one output column or row, each operand layout
     (3000, 1, 700, N, N), (3000, 1, 701, N, T), (2048, 1, 1024, T, N), (1500, 1, 333, T, T),
     (1, 3000, 700, N, N), (1, 2048, 1024, N, T), (1, 1501, 333, T, N), (1, 4096, 96, T, T),
     (5000, 1, 8, N, N), (1, 300, 5000, N, N),
+    # two to eight vectors against a matrix stored row by row along k (a small batch times W^T)
+    (4, 5000, 704, N, T), (8, 4200, 333, N, T), (5000, 2, 701, N, T), (4500, 7, 96, N, T), (3, 4099, 64, N, T),
 ]
 
 
