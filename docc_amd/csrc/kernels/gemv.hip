@@ -156,6 +156,82 @@ __device__ __forceinline__ void gemv_cols_partial(const In* __restrict__ M, long
     for (int e = 0; e < VEC; e++) P[(long) blockIdx.y * cols + col + e] = acc[e] + acc1[e];
 }
 
+// The columns form for a few vectors at once (a small batch times a weight matrix stored [k][n], y = x W):
+// P[slice][v][col] = sum over the slice's rows p of X[v * sx_v + p * sx_p] * M[p, col]; the matrix moves once.
+template <typename In, typename T, int VEC, int NV>
+__device__ __forceinline__ void gemv_cols_partial_multi(const In* __restrict__ M, long ld, const In* __restrict__ X, long sx_v, long sx_p, int nv,
+                                                        long rows, long cols, long chunk) {
+    typedef In V __attribute__((ext_vector_type(VEC)));
+    constexpr int STEP = 64;            // rows of the slice whose vector entries sit in LDS at a time
+    __shared__ T xs[STEP][NV];
+    T* P = reinterpret_cast<T*>(docc_gemv_scratch);
+    const long col = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
+    const bool live = col < cols;
+    const long r0 = (long) blockIdx.y * chunk;
+    const long r1 = r0 + chunk < rows ? r0 + chunk : rows;
+    T acc[NV][VEC];
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[v][e] = (T) 0;
+    for (long base = r0; base < r1; base += STEP) {
+        const int cnt = r1 - base < STEP ? (int) (r1 - base) : STEP;
+        __syncthreads();
+        for (int i = threadIdx.x; i < STEP * NV; i += 256) {
+            const int r = i / NV, v = i % NV;
+            xs[r][v] = (r < cnt && v < nv) ? gemv_value<T, In>(X[v * sx_v + (base + r) * sx_p]) : (T) 0;
+        }
+        __syncthreads();
+        if (!live) continue;
+#pragma unroll 4
+        for (int r = 0; r < cnt; r++) {
+            T a[VEC];
+            if (VEC > 1) {
+                const V av = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + (base + r) * ld + col));
+#pragma unroll
+                for (int e = 0; e < VEC; e++) a[e] = gemv_value<T, In>(av[e]);
+            } else {
+                a[0] = gemv_value<T, In>(M[(base + r) * ld + col]);
+            }
+#pragma unroll
+            for (int v = 0; v < NV; v++) {
+                const T w = xs[r][v];
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[v][e] += w * a[e];
+            }
+        }
+    }
+    if (!live) return;
+#pragma unroll
+    for (int v = 0; v < NV; v++)
+        if (v < nv)
+#pragma unroll
+            for (int e = 0; e < VEC; e++) P[((long) blockIdx.y * nv + v) * cols + col + e] = acc[v][e];
+}
+
+// y[v * sy_vec + col * sy_col] = alpha * (sum over the slices of P[s][v][col]) + beta * y[..]; entries = nv * cols
+template <typename T>
+__device__ __forceinline__ void gemv_cols_final_multi(T* __restrict__ y, long sy_vec, long sy_col, long cols, long entries, int slices, T alpha,
+                                                      T beta) {
+    // 64 neighbouring entries per work-group (256-byte segments of every slice), the slices dealt to its four waves
+    __shared__ T part[4][64];
+    const T* P = reinterpret_cast<const T*>(docc_gemv_scratch);
+    const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const long e = (long) blockIdx.x * 64 + c;
+    T acc = (T) 0;
+    if (e < entries) {
+#pragma unroll 4
+        for (long s = g; s < slices; s += 4) acc += P[s * entries + e];
+    }
+    part[g][c] = acc;
+    __syncthreads();
+    if (g == 0 && e < entries) {
+        const T r = (part[0][c] + part[1][c]) + (part[2][c] + part[3][c]);
+        T* out = y + (e / cols) * sy_vec + (e % cols) * sy_col;
+        *out = beta == (T) 0 ? alpha * r : __builtin_fma(beta, *out, alpha * r);
+    }
+}
+
 template <typename T>
 __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, long cols, int slices, T alpha, T beta) {
     // a work-group takes 16 neighbouring columns; 16 lanes per column each add every 16th slice, then one lane
@@ -194,12 +270,24 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
         const In* M, long ld, const In* X, long ldx, int nv, T* y, long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {     \
         docc_k::gemv_rows_multi<In, T, VEC, NV>(M, ld, X, ldx, nv, y, sy_row, sy_vec, rows, k, alpha, beta);                            \
     }
+// the columns form of the same; fp32 and fp64 only (for bf16 the MFMA tiles are as fast)
+#define DOCC_GEMV_MULTI_COLS(NAME, In, T, VEC, NV)                                                                                     \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colpm_##NAME##_v##VEC##_n##NV(                                          \
+        const In* M, long ld, const In* X, long sx_v, long sx_p, int nv, long rows, long cols, long chunk) {                          \
+        docc_k::gemv_cols_partial_multi<In, T, VEC, NV>(M, ld, X, sx_v, sx_p, nv, rows, cols, chunk);                                  \
+    }
 #define DOCC_GEMV_MULTI_ALL(NAME, In, T, VEC) \
     DOCC_GEMV_MULTI(NAME, In, T, VEC, 2) DOCC_GEMV_MULTI(NAME, In, T, VEC, 4) DOCC_GEMV_MULTI(NAME, In, T, VEC, 8)
+#define DOCC_GEMV_MULTI_COLS_ALL(NAME, In, T, VEC) \
+    DOCC_GEMV_MULTI_COLS(NAME, In, T, VEC, 2) DOCC_GEMV_MULTI_COLS(NAME, In, T, VEC, 4)
 DOCC_GEMV_MULTI_ALL(f32, float, float, 4)
 DOCC_GEMV_MULTI_ALL(f32, float, float, 1)
 DOCC_GEMV_MULTI_ALL(f64, double, double, 2)
 DOCC_GEMV_MULTI_ALL(f64, double, double, 1)
+DOCC_GEMV_MULTI_COLS_ALL(f32, float, float, 4)
+DOCC_GEMV_MULTI_COLS_ALL(f32, float, float, 1)
+DOCC_GEMV_MULTI_COLS_ALL(f64, double, double, 2)
+DOCC_GEMV_MULTI_COLS_ALL(f64, double, double, 1)
 DOCC_GEMV_MULTI_ALL(bf16, unsigned short, float, 8)
 DOCC_GEMV_MULTI_ALL(bf16, unsigned short, float, 1)
 
@@ -215,4 +303,12 @@ extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f32(float* y, l
 }
 extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f64(double* y, long incy, long cols, int slices, double alpha, double beta) {
     docc_k::gemv_cols_final<double>(y, incy, cols, slices, alpha, beta);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f32(float* y, long sy_vec, long sy_col, long cols, long entries, int slices,
+                                                                      float alpha, float beta) {
+    docc_k::gemv_cols_final_multi<float>(y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f64(double* y, long sy_vec, long sy_col, long cols, long entries, int slices,
+                                                                      double alpha, double beta) {
+    docc_k::gemv_cols_final_multi<double>(y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
 }

@@ -40,7 +40,54 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
     if (m > 1 && n > 1) {
         // two to eight rows or columns of output with both operands stored row by row along k (op(A) = A, op(B) = B^T,
         // the product of a small batch with a weight matrix): the larger operand moves once
-        if (ta || !tb || (m > 8 && n > 8)) return 1;
+        if (m > 8 && n > 8) return 1;
+        int cusm = compute_units();
+        if (cusm <= 0) cusm = 256;
+        const int64_t max_vectors = sizeof(T) == 2 ? 4 : 8;
+        if (sizeof(T) != 2 && ((m <= max_vectors && !ta && !tb) || (n <= max_vectors && ta && !tb && m > 8))) {
+            // the large operand is stored [k][columns] (y = x W with W as numpy holds it): columns form, sliced over k
+            const bool small_a = m <= max_vectors && !ta;
+            const int64_t nv = small_a ? m : n, cols = small_a ? n : m;
+            const T* mat = small_a ? B : A;
+            const T* vecs = small_a ? A : B;
+            const int64_t ldm = small_a ? ldb : lda;
+            const int64_t sx_v = small_a ? lda : 1, sx_p = small_a ? 1 : ldb;          // A[v][p] or B[p][v]
+            const int64_t sy_vec = small_a ? ldc : 1, sy_col = small_a ? 1 : ldc;
+            if (cols < 1024 || k < 64) return 1;
+            const int vecw = 16 / (int) sizeof(T);
+            const bool aligned = (uintptr_t) mat % 16 == 0 && ldm % vecw == 0 && cols % vecw == 0;
+            const int lanes = aligned ? vecw : 1;
+            const int64_t col_blocks = (cols / lanes + 255) / 256;
+            int64_t slices = (8 * (int64_t) cusm + col_blocks - 1) / col_blocks;
+            if (slices > k / 16) slices = k / 16;
+            // the partial sums are written and read back: keep them under a sixteenth of the matrix's bytes
+            const int64_t group = nv < 4 ? nv : 4;                                     // vectors per pass
+            int64_t cheap = k * (int64_t) sizeof(T) / (16 * (int64_t) sizeof(S) * group);
+            if (cheap * col_blocks < 4 * (int64_t) cusm) cheap *= 2;      // ... unless that leaves the chip short of work-groups
+            if (slices > cheap) slices = cheap;
+            const int64_t fit = (int64_t(8) << 20) / ((int64_t) sizeof(S) * cols * group);
+            if (slices > fit) slices = fit;
+            if (slices > 256) slices = 256;
+            if (slices < 1 || col_blocks > 0x7fffffffLL) return 1;
+            const int64_t chunk = (k + slices - 1) / slices;
+            slices = (k + chunk - 1) / chunk;
+            // five to eight vectors go as two passes of at most four: two reads of the matrix beat one with eight sums a lane
+            char kname[64], fname[64];
+            std::snprintf(fname, sizeof(fname), "docc_gemv_colfm_f%d", (int) sizeof(S) * 8);
+            for (int64_t v0 = 0; v0 < nv; v0 += 4) {
+                const int64_t gv = nv - v0 < 4 ? nv - v0 : 4;
+                std::snprintf(kname, sizeof(kname), "docc_gemv_colpm_%s_v%d_n%d", sizeof(T) == 4 ? "f32" : "f64", lanes, gv <= 2 ? 2 : 4);
+                int rcm = launch(kname, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, mat, (long) ldm, vecs + v0 * sx_v, (long) sx_v,
+                                 (long) sx_p, (int) gv, (long) k, (long) cols, (long) chunk);
+                if (rcm) return rcm;
+                const int64_t entries = gv * cols;
+                rcm = launch(fname, (uint32_t) ((entries + 63) / 64), 1, 1, 256, 0, s, C + v0 * sy_vec, (long) sy_vec, (long) sy_col,
+                             (long) cols, (long) entries, (int) slices, alpha, beta);
+                if (rcm) return rcm;
+            }
+            return 0;
+        }
+        if (ta || !tb) return 1;
         const bool small_a = m <= n;                  // the vectors: A's rows (m of them) or B's rows (n of them)
         const int64_t nv = small_a ? m : n, big = small_a ? n : m;
         int cus0 = compute_units();

@@ -268,6 +268,8 @@ GEMV_CASES = [  # m, n, k, ta, tb: one output column or row, each operand layout
     (5000, 1, 8, N, N), (1, 300, 5000, N, N),
     # two to eight vectors against a matrix stored row by row along k (a small batch times W^T)
     (4, 5000, 704, N, T), (8, 4200, 333, N, T), (5000, 2, 701, N, T), (4500, 7, 96, N, T), (3, 4099, 64, N, T),
+    # ... and against a matrix stored [k][n] (a small batch times W as numpy holds it), either side
+    (4, 5000, 704, N, N), (8, 4200, 333, N, N), (2, 1027, 4096, N, N), (5000, 3, 701, T, N), (4100, 8, 96, T, N),
 ]
 
 
