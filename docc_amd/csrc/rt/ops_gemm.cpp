@@ -199,8 +199,17 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
                                            bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
     }
-    if ((m <= 8 || n <= 8) && batch == 1 && !bias && activation < 0) {
+    const bool epilogue = bias || activation >= 0;
+    if ((m <= 8 || n <= 8) && batch == 1 && (!epilogue || ldc == n)) {
         rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
+        if (rc == 0 && epilogue) {
+            // the few rows or columns of output are a small tensor: bias and activation as one elementwise pass over it,
+            // the same roundings as the fused store
+            const int64_t shape[2] = {m, n}, row[2] = {1, n};
+            const int post[1] = {activation};
+            return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
+                                               bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
+        }
         if (rc != 1) return rc;
     }
     const size_t vec = 16 / sizeof(T);

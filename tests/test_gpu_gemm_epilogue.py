@@ -16,7 +16,9 @@ N, T = oracle.NO_TRANS, oracle.TRANS
 
 # m, n, k, ta, tb: aligned and ragged shapes, every tile family (small / large problems)
 SHAPES = [(64, 64, 64, N, N), (100, 130, 70, N, T), (257, 129, 100, T, N), (33, 17, 5, T, T), (512, 384, 256, N, N),
-          (1024, 1024, 128, N, T), (1, 300, 7, N, N), (40, 50, 0, N, N)]
+          (1024, 1024, 128, N, T), (1, 300, 7, N, N), (40, 50, 0, N, N),
+          # a small batch through a layer: the matrix-vector kernels, bias and activation as a pass over the few output rows
+          (4, 5000, 704, N, T), (3000, 1, 700, N, N), (4, 4200, 333, N, N), (1, 4096, 512, N, T)]
 ACTS = [None, "relu", "abs"]          # the activations built into the store
 
 
