@@ -62,11 +62,11 @@ __device__ __forceinline__ void gemv_rows(const In* __restrict__ M, long ld, con
 // A few vectors at once (a small batch against a weight matrix whose rows are contiguous, y = x W^T):
 // y[row * sy_row + v * sy_vec] = alpha * <M[row, :], X[v, :]> + beta * y[..] for v < nv <= NV. The matrix still
 // moves once; the vectors (nv * k elements) come from the caches.
-template <typename In, typename T, int VEC, int NV>
+// RW: matrix rows per wavefront; a piece of the vectors is loaded once for all of them
+template <typename In, typename T, int VEC, int NV, int RW>
 __device__ __forceinline__ void gemv_rows_multi(const In* __restrict__ M, long ld, const In* __restrict__ X, long ldx, int nv, T* __restrict__ y,
                                                 long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {
     typedef In V __attribute__((ext_vector_type(VEC)));
-    constexpr int RW = 4;   // matrix rows per wavefront: a piece of the vectors is loaded once for four rows
     const int lane = threadIdx.x & 63;
     const long row0 = ((long) blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
     if (row0 >= rows) return;
@@ -268,7 +268,13 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
 #define DOCC_GEMV_MULTI(NAME, In, T, VEC, NV)                                                                                          \
     extern "C" __global__ __launch_bounds__(256) void docc_gemv_rowsm_##NAME##_v##VEC##_n##NV(                                          \
         const In* M, long ld, const In* X, long ldx, int nv, T* y, long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {     \
-        docc_k::gemv_rows_multi<In, T, VEC, NV>(M, ld, X, ldx, nv, y, sy_row, sy_vec, rows, k, alpha, beta);                            \
+        docc_k::gemv_rows_multi<In, T, VEC, NV, 4>(M, ld, X, ldx, nv, y, sy_row, sy_vec, rows, k, alpha, beta);                         \
+    }
+// eight rows per wavefront: half the vector traffic, for matrices with enough rows to still fill the chip
+#define DOCC_GEMV_MULTI_R8(NAME, In, T, VEC, NV)                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_rowsm_##NAME##_v##VEC##_n##NV##_r8(                                     \
+        const In* M, long ld, const In* X, long ldx, int nv, T* y, long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {     \
+        docc_k::gemv_rows_multi<In, T, VEC, NV, 8>(M, ld, X, ldx, nv, y, sy_row, sy_vec, rows, k, alpha, beta);                         \
     }
 // the columns form of the same; fp32 and fp64 only (for bf16 the MFMA tiles are as fast)
 #define DOCC_GEMV_MULTI_COLS(NAME, In, T, VEC, NV)                                                                                     \
@@ -284,6 +290,10 @@ DOCC_GEMV_MULTI_ALL(f32, float, float, 4)
 DOCC_GEMV_MULTI_ALL(f32, float, float, 1)
 DOCC_GEMV_MULTI_ALL(f64, double, double, 2)
 DOCC_GEMV_MULTI_ALL(f64, double, double, 1)
+DOCC_GEMV_MULTI_R8(f32, float, float, 4, 2)
+DOCC_GEMV_MULTI_R8(f32, float, float, 4, 4)
+DOCC_GEMV_MULTI_R8(f64, double, double, 2, 2)
+DOCC_GEMV_MULTI_R8(f64, double, double, 2, 4)
 DOCC_GEMV_MULTI_COLS_ALL(f32, float, float, 4)
 DOCC_GEMV_MULTI_COLS_ALL(f32, float, float, 1)
 DOCC_GEMV_MULTI_COLS_ALL(f64, double, double, 2)

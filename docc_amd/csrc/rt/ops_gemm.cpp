@@ -43,7 +43,7 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         if (m > 8 && n > 8) return 1;
         int cusm = compute_units();
         if (cusm <= 0) cusm = 256;
-        const int64_t max_vectors = sizeof(T) == 2 ? 4 : 8;
+        const int64_t max_vectors = sizeof(T) == 4 ? 8 : 4;      // fp64 8 x 8192 x 8192: 296 us here, 172 through the tiles
         if (sizeof(T) != 2 && ((m <= max_vectors && !ta && !tb) || (n <= max_vectors && ta && !tb && m > 8))) {
             // the large operand is stored [k][columns] (y = x W with W as numpy holds it): columns form, sliced over k
             const bool small_a = m <= max_vectors && !ta;
@@ -93,18 +93,24 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         int cus0 = compute_units();
         if (cus0 <= 0) cus0 = 256;
         // bf16 from five vectors on is faster through the MFMA tiles (8 x 28672 x 8192: 111 us against 145 here)
-        const int64_t max_nv = sizeof(T) == 2 ? 4 : 8;
-        if (nv > max_nv || big < 16 * (int64_t) cus0 || (big + 15) / 16 > 0x7fffffffLL) return 1;   // 16 matrix rows per work-group
+        // ... and fp64 likewise (6 x 8192 x 8192: 168 us through the tiles against 170 here)
+        const int64_t max_nv = sizeof(T) == 4 ? 8 : 4;
+        const int vecw = 16 / (int) sizeof(T);
+        const bool aligned = ((uintptr_t) (small_a ? B : A) | (uintptr_t) (small_a ? A : B)) % 16 == 0 && (small_a ? ldb : lda) % vecw == 0 &&
+                             (small_a ? lda : ldb) % vecw == 0;
+        // a wavefront takes four matrix rows, or eight where that still leaves a work-group per CU (fp32 4 x 8192 x 8192:
+        // 79 -> 68 us; bf16 gains nothing from it)
+        const bool eight = nv <= 4 && aligned && sizeof(T) != 2 && big >= 32 * (int64_t) cus0;
+        const int64_t wg_rows = eight ? 32 : 16;
+        if (nv > max_nv || big < 16 * (int64_t) cus0 || (big + wg_rows - 1) / wg_rows > 0x7fffffffLL) return 1;
         const T* mat = small_a ? B : A;
         const T* vecs = small_a ? A : B;
         const int64_t ldm = small_a ? ldb : lda, ldx = small_a ? lda : ldb;
         const int64_t sy_row = small_a ? 1 : ldc, sy_vec = small_a ? ldc : 1;
-        const int vecw = 16 / (int) sizeof(T);
-        const bool aligned = ((uintptr_t) mat | (uintptr_t) vecs) % 16 == 0 && ldm % vecw == 0 && ldx % vecw == 0;
         char kname[64];
-        std::snprintf(kname, sizeof(kname), "docc_gemv_rowsm_%s_v%d_n%d", sizeof(T) == 2 ? "bf16" : sizeof(T) == 4 ? "f32" : "f64",
-                      aligned ? vecw : 1, nv <= 2 ? 2 : nv <= 4 ? 4 : 8);
-        return launch(kname, (uint32_t) ((big + 15) / 16), 1, 1, 256, 0, s, mat, (long) ldm, vecs, (long) ldx, (int) nv, C, (long) sy_row,
+        std::snprintf(kname, sizeof(kname), "docc_gemv_rowsm_%s_v%d_n%d%s", sizeof(T) == 2 ? "bf16" : sizeof(T) == 4 ? "f32" : "f64",
+                      aligned ? vecw : 1, nv <= 2 ? 2 : nv <= 4 ? 4 : 8, eight ? "_r8" : "");
+        return launch(kname, (uint32_t) ((big + wg_rows - 1) / wg_rows), 1, 1, 256, 0, s, mat, (long) ldm, vecs, (long) ldx, (int) nv, C, (long) sy_row,
                       (long) sy_vec, (long) big, (long) k, alpha, beta);
     }
     if (n == 1) {          // y = op(A) b: A as stored is [m][k] (rows form) or [k][m] (columns form)
