@@ -39,7 +39,7 @@ PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3, "bf16": 2516.6}
 
 # HBM bytes per softmax launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for the 128 MiB copy kernel; see profiles/softmax_f32_8192x4096_pmc.txt.
-SOFTMAX_TRAFFIC_BYTES = 268471498
+SOFTMAX_TRAFFIC_BYTES = 268470883
 
 
 def parse_args():
