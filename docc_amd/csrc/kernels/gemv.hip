@@ -61,15 +61,16 @@ __device__ __forceinline__ void gemv_rows(const In* __restrict__ M, long ld, con
 
 // A few vectors at once (a small batch against a weight matrix whose rows are contiguous, y = x W^T):
 // y[row * sy_row + v * sy_vec] = alpha * <M[row, :], X[v, :]> + beta * y[..] for v < nv <= NV. The matrix still
-// moves once; the vectors (nv * k elements) come from the caches.
-// RW: matrix rows per wavefront; a piece of the vectors is loaded once for all of them
+// moves once; a work-group stages the vectors through LDS, 256 lane-widths at a time, for all its rows.
+// RW: matrix rows per wavefront
 template <typename In, typename T, int VEC, int NV, int RW>
 __device__ __forceinline__ void gemv_rows_multi(const In* __restrict__ M, long ld, const In* __restrict__ X, long ldx, int nv, T* __restrict__ y,
                                                 long sy_row, long sy_vec, long rows, long k, T alpha, T beta) {
     typedef In V __attribute__((ext_vector_type(VEC)));
+    constexpr int STEP = 4, SPAN = STEP * 64;      // lane-widths of every vector in LDS at a time
+    __shared__ V xs[NV][SPAN];
     const int lane = threadIdx.x & 63;
     const long row0 = ((long) blockIdx.x * 4 + (threadIdx.x >> 6)) * RW;
-    if (row0 >= rows) return;
     const In* m[RW];
 #pragma unroll
     for (int r = 0; r < RW; r++) m[r] = M + (row0 + r < rows ? row0 + r : rows - 1) * ld;   // rows past the end repeat the last one
@@ -78,20 +79,36 @@ __device__ __forceinline__ void gemv_rows_multi(const In* __restrict__ M, long l
     for (int r = 0; r < RW; r++)
 #pragma unroll
         for (int v = 0; v < NV; v++) acc[r][v] = (T) 0;
-    const long nvec = VEC > 1 ? k / VEC : 0;
-    for (long c = lane; c < nvec; c += 64) {
-        V a[RW];
+    const long nvec = k / VEC;
+    for (long c0 = 0; c0 < nvec; c0 += SPAN) {
+        __syncthreads();
+        for (int i = threadIdx.x; i < NV * SPAN; i += 256) {
+            const int v = i / SPAN, j = i % SPAN;
+            V piece = {};
+            if (v < nv && c0 + j < nvec) piece = reinterpret_cast<const V*>(X + v * ldx)[c0 + j];
+            xs[v][j] = piece;
+        }
+        __syncthreads();
 #pragma unroll
-        for (int r = 0; r < RW; r++) a[r] = __builtin_nontemporal_load(reinterpret_cast<const V*>(m[r]) + c);
+        for (int st = 0; st < STEP; st++) {
+            const long c = c0 + st * 64 + lane;
+            if (c0 + st * 64 < nvec) {                      // uniform over the wavefront
+                const long cc = c < nvec ? c : nvec - 1;
+                V a[RW];
 #pragma unroll
-        for (int v = 0; v < NV; v++) {
-            if (v < nv) {
-                const V b = reinterpret_cast<const V*>(X + v * ldx)[c];
+                for (int r = 0; r < RW; r++) {
+                    a[r] = __builtin_nontemporal_load(reinterpret_cast<const V*>(m[r]) + cc);
+                    if (c >= nvec) a[r] = V{};              // past the end: zero times the zero in LDS
+                }
 #pragma unroll
-                for (int e = 0; e < VEC; e++) {
-                    const T bv = gemv_value<T, In>(b[e]);
+                for (int v = 0; v < NV; v++) {
+                    const V b = xs[v][st * 64 + lane];
 #pragma unroll
-                    for (int r = 0; r < RW; r++) acc[r][v] += gemv_value<T, In>(a[r][e]) * bv;
+                    for (int e = 0; e < VEC; e++) {
+                        const T bv = gemv_value<T, In>(b[e]);
+#pragma unroll
+                        for (int r = 0; r < RW; r++) acc[r][v] += gemv_value<T, In>(a[r][e]) * bv;
+                    }
                 }
             }
         }

@@ -92,9 +92,9 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         const int64_t nv = small_a ? m : n, big = small_a ? n : m;
         int cus0 = compute_units();
         if (cus0 <= 0) cus0 = 256;
-        // bf16 from five vectors on is faster through the MFMA tiles (8 x 28672 x 8192: 111 us against 145 here)
-        // ... and fp64 likewise (6 x 8192 x 8192: 168 us through the tiles against 170 here)
-        const int64_t max_nv = sizeof(T) == 4 ? 8 : 4;
+        // five to eight vectors: fp64 is faster through the MFMA tiles (8 x 8192 x 8192: 166 us against 218 here), bf16 too
+        // once the matrix is large (8 x 28672 x 8192: 111 us against 137; 8 x 8192 x 8192: 56 against 46 here)
+        const int64_t max_nv = sizeof(T) == 8 || (sizeof(T) == 2 && big * k > (int64_t(1) << 27)) ? 4 : 8;
         const int vecw = 16 / (int) sizeof(T);
         const bool aligned = ((uintptr_t) (small_a ? B : A) | (uintptr_t) (small_a ? A : B)) % 16 == 0 && (small_a ? ldb : lda) % vecw == 0 &&
                              (small_a ? lda : ldb) % vecw == 0;

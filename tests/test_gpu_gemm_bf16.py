@@ -135,7 +135,7 @@ def test_bgemm_every_tile_configuration(rt, cfg):
 BGEMV_CASES = [(3000, 1, 704, N, N), (3000, 1, 701, N, T), (2048, 1, 1024, T, N), (1504, 1, 333, T, T),
                (1, 3000, 700, N, N), (1, 2048, 1024, N, T), (1, 1501, 333, T, N), (1, 4096, 96, T, T),
                (4, 5000, 704, N, T), (3, 4200, 333, N, T), (5000, 2, 701, N, T), (4500, 4, 96, N, T),
-               (4, 5000, 704, N, N), (3, 4201, 333, N, N), (5000, 2, 701, T, N), (4104, 4, 96, T, N)]
+               (8, 5000, 704, N, T), (4500, 6, 333, N, T), (4, 5000, 704, N, N), (3, 4201, 333, N, N), (5000, 2, 701, T, N), (4104, 4, 96, T, N)]
 
 
 @pytest.mark.parametrize("case", BGEMV_CASES, ids=[f"{c[0]}x{c[1]}x{c[2]}" + "nt"[c[3] == T] + "nt"[c[4] == T] for c in BGEMV_CASES])
