@@ -242,6 +242,30 @@ def test_torch_compile_mlp_fp32():
     assert r["GEMM"] == 2 and r["H2D"] == 0 and r["D2H"] == 0      # device tensors: no transfers at all
 
 
+def test_torch_compile_small_batch_through_wide_layers():
+    """A batch of four through 2048-wide layers: the GEMMs have few output rows and take the matrix-vector kernels
+    (bias and activation as one pass over the output); same bar as any fp32 GEMM chain."""
+    class Decoder(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = torch.nn.Linear(2048, 8192)
+            self.down = torch.nn.Linear(8192, 2048, bias=False)
+
+        def forward(self, x):
+            return self.down(torch.relu(self.up(x)))
+
+    torch.manual_seed(3)
+    model = Decoder().cuda()
+    x = torch.randn(4, 2048, device="cuda")
+    program = docc_torch.compile_torch(model, x, target="rocm")
+    y = program(x)
+    assert y.is_cuda and y.shape == (4, 2048)
+    with torch.no_grad():
+        ref = model.double()(x.double())
+    assert rel_err_max(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+    assert program.last_sdfg.loop_report()["GEMM"] == 2
+
+
 @pytest.mark.parametrize("mode", ["", "aggregate"])
 def test_instrumented_program_writes_a_trace_with_device_times(tmp_path, mode):
     """`instrumentation_mode="ols"`: every rocm node and transfer is a region timed with HIP events;
