@@ -110,11 +110,15 @@ public:
             ops = operands();
             emit_transfers_begin(stream, ops);
         }
+        // the pointer a launcher receives: the connector's local as it is (a device pointer already), or the
+        // device copy this dispatcher made. A connector that is not among the copied operands would hand a
+        // host pointer to a kernel, so it is an error here rather than a fault on the device.
         auto name_of = [&](const std::string& connector) -> std::string {
             if (!with_transfers_) return connector;
             for (auto& op : ops)
                 if (op.connector == connector) return op.device;
-            return connector;
+            throw std::runtime_error("rocm dispatcher of " + node_.code() + ": connector '" + connector +
+                                     "' is passed to the launcher but is not one of the node's device operands");
         };
         emit_launch(stream, name_of);
         if (with_transfers_) emit_transfers_end(stream, ops);
@@ -138,6 +142,10 @@ protected:
     virtual std::string guard_condition() const { return ""; }
 
     DeviceOperand operand(const std::string& connector, bool in, bool out) const {
+        const auto& names = out ? node_.outputs() : node_.inputs();
+        if (std::find(names.begin(), names.end(), connector) == names.end() && data_flow_graph_.input(connector) == nullptr &&
+            data_flow_graph_.output(connector) == nullptr)
+            throw std::runtime_error("rocm dispatcher of " + node_.code() + ": the node has no connector '" + connector + "'");
         return DeviceOperand{connector, "d_" + connector, node_.connector_bytes(connector), in, out};
     }
 
@@ -209,7 +217,7 @@ protected:
     const tensor::MatMulNode& mm() const { return static_cast<const tensor::MatMulNode&>(node_); }
 
     std::vector<DeviceOperand> operands() const override {
-        return {operand("A", true, false), operand("B", true, false), operand("C", false, true)};
+        return {operand("A", true, false), operand("B", true, false), operand("Y", false, true)};
     }
 
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
@@ -1064,91 +1072,209 @@ bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, ana
 }
 
 bool RocmDataTransferMinimizationPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
+    // The root sequence is straight-line code, so the device copy of every host container can be
+    // tracked exactly: one forward walk keeps, per host container, the device buffer that holds its
+    // current value. An upload from a container whose value already sits in a buffer of the same
+    // extent is dropped and its buffer renamed to the first one (however many nodes read it, and
+    // whatever lies between them); a node that rewrites a container takes over the buffer the old
+    // value lived in; a download is kept only where the host looks at the data before the device
+    // writes it again; every buffer is freed once, behind its last use.
     StructuredSDFG& sdfg = builder.subject();
-    auto& blocks = sdfg.blocks();
+    std::vector<Block> old = std::move(sdfg.blocks());
+    std::vector<Block>& out = sdfg.blocks();
+    out.clear();
     bool applied = false;
 
-    auto uses_host = [&](const Block& b, const std::string& host) {
-        for (auto& in : b.inputs)
-            if (!in.is_constant && in.data == host) return true;
-        for (auto& out : b.outputs)
-            if (out.data == host) return true;
-        return false;
+    struct Resident {
+        std::string device;
+        Expression bytes;
+        int device_id = 0;
     };
-    auto needed_on_host = [&](const std::string& host, size_t from) {
-        const Container& c = sdfg.container(host);
-        if (c.is_argument || host == sdfg.return_container()) return true;
-        for (size_t j = from; j < blocks.size(); j++)
-            if (!is_offloading(blocks[j]) && uses_host(blocks[j], host)) return true;
-        return false;
-    };
+    std::map<std::string, Resident> current;          // host container -> buffer holding its value
+    std::map<std::string, std::string> stale;         // host container whose own memory is out of date -> that buffer
+    std::map<std::string, std::string> renamed;       // dropped device container -> the one used instead
+    std::map<std::string, Resident> allocated;        // device buffers of the function, in need of a FREE
+    std::vector<std::string> allocation_order;
 
-    bool changed = true;
-    while (changed) {
-        changed = false;
-        for (size_t i = 0; i < blocks.size() && !changed; i++) {
-            if (!is_offloading(blocks[i])) continue;
-            const auto& first = offloading(blocks[i]);
-            if (first.transfer_direction() == DataTransferDirection::NONE && first.is_free()) {
-                // a read-only operand freed here and uploaded again later from the same, unchanged
-                // host container: keep the first device copy alive instead
-                const std::string dev1 = blocks[i].inputs[0].data;
-                std::string host;
-                for (size_t k = 0; k < i; k++)
-                    if (is_offloading(blocks[k]) && offloading(blocks[k]).is_h2d() && blocks[k].outputs[0].data == dev1)
-                        host = blocks[k].inputs[0].data;
-                if (host.empty()) continue;
-                size_t j = i + 1;
-                while (j < blocks.size() && !uses_host(blocks[j], host)) j++;
-                if (j >= blocks.size() || !is_offloading(blocks[j])) continue;
-                const auto& again = offloading(blocks[j]);
-                if (!again.is_h2d() || !again.is_alloc() || again.size() != first.size() || again.device_id() != first.device_id()) continue;
-                const std::string dev2 = blocks[j].outputs[0].data;
-                blocks.erase(blocks.begin() + (long) j);
-                blocks.erase(blocks.begin() + (long) i);
-                for (size_t k = i; k < blocks.size(); k++) {
-                    for (auto& in : blocks[k].inputs)
-                        if (!in.is_constant && in.data == dev2) in.data = dev1;
-                    for (auto& out : blocks[k].outputs)
-                        if (out.data == dev2) out.data = dev1;
+    auto host_side = [&](const Block& b) { return !is_offloading(b) && !is_rocm_impl(b.node->implementation_type()); };
+    auto reads_container = [&](const Block& b, const std::string& name) {
+        for (auto& in : b.inputs)
+            if (!in.is_constant && in.data == name) return true;
+        return false;
+    };
+    auto writes_container = [&](const Block& b, const std::string& name) {
+        for (auto& o : b.outputs)
+            if (o.data == name) return true;
+        return false;
+    };
+    // does host code look at `host` after position `from` of the old sequence, before the device
+    // replaces all of it again?
+    auto host_needs = [&](const std::string& host, const Expression& bytes, size_t from) {
+        for (size_t j = from; j < old.size(); j++) {
+            const Block& b = old[j];
+            if (!b.node) continue;
+            if (is_offloading(b)) {
+                const auto& node = offloading(b);
+                if (node.is_d2h() && b.outputs[0].data == host && node.size() == bytes) return false;
+                if (node.is_h2d() && b.inputs[0].data == host) {
+                    const auto it = current.find(host);
+                    // an upload that will not be dropped reads the host memory
+                    if (it == current.end() || it->second.bytes != node.size() || it->second.device_id != node.device_id()) return true;
                 }
-                changed = applied = true;
                 continue;
             }
-            if (!first.is_d2h() || !first.is_free()) continue;
-            const std::string host = blocks[i].outputs[0].data, dev1 = blocks[i].inputs[0].data;
-            // next block that touches the host container
-            size_t j = i + 1;
-            while (j < blocks.size() && !uses_host(blocks[j], host)) j++;
-            if (j >= blocks.size() || !is_offloading(blocks[j])) continue;
-            const auto& second = offloading(blocks[j]);
-            if (!second.is_h2d() || !second.is_alloc() || !first.redundant_with(second)) continue;
-            const std::string dev2 = blocks[j].outputs[0].data;
-            // the upload disappears; every later use of its device buffer refers to the first buffer
-            blocks.erase(blocks.begin() + (long) j);
-            for (size_t k = j; k < blocks.size(); k++) {
-                for (auto& in : blocks[k].inputs)
-                    if (!in.is_constant && in.data == dev2) in.data = dev1;
-                for (auto& out : blocks[k].outputs)
-                    if (out.data == dev2) out.data = dev1;
-            }
-            // the download stays only if the host still looks at the data, and no longer frees
-            if (needed_on_host(host, i + 1)) {
-                auto keep = std::make_unique<ROCMDataOffloadingNode>(first.size(), first.device_id(), DataTransferDirection::D2H,
-                                                                     BufferLifecycle::NO_CHANGE);
-                keep->set_element_id(blocks[i].node->element_id());
-                blocks[i].node = std::move(keep);
-            } else {
-                blocks.erase(blocks.begin() + (long) i);
-                // a host transient nobody touches any more needs no host memory
-                Container& c = sdfg.container(host);
-                bool any = false;
-                for (auto& b : blocks)
-                    if (uses_host(b, host)) any = true;
-                if (!any && c.transient) c.size_bytes.clear();
-            }
-            changed = applied = true;
+            if (host_side(b) && (reads_container(b, host) || writes_container(b, host))) return true;
         }
+        const Container& c = sdfg.container(host);
+        return c.is_argument || host == sdfg.return_container();
+    };
+    auto emit_download = [&](const std::string& host, const Resident& from, const structured_control_flow::DebugInfo& dbg) {
+        Block blk;
+        blk.element_id = sdfg.next_element_id();
+        blk.debug_info = dbg;
+        blk.node = std::make_unique<ROCMDataOffloadingNode>(from.bytes, from.device_id, DataTransferDirection::D2H, BufferLifecycle::NO_CHANGE);
+        blk.node->set_element_id(sdfg.next_element_id());
+        blk.inputs = {make_binding("_src", from.device)};
+        blk.outputs = {make_binding("_dst", host)};
+        out.push_back(std::move(blk));
+    };
+
+    for (size_t i = 0; i < old.size(); i++) {
+        Block b = std::move(old[i]);
+        old[i].node.reset();
+        for (auto& in : b.inputs)
+            if (!in.is_constant && renamed.count(in.data)) in.data = renamed[in.data];
+        for (auto& o : b.outputs)
+            if (renamed.count(o.data)) o.data = renamed[o.data];
+
+        if (!is_offloading(b)) {
+            if (host_side(b)) {
+                // host code: bring in what it reads, forget device copies of what it writes
+                for (auto& in : b.inputs)
+                    if (!in.is_constant && stale.count(in.data)) {
+                        emit_download(in.data, current.at(in.data), b.debug_info);
+                        stale.erase(in.data);
+                    }
+                for (auto& o : b.outputs) {
+                    current.erase(o.data);
+                    stale.erase(o.data);
+                }
+            }
+            out.push_back(std::move(b));
+            continue;
+        }
+
+        const auto& node = offloading(b);
+        if (node.is_h2d()) {
+            const std::string host = b.inputs[0].data, device = b.outputs[0].data;
+            const auto it = current.find(host);
+            if (node.is_alloc() && it != current.end() && it->second.bytes == node.size() && it->second.device_id == node.device_id()) {
+                renamed[device] = it->second.device;      // the value is on the device already
+                applied = true;
+                continue;
+            }
+            if (stale.count(host)) {                      // an upload of another extent: the host memory must be current first
+                emit_download(host, current.at(host), b.debug_info);
+                stale.erase(host);
+            }
+            current[host] = Resident{device, node.size(), node.device_id()};
+            if (node.is_alloc() && !allocated.count(device)) {
+                allocated[device] = current[host];
+                allocation_order.push_back(device);
+            }
+            out.push_back(std::move(b));
+            continue;
+        }
+        if (node.is_d2h()) {
+            const std::string device = b.inputs[0].data, host = b.outputs[0].data;
+            const Resident here{device, node.size(), node.device_id()};
+            current[host] = here;
+            if (host_needs(host, node.size(), i + 1)) {
+                stale.erase(host);
+                emit_download(host, here, b.debug_info);
+                out.back().node->set_element_id(b.node->element_id());
+                out.back().element_id = b.element_id;
+            } else {
+                stale[host] = device;
+                applied = true;
+            }
+            continue;                                     // a FREE comes behind the buffer's last use
+        }
+        if (node.is_alloc()) {
+            // a buffer some node is about to fill: the download that follows names the host container
+            const std::string device = b.outputs[0].data;
+            std::string host;
+            for (size_t j = i + 1; j < old.size() && host.empty(); j++) {
+                if (!old[j].node || !is_offloading(old[j])) continue;
+                if (offloading(old[j]).is_d2h() && old[j].inputs[0].data == device) host = old[j].outputs[0].data;
+                else if (offloading(old[j]).is_free() && old[j].inputs[0].data == device) break;
+            }
+            const auto it = host.empty() ? current.end() : current.find(host);
+            if (it != current.end() && it->second.bytes == node.size() && it->second.device_id == node.device_id()) {
+                renamed[device] = it->second.device;      // the old value's buffer is overwritten in place
+                applied = true;
+                continue;
+            }
+            if (!allocated.count(device)) {
+                allocated[device] = Resident{device, node.size(), node.device_id()};
+                allocation_order.push_back(device);
+            }
+            out.push_back(std::move(b));
+            continue;
+        }
+        // a bare FREE: dropped here, placed behind the last use below
+        if (node.is_free()) continue;
+        out.push_back(std::move(b));
+    }
+
+    // one FREE per buffer, behind its last use; a download that is the last use frees as well
+    for (auto rit = allocation_order.rbegin(); rit != allocation_order.rend(); ++rit) {
+        const Resident& r = allocated.at(*rit);
+        size_t last = out.size();
+        for (size_t j = out.size(); j-- > 0;) {
+            if (reads_container(out[j], r.device) || writes_container(out[j], r.device)) {
+                last = j;
+                break;
+            }
+        }
+        if (last == out.size()) continue;
+        Block& user = out[last];
+        if (is_offloading(user) && offloading(user).is_d2h() && !offloading(user).is_free() && user.inputs[0].data == r.device) {
+            auto both = std::make_unique<ROCMDataOffloadingNode>(r.bytes, r.device_id, DataTransferDirection::D2H, BufferLifecycle::FREE);
+            both->set_element_id(user.node->element_id());
+            user.node = std::move(both);
+            continue;
+        }
+        Block blk;
+        blk.element_id = sdfg.next_element_id();
+        blk.debug_info = user.debug_info;
+        blk.node = std::make_unique<ROCMDataOffloadingNode>(r.bytes, r.device_id, DataTransferDirection::NONE, BufferLifecycle::FREE);
+        blk.node->set_element_id(sdfg.next_element_id());
+        blk.inputs = {make_binding("_ptr", r.device)};
+        // behind the other FREEs that already follow this position
+        size_t pos = last + 1;
+        while (pos < out.size() && is_offloading(out[pos]) && offloading(out[pos]).transfer_direction() == DataTransferDirection::NONE &&
+               offloading(out[pos]).is_free())
+            pos++;
+        out.insert(out.begin() + (long) pos, std::move(blk));
+    }
+
+    // device containers that were renamed away, and host memory of transients nobody touches any more
+    for (auto& kv : renamed) {
+        bool used = false;
+        for (auto& b : out)
+            if (reads_container(b, kv.first) || writes_container(b, kv.first)) used = true;
+        if (!used && sdfg.exists(kv.first)) sdfg.remove_container(kv.first);
+    }
+    std::vector<std::string> names;
+    for (auto& kv : sdfg.containers()) names.push_back(kv.first);
+    for (auto& name : names) {
+        Container& c = sdfg.container(name);
+        if (!c.transient || c.is_argument || c.storage != "CPU" || c.size_bytes.empty() || name == sdfg.return_container()) continue;
+        bool used = false;
+        for (auto& b : out)
+            if (reads_container(b, name) || writes_container(b, name)) used = true;
+        if (!used) c.size_bytes.clear();
     }
     return applied;
 }

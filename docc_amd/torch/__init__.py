@@ -634,6 +634,20 @@ class TorchProgram(DoccProgram):
             parts.append(f"{tuple(a.shape)}:{a.dtype}:{a.device.type}" if isinstance(a, torch.Tensor) else f"scalar({type(a).__name__})")
         return "|".join(parts)
 
+    def _model_code(self) -> str:
+        """Text that tells two models of the same name apart: the traced graph's code (it names every
+        operation and constant argument), else the source of forward()."""
+        try:
+            return self._graph_module().graph.python_code("self").src
+        except Exception:
+            pass
+        try:
+            import inspect
+
+            return inspect.getsource(type(self.model).forward)
+        except Exception:
+            return ""
+
     def _lower(self, examples):
         lowering = _FxLowering(self._graph_module(), examples, f"__docc_{self.name}")
         sdfg = lowering.lower()
@@ -654,7 +668,11 @@ class TorchProgram(DoccProgram):
         self._sdfg = sdfg
         folder = output_folder
         if folder is None:
-            stable_id = hashlib.sha256(f"{self.name}|{self.target}|{self.category}|{key}".encode()).hexdigest()[:16]
+            # the folder (and with it the path the library is loaded from) is specific to the graph: every
+            # graph torch.compile hands over is called "GraphModule", and dlopen returns the handle it already
+            # holds for a path, so two models sharing a folder would run the first one's code
+            # (reference mlir/docc/torch/__init__.py:110-131 hashes the model's code for the same reason)
+            stable_id = hashlib.sha256(f"{self.name}|{self.target}|{self.category}|{key}|{self._model_code()}".encode()).hexdigest()[:16]
             base = os.environ.get("DOCC_TMP") or f"/tmp/{os.getenv('USER') or getpass.getuser()}/DOCC"
             folder = f"{base}/{self.name}-{stable_id}"
         if os.path.exists(folder):

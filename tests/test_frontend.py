@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 import scipy.special
 import torch
+from pathlib import Path
 
 import docc_amd.torch as docc_torch
 from docc_amd.python import (conv2d, erf, native, register_target, register_target_overrides, relu, sigmoid, softmax,
@@ -366,6 +367,28 @@ def test_torch_backend_is_registered_and_reads_global_options():
     finally:
         unregister_target("probe")
         docc_torch.set_backend_options(target="rocm")
+
+
+def test_torch_models_of_one_name_and_shape_get_libraries_of_their_own(tmp_path, monkeypatch):
+    """Two different models with the same class name and input shapes (under torch.compile every graph is a
+    "GraphModule"): folder and library path differ, so loading the second cannot return the first's handle
+    (reference mlir/docc/torch/__init__.py:110-131)."""
+    monkeypatch.setenv("DOCC_TMP", str(tmp_path))
+
+    def make(fn):
+        return type("Net", (torch.nn.Module,), {"forward": lambda self, x: fn(x)})()
+
+    x = torch.randn(4, 8)
+    first = docc_torch.TorchProgram(make(torch.tanh), None, target="rocm").compile(x)
+    second = docc_torch.TorchProgram(make(torch.relu), None, target="rocm").compile(x)
+    assert first.sdfg.name == second.sdfg.name
+    assert first.lib_path != second.lib_path and Path(first.lib_path).parent != Path(second.lib_path).parent
+    assert first.lib._handle != second.lib._handle
+    codes = [c.sdfg.library_nodes() for c in (first, second)]
+    assert any(n["code"] == "ml::Tanh" for n in codes[0]) and any(n["code"] == "ml::ReLU" for n in codes[1])
+    # the same model again maps to the same place
+    again = docc_torch.TorchProgram(make(torch.tanh), None, target="rocm").compile(x)
+    assert again.lib_path == first.lib_path
 
 
 def test_reductions_and_softmax_pieces_used_on_their_own():

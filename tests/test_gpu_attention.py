@@ -66,6 +66,91 @@ def test_attention_closed_forms(rt):
     assert np.array_equal(O[0, 0], np.broadcast_to(Vd[0, 0, 17].float().numpy(), (32, 64)))
 
 
+def _ramp_case(SQ, SKV, steps, g):
+    """Keys whose scores grow (or fall) block by block for the queries that point along coordinate 0:
+    K[j, 0] = 32 * steps[j // 64], Q[i, 0] cycles through (+8, -8, +0.5, 0), so between two 64-key
+    blocks the row maximum of the +8 queries moves by 32 * 8 / 8 = 32 nats (46 in the log2 domain) per
+    unit of `steps`, that of the +0.5 queries by 2 nats, and the -8 queries see it fall."""
+    Q = torch.randn(1, 2, SQ, 64, generator=g)
+    K = torch.randn(1, 2, SKV, 64, generator=g)
+    V = torch.randn(1, 2, SKV, 64, generator=g)
+    Q[..., 0] = torch.tensor([8.0, -8.0, 0.5, 0.0]).repeat((SQ + 3) // 4)[:SQ]
+    blk = torch.arange(SKV) // 64
+    K[..., 0] = 32.0 * torch.tensor(steps, dtype=torch.float32)[blk]
+    return Q.bfloat16(), K.bfloat16(), V.bfloat16()
+
+
+@pytest.mark.parametrize("SQ,SKV,steps", [
+    (256, 1024, [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15]),     # the maximum grows in every block
+    (130, 1024, [3, 0, 1, 5, 5, 2, 9, 1, 0, 12, 4, 4, 13, 2, 15, 1]),        # grows, falls, grows again
+    (192, 1000, [0, 0, 2, 2, 1, 4, 0, 6, 3, 8, 8, 1, 10, 5, 2, 12]),         # ... with a partial last block
+    (64, 704, [15, 14, 13, 12, 11, 10, 9, 8, 7, 6, 5]),                      # falls: the first block dominates
+])
+def test_attention_reference_point_moves_between_blocks(rt, SQ, SKV, steps):
+    """The running reference point of the exponentials has to move, and the output and the running sum be
+    rescaled, in blocks after the first: row maxima that grow by more than 2^40 between key blocks."""
+    g = torch.Generator().manual_seed(SQ + SKV)
+    Q, K, V = _ramp_case(SQ, SKV, steps, g)
+    for out_bf16 in (False, True):
+        O = run_attention(rt, bits(Q), bits(K), bits(V), out_bf16=out_bf16)
+        ref = oracle.attention(bits(Q), bits(K), bits(V))
+        assert np.isfinite(O).all()
+        assert rel_err_max(O, ref) <= TOL_BF16
+
+
+@pytest.mark.parametrize("sigma,bound", [(1.0, 5e-3), (3.3, 5e-3), (4.5, 5e-3), (8.0, 5e-3)])
+def test_attention_large_logits(rt, sigma, bound):
+    """Scores far from N(0,1): with Q, K ~ N(0, sigma^2) the logits span about +-5 sigma^2 (+-60 at sigma 3.3,
+    +-110 at 4.5, +-330 at 8). The scale is applied to the fp32 scores, not folded into a re-rounded bf16 Q, so
+    the error does not grow with the logits: it stays at the bf16 rounding of the probabilities (measured
+    1.5e-3 .. 2.5e-3), well inside the 2e-2 of the bf16 configurations."""
+    g = torch.Generator().manual_seed(int(sigma * 10))
+    Q, K = ((torch.randn(1, 4, 512, 64, generator=g) * sigma).bfloat16() for _ in range(2))
+    V = torch.randn(1, 4, 512, 64, generator=g).bfloat16()
+    O = run_attention(rt, bits(Q), bits(K), bits(V))
+    ref = oracle.attention(bits(Q), bits(K), bits(V))
+    err = rel_err_max(O, ref)
+    print(f"attention sigma {sigma}: logits up to {float((Q.float() @ K.float().transpose(-1, -2)).abs().max()) / 8:.0f}, rel err {err:.2e}")
+    assert err <= bound <= TOL_BF16
+
+
+def _inf_nan_case():
+    g = torch.Generator().manual_seed(11)
+    SQ, SKV = 96, 320
+    Q = torch.randn(1, 4, SQ, 64, generator=g)
+    K = torch.randn(1, 4, SKV, 64, generator=g)
+    V = torch.randn(1, 4, SKV, 64, generator=g)
+    Q[..., 0] = Q[..., 0].abs() + 0.5               # positive: a key with -inf in coordinate 0 scores -inf
+    # head 0: the first 64 keys (all of the first block) and a scattering of later ones are excluded
+    K[0, 0, :64, 0] = -float("inf")
+    K[0, 0, 100:300:7, 0] = -float("inf")
+    # head 1: one key row holds a NaN -> every row of that head is NaN
+    K[0, 1, 77, 5] = float("nan")
+    # head 2: every second key excluded; queries 16..31 multiply the infinity by zero (NaN scores),
+    # queries 32..47 by a negative number (+inf scores): NaN rows, the other rows stay finite
+    K[0, 2, ::2, 0] = -float("inf")
+    Q[0, 2, 16:32, 0] = 0.0
+    Q[0, 2, 32:48, 0] *= -1.0
+    # head 3: every key excluded -> 0 / 0
+    K[0, 3, :, 0] = -float("inf")
+    return Q.bfloat16(), K.bfloat16(), V.bfloat16()
+
+
+def test_attention_infinite_and_nan_scores(rt):
+    """Scores of -inf (a key that is excluded), +inf and NaN: what the oracle's max / exp / sum / divide
+    chain gives. -inf scores weigh nothing, also when they fill the whole first block of keys; a row of
+    only -inf scores, a +inf score or a NaN score make the row NaN."""
+    Qb, Kb, Vb = _inf_nan_case()
+    ref = oracle.attention(bits(Qb), bits(Kb), bits(Vb))
+    assert np.isfinite(ref[0, 0]).all() and np.isnan(ref[0, 1]).all() and np.isnan(ref[0, 3]).all()
+    assert np.array_equal(np.isnan(ref[0, 2]).all(axis=1), (np.arange(96) >= 16) & (np.arange(96) < 48))
+    for out_bf16 in (False, True):
+        O = run_attention(rt, bits(Qb), bits(Kb), bits(Vb), out_bf16=out_bf16)
+        assert np.array_equal(np.isnan(O), np.isnan(ref))
+        ok = np.isfinite(ref)
+        assert rel_err_max(np.where(ok, O, 0.0), np.where(ok, ref, 0.0)) <= TOL_BF16
+
+
 def test_attention_errors(rt):
     from docc_amd.runtime import RocmRuntimeError
     t = torch.zeros(64 * 64, dtype=torch.bfloat16, device="cuda")

@@ -93,6 +93,21 @@ def test_native_chain_keeps_the_intermediate_on_the_device():
     assert r["H2D"] == 3 and r["D2H"] == 1
 
 
+def test_native_intermediate_with_two_readers():
+    @native(target="rocm")
+    def two_readers(a, b):
+        t = a @ b
+        return scipy.special.softmax(t, axis=-1) @ t
+
+    rng = np.random.default_rng(5)
+    a, b = (rng.standard_normal((80, 80)).astype(np.float32) * 0.3 for _ in range(2))
+    y = two_readers(a, b)
+    t = oracle.gemm(a, b)
+    assert rel_err_max(y, oracle.gemm(oracle.softmax(t), t)) <= 1e-5
+    r = two_readers.last_sdfg.loop_report()
+    assert r["H2D"] == 2 and r["D2H"] == 1          # the intermediate feeds both nodes from device memory
+
+
 def test_native_conv():
     @native(target="rocm")
     def conv(x, w, b):

@@ -311,6 +311,155 @@ def test_offloading_reuses_a_read_only_operand(tmp_path):
     assert len(d2h_only) == 1     # C's download no longer frees: the second GEMM still reads the device copy
 
 
+def every_node_type():
+    """One single-node program per node type the target lowers; arguments p0..p3 (names no connector has)."""
+    def build(name, fill, ptrs):
+        b = StructuredSDFGBuilder(name)
+        for n, t in ptrs.items():
+            b.add_container(n, t, True)
+        fill(b)
+        return b.move()
+
+    f3 = {"p0": F32, "p1": F32, "p3": F32}
+    yield build("n_gemm", lambda b: b.add_gemm("p0", "p1", "p3", "1.0", "0.5", 8, 8, 8), f3)
+    yield build("n_gemm_bf16", lambda b: b.add_gemm("p0", "p1", "p3", "1.0", "0.0", 8, 8, 8), {"p0": BF16, "p1": BF16, "p3": F32})
+    yield build("n_matmul", lambda b: b.add_matmul("p0", "p1", "p3", [6, 32, 16], [6, 16, 24]), f3)
+    yield build("n_softmax", lambda b: b.add_reduce_op("softmax", "p0", "p3", [4, 8], [-1]), {"p0": F32, "p3": F32})
+    yield build("n_softmax_inner", lambda b: b.add_reduce_op("softmax", "p0", "p3", [4, 8, 6], [1]), {"p0": F64, "p3": F64})
+    for op in ("sum", "max", "min", "mean"):
+        yield build("n_" + op, lambda b, op=op: b.add_reduce_op(op, "p0", "p3", [4, 8, 6], [1]), {"p0": F32, "p3": F32})
+    yield build("n_conv", lambda b: b.add_conv("p0", "p1", "p3", [2, 8, 9, 9], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 16, B="p2"),
+                {"p0": F32, "p1": F32, "p2": F32, "p3": F32})
+    yield build("n_conv_gemm", lambda b: b.add_conv("p0", "p1", "p3", [2, 7, 9, 9], [3, 3], [2, 2], [0, 0, 0, 0], [1, 1], 16),
+                {"p0": F32, "p1": F32, "p3": F32})
+    for d in (64, 128):
+        yield build(f"n_attention{d}", lambda b, d=d: b.add_attention("p0", "p1", "p2", "p3", [2, 4, 96, d], 80, 0.125),
+                    {"p0": BF16, "p1": BF16, "p2": BF16, "p3": F32})
+    for op in StructuredSDFGBuilder.UNARY_CODES:
+        yield build("n_" + op, lambda b, op=op: b.add_elementwise_unary_op(op, "p0", "p3", [4, 8]), {"p0": F32, "p3": F32})
+    for op in sorted(set(StructuredSDFGBuilder.BINARY_CODES) - {"max", "min"}):
+        yield build("n_" + op, lambda b, op=op: b.add_elementwise_op(op, "p0", "p1", "p3", [4, 8]), f3)
+    yield build("n_scalar", lambda b: b.add_elementwise_op("mul", "p0", 2.5, "p3", [4, 8]), {"p0": F64, "p3": F64})
+    yield build("n_broadcast", lambda b: b.add_broadcast("p0", "p3", [1, 8], [4, 8]), {"p0": F32, "p3": F32})
+    yield build("n_transpose", lambda b: b.add_transpose("p0", "p3", [4, 8, 3], [2, 0, 1]), {"p0": F32, "p3": F32})
+    yield build("n_cast", lambda b: b.add_cast_op("p0", "p3", [4, 8]), {"p0": F32, "p3": BF16})
+
+
+LAUNCHER_CALL = re.compile(r"DOCC_ROCM_CHECK\((docc_rocm_\w+)\((.*)\)\);")
+NOT_A_KERNEL = {"docc_rocm_malloc", "docc_rocm_free", "docc_rocm_memcpy_h2d_async", "docc_rocm_memcpy_d2h_async",
+                "docc_rocm_stream_sync"}
+
+
+@pytest.mark.parametrize("offload", ["node", "function", "none"])
+def test_every_node_type_generates_valid_code_on_device_pointers(tmp_path, offload):
+    """Each node type, alone, under each offloading mode: the emitted C++ passes the compiler's syntax and
+    type checks against the runtime headers, and where the function receives host pointers no launcher is
+    handed one of them (a host address in a kernel is a memory fault on the device)."""
+    include = Path(runtime.__file__).resolve().parent.parent / "include"
+    for s in every_node_type():
+        pointers = {n for n in s.arguments if s.containers[n].get("pointer", True)}
+        s.schedule("rocm", options={"offload": offload})
+        folder = tmp_path / s.name
+        src, report = source_of(s, folder)
+        cxx = __import__("os").environ.get("DOCC_CXX", "/opt/rocm/lib/llvm/bin/clang++")     # the compiler the target's JIT step runs
+        proc = __import__("subprocess").run([cxx, "-std=c++17", "-fsyntax-only", "-Wall",
+                                             "-I", str(include), "-I", str(folder), report["source"]], capture_output=True, text=True)
+        assert proc.returncode == 0, f"{s.name} under offload={offload}:\n{proc.stderr}\n{src}"
+        calls = [m for m in LAUNCHER_CALL.finditer(src) if m.group(1) not in NOT_A_KERNEL and not m.group(1).endswith("_workspace_bytes")]
+        assert calls, s.name
+        if offload == "none":
+            continue
+        connectors = set()
+        for node in s.library_nodes():
+            if node["code"] != "ROCMOffloading":
+                connectors |= {c for c in node.get("inputs", []) + node.get("outputs", [])}
+        for m in calls:
+            tokens = set(re.findall(r"[A-Za-z_]\w*", m.group(2)))
+            if offload == "node":
+                # the node's connector locals are host pointers here; only their device copies d_<connector> may be passed
+                bare = {t for t in tokens if t in connectors and not t.startswith("__alpha") and not t.startswith("__beta")}
+                assert not (bare & {"A", "B", "C", "X", "Y", "W", "Q", "K", "V", "O", "__A", "__B", "__C", "__bias"}), (s.name, m.group(0))
+            assert not (tokens & pointers), (s.name, m.group(0))
+
+
+def check_transfers(s):
+    """Walks the scheduled block list the way the generated code runs and fails on: an upload from host
+    memory that holds no value (a transient nothing has written or downloaded into), a node or download
+    that uses a device buffer before it is allocated or after it is freed, a buffer freed twice or never."""
+    live, host_valid = set(), set(s.arguments)
+    for child in s._data["root"]["children"]:
+        flow, node = child["dataflow"], child["dataflow"]["library_node"]
+        ins = [b["data"] for b in flow["inputs"] if "data" in b]
+        outs = [b["data"] for b in flow["outputs"]]
+        if node["code"] == "ROCMOffloading":
+            direction, life = node["transfer_direction"], node["buffer_lifecycle"]
+            if life == 1:
+                assert outs[0] not in live, f"{outs[0]} allocated twice"
+                live.add(outs[0])
+            if direction == 1:
+                assert ins[0] in host_valid, f"upload from {ins[0]}, which holds no value"
+                assert outs[0] in live
+            if direction == -1:
+                assert ins[0] in live
+                host_valid.add(outs[0])
+            if life == -1:
+                assert ins[0] in live, f"{ins[0]} freed while not allocated"
+                live.discard(ins[0])
+        else:
+            for name in ins + outs:
+                if s.containers[name].get("storage") == "ROCM_Generic":
+                    assert name in live, f"{node['code']} uses {name} outside its lifetime"
+    assert not live, f"never freed: {sorted(live)}"
+    return host_valid
+
+
+def test_offloading_a_transient_with_two_readers(tmp_path):
+    """T = A @ B; Y = softmax(T); Z = T @ B: both readers of T, and both readers of B, use the buffers
+    the first node filled; nothing is uploaded from T's (never written) host memory."""
+    b = StructuredSDFGBuilder("two_readers")
+    for n in ("A", "B", "Y", "Z"):
+        b.add_container(n, F32, True)
+    b.add_container("T", F32, False, transient_bytes=64 * 64 * 4)
+    b.add_gemm("A", "B", "T", "1.0", "0.0", 64, 64, 64)
+    b.add_reduce_op("softmax", "T", "Y", [64, 64], [-1])
+    b.add_gemm("T", "B", "Z", "1.0", "0.0", 64, 64, 64)
+    s = b.move()
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 2 and r["D2H"] == 2                     # A, B up; Y, Z down
+    valid = check_transfers(s)
+    assert "T" not in valid and "size" not in s.containers["T"]
+    src, _ = source_of(s, tmp_path)
+    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")
+    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(") == 5   # A B T Y Z
+
+
+def test_offloading_longer_chains_keep_every_lifetime_whole(tmp_path):
+    """Reuse patterns the pairwise view of transfers gets wrong: three readers with other nodes in between,
+    a container rewritten between its readers, an argument written twice."""
+    b = StructuredSDFGBuilder("lifetimes")
+    for n in ("A", "B", "C", "Y"):
+        b.add_container(n, F32, True)
+    for n in ("T", "U", "V"):
+        b.add_container(n, F32, False, transient_bytes=32 * 32 * 4)
+    b.add_gemm("A", "B", "T", "1.0", "0.0", 32, 32, 32)         # T = A B
+    b.add_gemm("T", "B", "U", "1.0", "0.0", 32, 32, 32)         # U = T B
+    b.add_reduce_op("softmax", "T", "V", [32, 32], [-1])        # V = softmax(T)
+    b.add_gemm("T", "U", "C", "1.0", "0.0", 32, 32, 32)         # C = T U      (third reader of T)
+    b.add_gemm("V", "C", "T", "1.0", "0.0", 32, 32, 32)         # T = V C      (T rewritten)
+    b.add_gemm("T", "A", "C", "1.0", "0.0", 32, 32, 32)         # C = T A      (C written a second time)
+    b.add_reduce_op("softmax", "C", "Y", [32, 32], [-1])
+    s = b.move()
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 2                                        # A and B, once each
+    assert r["D2H"] == 2                                        # C once (its first value is never seen by the host) and Y
+    valid = check_transfers(s)
+    assert not ({"T", "U", "V"} & valid)
+    src, _ = source_of(s, tmp_path)
+    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(")
+
+
 def test_generated_function_honours_the_calling_convention(tmp_path):
     """Compiles an emitted function and calls it through ctypes the way CompiledSDFG does. Without a
     GPU the first runtime call fails; the function must return early and report through the failure
