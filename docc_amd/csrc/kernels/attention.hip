@@ -9,8 +9,8 @@
 // head in memory. This kernel never stores scores: it walks the keys in
 // blocks of 64 with an online max/sum (flash-attention style).
 //
-// Layout of the computation (one work-group = 128 queries of one head, four
-// wavefronts of 32 queries each; K and V blocks are shared through LDS):
+// Layout of the computation (one work-group = four wavefronts of one head, each with QT tiles of 32
+// queries: 256 queries per work-group with QT = 2, 128 with QT = 1; K and V blocks are shared through LDS):
 //   S^T[key, q]  = K_blk[key, d] * Q^T[d, q]     v_mfma_f32_32x32x16_bf16, A = K (d-contiguous
 //                                                128-bit LDS reads), B = Q (kept in registers)
 //   the transposed product puts one query per lane (column = lane % 32) and 32 of
@@ -23,21 +23,26 @@
 //                                                are (the k-order of the MFMA is permuted to
 //                                                the accumulator's row order on both operands).
 //
-// The softmax arithmetic, not the MFMAs, is the longer half of a block (32 scores per lane), so
-// it is cut to exp2, pack and sum:
-//   - scale*log2(e) is folded into Q once (Q' = bf16(Q * scale * log2e)), so the score product
-//     already yields log2-domain scores;
-//   - the reference point m of the online softmax rides in the MFMA's C operand: S' = K Q'^T - m,
-//     p = exp2(S') with no subtraction pass;
+// On this device the kernel runs against the power limit, not against a pipe: with pieces of the block loop
+// taken out one at a time its time falls by the share of the instructions removed, whatever pipe they ran on
+// (16 MFMAs 56 %, the eight 128-bit K reads 10 %, the sixteen transposed V reads 6 %, the copies 9 %, 16 dot2
+// 7.6 %, 32 exp 17 %, 32 fma 7 %), and overlapping them better (score MFMAs of the next block issued between the
+// exponentials) changes nothing. So the design goal is the fewest instructions per flop:
+//   - QT = 2: a wavefront takes 64 queries, so every K and V operand read from LDS, and every block copied
+//     into LDS, serves twice the MFMAs (LDS reads and copies per flop halve);
+//   - p = exp2(s * c - m) with c = scale * log2(e) applied to the fp32 score by one fma: Q and K enter
+//     the MFMA as they are (folding c into a re-rounded bf16 Q costs 2^-9 of every product, which at
+//     logits of +-60 is an error of 1.6e-2 in the result);
 //   - m does not have to be the exact running maximum: softmax is shift invariant and fp32/bf16
 //     keep their relative precision at any magnitude, so m stays what the first block set until a
-//     block's row sum shows growth beyond 2^40 (or inf) - only then the block takes the slow path
-//     (true block maximum, rescale of the output and the sum, recomputed p). The usual block has no
-//     max pass and no rescale;
-//   - p is packed to bf16 by one v_perm_b32 per pair (truncation) and the row sum is taken from the
-//     packed values with v_dot2c_f32_bf16: it sums exactly what the second product multiplies, so
-//     the truncation bias cancels in O = PV / sum.
-// K/V blocks arrive in a ring of LDS stages by asynchronous global->LDS copies.
+//     block's row sum shows growth beyond 2^40 (or inf, or NaN) - only then the block takes the slow
+//     path (scores recomputed, true block maximum, rescale of the output and the sum, p again). The usual
+//     block has no max pass and no rescale. A lane that has seen nothing but -inf scores so far keeps
+//     m = -inf, which makes its next block's sum inf or NaN and so leads it through the slow path until a
+//     finite score turns up;
+//   - p is packed to bf16 with v_cvt_pk_bf16_f32 and the row sum is taken from the packed values with
+//     v_dot2c_f32_bf16: it sums exactly what the second product multiplies.
+// K/V blocks arrive in a ring of three LDS stages by asynchronous global->LDS copies, two blocks ahead.
 #include "gemm_mfma.h"
 #include <type_traits>
 
@@ -58,7 +63,6 @@ struct Mfma<uint16_t> {
 };
 
 constexpr int kHeadDim = 64;
-constexpr int kBlockQ = 128;     // queries per work-group
 constexpr int kBlockKV = 64;     // keys per step
 constexpr int kAttnStages = 3;   // LDS ring depth: blocks kb+1 and kb+2 are in flight while block kb is worked on
 constexpr int kTileElems = kBlockKV * kHeadDim;          // one K or V block, unpadded, 16-byte granules swizzled
@@ -81,17 +85,18 @@ __device__ __forceinline__ float half_swap(float x, int which) {
     return __builtin_bit_cast(float, which ? sw[1] : sw[0]);
 }
 
-template <bool OUT_BF16>
+template <bool OUT_BF16, int QT>
 __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                                                   const uint16_t* __restrict__ V, void* __restrict__ O, int SQ,
                                                   int SKV, float scale_log2e) {
     extern __shared__ __attribute__((aligned(16))) unsigned char docc_attn_lds[];
     uint16_t* const lds = reinterpret_cast<uint16_t*>(docc_attn_lds);
+    constexpr int kBlockQ = 128 * QT;     // queries per work-group
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qj = lane & 31, g = lane >> 5;
     // work-group -> (head, query block): consecutive work-group ids go round the 8 XCDs, so the id is
-    // renumbered to give each XCD whole heads - the 16 query blocks of a head then share one L2
+    // renumbered to give each XCD whole heads - the query blocks of a head then share one L2
     const int nqb = gridDim.x, total = gridDim.x * gridDim.y;
     int lid = blockIdx.y * gridDim.x + blockIdx.x;
     if (total % 8 == 0) lid = (lid % 8) * (total / 8) + lid / 8;
@@ -100,55 +105,59 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const uint16_t* Qh = Q + bh * (long) SQ * kHeadDim;
     const char* Kh = reinterpret_cast<const char*>(K + bh * (long) SKV * kHeadDim);
     const char* Vh = reinterpret_cast<const char*>(V + bh * (long) SKV * kHeadDim);
-    const int q = qblk * kBlockQ + wave * 32 + qj;   // this lane's query
+    const int q0 = qblk * kBlockQ + wave * (32 * QT) + qj;   // this lane's queries: q0 + 32 * qt
+    const float c = scale_log2e;
+    const float ninf = -__builtin_huge_valf();
 
-    // Q'^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q, times scale*log2e
-    bf16x8 bq[4];
+    // Q^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q0 + 32*qt
+    bf16x8 bq[QT][4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-        u16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
-        if (q < SQ) v = *reinterpret_cast<const u16x8_t*>(Qh + (long) q * kHeadDim + 16 * ks + 8 * g);
+    for (int qt = 0; qt < QT; qt++)
 #pragma unroll
-        for (int e = 0; e < 8; e++) v[e] = f32_to_bf16_rne(bf16_bits_to_f32(v[e]) * scale_log2e);
-        bq[ks] = __builtin_bit_cast(bf16x8, v);
-    }
+        for (int ks = 0; ks < 4; ks++) {
+            u16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (q0 + 32 * qt < SQ) v = *reinterpret_cast<const u16x8_t*>(Qh + (long) (q0 + 32 * qt) * kHeadDim + 16 * ks + 8 * g);
+            bq[qt][ks] = __builtin_bit_cast(bf16x8, v);
+        }
 
     const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
     const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
 
     // K/V copies: a block is 512 granules of 16 bytes per tensor, two per thread. LDS slot s (in copy
-    // order: lane-contiguous) holds row s/8, granule column (s%8) ^ swizzle(row).
-    unsigned koff[2], voff[2];     // byte offsets of this lane's granules inside a full block
-    int krow[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int s = (i * 4 + wave) * 64 + lane;
-        const int row = s >> 3, cs = s & 7;
-        krow[i] = row;
-        koff[i] = (unsigned) ((row * 8 + (cs ^ ((row >> 1) & 7))) * 16);
-        voff[i] = (unsigned) ((row * 8 + (cs ^ (((row >> 1) & 1) << 2))) * 16);
-    }
+    // order: lane-contiguous) holds row s/8, granule column (s%8) ^ swizzle(row). The second granule of a
+    // lane lies 32 rows below the first, where both swizzles repeat: one offset per tensor serves both.
+    const int copy_row = wave * 8 + (lane >> 3);
+    const unsigned koff = (unsigned) ((copy_row * 8 + ((lane & 7) ^ ((copy_row >> 1) & 7))) * 16);
+    const unsigned voff = (unsigned) ((copy_row * 8 + ((lane & 7) ^ (((copy_row >> 1) & 1) << 2))) * 16);
     auto issue = [&](int kb) {   // starts the copy of block kb into its stage
         uint16_t* st = lds + (kb % kAttnStages) * kStageElems;
         const char* kp = Kh + (long) kb * (kTileElems * 2);
         const char* vp = Vh + (long) kb * (kTileElems * 2);
-        const bool partial = kb >= full_blocks;     // rows past the end copy the last key (scores masked, V zeroed below)
+        if (kb < full_blocks) {
+            // scalar base + 32-bit lane offset: the empty asm keeps the compiler from adding the head's base to
+            // the offsets once, outside the loop, which would cost 64-bit addresses per lane
+            unsigned ko = koff, vo = voff;
+            asm volatile("" : "+v"(ko), "+v"(vo));
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + ko), (attn_lds_ptr_t) (st + wave * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + vo), (attn_lds_ptr_t) (st + kTileElems + wave * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + 4096 + ko), (attn_lds_ptr_t) (st + (4 + wave) * 512), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + 4096 + vo), (attn_lds_ptr_t) (st + kTileElems + (4 + wave) * 512), 16, 0, 0);
+        } else {
+            // the partial last block: rows past the end copy the last key (their scores are masked, their V rows zeroed)
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            unsigned ko = koff[i], vo = voff[i];
-            if (partial && krow[i] >= keys_left) {
-                ko -= (unsigned) ((krow[i] - (keys_left - 1)) * 128);
-                vo -= (unsigned) ((krow[i] - (keys_left - 1)) * 128);
+            for (int i = 0; i < 2; i++) {
+                const int row = copy_row + 32 * i;
+                const unsigned back = row >= keys_left ? (unsigned) ((row - (keys_left - 1)) * 128) : 0u;
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + (koff + 4096u * i - back)), (attn_lds_ptr_t) (st + (i * 4 + wave) * 512), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + (voff + 4096u * i - back)), (attn_lds_ptr_t) (st + kTileElems + (i * 4 + wave) * 512), 16, 0, 0);
             }
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + ko), (attn_lds_ptr_t) (st + (i * 4 + wave) * 512), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + vo), (attn_lds_ptr_t) (st + kTileElems + (i * 4 + wave) * 512), 16, 0, 0);
         }
     };
-    // block kb has landed in every wave's view; rows of a partial last V block are cleared so that
-    // 0 * (copied value) cannot produce a NaN
-    auto arrive = [&](int kb, int newer_blocks) {
+    // block kb has landed in every wave's view and every wave is done with block kb-1; rows of a partial
+    // last V block are cleared so that 0 * (copied value) cannot produce a NaN
+    auto arrive = [&](int kb) {
         // each block is four copies per lane; one newer block may still be in flight
-        if (newer_blocks > 0) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        if (kb + 1 < nblocks) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -160,16 +169,18 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         }
     };
 
-    f32x16 ot[2];   // O^T tiles: d = 32*dt + acc_row(lane, r), column = this lane's query
+    f32x16 ot[QT][2];   // O^T tiles: d = 32*dt + acc_row(lane, r), column = this lane's query of tile qt
+    float m_run[QT];    // reference point of the exponentials (log2 domain); -inf: nothing finite seen yet
+    float l_part[QT];   // this lane's part of the running sum (its 32 keys per block)
 #pragma unroll
-    for (int dt = 0; dt < 2; dt++)
+    for (int qt = 0; qt < QT; qt++) {
+        m_run[qt] = ninf;
+        l_part[qt] = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; r++) ot[dt][r] = 0.f;
-    float m_run = 0.f;                      // reference point of the exponentials (log2 domain)
-    f32x16 negm;                            // -m_run in every register: the C operand of the score MFMAs
+        for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) negm[r] = 0.f;
-    float l_part = 0.f;                     // this lane's part of the running sum (its 32 keys per block)
+            for (int r = 0; r < 16; r++) ot[qt][dt][r] = 0.f;
+    }
 
     // lane roles for the transposed V reads (see gemm_bf16.hip)
     const int ts = lane & 15, tgrp = lane >> 4;
@@ -177,12 +188,12 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const int tr_col = 16 * (tgrp & 1) + 4 * (ts & 3);         // + 32*dt
     typedef __attribute__((address_space(3))) s16x4_t lds_s16x4;
 
-    f32x16 st[2];
+    const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-    // scores relative to the reference point, transposed: s[t][r] = <K[32t + acc_row(r)], Q'[q]> - m_run
-    auto scores = [&](int kb, f32x16 (&s)[2]) {
+    // raw scores, transposed: s[qt][t][r] = <K[32t + acc_row(r)], Q[q0 + 32 qt]>; keys past the end score -inf.
+    // All eight K operands are requested before the first MFMA: one LDS round trip, not eight; each serves QT MFMAs.
+    auto scores = [&](int kb, f32x16 (&s)[QT][2]) {
         const uint16_t* ks_ = lds + (kb % kAttnStages) * kStageElems;
-        // all eight K operands are requested before the first MFMA: one LDS round trip, not eight
         u16x8_t kv[2][4];
 #pragma unroll
         for (int t = 0; t < 2; t++)
@@ -193,89 +204,99 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         for (int ks = 0; ks < 4; ks++)
 #pragma unroll
             for (int t = 0; t < 2; t++)
-                s[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv[t][ks]), bq[ks], ks == 0 ? negm : s[t], 0, 0, 0);
+#pragma unroll
+                for (int qt = 0; qt < QT; qt++)
+                    s[qt][t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kv[t][ks]), bq[qt][ks],
+                                                                      ks == 0 ? zero16 : s[qt][t], 0, 0, 0);
+        if ((kb + 1) * kBlockKV > SKV) {
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (kb * kBlockKV + 32 * t + Mfma<float>::acc_row(lane, r) >= SKV) {
+#pragma unroll
+                        for (int qt = 0; qt < QT; qt++) s[qt][t][r] = ninf;
+                    }
+        }
     };
 
-    bf16x2_t pk[2][8];
-    // p = exp2(s), packed to bf16 pairs in accumulator order; returns this lane's row sum of the packed values
-    auto exponentials = [&](f32x16 (&s)[2]) {
-        bf16x2_t ones;
-        ones[0] = (__bf16) 1.0f;
-        ones[1] = (__bf16) 1.0f;
+    bf16x2_t pk[QT][2][8];
+    bf16x2_t ones;
+    ones[0] = (__bf16) 1.0f;
+    ones[1] = (__bf16) 1.0f;
+    // p = exp2(s*c - mc), packed to bf16 pairs in accumulator order; returns the lane's row sum of the packed values
+    auto exponentials = [&](const f32x16 (&s)[2], bf16x2_t (&pq)[2][8], float mc) {
         float psum = 0.f;
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
             for (int r = 0; r < 16; r += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(s[t][r]);
-                const float p1 = __builtin_amdgcn_exp2f(s[t][r + 1]);
-                const bf16x2_t pp = __builtin_bit_cast(bf16x2_t, __builtin_amdgcn_perm(__builtin_bit_cast(unsigned, p1), __builtin_bit_cast(unsigned, p0), 0x07060302u));
-                pk[t][r / 2] = pp;
+                bf16x2_t pp;
+                pp[0] = (__bf16) __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r], c, -mc));
+                pp[1] = (__bf16) __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][r + 1], c, -mc));
+                pq[t][r / 2] = pp;
                 psum = __builtin_amdgcn_fdot2_f32_bf16(pp, ones, psum, false);
             }
         return psum;
     };
+    // reference point a lane subtracts: 0 while it has seen no finite score (its scores are all -inf then, p = 0)
+    auto base_of = [&](float m) { return m == ninf ? 0.f : m; };
+    // the maximum of the scaled scores of the lane pair's query (c > 0)
+    auto scaled_max = [&](const f32x16 (&s)[2]) {
+        float mx = s[0][0];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
+        return fmaxf(half_swap(mx, 0), half_swap(mx, 1)) * c;
+    };
 
-    // one block: scores -> exponentials -> O^T += V^T P^T. Sized for three to four waves per SIMD: a
-    // wave issues an instruction only every 4-5 cycles, so the arithmetic of one wave needs the other
-    // waves' MFMAs and arithmetic to fill the pipes; the same waves hide the latency of the copies,
-    // which run one block ahead.
+    f32x16 st[QT][2];
+    // one block: scores -> exponentials -> O^T += V^T P^T
     auto block = [&](int kb, auto first_c) {
         constexpr bool FIRST = decltype(first_c)::value;
-        f32x16 (&s)[2] = st;
         // block kb must have landed; after the barrier every wave is done with block kb-1, whose
         // stage takes block kb+2
-        arrive(kb, kb + 1 < nblocks ? 1 : 0);
+        arrive(kb);
         if (kb + 2 < nblocks) issue(kb + 2);
-        scores(kb, s);
-        // keys past the end (last block only) score -inf
-        if ((kb + 1) * kBlockKV > SKV) {
+        scores(kb, st);
+        if (FIRST) {
+            // the first block sets the reference point
 #pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = kb * kBlockKV + 32 * t + Mfma<float>::acc_row(lane, r);
-                    if (key >= SKV) s[t][r] = -__builtin_huge_valf();
-                }
+            for (int qt = 0; qt < QT; qt++) m_run[qt] = scaled_max(st[qt]);
         }
-        const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
-        float psum = 0.f;
-        bool slow = FIRST;
-        if (!FIRST) {
-            psum = exponentials(s);
-            // growth of the maximum beyond 2^40 over the reference point (or an overflow) shows in the sum
-            slow = __builtin_amdgcn_ballot_w64(!(psum < 0x1p40f)) != 0;
+        float psum[QT];
+        bool slow = false;
+#pragma unroll
+        for (int qt = 0; qt < QT; qt++) {
+            psum[qt] = exponentials(st[qt], pk[qt], base_of(m_run[qt]));
+            // growth of the maximum beyond 2^40 over the reference point (or an overflow, or a NaN) shows in the sum
+            slow = slow || !(psum[qt] < 0x1p40f);
         }
-        if (slow) {
-            // move the reference point to the true maximum of what this lane pair has seen
-            float mx = s[0][0];
+        if (__builtin_amdgcn_ballot_w64(slow) != 0) {
+            // the slow path: the reference point moves to the maximum of what the lane pair has seen. The raw
+            // scores were consumed by the packing, so they are computed again (K of block kb is still in LDS).
+            scores(kb, st);
 #pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[t][r]);
-            mx = fmaxf(half_swap(mx, 0), half_swap(mx, 1));
-            const float d = FIRST ? mx : fmaxf(mx, 0.f);             // s is relative to m_run (0 in the first block)
-            const float alpha = FIRST ? 0.f : __builtin_amdgcn_exp2f(-d);
-            m_run += d;
-#pragma unroll
-            for (int r = 0; r < 16; r++) negm[r] = -m_run;
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) s[t][r] -= d;
-            if (!FIRST) {
-                l_part *= alpha;
+            for (int qt = 0; qt < QT; qt++) {
+                const float m_new = fmaxf(m_run[qt], scaled_max(st[qt]));     // fmaxf drops a NaN: it shows up in p instead
+                // exp2(-inf - -inf) would be NaN: a lane that still has nothing finite has nothing to rescale either
+                const float alpha = m_new == ninf ? 1.f : __builtin_amdgcn_exp2f(m_run[qt] - m_new);
+                m_run[qt] = m_new;
+                l_part[qt] *= alpha;
 #pragma unroll
                 for (int dt = 0; dt < 2; dt++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) ot[dt][r] *= alpha;
+                    for (int r = 0; r < 16; r++) ot[qt][dt][r] *= alpha;
+                psum[qt] = exponentials(st[qt], pk[qt], base_of(m_new));
             }
-            psum = exponentials(s);
         }
-        l_part += psum;
+#pragma unroll
+        for (int qt = 0; qt < QT; qt++) l_part[qt] += psum[qt];
 
         // O^T += V^T P^T, 16 keys per MFMA; key order inside a step follows the accumulator rows.
-        // The V operands of two MFMA pairs are requested together (they do not depend on P).
+        // The V operands of two steps are requested together (they do not depend on P); each serves QT MFMAs.
+        const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
         auto pv_half = [&](int h) {
             s16x8_t va[2][2];
 #pragma unroll
@@ -296,11 +317,15 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 #pragma unroll
             for (int uu = 0; uu < 2; uu++) {
                 const int u = 2 * h + uu;
-                struct Pack { bf16x2_t v[4]; } pack = {{pk[u >> 1][4 * (u & 1)], pk[u >> 1][4 * (u & 1) + 1], pk[u >> 1][4 * (u & 1) + 2], pk[u >> 1][4 * (u & 1) + 3]}};
-                const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
 #pragma unroll
-                for (int dt = 0; dt < 2; dt++)
-                    ot[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[uu][dt]), pb, ot[dt], 0, 0, 0);
+                for (int qt = 0; qt < QT; qt++) {
+                    struct Pack { bf16x2_t v[4]; } pack = {{pk[qt][u >> 1][4 * (u & 1)], pk[qt][u >> 1][4 * (u & 1) + 1],
+                                                            pk[qt][u >> 1][4 * (u & 1) + 2], pk[qt][u >> 1][4 * (u & 1) + 3]}};
+                    const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
+#pragma unroll
+                    for (int dt = 0; dt < 2; dt++)
+                        ot[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[uu][dt]), pb, ot[qt][dt], 0, 0, 0);
+                }
             }
         };
         pv_half(0);
@@ -312,25 +337,29 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     block(0, std::true_type{});
     for (int kb = 1; kb < nblocks; kb++) block(kb, std::false_type{});
 
-    const float l = half_swap(l_part, 0) + half_swap(l_part, 1);
-    const float inv = 1.0f / l;
-    if (q < SQ) {
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++) {
+    for (int qt = 0; qt < QT; qt++) {
+        const int q = q0 + 32 * qt;
+        const float l = half_swap(l_part[qt], 0) + half_swap(l_part[qt], 1);
+        const float inv = 1.0f / l;
+        if (q < SQ) {
 #pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                const int d = 32 * dt + 8 * rq + 4 * g;   // registers 4*rq .. 4*rq+3 hold d .. d+3
-                const long off = (bh * (long) SQ + q) * kHeadDim + d;
-                if (OUT_BF16) {
-                    u16x4_t o;
+            for (int dt = 0; dt < 2; dt++) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = f32_to_bf16_rne(ot[dt][4 * rq + e] * inv);
-                    *reinterpret_cast<u16x4_t*>(reinterpret_cast<uint16_t*>(O) + off) = o;
-                } else {
-                    f32x4 o;
+                for (int rq = 0; rq < 4; rq++) {
+                    const int d = 32 * dt + 8 * rq + 4 * g;   // registers 4*rq .. 4*rq+3 hold d .. d+3
+                    const long off = (bh * (long) SQ + q) * kHeadDim + d;
+                    if (OUT_BF16) {
+                        u16x4_t o;
 #pragma unroll
-                    for (int e = 0; e < 4; e++) o[e] = ot[dt][4 * rq + e] * inv;
-                    *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(O) + off) = o;
+                        for (int e = 0; e < 4; e++) o[e] = f32_to_bf16_rne(ot[qt][dt][4 * rq + e] * inv);
+                        *reinterpret_cast<u16x4_t*>(reinterpret_cast<uint16_t*>(O) + off) = o;
+                    } else {
+                        f32x4 o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = ot[qt][dt][4 * rq + e] * inv;
+                        *reinterpret_cast<f32x4*>(reinterpret_cast<float*>(O) + off) = o;
+                    }
                 }
             }
         }
@@ -339,14 +368,15 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
 } // namespace docc_k
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void docc_attention_bf16_d64_f32out(const uint16_t* Q, const uint16_t* K,
-                                                                                 const uint16_t* V, void* O, int SQ,
-                                                                                 int SKV, float scale_log2e) {
-    docc_k::attention_fwd_d64<false>(Q, K, V, O, SQ, SKV, scale_log2e);
-}
+#define DOCC_ATTENTION_KERNEL(name, out_bf16, qt, waves)                                                                          \
+    extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(waves))) void name(                           \
+        const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int SQ, int SKV, float scale_log2e) {                   \
+        docc_k::attention_fwd_d64<out_bf16, qt>(Q, K, V, O, SQ, SKV, scale_log2e);                                                \
+    }
 
-extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3))) void docc_attention_bf16_d64_bf16out(const uint16_t* Q, const uint16_t* K,
-                                                                                  const uint16_t* V, void* O, int SQ,
-                                                                                  int SKV, float scale_log2e) {
-    docc_k::attention_fwd_d64<true>(Q, K, V, O, SQ, SKV, scale_log2e);
-}
+// 64 queries per wavefront (256 per work-group): the form for long query axes
+DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q256_f32out, false, 2, 2)
+DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q256_bf16out, true, 2, 2)
+// 32 queries per wavefront (128 per work-group): more work-groups where there are few queries
+DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q128_f32out, false, 1, 3)
+DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q128_bf16out, true, 1, 3)

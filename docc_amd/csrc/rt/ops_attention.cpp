@@ -1,5 +1,6 @@
 // Launcher for ml::Attention (see include/docc_rocm_ops.h).
 #include <cmath>
+#include <cstdlib>
 
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
@@ -23,13 +24,23 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
     // LDS: ring of 3 stages x (K block [64][64] + V block [64][64]) bf16
     const uint32_t lds = 3 * (2 * 64 * 64) * 2;
     const float scale_log2e = scale * 1.4426950408889634f;
-    // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
+    // Two forms: 256 queries per work-group (a wavefront takes 64, so each K/V operand read from LDS serves two
+    // MFMAs: fewer instructions per flop) once that still gives every CU its two resident work-groups, else 128
+    // per work-group (more, smaller work-groups). DOCC_ROCM_ATTENTION_Q=128|256 forces one (tuning and tests).
     const int64_t BH = B * H, out_bytes = out_bf16 ? 2 : 4;
+    int per_group = ((SQ + 255) / 256) * BH >= 2 * compute_units() ? 256 : 128;
+    if (const char* force = std::getenv("DOCC_ROCM_ATTENTION_Q")) {
+        const int v = std::atoi(force);
+        if (v == 128 || v == 256) per_group = v;
+    }
+    const char* kernel = per_group == 256 ? (out_bf16 ? "docc_attention_bf16_d64_q256_bf16out" : "docc_attention_bf16_d64_q256_f32out")
+                                          : (out_bf16 ? "docc_attention_bf16_d64_q128_bf16out" : "docc_attention_bf16_d64_q128_f32out");
+    // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
     for (int64_t h0 = 0; h0 < BH; h0 += 65535) {
         const int64_t nh = BH - h0 < 65535 ? BH - h0 : 65535;
-        rc = launch(out_bf16 ? "docc_attention_bf16_d64_bf16out" : "docc_attention_bf16_d64_f32out", (uint32_t) ((SQ + 127) / 128),
-                    (uint32_t) nh, 1, 256, lds, (hipStream_t) stream, Q + h0 * SQ * 64, K + h0 * SKV * 64, V + h0 * SKV * 64,
-                    (void*) ((char*) O + h0 * SQ * 64 * out_bytes), (int) SQ, (int) SKV, scale_log2e);
+        rc = launch(kernel, (uint32_t) ((SQ + per_group - 1) / per_group), (uint32_t) nh, 1, 256, lds, (hipStream_t) stream,
+                    Q + h0 * SQ * 64, K + h0 * SKV * 64, V + h0 * SKV * 64, (void*) ((char*) O + h0 * SQ * 64 * out_bytes), (int) SQ,
+                    (int) SKV, scale_log2e);
         if (rc) return rc;
     }
     return 0;

@@ -14,6 +14,16 @@ pytestmark = pytest.mark.gpu
 TOL_BF16 = 2e-2
 
 
+@pytest.fixture(autouse=True, params=["128", "256", None], ids=["q128", "q256", "auto"])
+def kernel_form(request, monkeypatch):
+    """Every test runs with 128 and with 256 queries per work-group forced, and with the launcher's own choice."""
+    if request.param is None:
+        monkeypatch.delenv("DOCC_ROCM_ATTENTION_Q", raising=False)
+    else:
+        monkeypatch.setenv("DOCC_ROCM_ATTENTION_Q", request.param)
+    return request.param
+
+
 def bits(t: torch.Tensor) -> np.ndarray:
     return t.contiguous().view(torch.int16).numpy().view(np.uint16)
 
@@ -149,6 +159,15 @@ def test_attention_infinite_and_nan_scores(rt):
         assert np.array_equal(np.isnan(O), np.isnan(ref))
         ok = np.isfinite(ref)
         assert rel_err_max(np.where(ok, O, 0.0), np.where(ok, ref, 0.0)) <= TOL_BF16
+
+
+def test_attention_is_deterministic(rt):
+    """The same inputs give the same bits on every launch (no order of arrival enters the sums)."""
+    g = torch.Generator().manual_seed(21)
+    Q, K, V = (torch.randn(2, 4, 520, 64, generator=g).bfloat16() for _ in range(3))
+    first = run_attention(rt, bits(Q), bits(K), bits(V))
+    for _ in range(5):
+        assert np.array_equal(run_attention(rt, bits(Q), bits(K), bits(V)), first)
 
 
 def test_attention_errors(rt):
