@@ -5,16 +5,13 @@
 //   rows   y[i] = alpha * <M[i, :], x> + beta * y[i]      the matrix's rows are contiguous: one wavefront per row,
 //          128-bit loads, the vector comes from the caches;
 //   cols   y[j] = alpha * sum_p x[p] * M[p, j] + beta * y[j]   a lane owns columns (contiguous across lanes), the
-//          rows are cut into slices over work-groups whose partial sums meet in a scratch array; a second
+//          rows are cut into slices over work-groups whose partial sums meet in a buffer of the launcher; a second
 //          launch adds them in slice order, so the result does not depend on scheduling.
 // fp32 sums in fp32, fp64 in fp64 (cblas_?gemm semantics, reference gemm_node.cpp:474-505), bf16 operands (raw
 // 16-bit words) in fp32 with an fp32 result, like the bf16 GEMM; when beta == 0, y is not read.
 #include "common.h"
 
 namespace docc_k {
-
-constexpr long kGemvScratchBytes = 8l << 20;
-__device__ __attribute__((aligned(256))) unsigned char docc_gemv_scratch[kGemvScratchBytes];
 
 template <typename T>
 __device__ __forceinline__ T gemv_wave_sum(T v) {
@@ -140,10 +137,10 @@ __device__ __forceinline__ void gemv_rows_multi(const In* __restrict__ M, long l
 
 // partial sums of rows [slice * chunk, ...) for VEC columns per lane; P[slice][col]
 template <typename In, typename T, int VEC>
-__device__ __forceinline__ void gemv_cols_partial(const In* __restrict__ M, long ld, const In* __restrict__ x, long incx, long rows, long cols,
+__device__ __forceinline__ void gemv_cols_partial(void* partials, const In* __restrict__ M, long ld, const In* __restrict__ x, long incx, long rows, long cols,
                                                   long chunk) {
     typedef In V __attribute__((ext_vector_type(VEC)));
-    T* P = reinterpret_cast<T*>(docc_gemv_scratch);
+    T* P = reinterpret_cast<T*>(partials);
     const long col = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
     if (col >= cols) return;
     const long r0 = (long) blockIdx.y * chunk;
@@ -176,12 +173,12 @@ __device__ __forceinline__ void gemv_cols_partial(const In* __restrict__ M, long
 // The columns form for a few vectors at once (a small batch times a weight matrix stored [k][n], y = x W):
 // P[slice][v][col] = sum over the slice's rows p of X[v * sx_v + p * sx_p] * M[p, col]; the matrix moves once.
 template <typename In, typename T, int VEC, int NV>
-__device__ __forceinline__ void gemv_cols_partial_multi(const In* __restrict__ M, long ld, const In* __restrict__ X, long sx_v, long sx_p, int nv,
+__device__ __forceinline__ void gemv_cols_partial_multi(void* partials, const In* __restrict__ M, long ld, const In* __restrict__ X, long sx_v, long sx_p, int nv,
                                                         long rows, long cols, long chunk) {
     typedef In V __attribute__((ext_vector_type(VEC)));
     constexpr int STEP = 64;            // rows of the slice whose vector entries sit in LDS at a time
     __shared__ T xs[STEP][NV];
-    T* P = reinterpret_cast<T*>(docc_gemv_scratch);
+    T* P = reinterpret_cast<T*>(partials);
     const long col = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
     const bool live = col < cols;
     const long r0 = (long) blockIdx.y * chunk;
@@ -228,11 +225,11 @@ __device__ __forceinline__ void gemv_cols_partial_multi(const In* __restrict__ M
 
 // y[v * sy_vec + col * sy_col] = alpha * (sum over the slices of P[s][v][col]) + beta * y[..]; entries = nv * cols
 template <typename T>
-__device__ __forceinline__ void gemv_cols_final_multi(T* __restrict__ y, long sy_vec, long sy_col, long cols, long entries, int slices, T alpha,
+__device__ __forceinline__ void gemv_cols_final_multi(const void* partials, T* __restrict__ y, long sy_vec, long sy_col, long cols, long entries, int slices, T alpha,
                                                       T beta) {
     // 64 neighbouring entries per work-group (256-byte segments of every slice), the slices dealt to its four waves
     __shared__ T part[4][64];
-    const T* P = reinterpret_cast<const T*>(docc_gemv_scratch);
+    const T* P = reinterpret_cast<const T*>(partials);
     const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
     const long e = (long) blockIdx.x * 64 + c;
     T acc = (T) 0;
@@ -250,11 +247,11 @@ __device__ __forceinline__ void gemv_cols_final_multi(T* __restrict__ y, long sy
 }
 
 template <typename T>
-__device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, long cols, int slices, T alpha, T beta) {
+__device__ __forceinline__ void gemv_cols_final(const void* partials, T* __restrict__ y, long incy, long cols, int slices, T alpha, T beta) {
     // a work-group takes 16 neighbouring columns; 16 lanes per column each add every 16th slice, then one lane
     // adds the 16 sums in order: the order of the additions is fixed by the launch geometry alone
     __shared__ T part[16][17];
-    const T* P = reinterpret_cast<const T*>(docc_gemv_scratch);
+    const T* P = reinterpret_cast<const T*>(partials);
     const int c = threadIdx.x & 15, g = threadIdx.x >> 4;
     const long col = (long) blockIdx.x * 16 + c;
     T acc = (T) 0;
@@ -278,9 +275,9 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
                                                                                      long incy, long rows, long k, T alpha, T beta) { \
         docc_k::gemv_rows<In, T, VEC>(M, ld, x, incx, y, incy, rows, k, alpha, beta);                                                  \
     }                                                                                                                                 \
-    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colp_##NAME##_v##VEC(const In* M, long ld, const In* x, long incx,      \
-                                                                                     long rows, long cols, long chunk) {              \
-        docc_k::gemv_cols_partial<In, T, VEC>(M, ld, x, incx, rows, cols, chunk);                                                      \
+    extern "C" __global__ __launch_bounds__(256) void docc_gemv_colp_##NAME##_v##VEC(void* partials, const In* M, long ld, const In* x, \
+                                                                                     long incx, long rows, long cols, long chunk) {   \
+        docc_k::gemv_cols_partial<In, T, VEC>(partials, M, ld, x, incx, rows, cols, chunk);                                            \
     }
 #define DOCC_GEMV_MULTI(NAME, In, T, VEC, NV)                                                                                          \
     extern "C" __global__ __launch_bounds__(256) void docc_gemv_rowsm_##NAME##_v##VEC##_n##NV(                                          \
@@ -296,8 +293,8 @@ __device__ __forceinline__ void gemv_cols_final(T* __restrict__ y, long incy, lo
 // the columns form of the same; fp32 and fp64 only (for bf16 the MFMA tiles are as fast)
 #define DOCC_GEMV_MULTI_COLS(NAME, In, T, VEC, NV)                                                                                     \
     extern "C" __global__ __launch_bounds__(256) void docc_gemv_colpm_##NAME##_v##VEC##_n##NV(                                          \
-        const In* M, long ld, const In* X, long sx_v, long sx_p, int nv, long rows, long cols, long chunk) {                          \
-        docc_k::gemv_cols_partial_multi<In, T, VEC, NV>(M, ld, X, sx_v, sx_p, nv, rows, cols, chunk);                                  \
+        void* partials, const In* M, long ld, const In* X, long sx_v, long sx_p, int nv, long rows, long cols, long chunk) {          \
+        docc_k::gemv_cols_partial_multi<In, T, VEC, NV>(partials, M, ld, X, sx_v, sx_p, nv, rows, cols, chunk);                        \
     }
 #define DOCC_GEMV_MULTI_ALL(NAME, In, T, VEC) \
     DOCC_GEMV_MULTI(NAME, In, T, VEC, 2) DOCC_GEMV_MULTI(NAME, In, T, VEC, 4) DOCC_GEMV_MULTI(NAME, In, T, VEC, 8)
@@ -325,17 +322,19 @@ DOCC_GEMV(f64, double, double, 1)
 DOCC_GEMV(bf16, unsigned short, float, 8)
 DOCC_GEMV(bf16, unsigned short, float, 1)
 
-extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f32(float* y, long incy, long cols, int slices, float alpha, float beta) {
-    docc_k::gemv_cols_final<float>(y, incy, cols, slices, alpha, beta);
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f32(const void* partials, float* y, long incy, long cols, int slices, float alpha,
+                                                                     float beta) {
+    docc_k::gemv_cols_final<float>(partials, y, incy, cols, slices, alpha, beta);
 }
-extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f64(double* y, long incy, long cols, int slices, double alpha, double beta) {
-    docc_k::gemv_cols_final<double>(y, incy, cols, slices, alpha, beta);
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colf_f64(const void* partials, double* y, long incy, long cols, int slices, double alpha,
+                                                                     double beta) {
+    docc_k::gemv_cols_final<double>(partials, y, incy, cols, slices, alpha, beta);
 }
-extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f32(float* y, long sy_vec, long sy_col, long cols, long entries, int slices,
-                                                                      float alpha, float beta) {
-    docc_k::gemv_cols_final_multi<float>(y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f32(const void* partials, float* y, long sy_vec, long sy_col, long cols, long entries,
+                                                                      int slices, float alpha, float beta) {
+    docc_k::gemv_cols_final_multi<float>(partials, y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
 }
-extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f64(double* y, long sy_vec, long sy_col, long cols, long entries, int slices,
-                                                                      double alpha, double beta) {
-    docc_k::gemv_cols_final_multi<double>(y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
+extern "C" __global__ __launch_bounds__(256) void docc_gemv_colfm_f64(const void* partials, double* y, long sy_vec, long sy_col, long cols, long entries,
+                                                                      int slices, double alpha, double beta) {
+    docc_k::gemv_cols_final_multi<double>(partials, y, sy_vec, sy_col, cols, entries, slices, alpha, beta);
 }

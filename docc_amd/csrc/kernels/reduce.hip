@@ -11,7 +11,7 @@
 //   inner  > 1  one lane per output element, walking the reduced extent with stride `inner`, so
 //               that neighbouring lanes read neighbouring addresses; when there are too few
 //               output elements to fill the device the reduced extent is cut into slices, one
-//               work-group row per slice, whose partial results go through a scratch array in
+//               work-group row per slice, whose partial results go through a buffer of the launcher in
 //               device memory and are combined, in slice order, by a second launch
 // Sums are therefore added in another order than the reference's loop: equal to it within the
 // usual bound (reduce * epsilon * sum|x|), exactly equal for Max and Min.
@@ -95,19 +95,17 @@ __device__ __forceinline__ void column_reduce(const T* X, T* Y, long outer, long
     }
 }
 
-// Partial results of the sliced column reduction: [slice][outer * inner] elements. Every call
-// that slices writes the part it reads back, so nothing has to be cleared; calls that overlap
-// on one device (different streams) would share it and must not.
-constexpr long kReduceScratchBytes = 8L << 20;
-__device__ __attribute__((aligned(256))) unsigned char docc_reduce_scratch[kReduceScratchBytes];
+// Partial results of the sliced column reduction live in `partials`, device memory of the launcher:
+// [slice][outer * inner] elements. Every call that slices writes the part it reads back, so nothing has
+// to be cleared.
 
 // P[s, o, i] = reduce over the rows of slice s of X[o, r, i]; grid.y = number of slices. Each lane
 // owns VEC neighbouring columns (inner % VEC == 0, X 16-byte aligned when VEC > 1): one 128-bit load
 // per row.
 template <typename T, int OP, int VEC>
-__device__ __forceinline__ void column_reduce_partial(const T* X, long outer, long R, long inner, long chunk) {
+__device__ __forceinline__ void column_reduce_partial(void* partials, const T* X, long outer, long R, long inner, long chunk) {
     typedef T V __attribute__((ext_vector_type(VEC)));
-    T* P = reinterpret_cast<T*>(docc_reduce_scratch);
+    T* P = reinterpret_cast<T*>(partials);
     const long total = outer * inner;
     const long idx = ((long) blockIdx.x * blockDim.x + threadIdx.x) * VEC;
     if (idx >= total) return;
@@ -141,9 +139,9 @@ __device__ __forceinline__ void column_reduce_partial(const T* X, long outer, lo
 // elements; 16 lanes per element each combine every 16th slice, then one lane combines the 16
 // partial values in order (the order of the additions is fixed by the launch geometry alone).
 template <typename T, int OP>
-__device__ __forceinline__ void column_reduce_final(T* Y, long total, long R, long slices) {
+__device__ __forceinline__ void column_reduce_final(const void* partials, T* Y, long total, long R, long slices) {
     __shared__ T part[16][17];
-    const T* P = reinterpret_cast<const T*>(docc_reduce_scratch);
+    const T* P = reinterpret_cast<const T*>(partials);
     const int col = threadIdx.x & 15, lane_s = threadIdx.x >> 4;
     const long idx = (long) blockIdx.x * 16 + col;
     T a = reduce_identity<OP, T>();
@@ -180,16 +178,17 @@ __device__ __forceinline__ void column_reduce_final(T* Y, long total, long R, lo
     }
 
 #define DOCC_REDUCE_SLICED(NAME, OP, SFX, T)                                                                                   \
-    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colp_##NAME##_##SFX(const T* X, long outer, long R, long inner, \
-                                                                                      long chunk) {                            \
-        docc_k::column_reduce_partial<T, docc_k::OP, 1>(X, outer, R, inner, chunk);                                            \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colp_##NAME##_##SFX(void* partials, const T* X, long outer, long R, \
+                                                                                      long inner, long chunk) {                \
+        docc_k::column_reduce_partial<T, docc_k::OP, 1>(partials, X, outer, R, inner, chunk);                                  \
     }                                                                                                                          \
-    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colpv_##NAME##_##SFX(const T* X, long outer, long R,            \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colpv_##NAME##_##SFX(void* partials, const T* X, long outer, long R, \
                                                                                        long inner, long chunk) {               \
-        docc_k::column_reduce_partial<T, docc_k::OP, 16 / sizeof(T)>(X, outer, R, inner, chunk);                               \
+        docc_k::column_reduce_partial<T, docc_k::OP, 16 / sizeof(T)>(partials, X, outer, R, inner, chunk);                     \
     }                                                                                                                          \
-    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colf_##NAME##_##SFX(T* Y, long total, long R, long slices) {    \
-        docc_k::column_reduce_final<T, docc_k::OP>(Y, total, R, slices);                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_colf_##NAME##_##SFX(const void* partials, T* Y, long total, long R, \
+                                                                                      long slices) {                           \
+        docc_k::column_reduce_final<T, docc_k::OP>(partials, Y, total, R, slices);                                             \
     }
 
 DOCC_REDUCE(sum, kSum)

@@ -331,11 +331,9 @@ __device__ __forceinline__ void softmax_strided_slab(const T* X, T* Y, long redu
 
 // Few columns and a long reduced extent leave the tile kernel with a handful of work-groups that each walk
 // the whole extent twice. The sliced pair spreads the rows as well: work-group (outer index, slice of rows,
-// 64-column tile) first leaves its running (maximum, sum) pairs in the scratch array below, then - in a second
+// 64-column tile) first leaves its running (maximum, sum) pairs in a buffer of the launcher, then - in a second
 // launch - every work-group merges the pairs of all slices of its columns and writes the results of its own
-// slice. The scratch array is shared by every such call on the device.
-constexpr long kSoftmaxScratchBytes = 8l << 20;
-__device__ __attribute__((aligned(256))) unsigned char docc_softmax_scratch[kSoftmaxScratchBytes];
+// slice. The pairs live in `partials`, device memory of the launcher: [outer][slice][column] x (maximum, sum).
 
 struct SlicedWork {
     long o, col, r0, r1;   // outer index, this lane's column, rows [r0, r1) of the slice
@@ -359,7 +357,7 @@ __device__ __forceinline__ SlicedWork sliced_work(long reduce, long inner, long 
 }
 
 template <typename T>
-__device__ __forceinline__ void softmax_sliced_partial(const T* X, long reduce, long inner, long tiles, int slices) {
+__device__ __forceinline__ void softmax_sliced_partial(void* partials, const T* X, long reduce, long inner, long tiles, int slices) {
     using M = SoftmaxMath<T>;
     __shared__ T lm[256];
     __shared__ T ls[256];
@@ -378,7 +376,7 @@ __device__ __forceinline__ void softmax_sliced_partial(const T* X, long reduce, 
         for (int i = 0; i < 4; i++) gm = M::max(gm, lm[(threadIdx.x & 63) + 64 * i]);
         T gs = (T) 0;
         for (int i = 0; i < 4; i++) gs += pair_weight(lm[(threadIdx.x & 63) + 64 * i], ls[(threadIdx.x & 63) + 64 * i], gm);
-        T* P = reinterpret_cast<T*>(docc_softmax_scratch);
+        T* P = reinterpret_cast<T*>(partials);
         const long at = ((w.o * slices + w.slice) * inner + w.col) * 2;
         P[at] = gm;
         P[at + 1] = gs;
@@ -386,13 +384,13 @@ __device__ __forceinline__ void softmax_sliced_partial(const T* X, long reduce, 
 }
 
 template <typename T>
-__device__ __forceinline__ void softmax_sliced_finish(const T* X, T* Y, long reduce, long inner, long tiles, int slices) {
+__device__ __forceinline__ void softmax_sliced_finish(const void* partials, const T* X, T* Y, long reduce, long inner, long tiles, int slices) {
     using M = SoftmaxMath<T>;
     __shared__ T lm[256];
     __shared__ T ls[256];
     const SlicedWork w = sliced_work(reduce, inner, tiles, slices);
     const int part = threadIdx.x >> 6;
-    const T* P = reinterpret_cast<const T*>(docc_softmax_scratch);
+    const T* P = reinterpret_cast<const T*>(partials);
     // the four waves share the slices of this column
     T m = M::neg_inf(), s = (T) 0;
     if (w.live)
@@ -417,13 +415,14 @@ __device__ __forceinline__ void softmax_sliced_finish(const T* X, T* Y, long red
 } // namespace
 
 #define DOCC_SOFTMAX_SLICED(T, SUFFIX)                                                                                        \
-    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_partial(const T* X, long reduce, long inner, \
-                                                                                            long tiles, int slices) {       \
-        softmax_sliced_partial<T>(X, reduce, inner, tiles, slices);                                                           \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_partial(void* partials, const T* X, long reduce, \
+                                                                                            long inner, long tiles, int slices) { \
+        softmax_sliced_partial<T>(partials, X, reduce, inner, tiles, slices);                                                 \
     }                                                                                                                         \
-    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_finish(const T* X, T* Y, long reduce,       \
-                                                                                           long inner, long tiles, int slices) { \
-        softmax_sliced_finish<T>(X, Y, reduce, inner, tiles, slices);                                                         \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_finish(const void* partials, const T* X, T* Y, \
+                                                                                           long reduce, long inner, long tiles, \
+                                                                                           int slices) {                      \
+        softmax_sliced_finish<T>(partials, X, Y, reduce, inner, tiles, slices);                                               \
     }
 DOCC_SOFTMAX_SLICED(float, f32)
 DOCC_SOFTMAX_SLICED(double, f64)

@@ -65,7 +65,7 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
             int64_t cheap = k * (int64_t) sizeof(T) / (16 * (int64_t) sizeof(S) * group);
             if (cheap * col_blocks < 4 * (int64_t) cusm) cheap *= 2;      // ... unless that leaves the chip short of work-groups
             if (slices > cheap) slices = cheap;
-            const int64_t fit = (int64_t(8) << 20) / ((int64_t) sizeof(S) * cols * group);
+            const int64_t fit = (int64_t) kPartialsBytes / ((int64_t) sizeof(S) * cols * group);
             if (slices > fit) slices = fit;
             if (slices > 256) slices = 256;
             if (slices < 1 || col_blocks > 0x7fffffffLL) return 1;
@@ -74,15 +74,17 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
             // five to eight vectors go as two passes of at most four: two reads of the matrix beat one with eight sums a lane
             char kname[64], fname[64];
             std::snprintf(fname, sizeof(fname), "docc_gemv_colfm_f%d", (int) sizeof(S) * 8);
+            PartialsLease partials;
+            if (int rcp = partials_for(s, &partials)) return rcp;
             for (int64_t v0 = 0; v0 < nv; v0 += 4) {
                 const int64_t gv = nv - v0 < 4 ? nv - v0 : 4;
                 std::snprintf(kname, sizeof(kname), "docc_gemv_colpm_%s_v%d_n%d", sizeof(T) == 4 ? "f32" : "f64", lanes, gv <= 2 ? 2 : 4);
-                int rcm = launch(kname, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, mat, (long) ldm, vecs + v0 * sx_v, (long) sx_v,
-                                 (long) sx_p, (int) gv, (long) k, (long) cols, (long) chunk);
+                int rcm = launch(kname, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, partials.ptr, mat, (long) ldm, vecs + v0 * sx_v,
+                                 (long) sx_v, (long) sx_p, (int) gv, (long) k, (long) cols, (long) chunk);
                 if (rcm) return rcm;
                 const int64_t entries = gv * cols;
-                rcm = launch(fname, (uint32_t) ((entries + 63) / 64), 1, 1, 256, 0, s, C + v0 * sy_vec, (long) sy_vec, (long) sy_col,
-                             (long) cols, (long) entries, (int) slices, alpha, beta);
+                rcm = launch(fname, (uint32_t) ((entries + 63) / 64), 1, 1, 256, 0, s, (const void*) partials.ptr, C + v0 * sy_vec, (long) sy_vec,
+                             (long) sy_col, (long) cols, (long) entries, (int) slices, alpha, beta);
                 if (rcm) return rcm;
             }
             return 0;
@@ -140,26 +142,29 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
                       (long) cols, alpha, beta);
     }
     // columns form: lanes own columns, the rows are sliced so that about eight work-groups per CU share the matrix;
-    // the slices' sums meet in the kernels' 8 MiB scratch array
+    // the slices' sums meet in the stream's partial-results buffer
     if (cols < 256 || rows < 64) return 1;
     const bool aligned = (uintptr_t) M % 16 == 0 && ld % vec == 0 && cols % vec == 0;
     const int lanes = aligned ? vec : 1;
     const int64_t col_blocks = (cols / lanes + 255) / 256;
     int64_t slices = (8 * (int64_t) cus + col_blocks - 1) / col_blocks;
     if (slices > rows / 16) slices = rows / 16;
-    const int64_t fit = (int64_t(8) << 20) / ((int64_t) sizeof(S) * cols);
+    const int64_t fit = (int64_t) kPartialsBytes / ((int64_t) sizeof(S) * cols);
     if (slices > fit) slices = fit;
     if (slices > 256) slices = 256;
     if (slices < 1) return 1;
     const int64_t chunk = (rows + slices - 1) / slices;
     slices = (rows + chunk - 1) / chunk;
     if (col_blocks > 0x7fffffffLL || slices > 65535) return 1;
+    PartialsLease partials;
+    if (int rcp = partials_for(s, &partials)) return rcp;
     std::snprintf(name, sizeof(name), "docc_gemv_colp_%s_v%d", type, lanes);
-    int rc = launch(name, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, M, (long) ld, x, (long) incx, (long) rows, (long) cols,
-                    (long) chunk);
+    int rc = launch(name, (uint32_t) col_blocks, (uint32_t) slices, 1, 256, 0, s, partials.ptr, M, (long) ld, x, (long) incx, (long) rows,
+                    (long) cols, (long) chunk);
     if (rc) return rc;
     std::snprintf(name, sizeof(name), "docc_gemv_colf_f%d", bits);
-    return launch(name, (uint32_t) ((cols + 15) / 16), 1, 1, 256, 0, s, C, (long) incy, (long) cols, (int) slices, alpha, beta);
+    return launch(name, (uint32_t) ((cols + 15) / 16), 1, 1, 256, 0, s, (const void*) partials.ptr, C, (long) incy, (long) cols, (int) slices,
+                  alpha, beta);
 }
 
 // T: element type of A and B; S: type of C, alpha and beta

@@ -34,12 +34,12 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
     const int64_t total = outer * inner;
     int64_t blocks = (total + 255) / 256;
     // Too few output elements to fill the device: cut the reduced extent into slices. Their partial
-    // results go through the kernels' 8 MiB scratch array (docc_reduce_scratch in reduce.hip).
+    // results go through the stream's partial-results buffer.
     if (blocks < (int64_t) cus * 2 && reduce >= 64) {
         const int per_vec = 128 / precision;
         const bool vec = inner % per_vec == 0 && (uintptr_t) X % 16 == 0;
         const int64_t pblocks = vec ? (total / per_vec + 255) / 256 : blocks;
-        const int64_t scratch_elems = (int64_t(8) << 20) / (precision / 8);
+        const int64_t scratch_elems = (int64_t) kPartialsBytes / (precision / 8);
         int64_t slices = ((int64_t) cus * 8 + pblocks - 1) / pblocks;
         if (slices > reduce / 16) slices = reduce / 16;
         if (slices > scratch_elems / total) slices = scratch_elems / total;
@@ -47,14 +47,16 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
         if (slices > 1) {
             const int64_t chunk = (reduce + slices - 1) / slices;
             slices = (reduce + chunk - 1) / chunk;
+            PartialsLease partials;
+            if (int rc = partials_for((hipStream_t) stream, &partials)) return rc;
             std::snprintf(name, sizeof(name), "docc_reduce_colp%s_%s_f%d", vec ? "v" : "", names[op], precision);
             // the partial pass of a mean adds; the division happens once, in the final pass
-            if (int rc = launch(name, (uint32_t) pblocks, (uint32_t) slices, 1, 256, 0, (hipStream_t) stream, X, (long) outer,
+            if (int rc = launch(name, (uint32_t) pblocks, (uint32_t) slices, 1, 256, 0, (hipStream_t) stream, partials.ptr, X, (long) outer,
                                 (long) reduce, (long) inner, (long) chunk))
                 return rc;
             std::snprintf(name, sizeof(name), "docc_reduce_colf_%s_f%d", names[op], precision);
-            return launch(name, (uint32_t) ((total + 15) / 16), 1, 1, 256, 0, (hipStream_t) stream, Y, (long) total, (long) reduce,
-                          (long) slices);
+            return launch(name, (uint32_t) ((total + 15) / 16), 1, 1, 256, 0, (hipStream_t) stream, (const void*) partials.ptr, Y, (long) total,
+                          (long) reduce, (long) slices);
         }
     }
     if (blocks > (int64_t) cus * 16) blocks = (int64_t) cus * 16;

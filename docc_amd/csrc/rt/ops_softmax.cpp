@@ -45,13 +45,28 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
     return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
 }
 
-int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y) {
-    if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: precision must be 32 or 64");
-    if (outer < 0 || reduce < 0 || inner < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
-    if (outer == 0 || reduce == 0 || inner == 0) return 0;
-    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
-    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
-    hipStream_t s = (hipStream_t) stream;
+} // extern "C"
+
+namespace docc::rt::rocm {
+
+// Number of row slices of the sliced form for softmax over the middle extent of an [outer, reduce, inner] view
+// (inner > 32 or not a power of two), 0 when the one-launch tile kernel is used. Few (outer index, column
+// tile) pairs and many rows: the rows are sliced as well, so that about four work-groups per CU share the
+// tensor; the (maximum, sum) pairs of the slices need outer * slices * inner * 2 elements of `capacity` bytes.
+int64_t softmax_slices(int precision, int64_t outer, int64_t reduce, int64_t inner, int cus, int64_t capacity) {
+    const int64_t tiles = (inner + 63) / 64, groups = outer * tiles;
+    if (groups >= 2 * (int64_t) cus || reduce < 256) return 0;
+    int64_t slices = (4 * (int64_t) cus + groups - 1) / groups;
+    if (slices > reduce / 64) slices = reduce / 64;
+    const int64_t pair_bytes = 2 * (precision / 8);
+    const int64_t fit = capacity / (outer * inner * pair_bytes);
+    if (slices > fit) slices = fit;
+    return slices >= 2 ? slices : 0;
+}
+
+// The general softmax. `partials` = nullptr: the sliced form takes the stream's partial-results buffer;
+// otherwise `partials` (at least softmax_slices(.., kPartialsBytes) slices' worth of pairs) is used.
+int softmax_general(hipStream_t s, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y, void* partials) {
     const char* t = precision == 32 ? "f32" : "f64";
     char name[64];
     if (inner == 1) {
@@ -66,27 +81,67 @@ int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, i
     }
     const int64_t tiles = (inner + 63) / 64;
     if (tiles > 0x7fffffffLL / outer) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 work-groups");
-    // Few (outer index, column tile) pairs and many rows: slice the rows as well, so that about four work-groups
-    // per CU share the tensor; the pairs of the slices go through the kernels' 8 MiB scratch array.
     int cus = compute_units();
     if (cus <= 0) cus = 256;
     const int64_t groups = outer * tiles;
-    if (groups < 2 * (int64_t) cus && reduce >= 256) {
-        int64_t slices = (4 * (int64_t) cus + groups - 1) / groups;
-        if (slices > reduce / 64) slices = reduce / 64;
-        const int64_t pair_bytes = 2 * (precision / 8);
-        const int64_t fit = (int64_t(8) << 20) / (outer * inner * pair_bytes);
-        if (slices > fit) slices = fit;
-        if (slices >= 2) {
-            std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_partial", t);
-            int rc = launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, X, (long) reduce, (long) inner, (long) tiles, (int) slices);
-            if (rc) return rc;
-            std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_finish", t);
-            return launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles, (int) slices);
+    const int64_t slices = softmax_slices(precision, outer, reduce, inner, cus, (int64_t) kPartialsBytes);
+    if (slices >= 2) {
+        PartialsLease lease;
+        if (!partials) {
+            if (int rc = partials_for(s, &lease)) return rc;
+            partials = lease.ptr;
         }
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_partial", t);
+        int rc = launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, partials, X, (long) reduce, (long) inner, (long) tiles, (int) slices);
+        if (rc) return rc;
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_finish", t);
+        return launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, (const void*) partials, X, Y, (long) reduce, (long) inner, (long) tiles,
+                      (int) slices);
     }
     std::snprintf(name, sizeof(name), "docc_softmax_%s_tile", t);
     return launch(name, (uint32_t) (outer * tiles), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles);
+}
+
+// argument checks shared by the entry points of the general softmax; 1 = nothing to do
+int softmax_check(int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, const void* Y) {
+    if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: precision must be 32 or 64");
+    if (outer < 0 || reduce < 0 || inner < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
+    if (outer == 0 || reduce == 0 || inner == 0) return 1;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
+    return 0;
+}
+
+} // namespace docc::rt::rocm
+
+extern "C" {
+
+int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y) {
+    if (int rc = softmax_check(precision, outer, reduce, inner, X, Y)) return rc == 1 ? 0 : rc;
+    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
+    if (int rc = ensure_device()) return rc;
+    return softmax_general((hipStream_t) stream, precision, outer, reduce, inner, X, Y, nullptr);
+}
+
+int64_t docc_rocm_softmax_workspace_bytes(int precision, int64_t outer, int64_t reduce, int64_t inner) {
+    if ((precision != 32 && precision != 64) || outer <= 0 || reduce <= 0 || inner <= 0) return 0;
+    if (inner == 1 || (inner <= 32 && (inner & (inner - 1)) == 0)) return 0;
+    if (ensure_device()) return 0;
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    const int64_t slices = softmax_slices(precision, outer, reduce, inner, cus, (int64_t) kPartialsBytes);
+    return (slices * outer * inner * 2 * (precision / 8) + 255) / 256 * 256;
+}
+
+int docc_rocm_softmax_ws(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y,
+                         void* workspace, int64_t workspace_bytes) {
+    if (int rc = softmax_check(precision, outer, reduce, inner, X, Y)) return rc == 1 ? 0 : rc;
+    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
+    if (int rc = ensure_device()) return rc;
+    const int64_t need = docc_rocm_softmax_workspace_bytes(precision, outer, reduce, inner);
+    if (need > 0 && (!workspace || workspace_bytes < need || ((uintptr_t) workspace % 256) != 0))
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: this shape needs a 256-byte aligned workspace of %lld bytes", (long long) need);
+    // need == 0: the shape runs as one launch and no partial results exist
+    return softmax_general((hipStream_t) stream, precision, outer, reduce, inner, X, Y, need > 0 ? workspace : nullptr);
 }
 
 static uint32_t grid_for(int64_t items) {

@@ -6,6 +6,7 @@
 
 #include <cstdarg>
 #include <cstdint>
+#include <mutex>
 #include <string>
 
 #include "docc_rocm_rt.h"
@@ -25,6 +26,18 @@ int kernel(const char* name, hipFunction_t* fn);
 
 // Number of compute units of the current device (after ensure_device()).
 int compute_units();
+
+// Partial results of the launchers that run as a pair of launches (sliced softmax, column reductions, column
+// matrix-vector products): kPartialsBytes of device memory per (device, stream), created on the first such call
+// on that stream and kept until the process ends. Two calls on different streams so never share a buffer; the
+// lease also holds the stream's lock, so that two host threads feeding one stream enqueue their pairs one after
+// the other. Keep the lease alive until the second launch of the pair has been issued.
+constexpr size_t kPartialsBytes = size_t(8) << 20;
+struct PartialsLease {
+    void* ptr = nullptr;
+    std::unique_lock<std::mutex> lock;
+};
+int partials_for(hipStream_t stream, PartialsLease* lease);
 
 // Launch helper: packs the addresses of `args` for hipModuleLaunchKernel.
 template <typename... Args>

@@ -176,6 +176,44 @@ int kernel(const char* name, hipFunction_t* fn) {
     return 0;
 }
 
+namespace {
+struct PartialsSlot {
+    void* ptr = nullptr;
+    std::mutex busy;
+};
+std::mutex g_partials_mutex;
+// never destroyed: the slots' mutexes may be held while the process exits
+std::map<std::pair<int, hipStream_t>, PartialsSlot*>& partials_slots() {
+    static auto* slots = new std::map<std::pair<int, hipStream_t>, PartialsSlot*>();
+    return *slots;
+}
+} // namespace
+
+int partials_for(hipStream_t stream, PartialsLease* lease) {
+    int dev = 0;
+    int rc = check(hipGetDevice(&dev), "hipGetDevice");
+    if (rc) return rc;
+    PartialsSlot* slot = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_partials_mutex);
+        auto& slots = partials_slots();
+        auto it = slots.find({dev, stream});
+        if (it == slots.end()) it = slots.emplace(std::make_pair(dev, stream), new PartialsSlot()).first;
+        slot = it->second;
+    }
+    std::unique_lock<std::mutex> busy(slot->busy);
+    if (!slot->ptr) {
+        rc = check(hipMalloc(&slot->ptr, kPartialsBytes), "hipMalloc (partial results)");
+        if (rc) {
+            slot->ptr = nullptr;
+            return rc;
+        }
+    }
+    lease->ptr = slot->ptr;
+    lease->lock = std::move(busy);
+    return 0;
+}
+
 int compute_units() {
     int dev = 0;
     (void) hipGetDevice(&dev);

@@ -74,6 +74,8 @@ _SIGNATURES = {
     "docc_rocm_bf16gemm_f32_batched": [_vp, _int, _int, _i64, _i64, _i64, _f32, _vp, _i64, _i64, _vp, _i64, _i64, _f32, _vp, _i64, _i64, _i64],
     "docc_rocm_softmax_f32": [_vp, _i64, _i64, _vp, _vp],
     "docc_rocm_softmax": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
+    "docc_rocm_softmax_workspace_bytes": [_int, _i64, _i64, _i64],
+    "docc_rocm_softmax_ws": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _i64],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_conv2d_f32_workspace_bytes": [_i64] * 13,
     "docc_rocm_conv2d_f32_ws": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp, _vp, _i64],
@@ -95,7 +97,7 @@ _SIGNATURES = {
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
-            "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64,
+            "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64, "docc_rocm_softmax_workspace_bytes": _i64,
             "docc_rocm_conv2d_f32_workspace_bytes": _i64}
 
 #: every symbol the two public headers declare
@@ -257,6 +259,15 @@ def gemm_batched(kind, batch, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b
 def softmax(precision, outer, reduce, inner, X, Y, stream=0) -> None:
     """Softmax over the middle extent of an [outer, reduce, inner] view; precision 32 or 64."""
     call("docc_rocm_softmax", stream, precision, outer, reduce, inner, X, Y)
+
+
+def softmax_workspace_bytes(precision, outer, reduce, inner) -> int:
+    return int(lib().docc_rocm_softmax_workspace_bytes(precision, outer, reduce, inner))
+
+
+def softmax_ws(precision, outer, reduce, inner, X, Y, workspace, workspace_bytes, stream=0) -> None:
+    """docc_rocm_softmax with the partial results of the sliced form in `workspace` (device memory of the caller)."""
+    call("docc_rocm_softmax_ws", stream, precision, outer, reduce, inner, X, Y, workspace or None, workspace_bytes)
 
 
 def softmax_f32(rows, cols, X, Y, stream=0) -> None:

@@ -44,8 +44,8 @@ extern "C" {
  * (reference gemm_node.cpp:474-505) and cublasDgemm / cublasSgemm
  * (reference opt/src/targets/cuda/blas/gemm.cpp:131-185).
  * Zero-sized m, n: nothing is done; k == 0: C = beta * C. Products with one output
- * column or row (bf16 ones too) run as matrix-vector kernels (HBM-bound); their partial sums may pass through a
- * scratch array in the kernel image: do not overlap such calls on different streams.
+ * column or row (bf16 ones too) run as matrix-vector kernels (HBM-bound); their partial sums may pass through
+ * 8 MiB of device memory that the library keeps per stream (see docc_rocm_softmax).
  */
 int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                     double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta,
@@ -122,12 +122,24 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
  * (double). The reference's node takes any axes and its element type from its memlets
  * (softmax_node.cpp:38-110). inner == 1 with precision 32 is docc_rocm_softmax_f32; the other
  * forms read X twice (running maximum and sum, then the results). With few columns and a long
- * reduced extent the intermediate (maximum, sum) pairs of row slices pass through an 8 MiB scratch
- * array in the kernel image, shared by every such call on the device: do not overlap them on
- * different streams.
+ * reduced extent the rows are sliced over work-groups as well and the (maximum, sum) pairs of the
+ * slices pass through 8 MiB of device memory that the library keeps per stream (allocated on the
+ * first such call on a stream, kept until the process ends), so calls on different streams, and from
+ * different threads, do not disturb each other.
  */
 int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner,
                       const void* X, void* Y);
+
+/*
+ * The same with the partial results in memory of the caller: `workspace` is device memory, 256-byte
+ * aligned, of at least docc_rocm_softmax_workspace_bytes(...) bytes (0 for the shapes that run as one
+ * launch; at most 8 MiB); it may be reused as soon as the call's kernels have run. Same kernels and
+ * launch geometry as docc_rocm_softmax, so the results are the same bits. Counterpart in the reference:
+ * the temporaries SoftmaxNode::expand allocates around its loop nests (softmax_node.cpp:112-140).
+ */
+int64_t docc_rocm_softmax_workspace_bytes(int precision, int64_t outer, int64_t reduce, int64_t inner);
+int docc_rocm_softmax_ws(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner,
+                         const void* X, void* Y, void* workspace, int64_t workspace_bytes);
 
 /*
  * ml::Conv, 2-d, NCHW fp32, group 1 (reference conv_node.h:9-22,48-217):

@@ -3,6 +3,7 @@
 (max|y - y_ref| / max|y_ref|), the fp32 bar."""
 import numpy as np
 import pytest
+import scipy.special
 import torch
 
 import oracle
@@ -135,6 +136,93 @@ def test_softmax_general_matches_oracle(rt, dt, tol, shape, axes):
     assert rel_err_max(Y, ref) <= tol
     np.testing.assert_allclose(Y, ref, rtol=20 * tol, atol=1e-300 if dt == np.float64 else 1e-30)
     np.testing.assert_allclose(Y.sum(axis=tuple(norm)), 1.0, rtol=0, atol=max(tol, 1e-14) * 4)
+
+
+def test_sliced_launch_pairs_on_two_streams_and_two_threads(rt):
+    """The launchers that run as two launches with partial results in between (sliced softmax, column reduction,
+    column matrix-vector product) keep those per stream: pairs issued to two streams, from two threads, many
+    times over, each give what the same call gives alone."""
+    import ctypes
+    import threading
+
+    streams = []
+    for _ in range(2):
+        h = ctypes.c_void_p()
+        rt.call("docc_rocm_stream_create", ctypes.byref(h))
+        streams.append(h.value)
+    rng = np.random.default_rng(77)
+    cases = []
+    for t, (rows, cols) in enumerate([(6000, 320), (4096, 1100)]):
+        X = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+        v = rng.standard_normal(rows).astype(np.float32)
+        x, vd = dev(X), dev(v)
+        outs = {"softmax": torch.empty_like(x), "sum": torch.empty(cols, device="cuda"), "gemv": torch.empty(cols, device="cuda")}
+        cases.append((X, v, x, vd, outs, rows, cols))
+    torch.cuda.synchronize()
+
+    def issue(case, stream):
+        X, v, x, vd, outs, rows, cols = case
+        rt.softmax(32, 1, rows, cols, x.data_ptr(), outs["softmax"].data_ptr(), stream=stream)
+        rt.reduce("sum", 32, 1, rows, cols, x.data_ptr(), outs["sum"].data_ptr(), stream=stream)
+        rt.sgemm(1, cols, rows, 1.0, vd.data_ptr(), rows, x.data_ptr(), cols, 0.0, outs["gemv"].data_ptr(), cols, stream=stream)
+
+    # what each call gives alone
+    alone = []
+    for case in cases:
+        issue(case, 0)
+        torch.cuda.synchronize()
+        alone.append({k: t.clone() for k, t in case[4].items()})
+        for t in case[4].values():
+            t.fill_(float("nan"))
+    errors = []
+
+    def worker(i):
+        try:
+            for _ in range(20):
+                issue(cases[i], streams[i])
+        except Exception as e:      # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors
+    for case, ref in zip(cases, alone):
+        for k in ref:
+            assert torch.equal(case[4][k], ref[k]), k
+        X = case[0]
+        # against the closed form in float64 (over 6000 rows the oracle's left-to-right fp32 sum is itself 1e-5 off)
+        assert rel_err_max(host(case[4]["softmax"]), scipy.special.softmax(X.astype(np.float64), axis=0)) <= TOL_F32
+        assert rel_err_max(host(case[4]["sum"]), X.sum(axis=0, dtype=np.float64)) <= TOL_F32
+    for h in streams:
+        rt.call("docc_rocm_stream_destroy", h)
+
+
+def test_softmax_with_the_callers_workspace(rt):
+    """docc_rocm_softmax_ws: same bits as docc_rocm_softmax, the partial results in memory of the caller."""
+    rng = np.random.default_rng(5)
+    for dt, precision in ((np.float32, 32), (np.float64, 64)):
+        for outer, reduce_, inner in ((1, 5000, 300), (3, 700, 130), (2, 64, 40), (4, 100, 1), (2, 300, 16)):
+            X = (rng.standard_normal((outer, reduce_, inner)) * 6).astype(dt)
+            x = dev(X)
+            y0, y1 = torch.empty_like(x), torch.full_like(x, float("nan"))
+            rt.softmax(precision, outer, reduce_, inner, x.data_ptr(), y0.data_ptr())
+            need = rt.softmax_workspace_bytes(precision, outer, reduce_, inner)
+            assert 0 <= need <= 8 << 20
+            ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+            rt.softmax_ws(precision, outer, reduce_, inner, x.data_ptr(), y1.data_ptr(), ws.data_ptr(), need)
+            torch.cuda.synchronize()
+            assert torch.equal(y0, y1)
+            if need:
+                from docc_amd.runtime import RocmRuntimeError
+                with pytest.raises(RocmRuntimeError, match="workspace"):
+                    rt.softmax_ws(precision, outer, reduce_, inner, x.data_ptr(), y1.data_ptr(), ws.data_ptr(), need - 1)
+                with pytest.raises(RocmRuntimeError, match="workspace"):
+                    rt.softmax_ws(precision, outer, reduce_, inner, x.data_ptr(), y1.data_ptr(), 0, 0)
+    assert rt.softmax_workspace_bytes(32, 1, 5000, 300) > 0      # the sliced form is among the cases
 
 
 def test_softmax_general_edge_values_and_empty(rt):
