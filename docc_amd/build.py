@@ -116,15 +116,23 @@ def build_kernels(force: bool = True, jobs: int = 8) -> list[Path]:
 
 def build_runtime(force: bool = True) -> Path:
     srcs = sorted((CSRC / "rt").glob("*.cpp"))
-    deps = srcs + sorted((CSRC / "rt").glob("*.h")) + sorted(INCLUDE.glob("*.h"))
+    hip_srcs = sorted((CSRC / "rt").glob("*.hip"))
+    deps = srcs + hip_srcs + sorted((CSRC / "rt").glob("*.h")) + sorted(INCLUDE.glob("*.h"))
     out = LIB / "libdocc_rt_rocm.so"
     if not force and _newer(out, deps):
         return out
     LIB.mkdir(parents=True, exist_ok=True)
+    # the one HIP source of the runtime (a device array whose address host code asks for) goes through hipcc;
+    # its object carries the device image and registers it when the library is loaded
+    objs = []
+    for src in hip_srcs:
+        obj = LIB / (src.stem + ".o")
+        _run([hipcc(), "-c", "-fPIC", *DEVICE_FLAGS, "-I", str(INCLUDE), "-I", str(CSRC / "rt"), str(src), "-o", str(obj)])
+        objs.append(obj)
     _run([
         "g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-D__HIP_PLATFORM_AMD__",
         "-I", str(INCLUDE), "-I", str(CSRC / "rt"), "-I", str(ROCM / "include"),
-        *map(str, srcs), "-o", str(out),
+        *map(str, srcs), *map(str, objs), "-o", str(out),
         "-L", str(ROCM / "lib"), "-lamdhip64", "-ldl", f"-Wl,-rpath,{ROCM / 'lib'}",
     ])
     return out

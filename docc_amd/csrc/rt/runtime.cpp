@@ -46,7 +46,8 @@ const char* const kKernelImages[] = {
 };
 
 struct DeviceState {
-    bool ready = false;
+    bool ready = false;          // kernel images loaded
+    bool noalloc_ready = false;  // set-up of docc_rocm_softmax_noalloc done
     std::vector<hipModule_t> modules;
     int compute_units = 0;
     std::unordered_map<std::string, hipFunction_t> functions;
@@ -115,10 +116,32 @@ int check(hipError_t err, const char* what) {
     return fail((int) err, "%s: %s (%s)", what, hipGetErrorString(err), hipGetErrorName(err));
 }
 
+int noalloc_setup_device(int dev);   // noalloc.hip
+
+namespace {
+int load_device_images(int dev);
+}
+
 int ensure_device() {
     int dev = 0;
     hipError_t err = hipGetDevice(&dev);
     if (err != hipSuccess) return fail(DOCC_ROCM_ERR_NO_DEVICE, "no HIP device: %s", hipGetErrorString(err));
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if ((size_t) dev < g_devices.size() && g_devices[dev].ready && g_devices[dev].noalloc_ready) return 0;
+    }
+    if (int rc = load_device_images(dev)) return rc;
+    // the entry point that allocates nothing gets its array's address and its kernels now (outside the lock:
+    // the kernel lookups take it)
+    if (int rc = noalloc_setup_device(dev)) return rc;
+    std::lock_guard<std::mutex> lock(g_mutex);
+    g_devices[dev].noalloc_ready = true;
+    return 0;
+}
+
+namespace {
+int load_device_images(int dev) {
+    hipError_t err;
     std::lock_guard<std::mutex> lock(g_mutex);
     if ((size_t) dev >= g_devices.size()) g_devices.resize(dev + 1);
     DeviceState& st = g_devices[dev];
@@ -147,12 +170,21 @@ int ensure_device() {
     st.ready = true;
     return 0;
 }
+} // namespace
 
 int kernel(const char* name, hipFunction_t* fn) {
-    int rc = ensure_device();
-    if (rc) return rc;
     int dev = 0;
     (void) hipGetDevice(&dev);
+    {
+        // not ensure_device(): the device's own set-up looks kernels up before it is complete
+        std::lock_guard<std::mutex> lock(g_mutex);
+        if ((size_t) dev >= g_devices.size() || !g_devices[dev].ready) dev = -1;
+    }
+    if (dev < 0) {
+        int rc = ensure_device();
+        if (rc) return rc;
+        (void) hipGetDevice(&dev);
+    }
     std::lock_guard<std::mutex> lock(g_mutex);
     DeviceState& st = g_devices[dev];
     auto it = st.functions.find(name);

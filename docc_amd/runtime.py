@@ -76,6 +76,7 @@ _SIGNATURES = {
     "docc_rocm_softmax": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_softmax_workspace_bytes": [_int, _i64, _i64, _i64],
     "docc_rocm_softmax_ws": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _i64],
+    "docc_rocm_softmax_noalloc": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_conv2d_f32_workspace_bytes": [_i64] * 13,
     "docc_rocm_conv2d_f32_ws": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp, _vp, _i64],
@@ -268,6 +269,11 @@ def softmax_workspace_bytes(precision, outer, reduce, inner) -> int:
 def softmax_ws(precision, outer, reduce, inner, X, Y, workspace, workspace_bytes, stream=0) -> None:
     """docc_rocm_softmax with the partial results of the sliced form in `workspace` (device memory of the caller)."""
     call("docc_rocm_softmax_ws", stream, precision, outer, reduce, inner, X, Y, workspace or None, workspace_bytes)
+
+
+def softmax_noalloc(precision, outer, reduce, inner, X, Y, stream=0) -> None:
+    """docc_rocm_softmax through the entry point that allocates nothing (fixed 1 MiB of partial results)."""
+    call("docc_rocm_softmax_noalloc", stream, precision, outer, reduce, inner, X, Y)
 
 
 def softmax_f32(rows, cols, X, Y, stream=0) -> None:

@@ -142,6 +142,20 @@ int docc_rocm_softmax_ws(docc_rocm_stream_t stream, int precision, int64_t outer
                          const void* X, void* Y, void* workspace, int64_t workspace_bytes);
 
 /*
+ * docc_rocm_softmax for callers that cannot allocate device memory: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc. No counterpart in the reference. The call itself allocates, loads and
+ * looks up nothing: the partial results of the sliced form go through a fixed 1 MiB array of the library's own
+ * device image, whose address and kernels are obtained when the device is set up, so docc_rocm_init(device)
+ * must have returned before the first call (otherwise the call fails with a message that says so).
+ * A shape whose partial results need more than the 1 MiB (docc_rocm_softmax_workspace_bytes(...) tells) is
+ * refused with DOCC_ROCM_ERR_UNSUPPORTED and a message naming both numbers; every other shape gives the bits of
+ * docc_rocm_softmax. All calls on a device share the array: it need not be cleared between calls (a call
+ * writes what it reads back), but calls that overlap on one device - two streams, two threads - race.
+ */
+int docc_rocm_softmax_noalloc(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner,
+                              const void* X, void* Y);
+
+/*
  * ml::Conv, 2-d, NCHW fp32, group 1 (reference conv_node.h:9-22,48-217):
  *   Y[n,oc,oh,ow] = bias[oc] + sum_{ic,kh,kw} X[n,ic,oh*sh-ph+kh*dh, ow*sw-pw+kw*dw] * W[oc,ic,kh,kw]
  * with zero padding (taps outside the image contribute 0); bias may be NULL.
