@@ -6,7 +6,11 @@
 Prints ONE JSON line. The headline (`value`, `roofline`, `cpu_baseline`) is the
 fp32 row softmax over [8192, 4096] (one step = one launch over one such
 tensor, inputs resident in HBM, rotating over four buffer pairs so that the
-256 MB Infinity Cache cannot serve the reads). The other benchmark
+256 MB Infinity Cache cannot serve the reads). `value` comes from a timed region
+of exactly --steps steps; where such a region is shorter than 50 ms it is timed
+again until 50 ms of timed work have run and the median region is reported
+(`timed_regions`). Inputs are the seeded arrays the benchmark configurations
+name (numpy / torch CPU generators), uploaded before the timed regions. The other benchmark
 configurations (fp64 GEMM 1000^3, fp32 and bf16 GEMM 4096^3, attention
 B8 H16 S2048 D64, conv2d N32 C64 56x56 3x3) are measured in the same run and
 reported under `kernels`, each with its own roofline fraction and CPU baseline.
@@ -38,8 +42,10 @@ PEAK_HBM_GBS = 8000.0
 PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3, "bf16": 2516.6}
 
 # HBM bytes per softmax launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
-# same counters read for the 128 MiB copy kernel; see profiles/softmax_f32_8192x4096_pmc.txt.
+# same counters read for the 128 MiB copy kernel. A stored figure (this run does not read counters):
+# the JSON line names the file it comes from.
 SOFTMAX_TRAFFIC_BYTES = 268470883
+SOFTMAX_TRAFFIC_SOURCE = "profiles/softmax_f32_8192x4096_pmc.txt (stored figure from a rocprofv3 --pmc run, not measured by this run)"
 
 
 def parse_args():
@@ -91,6 +97,21 @@ def main():
         e1.record(stream)
         return e0.elapsed_ms(e1) / iters
 
+    # The shader clock the device sustains under a train of launches: one wave on a stream of its own watches
+    # the clock counters for a millisecond while the launches run on the null stream.
+    probe_stream = rt.stream_create()
+    clock_out = torch.zeros(1, device="cuda")
+
+    def sustained_clock_ghz(fn, launch_ms):
+        n = max(8, int(4.0 / max(launch_ms, 1e-3)) + 4)     # at least 4 ms of back-to-back launches
+        rt.device_sync()
+        for i in range(n):
+            fn(i)
+            if i == min(n // 8, 16):
+                rt.clock_probe(1000, clock_out.data_ptr(), probe_stream)
+        rt.device_sync()
+        return round(float(clock_out.item()) / 1000.0, 3)
+
     # ---- CPU side -------------------------------------------------------------------
     cores = min(len(os.sched_getaffinity(0)), int(os.environ.get("OMP_NUM_THREADS", "1024")))
     oracle_lib = None
@@ -123,25 +144,36 @@ def main():
     if want("softmax"):
         R, C = 8192, 4096
         nbytes = 2 * R * C * 4
-        g = torch.Generator(device="cuda").manual_seed(1)
-        pairs = [(torch.randn(R, C, device="cuda", generator=g) * 8, torch.empty(R, C, device="cuda")) for _ in range(4)]
+        # the configuration's own array (seed 1) and three more draws of the same generator to rotate over
+        rng = np.random.default_rng(1)
+        pairs = [(torch.from_numpy((rng.standard_normal((R, C)) * 8).astype(np.float32)).cuda(), torch.empty(R, C, device="cuda"))
+                 for _ in range(4)]
         step = lambda i: rt.softmax_f32(R, C, pairs[i % 4][0].data_ptr(), pairs[i % 4][1].data_ptr(), stream)
         for i in range(args.warmup):
             step(i)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(i)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
+
+        def region():
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                step(i)
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0
+
+        regions = [region()]
+        while sum(regions) < 0.05 and len(regions) < 1000:
+            regions.append(region())
+        wall = statistics.median(regions)
         ms_per_step = wall * 1e3 / args.steps
-        kern_ms = time_kernel(step, args.steps, 5)
+        kern_ms = time_kernel(step, max(args.steps, 200), 5)
         achieved = nbytes / kern_ms / 1e6
-        out.update(value=nbytes / (wall / args.steps) / 1e9, ms_per_step=ms_per_step)
+        out.update(value=nbytes / (wall / args.steps) / 1e9, ms_per_step=ms_per_step, timed_regions=len(regions),
+                   timed_ms_total=round(sum(regions) * 1e3, 2))
         out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": SOFTMAX_TRAFFIC_BYTES,
+                           "traffic_source": SOFTMAX_TRAFFIC_SOURCE,
                            "kernel": "docc_softmax_f32_block8_v2", "kernel_us": round(kern_ms * 1e3, 2),
-                           "algorithmic_bytes": nbytes}
+                           "algorithmic_bytes": nbytes, "sustained_clock_ghz": sustained_clock_ghz(step, kern_ms)}
         # same number for a plain copy of the same bytes: the practical ceiling of this memory system
         copy_ms = time_kernel(lambda i: rt.copy_bytes(R * C * 4, pairs[i % 4][0].data_ptr(), pairs[i % 4][1].data_ptr(), stream), 50, 5)
         out["roofline"]["copy_kernel_GBps"] = round(nbytes / copy_ms / 1e6, 1)
@@ -164,7 +196,7 @@ def main():
         ops = torch.randn(4096, device="cuda")
         sink = torch.empty(2 * 256 * max(info["compute_units"], 1), device="cuda")
         iters = 4000
-        best = 0.0
+        best, best_clock = 0.0, 0.0
         for waves in (1, 2):
             flop = [0.0]
 
@@ -172,17 +204,22 @@ def main():
                 flop[0] = rt.mfma_probe(prec, waves, iters, ops.data_ptr(), sink.data_ptr(), stream)
 
             ms = time_kernel(probe, 5, 2)
-            best = max(best, flop[0] / ms / 1e9)
-        ceiling_cache[dtype] = round(best, 1)
+            if flop[0] / ms / 1e9 > best:
+                best, best_clock = flop[0] / ms / 1e9, sustained_clock_ghz(probe, ms)
+        ceiling_cache[dtype] = (round(best, 1), best_clock)
         return ceiling_cache[dtype]
 
-    def add_kernel(name, dtype, flops, ms, cpu=None, extra=None):
+    def add_kernel(name, dtype, flops, ms, cpu=None, extra=None, fn=None):
         tf = flops / ms / 1e9
-        ceiling = mfma_ceiling(dtype)
+        ceiling, ceiling_clock = mfma_ceiling(dtype)
         entry = {"tflops": round(tf, 2), "kernel_us": round(ms * 1e3, 2), "flop": flops,
                  "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
                               "frac": round(tf / PEAK_TFLOPS[dtype], 4), "mfma_loop_random_operands": ceiling,
+                              "mfma_loop_clock_ghz": ceiling_clock,
                               "frac_of_mfma_loop": round(tf / ceiling, 4) if ceiling else None}, "dtype": dtype}
+        if fn is not None:
+            # the clock under this kernel (nominal 2.4 GHz): what separates an idle pipe from a lowered clock
+            entry["roofline"]["sustained_clock_ghz"] = sustained_clock_ghz(fn, ms)
         if cpu:
             entry["cpu_baseline"] = cpu
         if extra:
@@ -192,10 +229,12 @@ def main():
     # ---- config 1: fp64 GEMM 1000^3 ---------------------------------------------------
     if want("dgemm"):
         n = 1000
-        A = torch.rand(n, n, device="cuda", dtype=torch.float64)
-        B = torch.rand(n, n, device="cuda", dtype=torch.float64)
+        rng = np.random.default_rng(0)
+        A = torch.from_numpy(rng.random((n, n))).cuda()
+        B = torch.from_numpy(rng.random((n, n))).cuda()
         Cm = torch.empty(n, n, device="cuda", dtype=torch.float64)
-        ms = time_kernel(lambda i: rt.dgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 200, 10)
+        run = lambda i: rt.dgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream)
+        ms = time_kernel(run, 200, 10)
         cpu = None
         if oracle_lib is not None:
             a, b = A.cpu().numpy(), B.cpu().numpy()
@@ -204,15 +243,17 @@ def main():
             cpu = {"value": round(2 * n**3 / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": "full 1000^3, the reference's expanded loop nest (omp over i)",
                    "host_blas_tflops": round(2 * n**3 / tb / 1e12, 4), "host_blas": "numpy/OpenBLAS dgemm (the call the reference's BLAS dispatcher emits)"}
-        add_kernel("dgemm_1000", "f64", 2 * n**3, ms, cpu)
+        add_kernel("dgemm_1000", "f64", 2 * n**3, ms, cpu, fn=run)
 
     # ---- config 3a: fp32 GEMM 4096^3 ----------------------------------------------------
     if want("sgemm"):
         n = 4096
-        A = torch.randn(n, n, device="cuda") / 64
-        B = torch.randn(n, n, device="cuda") / 64
+        rng = np.random.default_rng(2)
+        A = torch.from_numpy((rng.standard_normal((n, n)) / 64).astype(np.float32)).cuda()
+        B = torch.from_numpy((rng.standard_normal((n, n)) / 64).astype(np.float32)).cuda()
         Cm = torch.empty(n, n, device="cuda")
-        ms = time_kernel(lambda i: rt.sgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 20, 3)
+        run = lambda i: rt.sgemm(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream)
+        ms = time_kernel(run, 20, 3)
         cpu = None
         if oracle_lib is not None:
             rows = 128
@@ -223,7 +264,7 @@ def main():
             cpu = {"value": round(2 * rows * n * n / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"first {rows} rows of C ({rows}x4096x4096), the reference's expanded loop nest",
                    "host_blas_tflops": round(2 * n**3 / tb / 1e12, 4), "host_blas": "numpy/OpenBLAS sgemm, full 4096^3"}
-        add_kernel("sgemm_4096", "f32", 2 * n**3, ms, cpu)
+        add_kernel("sgemm_4096", "f32", 2 * n**3, ms, cpu, fn=run)
         # the same product with bias row + ReLU in its store (what the fusion pass makes of a dense layer)
         bias = torch.randn(n, device="cuda")
         ms_e = time_kernel(lambda i: rt.gemm_epilogue("s", n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n,
@@ -245,10 +286,12 @@ def main():
     # ---- config 3b: bf16 GEMM 4096^3, fp32 accumulate/output ------------------------------
     if want("bgemm"):
         n = 4096
-        A = (torch.randn(n, n, device="cuda") / 64).bfloat16()
-        B = (torch.randn(n, n, device="cuda") / 64).bfloat16()
+        rng = np.random.default_rng(2)      # the values of configuration 3a, rounded to bf16 (nearest even)
+        A = torch.from_numpy((rng.standard_normal((n, n)) / 64).astype(np.float32)).cuda().bfloat16()
+        B = torch.from_numpy((rng.standard_normal((n, n)) / 64).astype(np.float32)).cuda().bfloat16()
         Cm = torch.empty(n, n, device="cuda")
-        ms = time_kernel(lambda i: rt.bf16gemm_f32(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream), 50, 5)
+        run = lambda i: rt.bf16gemm_f32(n, n, n, 1.0, A.data_ptr(), n, B.data_ptr(), n, 0.0, Cm.data_ptr(), n, stream=stream)
+        ms = time_kernel(run, 50, 5)
         cpu = None
         if oracle_lib is not None:
             rows = 128
@@ -257,15 +300,17 @@ def main():
             t = cpu_time(lambda: oracle.gemm_bf16(a, b, lib=oracle_lib), reps=1)
             cpu = {"value": round(2 * rows * n * n / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"first {rows} rows of C, fp32 loop nest on the bf16 values (the reference has no bf16 GEMM)"}
-        add_kernel("bgemm_4096", "bf16", 2 * n**3, ms, cpu)
+        add_kernel("bgemm_4096", "bf16", 2 * n**3, ms, cpu, fn=run)
         del A, B, Cm
 
     # ---- config 4: attention B8 H16 S2048 D64 bf16 ----------------------------------------
     if want("attention"):
         Bn, H, S, D = 8, 16, 2048, 64
-        Q, K, V = (torch.randn(Bn, H, S, D, device="cuda").bfloat16() for _ in range(3))
+        torch.manual_seed(3)
+        Q, K, V = (torch.randn(Bn, H, S, D).bfloat16().cuda() for _ in range(3))
         O = torch.empty(Bn, H, S, D, device="cuda", dtype=torch.bfloat16)
-        ms = time_kernel(lambda i: rt.attention_bf16(Bn, H, S, S, D, 0.125, Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), out_bf16=True, stream=stream), 50, 5)
+        run = lambda i: rt.attention_bf16(Bn, H, S, S, D, 0.125, Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), out_bf16=True, stream=stream)
+        ms = time_kernel(run, 50, 5)
         cpu = None
         if oracle_lib is not None:
             heads = max(cores, 1)
@@ -274,16 +319,18 @@ def main():
             t = cpu_time(lambda: oracle.attention(q, k, v, 0.125, lib=oracle_lib), reps=1)
             cpu = {"value": round(4 * heads * S * S * D / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"{heads} of the 128 (batch, head) pairs, fp32 loop nests (the reference has no attention)"}
-        add_kernel("attention_b8h16s2048d64", "bf16", 4 * Bn * H * S * S * D, ms, cpu)
+        add_kernel("attention_b8h16s2048d64", "bf16", 4 * Bn * H * S * S * D, ms, cpu, fn=run)
         del Q, K, V, O
 
     # ---- config 5: conv2d N32 C64->64 56x56 3x3 s1 p1 + bias ------------------------------
     if want("conv"):
-        X = torch.randn(32, 64, 56, 56, device="cuda")
-        W = torch.randn(64, 64, 3, 3, device="cuda") * (2.0 / 576) ** 0.5
-        b = torch.randn(64, device="cuda") * 0.1
+        torch.manual_seed(4)
+        X = torch.randn(32, 64, 56, 56).cuda()
+        W = (torch.randn(64, 64, 3, 3) * (2.0 / 576) ** 0.5).cuda()      # Kaiming-normal: fan_in 576
+        b = (torch.randn(64) * 0.1).cuda()
         Y = torch.empty(32, 64, 56, 56, device="cuda")
-        ms = time_kernel(lambda i: rt.conv2d_f32(32, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), stream=stream), 100, 10)
+        run = lambda i: rt.conv2d_f32(32, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), stream=stream)
+        ms = time_kernel(run, 100, 10)
         flops = 2 * 32 * 64 * 56 * 56 * 64 * 9
         cpu = None
         if oracle_lib is not None:
@@ -291,7 +338,7 @@ def main():
             t = cpu_time(lambda: oracle.conv2d(x, w, bb, pad=(1, 1), lib=oracle_lib), reps=1)
             cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": "full problem, the reference's loop nest with a zero-padding guard (omp over n)"}
-        add_kernel("conv2d_n32c64hw56k3", "f32", flops, ms, cpu)
+        add_kernel("conv2d_n32c64hw56k3", "f32", flops, ms, cpu, fn=run)
 
     # ---- elementwise tensor nodes on the softmax tensor's shape (HBM-bound) --------------------
     if want("elementwise"):
@@ -380,12 +427,14 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(out.get("ms_per_step", 0.0), 5),
+        "timed_regions": out.get("timed_regions", 0),
+        "timed_ms_total": out.get("timed_ms_total", 0.0),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "configs[1]: fp32 row softmax over axis -1 of an [8192, 4096] tensor, N(0,1)*8; one step = one launch, 268435456 algorithmic bytes",
+        "config": {"workload": "configs[1]: fp32 row softmax over axis -1 of an [8192, 4096] tensor, N(0,1)*8 from numpy default_rng(1); one step = one launch, 268435456 algorithmic bytes",
                    "device": info["arch"], "compute_units": info["compute_units"]},
     }
     if "roofline" in out:

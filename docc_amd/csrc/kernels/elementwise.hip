@@ -58,6 +58,34 @@ __device__ __forceinline__ void binary_kernel(const T* A, const T* B, T* Y, long
     for (long i = nvec * N + tid; i < n; i += stride) Y[i] = binary<OP>(A[i], B[i]);
 }
 
+// Activations with scalar operands: Y[i] = f(X[i], alpha, beta)
+template <typename T, int OP>
+__device__ __forceinline__ void param_unary_kernel(const T* X, T* Y, long n, long nvec, T alpha, T beta) {
+    typedef typename Vec128<T>::type V;
+    constexpr int N = Vec128<T>::N;
+    const long stride = (long) gridDim.x * blockDim.x;
+    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = tid; i < nvec; i += stride) {
+        V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(X) + i);
+#pragma unroll
+        for (int e = 0; e < N; e++) v[e] = param_unary<OP>(v[e], alpha, beta);
+        __builtin_nontemporal_store(v, reinterpret_cast<V*>(Y) + i);
+    }
+    for (long i = nvec * N + tid; i < n; i += stride) Y[i] = param_unary<OP>(X[i], alpha, beta);
+}
+
+// ml::Fill: every element of Y becomes one value of 1, 2, 4 or 8 bytes (fill_node.cpp:29-41: an assign
+// tasklet from a scalar under the output's Maps). `pattern` holds the value repeated to 16 bytes.
+__device__ __forceinline__ void fill_kernel(unsigned char* Y, long bytes, long nvec, u32x4 pattern) {
+    const long stride = (long) gridDim.x * blockDim.x;
+    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = tid; i < nvec; i += stride) __builtin_nontemporal_store(pattern, reinterpret_cast<u32x4*>(Y) + i);
+    // the tail (and everything, when Y is not 16-byte aligned): byte b of the output is byte b % 16 of the pattern,
+    // because the element size divides 16 and Y starts on an element boundary
+    const unsigned char* pb = reinterpret_cast<const unsigned char*>(&pattern);
+    for (long b = nvec * 16 + tid; b < bytes; b += stride) Y[b] = pb[b & 15];
+}
+
 // One operand is a scalar (the reference binds a constant or scalar container to "A" or "B",
 // python/bindings/builder/py_structured_sdfg_builder.cpp:894-908): Y[i] = f(A[i], b), or
 // f(b, A[i]) when LEFT.
@@ -253,6 +281,23 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
     }                                                                                                                        \
     DOCC_EW_BINARY_SCALAR(NAME, OP, sr, false)                                                                               \
     DOCC_EW_BINARY_SCALAR(NAME, OP, sl, true)
+
+#define DOCC_EW_PARAM_UNARY(NAME, OP)                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f32(const float* X, float* Y, long n, long nvec, float alpha, \
+                                                                           float beta) {                                     \
+        docc_k::param_unary_kernel<float, docc_k::OP>(X, Y, n, nvec, alpha, beta);                                           \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_ew_##NAME##_f64(const double* X, double* Y, long n, long nvec,       \
+                                                                           double alpha, double beta) {                      \
+        docc_k::param_unary_kernel<double, docc_k::OP>(X, Y, n, nvec, alpha, beta);                                          \
+    }
+DOCC_EW_PARAM_UNARY(elu, kElu)
+DOCC_EW_PARAM_UNARY(leaky_relu, kLeakyReLU)
+DOCC_EW_PARAM_UNARY(hard_sigmoid, kHardSigmoid)
+
+extern "C" __global__ __launch_bounds__(256) void docc_fill_bytes(unsigned char* Y, long bytes, long nvec, docc_k::u32x4 pattern) {
+    docc_k::fill_kernel(Y, bytes, nvec, pattern);
+}
 
 DOCC_EW_UNARY(abs, kAbs)
 DOCC_EW_UNARY(exp, kExp)

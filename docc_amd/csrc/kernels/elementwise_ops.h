@@ -6,6 +6,13 @@
 //   Abs, Exp, Sqrt, Tanh, Erf        the libm function of the element type (cmath_node.h)
 //   Add, Sub, Mul, Div               the IEEE operation
 //   Pow      pow(a, b)               elementwise_ops/pow_node.cpp:52-54 (CMathFunction::pow)
+// Activations with scalar operands ("alpha", "beta" connectors; elu_node.cpp:21, leaky_relu_node.cpp:21,
+// hard_sigmoid_node.cpp:21-22). The reference's expansions of these three are unfinished (Elu has no branch for
+// x > 0, LeakyReLU's multiply has one operand, HardSigmoid's fma has one), so the semantics are the ONNX
+// operators the nodes are named after:
+//   Elu          x > 0 ? x : alpha * (exp(x) - 1)          (the reference's exp, subtract 1, times alpha for x <= 0)
+//   LeakyReLU    x >= 0 ? x : alpha * x
+//   HardSigmoid  fmax(0, fmin(1, alpha * x + beta))        (the reference's fma, fmin(.., 1), fmax(.., 0) order)
 #pragma once
 
 #include "common.h"
@@ -13,6 +20,7 @@
 namespace docc_k {
 
 enum UnaryOp : int { kAbs = 0, kExp = 1, kReLU = 2, kSigmoid = 3, kSqrt = 4, kTanh = 5, kErf = 6 };
+enum ParamUnaryOp : int { kElu = 7, kLeakyReLU = 8, kHardSigmoid = 9 };
 enum BinaryOp : int { kAdd = 0, kSub = 1, kMul = 2, kDiv = 3, kMaximum = 4, kMinimum = 5, kPow = 6 };
 
 template <int OP>
@@ -54,6 +62,19 @@ __device__ __forceinline__ double binary(double a, double b) {
     if (OP == kMaximum) return fmax(a, b);
     if (OP == kPow) return pow(a, b);
     return fmin(a, b);
+}
+
+template <int OP>
+__device__ __forceinline__ float param_unary(float x, float alpha, float beta) {
+    if (OP == kElu) return x > 0.0f ? x : alpha * (expf(x) - 1.0f);
+    if (OP == kLeakyReLU) return x >= 0.0f ? x : alpha * x;
+    return fmaxf(fminf(__builtin_fmaf(alpha, x, beta), 1.0f), 0.0f);
+}
+template <int OP>
+__device__ __forceinline__ double param_unary(double x, double alpha, double beta) {
+    if (OP == kElu) return x > 0.0 ? x : alpha * (exp(x) - 1.0);
+    if (OP == kLeakyReLU) return x >= 0.0 ? x : alpha * x;
+    return fmax(fmin(__builtin_fma(alpha, x, beta), 1.0), 0.0);
 }
 
 // operation chosen at run time; the code is uniform over a launch, so this is a scalar branch

@@ -157,7 +157,57 @@ __device__ __forceinline__ void column_reduce_final(const void* partials, T* Y, 
     }
 }
 
+// DOT::BLAS: sum_i x[i * incx] * y[i * incy] (reference dot_node.cpp:76-165: one fma per element; the BLAS
+// dispatcher prints cblas_?dot). Work-group b takes elements [b * chunk, (b + 1) * chunk) and leaves its sum in
+// partials[b]; the second launch (one work-group) adds the partial sums in order and writes the result behind
+// them, at partials[groups]. The split depends on n and the launch geometry alone, so the result is reproducible.
+template <typename T>
+__device__ __forceinline__ void dot_partial(void* partials, const T* __restrict__ x, long incx, const T* __restrict__ y, long incy, long n,
+                                            long chunk) {
+    __shared__ T part[4];
+    const long i0 = (long) blockIdx.x * chunk, i1 = min(n, i0 + chunk);
+    T a0 = (T) 0, a1 = (T) 0;
+    long i = i0 + threadIdx.x;
+    for (; i + 256 < i1; i += 512) {      // two independent chains
+        a0 = __builtin_fma(x[i * incx], y[i * incy], a0);
+        a1 = __builtin_fma(x[(i + 256) * incx], y[(i + 256) * incy], a1);
+    }
+    if (i < i1) a0 = __builtin_fma(x[i * incx], y[i * incy], a0);
+    T a = a0 + a1;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) a += __shfl_xor(a, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) reinterpret_cast<T*>(partials)[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+template <typename T>
+__device__ __forceinline__ void dot_final(void* partials, int groups) {
+    __shared__ T part[256];
+    T* P = reinterpret_cast<T*>(partials);
+    T a = (T) 0;
+    for (int g = threadIdx.x; g < groups; g += 256) a += P[g];
+    part[threadIdx.x] = a;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T r = (T) 0;
+        for (int k = 0; k < 256; k++) r += part[k];
+        P[groups] = r;
+    }
+}
+
 } // namespace docc_k
+
+#define DOCC_DOT(SFX, T)                                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_dot_partial_##SFX(void* partials, const T* x, long incx, const T* y, \
+                                                                             long incy, long n, long chunk) {                  \
+        docc_k::dot_partial<T>(partials, x, incx, y, incy, n, chunk);                                                          \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_dot_final_##SFX(void* partials, int groups) {                          \
+        docc_k::dot_final<T>(partials, groups);                                                                                \
+    }
+DOCC_DOT(f32, float)
+DOCC_DOT(f64, double)
 
 #define DOCC_REDUCE(NAME, OP)                                                                                                  \
     extern "C" __global__ __launch_bounds__(256) void docc_reduce_row_##NAME##_f32(const float* X, float* Y, long rows, long R,   \

@@ -26,6 +26,23 @@ extern "C" __global__ __launch_bounds__(256) void docc_bf16_to_f32(const uint16_
     for (; i < n; i += stride) dst[i] = bf16_bits_to_f32(src[i]);
 }
 
+// Shader clock observed over `ticks` ticks of the constant 100 MHz counter (s_memrealtime) by one wave that does
+// nothing but sleep and look at that counter: launched on a stream of its own next to a train of kernels, it
+// gives the clock the device sustains under them. out[0] = MHz. The wait is bounded twice over (ticks, and a
+// cap on the number of looks), so the wave always ends.
+extern "C" __global__ __launch_bounds__(64) void docc_clock_probe(float* __restrict__ out, long ticks) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const long r0 = (long) __builtin_amdgcn_s_memrealtime();
+    const long c0 = (long) __builtin_readcyclecounter();
+    long r1 = r0;
+    for (int looks = 0; looks < (1 << 20) && r1 - r0 < ticks; looks++) {
+        __builtin_amdgcn_s_sleep(16);
+        r1 = (long) __builtin_amdgcn_s_memrealtime();
+    }
+    const long c1 = (long) __builtin_readcyclecounter();
+    out[0] = r1 > r0 ? (float) ((double) (c1 - c0) / (double) (r1 - r0) * 100.0) : 0.f;
+}
+
 // MFMA rate probes: `iters` rounds of 32 back-to-back MFMAs per wave on operands taken from
 // `operands` (4096 floats; random values make the multipliers toggle as they do in a real GEMM,
 // zeros do not), four accumulators, eight operand register sets in rotation. They measure what the

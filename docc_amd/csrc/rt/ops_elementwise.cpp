@@ -96,6 +96,41 @@ extern "C" int docc_rocm_elementwise_unary(docc_rocm_stream_t stream, int op, in
                   256, 0, (hipStream_t) stream, X, Y, (long) n, nvec);
 }
 
+extern "C" int docc_rocm_elementwise_activation(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y,
+                                                double alpha, double beta) {
+    static const char* const names[] = {"elu", "leaky_relu", "hard_sigmoid"};
+    if (op < DOCC_ROCM_UNARY_ELU || op > DOCC_ROCM_UNARY_HARD_SIGMOID)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_activation: unknown operation %d", op);
+    if (int rc = check_precision("elementwise_activation", precision)) return rc;
+    if (n < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_activation: negative count");
+    if (n == 0) return 0;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "elementwise_activation: null pointer");
+    if (int rc = ensure_device()) return rc;
+    const int per_vec = precision == 32 ? 4 : 2;
+    const bool aligned = (((uintptr_t) X | (uintptr_t) Y) % 16) == 0;
+    const long nvec = aligned ? (long) (n / per_vec) : 0;
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_ew_%s_f%d", names[op - DOCC_ROCM_UNARY_ELU], precision);
+    const uint32_t grid = grid_for(aligned ? (n + per_vec - 1) / per_vec : n, op == DOCC_ROCM_UNARY_ELU ? kGridTranscendental : kGridStreaming);
+    if (precision == 32) return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) n, nvec, (float) alpha, (float) beta);
+    return launch(name, grid, 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) n, nvec, alpha, beta);
+}
+
+extern "C" int docc_rocm_fill(docc_rocm_stream_t stream, int element_bytes, int64_t n, const void* value, void* Y) {
+    if (element_bytes != 1 && element_bytes != 2 && element_bytes != 4 && element_bytes != 8)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "fill: element size must be 1, 2, 4 or 8 bytes");
+    if (n < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "fill: negative count");
+    if (n == 0) return 0;
+    if (!value || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "fill: null pointer");
+    if ((uintptr_t) Y % (uintptr_t) element_bytes) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "fill: the output is not aligned to its element size");
+    if (int rc = ensure_device()) return rc;
+    struct alignas(16) Pattern { unsigned char b[16]; } pattern;      // passed by value, like the kernel's uint4
+    for (int i = 0; i < 16; i++) pattern.b[i] = ((const unsigned char*) value)[i % element_bytes];
+    const long bytes = (long) n * element_bytes;
+    const long nvec = (uintptr_t) Y % 16 == 0 ? bytes / 16 : 0;
+    return launch("docc_fill_bytes", grid_for(nvec > 0 ? nvec : bytes, kGridStreaming), 1, 1, 256, 0, (hipStream_t) stream, Y, bytes, nvec, pattern);
+}
+
 extern "C" int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A,
                                             const void* B, void* Y) {
     if (op < 0 || op >= (int) (sizeof(kBinaryNames) / sizeof(kBinaryNames[0])))

@@ -1,5 +1,6 @@
 // Launcher for the reduce tensor nodes (see include/docc_rocm_ops.h).
 #include <cstdio>
+#include <cstring>
 
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
@@ -62,4 +63,40 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
     if (blocks > (int64_t) cus * 16) blocks = (int64_t) cus * 16;
     std::snprintf(name, sizeof(name), "docc_reduce_col_%s_f%d", names[op], precision);
     return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) outer, (long) reduce, (long) inner);
+}
+
+// DOT::BLAS. Like cblas_?dot / cublas?dot with the result in host memory (reference dot_node.cpp dispatcher,
+// opt/src/targets/cuda/blas/dot.cpp:55-68): the call returns when the value is there.
+extern "C" int docc_rocm_dot(docc_rocm_stream_t stream, int precision, int64_t n, const void* x, int64_t incx, const void* y, int64_t incy,
+                             void* result) {
+    if (precision != 32 && precision != 64) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "dot: precision must be 32 or 64");
+    if (n < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "dot: negative length");
+    if (!result) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "dot: null result");
+    const size_t elem = precision / 8;
+    if (n == 0) {
+        std::memset(result, 0, elem);
+        return 0;
+    }
+    if (!x || !y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "dot: null pointer");
+    if (incx < 0 || incy < 0) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "dot: negative increments are not supported");
+    if (int rc = ensure_device()) return rc;
+    int cus = compute_units();
+    if (cus <= 0) cus = 256;
+    // about four work-groups per CU, at least 2048 elements each
+    int64_t groups = (n + 2047) / 2048;
+    if (groups > 4 * (int64_t) cus) groups = 4 * (int64_t) cus;
+    const int64_t chunk = (n + groups - 1) / groups;
+    groups = (n + chunk - 1) / chunk;
+    hipStream_t s = (hipStream_t) stream;
+    PartialsLease partials;
+    if (int rc = partials_for(s, &partials)) return rc;
+    const char* t = precision == 32 ? "f32" : "f64";
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_dot_partial_%s", t);
+    if (int rc = launch(name, (uint32_t) groups, 1, 1, 256, 0, s, partials.ptr, x, (long) incx, y, (long) incy, (long) n, (long) chunk)) return rc;
+    std::snprintf(name, sizeof(name), "docc_dot_final_%s", t);
+    if (int rc = launch(name, 1, 1, 1, 256, 0, s, partials.ptr, (int) groups)) return rc;
+    if (int rc = check(hipMemcpyAsync(result, (const char*) partials.ptr + (size_t) groups * elem, elem, hipMemcpyDeviceToHost, s), "hipMemcpyAsync (dot)"))
+        return rc;
+    return check(hipStreamSynchronize(s), "hipStreamSynchronize (dot)");
 }

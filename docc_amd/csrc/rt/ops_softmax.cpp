@@ -182,6 +182,14 @@ int docc_rocm_mfma_probe(docc_rocm_stream_t stream, int precision, int waves_per
                   256, 0, (hipStream_t) stream, operands, sink, iters);
 }
 
+int docc_rocm_clock_probe(docc_rocm_stream_t stream, int microseconds, float* mhz) {
+    if (microseconds < 1 || microseconds > 100000) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "clock_probe: 1 .. 100000 microseconds");
+    if (!mhz) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "clock_probe: null pointer");
+    int rc = ensure_device();
+    if (rc) return rc;
+    return launch("docc_clock_probe", 1, 1, 1, 64, 0, (hipStream_t) stream, mhz, (long) microseconds * 100);
+}
+
 int docc_rocm_convert_f32_to_bf16(docc_rocm_stream_t stream, int64_t count, const float* src, uint16_t* dst) {
     if (count < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "convert: negative count");
     if (count == 0) return 0;

@@ -92,10 +92,14 @@ _SIGNATURES = {
     "docc_rocm_cast": [_vp, _int, _int, _i64, _vp, _vp],
     "docc_rocm_transpose": [_vp, _int, _int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), _vp, _vp],
     "docc_rocm_reduce": [_vp, ctypes.c_int, ctypes.c_int, _i64, _i64, _i64, _vp, _vp],
+    "docc_rocm_elementwise_activation": [_vp, _int, _int, _i64, _vp, _vp, ctypes.c_double, ctypes.c_double],
+    "docc_rocm_fill": [_vp, _int, _i64, _vp, _vp],
+    "docc_rocm_dot": [_vp, _int, _i64, _vp, _i64, _vp, _i64, _vp],
     "docc_rocm_elementwise_fused": [_vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_double, _vp, _vp,
                                     ctypes.c_double, ctypes.c_int, _vp, _vp],
     "docc_rocm_copy_bytes": [_vp, _i64, _vp, _vp],
     "docc_rocm_mfma_probe": [_vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp],
+    "docc_rocm_clock_probe": [_vp, ctypes.c_int, _vp],
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
             "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64, "docc_rocm_softmax_workspace_bytes": _i64,
@@ -342,6 +346,29 @@ def broadcast(precision, in_shape, out_shape, X, Y, stream=0) -> None:
 REDUCE_OPS = {"sum": 0, "max": 1, "min": 2, "mean": 3}
 
 
+ACTIVATION_OPS = {"elu": 7, "leaky_relu": 8, "hard_sigmoid": 9}
+
+
+def elementwise_activation(op, precision, n, X, Y, alpha, beta=0.0, stream=0) -> None:
+    """Y[i] = f(X[i]; alpha, beta) for ml::Elu / ml::LeakyReLU / ml::HardSigmoid."""
+    call("docc_rocm_elementwise_activation", stream, ACTIVATION_OPS[op] if isinstance(op, str) else op, precision, n, X, Y, float(alpha), float(beta))
+
+
+def fill(value, n, Y, stream=0) -> None:
+    """All n elements at Y become `value`, a numpy scalar (its item size is the element size)."""
+    import numpy as np
+
+    v = np.asarray(value).reshape(1)
+    call("docc_rocm_fill", stream, v.dtype.itemsize, n, v.ctypes.data, Y)
+
+
+def dot(precision, n, x, incx, y, incy, stream=0):
+    """sum_i x[i*incx] * y[i*incy] (device vectors), returned as a Python float once the stream has run."""
+    out = (ctypes.c_double if precision == 64 else ctypes.c_float)(0)
+    call("docc_rocm_dot", stream, precision, n, x, incx, y, incy, ctypes.addressof(out))
+    return out.value
+
+
 def reduce(op, precision, outer, extent, inner, X, Y, stream=0) -> None:
     """Y[o, i] = op over r of X[o, r, i] for X seen as [outer, extent, inner]."""
     call("docc_rocm_reduce", stream, REDUCE_OPS[op] if isinstance(op, str) else op, precision, outer, extent, inner, X, Y)
@@ -390,6 +417,22 @@ def mfma_probe(precision, waves_per_simd, iters, operands, sink, stream=0) -> fl
     flop = ctypes.c_double(0.0)
     call("docc_rocm_mfma_probe", stream, precision, waves_per_simd, iters, operands, sink, ctypes.addressof(flop))
     return flop.value
+
+
+def clock_probe(microseconds, mhz, stream=0) -> None:
+    """One wave samples the shader clock for `microseconds`; mhz: device address of one float."""
+    call("docc_rocm_clock_probe", stream, microseconds, mhz)
+
+
+def stream_create() -> int:
+    """A non-blocking stream (it does not wait for the null stream)."""
+    h = _vp()
+    call("docc_rocm_stream_create", ctypes.byref(h))
+    return h.value
+
+
+def stream_destroy(stream: int) -> None:
+    call("docc_rocm_stream_destroy", stream)
 
 
 def convert_f32_to_bf16(count, src, dst, stream=0) -> None:

@@ -232,6 +232,9 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
 #define DOCC_ROCM_UNARY_SQRT 4     /* ml::Sqrt     sqrt        */
 #define DOCC_ROCM_UNARY_TANH 5     /* ml::Tanh     tanh        */
 #define DOCC_ROCM_UNARY_ERF 6      /* ml::Erf      erf         */
+#define DOCC_ROCM_UNARY_ELU 7          /* ml::Elu          x > 0 ? x : alpha * (exp(x) - 1)      (elu_node.cpp:21-97)          */
+#define DOCC_ROCM_UNARY_LEAKY_RELU 8   /* ml::LeakyReLU    x >= 0 ? x : alpha * x                (leaky_relu_node.cpp:21-68)   */
+#define DOCC_ROCM_UNARY_HARD_SIGMOID 9 /* ml::HardSigmoid  fmax(0, fmin(1, alpha * x + beta))    (hard_sigmoid_node.cpp:21-83) */
 #define DOCC_ROCM_BINARY_ADD 0     /* ml::Add */
 #define DOCC_ROCM_BINARY_SUB 1     /* ml::Sub */
 #define DOCC_ROCM_BINARY_MUL 2     /* ml::Mul */
@@ -242,6 +245,15 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
 int docc_rocm_elementwise_unary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y);
 int docc_rocm_elementwise_binary(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* A, const void* B,
                                  void* Y);
+/* The unary nodes with scalar operands on their "alpha" / "beta" connectors (codes 7..9 above; beta is read by
+ * HardSigmoid only). The reference's expansions of these nodes are unfinished (no branch for positive inputs in
+ * Elu, one-operand multiplies), so the operations are the ONNX operators of the same names; the order of the
+ * steps the reference does spell out (exp, minus one, times alpha; fma, min with 1, max with 0) is kept. */
+int docc_rocm_elementwise_activation(docc_rocm_stream_t stream, int op, int precision, int64_t n, const void* X, void* Y, double alpha,
+                                     double beta);
+/* ml::Fill (fill_node.cpp:29-41: an assign tasklet from a scalar under Maps over the output's shape): the `n`
+ * elements of Y, of 1, 2, 4 or 8 bytes each, all become the element at `value` (host memory). */
+int docc_rocm_fill(docc_rocm_stream_t stream, int element_bytes, int64_t n, const void* value, void* Y);
 /* One operand is a scalar: the reference binds a constant or a scalar container to "A" or
  * "B" of the binary node (python/bindings/builder/py_structured_sdfg_builder.cpp:894-908).
  * Y[i] = f(A[i], scalar), or f(scalar, A[i]) when scalar_is_lhs != 0; the scalar is
@@ -307,6 +319,21 @@ int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision, int64_t o
 int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precision, int rank, const int64_t* shape, int binary_op,
                                 const int64_t* a_shape, const void* A, double a_scalar, const int64_t* b_shape, const void* B,
                                 double b_scalar, int n_post, const int* post_ops, void* Y);
+
+/* DOT::BLAS (reference dot_node.cpp:18-40 connectors __x, __y -> __out, :76-165 expansion; replaces cblas_?dot
+ * of its BLAS dispatcher and cublas?dot of opt/src/targets/cuda/blas/dot.cpp:55-68): *result = sum_i
+ * x[i * incx] * y[i * incy], precision 32 or 64, x and y in device memory, `result` in HOST memory; the call
+ * returns when the value is there (it waits for the stream). Increments must not be negative. The sum is
+ * split by n and the launch geometry alone: the same call gives the same bits. */
+int docc_rocm_dot(docc_rocm_stream_t stream, int precision, int64_t n, const void* x, int64_t incx, const void* y, int64_t incy,
+                  void* result);
+
+/* Measurement aid, no counterpart in the reference: one wave watches the constant 100 MHz counter for
+ * `microseconds` (1 .. 100000) and writes the shader clock it saw over that time, in MHz, to mhz[0] (device
+ * memory). Launched on a stream of its own (docc_rocm_stream_create gives non-blocking ones) while a train of
+ * kernels runs on another, it tells the clock the device sustains under those kernels - the figure that
+ * separates "the pipe is idle" from "the power limit lowered the clock". */
+int docc_rocm_clock_probe(docc_rocm_stream_t stream, int microseconds, float* mhz);
 
 /* Measurement aid, no counterpart in the reference: `iters` rounds of 32 back-to-back
  * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16) on

@@ -61,6 +61,12 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.oracle_attention_bf16.restype = ctypes.c_int
     lib.oracle_elementwise_unary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p]
     lib.oracle_elementwise_unary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p]
+    lib.oracle_elementwise_activation_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p, ctypes.c_float, ctypes.c_float]
+    lib.oracle_elementwise_activation_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p, ctypes.c_double, ctypes.c_double]
+    lib.oracle_dot_f32.argtypes = [_i64, _f32p, _i64, _f32p, _i64]
+    lib.oracle_dot_f32.restype = ctypes.c_float
+    lib.oracle_dot_f64.argtypes = [_i64, _f64p, _i64, _f64p, _i64]
+    lib.oracle_dot_f64.restype = ctypes.c_double
     lib.oracle_elementwise_binary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p, _f32p]
     lib.oracle_elementwise_binary_f64.argtypes = [ctypes.c_int, _i64, _f64p, _f64p, _f64p]
     lib.oracle_broadcast.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.POINTER(_i64), ctypes.POINTER(_i64), ctypes.c_void_p, ctypes.c_void_p]
@@ -249,6 +255,34 @@ def elementwise_unary(op: str, X, lib=None) -> np.ndarray:
     if fn(UNARY_OPS[op], X.size, _p(X, ptr), _p(out, ptr)) != 0:
         raise ValueError(f"unknown unary operation {op}")
     return out
+
+
+ACTIVATION_OPS = {"elu": 7, "leaky_relu": 8, "hard_sigmoid": 9}
+
+
+def elementwise_activation(op: str, X, alpha, beta=0.0, lib=None) -> np.ndarray:
+    """ml::Elu / ml::LeakyReLU / ml::HardSigmoid with their scalar operands, fp32 or fp64 X of any shape."""
+    lib = lib or load()
+    dt = np.float64 if np.asarray(X).dtype == np.float64 else np.float32
+    X = _c(X, dt)
+    out = np.empty_like(X)
+    ptr = _f64p if dt == np.float64 else _f32p
+    fn = lib.oracle_elementwise_activation_f64 if dt == np.float64 else lib.oracle_elementwise_activation_f32
+    if fn(ACTIVATION_OPS[op], X.size, _p(X, ptr), _p(out, ptr), float(alpha), float(beta)) != 0:
+        raise ValueError(f"unknown activation {op}")
+    return out
+
+
+def dot(x, y, incx=1, incy=1, n=None, lib=None):
+    """DOT::BLAS: sum_i x[i*incx] * y[i*incy], added left to right in the element type."""
+    lib = lib or load()
+    dt = np.float64 if np.asarray(x).dtype == np.float64 else np.float32
+    x, y = _c(x, dt).ravel(), _c(y, dt).ravel()
+    if n is None:
+        n = min((x.size + incx - 1) // incx if incx else x.size, (y.size + incy - 1) // incy if incy else y.size)
+    ptr = _f64p if dt == np.float64 else _f32p
+    fn = lib.oracle_dot_f64 if dt == np.float64 else lib.oracle_dot_f32
+    return dt(fn(n, _p(x, ptr), incx, _p(y, ptr), incy))
 
 
 def elementwise_binary(op: str, A, B, lib=None) -> np.ndarray:

@@ -490,6 +490,59 @@ ORACLE_API int oracle_elementwise_unary_f64(int op, int64_t n, const double* X, 
     return 0;
 }
 
+/* The unary nodes with scalar operands (connectors "alpha", "beta"): ml::Elu (elu_node.cpp:21-97), ml::LeakyReLU
+ * (leaky_relu_node.cpp:21-68), ml::HardSigmoid (hard_sigmoid_node.cpp:21-83), operation codes 7, 8, 9. The
+ * reference's expansions are unfinished - Elu computes alpha * (exp(x) - 1) for every x, LeakyReLU's multiply
+ * and HardSigmoid's fma have one operand - so this restates the ONNX operators the nodes are named after,
+ * keeping the steps the reference does spell out in their order (exp, minus 1.0, times alpha; a * x + b,
+ * fmin with 1, fmax with 0). Parity unpinned by the reference (no test of it computes values); pinned by
+ * torch's elu / leaky_relu / hardsigmoid and closed forms in tests/test_oracle.py. */
+#define ORACLE_ACTIVATION_BODY(T, SUF)                                                                     \
+    switch (op) {                                                                                          \
+        case 7: { T t = exp##SUF(x); t = t - (T) 1.0; t = alpha * t; y = x > (T) 0.0 ? x : t; break; }     \
+        case 8: y = x >= (T) 0.0 ? x : alpha * x; break;                                                   \
+        default: { T t = fma##SUF(alpha, x, beta); t = fmin##SUF(t, (T) 1.0); y = fmax##SUF(t, (T) 0.0); break; } \
+    }
+
+ORACLE_API int oracle_elementwise_activation_f32(int op, int64_t n, const float* X, float* Y, float alpha, float beta) {
+    if (op < 7 || op > 9) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const float x = X[i];
+        float y;
+        ORACLE_ACTIVATION_BODY(float, f)
+        Y[i] = y;
+    }
+    return 0;
+}
+
+ORACLE_API int oracle_elementwise_activation_f64(int op, int64_t n, const double* X, double* Y, double alpha, double beta) {
+    if (op < 7 || op > 9) return 1;
+#pragma omp parallel for schedule(static)
+    for (int64_t i = 0; i < n; i++) {
+        const double x = X[i];
+        double y;
+        ORACLE_ACTIVATION_BODY(double, )
+        Y[i] = y;
+    }
+    return 0;
+}
+
+/* DOT::BLAS as DotNode::expand writes it (dot_node.cpp:76-165): one sequential For over i with the tasklet
+ * fp_fma, res = x[i * incx] * y[i * incy] + res, printed "a * b + c" (cpp_language_extension.cpp:207-208) -
+ * started from zero, as cblas_?dot, which the node's BLAS dispatcher prints, returns the plain sum. */
+ORACLE_API float oracle_dot_f32(int64_t n, const float* x, int64_t incx, const float* y, int64_t incy) {
+    float res = 0.0f;
+    for (int64_t i = 0; i < n; i++) res = x[i * incx] * y[i * incy] + res;
+    return res;
+}
+
+ORACLE_API double oracle_dot_f64(int64_t n, const double* x, int64_t incx, const double* y, int64_t incy) {
+    double res = 0.0;
+    for (int64_t i = 0; i < n; i++) res = x[i * incx] * y[i * incy] + res;
+    return res;
+}
+
 ORACLE_API int oracle_elementwise_binary_f32(int op, int64_t n, const float* A, const float* B, float* Y) {
     if (op < 0 || op > 6) return 1;
 #pragma omp parallel for schedule(static)

@@ -311,3 +311,67 @@ def test_reduce_nodes_against_numpy_and_closed_forms():
         oracle.reduce("sum", np.zeros((2, 3, 4)), (0, 2))        # not a block of adjacent axes
     with pytest.raises(ValueError):
         oracle.reduce("mean", np.zeros((2, 0)), (1,))
+
+
+# ---- activations with scalar operands, fill, dot, transpose ------------------------------------------------
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_activations_against_torch_and_closed_forms(dt):
+    """ml::Elu / ml::LeakyReLU / ml::HardSigmoid: torch's functions of the same names (computed in float64),
+    and the points where a wrong branch or a dropped operand shows: f(0), the saturation of HardSigmoid,
+    the slope for negative inputs, alpha = 0."""
+    rng = np.random.default_rng(8)
+    x = np.concatenate([rng.standard_normal(5000) * 3, [0.0, -0.0, 1e-30, -1e-30, 50.0, -50.0, np.inf, -np.inf]]).astype(dt)
+    t = torch.from_numpy(x.astype(np.float64))
+    tol = 2e-7 if dt == np.float32 else 1e-15
+    cases = [("elu", 1.0, 0.0, torch.nn.functional.elu(t, 1.0)), ("elu", 0.3, 0.0, torch.nn.functional.elu(t, 0.3)),
+             ("leaky_relu", 0.01, 0.0, torch.nn.functional.leaky_relu(t, 0.01)), ("leaky_relu", 0.25, 0.0, torch.nn.functional.leaky_relu(t, 0.25)),
+             ("hard_sigmoid", 1.0 / 6.0, 0.5, torch.nn.functional.hardsigmoid(t)), ("hard_sigmoid", 0.2, 0.5, torch.clamp(0.2 * t + 0.5, 0.0, 1.0))]
+    for op, alpha, beta, ref in cases:
+        y = oracle.elementwise_activation(op, x, alpha, beta)
+        assert y.dtype == dt and y.shape == x.shape
+        ref = ref.numpy()
+        ok = np.isfinite(ref)
+        assert np.array_equal(np.isnan(y), np.isnan(ref)), op
+        np.testing.assert_allclose(y[ok], ref[ok], rtol=tol, atol=tol, err_msg=op)
+        assert np.array_equal(y[~ok & ~np.isnan(ref)], ref[~ok & ~np.isnan(ref)].astype(dt))      # the infinities
+    one = np.array([2.5, -2.5], dt)
+    assert np.array_equal(oracle.elementwise_activation("elu", one, 0.0), np.array([2.5, -0.0], dt))          # alpha = 0: negatives vanish
+    assert oracle.elementwise_activation("elu", one, 2.0)[1] == dt(2.0) * (np.exp(dt(-2.5)) - dt(1.0))
+    assert np.array_equal(oracle.elementwise_activation("leaky_relu", one, 0.5), np.array([2.5, -1.25], dt))
+    assert np.array_equal(oracle.elementwise_activation("hard_sigmoid", np.array([-10, 0, 1, 10], dt), 0.25, 0.5), np.array([0, 0.5, 0.75, 1], dt))
+    with pytest.raises(KeyError):
+        oracle.elementwise_activation("gelu", one, 1.0)
+
+
+def test_dot_against_numpy_and_exact_cases():
+    rng = np.random.default_rng(9)
+    for dt, tol in ((np.float32, 1e-5), (np.float64, 1e-13)):
+        x, y = rng.standard_normal(4097).astype(dt), rng.standard_normal(4097).astype(dt)
+        exact = np.dot(x.astype(np.longdouble), y.astype(np.longdouble))
+        scale = np.dot(np.abs(x).astype(np.longdouble), np.abs(y).astype(np.longdouble))
+        assert abs(oracle.dot(x, y) - exact) <= tol * scale
+        # increments: every third element of x against every second of y
+        n = 1000
+        assert abs(oracle.dot(x, y, 3, 2, n) - np.dot(x[:3 * n:3].astype(np.longdouble), y[:2 * n:2].astype(np.longdouble))) <= tol * scale
+        # integer values are exact in any order; a swapped increment or an off-by-one in n changes them
+        xi, yi = np.arange(1, 101, dtype=dt), np.arange(100, 0, -1, dtype=dt)
+        assert oracle.dot(xi, yi) == dt(sum(a * b for a, b in zip(range(1, 101), range(100, 0, -1))))
+        assert oracle.dot(xi, yi, 2, 1, 50) == dt(sum(a * b for a, b in zip(range(1, 101, 2), range(100, 50, -1))))
+        assert oracle.dot(xi, yi, 1, 1, 0) == 0
+        assert oracle.dot(xi, np.ones(1, dt), 1, 0, 100) == dt(5050)       # increment 0 repeats one element
+
+
+def test_transpose_matches_numpy_for_every_permutation():
+    """oracle_transpose against numpy.transpose: every permutation of rank 2-4 tensors, every element size; an
+    inverted permutation or a slip in the strides fails it (the extents are pairwise different)."""
+    import itertools
+
+    rng = np.random.default_rng(10)
+    for shape in ((3, 5), (2, 3, 5), (2, 3, 4, 5)):
+        for dt in (np.uint8, np.int16, np.float32, np.float64):
+            X = rng.integers(0, 200, size=shape).astype(dt)
+            for perm in itertools.permutations(range(len(shape))):
+                Y = oracle.transpose(X, perm)
+                assert Y.dtype == dt and Y.flags.c_contiguous
+                assert np.array_equal(Y, np.transpose(X, perm)), (shape, perm)
