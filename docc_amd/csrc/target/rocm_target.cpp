@@ -35,7 +35,10 @@ bool is_math_node(const LibraryNode& node) {
     const std::string& c = node.code();
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
            c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
-           c == tensor::LibraryNodeType_Transpose || c == tensor::LibraryNodeType_Cast || is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
+           c == tensor::LibraryNodeType_Transpose || c == tensor::LibraryNodeType_Cast || c == tensor::LibraryNodeType_Fill ||
+           c == blas::LibraryNodeType_DOT ||
+           std::find(tensor::ActivationNodeCodes.begin(), tensor::ActivationNodeCodes.end(), c) != tensor::ActivationNodeCodes.end() ||
+           is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
 }
 
 // Preamble every rocm dispatcher puts into the globals stream (duplicates are folded by the generator).
@@ -439,6 +442,75 @@ protected:
     }
 };
 
+// ml::Elu / ml::LeakyReLU / ml::HardSigmoid: "alpha" and "beta" are scalars (constants or scalar containers) and
+// travel by value; an operand the graph leaves unbound takes its operator's default.
+class ActivationNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("X", true, false), operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::ActivationNode&>(node_);
+        const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
+        auto scalar = [&](const std::string& connector) -> std::string {
+            const auto* in = data_flow_graph_.input(connector);
+            if (!in) return connector == "beta" && n.code() != "ml::HardSigmoid" ? "0.0" : n.default_operand(connector);
+            if (!in->is_constant && function_.container(in->data).is_pointer)
+                throw InvalidSDFGException(n.code() + ": operand '" + connector + "' must be a scalar");
+            return "(double) " + connector;
+        };
+        s << "DOCC_ROCM_CHECK(docc_rocm_elementwise_activation(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision << ", "
+          << n.count() << ", " << name_of("X") << ", " << name_of("Y") << ", " << scalar("alpha") << ", " << scalar("beta") << "));" << std::endl;
+    }
+};
+
+// ml::Fill: the value is the scalar (or constant) on "X", handed over through host memory
+class FillNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("Y", false, true)}; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const tensor::FillNode&>(node_);
+        const auto* in = data_flow_graph_.input("X");
+        if (!in) throw InvalidSDFGException("ml::Fill: no value on connector 'X'");
+        if (!in->is_constant && function_.container(in->data).is_pointer) throw InvalidSDFGException("ml::Fill: the value on 'X' must be a scalar");
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "const " << language_extension_.primitive_type(n.element()) << " __docc_value = (" << language_extension_.primitive_type(n.element())
+          << ") X;" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_fill(nullptr, (int) sizeof(__docc_value), " << n.count() << ", &__docc_value, " << name_of("Y") << "));"
+          << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+};
+
+// DOT::BLAS: the vectors are device operands, the result a scalar of the host function (reference cuBLAS form
+// opt/src/targets/cuda/blas/dot.cpp:55-68 passes &__out the same way); the launcher returns with the value.
+class DotNodeDispatcher_ROCM : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+protected:
+    std::vector<DeviceOperand> operands() const override { return {operand("__x", true, false), operand("__y", true, false)}; }
+
+    std::string guard_condition() const override { return ""; }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = static_cast<const blas::DotNode&>(node_);
+        const auto* out = data_flow_graph_.output("__out");
+        if (!out || function_.container(out->data).is_pointer) throw InvalidSDFGException("DOT: the result on '__out' must be a scalar container");
+        s << "DOCC_ROCM_CHECK(docc_rocm_dot(nullptr, " << (n.precision() == blas::d ? 64 : 32) << ", " << language_extension_.expression(n.n()) << ", "
+          << name_of("__x") << ", " << language_extension_.expression(n.incx()) << ", " << name_of("__y") << ", "
+          << language_extension_.expression(n.incy()) << ", &__out));" << std::endl;
+    }
+};
+
 class BroadcastNodeDispatcher_ROCM : public RocmMathDispatcher {
 public:
     using RocmMathDispatcher::RocmMathDispatcher;
@@ -637,6 +709,9 @@ void register_plugin(plugins::Context& context) {
     register_math<AttentionNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Attention);
     for (auto& code : tensor::UnaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
     for (auto& code : tensor::BinaryNodeCodes) register_math<ElementWiseNodeDispatcher_ROCM>(reg, code);
+    for (auto& code : tensor::ActivationNodeCodes) register_math<ActivationNodeDispatcher_ROCM>(reg, code);
+    register_math<FillNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Fill);
+    register_math<DotNodeDispatcher_ROCM>(reg, blas::LibraryNodeType_DOT);
     register_math<BroadcastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Broadcast);
     register_math<TransposeNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Transpose);
     register_math<CastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Cast);
@@ -697,6 +772,13 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (a->element() != P::BFloat) return decline("inputs must be BFloat");
         if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
         // head dimension 64 runs the fused kernel, any other the GEMM / softmax / GEMM sequence
+    } else if (auto* act = dynamic_cast<tensor::ActivationNode*>(&node)) {
+        if (act->element() != P::Float && act->element() != P::Double) return decline("element type must be Float or Double");
+    } else if (auto* fill = dynamic_cast<tensor::FillNode*>(&node)) {
+        const size_t size = types::primitive_type_size(fill->element());
+        if (size != 1 && size != 2 && size != 4 && size != 8) return decline("elements must be 1, 2, 4 or 8 bytes");
+    } else if (auto* dot = dynamic_cast<blas::DotNode*>(&node)) {
+        if (dot->precision() != blas::s && dot->precision() != blas::d) return decline("precision must be s or d");
     } else if (is_elementwise_code(node.code())) {
         auto* e = dynamic_cast<tensor::ElementWiseNode*>(&node);
         if (!e) return decline("not an elementwise node object");
@@ -993,7 +1075,7 @@ bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, ana
         for (auto& in : sdfg.blocks()[i].inputs)
             if (!in.is_constant && sdfg.container(in.data).storage == "CPU" && sdfg.container(in.data).is_pointer) on_host = true;
         for (auto& out : sdfg.blocks()[i].outputs)
-            if (sdfg.container(out.data).storage == "CPU") on_host = true;
+            if (sdfg.container(out.data).storage == "CPU" && sdfg.container(out.data).is_pointer) on_host = true;
         if (!on_host) continue;
 
         struct Plan {
@@ -1017,6 +1099,7 @@ bool RocmOffloadTransform::run_pass(builder::StructuredSDFGBuilder& builder, ana
                 if (blk.node->reads(in.connector, blk.inputs)) p.read = true;
             }
             for (auto& out : blk.outputs) {
+                if (!sdfg.container(out.data).is_pointer) continue;   // a scalar result (DOT's __out) stays a host scalar
                 Plan& p = plan_for(out.data);
                 p.bytes = blk.node->connector_bytes(out.connector);
                 p.written = true;

@@ -218,6 +218,44 @@ bool GEMMNode::reads(const std::string& connector, const std::vector<data_flow::
 
 // ----------------------------------------------------------- tensor nodes
 
+namespace math::blas {
+
+DotNode::DotNode(std::string implementation_type, BLAS_Precision precision, Expression n, Expression incx, Expression incy)
+    : LibraryNode(LibraryNodeType_DOT, {"__out"}, {"__x", "__y"}, false, std::move(implementation_type)), precision_(precision),
+      n_(std::move(n)), incx_(std::move(incx)), incy_(std::move(incy)) {}
+
+void DotNode::validate() const {
+    if (precision_ != s && precision_ != d) throw InvalidSDFGException("DOT: precision must be s or d");
+    if (n_.empty() || incx_.empty() || incy_.empty()) throw InvalidSDFGException("DOT: n, incx and incy are required");
+}
+
+Expression DotNode::flop() const { return "((" + n_ + ") + ((" + n_ + ") - 1))"; }
+
+void DotNode::to_json(json::Value& j) const {
+    j.set("precision", (int64_t) precision_);
+    j.set("n", n_);
+    j.set("incx", incx_);
+    j.set("incy", incy_);
+}
+
+std::unique_ptr<DotNode> DotNode::from_json(const json::Value& j) {
+    return std::make_unique<DotNode>(impl_of(j), (BLAS_Precision) j.at("precision").as_int(), j.at("n").as_expression(),
+                                     j.at("incx").as_expression(), j.at("incy").as_expression());
+}
+
+Expression DotNode::connector_bytes(const std::string& connector) const {
+    const types::PrimitiveType t = precision_input_type(precision_);
+    if (connector == "__out") return bytes_of("1", t);
+    const Expression& inc = connector == "__x" ? incx_ : incy_;
+    // the span of the n strided elements: (n - 1) * inc + 1
+    int64_t n = 0, step = 0;
+    if (symbolic::is_integer(inc, &step) && step == 1) return bytes_of(n_, t);
+    if (symbolic::is_integer(n_, &n) && symbolic::is_integer(inc, &step)) return bytes_of(symbolic::integer(n > 0 ? (n - 1) * step + 1 : 0), t);
+    return bytes_of("(((" + n_ + ") - 1) * (" + inc + ") + 1)", t);
+}
+
+} // namespace math::blas
+
 namespace math::tensor {
 
 SoftmaxNode::SoftmaxNode(std::string implementation_type, std::vector<Expression> shape, std::vector<int64_t> axes,
@@ -581,6 +619,70 @@ std::unique_ptr<BroadcastNode> BroadcastNode::from_json(const Value& j) {
 Expression BroadcastNode::connector_bytes(const std::string& connector) const {
     const auto& shape = connector == "X" ? input_shape_ : output_shape_;
     return bytes_of(product(shape, 0, shape.size()), element_);
+}
+
+ActivationNode::ActivationNode(std::string code, std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element)
+    // "alpha" (and "beta" of HardSigmoid) are connectors a graph may leave unbound, so they are not among the
+    // inputs whose binding validate() insists on
+    : LibraryNode(code, {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)), element_(element) {}
+
+int ActivationNode::operation() const {
+    for (size_t i = 0; i < ActivationNodeCodes.size(); i++)
+        if (ActivationNodeCodes[i] == code_) return 7 + (int) i;
+    return -1;
+}
+
+Expression ActivationNode::count() const { return product(shape_, 0, shape_.size()); }
+
+std::string ActivationNode::default_operand(const std::string& connector) const {
+    if (code_ == "ml::Elu") return "1.0";
+    if (code_ == "ml::LeakyReLU") return "0.01";
+    return connector == "alpha" ? "0.2" : "0.5";
+}
+
+void ActivationNode::validate() const {
+    if (operation() < 0) throw InvalidSDFGException(code_ + ": not an activation node code");
+    if (shape_.empty()) throw InvalidSDFGException(code_ + ": empty shape");
+}
+
+void ActivationNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<ActivationNode> ActivationNode::from_json(const Value& j) {
+    const Value* et = j.find("element_type");
+    return std::make_unique<ActivationNode>(j.at("code").as_string(), impl_of(j), exprs_from_json(j.at("shape")),
+                                            et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression ActivationNode::connector_bytes(const std::string& connector) const {
+    if (connector == "alpha" || connector == "beta") return bytes_of("1", element_);
+    return bytes_of(count(), element_);
+}
+
+FillNode::FillNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element)
+    : LibraryNode(LibraryNodeType_Fill, {"Y"}, {"X"}, false, std::move(implementation_type)), shape_(std::move(shape)), element_(element) {}
+
+Expression FillNode::count() const { return shape_.empty() ? Expression("1") : product(shape_, 0, shape_.size()); }
+
+void FillNode::validate() const {
+    if (element_ == types::PrimitiveType::Void) throw InvalidSDFGException("Fill: void element type");
+}
+
+void FillNode::to_json(Value& j) const {
+    j.set("shape", exprs_to_json(shape_));
+    j.set("element_type", types::primitive_type_to_string(element_));
+}
+
+std::unique_ptr<FillNode> FillNode::from_json(const Value& j) {
+    const Value* et = j.find("element_type");
+    return std::make_unique<FillNode>(impl_of(j), exprs_from_json(j.at("shape")),
+                                      et ? types::primitive_type_from_string(et->as_string()) : types::PrimitiveType::Float);
+}
+
+Expression FillNode::connector_bytes(const std::string& connector) const {
+    return connector == "X" ? bytes_of("1", element_) : bytes_of(count(), element_);
 }
 
 CastNode::CastNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element, types::PrimitiveType target)
@@ -1033,6 +1135,9 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     fns_[math::tensor::LibraryNodeType_Broadcast] = &deserialize<math::tensor::BroadcastNode>;
     fns_[math::tensor::LibraryNodeType_Transpose] = &deserialize<math::tensor::TransposeNode>;
     fns_[math::tensor::LibraryNodeType_Cast] = &deserialize<math::tensor::CastNode>;
+    for (auto& code : math::tensor::ActivationNodeCodes) fns_[code] = &deserialize<math::tensor::ActivationNode>;
+    fns_[math::tensor::LibraryNodeType_Fill] = &deserialize<math::tensor::FillNode>;
+    fns_[math::blas::LibraryNodeType_DOT] = &deserialize<math::blas::DotNode>;
     for (auto& code : math::tensor::ReduceNodeCodes) fns_[code] = &deserialize<math::tensor::ReduceNode>;
     fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
 }

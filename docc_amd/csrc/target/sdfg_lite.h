@@ -172,6 +172,29 @@ private:
     std::string epilogue_activation_;
 };
 
+// reference: sdfg/include/sdfg/data_flow/library_nodes/math/blas/dot_node.h, dot_node.cpp:18-40 (connectors
+// "__x", "__y" -> "__out", a scalar), JSON keys code, precision, n, incx, incy (dot_node.cpp:189-202)
+inline const std::string LibraryNodeType_DOT = "DOT";
+
+class DotNode : public data_flow::LibraryNode {
+public:
+    DotNode(std::string implementation_type, BLAS_Precision precision, Expression n, Expression incx, Expression incy);
+    BLAS_Precision precision() const { return precision_; }
+    const Expression& n() const { return n_; }
+    const Expression& incx() const { return incx_; }
+    const Expression& incy() const { return incy_; }
+
+    void validate() const override;
+    Expression flop() const override;   // n multiplications + n - 1 additions (dot_node.cpp:167-171)
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<DotNode> from_json(const json::Value& j);
+
+private:
+    BLAS_Precision precision_;
+    Expression n_, incx_, incy_;
+};
+
 } // namespace math::blas
 
 namespace math::tensor {
@@ -398,6 +421,56 @@ public:
 private:
     std::vector<Expression> shape_;
     types::PrimitiveType element_, target_;
+};
+
+// The unary nodes with scalar operands. reference: .../elementwise_ops/elu_node.cpp:21 ("X", "alpha" -> "Y"),
+// leaky_relu_node.cpp:21 (the same), hard_sigmoid_node.cpp:21-22 ("X", "alpha", "beta" -> "Y"); JSON keys code +
+// shape (ElementWiseUnaryNodeSerializer). "alpha" / "beta" are bound to constants or scalar containers; an
+// operand that is left unbound takes the ONNX default of its operator (Elu 1, LeakyReLU 0.01, HardSigmoid 0.2 / 0.5).
+inline const std::vector<std::string> ActivationNodeCodes = {"ml::Elu", "ml::LeakyReLU", "ml::HardSigmoid"};
+
+class ActivationNode : public data_flow::LibraryNode {
+public:
+    ActivationNode(std::string code, std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element);
+    const std::vector<Expression>& shape() const { return shape_; }
+    types::PrimitiveType element() const { return element_; }
+    // the runtime's operation code (DOCC_ROCM_UNARY_ELU ...)
+    int operation() const;
+    Expression count() const;
+    // the literal an unbound "alpha" / "beta" stands for
+    std::string default_operand(const std::string& connector) const;
+
+    void validate() const override;
+    Expression flop() const override { return count(); }
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ActivationNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    types::PrimitiveType element_;
+};
+
+// reference: .../elementwise_ops/fill_node.cpp:17-41 ("X" -> "Y" with X a scalar or a constant: every element
+// of Y becomes X; JSON keys code + shape)
+inline const std::string LibraryNodeType_Fill = "ml::Fill";
+
+class FillNode : public data_flow::LibraryNode {
+public:
+    FillNode(std::string implementation_type, std::vector<Expression> shape, types::PrimitiveType element);
+    const std::vector<Expression>& shape() const { return shape_; }
+    types::PrimitiveType element() const { return element_; }
+    Expression count() const;
+
+    void validate() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    bool reads(const std::string& connector, const std::vector<data_flow::ConnectorBinding>&) const override { return connector == "X"; }
+    static std::unique_ptr<FillNode> from_json(const json::Value& j);
+
+private:
+    std::vector<Expression> shape_;
+    types::PrimitiveType element_;
 };
 
 // reference: .../tensor/transpose_node.h:14-60 (connectors "X" -> "Y", JSON keys "shape" and "perm";

@@ -422,13 +422,45 @@ class StructuredSDFGBuilder:
                          "shape": [_expr(s) for s in shape], "element_type": elem.value},
                         [bind("A", A), bind("B", B)], [self._operand("C", C)])
 
-    def add_elementwise_unary_op(self, op: str, X: str, Y: str, shape: Sequence[Any]) -> None:
-        """Unary elementwise node "X" -> "Y" (reference add_elementwise_unary_op, same file :910-952)."""
+    #: unary nodes with scalar operands on "alpha" / "beta" (reference elu_node.cpp, leaky_relu_node.cpp, hard_sigmoid_node.cpp)
+    ACTIVATION_CODES = {"elu": "ml::Elu", "leaky_relu": "ml::LeakyReLU", "hard_sigmoid": "ml::HardSigmoid"}
+
+    def add_elementwise_unary_op(self, op: str, X: str, Y: str, shape: Sequence[Any], alpha: Any = None, beta: Any = None) -> None:
+        """Unary elementwise node "X" -> "Y" (reference add_elementwise_unary_op, same file :910-952). For elu,
+        leaky_relu and hard_sigmoid `alpha` / `beta` (a number or the name of a scalar container) are bound to the
+        connectors of those names; left out, the operator's default applies (1, 0.01, 0.2 / 0.5)."""
+        if op in self.ACTIVATION_CODES:
+            elem = self._element(X)
+            inputs = [self._operand("X", X)]
+            for connector, v in (("alpha", alpha), ("beta", beta if op == "hard_sigmoid" else None)):
+                if v is not None:
+                    inputs.append(self._operand(connector, v) if v in self._data["containers"] else self._operand(connector, repr(float(v)), elem))
+            self._add_block({"code": self.ACTIVATION_CODES[op], "implementation_type": "NONE", "side_effect": False,
+                             "shape": [_expr(s) for s in shape], "element_type": elem.value}, inputs, [self._operand("Y", Y)])
+            return
         if op not in self.UNARY_CODES:
             raise NotImplementedError(f"elementwise op '{op}' is not part of the rocm target")
         self._add_block({"code": self.UNARY_CODES[op], "implementation_type": "NONE", "side_effect": False,
                          "shape": [_expr(s) for s in shape], "element_type": self._element(X).value},
                         [self._operand("X", X)], [self._operand("Y", Y)])
+
+    def add_fill(self, value: Any, Y: str, shape: Sequence[Any]) -> None:
+        """ml::Fill: every element of Y becomes `value`, a number or the name of a scalar container (reference
+        fill_node.cpp:17-41; the torch path creates it for linalg.fill, LinalgToSDFGTranslator.cpp:456-500)."""
+        elem = self._element(Y)
+        x = self._operand("X", value) if value in self._data["containers"] else self._operand("X", repr(value), elem)
+        self._add_block({"code": "ml::Fill", "implementation_type": "NONE", "side_effect": False, "shape": [_expr(s) for s in shape],
+                         "element_type": elem.value}, [x], [self._operand("Y", Y)])
+
+    def add_dot(self, X: str, Y: str, result: str, n: Any, incx: Any = 1, incy: Any = 1) -> None:
+        """DOT::BLAS: result = sum_i X[i * incx] * Y[i * incy] with `result` a scalar container whose type sets the
+        precision (reference add_dot, python/bindings/builder/py_structured_sdfg_builder.cpp:776-840)."""
+        elem = self._element(result)
+        if elem not in (PrimitiveType.Float, PrimitiveType.Double):
+            raise InvalidSDFGException("DOT: the result must be a Float or Double scalar")
+        self._add_block({"code": "DOT", "implementation_type": "BLAS", "side_effect": False,
+                         "precision": ord("s") if elem == PrimitiveType.Float else ord("d"), "n": _expr(n), "incx": _expr(incx), "incy": _expr(incy)},
+                        [self._operand("__x", X), self._operand("__y", Y)], [self._operand("__out", result)])
 
     def add_broadcast(self, X: str, Y: str, input_shape: Sequence[Any], output_shape: Sequence[Any]) -> None:
         """ml::Broadcast (reference .../tensor/broadcast_node.h): equal ranks, extent-1 dimensions repeat."""

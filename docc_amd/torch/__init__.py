@@ -16,7 +16,8 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
                                            -> ml::Attention (bf16, head dim 64)
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
                                            -> ml::Add .. ml::Minimum, with ml::Broadcast where shapes differ
-    relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh)
+    relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh),
+    elu, leaky_relu, hardsigmoid (F.* and nn.ELU / nn.LeakyReLU / nn.Hardsigmoid)
                                            -> ml::ReLU .. ml::Erf
     F.linear / nn.Linear                   -> GEMM with the weight transposed, bias through Broadcast + Add
     sum / mean / amax / amin over one dim or a block of adjacent dims (keepdim) -> ml::Sum .. ml::Min
@@ -258,12 +259,15 @@ class _FxLowering:
         self.builder.add_elementwise_op(op, name(a), name(b), out.name, shape)
         return out
 
-    def unary(self, node, op: str, x, dest):
+    def unary(self, node, op: str, x, dest, alpha=None, beta=None):
         x = self.tensor(node, x)
         if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
         out = self.new_tensor(x.shape, x.dtype, dest)
-        self.builder.add_elementwise_unary_op(op, x.name, out.name, x.shape)
+        if alpha is None and beta is None:
+            self.builder.add_elementwise_unary_op(op, x.name, out.name, x.shape)
+        else:
+            self.builder.add_elementwise_unary_op(op, x.name, out.name, x.shape, alpha=alpha, beta=beta)
         return out
 
     def reduce(self, node, op: str, x, dim, keepdim: bool, dest):
@@ -385,6 +389,17 @@ class _FxLowering:
                 if type(mod) in activations:
                     self.env[node] = self.unary(node, activations[type(mod)], self.arg(node.args[0]), dest)
                     continue
+                # ml::Elu / ml::LeakyReLU / ml::HardSigmoid with their scalar operands (torch's hardsigmoid is relu6(x + 3) / 6)
+                if type(mod) in (torch.nn.ELU, torch.nn.LeakyReLU, torch.nn.Hardsigmoid):
+                    if getattr(mod, "inplace", False):
+                        self.fail(node, "an in-place activation")
+                    if isinstance(mod, torch.nn.ELU):
+                        self.env[node] = self.unary(node, "elu", self.arg(node.args[0]), dest, alpha=float(mod.alpha))
+                    elif isinstance(mod, torch.nn.LeakyReLU):
+                        self.env[node] = self.unary(node, "leaky_relu", self.arg(node.args[0]), dest, alpha=float(mod.negative_slope))
+                    else:
+                        self.env[node] = self.unary(node, "hard_sigmoid", self.arg(node.args[0]), dest, alpha=1.0 / 6.0, beta=0.5)
+                    continue
                 if isinstance(mod, torch.nn.Linear):
                     w = self.add_input(f"{node.name}_weight", list(mod.weight.shape), mod.weight.dtype, ("attr", f"{node.target}.weight"))
                     b = None
@@ -493,6 +508,14 @@ class _FxLowering:
                 if kwargs.get("inplace"):
                     self.fail(node, "an in-place activation")
                 return self.unary(node, op, args[0], dest)
+        if t in (F.elu, F.leaky_relu, F.hardsigmoid):
+            if kwargs.get("inplace") or (len(args) > 2 and args[2]):
+                self.fail(node, "an in-place activation")
+            if t is F.elu:
+                return self.unary(node, "elu", args[0], dest, alpha=float(kwargs.get("alpha", args[1] if len(args) > 1 else 1.0)))
+            if t is F.leaky_relu:
+                return self.unary(node, "leaky_relu", args[0], dest, alpha=float(kwargs.get("negative_slope", args[1] if len(args) > 1 else 0.01)))
+            return self.unary(node, "hard_sigmoid", args[0], dest, alpha=1.0 / 6.0, beta=0.5)
         reductions = {"sum": (torch.sum,), "mean": (torch.mean,), "amax": (torch.amax,), "amin": (torch.amin,)}
         for name, fns in reductions.items():
             if any(t is f for f in fns) or method == name:

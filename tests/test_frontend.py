@@ -343,6 +343,29 @@ def test_torch_lowering_of_elementwise_operations_and_linear():
         docc_torch.TorchProgram(Ints(), torch.ones(4, dtype=torch.int32), target="rocm").to_sdfg()
 
 
+def test_torch_lowering_of_activations_with_scalar_operands():
+    class Acts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.elu = torch.nn.ELU(alpha=0.7)
+            self.leaky = torch.nn.LeakyReLU(0.2)
+            self.hs = torch.nn.Hardsigmoid()
+
+        def forward(self, x):
+            return self.hs(self.leaky(self.elu(x))) + torch.nn.functional.leaky_relu(x) + torch.nn.functional.elu(x, alpha=1.5)
+
+    sdfg = docc_torch.TorchProgram(Acts(), (torch.randn(4, 6),), target="rocm").to_sdfg()
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes == ["ml::Elu", "ml::LeakyReLU", "ml::HardSigmoid", "ml::LeakyReLU", "ml::Add", "ml::Elu", "ml::Add"]
+    flows = [c["dataflow"] for c in sdfg._data["root"]["children"]]
+    operands = lambda f: {b["connector"]: b.get("constant") for b in f["inputs"] if "constant" in b}
+    assert operands(flows[0]) == {"alpha": "0.7"} and operands(flows[1]) == {"alpha": "0.2"}
+    assert operands(flows[2]) == {"alpha": repr(1.0 / 6.0), "beta": "0.5"}
+    assert operands(flows[3]) == {"alpha": "0.01"} and operands(flows[5]) == {"alpha": "1.5"}
+    sdfg.schedule("rocm")          # the mapper takes all of them
+    assert sdfg.loop_report()["ml::Elu::ROCMWithoutTransfers"] == 2
+
+
 def test_torch_backend_is_registered_and_reads_global_options():
     import torch._dynamo
 

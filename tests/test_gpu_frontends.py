@@ -257,6 +257,67 @@ def test_torch_compile_mlp_fp32():
     assert r["GEMM"] == 2 and r["H2D"] == 0 and r["D2H"] == 0      # device tensors: no transfers at all
 
 
+def test_torch_compile_activations_with_scalar_operands():
+    class Acts(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.elu = torch.nn.ELU(alpha=0.7)
+            self.leaky = torch.nn.LeakyReLU(0.2)
+            self.hs = torch.nn.Hardsigmoid()
+
+        def forward(self, x):
+            return self.hs(self.leaky(self.elu(x))) + torch.nn.functional.leaky_relu(x) + torch.nn.functional.elu(x, alpha=1.5)
+
+    torch.manual_seed(1)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.float64, 1e-12)):
+        x = (torch.randn(37, 129, dtype=dtype) * 3).cuda()
+        program = docc_torch.compile_torch(Acts(), x, target="rocm")
+        y = program(x)
+        with torch.no_grad():
+            ref = Acts()(x.double().cpu())
+        assert y.dtype == dtype and rel_err_max(y.cpu().numpy(), ref.numpy()) <= tol
+        # the same through the oracle's functions, node by node
+        xh = x.cpu().numpy()
+        o = oracle.elementwise_activation("hard_sigmoid", oracle.elementwise_activation("leaky_relu", oracle.elementwise_activation("elu", xh, 0.7), 0.2),
+                                          1.0 / 6.0, 0.5)
+        o = o + oracle.elementwise_activation("leaky_relu", xh, 0.01) + oracle.elementwise_activation("elu", xh, 1.5)
+        assert rel_err_max(y.cpu().numpy(), o) <= tol
+
+
+def test_builder_program_with_dot_fill_and_activations(tmp_path):
+    """DOT::BLAS with a scalar result, ml::Fill from that scalar, and the activations, through the builder and
+    the generated code on host arrays (function-level offloading)."""
+    import ctypes
+
+    from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFGBuilder
+
+    F64p = Pointer(Scalar(PrimitiveType.Double))
+    b = StructuredSDFGBuilder("dot_fill")
+    for name in ("x", "y", "filled", "act"):
+        b.add_container(name, F64p, True)
+    b.add_container("_s0", Scalar(PrimitiveType.Int64), True)
+    b.add_container("r", Scalar(PrimitiveType.Double), False)
+    b.add_dot("x", "y", "r", "_s0", 1, 1)
+    b.add_fill("r", "filled", ["_s0"])
+    b.add_elementwise_unary_op("elu", "x", "act", ["_s0"], alpha="r")
+    s = b.move()
+    s.schedule("rocm")
+    lib = s._compile(str(tmp_path))
+    fn = getattr(ctypes.CDLL(lib), "dot_fill")
+    fn.restype = None
+    n = 5000
+    rng = np.random.default_rng(12)
+    x, y = rng.standard_normal(n) * 0.01, rng.standard_normal(n)
+    filled, act = np.full(n, np.nan), np.full(n, np.nan)
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    fn(ptr(x), ptr(y), ptr(filled), ptr(act), ctypes.c_int64(n))
+    from docc_amd import runtime
+    assert runtime.take_failure()[0] == 0
+    r = float(np.dot(x.astype(np.longdouble), y.astype(np.longdouble)))
+    assert abs(filled[0] - r) <= 1e-12 * float(np.abs(x) @ np.abs(y)) and (filled == filled[0]).all()
+    assert rel_err_max(act, oracle.elementwise_activation("elu", x, filled[0])) <= 1e-12
+
+
 def test_torch_compile_small_batch_through_wide_layers():
     """A batch of four through 2048-wide layers: the GEMMs have few output rows and take the matrix-vector kernels
     (bias and activation as one pass over the output); same bar as any fp32 GEMM chain."""

@@ -37,7 +37,8 @@ def test_registry_holds_every_rocm_key():
     keys = registered_dispatchers()
     for code in ("GEMM", "ml::MatMul", "ml::Softmax", "ml::Conv", "ml::Attention", "ml::Broadcast", "ml::Abs", "ml::Exp",
                  "ml::ReLU", "ml::Sigmoid", "ml::Sqrt", "ml::Tanh", "ml::Erf", "ml::Add", "ml::Sub", "ml::Mul", "ml::Div",
-                 "ml::Maximum", "ml::Minimum", "ml::Sum", "ml::Max", "ml::Min", "ml::Mean", "ROCMFusedElementWise"):
+                 "ml::Maximum", "ml::Minimum", "ml::Sum", "ml::Max", "ml::Min", "ml::Mean", "ROCMFusedElementWise", "ml::Elu",
+                 "ml::LeakyReLU", "ml::HardSigmoid", "ml::Fill", "DOT"):
         assert f"{code}::ROCMWithTransfers" in keys and f"{code}::ROCMWithoutTransfers" in keys
     assert "ROCMOffloading::NONE" in keys
 
@@ -53,6 +54,42 @@ def test_gemm_node_json_uses_the_reference_keys():
     # a round trip through the native parser keeps everything
     again = StructuredSDFG.parse(gemm_sdfg().to_json())
     assert again.library_nodes()[0] == node and again.arguments == ["A", "B", "_s0", "_docc_ret_0"]
+
+
+def test_dot_and_activation_nodes_use_the_reference_keys(tmp_path):
+    b = StructuredSDFGBuilder("dots")
+    b.add_container("x", F32, True)
+    b.add_container("y", F32, True)
+    b.add_container("_s0", I64, True)
+    b.add_container("r", Scalar(PrimitiveType.Float), False)
+    b.add_container("out", F32, True)
+    b.add_dot("x", "y", "r", "_s0", 1, 2)
+    b.add_fill("r", "out", [1])
+    b.add_elementwise_unary_op("leaky_relu", "x", "y", ["_s0"], alpha="r")
+    s = b.move()
+    dot, fill, leaky = s.library_nodes()
+    # DotNodeSerializer (reference dot_node.cpp:189-202) and ElementWiseUnaryNodeSerializer keys
+    assert dot["code"] == "DOT" and dot["precision"] == ord("s") and (dot["n"], dot["incx"], dot["incy"]) == ("_s0", "1", "2")
+    assert dot["implementation_type"] == "BLAS"
+    assert fill["code"] == "ml::Fill" and fill["shape"] == ["1"]
+    assert leaky["code"] == "ml::LeakyReLU" and leaky["shape"] == ["_s0"]
+    again = StructuredSDFG.parse(s.to_json())
+    assert [n["code"] for n in again.library_nodes()] == ["DOT", "ml::Fill", "ml::LeakyReLU"]
+    s.schedule("rocm", options={"offload": "none"})
+    src, _ = source_of(s, tmp_path)
+    assert "docc_rocm_dot(nullptr, 32, _s0, __x, 1, __y, 2, &__out)" in src and "r = __out;" in src
+    assert "docc_rocm_fill(nullptr, (int) sizeof(__docc_value), 1, &__docc_value, Y)" in src
+    assert "docc_rocm_elementwise_activation(nullptr, 8 /* ml::LeakyReLU */, 32, _s0, X, Y, (double) alpha, 0.0)" in src
+    # a pointer where a scalar belongs is refused when the code is generated
+    b = StructuredSDFGBuilder("bad_dot")
+    for n in ("x", "y", "r"):
+        b.add_container(n, F64, True)
+    b._add_block({"code": "DOT", "implementation_type": "BLAS", "side_effect": False, "precision": ord("d"), "n": "4", "incx": "1", "incy": "1"},
+                 [b._operand("__x", "x"), b._operand("__y", "y")], [b._operand("__out", "r")])
+    bad = b.move()
+    bad.schedule("rocm", options={"offload": "none"})
+    with pytest.raises(InvalidSDFGException, match="scalar"):
+        bad.generate(str(tmp_path / "bad"))
 
 
 def test_validation_errors():
@@ -340,6 +377,16 @@ def every_node_type():
     for op in sorted(set(StructuredSDFGBuilder.BINARY_CODES) - {"max", "min"}):
         yield build("n_" + op, lambda b, op=op: b.add_elementwise_op(op, "p0", "p1", "p3", [4, 8]), f3)
     yield build("n_scalar", lambda b: b.add_elementwise_op("mul", "p0", 2.5, "p3", [4, 8]), {"p0": F64, "p3": F64})
+    yield build("n_elu", lambda b: b.add_elementwise_unary_op("elu", "p0", "p3", [4, 8], alpha=0.5), {"p0": F32, "p3": F32})
+    yield build("n_leaky", lambda b: b.add_elementwise_unary_op("leaky_relu", "p0", "p3", [4, 8]), {"p0": F64, "p3": F64})
+    yield build("n_hardsig", lambda b: b.add_elementwise_unary_op("hard_sigmoid", "p0", "p3", [4, 8], alpha=0.25, beta=0.5), {"p0": F32, "p3": F32})
+    yield build("n_fill", lambda b: b.add_fill(1.5, "p3", [4, 8]), {"p3": F32})
+
+    def dot(b):
+        b.add_container("res", Scalar(PrimitiveType.Double), False)
+        b.add_dot("p0", "p1", "res", 32, 1, 2)
+        b.add_fill("res", "p3", [1])          # the scalar result reaches an argument through a fill of one element
+    yield build("n_dot", dot, {"p0": F64, "p1": F64, "p3": F64})
     yield build("n_broadcast", lambda b: b.add_broadcast("p0", "p3", [1, 8], [4, 8]), {"p0": F32, "p3": F32})
     yield build("n_transpose", lambda b: b.add_transpose("p0", "p3", [4, 8, 3], [2, 0, 1]), {"p0": F32, "p3": F32})
     yield build("n_cast", lambda b: b.add_cast_op("p0", "p3", [4, 8]), {"p0": F32, "p3": BF16})
