@@ -13,8 +13,16 @@
 //              deallocation, allocation_size?}, ... }
 // What the rocm target can take from it is a root sequence of blocks that hold one library node
 // each (with its access and constant nodes), allocation and release of temporaries (Malloc / Free
-// nodes, managed storage) and a final return; loop nests, tasklets and branches have no lowering
-// here and are refused with the element that stopped the import.
+// nodes, managed storage), a final return, and the loop nests that are elementwise work in disguise:
+// a perfect nest of Maps (or of the Fors the front end writes before its For2Map pass) over one block
+// with one tasklet or CMath node whose operands are dense tensors indexed by the loop variables. That is
+// the form the elementwise tensor nodes expand to (elementwise_node.cpp:86-240) and the form of the copy
+// into the return buffer (python/docc/python/ast_parser.py:1186-1210, :2102-2270); it is folded back into
+// the node the target has a kernel for (ml::Transpose for a copy, ml::Fill, the elementwise nodes). The
+// reference's CUDA target instead prints a kernel per Map nest (opt/src/targets/cuda/codegen/
+// cuda_map_dispatcher.cpp:42-168); here the kernels exist already, so the nest is matched, not compiled.
+// A scalar stored through an assign tasklet (the scalar form of the return copy) becomes an ml::Fill of one
+// element. Other loops, tasklets and branches have no lowering and are refused with the element named.
 #include <algorithm>
 #include <cctype>
 #include <map>
@@ -123,6 +131,101 @@ Value debug_info_of(const Value& element) {
     return Value();
 }
 
+
+// ---- expressions of loop nests ---------------------------------------------------------------
+// Index arithmetic arrives as SymEngine prints it ("_i0", "_s1*_i0 + _i1", "1 + _i0", "_i0 < _s0"). The
+// matcher needs sums of products only: a term is an integer coefficient times a sorted list of symbols.
+
+std::string strip(const std::string& e) {
+    std::string s;
+    for (char c : e)
+        if (!std::isspace((unsigned char) c)) s += c;
+    // outer parentheses that span the whole expression
+    for (bool again = true; again && s.size() >= 2 && s.front() == '(' && s.back() == ')';) {
+        int depth = 0;
+        again = true;
+        for (size_t i = 0; i + 1 < s.size(); i++) {
+            if (s[i] == '(') depth++;
+            if (s[i] == ')') depth--;
+            if (depth == 0) {
+                again = false;
+                break;
+            }
+        }
+        if (again) s = s.substr(1, s.size() - 2);
+    }
+    return s;
+}
+
+std::vector<std::string> split_top(const std::string& e, char sep) {
+    std::vector<std::string> parts;
+    int depth = 0;
+    std::string cur;
+    for (char c : e) {
+        if (c == '(') depth++;
+        if (c == ')') depth--;
+        if (c == sep && depth == 0) {
+            parts.push_back(cur);
+            cur.clear();
+        } else {
+            cur += c;
+        }
+    }
+    parts.push_back(cur);
+    return parts;
+}
+
+struct Term {
+    int64_t coefficient = 1;
+    std::vector<std::string> symbols;   // sorted
+    bool operator==(const Term& o) const { return coefficient == o.coefficient && symbols == o.symbols; }
+};
+
+// a product of integers and symbols; false for anything else (sums inside, divisions, calls)
+bool parse_term(const std::string& text, Term* out) {
+    Term t;
+    for (auto& f : split_top(strip(text), '*')) {
+        const std::string factor = strip(f);
+        if (factor.empty()) return false;
+        int64_t v = 0;
+        if (symbolic::is_integer(factor, &v)) {
+            t.coefficient *= v;
+            continue;
+        }
+        for (char c : factor)
+            if (!(std::isalnum((unsigned char) c) || c == '_')) return false;
+        if (std::isdigit((unsigned char) factor[0])) return false;
+        t.symbols.push_back(factor);
+    }
+    std::sort(t.symbols.begin(), t.symbols.end());
+    *out = t;
+    return true;
+}
+
+Term term_product(const Term& a, const Term& b) {
+    Term t;
+    t.coefficient = a.coefficient * b.coefficient;
+    t.symbols = a.symbols;
+    t.symbols.insert(t.symbols.end(), b.symbols.begin(), b.symbols.end());
+    std::sort(t.symbols.begin(), t.symbols.end());
+    return t;
+}
+
+// One loop of a nest in the only form matched: for (var = 0; var < extent; var = var + 1)
+struct NestLoop {
+    std::string var;
+    Expression extent;
+    Term extent_term;
+};
+
+// How an operand walks memory: a stride (in elements) per loop of the nest; `dense` tells in which order of
+// the loops the strides are those of a C-contiguous tensor over the loops' extents (outermost first).
+struct OperandWalk {
+    bool scalar = false;               // a constant or a scalar container
+    Value binding;                     // {"data": ...} or {"constant": ..., "type": ...}
+    std::vector<int> order;            // loop indices, outermost dimension first
+};
+
 struct Import {
     const Value& src;
     Value out;
@@ -183,8 +286,11 @@ struct Import {
         for (auto& n : nodes) {
             by_id[n.at("element_id").as_int()] = &n;
             const std::string kind = n.at("type").as_string();
-            if (kind == "tasklet")
-                throw InvalidSDFGException(describe(n) + " in " + describe(block) + ": tasklets are not lowered by the rocm target");
+            if (kind == "tasklet" || (kind == "library_node" && n.at("code").as_string() == "CMath")) {
+                // a statement outside any loop: the scalar forms (a scalar stored into a buffer)
+                lower_tasklet_block(block, {}, children);
+                return true;
+            }
             if (kind == "library_node") {
                 if (lib) throw InvalidSDFGException(describe(block) + ": more than one library node in a block");
                 lib = &n;
@@ -283,6 +389,293 @@ struct Import {
         return true;
     }
 
+
+    [[noreturn]] void refuse(const Value& element, const std::string& why) {
+        throw InvalidSDFGException(describe(element) + ": " + why + " (the rocm target lowers library nodes and the elementwise loop nests "
+                                   "that match one of its kernels)");
+    }
+
+    // strides of `edge`'s operand per loop of the nest -> order of the loops in which it is dense
+    bool walk_of(const Value& block, const Value& edge, const Value& node, const std::vector<NestLoop>& loops, OperandWalk* walk) {
+        const std::string kind = node.at("type").as_string();
+        if (kind == "constant_node") {
+            walk->scalar = true;
+            walk->binding.set("constant", c_expression(node.at("data").as_expression()));
+            walk->binding.set("type", types::primitive_type_to_string(element_of(node.at("data_type"), describe(node))));
+            return true;
+        }
+        const std::string data = node.at("data").as_string();
+        walk->binding.set("data", data);
+        const Value& c = container(data);
+        if (c.at("type").as_string() == "scalar") {
+            walk->scalar = true;
+            return true;
+        }
+        const Value& type = edge.at("base_type");
+        const std::string tkind = type.at("type").as_string();
+        const Array& subset = edge.at("subset").as_array();
+        std::vector<Term> strides(loops.size());
+        std::vector<bool> seen(loops.size(), false);
+        auto loop_of = [&](const std::string& name) {
+            for (size_t l = 0; l < loops.size(); l++)
+                if (loops[l].var == name) return (int) l;
+            return -1;
+        };
+        if (tkind == "tensor") {
+            // one index per dimension, each a loop variable; the strides are the type's
+            const Array& tstrides = type.at("strides").as_array();
+            if (subset.size() != tstrides.size()) return false;
+            if (const Value* off = type.find("offset"))
+                if (strip(off->as_expression()) != "0") return false;
+            for (size_t d = 0; d < subset.size(); d++) {
+                const int l = loop_of(strip(subset[d].as_expression()));
+                Term st;
+                if (l < 0 || seen[l] || !parse_term(tstrides[d].as_expression(), &st)) return false;
+                seen[l] = true;
+                strides[l] = st;
+            }
+        } else if (tkind == "pointer" || tkind == "array") {
+            // one linearised index: a sum of (stride * loop variable) terms
+            if (subset.size() != 1) return false;
+            for (auto& part : split_top(strip(subset[0].as_expression()), '+')) {
+                Term t;
+                if (!parse_term(part, &t)) return false;
+                int l = -1;
+                for (size_t k = 0; k < t.symbols.size(); k++) {
+                    const int hit = loop_of(t.symbols[k]);
+                    if (hit >= 0) {
+                        if (l >= 0) return false;   // a product of two loop variables
+                        l = hit;
+                        t.symbols.erase(t.symbols.begin() + (long) k);
+                        k--;
+                    }
+                }
+                if (l < 0 || seen[l]) return false;   // a constant offset, or a variable twice
+                seen[l] = true;
+                strides[l] = t;
+            }
+        } else {
+            return false;
+        }
+        for (bool v : seen)
+            if (!v) return false;   // a repeated (broadcast) operand: not matched
+        // innermost: stride 1; then the loop whose stride is the product of the extents found so far; ...
+        std::vector<int> inner_first;
+        Term expect;
+        std::vector<bool> used(loops.size(), false);
+        for (size_t n = 0; n < loops.size(); n++) {
+            int found = -1;
+            for (size_t l = 0; l < loops.size(); l++)
+                if (!used[l] && strides[l] == expect) found = (int) l;
+            if (found < 0) {
+                // extents of 1 have any stride; nothing else may be left
+                for (size_t l = 0; l < loops.size(); l++)
+                    if (!used[l] && !(loops[l].extent_term == Term{})) return false;
+                for (size_t l = 0; l < loops.size(); l++)
+                    if (!used[l]) inner_first.push_back((int) l);
+                break;
+            }
+            used[found] = true;
+            inner_first.push_back(found);
+            expect = term_product(expect, loops[found].extent_term);
+        }
+        walk->order.assign(inner_first.rbegin(), inner_first.rend());
+        (void) block;
+        return true;
+    }
+
+    // `element` is a for or a map: the nest below it, matched against the elementwise forms
+    void import_loop_nest(const Value& element, Array& children) {
+        std::vector<NestLoop> loops;
+        const Value* at = &element;
+        const Value* block = nullptr;
+        while (true) {
+            const std::string kind = at->at("type").as_string();
+            if (kind == "for" || kind == "map") {
+                NestLoop loop;
+                loop.var = strip(at->at("indvar").as_expression());
+                if (strip(at->at("init").as_expression()) != "0") refuse(*at, "the loop does not start at 0");
+                const std::string update = strip(at->at("update").as_expression());
+                if (update != "1+" + loop.var && update != loop.var + "+1") refuse(*at, "the loop's step is not 1");
+                const std::string cond = strip(at->at("condition").as_expression());
+                if (cond.rfind(loop.var + "<", 0) != 0 || cond.find("<=") != std::string::npos) refuse(*at, "the loop's condition is not 'variable < bound'");
+                loop.extent = c_expression(strip(cond.substr(loop.var.size() + 1)));
+                if (!parse_term(loop.extent, &loop.extent_term)) refuse(*at, "the loop's bound is not a product of symbols and integers");
+                loops.push_back(loop);
+                const Value& body = at->at("root");
+                if (const Value* transitions = body.find("transitions"))
+                    for (auto& t : transitions->as_array())
+                        if (!t.at("assignments").as_array().empty()) refuse(t, "symbol assignments inside a loop nest");
+                const Value* only = nullptr;
+                for (auto& child : body.at("children").as_array()) {
+                    if (child.at("type").as_string() == "block" && child.at("dataflow").at("nodes").as_array().empty()) continue;
+                    if (only) refuse(*at, "more than one statement in a loop body");
+                    only = &child;
+                }
+                if (!only) return;   // an empty nest does nothing
+                at = only;
+                continue;
+            }
+            if (kind == "sequence") {
+                const Array& kids = at->at("children").as_array();
+                if (kids.size() != 1) refuse(*at, "more than one statement in a loop body");
+                at = &kids[0];
+                continue;
+            }
+            if (kind != "block") refuse(*at, "control flow inside a loop nest");
+            block = at;
+            break;
+        }
+        if (loops.size() > 6) refuse(element, "a loop nest deeper than 6");
+        lower_tasklet_block(*block, loops, children);
+    }
+
+    // One block with one tasklet (or CMath node) under `loops` (none: a scalar statement).
+    void lower_tasklet_block(const Value& block, const std::vector<NestLoop>& loops, Array& children) {
+        const Value& df = block.at("dataflow");
+        std::map<int64_t, const Value*> by_id;
+        const Value* op = nullptr;
+        for (auto& n : df.at("nodes").as_array()) {
+            by_id[n.at("element_id").as_int()] = &n;
+            const std::string kind = n.at("type").as_string();
+            if (kind == "tasklet" || kind == "library_node") {
+                if (op) refuse(block, "more than one operation in a loop body");
+                op = &n;
+            }
+        }
+        if (!op) return;
+        const int64_t op_id = op->at("element_id").as_int();
+        std::map<std::string, OperandWalk> in;
+        OperandWalk out;
+        const Value* out_type = nullptr;
+        bool out_is_pointer = false;
+        for (auto& e : df.at("edges").as_array()) {
+            const bool into = e.at("dst").as_int() == op_id, from = e.at("src").as_int() == op_id;
+            if (!into && !from) refuse(block, "data movement beside the operation");
+            const Value& other = *by_id.at(e.at(into ? "src" : "dst").as_int());
+            OperandWalk w;
+            if (!walk_of(block, e, other, loops, &w))
+                refuse(block, "operand '" + (other.contains("data") ? other.at("data").as_expression() : std::string("?")) +
+                                  "' is not a dense tensor indexed by the loop variables");
+            if (into) {
+                in[e.at("dst_conn").as_string()] = w;
+            } else {
+                if (out_type) refuse(block, "an operation with two results");
+                out = w;
+                out_type = &e.at("base_type");
+                out_is_pointer = other.at("type").as_string() == "access_node" && container(other.at("data").as_string()).at("type").as_string() == "pointer";
+                if (out.scalar && out_is_pointer) {
+                    // a scalar stored to element 0 of a buffer (the scalar form of the return copy)
+                    for (auto& sub : e.at("subset").as_array())
+                        if (strip(sub.as_expression()) != "0") refuse(block, "a store to one element other than the first");
+                }
+            }
+        }
+        if (!out_type) refuse(block, "an operation without a result");
+        const types::PrimitiveType element = element_of(*out_type, describe(block));
+
+        // what the operation is
+        std::string code;      // node code of the target
+        std::vector<std::string> operands;   // the operation's input connectors in order
+        if (op->at("type").as_string() == "tasklet") {
+            const int64_t tc = op->at("code").as_int();
+            for (auto& i : op->at("inputs").as_array()) operands.push_back(i.as_string());
+            // enum TaskletCode (reference sdfg/include/sdfg/data_flow/tasklet.h:94-153)
+            switch (tc) {
+                case 0: code = "assign"; break;
+                case 2: code = "ml::Add"; break;
+                case 3: code = "ml::Sub"; break;
+                case 4: code = "ml::Mul"; break;
+                case 5: code = "ml::Div"; break;
+                default: refuse(*op, "tasklet code " + std::to_string(tc) + " has no kernel");
+            }
+        } else {
+            if (op->at("code").as_string() != "CMath") refuse(*op, "a library node inside a loop nest");
+            const std::string stem = op->at("function_stem").as_string();
+            static const std::map<std::string, std::string> functions = {
+                {"exp", "ml::Exp"}, {"sqrt", "ml::Sqrt"}, {"tanh", "ml::Tanh"}, {"erf", "ml::Erf"}, {"fabs", "ml::Abs"},
+                {"fmax", "ml::Maximum"}, {"fmin", "ml::Minimum"}, {"pow", "ml::Pow"}};
+            auto it = functions.find(stem);
+            if (it == functions.end()) refuse(*op, "CMath function '" + stem + "' has no kernel");
+            code = it->second;
+            operands = {"_in1", "_in2"};
+            if (code == "ml::Exp" || code == "ml::Sqrt" || code == "ml::Tanh" || code == "ml::Erf" || code == "ml::Abs") operands = {"_in1"};
+        }
+        for (auto& name : operands)
+            if (!in.count(name)) refuse(*op, "input '" + name + "' is not connected");
+
+        auto shape_in = [&](const std::vector<int>& order) {
+            Array shape;
+            for (int l : order) shape.emplace_back(loops[(size_t) l].extent);
+            if (shape.empty()) shape.emplace_back("1");
+            return Value(std::move(shape));
+        };
+        auto bind = [&](const char* connector, const OperandWalk& w) {
+            Value b = w.binding;
+            b.set("connector", connector);
+            return b;
+        };
+        if (out.scalar && !out_is_pointer) refuse(block, "a scalar computed by a tasklet");
+
+        Value node{Object{}};
+        node.set("type", "library_node");
+        node.set("element_id", op_id);
+        node.set("implementation_type", "NONE");
+        node.set("side_effect", false);
+        node.set("element_type", types::primitive_type_to_string(element));
+        Array inputs, outputs;
+        if (code == "assign") {
+            const OperandWalk& x = in.at(operands.at(0));
+            if (x.scalar) {
+                node.set("code", "ml::Fill");
+                node.set("shape", shape_in(out.order));
+                inputs.push_back(bind("X", x));
+            } else {
+                if (out.scalar) refuse(block, "a tensor stored to one element");
+                // Y[loops in out.order] = X[loops in x.order]: output axis a is the input axis that runs over the same loop
+                Array perm;
+                for (int l : out.order) {
+                    auto pos = std::find(x.order.begin(), x.order.end(), l);
+                    perm.emplace_back((int64_t) (pos - x.order.begin()));
+                }
+                node.set("code", "ml::Transpose");
+                node.set("shape", shape_in(x.order));
+                node.set("perm", Value(std::move(perm)));
+                inputs.push_back(bind("X", x));
+            }
+            outputs.push_back(bind("Y", out));
+        } else if (operands.size() == 1) {
+            const OperandWalk& x = in.at(operands[0]);
+            if (x.scalar || out.scalar || x.order != out.order) refuse(block, "operand and result of the unary operation walk memory differently");
+            node.set("code", code);
+            node.set("shape", shape_in(out.order));
+            inputs.push_back(bind("X", x));
+            outputs.push_back(bind("Y", out));
+        } else {
+            const OperandWalk &a = in.at(operands[0]), &b = in.at(operands[1]);
+            if (out.scalar || (a.scalar && b.scalar)) refuse(block, "a binary operation on scalars only");
+            if ((!a.scalar && a.order != out.order) || (!b.scalar && b.order != out.order))
+                refuse(block, "operands and result of the binary operation walk memory differently");
+            node.set("code", code);
+            node.set("shape", shape_in(out.order));
+            inputs.push_back(bind("A", a));
+            inputs.push_back(bind("B", b));
+            outputs.push_back(bind("C", out));
+        }
+        Value flow;
+        flow.set("library_node", std::move(node));
+        flow.set("inputs", Value(std::move(inputs)));
+        flow.set("outputs", Value(std::move(outputs)));
+        Value b;
+        b.set("type", "block");
+        b.set("element_id", block.at("element_id").as_int());
+        Value dbg = debug_info_of(*op);
+        if (dbg.is_null()) dbg = debug_info_of(block);
+        if (!dbg.is_null()) b.set("debug_info", std::move(dbg));
+        b.set("dataflow", std::move(flow));
+        children.push_back(std::move(b));
+    }
+
     void import_sequence(const Value& seq, Array& children, std::string& returned) {
         if (const Value* transitions = seq.find("transitions"))
             for (auto& t : transitions->as_array())
@@ -296,13 +689,15 @@ struct Import {
                 import_block(child, children);
             } else if (kind == "sequence") {
                 import_sequence(child, children, returned);
+            } else if (kind == "for" || kind == "map") {
+                import_loop_nest(child, children);
             } else if (kind == "return") {
                 const std::string data = child.at("data").as_string();
                 if (child.contains("data_type")) throw InvalidSDFGException(describe(child) + ": returning a constant");
                 returned = data.empty() ? "\x01" : data;
             } else {
-                throw InvalidSDFGException(describe(child) + ": control flow other than a sequence of library-node blocks is not "
-                                           "lowered by the rocm target");
+                throw InvalidSDFGException(describe(child) + ": control flow other than a sequence of library-node blocks and elementwise "
+                                           "loop nests is not lowered by the rocm target");
             }
         }
     }

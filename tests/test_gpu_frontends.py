@@ -402,6 +402,46 @@ def test_program_in_docc_json_format_runs(tmp_path):
     assert rel_err_max(C, ref) <= 1e-12
 
 
+def test_docc_json_return_copy_and_elementwise_nests_run(tmp_path):
+    """`return A @ B` as the front end writes it (GEMM into a temporary, a For nest copying it into `_docc_ret_0`), and
+    Maps holding one tasklet or CMath call each: the nests are matched to the copy / elementwise / fill kernels."""
+    import ctypes
+    import json
+
+    from docc_amd import runtime
+    from docc_amd.sdfg import StructuredSDFG
+    from test_interchange import elementwise_nests_program, return_matmul_program
+
+    s = StructuredSDFG.parse(json.dumps(return_matmul_program()))
+    s.schedule("rocm")
+    fn = ctypes.CDLL(s._compile(str(tmp_path / "mm"))).f_sdfg
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    fn.restype = None
+    rng = np.random.default_rng(5)
+    n = 150
+    A, B = rng.random((n, n)), rng.random((n, n))
+    out = np.full((n, n), np.nan)
+    fn(A.ctypes.data, B.ctypes.data, n, out.ctypes.data)
+    assert runtime.take_failure() == (0, "")
+    assert rel_err_max(out, oracle.gemm(A, B, variant="ld")) <= 1e-12
+
+    s = StructuredSDFG.parse(json.dumps(elementwise_nests_program()))
+    s.schedule("rocm")
+    fn = ctypes.CDLL(s._compile(str(tmp_path / "ew"))).nests_sdfg
+    fn.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int64] * 2
+    fn.restype = None
+    r, c = 37, 129
+    X, Y = (rng.standard_normal((r, c)).astype(np.float32) for _ in range(2))
+    S, E, Z, W = (np.full((r, c), np.nan, np.float32) for _ in range(4))
+    T = np.full((c, r), np.nan, np.float32)
+    fn(*(a.ctypes.data for a in (X, Y, S, E, T, Z, W)), r, c)
+    assert runtime.take_failure() == (0, "")
+    assert np.array_equal(S, X + Y) and np.array_equal(Z, np.full((r, c), 0.5, np.float32))
+    ref = np.exp((X + Y).astype(np.float64))
+    assert rel_err_max(E, ref) <= 1e-5 and np.array_equal(T, E.T)
+    assert rel_err_max(W, E.astype(np.float64) / 3.0) <= 1e-5
+
+
 def test_native_reductions_and_layer_statistics():
     """np.sum / max / min / mean over rows, columns and blocks of axes; the softmax pieces as values of their own."""
     @native(target="rocm")

@@ -92,8 +92,8 @@ def gemm_program():
 
 def test_reference_data_file_pins_the_envelope_and_type_encoding():
     data = json.loads(GOLDEN.read_text())
-    # a loop nest has no lowering on this target: the import stops at the first map and says so
-    with pytest.raises(InvalidSDFGException, match=r"map \(element \d+\): control flow other than a sequence of library-node blocks"):
+    # a tiled loop nest (steps of 32, a reduction inside) matches no elementwise kernel: the import stops at the first map and says so
+    with pytest.raises(InvalidSDFGException, match=r"map \(element \d+\): the loop's step is not 1"):
         StructuredSDFG.from_docc_json(json.dumps(data))
     # its declarations alone import: arrays behind pointers decay to their element type, type numbers as in docc's enum
     head = dict(data, root={"type": "sequence", "element_id": 1, "debug_info": NO_DEBUG, "children": [], "transitions": []})
@@ -101,7 +101,7 @@ def test_reference_data_file_pins_the_envelope_and_type_encoding():
     assert s.name == "sdfg_test" and s.arguments == ["A", "B", "C", "K", "N", "M"]
     assert s.containers["A"] == {"type": "pointer", "element": "Float", "transient": False, "storage": "CPU"}
     assert s.containers["i"]["type"] == "scalar" and s.containers["i"]["element"] == "UInt64" and s.containers["K"]["element"] == "UInt64"
-    # a tasklet block on its own is refused with its element named
+    # a tasklet block on its own (an fma into C[i][j] outside its loops) is refused with its element named
     def first_block(n):
         if n.get("type") == "block":
             return n
@@ -113,7 +113,7 @@ def test_reference_data_file_pins_the_envelope_and_type_encoding():
     blk = first_block(data["root"])
     only = dict(data, root={"type": "sequence", "element_id": 1, "debug_info": NO_DEBUG, "children": [blk],
                             "transitions": [{"type": "transition", "element_id": 2, "debug_info": NO_DEBUG, "assignments": []}]})
-    with pytest.raises(InvalidSDFGException, match=r"tasklet \(element \d+\) in block"):
+    with pytest.raises(InvalidSDFGException, match=r"block \(element \d+\): "):
         StructuredSDFG.from_docc_json(json.dumps(only))
 
 
@@ -237,3 +237,169 @@ def test_cast_and_transpose_nodes_cross_the_formats():
     strip = lambda nodes: [{k: v for k, v in n.items() if k != "element_id"} for n in nodes]
     assert strip(again.library_nodes()) == strip(s.library_nodes())
     assert again.library_nodes()[0]["element_type"] == "Float" and again.library_nodes()[0]["target_type"] == "BFloat"
+
+
+# ---- loop nests that are elementwise work -------------------------------------------------------------
+# What the front end writes for `Y[:, :] = X` and for the copy into the return buffer (python/docc/python/
+# ast_parser.py:1186-1210, :2102-2270): one For per sliced dimension (var = 0; var < extent; var = 1 + var), and in
+# the innermost body a block with one assign tasklet whose memlets carry a Tensor type and one loop variable per
+# dimension. The elementwise tensor nodes expand to Maps of the same shape (elementwise_node.cpp:86-240).
+
+def tensor(prim, shape, strides=None):
+    if strides is None:
+        strides, acc = [], []
+        for d in reversed(shape):
+            strides.insert(0, "*".join(acc) if acc else "1")
+            acc.insert(0, d)
+    return {"type": "tensor", "element_type": scalar(prim), "shape": list(shape), "strides": list(strides), "offset": "0",
+            "storage_type": STACK, "initializer": "", "alignment": 0}
+
+
+def docc_nest(ids, kind, loops, op, inputs, output):
+    """loops: [(variable, extent)], outermost first; inputs: [(connector, container or (literal, prim), subset, base type)];
+    output: (connector, container, subset, base type); op: the tasklet or CMath node without its ids."""
+    op = {"element_id": ids(), "debug_info": NO_DEBUG, **op}
+    nodes, edges = [op], []
+    for conn, value, subset, base in inputs:
+        nid = ids()
+        if isinstance(value, tuple):
+            nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "constant_node", "data": value[0], "data_type": scalar(value[1])})
+        else:
+            nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "access_node", "data": value})
+        edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": nid, "dst": op["element_id"], "src_conn": "void", "dst_conn": conn,
+                      "subset": list(subset), "base_type": base})
+    conn, name, subset, base = output
+    nid = ids()
+    nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "access_node", "data": name})
+    edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": op["element_id"], "dst": nid, "src_conn": conn, "dst_conn": "void",
+                  "subset": list(subset), "base_type": base})
+    body = {"type": "block", "element_id": ids(), "debug_info": NO_DEBUG, "dataflow": {"type": "dataflow", "nodes": nodes, "edges": edges}}
+    for var, extent in reversed(loops):
+        seq = {"type": "sequence", "element_id": ids(), "debug_info": NO_DEBUG, "children": [body],
+               "transitions": [{"type": "transition", "element_id": ids(), "debug_info": NO_DEBUG, "assignments": []}]}
+        body = {"type": kind, "element_id": ids(), "debug_info": NO_DEBUG, "indvar": var, "init": "0", "condition": f"{var} < {extent}",
+                "update": f"1 + {var}", "root": seq}
+        if kind == "map":
+            body["schedule_type"] = {"value": "SEQUENTIAL", "category": 0, "properties": {}}
+    return body
+
+
+ASSIGN = {"type": "tasklet", "code": 0, "inputs": ["_in"], "output": "_out"}
+
+
+def return_matmul_program():
+    """`def f(A, B): return A @ B` as the front end leaves it: the product in a Malloc'ed temporary, a copy nest into
+    the return buffer, the temporary freed, return."""
+    ids = Ids()
+    containers = {n: pointer(DOUBLE) for n in ("A", "B", "_docc_ret_0", "_tmp_0")}
+    for n in ("_s0", "_slice_iter_0_", "_slice_iter_1_"):
+        containers[n] = scalar(INT64)
+    gemm = {"implementation_type": "BLAS", "code": "GEMM", "precision": ord("d"), "layout": 101, "trans_a": 111, "trans_b": 111,
+            "m": "_s0", "n": "_s0", "k": "_s0", "lda": "_s0", "ldb": "_s0", "ldc": "_s0"}
+    t = tensor(DOUBLE, ["_s0", "_s0"])
+    idx = ["_slice_iter_0_", "_slice_iter_1_"]
+    children = [
+        docc_block(ids, {"implementation_type": "NONE", "code": "Malloc", "size": "8*_s0**2"}, [], [("_ret", "_tmp_0")], containers),
+        docc_block(ids, gemm, [("__A", "A"), ("__B", "B"), ("__C", "_tmp_0"), ("__alpha", ("1.0", DOUBLE)), ("__beta", ("0.0", DOUBLE))],
+                   [("__C", "_tmp_0")], containers),
+        docc_nest(ids, "for", [("_slice_iter_0_", "_s0"), ("_slice_iter_1_", "_s0")], ASSIGN,
+                  [("_in", "_tmp_0", idx, t)], ("_out", "_docc_ret_0", idx, t)),
+        docc_block(ids, {"implementation_type": "NONE", "code": "Free"}, [("_ptr", "_tmp_0")], [("_ptr", "_tmp_0")], containers),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    return docc_sdfg("f_sdfg", containers, ["A", "B", "_s0", "_docc_ret_0"], children, ids)
+
+
+def elementwise_nests_program():
+    """Maps as the expanded tensor nodes leave them, over [_s0, _s1] fp32 buffers indexed by one linearised expression:
+    S = X + Y; E = exp(S); T[j][i] = E[i][j] (T is [_s1, _s0]); Z = 0.5 everywhere; W = E / 3."""
+    ids = Ids()
+    containers = {n: pointer(FLOAT) for n in ("X", "Y", "S", "E", "T", "Z", "W")}
+    for n in ("_s0", "_s1", "_i0", "_i1"):
+        containers[n] = scalar(INT64)
+    P = pointer(FLOAT)
+    loops = [("_i0", "_s0"), ("_i1", "_s1")]
+    rm, cm = ["_i1 + _i0*_s1"], ["_i0 + _i1*_s0"]
+    children = [
+        docc_nest(ids, "map", loops, {"type": "tasklet", "code": 2, "inputs": ["_in1", "_in2"], "output": "_out"},
+                  [("_in1", "X", rm, P), ("_in2", "Y", rm, P)], ("_out", "S", rm, P)),
+        docc_nest(ids, "map", loops, {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "expf",
+                                      "function_stem": "exp", "primitive_type": FLOAT},
+                  [("_in1", "S", rm, P)], ("_out", "E", rm, P)),
+        docc_nest(ids, "map", loops, ASSIGN, [("_in", "E", rm, P)], ("_out", "T", cm, P)),
+        docc_nest(ids, "map", loops, ASSIGN, [("_in", ("0.5f", FLOAT), [], scalar(FLOAT))], ("_out", "Z", rm, P)),
+        docc_nest(ids, "map", loops, {"type": "tasklet", "code": 5, "inputs": ["_in1", "_in2"], "output": "_out"},
+                  [("_in1", "E", rm, P), ("_in2", ("3.0f", FLOAT), [], scalar(FLOAT))], ("_out", "W", rm, P)),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    return docc_sdfg("nests_sdfg", containers, ["X", "Y", "S", "E", "T", "Z", "W", "_s0", "_s1"], children, ids)
+
+
+def test_return_copy_nest_imports_as_a_copy_kernel(tmp_path):
+    s = StructuredSDFG.from_docc_json(json.dumps(return_matmul_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["GEMM", "ml::Transpose"]
+    assert nodes[1]["shape"] == ["_s0", "_s0"] and nodes[1]["perm"] == [0, 1] and nodes[1]["element_type"] == "Double"
+    copy_block = s._data["root"]["children"][1]["dataflow"]
+    assert copy_block["inputs"] == [{"data": "_tmp_0", "connector": "X"}] and copy_block["outputs"] == [{"data": "_docc_ret_0", "connector": "Y"}]
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["H2D"] == 2 and r["D2H"] == 1            # A and B up, the return buffer down; the product never leaves the device
+    src = Path(s.generate(str(tmp_path))["source"]).read_text()
+    assert src.count("docc_rocm_dgemm(") == 1 and src.count("docc_rocm_transpose(") == 1
+    assert 'extern "C" void f_sdfg(double *A, double *B, int64_t _s0, double *_docc_ret_0)' in src
+
+
+def test_elementwise_nests_import_as_tensor_nodes():
+    s = StructuredSDFG.from_docc_json(json.dumps(elementwise_nests_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["ml::Add", "ml::Exp", "ml::Transpose", "ml::Fill", "ml::Div"]
+    assert all(n["shape"] == ["_s0", "_s1"] for n in nodes) and all(n["element_type"] == "Float" for n in nodes)
+    assert nodes[2]["perm"] == [1, 0]
+    blocks = [c["dataflow"] for c in s._data["root"]["children"][:5]]
+    assert blocks[0]["inputs"] == [{"data": "X", "connector": "A"}, {"data": "Y", "connector": "B"}] and blocks[0]["outputs"] == [{"data": "S", "connector": "C"}]
+    assert blocks[3]["inputs"] == [{"constant": "0.5f", "type": "Float", "connector": "X"}]
+    assert blocks[4]["inputs"][1] == {"constant": "3.0f", "type": "Float", "connector": "B"}
+    s.schedule("rocm")
+
+
+def test_loop_nests_outside_the_elementwise_forms_are_refused():
+    base = elementwise_nests_program()
+
+    def nest(i):
+        return base["root"]["children"][i]
+
+    def inner_block(n):
+        while n["type"] != "block":
+            n = n["root"]["children"][0] if n["type"] in ("for", "map") else n["children"][0]
+        return n
+
+    def refused(prog, why):
+        with pytest.raises(InvalidSDFGException, match=why):
+            StructuredSDFG.from_docc_json(json.dumps(prog))
+
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["init"] = "1"
+    refused(bad, r"map \(element \d+\): the loop does not start at 0")
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["condition"] = "_i0 <= _s0"
+    refused(bad, "condition is not 'variable < bound'")
+    bad = copy.deepcopy(base)
+    inner_block(bad["root"]["children"][0])["dataflow"]["edges"][0]["subset"] = ["_i1 + _i0*_s0"]      # wrong row pitch: not the dense tensor of the nest
+    refused(bad, "operand 'X' is not a dense tensor indexed by the loop variables")
+    bad = copy.deepcopy(base)
+    inner_block(bad["root"]["children"][0])["dataflow"]["edges"][0]["subset"] = ["1 + _i1 + _i0*_s1"]  # shifted by one element
+    refused(bad, "operand 'X' is not a dense tensor")
+    bad = copy.deepcopy(base)
+    inner_block(bad["root"]["children"][0])["dataflow"]["edges"][1]["subset"] = ["_i0 + _i1*_s0"]      # X + Y^T: no kernel walks the operands differently
+    refused(bad, "walk memory differently")
+    bad = copy.deepcopy(base)
+    inner_block(bad["root"]["children"][0])["dataflow"]["nodes"][0]["code"] = 6                        # fp_rem
+    refused(bad, r"tasklet code 6 has no kernel")
+    bad = copy.deepcopy(base)
+    inner_block(bad["root"]["children"][1])["dataflow"]["nodes"][0]["function_stem"] = "lgamma"
+    refused(bad, "CMath function 'lgamma' has no kernel")
+    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["root"]["children"].append(copy.deepcopy(inner_block(nest(1))))
+    bad["root"]["children"][0]["root"]["transitions"].append(copy.deepcopy(bad["root"]["children"][0]["root"]["transitions"][0]))
+    refused(bad, "more than one statement in a loop body")
