@@ -67,6 +67,49 @@ def _map_python_type(value: Any):
     raise TypeError(f"unsupported argument type {type(value).__name__}")
 
 
+def _map_annotation(ann: Any):
+    """One return annotation -> SDFG type, or None if it names nothing this front end can declare ahead of the body
+    (reference python_program.py:40-100: Annotated[np.ndarray, shape, dtype], np.ndarray[shape, dtype], float, int, ...)."""
+    import typing
+
+    if typing.get_origin(ann) is typing.Annotated:
+        base, *meta = typing.get_args(ann)
+        if base is np.ndarray:
+            elem = _map_annotation(meta[1]) if len(meta) > 1 else Scalar(PrimitiveType.Double)
+            return Pointer(elem) if isinstance(elem, Scalar) else None
+        return None
+    if typing.get_origin(ann) is np.ndarray:
+        args = typing.get_args(ann)
+        if len(args) >= 2:
+            dt = args[1]
+            inner = typing.get_args(dt)
+            elem = _map_annotation(inner[0] if typing.get_origin(dt) is np.dtype and inner else dt)
+            return Pointer(elem) if isinstance(elem, Scalar) else None
+        return None
+    table = {float: PrimitiveType.Double, np.float64: PrimitiveType.Double, np.float32: PrimitiveType.Float, bool: PrimitiveType.Bool,
+             np.bool_: PrimitiveType.Bool, int: PrimitiveType.Int64, np.int64: PrimitiveType.Int64, np.int32: PrimitiveType.Int32}
+    try:
+        return Scalar(table[ann]) if ann in table else None
+    except TypeError:   # unhashable annotation
+        return None
+
+
+def _return_annotation_types(func) -> Optional[List[Any]]:
+    """The types a return annotation declares (a tuple annotation: one per element), or None: no annotation, or one that
+    does not map - the outputs are then inferred from the body (reference python_program.py:478-512)."""
+    import typing
+
+    ann = inspect.signature(func).return_annotation
+    if ann is inspect.Signature.empty or isinstance(ann, str):
+        return None
+    if typing.get_origin(ann) is tuple:
+        items = [a for a in typing.get_args(ann) if a is not Ellipsis]
+    else:
+        items = [ann]
+    types = [_map_annotation(a) for a in items]
+    return None if any(t is None for t in types) else types
+
+
 def _mul(a: str, b: str) -> str:
     if a == "1":
         return b
@@ -133,6 +176,9 @@ class _Lowering(ast.NodeVisitor):
         if dest is not None:
             if not self.b.exists(dest):  # a `_docc_ret_<i>` output: becomes a trailing pointer argument
                 self.b.add_container(dest, Pointer(Scalar(elem)), True)
+            elif self.b._data["containers"][dest]["element"] != elem.value:   # declared by the return annotation
+                raise TypeError(f"{self.func.__name__}: the return annotation declares {self.b._data['containers'][dest]['element']} "
+                                f"for output {dest}, the returned value is {elem.value}")
             return _Array(dest, shape, elem)
         size = str(_SIZES[elem])
         for s in shape:
@@ -693,6 +739,11 @@ class PythonProgram(DoccProgram):
             raise TypeError(f"{self.name}() takes {len(params)} positional arguments but {len(args)} were given")
         builder = StructuredSDFGBuilder(f"{self.name}_sdfg")
         env: Dict[str, Any] = {}
+        # outputs a return annotation declares come first in the argument list: the reference adds them before it looks
+        # at the parameters (python_program.py:515-524); a scalar is returned through a pointer
+        declared = _return_annotation_types(self.func) or []
+        for i, t in enumerate(declared):
+            builder.add_container(f"_docc_ret_{i}", t if isinstance(t, Pointer) else Pointer(t), True)
         for i, (p, a, t) in enumerate(zip(params, args, arg_types)):
             builder.add_container(p, t, True)
             if isinstance(a, np.ndarray):

@@ -493,3 +493,38 @@ def test_transposes_lower_to_a_gemm_flag_or_a_transpose_node():
 
     with pytest.raises(ValueError, match="axes"):
         repeated_axis.to_sdfg(x)
+
+
+def test_return_annotation_puts_the_outputs_first():
+    """With a return annotation the reference declares `_docc_ret_<i>` before it looks at the parameters
+    (python/docc/python/python_program.py:515-524): the outputs lead the argument list of the generated function."""
+    from typing import Annotated, Tuple
+
+    @native(target="rocm")
+    def annotated(a, b) -> Annotated[np.ndarray, (None, None), np.float64]:
+        return a @ b
+
+    a = np.random.rand(6, 6)
+    sdfg = annotated.to_sdfg(a, a)
+    assert sdfg.arguments == ["_docc_ret_0", "a", "b", "_s0"]
+    sdfg.schedule("rocm")
+    src = Path(sdfg.generate(str(Path(__import__("os").environ["DOCC_TMP"]) / "annotated"))["source"]).read_text()
+    assert 'extern "C" void annotated_sdfg(double *_docc_ret_0, double *a, double *b, int64_t _s0)' in src
+
+    @native(target="rocm")
+    def two(a, b) -> Tuple[Annotated[np.ndarray, (None, None), np.float32], Annotated[np.ndarray, (None, None), np.float32]]:
+        return a @ b, relu(a)
+
+    f = np.zeros((4, 4), np.float32)
+    assert two.to_sdfg(f, f).arguments == ["_docc_ret_0", "_docc_ret_1", "a", "b", "_s0"]
+
+    # an element type other than the declared one is an error, not a silent reinterpretation
+    with pytest.raises(TypeError, match="declares Double for output _docc_ret_0, the returned value is Float"):
+        annotated.to_sdfg(f, f)
+
+    # an annotation that maps to nothing leaves the outputs to the body, as without one
+    @native(target="rocm")
+    def loose(a, b) -> "whatever":
+        return a @ b
+
+    assert loose.to_sdfg(a, a).arguments == ["a", "b", "_s0", "_docc_ret_0"]

@@ -46,6 +46,22 @@ def test_native_matmul_config_1():
     assert len(matmul.cache) == 1
 
 
+def test_native_matmul_with_a_return_annotation():
+    """The annotation moves `_docc_ret_0` to the front of the generated function's arguments
+    (reference python_program.py:515-524); the caller walks the arguments by name."""
+    from typing import Annotated
+
+    @native(target="rocm")
+    def annotated_mm(a, b) -> Annotated[np.ndarray, (None, None), np.float64]:
+        return a @ b
+
+    rng = np.random.default_rng(3)
+    A, B = rng.random((96, 80)), rng.random((80, 72))
+    C = annotated_mm(A, B)
+    assert annotated_mm.last_sdfg.arguments[0] == "_docc_ret_0"
+    assert C.shape == (96, 72) and rel_err_max(C, oracle.gemm(A, B, variant="ld")) <= 1e-12
+
+
 @pytest.mark.parametrize("offload", ["function", "node"])
 def test_native_polybench_gemm(offload):
     @native(target="rocm", offload=offload)
