@@ -330,6 +330,37 @@ bool CPPCodeGenerator::as_source(const std::filesystem::path& header_path, const
 
 } // namespace sdfg::codegen
 
+namespace sdfg::plugins {
+
+TargetMapperRegistry& TargetMapperRegistry::instance() {
+    static TargetMapperRegistry registry;
+    return registry;
+}
+
+const std::vector<std::shared_ptr<TargetMapperFactory>> TargetMapperRegistry::get_all_mappers() {
+    std::lock_guard<std::mutex> lock(mutex_);
+    return factories_;
+}
+
+void TargetMapperRegistry::register_target_mapper(std::shared_ptr<TargetMapperFactory> factory) {
+    if (!factory) return;
+    std::lock_guard<std::mutex> lock(mutex_);
+    // highest priority first; equal priorities in the order they were registered
+    const int p = factory->priority();
+    auto it = factories_.begin();
+    while (it != factories_.end() && (*it)->priority() >= p) ++it;
+    factories_.insert(it, std::move(factory));
+}
+
+std::vector<std::shared_ptr<TargetMapper>> TargetMapperRegistry::create_for_target(const std::string& target) {
+    std::vector<std::shared_ptr<TargetMapper>> mappers;
+    for (auto& f : get_all_mappers())
+        if (f->for_target() == target) mappers.push_back(f->create());
+    return mappers;
+}
+
+} // namespace sdfg::plugins
+
 namespace sdfg::passes {
 
 bool TargetMappingPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager) {

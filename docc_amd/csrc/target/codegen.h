@@ -165,7 +165,7 @@ private:
 class LibraryNodeDispatcher {
 public:
     LibraryNodeDispatcher(LanguageExtension& language_extension, const Function& function,
-                          const structured_control_flow::Block& data_flow_graph, const data_flow::LibraryNode& node)
+                          const data_flow::DataFlowGraph& data_flow_graph, const data_flow::LibraryNode& node)
         : language_extension_(language_extension), function_(function), data_flow_graph_(data_flow_graph), node_(node) {}
     virtual ~LibraryNodeDispatcher() = default;
 
@@ -180,12 +180,13 @@ public:
 protected:
     LanguageExtension& language_extension_;
     const Function& function_;
-    const structured_control_flow::Block& data_flow_graph_;
+    const data_flow::DataFlowGraph& data_flow_graph_;
     const data_flow::LibraryNode& node_;
 };
 
+// the reference's parameter list (codegen/dispatchers/node_dispatcher_registry.h:140-141)
 using LibraryNodeDispatcherFn = std::function<std::unique_ptr<LibraryNodeDispatcher>(
-    LanguageExtension&, const Function&, const structured_control_flow::Block&, const data_flow::LibraryNode&)>;
+    LanguageExtension&, const Function&, const data_flow::DataFlowGraph&, const data_flow::LibraryNode&)>;
 
 class LibraryNodeDispatcherRegistry {
 public:
@@ -259,6 +260,29 @@ public:
     virtual ~TargetMapper() = default;
     virtual bool try_map(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager,
                          data_flow::LibraryNode& node) const = 0;
+};
+
+// reference: sdfg/include/sdfg/plugins/target_mapping.h:24-37 (declared there, with no definition in the tree; the
+// registry here keeps the factories ordered by priority, highest first, and by registration within one priority)
+class TargetMapperFactory {
+public:
+    virtual ~TargetMapperFactory() = default;
+    virtual std::unique_ptr<TargetMapper> create() const = 0;
+    virtual int priority() = 0;
+    virtual const std::string& for_target() const = 0;
+};
+
+class TargetMapperRegistry {
+public:
+    static TargetMapperRegistry& instance();
+    const std::vector<std::shared_ptr<TargetMapperFactory>> get_all_mappers();
+    void register_target_mapper(std::shared_ptr<TargetMapperFactory> factory);
+    // the mappers of one target, in the order get_all_mappers() gives
+    std::vector<std::shared_ptr<TargetMapper>> create_for_target(const std::string& target);
+
+private:
+    std::mutex mutex_;
+    std::vector<std::shared_ptr<TargetMapperFactory>> factories_;
 };
 
 } // namespace sdfg::plugins

@@ -1,6 +1,7 @@
 #include "rocm_target.h"
 
 #include <algorithm>
+#include <mutex>
 #include <set>
 #include <sstream>
 
@@ -12,6 +13,7 @@ using codegen::LanguageExtension;
 using codegen::LibraryNodeDispatcher;
 using codegen::PrettyPrinter;
 using data_flow::ConnectorBinding;
+using data_flow::DataFlowGraph;
 using data_flow::LibraryNode;
 using structured_control_flow::Block;
 namespace blas = math::blas;
@@ -98,7 +100,7 @@ Expression sum_bytes(const std::vector<DeviceOperand>& ops) {
 // with or without the surrounding transfers.
 class RocmMathDispatcher : public LibraryNodeDispatcher {
 public:
-    RocmMathDispatcher(LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n, bool with_transfers)
+    RocmMathDispatcher(LanguageExtension& le, const Function& f, const DataFlowGraph& b, const LibraryNode& n, bool with_transfers)
         : LibraryNodeDispatcher(le, f, b, n), with_transfers_(with_transfers) {}
 
     void dispatch_code(PrettyPrinter& stream, PrettyPrinter& globals, CodeSnippetFactory&) override {
@@ -685,7 +687,7 @@ void register_math(codegen::LibraryNodeDispatcherRegistry& reg, const std::strin
     for (bool with : {true, false}) {
         reg.register_library_node_dispatcher(
             code + "::" + (with ? ImplementationType_ROCMWithTransfers : ImplementationType_ROCMWithoutTransfers),
-            [with](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
+            [with](LanguageExtension& le, const Function& f, const DataFlowGraph& b, const LibraryNode& n) {
                 return std::make_unique<D>(le, f, b, n, with);
             });
     }
@@ -719,7 +721,7 @@ void register_plugin(plugins::Context& context) {
     register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
     reg.register_library_node_dispatcher(
         LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
-        [](LanguageExtension& le, const Function& f, const Block& b, const LibraryNode& n) {
+        [](LanguageExtension& le, const Function& f, const DataFlowGraph& b, const LibraryNode& n) {
             return std::make_unique<ROCMDataOffloadingNodeDispatcher>(le, f, b, n);
         });
 }
@@ -727,6 +729,14 @@ void register_plugin(plugins::Context& context) {
 void register_rocm_plugin() {
     auto context = plugins::Context::global_context();
     register_plugin(context);
+    // the mapper's factory, once (the dispatcher registry ignores a second registration by itself)
+    static std::once_flag once;
+    std::call_once(once, [] { plugins::TargetMapperRegistry::instance().register_target_mapper(std::make_shared<RocmLibNodeMapperFactory>()); });
+}
+
+const std::string& RocmLibNodeMapperFactory::for_target() const {
+    static const std::string target = "rocm";
+    return target;
 }
 
 const plugins::Plugin rocm_plugin = {"rocm", "0.1", "MI355X (gfx950) target for the math library nodes", &register_plugin};

@@ -40,6 +40,22 @@ private:
     mutable std::string reason_;
 };
 
+// The mapper's factory as a docc plugin hands it over (plugins::TargetMapperFactory, reference
+// sdfg/include/sdfg/plugins/target_mapping.h:24-30): target "rocm", one factory per implementation type.
+// register_plugin() puts the ROCMWithoutTransfers one (the default schedule) into plugins::TargetMapperRegistry.
+class RocmLibNodeMapperFactory : public plugins::TargetMapperFactory {
+public:
+    explicit RocmLibNodeMapperFactory(std::string implementation_type = ImplementationType_ROCMWithoutTransfers, int priority = 100)
+        : implementation_type_(std::move(implementation_type)), priority_(priority) {}
+    std::unique_ptr<plugins::TargetMapper> create() const override { return std::make_unique<RocmLibNodeMapper>(implementation_type_); }
+    int priority() override { return priority_; }
+    const std::string& for_target() const override;
+
+private:
+    std::string implementation_type_;
+    int priority_;
+};
+
 // Surrounds every ROCMWithoutTransfers node with offloading blocks (ALLOC[+H2D] before,
 // [D2H+]FREE after) on device containers `__daisy_rocm_<element id>_<container>`.
 class RocmOffloadTransform {

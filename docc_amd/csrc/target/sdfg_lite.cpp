@@ -872,21 +872,21 @@ std::unique_ptr<ROCMDataOffloadingNode> ROCMDataOffloadingNode::from_json(const 
 
 // ------------------------------------------------------------------- SDFG
 
-namespace structured_control_flow {
+namespace data_flow {
 
-const data_flow::ConnectorBinding* Block::input(const std::string& connector) const {
+const data_flow::ConnectorBinding* DataFlowGraph::input(const std::string& connector) const {
     for (auto& b : inputs)
         if (b.connector == connector) return &b;
     return nullptr;
 }
 
-const data_flow::ConnectorBinding* Block::output(const std::string& connector) const {
+const data_flow::ConnectorBinding* DataFlowGraph::output(const std::string& connector) const {
     for (auto& b : outputs)
         if (b.connector == connector) return &b;
     return nullptr;
 }
 
-} // namespace structured_control_flow
+} // namespace data_flow
 
 const Container& StructuredSDFG::container(const std::string& name) const {
     auto it = containers_.find(name);

@@ -573,6 +573,23 @@ private:
 
 } // namespace rocm
 
+namespace data_flow {
+
+// The dataflow of a block as this target needs it: the one library node and what its connectors are bound to.
+// It stands where the reference's data_flow::DataFlowGraph stands in the dispatcher interfaces
+// (codegen/dispatchers/node_dispatcher_registry.h:140-141); there a dispatcher reaches the same facts through
+// in_edges(node) / out_edges(node) and the access or constant node at the other end of each memlet.
+struct DataFlowGraph {
+    std::unique_ptr<LibraryNode> node;
+    std::vector<ConnectorBinding> inputs;
+    std::vector<ConnectorBinding> outputs;
+
+    const ConnectorBinding* input(const std::string& connector) const;
+    const ConnectorBinding* output(const std::string& connector) const;
+};
+
+} // namespace data_flow
+
 namespace structured_control_flow {
 
 // Source position of an element (reference sdfg/include/sdfg/element.h DebugInfo; JSON keys of
@@ -584,16 +601,14 @@ struct DebugInfo {
     long start_line = 0, start_column = 0, end_line = 0, end_column = 0;
 };
 
-// One block of the root sequence: a dataflow graph with exactly one library node.
-struct Block {
+// One block of the root sequence: a dataflow graph with exactly one library node
+// (reference structured_control_flow/block.h: Block::dataflow()).
+struct Block : public data_flow::DataFlowGraph {
     size_t element_id = 0;
     DebugInfo debug_info;
-    std::unique_ptr<data_flow::LibraryNode> node;
-    std::vector<data_flow::ConnectorBinding> inputs;
-    std::vector<data_flow::ConnectorBinding> outputs;
 
-    const data_flow::ConnectorBinding* input(const std::string& connector) const;
-    const data_flow::ConnectorBinding* output(const std::string& connector) const;
+    const data_flow::DataFlowGraph& dataflow() const { return *this; }
+    data_flow::DataFlowGraph& dataflow() { return *this; }
 };
 
 } // namespace structured_control_flow

@@ -103,6 +103,20 @@ char* docc_rocm_target_dispatcher_keys(void) {
     });
 }
 
+char* docc_rocm_target_mappers(void) {
+    return guarded([] {
+        rocm::register_rocm_plugin();
+        json::Array a;
+        for (auto& f : plugins::TargetMapperRegistry::instance().get_all_mappers()) {
+            json::Value e;
+            e.set("target", f->for_target());
+            e.set("priority", (int64_t) f->priority());
+            a.push_back(std::move(e));
+        }
+        return json::Value(std::move(a)).dump();
+    });
+}
+
 char* docc_rocm_target_validate(const char* sdfg_json) {
     return guarded([&] { return parse(sdfg_json)->to_json().dump(2); });
 }

@@ -29,7 +29,7 @@ EXPORTED_SYMBOLS = (
     "docc_rocm_target_register", "docc_rocm_target_dispatcher_keys", "docc_rocm_target_validate",
     "docc_rocm_target_schedule", "docc_rocm_target_generate", "docc_rocm_target_compile",
     "docc_rocm_target_report", "docc_rocm_target_free", "docc_rocm_target_last_error",
-    "docc_rocm_target_import", "docc_rocm_target_export",
+    "docc_rocm_target_import", "docc_rocm_target_export", "docc_rocm_target_mappers",
 )
 
 
@@ -45,7 +45,7 @@ def _native() -> ctypes.CDLL:
         lib = ctypes.CDLL(str(_TARGET_LIB))
         cp = ctypes.c_char_p
         lib.docc_rocm_target_register.restype = ctypes.c_int
-        for name, args in (("docc_rocm_target_dispatcher_keys", []), ("docc_rocm_target_validate", [cp]),
+        for name, args in (("docc_rocm_target_dispatcher_keys", []), ("docc_rocm_target_mappers", []), ("docc_rocm_target_validate", [cp]),
                            ("docc_rocm_target_schedule", [cp, cp, cp]),
                            ("docc_rocm_target_import", [cp]), ("docc_rocm_target_export", [cp]), ("docc_rocm_target_generate", [cp, cp, cp]),
                            ("docc_rocm_target_compile", [cp, cp, cp, cp, cp]), ("docc_rocm_target_report", [cp])):
@@ -74,6 +74,11 @@ def _call(name: str, *args: Optional[str]) -> str:
 def registered_dispatchers() -> List[str]:
     """The "<code>::<implementation type>" keys the code generator can dispatch."""
     return json.loads(_call("docc_rocm_target_dispatcher_keys"))
+
+
+def registered_target_mappers() -> List[Dict[str, Any]]:
+    """The target mapper factories of the plugin registry, highest priority first: [{"target", "priority"}]."""
+    return json.loads(_call("docc_rocm_target_mappers"))
 
 
 class PrimitiveType(enum.Enum):

@@ -30,6 +30,10 @@ int docc_rocm_target_register(void);
 /* JSON array of the registered "<code>::<implementation type>" dispatcher keys. */
 char* docc_rocm_target_dispatcher_keys(void);
 
+/* JSON array of the target mapper factories in plugins::TargetMapperRegistry, highest priority first:
+ * [{"target": "rocm", "priority": 100}, ...] (reference sdfg/include/sdfg/plugins/target_mapping.h:24-37). */
+char* docc_rocm_target_mappers(void);
+
 /* Parses and validates an SDFG; returns its canonical JSON. Counterpart of
  * StructuredSDFG.parse + validate (reference bindings.cpp:136-160). */
 char* docc_rocm_target_validate(const char* sdfg_json);

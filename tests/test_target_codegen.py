@@ -764,3 +764,83 @@ def test_reduce_nodes_dispatch_and_decline(tmp_path):
     b.add_reduce_op("sum", "X", "Y", [4, 5], [2])
     with pytest.raises(InvalidSDFGException, match="Axis value out of bounds"):
         b.move().validate()
+
+
+def test_cpp_plugin_door_has_the_reference_signatures(tmp_path):
+    """A plugin source written against the reference's interfaces compiles against this target's headers and runs:
+    the dispatcher factory takes (LanguageExtension&, const Function&, const data_flow::DataFlowGraph&, const
+    data_flow::LibraryNode&) (sdfg/include/sdfg/codegen/dispatchers/node_dispatcher_registry.h:140-141), a dispatcher
+    overrides dispatch_code(PrettyPrinter&, PrettyPrinter&, CodeSnippetFactory&), target mappers arrive through
+    TargetMapperFactory / TargetMapperRegistry (sdfg/include/sdfg/plugins/target_mapping.h:24-37) and a plugin registers
+    through plugins::Context (targets/et/src/et/target.cpp:21-36)."""
+    import subprocess
+    from docc_amd.sdfg import registered_target_mappers
+
+    assert {"target": "rocm", "priority": 100} in registered_target_mappers()
+    root = Path(__file__).resolve().parent.parent
+    src = tmp_path / "plugin.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include <functional>
+#include <memory>
+#include <type_traits>
+#include "rocm_target.h"
+using namespace sdfg;
+
+// the reference's factory type, spelled out
+using RefFn = std::function<std::unique_ptr<codegen::LibraryNodeDispatcher>(codegen::LanguageExtension&, const Function&,
+                                                                             const data_flow::DataFlowGraph&, const data_flow::LibraryNode&)>;
+static_assert(std::is_same<codegen::LibraryNodeDispatcherFn, RefFn>::value, "dispatcher factory signature");
+static_assert(std::is_abstract<plugins::TargetMapperFactory>::value && std::is_abstract<plugins::TargetMapper>::value, "mapper interfaces");
+
+class MyDispatcher : public codegen::LibraryNodeDispatcher {
+public:
+    MyDispatcher(codegen::LanguageExtension& le, const Function& f, const data_flow::DataFlowGraph& g, const data_flow::LibraryNode& n)
+        : codegen::LibraryNodeDispatcher(le, f, g, n) {}
+    void dispatch_code(codegen::PrettyPrinter& stream, codegen::PrettyPrinter&, codegen::CodeSnippetFactory&) override {
+        stream << "/* " << node_.code() << " with " << data_flow_graph_.inputs.size() << " inputs */" << std::endl;
+    }
+};
+
+class MyMapper : public plugins::TargetMapper {
+public:
+    bool try_map(builder::StructuredSDFGBuilder&, analysis::AnalysisManager&, data_flow::LibraryNode&) const override { return false; }
+};
+class MyFactory : public plugins::TargetMapperFactory {
+public:
+    std::unique_ptr<plugins::TargetMapper> create() const override { return std::make_unique<MyMapper>(); }
+    int priority() override { return 500; }
+    const std::string& for_target() const override { static const std::string t = "mine"; return t; }
+};
+
+static void register_mine(plugins::Context& context) {
+    context.library_node_dispatcher_registry.register_library_node_dispatcher(
+        "GEMM::MINE", [](codegen::LanguageExtension& le, const Function& f, const data_flow::DataFlowGraph& g, const data_flow::LibraryNode& n) {
+            return std::make_unique<MyDispatcher>(le, f, g, n);
+        });
+}
+
+int main() {
+    auto context = plugins::Context::global_context();
+    rocm::register_plugin(context);     // the rocm plugin's own entry, as docc would call it
+    register_mine(context);
+    auto& reg = codegen::LibraryNodeDispatcherRegistry::instance();
+    if (!reg.get_library_node_dispatcher("GEMM::MINE") || !reg.get_library_node_dispatcher("GEMM::ROCMWithoutTransfers")) return 1;
+    rocm::register_rocm_plugin();
+    auto& mappers = plugins::TargetMapperRegistry::instance();
+    mappers.register_target_mapper(std::make_shared<MyFactory>());
+    auto all = mappers.get_all_mappers();
+    if (all.size() != 2 || all[0]->for_target() != "mine" || all[1]->for_target() != "rocm") return 2;     // by priority
+    auto rocm_mappers = mappers.create_for_target("rocm");
+    if (rocm_mappers.size() != 1 || dynamic_cast<rocm::RocmLibNodeMapper*>(rocm_mappers[0].get()) == nullptr) return 3;
+    std::puts("ok");
+    return 0;
+}
+''')
+    exe = tmp_path / "plugin"
+    lib_dir = root / "docc_amd" / "lib"
+    r = subprocess.run(["g++", "-std=c++17", "-I", str(root / "docc_amd" / "csrc" / "target"), str(src), "-o", str(exe),
+                        "-L", str(lib_dir), "-ldocc_rocm_target", f"-Wl,-rpath,{lib_dir}"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-3000:]
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", (r.returncode, r.stdout, r.stderr)
