@@ -1,5 +1,7 @@
 #include "codegen.h"
 
+#include <map>
+
 #include <algorithm>
 #include <fstream>
 
@@ -59,8 +61,42 @@ CodeSnippet& CodeSnippetFactory::require(const std::string& name, const std::str
 
 void LibraryNodeDispatcher::dispatch(PrettyPrinter& stream, PrettyPrinter& globals_stream,
                                      CodeSnippetFactory& library_snippet_factory) {
+    // A connector's local hides a container of the same name for the rest of the scope (and `T *X = X;` reads the
+    // local itself). The reference's connectors are spelled `__A`, `_in`, ... and never meet a container; the tensor
+    // nodes' are `X`, `Y`, `A`, `B`, `C`, which a user's arrays may be called too. Where a connector of this node and
+    // a container bound to it share a name, the containers are first copied under names nothing else uses.
+    bool clash = false;
+    auto bound = [&](const std::string& name) {
+        for (auto& in : data_flow_graph_.inputs)
+            if (!in.is_constant && in.data == name) return true;
+        for (auto& out : data_flow_graph_.outputs)
+            if (out.data == name) return true;
+        return false;
+    };
+    for (auto& in : data_flow_graph_.inputs) clash = clash || bound(in.connector);
+    for (auto& out : data_flow_graph_.outputs) clash = clash || bound(out.connector);
+
     stream << "{" << std::endl;
     stream.setIndent(stream.indent() + 4);
+    std::map<std::string, std::string> alias;   // connector -> the name its container's value is read from / written to
+    if (clash) {
+        size_t k = 0;
+        auto capture = [&](const std::string& connector, const std::string& data) {
+            const std::string name = "__docc_bound_" + std::to_string(k++);
+            stream << language_extension_.declaration(name, function_.container(data)) << " = " << data << ";" << std::endl;
+            alias[connector] = name;
+        };
+        for (auto& in : data_flow_graph_.inputs)
+            if (!in.is_constant) capture(in.connector, in.data);
+        for (auto& out : data_flow_graph_.outputs)
+            if (!data_flow_graph_.input(out.connector)) capture(out.connector, out.data);
+        stream << "{" << std::endl;
+        stream.setIndent(stream.indent() + 4);
+    }
+    auto source_of = [&](const std::string& connector, const std::string& data) {
+        auto it = alias.find(connector);
+        return it == alias.end() ? data : it->second;
+    };
 
     // one local per input connector: container value or constant literal
     for (auto& in : data_flow_graph_.inputs) {
@@ -68,21 +104,31 @@ void LibraryNodeDispatcher::dispatch(PrettyPrinter& stream, PrettyPrinter& globa
             stream << language_extension_.primitive_type(in.type) << " " << in.connector << " = " << in.data << ";" << std::endl;
         } else {
             const Container& c = function_.container(in.data);
-            stream << language_extension_.declaration(in.connector, c) << " = " << in.data << ";" << std::endl;
+            stream << language_extension_.declaration(in.connector, c) << " = " << source_of(in.connector, in.data) << ";" << std::endl;
         }
     }
     // outputs that are not inputs as well get a local too
     for (auto& out : data_flow_graph_.outputs) {
         if (data_flow_graph_.input(out.connector)) continue;
         const Container& c = function_.container(out.data);
-        stream << language_extension_.declaration(out.connector, c) << " = " << out.data << ";" << std::endl;
+        stream << language_extension_.declaration(out.connector, c) << " = " << source_of(out.connector, out.data) << ";" << std::endl;
     }
     stream << std::endl;
 
     this->dispatch_code(stream, globals_stream, library_snippet_factory);
 
     stream << std::endl;
-    for (auto& out : data_flow_graph_.outputs) stream << out.data << " = " << out.connector << ";" << std::endl;
+    if (clash) {
+        // out of the connectors' scope first, then into the containers
+        for (auto& out : data_flow_graph_.outputs)
+            if (alias.count(out.connector)) stream << alias[out.connector] << " = " << out.connector << ";" << std::endl;
+        stream.setIndent(stream.indent() - 4);
+        stream << "}" << std::endl;
+        for (auto& out : data_flow_graph_.outputs)
+            if (alias.count(out.connector)) stream << out.data << " = " << alias[out.connector] << ";" << std::endl;
+    } else {
+        for (auto& out : data_flow_graph_.outputs) stream << out.data << " = " << out.connector << ";" << std::endl;
+    }
 
     stream.setIndent(stream.indent() - 4);
     stream << "}" << std::endl;

@@ -614,8 +614,51 @@ protected:
     void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
         const auto& n = static_cast<const tensor::ReduceNode&>(node_);
         const int precision = n.element() == types::PrimitiveType::Double ? 64 : 32;
-        s << "DOCC_ROCM_CHECK(docc_rocm_reduce(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision << ", "
-          << n.outer() << ", " << n.extent() << ", " << n.inner() << ", " << name_of("X") << ", " << name_of("Y") << "));" << std::endl;
+        auto call = [&](const Expression& outer, const Expression& extent, const Expression& inner, const std::string& x, const std::string& y) {
+            s << "DOCC_ROCM_CHECK(docc_rocm_reduce(nullptr, " << n.operation() << " /* " << n.code() << " */, " << precision << ", "
+              << outer << ", " << extent << ", " << inner << ", " << x << ", " << y << "));" << std::endl;
+        };
+        if (n.adjacent_axes()) {
+            call(n.outer(), n.extent(), n.inner(), name_of("X"), name_of("Y"));
+            return;
+        }
+        // Axes in several blocks: one reduction per block of adjacent axes, the innermost block first, through device
+        // temporaries (a sum of sums, a maximum of maxima, and - the blocks being full extents - a mean of means).
+        // The reference's expansion is one loop nest over all the axes (reduce_node.cpp:188-333); for Sum and Mean the
+        // order of the additions differs from it, as it does inside one block.
+        const auto axes = n.sorted_axes();
+        std::vector<std::pair<size_t, size_t>> runs;   // [first, last] positions in the current shape
+        for (size_t i = 0; i < axes.size();) {
+            size_t j = i;
+            while (j + 1 < axes.size() && axes[j + 1] == axes[j] + 1) j++;
+            runs.emplace_back((size_t) axes[i], (size_t) axes[j]);
+            i = j + 1;
+        }
+        const Expression elem = symbolic::integer(precision / 8);
+        std::vector<Expression> shape = n.shape();
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        s << "void *__docc_part[2] = {nullptr, nullptr};" << std::endl;
+        std::string from = name_of("X");
+        for (size_t k = runs.size(); k-- > 0;) {
+            const auto [lo, hi] = runs[k];
+            const Expression outer = symbolic::product(shape, 0, lo), extent = symbolic::product(shape, lo, hi + 1),
+                             inner = symbolic::product(shape, hi + 1, shape.size());
+            std::string to = name_of("Y");
+            if (k > 0) {
+                const int slot = (int) ((runs.size() - 1 - k) & 1);
+                to = "__docc_part[" + std::to_string(slot) + "]";
+                if (runs.size() - 1 - k < 2)   // a later step reuses the slot: its result is never larger
+                    s << "DOCC_ROCM_CHECK(docc_rocm_malloc(&" << to << ", (size_t) (" << symbolic::mul(symbolic::mul(outer, inner), elem) << ")));" << std::endl;
+            }
+            call(outer, extent, inner, from, to);
+            shape.erase(shape.begin() + (long) lo, shape.begin() + (long) hi + 1);
+            from = to;
+        }
+        s << "if (__docc_part[0]) DOCC_ROCM_CHECK(docc_rocm_free(__docc_part[0]));" << std::endl;
+        s << "if (__docc_part[1]) DOCC_ROCM_CHECK(docc_rocm_free(__docc_part[1]));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
     }
 };
 
@@ -795,7 +838,6 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (e->element() != P::Float && e->element() != P::Double) return decline("element type must be Float or Double");
     } else if (auto* r = dynamic_cast<tensor::ReduceNode*>(&node)) {
         if (r->element() != P::Float && r->element() != P::Double) return decline("element type must be Float or Double");
-        if (!r->adjacent_axes()) return decline("the reduced axes must be adjacent (one block)");
     } else if (node.code() == tensor::LibraryNodeType_Broadcast) {
         auto* b = dynamic_cast<tensor::BroadcastNode*>(&node);
         if (!b) return decline("not a Broadcast node object");

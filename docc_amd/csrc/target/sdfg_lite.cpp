@@ -80,6 +80,12 @@ Expression mul(const Expression& a, const Expression& b) {
     return (is_atom(a) ? a : "(" + a + ")") + "*" + (is_atom(b) ? b : "(" + b + ")");
 }
 
+Expression product(const std::vector<Expression>& v, size_t begin, size_t end) {
+    Expression p = "1";
+    for (size_t i = begin; i < end; i++) p = mul(p, v[i]);
+    return p;
+}
+
 } // namespace symbolic
 
 namespace {
@@ -100,11 +106,7 @@ std::vector<Expression> exprs_from_json(const Value& v) {
     return out;
 }
 
-Expression product(const std::vector<Expression>& v, size_t begin, size_t end) {
-    Expression p = "1";
-    for (size_t i = begin; i < end; i++) p = symbolic::mul(p, v[i]);
-    return p;
-}
+Expression product(const std::vector<Expression>& v, size_t begin, size_t end) { return symbolic::product(v, begin, end); }
 
 Expression bytes_of(const Expression& elems, types::PrimitiveType t) {
     return symbolic::mul(elems, symbolic::integer((int64_t) types::primitive_type_size(t)));

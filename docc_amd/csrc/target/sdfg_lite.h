@@ -46,6 +46,8 @@ namespace symbolic {
 Expression mul(const Expression& a, const Expression& b);
 Expression integer(int64_t v);
 bool is_integer(const Expression& e, int64_t* value = nullptr);
+// v[begin] * ... * v[end - 1] ("1" for an empty range)
+Expression product(const std::vector<Expression>& v, size_t begin, size_t end);
 } // namespace symbolic
 
 // Implementation types, following the "<LIB>With[out]Transfers" naming of the

@@ -26,7 +26,7 @@ NotImplementedError (there is no CPU lowering behind it):
     np.abs, np.exp, np.sqrt, np.tanh, scipy.special.erf / expit, relu(x), sigmoid(x),
         np.maximum(x, 0)  (ReLU)
     np.sum / np.max / np.min / np.mean (and the array methods) over one axis or a block of
-        adjacent axes, with keepdims
+        axes, with keepdims
 """
 from __future__ import annotations
 
@@ -382,8 +382,6 @@ class _Lowering(ast.NodeVisitor):
         if any(not isinstance(a, int) or a < -rank or a >= rank for a in axes):
             raise ValueError(f"{self.func.__name__}: axis {axis} is out of bounds for an array of rank {rank}")
         axes = sorted({a % rank for a in axes})
-        if axes != list(range(axes[0], axes[-1] + 1)):
-            self.fail(node, "a reduction over axes that are not adjacent")
         shape = [("1" if d in axes else s) for d, s in enumerate(x.shape) if keepdims or d not in axes]
         out = self.new_array(shape, x.elem, dest)
         self.b.add_reduce_op(op, x.name, out.name, x.shape, axes, keepdims)

@@ -20,7 +20,7 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     elu, leaky_relu, hardsigmoid (F.* and nn.ELU / nn.LeakyReLU / nn.Hardsigmoid)
                                            -> ml::ReLU .. ml::Erf
     F.linear / nn.Linear                   -> GEMM with the weight transposed, bias through Broadcast + Add
-    sum / mean / amax / amin over one dim or a block of adjacent dims (keepdim) -> ml::Sum .. ml::Min
+    sum / mean / amax / amin over any dims (keepdim) -> ml::Sum .. ml::Min
 
 Tensors on a `cuda` device are passed to the generated function as device pointers (no
 transfers, the kernels run on the null stream in order with torch's default stream); CPU tensors
@@ -277,8 +277,6 @@ class _FxLowering:
         rank = len(x.shape)
         dims = list(range(rank)) if dim is None or dim == [] or dim == () else ([dim] if isinstance(dim, int) else list(dim))
         dims = sorted({int(d) % rank for d in dims})
-        if dims != list(range(dims[0], dims[-1] + 1)):
-            self.fail(node, "a reduction over dims that are not adjacent")
         shape = [(1 if d in dims else s) for d, s in enumerate(x.shape) if keepdim or d not in dims]
         out = self.new_tensor(shape, x.dtype, dest)
         self.builder.add_reduce_op(op, x.name, out.name, x.shape, dims, keepdim)

@@ -458,6 +458,63 @@ def test_docc_json_return_copy_and_elementwise_nests_run(tmp_path):
     assert rel_err_max(W, E.astype(np.float64) / 3.0) <= 1e-5
 
 
+def test_reductions_over_axes_that_are_not_adjacent():
+    """Axes in several blocks: the dispatcher reduces block by block through device temporaries. numpy is the pin
+    (a float64 reference; sums in another order than the reference's single loop nest, inside the usual bars)."""
+    @native(target="rocm")
+    def scattered(x):
+        return np.sum(x, axis=(0, 2)), np.max(x, axis=(0, 2, 4)), np.mean(x, axis=(1, 3), keepdims=True), np.min(x, axis=(0, 3))
+
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((6, 5, 7, 4, 9))
+    s, mx, mean, mn = scattered(x)
+    assert s.shape == (5, 4, 9) and mx.shape == (5, 4) and mean.shape == (6, 1, 7, 1, 9) and mn.shape == (5, 7, 9)
+    assert rel_err_max(s, x.sum(axis=(0, 2))) <= 1e-12 and np.array_equal(mx, x.max(axis=(0, 2, 4)))
+    assert rel_err_max(mean, x.mean(axis=(1, 3), keepdims=True)) <= 1e-12 and np.array_equal(mn, x.min(axis=(0, 3)))
+    x32 = x.astype(np.float32)
+    s32, _, mean32, _ = scattered(x32)
+    assert rel_err_max(s32, x32.astype(np.float64).sum(axis=(0, 2))) <= 1e-5
+    assert rel_err_max(mean32, x32.astype(np.float64).mean(axis=(1, 3), keepdims=True)) <= 1e-5
+
+    class M(torch.nn.Module):
+        def forward(self, t):
+            return t.sum(dim=(0, 2)) + t.amax(dim=(0, 2))
+
+    t = torch.randn(3, 8, 5, 16, device="cuda")
+    y = docc_torch.compile_torch(M(), t, target="rocm")(t)
+    ref = t.double().sum(dim=(0, 2)) + t.double().amax(dim=(0, 2))
+    assert rel_err_max(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+
+
+def test_arrays_named_like_the_nodes_connectors(tmp_path):
+    """Containers called A, B, C, X, Y under nodes whose connectors carry the same names, every operand copied by the
+    node itself (offload "node": the connectors are bound to the caller's own arrays)."""
+    import ctypes
+
+    from docc_amd import runtime
+    from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFGBuilder
+
+    F64p = Pointer(Scalar(PrimitiveType.Double))
+    b = StructuredSDFGBuilder("clash")
+    for name in ("X", "Y", "A", "B"):
+        b.add_container(name, F64p, True)
+    b.add_elementwise_op("add", "Y", "X", "A", [64])        # connectors A <- Y, B <- X, C -> A
+    b.add_elementwise_unary_op("relu", "A", "X", [64])      # connectors X <- A, Y -> X
+    b.add_elementwise_op("mul", "X", "A", "B", [64])        # connectors A <- X, B <- A, C -> B
+    s = b.move()
+    s.schedule("rocm", options={"offload": "node", "fuse_elementwise": False})
+    fn = ctypes.CDLL(s._compile(str(tmp_path))).clash
+    fn.restype = None
+    rng = np.random.default_rng(4)
+    X, Y = rng.standard_normal(64), rng.standard_normal(64)
+    x0 = X.copy()
+    A, B = np.full(64, np.nan), np.full(64, np.nan)
+    ptr = lambda a: a.ctypes.data_as(ctypes.c_void_p)
+    fn(ptr(X), ptr(Y), ptr(A), ptr(B))
+    assert runtime.take_failure()[0] == 0
+    assert np.array_equal(A, Y + x0) and np.array_equal(X, np.maximum(A, 0)) and np.array_equal(B, X * A)
+
+
 def test_native_reductions_and_layer_statistics():
     """np.sum / max / min / mean over rows, columns and blocks of axes; the softmax pieces as values of their own."""
     @native(target="rocm")

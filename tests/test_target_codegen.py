@@ -741,13 +741,20 @@ def test_reduce_nodes_dispatch_and_decline(tmp_path):
     assert "docc_rocm_reduce(nullptr, 0 /* ml::Sum */, 32, _n*64, 3136, 1, X, Y)" in flat
     assert "docc_rocm_reduce(nullptr, 1 /* ml::Max */, 32, _n, 64, 3136, X, Y)" in flat
     assert "(size_t) (_n*64*4)" in flat.replace("(_n*64)*4", "_n*64*4")                      # Y of the sum: the kept extents
-    # what the kernels do not cover is declined by the mapper, with the reason
+    # axes in several blocks are reduced block by block
     b = StructuredSDFGBuilder("scattered")
     for n in ("X", "Y"):
         b.add_container(n, F64, True)
-    b.add_reduce_op("mean", "X", "Y", [4, 5, 6], [0, 2])
-    with pytest.raises(InvalidSDFGException, match="adjacent"):
-        b.move().schedule("rocm")
+    b.add_container("_n", I64, True)
+    b.add_reduce_op("mean", "X", "Y", [4, 5, "_n", 6, 7], [0, 2, 3])
+    s = b.move()
+    s.schedule("rocm", options={"offload": "none"})
+    flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "scattered")[0])
+    # axes in two blocks: the inner block (axes 2, 3) first into a device temporary, then axis 0 of what is left
+    assert "docc_rocm_malloc(&__docc_part[0], (size_t) (1120))" in flat                      # [4, 5, 7] doubles
+    assert "docc_rocm_reduce(nullptr, 3 /* ml::Mean */, 64, 20, _n*6, 7, X, __docc_part[0])" in flat
+    assert "docc_rocm_reduce(nullptr, 3 /* ml::Mean */, 64, 1, 4, 35, __docc_part[0], Y)" in flat
+    assert "docc_rocm_free(__docc_part[0])" in flat
     # std is the chain of nodes the reference's StdNode expands to
     b = StructuredSDFGBuilder("s")
     for n in ("X", "Y"):
@@ -844,3 +851,36 @@ int main() {
     assert r.returncode == 0, r.stderr[-3000:]
     r = subprocess.run([str(exe)], capture_output=True, text=True)
     assert r.returncode == 0 and r.stdout.strip() == "ok", (r.returncode, r.stdout, r.stderr)
+
+
+def test_containers_named_like_connectors_do_not_shadow_each_other(tmp_path):
+    """The tensor nodes' connectors are X, Y, A, B, C - names a user's arrays may carry too. A connector's local would
+    hide such a container (`double *X = X;` reads the local itself), so the containers are captured under other names
+    first and written back outside the connectors' scope."""
+    import subprocess
+
+    b = StructuredSDFGBuilder("clash")
+    for n in ("X", "Y", "A"):
+        b.add_container(n, F64, True)
+    b.add_elementwise_op("add", "Y", "X", "A", [8])       # connector A <- Y, B <- X, C -> A
+    b.add_elementwise_unary_op("relu", "A", "X", [8])     # connector X <- A, Y -> X
+    s = b.move()
+    s.schedule("rocm", options={"offload": "none", "fuse_elementwise": False})
+    src_path = s.generate(str(tmp_path))["source"]
+    flat = re.sub(r"\s+", " ", Path(src_path).read_text())
+    assert "double *__docc_bound_0 = Y; double *__docc_bound_1 = X; double *__docc_bound_2 = A; { double *A = __docc_bound_0; double *B = __docc_bound_1; double *C = __docc_bound_2;" in flat
+    assert "__docc_bound_2 = C; } A = __docc_bound_2;" in flat
+    assert "double *X = X;" not in flat and "double *A = A;" not in flat
+    # nodes whose connectors meet no container keep the reference's plain text
+    b = StructuredSDFGBuilder("plain")
+    for n in ("P", "Q"):
+        b.add_container(n, F64, True)
+    b.add_elementwise_unary_op("relu", "P", "Q", [8])
+    s2 = b.move()
+    s2.schedule("rocm", options={"offload": "none"})
+    flat2 = re.sub(r"\s+", " ", Path(s2.generate(str(tmp_path / "plain"))["source"]).read_text())
+    assert "{ double *X = P; double *Y = Q;" in flat2 and "__docc_bound" not in flat2
+    root = Path(__file__).resolve().parent.parent
+    r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Werror=uninitialized", "-I", str(root / "include"), "-I", str(tmp_path), src_path],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
