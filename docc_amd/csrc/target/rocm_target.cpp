@@ -943,6 +943,106 @@ void make_fused(StructuredSDFG& sdfg, size_t i) {
 
 } // namespace
 
+bool RocmSoftmaxPatternPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
+    StructuredSDFG& sdfg = builder.subject();
+    auto& blocks = sdfg.blocks();
+    bool applied = false;
+    // the single block that writes `name`, or -1
+    auto writer_of = [&](const std::string& name) -> long {
+        const Uses u = uses_of(sdfg, name);
+        return u.writers.size() == 1 ? (long) u.writers[0] : -1;
+    };
+    auto private_value = [&](const std::string& name, std::vector<size_t> readers) {
+        const Container& c = sdfg.container(name);
+        if (c.is_argument || !c.transient || name == sdfg.return_container()) return false;
+        Uses u = uses_of(sdfg, name);
+        std::sort(readers.begin(), readers.end());
+        std::sort(u.readers.begin(), u.readers.end());
+        return u.writers.size() == 1 && u.readers == readers;
+    };
+    auto elementwise = [&](long i, const char* code, bool binary) -> tensor::ElementWiseNode* {
+        if (i < 0) return nullptr;
+        auto* e = dynamic_cast<tensor::ElementWiseNode*>(blocks[(size_t) i].node.get());
+        return e && e->code() == code && e->is_binary() == binary && e->implementation_type() == ImplementationType_NONE ? e : nullptr;
+    };
+    auto data_of = [&](size_t i, const char* connector) -> std::string {
+        const ConnectorBinding* b = blocks[i].input(connector);
+        return b && !b->is_constant ? b->data : std::string();
+    };
+    // Broadcast of a keepdims reduction `code` of `source` over `axes`: fills the two block indices
+    auto reduced_and_repeated = [&](const std::string& repeated, const char* code, const std::vector<Expression>& shape, long* bc_at, long* red_at,
+                                    std::vector<int64_t>* axes, std::string* source) {
+        *bc_at = repeated.empty() ? -1 : writer_of(repeated);
+        if (*bc_at < 0) return false;
+        auto* bc = dynamic_cast<tensor::BroadcastNode*>(blocks[(size_t) *bc_at].node.get());
+        if (!bc || bc->implementation_type() != ImplementationType_NONE || bc->output_shape() != shape) return false;
+        const std::string small = data_of((size_t) *bc_at, "X");
+        *red_at = small.empty() ? -1 : writer_of(small);
+        if (*red_at < 0) return false;
+        auto* red = dynamic_cast<tensor::ReduceNode*>(blocks[(size_t) *red_at].node.get());
+        if (!red || red->code() != code || red->implementation_type() != ImplementationType_NONE || !red->keepdims() || red->shape() != shape) return false;
+        // the broadcast repeats exactly the reduced axes
+        const auto ax = red->sorted_axes();
+        if (bc->input_shape().size() != shape.size()) return false;
+        for (size_t d = 0; d < shape.size(); d++) {
+            const bool reduced = std::find(ax.begin(), ax.end(), (int64_t) d) != ax.end();
+            if (bc->input_shape()[d] != (reduced ? Expression("1") : shape[d])) return false;
+        }
+        *axes = ax;
+        *source = data_of((size_t) *red_at, "X");
+        return !source->empty();
+    };
+    bool changed = true;
+    while (changed) {
+        changed = false;
+        for (size_t at = 0; at < blocks.size() && !changed; at++) {
+            auto* div = elementwise((long) at, "ml::Div", true);
+            if (!div) continue;
+            const std::vector<Expression> shape = div->shape();
+            const std::string e_name = data_of(at, "A"), den = data_of(at, "B");
+            long bc2, sum_at, bc1, max_at;
+            std::vector<int64_t> axes_sum, axes_max;
+            std::string sum_src, max_src;
+            if (e_name.empty() || !reduced_and_repeated(den, "ml::Sum", shape, &bc2, &sum_at, &axes_sum, &sum_src) || sum_src != e_name) continue;
+            const long exp_at = writer_of(e_name);
+            auto* ex = elementwise(exp_at, "ml::Exp", false);
+            if (!ex || ex->shape() != shape || ex->element() != div->element()) continue;
+            const std::string d_name = data_of((size_t) exp_at, "X");
+            const long sub_at = d_name.empty() ? -1 : writer_of(d_name);
+            auto* sub = elementwise(sub_at, "ml::Sub", true);
+            if (!sub || sub->shape() != shape) continue;
+            const std::string x_name = data_of((size_t) sub_at, "A"), shift = data_of((size_t) sub_at, "B");
+            if (x_name.empty() || !reduced_and_repeated(shift, "ml::Max", shape, &bc1, &max_at, &axes_max, &max_src)) continue;
+            if (max_src != x_name || axes_max != axes_sum) continue;
+            // program order, and every value in between private to the pattern
+            const size_t i_max = (size_t) max_at, i_bc1 = (size_t) bc1, i_sub = (size_t) sub_at, i_exp = (size_t) exp_at, i_sum = (size_t) sum_at, i_bc2 = (size_t) bc2;
+            if (!(i_max < i_bc1 && i_bc1 < i_sub && i_sub < i_exp && i_exp < i_sum && i_sum < i_bc2 && i_bc2 < at)) continue;
+            const std::string m_name = blocks[i_max].outputs[0].data, s_name = blocks[i_sum].outputs[0].data, y_name = blocks[at].outputs[0].data;
+            if (!private_value(m_name, {i_bc1}) || !private_value(shift, {i_sub}) || !private_value(d_name, {i_exp}) ||
+                !private_value(e_name, {i_sum, at}) || !private_value(s_name, {i_bc2}) || !private_value(den, {at}))
+                continue;
+            // X as the Max saw it must be what the Sub sees, and the result must not be looked at before the Div stood
+            if (!unwritten_between(sdfg, x_name, i_max, at) || (y_name != x_name && !untouched_between(sdfg, y_name, i_max, at))) continue;
+            if (y_name == x_name) continue;   // in place: the softmax kernels allow it, the pattern's readers of X in between do not
+            auto node = std::make_unique<tensor::SoftmaxNode>(ImplementationType_NONE, shape, axes_sum, div->element());
+            node->set_element_id(div->element_id());
+            Block& last = blocks[at];
+            last.node = std::move(node);
+            last.inputs.clear();
+            ConnectorBinding in;
+            in.connector = "X";
+            in.data = x_name;
+            last.inputs.push_back(in);
+            last.outputs[0].connector = "Y";
+            // the other six blocks go, highest index first, and their values with them
+            for (size_t i : {i_bc2, i_sum, i_exp, i_sub, i_bc1, i_max}) blocks.erase(blocks.begin() + (long) i);
+            for (auto& name : {m_name, shift, d_name, e_name, s_name, den}) sdfg.remove_container(name);
+            changed = applied = true;
+        }
+    }
+    return applied;
+}
+
 bool RocmElementwiseFusionPass::run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager&) {
     StructuredSDFG& sdfg = builder.subject();
     auto& blocks = sdfg.blocks();
@@ -1421,6 +1521,10 @@ void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::A
     if (options.offload != "function" && options.offload != "node" && options.offload != "none")
         throw std::invalid_argument("rocm: option offload must be 'function', 'node' or 'none'");
     const std::string impl = options.offload == "node" ? ImplementationType_ROCMWithTransfers : ImplementationType_ROCMWithoutTransfers;
+    if (options.match_softmax) {
+        RocmSoftmaxPatternPass pattern;
+        pattern.run_pass(builder, analysis_manager);
+    }
     auto mapper = std::make_shared<RocmLibNodeMapper>(impl);
     for (auto& blk : builder.subject().blocks()) {
         if (!is_math_node(*blk.node) || is_rocm_impl(blk.node->implementation_type())) continue;

@@ -83,6 +83,16 @@ public:
     bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
 };
 
+// Recognises softmax written out in its pieces - the form numpy code takes, and what the reference's SoftmaxNode
+// expands to (softmax_node.cpp:142-252): m = Max(X, axes, keepdims); e = Exp(X - broadcast(m)); Y = e / broadcast(Sum(e,
+// axes, keepdims)) - and replaces the seven nodes by one ml::Softmax when every value in between is a transient that
+// nothing else looks at. Runs before the mapping (on nodes without an implementation type).
+class RocmSoftmaxPatternPass {
+public:
+    std::string name() { return "RocmSoftmaxPattern"; }
+    bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
+};
+
 struct ScheduleOptions {
     // "function": nodes run WithoutTransfers between hoisted, minimised transfers (default)
     // "node":     every node copies its operands itself (ROCMWithTransfers)
@@ -92,6 +102,8 @@ struct ScheduleOptions {
     bool require_all_mapped = true;
     // run RocmElementwiseFusionPass after the mapping
     bool fuse_elementwise = true;
+    // run RocmSoftmaxPatternPass before the mapping
+    bool match_softmax = true;
 };
 
 // The scheduling entry of the target: mapping pass (+ offloading passes).

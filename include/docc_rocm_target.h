@@ -53,8 +53,9 @@ char* docc_rocm_target_export(const char* sdfg_json);
 
 /* Runs the rocm scheduling passes (node mapping, offloading, transfer minimisation) and
  * returns the scheduled SDFG. `options_json` may be NULL or an object with
- * "offload": "function" | "node" | "none", "require_all_mapped": bool and "fuse": bool (fold
- * Broadcast and unary elementwise nodes into their neighbours, default true).
+ * "offload": "function" | "node" | "none", "require_all_mapped": bool, "fuse": bool (fold
+ * Broadcast and unary elementwise nodes into their neighbours, default true) and "match_softmax": bool
+ * (replace softmax written out as Max, Sub, Exp, Sum, Div nodes by one ml::Softmax, default true).
  * Counterpart of PyStructuredSDFG::schedule (reference py_structured_sdfg.cpp:320-347). */
 char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, const char* options_json);
 

@@ -502,7 +502,7 @@ def test_arrays_named_like_the_nodes_connectors(tmp_path):
     b.add_elementwise_unary_op("relu", "A", "X", [64])      # connectors X <- A, Y -> X
     b.add_elementwise_op("mul", "X", "A", "B", [64])        # connectors A <- X, B <- A, C -> B
     s = b.move()
-    s.schedule("rocm", options={"offload": "node", "fuse_elementwise": False})
+    s.schedule("rocm", options={"offload": "node", "fuse": False})
     fn = ctypes.CDLL(s._compile(str(tmp_path))).clash
     fn.restype = None
     rng = np.random.default_rng(4)
@@ -513,6 +513,26 @@ def test_arrays_named_like_the_nodes_connectors(tmp_path):
     fn(ptr(X), ptr(Y), ptr(A), ptr(B))
     assert runtime.take_failure()[0] == 0
     assert np.array_equal(A, Y + x0) and np.array_equal(X, np.maximum(A, 0)) and np.array_equal(B, X * A)
+
+
+def test_softmax_written_in_pieces_runs_as_the_softmax_kernel(tmp_path):
+    """Seven nodes (Max, Broadcast, Sub, Exp, Sum, Broadcast, Div) are matched to one ml::Softmax before the mapping."""
+    import ctypes
+
+    from docc_amd import runtime
+    from test_target_codegen import softmax_in_pieces
+
+    s = softmax_in_pieces("pieces", [8, 16, 300], [-1])
+    s.schedule("rocm")
+    assert s.loop_report()["ml::Softmax::ROCMWithoutTransfers"] == 1
+    fn = ctypes.CDLL(s._compile(str(tmp_path))).pieces
+    fn.restype = None
+    rng = np.random.default_rng(8)
+    X = (rng.standard_normal((8, 16, 300)) * 8).astype(np.float32)
+    Y = np.full_like(X, np.nan)
+    fn(X.ctypes.data_as(ctypes.c_void_p), Y.ctypes.data_as(ctypes.c_void_p))
+    assert runtime.take_failure()[0] == 0
+    assert rel_err_max(Y, oracle.softmax(X.reshape(-1, 300)).reshape(X.shape)) <= 1e-5
 
 
 def test_native_reductions_and_layer_statistics():

@@ -865,7 +865,7 @@ def test_containers_named_like_connectors_do_not_shadow_each_other(tmp_path):
     b.add_elementwise_op("add", "Y", "X", "A", [8])       # connector A <- Y, B <- X, C -> A
     b.add_elementwise_unary_op("relu", "A", "X", [8])     # connector X <- A, Y -> X
     s = b.move()
-    s.schedule("rocm", options={"offload": "none", "fuse_elementwise": False})
+    s.schedule("rocm", options={"offload": "none", "fuse": False})
     src_path = s.generate(str(tmp_path))["source"]
     flat = re.sub(r"\s+", " ", Path(src_path).read_text())
     assert "double *__docc_bound_0 = Y; double *__docc_bound_1 = X; double *__docc_bound_2 = A; { double *A = __docc_bound_0; double *B = __docc_bound_1; double *C = __docc_bound_2;" in flat
@@ -884,3 +884,51 @@ def test_containers_named_like_connectors_do_not_shadow_each_other(tmp_path):
     r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-Wall", "-Werror=uninitialized", "-I", str(root / "include"), "-I", str(tmp_path), src_path],
                        capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
+
+
+def softmax_in_pieces(name, shape, axes, extra_reader=False):
+    """m = Max(X); e = Exp(X - broadcast(m)); Y = e / broadcast(Sum(e)) as seven nodes, the way a builder client or an
+    imported program spells softmax (the nodes the reference's SoftmaxNode::expand chains, softmax_node.cpp:142-252)."""
+    b = StructuredSDFGBuilder(name)
+    for n in ("X", "Y") + (("Z",) if extra_reader else ()):
+        b.add_container(n, F32, True)
+    kept = [1 if d in [a % len(shape) for a in axes] else s for d, s in enumerate(shape)]
+    count = 1
+    for s_ in shape:
+        count *= s_
+    for n in ("m", "mb", "d", "e", "s", "sb"):
+        b.add_container(n, F32, False, transient_bytes=4 * count)
+    b.add_reduce_op("max", "X", "m", shape, axes, True)
+    b.add_broadcast("m", "mb", kept, shape)
+    b.add_elementwise_op("sub", "X", "mb", "d", shape)
+    b.add_elementwise_unary_op("exp", "d", "e", shape)
+    b.add_reduce_op("sum", "e", "s", shape, axes, True)
+    b.add_broadcast("s", "sb", kept, shape)
+    b.add_elementwise_op("div", "e", "sb", "Y", shape)
+    if extra_reader:
+        b.add_elementwise_unary_op("relu", "e", "Z", shape)       # the exponentials are looked at from outside
+    return b.move()
+
+
+def test_softmax_written_in_pieces_becomes_one_node(tmp_path):
+    s = softmax_in_pieces("pieces", [8, 16, 32], [-1])
+    assert [n["code"] for n in s.library_nodes()] == ["ml::Max", "ml::Broadcast", "ml::Sub", "ml::Exp", "ml::Sum", "ml::Broadcast", "ml::Div"]
+    s.schedule("rocm")
+    nodes = [n for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert [n["code"] for n in nodes] == ["ml::Softmax"] and nodes[0]["axes"] == [2] and nodes[0]["shape"] == ["8", "16", "32"]
+    assert set(s.containers) >= {"X", "Y"} and not {"m", "mb", "d", "e", "s", "sb"} & set(s.containers)
+    r = s.loop_report()
+    assert r["H2D"] == 1 and r["D2H"] == 1
+    assert "docc_rocm_softmax_f32(nullptr, " in source_of(s, tmp_path)[0]
+    # a block of axes in the middle
+    s = softmax_in_pieces("middle", [4, 5, 6, 7], [1, 2])
+    s.schedule("rocm")
+    (node,) = [n for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert node["code"] == "ml::Softmax" and node["axes"] == [1, 2]
+    # not when a value in between is used elsewhere, and not when switched off
+    s = softmax_in_pieces("shared", [8, 32], [1], extra_reader=True)
+    s.schedule("rocm")
+    assert "ml::Softmax" not in [n["code"] for n in s.library_nodes()]
+    s = softmax_in_pieces("off", [8, 32], [1])
+    s.schedule("rocm", options={"match_softmax": False})
+    assert "ml::Softmax" not in [n["code"] for n in s.library_nodes()]
