@@ -298,8 +298,8 @@ int docc_rocm_cast(docc_rocm_stream_t stream, int src_type, int dst_type, int64_
  * attaches to Y. Max / Min use fmax / fmin like the reference (a NaN is ignored unless the
  * whole extent is NaN); an empty extent gives the identity (0, -inf, +inf). A reduction with
  * inner > 1 and few output elements is sliced along the reduced extent; the slices' partial
- * results pass through an 8 MiB array in device memory that belongs to the kernels' code object
- * and is shared by every such call on the device: do not overlap them on different streams. */
+ * results pass through 8 MiB of device memory that the library keeps per stream (see
+ * docc_rocm_softmax): calls on different streams do not share it. */
 #define DOCC_ROCM_REDUCE_SUM 0
 #define DOCC_ROCM_REDUCE_MAX 1
 #define DOCC_ROCM_REDUCE_MIN 2
