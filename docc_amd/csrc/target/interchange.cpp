@@ -414,6 +414,14 @@ struct Import {
         const Value& type = edge.at("base_type");
         const std::string tkind = type.at("type").as_string();
         const Array& subset = edge.at("subset").as_array();
+        if (loops.empty()) {
+            // a statement outside any loop touches one element of a buffer: only the first one has a form here
+            // (the caller allows it as the place a scalar is stored to)
+            for (auto& sub : subset)
+                if (strip(sub.as_expression()) != "0") return false;
+            walk->scalar = true;
+            return true;
+        }
         std::vector<Term> strides(loops.size());
         std::vector<bool> seen(loops.size(), false);
         auto loop_of = [&](const std::string& name) {
@@ -558,6 +566,8 @@ struct Import {
                 refuse(block, "operand '" + (other.contains("data") ? other.at("data").as_expression() : std::string("?")) +
                                   "' is not a dense tensor indexed by the loop variables");
             if (into) {
+                if (w.scalar && other.at("type").as_string() == "access_node" && container(other.at("data").as_string()).at("type").as_string() != "scalar")
+                    refuse(block, "one element of '" + other.at("data").as_string() + "' read outside a loop");
                 in[e.at("dst_conn").as_string()] = w;
             } else {
                 if (out_type) refuse(block, "an operation with two results");

@@ -457,6 +457,19 @@ def test_docc_json_return_copy_and_elementwise_nests_run(tmp_path):
     assert rel_err_max(E, ref) <= 1e-5 and np.array_equal(T, E.T)
     assert rel_err_max(W, E.astype(np.float64) / 3.0) <= 1e-5
 
+    # a copy that permutes the axes, a scalar on the left of a difference, a scalar stored into the return buffer
+    from test_interchange import permuted_copy_and_scalar_program
+    s = StructuredSDFG.parse(json.dumps(permuted_copy_and_scalar_program()))
+    s.schedule("rocm")
+    fn = ctypes.CDLL(s._compile(str(tmp_path / "perm"))).perm_sdfg
+    fn.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_double, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]
+    fn.restype = None
+    Xp = rng.standard_normal((11, 7, 5))
+    Tp, Sp, ret = np.full((5, 11, 7), np.nan), np.full((11, 7, 5), np.nan), np.full(1, np.nan)
+    fn(Xp.ctypes.data, Tp.ctypes.data, Sp.ctypes.data, 2.75, 11, 7, ret.ctypes.data)
+    assert runtime.take_failure() == (0, "")
+    assert np.array_equal(Tp, Xp.transpose(2, 0, 1)) and np.array_equal(Sp, 2.0 - Xp) and ret[0] == 2.75
+
 
 def test_reductions_over_axes_that_are_not_adjacent():
     """Axes in several blocks: the dispatcher reduces block by block through device temporaries. numpy is the pin

@@ -403,3 +403,47 @@ def test_loop_nests_outside_the_elementwise_forms_are_refused():
     bad["root"]["children"][0]["root"]["children"].append(copy.deepcopy(inner_block(nest(1))))
     bad["root"]["children"][0]["root"]["transitions"].append(copy.deepcopy(bad["root"]["children"][0]["root"]["transitions"][0]))
     refused(bad, "more than one statement in a loop body")
+
+
+def permuted_copy_and_scalar_program():
+    """T[k][i][j] = X[i][j][k] over a [_s0, _s1, 5] array (Tensor-typed memlets, the loop order of the source), a
+    difference with the scalar on the left (S = 2 - X, linearised pointers), and a scalar argument stored into the
+    one-element return buffer (the scalar form of the front end's return copy, ast_parser.py:1150-1157)."""
+    ids = Ids()
+    containers = {n: pointer(DOUBLE) for n in ("X", "T", "S", "_docc_ret_0")}
+    for n in ("_s0", "_s1", "_i0", "_i1", "_i2"):
+        containers[n] = scalar(INT64)
+    containers["v"] = scalar(DOUBLE)
+    tx = tensor(DOUBLE, ["_s0", "_s1", "5"])
+    tt = tensor(DOUBLE, ["5", "_s0", "_s1"])
+    P = pointer(DOUBLE)
+    loops = [("_i0", "_s0"), ("_i1", "_s1"), ("_i2", "5")]
+    lin = ["_i2 + 5*_i1 + 5*_i0*_s1"]
+    children = [
+        docc_nest(ids, "for", loops, ASSIGN, [("_in", "X", ["_i0", "_i1", "_i2"], tx)], ("_out", "T", ["_i2", "_i0", "_i1"], tt)),
+        docc_nest(ids, "map", loops, {"type": "tasklet", "code": 3, "inputs": ["_in1", "_in2"], "output": "_out"},
+                  [("_in1", ("2.0", DOUBLE), [], scalar(DOUBLE)), ("_in2", "X", lin, P)], ("_out", "S", lin, P)),
+        docc_nest(ids, "for", [], ASSIGN, [("_in", "v", [], scalar(DOUBLE))], ("_out", "_docc_ret_0", ["0"], P)),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    return docc_sdfg("perm_sdfg", containers, ["X", "T", "S", "v", "_s0", "_s1", "_docc_ret_0"], children, ids)
+
+
+def test_permuted_copies_scalar_operands_and_scalar_stores_import():
+    s = StructuredSDFG.from_docc_json(json.dumps(permuted_copy_and_scalar_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["ml::Transpose", "ml::Sub", "ml::Fill"]
+    # output axis a of the copy is the input axis that runs over the same loop: T's axes (k, i, j) are X's axes (2, 0, 1)
+    assert nodes[0]["shape"] == ["_s0", "_s1", "5"] and nodes[0]["perm"] == [2, 0, 1]
+    blocks = [c["dataflow"] for c in s._data["root"]["children"][:3]]
+    assert blocks[1]["inputs"] == [{"constant": "2.0", "type": "Double", "connector": "A"}, {"data": "X", "connector": "B"}]
+    assert nodes[2]["shape"] == ["1"] and blocks[2]["inputs"] == [{"data": "v", "connector": "X"}]
+    s.schedule("rocm")
+    # a tensor type that starts past its container's first element is not matched
+    bad = permuted_copy_and_scalar_program()
+    blk = bad["root"]["children"][0]
+    while blk["type"] != "block":
+        blk = blk["root"]["children"][0]
+    blk["dataflow"]["edges"][0]["base_type"]["offset"] = "3"
+    with pytest.raises(InvalidSDFGException, match="operand 'X' is not a dense tensor"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
