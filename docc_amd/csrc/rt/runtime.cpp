@@ -9,9 +9,11 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <condition_variable>
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -258,6 +260,150 @@ int compute_units() {
 
 using namespace docc::rt::rocm;
 
+// ---- uploads from pageable memory ---------------------------------------------------------------------------
+// hipMemcpyAsync from memory the driver has not pinned goes through the driver's own staging at about 30 GB/s on
+// these machines; from pinned memory the same bytes move at 57 GB/s. The caller's arrays (numpy's) are pageable, so a
+// large upload is staged here instead: helper threads copy the source into a ring of pinned chunks while the chunks
+// already filled travel over PCIe. The call returns when the last chunk has been handed to the stream, i.e. after the
+// source has been read completely (what hipMemcpyAsync guarantees for pageable memory as well).
+// DOCC_ROCM_H2D_THREADS=<n> sets the number of copying threads (default 4; 0 switches the staging off).
+namespace {
+
+constexpr size_t kStageMin = size_t(16) << 20;     // smaller uploads go straight to the driver (no gain measured below)
+constexpr size_t kStageChunk = size_t(8) << 20;
+constexpr int kStageBuffers = 4;
+
+std::mutex g_pinned_mutex;
+std::map<uintptr_t, size_t> g_pinned;   // blocks from docc_rocm_host_malloc: start -> bytes
+
+void note_pinned(void* p, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    g_pinned[(uintptr_t) p] = bytes;
+}
+
+void forget_pinned(void* p) {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    g_pinned.erase((uintptr_t) p);
+}
+
+bool is_pinned(const void* p, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_pinned_mutex);
+    auto it = g_pinned.upper_bound((uintptr_t) p);
+    if (it == g_pinned.begin()) return false;
+    --it;
+    return (uintptr_t) p + bytes <= it->first + it->second;
+}
+
+// A fixed pool of threads that copy slices of one chunk; never torn down (the threads sleep on a condition variable
+// until the process ends).
+class CopyPool {
+public:
+    explicit CopyPool(int threads) {
+        for (int i = 0; i < threads; i++) std::thread([this] { work(); }).detach();
+    }
+    // copies `bytes` from src to dst with every thread of the pool and the caller
+    void copy(char* dst, const char* src, size_t bytes, int parts) {
+        const size_t slice = ((bytes + (size_t) parts - 1) / (size_t) parts + 4095) & ~size_t(4095);
+        size_t first = slice < bytes ? slice : bytes;
+        {
+            std::lock_guard<std::mutex> lock(mutex_);
+            for (size_t off = first; off < bytes; off += slice) {
+                jobs_.push_back({dst + off, src + off, off + slice <= bytes ? slice : bytes - off});
+                pending_++;
+            }
+        }
+        wake_.notify_all();
+        std::memcpy(dst, src, first);
+        std::unique_lock<std::mutex> lock(mutex_);
+        done_.wait(lock, [this] { return pending_ == 0; });
+    }
+
+private:
+    struct Job {
+        char* dst;
+        const char* src;
+        size_t bytes;
+    };
+    void work() {
+        for (;;) {
+            Job job;
+            {
+                std::unique_lock<std::mutex> lock(mutex_);
+                wake_.wait(lock, [this] { return !jobs_.empty(); });
+                job = jobs_.back();
+                jobs_.pop_back();
+            }
+            std::memcpy(job.dst, job.src, job.bytes);
+            {
+                std::lock_guard<std::mutex> lock(mutex_);
+                pending_--;
+            }
+            done_.notify_all();
+        }
+    }
+    std::mutex mutex_;
+    std::condition_variable wake_, done_;
+    std::vector<Job> jobs_;
+    size_t pending_ = 0;
+};
+
+struct Stager {
+    std::mutex mutex;              // one staged upload at a time
+    bool tried = false, ready = false;
+    int threads = 0;
+    char* buffer[kStageBuffers] = {};
+    hipEvent_t sent[kStageBuffers] = {};
+    bool in_flight[kStageBuffers] = {};
+    CopyPool* pool = nullptr;
+};
+Stager g_stager;
+
+// 0: done, 1: not staged (the caller falls back to the plain copy), other: error
+int staged_h2d(void* dst_dev, const void* src_host, size_t bytes, hipStream_t stream) {
+    Stager& st = g_stager;
+    std::lock_guard<std::mutex> lock(st.mutex);
+    if (!st.tried) {
+        st.tried = true;
+        int threads = 4;
+        if (const char* e = std::getenv("DOCC_ROCM_H2D_THREADS")) threads = std::atoi(e);
+        if (threads > 64) threads = 64;
+        if (threads >= 1) {
+            bool ok = true;
+            for (int i = 0; i < kStageBuffers && ok; i++)
+                ok = hipHostMalloc((void**) &st.buffer[i], kStageChunk, hipHostMallocDefault) == hipSuccess &&
+                     hipEventCreateWithFlags(&st.sent[i], hipEventDisableTiming) == hipSuccess;
+            if (ok) {
+                st.threads = threads;
+                st.pool = new CopyPool(threads - 1);
+                st.ready = true;
+            } else {
+                (void) hipGetLastError();
+            }
+        }
+    }
+    if (!st.ready) return 1;
+    const char* src = (const char*) src_host;
+    char* dst = (char*) dst_dev;
+    int slot = 0;
+    for (size_t off = 0; off < bytes; off += kStageChunk, slot = (slot + 1) % kStageBuffers) {
+        const size_t n = bytes - off < kStageChunk ? bytes - off : kStageChunk;
+        if (st.in_flight[slot]) {
+            int rc = check(hipEventSynchronize(st.sent[slot]), "hipEventSynchronize(H2D staging)");
+            if (rc) return rc;
+            st.in_flight[slot] = false;
+        }
+        st.pool->copy(st.buffer[slot], src + off, n, st.threads);
+        int rc = check(hipMemcpyAsync(dst + off, st.buffer[slot], n, hipMemcpyHostToDevice, stream), "hipMemcpyAsync(H2D, staged)");
+        if (rc) return rc;
+        rc = check(hipEventRecord(st.sent[slot], stream), "hipEventRecord(H2D staging)");
+        if (rc) return rc;
+        st.in_flight[slot] = true;
+    }
+    return 0;
+}
+
+} // namespace
+
 extern "C" {
 
 int docc_rocm_device_count(void) {
@@ -420,16 +566,23 @@ int docc_rocm_host_malloc(void** host_ptr, size_t bytes) {
     if (!host_ptr) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "host_malloc: null argument");
     *host_ptr = nullptr;
     if (bytes == 0) return 0;
-    return check(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault), "hipHostMalloc");
+    const int rc = check(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault), "hipHostMalloc");
+    if (rc == 0) note_pinned(*host_ptr, bytes);
+    return rc;
 }
 
 int docc_rocm_host_free(void* host_ptr) {
     if (!host_ptr) return 0;
+    forget_pinned(host_ptr);
     return check(hipHostFree(host_ptr), "hipHostFree");
 }
 
 int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes, docc_rocm_stream_t stream) {
     if (bytes == 0) return 0;
+    if (bytes >= kStageMin && !is_pinned(src_host, bytes)) {
+        const int rc = staged_h2d(dst_dev, src_host, bytes, (hipStream_t) stream);
+        if (rc != 1) return rc;     // 1: staging is switched off or could not be set up
+    }
     return check(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t) stream), "hipMemcpyAsync(H2D)");
 }
 

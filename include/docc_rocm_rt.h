@@ -86,7 +86,11 @@ int docc_rocm_host_free(void* host_ptr);
 
 /* Copies on a stream. Replace the blocking cudaMemcpy H2D/D2H of the CUDA
  * offloading node (reference cuda_data_offloading_node.cpp:153-166); the
- * caller orders them with docc_rocm_stream_sync. */
+ * caller orders them with docc_rocm_stream_sync. An upload of 16 MiB or more
+ * from memory that docc_rocm_host_malloc did not return is staged through
+ * pinned chunks of the runtime (helper threads, DOCC_ROCM_H2D_THREADS): the
+ * source has been read when the call returns, as with hipMemcpyAsync from
+ * pageable memory. */
 int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes, docc_rocm_stream_t stream);
 int docc_rocm_memcpy_d2h_async(void* dst_host, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);
 int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);

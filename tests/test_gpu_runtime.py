@@ -97,3 +97,42 @@ def test_result_arrays_are_pinned_and_reused(rt):
     del b, c
     gc.collect()
     rt.pinned_trim()
+
+
+def test_large_uploads_from_pageable_memory_are_staged_through_pinned_chunks(rt):
+    """Uploads of 16 MiB and more from memory the runtime did not pin go through its ring of pinned 8 MiB chunks (helper
+    threads fill them while earlier chunks travel); sizes that are no multiple of the chunk, sources the call may not
+    keep, two uploads in a row, another stream, and pinned sources (straight to the driver) all arrive intact."""
+    import ctypes
+    rng = np.random.default_rng(5)
+    for nbytes in (4 << 20, (33 << 20) + 13, (16 << 20) - 1, (16 << 20), (24 << 20) + 1):
+        x = rng.integers(0, 256, nbytes, dtype=np.uint8)
+        expected = x.copy()
+        p = rt.malloc(nbytes)
+        rt.memcpy_h2d(p, x.ctypes.data, nbytes)
+        x[:] = 0                        # the source has been read when the call returns
+        y = np.empty(nbytes, np.uint8)
+        rt.memcpy_d2h(y.ctypes.data, p, nbytes)
+        rt.stream_sync()
+        assert np.array_equal(y, expected)
+        rt.free(p)
+    # a stream of its own, and a pinned source
+    s = ctypes.c_void_p()
+    rt.call("docc_rocm_stream_create", ctypes.byref(s))
+    n = (20 << 20) + 5
+    x = rng.integers(0, 256, n, dtype=np.uint8)
+    hp = ctypes.c_void_p()
+    rt.call("docc_rocm_host_malloc", ctypes.byref(hp), n)
+    pinned = np.frombuffer((ctypes.c_uint8 * n).from_address(hp.value), dtype=np.uint8)
+    pinned[:] = x[::-1]
+    p, q = rt.malloc(n), rt.malloc(n)
+    rt.memcpy_h2d(p, x.ctypes.data, n, s.value)
+    rt.memcpy_h2d(q, hp.value, n, s.value)
+    y, z = np.empty(n, np.uint8), np.empty(n, np.uint8)
+    rt.memcpy_d2h(y.ctypes.data, p, n, s.value)
+    rt.memcpy_d2h(z.ctypes.data, q, n, s.value)
+    rt.stream_sync(s.value)
+    assert np.array_equal(y, x) and np.array_equal(z, x[::-1])
+    rt.free(p); rt.free(q)
+    rt.call("docc_rocm_host_free", hp)
+    rt.call("docc_rocm_stream_destroy", s)
