@@ -103,11 +103,13 @@ def main():
     clock_out = torch.zeros(1, device="cuda")
 
     def sustained_clock_ghz(fn, launch_ms):
-        n = max(8, int(4.0 / max(launch_ms, 1e-3)) + 4)     # at least 4 ms of back-to-back launches
+        # the clocks settle over the first 10-20 ms of load: look at them after 30 ms of it, with launches still queued behind
+        per_ms = 1.0 / max(launch_ms, 1e-3)
+        at, n = max(2, int(30.0 * per_ms)), max(4, int(34.0 * per_ms) + 2)
         rt.device_sync()
         for i in range(n):
             fn(i)
-            if i == min(n // 8, 16):
+            if i == at:
                 rt.clock_probe(1000, clock_out.data_ptr(), probe_stream)
         rt.device_sync()
         return round(float(clock_out.item()) / 1000.0, 3)
@@ -195,7 +197,7 @@ def main():
         prec = {"f64": 64, "f32": 32, "bf16": 16}[dtype]
         ops = torch.randn(4096, device="cuda")
         sink = torch.empty(2 * 256 * max(info["compute_units"], 1), device="cuda")
-        iters = 4000
+        iters = 8000
         best, best_clock = 0.0, 0.0
         for waves in (1, 2):
             flop = [0.0]
@@ -203,7 +205,7 @@ def main():
             def probe(i, waves=waves):
                 flop[0] = rt.mfma_probe(prec, waves, iters, ops.data_ptr(), sink.data_ptr(), stream)
 
-            ms = time_kernel(probe, 5, 2)
+            ms = time_kernel(probe, 8, 2)
             if flop[0] / ms / 1e9 > best:
                 best, best_clock = flop[0] / ms / 1e9, sustained_clock_ghz(probe, ms)
         ceiling_cache[dtype] = (round(best, 1), best_clock)

@@ -52,10 +52,17 @@ typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
 typedef double probe_f64x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
 
+// Every index below is a compile-time constant once the loops are unrolled, so the operand sets live in
+// registers and the set-up is sixteen loads: with run-time indices the compiler builds the sets one lane
+// at a time, which costs as much as thousands of rounds and is then counted as matrix time. The MFMAs are
+// written as asm with the accumulators held in VGPRs: left to itself the compiler keeps them in AGPRs and,
+// for the fp64 loop, copies them across and back every round.
 extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f64(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
     probe_f64x4 acc[4];
+#pragma unroll
     for (int i = 0; i < 4; i++) acc[i] = {0, 0, 0, 0};
     double a[8], b[8];
+#pragma unroll
     for (int i = 0; i < 8; i++) {
         a[i] = operands[(threadIdx.x * 8 + i) & 4095];
         b[i] = operands[(threadIdx.x * 8 + i + 2048) & 4095];
@@ -64,18 +71,22 @@ extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f64(const floa
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+            for (int i = 0; i < 4; i++) asm volatile("v_mfma_f64_16x16x4_f64 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[(s + i) & 7]), "v"(b[s]));
     }
     double r = 0;
+#pragma unroll
     for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][3];
     sink[blockIdx.x * 256 + threadIdx.x] = (float) r;
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f32(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
     probe_f32x16 acc[4];
+#pragma unroll
     for (int i = 0; i < 4; i++)
+#pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0;
     float a[8], b[8];
+#pragma unroll
     for (int i = 0; i < 8; i++) {
         a[i] = operands[(threadIdx.x * 8 + i) & 4095];
         b[i] = operands[(threadIdx.x * 8 + i + 2048) & 4095];
@@ -84,30 +95,38 @@ extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_f32(const floa
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+            for (int i = 0; i < 4; i++) asm volatile("v_mfma_f32_32x32x2_f32 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[(s + i) & 7]), "v"(b[s]));
     }
     float r = 0;
+#pragma unroll
     for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][15];
     sink[blockIdx.x * 256 + threadIdx.x] = r;
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_bf16(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
     probe_f32x16 acc[4];
+#pragma unroll
     for (int i = 0; i < 4; i++)
+#pragma unroll
         for (int r = 0; r < 16; r++) acc[i][r] = 0;
+    // each lane's eight operand sets: 64 consecutive table entries (a), the 64 of the lane 28 further on (b)
+    const float4* row_a = reinterpret_cast<const float4*>(operands + ((threadIdx.x * 64) & 4095));
+    const float4* row_b = reinterpret_cast<const float4*>(operands + ((threadIdx.x * 64 + 1792) & 4095));
     probe_bf16x8 a[8], b[8];
-    for (int i = 0; i < 8; i++)
-        for (int e = 0; e < 8; e++) {
-            a[i][e] = (__bf16) operands[(threadIdx.x * 64 + i * 8 + e) & 4095];
-            b[i][e] = (__bf16) operands[(threadIdx.x * 64 + i * 8 + e + 1777) & 4095];
-        }
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float4 a0 = row_a[2 * i], a1 = row_a[2 * i + 1], b0 = row_b[2 * i], b1 = row_b[2 * i + 1];
+        a[i] = probe_bf16x8{(__bf16) a0.x, (__bf16) a0.y, (__bf16) a0.z, (__bf16) a0.w, (__bf16) a1.x, (__bf16) a1.y, (__bf16) a1.z, (__bf16) a1.w};
+        b[i] = probe_bf16x8{(__bf16) b0.x, (__bf16) b0.y, (__bf16) b0.z, (__bf16) b0.w, (__bf16) b1.x, (__bf16) b1.y, (__bf16) b1.z, (__bf16) b1.w};
+    }
     for (int it = 0; it < iters; it++) {
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[(s + i) & 7], b[s], acc[i], 0, 0, 0);
+            for (int i = 0; i < 4; i++) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[(s + i) & 7]), "v"(b[s]));
     }
     float r = 0;
+#pragma unroll
     for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][15];
     sink[blockIdx.x * 256 + threadIdx.x] = r;
 }
