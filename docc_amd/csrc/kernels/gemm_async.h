@@ -130,7 +130,9 @@ struct AsyncTile {
     }
 };
 
-template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool TA, bool TB>
+// SPREAD: the copies that refill a stage are dealt over the MFMAs of a whole K-step instead of being issued in
+// one run behind the barrier (needs three stages or more; see the pipeline comment in run()).
+template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool TA, bool TB, bool SPREAD = false>
 struct AsyncGemmKernel {
     typedef AsyncTraits<T> X;
     typedef typename X::acc_t acc_t;
@@ -148,6 +150,7 @@ struct AsyncGemmKernel {
     static constexpr int LOADS_PER_STEP = ATile::NV + BTile::NV;
     static_assert(BK % KG == 0, "BK must be a multiple of the k-group");
     static_assert(STAGES >= 2 && (STAGES - 1) * LOADS_PER_STEP < 64, "vmcnt holds at most 63 outstanding loads");
+    static_assert(!SPREAD || STAGES >= 3, "copies dealt over a K-step need a stage that nobody reads meanwhile");
 
     static __device__ __forceinline__ void run(const T* __restrict__ A, const T* __restrict__ B, out_t* __restrict__ C,
                                                long M, long N, long K, long lda, long ldb, long ldc, out_t alpha,
@@ -290,7 +293,7 @@ struct AsyncGemmKernel {
         for (int s = 0; s < STAGES - 1; s++)
             if (s < ksteps) fill(s);
         arrive(0);
-        if (STAGES - 1 < ksteps) fill(STAGES - 1);
+        if (!SPREAD && STAGES - 1 < ksteps) fill(STAGES - 1);
         fetch(stage_of(0), 0, 0);
 
         // the last K-step has no successor: it is peeled so that the loop body is free of branches
@@ -308,7 +311,7 @@ struct AsyncGemmKernel {
         constexpr int PPM = (NPIECE + NM - 1) / NM;                   // pieces per MFMA, inner steps but the last
         constexpr int PPL = (NPIECE + NM - 2) / (NM - 1);             // pieces per MFMA, last inner step
         constexpr int LPM = (LOADS_PER_STEP + NM - 2) / (NM - 1);     // copies per MFMA, last inner step
-        auto kstep = [&](int kt, auto mode_c) {
+        auto kstep_burst = [&](int kt, auto mode_c) {
             constexpr int MODE = decltype(mode_c)::value;
             constexpr bool NEXT = MODE != 2;
             const T* st = stage_of(kt);
@@ -357,8 +360,85 @@ struct AsyncGemmKernel {
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
+        // The same with the copies dealt out (SPREAD). All four waves leave the barrier together, and a run of
+        // copies from each of them at that moment queues up in the one vector-memory pipe of the CU; the waves
+        // then sit behind their own copies while the matrix pipe idles. Here K-step kt issues the copies of step
+        // kt+STAGES-1, one every LSTRIDE MFMAs over the whole step, into the stage that the barrier at the end
+        // of step kt-1 freed; nobody reads that stage before step kt+STAGES-1. At the wait in the last inner
+        // step the copies of step kt+1 are older than those of STAGES-3 whole steps and the EARLY copies this
+        // step has issued so far.
+        constexpr int SLOTS = NKI * NM;                                                        // MFMAs of a K-step
+        constexpr int LSTRIDE = SLOTS / LOADS_PER_STEP > 0 ? SLOTS / LOADS_PER_STEP : 1;       // MFMAs between two copies
+        constexpr int LPS = (LOADS_PER_STEP + SLOTS - 1) / SLOTS;                              // copies per slot when there are more copies than MFMAs
+        // copies issued behind MFMA `slot` (0-based over the K-step): indices [lo, hi)
+        auto copies_lo = [](int slot) constexpr { return SLOTS >= LOADS_PER_STEP ? (slot + 1) / LSTRIDE : slot * LPS; };
+        constexpr int WAIT_SLOT = (NKI - 1) * NM;                                              // the MFMA the wait follows
+        constexpr int EARLY_RAW = SLOTS >= LOADS_PER_STEP ? (WAIT_SLOT + 2) / LSTRIDE : (WAIT_SLOT + 1) * LPS;    // = copies_lo(WAIT_SLOT + 1)
+        constexpr int EARLY = EARLY_RAW < LOADS_PER_STEP ? EARLY_RAW : LOADS_PER_STEP;
+        auto kstep_spread = [&](int kt, auto mode_c) {
+            constexpr int MODE = decltype(mode_c)::value;
+            constexpr bool NEXT = MODE != 2;
+            const T* st = stage_of(kt);
+            T* dst = lds + ((kt + STAGES - 1) % STAGES) * STAGE_ELEMS;
+            if (MODE == 0) {
+                ta.advance();
+                tb.advance();
+            } else if (MODE == 1) {
+                if (kt + STAGES - 1 < ksteps) fill(kt + STAGES - 1);    // the K tail, through registers
+            }
+            auto copies = [&](int slot) {
+                if (MODE != 0) return;
+                int lo = copies_lo(slot), hi = copies_lo(slot + 1);
+                if (slot == SLOTS - 1) hi = LOADS_PER_STEP;
+#pragma unroll
+                for (int q = lo; q < hi && q < LOADS_PER_STEP; q++) {
+                    if (q < ATile::NV) ta.issue_one(dst, q, wave);
+                    else tb.issue_one(dst + ATile::ELEMS, q - ATile::NV, wave);
+                }
+            };
+#pragma unroll
+            for (int ki = 0; ki < NKI; ki++) {
+                if (ki + 1 < NKI) {
+#pragma unroll
+                    for (int n = 0; n < NM; n++) {
+                        mma(ki & 1, n, n + 1);
+#pragma unroll
+                        for (int q = n * PPM; q < (n + 1) * PPM && q < NPIECE; q++) fetch_piece(st, ki + 1, (ki + 1) & 1, q);
+                        copies(ki * NM + n);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else if (NEXT) {
+                    mma(ki & 1, 0, 1);
+                    copies(ki * NM);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (MODE == 0) {
+                        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 3) * LOADS_PER_STEP + EARLY) : "memory");
+                    } else {
+                        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+                    }
+                    __builtin_amdgcn_s_barrier();
+                    asm volatile("" ::: "memory");
+                    const T* nst = stage_of(kt + 1);
+#pragma unroll
+                    for (int n = 1; n < NM; n++) {
+                        mma(ki & 1, n, n + 1);
+#pragma unroll
+                        for (int q = (n - 1) * PPL; q < n * PPL && q < NPIECE; q++) fetch_piece(nst, 0, 0, q);
+                        copies(ki * NM + n);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
+                    mma(ki & 1, 0, NM);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        auto kstep = [&](int kt, auto mode_c) {
+            if constexpr (SPREAD) kstep_spread(kt, mode_c);
+            else kstep_burst(kt, mode_c);
+        };
         int kt = 0;
-        for (; kt + STAGES < full; kt++) kstep(kt, std::integral_constant<int, 0>{});
+        for (; kt + STAGES - (SPREAD ? 1 : 0) < full; kt++) kstep(kt, std::integral_constant<int, 0>{});
         for (; kt + 1 < ksteps; kt++) kstep(kt, std::integral_constant<int, 1>{});
         kstep(kt, std::integral_constant<int, 2>{});
 
@@ -380,6 +460,22 @@ struct AsyncGemmKernel {
         docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB>::run(A + z * batch_a, B + z * batch_b, C + z * batch_c, M, N, \
                                                                         K, lda, ldb, ldc, alpha, beta, bias, act); \
     }
+
+// the same with the copies dealt over the K-step: docc_<prefix>a_<BM>x<BN>x<BK>p<STAGES>_<nn|nt|tn|tt>
+#define DOCC_AGEMM_SPREAD_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, TA, TB, TAG)                                   \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void DOCC_GEMM_NAME(docc_##PREFIX##a_##BM##x##BN##x##BK##p##ST##_##TAG)(  \
+        const T* A, const T* B, OT* C, long M, long N, long K, long lda, long ldb, long ldc, OT alpha, OT beta,    \
+        const OT* bias, int act, long batch_a, long batch_b, long batch_c) {                                       \
+        const long z = blockIdx.y;                                                                                 \
+        docc_k::AsyncGemmKernel<T, BM, BN, BK, WM, WN, ST, TA, TB, true>::run(A + z * batch_a, B + z * batch_b, C + z * batch_c, \
+                                                                              M, N, K, lda, ldb, ldc, alpha, beta, bias, act);  \
+    }
+
+#define DOCC_AGEMM_SPREAD_CONFIG(PREFIX, T, OT, BM, BN, BK, WM, WN, ST)            \
+    DOCC_AGEMM_SPREAD_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, false, false, nn)   \
+    DOCC_AGEMM_SPREAD_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, false, true, nt)    \
+    DOCC_AGEMM_SPREAD_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, true, false, tn)    \
+    DOCC_AGEMM_SPREAD_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, true, true, tt)
 
 #define DOCC_AGEMM_CONFIG(PREFIX, T, OT, BM, BN, BK, WM, WN, ST)            \
     DOCC_AGEMM_ONE(PREFIX, T, OT, BM, BN, BK, WM, WN, ST, false, false, nn)   \

@@ -15,6 +15,7 @@ DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 256, 16, 2, 2, 3)
 DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 256, 16, 2, 2, 4)
 DOCC_AGEMM_CONFIG(sgemm, float, float, 128, 256, 32, 2, 2, 3)
 DOCC_AGEMM_CONFIG(sgemm, float, float, 64, 64, 32, 2, 2, 3)
+DOCC_AGEMM_SPREAD_CONFIG(sgemm, float, float, 128, 256, 32, 2, 2, 3)   // copies dealt over the K-step: 2-3 % slower here
 #endif
 
 #ifndef DOCC_GEMM_EPILOGUE

@@ -17,6 +17,7 @@ DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 16, 2, 2, 4)
 #ifndef DOCC_GEMM_EPILOGUE   // tuning alternative: no epilogue variant
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 32, 32, 2, 2, 3)
 DOCC_AGEMM_CONFIG(dgemm, double, double, 64, 64, 32, 2, 2, 3)
+DOCC_AGEMM_SPREAD_CONFIG(dgemm, double, double, 64, 32, 16, 2, 2, 4)   // copies dealt over the K-step: no difference here
 #endif
 
 #ifndef DOCC_GEMM_EPILOGUE

@@ -170,13 +170,14 @@ def test_sgemm_config_4096(rt):
     assert np.abs(lhs - rhs).max() / np.abs(rhs).max() <= 1e-5
 
 
-# every built tile configuration, selected through DOCC_ROCM_GEMM_CFG (BMxBNxBKxWAVES[xSTAGES]; a
-# trailing stage count picks the asynchronous multi-stage kernel), on shapes with ragged edges,
+# every built tile configuration, selected through DOCC_ROCM_GEMM_CFG (BMxBNxBKxWAVES[xSTAGES[p]]; a
+# trailing stage count picks the asynchronous multi-stage kernel, "p" its variant with a stage's copies
+# dealt over the K-step), on shapes with ragged edges,
 # a K tail and all four transpose combinations
 F64_CFGS = ["64x64x16x4", "128x128x16x4", "64x64x16x4x2", "64x64x16x4x4", "64x64x16x4x6", "128x128x16x4x3",
-            "64x32x16x4x4", "64x32x32x4x3", "64x64x32x4x3"]
+            "64x32x16x4x4", "64x32x32x4x3", "64x64x32x4x3", "64x32x16x4x4p"]
 F32_CFGS = ["64x64x16x4", "128x128x16x4", "128x128x16x4x3", "128x128x32x4x3", "128x256x16x4x3", "64x64x16x4x4",
-            "64x64x32x4x3", "128x256x32x4x2", "128x256x32x4x3", "128x256x16x4x4"]
+            "64x64x32x4x3", "128x256x32x4x2", "128x256x32x4x3", "128x256x16x4x4", "128x256x32x4x3p"]
 
 
 @pytest.mark.parametrize("dt,cfg", [(np.float64, c) for c in F64_CFGS] + [(np.float32, c) for c in F32_CFGS])

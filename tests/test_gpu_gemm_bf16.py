@@ -107,10 +107,10 @@ def test_device_bf16_conversion_matches_oracle(rt):
     assert np.array_equal(host(back), oracle.bf16_to_f32(bits))
 
 
-# every built tile configuration (DOCC_ROCM_GEMM_CFG = BMxBNxBKxWAVES[xSTAGES]; a stage count picks the
+# every built tile configuration (DOCC_ROCM_GEMM_CFG = BMxBNxBKxWAVES[xSTAGES[p]]; a stage count picks the
 # asynchronous kernel), ragged edges, a K tail, all transposes
 BF16_CFGS = ["128x128x64x4", "256x256x64x4", "128x128x64x4x3", "128x128x64x4x4", "128x128x32x4x4", "128x256x64x4x3",
-             "256x256x64x4x2", "256x256x32x4x4"]
+             "256x256x64x4x2", "256x256x32x4x4", "256x256x32x4x4p"]
 
 
 @pytest.mark.parametrize("cfg", BF16_CFGS)
