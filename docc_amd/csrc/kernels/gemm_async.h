@@ -306,10 +306,12 @@ struct AsyncGemmKernel {
         //   refill stage kt and the LDS reads of step kt+1's first operands.
         // mode 0: steady state (the refill is a full asynchronous step, nothing in the body branches);
         // mode 1: near the end (the refill may be the K tail or absent); mode 2: the last step
-        // shares per MFMA slot, dealt from the first slot on so that the last LDS read is issued well
-        // before the inner step ends (its latency would otherwise be waited for at the next step)
-        constexpr int PPM = (NPIECE + NM - 1) / NM;                   // pieces per MFMA, inner steps but the last
-        constexpr int PPL = (NPIECE + NM - 2) / (NM - 1);             // pieces per MFMA, last inner step
+        // shares per MFMA slot. The LDS reads are dealt over the first half of an inner step's slots only, so that
+        // the last of them is issued at least half an inner step before its operand is needed (with the four
+        // MFMAs of an fp64 inner step, one read per MFMA left the last read 64 cycles: the next step waited for it)
+        constexpr int PSLOTS = NM / 2 > 0 ? NM / 2 : 1, PSLOTS_LAST = NM / 2 > 0 ? NM / 2 : 1;
+        constexpr int PPM = (NPIECE + PSLOTS - 1) / PSLOTS;           // pieces per MFMA, inner steps but the last
+        constexpr int PPL = (NPIECE + PSLOTS_LAST - 1) / PSLOTS_LAST; // pieces per MFMA, last inner step
         constexpr int LPM = (LOADS_PER_STEP + NM - 2) / (NM - 1);     // copies per MFMA, last inner step
         auto kstep_burst = [&](int kt, auto mode_c) {
             constexpr int MODE = decltype(mode_c)::value;
