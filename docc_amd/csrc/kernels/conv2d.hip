@@ -211,14 +211,24 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 // are then one 128-bit LDS read per lane: the weights at [oc][t][4g..4g+3], the pixels at
 // [(r+kh)*WP + (c+kw)][4g..4g+3], whose address is a wave-uniform tap term plus a per-lane pixel
 // term: im2col costs one add per read.
+//
+// SPLIT: a strip of 13 column tiles (at most 416 pixels). The waves of a pixel group take six tiles each and
+// share the thirteenth: in every chunk group 0 multiplies it over the first half of the chunk's k-slices, group 1
+// over the second half (the work-group meets at a barrier per chunk, so the halves must balance inside a chunk),
+// and the two partial tiles are added through LDS before the store. Both groups run the same instructions: the
+// shared tile has operand registers of its own, and group 1 simply fetches them from the mirrored tap (tap 8 - t
+// where group 0 reads tap t; of the middle tap each takes two of the four slices). A wave then carries 6.5 tiles instead
+// of 7, which is what lets 8 strips of 7 rows (one work-group on each of 256 CUs) beat 7 strips of 8 rows on a
+// 56x56 image: both are one round of work-groups, and the round is as long as its waves' MFMA count.
 namespace docc_k {
 
-template <int KH, int KW>
+template <int KH, int KW, bool SPLIT = false>
 struct ConvHaloKernel {
     static constexpr int KHW = KH * KW;
     static constexpr int CI = 8;                 // input channels per chunk
     static constexpr int KC = CI * KHW;          // k per chunk
-    static constexpr int TN = 7;                 // MFMA column tiles per wave
+    static constexpr int TN = 7;                 // MFMA column tiles per wave (SPLIT: the seventh is the shared one)
+    static constexpr int TOWN = SPLIT ? 6 : 7;   // column tiles a wave has to itself
     static constexpr int LDA_S = KC + 4;
     static constexpr int A_ELEMS = 64 * LDA_S;
     static constexpr int NR = 3;                 // patch pixels per thread per chunk (upper bound)
@@ -227,7 +237,7 @@ struct ConvHaloKernel {
     static __device__ __forceinline__ void run(const ConvParams& p, int TH) {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_conv_lds[];
         float* const lds = reinterpret_cast<float*>(docc_conv_lds);
-        const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+        const int tid = threadIdx.x, lane = tid & 63, wave = SPLIT ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;   // SPLIT: the mirrored tap is a scalar
         const int l32 = lane & 31, g = lane >> 5;
         const int ocw = wave & 1, pg = wave >> 1;
 
@@ -240,10 +250,12 @@ struct ConvHaloKernel {
 
         // per-lane patch offsets (floats) of the 7 column tiles of this wave: pixel (r, c) of the
         // strip and the channel half of this lane
+        // first pixel of column tile j of this wave
+        auto tile_pixel0 = [&](int j) { return j < TOWN ? (pg * TOWN + j) * 32 : 2 * TOWN * 32; };
         int boff[TN];
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            int q = pg * (TN * 32) + j * 32 + l32;
+            int q = tile_pixel0(j) + l32;
             q = q < npix ? q : 0;
             boff[j] = ((q / p.OW) * WP + (q % p.OW)) * CI + 4 * g;
         }
@@ -333,12 +345,34 @@ struct ConvHaloKernel {
         constexpr int T0 = 0;
         constexpr int TB = KHW > 1 ? KHW - 2 : 0;
         f32x4 a[2], b[2][TN];
+        f32x4 a6[2];                                     // SPLIT: the shared tile's own weight operand (its pixels: b[.][TN - 1])
+        static_assert(!SPLIT || KHW % 2 == 1, "the shared tile is halved in the middle tap");
+        // slices of tap t that go into the shared tile (code order; group 1 maps them to the mirrored tap)
+        auto shared_slices = [](int t) constexpr { return !SPLIT ? 4 : 4 * t + 4 <= 2 * KHW ? 4 : 4 * t < 2 * KHW ? 2 : 0; };
         auto fetch = [&](int base, int t, int to) {
             const float* arow = lds + base + (ocw * 32 + l32) * LDA_S + 4 * g + t * CI;
             a[to] = *reinterpret_cast<const f32x4*>(arow);
             const float* bt = lds + base + A_ELEMS + ((t / KW) * WP + (t % KW)) * CI;     // wave-uniform
 #pragma unroll
-            for (int j = 0; j < TN; j++) b[to][j] = *reinterpret_cast<const f32x4*>(bt + boff[j]);
+            for (int j = 0; j < TOWN; j++) b[to][j] = *reinterpret_cast<const f32x4*>(bt + boff[j]);
+            if constexpr (SPLIT) {
+                const int n6 = shared_slices(t);
+                if (n6 > 0) {
+                    const int tt = pg ? KHW - 1 - t : t;                   // wave-uniform
+                    const int sh = (pg && n6 == 2) ? 2 : 0;                // the middle tap: group 1 takes its upper two slices
+                    const float* arow6 = lds + base + (ocw * 32 + l32) * LDA_S + 4 * g + tt * CI + sh;
+                    const float* b6 = lds + base + A_ELEMS + ((tt / KW) * WP + (tt % KW)) * CI + boff[TN - 1] + sh;
+                    if (n6 == 4) {
+                        a6[to] = *reinterpret_cast<const f32x4*>(arow6);
+                        b[to][TN - 1] = *reinterpret_cast<const f32x4*>(b6);
+                    } else {
+                        typedef float f32x2 __attribute__((ext_vector_type(2)));
+                        const f32x2 av = *reinterpret_cast<const f32x2*>(arow6), bv = *reinterpret_cast<const f32x2*>(b6);
+                        a6[to][0] = av[0], a6[to][1] = av[1];
+                        b[to][TN - 1][0] = bv[0], b[to][TN - 1][1] = bv[1];
+                    }
+                }
+            }
         };
         // par: parity of the chunk's first tap in the tap stream (operand registers alternate per tap).
         // Each tap is one scheduling region: its 28 MFMAs, the LDS reads of the next tap's operands,
@@ -367,8 +401,14 @@ struct ConvHaloKernel {
 #pragma unroll
                 for (int s = 0; s < 4; s++)
 #pragma unroll
-                    for (int j = 0; j < TN; j++)
-                        acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[so][s], b[so][j][s], acc[j], 0, 0, 0);
+                    for (int j = 0; j < TN; j++) {
+                        if (j < TOWN) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[so][s], b[so][j][s], acc[j], 0, 0, 0);
+                        else if (s < shared_slices(t)) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a6[so][s], b[so][j][s], acc[j], 0, 0, 0);
+                    }
+                const int nmfma = 4 * TOWN + (SPLIT ? shared_slices(t) : 0);
+                // LDS reads issued in this region: the next tap's weights, its own tiles' pixels and, if it has any, the shared tile's pair
+                const int tn = t + 1 < KHW ? t + 1 : 0;
+                const int nreads = 1 + TOWN + (SPLIT && shared_slices(tn) > 0 ? 2 : 0);
                 int writes = 0, loads = 0;
                 if constexpr (NEXT) {
                     const int i0 = t < T0 ? 0 : NSL * (t - T0) / (TB + 1 - T0);
@@ -382,11 +422,11 @@ struct ConvHaloKernel {
                     }
                 }
 #pragma unroll
-                for (int i = 0; i < 4 * TN; i++) {
+                for (int i = 0; i < nmfma; i++) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // MFMA
-                    if (reads && i < TN + 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS read
-                    if (i >= TN + 1 && i - (TN + 1) < writes) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS write
-                    if (i >= TN + 1 && ((i - (TN + 1)) & 1) == 0 && (i - (TN + 1)) / 2 < loads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // load
+                    if (reads && i < nreads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // LDS read
+                    if (i >= nreads && i - nreads < writes) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);   // LDS write
+                    if (i >= nreads && ((i - nreads) & 1) == 0 && (i - nreads) / 2 < loads) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);    // load
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 if constexpr (NEXT) {
@@ -411,47 +451,66 @@ struct ConvHaloKernel {
             if (nxt == 3 * stage_elems) nxt = 0;
         };
         constexpr int P1 = KHW & 1;      // parity of the second chunk of a pair
-        int ch = 0;
-        for (; ch + 2 < nch; ch += 2) {
-            step(std::integral_constant<int, 0>{}, std::true_type{}, cur, nxt, ch + 2);
-            advance();
-            step(std::integral_constant<int, P1>{}, std::true_type{}, cur, nxt, ch + 3 < nch ? ch + 3 : nch - 1);
-            advance();
+        typedef std::integral_constant<int, 0> Par0;
+        typedef std::integral_constant<int, P1> Par1;
+        {
+            int ch = 0;
+            for (; ch + 2 < nch; ch += 2) {
+                step(Par0{}, std::true_type{}, cur, nxt, ch + 2);
+                advance();
+                step(Par1{}, std::true_type{}, cur, nxt, ch + 3 < nch ? ch + 3 : nch - 1);
+                advance();
+            }
+            if (ch + 2 == nch) {
+                step(Par0{}, std::true_type{}, cur, nxt, nch - 1);
+                advance();
+                step(Par1{}, std::false_type{}, cur, nxt, 0);
+            } else {
+                step(Par0{}, std::false_type{}, cur, nxt, 0);
+            }
         }
-        if (ch + 2 == nch) {
-            step(std::integral_constant<int, 0>{}, std::true_type{}, cur, nxt, nch - 1);
-            advance();
-            step(std::integral_constant<int, P1>{}, std::false_type{}, cur, nxt, 0);
-        } else {
-            step(std::integral_constant<int, 0>{}, std::false_type{}, cur, nxt, 0);
+        if constexpr (SPLIT) {
+            // the two halves of the shared tile meet in LDS, [channel tile][accumulator register][lane]
+            __syncthreads();
+            float* xch = lds + ocw * (16 * 64);
+            if (pg == 1) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) xch[r * 64 + lane] = acc[TN - 1][r];
+            }
+            __syncthreads();
+            if (pg == 0) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[TN - 1][r] += xch[r * 64 + lane];
+            }
         }
 
         // epilogue: rows of the accumulator = output channels, columns = pixels of the strip. A tile
         // that lies wholly inside the output (the usual case) is stored by straight-line code; one
         // branch per element costs more in instruction fetch than the stores themselves.
-        const bool whole = oc0 + 64 <= p.OC && oh0 + TH <= p.OH && (pg + 1) * (TN * 32) <= npix;
+        const bool whole = oc0 + 64 <= p.OC && oh0 + TH <= p.OH && (pg + 1) * (TOWN * 32) <= npix;
         if (whole) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int q = pg * (TN * 32) + j * 32 + l32;
+            for (int j = 0; j < TOWN; j++) {
+                const int q = tile_pixel0(j) + l32;
                 float* ybase = p.Y + ((long) n * p.OC * p.OH + oh0 + q / p.OW) * p.OW + q % p.OW +
                                (long) (oc0 + ocw * 32 + 4 * g) * p.OH * p.OW;
 #pragma unroll
                 for (int r = 0; r < 16; r++)
                     ybase[(long) (8 * (r / 4) + r % 4) * p.OH * p.OW] = acc[j][r] + bias_r[r];
             }
-        } else {
+        }
+        // tiles that may leave the output: all of them on a ragged strip, and the shared tile (group 0 holds its sum)
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int q = pg * (TN * 32) + j * 32 + l32;
-                const int oh = oh0 + q / p.OW, ow = q % p.OW;
-                if (q >= npix || oh >= p.OH) continue;
-                float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+        for (int j = 0; j < TN; j++) {
+            if (j < TOWN ? whole : pg != 0) continue;
+            const int q = tile_pixel0(j) + l32;
+            const int oh = oh0 + q / p.OW, ow = q % p.OW;
+            if (q >= npix || oh >= p.OH) continue;
+            float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
-                    if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = acc[j][r] + bias_r[r];
-                }
+            for (int r = 0; r < 16; r++) {
+                const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
+                if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = acc[j][r] + bias_r[r];
             }
         }
     }
@@ -465,6 +524,10 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3(docc_
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_k::ConvParams p, int TH) {
     docc_k::ConvHaloKernel<1, 1>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, true>::run(p, TH);
 }
 
 // Explicit im2col for the layers the two kernels above serve badly (small images, many channels): the

@@ -42,6 +42,7 @@ CASES = [
     (1, 24, 5, 100, 64, 3, 3, (1, 1), (2, 1), (1, 1), True),    # wide rows: 4 rows per strip, asymmetric pad sizes
     (2, 32, 12, 12, 16, 1, 1, (1, 1), (0, 0), (1, 1), True),    # 1x1
     (1, 8, 3, 448, 8, 3, 3, (1, 1), (1, 1), (1, 1), False),     # one row per strip
+    (2, 32, 14, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),    # 7 rows of 56: 13 column tiles, the last shared by two waves
 ]
 
 
@@ -145,11 +146,12 @@ def run_conv_ws(rt, X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1),
     return host(y), need
 
 
-@pytest.mark.parametrize("force", ["gemm", "gather", "halo", ""])
+@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-whole", ""])
 @pytest.mark.parametrize("case", CASES)
 def test_conv_every_path_integer_exact(rt, monkeypatch, force, case):
-    """Each way to run a layer (forced through DOCC_ROCM_CONV; a path that does not apply falls back) and the
-    automatic choice give the oracle's integers."""
+    """Each way to run a layer (forced through DOCC_ROCM_CONV; a path that does not apply falls back; halo-split and
+    halo-whole are the LDS-halo kernel with strips of 13 shared and 14 whole column tiles) and the automatic choice
+    give the oracle's integers."""
     N, C, H, W, OC, KH, KW, stride, pad, dil, use_bias = case
     if force:
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
