@@ -255,8 +255,18 @@ __device__ __forceinline__ void gemv_cols_final(const void* partials, T* __restr
     const int c = threadIdx.x & 15, g = threadIdx.x >> 4;
     const long col = (long) blockIdx.x * 16 + c;
     T acc = (T) 0;
-    if (col < cols)
-        for (long s = g; s < slices; s += 16) acc += P[s * cols + col];
+    if (col < cols) {
+        // eight loads in flight, added in slice order
+        long s = g;
+        for (; s + 7 * 16 < slices; s += 8 * 16) {
+            T v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) v[k] = P[(s + 16 * k) * cols + col];
+#pragma unroll
+            for (int k = 0; k < 8; k++) acc += v[k];
+        }
+        for (; s < slices; s += 16) acc += P[s * cols + col];
+    }
     part[g][c] = acc;
     __syncthreads();
     if (g == 0 && col < cols) {

@@ -145,8 +145,18 @@ __device__ __forceinline__ void column_reduce_final(const void* partials, T* Y, 
     const int col = threadIdx.x & 15, lane_s = threadIdx.x >> 4;
     const long idx = (long) blockIdx.x * 16 + col;
     T a = reduce_identity<OP, T>();
-    if (idx < total)
-        for (long s = lane_s; s < slices; s += 16) a = combine<OP>(a, P[s * total + idx]);
+    if (idx < total) {
+        // eight loads in flight, combined in slice order: one load at a time is one memory round trip per slice
+        long s = lane_s;
+        for (; s + 7 * 16 < slices; s += 8 * 16) {
+            T v[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) v[k] = P[(s + 16 * k) * total + idx];
+#pragma unroll
+            for (int k = 0; k < 8; k++) a = combine<OP>(a, v[k]);
+        }
+        for (; s < slices; s += 16) a = combine<OP>(a, P[s * total + idx]);
+    }
     part[lane_s][col] = a;
     __syncthreads();
     if (lane_s == 0 && idx < total) {

@@ -1,5 +1,6 @@
 // Launcher for the reduce tensor nodes (see include/docc_rocm_ops.h).
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "docc_rocm_ops.h"
@@ -44,7 +45,9 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
         int64_t slices = ((int64_t) cus * 8 + pblocks - 1) / pblocks;
         if (slices > reduce / 16) slices = reduce / 16;
         if (slices > scratch_elems / total) slices = scratch_elems / total;
-        if (slices > 256) slices = 256;
+        int64_t cap = 256;
+        if (const char* e = std::getenv("DOCC_ROCM_REDUCE_SLICES")) cap = std::atoll(e) > 0 ? std::atoll(e) : cap;   // tuning
+        if (slices > cap) slices = cap;
         if (slices > 1) {
             const int64_t chunk = (reduce + slices - 1) / slices;
             slices = (reduce + chunk - 1) / chunk;
