@@ -136,3 +136,52 @@ def test_large_uploads_from_pageable_memory_are_staged_through_pinned_chunks(rt)
     rt.free(p); rt.free(q)
     rt.call("docc_rocm_host_free", hp)
     rt.call("docc_rocm_stream_destroy", s)
+
+
+@pytest.mark.parametrize("precision", [64, 32, 16])
+def test_mfma_probe_times_its_loop_and_nothing_else(rt, precision):
+    """The ceiling probe's launch time must be its MFMA loop: twice the rounds take twice as long (operand
+    set-up that costs as much as thousands of rounds once passed for matrix time), and the flop count it
+    reports is 32 MFMAs per round and wave."""
+    import statistics
+    import torch
+    ops = torch.randn(4096, device="cuda")
+    sink = torch.empty(2 * 256 * 512, device="cuda")
+
+    def timed(iters):
+        flop = rt.mfma_probe(precision, 1, iters, ops.data_ptr(), sink.data_ptr())
+        for _ in range(3):
+            rt.mfma_probe(precision, 1, iters, ops.data_ptr(), sink.data_ptr())
+        rt.device_sync()
+        ts = []
+        for _ in range(5):
+            e0, e1 = rt.Event(), rt.Event()
+            e0.record()
+            rt.mfma_probe(precision, 1, iters, ops.data_ptr(), sink.data_ptr())
+            e1.record()
+            ts.append(e0.elapsed_ms(e1))
+        return statistics.median(ts), flop
+
+    for _ in range(20):   # clocks up
+        rt.mfma_probe(precision, 1, 2000, ops.data_ptr(), sink.data_ptr())
+    t1, f1 = timed(2000)
+    t2, f2 = timed(4000)
+    per_mfma = {64: 2048, 32: 4096, 16: 32768}[precision]
+    groups = f1 / (per_mfma * 32.0 * 2000 * 4)
+    assert groups == int(groups) and groups >= 1 and f2 == 2 * f1
+    assert 1.85 < t2 / t1 < 2.15, (t1, t2)
+    assert torch.isfinite(sink[: int(groups) * 256]).all()
+    with pytest.raises(rt.RocmRuntimeError):
+        rt.mfma_probe(8, 1, 10, ops.data_ptr(), sink.data_ptr())
+    with pytest.raises(rt.RocmRuntimeError):
+        rt.mfma_probe(precision, 3, 10, ops.data_ptr(), sink.data_ptr())
+
+
+def test_clock_probe_reports_a_plausible_shader_clock(rt):
+    import torch
+    out = torch.zeros(1, device="cuda")
+    rt.clock_probe(200, out.data_ptr())
+    rt.device_sync()
+    assert 100.0 < float(out.item()) < 3000.0
+    with pytest.raises(rt.RocmRuntimeError):
+        rt.clock_probe(0, out.data_ptr())
