@@ -303,6 +303,13 @@ def main():
             cpu = {"value": round(2 * rows * n * n / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"first {rows} rows of C, fp32 loop nest on the bf16 values (the reference has no bf16 GEMM)"}
         add_kernel("bgemm_4096", "bf16", 2 * n**3, ms, cpu, fn=run)
+        # the same launch on all-zero operands: no data toggling, so the power limit does not bind and the
+        # difference to the figure above is what the limit costs this kernel
+        A.zero_()
+        B.zero_()
+        zero_ms = time_kernel(run, 50, 5)
+        kernels["bgemm_4096"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2), "tflops": round(2 * n**3 / zero_ms / 1e9, 1),
+                                                  "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
         del A, B, Cm
 
     # ---- config 4: attention B8 H16 S2048 D64 bf16 ----------------------------------------
@@ -322,6 +329,12 @@ def main():
             cpu = {"value": round(4 * heads * S * S * D / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"{heads} of the 128 (batch, head) pairs, fp32 loop nests (the reference has no attention)"}
         add_kernel("attention_b8h16s2048d64", "bf16", 4 * Bn * H * S * S * D, ms, cpu, fn=run)
+        for t in (Q, K, V):     # as for the bf16 GEMM: the same launch without data toggling
+            t.zero_()
+        zero_ms = time_kernel(run, 50, 5)
+        kernels["attention_b8h16s2048d64"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2),
+                                                               "tflops": round(4 * Bn * H * S * S * D / zero_ms / 1e9, 1),
+                                                               "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
         del Q, K, V, O
 
     # ---- config 5: conv2d N32 C64->64 56x56 3x3 s1 p1 + bias ------------------------------
