@@ -162,7 +162,17 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
     int rc = ensure_device();
     if (rc) return rc;
     long n16 = bytes / 16;
-    return launch("docc_copy_b128", grid_for(n16), 1, 1, 256, 0, (hipStream_t) stream, src, dst, n16);
+    // a work-group per 1024 vectors; more than 2^31 - 1 work-groups (32 TiB) in launches of that many
+    const long per_launch = 0x7fffffffL;
+    for (long done = 0; done < n16;) {
+        long groups = (n16 - done + 1023) / 1024;
+        if (groups > per_launch) groups = per_launch;
+        const long count = groups * 1024 < n16 - done ? groups * 1024 : n16 - done;
+        rc = launch("docc_copy_b128", (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, (const char*) src + done * 16, (char*) dst + done * 16, count);
+        if (rc) return rc;
+        done += count;
+    }
+    return 0;
 }
 
 int docc_rocm_mfma_probe(docc_rocm_stream_t stream, int precision, int waves_per_simd, int iters, const float* operands,

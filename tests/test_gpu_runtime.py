@@ -185,3 +185,15 @@ def test_clock_probe_reports_a_plausible_shader_clock(rt):
     assert 100.0 < float(out.item()) < 3000.0
     with pytest.raises(rt.RocmRuntimeError):
         rt.clock_probe(0, out.data_ptr())
+
+
+@pytest.mark.parametrize("nbytes", [16, 16 * 1023, 16 * 1024, 16 * 1025, 16 * 777777])
+def test_copy_bytes_moves_exactly_the_bytes_asked_for(rt, nbytes):
+    import torch
+    x = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda")
+    y = torch.zeros(nbytes + 64, dtype=torch.uint8, device="cuda")
+    rt.copy_bytes(nbytes, x.data_ptr(), y.data_ptr())
+    rt.device_sync()
+    assert torch.equal(x, y[:nbytes]) and int(y[nbytes:].sum().item()) == 0
+    with pytest.raises(rt.RocmRuntimeError):
+        rt.copy_bytes(24, x.data_ptr(), y.data_ptr())
