@@ -56,6 +56,8 @@ def parse_args():
     ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the PCIe-inclusive calls through @native")
+    ap.add_argument("--no-zero", action="store_true", help="skip the extra timing of the bf16 kernels on all-zero operands (profiling runs: "
+                                                            "one kind of launch per kernel name)")
     return ap.parse_args()
 
 
@@ -305,11 +307,12 @@ def main():
         add_kernel("bgemm_4096", "bf16", 2 * n**3, ms, cpu, fn=run)
         # the same launch on all-zero operands: no data toggling, so the power limit does not bind and the
         # difference to the figure above is what the limit costs this kernel
-        A.zero_()
-        B.zero_()
-        zero_ms = time_kernel(run, 50, 5)
-        kernels["bgemm_4096"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2), "tflops": round(2 * n**3 / zero_ms / 1e9, 1),
-                                                  "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
+        if not args.no_zero:
+            A.zero_()
+            B.zero_()
+            zero_ms = time_kernel(run, 50, 5)
+            kernels["bgemm_4096"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2), "tflops": round(2 * n**3 / zero_ms / 1e9, 1),
+                                                      "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
         del A, B, Cm
 
     # ---- config 4: attention B8 H16 S2048 D64 bf16 ----------------------------------------
@@ -329,12 +332,13 @@ def main():
             cpu = {"value": round(4 * heads * S * S * D / t / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
                    "sample": f"{heads} of the 128 (batch, head) pairs, fp32 loop nests (the reference has no attention)"}
         add_kernel("attention_b8h16s2048d64", "bf16", 4 * Bn * H * S * S * D, ms, cpu, fn=run)
-        for t in (Q, K, V):     # as for the bf16 GEMM: the same launch without data toggling
-            t.zero_()
-        zero_ms = time_kernel(run, 50, 5)
-        kernels["attention_b8h16s2048d64"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2),
-                                                               "tflops": round(4 * Bn * H * S * S * D / zero_ms / 1e9, 1),
-                                                               "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
+        if not args.no_zero:
+            for t in (Q, K, V):     # as for the bf16 GEMM: the same launch without data toggling
+                t.zero_()
+            zero_ms = time_kernel(run, 50, 5)
+            kernels["attention_b8h16s2048d64"]["zero_operands"] = {"kernel_us": round(zero_ms * 1e3, 2),
+                                                                   "tflops": round(4 * Bn * H * S * S * D / zero_ms / 1e9, 1),
+                                                                   "sustained_clock_ghz": sustained_clock_ghz(run, zero_ms)}
         del Q, K, V, O
 
     # ---- config 5: conv2d N32 C64->64 56x56 3x3 s1 p1 + bias ------------------------------
