@@ -169,7 +169,7 @@ def test_mfma_probe_times_its_loop_and_nothing_else(rt, precision):
     per_mfma = {64: 2048, 32: 4096, 16: 32768}[precision]
     groups = f1 / (per_mfma * 32.0 * 2000 * 4)
     assert groups == int(groups) and groups >= 1 and f2 == 2 * f1
-    assert 1.85 < t2 / t1 < 2.15, (t1, t2)
+    assert 1.75 < t2 / t1 < 2.25, (t1, t2)
     assert torch.isfinite(sink[: int(groups) * 256]).all()
     with pytest.raises(rt.RocmRuntimeError):
         rt.mfma_probe(8, 1, 10, ops.data_ptr(), sink.data_ptr())
