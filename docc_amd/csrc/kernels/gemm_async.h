@@ -11,7 +11,8 @@
 //   - because the LDS position of a granule is fixed by the lane that loads it, rows cannot be
 //     padded; bank conflicts are avoided by XOR-swizzling the granule index with the row
 //     (the lane simply fetches the global granule that belongs in its slot);
-//   - the partial last K-step (and nothing else) goes through registers, masked to zero.
+//   - the partial last K-step is copied the same way: the granules past K fetch the first valid k of their row
+//     (column) instead, and are cleared in LDS once they have landed (one extra barrier per product).
 // Requires 16-byte aligned operands with contiguous extents that are multiples of the vector
 // length (the launcher sends everything else to the gemm_mfma.h kernels).
 #pragma once
@@ -112,26 +113,36 @@ struct AsyncTile {
         for (int i = 0; i < NV; i++) issue_one(stage, i, wave);
     }
 
-    // the partial last K-step through registers: k >= kleft reads as zero
-    __device__ __forceinline__ void copy_tail(T* stage, int kleft, int tid) const {
-        const int wave = tid >> 6, lane = tid & 63;
+    // The partial last K-step: granule i holds k >= kleft when `past(i)` says so. Such a granule is copied from
+    // k = 0 of the step (same row / column, so the address stays inside the operand) and cleared afterwards.
+    __device__ __forceinline__ bool past(int i, int wave, int lane, int kleft, unsigned* back) const {
+        const int g = (i * NW + wave) * 64 + lane;
+        const int row = g / VPR, cv = (g % VPR) ^ swz(row);
+        const bool out = K_ALONG_COLS ? (cv * VEC >= kleft) : (row >= kleft);
+        // bytes from the granule's own position back to k = 0 of the step
+        *back = K_ALONG_COLS ? (unsigned) (cv * VEC * (int) sizeof(T)) : (unsigned) ((long) row * (kstep_bytes / ROWS));
+        return out;
+    }
+    __device__ __forceinline__ void issue_tail(T* stage, int kleft, int wave, int lane) const {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            const int g = (i * NW + wave) * 64 + lane;
-            const int row = g / VPR, cv = (g % VPR) ^ swz(row);
-            vec_t v;
+            unsigned back;
+            const unsigned o = past(i, wave, lane, kleft, &back) ? off[i] - back : off[i];
+            __builtin_amdgcn_global_load_lds((global_ptr_t) (base + o), (lds_ptr_t) (stage + (i * NW + wave) * 64 * VEC), 16, 0, 0);
+        }
+    }
+    __device__ __forceinline__ void clear_tail(T* stage, int kleft, int wave, int lane) const {
+        vec_t z;
 #pragma unroll
-            for (int e = 0; e < VEC; e++) {
-                const bool ok = K_ALONG_COLS ? (cv * VEC + e < kleft) : (row < kleft);
-                v[e] = ok ? reinterpret_cast<const T*>(base + off[i])[e] : (T) 0;
-            }
-            *reinterpret_cast<vec_t*>(stage + g * VEC) = v;
+        for (int e = 0; e < VEC; e++) z[e] = (T) 0;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            unsigned back;
+            if (past(i, wave, lane, kleft, &back)) *reinterpret_cast<vec_t*>(stage + ((i * NW + wave) * 64 + lane) * VEC) = z;
         }
     }
 };
 
-// SPREAD: the copies that refill a stage are dealt over the MFMAs of a whole K-step instead of being issued in
-// one run behind the barrier (needs three stages or more; see the pipeline comment in run()).
 template <typename T, int BM, int BN, int BK, int WM, int WN, int STAGES, bool TA, bool TB, bool SPREAD = false>
 struct AsyncGemmKernel {
     typedef AsyncTraits<T> X;
@@ -274,12 +285,24 @@ struct AsyncGemmKernel {
                 ta.issue(st, wave);
                 tb.issue(st + ATile::ELEMS, wave);
             } else {
-                ta.copy_tail(st, kleft, tid);
-                tb.copy_tail(st + ATile::ELEMS, kleft, tid);
+                ta.issue_tail(st, kleft, wave, lane);
+                tb.issue_tail(st + ATile::ELEMS, kleft, wave, lane);
             }
         };
         // step kt has landed once at most the loads of the STAGES-2 newer full steps are outstanding;
         // near the end fewer newer steps exist, so everything is awaited
+        // after the barrier that puts step kt into every wave's view: the partial last step has what lies past K
+        // cleared (every lane clears the granules it copied itself, which its own wait has seen land)
+        auto clear_if_tail = [&](int kt) {
+            if (kleft > 0 && kt == full) {
+                T* st = stage_of(kt);
+                ta.clear_tail(st, kleft, wave, lane);
+                tb.clear_tail(st + ATile::ELEMS, kleft, wave, lane);
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
+        };
         auto arrive = [&](int kt) {
             if (kt + STAGES - 2 < full) {
                 asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((STAGES - 2) * LOADS_PER_STEP) : "memory");
@@ -288,6 +311,7 @@ struct AsyncGemmKernel {
             }
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            clear_if_tail(kt);
         };
 #pragma unroll
         for (int s = 0; s < STAGES - 1; s++)
@@ -386,7 +410,7 @@ struct AsyncGemmKernel {
                 ta.advance();
                 tb.advance();
             } else if (MODE == 1) {
-                if (kt + STAGES - 1 < ksteps) fill(kt + STAGES - 1);    // the K tail, through registers
+                if (kt + STAGES - 1 < ksteps) fill(kt + STAGES - 1);    // the K tail
             }
             auto copies = [&](int slot) {
                 if (MODE != 0) return;
@@ -420,6 +444,7 @@ struct AsyncGemmKernel {
                     }
                     __builtin_amdgcn_s_barrier();
                     asm volatile("" ::: "memory");
+                    if (MODE != 0) clear_if_tail(kt + 1);
                     const T* nst = stage_of(kt + 1);
 #pragma unroll
                     for (int n = 1; n < NM; n++) {
