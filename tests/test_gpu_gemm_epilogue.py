@@ -101,3 +101,22 @@ def test_epilogue_on_the_benchmark_shapes_and_padded_c(rt):
         rt.gemm_epilogue("d", m, 64, k, 1.0, a2.data_ptr(), k, b2.data_ptr(), 64, 0.0, c2.data_ptr(), ldc, bias2.data_ptr(), "tanh")
     with pytest.raises(RocmRuntimeError):       # an empty product with an epilogue goes through the elementwise kernel: contiguous C only
         rt.gemm_epilogue("d", m, 64, 0, 1.0, a2.data_ptr(), k, b2.data_ptr(), 64, 0.0, c2.data_ptr(), ldc, bias2.data_ptr(), "relu")
+
+
+def test_bf16_epilogue_on_the_large_tile(rt):
+    """A product large enough for the 256x256 tile (the kernel that deals its copies over the K-step), with a
+    K tail: bias and ReLU in the store give the bits of the separate nodes."""
+    m, n, k = 4096, 3072, 264
+    g = torch.Generator(device="cuda").manual_seed(5)
+    a = (torch.randn(m, k, device="cuda", generator=g) / 8).bfloat16()
+    b = (torch.randn(k, n, device="cuda", generator=g) / 8).bfloat16()
+    bias = torch.randn(n, device="cuda", generator=g)
+    c0 = torch.randn(m, n, device="cuda", generator=g)
+    fused = c0.clone()
+    rt.gemm_epilogue("b", m, n, k, 1.5, a.data_ptr(), k, b.data_ptr(), n, -0.75, fused.data_ptr(), n, bias.data_ptr(), "relu")
+    plain = c0.clone()
+    rt.bf16gemm_f32(m, n, k, 1.5, a.data_ptr(), k, b.data_ptr(), n, -0.75, plain.data_ptr(), n)
+    torch.cuda.synchronize()
+    assert torch.equal(fused, torch.relu(plain + bias))
+    ref = 1.5 * (a[:64].double() @ b.double()) - 0.75 * c0[:64].double()
+    assert ((plain[:64].double() - ref).abs().max() / ref.abs().max()).item() <= 1e-5
