@@ -22,7 +22,11 @@
 // reference's CUDA target instead prints a kernel per Map nest (opt/src/targets/cuda/codegen/
 // cuda_map_dispatcher.cpp:42-168); here the kernels exist already, so the nest is matched, not compiled.
 // A scalar stored through an assign tasklet (the scalar form of the return copy) becomes an ml::Fill of one
-// element. Other loops, tasklets and branches have no lowering and are refused with the element named.
+// element. The expansion of a reduce node (reduce_node.cpp:186-330: a nest that stores the identity, then maps
+// around fors whose body accumulates onto the result) is folded back into ml::Sum / ml::Max / ml::Min, and a copy
+// whose source some loops do not index (broadcast_node.cpp:110-187) into ml::Broadcast, so that an expanded softmax
+// arrives as the seven nodes the softmax pattern pass knows. Other loops, tasklets and branches have no lowering
+// and are refused with the element named.
 #include <algorithm>
 #include <cctype>
 #include <map>
@@ -224,6 +228,10 @@ struct OperandWalk {
     bool scalar = false;               // a constant or a scalar container
     Value binding;                     // {"data": ...} or {"constant": ..., "type": ...}
     std::vector<int> order;            // loop indices, outermost dimension first
+    std::vector<int> missing;          // loops of the nest that do not index the operand (a reduced or a repeated extent)
+    int units = 0;                     // dimensions indexed by the constant 0 (extent 1: a kept or a repeated dimension)
+    bool partial() const { return !missing.empty() || units > 0; }
+    bool uses(int loop) const { return std::find(order.begin(), order.end(), loop) != order.end(); }
 };
 
 struct Import {
@@ -436,7 +444,12 @@ struct Import {
             if (const Value* off = type.find("offset"))
                 if (strip(off->as_expression()) != "0") return false;
             for (size_t d = 0; d < subset.size(); d++) {
-                const int l = loop_of(strip(subset[d].as_expression()));
+                const std::string index = strip(subset[d].as_expression());
+                if (index == "0") {   // a dimension of extent 1 (a reduced dimension that was kept, or one that is repeated)
+                    walk->units++;
+                    continue;
+                }
+                const int l = loop_of(index);
                 Term st;
                 if (l < 0 || seen[l] || !parse_term(tstrides[d].as_expression(), &st)) return false;
                 seen[l] = true;
@@ -465,12 +478,16 @@ struct Import {
         } else {
             return false;
         }
-        for (bool v : seen)
-            if (!v) return false;   // a repeated (broadcast) operand: not matched
+        // loops that do not index the operand: the callers that know reductions and broadcasts look at `missing`
+        std::vector<bool> used(loops.size(), false);
+        for (size_t l = 0; l < loops.size(); l++)
+            if (!seen[l]) {
+                walk->missing.push_back((int) l);
+                used[l] = true;
+            }
         // innermost: stride 1; then the loop whose stride is the product of the extents found so far; ...
         std::vector<int> inner_first;
         Term expect;
-        std::vector<bool> used(loops.size(), false);
         for (size_t n = 0; n < loops.size(); n++) {
             int found = -1;
             for (size_t l = 0; l < loops.size(); l++)
@@ -626,6 +643,118 @@ struct Import {
             return b;
         };
         if (out.scalar && !out_is_pointer) refuse(block, "a scalar computed by a tasklet");
+
+        // ---- reductions and repeated operands (ReduceNode::expand, reduce_node.cpp:122-345; BroadcastNode::expand,
+        // broadcast_node.cpp:110-187). A reduction is a binary operation whose second operand is its own result,
+        // in a nest some of whose loops do not index the result; the nest before it sets the result to the
+        // operation's identity.
+        auto extents_of = [&](const std::vector<int>& order) {
+            Array shape;
+            for (int l : order) shape.emplace_back(loops[(size_t) l].extent);
+            return shape;
+        };
+        auto subsequence = [](const std::vector<int>& part, const std::vector<int>& whole) {
+            size_t at = 0;
+            for (int l : whole)
+                if (at < part.size() && part[at] == l) at++;
+            return at == part.size();
+        };
+        auto emit = [&](Value node, Array inputs, Array outputs) {
+            node.set("type", "library_node");
+            node.set("element_id", op_id);
+            node.set("implementation_type", "NONE");
+            node.set("side_effect", false);
+            node.set("element_type", types::primitive_type_to_string(element));
+            Value flow;
+            flow.set("library_node", std::move(node));
+            flow.set("inputs", Value(std::move(inputs)));
+            flow.set("outputs", Value(std::move(outputs)));
+            Value b;
+            b.set("type", "block");
+            b.set("element_id", block.at("element_id").as_int());
+            Value dbg = debug_info_of(*op);
+            if (dbg.is_null()) dbg = debug_info_of(block);
+            if (!dbg.is_null()) b.set("debug_info", std::move(dbg));
+            b.set("dataflow", std::move(flow));
+            children.push_back(std::move(b));
+        };
+        if (operands.size() == 2 && !out.scalar && out.partial()) {
+            static const std::map<std::string, std::pair<std::string, int>> reductions = {
+                {"ml::Add", {"ml::Sum", 0}}, {"ml::Maximum", {"ml::Max", -1}}, {"ml::Minimum", {"ml::Min", +1}}};
+            auto red = reductions.find(code);
+            if (red == reductions.end()) refuse(block, "a result that some loops of the nest do not index, under an operation that is not a sum, maximum or minimum");
+            const std::string result = out.binding.at("data").as_string();
+            int acc = -1;
+            for (int k = 0; k < 2; k++) {
+                const OperandWalk& w = in.at(operands[(size_t) k]);
+                if (!w.scalar && w.binding.at("data").as_string() == result && w.order == out.order && w.missing == out.missing) acc = k;
+            }
+            if (acc < 0) refuse(block, "a result that some loops of the nest do not index and that is not accumulated onto");
+            const OperandWalk& x = in.at(operands[(size_t) (1 - acc)]);
+            if (x.scalar || x.partial()) refuse(block, "the operand of a reduction must be indexed by every loop of the nest");
+            if (!subsequence(out.order, x.order)) refuse(block, "operand and result of the reduction walk memory differently");
+            if (out.units != 0 && out.units != (int) out.missing.size()) refuse(block, "some reduced dimensions kept and others dropped");
+            // the nest before this one must have set the result to the identity of the operation
+            const auto identity_ok = [&](const Value& before) {
+                const Value* df = before.find("dataflow");
+                if (!df || !df->contains("library_node")) return false;
+                const Value& n = df->at("library_node");
+                if (n.at("code").as_string() != "ml::Fill") return false;
+                if (df->at("outputs").as_array().at(0).at("data").as_string() != result) return false;
+                const Value& x0 = df->at("inputs").as_array().at(0);
+                if (!x0.contains("constant")) return false;
+                std::string c = x0.at("constant").as_string();
+                c.erase(std::remove_if(c.begin(), c.end(), [](char ch) { return ch == '(' || ch == ')' || ch == ' '; }), c.end());
+                if (red->second.second == 0) {
+                    char* end = nullptr;
+                    const double v = std::strtod(c.c_str(), &end);
+                    return end != c.c_str() && v == 0.0;
+                }
+                const bool negative = !c.empty() && c[0] == '-';
+                const std::string mag = negative ? c.substr(1) : c;
+                return (mag == "INFINITY" || mag == "HUGE_VAL" || mag == "HUGE_VALF") && negative == (red->second.second < 0);
+            };
+            if (children.empty() || !identity_ok(children.back()))
+                refuse(block, "an accumulation whose result the nest before it does not set to the operation's identity");
+            children.pop_back();
+            Array axes;
+            for (size_t d = 0; d < x.order.size(); d++)
+                if (!out.uses(x.order[d])) axes.emplace_back((int64_t) d);
+            Value node{Object{}};
+            node.set("code", red->second.first);
+            node.set("shape", Value(extents_of(x.order)));
+            node.set("axes", Value(std::move(axes)));
+            node.set("keepdims", out.units > 0);
+            Array inputs, outputs;
+            Value bx = x.binding, by = out.binding;
+            bx.set("connector", "X");
+            by.set("connector", "Y");
+            inputs.push_back(std::move(bx));
+            outputs.push_back(std::move(by));
+            emit(std::move(node), std::move(inputs), std::move(outputs));
+            return;
+        }
+        if (code == "assign" && !out.scalar && !out.partial() && !in.at(operands.at(0)).scalar && in.at(operands.at(0)).partial()) {
+            const OperandWalk& x = in.at(operands[0]);
+            if (!subsequence(x.order, out.order)) refuse(block, "operand and result of the repeated copy walk memory differently");
+            Array in_shape;
+            for (int l : out.order) in_shape.emplace_back(x.uses(l) ? loops[(size_t) l].extent : std::string("1"));
+            Value node{Object{}};
+            node.set("code", "ml::Broadcast");
+            node.set("input_shape", Value(std::move(in_shape)));
+            node.set("output_shape", Value(extents_of(out.order)));
+            Array inputs, outputs;
+            Value bx = x.binding, by = out.binding;
+            bx.set("connector", "X");
+            by.set("connector", "Y");
+            inputs.push_back(std::move(bx));
+            outputs.push_back(std::move(by));
+            emit(std::move(node), std::move(inputs), std::move(outputs));
+            return;
+        }
+        if (out.partial()) refuse(block, "a result that some loops of the nest do not index");
+        for (auto& name : operands)
+            if (in.at(name).partial()) refuse(block, "operand '" + in.at(name).binding.at("data").as_string() + "' is not indexed by every loop of the nest");
 
         Value node{Object{}};
         node.set("type", "library_node");

@@ -471,6 +471,36 @@ def test_docc_json_return_copy_and_elementwise_nests_run(tmp_path):
     assert np.array_equal(Tp, Xp.transpose(2, 0, 1)) and np.array_equal(Sp, 2.0 - Xp) and ret[0] == 2.75
 
 
+def test_docc_json_expanded_softmax_runs_as_the_softmax_kernel_and_as_its_pieces(tmp_path):
+    """softmax after docc's tensor-node expansion - thirteen loop nests over six Malloc'ed temporaries - imports as
+    Max / Broadcast / Sub / Exp / Sum / Broadcast / Div; with the pattern pass it is one softmax launch, without it the
+    seven nodes run one by one (reduction nests as reduce kernels, repeated copies as broadcasts). Both against the oracle."""
+    import ctypes
+    import json
+
+    from docc_amd import runtime
+    from docc_amd.sdfg import StructuredSDFG
+    from test_interchange import expanded_softmax_program
+
+    rng = np.random.default_rng(11)
+    r, c = 77, 300
+    X = (rng.standard_normal((r, c)) * 8).astype(np.float32)
+    ref = oracle.softmax(X)
+    for name, options, launcher in (("one", {}, "docc_rocm_softmax_f32"), ("pieces", {"match_softmax": False}, "docc_rocm_reduce")):
+        s = StructuredSDFG.parse(json.dumps(expanded_softmax_program()))
+        s.schedule("rocm", options=options)
+        folder = tmp_path / name
+        lib = s._compile(str(folder))
+        assert launcher in (folder / "softmax_sdfg.cpp").read_text()
+        fn = ctypes.CDLL(lib).softmax_sdfg
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64]
+        fn.restype = None
+        Y = np.full((r, c), np.nan, np.float32)
+        fn(X.ctypes.data, Y.ctypes.data, r, c)
+        assert runtime.take_failure() == (0, "")
+        assert rel_err_max(Y, ref) <= 1e-5, name
+
+
 def test_reductions_over_axes_that_are_not_adjacent():
     """Axes in several blocks: the dispatcher reduces block by block through device temporaries. numpy is the pin
     (a float64 reference; sums in another order than the reference's single loop nest, inside the usual bars)."""

@@ -274,12 +274,14 @@ def docc_nest(ids, kind, loops, op, inputs, output):
     edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": op["element_id"], "dst": nid, "src_conn": conn, "dst_conn": "void",
                   "subset": list(subset), "base_type": base})
     body = {"type": "block", "element_id": ids(), "debug_info": NO_DEBUG, "dataflow": {"type": "dataflow", "nodes": nodes, "edges": edges}}
-    for var, extent in reversed(loops):
+    for loop in reversed(loops):
+        var, extent = loop[0], loop[1]
+        this_kind = loop[2] if len(loop) > 2 else kind      # a loop may name its own kind (maps around fors in a reduction)
         seq = {"type": "sequence", "element_id": ids(), "debug_info": NO_DEBUG, "children": [body],
                "transitions": [{"type": "transition", "element_id": ids(), "debug_info": NO_DEBUG, "assignments": []}]}
-        body = {"type": kind, "element_id": ids(), "debug_info": NO_DEBUG, "indvar": var, "init": "0", "condition": f"{var} < {extent}",
+        body = {"type": this_kind, "element_id": ids(), "debug_info": NO_DEBUG, "indvar": var, "init": "0", "condition": f"{var} < {extent}",
                 "update": f"1 + {var}", "root": seq}
-        if kind == "map":
+        if this_kind == "map":
             body["schedule_type"] = {"value": "SEQUENTIAL", "category": 0, "properties": {}}
     return body
 
@@ -446,4 +448,90 @@ def test_permuted_copies_scalar_operands_and_scalar_stores_import():
         blk = blk["root"]["children"][0]
     blk["dataflow"]["edges"][0]["base_type"]["offset"] = "3"
     with pytest.raises(InvalidSDFGException, match="operand 'X' is not a dense tensor"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+
+
+def reduce_nests(ids, cmath_or_tasklet, identity, x, y, rows, cols, tx, ty):
+    """Max / Sum over the last axis with keepdims as ReduceNode::expand leaves it (reduce_node.cpp:186-330): a nest of
+    maps that stores the identity into every result element, then maps over the kept extent around a for over the
+    reduced one, whose body combines X[i, k] with Y[i, 0] into Y[i, 0]."""
+    init = docc_nest(ids, "map", [("_i_init", rows), ("_i_init_1", "1")], ASSIGN, [("_in", (identity, FLOAT), [], scalar(FLOAT))],
+                     ("_out", y, ["_i_init", "_i_init_1"], ty))
+    body = docc_nest(ids, "map", [("_i", rows, "map"), ("_k", cols, "for")], cmath_or_tasklet,
+                     [("_in1", x, ["_i", "_k"], tx), ("_in2", y, ["_i", "0"], ty)], ("_out", y, ["_i", "0"], ty))
+    return [init, body]
+
+
+def expanded_softmax_program():
+    """`Y = softmax(X, axis=-1)` on fp32 [_s0, _s1] after the tensor nodes were expanded: the seven steps of
+    SoftmaxNode::expand (softmax_node.cpp:142-252) as the loop nests their own expansions leave (reduce_node.cpp,
+    broadcast_node.cpp:110-187, the elementwise maps), over Malloc'ed temporaries."""
+    ids = Ids()
+    names = ("X", "Y", "_max", "_max_b", "_sub", "_exp", "_sum", "_sum_b")
+    containers = {n: pointer(FLOAT) for n in names}
+    for n in ("_s0", "_s1", "_i_init", "_i_init_1", "_i", "_k", "_i0", "_i1"):
+        containers[n] = scalar(INT64)
+    full, red = tensor(FLOAT, ["_s0", "_s1"]), tensor(FLOAT, ["_s0", "1"])
+    both = [("_i0", "_s0"), ("_i1", "_s1")]
+    ij = ["_i0", "_i1"]
+    fmax = {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "fmaxf", "function_stem": "fmax", "primitive_type": FLOAT}
+    expf = {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "expf", "function_stem": "exp", "primitive_type": FLOAT}
+    add = {"type": "tasklet", "code": 2, "inputs": ["_in1", "_in2"], "output": "_out"}
+    sub = {"type": "tasklet", "code": 3, "inputs": ["_in1", "_in2"], "output": "_out"}
+    div = {"type": "tasklet", "code": 5, "inputs": ["_in1", "_in2"], "output": "_out"}
+    children = []
+    for name, size in (("_max", "4*_s0"), ("_max_b", "4*_s0*_s1"), ("_sub", "4*_s0*_s1"), ("_exp", "4*_s0*_s1"), ("_sum", "4*_s0"), ("_sum_b", "4*_s0*_s1")):
+        children.append(docc_block(ids, {"implementation_type": "NONE", "code": "Malloc", "size": size}, [], [("_ret", name)], containers))
+    children += reduce_nests(ids, fmax, "-INFINITY", "X", "_max", "_s0", "_s1", full, red)
+    children.append(docc_nest(ids, "map", both, ASSIGN, [("_in", "_max", ["_i0", "0"], red)], ("_out", "_max_b", ij, full)))
+    children.append(docc_nest(ids, "map", both, sub, [("_in1", "X", ij, full), ("_in2", "_max_b", ij, full)], ("_out", "_sub", ij, full)))
+    children.append(docc_nest(ids, "map", both, expf, [("_in1", "_sub", ij, full)], ("_out", "_exp", ij, full)))
+    children += reduce_nests(ids, add, "0.0", "_exp", "_sum", "_s0", "_s1", full, red)
+    children.append(docc_nest(ids, "map", both, ASSIGN, [("_in", "_sum", ["_i0", "0"], red)], ("_out", "_sum_b", ij, full)))
+    children.append(docc_nest(ids, "map", both, div, [("_in1", "_exp", ij, full), ("_in2", "_sum_b", ij, full)], ("_out", "Y", ij, full)))
+    for name in ("_max", "_max_b", "_sub", "_exp", "_sum", "_sum_b"):
+        children.append(docc_block(ids, {"implementation_type": "NONE", "code": "Free"}, [("_ptr", name)], [("_ptr", name)], containers))
+    children.append({"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG})
+    return docc_sdfg("softmax_sdfg", containers, ["X", "Y", "_s0", "_s1"], children, ids)
+
+
+def test_expanded_softmax_imports_as_its_nodes_and_becomes_one_kernel(tmp_path):
+    s = StructuredSDFG.from_docc_json(json.dumps(expanded_softmax_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["ml::Max", "ml::Broadcast", "ml::Sub", "ml::Exp", "ml::Sum", "ml::Broadcast", "ml::Div"]
+    assert nodes[0]["shape"] == ["_s0", "_s1"] and nodes[0]["axes"] == [1] and nodes[0]["keepdims"] is True
+    assert nodes[4]["axes"] == [1] and nodes[4]["keepdims"] is True
+    assert nodes[1]["input_shape"] == ["_s0", "1"] and nodes[1]["output_shape"] == ["_s0", "_s1"]
+    s.schedule("rocm")
+    assert [n["code"] for n in s.library_nodes() if n["code"].startswith("ml::")] == ["ml::Softmax"]
+    src = Path(s.generate(str(tmp_path))["source"]).read_text()
+    assert "docc_rocm_softmax" in src and "docc_rocm_reduce" not in src
+
+
+def test_accumulations_that_are_not_the_expansion_of_a_reduction_are_refused():
+    prog = expanded_softmax_program()
+    # without the nest that sets the maximum to -INFINITY the accumulation has no known starting value
+    kids = prog["root"]["children"] if "root" in prog else None
+    text = json.dumps(prog)
+    bad = json.loads(text)
+    root = bad["root"]
+    maps = [i for i, c in enumerate(root["children"]) if c["type"] == "map"]
+    del root["children"][maps[0]]
+    del root["transitions"][maps[0]]
+    with pytest.raises(Exception, match="identity"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
+    # a product accumulated over an axis is no node of the target
+    bad = json.loads(text)
+    for c in bad["root"]["children"]:
+        if c["type"] == "map":
+            stack = [c]
+            while stack:
+                e = stack.pop()
+                if isinstance(e, dict):
+                    if e.get("type") == "tasklet" and e.get("code") == 2:
+                        e["code"] = 4
+                    stack.extend(e.values())
+                elif isinstance(e, list):
+                    stack.extend(e)
+    with pytest.raises(Exception, match="sum, maximum or minimum"):
         StructuredSDFG.from_docc_json(json.dumps(bad))
