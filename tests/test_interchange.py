@@ -535,3 +535,57 @@ def test_accumulations_that_are_not_the_expansion_of_a_reduction_are_refused():
                     stack.extend(e)
     with pytest.raises(Exception, match="sum, maximum or minimum"):
         StructuredSDFG.from_docc_json(json.dumps(bad))
+
+
+def test_reduction_nests_over_other_axes_and_index_forms():
+    """The same pair of nests reducing the first axis (result without the reduced dimension), with one linearised index
+    per operand, and over two separated axes of a rank-3 tensor (kept as extents of 1)."""
+    add = {"type": "tasklet", "code": 2, "inputs": ["_in1", "_in2"], "output": "_out"}
+    fmax = {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "fmaxf", "function_stem": "fmax", "primitive_type": FLOAT}
+
+    def program(symbols, nests):
+        ids = Ids()
+        containers = {n: pointer(FLOAT) for n in ("X", "Y")}
+        for n in symbols:
+            containers[n] = scalar(INT64)
+        children = nests(ids) + [{"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG}]
+        return docc_sdfg("r_sdfg", containers, ["X", "Y"] + [n for n in symbols if n.startswith("_s")], children, ids)
+
+    def node(prog):
+        nodes = StructuredSDFG.from_docc_json(json.dumps(prog)).library_nodes()
+        assert len(nodes) == 1
+        return nodes[0]
+
+    def columns(ids):
+        tx, ty = tensor(FLOAT, ["_s0", "_s1"]), tensor(FLOAT, ["_s1"])
+        return [docc_nest(ids, "map", [("_ii", "_s1")], ASSIGN, [("_in", ("0.0", FLOAT), [], scalar(FLOAT))], ("_out", "Y", ["_ii"], ty)),
+                docc_nest(ids, "map", [("_i", "_s1", "map"), ("_k", "_s0", "for")], add,
+                          [("_in1", "X", ["_k", "_i"], tx), ("_in2", "Y", ["_i"], ty)], ("_out", "Y", ["_i"], ty))]
+    n = node(program(["_s0", "_s1", "_ii", "_i", "_k"], columns))
+    assert (n["code"], n["shape"], n["axes"], n["keepdims"]) == ("ml::Sum", ["_s0", "_s1"], [0], False)
+
+    def linear(ids):
+        P = pointer(FLOAT)
+        return [docc_nest(ids, "map", [("_ii", "_s0")], ASSIGN, [("_in", ("-INFINITY", FLOAT), [], scalar(FLOAT))], ("_out", "Y", ["_ii"], P)),
+                docc_nest(ids, "map", [("_i", "_s0", "map"), ("_k", "_s1", "for")], fmax,
+                          [("_in1", "X", ["_k + _i*_s1"], P), ("_in2", "Y", ["_i"], P)], ("_out", "Y", ["_i"], P))]
+    n = node(program(["_s0", "_s1", "_ii", "_i", "_k"], linear))
+    assert (n["code"], n["shape"], n["axes"], n["keepdims"]) == ("ml::Max", ["_s0", "_s1"], [1], False)
+
+    def two_axes(ids):
+        tx, ty = tensor(FLOAT, ["_s0", "_s1", "_s2"]), tensor(FLOAT, ["1", "_s1", "1"])
+        return [docc_nest(ids, "map", [("_a", "1"), ("_ii", "_s1"), ("_c", "1")], ASSIGN, [("_in", ("0.0", FLOAT), [], scalar(FLOAT))],
+                          ("_out", "Y", ["_a", "_ii", "_c"], ty)),
+                docc_nest(ids, "map", [("_i", "_s1", "map"), ("_k", "_s0", "for"), ("_k2", "_s2", "for")], add,
+                          [("_in1", "X", ["_k", "_i", "_k2"], tx), ("_in2", "Y", ["0", "_i", "0"], ty)], ("_out", "Y", ["0", "_i", "0"], ty))]
+    n = node(program(["_s0", "_s1", "_s2", "_ii", "_i", "_k", "_k2", "_a", "_c"], two_axes))
+    assert (n["code"], n["shape"], n["axes"], n["keepdims"]) == ("ml::Sum", ["_s0", "_s1", "_s2"], [0, 2], True)
+
+    # a maximum initialised with the identity of a sum is not the expansion of a node
+    def wrong_identity(ids):
+        P = pointer(FLOAT)
+        return [docc_nest(ids, "map", [("_ii", "_s0")], ASSIGN, [("_in", ("0.0", FLOAT), [], scalar(FLOAT))], ("_out", "Y", ["_ii"], P)),
+                docc_nest(ids, "map", [("_i", "_s0", "map"), ("_k", "_s1", "for")], fmax,
+                          [("_in1", "X", ["_k + _i*_s1"], P), ("_in2", "Y", ["_i"], P)], ("_out", "Y", ["_i"], P))]
+    with pytest.raises(Exception, match="identity"):
+        StructuredSDFG.from_docc_json(json.dumps(program(["_s0", "_s1", "_ii", "_i", "_k"], wrong_identity)))
