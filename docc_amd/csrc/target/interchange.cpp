@@ -417,6 +417,14 @@ struct Import {
         const Value& c = container(data);
         if (c.at("type").as_string() == "scalar") {
             walk->scalar = true;
+            auto known = assigned.find(data);
+            if (known != assigned.end()) {
+                // converted to the element type of the operation that reads it, as the generated C of the reference would
+                Value b{Object{}};
+                b.set("constant", "(" + c_expression(known->second) + ")");
+                b.set("type", types::primitive_type_to_string(element_of(edge.at("base_type"), describe(node))));
+                walk->binding = std::move(b);
+            }
             return true;
         }
         const Value& type = edge.at("base_type");
@@ -815,11 +823,77 @@ struct Import {
         children.push_back(std::move(b));
     }
 
+    // Symbols a transition sets to an expression of the function's scalar arguments (the element count a mean divides
+    // by, mean_node.cpp:96-107): the value is the same wherever the symbol is read, so a read of it is a read of
+    // the expression. Anything else assigned between blocks has no lowering here.
+    std::map<std::string, std::string> assigned;
+    // does `word` occur as an identifier in any string below `v`, other than as the name an access node refers to
+    // or as the left-hand side of an assignment?
+    static bool word_in_expressions(const Value& v, const std::string& word) {
+        if (v.is_string()) {
+            const std::string& text = v.as_string();
+            for (size_t at = text.find(word); at != std::string::npos; at = text.find(word, at + 1)) {
+                const bool left = at == 0 || !(std::isalnum((unsigned char) text[at - 1]) || text[at - 1] == '_');
+                const size_t end = at + word.size();
+                const bool right = end >= text.size() || !(std::isalnum((unsigned char) text[end]) || text[end] == '_');
+                if (left && right) return true;
+            }
+            return false;
+        }
+        if (v.is_array()) {
+            for (auto& e : v.as_array())
+                if (word_in_expressions(e, word)) return true;
+            return false;
+        }
+        if (v.is_object()) {
+            const Value* type = v.find("type");
+            const bool access = type && type->is_string() && type->as_string() == "access_node";
+            for (auto& kv : v.as_object()) {
+                if (access && kv.first == "data") continue;
+                if (kv.first == "symbol" && v.contains("expression")) continue;
+                if (word_in_expressions(kv.second, word)) return true;
+            }
+        }
+        return false;
+    }
+    void note_assignments(const Value& t) {
+        for (auto& a : t.at("assignments").as_array()) {
+            const std::string symbol = strip(a.at("symbol").as_string()), expr = strip(a.at("expression").as_expression());
+            std::string word;
+            auto check = [&]() {
+                if (word.empty() || std::isdigit((unsigned char) word[0])) return;
+                bool argument = false;
+                for (auto& arg : src.at("arguments").as_array()) argument = argument || arg.as_string() == word;
+                if (!argument || container(word).at("type").as_string() != "scalar")
+                    throw InvalidSDFGException(describe(t) + ": symbol '" + symbol + "' is assigned '" + expr +
+                                               "', which is not an expression of the function's scalar arguments");
+            };
+            for (char ch : expr) {
+                if (std::isalnum((unsigned char) ch) || ch == '_') word += ch;
+                else {
+                    check();
+                    word.clear();
+                }
+            }
+            check();
+            if (!src.at("containers").contains(symbol) || container(symbol).at("type").as_string() != "scalar")
+                throw InvalidSDFGException(describe(t) + ": symbol assignments between blocks are not lowered by the rocm target ('" + symbol +
+                                           "' is not a scalar of the function)");
+            // the symbol may be read through access nodes only: inside an index, a bound or a node's attribute it would
+            // have to be a variable of the generated function, which this target does not write assignments for
+            if (word_in_expressions(src.at("root"), symbol))
+                throw InvalidSDFGException(describe(t) + ": symbol assignments between blocks are not lowered by the rocm target ('" + symbol +
+                                           "' is read inside an expression)");
+            auto it = assigned.find(symbol);
+            if (it != assigned.end() && it->second != expr)
+                throw InvalidSDFGException(describe(t) + ": symbol '" + symbol + "' is assigned two different values");
+            assigned[symbol] = expr;
+        }
+    }
+
     void import_sequence(const Value& seq, Array& children, std::string& returned) {
         if (const Value* transitions = seq.find("transitions"))
-            for (auto& t : transitions->as_array())
-                if (!t.at("assignments").as_array().empty())
-                    throw InvalidSDFGException(describe(t) + ": symbol assignments between blocks are not lowered by the rocm target");
+            for (auto& t : transitions->as_array()) note_assignments(t);
         for (auto& child : seq.at("children").as_array()) {
             const std::string kind = child.at("type").as_string();
             if (!returned.empty())

@@ -501,6 +501,29 @@ def test_docc_json_expanded_softmax_runs_as_the_softmax_kernel_and_as_its_pieces
         assert rel_err_max(Y, ref) <= 1e-5, name
 
 
+def test_docc_json_expanded_mean_runs(tmp_path):
+    """A mean after expansion: the sum's two nests, the count set on a transition, the division by it."""
+    import ctypes
+    import json
+
+    from docc_amd import runtime
+    from docc_amd.sdfg import StructuredSDFG
+    from test_interchange import expanded_mean_program
+
+    s = StructuredSDFG.parse(json.dumps(expanded_mean_program()))
+    s.schedule("rocm")
+    fn = ctypes.CDLL(s._compile(str(tmp_path / "mean"))).mean_sdfg
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64]
+    fn.restype = None
+    rng = np.random.default_rng(12)
+    r, c = 130, 517
+    X = rng.standard_normal((r, c)).astype(np.float32)
+    Y = np.full(r, np.nan, np.float32)
+    fn(X.ctypes.data, Y.ctypes.data, r, c)
+    assert runtime.take_failure() == (0, "")
+    assert rel_err_max(Y, X.astype(np.float64).mean(axis=1)) <= 1e-5
+
+
 def test_reductions_over_axes_that_are_not_adjacent():
     """Axes in several blocks: the dispatcher reduces block by block through device temporaries. numpy is the pin
     (a float64 reference; sums in another order than the reference's single loop nest, inside the usual bars)."""

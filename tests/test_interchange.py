@@ -589,3 +589,43 @@ def test_reduction_nests_over_other_axes_and_index_forms():
                           [("_in1", "X", ["_k + _i*_s1"], P), ("_in2", "Y", ["_i"], P)], ("_out", "Y", ["_i"], P))]
     with pytest.raises(Exception, match="identity"):
         StructuredSDFG.from_docc_json(json.dumps(program(["_s0", "_s1", "_ii", "_i", "_k"], wrong_identity)))
+
+
+def expanded_mean_program():
+    """`Y = mean(X, axis=1)` on fp32 [_s0, _s1] after expansion (mean_node.cpp:24-125): the two nests of the sum, an empty
+    block whose transition sets `_mean_count = _s1`, and the map that divides the sums by that count."""
+    ids = Ids()
+    containers = {n: pointer(FLOAT) for n in ("X", "Y")}
+    for n in ("_s0", "_s1", "_ii", "_i", "_k", "_j", "_mean_count"):
+        containers[n] = scalar(INT64)
+    tx, ty = tensor(FLOAT, ["_s0", "_s1"]), tensor(FLOAT, ["_s0"])
+    add = {"type": "tasklet", "code": 2, "inputs": ["_in1", "_in2"], "output": "_out"}
+    div = {"type": "tasklet", "code": 5, "inputs": ["_in1", "_in2"], "output": "_out"}
+    children = [
+        docc_nest(ids, "map", [("_ii", "_s0")], ASSIGN, [("_in", ("0.0", FLOAT), [], scalar(FLOAT))], ("_out", "Y", ["_ii"], ty)),
+        docc_nest(ids, "map", [("_i", "_s0", "map"), ("_k", "_s1", "for")], add,
+                  [("_in1", "X", ["_i", "_k"], tx), ("_in2", "Y", ["_i"], ty)], ("_out", "Y", ["_i"], ty)),
+        {"type": "block", "element_id": ids(), "debug_info": NO_DEBUG, "dataflow": {"type": "dataflow", "nodes": [], "edges": []}},
+        docc_nest(ids, "map", [("_j", "_s0")], div, [("_in1", "Y", ["_j"], ty), ("_in2", "_mean_count", [], tensor(FLOAT, []))],
+                  ("_out", "Y", ["_j"], ty)),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    prog = docc_sdfg("mean_sdfg", containers, ["X", "Y", "_s0", "_s1"], children, ids)
+    prog["root"]["transitions"][2]["assignments"] = [{"symbol": "_mean_count", "expression": "_s1"}]
+    return prog
+
+
+def test_expanded_mean_imports_with_its_count_as_an_expression(tmp_path):
+    s = StructuredSDFG.from_docc_json(json.dumps(expanded_mean_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["ml::Sum", "ml::Div"]
+    div = s._data["root"]["children"][1]["dataflow"]
+    assert div["inputs"][1] == {"constant": "(_s1)", "type": "Float", "connector": "B"}
+    s.schedule("rocm")
+    src = Path(s.generate(str(tmp_path))["source"]).read_text()
+    assert "docc_rocm_reduce" in src and "(_s1)" in src
+    # a symbol set from something that is not an argument has no value the generated function could know
+    bad = expanded_mean_program()
+    bad["root"]["transitions"][2]["assignments"] = [{"symbol": "_mean_count", "expression": "_k + 1"}]
+    with pytest.raises(Exception, match="scalar arguments"):
+        StructuredSDFG.from_docc_json(json.dumps(bad))
