@@ -460,6 +460,10 @@ struct Import {
                 const int l = loop_of(index);
                 Term st;
                 if (l < 0 || seen[l] || !parse_term(tstrides[d].as_expression(), &st)) return false;
+                if (st.coefficient == 0) {   // a repeated dimension of a view (the front end's broadcasting, numpy.py:2679-2705)
+                    walk->units++;
+                    continue;                // the loop stays unseen: it does not index the operand's memory
+                }
                 seen[l] = true;
                 strides[l] = st;
             }
@@ -761,6 +765,45 @@ struct Import {
             return;
         }
         if (out.partial()) refuse(block, "a result that some loops of the nest do not index");
+        if (operands.size() == 2 && !out.scalar) {
+            // an operand of a binary operation that some loops do not move (a view with strides of 0): it is repeated into a
+            // temporary of the result's shape first; the fusion pass folds that copy back into the operation's kernel
+            for (auto& name : operands) {
+                OperandWalk& w = in.at(name);
+                if (w.scalar || !w.partial()) continue;
+                if (!subsequence(w.order, out.order)) refuse(block, "a repeated operand and the result walk memory differently");
+                const std::string temp = "_docc_repeat_" + std::to_string(op_id) + name;
+                std::string bytes = std::to_string(types::primitive_type_size(element));
+                for (int l : out.order) bytes += "*(" + loops[(size_t) l].extent + ")";
+                Value c;
+                c.set("type", "pointer");
+                c.set("element", types::primitive_type_to_string(element));
+                c.set("transient", true);
+                c.set("size", bytes);
+                c.set("storage", "CPU");
+                containers.emplace_back(temp, std::move(c));
+                Array in_shape;
+                for (int l : out.order) in_shape.emplace_back(w.uses(l) ? loops[(size_t) l].extent : std::string("1"));
+                Value node{Object{}};
+                node.set("code", "ml::Broadcast");
+                node.set("input_shape", Value(std::move(in_shape)));
+                node.set("output_shape", Value(extents_of(out.order)));
+                Array inputs, outputs;
+                Value bx = w.binding, by{Object{}};
+                bx.set("connector", "X");
+                by.set("data", temp);
+                by.set("connector", "Y");
+                inputs.push_back(std::move(bx));
+                outputs.push_back(std::move(by));
+                emit(std::move(node), std::move(inputs), std::move(outputs));
+                Value nb{Object{}};
+                nb.set("data", temp);
+                w.binding = std::move(nb);
+                w.order = out.order;
+                w.missing.clear();
+                w.units = 0;
+            }
+        }
         for (auto& name : operands)
             if (in.at(name).partial()) refuse(block, "operand '" + in.at(name).binding.at("data").as_string() + "' is not indexed by every loop of the nest");
 

@@ -480,19 +480,24 @@ def test_docc_json_expanded_softmax_runs_as_the_softmax_kernel_and_as_its_pieces
 
     from docc_amd import runtime
     from docc_amd.sdfg import StructuredSDFG
-    from test_interchange import expanded_softmax_program
+    from test_interchange import expanded_softmax_program, numpy_softmax_expanded_program
 
     rng = np.random.default_rng(11)
     r, c = 77, 300
     X = (rng.standard_normal((r, c)) * 8).astype(np.float32)
     ref = oracle.softmax(X)
-    for name, options, launcher in (("one", {}, "docc_rocm_softmax_f32"), ("pieces", {"match_softmax": False}, "docc_rocm_reduce")):
-        s = StructuredSDFG.parse(json.dumps(expanded_softmax_program()))
+    # the node's own expansion, and the numpy spelling with its stride-0 views of the row maximum and the row sum
+    cases = [("one", expanded_softmax_program, "softmax_sdfg", {}, "docc_rocm_softmax_f32"),
+             ("pieces", expanded_softmax_program, "softmax_sdfg", {"match_softmax": False}, "docc_rocm_reduce"),
+             ("np_one", numpy_softmax_expanded_program, "np_softmax_sdfg", {}, "docc_rocm_softmax_f32"),
+             ("np_pieces", numpy_softmax_expanded_program, "np_softmax_sdfg", {"match_softmax": False}, "docc_rocm_elementwise_fused")]
+    for name, program, function, options, launcher in cases:
+        s = StructuredSDFG.parse(json.dumps(program()))
         s.schedule("rocm", options=options)
         folder = tmp_path / name
         lib = s._compile(str(folder))
-        assert launcher in (folder / "softmax_sdfg.cpp").read_text()
-        fn = ctypes.CDLL(lib).softmax_sdfg
+        assert launcher in (folder / (function + ".cpp")).read_text()
+        fn = getattr(ctypes.CDLL(lib), function)
         fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64]
         fn.restype = None
         Y = np.full((r, c), np.nan, np.float32)

@@ -629,3 +629,48 @@ def test_expanded_mean_imports_with_its_count_as_an_expression(tmp_path):
     bad["root"]["transitions"][2]["assignments"] = [{"symbol": "_mean_count", "expression": "_k + 1"}]
     with pytest.raises(Exception, match="scalar arguments"):
         StructuredSDFG.from_docc_json(json.dumps(bad))
+
+
+def numpy_softmax_expanded_program():
+    """softmax as numpy code spells it - `m = max(x, -1, keepdims)`, `e = exp(x - m)`, `e / sum(e, -1, keepdims)` - after
+    expansion. The front end repeats `m` and the sum along the rows with views whose stride is 0 in the repeated
+    dimension (numpy.py:1193-1232, :2679-2705), so the subtraction and the division index them with both loop variables."""
+    ids = Ids()
+    names = ("X", "Y", "_m", "_d", "_e", "_s")
+    containers = {n: pointer(FLOAT) for n in names}
+    for n in ("_s0", "_s1", "_i_init", "_i_init_1", "_i", "_k", "_i0", "_i1"):
+        containers[n] = scalar(INT64)
+    full, red = tensor(FLOAT, ["_s0", "_s1"]), tensor(FLOAT, ["_s0", "1"])
+    view = tensor(FLOAT, ["_s0", "_s1"], ["1", "0"])          # [rows, 1] seen as [rows, cols]
+    both, ij = [("_i0", "_s0"), ("_i1", "_s1")], ["_i0", "_i1"]
+    fmax = {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "fmaxf", "function_stem": "fmax", "primitive_type": FLOAT}
+    expf = {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": "expf", "function_stem": "exp", "primitive_type": FLOAT}
+    add = {"type": "tasklet", "code": 2, "inputs": ["_in1", "_in2"], "output": "_out"}
+    sub = {"type": "tasklet", "code": 3, "inputs": ["_in1", "_in2"], "output": "_out"}
+    div = {"type": "tasklet", "code": 5, "inputs": ["_in1", "_in2"], "output": "_out"}
+    children = []
+    for name, size in (("_m", "4*_s0"), ("_d", "4*_s0*_s1"), ("_e", "4*_s0*_s1"), ("_s", "4*_s0")):
+        children.append(docc_block(ids, {"implementation_type": "NONE", "code": "Malloc", "size": size}, [], [("_ret", name)], containers))
+    children += reduce_nests(ids, fmax, "-INFINITY", "X", "_m", "_s0", "_s1", full, red)
+    children.append(docc_nest(ids, "map", both, sub, [("_in1", "X", ij, full), ("_in2", "_m", ij, view)], ("_out", "_d", ij, full)))
+    children.append(docc_nest(ids, "map", both, expf, [("_in1", "_d", ij, full)], ("_out", "_e", ij, full)))
+    children += reduce_nests(ids, add, "0.0", "_e", "_s", "_s0", "_s1", full, red)
+    children.append(docc_nest(ids, "map", both, div, [("_in1", "_e", ij, full), ("_in2", "_s", ij, view)], ("_out", "Y", ij, full)))
+    for name in ("_m", "_d", "_e", "_s"):
+        children.append(docc_block(ids, {"implementation_type": "NONE", "code": "Free"}, [("_ptr", name)], [("_ptr", name)], containers))
+    children.append({"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG})
+    return docc_sdfg("np_softmax_sdfg", containers, ["X", "Y", "_s0", "_s1"], children, ids)
+
+
+def test_views_with_a_stride_of_zero_import_as_repeated_operands(tmp_path):
+    s = StructuredSDFG.from_docc_json(json.dumps(numpy_softmax_expanded_program()))
+    nodes = s.library_nodes()
+    assert [n["code"] for n in nodes] == ["ml::Max", "ml::Broadcast", "ml::Sub", "ml::Exp", "ml::Sum", "ml::Broadcast", "ml::Div"]
+    assert nodes[1]["input_shape"] == ["_s0", "1"] and nodes[1]["output_shape"] == ["_s0", "_s1"]
+    s.schedule("rocm", options={"match_softmax": False})
+    codes = [n["code"] for n in s.library_nodes() if n["code"].startswith("ml::")]
+    assert "ml::Broadcast" not in codes                 # folded into the subtraction and the division
+    s = StructuredSDFG.from_docc_json(json.dumps(numpy_softmax_expanded_program()))
+    s.schedule("rocm")
+    assert [n["code"] for n in s.library_nodes() if n["code"].startswith("ml::")] == ["ml::Softmax"]
+    assert "docc_rocm_softmax_f32" in Path(s.generate(str(tmp_path))["source"]).read_text()
