@@ -24,13 +24,17 @@ struct Vec128<double> {
     static constexpr int N = 2;
 };
 
+// Every kernel here is launched with work-groups of kGroup lanes. (blockDim.x would be a load from the hidden
+// kernel arguments that each wave waits for before its first data load: waves that live for one or four vectors feel it.)
+constexpr int kGroup = 256;
+
 // nvec: number of whole 128-bit vectors to process vectorised (0 when an operand is unaligned)
 template <typename T, int OP>
 __device__ __forceinline__ void unary_kernel(const T* X, T* Y, long n, long nvec) {
     typedef typename Vec128<T>::type V;
     constexpr int N = Vec128<T>::N;
-    const long stride = (long) gridDim.x * blockDim.x;
-    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long) gridDim.x * kGroup;
+    const long tid = (long) blockIdx.x * kGroup + threadIdx.x;
     for (long i = tid; i < nvec; i += stride) {
         V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(X) + i);
 #pragma unroll
@@ -45,8 +49,8 @@ __device__ __forceinline__ void binary_kernel(const T* A, const T* B, T* Y, long
                                               long nvec) {
     typedef typename Vec128<T>::type V;
     constexpr int N = Vec128<T>::N;
-    const long stride = (long) gridDim.x * blockDim.x;
-    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long) gridDim.x * kGroup;
+    const long tid = (long) blockIdx.x * kGroup + threadIdx.x;
     for (long i = tid; i < nvec; i += stride) {
         const V a = __builtin_nontemporal_load(reinterpret_cast<const V*>(A) + i);
         const V b = __builtin_nontemporal_load(reinterpret_cast<const V*>(B) + i);
@@ -63,8 +67,8 @@ template <typename T, int OP>
 __device__ __forceinline__ void param_unary_kernel(const T* X, T* Y, long n, long nvec, T alpha, T beta) {
     typedef typename Vec128<T>::type V;
     constexpr int N = Vec128<T>::N;
-    const long stride = (long) gridDim.x * blockDim.x;
-    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long) gridDim.x * kGroup;
+    const long tid = (long) blockIdx.x * kGroup + threadIdx.x;
     for (long i = tid; i < nvec; i += stride) {
         V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(X) + i);
 #pragma unroll
@@ -77,8 +81,8 @@ __device__ __forceinline__ void param_unary_kernel(const T* X, T* Y, long n, lon
 // ml::Fill: every element of Y becomes one value of 1, 2, 4 or 8 bytes (fill_node.cpp:29-41: an assign
 // tasklet from a scalar under the output's Maps). `pattern` holds the value repeated to 16 bytes.
 __device__ __forceinline__ void fill_kernel(unsigned char* Y, long bytes, long nvec, u32x4 pattern) {
-    const long stride = (long) gridDim.x * blockDim.x;
-    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long) gridDim.x * kGroup;
+    const long tid = (long) blockIdx.x * kGroup + threadIdx.x;
     for (long i = tid; i < nvec; i += stride) __builtin_nontemporal_store(pattern, reinterpret_cast<u32x4*>(Y) + i);
     // the tail (and everything, when Y is not 16-byte aligned): byte b of the output is byte b % 16 of the pattern,
     // because the element size divides 16 and Y starts on an element boundary
@@ -93,8 +97,8 @@ template <typename T, int OP, bool LEFT>
 __device__ __forceinline__ void binary_scalar_kernel(const T* A, T b, T* Y, long n, long nvec) {
     typedef typename Vec128<T>::type V;
     constexpr int N = Vec128<T>::N;
-    const long stride = (long) gridDim.x * blockDim.x;
-    const long tid = (long) blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long) gridDim.x * kGroup;
+    const long tid = (long) blockIdx.x * kGroup + threadIdx.x;
     for (long i = tid; i < nvec; i += stride) {
         V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(A) + i);
 #pragma unroll
@@ -120,13 +124,13 @@ struct BroadcastParams {
 template <typename T, int VEC, typename I>
 __device__ __forceinline__ void broadcast_kernel(const T* X, T* Y, const BroadcastParams& p) {
     typedef T V __attribute__((ext_vector_type(VEC)));
-    const I stride = (I) gridDim.x * blockDim.x;
+    const I stride = (I) gridDim.x * kGroup;
     const I nv = (I) (p.n / VEC);
     const int last = p.rank - 1;
     const I inner = (I) p.out_dims[last] / VEC;
     const bool inner_repeats = p.in_strides[last] == 0;
     // position of the lane's vector as (row, column) of the innermost dimension, advanced without divisions
-    I v = (I) blockIdx.x * blockDim.x + threadIdx.x;
+    I v = (I) blockIdx.x * kGroup + threadIdx.x;
     I col = v % inner, row = v / inner;
     const I step_col = stride % inner, step_row = stride / inner;
     for (; v < nv; v += stride) {
@@ -185,13 +189,13 @@ struct FusedParams {
 template <typename T, int VEC, typename I>
 __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const FusedParams& p) {
     typedef T V __attribute__((ext_vector_type(VEC)));
-    const I stride = (I) gridDim.x * blockDim.x;
+    const I stride = (I) gridDim.x * kGroup;
     const I nv = (I) (p.n / VEC);
     const int last = p.rank - 1;
     const I inner = (I) p.dims[last] / VEC;
     const bool a_inner = !p.a_scalar && p.a_strides[last] != 0, b_inner = !p.b_scalar && p.b_strides[last] != 0;
     const bool has_b = p.binary >= 0;
-    I v = (I) blockIdx.x * blockDim.x + threadIdx.x;
+    I v = (I) blockIdx.x * kGroup + threadIdx.x;
     I col = v % inner, row = v / inner;
     const I step_col = stride % inner, step_row = stride / inner;
     for (; v < nv; v += stride) {
@@ -250,6 +254,82 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
         }
         __builtin_nontemporal_store(a, reinterpret_cast<V*>(Y) + v);
     }
+}
+
+// The same chain for outputs that collapse to rows x columns with both operands contiguous or repeated along
+// the columns (address = base + row * s0 + column * s1, s1 0 or 1): the common cases - a bias row, a column of row
+// statistics, two equal shapes, a scalar. A work-group is 2^cx_log2 column vectors wide and 256 >> cx_log2 rows
+// high (narrow rows stack up in a wave, consecutive rows being consecutive memory), and a lane takes the same column
+// vector of four rows, a group height apart: four loads in flight and no index arithmetic beyond an add per row; an
+// operand that does not change from row to row (the bias row) is loaded once. The general kernel above recomputes
+// every operand offset per vector and keeps one load in flight: 47.5 us against 41.0 here for relu(x + bias row) on
+// [8192,4096] fp32. Groups are numbered along the columns first.
+template <typename T, int VEC, bool WIDE>
+__device__ __forceinline__ void fused_rows_body(const T* A, const T* B, T* Y, const FusedParams& p, int cx_log2_arg, uint32_t groups_x) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    constexpr int PER_LANE = 4;
+    // WIDE: a group is one row high, so the row numbers (and a column operand's addresses) are the same for the whole group
+    const int cx_log2 = WIDE ? 8 : cx_log2_arg;
+    const long rows = p.rank == 2 ? p.dims[0] : 1, cols = p.dims[p.rank - 1];
+    const long sa0 = p.rank == 2 ? p.a_strides[0] : 0, sb0 = p.rank == 2 ? p.b_strides[0] : 0;
+    const bool a_cols = !p.a_scalar && p.a_strides[p.rank - 1] != 0, b_cols = !p.b_scalar && p.b_strides[p.rank - 1] != 0;
+    const bool has_b = p.binary >= 0;
+    const int height = 256 >> cx_log2;
+    const uint32_t gy = blockIdx.x / groups_x, gx = blockIdx.x - gy * groups_x;
+    const long cv = ((long) gx << cx_log2) + (threadIdx.x & ((1u << cx_log2) - 1));
+    if (cv * VEC >= cols) return;
+    const long r0 = (long) gy * (PER_LANE * height) + (WIDE ? 0 : threadIdx.x >> cx_log2);
+    auto load = [&](const T* base, bool scalar, double value, bool along_cols, long s0, bool reused, long r) {
+        V v;
+        if (scalar) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) v[e] = (T) value;
+        } else if (along_cols) {
+            const V* q = reinterpret_cast<const V*>(base + r * s0 + cv * VEC);
+            v = reused ? *q : __builtin_nontemporal_load(q);
+        } else {
+            const T x = base[r * s0];
+#pragma unroll
+            for (int e = 0; e < VEC; e++) v[e] = x;
+        }
+        return v;
+    };
+    // an operand that is the same in every row (a scalar, a row vector) is fetched once
+    const bool a_fixed = p.a_scalar || sa0 == 0, b_fixed = !has_b || p.b_scalar || sb0 == 0;
+    V a0 = load(A, p.a_scalar, p.scalar_a, a_cols, 0, true, 0), b0 = a0;
+    if (has_b) b0 = load(B, p.b_scalar, p.scalar_b, b_cols, 0, true, 0);
+    auto finish = [&](V a, V b, long r) {
+        if (has_b) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = apply_binary<T>(p.binary, a[e], b[e]);
+        }
+        for (int k = 0; k < p.npost; k++) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a[e] = apply_unary<T>(p.post[k], a[e]);
+        }
+        __builtin_nontemporal_store(a, reinterpret_cast<V*>(Y + r * cols) + cv);
+    };
+    if (r0 + (PER_LANE - 1) * height < rows) {
+        V a[PER_LANE], b[PER_LANE];
+#pragma unroll
+        for (int u = 0; u < PER_LANE; u++) {
+            a[u] = a_fixed ? a0 : load(A, false, 0, a_cols, sa0, p.a_reused, r0 + u * height);
+            b[u] = b_fixed ? b0 : load(B, false, 0, b_cols, sb0, p.b_reused, r0 + u * height);
+        }
+#pragma unroll
+        for (int u = 0; u < PER_LANE; u++) finish(a[u], b[u], r0 + u * height);
+    } else {
+        for (long r = r0; r < rows; r += height)
+            finish(a_fixed ? a0 : load(A, false, 0, a_cols, sa0, p.a_reused, r), b_fixed ? b0 : load(B, false, 0, b_cols, sb0, p.b_reused, r), r);
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void fused_rows_kernel(const T* A, const T* B, T* Y, const FusedParams& p, int cx_log2, uint32_t groups_x) {
+    if (cx_log2 == 8)
+        fused_rows_body<T, VEC, true>(A, B, Y, p, cx_log2, groups_x);
+    else
+        fused_rows_body<T, VEC, false>(A, B, Y, p, cx_log2, groups_x);
 }
 
 } // namespace docc_k
@@ -333,6 +413,14 @@ DOCC_BROADCAST(f64_v1_i64, double, 1, long)
                                                                            docc_k::FusedParams p) {                         \
         docc_k::fused_kernel<T, VEC, I>(A, B, Y, p);                                                                        \
     }
+extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f32_v4(const float* A, const float* B, float* Y, docc_k::FusedParams p,
+                                                                            int cx_log2, uint32_t groups_x) {
+    docc_k::fused_rows_kernel<float, 4>(A, B, Y, p, cx_log2, groups_x);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f64_v2(const double* A, const double* B, double* Y, docc_k::FusedParams p,
+                                                                            int cx_log2, uint32_t groups_x) {
+    docc_k::fused_rows_kernel<double, 2>(A, B, Y, p, cx_log2, groups_x);
+}
 DOCC_EW_FUSED(f32_v4_i32, float, 4, unsigned)
 DOCC_EW_FUSED(f32_v1_i32, float, 1, unsigned)
 DOCC_EW_FUSED(f32_v4_i64, float, 4, long)

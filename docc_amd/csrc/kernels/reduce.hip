@@ -53,8 +53,8 @@ template <typename T, int OP, int VEC>
 __device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, long nvec) {
     typedef T V __attribute__((ext_vector_type(VEC)));
     const int lane = threadIdx.x & 63;
-    const long waves = (long) gridDim.x * (blockDim.x >> 6);
-    for (long row = (long) blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
+    const long waves = (long) gridDim.x * (256 >> 6);
+    for (long row = (long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
         const T* x = X + row * R;
         T acc[VEC];
 #pragma unroll
@@ -77,8 +77,8 @@ __device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, 
 template <typename T, int OP>
 __device__ __forceinline__ void column_reduce(const T* X, T* Y, long outer, long R, long inner) {
     const long total = outer * inner;
-    const long stride = (long) gridDim.x * blockDim.x;
-    for (long idx = (long) blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const long stride = (long) gridDim.x * 256;
+    for (long idx = (long) blockIdx.x * 256 + threadIdx.x; idx < total; idx += stride) {
         const long o = idx / inner, i = idx % inner;
         const T* x = X + o * R * inner + i;
         T a0 = reduce_identity<OP, T>(), a1 = a0, a2 = a0, a3 = a0;
@@ -107,7 +107,7 @@ __device__ __forceinline__ void column_reduce_partial(void* partials, const T* X
     typedef T V __attribute__((ext_vector_type(VEC)));
     T* P = reinterpret_cast<T*>(partials);
     const long total = outer * inner;
-    const long idx = ((long) blockIdx.x * blockDim.x + threadIdx.x) * VEC;
+    const long idx = ((long) blockIdx.x * 256 + threadIdx.x) * VEC;
     if (idx >= total) return;
     const long r0 = (long) blockIdx.y * chunk, r1 = min(R, r0 + chunk);
     const long o = idx / inner, i = idx % inner;

@@ -69,7 +69,7 @@ __device__ __forceinline__ void softmax_row_wave(const float* __restrict__ x, fl
 template <int NV>
 __device__ __forceinline__ void softmax_wave_kernel(const float* X, float* Y, long rows, int cols) {
     const int lane = threadIdx.x & (kWave - 1);
-    const long row = (long) blockIdx.x * (blockDim.x / kWave) + (threadIdx.x / kWave);
+    const long row = (long) blockIdx.x * (256 / kWave) + (threadIdx.x / kWave);   // launched with 256 lanes; blockDim.x would be a load to wait for
     if (row >= rows) return;
     softmax_row_wave<NV>(X + row * (long) cols, Y + row * (long) cols, cols, lane);
 }

@@ -290,6 +290,29 @@ extern "C" int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precis
                      (!has_b || vector_ok(p.b_scalar, B, p.b_strides[r - 1]));
     const int lanes = vec ? per_vec : 1;
     char name[64];
+    // rows x columns with every operand contiguous or repeated along the columns: the kernel that walks rows
+    // one long run of full and scalar operands is cut into rows of 256 vectors for it
+    const long run_vecs = r == 1 ? p.dims[0] / per_vec : 0;
+    const bool general_only = std::getenv("DOCC_ROCM_EW_FUSED_GENERAL") != nullptr;
+    if (vec && !general_only && run_vecs > 256 && run_vecs % 256 == 0) {
+        p.rank = 2;
+        p.dims[0] = run_vecs / 256, p.dims[1] = 256 * per_vec;
+        p.a_strides[1] = p.a_strides[0], p.a_strides[0] *= p.dims[1];
+        p.b_strides[1] = p.b_strides[0], p.b_strides[0] *= p.dims[1];
+    }
+    if (vec && p.rank <= 2 && !general_only) {
+        const long rows = p.rank == 2 ? p.dims[0] : 1, cvecs = p.dims[p.rank - 1] / per_vec;
+        // a group: 2^cx_log2 column vectors by 256 >> cx_log2 rows, four rows a lane
+        int cx_log2 = 0;
+        while (cx_log2 < 8 && (1L << cx_log2) < cvecs) cx_log2++;
+        const long groups_x = (cvecs + (1L << cx_log2) - 1) >> cx_log2, rows_per_group = 4L * (256 >> cx_log2);
+        const long groups = groups_x * ((rows + rows_per_group - 1) / rows_per_group);
+        // not for widths that leave more than a quarter of the lanes without a column
+        if (groups <= 0x7fffffffL && cvecs * 4 >= (groups_x << cx_log2) * 3) {
+            std::snprintf(name, sizeof(name), "docc_ew_fused_rows_f%d_v%d", precision, per_vec);
+            return launch(name, (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, p, cx_log2, (uint32_t) groups_x);
+        }
+    }
     std::snprintf(name, sizeof(name), "docc_ew_fused_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
     return launch(name, grid_for(n / lanes, kGridFused), 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, p);
 }

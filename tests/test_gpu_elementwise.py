@@ -184,6 +184,16 @@ FUSED_CASES = [
     ((3, 5, 7), (3, 1, 7), (1, 5, 1), "minimum", ["abs"]),               # both operands repeat
     ((2, 3, 2, 3, 2, 4), (2, 3, 2, 3, 2, 4), (4,), "add", ["relu"]),     # rank 6
     ((8192, 4096), (8192, 4096), (4096,), "add", ["relu"]),              # the softmax tensor's shape
+    # rows x columns of whole vectors: the kernel that walks rows (groups 2^k column vectors wide)
+    ((1003, 64), (1003, 64), (64,), "add", ["relu"]),                    # narrow rows stacked in a group, a ragged last group
+    ((1001, 16), (1001, 1), (1001, 16), "sub", ["abs"]),                 # column operand, four column vectors
+    ((4099, 1024), (4099, 1024), (4099, 1024), "mul", ["relu"]),         # equal shapes: collapses to one run, not a multiple of 256 vectors
+    ((4096, 1024), (4096, 1024), (4096, 1024), "mul", ["relu"]),         # equal shapes: one run cut into rows of 256 vectors
+    ((1 << 20,), (1 << 20,), None, "maximum", ["abs", "sqrt"]),          # one run with a scalar
+    ((5, 4096), (4096,), (5, 1), "add", []),                             # fewer rows than a lane takes: row and column operands
+    ((7, 100), (7, 100), (100,), "minimum", ["relu"]),                   # 25 column vectors in a group of 32
+    ((9, 2052), (9, 2052), (2052,), "add", ["relu"]),                    # 513 column vectors: left to the general kernel
+    ((3, 70000), (3, 70000), (3, 1), "mul", []),                         # many groups along the columns
 ]
 
 
@@ -212,6 +222,31 @@ def test_fused_chain_equals_the_separate_nodes_bit_for_bit(rt, dt, case):
                          db.data_ptr() if db is not None else b, b_shape if binary is not None else None, post, out.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(host(out), ref, equal_nan=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_fused_rows_kernel_equals_the_general_kernel_and_works_in_place(rt, dt, monkeypatch):
+    """The kernel for rows x columns against the general one (DOCC_ROCM_EW_FUSED_GENERAL) on the same operands,
+    libm operations included (the same device functions: equal bit for bit), then with the output on the left operand."""
+    rng = np.random.default_rng(31)
+    tdt = torch.float64 if dt == np.float64 else torch.float32
+    for shape, b_shape in [((777, 256), (256,)), ((777, 256), (777, 1)), ((777, 256), (777, 256)), ((130, 24), (24,)), ((65536,), (65536,))]:
+        x, b = dev(rng.standard_normal(shape).astype(dt)), dev(rng.standard_normal(b_shape).astype(dt))
+        outs = []
+        for general in (False, True):
+            if general:
+                monkeypatch.setenv("DOCC_ROCM_EW_FUSED_GENERAL", "1")
+            else:
+                monkeypatch.delenv("DOCC_ROCM_EW_FUSED_GENERAL", raising=False)
+            out = torch.full(shape, float("nan"), device="cuda", dtype=tdt)
+            rt.elementwise_fused(prec(dt), shape, "add", x.data_ptr(), shape, b.data_ptr(), b_shape, ["tanh", "sigmoid"], out.data_ptr())
+            torch.cuda.synchronize()
+            outs.append(host(out))
+        assert np.array_equal(outs[0], outs[1], equal_nan=True), (shape, b_shape)
+        monkeypatch.delenv("DOCC_ROCM_EW_FUSED_GENERAL", raising=False)
+        rt.elementwise_fused(prec(dt), shape, "add", x.data_ptr(), shape, b.data_ptr(), b_shape, ["tanh", "sigmoid"], x.data_ptr())
+        torch.cuda.synchronize()
+        assert np.array_equal(host(x), outs[0], equal_nan=True), (shape, b_shape)
 
 
 def test_fused_chain_with_libm_operations_and_unaligned_operands(rt):
