@@ -11,6 +11,10 @@
 // 16-bit words) in fp32 with an fp32 result, like the bf16 GEMM; when beta == 0, y is not read.
 #include "common.h"
 
+#ifndef DOCC_GEMV_COL_CHAINS
+#define DOCC_GEMV_COL_CHAINS 2
+#endif
+
 namespace docc_k {
 
 template <typename T>
@@ -145,29 +149,40 @@ __device__ __forceinline__ void gemv_cols_partial(void* partials, const In* __re
     if (col >= cols) return;
     const long r0 = (long) blockIdx.y * chunk;
     const long r1 = r0 + chunk < rows ? r0 + chunk : rows;
-    T acc[VEC], acc1[VEC];
+    constexpr int CH = DOCC_GEMV_COL_CHAINS;   // independent chains: that many rows' loads in flight per lane (4 and 8 are slower)
+    T acc[CH][VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; e++) acc[e] = acc1[e] = (T) 0;
+    for (int u = 0; u < CH; u++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[u][e] = (T) 0;
     long r = r0;
     if (VEC > 1) {
-        for (; r + 2 <= r1; r += 2) {   // two independent chains keep the loads in flight
-            const V a0 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + r * ld + col));
-            const V a1 = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + (r + 1) * ld + col));
-            const T w0 = gemv_value<T, In>(x[r * incx]), w1 = gemv_value<T, In>(x[(r + 1) * incx]);
+        for (; r + CH <= r1; r += CH) {
+            V a[CH];
+            T w[CH];
 #pragma unroll
-            for (int e = 0; e < VEC; e++) {
-                acc[e] += w0 * gemv_value<T, In>(a0[e]);
-                acc1[e] += w1 * gemv_value<T, In>(a1[e]);
+            for (int u = 0; u < CH; u++) {
+                a[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(M + (r + u) * ld + col));
+                w[u] = gemv_value<T, In>(x[(r + u) * incx]);
             }
+#pragma unroll
+            for (int u = 0; u < CH; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[u][e] += w[u] * gemv_value<T, In>(a[u][e]);
         }
     }
     for (; r < r1; r++) {
         const T w = gemv_value<T, In>(x[r * incx]);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) acc[e] += w * gemv_value<T, In>(M[r * ld + col + e]);
+        for (int e = 0; e < VEC; e++) acc[0][e] += w * gemv_value<T, In>(M[r * ld + col + e]);
     }
 #pragma unroll
-    for (int e = 0; e < VEC; e++) P[(long) blockIdx.y * cols + col + e] = acc[e] + acc1[e];
+    for (int e = 0; e < VEC; e++) {
+        T sum = acc[0][e];
+#pragma unroll
+        for (int u = 1; u < CH; u++) sum += acc[u][e];
+        P[(long) blockIdx.y * cols + col + e] = sum;
+    }
 }
 
 // The columns form for a few vectors at once (a small batch times a weight matrix stored [k][n], y = x W):

@@ -59,7 +59,9 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
             const bool aligned = (uintptr_t) mat % 16 == 0 && ldm % vecw == 0 && cols % vecw == 0;
             const int lanes = aligned ? vecw : 1;
             const int64_t col_blocks = (cols / lanes + 255) / 256;
-            int64_t slices = (8 * (int64_t) cusm + col_blocks - 1) / col_blocks;
+            // 1.75 work-groups per CU (measured against 0.75 .. 6 per CU on five shapes: 4 x 8192 x 8192 in 46.9 us against
+            // 51.7 with two, 8 x 8192 x 8192 in 93.9 against 102.3, 4 x 4096 x 11008 in 32.9 against 35.3)
+            int64_t slices = (7 * (int64_t) cusm / 4 + col_blocks - 1) / col_blocks;
             if (slices > k / 16) slices = k / 16;
             // the partial sums are written and read back: keep them under a sixteenth of the matrix's bytes
             const int64_t group = nv < 4 ? nv : 4;                                     // vectors per pass
@@ -69,6 +71,10 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
             const int64_t fit = (int64_t) kPartialsBytes / ((int64_t) sizeof(S) * cols * group);
             if (slices > fit) slices = fit;
             if (slices > 256) slices = 256;
+            if (const char* e = std::getenv("DOCC_ROCM_GEMV_SLICES")) {   // tuning: a cap on the slices
+                const int64_t cap = std::atoi(e);
+                if (cap >= 1 && cap < slices) slices = cap;
+            }
             if (slices < 1 || col_blocks > 0x7fffffffLL) return 1;
             const int64_t chunk = (k + slices - 1) / slices;
             slices = (k + chunk - 1) / chunk;
@@ -142,17 +148,23 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         return launch(name, (uint32_t) ((rows + 3) / 4), 1, 1, 256, 0, s, M, (long) ld, x, (long) incx, C, (long) incy, (long) rows,
                       (long) cols, alpha, beta);
     }
-    // columns form: lanes own columns, the rows are sliced so that about eight work-groups per CU share the matrix;
+    // columns form: lanes own columns, the rows are sliced so that 2.6 work-groups per CU share the matrix (measured
+    // on eight shapes from 4096 x 4096 to 28672 x 8192 against 1.5, 2, 3, 4, 6 and 8 per CU: the fastest on every one,
+    // 8192 x 8192 fp32 in 42 us against 50 with eight - fewer slices also leave less for the second launch to add);
     // the slices' sums meet in the stream's partial-results buffer
     if (cols < 256 || rows < 64) return 1;
     const bool aligned = (uintptr_t) M % 16 == 0 && ld % vec == 0 && cols % vec == 0;
     const int lanes = aligned ? vec : 1;
     const int64_t col_blocks = (cols / lanes + 255) / 256;
-    int64_t slices = (8 * (int64_t) cus + col_blocks - 1) / col_blocks;
+    int64_t slices = (21 * (int64_t) cus / 8 + col_blocks - 1) / col_blocks;
     if (slices > rows / 16) slices = rows / 16;
     const int64_t fit = (int64_t) kPartialsBytes / ((int64_t) sizeof(S) * cols);
     if (slices > fit) slices = fit;
     if (slices > 256) slices = 256;
+    if (const char* e = std::getenv("DOCC_ROCM_GEMV_SLICES")) {   // tuning: a cap on the slices
+        const int64_t cap = std::atoi(e);
+        if (cap >= 1 && cap < slices) slices = cap;
+    }
     if (slices < 1) return 1;
     const int64_t chunk = (rows + slices - 1) / slices;
     slices = (rows + chunk - 1) / chunk;
