@@ -43,7 +43,23 @@ __device__ __forceinline__ void gemv_rows(const In* __restrict__ M, long ld, con
         const long nv = k / VEC;
         const V* mv = reinterpret_cast<const V*>(m);
         const V* xv = reinterpret_cast<const V*>(x);
-        for (long c = lane; c < nv; c += 64) {
+        // four loads of the row in flight per lane (one at a time the wave waited out every load: 43.7 us for 8192 x 8192
+        // fp32); the products are added in the order of the plain loop
+        constexpr int U = 4;
+        long c = lane;
+        for (; c + (U - 1) * 64 < nv; c += U * 64) {
+            V a[U], b[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                a[u] = __builtin_nontemporal_load(mv + c + u * 64);
+                b[u] = xv[c + u * 64];
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc += gemv_value<T, In>(a[u][e]) * gemv_value<T, In>(b[u][e]);
+        }
+        for (; c < nv; c += 64) {
             const V a = __builtin_nontemporal_load(mv + c);
             const V b = xv[c];
 #pragma unroll

@@ -59,7 +59,19 @@ __device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, 
         T acc[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; e++) acc[e] = reduce_identity<OP, T>();
-        for (long i = lane; i < nvec; i += kWave) {
+        // four loads in flight per lane, combined in the order of the plain loop
+        constexpr int U = 4;
+        long i = lane;
+        for (; i + (U - 1) * kWave < nvec; i += U * kWave) {
+            V v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) v[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(x) + i + u * kWave);
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[e] = combine<OP>(acc[e], v[u][e]);
+        }
+        for (; i < nvec; i += kWave) {
             const V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(x) + i);
 #pragma unroll
             for (int e = 0; e < VEC; e++) acc[e] = combine<OP>(acc[e], v[e]);
