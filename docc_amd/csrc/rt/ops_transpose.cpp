@@ -1,5 +1,6 @@
 // Launcher for ml::Transpose (see include/docc_rocm_ops.h).
 #include <cstdio>
+#include <cstdlib>
 
 #include "docc_rocm_ops.h"
 #include "rt_state.h"
@@ -133,6 +134,11 @@ extern "C" int docc_rocm_transpose(docc_rocm_stream_t stream, int element_bytes,
     p.rank = k;
     const int64_t blocks = planes * p.tiles_a * p.tiles_b;
     if (blocks > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "transpose: more than 2^31-1 tiles");
+    // 4-byte elements, every extent, stride and address a multiple of four elements: the tile in 128-bit units
+    bool quads = element_bytes == 4 && p.a_ext % 4 == 0 && p.b_ext % 4 == 0 && p.b_in_stride % 4 == 0 && p.a_out_stride % 4 == 0 &&
+                 ((uintptr_t) X | (uintptr_t) Y) % 16 == 0 && !std::getenv("DOCC_ROCM_TRANSPOSE_SCALAR");
+    for (int i = 0; i < p.rank; i++) quads = quads && p.in_stride[i] % 4 == 0 && p.out_stride[i] % 4 == 0;
+    if (quads) return launch("docc_transpose_tile4_b32", (uint32_t) blocks, 1, 1, 256, 0, st, X, Y, p);
     std::snprintf(name, sizeof(name), "docc_transpose_tile_b%d", element_bytes * 8);
     return launch(name, (uint32_t) blocks, 1, 1, 256, 0, st, X, Y, p);
 }

@@ -47,6 +47,8 @@ CASES = [  # shape, perm: tiles with ragged edges, merged axes, unit axes, rank 
     ((8, 16, 200, 64), (0, 2, 1, 3)), ((8, 16, 200, 64), (0, 1, 3, 2)), ((32, 64, 14, 14), (0, 2, 3, 1)), ((32, 14, 14, 64), (0, 3, 1, 2)),
     ((2, 3, 4, 5, 6, 7), (5, 3, 1, 0, 2, 4)), ((2, 3, 4, 5, 6, 7), (0, 1, 2, 3, 4, 5)), ((2, 1, 3, 1, 5), (4, 3, 2, 1, 0)),
     ((5, 6, 7), (1, 0, 2)), ((0, 5), (1, 0)), ((7,), (0,)), ((3, 4, 65, 2), (2, 0, 1, 3)),
+    # everything a multiple of four elements: 4-byte elements take the tile that moves 128-bit units (ragged tiles of 4, 8, 60)
+    ((132, 260), (1, 0)), ((3, 68, 12, 8), (0, 3, 2, 1)), ((4, 200), (1, 0)), ((2, 124, 8, 60), (0, 3, 2, 1)),
 ]
 
 
@@ -55,6 +57,22 @@ def test_transpose_shapes(rt, shape, perm):
     for dt in (np.float32, np.float64, np.int16):
         X = values(shape, dt, len(shape) + sum(perm))
         assert np.array_equal(run_transpose(rt, X, perm), oracle.transpose(X, perm)), dt
+
+
+def test_tile_in_128_bit_units_equals_the_one_element_tile(rt, monkeypatch):
+    """4-byte elements with every extent and stride a multiple of four take another kernel: both against numpy, and a
+    tensor whose address is not a multiple of 16 bytes (the one-element tile again)."""
+    X = values((260, 516), np.float32, 5)
+    want = np.ascontiguousarray(X.T)
+    assert np.array_equal(run_transpose(rt, X, (1, 0)), want)
+    monkeypatch.setenv("DOCC_ROCM_TRANSPOSE_SCALAR", "1")
+    assert np.array_equal(run_transpose(rt, X, (1, 0)), want)
+    monkeypatch.delenv("DOCC_ROCM_TRANSPOSE_SCALAR")
+    buf = dev(np.concatenate([np.zeros(1, np.float32), X.ravel()]))
+    y = torch.empty(X.size, dtype=torch.float32, device="cuda")
+    rt.transpose(4, X.shape, (1, 0), buf.data_ptr() + 4, y.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y).reshape(want.shape), want)
 
 
 def test_transpose_involution_at_full_size_and_errors(rt):
