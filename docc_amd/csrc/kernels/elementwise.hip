@@ -264,15 +264,32 @@ __device__ __forceinline__ void fused_kernel(const T* A, const T* B, T* Y, const
 // operand that does not change from row to row (the bias row) is loaded once. The general kernel above recomputes
 // every operand offset per vector and keeps one load in flight: 47.5 us against 41.0 here for relu(x + bias row) on
 // [8192,4096] fp32. Groups are numbered along the columns first.
+// What the rows kernel needs, at fixed places (a kernel argument indexed by the rank is a second, dependent load,
+// and every wave waited for it before its first data load). Mirrored by the launcher.
+struct FusedRowsParams {
+    long rows, cols;
+    long a_row_stride, b_row_stride;   // in elements; 0: the same in every row
+    int a_along_cols, b_along_cols;    // operand varies along the columns (stride 1) or repeats (stride 0)
+    int binary;                        // BinaryOp or -1
+    int a_scalar, b_scalar;
+    int a_reused, b_reused;
+    int npost;
+    int post[4];
+    double scalar_a, scalar_b;
+    int cx_log2;
+    unsigned groups_x;
+};
+
 template <typename T, int VEC, bool WIDE>
-__device__ __forceinline__ void fused_rows_body(const T* A, const T* B, T* Y, const FusedParams& p, int cx_log2_arg, uint32_t groups_x) {
+__device__ __forceinline__ void fused_rows_body(const T* A, const T* B, T* Y, const FusedRowsParams& p) {
     typedef T V __attribute__((ext_vector_type(VEC)));
     constexpr int PER_LANE = 4;
     // WIDE: a group is one row high, so the row numbers (and a column operand's addresses) are the same for the whole group
-    const int cx_log2 = WIDE ? 8 : cx_log2_arg;
-    const long rows = p.rank == 2 ? p.dims[0] : 1, cols = p.dims[p.rank - 1];
-    const long sa0 = p.rank == 2 ? p.a_strides[0] : 0, sb0 = p.rank == 2 ? p.b_strides[0] : 0;
-    const bool a_cols = !p.a_scalar && p.a_strides[p.rank - 1] != 0, b_cols = !p.b_scalar && p.b_strides[p.rank - 1] != 0;
+    const int cx_log2 = WIDE ? 8 : p.cx_log2;
+    const uint32_t groups_x = p.groups_x;
+    const long rows = p.rows, cols = p.cols;
+    const long sa0 = p.a_row_stride, sb0 = p.b_row_stride;
+    const bool a_cols = !p.a_scalar && p.a_along_cols, b_cols = !p.b_scalar && p.b_along_cols;
     const bool has_b = p.binary >= 0;
     const int height = 256 >> cx_log2;
     const uint32_t gy = blockIdx.x / groups_x, gx = blockIdx.x - gy * groups_x;
@@ -325,11 +342,11 @@ __device__ __forceinline__ void fused_rows_body(const T* A, const T* B, T* Y, co
 }
 
 template <typename T, int VEC>
-__device__ __forceinline__ void fused_rows_kernel(const T* A, const T* B, T* Y, const FusedParams& p, int cx_log2, uint32_t groups_x) {
-    if (cx_log2 == 8)
-        fused_rows_body<T, VEC, true>(A, B, Y, p, cx_log2, groups_x);
+__device__ __forceinline__ void fused_rows_kernel(const T* A, const T* B, T* Y, const FusedRowsParams& p) {
+    if (p.cx_log2 == 8)
+        fused_rows_body<T, VEC, true>(A, B, Y, p);
     else
-        fused_rows_body<T, VEC, false>(A, B, Y, p, cx_log2, groups_x);
+        fused_rows_body<T, VEC, false>(A, B, Y, p);
 }
 
 } // namespace docc_k
@@ -413,13 +430,11 @@ DOCC_BROADCAST(f64_v1_i64, double, 1, long)
                                                                            docc_k::FusedParams p) {                         \
         docc_k::fused_kernel<T, VEC, I>(A, B, Y, p);                                                                        \
     }
-extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f32_v4(const float* A, const float* B, float* Y, docc_k::FusedParams p,
-                                                                            int cx_log2, uint32_t groups_x) {
-    docc_k::fused_rows_kernel<float, 4>(A, B, Y, p, cx_log2, groups_x);
+extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f32_v4(const float* A, const float* B, float* Y, docc_k::FusedRowsParams p) {
+    docc_k::fused_rows_kernel<float, 4>(A, B, Y, p);
 }
-extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f64_v2(const double* A, const double* B, double* Y, docc_k::FusedParams p,
-                                                                            int cx_log2, uint32_t groups_x) {
-    docc_k::fused_rows_kernel<double, 2>(A, B, Y, p, cx_log2, groups_x);
+extern "C" __global__ __launch_bounds__(256) void docc_ew_fused_rows_f64_v2(const double* A, const double* B, double* Y, docc_k::FusedRowsParams p) {
+    docc_k::fused_rows_kernel<double, 2>(A, B, Y, p);
 }
 DOCC_EW_FUSED(f32_v4_i32, float, 4, unsigned)
 DOCC_EW_FUSED(f32_v1_i32, float, 1, unsigned)

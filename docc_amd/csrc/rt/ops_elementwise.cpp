@@ -59,6 +59,21 @@ struct FusedParams {
     int post[4];
 };
 
+// mirrors docc_k::FusedRowsParams
+struct FusedRowsParams {
+    long rows, cols;
+    long a_row_stride, b_row_stride;
+    int a_along_cols, b_along_cols;
+    int binary;
+    int a_scalar, b_scalar;
+    int a_reused, b_reused;
+    int npost;
+    int post[4];
+    double scalar_a, scalar_b;
+    int cx_log2;
+    unsigned groups_x;
+};
+
 // element strides of an operand of shape `in` (extent 1 repeats) inside the output shape
 int operand_strides(const char* what, int rank, const int64_t* in, const int64_t* out, long* strides) {
     long stride = 1;
@@ -309,8 +324,18 @@ extern "C" int docc_rocm_elementwise_fused(docc_rocm_stream_t stream, int precis
         const long groups = groups_x * ((rows + rows_per_group - 1) / rows_per_group);
         // not for widths that leave more than a quarter of the lanes without a column
         if (groups <= 0x7fffffffL && cvecs * 4 >= (groups_x << cx_log2) * 3) {
+            FusedRowsParams q{};
+            const int last = p.rank - 1;
+            q.rows = rows, q.cols = p.dims[last];
+            q.a_row_stride = p.rank == 2 ? p.a_strides[0] : 0, q.b_row_stride = p.rank == 2 ? p.b_strides[0] : 0;
+            q.a_along_cols = p.a_strides[last] != 0, q.b_along_cols = p.b_strides[last] != 0;
+            q.binary = p.binary, q.a_scalar = p.a_scalar, q.b_scalar = p.b_scalar, q.a_reused = p.a_reused, q.b_reused = p.b_reused;
+            q.npost = p.npost;
+            for (int k = 0; k < 4; k++) q.post[k] = p.post[k];
+            q.scalar_a = p.scalar_a, q.scalar_b = p.scalar_b;
+            q.cx_log2 = cx_log2, q.groups_x = (unsigned) groups_x;
             std::snprintf(name, sizeof(name), "docc_ew_fused_rows_f%d_v%d", precision, per_vec);
-            return launch(name, (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, p, cx_log2, (uint32_t) groups_x);
+            return launch(name, (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, A, B, Y, q);
         }
     }
     std::snprintf(name, sizeof(name), "docc_ew_fused_f%d_v%d_i%d", precision, lanes, n < (1L << 31) ? 32 : 64);
