@@ -220,14 +220,21 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 // where group 0 reads tap t; of the middle tap each takes two of the four slices). A wave then carries 6.5 tiles instead
 // of 7, which is what lets 8 strips of 7 rows (one work-group on each of 256 CUs) beat 7 strips of 8 rows on a
 // 56x56 image: both are one round of work-groups, and the round is as long as its waves' MFMA count.
+//
+// NARROW: the shared tile holds at most 16 pixels of the strip (8 of 392 on a 56-wide image). It is then multiplied
+// with the 16x16x4 MFMA - two of them for the wave's 32 output channels and four of a tap's eight channels, half the
+// matrix-pipe time of the 32-pixel form - from operands read as single words: lane l holds the weight of output
+// channel l % 16 and the pixel l % 16 for channel l / 16 (+ 4 for the tap's second half). The two pixel groups still
+// share it by taps, the middle tap by its channel halves.
 #ifndef DOCC_CONV_EARLY_STORE
 #define DOCC_CONV_EARLY_STORE 1
 #endif
 
 namespace docc_k {
 
-template <int KH, int KW, bool SPLIT = false>
+template <int KH, int KW, bool SPLIT = false, bool NARROW = false>
 struct ConvHaloKernel {
+    static_assert(!NARROW || SPLIT, "the narrow tile is the shared tile of a split strip");
     static constexpr int KHW = KH * KW;
     static constexpr int CI = 8;                 // input channels per chunk
     static constexpr int KC = CI * KHW;          // k per chunk
@@ -350,16 +357,43 @@ struct ConvHaloKernel {
         constexpr int TB = KHW > 1 ? KHW - 2 : 0;
         f32x4 a[2], b[2][TN];
         f32x4 a6[2];                                     // SPLIT: the shared tile's own weight operand (its pixels: b[.][TN - 1])
+        float an6[2][2][2], bn6[2][2];                   // NARROW: weights [operand set][channel tile of 16][half of the tap], pixels [set][half]
+        f32x4 accn[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};   // NARROW: the shared tile, 16 channels x 16 pixels each
+        // NARROW: first pixel of the shared tile for this lane (lane % 16), as a patch offset, and the lane's channel of four
+        int boffn = 0;
+        if constexpr (NARROW) {
+            int q = 2 * TOWN * 32 + (lane & 15);
+            q = q < npix ? q : 0;
+            boffn = ((q / p.OW) * WP + (q % p.OW)) * CI + (lane >> 4);
+        }
         static_assert(!SPLIT || KHW % 2 == 1, "the shared tile is halved in the middle tap");
         // slices of tap t that go into the shared tile (code order; group 1 maps them to the mirrored tap)
         auto shared_slices = [](int t) constexpr { return !SPLIT ? 4 : 4 * t + 4 <= 2 * KHW ? 4 : 4 * t < 2 * KHW ? 2 : 0; };
+        // NARROW: the shared tile's operands of (code-order) tap t; group 1 reads the mirrored tap, of the middle tap each its half
+        auto read_narrow = [&](int base, int t, float (&an)[2][2], float (&bn)[2]) {
+            const int n6 = shared_slices(t);        // 4: both halves of the tap's channels, 2: one half
+            if (n6 == 0) return;
+            const int tt = pg ? KHW - 1 - t : t;                   // wave-uniform
+            const int sh = (pg && n6 == 2) ? 4 : 0;                // the middle tap: group 1 takes its upper four channels
+            const float* arown = lds + base + (ocw * 32 + (lane & 15)) * LDA_S + (lane >> 4) + tt * CI + sh;
+            const float* bnp = lds + base + A_ELEMS + ((tt / KW) * WP + (tt % KW)) * CI + boffn + sh;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                if (h == 1 && n6 == 2) break;
+                an[0][h] = arown[4 * h];
+                an[1][h] = arown[16 * LDA_S + 4 * h];
+                bn[h] = bnp[4 * h];
+            }
+        };
         auto fetch = [&](int base, int t, int to) {
             const float* arow = lds + base + (ocw * 32 + l32) * LDA_S + 4 * g + t * CI;
             a[to] = *reinterpret_cast<const f32x4*>(arow);
             const float* bt = lds + base + A_ELEMS + ((t / KW) * WP + (t % KW)) * CI;     // wave-uniform
 #pragma unroll
             for (int j = 0; j < TOWN; j++) b[to][j] = *reinterpret_cast<const f32x4*>(bt + boff[j]);
-            if constexpr (SPLIT) {
+            if constexpr (NARROW) {
+                read_narrow(base, t, an6[to], bn6[to]);
+            } else if constexpr (SPLIT) {
                 const int n6 = shared_slices(t);
                 if (n6 > 0) {
                     const int tt = pg ? KHW - 1 - t : t;                   // wave-uniform
@@ -384,6 +418,18 @@ struct ConvHaloKernel {
         // end of the region lay these out as "one MFMA, then one LDS read or one LDS write and one
         // load" so that the matrix pipe is fed while the other pipes work.
         float bias_r[16];
+        float biasn[2][4];                               // NARROW: bias of the shared tile's rows (channel tile, accumulator register)
+        auto load_biasn = [&]() {
+            if constexpr (NARROW) {
+#pragma unroll
+                for (int sub = 0; sub < 2; sub++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) {
+                        const int oc = oc0 + ocw * 32 + sub * 16 + 4 * (lane >> 4) + r;
+                        biasn[sub][r] = p.bias ? p.bias[oc < p.OC ? oc : p.OC - 1] : 0.f;
+                    }
+            }
+        };
         auto step = [&](auto par_c, auto has_next_c, int cur, int nxt, int after) {
             constexpr int PAR = decltype(par_c)::value;
             constexpr bool NEXT = decltype(has_next_c)::value;
@@ -394,6 +440,7 @@ struct ConvHaloKernel {
                     const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
                     bias_r[r] = p.bias ? p.bias[oc < p.OC ? oc : p.OC - 1] : 0.f;
                 }
+                load_biasn();
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
@@ -407,12 +454,15 @@ struct ConvHaloKernel {
 #pragma unroll
                     for (int j = 0; j < TN; j++) {
                         if (j < TOWN) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[so][s], b[so][j][s], acc[j], 0, 0, 0);
-                        else if (s < shared_slices(t)) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a6[so][s], b[so][j][s], acc[j], 0, 0, 0);
+                        else if (NARROW) {
+                            // slices 0 .. 3 of the code order stand for (channel tile, half of the tap): halves first
+                            if (s < shared_slices(t)) accn[s & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(an6[so][s & 1][s >> 1], bn6[so][s >> 1], accn[s & 1], 0, 0, 0);
+                        } else if (s < shared_slices(t)) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a6[so][s], b[so][j][s], acc[j], 0, 0, 0);
                     }
                 const int nmfma = 4 * TOWN + (SPLIT ? shared_slices(t) : 0);
                 // LDS reads issued in this region: the next tap's weights, its own tiles' pixels and, if it has any, the shared tile's pair
                 const int tn = t + 1 < KHW ? t + 1 : 0;
-                const int nreads = 1 + TOWN + (SPLIT && shared_slices(tn) > 0 ? 2 : 0);
+                const int nreads = 1 + TOWN + (SPLIT && shared_slices(tn) > 0 ? (NARROW ? 3 : 2) : 0);
                 int writes = 0, loads = 0;
                 if constexpr (NEXT) {
                     const int i0 = t < T0 ? 0 : NSL * (t - T0) / (TB + 1 - T0);
@@ -456,6 +506,7 @@ struct ConvHaloKernel {
                 const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
                 bias_r[r] = p.bias ? p.bias[oc] : 0.f;
             }
+            load_biasn();
             f32x4 aw[KHW];
             const float* arow = lds + cur + (ocw * 32 + l32) * LDA_S + 4 * g;
             aw[0] = a[SO];
@@ -508,6 +559,14 @@ struct ConvHaloKernel {
 #pragma unroll
                         for (int u = 0; u < group_size(gi + 1); u++) bb[u][1] = bread(group_first(gi + 1) + u, 1);
                     }
+                    if constexpr (NARROW) {
+                        if (gi == 1 && t == 1) {
+                            // have the shared tile's bias in registers now, where the first stores wait for theirs: met for
+                            // the first time at the end, its loads would be waited for together with every store before
+#pragma unroll
+                            for (int k = 0; k < 8; k++) asm volatile("" ::"v"(biasn[k / 4][k % 4]));
+                        }
+                    }
                     // a region per slice pins the order: the tiles take turns, the stores sit between their MFMAs
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -520,7 +579,25 @@ struct ConvHaloKernel {
                     }
                 }
             }
-            if constexpr (SPLIT) {
+            if constexpr (NARROW) {
+                // the shared tile in its narrow form: this group's half of the chunk's taps, under them the store of the last own tiles
+                float anl[2][2][2], bnl[2][2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) anl[0][0][h] = an6[SO][0][h], anl[0][1][h] = an6[SO][1][h], bnl[0][h] = bn6[SO][h];
+                constexpr int NT6 = (KHW + 1) / 2;
+#pragma unroll
+                for (int t = 0; t < NT6; t++) {
+                    if (t + 1 < NT6) read_narrow(cur, t + 1, anl[(t + 1) & 1], bnl[(t + 1) & 1]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        if (s < shared_slices(t))
+                            accn[s & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(anl[t & 1][s & 1][s >> 1], bnl[t & 1][s >> 1], accn[s & 1], 0, 0, 0);
+                        store_part(NG - 1, t, s, NT6);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            } else if constexpr (SPLIT) {
                 // the shared tile: this group's half of the chunk's slices, under them the store of the last own tile
                 auto read6 = [&](int t, f32x4& av, f32x4& bv) {
                     const int n6 = shared_slices(t);
@@ -595,7 +672,10 @@ struct ConvHaloKernel {
         // joined, the bias registers would be waited for as loads that may still be in flight, and that wait would
         // also sit out every store issued before it.
         auto bias_shared_tile = [&]() {
-            if constexpr (SPLIT) {
+            if constexpr (NARROW) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) accn[k / 4][k % 4] += pg == 0 ? biasn[k / 4][k % 4] : 0.f;
+            } else if constexpr (SPLIT) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[TN - 1][r] += pg == 0 ? bias_r[r] : 0.f;
             }
@@ -644,7 +724,28 @@ struct ConvHaloKernel {
                 last_chunk(Par0{});
             }
         }
-        if constexpr (SPLIT) {
+        if constexpr (NARROW) {
+            // the two halves of the shared tile meet in LDS, [channel tile of 32][accumulator register][lane]; group 0 stores the sum
+            __syncthreads();
+            float* xch = lds + ocw * (8 * 64);
+            if (pg == 1) {
+#pragma unroll
+                for (int k = 0; k < 8; k++) xch[k * 64 + lane] = accn[k / 4][k % 4];
+            }
+            __syncthreads();
+            if (pg == 0) {
+                const int q = 2 * TOWN * 32 + (lane & 15);
+                const int oh = oh0 + q / p.OW, ow = q % p.OW;
+                if (q < npix && oh < p.OH) {
+                    float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        const int oc = oc0 + ocw * 32 + (k / 4) * 16 + 4 * (lane >> 4) + k % 4;
+                        if (oc < p.OC) ybase[(long) oc * p.OH * p.OW] = accn[k / 4][k % 4] + xch[k * 64 + lane];
+                    }
+                }
+            }
+        } else if constexpr (SPLIT) {
             // the two halves of the shared tile meet in LDS, [channel tile][accumulator register][lane]; group 0 stores the sum
             __syncthreads();
             float* xch = lds + ocw * (16 * 64);
@@ -674,6 +775,10 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split(docc_k::ConvParams p, int TH) {
     docc_k::ConvHaloKernel<3, 3, true>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split16(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, true, true>::run(p, TH);
 }
 
 // Explicit im2col for the layers the two kernels above serve badly (small images, many channels): the

@@ -184,7 +184,9 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         // the shorter strips pay about 3.5 % more for halo rows and per-work-group set-up (measured on 32 x 64 x 56 x 56:
         // 7 strips of 8 rows 68.4 us, 8 strips of 7 rows 70.9 us with 7 tiles a wave, 67.0 us with 6.5).
         // DOCC_ROCM_CONV=halo-split / halo-whole force one of the two (tests, tuning).
-        bool split = false;
+        // A thirteenth tile with at most 16 pixels of the strip (8 of 7 x 56) goes through the 16-pixel MFMA at half the
+        // cost: 6.25 tiles a wave (_split16; DOCC_ROCM_CONV=halo-split-wide keeps the 32-pixel form).
+        bool split = false, narrow = false;
         if (KH == 3) {
             int64_t THs = 416 / OW;
             if (THs > OH) THs = OH;
@@ -193,9 +195,11 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
                 if (cus <= 0) cus = 256;
                 const int64_t ocb = (OC + 63) / 64;
                 auto rounds = [&](int64_t th) { return (double) ((N * ((OH + th - 1) / th) * ocb + cus - 1) / cus); };
-                split = rounds(THs) * 6.5 * 1.035 < rounds(TH) * 7.0;
+                narrow = THs * OW <= 12 * 32 + 16;
+                split = rounds(THs) * (narrow ? 6.25 : 6.5) * 1.035 < rounds(TH) * 7.0;
                 if (const char* force = std::getenv("DOCC_ROCM_CONV")) {
-                    if (std::strcmp(force, "halo-split") == 0) split = true;
+                    if (std::strncmp(force, "halo-split", 10) == 0) split = true;
+                    if (std::strcmp(force, "halo-split-wide") == 0) narrow = false;
                     if (std::strcmp(force, "halo-whole") == 0) split = false;
                 }
                 if (split) TH = THs;
@@ -205,7 +209,8 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
         if (PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
-            return launch(KH == 3 ? (split ? "docc_conv2d_f32_halo_3x3_split" : "docc_conv2d_f32_halo_3x3") : "docc_conv2d_f32_halo_1x1",
+            return launch(KH == 3 ? (split ? (narrow ? "docc_conv2d_f32_halo_3x3_split16" : "docc_conv2d_f32_halo_3x3_split") : "docc_conv2d_f32_halo_3x3")
+                                  : "docc_conv2d_f32_halo_1x1",
                           (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
         }
     }

@@ -146,11 +146,12 @@ def run_conv_ws(rt, X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1),
     return host(y), need
 
 
-@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-whole", ""])
+@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-split-wide", "halo-whole", ""])
 @pytest.mark.parametrize("case", CASES)
 def test_conv_every_path_integer_exact(rt, monkeypatch, force, case):
     """Each way to run a layer (forced through DOCC_ROCM_CONV; a path that does not apply falls back; halo-split and
-    halo-whole are the LDS-halo kernel with strips of 13 shared and 14 whole column tiles) and the automatic choice
+    halo-whole are the LDS-halo kernel with strips of 13 shared and 14 whole column tiles, halo-split-wide keeps the
+    shared tile 32 pixels wide where the 16-pixel form would apply) and the automatic choice
     give the oracle's integers."""
     N, C, H, W, OC, KH, KW, stride, pad, dil, use_bias = case
     if force:
