@@ -264,12 +264,15 @@ struct ConvHaloKernel {
         // first pixel of column tile j of this wave
         auto tile_pixel0 = [&](int j) { return j < TOWN ? (pg * TOWN + j) * 32 : 2 * TOWN * 32; };
         int boff[TN];
+        // (filled in below, while the first chunk's loads are under way)
+        auto pixel_offsets = [&]() {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            int q = tile_pixel0(j) + l32;
-            q = q < npix ? q : 0;
-            boff[j] = ((q / p.OW) * WP + (q % p.OW)) * CI + 4 * g;
-        }
+            for (int j = 0; j < TN; j++) {
+                int q = tile_pixel0(j) + l32;
+                q = q < npix ? q : 0;
+                boff[j] = ((q / p.OW) * WP + (q % p.OW)) * CI + 4 * g;
+            }
+        };
 
         // patch pixels this thread moves per chunk: byte offset inside one channel plane (0 when the
         // value is a zero of the padding), validity, and the LDS pixel slot (the spare one for
@@ -361,11 +364,13 @@ struct ConvHaloKernel {
         f32x4 accn[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};   // NARROW: the shared tile, 16 channels x 16 pixels each
         // NARROW: first pixel of the shared tile for this lane (lane % 16), as a patch offset, and the lane's channel of four
         int boffn = 0;
-        if constexpr (NARROW) {
-            int q = 2 * TOWN * 32 + (lane & 15);
-            q = q < npix ? q : 0;
-            boffn = ((q / p.OW) * WP + (q % p.OW)) * CI + (lane >> 4);
-        }
+        auto narrow_pixel_offset = [&]() {
+            if constexpr (NARROW) {
+                int q = 2 * TOWN * 32 + (lane & 15);
+                q = q < npix ? q : 0;
+                boffn = ((q / p.OW) * WP + (q % p.OW)) * CI + (lane >> 4);
+            }
+        };
         static_assert(!SPLIT || KHW % 2 == 1, "the shared tile is halved in the middle tap");
         // slices of tap t that go into the shared tile (code order; group 1 maps them to the mirrored tap)
         auto shared_slices = [](int t) constexpr { return !SPLIT ? 4 : 4 * t + 4 <= 2 * KHW ? 4 : 4 * t < 2 * KHW ? 2 : 0; };
@@ -639,6 +644,17 @@ struct ConvHaloKernel {
 
         const int nch = p.C / CI;
         gload(0);
+        // the index arithmetic nothing needs before the first operand read goes here, under the loads' way to memory and back
+        // (left to the compiler it lands behind the barrier, in front of the first MFMA)
+        pixel_offsets();
+        narrow_pixel_offset();
+        // (an empty asm that takes the value: without it the arithmetic is moved to the first use)
+#pragma unroll
+        for (int j = 0; j < TN; j++) asm volatile("" : "+v"(boff[j]));
+        asm volatile("" : "+v"(boffn));
+        // the accumulators are cleared here as well (112 register writes that otherwise stand between the barrier and the first MFMA)
+#pragma unroll
+        for (int j = 0; j < TN; j++) asm volatile("" : "+a"(acc[j]));
 #pragma unroll
         for (int i = 0; i < NSL; i++) stage_slice(i, 0);
         if (nch > 1) gload(1);
@@ -725,9 +741,10 @@ struct ConvHaloKernel {
             }
         }
         if constexpr (NARROW) {
-            // the two halves of the shared tile meet in LDS, [channel tile of 32][accumulator register][lane]; group 0 stores the sum
-            __syncthreads();
-            float* xch = lds + ocw * (8 * 64);
+            // The two halves of the shared tile meet in LDS, [channel tile of 32][accumulator register][lane]; group 0 stores
+            // the sum. They meet in the ring's third buffer, the one after the last chunk's: what it held was read two chunks
+            // ago, before the barrier every wave has passed to get here, so group 1 can write without another barrier.
+            float* xch = lds + nxt + ocw * (8 * 64);
             if (pg == 1) {
 #pragma unroll
                 for (int k = 0; k < 8; k++) xch[k * 64 + lane] = accn[k / 4][k % 4];
@@ -746,9 +763,8 @@ struct ConvHaloKernel {
                 }
             }
         } else if constexpr (SPLIT) {
-            // the two halves of the shared tile meet in LDS, [channel tile][accumulator register][lane]; group 0 stores the sum
-            __syncthreads();
-            float* xch = lds + ocw * (16 * 64);
+            // the two halves of the shared tile meet in LDS (the ring's free buffer, as above), [channel tile][accumulator register][lane]
+            float* xch = lds + nxt + ocw * (16 * 64);
             if (pg == 1) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) xch[r * 64 + lane] = acc[TN - 1][r];
