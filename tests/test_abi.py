@@ -48,6 +48,23 @@ def test_kernel_images_are_built():
     assert listed == set(build.KERNEL_FAMILIES)
 
 
+def test_kernels_the_launchers_name_are_in_the_images():
+    """Every kernel a launcher names outright (a string literal, not a pattern filled in at run time) is a symbol
+    of one of the built images."""
+    from docc_amd import runtime
+
+    # the images are offload bundles around an ELF object: a kernel's name stands in its string table, NUL-terminated
+    images = b"\0".join(image.read_bytes() for image in sorted(runtime.LIB_DIR.glob("docc_rocm_*.hsaco")))
+    named = set()
+    for src in (ROOT / "docc_amd" / "csrc" / "rt").glob("*.cpp"):
+        named.update(re.findall(r'"(docc_[a-z0-9_]+)"', src.read_text()))
+    named = {n for n in named if not n.startswith("docc_rocm_")}      # entry points of the library itself, not kernels
+    assert {"docc_conv2d_f32_halo_3x3_split16", "docc_transpose_tile4_b32", "docc_copy_b128", "docc_softmax_f32_block8_v2"} <= named
+    missing = sorted(n for n in named if b"\0" + n.encode() + b"\0" not in images)
+    assert not missing, missing
+    assert b"\0docc_conv2d_f32_halo_3x3_split17\0" not in images      # the check can fail
+
+
 def test_runtime_reports_errors_without_a_gpu_or_with_bad_arguments():
     import torch
 
