@@ -1025,6 +1025,9 @@ bool RocmSoftmaxPatternPass::run_pass(builder::StructuredSDFGBuilder& builder, a
             if (!unwritten_between(sdfg, x_name, i_max, at) || (y_name != x_name && !untouched_between(sdfg, y_name, i_max, at))) continue;
             if (y_name == x_name) continue;   // in place: the softmax kernels allow it, the pattern's readers of X in between do not
             auto node = std::make_unique<tensor::SoftmaxNode>(ImplementationType_NONE, shape, axes_sum, div->element());
+            // only a node the mapper takes (RocmLibNodeMapper::try_map): otherwise the seven nodes, which it maps
+            // one by one, would become one that it declines
+            if ((div->element() != types::PrimitiveType::Float && div->element() != types::PrimitiveType::Double) || !node->adjacent_axes()) continue;
             node->set_element_id(div->element_id());
             Block& last = blocks[at];
             last.node = std::move(node);

@@ -932,3 +932,10 @@ def test_softmax_written_in_pieces_becomes_one_node(tmp_path):
     s = softmax_in_pieces("off", [8, 32], [1])
     s.schedule("rocm", options={"match_softmax": False})
     assert "ml::Softmax" not in [n["code"] for n in s.library_nodes()]
+    # reduced axes that are not one block: no softmax kernel takes them, so the seven nodes stay (the mapper takes
+    # each of them: reductions over several blocks run block by block) and the schedule does not fail
+    s = softmax_in_pieces("apart", [4, 5, 6], [0, 2])
+    s.schedule("rocm", options={"require_all_mapped": True})
+    codes = [n["code"] for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert "ml::Softmax" not in codes and "ml::Max" in codes and "ml::Sum" in codes
+    assert all(n["implementation_type"].startswith("ROCM") for n in s.library_nodes() if n["code"] != "ROCMOffloading")
