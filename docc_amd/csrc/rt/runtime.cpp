@@ -61,10 +61,28 @@ std::vector<DeviceState> g_devices;
 // Device blocks that docc_rocm_free keeps for the next docc_rocm_malloc of the same (rounded) size: generated
 // code allocates and frees the same buffers on every call of a compiled function, and hipMalloc / hipFree
 // cost more than a small kernel. Keyed by (device, bytes); `live` remembers the size of what is handed out.
+//
+// A cached block carries the point in a stream behind which its last owner's work is over: docc_rocm_free_async
+// records an event on the stream the owner worked on instead of waiting for the device, and the next owner either
+// continues on that same stream (stream order keeps it behind the old work), makes its own stream wait for the event
+// (docc_rocm_malloc_async), or waits for it on the host (docc_rocm_malloc). docc_rocm_free has waited for the whole
+// device and leaves `pending` false.
+struct CachedBlock {
+    void* ptr = nullptr;
+    hipEvent_t released = nullptr;   // created the first time the block is freed on a stream, reused afterwards
+    hipStream_t stream = nullptr;    // the stream `released` was recorded on
+    bool pending = false;            // `released` may not have happened yet
+};
+
 struct BlockCache {
     std::mutex mutex;
-    std::multimap<std::pair<int, size_t>, void*> free_blocks;
-    std::unordered_map<void*, std::pair<int, size_t>> live;
+    std::multimap<std::pair<int, size_t>, CachedBlock> free_blocks;
+    struct Live {
+        int device;
+        size_t bytes;
+        hipEvent_t released;         // travels with the block so that it is created once
+    };
+    std::unordered_map<void*, Live> live;
     size_t cached_bytes = 0;
     size_t limit = 0;   // bytes the cache may hold; 0 switches it off
 };
@@ -248,6 +266,31 @@ int partials_for(hipStream_t stream, PartialsLease* lease) {
     return 0;
 }
 
+// The stream goes away: its partial-results buffers (one per device it was used on) go with it. A launcher still
+// running on the stream from another thread would be the caller's error, as with hipStreamDestroy itself.
+void release_partials(hipStream_t stream) {
+    std::vector<PartialsSlot*> gone;
+    {
+        std::lock_guard<std::mutex> lock(g_partials_mutex);
+        auto& slots = partials_slots();
+        for (auto it = slots.begin(); it != slots.end();)
+            if (it->first.second == stream) {
+                gone.push_back(it->second);
+                it = slots.erase(it);
+            } else {
+                ++it;
+            }
+    }
+    for (PartialsSlot* slot : gone) {
+        {
+            std::lock_guard<std::mutex> busy(slot->busy);
+            if (slot->ptr) (void) hipFree(slot->ptr);   // waits for the kernels that still use it
+            slot->ptr = nullptr;
+        }
+        delete slot;
+    }
+}
+
 int compute_units() {
     int dev = 0;
     (void) hipGetDevice(&dev);
@@ -287,11 +330,22 @@ void forget_pinned(void* p) {
 }
 
 bool is_pinned(const void* p, size_t bytes) {
-    std::lock_guard<std::mutex> lock(g_pinned_mutex);
-    auto it = g_pinned.upper_bound((uintptr_t) p);
-    if (it == g_pinned.begin()) return false;
-    --it;
-    return (uintptr_t) p + bytes <= it->first + it->second;
+    {
+        std::lock_guard<std::mutex> lock(g_pinned_mutex);
+        auto it = g_pinned.upper_bound((uintptr_t) p);
+        if (it != g_pinned.begin()) {
+            --it;
+            if ((uintptr_t) p + bytes <= it->first + it->second) return true;
+        }
+    }
+    // memory the caller pinned itself (hipHostMalloc, torch's pin_memory): the driver knows it. A pointer it has
+    // never seen makes the query fail, which is the answer "pageable"; the error it leaves is cleared.
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void) hipGetLastError();
+        return false;
+    }
+    return attr.type == hipMemoryTypeHost;
 }
 
 // A fixed pool of threads that copy slices of one chunk; never torn down (the threads sleep on a condition variable
@@ -459,7 +513,11 @@ int docc_rocm_module_get_function(docc_rocm_module_t module, const char* name, d
     return 0;
 }
 
-int docc_rocm_malloc(void** dev_ptr, size_t bytes) {
+namespace {
+
+// `stream` matters only if `ordered`: then a block whose release is still pending is handed out behind that release
+// in `stream`'s own order; otherwise the host waits for the release.
+int pool_malloc(void** dev_ptr, size_t bytes, bool ordered, hipStream_t stream) {
     if (!dev_ptr) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "malloc: null argument");
     *dev_ptr = nullptr;
     if (bytes == 0) return 0;
@@ -469,16 +527,32 @@ int docc_rocm_malloc(void** dev_ptr, size_t bytes) {
     int dev = 0;
     int rc = check(hipGetDevice(&dev), "hipGetDevice");
     if (rc) return rc;
+    CachedBlock got;
     {
         std::lock_guard<std::mutex> lock(c.mutex);
-        auto it = c.free_blocks.find({dev, rounded});
-        if (it != c.free_blocks.end()) {
-            *dev_ptr = it->second;
+        auto range = c.free_blocks.equal_range({dev, rounded});
+        auto pick = range.first;
+        // prefer a block that needs no wait: released on this very stream, or not pending at all
+        for (auto it = range.first; it != range.second; ++it)
+            if (!it->second.pending || (ordered && it->second.stream == stream)) {
+                pick = it;
+                break;
+            }
+        if (pick != range.second) {
+            got = pick->second;
             c.cached_bytes -= rounded;
-            c.free_blocks.erase(it);
-            c.live[*dev_ptr] = {dev, rounded};
-            return 0;
+            c.free_blocks.erase(pick);
+            c.live[got.ptr] = {dev, rounded, got.released};
         }
+    }
+    if (got.ptr) {
+        if (got.pending && !(ordered && got.stream == stream)) {
+            rc = ordered ? check(hipStreamWaitEvent(stream, got.released, 0), "hipStreamWaitEvent(block release)")
+                         : check(hipEventSynchronize(got.released), "hipEventSynchronize(block release)");
+            if (rc) return rc;   // the block stays in `live`; its owner-to-be never sees it
+        }
+        *dev_ptr = got.ptr;
+        return 0;
     }
     hipError_t e = hipMalloc(dev_ptr, rounded);
     if (e == hipErrorOutOfMemory) {   // give the cached blocks back and try once more
@@ -489,41 +563,68 @@ int docc_rocm_malloc(void** dev_ptr, size_t bytes) {
     rc = check(e, "hipMalloc");
     if (rc) return rc;
     std::lock_guard<std::mutex> lock(c.mutex);
-    c.live[*dev_ptr] = {dev, rounded};
+    c.live[*dev_ptr] = {dev, rounded, nullptr};
     return 0;
 }
 
-int docc_rocm_free(void* dev_ptr) {
+int pool_free(void* dev_ptr, bool ordered, hipStream_t stream) {
     if (!dev_ptr) return 0;
     BlockCache& c = block_cache();
-    std::pair<int, size_t> key{0, 0};
+    BlockCache::Live info{0, 0, nullptr};
     bool keep = false;
     {
         std::lock_guard<std::mutex> lock(c.mutex);
         auto it = c.live.find(dev_ptr);
         if (it != c.live.end()) {
-            key = it->second;
+            info = it->second;
             c.live.erase(it);
-            keep = c.limit > 0 && key.second <= c.limit - (c.cached_bytes < c.limit ? c.cached_bytes : c.limit);
+            keep = c.limit > 0 && info.bytes <= c.limit - (c.cached_bytes < c.limit ? c.cached_bytes : c.limit);
         }
     }
-    if (!keep) return check(hipFree(dev_ptr), "hipFree");
-    // hipFree waits for the device before it releases memory; a block that stays allocated must do the same
-    // before another caller can get it
-    int rc = check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    if (!keep) {
+        if (info.released) (void) hipEventDestroy(info.released);
+        return check(hipFree(dev_ptr), "hipFree");   // waits for the device itself
+    }
+    CachedBlock blk;
+    blk.ptr = dev_ptr;
+    blk.released = info.released;
+    int rc = 0;
+    if (ordered) {
+        if (!blk.released) rc = check(hipEventCreateWithFlags(&blk.released, hipEventDisableTiming), "hipEventCreate(block release)");
+        if (!rc) rc = check(hipEventRecord(blk.released, stream), "hipEventRecord(block release)");
+        blk.stream = stream;
+        blk.pending = true;
+    } else {
+        // hipFree waits for the device before it releases memory; a block that stays allocated must do the same
+        // before another caller can get it
+        rc = check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    }
     if (rc) {
+        if (blk.released) (void) hipEventDestroy(blk.released);
         (void) hipFree(dev_ptr);
         return rc;
     }
     std::lock_guard<std::mutex> lock(c.mutex);
-    c.free_blocks.insert({key, dev_ptr});
-    c.cached_bytes += key.second;
+    c.free_blocks.insert({{info.device, info.bytes}, blk});
+    c.cached_bytes += info.bytes;
     return 0;
 }
 
+} // namespace
+
+int docc_rocm_malloc(void** dev_ptr, size_t bytes) { return pool_malloc(dev_ptr, bytes, false, nullptr); }
+
+int docc_rocm_malloc_async(void** dev_ptr, size_t bytes, docc_rocm_stream_t stream) {
+    return pool_malloc(dev_ptr, bytes, true, (hipStream_t) stream);
+}
+
+int docc_rocm_free(void* dev_ptr) { return pool_free(dev_ptr, false, nullptr); }
+
+int docc_rocm_free_async(void* dev_ptr, docc_rocm_stream_t stream) { return pool_free(dev_ptr, true, (hipStream_t) stream); }
+
 int docc_rocm_pool_trim(void) {
     BlockCache& c = block_cache();
-    std::multimap<std::pair<int, size_t>, void*> blocks;
+    std::multimap<std::pair<int, size_t>, CachedBlock> blocks;
     {
         std::lock_guard<std::mutex> lock(c.mutex);
         blocks.swap(c.free_blocks);
@@ -531,7 +632,9 @@ int docc_rocm_pool_trim(void) {
     }
     int rc = 0;
     for (auto& b : blocks) {
-        const int r = check(hipFree(b.second), "hipFree");
+        // hipFree waits for the device, which covers a release that is still pending
+        const int r = check(hipFree(b.second.ptr), "hipFree");
+        if (b.second.released) (void) hipEventDestroy(b.second.released);
         if (r && !rc) rc = r;
     }
     return rc;
@@ -607,6 +710,7 @@ int docc_rocm_stream_create(docc_rocm_stream_t* stream) {
 
 int docc_rocm_stream_destroy(docc_rocm_stream_t stream) {
     if (!stream) return 0;
+    release_partials((hipStream_t) stream);
     return check(hipStreamDestroy((hipStream_t) stream), "hipStreamDestroy");
 }
 

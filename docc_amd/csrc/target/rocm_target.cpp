@@ -70,7 +70,7 @@ void emit_transfers_begin(PrettyPrinter& s, const std::vector<DeviceOperand>& op
     for (auto& op : ops) {
         s << "void *" << op.device << " = nullptr;" << std::endl;
         s << "const size_t " << op.device << "_bytes = (size_t) (" << op.bytes << ");" << std::endl;
-        s << "DOCC_ROCM_CHECK(docc_rocm_malloc(&" << op.device << ", " << op.device << "_bytes));" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_malloc_async(&" << op.device << ", " << op.device << "_bytes, nullptr));" << std::endl;
     }
     for (auto& op : ops)
         if (op.copy_in)
@@ -84,7 +84,7 @@ void emit_transfers_end(PrettyPrinter& s, const std::vector<DeviceOperand>& ops)
             s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_d2h_async(" << op.connector << ", " << op.device << ", " << op.device
               << "_bytes, nullptr));" << std::endl;
     s << "DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
-    for (auto& op : ops) s << "DOCC_ROCM_CHECK(docc_rocm_free(" << op.device << "));" << std::endl;
+    for (auto& op : ops) s << "DOCC_ROCM_CHECK(docc_rocm_free_async(" << op.device << ", nullptr));" << std::endl;
 }
 
 Expression sum_bytes(const std::vector<DeviceOperand>& ops) {
@@ -298,15 +298,12 @@ protected:
         s.setIndent(s.indent() + 4);
         s << "const int64_t __ws_bytes = docc_rocm_conv2d_f32_workspace_bytes(" << dims.str() << ");" << std::endl;
         s << "void *__ws = nullptr;" << std::endl;
-        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc(&__ws, (size_t) __ws_bytes));" << std::endl;
+        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc_async(&__ws, (size_t) __ws_bytes, nullptr));" << std::endl;
         s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32_ws(nullptr, " << dims.str() << ", (const float *) " << name_of("X")
           << ", (const float *) " << name_of("W") << ", "
           << (c.has_bias() ? "(const float *) " + name_of("B") : std::string("nullptr")) << ", (float *) " << name_of("Y")
           << ", __ws, __ws_bytes));" << std::endl;
-        s << "if (__ws) {" << std::endl;
-        s << "    DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
-        s << "    DOCC_ROCM_CHECK(docc_rocm_free(__ws));" << std::endl;
-        s << "}" << std::endl;
+        s << "if (__ws) DOCC_ROCM_CHECK(docc_rocm_free_async(__ws, nullptr));" << std::endl;
         s.setIndent(s.indent() - 4);
         s << "}" << std::endl;
     }
@@ -343,14 +340,11 @@ protected:
         s.setIndent(s.indent() + 4);
         s << "const int64_t __ws_bytes = docc_rocm_attention_bf16_workspace_bytes(" << dims.str() << ", " << out_bf16 << ");" << std::endl;
         s << "void *__ws = nullptr;" << std::endl;
-        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc(&__ws, (size_t) __ws_bytes));" << std::endl;
+        s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc_async(&__ws, (size_t) __ws_bytes, nullptr));" << std::endl;
         s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16_ws(nullptr, " << dims.str() << ", (float) (" << a.scale()
           << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) " << name_of("K") << ", (const uint16_t *) "
           << name_of("V") << ", (void *) " << name_of("O") << ", " << out_bf16 << ", __ws, __ws_bytes));" << std::endl;
-        s << "if (__ws) {" << std::endl;
-        s << "    DOCC_ROCM_CHECK(docc_rocm_stream_sync(nullptr));" << std::endl;
-        s << "    DOCC_ROCM_CHECK(docc_rocm_free(__ws));" << std::endl;
-        s << "}" << std::endl;
+        s << "if (__ws) DOCC_ROCM_CHECK(docc_rocm_free_async(__ws, nullptr));" << std::endl;
         s.setIndent(s.indent() - 4);
         s << "}" << std::endl;
     }
@@ -370,7 +364,7 @@ public:
         // allocate, copy, free; copies are followed by a stream wait because the node is blocking
         if (n.is_alloc()) {
             const std::string dst = n.is_h2d() ? "_dst" : "_ret";
-            s << "DOCC_ROCM_CHECK(docc_rocm_malloc((void **) &" << dst << ", (size_t) (" << size << ")));" << std::endl;
+            s << "DOCC_ROCM_CHECK(docc_rocm_malloc_async((void **) &" << dst << ", (size_t) (" << size << "), nullptr));" << std::endl;
         }
         if (n.is_h2d()) {
             s << "DOCC_ROCM_CHECK(docc_rocm_memcpy_h2d_async(_dst, _src, (size_t) (" << size << "), nullptr));" << std::endl;
@@ -380,7 +374,7 @@ public:
         }
         if (n.is_free()) {
             const std::string ptr = n.is_d2h() ? "_src" : "_ptr";
-            s << "DOCC_ROCM_CHECK(docc_rocm_free(" << ptr << "));" << std::endl;
+            s << "DOCC_ROCM_CHECK(docc_rocm_free_async(" << ptr << ", nullptr));" << std::endl;
         }
     }
 
@@ -649,14 +643,14 @@ protected:
                 const int slot = (int) ((runs.size() - 1 - k) & 1);
                 to = "__docc_part[" + std::to_string(slot) + "]";
                 if (runs.size() - 1 - k < 2)   // a later step reuses the slot: its result is never larger
-                    s << "DOCC_ROCM_CHECK(docc_rocm_malloc(&" << to << ", (size_t) (" << symbolic::mul(symbolic::mul(outer, inner), elem) << ")));" << std::endl;
+                    s << "DOCC_ROCM_CHECK(docc_rocm_malloc_async(&" << to << ", (size_t) (" << symbolic::mul(symbolic::mul(outer, inner), elem) << "), nullptr));" << std::endl;
             }
             call(outer, extent, inner, from, to);
             shape.erase(shape.begin() + (long) lo, shape.begin() + (long) hi + 1);
             from = to;
         }
-        s << "if (__docc_part[0]) DOCC_ROCM_CHECK(docc_rocm_free(__docc_part[0]));" << std::endl;
-        s << "if (__docc_part[1]) DOCC_ROCM_CHECK(docc_rocm_free(__docc_part[1]));" << std::endl;
+        s << "if (__docc_part[0]) DOCC_ROCM_CHECK(docc_rocm_free_async(__docc_part[0], nullptr));" << std::endl;
+        s << "if (__docc_part[1]) DOCC_ROCM_CHECK(docc_rocm_free_async(__docc_part[1], nullptr));" << std::endl;
         s.setIndent(s.indent() - 4);
         s << "}" << std::endl;
     }

@@ -40,6 +40,8 @@ _SIGNATURES = {
     "docc_rocm_module_unload": [_vp],
     "docc_rocm_module_get_function": [_vp, ctypes.c_char_p, ctypes.POINTER(_vp)],
     "docc_rocm_malloc": [ctypes.POINTER(_vp), ctypes.c_size_t],
+    "docc_rocm_malloc_async": [ctypes.POINTER(_vp), ctypes.c_size_t, _vp],
+    "docc_rocm_free_async": [_vp, _vp],
     "docc_rocm_pool_trim": [],
     "docc_rocm_pool_stats": [ctypes.POINTER(ctypes.c_size_t)] * 3,
     "docc_rocm_pool_set_limit": [ctypes.c_size_t],
@@ -172,6 +174,18 @@ def malloc(nbytes: int) -> int:
 
 def free(ptr: int) -> None:
     call("docc_rocm_free", ptr)
+
+
+def malloc_async(nbytes: int, stream: int = 0) -> int:
+    """A block for work on `stream`: one that free_async released on that stream comes back without a wait."""
+    p = _vp()
+    call("docc_rocm_malloc_async", ctypes.byref(p), nbytes, stream)
+    return p.value or 0
+
+
+def free_async(ptr: int, stream: int = 0) -> None:
+    """Returns a block whose uses were all issued on `stream`; does not wait for them."""
+    call("docc_rocm_free_async", ptr, stream)
 
 
 def pool_trim() -> None:

@@ -74,6 +74,16 @@ int docc_rocm_free(void* dev_ptr);
  * same buffers on every call. The cache holds at most DOCC_ROCM_POOL_BYTES bytes (default 4 GiB,
  * 0 = every call goes to hipMalloc / hipFree) and is emptied when hipMalloc runs out of memory.
  * No counterpart in the reference, whose CUDA nodes call cudaMalloc / cudaFree each time. */
+/* Stream-ordered forms, what generated code calls: docc_rocm_free_async does not wait; it records, on `stream`,
+ * the point behind which the block's last use lies (the caller must have issued every use of the block on
+ * `stream`, or have ordered `stream` behind them), and the block goes to the cache at once. The next
+ * docc_rocm_malloc_async on the same stream gets it without any wait, on another stream after that stream has
+ * been made to wait for the recorded point (hipStreamWaitEvent; the new owner must then start using the
+ * block on the stream it named), and a plain docc_rocm_malloc after the host has waited for it. A compiled
+ * function that frees its buffers and is called again therefore never waits for the device on their account.
+ * The counterpart in CUDA terms is cudaMallocAsync / cudaFreeAsync; the reference's nodes use the blocking pair. */
+int docc_rocm_malloc_async(void** dev_ptr, size_t bytes, docc_rocm_stream_t stream);
+int docc_rocm_free_async(void* dev_ptr, docc_rocm_stream_t stream);
 int docc_rocm_pool_trim(void);
 int docc_rocm_pool_stats(size_t* cached_bytes, size_t* cached_blocks, size_t* limit_bytes);
 int docc_rocm_pool_set_limit(size_t limit_bytes);
@@ -95,7 +105,10 @@ int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes
 int docc_rocm_memcpy_d2h_async(void* dst_host, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);
 int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes, docc_rocm_stream_t stream);
 
-/* Streams (default priority only). */
+/* Streams (default priority only). docc_rocm_stream_destroy also releases the 8 MiB of partial results that
+ * the two-launch kernels (sliced softmax, column reductions, column matrix-vector products, dot) keep per
+ * stream; they allocate it with hipMalloc on their first call on a stream, so that first call waits for the
+ * device and cannot be captured into a HIP graph. */
 int docc_rocm_stream_create(docc_rocm_stream_t* stream);
 int docc_rocm_stream_destroy(docc_rocm_stream_t stream);
 int docc_rocm_stream_sync(docc_rocm_stream_t stream);

@@ -88,7 +88,7 @@ def test_runtime_reports_errors_without_a_gpu_or_with_bad_arguments():
     with pytest.raises(runtime.RocmRuntimeError):
         runtime.softmax_f32(4, 4, 16, 16)
     # the failure channel of generated code keeps the first report
-    runtime.lib().docc_rocm_report_failure(b"f", b"docc_rocm_malloc(...)", 2)
+    runtime.lib().docc_rocm_report_failure(b"f", b"docc_rocm_malloc_async(...)", 2)
     runtime.lib().docc_rocm_report_failure(b"g", b"later", 3)
     code, message = runtime.take_failure()
     assert code == 2 and "docc_rocm_malloc" in message

@@ -68,6 +68,100 @@ def test_cached_blocks_hold_no_stale_work(rt):
     assert np.array_equal(out, np.arange(n, dtype=np.float32))
 
 
+def test_blocks_freed_on_a_stream_come_back_in_stream_order(rt):
+    """free_async records the release on the stream and does not wait; the next owner sees the block only behind that
+    release: on the same stream by stream order, on another stream through an event wait, on the host after a wait."""
+    import torch
+    n = 1 << 24
+    src = torch.arange(n, dtype=torch.float32, device="cuda")
+    neg, neg2 = -src, -2 * src
+    expected = np.arange(n, dtype=np.float32)
+    a, b = rt.stream_create(), rt.stream_create()
+    try:
+        torch.cuda.synchronize()
+        rt.pool_trim()
+        # same stream: a chain of kernels into p, release, the block again, its contents are the chain's result
+        p = rt.malloc_async(n * 4, a)
+        for _ in range(8):
+            rt.elementwise_unary("abs", 32, n, neg.data_ptr(), p, stream=a)
+        rt.free_async(p, a)
+        assert rt.pool_stats()[1] == 1                     # kept at once, nothing was waited for
+        q = rt.malloc_async(n * 4, a)
+        assert q == p
+        out = np.empty(n, np.float32)
+        rt.memcpy_d2h(out.ctypes.data, q, n * 4, a)
+        rt.stream_sync(a)
+        assert np.array_equal(out, expected)
+        # another stream: its work on the block starts behind the first stream's
+        for _ in range(8):
+            rt.elementwise_unary("abs", 32, n, neg.data_ptr(), q, stream=a)
+        rt.free_async(q, a)
+        r = rt.malloc_async(n * 4, b)
+        assert r == p
+        rt.elementwise_unary("abs", 32, n, neg2.data_ptr(), r, stream=b)     # must land after the eight launches on a
+        rt.memcpy_d2h(out.ctypes.data, r, n * 4, b)
+        rt.stream_sync(b)
+        rt.stream_sync(a)
+        assert np.array_equal(out, expected * 2)
+        # the host-ordered malloc waits for a release that is still pending
+        for _ in range(8):
+            rt.elementwise_unary("abs", 32, n, neg.data_ptr(), r, stream=b)
+        rt.free_async(r, b)
+        t = rt.malloc(n * 4)
+        assert t == p
+        rt.memcpy_d2h(out.ctypes.data, t, n * 4)           # the null stream does not wait for b by itself
+        rt.stream_sync()
+        assert np.array_equal(out, expected)
+        rt.free(t)
+        # a block freed the plain way is not pending: any stream takes it without an event
+        assert rt.malloc_async(n * 4, b) == p
+        rt.free_async(p, b)
+    finally:
+        rt.stream_sync(a)
+        rt.stream_sync(b)
+        rt.stream_destroy(a)
+        rt.stream_destroy(b)
+        rt.pool_trim()
+
+
+def test_a_destroyed_stream_gives_its_partial_results_back(rt):
+    """The two-launch kernels keep 8 MiB per stream they ran on; destroying the stream releases it."""
+    import torch
+    x = torch.randn(8192, 256, device="cuda")
+    y = torch.empty(256, device="cuda")
+    ref = x.double().sum(0)
+
+    def once():
+        s = rt.stream_create()
+        rt.reduce("sum", 32, 1, 8192, 256, x.data_ptr(), y.data_ptr(), stream=s)      # few columns, long extent: sliced
+        rt.stream_sync(s)
+        rt.stream_destroy(s)
+
+    once()
+    torch.cuda.synchronize()
+    assert float((y.double() - ref).abs().max() / ref.abs().max()) < 1e-5
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(12):
+        once()
+    torch.cuda.synchronize()
+    assert free_before - torch.cuda.mem_get_info()[0] < (16 << 20), "partial-result buffers of destroyed streams were kept"
+
+
+def test_uploads_from_memory_the_caller_pinned_go_straight_to_the_driver(rt):
+    """Memory pinned by someone else (torch's pin_memory) is recognised: the upload is one asynchronous copy, and
+    arrives intact."""
+    import torch
+    n = (24 << 20) + 3
+    host = torch.randint(0, 255, (n,), dtype=torch.uint8).pin_memory()
+    p = rt.malloc(n)
+    rt.memcpy_h2d(p, host.data_ptr(), n)
+    back = torch.empty(n, dtype=torch.uint8)
+    rt.memcpy_d2h(back.data_ptr(), p, n)
+    rt.stream_sync()
+    rt.free(p)
+    assert torch.equal(host, back)
+
+
 def test_result_arrays_are_pinned_and_reused(rt):
     import gc
     rt.pinned_trim()

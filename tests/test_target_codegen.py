@@ -168,7 +168,7 @@ def test_with_transfers_dispatcher_text(tmp_path):
                   "double __beta = 0.0;", "_docc_ret_0 = __C;"):
         assert piece in flat
     # alloc x3, upload of A and B only (beta == 0: C is not read), launch, download, sync, free x3
-    assert flat.count("docc_rocm_malloc(") == 3 and flat.count("docc_rocm_free(") == 3
+    assert flat.count("docc_rocm_malloc_async(") == 3 and flat.count("docc_rocm_free_async(") == 3
     assert flat.count("docc_rocm_memcpy_h2d_async(") == 2 and flat.count("docc_rocm_memcpy_d2h_async(") == 1
     assert "docc_rocm_dgemm(nullptr, 111, 111, _s0, _s0, _s0, __alpha, (const double *) d___A, _s0, (const double *) d___B, _s0, __beta, (double *) d___C, _s0)" in flat
     assert flat.index("docc_rocm_memcpy_h2d_async") < flat.index("docc_rocm_dgemm") < flat.index("docc_rocm_memcpy_d2h_async") < flat.index("docc_rocm_stream_sync")
@@ -231,7 +231,7 @@ def test_attention_with_another_head_dimension_brings_its_workspace(tmp_path):
         else:
             assert "docc_rocm_attention_bf16_workspace_bytes(2, 4, 256, 192, 128, 1);" in src
             assert "docc_rocm_attention_bf16_ws(nullptr, 2, 4, 256, 192, 128, (float) (0.125), (const uint16_t *) Q" in src
-            assert src.index("docc_rocm_malloc(&__ws") < src.index("docc_rocm_attention_bf16_ws(") < src.index("docc_rocm_free(__ws)")
+            assert src.index("docc_rocm_malloc_async(&__ws") < src.index("docc_rocm_attention_bf16_ws(") < src.index("docc_rocm_free_async(__ws, nullptr)")
 
 
 def test_transpose_node_round_trips_and_dispatches(tmp_path):
@@ -320,8 +320,8 @@ def test_offloading_keeps_intermediates_on_the_device(tmp_path):
     codes = [(n["code"], n.get("transfer_direction"), n.get("buffer_lifecycle")) for n in s.library_nodes()]
     assert codes.index(("GEMM", None, None)) < codes.index(("ml::Softmax", None, None))
     src, _ = source_of(s, tmp_path)
-    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")  # no host allocation left
-    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(") == 4
+    assert "malloc(" not in src.replace("docc_rocm_malloc_async(", "")  # no host allocation left
+    assert src.count("docc_rocm_malloc_async(") == src.count("docc_rocm_free_async(") == 4
     # without minimisation (per-node transfers) T would cross twice
     s2 = chain_sdfg()
     s2.schedule("rocm", options={"offload": "node"})
@@ -393,7 +393,7 @@ def every_node_type():
 
 
 LAUNCHER_CALL = re.compile(r"DOCC_ROCM_CHECK\((docc_rocm_\w+)\((.*)\)\);")
-NOT_A_KERNEL = {"docc_rocm_malloc", "docc_rocm_free", "docc_rocm_memcpy_h2d_async", "docc_rocm_memcpy_d2h_async",
+NOT_A_KERNEL = {"docc_rocm_malloc_async", "docc_rocm_free_async", "docc_rocm_memcpy_h2d_async", "docc_rocm_memcpy_d2h_async",
                 "docc_rocm_stream_sync"}
 
 
@@ -477,8 +477,8 @@ def test_offloading_a_transient_with_two_readers(tmp_path):
     valid = check_transfers(s)
     assert "T" not in valid and "size" not in s.containers["T"]
     src, _ = source_of(s, tmp_path)
-    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")
-    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(") == 5   # A B T Y Z
+    assert "malloc(" not in src.replace("docc_rocm_malloc_async(", "")
+    assert src.count("docc_rocm_malloc_async(") == src.count("docc_rocm_free_async(") == 5   # A B T Y Z
 
 
 def test_offloading_longer_chains_keep_every_lifetime_whole(tmp_path):
@@ -504,7 +504,7 @@ def test_offloading_longer_chains_keep_every_lifetime_whole(tmp_path):
     valid = check_transfers(s)
     assert not ({"T", "U", "V"} & valid)
     src, _ = source_of(s, tmp_path)
-    assert src.count("docc_rocm_malloc(") == src.count("docc_rocm_free(")
+    assert src.count("docc_rocm_malloc_async(") == src.count("docc_rocm_free_async(")
 
 
 def test_generated_function_honours_the_calling_convention(tmp_path):
@@ -543,10 +543,10 @@ def test_device_pointer_mode_allocates_transients_on_the_device(tmp_path):
     assert r["H2D"] == 0 and r["D2H"] == 0 and r["ROCMOffloading"] == 2       # ALLOC and FREE of T
     assert s.containers["T"]["storage"] == "ROCM_Generic" and "size" not in s.containers["T"]
     src, _ = source_of(s, tmp_path)
-    assert "malloc(" not in src.replace("docc_rocm_malloc(", "")
+    assert "malloc(" not in src.replace("docc_rocm_malloc_async(", "")
     flat = re.sub(r"\s+", " ", src)
-    assert flat.index("docc_rocm_malloc(") < flat.index("docc_rocm_sgemm(") < flat.index("docc_rocm_softmax_f32(") < flat.index("docc_rocm_free(")
-    assert src.count("docc_rocm_malloc(") == 1 and src.count("docc_rocm_free(") == 1
+    assert flat.index("docc_rocm_malloc_async(") < flat.index("docc_rocm_sgemm(") < flat.index("docc_rocm_softmax_f32(") < flat.index("docc_rocm_free_async(")
+    assert src.count("docc_rocm_malloc_async(") == 1 and src.count("docc_rocm_free_async(") == 1
 
 
 def dense_sdfg():
@@ -602,7 +602,7 @@ def test_elementwise_with_transfers_and_scalar_on_the_left(tmp_path):
     src, report = source_of(s, tmp_path)
     flat = re.sub(r"\s+", " ", src)
     assert "docc_rocm_elementwise_binary_scalar(nullptr, 1 /* ml::Sub */, 64, _n, d_B, (double) A, 1, d_C)" in flat
-    assert flat.count("docc_rocm_malloc(") == 2 and flat.count("docc_rocm_memcpy_h2d_async(") == 1   # the scalar is not an operand buffer
+    assert flat.count("docc_rocm_malloc_async(") == 2 and flat.count("docc_rocm_memcpy_h2d_async(") == 1   # the scalar is not an operand buffer
     assert flat.count("docc_rocm_memcpy_d2h_async(") == 1
     # what the kernels lack is declined, not run elsewhere
     b = StructuredSDFGBuilder("ints")
@@ -639,7 +639,7 @@ def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
     assert ("docc_rocm_sgemm_epilogue(nullptr, 111, 111, 32, 16, 8, __alpha, (const float *) __A, 8, (const float *) __B, 16, __beta, "
             "(float *) __C, 16, (const float *) __bias, 2 /* ml::ReLU */)") in flat
     assert "float *__bias = __daisy_rocm_" in flat
-    assert flat.count("docc_rocm_malloc(") == 5      # X W bias on the device, T3, Y
+    assert flat.count("docc_rocm_malloc_async(") == 5      # X W bias on the device, T3, Y
 
     # without the GEMM in front the chain is one elementwise launch
     b = StructuredSDFGBuilder("ew")
@@ -751,10 +751,10 @@ def test_reduce_nodes_dispatch_and_decline(tmp_path):
     s.schedule("rocm", options={"offload": "none"})
     flat = re.sub(r"\s+", " ", source_of(s, tmp_path / "scattered")[0])
     # axes in two blocks: the inner block (axes 2, 3) first into a device temporary, then axis 0 of what is left
-    assert "docc_rocm_malloc(&__docc_part[0], (size_t) (1120))" in flat                      # [4, 5, 7] doubles
+    assert "docc_rocm_malloc_async(&__docc_part[0], (size_t) (1120), nullptr)" in flat                      # [4, 5, 7] doubles
     assert "docc_rocm_reduce(nullptr, 3 /* ml::Mean */, 64, 20, _n*6, 7, X, __docc_part[0])" in flat
     assert "docc_rocm_reduce(nullptr, 3 /* ml::Mean */, 64, 1, 4, 35, __docc_part[0], Y)" in flat
-    assert "docc_rocm_free(__docc_part[0])" in flat
+    assert "docc_rocm_free_async(__docc_part[0], nullptr)" in flat
     # std is the chain of nodes the reference's StdNode expands to
     b = StructuredSDFGBuilder("s")
     for n in ("X", "Y"):
