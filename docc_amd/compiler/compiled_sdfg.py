@@ -77,6 +77,8 @@ class CompiledSDFG:
             if c["type"] == "pointer":
                 want = _NUMPY[elem]
                 arr = value if isinstance(value, np.ndarray) else np.asarray(value)
+                if elem == PrimitiveType.BFloat and arr.dtype.name == "bfloat16" and arr.dtype.itemsize == 2:
+                    arr = arr.view(np.uint16)      # an ml_dtypes array: the same words
                 if arr.dtype != want:
                     raise TypeError(f"argument '{name}' must have dtype {np.dtype(want).name}, got {arr.dtype}")
                 if not arr.flags.c_contiguous:

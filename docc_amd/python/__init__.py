@@ -4,7 +4,7 @@ reference exports from `docc.python` (python/docc/python/__init__.py:1-13).
 Importing this package registers the `rocm` target through the same hook a third-party
 target would use (`register_target_overrides`)."""
 from docc_amd.python.functions import conv2d, erf, relu, sigmoid, softmax
-from docc_amd.python.python_program import PythonProgram, _map_python_type, native
+from docc_amd.python.python_program import PythonProgram, _map_python_type, bfloat16, native
 from docc_amd.python.target_registry import (get_target_compile_fn, get_target_schedule_fn, register_target,
                                              register_target_overrides, unregister_target)
 
@@ -21,5 +21,5 @@ def _rocm_compile(sdfg, output_folder, instrumentation_mode, capture_args, optio
 
 register_target_overrides("rocm", _rocm_schedule, _rocm_compile)
 
-__all__ = ["PythonProgram", "native", "register_target", "register_target_overrides", "unregister_target",
+__all__ = ["PythonProgram", "native", "bfloat16", "register_target", "register_target_overrides", "unregister_target",
            "get_target_schedule_fn", "get_target_compile_fn", "softmax", "conv2d", "relu", "sigmoid", "erf", "_map_python_type"]

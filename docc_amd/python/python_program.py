@@ -52,9 +52,23 @@ _DTYPES = {np.dtype(np.float64): PrimitiveType.Double, np.dtype(np.float32): Pri
 _SIZES = {PrimitiveType.Double: 8, PrimitiveType.Float: 4}
 
 
+class bfloat16:
+    """Names the bf16 element type in a parameter annotation: `Annotated[np.ndarray, (m, k), bfloat16]` or
+    `np.ndarray[Any, np.dtype[bfloat16]]` on a parameter whose arrays arrive as `np.uint16` (the raw 16-bit words, which
+    is how bf16 crosses the ctypes boundary: reference compiled_sdfg.py:28-31). The reference recognises
+    `ml_dtypes.bfloat16` arrays (python_program.py:432-433); such arrays are taken here too where that package exists.
+    Products of bf16 operands accumulate and return float32 (GEMM precision `b`)."""
+
+
+def _is_ml_bfloat16(dtype) -> bool:
+    return getattr(dtype, "name", "") == "bfloat16" and getattr(dtype, "itemsize", 0) == 2
+
+
 def _map_python_type(value: Any):
     """Python/numpy value -> SDFG type (reference python_program.py:401-464)."""
     if isinstance(value, np.ndarray):
+        if _is_ml_bfloat16(value.dtype):
+            return Pointer(Scalar(PrimitiveType.BFloat))
         if value.dtype not in _DTYPES:
             raise TypeError(f"unsupported array dtype {value.dtype}")
         return Pointer(Scalar(_DTYPES[value.dtype]))
@@ -86,6 +100,8 @@ def _map_annotation(ann: Any):
             elem = _map_annotation(inner[0] if typing.get_origin(dt) is np.dtype and inner else dt)
             return Pointer(elem) if isinstance(elem, Scalar) else None
         return None
+    if ann is bfloat16 or _is_ml_bfloat16(ann) or getattr(ann, "__name__", "") == "bfloat16":
+        return Scalar(PrimitiveType.BFloat)
     table = {float: PrimitiveType.Double, np.float64: PrimitiveType.Double, np.float32: PrimitiveType.Float, bool: PrimitiveType.Bool,
              np.bool_: PrimitiveType.Bool, int: PrimitiveType.Int64, np.int64: PrimitiveType.Int64, np.int32: PrimitiveType.Int32}
     try:
@@ -233,12 +249,14 @@ class _Lowering(ast.NodeVisitor):
             self.fail(node, "a matrix product of non-array operands")
         if left.elem != right.elem:
             self.fail(node, "a matrix product of mixed element types")
+        # bf16 operands: the products are accumulated and returned in float32 (GEMM precision `b`, ml::MatMul on BFloat)
+        out_elem = PrimitiveType.Float if left.elem == PrimitiveType.BFloat else left.elem
         if len(left.shape) == 2 and len(right.shape) == 2:
             m, k = (left.shape[1], left.shape[0]) if ta else left.shape
             k2, n = (right.shape[1], right.shape[0]) if tb else right.shape
             if k != k2:
                 raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({k} vs {k2})")
-            out = self.new_array([m, n], left.elem, dest)
+            out = self.new_array([m, n], out_elem, dest)
             self.b.add_gemm(left.name, right.name, out.name, alpha, beta, m, n, k, ta, tb, left.shape[1], right.shape[1], n)
             return out
         # vectors, numpy's rules: matrix @ vector and vector @ matrix are GEMMs with one column / one row, the result
@@ -247,16 +265,18 @@ class _Lowering(ast.NodeVisitor):
             m, k = (left.shape[1], left.shape[0]) if ta else left.shape
             if k != right.shape[0]:
                 raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({k} vs {right.shape[0]})")
-            out = self.new_array([m], left.elem, dest)
+            out = self.new_array([m], out_elem, dest)
             self.b.add_gemm(left.name, right.name, out.name, alpha, beta, m, "1", k, ta, False, left.shape[1], "1", "1")
             return out
         if len(left.shape) == 1 and len(right.shape) == 2 and not ta:
             k2, n = (right.shape[1], right.shape[0]) if tb else right.shape
             if left.shape[0] != k2:
                 raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({left.shape[0]} vs {k2})")
-            out = self.new_array([n], left.elem, dest)
+            out = self.new_array([n], out_elem, dest)
             self.b.add_gemm(left.name, right.name, out.name, alpha, beta, "1", n, left.shape[0], False, tb, left.shape[0], right.shape[1], n)
             return out
+        if len(left.shape) == 1 and len(right.shape) == 1 and left.elem == PrimitiveType.BFloat:
+            self.fail(node, "the inner product of two bf16 vectors")
         if len(left.shape) == 1 and len(right.shape) == 1 and not (ta or tb) and alpha == "1.0" and beta == "0.0":
             if left.shape[0] != right.shape[0]:
                 raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ ({left.shape[0]} vs {right.shape[0]})")
@@ -267,7 +287,7 @@ class _Lowering(ast.NodeVisitor):
             self.fail(node, "this broadcast in a batched product")
         if left.shape[-1] != right.shape[-2]:
             raise ValueError(f"{self.func.__name__}: matmul inner dimensions differ")
-        out = self.new_array(left.shape[:-1] + [right.shape[-1]], left.elem, dest)
+        out = self.new_array(left.shape[:-1] + [right.shape[-1]], out_elem, dest)
         self.b.add_matmul(left.name, right.name, out.name, left.shape, right.shape)
         return out
 
@@ -709,7 +729,17 @@ class PythonProgram(DoccProgram):
     def _analyse(self, args: Sequence[Any]):
         """Shape symbols: every distinct dimension value (other than 1) gets one `_s<i>`, in order
         of first appearance; returns (types, mapping, shape_sources, signature)."""
-        arg_types = [_map_python_type(a) for a in args]
+        # a parameter annotated as bf16 takes the raw 16-bit words
+        hints = self._parameter_annotations()
+        arg_types = []
+        for i, a in enumerate(args):
+            declared = hints[i] if i < len(hints) else None
+            if isinstance(a, np.ndarray) and isinstance(declared, Pointer) and declared.primitive_type == PrimitiveType.BFloat:
+                if a.dtype != np.uint16 and not _is_ml_bfloat16(a.dtype):
+                    raise TypeError(f"{self.name}: parameter {i} is annotated as bfloat16 and takes uint16 words, got {a.dtype}")
+                arg_types.append(declared)
+            else:
+                arg_types.append(_map_python_type(a))
         values: List[int] = []
         sources: List[Tuple[int, int]] = []
         mapping: Dict[Tuple[int, int], int] = {}
@@ -727,6 +757,16 @@ class PythonProgram(DoccProgram):
         ones = sorted((i, d) for i, a in enumerate(args) if isinstance(a, np.ndarray) for d, v in enumerate(a.shape) if v == 1)
         signature = f"{type_sig}|{sorted(mapping.items())}|{ones}"
         return arg_types, mapping, sources, signature
+
+    def _parameter_annotations(self) -> List[Any]:
+        """The SDFG type each parameter's annotation names, or None (no annotation, a string, one that does not map)."""
+        if getattr(self, "_hints", None) is None:
+            out = []
+            for p in inspect.signature(self.func).parameters.values():
+                ann = p.annotation
+                out.append(None if ann is inspect.Parameter.empty or isinstance(ann, str) else _map_annotation(ann))
+            self._hints = out
+        return self._hints
 
     def _get_cache_key(self, *args: Any) -> str:
         return self._analyse(args)[3]

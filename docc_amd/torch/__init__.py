@@ -68,6 +68,23 @@ class _Transposed:
         self.base = base
 
 
+class _Widened:
+    """A bf16 tensor converted to float32 (`x.float()`), kept symbolic: as both operands of a product it selects the
+    bf16 GEMM with float32 accumulation and result, which computes exactly that expression; anywhere else it becomes
+    the ml::Cast it stands for."""
+
+    def __init__(self, base: _T, dtype):
+        self.base, self.shape, self.dtype = base, base.shape, dtype
+
+
+class _Bf16Product:
+    """`a @ b` of bf16 operands, kept symbolic until `.float()` / `.to(torch.float32)` asks for the float32 result:
+    the GEMM then writes its float32 accumulators (without the rounding to bf16 that eager torch inserts in between)."""
+
+    def __init__(self, a: _T, b: _T, ta: bool, tb: bool):
+        self.a, self.b, self.ta, self.tb = a, b, ta, tb
+
+
 class _Scores:
     """scale * q @ k^T, kept symbolic until a softmax and a product with v complete the pattern."""
 
@@ -146,6 +163,10 @@ class _FxLowering:
             ta, a = True, a.base
         if isinstance(b, _Transposed):
             tb, b = True, b.base
+        if isinstance(a, _Widened) and isinstance(b, _Widened) and a.dtype == b.dtype == torch.float32:
+            # a.float() @ b.float() of bf16 tensors: the bf16 GEMM with float32 accumulation is that product
+            return self.product(node, a.base, b.base, ta, tb, torch.float32, dest)
+        a, b = self.tensor(node, a), self.tensor(node, b)
         if not isinstance(a, _T) or not isinstance(b, _T):
             self.fail(node, "a product of these operands")
         if a.dtype != b.dtype:
@@ -153,21 +174,31 @@ class _FxLowering:
         if len(a.shape) > 2 and tb and not ta and a.dtype == torch.bfloat16 and len(b.shape) == len(a.shape):
             return _Scores(a, b)  # q @ k^T: waits for its softmax
         if a.dtype == torch.bfloat16:
-            self.fail(node, "a bf16 product outside the attention pattern (its result would have to be rounded back to bf16)")
+            # bf16 operands: only the float32 result exists as a kernel; `.float()` on the product asks for it
+            return _Bf16Product(a, b, ta, tb)
+        return self.product(node, a, b, ta, tb, a.dtype, dest)
+
+    def product(self, node, a: _T, b: _T, ta: bool, tb: bool, out_dtype, dest):
+        """GEMM (2-d operands, transposes by flag) or ml::MatMul (batched) into a tensor of `out_dtype`: the operands'
+        dtype, or float32 for bf16 operands."""
         if len(a.shape) == 2 and len(b.shape) == 2:
             m, k = (a.shape[1], a.shape[0]) if ta else a.shape
             k2, n = (b.shape[1], b.shape[0]) if tb else b.shape
             if k != k2:
                 self.fail(node, f"inner dimensions {k} and {k2}")
-            out = self.new_tensor([m, n], a.dtype, dest)
+            out = self.new_tensor([m, n], out_dtype, dest)
             one, zero = "1.0", "0.0"
             self.builder.add_gemm(a.name, b.name, out.name, one, zero, m, n, k, ta, tb, a.shape[1], b.shape[1], n)
             return out
         if ta or tb:
             self.fail(node, "a transposed operand in a batched product")
+        if len(a.shape) < 2 or len(b.shape) < 2:
+            self.fail(node, "a product with a vector operand")
         if len(b.shape) > 2 and b.shape[:-2] != a.shape[:-2]:
             self.fail(node, "broadcasting batch dimensions")
-        out = self.new_tensor(a.shape[:-1] + [b.shape[-1]], a.dtype, dest)
+        if a.shape[-1] != b.shape[-2]:
+            self.fail(node, f"inner dimensions {a.shape[-1]} and {b.shape[-2]}")
+        out = self.new_tensor(a.shape[:-1] + [b.shape[-1]], out_dtype, dest)
         self.builder.add_matmul(a.name, b.name, out.name, a.shape, b.shape)
         return out
 
@@ -284,20 +315,27 @@ class _FxLowering:
 
     def linear(self, node, x, w, bias, dest):
         """x [..., K] times w[N, K] transposed, plus bias [N]: one GEMM over the flattened rows."""
+        out_dtype = None
+        if isinstance(x, _Widened) and isinstance(w, _Widened):      # bf16 operands widened for the product: the bf16 GEMM
+            x, w, out_dtype = x.base, w.base, self.torch.float32
+        else:
+            x, w = self.tensor(node, x), self.tensor(node, w)
         if not isinstance(x, _T) or not isinstance(w, _T) or len(w.shape) != 2 or len(x.shape) < 1 or x.shape[-1] != w.shape[1]:
             self.fail(node, "linear on these operands")
-        if x.dtype != w.dtype or x.dtype not in (self.torch.float32, self.torch.float64):
-            self.fail(node, "linear on dtypes other than float32 / float64")
+        if x.dtype != w.dtype or (out_dtype is None and x.dtype not in (self.torch.float32, self.torch.float64)):
+            self.fail(node, "linear on dtypes other than float32 / float64 (bf16 operands: pass x.float(), w.float())")
         n, k = w.shape
         m = int(math.prod(x.shape[:-1]))
         shape = x.shape[:-1] + [n]
-        out = self.new_tensor(shape, x.dtype, dest if bias is None else None)
+        out = self.new_tensor(shape, out_dtype or x.dtype, dest if bias is None else None)
         self.builder.add_gemm(x.name, w.name, out.name, "1.0", "0.0", m, n, k, False, True, k, k, n)
         if bias is None:
             return out
         return self.elementwise(node, "add", out, bias, dest)
 
     def transpose(self, node, x, d0: int, d1: int, dest=None):
+        if isinstance(x, _Widened) and dest is None and {d0 % len(x.shape), d1 % len(x.shape)} == {len(x.shape) - 2, len(x.shape) - 1}:
+            return _Transposed(x)   # still an operand of a bf16 product, or cast and transposed where it is used
         x = self.tensor(node, x)
         if not isinstance(x, _T):
             self.fail(node, "transposing this value")
@@ -325,6 +363,17 @@ class _FxLowering:
 
     def cast(self, node, x, dtype, dest=None):
         """ml::Cast; the same dtype passes the tensor on."""
+        torch = self.torch
+        if isinstance(x, _Bf16Product):
+            if dtype != torch.float32:
+                self.fail(node, f"a bf16 product converted to {dtype} (only its float32 result is computed)")
+            return self.product(node, x.a, x.b, x.ta, x.tb, torch.float32, dest)
+        if dtype == torch.float32 and dest is None:
+            # bf16 -> float32 that may be an operand of a product: decided where it is used
+            if isinstance(x, _T) and x.dtype == torch.bfloat16:
+                return _Widened(x, dtype)
+            if isinstance(x, _Transposed) and isinstance(x.base, _T) and x.base.dtype == torch.bfloat16:
+                return _Transposed(_Widened(x.base, dtype))
         x = self.tensor(node, x)
         if not isinstance(x, _T):
             self.fail(node, "converting this value")
@@ -345,6 +394,13 @@ class _FxLowering:
         if isinstance(v, _Transposed):
             rank = len(v.base.shape)
             return self.permute(node, v.base, list(range(rank - 2)) + [rank - 1, rank - 2], dest)
+        if isinstance(v, _Widened):
+            out = self.new_tensor(v.shape, v.dtype, dest)
+            self.builder.add_cast_op(v.base.name, out.name, v.shape)
+            return out
+        if isinstance(v, _Bf16Product):
+            self.fail(node, "a bf16 product used without `.float()` (the target computes its float32 result; rounding it "
+                            "back to bf16 is not built)")
         return v
 
     # ---- graph walk -------------------------------------------------------------------------
@@ -419,7 +475,7 @@ class _FxLowering:
             elif node.op == "output":
                 for i, n in enumerate(out_list):
                     v = self.env[n]
-                    if isinstance(v, _Transposed):
+                    if isinstance(v, (_Transposed, _Widened, _Bf16Product)):
                         v = self.tensor(n, v, f"_docc_ret_{i}")
                     elif isinstance(v, _T) and v.name != f"_docc_ret_{i}" and 1 <= len(v.shape) <= 6:
                         # a value that lives elsewhere (an input, the operand of a view): copied into the result

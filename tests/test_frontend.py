@@ -528,3 +528,77 @@ def test_return_annotation_puts_the_outputs_first():
         return a @ b
 
     assert loose.to_sdfg(a, a).arguments == ["a", "b", "_s0", "_docc_ret_0"]
+
+
+def test_bf16_products_lower_to_the_gemm_with_float32_accumulation():
+    """bf16 operands reach GEMM precision `b` (float32 accumulate and result) from both front ends: `@native` through a
+    parameter annotation on arrays of the 16-bit words (the reference carries bf16 across ctypes as c_uint16,
+    compiled_sdfg.py:28-31), torch through `(a @ b).float()` or `a.float() @ b.float()`."""
+    from typing import Annotated, Any
+
+    from docc_amd.python import bfloat16
+
+    @native(target="rocm")
+    def mm(a: Annotated[np.ndarray, ("M", "K"), bfloat16], b: np.ndarray[Any, np.dtype[bfloat16]]):
+        return a @ b
+
+    a, b = np.zeros((64, 32), np.uint16), np.zeros((32, 48), np.uint16)
+    sdfg = mm.to_sdfg(a, b)
+    (node,) = sdfg.library_nodes()
+    assert node["code"] == "GEMM" and node["precision"] == ord("b")
+    elements = {k: v["element"] for k, v in sdfg.containers.items()}
+    assert elements["a"] == elements["b"] == "BFloat" and elements["_docc_ret_0"] == "Float"
+    assert "BFloat" in mm._get_cache_key(a, b)
+    with pytest.raises(TypeError, match="bfloat16"):
+        mm.to_sdfg(np.zeros((64, 32), np.float32), b)
+
+    @native(target="rocm")
+    def batched(a: Annotated[np.ndarray, (), bfloat16], b: Annotated[np.ndarray, (), bfloat16]):
+        return a @ b
+
+    sdfg = batched.to_sdfg(np.zeros((4, 64, 32), np.uint16), np.zeros((4, 32, 48), np.uint16))
+    (node,) = sdfg.library_nodes()
+    assert node["code"] == "ml::MatMul" and sdfg.containers["_docc_ret_0"]["element"] == "Float"
+
+    @native(target="rocm")
+    def plain_words(a, b):          # no annotation: uint16 is not an element type of the math nodes
+        return a @ b
+
+    with pytest.raises(TypeError, match="uint16"):
+        plain_words.to_sdfg(a, b)
+
+    class ProductThenFloat(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.matmul(a, b).float()
+
+    class Widened(torch.nn.Module):
+        def forward(self, a, b):
+            return a.float() @ b.float().T
+
+    class WidenedLinear(torch.nn.Module):
+        def forward(self, x, w):
+            return torch.nn.functional.linear(x.float(), w.float())
+
+    class OneWidened(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.relu(a.float()) @ b.float()
+
+    class Rounded(torch.nn.Module):
+        def forward(self, a, b):
+            return torch.matmul(a, b)
+
+    ta, tb, tbt = (torch.zeros(s, dtype=torch.bfloat16) for s in ((64, 32), (32, 48), (48, 32)))
+    for model, args, trans_b in ((ProductThenFloat(), (ta, tb), 111), (Widened(), (ta, tbt), 112), (WidenedLinear(), (ta, tbt), 112)):
+        sdfg = docc_torch.TorchProgram(model, target="rocm").to_sdfg(*args)
+        (node,) = sdfg.library_nodes()
+        assert (node["code"], node["precision"], node["trans_b"]) == ("GEMM", ord("b"), trans_b), type(model).__name__
+        assert sdfg.containers["_docc_ret_0"]["element"] == "Float"
+    sdfg = docc_torch.TorchProgram(ProductThenFloat(), target="rocm").to_sdfg(torch.zeros(4, 64, 32, dtype=torch.bfloat16), torch.zeros(4, 32, 48, dtype=torch.bfloat16))
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::MatMul"] and sdfg.containers["_docc_ret_0"]["element"] == "Float"
+    # one operand that is more than a widened bf16 tensor: the casts are real, the product is a float32 GEMM
+    sdfg = docc_torch.TorchProgram(OneWidened(), target="rocm").to_sdfg(ta, tb)
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Cast", "ml::ReLU", "ml::Cast", "GEMM"]
+    assert sdfg.library_nodes()[-1]["precision"] == ord("s")
+    # the product rounded back to bf16 is not built
+    with pytest.raises(NotImplementedError, match="float"):
+        docc_torch.TorchProgram(Rounded(), target="rocm").to_sdfg(ta, tb)
