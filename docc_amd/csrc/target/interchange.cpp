@@ -521,13 +521,18 @@ struct Import {
         return true;
     }
 
-    // `element` is a for or a map: the nest below it, matched against the elementwise forms
+    // `element` is a for or a map: the nest below it. A body of one operation is matched against the prebuilt kernels
+    // first (elementwise nodes, copies, fills, reductions, repeated operands); what they do not cover - several
+    // operations, operands that walk memory in different orders, operations without a node - becomes one generated
+    // kernel (ROCMMap) if every loop of the nest is a map, i.e. its iterations are independent by construction.
     void import_loop_nest(const Value& element, Array& children) {
         std::vector<NestLoop> loops;
+        std::vector<const Value*> body;
+        bool all_maps = true;
         const Value* at = &element;
-        const Value* block = nullptr;
-        while (true) {
+        while (body.empty()) {
             const std::string kind = at->at("type").as_string();
+            const Value* seq = nullptr;
             if (kind == "for" || kind == "map") {
                 NestLoop loop;
                 loop.var = strip(at->at("indvar").as_expression());
@@ -539,32 +544,353 @@ struct Import {
                 loop.extent = c_expression(strip(cond.substr(loop.var.size() + 1)));
                 if (!parse_term(loop.extent, &loop.extent_term)) refuse(*at, "the loop's bound is not a product of symbols and integers");
                 loops.push_back(loop);
-                const Value& body = at->at("root");
-                if (const Value* transitions = body.find("transitions"))
-                    for (auto& t : transitions->as_array())
-                        if (!t.at("assignments").as_array().empty()) refuse(t, "symbol assignments inside a loop nest");
-                const Value* only = nullptr;
-                for (auto& child : body.at("children").as_array()) {
-                    if (child.at("type").as_string() == "block" && child.at("dataflow").at("nodes").as_array().empty()) continue;
-                    if (only) refuse(*at, "more than one statement in a loop body");
-                    only = &child;
-                }
-                if (!only) return;   // an empty nest does nothing
-                at = only;
+                all_maps = all_maps && kind == "map";
+                seq = &at->at("root");
+            } else if (kind == "sequence") {
+                seq = at;
+            } else if (kind == "block") {
+                body.push_back(at);
+                break;
+            } else {
+                refuse(*at, "control flow inside a loop nest");
+            }
+            if (const Value* transitions = seq->find("transitions"))
+                for (auto& t : transitions->as_array())
+                    if (!t.at("assignments").as_array().empty()) refuse(t, "symbol assignments inside a loop nest");
+            std::vector<const Value*> kids;
+            for (auto& child : seq->at("children").as_array()) {
+                if (child.at("type").as_string() == "block" && child.at("dataflow").at("nodes").as_array().empty()) continue;
+                kids.push_back(&child);
+            }
+            if (kids.empty()) return;   // an empty nest does nothing
+            if (kids.size() == 1) {
+                at = kids[0];
                 continue;
             }
-            if (kind == "sequence") {
-                const Array& kids = at->at("children").as_array();
-                if (kids.size() != 1) refuse(*at, "more than one statement in a loop body");
-                at = &kids[0];
-                continue;
-            }
-            if (kind != "block") refuse(*at, "control flow inside a loop nest");
-            block = at;
-            break;
+            // several statements: the body of the innermost loop, a run of blocks
+            for (const Value* k : kids)
+                if (k->at("type").as_string() != "block") refuse(*at, "more than one statement in a loop body, one of them control flow");
+            if (!all_maps) refuse(*at, "more than one statement in a loop body (several statements are lowered under maps only)");
+            body = kids;
         }
         if (loops.size() > 6) refuse(element, "a loop nest deeper than 6");
-        lower_tasklet_block(*block, loops, children);
+        size_t operations = 0;
+        for (const Value* b : body)
+            for (auto& n : b->at("dataflow").at("nodes").as_array()) {
+                const std::string kind = n.at("type").as_string();
+                operations += kind == "tasklet" || kind == "library_node";
+            }
+        if (body.size() == 1 && operations <= 1) {
+            if (!all_maps) {
+                lower_tasklet_block(*body[0], loops, children);
+                return;
+            }
+            // what the attempt adds before it gives up (a repeated operand's temporary and its Broadcast) goes again
+            const size_t n_children = children.size(), n_containers = containers.size();
+            try {
+                lower_tasklet_block(*body[0], loops, children);
+                return;
+            } catch (const InvalidSDFGException&) {
+                children.resize(n_children);
+                containers.resize(n_containers);
+            }
+        }
+        lower_map_nest(element, body, loops, children);
+    }
+
+    // The body blocks of a nest of maps as one ROCMMap node (see sdfg_lite.h): loads, a list of statements, stores.
+    void lower_map_nest(const Value& element, const std::vector<const Value*>& body, const std::vector<NestLoop>& loops, Array& children) {
+        static const std::map<int64_t, std::string> tasklet_names = {{0, "assign"}, {1, "fp_neg"}, {2, "fp_add"}, {3, "fp_sub"},
+                                                                     {4, "fp_mul"}, {5, "fp_div"}, {6, "fp_rem"}, {7, "fp_fma"}};
+        using P = types::PrimitiveType;
+        Array reads, writes, scalars, statements, inputs, outputs;
+        std::map<std::string, std::string> current;      // scalar container written in the body -> the value it holds now
+        std::map<std::string, std::string> stored;       // container|strides -> the value this nest stores there
+        std::map<std::string, size_t> write_at;          // container|strides -> index in `writes`
+        std::map<std::string, std::string> read_conn;    // container|strides -> connector of the load
+        std::map<std::string, std::string> scalar_conn;  // scalar container -> connector
+        std::map<std::string, std::set<std::string>> read_keys, write_keys;   // per container: how it is indexed
+        size_t n_values = 0;
+
+        auto is_argument = [&](const std::string& name) {
+            for (auto& arg : src.at("arguments").as_array())
+                if (arg.as_string() == name) return true;
+            return false;
+        };
+        auto floating = [&](P t, const Value& where) {
+            if (t != P::Float && t != P::Double) refuse(where, std::string("a value of type ") + types::primitive_type_to_string(t) + " in a loop body (Float and Double only)");
+            return t;
+        };
+        // strides (elements) per loop and the element count of a dense operand
+        auto layout_of = [&](const OperandWalk& w, Array* strides, std::string* extent, std::string* key) {
+            std::vector<std::string> per_loop(loops.size(), "0");
+            std::string run = "1";
+            for (size_t k = w.order.size(); k-- > 0;) {
+                per_loop[(size_t) w.order[k]] = run;
+                run = run == "1" ? loops[(size_t) w.order[k]].extent : "(" + loops[(size_t) w.order[k]].extent + ")*" + run;
+            }
+            *extent = run;
+            for (auto& st : per_loop) {
+                strides->emplace_back(st);
+                *key += "|" + st;
+            }
+        };
+
+        for (const Value* block : body) {
+            const Value& df = block->at("dataflow");
+            std::map<int64_t, const Value*> by_id;
+            std::vector<const Value*> ops;
+            for (auto& n : df.at("nodes").as_array()) {
+                by_id[n.at("element_id").as_int()] = &n;
+                const std::string kind = n.at("type").as_string();
+                if (kind == "tasklet") ops.push_back(&n);
+                else if (kind == "library_node") {
+                    if (n.at("code").as_string() != "CMath") refuse(n, "a library node inside a loop nest");
+                    ops.push_back(&n);
+                }
+            }
+            std::map<int64_t, std::map<std::string, const Value*>> in_edges;   // op -> connector -> edge
+            std::map<int64_t, std::vector<const Value*>> out_edges;            // op -> edges
+            std::map<int64_t, int64_t> producer;                                // access node -> op that writes it here
+            auto is_op = [&](int64_t id) {
+                for (const Value* o : ops)
+                    if (o->at("element_id").as_int() == id) return true;
+                return false;
+            };
+            for (auto& e : df.at("edges").as_array()) {
+                const int64_t from = e.at("src").as_int(), to = e.at("dst").as_int();
+                if (!by_id.count(from) || !by_id.count(to)) refuse(*block, "an edge refers to an unknown node");
+                if (is_op(to) && !is_op(from)) in_edges[to][e.at("dst_conn").as_string()] = &e;
+                else if (is_op(from) && !is_op(to)) {
+                    out_edges[from].push_back(&e);
+                    producer[to] = from;
+                } else
+                    refuse(*block, "data movement beside the operations");
+            }
+            // the operations in an order in which every value is computed before it is used
+            std::vector<const Value*> order;
+            std::set<int64_t> done;
+            while (order.size() < ops.size()) {
+                bool progress = false;
+                for (const Value* op : ops) {
+                    const int64_t id = op->at("element_id").as_int();
+                    if (done.count(id)) continue;
+                    bool ready = true;
+                    for (auto& kv : in_edges[id]) {
+                        auto p = producer.find(kv.second->at("src").as_int());
+                        ready = ready && (p == producer.end() || done.count(p->second));
+                    }
+                    if (!ready) continue;
+                    order.push_back(op);
+                    done.insert(id);
+                    progress = true;
+                }
+                if (!progress) refuse(*block, "operations that depend on each other in a cycle");
+            }
+
+            for (const Value* op : order) {
+                const int64_t id = op->at("element_id").as_int();
+                std::string name;
+                std::vector<std::string> connectors;
+                if (op->at("type").as_string() == "tasklet") {
+                    auto it = tasklet_names.find(op->at("code").as_int());
+                    if (it == tasklet_names.end()) refuse(*op, "tasklet code " + std::to_string(op->at("code").as_int()) + " has no kernel");
+                    name = it->second;
+                    for (auto& i : op->at("inputs").as_array()) connectors.push_back(i.as_string());
+                } else {
+                    name = op->at("function_stem").as_string();
+                    if (!rocm::ROCMMapNode::is_cmath(name)) refuse(*op, "CMath function '" + name + "' has no kernel");
+                    for (int k = 1; k <= rocm::ROCMMapNode::arity(name); k++) connectors.push_back("_in" + std::to_string(k));
+                }
+                if ((int) connectors.size() != rocm::ROCMMapNode::arity(name)) refuse(*op, "operation " + name + " with " + std::to_string(connectors.size()) + " inputs");
+                Array args;
+                for (auto& conn : connectors) {
+                    auto hit = in_edges[id].find(conn);
+                    if (hit == in_edges[id].end()) refuse(*op, "input '" + conn + "' is not connected");
+                    const Value& e = *hit->second;
+                    const Value& node = *by_id.at(e.at("src").as_int());
+                    if (node.at("type").as_string() == "constant_node") {
+                        floating(element_of(node.at("data_type"), describe(node)), node);
+                        args.emplace_back("#" + c_expression(node.at("data").as_expression()));
+                        continue;
+                    }
+                    const std::string data = node.at("data").as_string();
+                    const Value& c = container(data);
+                    const P element = types::primitive_type_from_string(c.at("element").as_string());
+                    if (c.at("type").as_string() == "scalar") {
+                        auto cur = current.find(data);
+                        auto known = assigned.find(data);
+                        if (cur != current.end()) {
+                            args.emplace_back(cur->second);
+                        } else if (known != assigned.end()) {
+                            args.emplace_back("#(" + c_expression(known->second) + ")");
+                        } else {
+                            floating(element, node);
+                            auto sc = scalar_conn.find(data);
+                            if (sc == scalar_conn.end()) {
+                                sc = scalar_conn.emplace(data, "_c" + std::to_string(scalar_conn.size())).first;
+                                Value s;
+                                s.set("connector", sc->second);
+                                s.set("element_type", types::primitive_type_to_string(element));
+                                scalars.push_back(std::move(s));
+                                Value b;
+                                b.set("data", data);
+                                b.set("connector", sc->second);
+                                inputs.push_back(std::move(b));
+                            }
+                            args.emplace_back(sc->second);
+                        }
+                        continue;
+                    }
+                    floating(element, node);
+                    OperandWalk w;
+                    if (loops.empty() || !walk_of(*block, e, node, loops, &w) || w.scalar)
+                        refuse(*block, "operand '" + data + "' is not a dense tensor indexed by the loop variables");
+                    Array strides;
+                    std::string extent, key = data;
+                    layout_of(w, &strides, &extent, &key);
+                    auto st = stored.find(key);
+                    if (st != stored.end()) {   // the element this iteration has just computed
+                        args.emplace_back(st->second);
+                        continue;
+                    }
+                    read_keys[data].insert(key);
+                    auto rc = read_conn.find(key);
+                    if (rc == read_conn.end()) {
+                        rc = read_conn.emplace(key, "_in" + std::to_string(read_conn.size())).first;
+                        Value r;
+                        r.set("connector", rc->second);
+                        r.set("strides", Value(std::move(strides)));
+                        r.set("extent", extent);
+                        r.set("element_type", types::primitive_type_to_string(element));
+                        reads.push_back(std::move(r));
+                        Value b;
+                        b.set("data", data);
+                        b.set("connector", rc->second);
+                        inputs.push_back(std::move(b));
+                    }
+                    args.emplace_back(rc->second);
+                }
+                auto outs = out_edges.find(id);
+                if (outs == out_edges.end() || outs->second.empty()) refuse(*op, "an operation without a result");
+                const std::string value = "_v" + std::to_string(n_values++);
+                P type = P::Void;
+                if (op->at("type").as_string() != "tasklet" && op->contains("primitive_type")) type = primitive_of(op->at("primitive_type"), describe(*op));
+                if (type == P::Void) type = element_of(outs->second[0]->at("base_type"), describe(*block));
+                floating(type, *op);
+                Value stmt;
+                stmt.set("out", value);
+                stmt.set("type", types::primitive_type_to_string(type));
+                stmt.set("op", name);
+                stmt.set("args", Value(std::move(args)));
+                statements.push_back(std::move(stmt));
+                for (const Value* e : outs->second) {
+                    const Value& node = *by_id.at(e->at("dst").as_int());
+                    if (node.at("type").as_string() != "access_node") refuse(*block, "a result that does not go to a container");
+                    const std::string data = node.at("data").as_string();
+                    const Value& c = container(data);
+                    const P element = floating(types::primitive_type_from_string(c.at("element").as_string()), node);
+                    if (c.at("type").as_string() == "scalar") {
+                        if (is_argument(data)) refuse(*block, "a scalar argument ('" + data + "') written inside a loop nest");
+                        current[data] = value;
+                        continue;
+                    }
+                    OperandWalk w;
+                    if (loops.empty() || !walk_of(*block, *e, node, loops, &w) || w.scalar)
+                        refuse(*block, "operand '" + data + "' is not a dense tensor indexed by the loop variables");
+                    if (w.partial()) refuse(*block, "a result that some loops of the nest do not index");
+                    Array strides;
+                    std::string extent, key = data;
+                    layout_of(w, &strides, &extent, &key);
+                    write_keys[data].insert(key);
+                    auto at = write_at.find(key);
+                    if (at != write_at.end()) {
+                        writes[at->second].set("value", value);   // stored again: the later value stays
+                    } else {
+                        write_at[key] = writes.size();
+                        Value wv;
+                        const std::string connector = "_out" + std::to_string(writes.size());
+                        wv.set("connector", connector);
+                        wv.set("strides", Value(std::move(strides)));
+                        wv.set("extent", extent);
+                        wv.set("element_type", types::primitive_type_to_string(element));
+                        wv.set("value", value);
+                        writes.push_back(std::move(wv));
+                        Value b;
+                        b.set("data", data);
+                        b.set("connector", connector);
+                        outputs.push_back(std::move(b));
+                    }
+                    stored[key] = value;
+                }
+            }
+        }
+        if (writes.empty()) refuse(element, "a loop nest that stores nothing to a tensor");
+        // iterations are independent only if nobody reads or writes an element that another iteration writes
+        for (auto& kv : write_keys) {
+            if (kv.second.size() > 1) refuse(element, "'" + kv.first + "' is written through two different index forms in one nest");
+            auto r = read_keys.find(kv.first);
+            if (r != read_keys.end() && (r->second.size() > 1 || *r->second.begin() != *kv.second.begin()))
+                refuse(element, "'" + kv.first + "' is read at other elements than the one the iteration writes");
+        }
+        // the integer scalars that bounds and strides mention
+        Array symbols, indvars, bounds;
+        std::set<std::string> seen;
+        auto scan = [&](const std::string& text) {
+            std::string word;
+            auto flush = [&]() {
+                if (!word.empty() && !std::isdigit((unsigned char) word[0]) && !seen.count(word)) {
+                    bool is_var = false;
+                    for (auto& l : loops) is_var = is_var || l.var == word;
+                    if (!is_var) {
+                        bool exists = false;
+                        for (auto& kv : containers) exists = exists || kv.first == word;
+                        if (!exists || container(word).at("type").as_string() != "scalar")
+                            refuse(element, "'" + word + "' in a bound or an index is not a scalar of the function");
+                        seen.insert(word);
+                        symbols.emplace_back(word);
+                    }
+                }
+                word.clear();
+            };
+            for (char ch : text) {
+                if (std::isalnum((unsigned char) ch) || ch == '_') word += ch;
+                else flush();
+            }
+            flush();
+        };
+        for (auto& l : loops) {
+            indvars.emplace_back(l.var);
+            bounds.emplace_back(l.extent);
+            scan(l.extent);
+        }
+        for (auto* list : {&reads, &writes})
+            for (auto& a : *list)
+                for (auto& st : a.at("strides").as_array()) scan(st.as_string());
+        Value node{Object{}};
+        node.set("type", "library_node");
+        node.set("element_id", element.at("element_id").as_int());
+        node.set("code", rocm::LibraryNodeType_ROCM_Map);
+        node.set("implementation_type", "NONE");
+        node.set("side_effect", false);
+        node.set("indvars", Value(std::move(indvars)));
+        node.set("bounds", Value(std::move(bounds)));
+        node.set("symbols", Value(std::move(symbols)));
+        node.set("reads", Value(std::move(reads)));
+        node.set("writes", Value(std::move(writes)));
+        node.set("scalars", Value(std::move(scalars)));
+        node.set("statements", Value(std::move(statements)));
+        Value flow;
+        flow.set("library_node", std::move(node));
+        flow.set("inputs", Value(std::move(inputs)));
+        flow.set("outputs", Value(std::move(outputs)));
+        Value b;
+        b.set("type", "block");
+        b.set("element_id", body[0]->at("element_id").as_int());
+        Value dbg = debug_info_of(element);
+        if (!dbg.is_null()) b.set("debug_info", std::move(dbg));
+        b.set("dataflow", std::move(flow));
+        children.push_back(std::move(b));
     }
 
     // One block with one tasklet (or CMath node) under `loops` (none: a scalar statement).

@@ -38,7 +38,7 @@ bool is_math_node(const LibraryNode& node) {
     return c == blas::LibraryNodeType_GEMM || c == tensor::LibraryNodeType_Softmax || c == tensor::LibraryNodeType_Conv ||
            c == tensor::LibraryNodeType_MatMul || c == tensor::LibraryNodeType_Attention || c == tensor::LibraryNodeType_Broadcast ||
            c == tensor::LibraryNodeType_Transpose || c == tensor::LibraryNodeType_Cast || c == tensor::LibraryNodeType_Fill ||
-           c == blas::LibraryNodeType_DOT ||
+           c == blas::LibraryNodeType_DOT || c == LibraryNodeType_ROCM_Map ||
            std::find(tensor::ActivationNodeCodes.begin(), tensor::ActivationNodeCodes.end(), c) != tensor::ActivationNodeCodes.end() ||
            is_elementwise_code(c) || std::find(tensor::ReduceNodeCodes.begin(), tensor::ReduceNodeCodes.end(), c) != tensor::ReduceNodeCodes.end();
 }
@@ -719,6 +719,146 @@ protected:
     }
 };
 
+// ---- Map nests -------------------------------------------------------------------------------
+// Counterpart of CUDAMapDispatcher (reference opt/src/targets/cuda/cuda_map_dispatcher.cpp:42-262): the kernel goes
+// into a snippet file of its own (there "<kernel>.cu", compiled with nvcc by the driver and linked in,
+// py_structured_sdfg.cpp:445-466; here "<kernel>.hip", compiled to the code object "<kernel>.hsaco" that lies next
+// to the generated library), and the host side launches it - there `kernel<<<grid, block>>>(args)`, here the
+// runtime's module_load / module_get_function / launch, since the host code is compiled by a plain C++ compiler.
+
+class ROCMMapDispatcher : public RocmMathDispatcher {
+public:
+    using RocmMathDispatcher::RocmMathDispatcher;
+
+    void dispatch_code(PrettyPrinter& stream, PrettyPrinter& globals, CodeSnippetFactory& snippets) override {
+        globals_ = &globals;
+        snippets_ = &snippets;
+        RocmMathDispatcher::dispatch_code(stream, globals, snippets);
+    }
+
+protected:
+    const ROCMMapNode& map() const { return static_cast<const ROCMMapNode&>(node_); }
+
+    std::vector<DeviceOperand> operands() const override {
+        std::vector<DeviceOperand> ops;
+        for (auto& r : map().reads()) ops.push_back(operand(r.connector, true, false));
+        for (auto& w : map().writes()) ops.push_back(operand(w.connector, false, true));
+        return ops;
+    }
+
+    static void emit_loader(PrettyPrinter& globals) {
+        if (globals.str().find("__docc_rocm_map_kernel(") != std::string::npos) return;   // once per file
+        globals << "#include <dlfcn.h>" << std::endl;
+        globals << "#include <mutex>" << std::endl;
+        globals << "#include <string>" << std::endl;
+        globals << "namespace {" << std::endl;
+        globals << "// a generated kernel image and its entry points; the image lies next to this library" << std::endl;
+        globals << "struct __docc_rocm_map_image {" << std::endl;
+        globals << "    std::mutex mutex;" << std::endl;
+        globals << "    docc_rocm_module_t module = nullptr;" << std::endl;
+        globals << "    docc_rocm_function_t functions[4] = {nullptr, nullptr, nullptr, nullptr};" << std::endl;
+        globals << "};" << std::endl;
+        globals << "int __docc_rocm_map_kernel(__docc_rocm_map_image &image, const char *file, const char *name, int slot, docc_rocm_function_t *function) {" << std::endl;
+        globals << "    std::lock_guard<std::mutex> lock(image.mutex);" << std::endl;
+        globals << "    if (!image.module) {" << std::endl;
+        globals << "        std::string path = file;" << std::endl;
+        globals << "        Dl_info info;" << std::endl;
+        globals << "        if (dladdr((const void *) &__docc_rocm_map_kernel, &info) && info.dli_fname) {" << std::endl;
+        globals << "            const std::string lib = info.dli_fname;" << std::endl;
+        globals << "            const size_t slash = lib.find_last_of('/');" << std::endl;
+        globals << "            if (slash != std::string::npos) path = lib.substr(0, slash + 1) + file;" << std::endl;
+        globals << "        }" << std::endl;
+        globals << "        const int rc = docc_rocm_module_load(path.c_str(), &image.module);" << std::endl;
+        globals << "        if (rc != 0) return rc;" << std::endl;
+        globals << "    }" << std::endl;
+        globals << "    if (!image.functions[slot]) {" << std::endl;
+        globals << "        const int rc = docc_rocm_module_get_function(image.module, name, &image.functions[slot]);" << std::endl;
+        globals << "        if (rc != 0) return rc;" << std::endl;
+        globals << "    }" << std::endl;
+        globals << "    *function = image.functions[slot];" << std::endl;
+        globals << "    return 0;" << std::endl;
+        globals << "}" << std::endl;
+        globals << "} // namespace" << std::endl;
+    }
+
+    void emit_launch(PrettyPrinter& s, const std::function<std::string(const std::string&)>& name_of) override {
+        const auto& n = map();
+        for (auto& sym : n.symbols())
+            if (!function_.exists(sym) || function_.container(sym).is_pointer)
+                throw std::runtime_error("ROCMMap: '" + sym + "' in a bound or a stride is not a scalar of the function");
+        // the reference's kernel name (cuda_map_dispatcher.cpp:135)
+        const std::string kernel = "kernel_" + function_.name() + "_" + std::to_string(node_.element_id());
+        const RocmMapKernelPlan plan = plan_rocm_map_kernel(n, kernel);
+        auto& snippet = snippets_->require(kernel, "hip", true).stream();
+        if (snippet.str().empty()) snippet << plan.source;
+        emit_loader(*globals_);
+        *globals_ << "static __docc_rocm_map_image __docc_image_" << kernel << ";" << std::endl;
+
+        const size_t depth = plan.bounds.size();
+        const int V = plan.vector_width;
+        s << "{" << std::endl;
+        s.setIndent(s.indent() + 4);
+        for (size_t l = 0; l < depth; l++) s << "long long __docc_b" << l << " = (long long) (" << plan.bounds[l] << ");" << std::endl;
+        s << "bool __docc_empty = false, __docc_wide = false;" << std::endl;
+        for (size_t l = 0; l < depth; l++) s << "__docc_empty = __docc_empty || __docc_b" << l << " <= 0;" << std::endl;
+        // 32-bit indices when every operand and the iteration count stay below 2^31
+        for (auto& op : plan.operands) s << "__docc_wide = __docc_wide || (long long) (" << op.extent << ") > 0x7fffffffLL;" << std::endl;
+        s << "if (!__docc_empty) {" << std::endl;
+        s.setIndent(s.indent() + 4);
+        for (auto& op : plan.operands)
+            s << (op.write ? "" : "const ") << (op.element == types::PrimitiveType::Double ? "double" : "float") << " *__docc_p_" << op.connector
+              << " = (" << (op.write ? "" : "const ") << (op.element == types::PrimitiveType::Double ? "double" : "float") << " *) " << name_of(op.connector) << ";" << std::endl;
+        for (auto& op : plan.operands)
+            for (size_t l = 0; l < depth; l++)
+                if (op.strides[l] != "0" && op.strides[l] != "1")
+                    s << "long long __docc_st_" << op.connector << "_" << l << " = (long long) (" << op.strides[l] << ");" << std::endl;
+        if (V > 1) {
+            s << "bool __docc_vector = __docc_b" << depth - 1 << " % " << V << " == 0;" << std::endl;
+            for (auto& op : plan.operands)
+                if (op.vector)
+                    s << "__docc_vector = __docc_vector && ((uintptr_t) __docc_p_" << op.connector << ") % "
+                      << V * (op.element == types::PrimitiveType::Double ? 8 : 4) << " == 0;" << std::endl;
+        } else {
+            s << "const bool __docc_vector = false;" << std::endl;
+        }
+        s << "unsigned long long __docc_threads = (unsigned long long) (__docc_vector ? __docc_b" << depth - 1 << " / " << V << " : __docc_b" << depth - 1 << ");" << std::endl;
+        for (size_t l = 0; l + 1 < depth; l++) s << "__docc_threads *= (unsigned long long) __docc_b" << l << ";" << std::endl;
+        s << "__docc_wide = __docc_wide || __docc_threads > 0x7fffffffULL;" << std::endl;
+        s << "const unsigned long long __docc_groups = (__docc_threads + 255) / 256;" << std::endl;
+        s << "if (__docc_groups > 0x7fffffffULL) {" << std::endl;
+        s << "    docc_rocm_report_failure(__func__, \"" << kernel << ": more than 2^31 work-groups\", DOCC_ROCM_ERR_UNSUPPORTED);" << std::endl;
+        s << "    DOCC_ROCM_ON_FAILURE;" << std::endl;
+        s << "}" << std::endl;
+        s << "static const char *const __docc_names[4] = {\"" << kernel << "_s32\", \"" << kernel << "_s64\", \"" << kernel << "_v32\", \"" << kernel << "_v64\"};" << std::endl;
+        s << "const int __docc_slot = (__docc_vector ? 2 : 0) + (__docc_wide ? 1 : 0);" << std::endl;
+        s << "docc_rocm_function_t __docc_fn = nullptr;" << std::endl;
+        s << "DOCC_ROCM_CHECK(__docc_rocm_map_kernel(__docc_image_" << kernel << ", \"" << kernel << ".hsaco\", __docc_names[__docc_slot], __docc_slot, &__docc_fn));" << std::endl;
+        s << "void *__docc_args[] = {";
+        bool first = true;
+        auto arg = [&](const std::string& name) {
+            s << (first ? "" : ", ") << "(void *) &" << name;
+            first = false;
+        };
+        for (auto& op : plan.operands) arg("__docc_p_" + op.connector);
+        for (auto& sc : n.scalars()) arg(sc.connector);
+        for (size_t l = 0; l < depth; l++) arg("__docc_b" + std::to_string(l));
+        for (auto& op : plan.operands)
+            for (size_t l = 0; l < depth; l++)
+                if (op.strides[l] != "0" && op.strides[l] != "1") arg("__docc_st_" + op.connector + "_" + std::to_string(l));
+        s << "};" << std::endl;
+        s << "const uint32_t __docc_grid[3] = {(uint32_t) __docc_groups, 1, 1}, __docc_block[3] = {256, 1, 1};" << std::endl;
+        s << "DOCC_ROCM_CHECK(docc_rocm_launch(__docc_fn, __docc_grid, __docc_block, 0, nullptr, __docc_args));" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+        s.setIndent(s.indent() - 4);
+        s << "}" << std::endl;
+    }
+
+private:
+    PrettyPrinter* globals_ = nullptr;
+    CodeSnippetFactory* snippets_ = nullptr;
+};
+
 template <typename D>
 void register_math(codegen::LibraryNodeDispatcherRegistry& reg, const std::string& code) {
     for (bool with : {true, false}) {
@@ -756,6 +896,7 @@ void register_plugin(plugins::Context& context) {
     register_math<CastNodeDispatcher_ROCM>(reg, tensor::LibraryNodeType_Cast);
     for (auto& code : tensor::ReduceNodeCodes) register_math<ReduceNodeDispatcher_ROCM>(reg, code);
     register_math<FusedElementWiseDispatcher_ROCM>(reg, LibraryNodeType_ROCM_FusedElementWise);
+    register_math<ROCMMapDispatcher>(reg, LibraryNodeType_ROCM_Map);
     reg.register_library_node_dispatcher(
         LibraryNodeType_ROCM_Offloading + "::" + ImplementationType_NONE,
         [](LanguageExtension& le, const Function& f, const DataFlowGraph& b, const LibraryNode& n) {
@@ -843,6 +984,9 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!cast_is_built(cast_type_code(c->element()), cast_type_code(c->target_type())))
             return decline(std::string("conversion ") + types::primitive_type_to_string(c->element()) + " -> " +
                            types::primitive_type_to_string(c->target_type()) + " is not built");
+    } else if (node.code() == LibraryNodeType_ROCM_Map) {
+        // a nest of maps over dense tensors: always has a kernel, it is generated for the node
+        if (!dynamic_cast<ROCMMapNode*>(&node)) return decline("not a ROCMMap node object");
     } else if (node.code() == tensor::LibraryNodeType_Transpose) {
         auto* t = dynamic_cast<tensor::TransposeNode*>(&node);
         if (!t) return decline("not a Transpose node object");

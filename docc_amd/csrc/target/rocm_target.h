@@ -93,6 +93,30 @@ public:
     bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
 };
 
+// The kernel a ROCMMap node becomes (map_kernel.cpp) and what the host side needs to launch it: the loops as the
+// kernel sees them (adjacent loops that every operand walks as one are merged), the operands in parameter order,
+// and the source text. Kernel parameters: one pointer per operand, the scalar operands by value, one `long long` per
+// bound, then one `long long` per stride that is neither 0 nor 1 (operand by operand, loop by loop). The text defines
+// `<kernel_name>_s32` / `_s64` (one iteration per thread, indices in 32 / 64 bits) and, when some operand is contiguous
+// along the innermost loop, `_v32` / `_v64` (`vector_width` iterations per thread, 128-bit accesses).
+struct RocmMapKernelPlan {
+    struct Operand {
+        std::string connector;
+        bool write;
+        types::PrimitiveType element;
+        std::vector<Expression> strides;   // per merged loop
+        Expression extent;
+        bool vector;                       // contiguous along the innermost loop
+        bool streamed;                     // no loop repeats it
+    };
+    std::string kernel_name;
+    std::vector<Expression> bounds;
+    std::vector<Operand> operands;
+    int vector_width = 1;
+    std::string source;
+};
+RocmMapKernelPlan plan_rocm_map_kernel(const ROCMMapNode& node, const std::string& kernel_name);
+
 struct ScheduleOptions {
     // "function": nodes run WithoutTransfers between hoisted, minimised transfers (default)
     // "node":     every node copies its operands itself (ROCMWithTransfers)

@@ -823,6 +823,178 @@ Expression ROCMFusedElementWiseNode::connector_bytes(const std::string& connecto
     return bytes_of(s.empty() ? Expression("1") : product(s, 0, s.size()), element_);
 }
 
+// ---- ROCMMap
+
+namespace {
+std::vector<std::string> map_inputs(const std::vector<ROCMMapNode::Access>& reads, const std::vector<ROCMMapNode::ScalarOperand>& scalars) {
+    std::vector<std::string> names;
+    for (auto& r : reads) names.push_back(r.connector);
+    for (auto& s : scalars) names.push_back(s.connector);
+    return names;
+}
+std::vector<std::string> map_outputs(const std::vector<ROCMMapNode::Access>& writes) {
+    std::vector<std::string> names;
+    for (auto& w : writes) names.push_back(w.connector);
+    return names;
+}
+const std::map<std::string, int>& map_operations() {
+    static const std::map<std::string, int> ops = {
+        {"assign", 1}, {"fp_neg", 1}, {"fp_add", 2}, {"fp_sub", 2}, {"fp_mul", 2}, {"fp_div", 2}, {"fp_rem", 2}, {"fp_fma", 3},
+        // CMath stems (reference cmath_node.h:21-96) that take and return the element type
+        {"sin", 1}, {"cos", 1}, {"tan", 1}, {"asin", 1}, {"acos", 1}, {"atan", 1}, {"atan2", 2}, {"sinh", 1}, {"cosh", 1}, {"tanh", 1},
+        {"asinh", 1}, {"acosh", 1}, {"atanh", 1}, {"exp", 1}, {"exp2", 1}, {"exp10", 1}, {"expm1", 1}, {"log", 1}, {"log10", 1},
+        {"log2", 1}, {"log1p", 1}, {"pow", 2}, {"sqrt", 1}, {"cbrt", 1}, {"hypot", 2}, {"erf", 1}, {"erfc", 1}, {"tgamma", 1},
+        {"lgamma", 1}, {"fabs", 1}, {"ceil", 1}, {"floor", 1}, {"trunc", 1}, {"round", 1}, {"nearbyint", 1}, {"rint", 1},
+        {"fmod", 2}, {"remainder", 2}, {"copysign", 2}, {"fmax", 2}, {"fmin", 2}, {"fdim", 2}, {"fma", 3}};
+    return ops;
+}
+} // namespace
+
+ROCMMapNode::ROCMMapNode(std::string implementation_type, std::vector<std::string> indvars, std::vector<Expression> bounds,
+                         std::vector<std::string> symbols, std::vector<Access> reads, std::vector<Access> writes,
+                         std::vector<ScalarOperand> scalars, std::vector<Statement> statements)
+    : LibraryNode(LibraryNodeType_ROCM_Map, map_outputs(writes), map_inputs(reads, scalars), false, std::move(implementation_type)),
+      indvars_(std::move(indvars)), bounds_(std::move(bounds)), symbols_(std::move(symbols)), reads_(std::move(reads)),
+      writes_(std::move(writes)), scalars_(std::move(scalars)), statements_(std::move(statements)) {}
+
+int ROCMMapNode::arity(const std::string& op) {
+    auto it = map_operations().find(op);
+    return it == map_operations().end() ? -1 : it->second;
+}
+
+bool ROCMMapNode::is_cmath(const std::string& op) { return arity(op) >= 0 && op != "assign" && op.rfind("fp_", 0) != 0; }
+
+void ROCMMapNode::validate() const {
+    using P = types::PrimitiveType;
+    auto floating = [](P t) { return t == P::Float || t == P::Double; };
+    if (indvars_.empty() || indvars_.size() > 6 || indvars_.size() != bounds_.size())
+        throw InvalidSDFGException(code_ + ": one bound per induction variable, 1..6 of them");
+    if (writes_.empty()) throw InvalidSDFGException(code_ + ": a nest that stores nothing");
+    std::vector<std::string> defined;
+    auto define = [&](const std::string& name) {
+        if (name.empty() || name[0] == '#' || std::find(defined.begin(), defined.end(), name) != defined.end())
+            throw InvalidSDFGException(code_ + ": name '" + name + "' is empty, a literal, or defined twice");
+        defined.push_back(name);
+    };
+    for (auto* list : {&reads_, &writes_})
+        for (auto& a : *list) {
+            if (a.strides.size() != indvars_.size()) throw InvalidSDFGException(code_ + ": operand " + a.connector + " needs one stride per induction variable");
+            if (!floating(a.element)) throw InvalidSDFGException(code_ + ": operand " + a.connector + " must be Float or Double");
+        }
+    for (auto& r : reads_) define(r.connector);
+    for (auto& s : scalars_) {
+        if (!floating(s.element)) throw InvalidSDFGException(code_ + ": scalar " + s.connector + " must be Float or Double");
+        define(s.connector);
+    }
+    auto known = [&](const std::string& name) {
+        return (name.size() > 1 && name[0] == '#') || std::find(defined.begin(), defined.end(), name) != defined.end();
+    };
+    for (auto& st : statements_) {
+        const int n = arity(st.op);
+        if (n < 0) throw InvalidSDFGException(code_ + ": unknown operation '" + st.op + "'");
+        if ((int) st.args.size() != n) throw InvalidSDFGException(code_ + ": operation " + st.op + " takes " + std::to_string(n) + " arguments");
+        if (!floating(st.type)) throw InvalidSDFGException(code_ + ": statement " + st.out + " must be Float or Double");
+        for (auto& a : st.args)
+            if (!known(a)) throw InvalidSDFGException(code_ + ": statement " + st.out + " uses '" + a + "' before it is defined");
+        define(st.out);
+    }
+    for (auto& w : writes_) {
+        if (!known(w.value)) throw InvalidSDFGException(code_ + ": " + w.connector + " stores '" + w.value + "', which nothing defines");
+        for (auto& other : writes_)
+            if (&other != &w && other.connector == w.connector) throw InvalidSDFGException(code_ + ": connector " + w.connector + " written twice");
+    }
+}
+
+Expression ROCMMapNode::flop() const {
+    size_t ops = 0;
+    for (auto& st : statements_) ops += st.op == "assign" ? 0 : st.op == "fp_fma" || st.op == "fma" ? 2 : 1;
+    return symbolic::mul(std::to_string(ops), product(bounds_, 0, bounds_.size()));
+}
+
+void ROCMMapNode::to_json(Value& j) const {
+    auto names = [](const std::vector<std::string>& v) {
+        Array a;
+        for (auto& n : v) a.emplace_back(n);
+        return Value(std::move(a));
+    };
+    auto accesses = [&](const std::vector<Access>& list, bool with_value) {
+        Array out;
+        for (auto& a : list) {
+            Value v;
+            v.set("connector", a.connector);
+            v.set("strides", exprs_to_json(a.strides));
+            v.set("extent", a.extent);
+            v.set("element_type", types::primitive_type_to_string(a.element));
+            if (with_value) v.set("value", a.value);
+            out.push_back(std::move(v));
+        }
+        return Value(std::move(out));
+    };
+    j.set("indvars", names(indvars_));
+    j.set("bounds", exprs_to_json(bounds_));
+    j.set("symbols", names(symbols_));
+    j.set("reads", accesses(reads_, false));
+    j.set("writes", accesses(writes_, true));
+    Array scalars;
+    for (auto& s : scalars_) {
+        Value v;
+        v.set("connector", s.connector);
+        v.set("element_type", types::primitive_type_to_string(s.element));
+        scalars.push_back(std::move(v));
+    }
+    j.set("scalars", Value(std::move(scalars)));
+    Array statements;
+    for (auto& st : statements_) {
+        Value v;
+        v.set("out", st.out);
+        v.set("type", types::primitive_type_to_string(st.type));
+        v.set("op", st.op);
+        v.set("args", names(st.args));
+        statements.push_back(std::move(v));
+    }
+    j.set("statements", Value(std::move(statements)));
+}
+
+std::unique_ptr<ROCMMapNode> ROCMMapNode::from_json(const Value& j) {
+    auto names = [](const Value& v) {
+        std::vector<std::string> out;
+        for (auto& n : v.as_array()) out.push_back(n.as_string());
+        return out;
+    };
+    auto accesses = [&](const Value& v, bool with_value) {
+        std::vector<Access> out;
+        for (auto& a : v.as_array()) {
+            Access acc;
+            acc.connector = a.at("connector").as_string();
+            acc.strides = exprs_from_json(a.at("strides"));
+            acc.extent = a.at("extent").as_expression();
+            acc.element = types::primitive_type_from_string(a.at("element_type").as_string());
+            if (with_value) acc.value = a.at("value").as_string();
+            out.push_back(std::move(acc));
+        }
+        return out;
+    };
+    std::vector<ScalarOperand> scalars;
+    for (auto& s : j.at("scalars").as_array())
+        scalars.push_back({s.at("connector").as_string(), types::primitive_type_from_string(s.at("element_type").as_string())});
+    std::vector<Statement> statements;
+    for (auto& s : j.at("statements").as_array())
+        statements.push_back({s.at("out").as_string(), types::primitive_type_from_string(s.at("type").as_string()), s.at("op").as_string(),
+                              names(s.at("args"))});
+    return std::make_unique<ROCMMapNode>(impl_of(j), names(j.at("indvars")), exprs_from_json(j.at("bounds")), names(j.at("symbols")),
+                                         accesses(j.at("reads"), false), accesses(j.at("writes"), true), std::move(scalars),
+                                         std::move(statements));
+}
+
+Expression ROCMMapNode::connector_bytes(const std::string& connector) const {
+    for (auto* list : {&reads_, &writes_})
+        for (auto& a : *list)
+            if (a.connector == connector) return bytes_of(a.extent, a.element);
+    for (auto& s : scalars_)
+        if (s.connector == connector) return bytes_of("1", s.element);
+    throw InvalidSDFGException(code_ + ": no connector '" + connector + "'");
+}
+
 ROCMDataOffloadingNode::ROCMDataOffloadingNode(Expression size, int device_id, DataTransferDirection direction,
                                                BufferLifecycle lifecycle)
     : LibraryNode(LibraryNodeType_ROCM_Offloading, offload_outputs(direction, lifecycle), offload_inputs(direction, lifecycle),
@@ -1142,6 +1314,7 @@ LibraryNodeSerializerRegistry::LibraryNodeSerializerRegistry() {
     fns_[math::blas::LibraryNodeType_DOT] = &deserialize<math::blas::DotNode>;
     for (auto& code : math::tensor::ReduceNodeCodes) fns_[code] = &deserialize<math::tensor::ReduceNode>;
     fns_[rocm::LibraryNodeType_ROCM_FusedElementWise] = &deserialize<rocm::ROCMFusedElementWiseNode>;
+    fns_[rocm::LibraryNodeType_ROCM_Map] = &deserialize<rocm::ROCMMapNode>;
 }
 
 LibraryNodeSerializerRegistry& LibraryNodeSerializerRegistry::instance() {

@@ -573,6 +573,74 @@ private:
     std::vector<std::string> post_;
 };
 
+// A perfect nest of Maps (from 0, step 1, `indvar < bound`) whose body is a chain of tasklets and CMath calls over
+// dense tensors: what the reference hands to its CUDAMapDispatcher (opt/src/targets/cuda/cuda_map_dispatcher.cpp:42-262)
+// as a Map element with a body sequence. The block list has no nested control flow, so the nest travels as one node
+// that spells the body out:
+//   reads   - tensor elements loaded once per iteration: connector, one stride per induction variable ("0": the
+//             variable does not index the operand, i.e. it is repeated along that loop), element count, element type;
+//   scalars - values passed to the kernel by value (scalar containers, constants bound to a connector);
+//   statements - in order: `out = op(args)`; an argument names a read or scalar connector, the `out` of an earlier
+//             statement, or a literal spelled "#<text>"; `op` is a tasklet code by name (assign, fp_neg, fp_add, fp_sub,
+//             fp_mul, fp_div, fp_rem, fp_fma: reference sdfg/include/sdfg/data_flow/tasklet.h:94-153) or the stem of
+//             a CMath function (cmath_node.h:21-96);
+//   writes  - tensor elements stored once per iteration, each naming the value it stores;
+//   symbols - the integer scalar containers that bounds and strides mention.
+// Written by the importer of docc's JSON for nests that are not one of the prebuilt kernels
+// (serializer::import_reference_json); dispatched by ROCMMapDispatcher as a generated gfx950 kernel.
+inline const std::string LibraryNodeType_ROCM_Map = "ROCMMap";
+
+class ROCMMapNode : public data_flow::LibraryNode {
+public:
+    struct Access {
+        std::string connector;
+        std::vector<Expression> strides;   // elements, one per induction variable
+        Expression extent;                 // elements the operand spans
+        types::PrimitiveType element;
+        std::string value;                 // writes: the statement result (or read / scalar) stored
+    };
+    struct ScalarOperand {
+        std::string connector;
+        types::PrimitiveType element;
+    };
+    struct Statement {
+        std::string out;
+        types::PrimitiveType type;
+        std::string op;
+        std::vector<std::string> args;
+    };
+
+    ROCMMapNode(std::string implementation_type, std::vector<std::string> indvars, std::vector<Expression> bounds,
+                std::vector<std::string> symbols, std::vector<Access> reads, std::vector<Access> writes,
+                std::vector<ScalarOperand> scalars, std::vector<Statement> statements);
+
+    const std::vector<std::string>& indvars() const { return indvars_; }
+    const std::vector<Expression>& bounds() const { return bounds_; }
+    const std::vector<std::string>& symbols() const { return symbols_; }
+    const std::vector<Access>& reads() const { return reads_; }
+    const std::vector<Access>& writes() const { return writes_; }
+    const std::vector<ScalarOperand>& scalars() const { return scalars_; }
+    const std::vector<Statement>& statements() const { return statements_; }
+
+    // number of arguments of a body operation, or -1 for one the kernels cannot spell
+    static int arity(const std::string& op);
+    static bool is_cmath(const std::string& op);
+
+    void validate() const override;
+    Expression flop() const override;
+    void to_json(json::Value& j) const override;
+    Expression connector_bytes(const std::string& connector) const override;
+    static std::unique_ptr<ROCMMapNode> from_json(const json::Value& j);
+
+private:
+    std::vector<std::string> indvars_;
+    std::vector<Expression> bounds_;
+    std::vector<std::string> symbols_;
+    std::vector<Access> reads_, writes_;
+    std::vector<ScalarOperand> scalars_;
+    std::vector<Statement> statements_;
+};
+
 } // namespace rocm
 
 namespace data_flow {

@@ -85,6 +85,30 @@ Generated generate(StructuredSDFG& sdfg, const char* output_dir, const char* ins
 
 std::string quote(const std::string& s) { return "'" + s + "'"; }
 
+std::string device_compiler() {
+    if (const char* hipcc = std::getenv("DOCC_HIPCC"))
+        if (*hipcc) return hipcc;
+    const char* rocm = std::getenv("ROCM_PATH");
+    return (std::filesystem::path(rocm && *rocm ? rocm : "/opt/rocm") / "bin" / "hipcc").string();
+}
+
+// The kernels the map dispatcher wrote ("<kernel>.hip") become code objects next to the library ("<kernel>.hsaco"),
+// one compiler process per file, as the reference's driver compiles its ".cu" snippets
+// (python/bindings/py_structured_sdfg.cpp:445-466). No contraction of separate statements into fused multiply-adds:
+// every tasklet rounds by itself, as in the host code the reference generates. Packed fp32 instructions are switched
+// off as for every kernel of this target.
+void compile_device_snippets(const Generated& g, const std::filesystem::path& log) {
+    for (auto& file : g.snippet_files) {
+        if (file.extension() != ".hip") continue;
+        std::filesystem::path object = file;
+        object.replace_extension(".hsaco");
+        const std::string cmd = device_compiler() + " --genco --offload-arch=gfx950 -O3 -std=c++17 -ffp-contract=off "
+                                "-Xclang -target-feature -Xclang -packed-fp32-ops -Wno-unused-command-line-argument " +
+                                quote(file.string()) + " -o " + quote(object.string()) + " >> " + quote(log.string()) + " 2>&1";
+        if (std::system(cmd.c_str()) != 0) throw std::runtime_error("Compilation failed: " + cmd);
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -196,6 +220,7 @@ char* docc_rocm_target_compile(const char* sdfg_json, const char* output_dir, co
         std::string compile = cxx + " -c -fPIC -O3 -march=native -mtune=native -funroll-loops -std=c++17 -I" + quote(include_dir) +
                               " " + quote(g.source.string()) + " -o " + quote(object.string()) + " > " + quote(log.string()) + " 2>&1";
         if (std::system(compile.c_str()) != 0) throw std::runtime_error("Compilation failed: " + compile);
+        compile_device_snippets(g, log);
         const std::filesystem::path lib = dir / ("lib" + sdfg->name() + ".so");
         std::string link = cxx + " -shared " + quote(object.string()) + " -o " + quote(lib.string()) + " -L" + quote(runtime_lib_dir) +
                            (instrumented ? " -ldocc_rtl_rocm" : "") + " -ldocc_rt_rocm -Wl,-rpath," + quote(runtime_lib_dir) + " -lm -lstdc++ >> " + quote(log.string()) + " 2>&1";

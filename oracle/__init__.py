@@ -368,3 +368,97 @@ def cast(X, dtype) -> np.ndarray:
         return bf16_to_f32(X).astype(dtype, copy=False)
     with np.errstate(all="ignore"):
         return X.astype(dtype)
+
+
+def _literal(text: str) -> float:
+    """A constant as generated C spells it: "0.5f", "3.0", "-INFINITY", "(2.0)"."""
+    t = text.strip()
+    while t.startswith("(") and t.endswith(")"):
+        t = t[1:-1].strip()
+    sign = 1.0
+    if t.startswith("-"):
+        sign, t = -1.0, t[1:].strip()
+    if t in ("INFINITY", "HUGE_VAL", "HUGE_VALF"):
+        return sign * float("inf")
+    if t in ("NAN",):
+        return float("nan")
+    if t.endswith(("f", "F")) and not t.lower().startswith("0x"):
+        return sign * float(np.float32(float(t[:-1])))
+    return sign * float(t)
+
+
+def map_nest(node: dict, operands: dict, scalars: dict | None = None, symbols: dict | None = None, lib=None) -> dict:
+    """Runs a ROCMMap node's body (the payload the importer writes: indvars, bounds, reads, scalars, statements,
+    writes) the way the reference's openmp target would print the nest: nested loops, one statement per tasklet.
+    operands: connector -> flat numpy array (reads and writes; arrays of writes are updated in place and returned);
+    scalars: connector -> value; symbols: name -> integer, for bounds and strides. Returns {write connector: array}."""
+    lib = lib or load()
+    lib.oracle_map_nest.restype = ctypes.c_int
+    symbols = {k: int(v) for k, v in (symbols or {}).items()}
+    ev = lambda e: int(eval(str(e), {"__builtins__": {}}, symbols))
+    depth = len(node["indvars"])
+    bounds = (ctypes.c_int64 * depth)(*[ev(b) for b in node["bounds"]])
+    np_type = lambda name: np.float64 if name == "Double" else np.float32
+    slots: dict = {}
+    reads = node["reads"]
+    keep = []
+    read_ptrs = (ctypes.c_void_p * max(1, len(reads)))()
+    read_strides = (ctypes.c_int64 * max(1, len(reads) * depth))()
+    read_f64 = (ctypes.c_int * max(1, len(reads)))()
+    for r, acc in enumerate(reads):
+        a = np.ascontiguousarray(operands[acc["connector"]], dtype=np_type(acc["element_type"])).reshape(-1)
+        if a.size < ev(acc["extent"]):
+            raise ValueError(f"operand {acc['connector']} holds {a.size} elements, the nest walks {ev(acc['extent'])}")
+        keep.append(a)
+        read_ptrs[r] = a.ctypes.data
+        read_f64[r] = int(acc["element_type"] == "Double")
+        for l in range(depth):
+            read_strides[r * depth + l] = ev(acc["strides"][l])
+        slots[acc["connector"]] = r
+    consts = []
+    for sc in node.get("scalars", []):
+        slots[sc["connector"]] = len(reads) + len(consts)
+        v = (scalars or {})[sc["connector"]]
+        consts.append(float(np.float32(v)) if sc["element_type"] != "Double" else float(v))
+    stmts = node["statements"]
+    for st in stmts:                      # literals become constants too
+        for a in st["args"]:
+            if a.startswith("#") and a not in slots:
+                slots[a] = len(reads) + len(consts)
+                consts.append(_literal(a[1:]))
+    for w in node["writes"]:
+        if w["value"].startswith("#") and w["value"] not in slots:
+            slots[w["value"]] = len(reads) + len(consts)
+            consts.append(_literal(w["value"][1:]))
+    base = len(reads) + len(consts)
+    ops = (ctypes.c_char_p * max(1, len(stmts)))()
+    stmt_f64 = (ctypes.c_int * max(1, len(stmts)))()
+    stmt_args = (ctypes.c_int * max(1, 3 * len(stmts)))(*([-1] * max(1, 3 * len(stmts))))
+    for s, st in enumerate(stmts):
+        ops[s] = st["op"].encode()
+        stmt_f64[s] = int(st["type"] == "Double")
+        for k, a in enumerate(st["args"]):
+            stmt_args[3 * s + k] = slots[a]
+        slots[st["out"]] = base + s
+    writes = node["writes"]
+    out = {}
+    write_ptrs = (ctypes.c_void_p * len(writes))()
+    write_strides = (ctypes.c_int64 * (len(writes) * depth))()
+    write_f64 = (ctypes.c_int * len(writes))()
+    write_slots = (ctypes.c_int * len(writes))()
+    for w, acc in enumerate(writes):
+        dt = np_type(acc["element_type"])
+        given = operands.get(acc["connector"])
+        a = np.zeros(ev(acc["extent"]), dt) if given is None else np.ascontiguousarray(given, dtype=dt).reshape(-1)
+        out[acc["connector"]] = a
+        write_ptrs[w] = a.ctypes.data
+        write_f64[w] = int(acc["element_type"] == "Double")
+        write_slots[w] = slots[acc["value"]]
+        for l in range(depth):
+            write_strides[w * depth + l] = ev(acc["strides"][l])
+    cv = (ctypes.c_double * max(1, len(consts)))(*consts)
+    rc = lib.oracle_map_nest(depth, bounds, len(reads), read_ptrs, read_strides, read_f64, len(consts), cv, len(stmts), ops, stmt_f64,
+                             stmt_args, len(writes), write_ptrs, write_strides, write_f64, write_slots)
+    if rc != 0:
+        raise ValueError("oracle_map_nest: a depth outside 1..8, an unknown operation or a value used before it is computed")
+    return out

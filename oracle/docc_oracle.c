@@ -659,3 +659,154 @@ ORACLE_API int oracle_transpose(int element_bytes, int rank, const int64_t* shap
     }
     return 0;
 }
+
+
+/* ------------------------------------------------------- Map nests (tasklet bodies) */
+
+/*
+ * A perfect nest of Maps whose body is a chain of tasklets and CMath calls, as the reference's openmp target prints
+ * it: the outermost Map becomes `#pragma omp parallel for schedule(static)` (opt/src/targets/omp/codegen/
+ * omp_map_dispatcher.cpp:46-82), the inner ones plain `for` loops, and every tasklet a statement of its own
+ *     <type> _out = <expression over the input connectors>;
+ * (sdfg/src/codegen/dispatchers/block_dispatcher.cpp:219-331 with the expressions of
+ * sdfg/src/codegen/language_extensions/cpp_language_extension.cpp:186-239), so every operation rounds by itself to the
+ * type of its result; only fp_fma, printed as `a * b + c` in one expression, is contracted by the compiler into one
+ * fused multiply-add. CMath nodes print the libm call of their stem, with the `f` suffix for float
+ * (sdfg/src/data_flow/library_nodes/math/cmath/cmath_node.cpp).
+ *
+ * The body is handed over as a small program. Value slots: first the `n_reads` tensor elements loaded by the
+ * iteration, then the `n_consts` constants (scalar operands and literals), then one slot per statement.
+ *   read r:   element type (`read_f64[r]`), base pointer, one stride in elements per loop (read_strides[r * depth + l])
+ *   statement s: operation name, result type (`stmt_f64[s]`), up to three argument slots (stmt_args[3 * s + k], -1: none)
+ *   write w:  the slot stored, element type, base pointer, strides
+ * Returns 0, or 1 for a depth outside 1..8, an unknown operation or a bad slot.
+ */
+enum oracle_map_op {
+    MAP_ASSIGN, MAP_NEG, MAP_ADD, MAP_SUB, MAP_MUL, MAP_DIV, MAP_REM, MAP_FMA,
+    MAP_SIN, MAP_COS, MAP_TAN, MAP_ASIN, MAP_ACOS, MAP_ATAN, MAP_ATAN2, MAP_SINH, MAP_COSH, MAP_TANH, MAP_ASINH, MAP_ACOSH, MAP_ATANH,
+    MAP_EXP, MAP_EXP2, MAP_EXP10, MAP_EXPM1, MAP_LOG, MAP_LOG10, MAP_LOG2, MAP_LOG1P, MAP_POW, MAP_SQRT, MAP_CBRT, MAP_HYPOT,
+    MAP_ERF, MAP_ERFC, MAP_TGAMMA, MAP_LGAMMA, MAP_FABS, MAP_CEIL, MAP_FLOOR, MAP_TRUNC, MAP_ROUND, MAP_NEARBYINT, MAP_RINT,
+    MAP_FMOD, MAP_REMAINDER, MAP_COPYSIGN, MAP_FMAX, MAP_FMIN, MAP_FDIM, MAP_OP_COUNT
+};
+static const char* const oracle_map_op_names[MAP_OP_COUNT] = {
+    "assign", "fp_neg", "fp_add", "fp_sub", "fp_mul", "fp_div", "fp_rem", "fp_fma",
+    "sin", "cos", "tan", "asin", "acos", "atan", "atan2", "sinh", "cosh", "tanh", "asinh", "acosh", "atanh",
+    "exp", "exp2", "exp10", "expm1", "log", "log10", "log2", "log1p", "pow", "sqrt", "cbrt", "hypot",
+    "erf", "erfc", "tgamma", "lgamma", "fabs", "ceil", "floor", "trunc", "round", "nearbyint", "rint",
+    "fmod", "remainder", "copysign", "fmax", "fmin", "fdim"};
+
+static float oracle_map_eval_f32(int op, float a, float b, float c) {
+    switch (op) {
+        case MAP_ASSIGN: return a;
+        case MAP_NEG: return -a;
+        case MAP_ADD: { volatile float r = a + b; return r; }
+        case MAP_SUB: { volatile float r = a - b; return r; }
+        case MAP_MUL: { volatile float r = a * b; return r; }
+        case MAP_DIV: return a / b;
+        case MAP_REM: case MAP_FMOD: return fmodf(a, b);
+        case MAP_FMA: return fmaf(a, b, c);
+        case MAP_SIN: return sinf(a); case MAP_COS: return cosf(a); case MAP_TAN: return tanf(a);
+        case MAP_ASIN: return asinf(a); case MAP_ACOS: return acosf(a); case MAP_ATAN: return atanf(a);
+        case MAP_ATAN2: return atan2f(a, b);
+        case MAP_SINH: return sinhf(a); case MAP_COSH: return coshf(a); case MAP_TANH: return tanhf(a);
+        case MAP_ASINH: return asinhf(a); case MAP_ACOSH: return acoshf(a); case MAP_ATANH: return atanhf(a);
+        case MAP_EXP: return expf(a); case MAP_EXP2: return exp2f(a); case MAP_EXP10: return powf(10.0f, a);
+        case MAP_EXPM1: return expm1f(a); case MAP_LOG: return logf(a); case MAP_LOG10: return log10f(a);
+        case MAP_LOG2: return log2f(a); case MAP_LOG1P: return log1pf(a); case MAP_POW: return powf(a, b);
+        case MAP_SQRT: return sqrtf(a); case MAP_CBRT: return cbrtf(a); case MAP_HYPOT: return hypotf(a, b);
+        case MAP_ERF: return erff(a); case MAP_ERFC: return erfcf(a); case MAP_TGAMMA: return tgammaf(a);
+        case MAP_LGAMMA: return lgammaf(a); case MAP_FABS: return fabsf(a); case MAP_CEIL: return ceilf(a);
+        case MAP_FLOOR: return floorf(a); case MAP_TRUNC: return truncf(a); case MAP_ROUND: return roundf(a);
+        case MAP_NEARBYINT: return nearbyintf(a); case MAP_RINT: return rintf(a);
+        case MAP_REMAINDER: return remainderf(a, b); case MAP_COPYSIGN: return copysignf(a, b);
+        case MAP_FMAX: return fmaxf(a, b); case MAP_FMIN: return fminf(a, b); case MAP_FDIM: return fdimf(a, b);
+    }
+    return NAN;
+}
+
+static double oracle_map_eval_f64(int op, double a, double b, double c) {
+    switch (op) {
+        case MAP_ASSIGN: return a;
+        case MAP_NEG: return -a;
+        case MAP_ADD: { volatile double r = a + b; return r; }
+        case MAP_SUB: { volatile double r = a - b; return r; }
+        case MAP_MUL: { volatile double r = a * b; return r; }
+        case MAP_DIV: return a / b;
+        case MAP_REM: case MAP_FMOD: return fmod(a, b);
+        case MAP_FMA: return fma(a, b, c);
+        case MAP_SIN: return sin(a); case MAP_COS: return cos(a); case MAP_TAN: return tan(a);
+        case MAP_ASIN: return asin(a); case MAP_ACOS: return acos(a); case MAP_ATAN: return atan(a);
+        case MAP_ATAN2: return atan2(a, b);
+        case MAP_SINH: return sinh(a); case MAP_COSH: return cosh(a); case MAP_TANH: return tanh(a);
+        case MAP_ASINH: return asinh(a); case MAP_ACOSH: return acosh(a); case MAP_ATANH: return atanh(a);
+        case MAP_EXP: return exp(a); case MAP_EXP2: return exp2(a); case MAP_EXP10: return pow(10.0, a);
+        case MAP_EXPM1: return expm1(a); case MAP_LOG: return log(a); case MAP_LOG10: return log10(a);
+        case MAP_LOG2: return log2(a); case MAP_LOG1P: return log1p(a); case MAP_POW: return pow(a, b);
+        case MAP_SQRT: return sqrt(a); case MAP_CBRT: return cbrt(a); case MAP_HYPOT: return hypot(a, b);
+        case MAP_ERF: return erf(a); case MAP_ERFC: return erfc(a); case MAP_TGAMMA: return tgamma(a);
+        case MAP_LGAMMA: return lgamma(a); case MAP_FABS: return fabs(a); case MAP_CEIL: return ceil(a);
+        case MAP_FLOOR: return floor(a); case MAP_TRUNC: return trunc(a); case MAP_ROUND: return round(a);
+        case MAP_NEARBYINT: return nearbyint(a); case MAP_RINT: return rint(a);
+        case MAP_REMAINDER: return remainder(a, b); case MAP_COPYSIGN: return copysign(a, b);
+        case MAP_FMAX: return fmax(a, b); case MAP_FMIN: return fmin(a, b); case MAP_FDIM: return fdim(a, b);
+    }
+    return NAN;
+}
+
+ORACLE_API int oracle_map_nest(int depth, const int64_t* bounds,
+                               int n_reads, const void* const* read_ptrs, const int64_t* read_strides, const int* read_f64,
+                               int n_consts, const double* consts,
+                               int n_stmts, const char* const* stmt_ops, const int* stmt_f64, const int* stmt_args,
+                               int n_writes, void* const* write_ptrs, const int64_t* write_strides, const int* write_f64, const int* write_slots) {
+    enum { MAX_SLOTS = 256 };
+    if (depth < 1 || depth > 8 || n_reads < 0 || n_consts < 0 || n_stmts < 0 || n_writes < 1) return 1;
+    const int n_slots = n_reads + n_consts + n_stmts;
+    if (n_slots > MAX_SLOTS) return 1;
+    int ops[MAX_SLOTS];
+    for (int s = 0; s < n_stmts; s++) {
+        ops[s] = -1;
+        for (int k = 0; k < MAP_OP_COUNT; k++)
+            if (strcmp(stmt_ops[s], oracle_map_op_names[k]) == 0) ops[s] = k;
+        if (strcmp(stmt_ops[s], "fma") == 0) ops[s] = MAP_FMA;
+        if (ops[s] < 0) return 1;
+        for (int k = 0; k < 3; k++)
+            if (stmt_args[3 * s + k] >= n_reads + n_consts + s) return 1;   /* only values computed before */
+    }
+    for (int w = 0; w < n_writes; w++)
+        if (write_slots[w] < 0 || write_slots[w] >= n_slots) return 1;
+    int64_t inner = 1;
+    for (int l = 1; l < depth; l++) inner *= bounds[l];
+#pragma omp parallel for schedule(static)
+    for (int64_t i0 = 0; i0 < bounds[0]; i0++) {
+        double slot[MAX_SLOTS];
+        for (int c = 0; c < n_consts; c++) slot[n_reads + c] = consts[c];
+        for (int64_t rest = 0; rest < inner; rest++) {
+            int64_t idx[8];
+            idx[0] = i0;
+            int64_t rem = rest;
+            for (int l = depth - 1; l >= 1; l--) {
+                idx[l] = rem % bounds[l];
+                rem /= bounds[l];
+            }
+            for (int r = 0; r < n_reads; r++) {
+                int64_t off = 0;
+                for (int l = 0; l < depth; l++) off += idx[l] * read_strides[r * depth + l];
+                slot[r] = read_f64[r] ? ((const double*) read_ptrs[r])[off] : (double) ((const float*) read_ptrs[r])[off];
+            }
+            for (int s = 0; s < n_stmts; s++) {
+                const int* a = stmt_args + 3 * s;
+                const double x = a[0] >= 0 ? slot[a[0]] : 0.0, y = a[1] >= 0 ? slot[a[1]] : 0.0, z = a[2] >= 0 ? slot[a[2]] : 0.0;
+                /* the inputs are converted to the type of the statement, then the operation rounds once */
+                slot[n_reads + n_consts + s] = stmt_f64[s] ? oracle_map_eval_f64(ops[s], x, y, z)
+                                                           : (double) oracle_map_eval_f32(ops[s], (float) x, (float) y, (float) z);
+            }
+            for (int w = 0; w < n_writes; w++) {
+                int64_t off = 0;
+                for (int l = 0; l < depth; l++) off += idx[l] * write_strides[w * depth + l];
+                if (write_f64[w]) ((double*) write_ptrs[w])[off] = slot[write_slots[w]];
+                else ((float*) write_ptrs[w])[off] = (float) slot[write_slots[w]];
+            }
+        }
+    }
+    return 0;
+}

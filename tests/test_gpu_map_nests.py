@@ -1,0 +1,172 @@
+"""Loop nests of maps that are not one of the prebuilt kernels, run as generated gfx950 kernels: a docc-layout program is
+imported (ROCMMap nodes), scheduled, its kernels are compiled with hipcc next to the generated library, and the host
+code launches them through docc_rocm_module_load / _module_get_function / _launch. Checked against the oracle's
+interpreter of the same body (the loop the reference's openmp target prints) and against numpy spelled by hand.
+
+The arithmetic tasklets are IEEE operations compiled without contraction: bit-exact. Calls into the math library
+(CMath): 1e-5 (fp32) / 1e-12 (fp64) norm-wise relative error."""
+import ctypes
+import json
+
+import numpy as np
+import pytest
+
+import oracle
+from docc_amd import runtime
+from docc_amd.sdfg import StructuredSDFG
+from gpu_util import rel_err_max
+from test_interchange import (DOUBLE, FLOAT, INT64, NO_DEBUG, Ids, cmath, docc_map_nest, docc_sdfg, fused_map_program, pointer,
+                              scalar, tasklet)
+
+pytestmark = pytest.mark.gpu
+
+
+def compiled(program, folder, name, argtypes):
+    s = StructuredSDFG.from_docc_json(json.dumps(program))
+    nodes = [n for n in s.library_nodes()]
+    s.schedule("rocm")
+    fn = getattr(ctypes.CDLL(s._compile(str(folder))), name)
+    fn.argtypes = argtypes
+    fn.restype = None
+    return fn, nodes
+
+
+@pytest.mark.parametrize("prim,shape", [(FLOAT, (64, 256)), (FLOAT, (37, 129)), (DOUBLE, (33, 64)), (DOUBLE, (5, 7)), (FLOAT, (1, 4)),
+                                        (FLOAT, (1024, 2048))])
+def test_fused_maps_run_as_generated_kernels(tmp_path, prim, shape, rt):
+    """Y = relu(A * B + c) as MapFusion leaves it (three blocks, scalar temporaries), then Z = (A - Y) / 3 with W = Z^T from
+    one chain. Inner extents that are multiples of the vector width take the 128-bit variant, the others the scalar one."""
+    dt = np.float32 if prim == FLOAT else np.float64
+    fn, nodes = compiled(fused_map_program(prim), tmp_path, "fused_maps_sdfg", [ctypes.c_void_p] * 6 + [ctypes.c_int64] * 2)
+    assert [n["code"] for n in nodes] == ["ROCMMap", "ROCMMap"]
+    rng = np.random.default_rng(21)
+    r, c = shape
+    A, B = (rng.standard_normal((r, c)).astype(dt) for _ in range(2))
+    C = rng.standard_normal(c).astype(dt)
+    Y, Z = (np.full((r, c), np.nan, dt) for _ in range(2))
+    W = np.full((c, r), np.nan, dt)
+    fn(*(a.ctypes.data for a in (A, B, C, Y, Z, W)), r, c)
+    assert runtime.take_failure() == (0, "")
+    # numpy, spelled by hand
+    y_ref = np.maximum(dt(0), A * B + C)
+    z_ref = (A - y_ref) / dt(3)
+    assert np.array_equal(Y, y_ref) and np.array_equal(Z, z_ref) and np.array_equal(W, z_ref.T)
+    # the oracle on the imported bodies
+    syms = {"_s0": r, "_s1": c}
+    first = oracle.map_nest(nodes[0], {"_in0": A, "_in1": B, "_in2": C}, symbols=syms)
+    assert np.array_equal(Y.reshape(-1), first["_out0"])
+    second = oracle.map_nest(nodes[1], {"_in0": A, "_in1": Y}, symbols=syms)
+    assert np.array_equal(Z.reshape(-1), second["_out0"]) and np.array_equal(W.reshape(-1), second["_out1"])
+
+
+def math_program(prim):
+    """One nest over [_s0, _s1, 6]: E = exp(X) * s + lgamma(|X| + 1) (a scalar argument, four operations in one block),
+    F = fma(X, X, E) rounded once, G[k][i][j] = tanh(F[i][j][k]) stored permuted, H = fmod(X, 0.75) in place of X's copy."""
+    ids = Ids()
+    containers = {n: pointer(prim) for n in ("X", "E", "F", "G", "H")}
+    for n in ("_s0", "_s1", "_i0", "_i1", "_i2"):
+        containers[n] = scalar(INT64)
+    for n in ("s", "_t0", "_t1", "_t2", "_t3", "_t4"):
+        containers[n] = scalar(prim)
+    P, S = pointer(prim), scalar(prim)
+    loops = [("_i0", "_s0"), ("_i1", "_s1"), ("_i2", "6")]
+    lin = ["_i2 + 6*_i1 + 6*_i0*_s1"]
+    perm = ["_i1 + _i0*_s1 + _i2*_s0*_s1"]
+    lit = (lambda v: (v + "f", prim)) if prim == FLOAT else (lambda v: (v, prim))
+    body = [
+        [(cmath("exp", prim), [("_in1", "X", lin, P)], [("_t0", [], S)]),
+         (tasklet(4, 2), [("_in1", "_t0", [], S), ("_in2", "s", [], S)], [("_t1", [], S)]),
+         (cmath("fabs", prim), [("_in1", "X", lin, P)], [("_t2", [], S)]),
+         (tasklet(2, 2), [("_in1", "_t2", [], S), ("_in2", lit("1.0"), [], S)], [("_t3", [], S)]),
+         (cmath("lgamma", prim), [("_in1", "_t3", [], S)], [("_t4", [], S)])],
+        [(tasklet(2, 2), [("_in1", "_t1", [], S), ("_in2", "_t4", [], S)], [("E", lin, P)])],
+        [(tasklet(7, 3), [("_in1", "X", lin, P), ("_in2", "X", lin, P), ("_in3", "E", lin, P)], [("F", lin, P)])],
+        [(cmath("tanh", prim), [("_in1", "F", lin, P)], [("G", perm, P)])],
+        [(tasklet(6, 2), [("_in1", "X", lin, P), ("_in2", lit("0.75"), [], S)], [("H", lin, P)])],
+    ]
+    children = [docc_map_nest(ids, loops, body), {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG}]
+    return docc_sdfg("math_maps_sdfg", containers, ["X", "E", "F", "G", "H", "s", "_s0", "_s1"], children, ids)
+
+
+@pytest.mark.parametrize("prim", [FLOAT, DOUBLE])
+def test_math_calls_scalar_arguments_and_permuted_stores(tmp_path, prim, rt):
+    dt, ct = (np.float32, ctypes.c_float) if prim == FLOAT else (np.float64, ctypes.c_double)
+    tol = 1e-5 if prim == FLOAT else 1e-12
+    fn, nodes = compiled(math_program(prim), tmp_path, "math_maps_sdfg", [ctypes.c_void_p] * 5 + [ct, ctypes.c_int64, ctypes.c_int64])
+    (node,) = nodes
+    assert node["code"] == "ROCMMap" and len(node["reads"]) == 1 and len(node["writes"]) == 4 and [s["connector"] for s in node["scalars"]] == ["_c0"]
+    rng = np.random.default_rng(22)
+    r, c = 19, 10
+    X = (rng.standard_normal((r, c, 6)) * 1.5).astype(dt)
+    E, F, H = (np.full((r, c, 6), np.nan, dt) for _ in range(3))
+    G = np.full((6, r, c), np.nan, dt)
+    fn(*(a.ctypes.data for a in (X, E, F, G, H)), 0.625, r, c)
+    assert runtime.take_failure() == (0, "")
+    ref = oracle.map_nest(node, {"_in0": X}, scalars={"_c0": 0.625}, symbols={"_s0": r, "_s1": c})
+    by_container = dict(zip(("E", "F", "G", "H"), (ref[w["connector"]] for w in node["writes"])))
+    assert rel_err_max(E, by_container["E"].reshape(E.shape)) <= tol
+    assert rel_err_max(F, by_container["F"].reshape(F.shape)) <= tol
+    assert rel_err_max(G, by_container["G"].reshape(G.shape)) <= tol
+    assert np.array_equal(H, by_container["H"].reshape(H.shape))                        # fmod is exact
+    # by hand, in float64
+    import scipy.special as sp
+    Xd = X.astype(np.float64)
+    e = np.exp(Xd) * 0.625 + sp.gammaln(np.abs(Xd) + 1.0)
+    assert rel_err_max(E, e) <= tol and rel_err_max(F, Xd * Xd + e) <= tol
+    assert rel_err_max(G, np.tanh(Xd * Xd + e).transpose(2, 0, 1)) <= tol and np.array_equal(H, np.fmod(X, dt(0.75)))
+
+
+def test_generated_kernel_at_the_size_of_the_memory_bound_configuration(tmp_path, rt):
+    """[8192, 4096] fp32: the nest collapses to one loop, 32-bit indices, 128-bit accesses; checked whole against numpy."""
+    fn, _ = compiled(fused_map_program(FLOAT), tmp_path, "fused_maps_sdfg", [ctypes.c_void_p] * 6 + [ctypes.c_int64] * 2)
+    rng = np.random.default_rng(23)
+    r, c = 8192, 4096
+    A, B = (rng.standard_normal((r, c), dtype=np.float32) for _ in range(2))
+    C = rng.standard_normal(c, dtype=np.float32)
+    Y, Z = (np.empty((r, c), np.float32) for _ in range(2))
+    W = np.empty((c, r), np.float32)
+    fn(*(a.ctypes.data for a in (A, B, C, Y, Z, W)), r, c)
+    assert runtime.take_failure() == (0, "")
+    y_ref = np.maximum(np.float32(0), A * B + C)
+    assert np.array_equal(Y, y_ref)
+    z_ref = (A - y_ref) / np.float32(3)
+    assert np.array_equal(Z, z_ref) and np.array_equal(W, z_ref.T)
+
+
+def test_module_load_get_function_and_launch(tmp_path, rt):
+    """The three runtime calls generated host code reaches its kernels through, called directly: a kernel image compiled
+    from a generated snippet is loaded, its entry points are found by name, and a launch with the parameter list of
+    the kernel runs it; a missing image, a missing name and an oversized block are reported as errors."""
+    import torch
+    s = StructuredSDFG.from_docc_json(json.dumps(fused_map_program(FLOAT)))
+    s.schedule("rocm", options={"offload": "none"})
+    s._compile(str(tmp_path))
+    images = sorted(tmp_path.glob("kernel_*.hsaco"))
+    assert len(images) == 2
+    (first,) = [i for i in images if "p__in2" in i.with_suffix(".hip").read_text()]      # the nest with three operands read
+    module = ctypes.c_void_p()
+    rt.call("docc_rocm_module_load", str(first).encode(), ctypes.byref(module))
+    fn = ctypes.c_void_p()
+    rt.call("docc_rocm_module_get_function", module, (first.stem + "_v32").encode(), ctypes.byref(fn))
+    assert fn.value
+    with pytest.raises(rt.RocmRuntimeError, match="not found"):
+        rt.call("docc_rocm_module_get_function", module, b"no_such_kernel", ctypes.byref(ctypes.c_void_p()))
+    with pytest.raises(rt.RocmRuntimeError, match="cannot load"):
+        rt.call("docc_rocm_module_load", str(tmp_path / "missing.hsaco").encode(), ctypes.byref(ctypes.c_void_p()))
+    r, c = 48, 64
+    a, b = torch.randn(r, c, device="cuda"), torch.randn(r, c, device="cuda")
+    bias = torch.randn(c, device="cuda")
+    y = torch.full((r, c), float("nan"), device="cuda")
+    # parameters of the first nest's kernel: the four pointers, two bounds, three row strides
+    values = [ctypes.c_void_p(t.data_ptr()) for t in (a, b, bias, y)] + [ctypes.c_longlong(v) for v in (r, c, c, c, c)]
+    args = (ctypes.c_void_p * len(values))(*[ctypes.cast(ctypes.pointer(v), ctypes.c_void_p) for v in values])
+    grid, block = (ctypes.c_uint32 * 3)((r * c // 4 + 255) // 256, 1, 1), (ctypes.c_uint32 * 3)(256, 1, 1)
+    torch.cuda.synchronize()
+    rt.call("docc_rocm_launch", fn, grid, block, 0, None, args)
+    rt.device_sync()
+    assert torch.equal(y, torch.relu(a * b + bias))
+    # an empty grid is no launch; a block of more than 1024 threads is refused before the driver sees it
+    rt.call("docc_rocm_launch", fn, (ctypes.c_uint32 * 3)(0, 1, 1), block, 0, None, args)
+    with pytest.raises(rt.RocmRuntimeError, match="block of 2048 threads"):
+        rt.call("docc_rocm_launch", fn, grid, (ctypes.c_uint32 * 3)(2048, 1, 1), 0, None, args)
+    rt.call("docc_rocm_module_unload", module)

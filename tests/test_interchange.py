@@ -392,16 +392,9 @@ def test_loop_nests_outside_the_elementwise_forms_are_refused():
     bad = copy.deepcopy(base)
     inner_block(bad["root"]["children"][0])["dataflow"]["edges"][0]["subset"] = ["1 + _i1 + _i0*_s1"]  # shifted by one element
     refused(bad, "operand 'X' is not a dense tensor")
+    # several statements under a sequential loop (under maps they become a generated kernel)
     bad = copy.deepcopy(base)
-    inner_block(bad["root"]["children"][0])["dataflow"]["edges"][1]["subset"] = ["_i0 + _i1*_s0"]      # X + Y^T: no kernel walks the operands differently
-    refused(bad, "walk memory differently")
-    bad = copy.deepcopy(base)
-    inner_block(bad["root"]["children"][0])["dataflow"]["nodes"][0]["code"] = 6                        # fp_rem
-    refused(bad, r"tasklet code 6 has no kernel")
-    bad = copy.deepcopy(base)
-    inner_block(bad["root"]["children"][1])["dataflow"]["nodes"][0]["function_stem"] = "lgamma"
-    refused(bad, "CMath function 'lgamma' has no kernel")
-    bad = copy.deepcopy(base)
+    bad["root"]["children"][0]["type"] = "for"
     bad["root"]["children"][0]["root"]["children"].append(copy.deepcopy(inner_block(nest(1))))
     bad["root"]["children"][0]["root"]["transitions"].append(copy.deepcopy(bad["root"]["children"][0]["root"]["transitions"][0]))
     refused(bad, "more than one statement in a loop body")
@@ -674,3 +667,181 @@ def test_views_with_a_stride_of_zero_import_as_repeated_operands(tmp_path):
     s.schedule("rocm")
     assert [n["code"] for n in s.library_nodes() if n["code"].startswith("ml::")] == ["ml::Softmax"]
     assert "docc_rocm_softmax_f32" in Path(s.generate(str(tmp_path))["source"]).read_text()
+
+
+# ---- loop nests that are not one of the prebuilt kernels: the generated-kernel path (ROCMMap) -------------------
+
+def docc_map_nest(ids, loops, blocks):
+    """A nest of maps whose innermost body is a run of blocks. blocks: one list of operations per block; an operation is
+    (op, inputs, outputs) with inputs [(connector, container or (literal, prim), subset, base type)] and outputs
+    [(container, subset, base type)]. Within a block an access node is shared by every edge that names its container,
+    so a scalar written by one operation and read by the next forms the chain tasklet -> access node -> tasklet."""
+    kids = []
+    for ops in blocks:
+        nodes, edges, access = [], [], {}
+
+        def access_node(name):
+            if name not in access:
+                access[name] = ids()
+                nodes.append({"element_id": access[name], "debug_info": NO_DEBUG, "type": "access_node", "data": name})
+            return access[name]
+
+        for op, inputs, outputs in ops:
+            op = {"element_id": ids(), "debug_info": NO_DEBUG, **op}
+            nodes.append(op)
+            for conn, value, subset, base in inputs:
+                if isinstance(value, tuple):
+                    nid = ids()
+                    nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "constant_node", "data": value[0], "data_type": scalar(value[1])})
+                else:
+                    nid = access_node(value)
+                edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": nid, "dst": op["element_id"], "src_conn": "void",
+                              "dst_conn": conn, "subset": list(subset), "base_type": base})
+            for name, subset, base in outputs:
+                # a container that is read and written in one block has two access nodes: the value before, the value after
+                nid = ids()
+                nodes.append({"element_id": nid, "debug_info": NO_DEBUG, "type": "access_node", "data": name})
+                access[name] = nid
+                edges.append({"element_id": ids(), "debug_info": NO_DEBUG, "src": op["element_id"], "dst": nid, "src_conn": "_out",
+                              "dst_conn": "void", "subset": list(subset), "base_type": base})
+        kids.append({"type": "block", "element_id": ids(), "debug_info": NO_DEBUG, "dataflow": {"type": "dataflow", "nodes": nodes, "edges": edges}})
+    body = None
+    for var, extent in reversed(loops):
+        children = kids if body is None else [body]
+        seq = {"type": "sequence", "element_id": ids(), "debug_info": NO_DEBUG, "children": children,
+               "transitions": [{"type": "transition", "element_id": ids(), "debug_info": NO_DEBUG, "assignments": []} for _ in children]}
+        body = {"type": "map", "element_id": ids(), "debug_info": NO_DEBUG, "indvar": var, "init": "0", "condition": f"{var} < {extent}",
+                "update": f"1 + {var}", "root": seq, "schedule_type": {"value": "SEQUENTIAL", "category": 0, "properties": {}}}
+    return body
+
+
+def tasklet(code, n_inputs):
+    names = ["_in"] if n_inputs == 1 and code == 0 else [f"_in{i + 1}" for i in range(n_inputs)]
+    return {"type": "tasklet", "code": code, "inputs": names, "output": "_out"}
+
+
+def cmath(stem, prim):
+    return {"type": "library_node", "implementation_type": "NONE", "code": "CMath", "name": stem + ("f" if prim == FLOAT else ""),
+            "function_stem": stem, "primitive_type": prim}
+
+
+def fused_map_program(prim=FLOAT):
+    """Y = relu(A * B + C) over [_s0, _s1] as MapFusion leaves three elementwise maps (map_fusion.cpp:246-330): one map
+    nest whose body is three blocks, the product and the sum handed on through scalar temporaries `_fused_tmp*`, the
+    last block the fmax(0, x) that ReLU expands to (relu_node.cpp:27-50). C is a row of _s1 entries repeated over the
+    rows (no index in _i0). A second nest, one block holding two chained tasklets: Z = (A - Y) / 3, and W[j][i] = Z[i][j]
+    stored by the same iteration."""
+    ids = Ids()
+    containers = {n: pointer(prim) for n in ("A", "B", "C", "Y", "Z", "W")}
+    for n in ("_s0", "_s1", "_i0", "_i1"):
+        containers[n] = scalar(INT64)
+    for n in ("_fused_tmp", "_fused_tmp_0", "_d"):
+        containers[n] = scalar(prim)
+    P, S = pointer(prim), scalar(prim)
+    loops = [("_i0", "_s0"), ("_i1", "_s1")]
+    rm, cm, row = ["_i1 + _i0*_s1"], ["_i0 + _i1*_s0"], ["_i1"]
+    lit = (lambda v: (v + "f", prim)) if prim == FLOAT else (lambda v: (v, prim))
+    children = [
+        docc_map_nest(ids, loops, [
+            [(tasklet(4, 2), [("_in1", "A", rm, P), ("_in2", "B", rm, P)], [("_fused_tmp", [], S)])],
+            [(tasklet(2, 2), [("_in1", "_fused_tmp", [], S), ("_in2", "C", row, P)], [("_fused_tmp_0", [], S)])],
+            [(cmath("fmax", prim), [("_in1", lit("0.0"), [], S), ("_in2", "_fused_tmp_0", [], S)], [("Y", rm, P)])],
+        ]),
+        docc_map_nest(ids, loops, [
+            [(tasklet(3, 2), [("_in1", "A", rm, P), ("_in2", "Y", rm, P)], [("_d", [], S)]),
+             (tasklet(5, 2), [("_in1", "_d", [], S), ("_in2", lit("3.0"), [], S)], [("Z", rm, P), ("W", cm, P)])],
+        ]),
+        {"type": "return", "element_id": ids(), "data": "", "debug_info": NO_DEBUG},
+    ]
+    return docc_sdfg("fused_maps_sdfg", containers, ["A", "B", "C", "Y", "Z", "W", "_s0", "_s1"], children, ids)
+
+
+def test_map_nests_with_several_operations_import_as_generated_kernels(tmp_path):
+    s = StructuredSDFG.from_docc_json(json.dumps(fused_map_program()))
+    first, second = s.library_nodes()
+    assert first["code"] == second["code"] == "ROCMMap"
+    assert first["indvars"] == ["_i0", "_i1"] and first["bounds"] == ["_s0", "_s1"] and first["symbols"] == ["_s0", "_s1"]
+    assert [(r["connector"], r["strides"], r["extent"]) for r in first["reads"]] == [
+        ("_in0", ["_s1", "1"], "(_s0)*_s1"), ("_in1", ["_s1", "1"], "(_s0)*_s1"), ("_in2", ["0", "1"], "_s1")]
+    assert [(st["op"], st["args"]) for st in first["statements"]] == [
+        ("fp_mul", ["_in0", "_in1"]), ("fp_add", ["_v0", "_in2"]), ("fmax", ["#0.0f", "_v1"])]
+    assert [(w["connector"], w["strides"], w["value"]) for w in first["writes"]] == [("_out0", ["_s1", "1"], "_v2")]
+    blocks = [c["dataflow"] for c in s._data["root"]["children"][:2]]
+    assert blocks[0]["inputs"] == [{"data": "A", "connector": "_in0"}, {"data": "B", "connector": "_in1"}, {"data": "C", "connector": "_in2"}]
+    assert blocks[0]["outputs"] == [{"data": "Y", "connector": "_out0"}]
+    # two results of one statement, one of them transposed
+    assert [(w["connector"], w["strides"], w["value"]) for w in second["writes"]] == [
+        ("_out0", ["_s1", "1"], "_v1"), ("_out1", ["1", "_s0"], "_v1")]
+    assert [(st["op"], st["args"]) for st in second["statements"]] == [("fp_sub", ["_in0", "_in1"]), ("fp_div", ["_v0", "#3.0f"])]
+    # the node survives the target's own JSON
+    again = StructuredSDFG.parse(s.to_json())
+    assert again.library_nodes() == s.library_nodes()
+
+    s.schedule("rocm")
+    assert [n["implementation_type"] for n in s.library_nodes() if n["code"] == "ROCMMap"] == ["ROCMWithoutTransfers"] * 2
+    r = s.loop_report()
+    assert r["H2D"] == 3 and r["D2H"] == 3            # A B C up; Y Z W down; Y stays on the device between the nests
+    report = s.generate(str(tmp_path))
+    src = Path(report["source"]).read_text()
+    kernels = sorted(p.name for p in tmp_path.glob("kernel_*.hip"))
+    assert len(kernels) == 2 and all(k.startswith("kernel_fused_maps_sdfg_") for k in kernels)
+    stem = kernels[0][:-4]
+    assert f'"{stem}.hsaco"' in src and "docc_rocm_module_load(" in src and "docc_rocm_module_get_function(" in src
+    assert src.count("docc_rocm_launch(__docc_fn, __docc_grid, __docc_block, 0, nullptr, __docc_args)") == 2
+    text = (tmp_path / kernels[0]).read_text()
+    assert f'extern "C" __global__ void __launch_bounds__(256) {stem}_v32(' in text and f"{stem}_s64(" in text
+    assert "const float _v0 = (float) (_in0) * (float) (_in1);" in text and "fmaxf((float) (0.0f), (float) (_v1))" in text
+    assert "if (gid < total) {" in text
+    # the kernel text is valid gfx950 code
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    for k in kernels:
+        r = subprocess.run([hipcc, "--genco", "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature",
+                            "-Xclang", "-packed-fp32-ops", str(tmp_path / k), "-o", str(tmp_path / (k[:-4] + ".hsaco"))], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_what_the_prebuilt_kernels_decline_goes_to_a_generated_kernel_under_maps_only():
+    base = elementwise_nests_program()
+
+    def inner_block(n):
+        while n["type"] != "block":
+            n = n["root"]["children"][0] if n["type"] in ("for", "map") else n["children"][0]
+        return n
+
+    # X + Y^T: the operands walk memory in different orders
+    prog = copy.deepcopy(base)
+    inner_block(prog["root"]["children"][0])["dataflow"]["edges"][1]["subset"] = ["_i0 + _i1*_s0"]
+    node = StructuredSDFG.from_docc_json(json.dumps(prog)).library_nodes()[0]
+    assert node["code"] == "ROCMMap" and [r["strides"] for r in node["reads"]] == [["_s1", "1"], ["1", "_s0"]]
+    # a remainder and a gamma function have no node of their own
+    prog = copy.deepcopy(base)
+    inner_block(prog["root"]["children"][0])["dataflow"]["nodes"][0]["code"] = 6
+    inner_block(prog["root"]["children"][1])["dataflow"]["nodes"][0]["function_stem"] = "lgamma"
+    nodes = StructuredSDFG.from_docc_json(json.dumps(prog)).library_nodes()
+    assert [n["code"] for n in nodes[:2]] == ["ROCMMap", "ROCMMap"]
+    assert nodes[0]["statements"][0]["op"] == "fp_rem" and nodes[1]["statements"][0]["op"] == "lgamma"
+    # the same under a sequential loop: nothing says that its iterations are independent
+    prog = copy.deepcopy(base)
+    prog["root"]["children"][0]["type"] = "for"
+    inner_block(prog["root"]["children"][0])["dataflow"]["nodes"][0]["code"] = 6
+    with pytest.raises(InvalidSDFGException, match="tasklet code 6 has no kernel"):
+        StructuredSDFG.from_docc_json(json.dumps(prog))
+    # an element other iterations write is read: not a nest the target may run in parallel. The second nest reads Y
+    # row by row and writes W column by column; reading W row by row instead meets elements of other iterations
+    prog = fused_map_program()
+    blk = inner_block(prog["root"]["children"][1])
+    for n in blk["dataflow"]["nodes"]:
+        if n["type"] == "access_node" and n["data"] == "Y":
+            n["data"] = "W"
+    with pytest.raises(InvalidSDFGException, match="'W' is read at other elements than the one the iteration writes"):
+        StructuredSDFG.from_docc_json(json.dumps(prog))
+    # a result that one loop of the nest does not index would be written by many iterations
+    prog = fused_map_program()
+    last = prog["root"]["children"][0]["root"]["children"][0]["root"]["children"][2]
+    for e in last["dataflow"]["edges"]:
+        if e["src_conn"] == "_out":
+            e["subset"] = ["_i1"]
+    with pytest.raises(InvalidSDFGException, match="a result that some loops of the nest do not index"):
+        StructuredSDFG.from_docc_json(json.dumps(prog))

@@ -375,3 +375,102 @@ def test_transpose_matches_numpy_for_every_permutation():
                 Y = oracle.transpose(X, perm)
                 assert Y.dtype == dt and Y.flags.c_contiguous
                 assert np.array_equal(Y, np.transpose(X, perm)), (shape, perm)
+
+
+# ---- map nests: the interpreter of tasklet bodies -------------------------------------------------------------------
+
+def _map_node(bounds, reads, statements, writes, scalars=()):
+    """A ROCMMap payload written by hand: reads / writes are (connector, strides, extent, type[, value])."""
+    acc = lambda t: {"connector": t[0], "strides": [str(x) for x in t[1]], "extent": str(t[2]), "element_type": t[3], **({"value": t[4]} if len(t) > 4 else {})}
+    return {"indvars": [f"i{k}" for k in range(len(bounds))], "bounds": [str(b) for b in bounds], "symbols": [],
+            "reads": [acc(r) for r in reads], "writes": [acc(w) for w in writes],
+            "scalars": [{"connector": c, "element_type": t} for c, t in scalars],
+            "statements": [{"out": o, "type": t, "op": op, "args": list(args)} for o, t, op, args in statements]}
+
+
+def test_map_nest_follows_strides_statement_order_and_roundings():
+    rng = np.random.default_rng(11)
+    n, m = 7, 12
+    A, B = rng.standard_normal((n, m)).astype(np.float32), rng.standard_normal((n, m)).astype(np.float32)
+    c = rng.standard_normal(m).astype(np.float32)
+    # relu(A * B + c), c repeated over the rows, stored row by row and transposed: pinned by numpy, whose ufuncs round
+    # after every operation as separate statements do
+    node = _map_node([n, m], [("a", [m, 1], n * m, "Float"), ("b", [m, 1], n * m, "Float"), ("c", [0, 1], m, "Float")],
+                     [("t0", "Float", "fp_mul", ["a", "b"]), ("t1", "Float", "fp_add", ["t0", "c"]), ("t2", "Float", "fmax", ["#0.0f", "t1"])],
+                     [("y", [m, 1], n * m, "Float", "t2"), ("yt", [1, n], n * m, "Float", "t2")])
+    out = oracle.map_nest(node, {"a": A, "b": B, "c": c})
+    ref = np.maximum(np.float32(0), A * B + c)
+    assert np.array_equal(out["y"].reshape(n, m), ref) and np.array_equal(out["yt"].reshape(m, n), ref.T)
+    # a transposed operand: a slip between the two stride lists fails this
+    node = _map_node([n, m], [("a", [m, 1], n * m, "Float"), ("bt", [1, n], n * m, "Float")],
+                     [("t0", "Float", "fp_sub", ["a", "bt"])], [("y", [m, 1], n * m, "Float", "t0")])
+    Bt = rng.standard_normal((m, n)).astype(np.float32)
+    assert np.array_equal(oracle.map_nest(node, {"a": A, "bt": Bt})["y"].reshape(n, m), A - Bt.T)
+    # argument order of the non-commutative operations, a scalar operand, a literal, three loops
+    X = rng.standard_normal((3, 4, 5))
+    node = _map_node([3, 4, 5], [("x", [20, 5, 1], 60, "Double")],
+                     [("t0", "Double", "fp_div", ["s", "x"]), ("t1", "Double", "fp_sub", ["t0", "#0.25"]), ("t2", "Double", "fp_neg", ["t1"]),
+                      ("t3", "Double", "pow", ["t2", "#2.0"]), ("t4", "Double", "fp_rem", ["t3", "s"]), ("t5", "Double", "atan2", ["t4", "x"])],
+                     [("y", [20, 5, 1], 60, "Double", "t5")], scalars=[("s", "Double")])
+    ref = np.arctan2(np.fmod((-(1.5 / X - 0.25)) ** 2.0, 1.5), X)
+    assert np.allclose(oracle.map_nest(node, {"x": X}, scalars={"s": 1.5})["y"].reshape(X.shape), ref, rtol=1e-15, atol=0)
+    # fp_fma is one rounding: the float64 product of two float32 values is exact, so rounding a*b+c once from
+    # float64 differs from the two roundings of mul-then-add on some elements and equals the fused result on all but
+    # double-rounding cases (none in this sample)
+    a32, b32, c32 = (rng.standard_normal(4096).astype(np.float32) for _ in range(3))
+    fused = _map_node([4096], [("a", [1], 4096, "Float"), ("b", [1], 4096, "Float"), ("c", [1], 4096, "Float")],
+                      [("t0", "Float", "fp_fma", ["a", "b", "c"])], [("y", [1], 4096, "Float", "t0")])
+    two = _map_node([4096], [("a", [1], 4096, "Float"), ("b", [1], 4096, "Float"), ("c", [1], 4096, "Float")],
+                    [("t0", "Float", "fp_mul", ["a", "b"]), ("t1", "Float", "fp_add", ["t0", "c"])], [("y", [1], 4096, "Float", "t1")])
+    yf, y2 = oracle.map_nest(fused, {"a": a32, "b": b32, "c": c32})["y"], oracle.map_nest(two, {"a": a32, "b": b32, "c": c32})["y"]
+    exact = a32.astype(np.float64) * b32.astype(np.float64) + c32.astype(np.float64)
+    assert np.array_equal(y2, a32 * b32 + c32)
+    assert (yf != y2).any() and np.abs(yf - exact).max() <= np.abs(y2 - exact).max()
+    assert np.abs(yf.astype(np.float64) - exact).max() <= np.abs(exact).max() * 2.0 ** -24
+    # a float32 statement on float64 operands converts first; a float64 statement on float32 operands widens
+    node = _map_node([64], [("a", [1], 64, "Double")], [("t0", "Float", "fp_mul", ["a", "a"]), ("t1", "Double", "fp_add", ["t0", "a"])],
+                     [("y", [1], 64, "Double", "t1")])
+    a64 = rng.standard_normal(64)
+    assert np.array_equal(oracle.map_nest(node, {"a": a64})["y"], (a64.astype(np.float32) * a64.astype(np.float32)).astype(np.float64) + a64)
+    # errors: an unknown operation, a value used before it exists, an operand that is too small
+    bad = _map_node([4], [("a", [1], 4, "Float")], [("t0", "Float", "fp_nope", ["a"])], [("y", [1], 4, "Float", "t0")])
+    with pytest.raises(ValueError):
+        oracle.map_nest(bad, {"a": np.zeros(4, np.float32)})
+    with pytest.raises(ValueError, match="holds 3 elements"):
+        oracle.map_nest(_map_node([4], [("a", [1], 4, "Float")], [("t0", "Float", "assign", ["a"])], [("y", [1], 4, "Float", "t0")]), {"a": np.zeros(3, np.float32)})
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_map_nest_cmath_calls_are_the_libm_functions(dtype):
+    """Every CMath stem against numpy / scipy / math in float64 (a wrong table entry - exp for exp2, ceil for floor,
+    swapped arguments - is off by far more than the tolerance)."""
+    import math
+    import scipy.special as sp
+    rng = np.random.default_rng(12)
+    n = 257
+    tname = "Double" if dtype == np.float64 else "Float"
+    tol = 4e-15 if dtype == np.float64 else 4e-7
+    pos, unit, anyv = (rng.random(n) * 4 + 0.1).astype(dtype), (rng.random(n) * 1.8 - 0.9).astype(dtype), (rng.standard_normal(n) * 3).astype(dtype)
+    other = (rng.standard_normal(n) * 2 + 0.3).astype(dtype)
+    unary = {"sin": (np.sin, anyv), "cos": (np.cos, anyv), "tan": (np.tan, unit), "asin": (np.arcsin, unit), "acos": (np.arccos, unit),
+             "atan": (np.arctan, anyv), "sinh": (np.sinh, anyv), "cosh": (np.cosh, anyv), "tanh": (np.tanh, anyv), "asinh": (np.arcsinh, anyv),
+             "acosh": (np.arccosh, pos + 1), "atanh": (np.arctanh, unit), "exp": (np.exp, anyv), "exp2": (np.exp2, anyv),
+             "exp10": (lambda x: 10.0 ** x, unit), "expm1": (np.expm1, unit), "log": (np.log, pos), "log10": (np.log10, pos),
+             "log2": (np.log2, pos), "log1p": (np.log1p, pos), "sqrt": (np.sqrt, pos), "cbrt": (np.cbrt, anyv), "erf": (sp.erf, anyv),
+             "erfc": (sp.erfc, unit), "tgamma": (sp.gamma, pos), "lgamma": (sp.gammaln, pos), "fabs": (np.abs, anyv), "ceil": (np.ceil, anyv),
+             "floor": (np.floor, anyv), "trunc": (np.trunc, anyv), "round": (lambda x: np.sign(x) * np.floor(np.abs(x) + 0.5), anyv),
+             "nearbyint": (np.rint, anyv), "rint": (np.rint, anyv)}
+    for stem, (fn, x) in unary.items():
+        node = _map_node([n], [("x", [1], n, tname)], [("t", tname, stem, ["x"])], [("y", [1], n, tname, "t")])
+        got = oracle.map_nest(node, {"x": x})["y"].astype(np.float64)
+        ref = fn(x.astype(np.float64))
+        assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max()), stem
+    binary = {"atan2": np.arctan2, "pow": lambda a, b: np.abs(a) ** b, "hypot": np.hypot, "fmod": np.fmod,
+              "remainder": lambda a, b: np.array([math.remainder(u, v) for u, v in zip(a, b)]), "copysign": np.copysign,
+              "fmax": np.fmax, "fmin": np.fmin, "fdim": lambda a, b: np.maximum(a - b, 0.0)}
+    for stem, fn in binary.items():
+        a = np.abs(anyv) if stem == "pow" else anyv
+        node = _map_node([n], [("a", [1], n, tname), ("b", [1], n, tname)], [("t", tname, stem, ["a", "b"])], [("y", [1], n, tname, "t")])
+        got = oracle.map_nest(node, {"a": a, "b": other})["y"].astype(np.float64)
+        ref = fn(a.astype(np.float64), other.astype(np.float64))
+        assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max()), stem
