@@ -495,7 +495,10 @@ int docc_rocm_module_load(const char* path, docc_rocm_module_t* module) {
     if (!path || !module) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "module_load: null argument");
     hipModule_t m;
     hipError_t err = hipModuleLoad(&m, path);
-    if (err != hipSuccess) return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "cannot load %s: %s", path, hipGetErrorString(err));
+    if (err != hipSuccess) {
+        (void) hipGetLastError();   // reported here; other users of the HIP runtime in this process must not pick it up
+        return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "cannot load %s: %s", path, hipGetErrorString(err));
+    }
     *module = m;
     return 0;
 }
@@ -508,7 +511,10 @@ int docc_rocm_module_get_function(docc_rocm_module_t module, const char* name, d
     if (!module || !name || !function) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "get_function: null argument");
     hipFunction_t f;
     hipError_t err = hipModuleGetFunction(&f, (hipModule_t) module, name);
-    if (err != hipSuccess) return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "kernel %s not found: %s", name, hipGetErrorString(err));
+    if (err != hipSuccess) {
+        (void) hipGetLastError();
+        return fail(DOCC_ROCM_ERR_KERNEL_IMAGE, "kernel %s not found: %s", name, hipGetErrorString(err));
+    }
     *function = f;
     return 0;
 }
