@@ -37,6 +37,10 @@ sys.path.insert(0, str(ROOT))
 
 METRIC = "GEMM/attn/conv TFLOP/s + softmax GB/s, % of roofline, vs openmp host target"
 
+# HBM-bound kernels walk this many sets of operands in turn (each set 256 MiB or more), so that no launch meets data
+# that an earlier one left in the 256 MiB Infinity Cache
+ROTATE = 4
+
 # MI355X published peaks
 PEAK_HBM_GBS = 8000.0
 PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3, "bf16": 2516.6}
@@ -173,9 +177,14 @@ def main():
         achieved = nbytes / kern_ms / 1e6
         out.update(value=nbytes / (wall / args.steps) / 1e9, ms_per_step=ms_per_step, timed_regions=len(regions),
                    timed_ms_total=round(sum(regions) * 1e3, 2))
+        # two clocks, named: `value` / `ms_per_step` are the host's wall clock around K launches (launch overhead and the
+        # final synchronisation included); `roofline.achieved` / `frac` are HIP events around launches on the stream
+        out["value_clock"] = "host wall clock around --steps launches between two device synchronisations"
         out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": SOFTMAX_TRAFFIC_BYTES,
                            "traffic_source": SOFTMAX_TRAFFIC_SOURCE,
+                           "clock": "HIP events on the launch stream around back-to-back launches",
+                           "frac_of_value": round(out["value"] / PEAK_HBM_GBS, 4),
                            "kernel": "docc_softmax_f32_block8_v2", "kernel_us": round(kern_ms * 1e3, 2),
                            "algorithmic_bytes": nbytes, "sustained_clock_ghz": sustained_clock_ghz(step, kern_ms)}
         # same number for a plain copy of the same bytes: the practical ceiling of this memory system
@@ -276,16 +285,18 @@ def main():
         add_kernel("sgemm_4096_bias_relu", "f32", 2 * n**3, ms_e)
         del A, B, Cm, bias
         # one output column / one output row: the matrix-vector kernels, HBM-bound (the matrix moves once)
+        # (four matrices taken in turn, 1 GiB: nothing is met again in the 256 MiB Infinity Cache)
         nv = 8192
-        Mx, xv, yv = torch.randn(nv, nv, device="cuda"), torch.randn(nv, device="cuda"), torch.empty(nv, device="cuda")
-        for name, call in (("sgemv_8192x8192_rows", lambda i: rt.sgemm(nv, 1, nv, 1.0, Mx.data_ptr(), nv, xv.data_ptr(), 1, 0.0, yv.data_ptr(), 1, stream=stream)),
-                           ("sgemv_8192x8192_columns", lambda i: rt.sgemm(1, nv, nv, 1.0, xv.data_ptr(), nv, Mx.data_ptr(), nv, 0.0, yv.data_ptr(), nv, stream=stream))):
-            ms_v = time_kernel(call, 50, 5)
+        Ms = [torch.randn(nv, nv, device="cuda") for _ in range(ROTATE)]
+        xv, yv = torch.randn(nv, device="cuda"), torch.empty(nv, device="cuda")
+        for name, call in (("sgemv_8192x8192_rows", lambda i: rt.sgemm(nv, 1, nv, 1.0, Ms[i % ROTATE].data_ptr(), nv, xv.data_ptr(), 1, 0.0, yv.data_ptr(), 1, stream=stream)),
+                           ("sgemv_8192x8192_columns", lambda i: rt.sgemm(1, nv, nv, 1.0, xv.data_ptr(), nv, Ms[i % ROTATE].data_ptr(), nv, 0.0, yv.data_ptr(), nv, stream=stream))):
+            ms_v = time_kernel(call, 48, 8)
             nbytes_v = 4 * (nv * nv + 2 * nv)
-            kernels[name] = {"kernel_us": round(ms_v * 1e3, 2), "dtype": "f32",
+            kernels[name] = {"kernel_us": round(ms_v * 1e3, 2), "dtype": "f32", "buffers_rotated": ROTATE,
                              "roofline": {"bound": "hbm", "achieved": round(nbytes_v / ms_v / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                           "frac": round(nbytes_v / ms_v / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_v}}
-        del Mx, xv, yv
+        del Ms, xv, yv
 
     # ---- config 3b: bf16 GEMM 4096^3, fp32 accumulate/output ------------------------------
     if want("bgemm"):
@@ -362,44 +373,74 @@ def main():
     # ---- elementwise tensor nodes on the softmax tensor's shape (HBM-bound) --------------------
     if want("elementwise"):
         n = 8192 * 4096
-        a, b2, y = (torch.randn(n, device="cuda") for _ in range(3))
-        cases = {"add_f32": (12 * n, lambda i: rt.elementwise_binary("add", 32, n, a.data_ptr(), b2.data_ptr(), y.data_ptr(), stream)),
-                 "relu_f32": (8 * n, lambda i: rt.elementwise_unary("relu", 32, n, a.data_ptr(), y.data_ptr(), stream)),
-                 "sigmoid_f32": (8 * n, lambda i: rt.elementwise_unary("sigmoid", 32, n, a.data_ptr(), y.data_ptr(), stream)),
-                 "broadcast_row_f32": (4 * n + 4 * 4096, lambda i: rt.broadcast(32, (1, 4096), (8192, 4096), a.data_ptr(), y.data_ptr(), stream)),
+        As, Bs, Ys = ([torch.randn(n, device="cuda") for _ in range(ROTATE)] for _ in range(3))
+        a_, b_, y_ = (lambda i: As[i % ROTATE].data_ptr()), (lambda i: Bs[i % ROTATE].data_ptr()), (lambda i: Ys[i % ROTATE].data_ptr())
+        cases = {"add_f32": (12 * n, lambda i: rt.elementwise_binary("add", 32, n, a_(i), b_(i), y_(i), stream)),
+                 "relu_f32": (8 * n, lambda i: rt.elementwise_unary("relu", 32, n, a_(i), y_(i), stream)),
+                 "sigmoid_f32": (8 * n, lambda i: rt.elementwise_unary("sigmoid", 32, n, a_(i), y_(i), stream)),
+                 "broadcast_row_f32": (4 * n + 4 * 4096, lambda i: rt.broadcast(32, (1, 4096), (8192, 4096), a_(i), y_(i), stream)),
                  # relu(a + bias row): what the fusion pass makes of Broadcast + Add + ReLU (28 B/element as three nodes)
-                 "fused_bias_relu_f32": (8 * n + 4 * 4096, lambda i: rt.elementwise_fused(32, (8192, 4096), "add", a.data_ptr(), (8192, 4096),
-                                                                                        b2.data_ptr(), (4096,), ["relu"], y.data_ptr(), stream))}
+                 "fused_bias_relu_f32": (8 * n + 4 * 4096, lambda i: rt.elementwise_fused(32, (8192, 4096), "add", a_(i), (8192, 4096),
+                                                                                        Bs[0].data_ptr(), (4096,), ["relu"], y_(i), stream))}
+        hbm_entry = lambda ms, nbytes_e, dtype="f32": {
+            "kernel_us": round(ms * 1e3, 2), "dtype": dtype, "buffers_rotated": ROTATE,
+            "roofline": {"bound": "hbm", "achieved": round(nbytes_e / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(nbytes_e / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_e}}
         for name, (nbytes_e, fn) in cases.items():
-            ms = time_kernel(fn, 50, 5)
-            gbs = nbytes_e / ms / 1e6
-            kernels[f"elementwise_{name}_8192x4096"] = {
-                "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
-                "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(gbs / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_e}}
+            kernels[f"elementwise_{name}_8192x4096"] = hbm_entry(time_kernel(fn, 48, 8), nbytes_e)
         # reduce nodes on the same tensor: over the rows' extent (one wavefront per row) and over the rows (one lane per column)
         for name, (outer, extent, inner) in {"sum_rows_f32": (8192, 4096, 1), "max_columns_f32": (1, 8192, 4096)}.items():
             op = name.split("_")[0]
-            ms = time_kernel(lambda i: rt.reduce(op, 32, outer, extent, inner, a.data_ptr(), y.data_ptr(), stream), 50, 5)
-            nbytes_r = 4 * n + 4 * outer * inner
-            kernels[f"reduce_{name}_8192x4096"] = {
-                "kernel_us": round(ms * 1e3, 2), "dtype": "f32",
-                "roofline": {"bound": "hbm", "achieved": round(nbytes_r / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": round(nbytes_r / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes_r}}
+            ms = time_kernel(lambda i: rt.reduce(op, 32, outer, extent, inner, a_(i), y_(i), stream), 48, 8)
+            kernels[f"reduce_{name}_8192x4096"] = hbm_entry(ms, 4 * n + 4 * outer * inner)
         # ml::Transpose of the same tensor (64 x 64 tiles through LDS) and of a [64, 128, 64, 64] tensor with its two
         # middle axes swapped (rows of 64 elements move as they are)
         for name, shape, perm in (("transpose_f32_8192x4096", (8192, 4096), (1, 0)), ("transpose_f32_64x128x64x64_0213", (64, 128, 64, 64), (0, 2, 1, 3))):
-            ms = time_kernel(lambda i: rt.transpose(4, shape, perm, a.data_ptr(), y.data_ptr(), stream), 50, 5)
-            kernels[name] = {"kernel_us": round(ms * 1e3, 2), "dtype": "b32",
-                             "roofline": {"bound": "hbm", "achieved": round(8 * n / ms / 1e6, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                          "frac": round(8 * n / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": 8 * n}}
+            ms = time_kernel(lambda i: rt.transpose(4, shape, perm, a_(i), y_(i), stream), 48, 8)
+            kernels[name] = hbm_entry(ms, 8 * n, "b32")
+        # loop nests compiled into kernels by the map dispatcher (ROCMMap): y = relu(a + bias row), the work of the fused
+        # elementwise kernel above, and y = fma(a, b, y0) over three full operands, both written as tasklets
+        if True:
+            import ctypes
+
+            from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFGBuilder
+
+            mb = StructuredSDFGBuilder("bench_maps")
+            for nm in ("A", "B", "bias", "Y", "Z"):
+                mb.add_container(nm, Pointer(Scalar(PrimitiveType.Float)), True)
+            row = ["4096", "1"]
+            mb.add_map_nest([("i", 8192), ("j", 4096)], [("a", "A", row), ("c", "bias", ["0", "1"])],
+                            [("s", "fp_add", ["a", "c"]), ("r", "fmax", [0.0, "s"])], [("Y", row, "r")])
+            one = mb.move()
+            mb2 = StructuredSDFGBuilder("bench_maps2")
+            for nm in ("A", "B", "Y", "Z"):
+                mb2.add_container(nm, Pointer(Scalar(PrimitiveType.Float)), True)
+            mb2.add_map_nest([("i", 8192), ("j", 4096)], [("a", "A", row), ("b", "B", row), ("y", "Y", row)],
+                             [("r", "fp_fma", ["a", "b", "y"])], [("Z", row, "r")])
+            two = mb2.move()
+            folder = Path(tempfile.gettempdir()) / f"docc_bench_maps_{os.getpid()}"
+            fns = []
+            for sd in (one, two):
+                sd.schedule("rocm", options={"offload": "none"})
+                lib = ctypes.CDLL(sd._compile(str(folder / sd.name)))
+                f = getattr(lib, sd.name)
+                f.argtypes = [ctypes.c_void_p] * len(sd.arguments)
+                f.restype = None
+                fns.append(f)
+            kernels["map_relu_bias_row_f32_8192x4096"] = hbm_entry(
+                time_kernel(lambda i: fns[0](a_(i), 0, Bs[0].data_ptr(), y_(i), 0), 48, 8), 8 * n + 4 * 4096)
+            kernels["map_fma_f32_8192x4096"] = hbm_entry(
+                time_kernel(lambda i: fns[1](a_(i), b_(i), y_(i), Ys[(i + 1) % ROTATE].data_ptr()), 48, 8), 16 * n)
+            code, message = rt.take_failure()
+            if code:
+                raise RuntimeError(message)
         if oracle_lib is not None:
-            ah, bh = a.cpu().numpy(), b2.cpu().numpy()
+            ah, bh = As[0].cpu().numpy(), Bs[0].cpu().numpy()
             t = cpu_time(lambda: oracle.elementwise_binary("add", ah, bh, lib=oracle_lib))
             kernels["elementwise_add_f32_8192x4096"]["cpu_baseline"] = {
                 "value": round(12 * n / t / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port",
                 "sample": "full tensor, the Map the reference's ElementWiseBinaryNode expands to (omp parallel for)"}
-        del a, b2, y
+        del As, Bs, Ys
 
     # ---- PCIe-inclusive: host arrays in, host array out, through @native (never the reported `value`) ----
     end_to_end = {}
@@ -448,6 +489,7 @@ def main():
         "ms_per_step": round(out.get("ms_per_step", 0.0), 5),
         "timed_regions": out.get("timed_regions", 0),
         "timed_ms_total": out.get("timed_ms_total", 0.0),
+        "value_clock": out.get("value_clock", ""),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -16,7 +16,8 @@ import enum
 import json
 import os
 from pathlib import Path
-from typing import Any, Dict, List, Optional, Sequence
+import re
+from typing import Any, Dict, List, Optional, Sequence, Tuple
 
 _LIB_DIR = Path(__file__).resolve().parent.parent / "lib"
 _TARGET_LIB = _LIB_DIR / "libdocc_rocm_target.so"
@@ -404,6 +405,61 @@ class StructuredSDFGBuilder:
                          "dilations": [_expr(s) for s in dilations], "output_channels": _expr(output_channels),
                          "group": _expr(group), "has_bias": B is not None, "element_type": self._element(X).value},
                         inputs, [self._operand("Y", Y)])
+
+    def add_map_nest(self, loops: Sequence[Tuple[str, Any]], reads: Sequence[Tuple[str, str, Sequence[Any]]],
+                     statements: Sequence[Tuple[str, str, Sequence[Any]]], writes: Sequence[Tuple[str, Sequence[Any], str]],
+                     scalars: Sequence[Tuple[str, Any]] = ()) -> None:
+        """A perfect nest of maps with a body of tasklets, run as one generated kernel (node code ROCMMap). The reference's
+        builder spells such a nest with begin_map / add_block / add_tasklet / add_memlet calls
+        (python/bindings/builder/py_structured_sdfg_builder.cpp); the block list has no nested scopes, so the nest is
+        given whole:
+          loops      [(induction variable, bound)], outermost first; every loop runs from 0 in steps of 1
+          reads      [(name, container, strides)]: `name` = container[sum(stride_l * variable_l)], loaded once per iteration
+          scalars    [(name, scalar container or number)]
+          statements [(name, operation, arguments)]: a tasklet code (assign, fp_neg, fp_add, fp_sub, fp_mul, fp_div,
+                     fp_rem, fp_fma) or a libm function stem (exp, tanh, fmax, pow, ...) applied to names defined
+                     before it or to numbers; every statement rounds by itself, in the element type of the first write
+          writes     [(container, strides, name)]
+        Iterations must be independent: no iteration may read or write an element another one writes."""
+        elem = self._element(writes[0][0])
+        literal = lambda v: "#" + (repr(float(v)) + ("f" if elem == PrimitiveType.Float else ""))
+        names: Dict[str, str] = {}
+        depth = len(loops)
+
+        def access(connector: str, container: str, strides: Sequence[Any]) -> Dict[str, Any]:
+            if len(strides) != depth:
+                raise InvalidSDFGException(f"map nest: '{container}' needs one stride per loop")
+            st = [_expr(x) for x in strides]
+            extent = " + ".join(["1"] + [f"(({_expr(b)}) - 1)*({x})" for (_, b), x in zip(loops, st) if x != "0"])
+            return {"connector": connector, "strides": st, "extent": extent, "element_type": self._element(container).value}
+
+        node_reads, node_scalars, node_statements, node_writes, inputs, outputs = [], [], [], [], [], []
+        for k, (name, container, strides) in enumerate(reads):
+            names[name] = f"_in{k}"
+            node_reads.append(access(names[name], container, strides))
+            inputs.append(self._operand(names[name], container))
+        for k, (name, value) in enumerate(scalars):
+            names[name] = f"_c{k}"
+            is_container = isinstance(value, str) and value in self._data["containers"]
+            node_scalars.append({"connector": names[name], "element_type": (self._element(value) if is_container else elem).value})
+            inputs.append(self._operand(names[name], value) if is_container else self._operand(names[name], value, elem))
+        resolve = lambda a: names[a] if isinstance(a, str) and a in names else literal(a) if isinstance(a, (int, float)) else str(a)
+        for k, (name, op, args) in enumerate(statements):
+            node_statements.append({"out": f"_v{k}", "type": elem.value, "op": op, "args": [resolve(a) for a in args]})
+            names[name] = f"_v{k}"
+        for k, (container, strides, value) in enumerate(writes):
+            w = access(f"_out{k}", container, strides)
+            w["value"] = resolve(value)
+            node_writes.append(w)
+            outputs.append(self._operand(f"_out{k}", container))
+        words = set()
+        for text in [_expr(b) for _, b in loops] + [x for a in node_reads + node_writes for x in a["strides"]]:
+            words.update(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", text))
+        symbols = sorted(w for w in words if w in self._data["containers"] and self._data["containers"][w]["type"] == "scalar")
+        self._add_block({"code": "ROCMMap", "implementation_type": "NONE", "side_effect": False,
+                         "indvars": [v for v, _ in loops], "bounds": [_expr(b) for _, b in loops], "symbols": symbols,
+                         "reads": node_reads, "writes": node_writes, "scalars": node_scalars, "statements": node_statements},
+                        inputs, outputs)
 
     #: elementwise tensor node codes (reference .../tensor/elementwise_ops/*.h)
     UNARY_CODES = {"abs": "ml::Abs", "exp": "ml::Exp", "relu": "ml::ReLU", "sigmoid": "ml::Sigmoid", "sqrt": "ml::Sqrt",

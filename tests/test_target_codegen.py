@@ -939,3 +939,47 @@ def test_softmax_written_in_pieces_becomes_one_node(tmp_path):
     codes = [n["code"] for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
     assert "ml::Softmax" not in codes and "ml::Max" in codes and "ml::Sum" in codes
     assert all(n["implementation_type"].startswith("ROCM") for n in s.library_nodes() if n["code"] != "ROCMOffloading")
+
+
+def test_builder_map_nest_generates_a_kernel_and_its_launch(tmp_path):
+    """add_map_nest: relu(a * b + bias row) over [_s0, _s1] spelled as three statements. The two loops are one walk
+    for a, b and y but not for the bias, so the kernel keeps both; with equally shaped operands only, the nest
+    collapses to a single loop and the kernel takes no strides."""
+    b = StructuredSDFGBuilder("mapped")
+    for n in ("A", "B", "Y"):
+        b.add_container(n, F32, True)
+    b.add_container("bias", F32, True)
+    b.add_container("alpha", Scalar(PrimitiveType.Float), True)
+    for n in ("_s0", "_s1"):
+        b.add_container(n, Scalar(PrimitiveType.Int64), True)
+    row = ["_s1", "1"]
+    b.add_map_nest([("i", "_s0"), ("j", "_s1")], [("a", "A", row), ("b", "B", row), ("c", "bias", ["0", "1"])],
+                   [("p", "fp_mul", ["a", "b"]), ("q", "fp_fma", ["p", "s", "c"]), ("r", "fmax", [0.0, "q"])], [("Y", row, "r")],
+                   scalars=[("s", "alpha")])
+    b.add_map_nest([("i", "_s0"), ("j", "_s1")], [("a", "A", row)], [("t", "tanh", ["a"]), ("u", "fp_sub", ["t", 0.5])], [("B", row, "u")])
+    s = b.move()
+    s.validate()
+    first, second = s.library_nodes()
+    assert first["symbols"] == ["_s0", "_s1"] and first["reads"][2]["extent"] == "1 + ((_s1) - 1)*(1)"
+    assert first["statements"][2] == {"out": "_v2", "type": "Float", "op": "fmax", "args": ["#0.0f", "_v1"]}
+    s.schedule("rocm", options={"offload": "none"})
+    report = s.generate(str(tmp_path))
+    src = Path(report["source"]).read_text()
+    texts = {p.name: p.read_text() for p in sorted(tmp_path.glob("kernel_mapped_*.hip"))}
+    assert len(texts) == 2
+    one, two = texts.values()
+    assert "float _c0, long long b0, long long b1, long long st__in0_0" in one and "__builtin_fmaf((float) (_v0), (float) (_c0), (float) (_in2))" in one
+    assert "long long b0)" in two and "b1" not in two and "st_" not in two          # one merged loop, no strides
+    assert "const I i0 = gid * V;" in two and "tanhf(" in two
+    assert '(void *) &_c0' in src and "(long long) ((_s0)*(_s1))" in src
+    # statements may only use what is defined before them; operations must be known
+    bad = StructuredSDFGBuilder("bad")
+    bad.add_container("A", F32, True)
+    bad.add_map_nest([("i", 8)], [("a", "A", ["1"])], [("p", "fp_add", ["a", "later"]), ("later", "assign", ["a"])], [("A", ["1"], "p")])
+    with pytest.raises(InvalidSDFGException, match="before it is defined"):
+        bad.move().validate()
+    bad = StructuredSDFGBuilder("bad2")
+    bad.add_container("A", F32, True)
+    bad.add_map_nest([("i", 8)], [("a", "A", ["1"])], [("p", "fp_sqrt", ["a"])], [("A", ["1"], "p")])
+    with pytest.raises(InvalidSDFGException, match="unknown operation 'fp_sqrt'"):
+        bad.move().validate()
