@@ -19,9 +19,9 @@ struct ConvParams {
     int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
 };
 
-int64_t out_dim(int64_t d_in, int64_t pad, int64_t dil, int64_t kernel, int64_t stride) {
-    // reference conv_node.cpp:224-233 with pads_begin == pads_end
-    const int64_t num = d_in + 2 * pad - (dil * (kernel - 1) + 1);
+int64_t out_dim(int64_t d_in, int64_t pad_begin, int64_t pad_end, int64_t dil, int64_t kernel, int64_t stride) {
+    // reference conv_node.cpp:224-233
+    const int64_t num = d_in + pad_begin + pad_end - (dil * (kernel - 1) + 1);
     return num < 0 ? 0 : num / stride + 1;
 }
 
@@ -92,12 +92,16 @@ ConvPath choose_path(int64_t N, int64_t C, int64_t OC, int64_t KH, int64_t KW, i
 
 } // namespace
 
-extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
-                                                        int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
-                                                        int64_t dil_w) {
+extern "C" int64_t docc_rocm_conv2d_f32_pads_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                                             int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                                                             int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h, int64_t dil_w) {
     if (N <= 0 || C <= 0 || OC <= 0 || KH <= 0 || KW <= 0 || stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0) return 0;
-    const int64_t OH = out_dim(H, pad_h, dil_h, KH, stride_h), OW = out_dim(W, pad_w, dil_w, KW, stride_w);
+    if (pad_h < 0 || pad_w < 0 || pad_h_end < 0 || pad_w_end < 0) return 0;
+    const int64_t OH = out_dim(H, pad_h, pad_h_end, dil_h, KH, stride_h), OW = out_dim(W, pad_w, pad_w_end, dil_w, KW, stride_w);
     if (OH <= 0 || OW <= 0) return 0;
+    // what decides between the paths is whether there is padding at all: the larger of begin and end stands for both
+    pad_h = pad_h > pad_h_end ? pad_h : pad_h_end;
+    pad_w = pad_w > pad_w_end ? pad_w : pad_w_end;
     if (KH == 1 && KW == 1 && stride_h == 1 && stride_w == 1 && pad_h == 0 && pad_w == 0) return 0;   // the input is the column matrix
     // nothing either when one of the direct kernels would be chosen anyway (operands assumed aligned)
     const bool halo_ok = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w);
@@ -109,14 +113,23 @@ extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, in
     return images * per_image;
 }
 
+extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                                        int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
+                                                        int64_t dil_w) {
+    return docc_rocm_conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, dil_h, dil_w);
+}
+
+// The kernels place the window with the begin pads and test every tap against the image, so the end pads only
+// enter through the output extents.
 static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
-                      int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X,
-                      const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
+                      int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h,
+                      int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
     if (N < 0 || C < 0 || H < 0 || W < 0 || OC < 0 || KH <= 0 || KW <= 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
-    if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0)
+    if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0 || pad_h_end < 0 || pad_w_end < 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: stride and dilation must be positive, padding non-negative");
-    const int64_t OH = out_dim(H, pad_h, dil_h, KH, stride_h), OW = out_dim(W, pad_w, dil_w, KW, stride_w);
+    const int64_t OH = out_dim(H, pad_h, pad_h_end, dil_h, KH, stride_h), OW = out_dim(W, pad_w, pad_w_end, dil_w, KW, stride_w);
+    const int64_t any_pad_h = pad_h > pad_h_end ? pad_h : pad_h_end, any_pad_w = pad_w > pad_w_end ? pad_w : pad_w_end;
     if (N == 0 || OC == 0 || OH == 0 || OW == 0) return 0;
     if (!Y || !Wt || (C > 0 && !X)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: null pointer");
     const int64_t lim = 0x7fffffffLL;
@@ -130,10 +143,11 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     // Stride-1, dilation-1 3x3 and 1x1 convolutions take the LDS-halo kernel: 64 output channels x a
     // strip of TH full output rows (at most 448 pixels) per work-group, 8 input channels per chunk.
     const bool halo_shape = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w) && ((uintptr_t) Wt % 16 == 0);
-    const int64_t need = docc_rocm_conv2d_f32_workspace_bytes(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w);
+    const int64_t need = docc_rocm_conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end,
+                                                                   dil_h, dil_w);
     const bool have_workspace = workspace && workspace_bytes >= need && need > 0 && ((uintptr_t) workspace % 256) == 0;
     const ConvPath path = C == 0 ? ConvPath::Gather
-                                 : choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, pad_h, pad_w, halo_shape, have_workspace);
+                                 : choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, any_pad_h, any_pad_w, halo_shape, have_workspace);
     if (path == ConvPath::Gemm1x1) {
         // Y[n] (OC x P) = W (OC x C) X[n] (C x P): one batched GEMM on the tensors as they lie; the bias is
         // written first and accumulated onto
@@ -229,13 +243,21 @@ extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_
                                     int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h,
                                     int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
                                     const float* bias, float* Y) {
-    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, nullptr, 0);
+    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, nullptr, 0);
 }
 
 extern "C" int docc_rocm_conv2d_f32_ws(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
                                        int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h,
                                        int64_t pad_w, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
                                        const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
-    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, workspace,
+    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y, workspace,
                       workspace_bytes);
+}
+
+extern "C" int docc_rocm_conv2d_f32_pads(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                                         int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                                         int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h, int64_t dil_w, const float* X,
+                                         const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
+    return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w, X, Wt, bias, Y,
+                      workspace, workspace_bytes);
 }

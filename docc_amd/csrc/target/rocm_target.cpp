@@ -290,16 +290,16 @@ protected:
         std::ostringstream dims;
         dims << c.shape()[0] << ", " << c.shape()[1] << ", " << c.shape()[2] << ", " << c.shape()[3] << ", " << c.output_channels() << ", "
              << c.kernel_shape()[0] << ", " << c.kernel_shape()[1] << ", " << get(c.strides(), 0, "1") << ", " << get(c.strides(), 1, "1")
-             << ", " << get(c.pads(), 0, "0") << ", " << get(c.pads(), 1, "0") << ", " << get(c.dilations(), 0, "1") << ", "
-             << get(c.dilations(), 1, "1");
+             << ", " << get(c.pads(), 0, "0") << ", " << get(c.pads(), 1, "0") << ", " << get(c.pads(), 2, "0") << ", " << get(c.pads(), 3, "0")
+             << ", " << get(c.dilations(), 0, "1") << ", " << get(c.dilations(), 1, "1");   // pads: begins, then ends
         // layers that run as im2col + GEMM take their column matrix from a workspace that lives around the node;
         // for the others the size is 0 and nothing is allocated
         s << "{" << std::endl;
         s.setIndent(s.indent() + 4);
-        s << "const int64_t __ws_bytes = docc_rocm_conv2d_f32_workspace_bytes(" << dims.str() << ");" << std::endl;
+        s << "const int64_t __ws_bytes = docc_rocm_conv2d_f32_pads_workspace_bytes(" << dims.str() << ");" << std::endl;
         s << "void *__ws = nullptr;" << std::endl;
         s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc_async(&__ws, (size_t) __ws_bytes, nullptr));" << std::endl;
-        s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32_ws(nullptr, " << dims.str() << ", (const float *) " << name_of("X")
+        s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32_pads(nullptr, " << dims.str() << ", (const float *) " << name_of("X")
           << ", (const float *) " << name_of("W") << ", "
           << (c.has_bias() ? "(const float *) " + name_of("B") : std::string("nullptr")) << ", (float *) " << name_of("Y")
           << ", __ws, __ws_bytes));" << std::endl;
@@ -952,8 +952,6 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (c->kernel_shape().size() != 2) return decline("only 2-d convolution is supported");
         int64_t group = 0;
         if (!symbolic::is_integer(c->group(), &group) || group != 1) return decline("only group == 1 is supported");
-        if (!c->pads().empty() && (c->pads()[0] != c->pads()[2] || c->pads()[1] != c->pads()[3]))
-            return decline("padding must be symmetric (begin == end)");
     } else if (node.code() == tensor::LibraryNodeType_Attention) {
         auto* a = dynamic_cast<tensor::AttentionNode*>(&node);
         if (!a) return decline("not an Attention node object");

@@ -80,6 +80,8 @@ _SIGNATURES = {
     "docc_rocm_softmax_ws": [_vp, _int, _i64, _i64, _i64, _vp, _vp, _vp, _i64],
     "docc_rocm_softmax_noalloc": [_vp, _int, _i64, _i64, _i64, _vp, _vp],
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
+    "docc_rocm_conv2d_f32_pads_workspace_bytes": [_i64] * 15,
+    "docc_rocm_conv2d_f32_pads": [_vp] + [_i64] * 15 + [_vp, _vp, _vp, _vp, _vp, _i64],
     "docc_rocm_conv2d_f32_workspace_bytes": [_i64] * 13,
     "docc_rocm_conv2d_f32_ws": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp, _vp, _i64],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
@@ -105,7 +107,7 @@ _SIGNATURES = {
 }
 _RESTYPE = {"docc_rocm_last_error": ctypes.c_char_p, "docc_rocm_version": ctypes.c_char_p,
             "docc_rocm_report_failure": None, "docc_rocm_attention_bf16_workspace_bytes": _i64, "docc_rocm_softmax_workspace_bytes": _i64,
-            "docc_rocm_conv2d_f32_workspace_bytes": _i64}
+            "docc_rocm_conv2d_f32_workspace_bytes": _i64, "docc_rocm_conv2d_f32_pads_workspace_bytes": _i64}
 
 #: every symbol the two public headers declare
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -310,6 +312,18 @@ def conv2d_f32_workspace_bytes(N, C, H, W, OC, KH, KW, stride, pad, dilation) ->
 def conv2d_f32_ws(N, C, H, W, OC, KH, KW, stride, pad, dilation, X, Wt, bias, Y, workspace, workspace_bytes, stream=0) -> None:
     """conv2d_f32 with device memory for a column matrix (conv2d_f32_workspace_bytes(...) bytes, 0 = none needed)."""
     call("docc_rocm_conv2d_f32_ws", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pad[0], pad[1],
+         dilation[0], dilation[1], X, Wt, bias or None, Y, workspace or None, workspace_bytes)
+
+
+def conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride, pads, dilation) -> int:
+    """`pads`: (top, left, bottom, right), the node's order (begins, then ends)."""
+    return int(lib().docc_rocm_conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride[0], stride[1], pads[0], pads[1], pads[2], pads[3],
+                                                                dilation[0], dilation[1]))
+
+
+def conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, pads, dilation, X, Wt, bias, Y, workspace=0, workspace_bytes=0, stream=0) -> None:
+    """The convolution with a begin and an end pad per axis: `pads` = (top, left, bottom, right)."""
+    call("docc_rocm_conv2d_f32_pads", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pads[0], pads[1], pads[2], pads[3],
          dilation[0], dilation[1], X, Wt, bias or None, Y, workspace or None, workspace_bytes)
 
 

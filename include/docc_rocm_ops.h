@@ -186,6 +186,20 @@ int docc_rocm_conv2d_f32_ws(docc_rocm_stream_t stream, int64_t N, int64_t C, int
                             float* Y, void* workspace, int64_t workspace_bytes);
 
 /*
+ * The same node with the pads the reference's node carries: a begin and an end per spatial axis
+ * (conv_node.cpp:76-77 `pads`: begins, then ends; :169-176 validation; :224-233 output extents)
+ *   ih = oh*stride_h - pad_h + kh*dil_h,   OH = (H + pad_h + pad_h_end - dil_h*(KH-1) - 1) / stride_h + 1   (same for W).
+ * `workspace` as for docc_rocm_conv2d_f32_ws (NULL: the direct kernels only).
+ */
+int64_t docc_rocm_conv2d_f32_pads_workspace_bytes(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                                  int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                                                  int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h, int64_t dil_w);
+int docc_rocm_conv2d_f32_pads(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
+                              int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w,
+                              int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h, int64_t dil_w, const float* X,
+                              const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes);
+
+/*
  * ml::Attention (a node the rocm target adds; the reference has none):
  *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
  * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32

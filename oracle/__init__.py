@@ -57,6 +57,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.oracle_conv_out_dim.argtypes = [_i64] * 6
     lib.oracle_conv_out_dim.restype = _i64
     lib.oracle_conv2d_f32.argtypes = [_i64] * 13 + [_f32p, _f32p, _f32p, _f32p]
+    lib.oracle_conv2d_f32_pads.argtypes = [_i64] * 15 + [_f32p, _f32p, _f32p, _f32p]
     lib.oracle_attention_bf16.argtypes = [_i64] * 5 + [ctypes.c_float, _u16p, _u16p, _u16p, _f32p]
     lib.oracle_attention_bf16.restype = ctypes.c_int
     lib.oracle_elementwise_unary_f32.argtypes = [ctypes.c_int, _i64, _f32p, _f32p]
@@ -208,6 +209,7 @@ def conv_out_dim(d_in, pad, dilation, kernel, stride) -> int:
 
 
 def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None) -> np.ndarray:
+    """`pad`: (height, width) on both sides, or (top, left, bottom, right) as the node orders them (begins, then ends)."""
     lib = lib or load()
     X = _c(X, np.float32)
     W = _c(W, np.float32)
@@ -215,12 +217,13 @@ def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None
     OC, C2, KH, KW = W.shape
     if C2 != C:
         raise ValueError("group != 1 is not supported")
-    OH = conv_out_dim(H, pad[0], dilation[0], KH, stride[0])
-    OW = conv_out_dim(Wd, pad[1], dilation[1], KW, stride[1])
+    pad = tuple(pad) if len(pad) == 4 else (pad[0], pad[1], pad[0], pad[1])
+    OH = int(lib.oracle_conv_out_dim(H, pad[0], pad[2], dilation[0], KH, stride[0]))
+    OW = int(lib.oracle_conv_out_dim(Wd, pad[1], pad[3], dilation[1], KW, stride[1]))
     Y = np.empty((N, OC, OH, OW), np.float32)
     b = None if bias is None else _c(bias, np.float32)
-    lib.oracle_conv2d_f32(N, C, H, Wd, OC, KH, KW, stride[0], stride[1], pad[0], pad[1], dilation[0], dilation[1],
-                          _p(X, _f32p), _p(W, _f32p), _p(b, _f32p) if b is not None else None, _p(Y, _f32p))
+    lib.oracle_conv2d_f32_pads(N, C, H, Wd, OC, KH, KW, stride[0], stride[1], pad[0], pad[1], pad[2], pad[3], dilation[0], dilation[1],
+                               _p(X, _f32p), _p(W, _f32p), _p(b, _f32p) if b is not None else None, _p(Y, _f32p))
     return Y
 
 

@@ -356,11 +356,14 @@ ORACLE_API int64_t oracle_conv_out_dim(int64_t d_in, int64_t pad_begin, int64_t 
  * of bounds; the ONNX Conv definition its header cites (conv_node.h:9-22)
  * pads with zeros, which is what the guard below does.
  */
-ORACLE_API void oracle_conv2d_f32(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
-                                  int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
-                                  int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y) {
-    int64_t OH = oracle_conv_out_dim(H, pad_h, pad_h, dil_h, KH, stride_h);
-    int64_t OW = oracle_conv_out_dim(W, pad_w, pad_w, dil_w, KW, stride_w);
+/* pads as the node carries them (conv_node.cpp:76-77, 169-176): a begin and an end per spatial axis; the begin pad
+ * moves the window, the end pad only adds output positions (conv_node.cpp:224-233). */
+ORACLE_API void oracle_conv2d_f32_pads(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                       int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end,
+                                       int64_t pad_w_end, int64_t dil_h, int64_t dil_w, const float* X, const float* Wt,
+                                       const float* bias, float* Y) {
+    int64_t OH = oracle_conv_out_dim(H, pad_h, pad_h_end, dil_h, KH, stride_h);
+    int64_t OW = oracle_conv_out_dim(W, pad_w, pad_w_end, dil_w, KW, stride_w);
 #pragma omp parallel for schedule(static)
     for (int64_t n = 0; n < N; n++) {
         for (int64_t oc = 0; oc < OC; oc++) {
@@ -383,6 +386,12 @@ ORACLE_API void oracle_conv2d_f32(int64_t N, int64_t C, int64_t H, int64_t W, in
             }
         }
     }
+}
+
+ORACLE_API void oracle_conv2d_f32(int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
+                                  int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t dil_h,
+                                  int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y) {
+    oracle_conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h, pad_w, dil_h, dil_w, X, Wt, bias, Y);
 }
 
 /* ------------------------------------------------------------- Attention */

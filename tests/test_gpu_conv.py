@@ -200,3 +200,50 @@ def test_conv_workspace_chunks_over_images(rt, monkeypatch):
     assert need > 0 and need % N == 0
     Y, _ = run_conv_ws(rt, X, Wt, b, (1, 1), (1, 1), (1, 1), workspace_bytes=need)
     assert np.array_equal(Y, oracle.conv2d(X, Wt, b, (1, 1), (1, 1), (1, 1)))
+
+
+# ---- a begin and an end pad per axis (the node's `pads`: begins, then ends; conv_node.cpp:76-77, 224-233) ------------
+
+PAD_CASES = [  # (N, C, H, W, OC, KH, KW, stride, (top, left, bottom, right), dilation, bias)
+    (2, 16, 12, 20, 70, 3, 3, (1, 1), (0, 1, 2, 0), (1, 1), True),     # halo shape, nothing above, two rows below
+    (1, 8, 9, 9, 64, 3, 3, (1, 1), (2, 2, 0, 1), (1, 1), False),      # halo shape, more before than after
+    (3, 5, 11, 13, 17, 3, 2, (2, 1), (1, 0, 0, 3), (1, 2), True),     # strides, dilation, odd channels: the gather kernel
+    (2, 24, 7, 7, 32, 1, 1, (1, 1), (0, 0, 1, 1), (1, 1), True),      # 1x1 with padding at the end only: not the pointwise GEMM
+    (2, 32, 10, 10, 40, 5, 5, (1, 1), (4, 0, 0, 4), (1, 1), False),   # a large filter hanging over one corner
+]
+
+
+@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", ""])
+@pytest.mark.parametrize("case", PAD_CASES)
+def test_conv_with_different_pads_before_and_after(rt, monkeypatch, force, case):
+    N, C, H, W, OC, KH, KW, stride, pads, dil, use_bias = case
+    if force:
+        monkeypatch.setenv("DOCC_ROCM_CONV", force)
+    rng = np.random.default_rng(hash(case[:7]) & 0xffff)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, C, KH, KW)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    ref = oracle.conv2d(X, Wt, b, stride, pads, dil)
+    # the extents follow begin + end; an independent statement of the same: pad the image by hand, convolve without pads
+    Xp = np.pad(X, ((0, 0), (0, 0), (pads[0], pads[2]), (pads[1], pads[3])))
+    assert np.array_equal(ref, oracle.conv2d(Xp, Wt, b, stride, (0, 0), dil))
+    x, w = dev(X), dev(Wt)
+    bd = dev(b) if b is not None else None
+    y = torch.full(ref.shape, float("nan"), device="cuda")
+    need = rt.conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride, pads, dil)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+    rt.conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, pads, dil, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0,
+                       y.data_ptr(), ws.data_ptr() if need else 0, need)
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    # equal pads through the new entry point are the old entry point
+    if force == "":
+        sym = (pads[0], pads[1], pads[0], pads[1])
+        y1 = torch.full(oracle.conv2d(X, Wt, b, stride, sym, dil).shape, float("nan"), device="cuda")
+        y2 = torch.full_like(y1, float("nan"))
+        rt.conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, sym, dil, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y1.data_ptr())
+        rt.conv2d_f32(N, C, H, W, OC, KH, KW, stride, sym[:2], dil, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y2.data_ptr())
+        torch.cuda.synchronize()
+        assert torch.equal(y1, y2)
+    with pytest.raises(rt.RocmRuntimeError, match="padding non-negative"):
+        rt.conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, (0, 0, -1, 0), dil, x.data_ptr(), w.data_ptr(), 0, y.data_ptr())

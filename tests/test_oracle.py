@@ -474,3 +474,20 @@ def test_map_nest_cmath_calls_are_the_libm_functions(dtype):
         got = oracle.map_nest(node, {"a": a, "b": other})["y"].astype(np.float64)
         ref = fn(a.astype(np.float64), other.astype(np.float64))
         assert np.abs(got - ref).max() <= tol * max(1.0, np.abs(ref).max()), stem
+
+
+def test_conv2d_with_a_begin_and_an_end_pad_per_axis():
+    """torch pads by hand (F.pad takes left, right, top, bottom) and convolves without padding, in float64: the begin pad
+    moves the window, the end pad only adds output positions. Swapping begin and end, or rows and columns, fails."""
+    rng = np.random.default_rng(31)
+    X = rng.standard_normal((2, 3, 9, 11)).astype(np.float32)
+    W = rng.standard_normal((4, 3, 3, 2)).astype(np.float32)
+    b = rng.standard_normal(4).astype(np.float32)
+    for pads, stride, dil in (((0, 1, 2, 0), (1, 1), (1, 1)), ((2, 0, 1, 3), (2, 1), (1, 2)), ((1, 2, 3, 4), (1, 2), (2, 1))):
+        top, left, bottom, right = pads
+        xp = torch.nn.functional.pad(torch.from_numpy(X).double(), (left, right, top, bottom))
+        ref = torch.nn.functional.conv2d(xp, torch.from_numpy(W).double(), torch.from_numpy(b).double(), stride=stride, dilation=dil).numpy()
+        got = oracle.conv2d(X, W, b, stride, pads, dil)
+        assert got.shape == ref.shape and np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    # two-element pads mean the same on both sides
+    assert np.array_equal(oracle.conv2d(X, W, b, pad=(1, 2)), oracle.conv2d(X, W, b, pad=(1, 2, 1, 2)))

@@ -146,6 +146,19 @@ def test_mapper_sets_implementation_types_and_declines_what_the_kernels_lack():
     b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 4, group=2)
     with pytest.raises(InvalidSDFGException, match="group"):
         b.move().schedule("rocm")
+    # a convolution whose pads differ between begin and end is taken: the launcher gets all four (begins, then ends)
+    b = StructuredSDFGBuilder("cp")
+    for n in ("X", "W", "Y"):
+        b.add_container(n, F32, True)
+    b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [0, 1, 2, 0], [1, 1], 4)
+    s = b.move()
+    s.schedule("rocm", options={"offload": "none"})
+    assert s.library_nodes()[0]["implementation_type"] == "ROCMWithoutTransfers"
+    import tempfile
+    with tempfile.TemporaryDirectory() as folder:
+        text = re.sub(r"\s+", " ", Path(s.generate(folder)["source"]).read_text())
+    assert "docc_rocm_conv2d_f32_pads(nullptr, 1, 4, 8, 8, 4, 3, 3, 1, 1, 0, 1, 2, 0, 1, 1, (const float *) X" in text
+    assert "docc_rocm_conv2d_f32_pads_workspace_bytes(1, 4, 8, 8, 4, 3, 3, 1, 1, 0, 1, 2, 0, 1, 1)" in text
     b = StructuredSDFGBuilder("a")
     for n in ("Q", "K", "V"):
         b.add_container(n, F32, True)
