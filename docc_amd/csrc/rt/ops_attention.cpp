@@ -28,7 +28,10 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
     // MFMAs: fewer instructions per flop) once that still gives every CU its two resident work-groups, else 128
     // per work-group (more, smaller work-groups). DOCC_ROCM_ATTENTION_Q=128|256 forces one (tuning and tests).
     const int64_t BH = B * H, out_bytes = out_bf16 ? 2 : 4;
-    int per_group = ((SQ + 255) / 256) * BH >= 2 * compute_units() ? 256 : 128;
+    // ... and only where the larger groups do not add padded queries: a wavefront multiplies its 64 queries whether they
+    // exist or not (SQ = 100 would run 256 queries in the large form and 128 in the small one)
+    const bool no_extra_padding = (SQ + 255) / 256 * 256 <= (SQ + 127) / 128 * 128 || SQ >= 1024;
+    int per_group = ((SQ + 255) / 256) * BH >= 2 * compute_units() && no_extra_padding ? 256 : 128;
     if (const char* force = std::getenv("DOCC_ROCM_ATTENTION_Q")) {
         const int v = std::atoi(force);
         if (v == 128 || v == 256) per_group = v;

@@ -267,3 +267,44 @@ def test_attention_more_pairs_than_one_grid_holds(rt):
     for p in (0, 65534, 65535, 69999):
         ref = oracle.attention(bits(flat(Q)[:, p:p + 1].cpu()), bits(flat(K)[:, p:p + 1].cpu()), bits(flat(V)[:, p:p + 1].cpu()))
         assert rel_err_max(flat(o)[:, p:p + 1].cpu().numpy(), ref) <= TOL_BF16, p
+
+
+def test_many_heads_with_few_queries(rt, kernel_form):
+    """Enough (batch, head) pairs to fill the device with 256-query groups, but only 100 queries each: the launcher's
+    own choice must be the 128-query form (the other would multiply 256 queries, 156 of them padding), and every form
+    gives the oracle's result."""
+    import time
+    g = torch.Generator().manual_seed(100)
+    B, H, SQ, SKV = 8, 128, 100, 192
+    Q, K, V = (torch.randn(B, H, s, 64, generator=g).bfloat16() for s in (SQ, SKV, SKV))
+    O = run_attention(rt, bits(Q), bits(K), bits(V))
+    heads = [(0, 0), (3, 77), (7, 127)]
+    for b, h in heads:
+        ref = oracle.attention(bits(Q[b:b + 1, h:h + 1]), bits(K[b:b + 1, h:h + 1]), bits(V[b:b + 1, h:h + 1]))
+        assert rel_err_max(O[b, h], ref[0, 0]) <= TOL_BF16
+    if kernel_form is None:
+        # the choice itself, seen from outside: the automatic launch takes about as long as the forced 128-query form
+        q, k, v = dev(bits(Q)), dev(bits(K)), dev(bits(V))
+        o = torch.empty(B, H, SQ, 64, device="cuda")
+
+        def timed(force):
+            import os
+            if force:
+                os.environ["DOCC_ROCM_ATTENTION_Q"] = force
+            else:
+                os.environ.pop("DOCC_ROCM_ATTENTION_Q", None)
+            try:
+                for _ in range(5):
+                    rt.attention_bf16(B, H, SQ, SKV, 64, 0.125, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr())
+                rt.device_sync()
+                e0, e1 = rt.Event(), rt.Event()
+                e0.record()
+                for _ in range(20):
+                    rt.attention_bf16(B, H, SQ, SKV, 64, 0.125, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr())
+                e1.record()
+                return e0.elapsed_ms(e1)
+            finally:
+                os.environ.pop("DOCC_ROCM_ATTENTION_Q", None)
+
+        auto, small, large = timed(None), timed("128"), timed("256")
+        assert abs(auto - small) <= 0.25 * small and small < large, (auto, small, large)
