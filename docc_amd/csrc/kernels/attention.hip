@@ -23,11 +23,15 @@
 //                                                are (the k-order of the MFMA is permuted to
 //                                                the accumulator's row order on both operands).
 //
-// On this device the kernel runs against the power limit, not against a pipe: with pieces of the block loop
-// taken out one at a time its time falls by the share of the instructions removed, whatever pipe they ran on
-// (16 MFMAs 56 %, the eight 128-bit K reads 10 %, the sixteen transposed V reads 6 %, the copies 9 %, 16 dot2
-// 7.6 %, 32 exp 17 %, 32 fma 7 %), and overlapping them better (score MFMAs of the next block issued between the
-// exponentials) changes nothing. So the design goal is the fewest instructions per flop:
+// What bounds it on this device: the vector ALU next to the matrix pipe. Per 64-key block and 64 queries a wave issues
+// 32 MFMAs (1024 cycles of the matrix pipe) and 64 exp2, 64 fma, 32 cvt_pk, 32 dot2 (about as many cycles of the vector
+// pipe), and the two hardly overlap: with pieces of the block loop taken out one at a time the time falls by the share
+// of the instructions removed, whatever pipe they ran on (16 MFMAs 56 %, the eight 128-bit K reads 10 %, the sixteen
+// transposed V reads 6 %, the copies 9 %, 16 dot2 7.6 %, 32 exp 17 %, 32 fma 7 %), and a wave that streams MFMAs
+// leaves the other wave of its SIMD about 55 % of the vector pipe's rate (measured with two-wave probes: 24 such vector
+// instructions take 71 ns alone and 128 ns beside a wave issuing MFMAs back to back, which itself is not slowed).
+// Issuing the score MFMAs of the next block between the exponentials changes nothing. The power limit adds about 8 %
+// on N(0,1) operands (the same launch on zeros). So the design goal is the fewest instructions per flop:
 //   - QT = 2: a wavefront takes 64 queries, so every K and V operand read from LDS, and every block copied
 //     into LDS, serves twice the MFMAs (LDS reads and copies per flop halve);
 //   - p = exp2(s * c - m) with c = scale * log2(e) applied to the fp32 score by one fma: Q and K enter
