@@ -170,3 +170,40 @@ def test_module_load_get_function_and_launch(tmp_path, rt):
     with pytest.raises(rt.RocmRuntimeError, match="block of 2048 threads"):
         rt.call("docc_rocm_launch", fn, grid, (ctypes.c_uint32 * 3)(2048, 1, 1), 0, None, args)
     rt.call("docc_rocm_module_unload", module)
+
+
+def test_generated_kernel_with_64_bit_indices(tmp_path, rt):
+    """More than 2^31 elements per operand: the host code picks the entry points that compute indices in 64 bits (the
+    vector form for the aligned extent, the element form for an extent that is no multiple of four)."""
+    import torch
+    from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFGBuilder
+
+    b = StructuredSDFGBuilder("wide_map")
+    for n in ("A", "Y"):
+        b.add_container(n, Pointer(Scalar(PrimitiveType.Float)), True)
+    b.add_container("_s0", Scalar(PrimitiveType.Int64), True)
+    b.add_map_nest([("i", "_s0")], [("a", "A", ["1"])], [("t", "fp_mul", ["a", 2.0]), ("u", "fp_add", ["t", 1.0])], [("Y", ["1"], "u")])
+    s = b.move()
+    s.schedule("rocm", options={"offload": "none"})
+    fn = ctypes.CDLL(s._compile(str(tmp_path))).wide_map
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64]
+    fn.restype = None
+    n = (1 << 31) + 4096
+    a = torch.empty(n + 3, device="cuda")
+    a[: 1 << 20] = torch.arange(1 << 20, device="cuda", dtype=torch.float32)
+    a[1 << 20:] = 3.0
+    a[n - 5:] = torch.arange(8, device="cuda", dtype=torch.float32)        # the far end, past 2^31
+    y = torch.zeros(n + 3, device="cuda")
+    for count in (n, n + 3):                                                 # a multiple of four, then not
+        y.zero_()
+        torch.cuda.synchronize()
+        fn(a.data_ptr(), y.data_ptr(), count)
+        torch.cuda.synchronize()
+        assert runtime.take_failure() == (0, "")
+        assert torch.equal(y[: 1 << 20], a[: 1 << 20] * 2 + 1)
+        assert torch.equal(y[count - 8:count], a[count - 8:count] * 2 + 1)
+        assert float(y[(1 << 31) + 7]) == 7.0 and (count == n + 3 or float(y[n:].abs().max()) == 0.0)
+        # a checksum over everything: 2 * sum(a) + count, in float64 by chunks
+        total = sum(float(y[i:i + (1 << 28)].double().sum()) for i in range(0, count, 1 << 28))
+        ref = sum(float(a[i:min(i + (1 << 28), count)].double().sum()) for i in range(0, count, 1 << 28)) * 2 + count
+        assert abs(total - ref) <= 1e-9 * ref
