@@ -1489,11 +1489,11 @@ bool RocmDataTransferMinimizationPass::run_pass(builder::StructuredSDFGBuilder& 
             if (!b.node) continue;
             if (is_offloading(b)) {
                 const auto& node = offloading(b);
-                if (node.is_d2h() && b.outputs[0].data == host && node.size() == bytes) return false;
+                if (node.is_d2h() && b.outputs[0].data == host && symbolic::equal(node.size(), bytes)) return false;
                 if (node.is_h2d() && b.inputs[0].data == host) {
                     const auto it = current.find(host);
                     // an upload that will not be dropped reads the host memory
-                    if (it == current.end() || it->second.bytes != node.size() || it->second.device_id != node.device_id()) return true;
+                    if (it == current.end() || !symbolic::equal(it->second.bytes, node.size()) || it->second.device_id != node.device_id()) return true;
                 }
                 continue;
             }
@@ -1542,7 +1542,7 @@ bool RocmDataTransferMinimizationPass::run_pass(builder::StructuredSDFGBuilder& 
         if (node.is_h2d()) {
             const std::string host = b.inputs[0].data, device = b.outputs[0].data;
             const auto it = current.find(host);
-            if (node.is_alloc() && it != current.end() && it->second.bytes == node.size() && it->second.device_id == node.device_id()) {
+            if (node.is_alloc() && it != current.end() && symbolic::equal(it->second.bytes, node.size()) && it->second.device_id == node.device_id()) {
                 renamed[device] = it->second.device;      // the value is on the device already
                 applied = true;
                 continue;
@@ -1584,7 +1584,7 @@ bool RocmDataTransferMinimizationPass::run_pass(builder::StructuredSDFGBuilder& 
                 else if (offloading(old[j]).is_free() && old[j].inputs[0].data == device) break;
             }
             const auto it = host.empty() ? current.end() : current.find(host);
-            if (it != current.end() && it->second.bytes == node.size() && it->second.device_id == node.device_id()) {
+            if (it != current.end() && symbolic::equal(it->second.bytes, node.size()) && it->second.device_id == node.device_id()) {
                 renamed[device] = it->second.device;      // the old value's buffer is overwritten in place
                 applied = true;
                 continue;
@@ -1674,6 +1674,10 @@ void rocm_scheduling_passes(builder::StructuredSDFGBuilder& builder, analysis::A
     if (options.fuse_elementwise) {
         RocmElementwiseFusionPass fusion;
         fusion.run_pass(builder, analysis_manager);
+    }
+    if (options.fuse_elementwise && options.fuse_maps) {
+        RocmMapFusionPass maps;
+        maps.run_pass(builder, analysis_manager);
     }
     if (options.offload == "none") {
         // the caller's pointers are device pointers, so every array the nodes touch lives in HBM:

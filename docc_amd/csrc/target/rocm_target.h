@@ -83,6 +83,17 @@ public:
     bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
 };
 
+// Merges blocks of elementwise kind (tensor elementwise nodes, ROCMFusedElementWise, ml::Broadcast, ROCMMap with one
+// result) that the fusion pass above left as separate launches into one ROCMMap node, when the value in between is
+// a transient that only the later block reads: one generated kernel per chain, whatever its length and however many
+// of its operands are repeated rows or scalars. The merged block stands where the later one stood. Runs after
+// RocmElementwiseFusionPass, so a chain the prebuilt fused kernel takes whole needs no device compiler.
+class RocmMapFusionPass {
+public:
+    std::string name() { return "RocmMapFusion"; }
+    bool run_pass(builder::StructuredSDFGBuilder& builder, analysis::AnalysisManager& analysis_manager);
+};
+
 // Recognises softmax written out in its pieces - the form numpy code takes, and what the reference's SoftmaxNode
 // expands to (softmax_node.cpp:142-252): m = Max(X, axes, keepdims); e = Exp(X - broadcast(m)); Y = e / broadcast(Sum(e,
 // axes, keepdims)) - and replaces the seven nodes by one ml::Softmax when every value in between is a transient that
@@ -128,6 +139,9 @@ struct ScheduleOptions {
     bool fuse_elementwise = true;
     // run RocmSoftmaxPatternPass before the mapping
     bool match_softmax = true;
+    // run RocmMapFusionPass after the elementwise fusion, if that runs (its kernels are compiled by hipcc when the
+    // program is)
+    bool fuse_maps = true;
 };
 
 // The scheduling entry of the target: mapping pass (+ offloading passes).

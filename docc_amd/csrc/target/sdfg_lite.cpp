@@ -86,6 +86,94 @@ Expression product(const std::vector<Expression>& v, size_t begin, size_t end) {
     return p;
 }
 
+namespace {
+
+// integer polynomials over the symbols: sorted symbol list -> coefficient
+using Polynomial = std::map<std::vector<std::string>, int64_t>;
+
+struct PolynomialParser {
+    const std::string& text;
+    size_t at = 0;
+    bool ok = true;
+
+    void skip() {
+        while (at < text.size() && std::isspace((unsigned char) text[at])) at++;
+    }
+    static Polynomial times(const Polynomial& a, const Polynomial& b) {
+        Polynomial out;
+        for (auto& x : a)
+            for (auto& y : b) {
+                std::vector<std::string> symbols = x.first;
+                symbols.insert(symbols.end(), y.first.begin(), y.first.end());
+                std::sort(symbols.begin(), symbols.end());
+                out[symbols] += x.second * y.second;
+            }
+        return out;
+    }
+    Polynomial factor() {
+        skip();
+        Polynomial p;
+        if (at >= text.size()) {
+            ok = false;
+        } else if (text[at] == '(') {
+            at++;
+            p = sum();
+            skip();
+            if (at < text.size() && text[at] == ')') at++;
+            else ok = false;
+        } else if (text[at] == '-') {
+            at++;
+            p = times(Polynomial{{{}, -1}}, factor());
+        } else if (std::isdigit((unsigned char) text[at])) {
+            int64_t v = 0;
+            while (at < text.size() && std::isdigit((unsigned char) text[at])) v = v * 10 + (text[at++] - '0');
+            p[{}] = v;
+        } else if (std::isalpha((unsigned char) text[at]) || text[at] == '_') {
+            std::string name;
+            while (at < text.size() && (std::isalnum((unsigned char) text[at]) || text[at] == '_')) name += text[at++];
+            skip();
+            if (at < text.size() && text[at] == '(') ok = false;   // a call
+            p[{name}] = 1;
+        } else {
+            ok = false;
+        }
+        return p;
+    }
+    Polynomial product() {
+        Polynomial p = factor();
+        for (skip(); ok && at < text.size() && text[at] == '*'; skip()) {
+            at++;
+            p = times(p, factor());
+        }
+        return p;
+    }
+    Polynomial sum() {
+        Polynomial p = product();
+        for (skip(); ok && at < text.size() && (text[at] == '+' || text[at] == '-'); skip()) {
+            const int64_t sign = text[at++] == '+' ? 1 : -1;
+            for (auto& term : product()) p[term.first] += sign * term.second;
+        }
+        return p;
+    }
+    bool parse(Polynomial* out) {
+        Polynomial p = sum();
+        skip();
+        if (!ok || at != text.size()) return false;
+        for (auto it = p.begin(); it != p.end();) it = it->second == 0 ? p.erase(it) : std::next(it);
+        *out = std::move(p);
+        return true;
+    }
+};
+
+} // namespace
+
+bool equal(const Expression& a, const Expression& b) {
+    if (a == b) return true;
+    Polynomial pa, pb;
+    PolynomialParser parse_a{a}, parse_b{b};
+    return parse_a.parse(&pa) && parse_b.parse(&pb) && pa == pb;
+}
+
 } // namespace symbolic
 
 namespace {

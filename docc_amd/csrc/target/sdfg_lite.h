@@ -48,6 +48,9 @@ Expression integer(int64_t v);
 bool is_integer(const Expression& e, int64_t* value = nullptr);
 // v[begin] * ... * v[end - 1] ("1" for an empty range)
 Expression product(const std::vector<Expression>& v, size_t begin, size_t end);
+// Whether the two expressions denote the same value for every value of their symbols, as far as sums and products of
+// integers and symbols go ("(32)*16" and "512", "(n)*m" and "m*n"); anything else (quotients, calls) compares as text.
+bool equal(const Expression& a, const Expression& b);
 } // namespace symbolic
 
 // Implementation types, following the "<LIB>With[out]Transfers" naming of the

@@ -171,6 +171,7 @@ char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, con
             if (const json::Value* v = o.find("require_all_mapped")) options.require_all_mapped = v->as_bool();
             if (const json::Value* v = o.find("fuse")) options.fuse_elementwise = v->as_bool();
             if (const json::Value* v = o.find("match_softmax")) options.match_softmax = v->as_bool();
+            if (const json::Value* v = o.find("fuse_maps")) options.fuse_maps = v->as_bool();
         }
         builder::StructuredSDFGBuilder builder(*sdfg);
         analysis::AnalysisManager analysis_manager(*sdfg);

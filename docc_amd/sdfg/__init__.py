@@ -230,7 +230,7 @@ class StructuredSDFG:
             return
         if target != "rocm":
             raise NotImplementedError(f"Target '{target}' is not supported: this package provides the 'rocm' target only")
-        opts = {k: v for k, v in (options or {}).items() if k in ("offload", "require_all_mapped", "fuse", "match_softmax")}
+        opts = {k: v for k, v in (options or {}).items() if k in ("offload", "require_all_mapped", "fuse", "match_softmax", "fuse_maps")}
         self._data = json.loads(_call("docc_rocm_target_schedule", self.to_json(), category, json.dumps(opts)))
 
     def generate(self, output_folder: str, instrumentation_mode: str = "") -> Dict[str, Any]:

@@ -705,7 +705,9 @@ def test_power_operator_through_both_front_ends():
     got = norms(x, y)
     ref = np.sqrt(x ** 2 + y ** 2) ** (y / 4)
     np.testing.assert_allclose(got, ref, rtol=1e-13)
-    assert [n["code"] for n in norms.last_sdfg.library_nodes()].count("ml::Pow") == 3
+    # the whole expression is one chain of elementwise nodes: scheduled, it is one generated kernel with the three powers
+    (nest,) = [n for n in norms.last_sdfg.library_nodes() if n["code"] == "ROCMMap"]
+    assert [st["op"] for st in nest["statements"]].count("pow") == 3 and len(nest["reads"]) == 2
 
     class P(torch.nn.Module):
         def forward(self, a, b):
@@ -778,7 +780,10 @@ def test_casts_through_both_front_ends():
     got = widen(x, k)
     assert got.dtype == np.float64
     np.testing.assert_array_equal(got, np.sqrt(x.astype(np.float64)) + k.astype(np.float64))
-    assert [n["code"] for n in widen.last_sdfg.library_nodes() if n["code"].startswith("ml::")] == ["ml::Cast", "ml::Sqrt", "ml::Cast", "ml::Add"]
+    # the two casts are prebuilt kernels; the square root and the addition behind them are one generated kernel
+    nodes = [n for n in widen.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert [n["code"] for n in nodes] == ["ml::Cast", "ml::Cast", "ROCMMap"]
+    assert [st["op"] for st in nodes[2]["statements"]] == ["sqrt", "fp_add"]
 
     class Mixed(torch.nn.Module):
         def forward(self, q, k, v):

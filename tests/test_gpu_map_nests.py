@@ -207,3 +207,76 @@ def test_generated_kernel_with_64_bit_indices(tmp_path, rt):
         total = sum(float(y[i:i + (1 << 28)].double().sum()) for i in range(0, count, 1 << 28))
         ref = sum(float(a[i:min(i + (1 << 28), count)].double().sum()) for i in range(0, count, 1 << 28)) * 2 + count
         assert abs(total - ref) <= 1e-9 * ref
+
+
+# ---- chains of tensor nodes merged into one generated kernel (RocmMapFusionPass)
+
+def chain_program(name, elem, shape):
+    """y = sigmoid((a + b) * c - bias_row) * 0.5 + max(a, col) over `shape` = [r, c]: five two-operand operations, a
+    repeated row, a repeated column and a constant, which the prebuilt fused kernel (one two-operand operation) cannot
+    take in one launch."""
+    from docc_amd.sdfg import Pointer, PrimitiveType, Scalar, StructuredSDFGBuilder
+    T = Pointer(Scalar(PrimitiveType.Float if elem == np.float32 else PrimitiveType.Double))
+    r, c = shape
+    size = np.dtype(elem).itemsize
+    b = StructuredSDFGBuilder(name)
+    for n in ("A", "B", "C", "bias", "col", "Y"):
+        b.add_container(n, T, True)
+    for n in ("T0", "T1", "T2", "T3", "T4", "T5", "T6", "T7"):
+        b.add_container(n, T, False, transient_bytes=r * c * size)
+    b.add_elementwise_op("add", "A", "B", "T0", [r, c])
+    b.add_elementwise_op("mul", "T0", "C", "T1", [r, c])
+    b.add_broadcast("bias", "T2", [1, c], [r, c])
+    b.add_elementwise_op("sub", "T1", "T2", "T3", [r, c])
+    b.add_elementwise_unary_op("sigmoid", "T3", "T4", [r, c])
+    b.add_elementwise_op("mul", "T4", "0.5", "T5", [r, c])
+    b.add_broadcast("col", "T6", [r, 1], [r, c])
+    b.add_elementwise_op("max", "A", "T6", "T7", [r, c])
+    b.add_elementwise_op("add", "T5", "T7", "Y", [r, c])
+    return b.move()
+
+
+@pytest.mark.parametrize("elem,shape", [(np.float32, (64, 256)), (np.float32, (37, 129)), (np.float64, (33, 64)), (np.float32, (1, 8)),
+                                        (np.float32, (2048, 1024))])
+def test_chain_of_tensor_nodes_runs_as_one_generated_kernel(tmp_path, rt, elem, shape):
+    r, c = shape
+    rng = np.random.default_rng(31)
+    A, B, C = (rng.standard_normal((r, c)).astype(elem) for _ in range(3))
+    bias, col = rng.standard_normal(c).astype(elem), rng.standard_normal(r).astype(elem)
+    results = {}
+    for fuse_maps in (True, False):
+        s = chain_program(f"chain_{int(fuse_maps)}", elem, shape)
+        s.schedule("rocm", options={"fuse_maps": fuse_maps})
+        kernels = [n for n in s.library_nodes() if n["code"] != "ROCMOffloading"]
+        if fuse_maps:
+            assert [n["code"] for n in kernels] == ["ROCMMap"] and s.loop_report()["H2D"] == 5 and s.loop_report()["D2H"] == 1
+            node, fused_text = kernels[0], s.to_json()
+        else:
+            assert len(kernels) >= 4 and not any(n["code"] == "ROCMMap" for n in kernels)
+        fn = getattr(ctypes.CDLL(s._compile(str(tmp_path / str(fuse_maps)))), f"chain_{int(fuse_maps)}")
+        fn.argtypes = [ctypes.c_void_p] * 6
+        fn.restype = None
+        Y = np.full((r, c), np.nan, elem)
+        fn(*(a.ctypes.data for a in (A, B, C, bias, col, Y)))
+        assert runtime.take_failure() == (0, "")
+        results[fuse_maps] = Y
+    # the same operations in the same order, each rounded once: the merged kernel gives the bits of the launches it replaces
+    assert np.array_equal(results[True], results[False])
+    # the oracle's interpreter on the merged body, each load bound to the array its connector names
+    arrays = {"A": A, "B": B, "C": C, "bias": bias, "col": col}
+    operands, scalars = {}, {}
+    for blk in json.loads(fused_text)["root"]["children"]:
+        if blk["dataflow"]["library_node"]["code"] != "ROCMMap":
+            continue
+        for binding in blk["dataflow"]["inputs"]:
+            if "constant" in binding:
+                scalars[binding["connector"]] = float(binding["constant"])
+            else:
+                operands[binding["connector"]] = arrays[binding["data"].rsplit("_", 1)[1]]
+    assert len(operands) == 5 and list(scalars.values()) == [0.5]           # A is loaded once for its two uses
+    ref = oracle.map_nest(node, operands, scalars=scalars)
+    assert rel_err_max(results[True], ref["_out0"].reshape(r, c)) <= (1e-5 if elem == np.float32 else 1e-12)
+    # by hand, in float64
+    d = lambda x: x.astype(np.float64)
+    hand = 1.0 / (1.0 + np.exp(-((d(A) + d(B)) * d(C) - d(bias)[None, :]))) * 0.5 + np.maximum(d(A), d(col)[:, None])
+    assert rel_err_max(results[True], hand) <= (2e-6 if elem == np.float32 else 1e-12)

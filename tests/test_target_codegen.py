@@ -716,10 +716,21 @@ def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
     b.add_elementwise_op("sub", "T2", "T1", "Y", [100])        # T1 has a second reader
     b.add_elementwise_unary_op("exp", "Y", "Z", [100])         # Y is an argument: stays
     s = b.move()
-    s.schedule("rocm")
+    text = s.to_json()
+    s.schedule("rocm", options={"fuse_maps": False})
     nodes = [(n["code"], n.get("post"), n.get("binary")) for n in s.library_nodes() if not n["code"].startswith("ROCMOff")]
     assert nodes == [("ROCMFusedElementWise", ["ml::Abs", "ml::Sqrt"], ""), ("ml::Tanh", None, None), ("ml::Sub", None, None),
                      ("ml::Exp", None, None)]
+    # what the prebuilt kernels leave as separate launches becomes one generated kernel: tanh and the subtraction are
+    # one nest, which is then the only reader of T1, so the chain in front joins it; Y, an argument, is still written
+    s = StructuredSDFG.parse(text)
+    s.schedule("rocm")
+    nodes = [n for n in s.library_nodes() if not n["code"].startswith("ROCMOff")]
+    assert [n["code"] for n in nodes] == ["ROCMMap", "ml::Exp"]
+    assert [(st["op"], st["args"]) for st in nodes[0]["statements"]] == [
+        ("fabs", ["_in0"]), ("sqrt", ["_v0"]), ("tanh", ["_v1"]), ("fp_sub", ["_v2", "_v1"])]
+    assert nodes[0]["bounds"] == ["100"] and len(nodes[0]["reads"]) == 1 and nodes[0]["writes"][0]["value"] == "_v3"
+    assert not {"T0", "T1", "T2"} & set(s.containers)
 
     # per-node transfers keep working on the fused node, scalars are passed by value
     b = StructuredSDFGBuilder("scalar")
