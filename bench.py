@@ -431,6 +431,32 @@ def main():
                 time_kernel(lambda i: fns[0](a_(i), 0, Bs[0].data_ptr(), y_(i), 0), 48, 8), 8 * n + 4 * 4096)
             kernels["map_fma_f32_8192x4096"] = hbm_entry(
                 time_kernel(lambda i: fns[1](a_(i), b_(i), y_(i), Ys[(i + 1) % ROTATE].data_ptr()), 48, 8), 16 * n)
+            # a chain of tensor nodes, y = sigmoid((a + b) * c - bias row) * 0.5: merged into one generated kernel by the
+            # map fusion pass (three full reads, one write), and as the launches of the prebuilt kernels it replaces
+            # (add, multiply, subtract + sigmoid, multiply by the constant: ten passes over the tensor)
+            chain_fns = {}
+            for merged in (True, False):
+                cb = StructuredSDFGBuilder("bench_chain" if merged else "bench_chain_apart")
+                for nm in ("A", "B", "C", "bias", "Y"):
+                    cb.add_container(nm, Pointer(Scalar(PrimitiveType.Float)), True)
+                for nm in ("T0", "T1", "T2", "T3", "T4"):
+                    cb.add_container(nm, Pointer(Scalar(PrimitiveType.Float)), False, transient_bytes=4 * n)
+                cb.add_elementwise_op("add", "A", "B", "T0", [8192, 4096])
+                cb.add_elementwise_op("mul", "T0", "C", "T1", [8192, 4096])
+                cb.add_broadcast("bias", "T2", [1, 4096], [8192, 4096])
+                cb.add_elementwise_op("sub", "T1", "T2", "T3", [8192, 4096])
+                cb.add_elementwise_unary_op("sigmoid", "T3", "T4", [8192, 4096])
+                cb.add_elementwise_op("mul", "T4", "0.5", "Y", [8192, 4096])
+                sd = cb.move()
+                sd.schedule("rocm", options={"offload": "none", "fuse_maps": merged})
+                lib = ctypes.CDLL(sd._compile(str(folder / sd.name)))
+                f = getattr(lib, sd.name)
+                f.argtypes = [ctypes.c_void_p] * 5
+                f.restype = None
+                chain_fns[merged] = f
+            chain = lambda f: (lambda i: f(a_(i), b_(i), Ys[(i + 1) % ROTATE].data_ptr(), Bs[0].data_ptr(), y_(i)))
+            kernels["map_chain_f32_8192x4096"] = hbm_entry(time_kernel(chain(chain_fns[True]), 48, 8), 16 * n + 4 * 4096)
+            kernels["map_chain_f32_8192x4096"]["apart_ms"] = round(time_kernel(chain(chain_fns[False]), 24, 4), 4)
             code, message = rt.take_failure()
             if code:
                 raise RuntimeError(message)

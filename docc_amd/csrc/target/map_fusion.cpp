@@ -63,6 +63,7 @@ public:
         if (auto* e = dynamic_cast<const tensor::ElementWiseNode*>(blk.node.get())) return from_elementwise(blk, *e);
         if (auto* f = dynamic_cast<const ROCMFusedElementWiseNode*>(blk.node.get())) return from_fused(blk, *f);
         if (auto* b = dynamic_cast<const tensor::BroadcastNode*>(blk.node.get())) return from_broadcast(blk, *b);
+        if (auto* c = dynamic_cast<const tensor::CastNode*>(blk.node.get())) return from_cast(blk, *c);
         return std::nullopt;
     }
 
@@ -106,7 +107,7 @@ private:
 
     // a connector's value: a load (array), a kernel argument (scalar container or constant)
     bool operand(MapForm& f, const Block& blk, const std::string& connector, const std::vector<Expression>& shape,
-                 const std::vector<Expression>& own_shape, std::string* value) {
+                 const std::vector<Expression>& own_shape, std::string* value, std::optional<P> loaded_as = std::nullopt) {
         const ConnectorBinding* in = blk.input(connector);
         if (!in) return false;
         if (in->is_constant || !sdfg_.container(in->data).is_pointer) {
@@ -120,7 +121,7 @@ private:
         }
         MapForm::Read r;
         r.data = in->data;
-        r.element = f.element;
+        r.element = loaded_as.value_or(f.element);
         if (!layout(shape, own_shape, &r.strides, &r.extent)) return false;
         r.value = fresh("r");
         *value = r.value;
@@ -213,6 +214,20 @@ private:
         std::string x;
         if (!operand(f, blk, "X", b.output_shape(), b.input_shape(), &x)) return std::nullopt;
         if (!result(f, blk, b.output_shape(), emit(f, "assign", {x}))) return std::nullopt;
+        return f;
+    }
+
+    // between the two floating point types only: the conversion is the assignment's
+    std::optional<MapForm> from_cast(const Block& blk, const tensor::CastNode& c) {
+        if (!floating(c.element()) || !floating(c.target_type()) || c.shape().empty()) return std::nullopt;
+        MapForm f;
+        f.element = c.target_type();
+        f.bounds = bounds_of(c.shape());
+        std::string x;
+        const ConnectorBinding* in = blk.input("X");
+        if (!in || in->is_constant || !sdfg_.container(in->data).is_pointer) return std::nullopt;
+        if (!operand(f, blk, "X", c.shape(), c.shape(), &x, c.element())) return std::nullopt;
+        if (!result(f, blk, c.shape(), emit(f, "assign", {x}))) return std::nullopt;
         return f;
     }
 
@@ -372,7 +387,7 @@ bool RocmMapFusionPass::run_pass(builder::StructuredSDFGBuilder& builder, analys
                 const size_t i = (size_t) writer;
                 if (blocks[i].node->implementation_type() != blocks[j].node->implementation_type()) continue;
                 std::optional<MapForm> producer = convert.form_of(blocks[i]);
-                if (!producer || producer->bounds != consumer->bounds || producer->element != consumer->element) continue;
+                if (!producer || producer->bounds != consumer->bounds) continue;
                 // every load of the link takes the element the producer's iteration stores
                 bool same_elements = true;
                 for (auto& r : consumer->reads)

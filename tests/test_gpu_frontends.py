@@ -780,10 +780,11 @@ def test_casts_through_both_front_ends():
     got = widen(x, k)
     assert got.dtype == np.float64
     np.testing.assert_array_equal(got, np.sqrt(x.astype(np.float64)) + k.astype(np.float64))
-    # the two casts are prebuilt kernels; the square root and the addition behind them are one generated kernel
+    # the cast from integers is a prebuilt kernel; the widening of x, the square root and the addition are one generated kernel
     nodes = [n for n in widen.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"]
-    assert [n["code"] for n in nodes] == ["ml::Cast", "ml::Cast", "ROCMMap"]
-    assert [st["op"] for st in nodes[2]["statements"]] == ["sqrt", "fp_add"]
+    assert [n["code"] for n in nodes] == ["ml::Cast", "ROCMMap"]
+    assert [(st["op"], st["type"]) for st in nodes[1]["statements"]] == [("assign", "Double"), ("sqrt", "Double"), ("fp_add", "Double")]
+    assert sorted(r["element_type"] for r in nodes[1]["reads"]) == ["Double", "Float"]
 
     class Mixed(torch.nn.Module):
         def forward(self, q, k, v):
