@@ -55,8 +55,10 @@ struct AsyncTraits<uint16_t> {   // bf16 bits
     static __device__ __forceinline__ int swz_mn(int k) { return (k & 3) << 2; }
 };
 
-// One operand tile of ROWS x COLS elements (COLS contiguous) in an LDS stage.
-template <typename T, int ROWS, int COLS, int NT, bool K_ALONG_COLS>
+// One operand tile of ROWS x COLS elements (COLS contiguous) in an LDS stage. LAYOUT: where a granule lies in the
+// stage. 0: row after row, the granule index XORed with a function of the row - for fragments of 32 rows (columns) and
+// two k-groups of lanes. 1: for the fragments of the 16x16x32 MFMA (16 rows, four k-groups, gemm_async16.h).
+template <typename T, int ROWS, int COLS, int NT, bool K_ALONG_COLS, int LAYOUT = 0>
 struct AsyncTile {
     typedef AsyncTraits<T> X;
     typedef typename X::vec_t vec_t;
@@ -70,14 +72,28 @@ struct AsyncTile {
     static_assert(NG % NT == 0, "tile does not divide among the threads");
     static_assert(K_ALONG_COLS ? (VPR == 16 || VPR == 8 || VPR == 4) : (VPR >= 16), "row length not covered by the swizzles");
 
+    static_assert(LAYOUT == 0 || (sizeof(T) == 2 && (K_ALONG_COLS ? VPR == 4 : VPR >= 16)), "layout 1: bf16 tiles 32 k deep");
     // granule-index swizzle of a row
     static __device__ __forceinline__ int swz(int row) {
+        if (LAYOUT == 1) {
+            // k along the columns: a fragment read is 16 rows x 4 granules (lane = 16 * granule + row); timed per
+            // pattern, the reads run without bank conflicts with the granule XORed by (row >> 1) & 3.
+            // k-major tile, read by transposing 64-bit reads: the lanes of half a wave read 32 bytes each of rows
+            // k, k+1, k+2, k+3 and k+8 .. k+11 at once - eight shifts of 32 bytes
+            return K_ALONG_COLS ? ((row >> 1) & 3) : 2 * ((row & 3) | (((row >> 3) & 1) << 2));
+        }
         // 16 consecutive rows read the same k-granule at once: spread them over the 16 slots of 256 bytes
         if (K_ALONG_COLS) return VPR == 16 ? (row & 15) : VPR == 8 ? ((row >> 1) & 7) : ((row >> 2) & 3);
         return X::swz_mn(row);
     }
-    // element offset (inside a stage) of the granule that holds columns cv*VEC .. of `row`
-    static __device__ __forceinline__ int granule_offset(int row, int cv) { return (row * VPR + (cv ^ swz(row))) * VEC; }
+    // slot (16-byte unit inside a stage) of the granule that holds columns cv*VEC .. of `row`, and the inverse
+    static __device__ __forceinline__ int slot_of(int row, int cv) { return row * VPR + (cv ^ swz(row)); }
+    static __device__ __forceinline__ void granule_of(int g, int& row, int& cv) {
+        row = g / VPR;
+        cv = (g % VPR) ^ swz(row);
+    }
+    // element offset (inside a stage) of that granule
+    static __device__ __forceinline__ int granule_offset(int row, int cv) { return slot_of(row, cv) * VEC; }
 
     const char* base;      // wave-uniform: origin of the tile of the current K-step
     unsigned off[NV];      // this lane's granules: byte offsets from the origin
@@ -94,7 +110,8 @@ struct AsyncTile {
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             const int g = (i * NW + wave) * 64 + lane;   // the LDS slot this lane fills
-            const int row = g / VPR, cv = (g % VPR) ^ swz(row);
+            int row, cv;
+            granule_of(g, row, cv);
             long r = r0 + row, c = c0 + (long) cv * VEC;
             if (K_ALONG_COLS) r = r < rmax ? r : rmax - 1;
             else c = c + VEC <= cmax ? c : cmax - VEC;
@@ -117,7 +134,8 @@ struct AsyncTile {
     // k = 0 of the step (same row / column, so the address stays inside the operand) and cleared afterwards.
     __device__ __forceinline__ bool past(int i, int wave, int lane, int kleft, unsigned* back) const {
         const int g = (i * NW + wave) * 64 + lane;
-        const int row = g / VPR, cv = (g % VPR) ^ swz(row);
+        int row, cv;
+        granule_of(g, row, cv);
         const bool out = K_ALONG_COLS ? (cv * VEC >= kleft) : (row >= kleft);
         // bytes from the granule's own position back to k = 0 of the step
         *back = K_ALONG_COLS ? (unsigned) (cv * VEC * (int) sizeof(T)) : (unsigned) ((long) row * (kstep_bytes / ROWS));

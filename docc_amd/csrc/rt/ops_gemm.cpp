@@ -15,6 +15,7 @@ struct TileConfig {
     int bm, bn, bk, waves;
     int stages;  // > 0: asynchronous multi-stage kernel (gemm_async.h), aligned operands only
     bool spread = false;  // asynchronous kernels: the variant that deals a stage's copies over the whole K-step (3 stages or more)
+    bool small = false;   // asynchronous bf16 kernels: the variant built on the 16x16x32 MFMA
 };
 
 // LDS bytes of GemmKernel<T, BM, BN, BK, ...> (csrc/kernels/gemm_mfma.h)
@@ -246,14 +247,17 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
     const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
     TileConfig cfg = pick(m, n, batch, aligned, force && force[0] == 'b' ? 1 : force && force[0] == 's' ? -1 : 0);
-    // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES[xSTAGES[p]] selects a built configuration directly (tuning)
+    // DOCC_ROCM_GEMM_CFG=BMxBNxBKxWAVES[xSTAGES[p|q]] selects a built configuration directly (tuning)
     if (const char* c = std::getenv("DOCC_ROCM_GEMM_CFG")) {
         TileConfig t{};
         char tag = 0;
         const int got = std::sscanf(c, "%dx%dx%dx%dx%d%c", &t.bm, &t.bn, &t.bk, &t.waves, &t.stages, &tag);
         t.spread = got == 6 && tag == 'p';
+        t.small = got == 6 && tag == 'q';
         if (got >= 4 && t.bm > 0 && t.bn > 0 && t.bk > 0 && t.waves > 0) cfg = t;
     }
+    // the 16x16x32 kernels (gemm_async16.h) take whole pairs of K-steps, at least a ring of them
+    if (cfg.small && !(k % (2 * cfg.bk) == 0 && k >= (int64_t) cfg.stages * cfg.bk)) cfg.small = false;
     // the asynchronous kernels need aligned operands and address a tile with 32-bit byte offsets
     const int64_t max_edge = cfg.bm > cfg.bn ? (cfg.bm > cfg.bk ? cfg.bm : cfg.bk) : (cfg.bn > cfg.bk ? cfg.bn : cfg.bk);
     const bool offsets_fit = max_edge * (lda > ldb ? lda : ldb) * (int64_t) sizeof(T) < (int64_t(1) << 32);
@@ -262,7 +266,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
     size_t lds;
     if (cfg.stages > 0) {
-        std::snprintf(name, sizeof(name), "docc_%sa_%dx%dx%d%c%d_%c%c", prefix, cfg.bm, cfg.bn, cfg.bk, cfg.spread ? 'p' : 's', cfg.stages,
+        std::snprintf(name, sizeof(name), "docc_%sa_%dx%dx%d%c%d_%c%c", prefix, cfg.bm, cfg.bn, cfg.bk, cfg.small ? 'q' : cfg.spread ? 'p' : 's', cfg.stages,
                       ta ? 't' : 'n', tb ? 't' : 'n');
         lds = (size_t) cfg.stages * ((size_t) cfg.bm * cfg.bk + (size_t) cfg.bk * cfg.bn) * sizeof(T);
     } else {
@@ -333,7 +337,8 @@ static TileConfig pick_dgemm(int64_t m, int64_t n, int64_t batch, bool aligned, 
 }
 
 static TileConfig pick_bgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
-    const TileConfig big{256, 256, 32, 4, 4, true}, small{128, 128, 32, 4, 4};
+    // big: on the 16x16x32 MFMA where K allows it (see gemm_launch), else on the 32x32x16 one with the copies dealt out
+    const TileConfig big{256, 256, 32, 4, 4, true, true}, small{128, 128, 32, 4, 4};
     const TileConfig plain_big{256, 256, 64, 4, 0}, plain_small{128, 128, 64, 4, 0};
     if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 256, 256, batch) >= 256 ? plain_big : plain_small);
     if (force) return force > 0 ? big : small;

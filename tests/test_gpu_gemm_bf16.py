@@ -107,10 +107,11 @@ def test_device_bf16_conversion_matches_oracle(rt):
     assert np.array_equal(host(back), oracle.bf16_to_f32(bits))
 
 
-# every built tile configuration (DOCC_ROCM_GEMM_CFG = BMxBNxBKxWAVES[xSTAGES[p]]; a stage count picks the
-# asynchronous kernel), ragged edges, a K tail, all transposes
+# every built tile configuration (DOCC_ROCM_GEMM_CFG = BMxBNxBKxWAVES[xSTAGES[p|q]]; a stage count picks the
+# asynchronous kernel, q the one on the 16x16x32 MFMA, which here falls back for want of a K that suits it), ragged
+# edges, a K tail, all transposes
 BF16_CFGS = ["128x128x64x4", "256x256x64x4", "128x128x64x4x3", "128x128x64x4x4", "128x128x32x4x4", "128x256x64x4x3",
-             "256x256x64x4x2", "256x256x32x4x4", "256x256x32x4x4p"]
+             "256x256x64x4x2", "256x256x32x4x4", "256x256x32x4x4p", "256x256x32x4x4q"]
 
 
 @pytest.mark.parametrize("cfg", BF16_CFGS)
@@ -128,6 +129,36 @@ def test_bgemm_every_tile_configuration(rt, cfg):
                     out = run_bgemm(rt, Ab, Bb, C0, alpha=2.0, beta=-1.0, ta=ta, tb=tb)
                     ref = oracle.gemm_bf16(Ab, Bb, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb)
                     assert np.array_equal(out, ref), (cfg, m, n, k, ta, tb)
+    finally:
+        os.environ.pop("DOCC_ROCM_GEMM_CFG", None)
+
+
+@pytest.mark.parametrize("ta,tb", [(N, N), (N, T), (T, N), (T, T)])
+def test_bgemm_on_the_16x16x32_mfma(rt, ta, tb):
+    """The kernel the 4096^3 configuration runs on (K a multiple of 64, four K-steps or more): exact on small integers
+    for ragged m and n, the shortest K it takes, an odd number of step pairs, alpha and beta; and N(0,1) operands
+    against the oracle. The same entry point on a K it does not take gives the same bits through the other kernel."""
+    rng = np.random.default_rng(16 + ta + 3 * tb)
+    os.environ["DOCC_ROCM_GEMM_CFG"] = "256x256x32x4x4q"
+    try:
+        for (m, n, k) in [(304, 264, 192), (136, 520, 128), (8, 16, 1024), (512, 256, 320), (257, 511, 448)]:
+            A = rng.integers(-4, 5, (k, m) if ta == T else (m, k)).astype(np.float32)
+            B = rng.integers(-4, 5, (n, k) if tb == T else (k, n)).astype(np.float32)
+            C0 = rng.integers(-4, 5, (m, n)).astype(np.float32)
+            Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+            out = run_bgemm(rt, Ab, Bb, C0, alpha=2.0, beta=-1.0, ta=ta, tb=tb)
+            assert np.array_equal(out, oracle.gemm_bf16(Ab, Bb, C0, alpha=2.0, beta=-1.0, trans_a=ta, trans_b=tb)), (m, n, k)
+            out = run_bgemm(rt, Ab, Bb, ta=ta, tb=tb)              # beta == 0 over a C full of NaN
+            assert np.array_equal(out, oracle.gemm_bf16(Ab, Bb, trans_a=ta, trans_b=tb)), (m, n, k)
+        m, n, k = 384, 320, 1024
+        A = (rng.standard_normal((k, m) if ta == T else (m, k)) / np.sqrt(k)).astype(np.float32)
+        B = (rng.standard_normal((n, k) if tb == T else (k, n)) / np.sqrt(k)).astype(np.float32)
+        Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+        C = run_bgemm(rt, Ab, Bb, ta=ta, tb=tb)
+        assert rel_err_max(C, oracle.gemm_bf16(Ab, Bb, trans_a=ta, trans_b=tb)) <= 1e-5
+        # the two MFMA forms add the same products in the same order of k-groups: the other kernel gives the same bits
+        os.environ["DOCC_ROCM_GEMM_CFG"] = "256x256x32x4x4p"
+        assert np.array_equal(C, run_bgemm(rt, Ab, Bb, ta=ta, tb=tb))
     finally:
         os.environ.pop("DOCC_ROCM_GEMM_CFG", None)
 

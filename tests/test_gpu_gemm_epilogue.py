@@ -103,10 +103,11 @@ def test_epilogue_on_the_benchmark_shapes_and_padded_c(rt):
         rt.gemm_epilogue("d", m, 64, 0, 1.0, a2.data_ptr(), k, b2.data_ptr(), 64, 0.0, c2.data_ptr(), ldc, bias2.data_ptr(), "relu")
 
 
-def test_bf16_epilogue_on_the_large_tile(rt):
-    """A product large enough for the 256x256 tile (the kernel that deals its copies over the K-step), with a
-    K tail: bias and ReLU in the store give the bits of the separate nodes."""
-    m, n, k = 4096, 3072, 264
+@pytest.mark.parametrize("k", [264, 320])
+def test_bf16_epilogue_on_the_large_tile(rt, k):
+    """A product large enough for the 256x256 tile, with a K tail (the 32x32x16 kernel that deals its copies over the
+    K-step) and with K a multiple of 64 (the 16x16x32 kernel): bias and ReLU in the store give the bits of the separate nodes."""
+    m, n = 4096, 3072
     g = torch.Generator(device="cuda").manual_seed(5)
     a = (torch.randn(m, k, device="cuda", generator=g) / 8).bfloat16()
     b = (torch.randn(k, n, device="cuda", generator=g) / 8).bfloat16()
