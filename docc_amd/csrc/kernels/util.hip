@@ -60,6 +60,7 @@ extern "C" __global__ __launch_bounds__(64) void docc_clock_probe(float* __restr
 // kernel can reach with that data. One wave per SIMD per work-group; launch 2 per CU for two.
 typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
 typedef double probe_f64x4 __attribute__((ext_vector_type(4)));
+typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
 
 // Every index below is a compile-time constant once the loops are unrolled, so the operand sets live in
@@ -138,5 +139,32 @@ extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_bf16(const flo
     float r = 0;
 #pragma unroll
     for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][15];
+    sink[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+// the same on the other form of the bf16 instruction: a quarter of the output tile, twice the k
+extern "C" __global__ __launch_bounds__(256) void docc_mfma_probe_bf16_16x16x32(const float* __restrict__ operands, float* __restrict__ sink, int iters) {
+    probe_f32x4 acc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) acc[i] = {0, 0, 0, 0};
+    // each lane's eight operand sets: 64 consecutive table entries (a), the 64 of the lane 28 further on (b)
+    const float4* row_a = reinterpret_cast<const float4*>(operands + ((threadIdx.x * 64) & 4095));
+    const float4* row_b = reinterpret_cast<const float4*>(operands + ((threadIdx.x * 64 + 1792) & 4095));
+    probe_bf16x8 a[8], b[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const float4 a0 = row_a[2 * i], a1 = row_a[2 * i + 1], b0 = row_b[2 * i], b1 = row_b[2 * i + 1];
+        a[i] = probe_bf16x8{(__bf16) a0.x, (__bf16) a0.y, (__bf16) a0.z, (__bf16) a0.w, (__bf16) a1.x, (__bf16) a1.y, (__bf16) a1.z, (__bf16) a1.w};
+        b[i] = probe_bf16x8{(__bf16) b0.x, (__bf16) b0.y, (__bf16) b0.z, (__bf16) b0.w, (__bf16) b1.x, (__bf16) b1.y, (__bf16) b1.z, (__bf16) b1.w};
+    }
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[i]) : "v"(a[(s + i) & 7]), "v"(b[s]));
+    }
+    float r = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) r += acc[i][0] + acc[i][3];
     sink[blockIdx.x * 256 + threadIdx.x] = r;
 }

@@ -177,7 +177,8 @@ int docc_rocm_copy_bytes(docc_rocm_stream_t stream, int64_t bytes, const void* s
 
 int docc_rocm_mfma_probe(docc_rocm_stream_t stream, int precision, int waves_per_simd, int iters, const float* operands,
                          float* sink, double* flop) {
-    if (precision != 64 && precision != 32 && precision != 16) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "mfma_probe: precision must be 64, 32 or 16");
+    if (precision != 64 && precision != 32 && precision != 16 && precision != 116)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "mfma_probe: precision must be 64, 32, 16 or 116");
     if (waves_per_simd < 1 || waves_per_simd > 2 || iters < 1) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "mfma_probe: waves_per_simd in 1..2, iters >= 1");
     if (!operands || !sink) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "mfma_probe: null pointer");
     int rc = ensure_device();
@@ -185,10 +186,10 @@ int docc_rocm_mfma_probe(docc_rocm_stream_t stream, int precision, int waves_per
     int cus = compute_units();
     if (cus <= 0) cus = 256;
     const uint32_t groups = (uint32_t) (cus * waves_per_simd);
-    // flop per MFMA: 16x16x4 fp64 = 2048, 32x32x2 fp32 = 4096, 32x32x16 bf16 = 32768; 32 MFMAs per round, 4 waves per group
-    const double per_mfma = precision == 64 ? 2048.0 : precision == 32 ? 4096.0 : 32768.0;
+    // flop per MFMA: 16x16x4 fp64 = 2048, 32x32x2 fp32 = 4096, 32x32x16 bf16 = 32768, 16x16x32 bf16 = 16384; 32 MFMAs per round, 4 waves per group
+    const double per_mfma = precision == 64 ? 2048.0 : precision == 32 ? 4096.0 : precision == 16 ? 32768.0 : 16384.0;
     if (flop) *flop = per_mfma * 32.0 * iters * 4.0 * groups;
-    return launch(precision == 64 ? "docc_mfma_probe_f64" : precision == 32 ? "docc_mfma_probe_f32" : "docc_mfma_probe_bf16", groups, 1, 1,
+    return launch(precision == 64 ? "docc_mfma_probe_f64" : precision == 32 ? "docc_mfma_probe_f32" : precision == 16 ? "docc_mfma_probe_bf16" : "docc_mfma_probe_bf16_16x16x32", groups, 1, 1,
                   256, 0, (hipStream_t) stream, operands, sink, iters);
 }
 

@@ -350,7 +350,7 @@ int docc_rocm_dot(docc_rocm_stream_t stream, int precision, int64_t n, const voi
 int docc_rocm_clock_probe(docc_rocm_stream_t stream, int microseconds, float* mhz);
 
 /* Measurement aid, no counterpart in the reference: `iters` rounds of 32 back-to-back
- * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16) on
+ * MFMAs per wave (precision 64: 16x16x4 fp64, 32: 32x32x2 fp32, 16: 32x32x16 bf16, 116: 16x16x32 bf16) on
  * every SIMD, `waves_per_simd` (1 or 2) waves each, operands taken from `operands`
  * (4096 floats on the device). `sink` receives 256 floats per work-group (CUs *
  * waves_per_simd groups); *flop (host, optional) the floating-point operations of

@@ -232,7 +232,7 @@ def test_large_uploads_from_pageable_memory_are_staged_through_pinned_chunks(rt)
     rt.call("docc_rocm_stream_destroy", s)
 
 
-@pytest.mark.parametrize("precision", [64, 32, 16])
+@pytest.mark.parametrize("precision", [64, 32, 16, 116])
 def test_mfma_probe_times_its_loop_and_nothing_else(rt, precision):
     """The ceiling probe's launch time must be its MFMA loop: twice the rounds take twice as long (operand
     set-up that costs as much as thousands of rounds once passed for matrix time), and the flop count it
@@ -260,7 +260,7 @@ def test_mfma_probe_times_its_loop_and_nothing_else(rt, precision):
         rt.mfma_probe(precision, 1, 2000, ops.data_ptr(), sink.data_ptr())
     t1, f1 = timed(2000)
     t2, f2 = timed(4000)
-    per_mfma = {64: 2048, 32: 4096, 16: 32768}[precision]
+    per_mfma = {64: 2048, 32: 4096, 16: 32768, 116: 16384}[precision]
     groups = f1 / (per_mfma * 32.0 * 2000 * 4)
     assert groups == int(groups) and groups >= 1 and f2 == 2 * f1
     assert 1.75 < t2 / t1 < 2.25, (t1, t2)
