@@ -44,6 +44,8 @@ KERNEL_FAMILIES = {
     "gemm_bf16_epilogue": "gemm_bf16_epilogue.hip",
     "gemm_bf16_async_epilogue": "gemm_bf16_async_epilogue.hip",
     "gemm_bf16_async_big_epilogue": "gemm_bf16_async_big_epilogue.hip",
+    "gemm_f32_big": "gemm_f32_big.hip",
+    "gemm_f32_big_epilogue": "gemm_f32_big_epilogue.hip",
     "conv2d": "conv2d.hip",
     "attention": "attention.hip",
     "elementwise": "elementwise.hip",

@@ -309,13 +309,13 @@ extern "C" {
 static int64_t tiles_of(int64_t m, int64_t n, int bm, int bn, int64_t batch = 1) { return ((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch; }
 
 static TileConfig pick_sgemm(int64_t m, int64_t n, int64_t batch, bool aligned, int force) {
-    const TileConfig wide{128, 256, 32, 4, 2}, big{128, 128, 32, 4, 3}, small{64, 64, 16, 4, 4};
+    const TileConfig huge{256, 256, 32, 4, 2}, wide{128, 256, 32, 4, 2}, big{128, 128, 32, 4, 3}, small{64, 64, 16, 4, 4};
     const TileConfig plain_big{128, 128, 16, 4, 0}, plain_small{64, 64, 16, 4, 0};
     if (!aligned) return force > 0 ? plain_big : force < 0 ? plain_small : (tiles_of(m, n, 128, 128, batch) >= 256 ? plain_big : plain_small);
-    if (force) return force > 0 ? wide : small;
+    if (force) return force > 0 ? huge : small;
     // Score = share of a tile's area that is real output x share of the CUs that get a work-group x what the
-    // tile sustains relative to the widest (141 / 138 / about 105 TFLOP/s on large problems): a 64-row product
-    // wastes half of a 128-row tile, a 1000^2 one leaves most CUs idle with the large tiles.
+    // tile sustains relative to the 128x256 one (146 / 141 / 138 / about 105 TFLOP/s on large problems): a 64-row
+    // product wastes half of a 128-row tile, a 1000^2 one leaves most CUs idle with the large tiles.
     int cus = compute_units();
     if (cus <= 0) cus = 256;
     auto score = [&](const TileConfig& c, double rel) {
@@ -323,7 +323,11 @@ static TileConfig pick_sgemm(int64_t m, int64_t n, int64_t batch, bool aligned, 
         const double fill = (double) tiles_of(m, n, c.bm, c.bn, batch) / cus;
         return rel * ((double) m * (double) n / padded) * (fill < 1.0 ? fill : 1.0);
     };
-    const double sw = score(wide, 1.0), sb = score(big, 0.97), ss = score(small, 0.75);
+    const double sh = score(huge, 1.03), sw = score(wide, 1.0), sb = score(big, 0.97), ss = score(small, 0.75);
+    // one work-group of the two largest tiles owns a CU, so their work-groups run in rounds: the 256x256 tile only
+    // where its rounds take no longer than those of the 128x256 one
+    auto rounds = [&](const TileConfig& c) { return (double) ((tiles_of(m, n, c.bm, c.bn, batch) + cus - 1) / cus) * c.bm * c.bn; };
+    if (sh >= sw && sh >= sb && sh >= ss && rounds(huge) / 1.03 <= rounds(wide)) return huge;
     return sw >= sb && sw >= ss ? wide : sb >= ss ? big : small;
 }
 

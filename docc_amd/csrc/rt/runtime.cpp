@@ -39,6 +39,8 @@ const char* const kKernelImages[] = {
     "docc_rocm_gemm_bf16_epilogue.hsaco",
     "docc_rocm_gemm_bf16_async_epilogue.hsaco",
     "docc_rocm_gemm_bf16_async_big_epilogue.hsaco",
+    "docc_rocm_gemm_f32_big.hsaco",
+    "docc_rocm_gemm_f32_big_epilogue.hsaco",
     "docc_rocm_conv2d.hsaco",
     "docc_rocm_attention.hsaco",
     "docc_rocm_elementwise.hsaco",

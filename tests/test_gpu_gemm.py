@@ -176,7 +176,7 @@ def test_sgemm_config_4096(rt):
 # a K tail and all four transpose combinations
 F64_CFGS = ["64x64x16x4", "128x128x16x4", "64x64x16x4x2", "64x64x16x4x4", "64x64x16x4x6", "128x128x16x4x3",
             "64x32x16x4x4", "64x32x32x4x3", "64x64x32x4x3", "64x32x16x4x4p"]
-F32_CFGS = ["64x64x16x4", "128x128x16x4", "128x128x16x4x3", "128x128x32x4x3", "128x256x16x4x3", "64x64x16x4x4",
+F32_CFGS = ["64x64x16x4", "128x128x16x4", "128x128x16x4x3", "128x128x32x4x3", "128x256x16x4x3", "64x64x16x4x4", "256x256x32x4x2",
             "64x64x32x4x3", "128x256x32x4x2", "128x256x32x4x3", "128x256x16x4x4", "128x256x32x4x3p"]
 
 
