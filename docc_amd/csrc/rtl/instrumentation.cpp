@@ -68,10 +68,19 @@ struct Region {
     long long first_start = 0, last_start = 0;
     Stats runtime;
     std::map<std::string, Stats> static_counters;
-    // ROCm event set
+    // ROCm event set: the events of the execution that is open
     docc_rocm_event_t begin = nullptr, end = nullptr;
     bool events_recorded = false;
     bool open = false;
+};
+
+// An execution whose events are recorded but not read yet: the device time of a region is taken from its two events
+// when the trace is written (or when many are waiting), so that a region costs the host two event records and no
+// wait - the stream keeps running under instrumented code as it does without.
+struct Pending {
+    size_t region;
+    size_t index;     // into Region::durations (individual mode)
+    docc_rocm_event_t begin, end;
 };
 
 std::string json_string(const std::string& s) {
@@ -109,6 +118,8 @@ std::string base_name(const std::string& path) {
     return p == std::string::npos ? path : path.substr(p + 1);
 }
 
+void state_flush();
+
 class State {
 public:
     State() {
@@ -131,6 +142,10 @@ public:
     }
 
     ~State() { write(); }
+
+    // events are read while the HIP runtime is still there: at exit before its own tear-down (registered after its
+    // start-up, so run before), not from this object's destructor
+    static void at_exit() { state_flush(); }
 
     size_t init(const __daisy_metadata_t* m, __daisy_event_set set) {
         std::lock_guard<std::mutex> lock(mutex_);
@@ -181,9 +196,15 @@ public:
         if (r.event_set == __DAISY_EVENT_SET_ROCM) {
             if (range_push_) range_push_(r.md.region_uuid.c_str());
             if (gpu_) {
-                // what is already queued on the stream is not part of the region
-                if (!r.begin && (docc_rocm_event_create(&r.begin) != 0 || docc_rocm_event_create(&r.end) != 0)) r.begin = r.end = nullptr;
-                if (r.begin && docc_rocm_stream_sync(nullptr) == 0 && docc_rocm_event_record(r.begin, nullptr) == 0) r.events_recorded = true;
+                // the begin event completes when what is already queued on the stream has: that work is not part of
+                // the region, and the host does not wait for it
+                if (!exit_hook_) {
+                    exit_hook_ = true;
+                    std::atexit(&State::at_exit);
+                }
+                r.begin = take_event();
+                r.end = take_event();
+                if (r.begin && r.end && docc_rocm_event_record(r.begin, nullptr) == 0) r.events_recorded = true;
             }
         }
         const long long now = wall_ns();
@@ -201,21 +222,27 @@ public:
         Region& r = region(id, "exiting");
         if (r.event_set == __DAISY_EVENT_SET_NONE || !r.open) return;
         r.open = false;
-        long long duration = -1;
+        bool deferred = false;
         if (r.event_set == __DAISY_EVENT_SET_ROCM) {
-            if (r.events_recorded) {
-                float ms = 0.f;
-                if (docc_rocm_event_record(r.end, nullptr) == 0 && docc_rocm_event_elapsed_ms(r.begin, r.end, &ms) == 0)
-                    duration = (long long) ((double) ms * 1e6);
+            if (r.events_recorded && docc_rocm_event_record(r.end, nullptr) == 0) {
+                if (!aggregate_) r.durations.push_back(-1);
+                pending_.push_back(Pending{id, aggregate_ ? 0 : r.durations.size() - 1, r.begin, r.end});
+                deferred = true;
+            } else {
+                give_event(r.begin);
+                give_event(r.end);
             }
+            r.begin = r.end = nullptr;
             if (range_pop_) range_pop_();
         }
-        const long long start = aggregate_ ? r.last_start : r.starts.back();
-        if (duration < 0) duration = wall_ns() - start;
-        if (aggregate_)
-            r.runtime.add((double) duration);
-        else
-            r.durations.push_back(duration);
+        if (!deferred) {
+            const long long duration = wall_ns() - (aggregate_ ? r.last_start : r.starts.back());
+            if (aggregate_)
+                r.runtime.add((double) duration);
+            else
+                r.durations.push_back(duration);
+        }
+        if (pending_.size() >= kMaxPending) resolve();
     }
 
     void metric(size_t id, const char* name, double value) {
@@ -232,6 +259,7 @@ public:
 
     int write() {
         std::lock_guard<std::mutex> lock(mutex_);
+        resolve();
         if (regions_.empty() && written_) return 0;
         FILE* f = std::fopen(output_file_.c_str(), "w");
         if (!f) {
@@ -262,6 +290,38 @@ public:
     }
 
 private:
+    static constexpr size_t kMaxPending = 4096;
+
+    docc_rocm_event_t take_event() {
+        if (!free_events_.empty()) {
+            docc_rocm_event_t e = free_events_.back();
+            free_events_.pop_back();
+            return e;
+        }
+        docc_rocm_event_t e = nullptr;
+        return docc_rocm_event_create(&e) == 0 ? e : nullptr;
+    }
+    void give_event(docc_rocm_event_t e) {
+        if (e) free_events_.push_back(e);
+    }
+
+    // reads the events of the executions that are waiting (the caller holds the lock); an execution whose events cannot
+    // be read is reported with a duration of 0
+    void resolve() {
+        for (auto& p : pending_) {
+            float ms = 0.f;
+            const long long duration = docc_rocm_event_elapsed_ms(p.begin, p.end, &ms) == 0 ? (long long) ((double) ms * 1e6) : 0;
+            Region& r = regions_.at(p.region);
+            if (aggregate_)
+                r.runtime.add((double) duration);
+            else
+                r.durations[p.index] = duration;
+            give_event(p.begin);
+            give_event(p.end);
+        }
+        pending_.clear();
+    }
+
     Region& region(size_t id, const char* what) {
         auto it = regions_.find(id);
         if (it == regions_.end()) {
@@ -326,7 +386,9 @@ private:
     size_t next_id_ = 1;
     std::map<size_t, Region> regions_;
     std::map<std::string, size_t> by_uuid_;
-    bool aggregate_ = false, gpu_ = false, written_ = false;
+    std::vector<Pending> pending_;
+    std::vector<docc_rocm_event_t> free_events_;
+    bool aggregate_ = false, gpu_ = false, written_ = false, exit_hook_ = false;
     std::string output_file_;
     int (*range_push_)(const char*) = nullptr;
     int (*range_pop_)() = nullptr;
@@ -336,6 +398,8 @@ State& state() {
     static State s;
     return s;
 }
+
+void state_flush() { (void) state().write(); }
 
 } // namespace
 

@@ -17,8 +17,10 @@
  * event set:
  *   CPU, CUDA  wall-clock time of the region (no PAPI counters here)
  *   ROCM       the region is bracketed on the device's null stream: enter and exit record a
- *              HIP event each, exit waits for its event, the duration is the time between the
- *              two events; without a GPU it degrades to wall-clock time. While a region is
+ *              HIP event each and return; the duration is the time between the two events,
+ *              read when the trace is written (no host wait inside instrumented code: the
+ *              stream runs on as it does without instrumentation); without a GPU it degrades
+ *              to wall-clock time. While a region is
  *              open a roctx range named after its region_uuid is pushed (when
  *              librocprofiler-sdk-roctx.so or libroctx64.so can be loaded), so that rocprofv3 --marker-trace shows the regions.
  *   NONE       metrics only
