@@ -48,7 +48,7 @@ PEAK_TFLOPS = {"f64": 78.6, "f32": 157.3, "bf16": 2516.6}
 # HBM bytes per softmax launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by what the
 # same counters read for the 128 MiB copy kernel. A stored figure (this run does not read counters):
 # the JSON line names the file it comes from.
-SOFTMAX_TRAFFIC_BYTES = 268450098
+SOFTMAX_TRAFFIC_BYTES = 268436685
 SOFTMAX_TRAFFIC_SOURCE = "profiles/softmax_f32_8192x4096_pmc.txt (stored figure from a rocprofv3 --pmc run, not measured by this run)"
 
 
