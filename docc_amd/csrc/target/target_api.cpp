@@ -173,6 +173,10 @@ char* docc_rocm_target_schedule(const char* sdfg_json, const char* category, con
             if (const json::Value* v = o.find("match_softmax")) options.match_softmax = v->as_bool();
             if (const json::Value* v = o.find("fuse_maps")) options.fuse_maps = v->as_bool();
         }
+        // merged chains are kernels this machine has to compile: without a device compiler the nodes keep their
+        // prebuilt kernels (a program that holds map nests of its own still needs one, and says so when compiled)
+        if (options.fuse_maps && device_compiler().find('/') != std::string::npos && !std::filesystem::exists(device_compiler()))
+            options.fuse_maps = false;
         builder::StructuredSDFGBuilder builder(*sdfg);
         analysis::AnalysisManager analysis_manager(*sdfg);
         rocm::rocm_scheduling_passes(builder, analysis_manager, category ? category : "server", options);

@@ -732,6 +732,35 @@ def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
     assert nodes[0]["bounds"] == ["100"] and len(nodes[0]["reads"]) == 1 and nodes[0]["writes"][0]["value"] == "_v3"
     assert not {"T0", "T1", "T2"} & set(s.containers)
 
+    # without a device compiler on the machine the chain keeps its prebuilt kernels
+    import os
+    s = StructuredSDFG.parse(text)
+    saved = os.environ.get("DOCC_HIPCC")
+    os.environ["DOCC_HIPCC"] = "/nonexistent/bin/hipcc"
+    try:
+        s.schedule("rocm")
+    finally:
+        if saved is None:
+            del os.environ["DOCC_HIPCC"]
+        else:
+            os.environ["DOCC_HIPCC"] = saved
+    assert "ROCMMap" not in [n["code"] for n in s.library_nodes()]
+
+    # a GEMM in front of a merged chain: its result stays on the device although the two nodes spell its size differently
+    b = StructuredSDFGBuilder("gemm_chain")
+    for n in ("X", "W", "C", "D", "Y"):
+        b.add_container(n, F32, True)
+    for n in ("T0", "T1", "T2"):
+        b.add_container(n, F32, False, transient_bytes=32 * 16 * 4)
+    b.add_gemm("X", "W", "T0", "1.0", "0.0", 32, 16, 8)
+    b.add_elementwise_op("mul", "T0", "C", "T1", [32, 16])
+    b.add_elementwise_op("sub", "T1", "D", "T2", [32, 16])
+    b.add_elementwise_op("mul", "T2", "0.5", "Y", [32, 16])
+    s = b.move()
+    s.schedule("rocm")
+    r = s.loop_report()
+    assert r["GEMM"] == 1 and r["ROCMMap"] == 1 and r["H2D"] == 4 and r["D2H"] == 1
+
     # per-node transfers keep working on the fused node, scalars are passed by value
     b = StructuredSDFGBuilder("scalar")
     b.add_container("x", F32, True)
