@@ -59,12 +59,14 @@ public:
     // nullopt: the block is not of elementwise kind (or uses an operation the statements cannot spell)
     std::optional<MapForm> form_of(const Block& blk) {
         if (!is_rocm_type(blk.node->implementation_type()) || blk.outputs.size() != 1) return std::nullopt;
-        if (auto* m = dynamic_cast<const ROCMMapNode*>(blk.node.get())) return from_map(blk, *m);
-        if (auto* e = dynamic_cast<const tensor::ElementWiseNode*>(blk.node.get())) return from_elementwise(blk, *e);
-        if (auto* f = dynamic_cast<const ROCMFusedElementWiseNode*>(blk.node.get())) return from_fused(blk, *f);
-        if (auto* b = dynamic_cast<const tensor::BroadcastNode*>(blk.node.get())) return from_broadcast(blk, *b);
-        if (auto* c = dynamic_cast<const tensor::CastNode*>(blk.node.get())) return from_cast(blk, *c);
-        return std::nullopt;
+        std::optional<MapForm> f;
+        if (auto* m = dynamic_cast<const ROCMMapNode*>(blk.node.get())) f = from_map(blk, *m);
+        else if (auto* e = dynamic_cast<const tensor::ElementWiseNode*>(blk.node.get())) f = from_elementwise(blk, *e);
+        else if (auto* fe = dynamic_cast<const ROCMFusedElementWiseNode*>(blk.node.get())) f = from_fused(blk, *fe);
+        else if (auto* b = dynamic_cast<const tensor::BroadcastNode*>(blk.node.get())) f = from_broadcast(blk, *b);
+        else if (auto* c = dynamic_cast<const tensor::CastNode*>(blk.node.get())) f = from_cast(blk, *c);
+        if (f && f->bounds.size() > 6) return std::nullopt;   // a ROCMMap node holds at most six loops
+        return f;
     }
 
     std::string fresh(const char* kind) { return std::string(kind) + std::to_string(counter_++); }

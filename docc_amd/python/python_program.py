@@ -490,6 +490,14 @@ class _Lowering(ast.NodeVisitor):
             return self.transpose(node, base, None, dest)
         if isinstance(node, ast.BinOp):
             return self.binop(node, dest)
+        if isinstance(node, ast.UnaryOp) and isinstance(node.op, (ast.USub, ast.UAdd)):
+            # -x of an array: the product with -1.0, which flips the sign of every value, zeros and NaNs included
+            v = self.array_of(node, self.ev(node.operand))
+            if not isinstance(v, _Array):
+                self.fail(node, "a sign in front of something that is not an array or a literal")
+            if isinstance(node.op, ast.UAdd):
+                return v
+            return self.elementwise(node, "mul", v, _ScalarValue("-1.0"), dest)
         if isinstance(node, ast.Call):
             return self.call(node, dest)
         self.fail(node, f"expression {ast.dump(node)[:60]}")

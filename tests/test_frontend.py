@@ -148,6 +148,10 @@ def test_elementwise_expressions_lower_to_tensor_nodes():
     def in_place(x, y):
         y[:] = np.exp(x) + y
 
+    @native
+    def negated(x, y):
+        return np.exp(-np.abs(x)) + -2.5
+
     x, w, b = np.zeros((8, 5), np.float32), np.zeros((5, 3), np.float32), np.zeros(3, np.float32)
     sdfg = dense.to_sdfg(x, w, b)
     codes = [n["code"] for n in sdfg.library_nodes()]
@@ -171,6 +175,12 @@ def test_elementwise_expressions_lower_to_tensor_nodes():
     assert all(n["element_type"] == "Double" for n in sdfg.library_nodes())
 
     assert [n["code"] for n in clip.to_sdfg(z, z).library_nodes()] == ["ml::ReLU", "ml::Abs", "ml::Minimum"]
+    # a sign in front of an array is the product with -1.0; in front of a literal it is the literal's
+    sdfg = negated.to_sdfg(z, z)
+    assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Abs", "ml::Mul", "ml::Exp", "ml::Add"]
+    blocks = [c["dataflow"] for c in sdfg._data["root"]["children"]]
+    assert {i["connector"]: i.get("constant") for i in blocks[1]["inputs"]}["B"] == "-1.0"
+    assert {i["connector"]: i.get("constant") for i in blocks[3]["inputs"]}["B"] == "-2.5"
     sdfg = in_place.to_sdfg(z, z)
     assert sdfg.arguments == ["x", "y", "_s0", "_s1"]
     assert sdfg._data["root"]["children"][1]["dataflow"]["outputs"][0]["data"] == "y"

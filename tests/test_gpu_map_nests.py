@@ -280,3 +280,46 @@ def test_chain_of_tensor_nodes_runs_as_one_generated_kernel(tmp_path, rt, elem, 
     d = lambda x: x.astype(np.float64)
     hand = 1.0 / (1.0 + np.exp(-((d(A) + d(B)) * d(C) - d(bias)[None, :]))) * 0.5 + np.maximum(d(A), d(col)[:, None])
     assert rel_err_max(results[True], hand) <= (2e-6 if elem == np.float32 else 1e-12)
+
+
+CHAIN_SOURCES = [
+    ("np.tanh(x * y + b) / (np.abs(z) + 1.5)", 1),
+    ("np.maximum(x, c) - np.minimum(y, z) * np.exp(-np.abs(x))", 1),
+    ("(x + b) * (y + c) + np.sqrt(np.abs(z)) * 0.25", 2),
+    ("1.0 / (1.0 + np.exp(-(x * 0.5 + y * z)))", 1),
+    ("np.sqrt(x * x + y * y + z * z) - b", 1),
+    ("((x - y) ** 2 + c) * np.tanh(z)", 1),
+]
+
+
+@pytest.mark.parametrize("case", range(len(CHAIN_SOURCES)))
+@pytest.mark.parametrize("dt", [np.float32, np.float64], ids=["f32", "f64"])
+def test_numpy_expressions_merge_into_generated_kernels(tmp_path, case, dt):
+    """numpy expressions with several two-operand operations, a bias row `b` and a column `c`, through @native: merged into
+    generated kernels (at most as many as the comment says), with the bits of the unmerged program and numpy's values."""
+    import importlib.util
+    import sys
+    from docc_amd.python import native    # noqa: F401  (the generated module imports it)
+    expr, max_kernels = CHAIN_SOURCES[case]
+    src = ("import numpy as np\nfrom docc_amd.python import native\n\n"
+           f"@native(target='rocm')\ndef merged(x, y, z, b, c):\n    return {expr}\n\n"
+           f"@native(target='rocm', fuse_maps=False)\ndef apart(x, y, z, b, c):\n    return {expr}\n")
+    path = tmp_path / f"chain_case_{case}_{np.dtype(dt).name}.py"
+    path.write_text(src)
+    spec = importlib.util.spec_from_file_location(path.stem, path)
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[path.stem] = mod
+    spec.loader.exec_module(mod)
+    rng = np.random.default_rng(40 + case)
+    r, cols = 96, 200
+    x, y, z = (rng.standard_normal((r, cols)).astype(dt) for _ in range(3))
+    b, c = rng.standard_normal((1, cols)).astype(dt), rng.standard_normal((r, 1)).astype(dt)
+    got, ref = mod.merged(x, y, z, b, c), mod.apart(x, y, z, b, c)
+    assert got.dtype == dt and got.shape == (r, cols)
+    assert np.array_equal(got, ref)
+    want = eval(expr, {"np": np, "x": x.astype(np.float64), "y": y.astype(np.float64), "z": z.astype(np.float64),
+                       "b": b.astype(np.float64), "c": c.astype(np.float64)})
+    assert rel_err_max(got, want) <= (2e-5 if dt == np.float32 else 1e-12)
+    kinds = [n["code"] for n in mod.merged.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert kinds.count("ROCMMap") >= 1 and len(kinds) <= max_kernels, kinds
+    assert "ROCMMap" not in [n["code"] for n in mod.apart.last_sdfg.library_nodes()]
