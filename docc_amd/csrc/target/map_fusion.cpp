@@ -44,12 +44,15 @@ struct MapForm {
     std::vector<Expression> bounds;
     std::vector<Read> reads;
     std::vector<Scalar> scalars;
+    struct Result {
+        std::string value, data;
+        std::vector<Expression> strides;
+        Expression extent;
+        P element;
+    };
     std::vector<Statement> statements;
-    // the one result
-    std::string result_value, result_data;
-    std::vector<Expression> result_strides;
-    Expression result_extent;
-    P element = P::Float;
+    std::vector<Result> results;   // the tensor nodes have one; a nest that was imported, or merged, may store several
+    P element = P::Float;          // of the statements a tensor node becomes
 };
 
 class Converter {
@@ -58,7 +61,7 @@ public:
 
     // nullopt: the block is not of elementwise kind (or uses an operation the statements cannot spell)
     std::optional<MapForm> form_of(const Block& blk) {
-        if (!is_rocm_type(blk.node->implementation_type()) || blk.outputs.size() != 1) return std::nullopt;
+        if (!is_rocm_type(blk.node->implementation_type()) || blk.outputs.empty()) return std::nullopt;
         std::optional<MapForm> f;
         if (auto* m = dynamic_cast<const ROCMMapNode*>(blk.node.get())) f = from_map(blk, *m);
         else if (auto* e = dynamic_cast<const tensor::ElementWiseNode*>(blk.node.get())) f = from_elementwise(blk, *e);
@@ -132,9 +135,13 @@ private:
     }
 
     bool result(MapForm& f, const Block& blk, const std::vector<Expression>& shape, const std::string& value) {
-        f.result_data = blk.outputs[0].data;
-        f.result_value = value;
-        return layout(shape, shape, &f.result_strides, &f.result_extent);
+        MapForm::Result r;
+        r.data = blk.outputs[0].data;
+        r.value = value;
+        r.element = f.element;
+        if (!layout(shape, shape, &r.strides, &r.extent)) return false;
+        f.results.push_back(std::move(r));
+        return true;
     }
 
     std::string emit(MapForm& f, const std::string& op, std::vector<std::string> args) {
@@ -234,7 +241,6 @@ private:
     }
 
     std::optional<MapForm> from_map(const Block& blk, const ROCMMapNode& m) {
-        if (m.writes().size() != 1) return std::nullopt;
         MapForm f;
         f.bounds = m.bounds();
         f.element = m.writes()[0].element;
@@ -258,12 +264,11 @@ private:
             names[st.out] = out.out;
             f.statements.push_back(std::move(out));
         }
-        const auto& w = m.writes()[0];
-        f.result_data = blk.outputs[0].data;
-        f.result_value = renamed(w.value);
-        if (f.result_value[0] == '#') return std::nullopt;
-        f.result_strides = w.strides;
-        f.result_extent = w.extent;
+        for (auto& w : m.writes()) {
+            const ConnectorBinding* out = blk.output(w.connector);
+            if (!out) return std::nullopt;
+            f.results.push_back({renamed(w.value), out->data, w.strides, w.extent, w.element});
+        }
         return f;
     }
 
@@ -333,7 +338,14 @@ void install(const StructuredSDFG& sdfg, Block& blk, const MapForm& f) {
         names[st.out] = out.out;
         statements.push_back(std::move(out));
     }
-    writes.push_back({"_out0", f.result_strides, f.result_extent, f.element, renamed(f.result_value)});
+    std::vector<ConnectorBinding> outputs;
+    for (auto& r : f.results) {
+        ConnectorBinding b;
+        b.connector = "_out" + std::to_string(writes.size());
+        b.data = r.data;
+        writes.push_back({b.connector, r.strides, r.extent, r.element, renamed(r.value)});
+        outputs.push_back(b);
+    }
     std::vector<std::string> indvars, symbols;
     for (size_t l = 0; l < f.bounds.size(); l++) {
         indvars.push_back("_i" + std::to_string(l));
@@ -346,7 +358,7 @@ void install(const StructuredSDFG& sdfg, Block& blk, const MapForm& f) {
     node->set_element_id(blk.node->element_id());
     blk.node = std::move(node);
     blk.inputs = std::move(inputs);
-    blk.outputs[0].connector = "_out0";
+    blk.outputs = std::move(outputs);
 }
 
 bool written_between(const StructuredSDFG& sdfg, const std::string& name, size_t from, size_t to) {
@@ -354,6 +366,29 @@ bool written_between(const StructuredSDFG& sdfg, const std::string& name, size_t
         for (auto& out : sdfg.blocks()[i].outputs)
             if (out.data == name) return true;
     return false;
+}
+
+bool touched_between(const StructuredSDFG& sdfg, const std::string& name, size_t from, size_t to) {
+    for (size_t i = from + 1; i < to; i++) {
+        for (auto& in : sdfg.blocks()[i].inputs)
+            if (!in.is_constant && in.data == name) return true;
+        for (auto& out : sdfg.blocks()[i].outputs)
+            if (out.data == name) return true;
+    }
+    return false;
+}
+
+// a value that only block `reader` reads and only block `writer` writes, and that nobody outside the function sees
+bool private_to(const StructuredSDFG& sdfg, const std::string& name, size_t writer, size_t reader) {
+    const Container& c = sdfg.container(name);
+    if (c.is_argument || !c.transient || name == sdfg.return_container()) return false;
+    for (size_t b = 0; b < sdfg.blocks().size(); b++) {
+        for (auto& in : sdfg.blocks()[b].inputs)
+            if (!in.is_constant && in.data == name && b != reader) return false;
+        for (auto& out : sdfg.blocks()[b].outputs)
+            if (out.data == name && b != writer) return false;
+    }
+    return true;
 }
 
 } // namespace
@@ -370,51 +405,95 @@ bool RocmMapFusionPass::run_pass(builder::StructuredSDFGBuilder& builder, analys
             std::optional<MapForm> consumer = convert.form_of(blocks[j]);
             if (!consumer) continue;
             for (size_t k = 0; k < consumer->reads.size() && !changed; k++) {
+                // the block that wrote what this load reads: the last writer before j, and the only one
                 const std::string link = consumer->reads[k].data;
-                // the value in between: a transient that one earlier block writes and only block j reads
-                const Container& lc = sdfg.container(link);
-                if (lc.is_argument || !lc.transient || link == sdfg.return_container()) continue;
                 long writer = -1;
-                bool private_link = true;
-                for (size_t b = 0; b < blocks.size(); b++) {
-                    for (auto& in : blocks[b].inputs)
-                        if (!in.is_constant && in.data == link && b != j) private_link = false;
+                size_t writers = 0;
+                for (size_t b = 0; b < blocks.size(); b++)
                     for (auto& out : blocks[b].outputs)
                         if (out.data == link) {
-                            if (writer >= 0 || b >= j) private_link = false;
-                            writer = (long) b;
+                            writers++;
+                            if (b < j) writer = (long) b;
                         }
-                }
-                if (!private_link || writer < 0) continue;
+                if (writer < 0 || writers != 1) continue;
                 const size_t i = (size_t) writer;
                 if (blocks[i].node->implementation_type() != blocks[j].node->implementation_type()) continue;
                 std::optional<MapForm> producer = convert.form_of(blocks[i]);
-                if (!producer || producer->bounds != consumer->bounds) continue;
-                // every load of the link takes the element the producer's iteration stores
+                if (!producer) continue;
+
+                // The producer's loops among the consumer's. Equal bounds: loop for loop. Fewer loops (a value per row
+                // that the consumer repeats along the others): the consumer's loops along which the link is indexed,
+                // in order; the producer's work is then done again for every iteration of the other loops, which is
+                // cheaper than a launch and a round trip through memory for values this small.
+                std::vector<long> at(consumer->bounds.size(), -1);     // consumer loop -> producer loop
+                const MapForm::Result* linked = nullptr;
+                for (auto& r : producer->results)
+                    if (r.data == link) linked = &r;
+                if (!linked) continue;
+                const bool same_loops = producer->bounds == consumer->bounds;
+                if (same_loops) {
+                    for (size_t l = 0; l < at.size(); l++) at[l] = (long) l;
+                } else {
+                    size_t next = 0;
+                    bool fits = true;
+                    for (size_t l = 0; l < at.size(); l++) {
+                        if (consumer->reads[k].strides[l] == "0") continue;
+                        if (next >= producer->bounds.size() || producer->bounds[next] != consumer->bounds[l]) fits = false;
+                        else at[l] = (long) next++;
+                    }
+                    // (a short chain only: it is repeated for every element of the consumer)
+                    if (!fits || next != producer->bounds.size() || producer->statements.size() > 8) continue;
+                }
+                auto along_consumer = [&](const std::vector<Expression>& strides) {
+                    std::vector<Expression> out(at.size(), "0");
+                    for (size_t l = 0; l < at.size(); l++)
+                        if (at[l] >= 0) out[l] = strides[(size_t) at[l]];
+                    return out;
+                };
+                // every load of a producer result takes the element the producer's iteration stores
                 bool same_elements = true;
                 for (auto& r : consumer->reads)
-                    if (r.data == link && (r.strides != producer->result_strides || r.element != producer->element)) same_elements = false;
+                    for (auto& pr : producer->results)
+                        if (r.data == pr.data && (r.strides != along_consumer(pr.strides) || r.element != pr.element)) same_elements = false;
                 if (!same_elements) continue;
-                // the producer's work moves to where the consumer stands: what it reads must still hold the same
-                // values there, and the consumer's result may alias a producer operand only element by element
-                bool movable = true;
-                for (auto& r : producer->reads) {
-                    if (written_between(sdfg, r.data, i, j)) movable = false;
-                    if (r.data == consumer->result_data && r.strides != consumer->result_strides) movable = false;
+                // Which producer results are still stored: those somebody else looks at. They are stored where the
+                // consumer stands, so nobody may look at them in between; with fewer loops than the consumer they
+                // would be stored over and over, so there all of them must be private to the two blocks.
+                std::vector<MapForm::Result> kept;
+                bool ok = true;
+                for (auto& pr : producer->results) {
+                    if (private_to(sdfg, pr.data, i, j)) continue;
+                    if (!same_loops || touched_between(sdfg, pr.data, i, j)) ok = false;
+                    for (auto& cr : consumer->results)
+                        if (cr.data == pr.data) ok = false;
+                    kept.push_back(pr);
                 }
-                for (auto& s : producer->scalars)
-                    if (!s.source.is_constant && written_between(sdfg, s.source.data, i, j)) movable = false;
-                if (!movable) continue;
+                // the producer's work moves to where the consumer stands: what it reads must still hold the same
+                // values there, and a consumer result may alias a producer operand only element by element
+                for (auto& r : producer->reads) {
+                    if (written_between(sdfg, r.data, i, j)) ok = false;
+                    for (auto& cr : consumer->results)
+                        if (r.data == cr.data && along_consumer(r.strides) != cr.strides) ok = false;
+                }
+                for (auto& sc : producer->scalars)
+                    if (!sc.source.is_constant && written_between(sdfg, sc.source.data, i, j)) ok = false;
+                if (!ok) continue;
 
                 MapForm merged;
                 merged.bounds = consumer->bounds;
                 merged.element = consumer->element;
-                merged.reads = producer->reads;
+                for (auto r : producer->reads) {
+                    r.strides = along_consumer(r.strides);
+                    merged.reads.push_back(std::move(r));
+                }
                 merged.scalars = producer->scalars;
                 merged.statements = producer->statements;
-                std::map<std::string, std::string> forwarded;   // consumer loads of the link -> the producer's value
+                std::map<std::string, std::string> forwarded;   // consumer loads of producer results -> the producer's values
                 for (auto& r : consumer->reads) {
-                    if (r.data == link) forwarded[r.value] = producer->result_value;
+                    const MapForm::Result* from = nullptr;
+                    for (auto& pr : producer->results)
+                        if (pr.data == r.data) from = &pr;
+                    if (from) forwarded[r.value] = from->value;
                     else merged.reads.push_back(r);
                 }
                 merged.scalars.insert(merged.scalars.end(), consumer->scalars.begin(), consumer->scalars.end());
@@ -426,13 +505,27 @@ bool RocmMapFusionPass::run_pass(builder::StructuredSDFGBuilder& builder, analys
                     for (auto& a : st.args) a = through(a);
                     merged.statements.push_back(std::move(st));
                 }
-                merged.result_value = through(consumer->result_value);
-                merged.result_data = consumer->result_data;
-                merged.result_strides = consumer->result_strides;
-                merged.result_extent = consumer->result_extent;
+                merged.results = kept;
+                for (auto r : consumer->results) {
+                    r.value = through(r.value);
+                    merged.results.push_back(std::move(r));
+                }
+                // a result that is a loaded value or a literal as it stands needs a statement of its own
+                for (auto& r : merged.results) {
+                    bool is_statement = false;
+                    for (auto& st : merged.statements) is_statement = is_statement || st.out == r.value;
+                    if (!is_statement) {
+                        Statement copy{convert.fresh("t"), r.element, "assign", {r.value}};
+                        r.value = copy.out;
+                        merged.statements.push_back(std::move(copy));
+                    }
+                }
+                std::vector<std::string> dropped;
+                for (auto& pr : producer->results)
+                    if (private_to(sdfg, pr.data, i, j)) dropped.push_back(pr.data);
                 install(sdfg, blocks[j], merged);
                 blocks.erase(blocks.begin() + (long) i);
-                sdfg.remove_container(link);
+                for (auto& name : dropped) sdfg.remove_container(name);
                 changed = applied = true;
             }
         }

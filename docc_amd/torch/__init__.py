@@ -19,6 +19,9 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh),
     elu, leaky_relu, hardsigmoid (F.* and nn.ELU / nn.LeakyReLU / nn.Hardsigmoid)
                                            -> ml::ReLU .. ml::Erf
+    gelu (erf and tanh forms), silu, neg, reciprocal, rsqrt, square, layer_norm (F.* / methods / nn.GELU, nn.SiLU,
+    nn.LayerNorm)                          -> the chains of those nodes (and ml::Mean) that spell them; the target's map
+                                              fusion makes one generated kernel of each chain
     F.linear / nn.Linear                   -> GEMM with the weight transposed, bias through Broadcast + Add
     sum / mean / amax / amin over any dims (keepdim) -> ml::Sum .. ml::Min
 
@@ -313,6 +316,46 @@ class _FxLowering:
         self.builder.add_reduce_op(op, x.name, out.name, x.shape, dims, keepdim)
         return out
 
+    # Operations torch has one name for and the node set spells in several: the pieces are tensor nodes, and the map
+    # fusion pass of the target makes one generated kernel of each chain.
+    def gelu(self, node, x, approximate: str, dest):
+        """0.5 x (1 + erf(x / sqrt 2)), or with tanh(sqrt(2 / pi) (x + 0.044715 x^3)) in place of the erf."""
+        if approximate == "tanh":
+            cube = self.elementwise(node, "mul", self.elementwise(node, "mul", x, x, None), x, None)
+            inner = self.elementwise(node, "mul", self.elementwise(node, "add", x, self.elementwise(node, "mul", cube, 0.044715, None), None),
+                                     math.sqrt(2.0 / math.pi), None)
+            gate = self.unary(node, "tanh", inner, None)
+        elif approximate == "none":
+            gate = self.unary(node, "erf", self.elementwise(node, "mul", x, 1.0 / math.sqrt(2.0), None), None)
+        else:
+            self.fail(node, f"gelu with approximate='{approximate}'")
+        half = self.elementwise(node, "mul", x, 0.5, None)
+        return self.elementwise(node, "mul", half, self.elementwise(node, "add", gate, 1.0, None), dest)
+
+    def silu(self, node, x, dest):
+        return self.elementwise(node, "mul", x, self.unary(node, "sigmoid", x, None), dest)
+
+    def layer_norm(self, node, x, normalized_shape, weight, bias, eps: float, dest):
+        """(x - mean) / sqrt(var + eps) * weight + bias over the last len(normalized_shape) axes, the variance as the
+        mean of the squared differences (what torch computes)."""
+        x = self.tensor(node, x)
+        if not isinstance(x, _T):
+            self.fail(node, "layer_norm of this value")
+        shape = [int(v) for v in ([normalized_shape] if isinstance(normalized_shape, int) else normalized_shape)]
+        if not shape or x.shape[-len(shape):] != shape:
+            self.fail(node, "layer_norm whose normalized_shape is not the tensor's last axes")
+        dims = list(range(len(x.shape) - len(shape), len(x.shape)))
+        centred = self.elementwise(node, "sub", x, self.reduce(node, "mean", x, dims, True, None), None)
+        var = self.reduce(node, "mean", self.elementwise(node, "mul", centred, centred, None), dims, True, None)
+        scale = self.unary(node, "sqrt", self.elementwise(node, "add", var, float(eps), None), None)
+        last = weight is None and bias is None
+        y = self.elementwise(node, "div", centred, scale, dest if last else None)
+        if weight is not None:
+            y = self.elementwise(node, "mul", y, weight, dest if bias is None else None)
+        if bias is not None:
+            y = self.elementwise(node, "add", y, bias, dest)
+        return y
+
     def linear(self, node, x, w, bias, dest):
         """x [..., K] times w[N, K] transposed, plus bias [N]: one GEMM over the flattened rows."""
         out_dtype = None
@@ -454,6 +497,22 @@ class _FxLowering:
                     else:
                         self.env[node] = self.unary(node, "hard_sigmoid", self.arg(node.args[0]), dest, alpha=1.0 / 6.0, beta=0.5)
                     continue
+                if isinstance(mod, torch.nn.GELU):
+                    self.env[node] = self.gelu(node, self.arg(node.args[0]), mod.approximate, dest)
+                    continue
+                if isinstance(mod, torch.nn.SiLU):
+                    if mod.inplace:
+                        self.fail(node, "an in-place activation")
+                    self.env[node] = self.silu(node, self.arg(node.args[0]), dest)
+                    continue
+                if isinstance(mod, torch.nn.LayerNorm):
+                    w = b = None
+                    if mod.weight is not None:
+                        w = self.add_input(f"{node.name}_weight", list(mod.weight.shape), mod.weight.dtype, ("attr", f"{node.target}.weight"))
+                    if mod.bias is not None:
+                        b = self.add_input(f"{node.name}_bias", list(mod.bias.shape), mod.bias.dtype, ("attr", f"{node.target}.bias"))
+                    self.env[node] = self.layer_norm(node, self.arg(node.args[0]), list(mod.normalized_shape), w, b, mod.eps, dest)
+                    continue
                 if isinstance(mod, torch.nn.Linear):
                     w = self.add_input(f"{node.name}_weight", list(mod.weight.shape), mod.weight.dtype, ("attr", f"{node.target}.weight"))
                     b = None
@@ -562,6 +621,24 @@ class _FxLowering:
                 if kwargs.get("inplace"):
                     self.fail(node, "an in-place activation")
                 return self.unary(node, op, args[0], dest)
+        if t is F.gelu:
+            return self.gelu(node, args[0], kwargs.get("approximate", args[1] if len(args) > 1 else "none"), dest)
+        if t is F.silu:
+            if kwargs.get("inplace") or (len(args) > 1 and args[1]):
+                self.fail(node, "an in-place activation")
+            return self.silu(node, args[0], dest)
+        if t in (torch.neg, torch.negative, operator.neg) or method in ("neg", "negative"):
+            return self.elementwise(node, "mul", args[0], -1.0, dest)
+        if t is torch.reciprocal or method == "reciprocal":
+            return self.elementwise(node, "div", 1.0, args[0], dest)
+        if t is torch.rsqrt or method == "rsqrt":
+            return self.elementwise(node, "div", 1.0, self.unary(node, "sqrt", args[0], None), dest)
+        if t is torch.square or method == "square":
+            return self.elementwise(node, "mul", args[0], args[0], dest)
+        if t is F.layer_norm:
+            names = ["input", "normalized_shape", "weight", "bias", "eps"]
+            bound = {"weight": None, "bias": None, "eps": 1e-5, **dict(zip(names, args)), **kwargs}
+            return self.layer_norm(node, bound["input"], bound["normalized_shape"], bound["weight"], bound["bias"], bound["eps"], dest)
         if t in (F.elu, F.leaky_relu, F.hardsigmoid):
             if kwargs.get("inplace") or (len(args) > 2 and args[2]):
                 self.fail(node, "an in-place activation")

@@ -612,3 +612,51 @@ def test_bf16_products_lower_to_the_gemm_with_float32_accumulation():
     # the product rounded back to bf16 is not built
     with pytest.raises(NotImplementedError, match="float"):
         docc_torch.TorchProgram(Rounded(), target="rocm").to_sdfg(ta, tb)
+
+
+def test_torch_lowering_of_composite_activations_and_layer_norm():
+    """gelu, silu, neg, reciprocal, rsqrt, square and layer_norm are spelled with the tensor nodes there are; scheduled, the
+    chains between the reductions and products are single generated kernels."""
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.LayerNorm(16)
+            self.fc1 = torch.nn.Linear(16, 32)
+            self.act = torch.nn.GELU()
+            self.fc2 = torch.nn.Linear(32, 16)
+
+        def forward(self, x):
+            return x + self.fc2(self.act(self.fc1(self.norm(x))))
+
+    x = torch.randn(2, 5, 16)
+    sdfg = docc_torch.TorchProgram(Block(), (x,), target="rocm").to_sdfg()
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    # layer norm: mean, centre, mean of squares, + eps, sqrt, divide, weight, bias
+    assert codes[:13] == ["ml::Mean", "ml::Broadcast", "ml::Sub", "ml::Mul", "ml::Mean", "ml::Add", "ml::Sqrt", "ml::Broadcast", "ml::Div",
+                          "ml::Broadcast", "ml::Mul", "ml::Broadcast", "ml::Add"]
+    assert codes[13:] == ["GEMM", "ml::Broadcast", "ml::Add", "ml::Mul", "ml::Erf", "ml::Mul", "ml::Add", "ml::Mul",
+                          "GEMM", "ml::Broadcast", "ml::Add", "ml::Add"]
+    sdfg.schedule("rocm")
+    kernels = [n["code"] for n in sdfg.library_nodes() if n["code"] != "ROCMOffloading"]
+    # mean | centre and square in one kernel each (the centred value has two readers) | mean | the rest of the norm |
+    # GEMM with its bias | gelu | GEMM with its bias | the residual
+    assert kernels.count("GEMM") == 2 and kernels.count("ml::Mean") == 2 and kernels.count("ROCMMap") >= 2
+    assert len(kernels) <= 9, kernels
+
+    class Misc(torch.nn.Module):
+        def forward(self, a, b):
+            return F.silu(a) * torch.rsqrt(b.square() + 1.0) - (-a).reciprocal() + F.gelu(b, approximate="tanh")
+
+    F = torch.nn.functional
+    sdfg = docc_torch.TorchProgram(Misc(), (torch.randn(6, 7), torch.randn(6, 7)), target="rocm").to_sdfg()
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes.count("ml::Sigmoid") == 1 and codes.count("ml::Sqrt") == 1 and codes.count("ml::Tanh") == 1 and codes.count("ml::Div") == 2
+    sdfg.schedule("rocm")
+    assert [n["code"] for n in sdfg.library_nodes() if n["code"] != "ROCMOffloading"] == ["ROCMMap"]      # one kernel for all of it
+
+    class Bad(torch.nn.Module):
+        def forward(self, a):
+            return F.gelu(a, approximate="sigmoid")
+
+    with pytest.raises((NotImplementedError, RuntimeError)):      # torch itself refuses the word while it traces
+        docc_torch.TorchProgram(Bad(), (torch.randn(4),), target="rocm").to_sdfg()

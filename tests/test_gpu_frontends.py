@@ -812,3 +812,58 @@ def test_products_with_vectors_follow_numpy():
     np.testing.assert_allclose(xx, x @ x, rtol=1e-13)
     codes = [n["code"] for n in products.last_sdfg.library_nodes() if not n["code"].startswith("ROCM")]
     assert codes == ["GEMM", "GEMM", "ml::Mul", "ml::Sum", "GEMM"]
+
+
+@pytest.mark.parametrize("approximate", ["none", "tanh"])
+def test_torch_compile_transformer_mlp_block(approximate):
+    """LayerNorm -> Linear -> GELU -> Linear and the residual, on device tensors: the pieces of the norm and of the
+    activation are tensor nodes that the target merges into generated kernels. Against the model in float64."""
+    class Block(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.norm = torch.nn.LayerNorm(256)
+            self.fc1 = torch.nn.Linear(256, 1024)
+            self.act = torch.nn.GELU(approximate=approximate)
+            self.fc2 = torch.nn.Linear(1024, 256)
+
+        def forward(self, x):
+            return x + self.fc2(self.act(self.fc1(self.norm(x))))
+
+    torch.manual_seed(3)
+    model = Block().cuda()
+    with torch.no_grad():
+        model.norm.weight.uniform_(0.5, 1.5)
+        model.norm.bias.uniform_(-0.5, 0.5)
+    x = torch.randn(8, 128, 256, device="cuda") * 2 + 0.5
+    program = docc_torch.compile_torch(model, x, target="rocm")
+    y = program(x)
+    assert y.is_cuda and y.shape == x.shape
+    with torch.no_grad():
+        ref = model.double()(x.double())
+    assert rel_err_max(y.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+    kernels = [n["code"] for n in program.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"]
+    assert kernels.count("GEMM") == 2 and kernels.count("ml::Mean") == 2 and kernels.count("ROCMMap") == 3 and len(kernels) == 8, kernels
+
+
+def test_torch_compile_composite_elementwise_operations():
+    class Misc(torch.nn.Module):
+        def forward(self, a, b):
+            F = torch.nn.functional
+            return F.silu(a) * torch.rsqrt(b.square() + 1.0) - (-a).reciprocal() + F.gelu(b, approximate="tanh")
+
+    torch.manual_seed(4)
+    for dtype, tol in ((torch.float32, 1e-5), (torch.float64, 1e-12)):
+        a, b = torch.randn(37, 129, dtype=dtype) + 3.0, torch.randn(37, 129, dtype=dtype)
+        program = docc_torch.compile_torch(Misc(), (a, b), target="rocm")
+        out = program(a, b)
+        ref = Misc()(a.double(), b.double())
+        assert out.dtype == dtype and rel_err_max(out.numpy(), ref.numpy()) <= tol
+        assert [n["code"] for n in program.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"] == ["ROCMMap"]
+
+    class Norm(torch.nn.Module):
+        def forward(self, x, w):
+            return torch.nn.functional.layer_norm(x, (6, 40), weight=w, eps=1e-3)
+
+    x, w = torch.randn(5, 7, 6, 40), torch.rand(6, 40) + 0.5
+    out = docc_torch.compile_torch(Norm(), (x, w), target="rocm")(x, w)
+    assert rel_err_max(out.numpy(), Norm()(x.double(), w.double()).numpy()) <= 1e-5

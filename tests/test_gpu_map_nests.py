@@ -139,7 +139,7 @@ def test_module_load_get_function_and_launch(tmp_path, rt):
     the kernel runs it; a missing image, a missing name and an oversized block are reported as errors."""
     import torch
     s = StructuredSDFG.from_docc_json(json.dumps(fused_map_program(FLOAT)))
-    s.schedule("rocm", options={"offload": "none"})
+    s.schedule("rocm", options={"offload": "none", "fuse_maps": False})      # the two nests as they were written: two kernels
     s._compile(str(tmp_path))
     images = sorted(tmp_path.glob("kernel_*.hsaco"))
     assert len(images) == 2

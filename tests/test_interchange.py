@@ -777,7 +777,13 @@ def test_map_nests_with_several_operations_import_as_generated_kernels(tmp_path)
     again = StructuredSDFG.parse(s.to_json())
     assert again.library_nodes() == s.library_nodes()
 
-    s.schedule("rocm")
+    # the two nests as two kernels (the map fusion pass would make one of them: Y of the first is what the second reads)
+    merged = StructuredSDFG.parse(s.to_json())
+    merged.schedule("rocm")
+    (one,) = [n for n in merged.library_nodes() if n["code"] == "ROCMMap"]
+    assert [w["value"] for w in one["writes"]] == ["_v2", "_v4", "_v4"] and len(one["reads"]) == 3      # Y, Z, W; Y is not read back
+    assert merged.loop_report()["H2D"] == 3 and merged.loop_report()["D2H"] == 3
+    s.schedule("rocm", options={"fuse_maps": False})
     assert [n["implementation_type"] for n in s.library_nodes() if n["code"] == "ROCMMap"] == ["ROCMWithoutTransfers"] * 2
     r = s.loop_report()
     assert r["H2D"] == 3 and r["D2H"] == 3            # A B C up; Y Z W down; Y stays on the device between the nests

@@ -722,15 +722,17 @@ def test_fusion_folds_the_chain_into_one_kernel(tmp_path):
     assert nodes == [("ROCMFusedElementWise", ["ml::Abs", "ml::Sqrt"], ""), ("ml::Tanh", None, None), ("ml::Sub", None, None),
                      ("ml::Exp", None, None)]
     # what the prebuilt kernels leave as separate launches becomes one generated kernel: tanh and the subtraction are
-    # one nest, which is then the only reader of T1, so the chain in front joins it; Y, an argument, is still written
+    # one nest, which is then the only reader of T1, so the chain in front joins it; Y, an argument, is still written,
+    # and the exponential of it is a second result of the same nest
     s = StructuredSDFG.parse(text)
     s.schedule("rocm")
     nodes = [n for n in s.library_nodes() if not n["code"].startswith("ROCMOff")]
-    assert [n["code"] for n in nodes] == ["ROCMMap", "ml::Exp"]
+    assert [n["code"] for n in nodes] == ["ROCMMap"]
     assert [(st["op"], st["args"]) for st in nodes[0]["statements"]] == [
-        ("fabs", ["_in0"]), ("sqrt", ["_v0"]), ("tanh", ["_v1"]), ("fp_sub", ["_v2", "_v1"])]
-    assert nodes[0]["bounds"] == ["100"] and len(nodes[0]["reads"]) == 1 and nodes[0]["writes"][0]["value"] == "_v3"
+        ("fabs", ["_in0"]), ("sqrt", ["_v0"]), ("tanh", ["_v1"]), ("fp_sub", ["_v2", "_v1"]), ("exp", ["_v3"])]
+    assert nodes[0]["bounds"] == ["100"] and len(nodes[0]["reads"]) == 1 and [w["value"] for w in nodes[0]["writes"]] == ["_v3", "_v4"]
     assert not {"T0", "T1", "T2"} & set(s.containers)
+    assert s.loop_report()["H2D"] == 1 and s.loop_report()["D2H"] == 2
 
     # without a device compiler on the machine the chain keeps its prebuilt kernels
     import os
