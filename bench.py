@@ -57,7 +57,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise")
+    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise,graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the PCIe-inclusive calls through @native")
     ap.add_argument("--no-zero", action="store_true", help="skip the extra timing of the bf16 kernels on all-zero operands (profiling runs: "
@@ -470,6 +470,61 @@ def main():
                 "sample": "full tensor, the Map the reference's ElementWiseBinaryNode expands to (omp parallel for)"}
         del As, Bs, Ys
 
+    # ---- a launch-bound function: kernel by kernel, and replayed as a HIP graph --------------------------
+    # LayerNorm -> Linear -> GELU -> Linear + residual on [8, 128, 256] device tensors compiles to eight kernels of a
+    # few microseconds each. Wall time per call of the generated function (the host submits eight launches and the
+    # cached allocations between them) against a replay of the same call recorded once (one submission).
+    graph_replay = {}
+    if want("graph"):
+        import docc_amd.torch as docc_torch
+
+        os.environ.setdefault("DOCC_TMP", str(Path(tempfile.gettempdir()) / f"docc_bench_{os.getpid()}"))
+
+        class Block(torch.nn.Module):
+            def __init__(self):
+                super().__init__()
+                self.norm = torch.nn.LayerNorm(256)
+                self.fc1 = torch.nn.Linear(256, 1024)
+                self.act = torch.nn.GELU()
+                self.fc2 = torch.nn.Linear(1024, 256)
+
+            def forward(self, x):
+                return x + self.fc2(self.act(self.fc1(self.norm(x))))
+
+        torch.manual_seed(0)
+        xb = torch.randn(8, 128, 256, device="cuda")
+        program = docc_torch.compile_torch(Block().cuda(), xb, target="rocm")
+        compiled = program.compile(xb)
+        recorded = compiled.record(xb)
+        keep, ptrs = compiled._operands((xb,), xb.device)
+        result = torch.empty_like(recorded.result)
+        ptrs = ptrs + [result.data_ptr()]
+
+        def wall_us(submit, wait, calls=400):
+            for _ in range(50):
+                submit()
+            wait()
+            best = float("inf")
+            for _ in range(5):
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    submit()
+                wait()
+                best = min(best, (time.perf_counter() - t0) / calls)
+            return round(best * 1e6, 2)
+
+        eager_us = wall_us(lambda: compiled.func(*ptrs), rt.device_sync)
+        replay_us = wall_us(lambda: recorded.replay(wait=False), recorded.wait)
+        same = bool(torch.equal(result, recorded.result))
+        kernels_per_call = len([n for n in program.last_sdfg.library_nodes() if n["code"] != "ROCMOffloading"])
+        graph_replay["transformer_mlp_block_f32_8x128x256"] = {
+            "kernels_per_call": kernels_per_call, "kernel_by_kernel_us_per_call": eager_us, "graph_replay_us_per_call": replay_us,
+            "same_bits": same}
+        recorded.close()
+        code, message = rt.take_failure()
+        if code:
+            raise RuntimeError(message)
+
     # ---- PCIe-inclusive: host arrays in, host array out, through @native (never the reported `value`) ----
     end_to_end = {}
     if not args.no_e2e and (want("softmax") or want("dgemm")):
@@ -531,6 +586,8 @@ def main():
     if "cpu_baseline" in out:
         line["cpu_baseline"] = out["cpu_baseline"]
     line["kernels"] = kernels
+    if graph_replay:
+        line["graph_replay"] = graph_replay
     if end_to_end:
         line["end_to_end_through_native"] = end_to_end
     print(json.dumps(line))

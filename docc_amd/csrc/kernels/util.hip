@@ -22,6 +22,26 @@ extern "C" __global__ __launch_bounds__(256) void docc_copy_b128(const u32x4* __
     }
 }
 
+// Byte fill, what hipMemsetAsync does, as a kernel: a memset recorded into a HIP graph is a node of its own kind,
+// a kernel is a kernel. Bytes up to the first 16-byte boundary and after the last one are written singly (by the
+// first work-group), the rest as 16-byte vectors.
+extern "C" __global__ __launch_bounds__(256) void docc_fill_b8(uint8_t* __restrict__ dst, int value, long n) {
+    const uint8_t b = (uint8_t) value;
+    long head = (long) ((16 - ((uintptr_t) dst & 15)) & 15);
+    if (head > n) head = n;
+    const long n16 = (n - head) / 16;
+    const long tail = head + n16 * 16;
+    if (blockIdx.x == 0) {
+        for (long i = threadIdx.x; i < head; i += 256) dst[i] = b;
+        for (long i = tail + threadIdx.x; i < n; i += 256) dst[i] = b;
+    }
+    const uint32_t w = 0x01010101u * b;
+    const u32x4 v = {w, w, w, w};
+    u32x4* body = (u32x4*) (dst + head);
+    const long stride = (long) gridDim.x * 256;
+    for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) body[i] = v;
+}
+
 extern "C" __global__ __launch_bounds__(256) void docc_f32_to_bf16(const float* __restrict__ src,
                                                                      uint16_t* __restrict__ dst, long n) {
     long i = (long) blockIdx.x * 256 + threadIdx.x;

@@ -352,7 +352,7 @@ extern "C" int docc_rocm_cast(docc_rocm_stream_t stream, int src_type, int dst_t
     if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "cast: null pointer");
     if (src_type == dst_type) {
         if (X == Y) return 0;
-        return check(hipMemcpyAsync(Y, X, (size_t) n * kSize[src_type], hipMemcpyDeviceToDevice, (hipStream_t) stream), "hipMemcpyAsync");
+        return check(hipMemcpyAsync(Y, X, (size_t) n * kSize[src_type], hipMemcpyDeviceToDevice, resolve_stream((hipStream_t) stream)), "hipMemcpyAsync");
     }
     // built: fp32 <-> fp64 / bf16 / fp16, int32 / int64 <-> fp32 / fp64
     const bool f = src_type == DOCC_ROCM_TYPE_F32 || src_type == DOCC_ROCM_TYPE_F64, g = dst_type == DOCC_ROCM_TYPE_F32 || dst_type == DOCC_ROCM_TYPE_F64;

@@ -90,7 +90,8 @@ extern "C" int docc_rocm_dot(docc_rocm_stream_t stream, int precision, int64_t n
     if (groups > 4 * (int64_t) cus) groups = 4 * (int64_t) cus;
     const int64_t chunk = (n + groups - 1) / groups;
     groups = (n + chunk - 1) / chunk;
-    hipStream_t s = (hipStream_t) stream;
+    if (capturing()) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "dot: returns its result to the host and cannot be captured into a graph");
+    hipStream_t s = resolve_stream((hipStream_t) stream);
     PartialsLease partials;
     if (int rc = partials_for(s, &partials)) return rc;
     const char* t = precision == 32 ? "f32" : "f64";

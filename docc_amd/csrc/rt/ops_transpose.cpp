@@ -76,7 +76,7 @@ extern "C" int docc_rocm_transpose(docc_rocm_stream_t stream, int element_bytes,
         }
     }
     r = m;
-    hipStream_t st = (hipStream_t) stream;
+    hipStream_t st = resolve_stream((hipStream_t) stream);
     if (r <= 1)   // nothing moves
         return check(hipMemcpyAsync(Y, X, (size_t) n * element_bytes, hipMemcpyDeviceToDevice, st), "hipMemcpyAsync");
 

@@ -39,6 +39,12 @@ struct PartialsLease {
 };
 int partials_for(hipStream_t stream, PartialsLease* lease);
 
+// The stream work is enqueued on: `stream` itself, or - where generated code and callers pass the null stream -
+// the stream the calling thread has named with docc_rocm_set_default_stream (the null stream if none).
+hipStream_t resolve_stream(hipStream_t stream);
+// True while the calling thread has a graph capture open: calls that must wait for the device refuse then.
+bool capturing();
+
 // Launch helper: packs the addresses of `args` for hipModuleLaunchKernel.
 template <typename... Args>
 int launch(const char* name, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t block, uint32_t shared_bytes,
@@ -46,6 +52,7 @@ int launch(const char* name, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t blo
     hipFunction_t fn;
     int rc = kernel(name, &fn);
     if (rc) return rc;
+    stream = resolve_stream(stream);
     void* ptrs[] = {(void*) &args...};
     if (gx == 0 || gy == 0 || gz == 0) return 0;
     if (gy > 65535u || gz > 65535u) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "%s: grid y/z too large", name);

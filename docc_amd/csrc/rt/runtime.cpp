@@ -99,6 +99,24 @@ BlockCache& block_cache() {
     return *cache;
 }
 
+// A graph capture in progress on the calling thread. Device memory that the captured code takes from the block cache
+// belongs to the graph from then on (every replay writes to those addresses): blocks "freed" during the capture go to
+// a list of the capture's own, from which later allocations of the same capture are served (the captured work is one
+// chain in stream order, so a block's next user starts after its last one), and all of them return to the cache when
+// the graph is destroyed.
+struct Capture {
+    hipStream_t stream = nullptr;
+    hipStream_t previous_default = nullptr;
+    std::vector<std::pair<void*, size_t>> blocks;          // every block the capture holds
+    std::multimap<size_t, void*> free_blocks;              // those not in use at this point of the capture
+};
+
+struct Graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<std::pair<void*, size_t>> blocks;
+};
+
 std::mutex g_failure_mutex;
 int g_failure_code = 0;
 std::string g_failure_message;
@@ -122,6 +140,16 @@ std::string kernel_image_dir() {
 }
 
 } // namespace
+
+namespace {
+// What the calling thread has set with docc_rocm_set_default_stream, and the capture it has open (if any).
+thread_local hipStream_t t_default_stream = nullptr;
+thread_local Capture* t_capture = nullptr;
+} // namespace
+
+hipStream_t resolve_stream(hipStream_t stream) { return stream ? stream : t_default_stream; }
+
+bool capturing() { return t_capture != nullptr; }
 
 int fail(int code, const char* fmt, ...) {
     char buf[512];
@@ -244,6 +272,7 @@ std::map<std::pair<int, hipStream_t>, PartialsSlot*>& partials_slots() {
 } // namespace
 
 int partials_for(hipStream_t stream, PartialsLease* lease) {
+    stream = resolve_stream(stream);
     int dev = 0;
     int rc = check(hipGetDevice(&dev), "hipGetDevice");
     if (rc) return rc;
@@ -535,14 +564,28 @@ int pool_malloc(void** dev_ptr, size_t bytes, bool ordered, hipStream_t stream) 
     int dev = 0;
     int rc = check(hipGetDevice(&dev), "hipGetDevice");
     if (rc) return rc;
+    stream = resolve_stream(stream);
+    Capture* capture = t_capture;
+    if (capture) {
+        // a block of the capture's own first; from the cache only one that needs no wait (no event may be waited for
+        // or recorded while the stream is being captured)
+        auto mine = capture->free_blocks.find(rounded);
+        if (mine != capture->free_blocks.end()) {
+            *dev_ptr = mine->second;
+            capture->free_blocks.erase(mine);
+            return 0;
+        }
+        ordered = true;
+        stream = capture->stream;
+    }
     CachedBlock got;
     {
         std::lock_guard<std::mutex> lock(c.mutex);
         auto range = c.free_blocks.equal_range({dev, rounded});
-        auto pick = range.first;
+        auto pick = capture ? range.second : range.first;
         // prefer a block that needs no wait: released on this very stream, or not pending at all
         for (auto it = range.first; it != range.second; ++it)
-            if (!it->second.pending || (ordered && it->second.stream == stream)) {
+            if (!it->second.pending || (!capture && ordered && it->second.stream == stream)) {
                 pick = it;
                 break;
             }
@@ -560,6 +603,7 @@ int pool_malloc(void** dev_ptr, size_t bytes, bool ordered, hipStream_t stream) 
             if (rc) return rc;   // the block stays in `live`; its owner-to-be never sees it
         }
         *dev_ptr = got.ptr;
+        if (capture) capture->blocks.push_back({got.ptr, rounded});
         return 0;
     }
     hipError_t e = hipMalloc(dev_ptr, rounded);
@@ -572,12 +616,29 @@ int pool_malloc(void** dev_ptr, size_t bytes, bool ordered, hipStream_t stream) 
     if (rc) return rc;
     std::lock_guard<std::mutex> lock(c.mutex);
     c.live[*dev_ptr] = {dev, rounded, nullptr};
+    if (capture) capture->blocks.push_back({*dev_ptr, rounded});
     return 0;
 }
 
 int pool_free(void* dev_ptr, bool ordered, hipStream_t stream) {
     if (!dev_ptr) return 0;
     BlockCache& c = block_cache();
+    stream = resolve_stream(stream);
+    if (Capture* capture = t_capture) {
+        // the block stays with the capture (and later with its graph); a block from before the capture joins it
+        size_t bytes = 0;
+        for (auto& b : capture->blocks)
+            if (b.first == dev_ptr) bytes = b.second;
+        if (bytes == 0) {
+            std::lock_guard<std::mutex> lock(c.mutex);
+            auto it = c.live.find(dev_ptr);
+            if (it == c.live.end()) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "free during a graph capture: not a block of this runtime");
+            bytes = it->second.bytes;
+            capture->blocks.push_back({dev_ptr, bytes});
+        }
+        capture->free_blocks.insert({bytes, dev_ptr});
+        return 0;
+    }
     BlockCache::Live info{0, 0, nullptr};
     bool keep = false;
     {
@@ -670,7 +731,14 @@ int docc_rocm_pool_set_limit(size_t limit_bytes) {
 
 int docc_rocm_memset_async(void* dev_ptr, int value, size_t bytes, docc_rocm_stream_t stream) {
     if (bytes == 0) return 0;
-    return check(hipMemsetAsync(dev_ptr, value, bytes, (hipStream_t) stream), "hipMemsetAsync");
+    if (capturing()) {
+        // a kernel instead of a memset node in the graph
+        long groups = (long) ((bytes / 16 + 1023) / 1024);
+        if (groups < 1) groups = 1;
+        if (groups > 4096) groups = 4096;
+        return launch("docc_fill_b8", (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, dev_ptr, value, (long) bytes);
+    }
+    return check(hipMemsetAsync(dev_ptr, value, bytes, resolve_stream((hipStream_t) stream)), "hipMemsetAsync");
 }
 
 int docc_rocm_host_malloc(void** host_ptr, size_t bytes) {
@@ -690,21 +758,21 @@ int docc_rocm_host_free(void* host_ptr) {
 
 int docc_rocm_memcpy_h2d_async(void* dst_dev, const void* src_host, size_t bytes, docc_rocm_stream_t stream) {
     if (bytes == 0) return 0;
-    if (bytes >= kStageMin && !is_pinned(src_host, bytes)) {
-        const int rc = staged_h2d(dst_dev, src_host, bytes, (hipStream_t) stream);
+    if (bytes >= kStageMin && !capturing() && !is_pinned(src_host, bytes)) {
+        const int rc = staged_h2d(dst_dev, src_host, bytes, resolve_stream((hipStream_t) stream));
         if (rc != 1) return rc;     // 1: staging is switched off or could not be set up
     }
-    return check(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, (hipStream_t) stream), "hipMemcpyAsync(H2D)");
+    return check(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, resolve_stream((hipStream_t) stream)), "hipMemcpyAsync(H2D)");
 }
 
 int docc_rocm_memcpy_d2h_async(void* dst_host, const void* src_dev, size_t bytes, docc_rocm_stream_t stream) {
     if (bytes == 0) return 0;
-    return check(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, (hipStream_t) stream), "hipMemcpyAsync(D2H)");
+    return check(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, resolve_stream((hipStream_t) stream)), "hipMemcpyAsync(D2H)");
 }
 
 int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes, docc_rocm_stream_t stream) {
     if (bytes == 0) return 0;
-    return check(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, (hipStream_t) stream), "hipMemcpyAsync(D2D)");
+    return check(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, resolve_stream((hipStream_t) stream)), "hipMemcpyAsync(D2D)");
 }
 
 int docc_rocm_stream_create(docc_rocm_stream_t* stream) {
@@ -718,12 +786,13 @@ int docc_rocm_stream_create(docc_rocm_stream_t* stream) {
 
 int docc_rocm_stream_destroy(docc_rocm_stream_t stream) {
     if (!stream) return 0;
+    if (t_default_stream == (hipStream_t) stream) t_default_stream = nullptr;
     release_partials((hipStream_t) stream);
     return check(hipStreamDestroy((hipStream_t) stream), "hipStreamDestroy");
 }
 
 int docc_rocm_stream_sync(docc_rocm_stream_t stream) {
-    return check(hipStreamSynchronize((hipStream_t) stream), "hipStreamSynchronize");
+    return check(hipStreamSynchronize(resolve_stream((hipStream_t) stream)), "hipStreamSynchronize");
 }
 
 int docc_rocm_device_sync(void) { return check(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
@@ -735,7 +804,7 @@ int docc_rocm_launch(docc_rocm_function_t function, const uint32_t grid[3], cons
     uint64_t threads = (uint64_t) block[0] * block[1] * block[2];
     if (threads == 0 || threads > 1024) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "launch: block of %llu threads", (unsigned long long) threads);
     return check(hipModuleLaunchKernel((hipFunction_t) function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
-                                       shared_bytes, (hipStream_t) stream, args, nullptr),
+                                       shared_bytes, resolve_stream((hipStream_t) stream), args, nullptr),
                  "hipModuleLaunchKernel");
 }
 
@@ -754,7 +823,7 @@ int docc_rocm_event_destroy(docc_rocm_event_t event) {
 }
 
 int docc_rocm_event_record(docc_rocm_event_t event, docc_rocm_stream_t stream) {
-    return check(hipEventRecord((hipEvent_t) event, (hipStream_t) stream), "hipEventRecord");
+    return check(hipEventRecord((hipEvent_t) event, resolve_stream((hipStream_t) stream)), "hipEventRecord");
 }
 
 int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, float* ms) {
@@ -762,6 +831,110 @@ int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, 
     int rc = check(hipEventSynchronize((hipEvent_t) stop), "hipEventSynchronize");
     if (rc) return rc;
     return check(hipEventElapsedTime(ms, (hipEvent_t) start, (hipEvent_t) stop), "hipEventElapsedTime");
+}
+
+int docc_rocm_set_default_stream(docc_rocm_stream_t stream) {
+    if (t_capture) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "set_default_stream: a graph capture is open on this thread");
+    t_default_stream = (hipStream_t) stream;
+    return 0;
+}
+
+int docc_rocm_graph_capture_begin(docc_rocm_stream_t stream) {
+    if (!stream) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_capture_begin: the null stream cannot be captured; create one");
+    if (t_capture) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_capture_begin: a capture is already open on this thread");
+    int rc = ensure_device();
+    if (rc) return rc;
+    // Everything released so far is over once the device has been waited for, so every cached block can be handed
+    // out during the capture without a wait (which a capturing stream could not record).
+    rc = check(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    if (rc) return rc;
+    {
+        BlockCache& c = block_cache();
+        std::lock_guard<std::mutex> lock(c.mutex);
+        for (auto& b : c.free_blocks) b.second.pending = false;
+    }
+    // relaxed: the block cache may still have to call hipMalloc for a size it has not seen
+    rc = check(hipStreamBeginCapture((hipStream_t) stream, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture");
+    if (rc) return rc;
+    auto* capture = new Capture();
+    capture->stream = (hipStream_t) stream;
+    capture->previous_default = t_default_stream;
+    t_default_stream = (hipStream_t) stream;
+    t_capture = capture;
+    return 0;
+}
+
+namespace {
+// the blocks go back to the cache, free for anybody: the device has finished with them
+void return_blocks(const std::vector<std::pair<void*, size_t>>& blocks) {
+    if (blocks.empty()) return;
+    (void) hipDeviceSynchronize();
+    BlockCache& c = block_cache();
+    int dev = 0;
+    (void) hipGetDevice(&dev);
+    for (auto& b : blocks) {
+        hipEvent_t released = nullptr;
+        bool keep = false;
+        {
+            std::lock_guard<std::mutex> lock(c.mutex);
+            auto it = c.live.find(b.first);
+            if (it != c.live.end()) {
+                released = it->second.released;
+                dev = it->second.device;
+                c.live.erase(it);
+            }
+            keep = c.limit > 0 && b.second <= c.limit - (c.cached_bytes < c.limit ? c.cached_bytes : c.limit);
+            if (keep) {
+                CachedBlock blk;
+                blk.ptr = b.first;
+                blk.released = released;
+                c.free_blocks.insert({{dev, b.second}, blk});
+                c.cached_bytes += b.second;
+            }
+        }
+        if (!keep) {
+            if (released) (void) hipEventDestroy(released);
+            (void) hipFree(b.first);
+        }
+    }
+}
+} // namespace
+
+int docc_rocm_graph_capture_end(docc_rocm_graph_t* graph) {
+    Capture* capture = t_capture;
+    if (!capture) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_capture_end: no capture is open on this thread");
+    t_capture = nullptr;
+    t_default_stream = capture->previous_default;
+    auto* g = new Graph();
+    g->blocks = std::move(capture->blocks);
+    int rc = check(hipStreamEndCapture(capture->stream, &g->graph), "hipStreamEndCapture");
+    delete capture;
+    if (!rc && !graph) rc = fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_capture_end: null argument");
+    if (!rc) rc = check(hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0), "hipGraphInstantiate");
+    if (rc) {
+        if (g->graph) (void) hipGraphDestroy(g->graph);
+        return_blocks(g->blocks);
+        delete g;
+        return rc;
+    }
+    *graph = g;
+    return 0;
+}
+
+int docc_rocm_graph_launch(docc_rocm_graph_t graph, docc_rocm_stream_t stream) {
+    if (!graph) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_launch: null graph");
+    if (t_capture) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "graph_launch: a capture is open on this thread");
+    return check(hipGraphLaunch(((Graph*) graph)->exec, resolve_stream((hipStream_t) stream)), "hipGraphLaunch");
+}
+
+int docc_rocm_graph_destroy(docc_rocm_graph_t graph) {
+    if (!graph) return 0;
+    auto* g = (Graph*) graph;
+    return_blocks(g->blocks);          // waits for the device first: a replay may still be running
+    int rc = check(hipGraphExecDestroy(g->exec), "hipGraphExecDestroy");
+    const int rc2 = check(hipGraphDestroy(g->graph), "hipGraphDestroy");
+    delete g;
+    return rc ? rc : rc2;
 }
 
 void docc_rocm_report_failure(const char* function, const char* call, int code) {

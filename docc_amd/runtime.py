@@ -8,6 +8,7 @@ from __future__ import annotations
 import ctypes
 import os
 from pathlib import Path
+from typing import Optional
 
 LIB_DIR = Path(__file__).resolve().parent / "lib"
 LIB_PATH = LIB_DIR / "libdocc_rt_rocm.so"
@@ -61,6 +62,11 @@ _SIGNATURES = {
     "docc_rocm_event_destroy": [_vp],
     "docc_rocm_event_record": [_vp, _vp],
     "docc_rocm_event_elapsed_ms": [_vp, _vp, ctypes.POINTER(_f32)],
+    "docc_rocm_set_default_stream": [_vp],
+    "docc_rocm_graph_capture_begin": [_vp],
+    "docc_rocm_graph_capture_end": [ctypes.POINTER(_vp)],
+    "docc_rocm_graph_launch": [_vp, _vp],
+    "docc_rocm_graph_destroy": [_vp],
     "docc_rocm_report_failure": [ctypes.c_char_p, ctypes.c_char_p, _int],
     "docc_rocm_take_failure": [ctypes.c_char_p, ctypes.c_size_t],
     "docc_rocm_last_error": [],
@@ -204,6 +210,15 @@ def pool_stats() -> tuple[int, int, int]:
 
 def pool_set_limit(nbytes: int) -> None:
     call("docc_rocm_pool_set_limit", nbytes)
+
+
+def memset(ptr: int, value: int, nbytes: int, stream: int = 0) -> None:
+    """Fills `nbytes` bytes of device memory with the byte `value`, in stream order."""
+    call("docc_rocm_memset_async", ptr, value, nbytes, stream)
+
+
+def memcpy_d2d(dst_dev: int, src_dev: int, nbytes: int, stream: int = 0) -> None:
+    call("docc_rocm_memcpy_d2d_async", dst_dev, src_dev, nbytes, stream)
 
 
 def memcpy_h2d(dst_dev: int, src_host: int, nbytes: int, stream: int = 0) -> None:
@@ -461,6 +476,73 @@ def stream_create() -> int:
 
 def stream_destroy(stream: int) -> None:
     call("docc_rocm_stream_destroy", stream)
+
+
+def set_default_stream(stream: int = 0) -> None:
+    """Names the stream that stands in for the null stream in this thread's calls of the runtime (generated code
+    passes the null stream everywhere); 0 restores the null stream."""
+    call("docc_rocm_set_default_stream", stream)
+
+
+class Graph:
+    """A recorded run of runtime calls (kernels, device copies, cached allocations) that replays with one submission.
+
+        stream = runtime.stream_create()
+        runtime.set_default_stream(stream); f(); runtime.stream_sync(stream)   # once, outside the record
+        with runtime.Graph.capture(stream) as graph:
+            f()                           # recorded, not run
+        graph.launch(); runtime.stream_sync(stream)
+
+    The device blocks `f` allocates while it is recorded belong to the graph until destroy(); the buffers it reads and
+    writes must stay where they are. launch() without a stream replays on the stream of the capture."""
+
+    def __init__(self, stream: int):
+        self.stream = stream
+        self.handle = None
+
+    class _Capture:
+        def __init__(self, graph: "Graph"):
+            self.graph = graph
+
+        def __enter__(self) -> "Graph":
+            call("docc_rocm_graph_capture_begin", self.graph.stream)
+            return self.graph
+
+        def __exit__(self, kind, value, trace) -> bool:
+            h = _vp()
+            code = lib().docc_rocm_graph_capture_end(ctypes.byref(h))
+            if kind is None:
+                failed, message = take_failure()    # a failing call in generated code ends that function early
+                if code != 0:
+                    raise RocmRuntimeError("docc_rocm_graph_capture_end", code, last_error())
+                self.graph.handle = h.value
+                if failed != 0:
+                    self.graph.destroy()
+                    raise RocmRuntimeError("graph capture", failed, message)
+            elif code == 0 and h.value:
+                lib().docc_rocm_graph_destroy(h.value)
+            return False
+
+    @classmethod
+    def capture(cls, stream: int) -> "Graph._Capture":
+        return cls._Capture(cls(stream))
+
+    def launch(self, stream: Optional[int] = None) -> None:
+        if not self.handle:
+            raise RuntimeError("the graph holds no record")
+        call("docc_rocm_graph_launch", self.handle, self.stream if stream is None else stream)
+
+    def destroy(self) -> None:
+        if self.handle:
+            handle, self.handle = self.handle, None
+            call("docc_rocm_graph_destroy", handle)
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().docc_rocm_graph_destroy(self.handle)
+        except Exception:
+            pass
 
 
 def convert_f32_to_bf16(count, src, dst, stream=0) -> None:

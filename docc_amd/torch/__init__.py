@@ -713,10 +713,8 @@ class _CompiledTorch:
         self.func.restype = None
         self.inputs, self.outputs, self.gm, self.on_device = inputs, outputs, gm, on_device
 
-    def __call__(self, *args):
-        import torch
-
-        device = torch.device("cuda", torch.cuda.current_device()) if self.on_device else torch.device("cpu")
+    def _operands(self, args, device):
+        """The tensors the generated function reads (kept alive by the caller) and their addresses."""
         keep, ptrs = [], []
         for name, (kind, ref) in self.inputs:
             if kind == "arg":
@@ -731,6 +729,47 @@ class _CompiledTorch:
             t = t.contiguous()
             keep.append(t)
             ptrs.append(t.data_ptr())
+        return keep, ptrs
+
+    def record(self, *args) -> "RecordedCall":
+        """Runs the function once on a stream of its own, records a second run there as a HIP graph and returns the
+        record: replay() repeats the whole function - every kernel of it - with one submission, reading the same
+        input tensors (fill them in place, with copy_) and writing the same result tensors."""
+        import torch
+
+        if not self.on_device:
+            raise ValueError("only a program compiled for device tensors can be recorded: its host variant waits for copies")
+        device = torch.device("cuda", torch.cuda.current_device())
+        keep, ptrs = self._operands(args, device)
+        outs = [torch.empty(shape, dtype=dtype, device=device) for _, shape, dtype in self.outputs]
+        runtime.init(device.index or 0)
+        torch.cuda.synchronize()
+        stream = runtime.stream_create()
+        runtime.set_default_stream(stream)
+        try:
+            for recording in (False, True):
+                if recording:
+                    with runtime.Graph.capture(stream) as graph:
+                        self.func(*ptrs, *[o.data_ptr() for o in outs])
+                else:
+                    # outside the record: kernel images load, per-stream buffers come into being
+                    self.func(*ptrs, *[o.data_ptr() for o in outs])
+                    code, message = runtime.take_failure()
+                    if code != 0:
+                        raise runtime.RocmRuntimeError(self.sdfg.name, code, message)
+                    runtime.stream_sync(stream)
+        except Exception:
+            runtime.set_default_stream(0)
+            runtime.stream_destroy(stream)
+            raise
+        runtime.set_default_stream(0)
+        return RecordedCall(graph, stream, keep, outs)
+
+    def __call__(self, *args):
+        import torch
+
+        device = torch.device("cuda", torch.cuda.current_device()) if self.on_device else torch.device("cpu")
+        keep, ptrs = self._operands(args, device)
         # results for CPU callers of 1 MiB and more are pinned (torch caches such blocks): the device-to-host copy runs
         # at link speed instead of through the driver's staging of pageable memory
         pin = lambda shape, dtype: (not self.on_device and torch.cuda.is_available() and
@@ -748,6 +787,43 @@ class _CompiledTorch:
         if self.on_device and torch.cuda.current_stream() != torch.cuda.default_stream():
             torch.cuda.default_stream().synchronize()
         return outs[0] if len(outs) == 1 else tuple(outs)
+
+
+class RecordedCall:
+    """One call of a compiled program on device tensors, recorded as a HIP graph (see _CompiledTorch.record).
+
+    inputs: the tensors the record reads, in the order of the function's operands; outputs: the tensors it writes.
+    replay() enqueues one run on the record's own stream and, unless wait=False, waits for it; torch's streams do
+    not order themselves against that stream, so synchronize torch's work on the inputs before a replay and call
+    wait() before reading the outputs of a replay(wait=False)."""
+
+    def __init__(self, graph, stream, inputs, outputs):
+        self.graph, self.stream, self.inputs, self.outputs = graph, stream, inputs, outputs
+
+    @property
+    def result(self):
+        return self.outputs[0] if len(self.outputs) == 1 else tuple(self.outputs)
+
+    def replay(self, wait: bool = True):
+        self.graph.launch()
+        if wait:
+            runtime.stream_sync(self.stream)
+        return self.result
+
+    def wait(self) -> None:
+        runtime.stream_sync(self.stream)
+
+    def close(self) -> None:
+        if self.graph is not None:
+            self.graph.destroy()
+            runtime.stream_destroy(self.stream)
+            self.graph = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class TorchProgram(DoccProgram):
@@ -862,6 +938,10 @@ class TorchProgram(DoccProgram):
     def __call__(self, *args: Any) -> Any:
         compiled = self.compile(*args)
         return self._convert_outputs(compiled(*self._convert_inputs(args)), args)
+
+    def record(self, *args: Any) -> RecordedCall:
+        """Compiles for `args` (device tensors) and records one call on them as a HIP graph."""
+        return self.compile(*args).record(*args)
 
     def _convert_inputs(self, args: tuple) -> tuple:
         return args

@@ -108,7 +108,7 @@ int docc_rocm_memcpy_d2d_async(void* dst_dev, const void* src_dev, size_t bytes,
 /* Streams (default priority only). docc_rocm_stream_destroy also releases the 8 MiB of partial results that
  * the two-launch kernels (sliced softmax, column reductions, column matrix-vector products, dot) keep per
  * stream; they allocate it with hipMalloc on their first call on a stream, so that first call waits for the
- * device and cannot be captured into a HIP graph. */
+ * device: run a function once on a stream before capturing it there. */
 int docc_rocm_stream_create(docc_rocm_stream_t* stream);
 int docc_rocm_stream_destroy(docc_rocm_stream_t stream);
 int docc_rocm_stream_sync(docc_rocm_stream_t stream);
@@ -127,6 +127,40 @@ int docc_rocm_event_create(docc_rocm_event_t* event);
 int docc_rocm_event_destroy(docc_rocm_event_t event);
 int docc_rocm_event_record(docc_rocm_event_t event, docc_rocm_stream_t stream);
 int docc_rocm_event_elapsed_ms(docc_rocm_event_t start, docc_rocm_event_t stop, float* ms);
+
+/*
+ * Graph capture of generated code. A compiled function is a fixed chain of launches, copies and (cached)
+ * allocations on the null stream; a caller that runs it many times on the same buffers records it once and replays
+ * the record, which costs one submission instead of one per kernel. No counterpart in the reference: its CUDA
+ * target launches kernel by kernel and synchronizes after each (reference
+ * opt/src/targets/cuda/codegen/cuda_map_dispatcher.cpp:236-262).
+ *
+ * docc_rocm_set_default_stream names, for the calling thread, the stream that stands in wherever generated code or
+ * a caller passes the null stream to this library (kernels, copies, allocations, docc_rocm_stream_sync); null
+ * restores the null stream. docc_rocm_graph_capture_begin waits for the device, starts a relaxed-mode capture on
+ * `stream` (not null) and makes it the thread's default stream; every call of this library on that thread up to
+ * docc_rocm_graph_capture_end is recorded instead of run. During a capture
+ *   - docc_rocm_malloc[_async] hands out blocks that then belong to the graph (every replay uses those addresses);
+ *     docc_rocm_free[_async] returns them to the capture, which serves its own later allocations from them, and
+ *     neither waits for anything. The blocks go back to the block cache in docc_rocm_graph_destroy;
+ *   - calls that hand a result to the host refuse (docc_rocm_dot) or end the capture with an error from HIP
+ *     (docc_rocm_stream_sync, docc_rocm_device_sync, docc_rocm_event_elapsed_ms): a function that copies results
+ *     to host memory and waits for them is captured up to that wait at most. Capture functions whose arguments
+ *     stay on the device;
+ *   - copies from or to host memory need pinned memory (docc_rocm_host_malloc) and are replayed from / to the
+ *     same addresses.
+ * Run the function once on `stream` (docc_rocm_set_default_stream) before capturing it, so that kernel images
+ * are loaded and the per-stream partial results exist. Kernels that keep partial results (see Streams above)
+ * record the capture stream's buffer: replay on that stream, or keep it idle while a replay runs elsewhere.
+ * docc_rocm_graph_launch enqueues one replay on `stream` (null: the thread's default). docc_rocm_graph_destroy
+ * waits for the device. The library records no memset nodes.
+ */
+typedef void* docc_rocm_graph_t;
+int docc_rocm_set_default_stream(docc_rocm_stream_t stream);
+int docc_rocm_graph_capture_begin(docc_rocm_stream_t stream);
+int docc_rocm_graph_capture_end(docc_rocm_graph_t* graph);
+int docc_rocm_graph_launch(docc_rocm_graph_t graph, docc_rocm_stream_t stream);
+int docc_rocm_graph_destroy(docc_rocm_graph_t graph);
 
 /*
  * Failure channel of generated code. The generated `extern "C"` functions have
