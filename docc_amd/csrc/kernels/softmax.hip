@@ -6,7 +6,9 @@
 // Max -> Broadcast -> Sub -> Exp -> Sum -> Broadcast -> Div with six
 // temporaries) by one kernel that reads X once and writes Y once.
 //
-// HBM-bound: algorithmic traffic is 8 bytes per element. Three shapes:
+// HBM-bound: algorithmic traffic is 8 bytes per element. The shapes of the fp32 row kernels:
+//   rows sharing a wavefront (cols <= 128, cols % 4 == 0): 1 to 32 lanes a row, 64 to 2 rows per
+//       wavefront and four such sets per wavefront, butterflies inside the lanes of a row;
 //   wave-per-row  (cols <= 1024, cols % 4 == 0; built up to 4096): a 64-lane wavefront
 //       holds the whole row in registers (NV float4 per lane, 128-bit coalesced loads),
 //       reduces max and sum with wave shuffles only - no LDS, no barrier;
@@ -14,8 +16,13 @@
 //       partial results cross the four waves through LDS; ahead of the wavefront
 //       per row from 2048 columns on (more rows in flight per register); rows of
 //       2049..4096 columns use 512 threads (two vectors per lane), the others 256;
-//   streaming     (any cols): per-lane online max/sum over the row, then a
-//       second read (served by L2 / Infinity Cache) to write the result.
+//       rows of up to 65536 columns 1024 threads, where there are rows enough for half the CUs;
+//   block-per-row for rows that start off a 16-byte boundary (any cols from 256 on): single
+//       elements up to the first boundary and after the last, vectors between;
+//   rows cut into slices (longer rows, or too few of them): two launches around one
+//       (maximum, sum) pair per slice, the second reading the slice again (12 bytes per element);
+//   streaming     (what is left: operands placed unequally, short ragged rows): per-lane
+//       online max/sum over the row, then a second read to write the result.
 #include "common.h"
 
 using namespace docc_k;
@@ -144,7 +151,76 @@ __device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, l
     }
 }
 
+// The work-group per row for rows that do not start on a 16-byte boundary (cols not a multiple of four, or operands
+// placed off it): up to three single elements, the vectors between the first and the last boundary, up to three single
+// elements; a lane holds NV vectors of the middle part and at most one of the single elements. X and Y must be placed
+// equally relative to 16 bytes, so that a row's boundaries are the same in both.
+template <int NV, int NW>
+__device__ __forceinline__ void softmax_block_any_kernel(const float* X, float* Y, long rows, int cols) {
+    constexpr int NT = NW * kWave;
+    __shared__ float lds[NW];
+    const long row = blockIdx.x;
+    const float* x = X + row * (long) cols;
+    float* y = Y + row * (long) cols;
+    const int mis = (int) ((reinterpret_cast<uintptr_t>(x) >> 2) & 3);
+    int head = mis ? 4 - mis : 0;
+    if (head > cols) head = cols;
+    const int nvec = (cols - head) >> 2;
+    const int tail0 = head + nvec * 4;
+    const int t = threadIdx.x;
+    const int edge = t < head ? t : (t - head < cols - tail0 ? tail0 + t - head : -1);   // this lane's single element, if any
+    float e = edge >= 0 ? x[edge] : kNegInf;
+    const f32x4* xv = reinterpret_cast<const f32x4*>(x + head);
+    f32x4* yv = reinterpret_cast<f32x4*>(y + head);
+    f32x4 v[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        int c = t + i * NT;
+        if (c < nvec) {
+            v[i] = __builtin_nontemporal_load(xv + c);
+        } else {
+            v[i] = f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+        }
+    }
+    float m = e;
+#pragma unroll
+    for (int i = 0; i < NV; i++) m = fmaxf(fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)), m);
+    m = block_max<NW>(m, lds);
+    e = exp_neg(e - m);
+    float s = edge >= 0 ? e : 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        v[i].x = exp_neg(v[i].x - m);
+        v[i].y = exp_neg(v[i].y - m);
+        v[i].z = exp_neg(v[i].z - m);
+        v[i].w = exp_neg(v[i].w - m);
+        if (t + i * NT < nvec) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);   // a vector past the row's end is NaN when the whole row is -inf
+    }
+    s = block_sum<NW>(s, lds);
+    const float inv = 1.0f / s;
+    if (edge >= 0) y[edge] = e * inv;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        int c = t + i * NT;
+        if (c < nvec) {
+            f32x4 o = v[i] * inv;
+            __builtin_nontemporal_store(o, yv + c);
+        }
+    }
+}
+
 } // namespace
+
+#define DOCC_SOFTMAX_BLOCK_ANY(NV, NW)                                                                                  \
+    extern "C" __global__ __launch_bounds__(NW * 64) void docc_softmax_f32_any##NW##_v##NV(const float* X, float* Y,    \
+                                                                                           long rows, int cols) {       \
+        softmax_block_any_kernel<NV, NW>(X, Y, rows, cols);                                                             \
+    }
+DOCC_SOFTMAX_BLOCK_ANY(1, 4)
+DOCC_SOFTMAX_BLOCK_ANY(4, 4)
+DOCC_SOFTMAX_BLOCK_ANY(16, 4)
+DOCC_SOFTMAX_BLOCK_ANY(8, 16)
+DOCC_SOFTMAX_BLOCK_ANY(16, 16)
 
 #define DOCC_SOFTMAX_WAVE(NV)                                                                             \
     extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_wave_v##NV(const float* X, float* Y, \
@@ -174,6 +250,70 @@ DOCC_SOFTMAX_BLOCK(2)
 DOCC_SOFTMAX_BLOCK(4)
 DOCC_SOFTMAX_BLOCK(8)
 DOCC_SOFTMAX_BLOCK(16)
+// sixteen wavefronts per row: rows of up to 65536 columns stay in registers (one read, one write), for tensors with
+// enough rows to give every CU one
+#define DOCC_SOFTMAX_BLOCK16(NV)                                                                             \
+    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_f32_block16_v##NV(const float* X, float* Y, \
+                                                                                      long rows, int cols) {  \
+        softmax_block_kernel<NV, 16>(X, Y, rows, cols);                                                      \
+    }
+DOCC_SOFTMAX_BLOCK16(8)
+DOCC_SOFTMAX_BLOCK16(16)
+
+// Rows of at most 128 columns: LPR lanes of a wavefront share a row (one vector each, cols <= 4 * LPR), so a
+// wavefront holds 64 / LPR rows at a time and four such sets in turn, all loaded before the first is reduced; the
+// reductions are butterflies inside the LPR lanes. A wavefront per row would leave 32 of its 64 lanes (128 columns)
+// to 63 of them (4 columns) idle.
+namespace {
+template <int LPR>
+__device__ __forceinline__ void softmax_subwave_kernel(const float* X, float* Y, long rows, int cols) {
+    constexpr int RPW = kWave / LPR;   // rows of a wavefront per set
+    constexpr int SETS = 4;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int l = lane % LPR, g = lane / LPR;
+    const int nvec = cols >> 2;
+    const long first = ((long) blockIdx.x * (256 / kWave) + threadIdx.x / kWave) * (RPW * SETS) + g;
+    const f32x4* xv = reinterpret_cast<const f32x4*>(X);
+    f32x4* yv = reinterpret_cast<f32x4*>(Y);
+    f32x4 v[SETS];
+    bool live[SETS];
+#pragma unroll
+    for (int i = 0; i < SETS; i++) {
+        const long row = first + (long) i * RPW;
+        live[i] = row < rows && l < nvec;
+        v[i] = live[i] ? __builtin_nontemporal_load(xv + row * nvec + l) : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+    }
+#pragma unroll
+    for (int i = 0; i < SETS; i++) {
+        float m = fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w));
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+        v[i].x = exp_neg(v[i].x - m);
+        v[i].y = exp_neg(v[i].y - m);
+        v[i].z = exp_neg(v[i].z - m);
+        v[i].w = exp_neg(v[i].w - m);
+        float s = (v[i].x + v[i].y) + (v[i].z + v[i].w);
+        if (!(l < nvec)) s = 0.f;   // a lane past the row's end holds -inf, which is NaN after the subtraction when the whole row is -inf
+#pragma unroll
+        for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
+        const float inv = 1.0f / s;
+        if (live[i]) {
+            f32x4 out = v[i] * inv;
+            __builtin_nontemporal_store(out, yv + (first + (long) i * RPW) * nvec + l);
+        }
+    }
+}
+} // namespace
+#define DOCC_SOFTMAX_SUB(LPR)                                                                                                  \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_sub##LPR(const float* X, float* Y, long rows, int cols) { \
+        softmax_subwave_kernel<LPR>(X, Y, rows, cols);                                                                         \
+    }
+DOCC_SOFTMAX_SUB(1)
+DOCC_SOFTMAX_SUB(2)
+DOCC_SOFTMAX_SUB(4)
+DOCC_SOFTMAX_SUB(8)
+DOCC_SOFTMAX_SUB(16)
+DOCC_SOFTMAX_SUB(32)
 
 // Any cols, any alignment: one 256-thread block per row. Pass 1 keeps a
 // per-thread running (max, sum) pair that is rescaled whenever the max moves
@@ -412,7 +552,172 @@ __device__ __forceinline__ void softmax_sliced_finish(const void* partials, cons
     for (long r = w.r0 + part; r < w.r1; r += 4) y[r * inner] = M::exp_le0(x[r * inner] - gm) / gs;
 }
 
+// Rows cut into slices (inner == 1): rows longer than a work-group's registers hold, or too few of them to give every
+// CU one. Work-group (row, slice) first leaves the (maximum, sum) pair of its `per` columns in the launcher's buffer,
+// then - in a second launch - merges the pairs of its row and writes its own columns. Both launches read with 16-byte
+// vectors wherever the row's address allows it: a row may start anywhere (cols need not be a multiple of the vector),
+// so each slice is walked as a head of single elements up to the first 16-byte boundary, a body of vectors and a tail.
+// X and Y must be equally placed relative to 16 bytes for the vector form (`vec`), else every access is one element.
+
+template <typename T> struct RowVec;
+template <> struct RowVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+template <> struct RowVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
+
+// the running pair after the elements of one vector: one rescaling per vector instead of one per element
+template <typename T>
+__device__ __forceinline__ void online_vector(typename RowVec<T>::type v, T& m, T& s) {
+    using M = SoftmaxMath<T>;
+    T cm = v[0];
+#pragma unroll
+    for (int i = 1; i < RowVec<T>::N; i++) cm = M::max(cm, v[i]);   // NaN elements do not move the maximum
+    const T nm = M::max(m, cm);
+    if (nm != m) {            // m == -inf: s is 0 (or NaN) and exp(-inf) is 0
+        s = s * M::exp_le0(m - nm);
+        m = nm;
+    }
+#pragma unroll
+    for (int i = 0; i < RowVec<T>::N; i++) s += (v[i] == M::neg_inf()) ? (T) 0 : M::exp_le0(v[i] - m);   // -inf weighs nothing; NaN poisons s
+}
+
+struct RowSlice {
+    long c0, c1;          // columns [c0, c1) of the row
+    long head, nvec;      // single elements before the vector body, vectors of the body
+};
+
+template <typename T>
+__device__ __forceinline__ RowSlice row_slice(const T* x, long cols, long per, long slice, int vec) {
+    RowSlice r;
+    r.c0 = slice * per;
+    r.c1 = r.c0 + per < cols ? r.c0 + per : cols;
+    constexpr int N = RowVec<T>::N;
+    if (vec) {
+        const long mis = (long) ((reinterpret_cast<uintptr_t>(x + r.c0) / sizeof(T)) & (N - 1));
+        r.head = mis ? N - mis : 0;
+        if (r.head > r.c1 - r.c0) r.head = r.c1 - r.c0;
+        r.nvec = (r.c1 - r.c0 - r.head) / N;
+    } else {
+        r.head = r.c1 - r.c0;
+        r.nvec = 0;
+    }
+    return r;
+}
+
+// tree over the 256 pairs of a work-group; the result is in lm[0], ls[0]
+template <typename T>
+__device__ __forceinline__ void merge_block_pairs(T m, T s, T* lm, T* ls) {
+    using M = SoftmaxMath<T>;
+    lm[threadIdx.x] = m;
+    ls[threadIdx.x] = s;
+    __syncthreads();
+    for (int half = 128; half > 0; half >>= 1) {
+        if ((int) threadIdx.x < half) {
+            const T m2 = lm[threadIdx.x + half], s2 = ls[threadIdx.x + half];
+            const T m1 = lm[threadIdx.x], s1 = ls[threadIdx.x];
+            const T g = M::max(m1, m2);
+            lm[threadIdx.x] = g;
+            ls[threadIdx.x] = pair_weight(m1, s1, g) + pair_weight(m2, s2, g);
+        }
+        __syncthreads();
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void softmax_rowslice_partial(void* partials, const T* X, long cols, long per, int slices, int vec) {
+    using M = SoftmaxMath<T>;
+    using V = typename RowVec<T>::type;
+    constexpr int N = RowVec<T>::N;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const long row = blockIdx.x / slices, slice = blockIdx.x % slices;
+    const T* x = X + row * cols;
+    const RowSlice r = row_slice(x, cols, per, slice, vec);
+    T m = M::neg_inf(), s = (T) 0;
+    // head and tail: at most N - 1 elements each in the vector form, the whole slice otherwise
+    for (long c = r.c0 + threadIdx.x; c < r.c0 + r.head; c += 256) online_step(x[c], m, s);
+    const V* xv = reinterpret_cast<const V*>(x + r.c0 + r.head);
+    long i = threadIdx.x;
+    for (; i + 768 < r.nvec; i += 1024) {   // four loads in flight per lane; ordinary loads: the second launch reads the slice again
+        const V v0 = xv[i], v1 = xv[i + 256], v2 = xv[i + 512], v3 = xv[i + 768];
+        online_vector<T>(v0, m, s);
+        online_vector<T>(v1, m, s);
+        online_vector<T>(v2, m, s);
+        online_vector<T>(v3, m, s);
+    }
+    for (; i < r.nvec; i += 256) online_vector<T>(xv[i], m, s);
+    for (long c = r.c0 + r.head + r.nvec * N + threadIdx.x; c < r.c1; c += 256) online_step(x[c], m, s);
+    merge_block_pairs(m, s, lm, ls);
+    if (threadIdx.x == 0) {
+        T* P = reinterpret_cast<T*>(partials);
+        P[blockIdx.x * 2] = lm[0];
+        P[blockIdx.x * 2 + 1] = ls[0];
+    }
+}
+
+template <typename T> __device__ __forceinline__ T softmax_scale(T gs);
+template <> __device__ __forceinline__ float softmax_scale<float>(float gs) { return 1.0f / gs; }   // one division per row, then multiplies
+template <> __device__ __forceinline__ double softmax_scale<double>(double gs) { return gs; }
+__device__ __forceinline__ float softmax_result(float e, float scale) { return e * scale; }
+__device__ __forceinline__ double softmax_result(double e, double scale) { return e / scale; }
+
+template <typename T>
+__device__ __forceinline__ void softmax_rowslice_finish(const void* partials, const T* X, T* Y, long cols, long per, int slices, int vec) {
+    using M = SoftmaxMath<T>;
+    using V = typename RowVec<T>::type;
+    constexpr int N = RowVec<T>::N;
+    __shared__ T lm[256];
+    __shared__ T ls[256];
+    const long row = blockIdx.x / slices, slice = blockIdx.x % slices;
+    const T* P = reinterpret_cast<const T*>(partials) + row * slices * 2;
+    T m = M::neg_inf(), s = (T) 0;
+    for (int sl = threadIdx.x; sl < slices; sl += 256) {
+        const T pm = P[sl * 2], ps = P[sl * 2 + 1];
+        const T g = M::max(m, pm);
+        s = pair_weight(m, s, g) + pair_weight(pm, ps, g);
+        m = g;
+    }
+    merge_block_pairs(m, s, lm, ls);
+    const T gm = lm[0];
+    const T scale = softmax_scale<T>(ls[0] + (gm - gm));   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
+    const T* x = X + row * cols;
+    T* y = Y + row * cols;
+    const RowSlice r = row_slice(x, cols, per, slice, vec);
+    for (long c = r.c0 + threadIdx.x; c < r.c0 + r.head; c += 256) y[c] = softmax_result(M::exp_le0(x[c] - gm), scale);
+    const V* xv = reinterpret_cast<const V*>(x + r.c0 + r.head);
+    V* yv = reinterpret_cast<V*>(y + r.c0 + r.head);
+    long i = threadIdx.x;
+    for (; i + 768 < r.nvec; i += 1024) {
+        V v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = __builtin_nontemporal_load(xv + i + 256 * j);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int e = 0; e < N; e++) v[j][e] = softmax_result(M::exp_le0(v[j][e] - gm), scale);
+            __builtin_nontemporal_store(v[j], yv + i + 256 * j);
+        }
+    }
+    for (; i < r.nvec; i += 256) {
+        V v = __builtin_nontemporal_load(xv + i);
+#pragma unroll
+        for (int e = 0; e < N; e++) v[e] = softmax_result(M::exp_le0(v[e] - gm), scale);
+        __builtin_nontemporal_store(v, yv + i);
+    }
+    for (long c = r.c0 + r.head + r.nvec * N + threadIdx.x; c < r.c1; c += 256) y[c] = softmax_result(M::exp_le0(x[c] - gm), scale);
+}
+
 } // namespace
+
+#define DOCC_SOFTMAX_ROWSLICE(T, SUFFIX)                                                                                           \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_rowslice_partial(void* partials, const T* X, long cols, \
+                                                                                              long per, int slices, int vec) {      \
+        softmax_rowslice_partial<T>(partials, X, cols, per, slices, vec);                                                          \
+    }                                                                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_rowslice_finish(const void* partials, const T* X, T* Y, \
+                                                                                             long cols, long per, int slices, int vec) { \
+        softmax_rowslice_finish<T>(partials, X, Y, cols, per, slices, vec);                                                        \
+    }
+DOCC_SOFTMAX_ROWSLICE(float, f32)
+DOCC_SOFTMAX_ROWSLICE(double, f64)
 
 #define DOCC_SOFTMAX_SLICED(T, SUFFIX)                                                                                        \
     extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_partial(void* partials, const T* X, long reduce, \

@@ -30,6 +30,7 @@ namespace docc::rt::rocm {
 int64_t softmax_slices(int precision, int64_t outer, int64_t reduce, int64_t inner, int cus, int64_t capacity);
 int softmax_general(hipStream_t s, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y, void* partials);
 int softmax_check(int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, const void* Y);
+int64_t softmax_row_slices(int precision, int64_t rows, int64_t cols, bool in_registers, int cus, int64_t capacity, int64_t* per);
 
 // Part of a device's set-up (docc_rocm_init, or the first launcher call on the device), with that device
 // current: asks for the address of the array on this device and resolves the kernels the entry point
@@ -49,7 +50,11 @@ int noalloc_setup_device(int dev) {
         "docc_softmax_f64_sliced_finish",  "docc_softmax_f32_wave_v1",       "docc_softmax_f32_wave_v2",       "docc_softmax_f32_wave_v4",
         "docc_softmax_f32_wave_v8",        "docc_softmax_f32_wave_v16",      "docc_softmax_f32_block8_v2",     "docc_softmax_f32_block_v1",
         "docc_softmax_f32_block_v2",       "docc_softmax_f32_block_v4",      "docc_softmax_f32_block_v8",      "docc_softmax_f32_block_v16",
-        "docc_softmax_f32_stream",
+        "docc_softmax_f32_stream",         "docc_softmax_f32_block16_v8",    "docc_softmax_f32_block16_v16",   "docc_softmax_f32_sub1",
+        "docc_softmax_f32_sub2",           "docc_softmax_f32_sub4",          "docc_softmax_f32_sub8",          "docc_softmax_f32_sub16",
+        "docc_softmax_f32_sub32",          "docc_softmax_f32_rowslice_partial", "docc_softmax_f64_rowslice_partial",
+        "docc_softmax_f32_rowslice_finish", "docc_softmax_f64_rowslice_finish", "docc_softmax_f32_any4_v1",      "docc_softmax_f32_any4_v4",
+        "docc_softmax_f32_any4_v16",       "docc_softmax_f32_any16_v8",      "docc_softmax_f32_any16_v16",
     };
     for (const char* name : kernels) {
         hipFunction_t fn;
@@ -73,8 +78,17 @@ extern "C" int docc_rocm_softmax_noalloc(docc_rocm_stream_t stream, int precisio
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT,
                     "softmax_noalloc: device %d has not been set up; call docc_rocm_init(%d) first (this entry point loads and allocates nothing)",
                     dev, dev);
-    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
-    if (inner != 1 && !(inner <= 32 && (inner & (inner - 1)) == 0)) {
+    if (inner == 1) {
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        // rows cut into slices leave one (maximum, sum) pair per row and slice
+        const int64_t need = softmax_row_slices(precision, outer, reduce, false, cus, (int64_t) kPartialsBytes, nullptr) * outer * 2 * (precision / 8);
+        if (need > (int64_t) kScratchBytes)
+            return fail(DOCC_ROCM_ERR_UNSUPPORTED,
+                        "softmax_noalloc: this shape needs %lld bytes of partial results, the entry point holds %lld; use docc_rocm_softmax or "
+                        "docc_rocm_softmax_ws",
+                        (long long) need, (long long) kScratchBytes);
+    } else if (!(inner <= 32 && (inner & (inner - 1)) == 0)) {
         int cus = compute_units();
         if (cus <= 0) cus = 256;
         // the slices docc_rocm_softmax would cut the rows into, and the bytes their (maximum, sum) pairs take

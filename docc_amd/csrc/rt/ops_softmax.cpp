@@ -7,20 +7,85 @@
 
 using namespace docc::rt::rocm;
 
-extern "C" {
+namespace docc::rt::rocm {
 
-int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols, const float* X, float* Y) {
-    if (rows < 0 || cols < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
-    if (rows == 0 || cols == 0) return 0;
-    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
+// Slices of the row-sliced form of a softmax over the rows of [rows, cols] (two launches around (maximum, sum) pairs,
+// rows * slices * 2 elements of them), 0 where a one-launch kernel serves; *per = columns of a slice. Rows that a
+// work-group's registers hold (16384 columns; 65536 with sixteen wavefronts, `in_registers`, where there are rows
+// enough to occupy half the CUs that way) stay with the one-launch kernels; longer rows, or rows too few to fill the
+// device one work-group each, are cut so that about eight work-groups per CU share the tensor, no slice shorter
+// than 4096 columns.
+int64_t softmax_row_slices(int precision, int64_t rows, int64_t cols, bool in_registers, int cus, int64_t capacity, int64_t* per) {
+    if (precision == 32) {
+        if (cols <= 16384) return 0;
+        if (in_registers && cols <= 65536 && rows >= cus / 2) return 0;
+    } else {
+        if (cols < 8192 || (rows >= 2 * (int64_t) cus && cols <= 65536)) return 0;
+    }
+    int64_t slices = (8 * (int64_t) cus + rows - 1) / rows;
+    if (slices > cols / 4096) slices = cols / 4096;
+    if (slices > 1024) slices = 1024;
+    if (slices < 1) slices = 1;
+    const int64_t width = ((cols + slices - 1) / slices + 1023) / 1024 * 1024;
+    slices = (cols + width - 1) / width;
+    if (rows > 0x7fffffffLL / slices) return 0;
+    if (rows * slices * 2 * (precision / 8) > capacity) return 0;
+    if (per) *per = width;
+    return slices;
+}
+
+namespace {
+int softmax_rowsliced(hipStream_t s, int precision, int64_t rows, int64_t cols, int64_t slices, int64_t per, const void* X, void* Y, void* partials) {
+    PartialsLease lease;
+    if (!partials) {
+        if (int rc = partials_for(s, &lease)) return rc;
+        partials = lease.ptr;
+    }
+    const size_t elem = (size_t) precision / 8;
+    const int vec = ((uintptr_t) X % elem == 0) && ((uintptr_t) Y % elem == 0) && ((uintptr_t) X % 16 == (uintptr_t) Y % 16);
+    const char* t = precision == 32 ? "f32" : "f64";
+    char name[64];
+    std::snprintf(name, sizeof(name), "docc_softmax_%s_rowslice_partial", t);
+    if (int rc = launch(name, (uint32_t) (rows * slices), 1, 1, 256, 0, s, partials, X, (long) cols, (long) per, (int) slices, vec)) return rc;
+    std::snprintf(name, sizeof(name), "docc_softmax_%s_rowslice_finish", t);
+    return launch(name, (uint32_t) (rows * slices), 1, 1, 256, 0, s, (const void*) partials, X, Y, (long) cols, (long) per, (int) slices, vec);
+}
+} // namespace
+
+// The fp32 row softmax; `partials` as for softmax_general.
+int softmax_rows_f32(hipStream_t s, int64_t rows, int64_t cols, const float* X, float* Y, void* partials) {
     if (rows > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
-    hipStream_t s = (hipStream_t) stream;
     const bool vec_ok = (cols % 4 == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
+    // rows that start off a 16-byte boundary are still read in vectors when they start equally far off it in X and Y
+    const bool same_place = (((uintptr_t) X | (uintptr_t) Y) % 4 == 0) && ((uintptr_t) X % 16 == (uintptr_t) Y % 16);
+    if (cols > 16384) {
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        int64_t per = 0;
+        const int64_t slices = softmax_row_slices(32, rows, cols, vec_ok || same_place, cus, (int64_t) kPartialsBytes, &per);
+        if (slices > 0) return softmax_rowsliced(s, 32, rows, cols, slices, per, X, Y, partials);
+        if (vec_ok && cols <= 65536)
+            return launch(cols <= 32768 ? "docc_softmax_f32_block16_v8" : "docc_softmax_f32_block16_v16", (uint32_t) rows, 1, 1, 1024, 0, s, X, Y,
+                          (long) rows, (int) cols);
+        if (same_place && cols <= 65536)
+            return launch(cols <= 32768 ? "docc_softmax_f32_any16_v8" : "docc_softmax_f32_any16_v16", (uint32_t) rows, 1, 1, 1024, 0, s, X, Y,
+                          (long) rows, (int) cols);
+        return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+    }
     // Up to 1024 columns one wavefront per row moves the most bytes (6.1-6.4 TB/s measured against 2.6-5.6
     // for a work-group per row); from 2048 columns on the work-group per row is ahead (6.1-6.3 against
     // 5.8-6.0 TB/s). DOCC_ROCM_SOFTMAX=wave|block overrides the choice (tuning; block = four wavefronts per row).
     const char* force = std::getenv("DOCC_ROCM_SOFTMAX");
     const bool wave = force && force[0] == 'w' ? true : force && force[0] == 'b' ? false : cols <= 1024;
+    if (vec_ok && cols <= 128 && !force) {
+        // several rows per wavefront: LPR lanes a row, four sets of 64 / LPR rows per wavefront, four wavefronts
+        int lpr = 1;
+        while (4 * lpr < cols) lpr *= 2;
+        char name[48];
+        std::snprintf(name, sizeof(name), "docc_softmax_f32_sub%d", lpr);
+        const int64_t rows_per_group = 4 * 4 * (64 / lpr);
+        return launch(name, (uint32_t) ((rows + rows_per_group - 1) / rows_per_group), 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
+    }
     if (vec_ok && cols <= 4096 && wave) {
         // one wavefront per row, 4 rows per 256-thread block
         const char* name = cols <= 256    ? "docc_softmax_f32_wave_v1"
@@ -34,7 +99,7 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
     if (vec_ok && cols > 2048 && cols <= 4096 && !(force && force[0] == 'b'))
         // eight wavefronts per row, two vectors per lane: 6.24 TB/s against 6.09 with four wavefronts at 4096 columns
         return launch("docc_softmax_f32_block8_v2", (uint32_t) rows, 1, 1, 512, 0, s, X, Y, (long) rows, (int) cols);
-    if (vec_ok && cols <= 16384) {
+    if (vec_ok) {
         const char* name = cols <= 1024   ? "docc_softmax_f32_block_v1"
                            : cols <= 2048 ? "docc_softmax_f32_block_v2"
                            : cols <= 4096 ? "docc_softmax_f32_block_v4"
@@ -42,7 +107,22 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
                                           : "docc_softmax_f32_block_v16";
         return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     }
+    if (same_place && cols >= 256 && !force)
+        return launch(cols <= 1024 ? "docc_softmax_f32_any4_v1" : cols <= 4096 ? "docc_softmax_f32_any4_v4" : "docc_softmax_f32_any4_v16", (uint32_t) rows,
+                      1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
     return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+}
+
+} // namespace docc::rt::rocm
+
+extern "C" {
+
+int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols, const float* X, float* Y) {
+    if (rows < 0 || cols < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: negative shape");
+    if (rows == 0 || cols == 0) return 0;
+    if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
+    if (int rc = ensure_device()) return rc;
+    return softmax_rows_f32((hipStream_t) stream, rows, cols, X, Y, nullptr);
 }
 
 } // extern "C"
@@ -70,7 +150,13 @@ int softmax_general(hipStream_t s, int precision, int64_t outer, int64_t reduce,
     const char* t = precision == 32 ? "f32" : "f64";
     char name[64];
     if (inner == 1) {
+        if (precision == 32) return softmax_rows_f32(s, outer, reduce, (const float*) X, (float*) Y, partials);
         if (outer > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        int64_t per = 0;
+        const int64_t slices = softmax_row_slices(64, outer, reduce, false, cus, (int64_t) kPartialsBytes, &per);
+        if (slices > 0) return softmax_rowsliced(s, 64, outer, reduce, slices, per, X, Y, partials);
         return launch("docc_softmax_f64_stream", (uint32_t) outer, 1, 1, 256, 0, s, X, Y, (long) outer, (long) reduce);
     }
     if (inner <= 32 && (inner & (inner - 1)) == 0) {
@@ -117,17 +203,18 @@ extern "C" {
 
 int docc_rocm_softmax(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y) {
     if (int rc = softmax_check(precision, outer, reduce, inner, X, Y)) return rc == 1 ? 0 : rc;
-    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
     if (int rc = ensure_device()) return rc;
     return softmax_general((hipStream_t) stream, precision, outer, reduce, inner, X, Y, nullptr);
 }
 
 int64_t docc_rocm_softmax_workspace_bytes(int precision, int64_t outer, int64_t reduce, int64_t inner) {
     if ((precision != 32 && precision != 64) || outer <= 0 || reduce <= 0 || inner <= 0) return 0;
-    if (inner == 1 || (inner <= 32 && (inner & (inner - 1)) == 0)) return 0;
+    if (inner != 1 && inner <= 32 && (inner & (inner - 1)) == 0) return 0;
     if (ensure_device()) return 0;
     int cus = compute_units();
     if (cus <= 0) cus = 256;
+    if (inner == 1)   // for any placement of the operands: rows that could stay in registers are cut when a pointer is not 16-byte aligned
+        return (softmax_row_slices(precision, outer, reduce, false, cus, (int64_t) kPartialsBytes, nullptr) * outer * 2 * (precision / 8) + 255) / 256 * 256;
     const int64_t slices = softmax_slices(precision, outer, reduce, inner, cus, (int64_t) kPartialsBytes);
     return (slices * outer * inner * 2 * (precision / 8) + 255) / 256 * 256;
 }
@@ -135,7 +222,6 @@ int64_t docc_rocm_softmax_workspace_bytes(int precision, int64_t outer, int64_t 
 int docc_rocm_softmax_ws(docc_rocm_stream_t stream, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y,
                          void* workspace, int64_t workspace_bytes) {
     if (int rc = softmax_check(precision, outer, reduce, inner, X, Y)) return rc == 1 ? 0 : rc;
-    if (inner == 1 && precision == 32) return docc_rocm_softmax_f32(stream, outer, reduce, (const float*) X, (float*) Y);
     if (int rc = ensure_device()) return rc;
     const int64_t need = docc_rocm_softmax_workspace_bytes(precision, outer, reduce, inner);
     if (need > 0 && (!workspace || workspace_bytes < need || ((uintptr_t) workspace % 256) != 0))

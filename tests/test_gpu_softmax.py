@@ -40,6 +40,119 @@ def test_softmax_matches_oracle(rt, rows, cols):
     np.testing.assert_allclose(Y.sum(axis=-1), 1.0, rtol=0, atol=1e-5)
 
 
+@pytest.mark.parametrize(
+    "rows,cols",
+    [(1000, 4), (999, 8), (77, 12), (513, 16), (130, 28), (4099, 32), (65, 60), (1025, 64), (300, 100), (259, 128)],
+)
+def test_softmax_rows_that_share_a_wavefront(rt, rows, cols):
+    """Up to 128 columns several rows share a wavefront (1 to 32 lanes a row, four sets of rows per wavefront): row counts
+    that end inside a set, inside a wavefront and inside a work-group, widths that fill the lanes of a row and that do not."""
+    rng = np.random.default_rng(rows * 1009 + cols)
+    X = (rng.standard_normal((rows, cols)) * 8).astype(np.float32)
+    X[rows // 2] = -np.inf                       # max = -inf: NaN for that row only
+    X[rows // 3, cols // 2] = -np.inf            # weight 0
+    Y = run_softmax(rt, X)
+    with np.errstate(invalid="ignore"):
+        ref = oracle.softmax(X)
+    assert np.isnan(Y[rows // 2]).all() and not np.isnan(np.delete(Y, rows // 2, axis=0)).any()
+    ok = ~np.isnan(ref)
+    assert Y[rows // 3, cols // 2] == 0.0
+    np.testing.assert_allclose(Y[ok], ref[ok], rtol=2e-5, atol=1e-30)
+
+
+@pytest.mark.parametrize(
+    "rows,cols",
+    [(130, 16388), (128, 32768), (200, 32772), (140, 65536), (129, 50000), (130, 20001), (129, 65535), (128, 32770),   # sixteen wavefronts hold a row
+     (3, 16388), (2, 40000), (100, 65540), (5, 300000), (1, 1 << 22), (7, 123457), (600, 70001), (2, 4097 * 4)],  # rows cut into slices
+)
+def test_softmax_long_rows(rt, rows, cols):
+    """Rows past 16384 columns: in the registers of sixteen wavefronts where there are rows enough for half the CUs,
+    else cut into slices over two launches (any width: a row need not start on a vector boundary)."""
+    rng = np.random.default_rng(rows * 7 + cols)
+    X = (rng.standard_normal((rows, cols)) * 8).astype(np.float32)
+    Y = run_softmax(rt, X)
+    ref = scipy.special.softmax(X.astype(np.float64), axis=-1)
+    assert rel_err_max(Y, ref) <= TOL_F32
+    np.testing.assert_allclose(Y, ref, rtol=3e-5, atol=1e-30)
+    np.testing.assert_allclose(Y.sum(axis=-1, dtype=np.float64), 1.0, rtol=0, atol=1e-5)
+
+
+@pytest.mark.parametrize("cols", [257, 259, 1001, 1023, 1026, 4095, 4097, 6282, 16383])
+def test_softmax_rows_that_start_off_a_vector_boundary(rt, cols):
+    """A width that is not a multiple of four puts most rows off a 16-byte boundary; the work-group per row then reads
+    up to three single elements, the vectors between the boundaries, and up to three single elements."""
+    rng = np.random.default_rng(cols)
+    X = (rng.standard_normal((13, cols)) * 8).astype(np.float32)
+    X[5] = -np.inf
+    X[6, cols - 1] = np.nan
+    X[7, :3] = -np.inf
+    Y = run_softmax(rt, X)
+    with np.errstate(invalid="ignore"):
+        ref = scipy.special.softmax(X.astype(np.float64), axis=-1)
+    assert np.isnan(Y[5]).all() and np.isnan(Y[6]).all() and (Y[7, :3] == 0).all()
+    ok = ~np.isnan(ref)
+    assert not np.isnan(Y[ok]).any()
+    np.testing.assert_allclose(Y[ok], ref[ok], rtol=3e-5, atol=1e-30)
+    # operands placed off the boundary themselves, equally and unequally (the second goes element by element)
+    for off_x, off_y in ((2, 2), (1, 3)):
+        bx = torch.zeros(X.size + 8, device="cuda")
+        by = torch.zeros(X.size + 8, device="cuda")
+        bx[off_x:off_x + X.size] = dev(X).view(-1)
+        rt.softmax_f32(13, cols, bx.data_ptr() + 4 * off_x, by.data_ptr() + 4 * off_y)
+        torch.cuda.synchronize()
+        got = host(by)
+        np.testing.assert_allclose(got[off_y:off_y + X.size].reshape(X.shape)[ok], ref[ok], rtol=3e-5, atol=1e-30)
+        assert (got[:off_y] == 0).all() and (got[off_y + X.size:] == 0).all()
+
+
+def test_softmax_long_rows_fp64_and_misplaced_operands(rt):
+    """The sliced rows in fp64 (vectors of two), and fp32 operands that are not 16-byte aligned: equally misplaced
+    operands keep the vector form (head and tail by single elements), unequally placed ones go element by element."""
+    rng = np.random.default_rng(12)
+    X = rng.standard_normal((3, 100003)) * 9
+    x = dev(X)
+    y = torch.empty_like(x)
+    rt.softmax(64, 3, 100003, 1, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    np.testing.assert_allclose(host(y), scipy.special.softmax(X, axis=-1), rtol=1e-12, atol=1e-300)
+    Xf = (rng.standard_normal((2, 70000)) * 8).astype(np.float32)
+    ref = scipy.special.softmax(Xf.astype(np.float64), axis=-1)
+    for off_x, off_y in ((1, 1), (3, 3), (1, 2), (0, 3)):
+        bx = torch.zeros(Xf.size + 8, device="cuda")
+        by = torch.zeros(Xf.size + 8, device="cuda")
+        bx[off_x:off_x + Xf.size] = dev(Xf).view(-1)
+        rt.softmax_f32(2, 70000, bx.data_ptr() + 4 * off_x, by.data_ptr() + 4 * off_y)
+        torch.cuda.synchronize()
+        got = host(by)
+        np.testing.assert_allclose(got[off_y:off_y + Xf.size].reshape(Xf.shape), ref, rtol=3e-5, atol=1e-30)
+        assert (got[:off_y] == 0).all() and (got[off_y + Xf.size:] == 0).all()      # nothing written outside the rows
+
+
+def test_softmax_long_rows_edge_values(rt):
+    """Infinite and NaN entries in rows that are cut into slices or held by sixteen wavefronts poison their own row only."""
+    for rows, cols in ((4, 200000), (140, 20000)):
+        X = np.zeros((rows, cols), np.float32)
+        X[0, cols - 5] = np.inf
+        X[1, 70] = np.nan
+        X[2, :] = -np.inf
+        X[3, 9::2] = -np.inf
+        Y = run_softmax(rt, X)
+        assert np.isnan(Y[:3]).all()
+        live = np.ones(cols, bool)
+        live[9::2] = False
+        assert (Y[3, ~live] == 0).all() and np.allclose(Y[3, live], 1.0 / live.sum(), rtol=1e-5)
+        if rows > 4:
+            assert np.allclose(Y[4:], 1.0 / cols, rtol=1e-5)
+    # a slice that holds nothing but -inf next to slices with finite values, and a NaN in a slice of -inf
+    X = np.full((2, 1 << 20), -np.inf, np.float32)
+    X[0, 5] = 1.0
+    X[0, (1 << 20) - 3] = 1.0
+    X[1, 5] = 2.0
+    X[1, 600000] = np.nan
+    Y = run_softmax(rt, X)
+    assert Y[0, 5] == 0.5 and Y[0, (1 << 20) - 3] == 0.5 and Y[0].sum() == 1.0 and np.isnan(Y[1]).all()
+
+
 @pytest.mark.parametrize("force", ["wave", "block"])
 @pytest.mark.parametrize("cols", [512, 1024, 2048, 3000, 4096])
 def test_softmax_every_built_variant(rt, monkeypatch, force, cols):
@@ -205,7 +318,7 @@ def test_softmax_with_the_callers_workspace(rt):
     """docc_rocm_softmax_ws: same bits as docc_rocm_softmax, the partial results in memory of the caller."""
     rng = np.random.default_rng(5)
     for dt, precision in ((np.float32, 32), (np.float64, 64)):
-        for outer, reduce_, inner in ((1, 5000, 300), (3, 700, 130), (2, 64, 40), (4, 100, 1), (2, 300, 16)):
+        for outer, reduce_, inner in ((1, 5000, 300), (3, 700, 130), (2, 64, 40), (4, 100, 1), (2, 300, 16), (3, 90000, 1), (300, 20000, 1)):
             X = (rng.standard_normal((outer, reduce_, inner)) * 6).astype(dt)
             x = dev(X)
             y0, y1 = torch.empty_like(x), torch.full_like(x, float("nan"))
@@ -223,6 +336,7 @@ def test_softmax_with_the_callers_workspace(rt):
                 with pytest.raises(RocmRuntimeError, match="workspace"):
                     rt.softmax_ws(precision, outer, reduce_, inner, x.data_ptr(), y1.data_ptr(), 0, 0)
     assert rt.softmax_workspace_bytes(32, 1, 5000, 300) > 0      # the sliced form is among the cases
+    assert rt.softmax_workspace_bytes(32, 3, 90000, 1) > 0 and rt.softmax_workspace_bytes(64, 3, 90000, 1) > 0      # and rows cut into slices
 
 
 def test_softmax_general_edge_values_and_empty(rt):

@@ -26,7 +26,8 @@ def both(rt, X, precision):
 def test_no_alloc_softmax_matches_the_allocating_entry_point(rt, dt, precision, tol):
     rng = np.random.default_rng(precision)
     # sliced form (partial results in the fixed array), large then small, then shapes of the one-launch forms
-    shapes = [(1, 6000, 320), (1, 900, 130), (2, 512, 70), (3, 700, 130), (1, 257, 64), (4, 100, 1), (2, 300, 16), (5, 40, 33)]
+    shapes = [(1, 6000, 320), (1, 900, 130), (2, 512, 70), (3, 700, 130), (1, 257, 64), (4, 100, 1), (2, 300, 16), (5, 40, 33),
+              (2, 150000, 1), (3, 20000, 1)]      # rows cut into slices: their pairs go through the fixed array as well
     assert rt.softmax_workspace_bytes(precision, *shapes[0]) > rt.softmax_workspace_bytes(precision, *shapes[1]) > 0
     for shape in shapes:
         X = (rng.standard_normal(shape) * 6).astype(dt)
