@@ -1,4 +1,4 @@
-// ml::Attention forward (non-causal), bf16 inputs, head dim 64, for gfx950:
+// ml::Attention forward (non-causal), bf16 inputs, head dim 32, 64 or 128, for gfx950:
 //   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) V[b,h,j,:]
 // with fp32 scores, softmax statistics and accumulation.
 //
@@ -9,8 +9,9 @@
 // head in memory. This kernel never stores scores: it walks the keys in
 // blocks of 64 with an online max/sum (flash-attention style).
 //
-// Layout of the computation (one work-group = four wavefronts of one head, each with QT tiles of 32
-// queries: 256 queries per work-group with QT = 2, 128 with QT = 1; K and V blocks are shared through LDS):
+// Layout of the computation (one work-group = four wavefronts of one head - eight at head dim 128 -, each with QT
+// tiles of 32 queries: 256 queries per work-group with QT = 2, 128 with QT = 1; K and V blocks are shared through LDS;
+// the figures below are those of head dim 64, the case the kernel was tuned on):
 //   S^T[key, q]  = K_blk[key, d] * Q^T[d, q]     v_mfma_f32_32x32x16_bf16, A = K (d-contiguous
 //                                                128-bit LDS reads), B = Q (kept in registers)
 //   the transposed product puts one query per lane (column = lane % 32) and 32 of
@@ -66,17 +67,23 @@ struct Mfma<uint16_t> {
     typedef u16x8_t vec_t;
 };
 
-constexpr int kHeadDim = 64;
 constexpr int kBlockKV = 64;     // keys per step
 constexpr int kAttnStages = 3;   // LDS ring depth: blocks kb+1 and kb+2 are in flight while block kb is worked on
-constexpr int kTileElems = kBlockKV * kHeadDim;          // one K or V block, unpadded, 16-byte granules swizzled
-constexpr int kStageElems = 2 * kTileElems;              // [K | V]
 
-// granule (8 bf16) index inside a row of 8 granules, swizzled so that the reads below are conflict-free:
-// K: a 128-bit read touches 16 consecutive rows at one granule column; V: a transposed 64-bit read
-// touches 4 consecutive rows x 4 granule columns
-__device__ __forceinline__ int attn_k_off(int row, int cv) { return (row * 8 + (cv ^ ((row >> 1) & 7))) * 8; }
-__device__ __forceinline__ int attn_v_off(int row, int cv) { return (row * 8 + (cv ^ (((row >> 1) & 1) << 2))) * 8; }
+// granule (8 bf16) index inside a row of HD / 8 granules, swizzled so that the reads below are conflict-free:
+// K: sixteen lanes of a 128-bit read touch 16 consecutive rows at one granule column; V: half a wavefront of a
+// transposed 64-bit read touches 4 consecutive rows x 4 granule columns. The LDS moves 256 bytes a cycle, which is
+// four rows at head dim 32, two at 64 and one at 128: the swizzle spreads the rows that would meet in the same banks.
+template <int HD> __device__ __forceinline__ int attn_k_swz(int row);
+template <> __device__ __forceinline__ int attn_k_swz<32>(int row) { return (row >> 2) & 3; }
+template <> __device__ __forceinline__ int attn_k_swz<64>(int row) { return (row >> 1) & 7; }
+template <> __device__ __forceinline__ int attn_k_swz<128>(int row) { return row & 15; }
+template <int HD> __device__ __forceinline__ int attn_v_swz(int row);
+template <> __device__ __forceinline__ int attn_v_swz<32>(int) { return 0; }
+template <> __device__ __forceinline__ int attn_v_swz<64>(int row) { return ((row >> 1) & 1) << 2; }
+template <> __device__ __forceinline__ int attn_v_swz<128>(int row) { return (row & 3) << 2; }
+template <int HD> __device__ __forceinline__ int attn_k_off(int row, int cv) { return (row * (HD / 8) + (cv ^ attn_k_swz<HD>(row))) * 8; }
+template <int HD> __device__ __forceinline__ int attn_v_off(int row, int cv) { return (row * (HD / 8) + (cv ^ attn_v_swz<HD>(row))) * 8; }
 
 // x of lanes 0..31 (which = 0) or of lanes 32..63 (which = 1), seen from both halves of the wave:
 // v_permlane32_swap exchanges the upper half of its first operand with the lower half of its second.
@@ -89,13 +96,21 @@ __device__ __forceinline__ float half_swap(float x, int which) {
     return __builtin_bit_cast(float, which ? sw[1] : sw[0]);
 }
 
-template <bool OUT_BF16, int QT>
-__device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
-                                                  const uint16_t* __restrict__ V, void* __restrict__ O, int SQ,
-                                                  int SKV, float scale_log2e) {
+template <bool OUT_BF16, int QT, int HD, int NW>
+__device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
+                                              const uint16_t* __restrict__ V, void* __restrict__ O, int SQ,
+                                              int SKV, float scale_log2e) {
     extern __shared__ __attribute__((aligned(16))) unsigned char docc_attn_lds[];
     uint16_t* const lds = reinterpret_cast<uint16_t*>(docc_attn_lds);
-    constexpr int kBlockQ = 128 * QT;     // queries per work-group
+    constexpr int kHeadDim = HD;
+    constexpr int kBlockQ = NW * 32 * QT;                    // queries per work-group
+    constexpr int kTileElems = kBlockKV * kHeadDim;          // one K or V block, unpadded, 16-byte granules swizzled
+    constexpr int kStageElems = 2 * kTileElems;              // [K | V]
+    constexpr int GR = HD / 8;                               // granules per row of a block
+    constexpr int RP = NW * 64 / GR;                         // rows of a block that the work-group copies at a time
+    constexpr int PASSES = kBlockKV / RP;
+    constexpr int KS = HD / 16, DT = HD / 32;                // MFMA steps over d of the score product, 32-row tiles of O^T
+    static_assert(PASSES >= 1 && PASSES * RP == kBlockKV, "the work-group's lanes must tile a block");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qj = lane & 31, g = lane >> 5;
@@ -114,11 +129,11 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const float ninf = -__builtin_huge_valf();
 
     // Q^T as the B operand of the score product: d = 16*ks + 8*g .. +7 of query q0 + 32*qt
-    bf16x8 bq[QT][4];
+    bf16x8 bq[QT][KS];
 #pragma unroll
     for (int qt = 0; qt < QT; qt++)
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
+        for (int ks = 0; ks < KS; ks++) {
             u16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
             if (q0 + 32 * qt < SQ) v = *reinterpret_cast<const u16x8_t*>(Qh + (long) (q0 + 32 * qt) * kHeadDim + 16 * ks + 8 * g);
             bq[qt][ks] = __builtin_bit_cast(bf16x8, v);
@@ -127,12 +142,13 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
     const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
 
-    // K/V copies: a block is 512 granules of 16 bytes per tensor, two per thread. LDS slot s (in copy
-    // order: lane-contiguous) holds row s/8, granule column (s%8) ^ swizzle(row). The second granule of a
-    // lane lies 32 rows below the first, where both swizzles repeat: one offset per tensor serves both.
-    const int copy_row = wave * 8 + (lane >> 3);
-    const unsigned koff = (unsigned) ((copy_row * 8 + ((lane & 7) ^ ((copy_row >> 1) & 7))) * 16);
-    const unsigned voff = (unsigned) ((copy_row * 8 + ((lane & 7) ^ (((copy_row >> 1) & 1) << 2))) * 16);
+    // K/V copies: a block is 64 * GR granules of 16 bytes per tensor, PASSES per thread. LDS slot s (in copy
+    // order: lane-contiguous) holds row s / GR, granule column (s % GR) ^ swizzle(row). The later granules of a
+    // lane lie RP rows below the first, where both swizzles repeat: one offset per tensor serves all.
+    const int copy_row = wave * (64 / GR) + lane / GR;
+    const unsigned koff = (unsigned) ((copy_row * GR + ((lane % GR) ^ attn_k_swz<HD>(copy_row))) * 16);
+    const unsigned voff = (unsigned) ((copy_row * GR + ((lane % GR) ^ attn_v_swz<HD>(copy_row))) * 16);
+    constexpr unsigned kPassBytes = RP * HD * 2;
     auto issue = [&](int kb) {   // starts the copy of block kb into its stage
         uint16_t* st = lds + (kb % kAttnStages) * kStageElems;
         const char* kp = Kh + (long) kb * (kTileElems * 2);
@@ -142,38 +158,39 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
             // the offsets once, outside the loop, which would cost 64-bit addresses per lane
             unsigned ko = koff, vo = voff;
             asm volatile("" : "+v"(ko), "+v"(vo));
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + ko), (attn_lds_ptr_t) (st + wave * 512), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + vo), (attn_lds_ptr_t) (st + kTileElems + wave * 512), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + 4096 + ko), (attn_lds_ptr_t) (st + (4 + wave) * 512), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + 4096 + vo), (attn_lds_ptr_t) (st + kTileElems + (4 + wave) * 512), 16, 0, 0);
+#pragma unroll
+            for (int i = 0; i < PASSES; i++) {
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + kPassBytes * i + ko), (attn_lds_ptr_t) (st + (i * NW + wave) * 512), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + kPassBytes * i + vo), (attn_lds_ptr_t) (st + kTileElems + (i * NW + wave) * 512), 16, 0, 0);
+            }
         } else {
             // the partial last block: rows past the end copy the last key (their scores are masked, their V rows zeroed)
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const int row = copy_row + 32 * i;
-                const unsigned back = row >= keys_left ? (unsigned) ((row - (keys_left - 1)) * 128) : 0u;
-                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + (koff + 4096u * i - back)), (attn_lds_ptr_t) (st + (i * 4 + wave) * 512), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + (voff + 4096u * i - back)), (attn_lds_ptr_t) (st + kTileElems + (i * 4 + wave) * 512), 16, 0, 0);
+            for (int i = 0; i < PASSES; i++) {
+                const int row = copy_row + RP * i;
+                const unsigned back = row >= keys_left ? (unsigned) ((row - (keys_left - 1)) * (HD * 2)) : 0u;
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (kp + (koff + kPassBytes * i - back)), (attn_lds_ptr_t) (st + (i * NW + wave) * 512), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((attn_global_ptr_t) (vp + (voff + kPassBytes * i - back)), (attn_lds_ptr_t) (st + kTileElems + (i * NW + wave) * 512), 16, 0, 0);
             }
         }
     };
     // block kb has landed in every wave's view and every wave is done with block kb-1; rows of a partial
     // last V block are cleared so that 0 * (copied value) cannot produce a NaN
     auto arrive = [&](int kb) {
-        // each block is four copies per lane; one newer block may still be in flight
-        if (kb + 1 < nblocks) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        // each block is 2 * PASSES copies per lane; one newer block may still be in flight
+        if (kb + 1 < nblocks) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(2 * PASSES) : "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (kb >= full_blocks) {
             uint16_t* vt = lds + (kb % kAttnStages) * kStageElems + kTileElems;
             const u16x8_t z = {0, 0, 0, 0, 0, 0, 0, 0};
-            for (int s = keys_left * 8 + tid; s < 512; s += 256) *reinterpret_cast<u16x8_t*>(vt + s * 8) = z;
+            for (int s = keys_left * GR + tid; s < kBlockKV * GR; s += 64 * NW) *reinterpret_cast<u16x8_t*>(vt + s * 8) = z;
             __syncthreads();
         }
     };
 
-    f32x16 ot[QT][2];   // O^T tiles: d = 32*dt + acc_row(lane, r), column = this lane's query of tile qt
+    f32x16 ot[QT][DT];  // O^T tiles: d = 32*dt + acc_row(lane, r), column = this lane's query of tile qt
     float m_run[QT];    // reference point of the exponentials (log2 domain); -inf: nothing finite seen yet
     float l_part[QT];   // this lane's part of the running sum (its 32 keys per block)
 #pragma unroll
@@ -181,7 +198,7 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         m_run[qt] = ninf;
         l_part[qt] = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < 2; dt++)
+        for (int dt = 0; dt < DT; dt++)
 #pragma unroll
             for (int r = 0; r < 16; r++) ot[qt][dt][r] = 0.f;
     }
@@ -195,17 +212,17 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
     const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // raw scores, transposed: s[qt][t][r] = <K[32t + acc_row(r)], Q[q0 + 32 qt]>; keys past the end score -inf.
-    // All eight K operands are requested before the first MFMA: one LDS round trip, not eight; each serves QT MFMAs.
+    // All K operands are requested before the first MFMA: one LDS round trip, not eight; each serves QT MFMAs.
     auto scores = [&](int kb, f32x16 (&s)[QT][2]) {
         const uint16_t* ks_ = lds + (kb % kAttnStages) * kStageElems;
-        u16x8_t kv[2][4];
+        u16x8_t kv[2][KS];
 #pragma unroll
         for (int t = 0; t < 2; t++)
 #pragma unroll
-            for (int ks = 0; ks < 4; ks++) kv[t][ks] = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off(32 * t + qj, 2 * ks + g));
+            for (int ks = 0; ks < KS; ks++) kv[t][ks] = *reinterpret_cast<const u16x8_t*>(ks_ + attn_k_off<HD>(32 * t + qj, 2 * ks + g));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++)
+        for (int ks = 0; ks < KS; ks++)
 #pragma unroll
             for (int t = 0; t < 2; t++)
 #pragma unroll
@@ -289,7 +306,7 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
                 m_run[qt] = m_new;
                 l_part[qt] *= alpha;
 #pragma unroll
-                for (int dt = 0; dt < 2; dt++)
+                for (int dt = 0; dt < DT; dt++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) ot[qt][dt][r] *= alpha;
                 psum[qt] = exponentials(st[qt], pk[qt], base_of(m_new));
@@ -302,16 +319,16 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         // The V operands of two steps are requested together (they do not depend on P); each serves QT MFMAs.
         const uint16_t* vs_ = lds + (kb % kAttnStages) * kStageElems + kTileElems;
         auto pv_half = [&](int h) {
-            s16x8_t va[2][2];
+            s16x8_t va[2][DT];
 #pragma unroll
             for (int uu = 0; uu < 2; uu++) {
                 const int u = 2 * h + uu;
                 const int row = 32 * (u >> 1) + 16 * (u & 1) + tr_row;
 #pragma unroll
-                for (int dt = 0; dt < 2; dt++) {
+                for (int dt = 0; dt < DT; dt++) {
                     const int col = 32 * dt + tr_col;
-                    const uint16_t* plo = vs_ + attn_v_off(row, col >> 3) + (col & 7);
-                    const uint16_t* phi = vs_ + attn_v_off(row + 8, col >> 3) + (col & 7);
+                    const uint16_t* plo = vs_ + attn_v_off<HD>(row, col >> 3) + (col & 7);
+                    const uint16_t* phi = vs_ + attn_v_off<HD>(row + 8, col >> 3) + (col & 7);
                     const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) plo);
                     const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*) phi);
                     va[uu][dt] = s16x8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -327,7 +344,7 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
                                                             pk[qt][u >> 1][4 * (u & 1) + 2], pk[qt][u >> 1][4 * (u & 1) + 3]}};
                     const bf16x8 pb = __builtin_bit_cast(bf16x8, pack);
 #pragma unroll
-                    for (int dt = 0; dt < 2; dt++)
+                    for (int dt = 0; dt < DT; dt++)
                         ot[qt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[uu][dt]), pb, ot[qt][dt], 0, 0, 0);
                 }
             }
@@ -348,7 +365,7 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
         const float inv = 1.0f / l;
         if (q < SQ) {
 #pragma unroll
-            for (int dt = 0; dt < 2; dt++) {
+            for (int dt = 0; dt < DT; dt++) {
 #pragma unroll
                 for (int rq = 0; rq < 4; rq++) {
                     const int d = 32 * dt + 8 * rq + 4 * g;   // registers 4*rq .. 4*rq+3 hold d .. d+3
@@ -372,11 +389,12 @@ __device__ __forceinline__ void attention_fwd_d64(const uint16_t* __restrict__ Q
 
 } // namespace docc_k
 
-#define DOCC_ATTENTION_KERNEL(name, out_bf16, qt, waves)                                                                          \
-    extern "C" __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(waves))) void name(                           \
+#define DOCC_ATTENTION_KERNEL_D(name, out_bf16, qt, waves, hd, nw)                                                                \
+    extern "C" __global__ __launch_bounds__(64 * nw) __attribute__((amdgpu_waves_per_eu(waves))) void name(                       \
         const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int SQ, int SKV, float scale_log2e) {                   \
-        docc_k::attention_fwd_d64<out_bf16, qt>(Q, K, V, O, SQ, SKV, scale_log2e);                                                \
+        docc_k::attention_fwd<out_bf16, qt, hd, nw>(Q, K, V, O, SQ, SKV, scale_log2e);                                            \
     }
+#define DOCC_ATTENTION_KERNEL(name, out_bf16, qt, waves) DOCC_ATTENTION_KERNEL_D(name, out_bf16, qt, waves, 64, 4)
 
 // 64 queries per wavefront (256 per work-group): the form for long query axes
 DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q256_f32out, false, 2, 2)
@@ -384,3 +402,15 @@ DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q256_bf16out, true, 2, 2)
 // 32 queries per wavefront (128 per work-group): more work-groups where there are few queries
 DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q128_f32out, false, 1, 3)
 DOCC_ATTENTION_KERNEL(docc_attention_bf16_d64_q128_bf16out, true, 1, 3)
+// head dim 32: the same two forms (half the MFMAs per block, the vector work of the softmax unchanged)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d32_q256_f32out, false, 2, 2, 32, 4)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d32_q256_bf16out, true, 2, 2, 32, 4)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d32_q128_f32out, false, 1, 3, 32, 4)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d32_q128_bf16out, true, 1, 3, 32, 4)
+// head dim 128: 32 queries per wavefront (the registers hold one tile of queries: 64 of O^T, 32 of Q, 64 of K operands),
+// eight wavefronts share the K and V blocks of a work-group (96 KB of LDS: one work-group per CU, two wavefronts per SIMD);
+// the four-wavefront form is for short query axes
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d128_q256_f32out, false, 1, 2, 128, 8)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d128_q256_bf16out, true, 1, 2, 128, 8)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d128_q128_f32out, false, 1, 1, 128, 4)
+DOCC_ATTENTION_KERNEL_D(docc_attention_bf16_d128_q128_bf16out, true, 1, 1, 128, 4)

@@ -42,6 +42,57 @@ extern "C" __global__ __launch_bounds__(256) void docc_fill_b8(uint8_t* __restri
     for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < n16; i += stride) body[i] = v;
 }
 
+// Rows of `d` 16-bit elements copied into rows of `dp` >= d (a multiple of 8), the rest of each row cleared: attention
+// operands of a head dimension that is not built, widened to one that is. One 16-byte piece of the result per lane.
+extern "C" __global__ __launch_bounds__(256) void docc_pad_rows_b16(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                                      long rows, int d, int dp) {
+    const int per_row = dp >> 3;
+    const long pieces = rows * per_row;
+    const long stride = (long) gridDim.x * 256;
+    for (long p = (long) blockIdx.x * 256 + threadIdx.x; p < pieces; p += stride) {
+        const long row = p / per_row;
+        const int c0 = (int) (p % per_row) * 8;
+        const uint16_t* from = src + row * d + c0;
+        u32x4 out;
+        if ((d & 7) == 0 && (reinterpret_cast<uintptr_t>(src) & 15) == 0) {   // whole pieces on both sides
+            out = c0 < d ? *reinterpret_cast<const u32x4*>(from) : u32x4{0u, 0u, 0u, 0u};
+            *reinterpret_cast<u32x4*>(dst + row * dp + c0) = out;
+            continue;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint32_t lo = c0 + 2 * i < d ? from[2 * i] : 0u;
+            const uint32_t hi = c0 + 2 * i + 1 < d ? from[2 * i + 1] : 0u;
+            out[i] = lo | (hi << 16);
+        }
+        *reinterpret_cast<u32x4*>(dst + row * dp + c0) = out;
+    }
+}
+
+// The first `d` elements of rows of `dp` elements, packed: the result of the widened attention, narrowed again.
+// WORD = uint16_t (bf16 result) or uint32_t (fp32 result).
+template <typename WORD>
+__device__ __forceinline__ void unpad_rows(const WORD* __restrict__ src, WORD* __restrict__ dst, long rows, int d, int dp) {
+    const long stride = (long) gridDim.x * 256;
+    constexpr int PER = 16 / sizeof(WORD);
+    if (d % PER == 0 && dp % PER == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0) {
+        // rows of whole 16-byte pieces on both sides
+        const int per_row = d / PER;
+        const long pieces = rows * per_row;
+        for (long p = (long) blockIdx.x * 256 + threadIdx.x; p < pieces; p += stride)
+            reinterpret_cast<u32x4*>(dst)[p] = *reinterpret_cast<const u32x4*>(src + (p / per_row) * dp + (p % per_row) * PER);
+        return;
+    }
+    const long n = rows * d;
+    for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = src[(i / d) * dp + i % d];
+}
+extern "C" __global__ __launch_bounds__(256) void docc_unpad_rows_b16(const uint16_t* src, uint16_t* dst, long rows, int d, int dp) {
+    unpad_rows(src, dst, rows, d, dp);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_unpad_rows_b32(const uint32_t* src, uint32_t* dst, long rows, int d, int dp) {
+    unpad_rows(src, dst, rows, d, dp);
+}
+
 extern "C" __global__ __launch_bounds__(256) void docc_f32_to_bf16(const float* __restrict__ src,
                                                                      uint16_t* __restrict__ dst, long n) {
     long i = (long) blockIdx.x * 256 + threadIdx.x;

@@ -1,5 +1,6 @@
 // Launcher for ml::Attention (see include/docc_rocm_ops.h).
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 
 #include "docc_rocm_ops.h"
@@ -11,7 +12,8 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
                                         int64_t D, float scale, const uint16_t* Q, const uint16_t* K,
                                         const uint16_t* V, void* O, int out_bf16) {
     if (B < 0 || H < 0 || SQ < 0 || SKV < 0 || D < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: negative shape");
-    if (D != 64) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: head dim %lld (only 64 is built)", (long long) D);
+    if (D != 32 && D != 64 && D != 128)
+        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: head dim %lld (32, 64 and 128 are built; docc_rocm_attention_bf16_ws takes any)", (long long) D);
     if (B == 0 || H == 0 || SQ == 0) return 0;
     if (SKV == 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: no keys (softmax over an empty axis)");
     if (!Q || !K || !V || !O) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: null pointer");
@@ -21,8 +23,8 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
     if (SQ > 0x7fffffffLL - 128 || SKV > 0x7fffffffLL - 64) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: sequences must be < 2^31");
     int rc = ensure_device();
     if (rc) return rc;
-    // LDS: ring of 3 stages x (K block [64][64] + V block [64][64]) bf16
-    const uint32_t lds = 3 * (2 * 64 * 64) * 2;
+    // LDS: ring of 3 stages x (K block [64][D] + V block [64][D]) bf16
+    const uint32_t lds = 3 * (2 * 64 * (uint32_t) D) * 2;
     const float scale_log2e = scale * 1.4426950408889634f;
     // Two forms: 256 queries per work-group (a wavefront takes 64, so each K/V operand read from LDS serves two
     // MFMAs: fewer instructions per flop) once that still gives every CU its two resident work-groups, else 128
@@ -36,13 +38,16 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
         const int v = std::atoi(force);
         if (v == 128 || v == 256) per_group = v;
     }
-    const char* kernel = per_group == 256 ? (out_bf16 ? "docc_attention_bf16_d64_q256_bf16out" : "docc_attention_bf16_d64_q256_f32out")
-                                          : (out_bf16 ? "docc_attention_bf16_d64_q128_bf16out" : "docc_attention_bf16_d64_q128_f32out");
+    // head dim 128: the large form is eight wavefronts of 32 queries (one work-group per CU), the small one four
+    if (D == 128 && !std::getenv("DOCC_ROCM_ATTENTION_Q")) per_group = ((SQ + 255) / 256) * BH >= compute_units() && no_extra_padding ? 256 : 128;
+    char kernel[64];
+    std::snprintf(kernel, sizeof(kernel), "docc_attention_bf16_d%d_q%d_%s", (int) D, per_group, out_bf16 ? "bf16out" : "f32out");
+    const uint32_t threads = D == 128 && per_group == 256 ? 512 : 256;
     // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
     for (int64_t h0 = 0; h0 < BH; h0 += 65535) {
         const int64_t nh = BH - h0 < 65535 ? BH - h0 : 65535;
-        rc = launch(kernel, (uint32_t) ((SQ + per_group - 1) / per_group), (uint32_t) nh, 1, 256, lds, (hipStream_t) stream,
-                    Q + h0 * SQ * 64, K + h0 * SKV * 64, V + h0 * SKV * 64, (void*) ((char*) O + h0 * SQ * 64 * out_bytes), (int) SQ,
+        rc = launch(kernel, (uint32_t) ((SQ + per_group - 1) / per_group), (uint32_t) nh, 1, threads, lds, (hipStream_t) stream,
+                    Q + h0 * SQ * D, K + h0 * SKV * D, V + h0 * SKV * D, (void*) ((char*) O + h0 * SQ * D * out_bytes), (int) SQ,
                     (int) SKV, scale_log2e);
         if (rc) return rc;
     }
@@ -52,6 +57,17 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
 // ---- any head dimension, through a caller-provided workspace -----------------------------------
 
 namespace {
+
+bool fused_head_dim(int64_t D) { return D == 32 || D == 64 || D == 128; }
+
+// the head dimension of the fused kernel that a smaller one is widened to (zero columns change neither the scores
+// nor the first D columns of the result); 0: none, the separate kernels run
+int64_t widened_head_dim(int64_t D) { return D < 32 ? 32 : D < 64 ? 64 : D < 128 ? 128 : 0; }
+
+// bytes of the widened Q, K, V and result per (batch, head) pair
+int64_t widened_bytes_per_head(int64_t SQ, int64_t SKV, int64_t Dp, int out_bf16) {
+    return (SQ + 2 * SKV) * Dp * 2 + SQ * Dp * (out_bf16 ? 2 : 4);   // Dp is a multiple of 32: every part stays 64-byte aligned
+}
 
 // bytes of scores (fp32) + probabilities (bf16) + an fp32 result per (batch, head) pair
 int64_t attention_bytes_per_head(int64_t SQ, int64_t SKV, int64_t D, int out_bf16) {
@@ -72,15 +88,16 @@ int64_t attention_heads_per_chunk(int64_t BH, int64_t per_head) {
 
 extern "C" int64_t docc_rocm_attention_bf16_workspace_bytes(int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, int out_bf16) {
     if (B <= 0 || H <= 0 || SQ <= 0 || SKV <= 0 || D <= 0) return 0;
-    if (D == 64) return 0;   // the fused kernel keeps scores and probabilities in registers
-    const int64_t per_head = attention_bytes_per_head(SQ, SKV, D, out_bf16);
+    if (fused_head_dim(D)) return 0;   // the fused kernel keeps scores and probabilities in registers
+    const int64_t per_head = widened_head_dim(D) ? widened_bytes_per_head(SQ, SKV, widened_head_dim(D), out_bf16)
+                                                 : attention_bytes_per_head(SQ, SKV, D, out_bf16);
     return attention_heads_per_chunk(B * H, per_head) * per_head;
 }
 
 extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
                                            float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
                                            int out_bf16, void* workspace, int64_t workspace_bytes) {
-    if (D == 64) return docc_rocm_attention_bf16(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16);
+    if (fused_head_dim(D)) return docc_rocm_attention_bf16(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16);
     if (B < 0 || H < 0 || SQ < 0 || SKV < 0 || D < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: negative shape");
     if (B == 0 || H == 0 || SQ == 0) return 0;
     if (SKV == 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: no keys (softmax over an empty axis)");
@@ -91,6 +108,37 @@ extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B,
     if (!workspace || workspace_bytes < need || ((uintptr_t) workspace % 256) != 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: head dim %lld needs a 256-byte aligned workspace of %lld bytes",
                     (long long) D, (long long) need);
+    if (const int64_t Dp = widened_head_dim(D)) {
+        // a head dimension below 128 that is not built: the operands are widened with zero columns to the next one
+        // that is, the fused kernel runs on them, and the first D columns of its result are the answer
+        if (((uintptr_t) Q | (uintptr_t) K | (uintptr_t) V) % 2 != 0 || (uintptr_t) O % (out_bf16 ? 2 : 4) != 0)
+            return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: misaligned pointer");
+        if (int rc = ensure_device()) return rc;
+        const int64_t BH = B * H, per_head = widened_bytes_per_head(SQ, SKV, Dp, out_bf16);
+        const int64_t chunk = attention_heads_per_chunk(BH, per_head);
+        hipStream_t s = (hipStream_t) stream;
+        auto grid = [](int64_t items) { return (uint32_t) (items < 256 * 4096 ? (items + 255) / 256 : 4096); };
+        for (int64_t h0 = 0; h0 < BH; h0 += chunk) {
+            const int64_t nh = BH - h0 < chunk ? BH - h0 : chunk;
+            uint16_t* Qp = (uint16_t*) workspace;
+            uint16_t* Kp = Qp + nh * SQ * Dp;
+            uint16_t* Vp = Kp + nh * SKV * Dp;
+            void* Op = (void*) (Vp + nh * SKV * Dp);
+            const struct { const uint16_t* from; uint16_t* to; int64_t rows; } parts[3] = {
+                {Q + h0 * SQ * D, Qp, nh * SQ}, {K + h0 * SKV * D, Kp, nh * SKV}, {V + h0 * SKV * D, Vp, nh * SKV}};
+            for (const auto& part : parts)
+                if (int rc = launch("docc_pad_rows_b16", grid(part.rows * (Dp / 8)), 1, 1, 256, 0, s, part.from, part.to, (long) part.rows, (int) D, (int) Dp))
+                    return rc;
+            if (int rc = docc_rocm_attention_bf16(stream, 1, nh, SQ, SKV, Dp, scale, Qp, Kp, Vp, Op, out_bf16)) return rc;
+            const int64_t rows = nh * SQ;
+            int rc = out_bf16 ? launch("docc_unpad_rows_b16", grid(rows * D), 1, 1, 256, 0, s, (const uint16_t*) Op, (uint16_t*) O + h0 * SQ * D, (long) rows,
+                                       (int) D, (int) Dp)
+                              : launch("docc_unpad_rows_b32", grid(rows * D), 1, 1, 256, 0, s, (const uint32_t*) Op, (uint32_t*) O + h0 * SQ * D, (long) rows,
+                                       (int) D, (int) Dp);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     // S = scale * Q K^T (batched bf16 GEMM, fp32 out), P = softmax rows of S, rounded to bf16, O = P V
     const int64_t BH = B * H, per_head = attention_bytes_per_head(SQ, SKV, D, out_bf16);
     const int64_t chunk = attention_heads_per_chunk(BH, per_head);

@@ -325,7 +325,7 @@ protected:
         const auto& q = a.shape_q();
         const int out_bf16 = a.output_element() == types::PrimitiveType::BFloat ? 1 : 0;
         int64_t d = 0;
-        if (symbolic::is_integer(q[3], &d) && d == 64) {
+        if (symbolic::is_integer(q[3], &d) && (d == 32 || d == 64 || d == 128)) {   // the head dimensions of the fused kernel
             s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16(nullptr, " << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv()
               << ", " << q[3] << ", (float) (" << a.scale() << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) "
               << name_of("K") << ", (const uint16_t *) " << name_of("V") << ", (void *) " << name_of("O") << ", " << out_bf16
@@ -957,7 +957,7 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!a) return decline("not an Attention node object");
         if (a->element() != P::BFloat) return decline("inputs must be BFloat");
         if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
-        // head dimension 64 runs the fused kernel, any other the GEMM / softmax / GEMM sequence
+        // head dimensions 32, 64 and 128 run the fused kernel, any other the GEMM / softmax / GEMM sequence
     } else if (auto* act = dynamic_cast<tensor::ActivationNode*>(&node)) {
         if (act->element() != P::Float && act->element() != P::Double) return decline("element type must be Float or Double");
     } else if (auto* fill = dynamic_cast<tensor::FillNode*>(&node)) {

@@ -13,7 +13,7 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     softmax(x, dim=-1) on fp32             -> ml::Softmax
     F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
-                                           -> ml::Attention (bf16, head dim 64)
+                                           -> ml::Attention (bf16; head dims 32, 64, 128 fused)
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
                                            -> ml::Add .. ml::Minimum, with ml::Broadcast where shapes differ
     relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh),

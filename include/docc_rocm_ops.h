@@ -204,7 +204,7 @@ int docc_rocm_conv2d_f32_pads(docc_rocm_stream_t stream, int64_t N, int64_t C, i
  *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
  * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32
  * scores, softmax and accumulation; non-causal. O is [B,H,SQ,D], fp32 when
- * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 64
+ * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 32, 64 or 128
  * (docc_rocm_attention_bf16_ws takes any D).
  */
 int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
@@ -213,9 +213,11 @@ int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, in
 
 /*
  * The same node for any head dimension D, with device memory of the caller for the scores:
- * D == 64 runs the kernel above and needs none; otherwise S = scale * Q K^T (batched bf16
- * GEMM, fp32 out), a row softmax, the probabilities rounded to bf16 and O = P V run as
- * separate kernels over chunks of (batch, head) pairs that keep the workspace under 2 GiB.
+ * D == 32, 64 or 128 runs the kernel above and needs none; another D below 128 is widened with zero
+ * columns to the next of these in the workspace (Q, K, V and the result), the kernel above runs on the
+ * widened operands and the first D columns of its result are copied out; above 128 S = scale * Q K^T
+ * (batched bf16 GEMM, fp32 out), a row softmax, the probabilities rounded to bf16 and O = P V run as
+ * separate kernels. Either way over chunks of (batch, head) pairs that keep the workspace under 2 GiB.
  * `workspace` must be 256-byte aligned and hold what _workspace_bytes returns for the
  * same arguments (0 when no workspace is needed). Calls on one stream may share a workspace.
  */

@@ -42,9 +42,10 @@ def run_attention(rt, Qb, Kb, Vb, scale=None, out_bf16=False):
 @pytest.mark.parametrize("B,H,SQ,SKV", [(1, 2, 96, 96), (1, 1, 1, 1), (2, 3, 128, 64), (1, 2, 130, 200), (1, 1, 33, 65),
                                         (2, 2, 256, 512), (1, 1, 7, 1000)])
 @pytest.mark.parametrize("out_bf16", [False, True])
-def test_attention_matches_oracle(rt, B, H, SQ, SKV, out_bf16):
-    g = torch.Generator().manual_seed(B * 7 + H * 5 + SQ * 3 + SKV)
-    Q, K, V = (torch.randn(B, H, s, 64, generator=g).bfloat16() for s in (SQ, SKV, SKV))
+@pytest.mark.parametrize("D", [64, 32, 128])
+def test_attention_matches_oracle(rt, B, H, SQ, SKV, out_bf16, D):
+    g = torch.Generator().manual_seed(B * 7 + H * 5 + SQ * 3 + SKV + (D if D != 64 else 0))
+    Q, K, V = (torch.randn(B, H, s, D, generator=g).bfloat16() for s in (SQ, SKV, SKV))
     O = run_attention(rt, bits(Q), bits(K), bits(V), out_bf16=out_bf16)
     ref = oracle.attention(bits(Q), bits(K), bits(V))
     assert np.isfinite(O).all()
@@ -106,6 +107,62 @@ def test_attention_reference_point_moves_between_blocks(rt, SQ, SKV, steps):
         ref = oracle.attention(bits(Q), bits(K), bits(V))
         assert np.isfinite(O).all()
         assert rel_err_max(O, ref) <= TOL_BF16
+
+
+@pytest.mark.parametrize("D", [32, 128])
+def test_attention_other_head_dimensions_closed_forms_and_edge_values(rt, D):
+    """Head dims 32 and 128 run the same kernel with other tile constants: equal keys give the mean of V, a dominant key
+    its V row, excluded keys (-inf scores) weigh nothing, a key axis that ends inside a block is masked, and a reference
+    point that has to move (scores growing by e^32 from block to block) takes the slow path."""
+    g = torch.Generator().manual_seed(D)
+    Q = torch.randn(1, 2, 70, D, generator=g).bfloat16()
+    V = torch.randn(1, 2, 150, D, generator=g).bfloat16()
+    K = torch.randn(1, 2, 1, D, generator=g).bfloat16().expand(1, 2, 150, D).contiguous()
+    O = run_attention(rt, bits(Q), bits(K), bits(V))
+    assert rel_err_max(O, np.broadcast_to(V.float().mean(dim=2, keepdim=True).numpy(), O.shape)) <= 5e-3
+    Kd = torch.zeros(1, 1, 100, D).bfloat16()
+    Qd = torch.zeros(1, 1, 40, D).bfloat16()
+    Qd[..., D - 1] = 64.0
+    Kd[0, 0, 77, D - 1] = 64.0
+    Vd = torch.randn(1, 1, 100, D, generator=g).bfloat16()
+    O = run_attention(rt, bits(Qd), bits(Kd), bits(Vd), scale=0.125)
+    assert np.array_equal(O[0, 0], np.broadcast_to(Vd[0, 0, 77].float().numpy(), (40, D)))
+    # -inf scores: keys whose first component is -inf against queries with a positive first component
+    Q = torch.randn(1, 2, 130, D, generator=g)
+    K = torch.randn(1, 2, 333, D, generator=g)
+    V = torch.randn(1, 2, 333, D, generator=g)
+    Q[..., 0] = Q[..., 0].abs() + 0.5
+    K[0, 0, :64, 0] = -float("inf")
+    K[0, 1, 5::3, 0] = -float("inf")
+    Q, K, V = Q.bfloat16(), K.bfloat16(), V.bfloat16()
+    O = run_attention(rt, bits(Q), bits(K), bits(V))
+    ref = oracle.attention(bits(Q), bits(K), bits(V))
+    assert np.isfinite(O).all() and rel_err_max(O, ref) <= TOL_BF16
+    # the reference point moves: K[j, 0] grows by 32 per block of 64 keys, Q[i, 0] = +-8
+    Q = torch.randn(1, 1, 64, D, generator=g)
+    K = torch.randn(1, 1, 448, D, generator=g)
+    V = torch.randn(1, 1, 448, D, generator=g).bfloat16()
+    Q[..., 0] = torch.tensor([8.0, -8.0, 0.5, 0.0]).repeat(16)
+    K[0, 0, :, 0] = 32.0 * (torch.arange(448) // 64)
+    Q, K = Q.bfloat16(), K.bfloat16()
+    O = run_attention(rt, bits(Q), bits(K), bits(V), scale=0.125)
+    ref = oracle.attention(bits(Q), bits(K), bits(V), scale=0.125)
+    assert np.isfinite(O).all() and rel_err_max(O, ref) <= TOL_BF16
+
+
+def test_attention_head_dim_128_at_size(rt):
+    """B4 H16 S2048 D128 (what a 2048-wide model's attention layer asks for): bands of queries of three heads against
+    the oracle, and every output row inside the envelope of V."""
+    torch.manual_seed(5)
+    Q, K, V = (torch.randn(4, 16, 2048, 128).bfloat16() for _ in range(3))
+    O = run_attention(rt, bits(Q), bits(K), bits(V), out_bf16=True)
+    assert np.isfinite(O).all()
+    for (b, h) in [(0, 0), (2, 7), (3, 15)]:
+        ref = oracle.attention(bits(Q[b:b + 1, h:h + 1, 900:1028]), bits(K[b:b + 1, h:h + 1]), bits(V[b:b + 1, h:h + 1]))
+        assert rel_err_max(O[b, h, 900:1028], ref[0, 0]) <= TOL_BF16
+    vmin = V.float().amin(dim=2, keepdim=True).numpy()
+    vmax = V.float().amax(dim=2, keepdim=True).numpy()
+    assert (O >= vmin - 0.02).all() and (O <= vmax + 0.02).all()
 
 
 @pytest.mark.parametrize("sigma,bound", [(1.0, 5e-3), (3.3, 5e-3), (4.5, 5e-3), (8.0, 5e-3)])
@@ -175,7 +232,7 @@ def test_attention_errors(rt):
     t = torch.zeros(64 * 64, dtype=torch.bfloat16, device="cuda")
     p = t.data_ptr()
     with pytest.raises(RocmRuntimeError):
-        rt.attention_bf16(1, 1, 8, 8, 128, 0.1, p, p, p, p)   # head dim not built
+        rt.attention_bf16(1, 1, 8, 8, 96, 0.1, p, p, p, p)    # head dim not built
     with pytest.raises(RocmRuntimeError):
         rt.attention_bf16(1, 1, 8, 0, 64, 0.1, p, p, p, p)    # empty key axis
     rt.attention_bf16(0, 1, 8, 8, 64, 0.1, 0, 0, 0, 0)         # empty batch: no-op
@@ -215,15 +272,15 @@ def run_attention_ws(rt, Qb, Kb, Vb, scale=None, out_bf16=False, slack=0):
     return o.float().cpu().numpy(), need
 
 
-@pytest.mark.parametrize("B,H,SQ,SKV,D", [(1, 2, 96, 96, 128), (2, 3, 128, 64, 32), (1, 2, 130, 200, 128), (1, 1, 33, 65, 80),
-                                          (1, 1, 1, 1, 8), (2, 2, 256, 512, 128), (1, 1, 7, 1000, 16), (1, 2, 50, 70, 7),
-                                          (1, 2, 96, 96, 64)])
+@pytest.mark.parametrize("B,H,SQ,SKV,D", [(1, 2, 96, 96, 96), (2, 3, 128, 64, 48), (1, 2, 130, 200, 256), (1, 1, 33, 65, 80),
+                                          (1, 1, 1, 1, 8), (2, 2, 256, 512, 160), (1, 1, 7, 1000, 16), (1, 2, 50, 70, 7),
+                                          (1, 2, 96, 96, 64), (1, 2, 96, 96, 128), (1, 2, 96, 96, 32)])
 @pytest.mark.parametrize("out_bf16", [False, True])
 def test_attention_any_head_dimension_matches_oracle(rt, B, H, SQ, SKV, D, out_bf16):
     g = torch.Generator().manual_seed(B * 7 + H * 5 + SQ * 3 + SKV + D)
     Q, K, V = (torch.randn(B, H, s, D, generator=g).bfloat16() for s in (SQ, SKV, SKV))
     O, need = run_attention_ws(rt, bits(Q), bits(K), bits(V), out_bf16=out_bf16)
-    assert (need == 0) == (D == 64)        # head dim 64 runs the fused kernel and needs no workspace
+    assert (need == 0) == (D in (32, 64, 128))        # these run the fused kernel and need no workspace
     ref = oracle.attention(bits(Q), bits(K), bits(V))
     assert np.isfinite(O).all()
     assert rel_err_max(O, ref) <= TOL_BF16
@@ -233,14 +290,14 @@ def test_attention_workspace_is_checked_and_chunked(rt):
     from docc_amd.runtime import RocmRuntimeError
     t = torch.zeros(1 << 16, dtype=torch.bfloat16, device="cuda")
     p = t.data_ptr()
-    need = rt.attention_bf16_workspace_bytes(1, 1, 8, 8, 128)
+    need = rt.attention_bf16_workspace_bytes(1, 1, 8, 8, 96)
     assert need >= 8 * 8 * 6
     with pytest.raises(RocmRuntimeError, match="workspace"):
-        rt.attention_bf16_ws(1, 1, 8, 8, 128, 0.1, p, p, p, p, 0, 0)
+        rt.attention_bf16_ws(1, 1, 8, 8, 96, 0.1, p, p, p, p, 0, 0)
     with pytest.raises(RocmRuntimeError, match="workspace"):
-        rt.attention_bf16_ws(1, 1, 8, 8, 128, 0.1, p, p, p, p, p, need - 1)
+        rt.attention_bf16_ws(1, 1, 8, 8, 96, 0.1, p, p, p, p, p, need - 1)
     # more (batch, head) pairs than one 2 GiB chunk of scores holds: 40 x 4096 x 4096 x 6 B = 3.75 GiB
-    B, H, S, D = 1, 40, 4096, 32
+    B, H, S, D = 1, 40, 4096, 160
     need = rt.attention_bf16_workspace_bytes(B, H, S, S, D)
     assert need <= 2 << 30 and need < H * S * S * 6
     g = torch.Generator(device="cuda").manual_seed(9)
@@ -252,6 +309,26 @@ def test_attention_workspace_is_checked_and_chunked(rt):
     for h in (0, 21, 39):       # heads of the first and of the second chunk
         ref = oracle.attention(bits(Q[:, h:h + 1, :256].cpu()), bits(K[:, h:h + 1].cpu()), bits(V[:, h:h + 1].cpu()))
         assert rel_err_max(o[:, h:h + 1, :256].cpu().numpy(), ref) <= TOL_BF16
+
+
+def test_attention_widened_head_dimension_in_chunks(rt):
+    """Head dim 96 runs as head dim 128 on operands widened with zero columns; 1100 heads of 2048 keys need 2.3 GB for
+    the widened copies, so they go in two chunks. Heads of both chunks against the oracle; the rest inside V's envelope."""
+    B, H, S, D = 1, 1100, 2048, 96
+    need = rt.attention_bf16_workspace_bytes(B, H, S, S, D, True)
+    assert need <= 2 << 30 and need < H * ((3 * S) * 128 * 2 + S * 128 * 2)
+    g = torch.Generator(device="cuda").manual_seed(10)
+    Q, K, V = (torch.randn(B, H, S, D, device="cuda", generator=g).bfloat16() for _ in range(3))
+    o = torch.full((B, H, S, D), float("nan"), device="cuda", dtype=torch.bfloat16)
+    ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+    rt.attention_bf16_ws(B, H, S, S, D, D ** -0.5, Q.data_ptr(), K.data_ptr(), V.data_ptr(), o.data_ptr(), ws.data_ptr(), need, out_bf16=True)
+    torch.cuda.synchronize()
+    for h in (0, 500, 1099):
+        ref = oracle.attention(bits(Q[:, h:h + 1, :128].cpu()), bits(K[:, h:h + 1].cpu()), bits(V[:, h:h + 1].cpu()))
+        assert rel_err_max(o[:, h:h + 1, :128].float().cpu().numpy(), ref) <= TOL_BF16
+    assert bool(torch.isfinite(o.float()).all())
+    vmin, vmax = V.float().amin(dim=2, keepdim=True), V.float().amax(dim=2, keepdim=True)
+    assert bool(((o.float() >= vmin - 0.02) & (o.float() <= vmax + 0.02)).all())
 
 
 def test_attention_more_pairs_than_one_grid_holds(rt):

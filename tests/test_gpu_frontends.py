@@ -683,14 +683,16 @@ def test_softmax_over_other_axes_and_fp64_through_both_front_ends():
     assert rel_err_max(out.numpy(), oracle.softmax_axes(a.numpy(), (0,))) <= 1e-12
 
 
-def test_torch_attention_with_head_dimension_128():
-    """Another head dimension than 64: the node brings a workspace for its scores (GEMM, softmax, GEMM)."""
+@pytest.mark.parametrize("D", [128, 96])
+def test_torch_attention_with_other_head_dimensions(D):
+    """Head dimension 128 runs the fused kernel like 64; 96 is not built, and the node brings a workspace for its
+    scores (GEMM, softmax, GEMM)."""
     torch.manual_seed(5)
-    Q, K, V = (torch.randn(2, 3, 200, 128).bfloat16() for _ in range(3))
+    Q, K, V = (torch.randn(2, 3, 200, D).bfloat16() for _ in range(3))
     for dev_in in ("cuda", "cpu"):
         program = docc_torch.compile_torch(Attn(), tuple(t.to(dev_in) for t in (Q, K, V)), target="rocm")
         out = program(*(t.to(dev_in) for t in (Q, K, V)))
-        assert out.device.type == dev_in and out.dtype == torch.bfloat16 and out.shape == (2, 3, 200, 128)
+        assert out.device.type == dev_in and out.dtype == torch.bfloat16 and out.shape == (2, 3, 200, D)
         assert rel_err_max(out.float().cpu().numpy(), oracle.attention(bits(Q), bits(K), bits(V))) <= 2e-2
 
 

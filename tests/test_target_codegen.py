@@ -231,7 +231,7 @@ def test_softmax_over_inner_axes_and_fp64(tmp_path):
 
 
 def test_attention_with_another_head_dimension_brings_its_workspace(tmp_path):
-    for d, fused in ((64, True), (128, False)):
+    for d, fused in ((64, True), (128, True), (32, True), (96, False)):
         b = StructuredSDFGBuilder("att")
         for n in ("Q", "K", "V", "O"):
             b.add_container(n, BF16, True)
@@ -240,10 +240,10 @@ def test_attention_with_another_head_dimension_brings_its_workspace(tmp_path):
         s.schedule("rocm", options={"offload": "none"})
         src, _ = source_of(s, tmp_path)
         if fused:
-            assert "docc_rocm_attention_bf16(nullptr, 2, 4, 256, 192, 64, (float) (0.125)," in src and "_ws" not in src
+            assert f"docc_rocm_attention_bf16(nullptr, 2, 4, 256, 192, {d}, (float) (0.125)," in src and "_ws" not in src
         else:
-            assert "docc_rocm_attention_bf16_workspace_bytes(2, 4, 256, 192, 128, 1);" in src
-            assert "docc_rocm_attention_bf16_ws(nullptr, 2, 4, 256, 192, 128, (float) (0.125), (const uint16_t *) Q" in src
+            assert "docc_rocm_attention_bf16_workspace_bytes(2, 4, 256, 192, 96, 1);" in src
+            assert "docc_rocm_attention_bf16_ws(nullptr, 2, 4, 256, 192, 96, (float) (0.125), (const uint16_t *) Q" in src
             assert src.index("docc_rocm_malloc_async(&__ws") < src.index("docc_rocm_attention_bf16_ws(") < src.index("docc_rocm_free_async(__ws, nullptr)")
 
 
