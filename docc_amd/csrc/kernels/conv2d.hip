@@ -200,6 +200,8 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 // One work-group computes 64 output channels x a strip of TH full output rows of one image
 // (TH*OW <= 448 pixels = 14 MFMA column tiles). Wave w takes output-channel tile (w & 1) and
 // pixel tiles 7*(w >> 1) .. +6, so the four waves hold the whole strip in 7 accumulators each.
+// TILES = 4 or 2 instead of 7 tiles per wave (strips of 256 or 128 pixels) are for layers whose images are
+// too small to give every CU a strip of 448: a work-group costs what its tiles cost, filled or not.
 // K = C*KH*KW is walked in chunks of 8 input channels. Per chunk the work-group stages
 //   - the input patch [TH+KH-1][OW+KW-1][8] (halo rows and columns included, zeros where the
 //     patch leaves the image, the eight channels of a pixel adjacent): every input pixel is read
@@ -232,14 +234,15 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 
 namespace docc_k {
 
-template <int KH, int KW, bool SPLIT = false, bool NARROW = false>
+template <int KH, int KW, bool SPLIT = false, bool NARROW = false, int TILES = 7>
 struct ConvHaloKernel {
     static_assert(!NARROW || SPLIT, "the narrow tile is the shared tile of a split strip");
+    static_assert(TILES >= 2 && (!SPLIT || TILES == 7), "the last chunk goes in groups of at least two tiles; the split strip is 13 tiles");
     static constexpr int KHW = KH * KW;
     static constexpr int CI = 8;                 // input channels per chunk
     static constexpr int KC = CI * KHW;          // k per chunk
-    static constexpr int TN = 7;                 // MFMA column tiles per wave (SPLIT: the seventh is the shared one)
-    static constexpr int TOWN = SPLIT ? 6 : 7;   // column tiles a wave has to itself
+    static constexpr int TN = TILES;             // MFMA column tiles per wave (SPLIT: the seventh is the shared one)
+    static constexpr int TOWN = SPLIT ? TN - 1 : TN;   // column tiles a wave has to itself
     static constexpr int LDA_S = KC + 4;
     static constexpr int A_ELEMS = 64 * LDA_S;
     static constexpr int NR = 3;                 // patch pixels per thread per chunk (upper bound)
@@ -790,6 +793,22 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3(docc_
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_k::ConvParams p, int TH) {
     docc_k::ConvHaloKernel<1, 1>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 4>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 2>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 4>::run(p, TH);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 2>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split(docc_k::ConvParams p, int TH) {

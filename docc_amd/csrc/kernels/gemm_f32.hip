@@ -28,4 +28,17 @@ extern "C" __global__ __launch_bounds__(256) void docc_sgemm_scale_c(float* C, l
         *p = (beta == 0.f) ? 0.f : beta * (*p);
     }
 }
+// The end of a product whose K extent was cut into `splits` parts (each part's product in P[z], an m x n matrix of its
+// own): C = alpha * (P[0] + P[1] + ...) + beta * C, the parts added in order; beta == 0 does not read C.
+extern "C" __global__ __launch_bounds__(256) void docc_splitk_combine_f32(const float* __restrict__ P, float* __restrict__ C, long M, long N,
+                                                                         long ldc, int splits, float alpha, float beta) {
+    const long total = M * N;
+    const long stride = (long) gridDim.x * 256;
+    for (long i = (long) blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+        float sum = P[i];
+        for (int z = 1; z < splits; z++) sum += P[(long) z * total + i];
+        float* p = C + (i / N) * ldc + (i % N);
+        *p = (beta == 0.f) ? alpha * sum : alpha * sum + beta * (*p);
+    }
+}
 #endif

@@ -1,4 +1,6 @@
 // Launcher for ml::Conv (see include/docc_rocm_ops.h).
+#include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -31,24 +33,89 @@ namespace {
 
 constexpr int64_t kConvWorkspaceCap = int64_t(2) << 30;   // images are processed in chunks that fit this
 
-// Rough times (us) of the three ways to run a layer, from what the kernels were measured to sustain. The halo
-// kernel computes 64 channels x 448 pixels per work-group whatever the strip really holds, one work-group per CU
-// at a time, at about 490 GFLOP/s per CU. The gather kernel sustains about 55 TFLOP/s when its 64 x 128 tiles
-// fill the CUs evenly. The GEMM on a column matrix runs at about 75 TFLOP/s on these shapes; the columns are
-// written and read once at about 5 TB/s, and the extra launches (columns, bias, transpose) cost about 15 us.
-double halo_time_us(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t K, int cus) {
-    int64_t TH = 448 / OW;
-    if (TH > OH) TH = OH;
-    if (TH < 1) TH = 1;
-    const int64_t groups = N * ((OH + TH - 1) / TH) * ((OC + 63) / 64);
-    const int64_t rounds = (groups + cus - 1) / cus;
-    return (double) rounds * (2.0 * 64 * 448 * (double) K) / 490e3;
+// How a layer runs on the LDS-halo kernel. A work-group takes 64 output channels x a strip of TH full output rows
+// and costs what its 2 x `tiles` column tiles of 32 pixels cost, filled or not; one work-group owns a CU at a time
+// (the forms with 7 and 4 tiles per wave by their registers), so a launch takes rounds of work-groups x tiles per wave.
+// Strips of 448 pixels (7 tiles per wave) where the images give every CU one; of 416 with the thirteenth tile shared
+// by the two pixel groups (6.5 tiles per wave, or 6.25 when that tile holds at most 16 pixels and goes through the
+// 16-pixel MFMA) where that saves a round's worth - the shorter strips pay about 3.5 % more for halo rows and
+// per-work-group set-up (measured on 32 x 64 x 56 x 56: 7 strips of 8 rows 68.4 us, 8 strips of 7 rows 70.9 us
+// with 7 tiles a wave, 67.0 us with 6.5); strips of 256 or 128 pixels (4 or 2 tiles per wave) for small images,
+// whose staging of weights per chunk is spread over fewer MFMAs (taken as 8 % and 20 %).
+// DOCC_ROCM_CONV=halo-split / halo-split-wide / halo-whole / halo-t4 / halo-t2 force a form (tests, tuning).
+struct HaloPlan {
+    int tiles = 7;        // column tiles per wave
+    int64_t TH = 1;       // output rows per strip
+    bool split = false, narrow = false;
+    double cost = 0;      // rounds x tiles per wave x overhead
+};
+
+HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int cus) {
+    const int64_t ocb = (OC + 63) / 64;
+    auto rows_for = [&](int64_t pixels) {
+        int64_t th = pixels / OW;
+        if (th > OH) th = OH;
+        if (th >= 1) th = (OH + (OH + th - 1) / th - 1) / ((OH + th - 1) / th);   // the same number of strips, evenly high
+        return th;
+    };
+    auto rounds = [&](int64_t th) { return (double) ((N * ((OH + th - 1) / th) * ocb + cus - 1) / cus); };
+    HaloPlan plan;
+    plan.TH = 448 / OW < OH ? 448 / OW : OH;   // (not evened out: the strips of the whole form stay as high as they can be)
+    if (plan.TH < 1) plan.TH = 1;
+    plan.cost = rounds(plan.TH) * 7.0;
+    const char* force = std::getenv("DOCC_ROCM_CONV");
+    const bool forced = force && std::strncmp(force, "halo-", 5) == 0;
+    if (KH == 3) {
+        int64_t ths = 416 / OW < OH ? 416 / OW : OH;
+        if (ths >= 1) {
+            const bool narrow = ths * OW <= 12 * 32 + 16;
+            const double cost = rounds(ths) * (narrow ? 6.25 : 6.5) * 1.035;
+            bool split = cost < plan.cost;
+            bool narrow_form = narrow;
+            if (forced) {
+                if (std::strncmp(force, "halo-split", 10) == 0) split = true;
+                if (std::strcmp(force, "halo-split-wide") == 0) narrow_form = false;
+                if (std::strcmp(force, "halo-whole") == 0) split = false;
+            }
+            if (split) {
+                plan.TH = ths;
+                plan.split = true;
+                plan.narrow = narrow_form;
+                plan.cost = cost;
+            }
+        }
+    }
+    const struct { int tiles; double overhead; const char* name; } small[2] = {{4, 1.08, "halo-t4"}, {2, 1.20, "halo-t2"}};
+    for (const auto& form : small) {
+        const int64_t th = rows_for(64 * form.tiles);
+        if (th < 1) continue;
+        const double cost = rounds(th) * form.tiles * form.overhead;
+        const bool take = forced ? std::strcmp(force, form.name) == 0 : cost < plan.cost;
+        if (take) {
+            plan.tiles = form.tiles;
+            plan.TH = th;
+            plan.split = plan.narrow = false;
+            plan.cost = cost;
+        }
+    }
+    return plan;
+}
+
+// Rough times (us) of the three ways to run a layer, from what the kernels were measured to sustain: the halo kernel
+// about 490 GFLOP/s per CU on the tiles it computes. The gather kernel sustains about 55 TFLOP/s when its 64 x 128
+// tiles fill the CUs evenly. The GEMM on a column matrix runs at
+// about 75 TFLOP/s on these shapes; the columns are written and read once at about 5 TB/s, and the extra launches
+// (columns, bias, transpose) cost about 15 us.
+double halo_time_us(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int64_t K, int cus) {
+    return plan_halo(N, OC, OH, OW, KH, cus).cost * (2.0 * 64 * 64 * (double) K) / 490e3;
 }
 
 double gather_time_us(int64_t N, int64_t OC, int64_t P, int64_t K, int cus) {
     const int64_t tiles = ((OC + 63) / 64) * ((N * P + 127) / 128);
     const int64_t rounds = (tiles + cus - 1) / cus;
-    return (double) rounds * cus * (2.0 * 64 * 128 * (double) K) / 55e6;
+    // past K = 1152 (128 channels of a 3x3 kernel) a tile's share of the input no longer stays close: 35 TFLOP/s at K = 2304
+    const double rate = 55e6 * (K > 1152 ? std::pow(1152.0 / (double) K, 0.65) : 1.0);
+    return (double) rounds * cus * (2.0 * 64 * 128 * (double) K) / rate;
 }
 
 double gemm_time_us(int64_t N, int64_t OC, int64_t P, int64_t K, bool needs_columns) {
@@ -85,7 +152,7 @@ ConvPath choose_path(int64_t N, int64_t C, int64_t OC, int64_t KH, int64_t KW, i
     // 1x1 layers move more bytes than they compute, which the models above do not see: measured, the batched GEMM
     // wins from 128 input channels on (C 256 -> 64 on 56 x 56: 50 against 65 us; C 64 -> 256: 99 against 74)
     if (pointwise) return gemm_fast && C >= 128 ? gemm : halo_ok ? ConvPath::Halo : ConvPath::Gather;
-    const double direct = halo_ok ? halo_time_us(N, OC, OH, OW, K, cus) : gather_time_us(N, OC, P, K, cus);
+    const double direct = halo_ok ? halo_time_us(N, OC, OH, OW, KH, K, cus) : gather_time_us(N, OC, P, K, cus);
     if (gemm_fast && gemm_time_us(N, OC, P, K, true) < 0.75 * direct) return gemm;
     return halo_ok ? ConvPath::Halo : ConvPath::Gather;
 }
@@ -191,41 +258,18 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         return 0;
     }
     if (path == ConvPath::Halo) {
-        int64_t TH = 448 / OW;
-        if (TH > OH) TH = OH;
-        // The 3x3 kernel also comes with strips of 13 column tiles (416 pixels), of which a wave multiplies 6.5 instead
-        // of 7 (the two pixel groups share the thirteenth). A launch takes rounds-of-work-groups x tiles-per-wave;
-        // the shorter strips pay about 3.5 % more for halo rows and per-work-group set-up (measured on 32 x 64 x 56 x 56:
-        // 7 strips of 8 rows 68.4 us, 8 strips of 7 rows 70.9 us with 7 tiles a wave, 67.0 us with 6.5).
-        // DOCC_ROCM_CONV=halo-split / halo-whole force one of the two (tests, tuning).
-        // A thirteenth tile with at most 16 pixels of the strip (8 of 7 x 56) goes through the 16-pixel MFMA at half the
-        // cost: 6.25 tiles a wave (_split16; DOCC_ROCM_CONV=halo-split-wide keeps the 32-pixel form).
-        bool split = false, narrow = false;
-        if (KH == 3) {
-            int64_t THs = 416 / OW;
-            if (THs > OH) THs = OH;
-            if (THs >= 1) {
-                int cus = compute_units();
-                if (cus <= 0) cus = 256;
-                const int64_t ocb = (OC + 63) / 64;
-                auto rounds = [&](int64_t th) { return (double) ((N * ((OH + th - 1) / th) * ocb + cus - 1) / cus); };
-                narrow = THs * OW <= 12 * 32 + 16;
-                split = rounds(THs) * (narrow ? 6.25 : 6.5) * 1.035 < rounds(TH) * 7.0;
-                if (const char* force = std::getenv("DOCC_ROCM_CONV")) {
-                    if (std::strncmp(force, "halo-split", 10) == 0) split = true;
-                    if (std::strcmp(force, "halo-split-wide") == 0) narrow = false;
-                    if (std::strcmp(force, "halo-whole") == 0) split = false;
-                }
-                if (split) TH = THs;
-            }
-        }
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        const HaloPlan plan = plan_halo(N, OC, OH, OW, KH, cus);
+        const int64_t TH = plan.TH;
         const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch pixels
         const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
         if (PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
-            return launch(KH == 3 ? (split ? (narrow ? "docc_conv2d_f32_halo_3x3_split16" : "docc_conv2d_f32_halo_3x3_split") : "docc_conv2d_f32_halo_3x3")
-                                  : "docc_conv2d_f32_halo_1x1",
-                          (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
+            char name[64];
+            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s", KH == 3 ? "3x3" : "1x1",
+                          plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "");
+            return launch(name, (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
         }
     }
     constexpr int BM = 64, BN = 128, BK = 16;

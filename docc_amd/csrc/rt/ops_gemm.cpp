@@ -264,6 +264,33 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     if (cfg.stages > 0 && !(aligned && offsets_fit)) cfg = pick(m, n, batch, false, 0);
     const int64_t tiles = ((m + cfg.bm - 1) / cfg.bm) * ((n + cfg.bn - 1) / cfg.bn);
     if (tiles > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "%s: too many tiles", prefix);
+    // Few output tiles and a long K extent (a handful of rows against a wide matrix: the product is bound by reading
+    // that matrix, and a work-group per tile reads it on a few CUs only): K is cut into parts, each part's product is
+    // one entry of a batched launch into the stream's buffer of partial results, and a second launch adds the parts
+    // (in order: the result does not depend on the device's scheduling). DOCC_ROCM_GEMM_SPLITK=0 switches it off,
+    // another number forces that many parts where K allows it (tests, tuning).
+    if (batch == 1 && !epilogue && aligned && k >= 1024) {
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        const char* env = std::getenv("DOCC_ROCM_GEMM_SPLITK");
+        const int64_t wanted = env ? std::atoll(env) : (2 * tiles <= cus ? 2 * (int64_t) cus / tiles : 1);
+        int64_t splits = 1;
+        while (splits * 2 <= wanted && splits * 2 <= 64 && k % (splits * 2) == 0 && (k / (splits * 2)) % 64 == 0 && k / (splits * 2) >= 256 &&
+               splits * 2 * m * n * (int64_t) sizeof(S) <= (int64_t) kPartialsBytes)
+            splits *= 2;
+        if (splits >= 2) {
+            PartialsLease partials;
+            if ((rc = partials_for(s, &partials))) return rc;
+            const int64_t part = k / splits;
+            rc = gemm_launch<T, S>(prefix, stream, trans_a, trans_b, m, n, part, (S) 1, A, lda, B, ldb, (S) 0, (S*) partials.ptr, n, pick, nullptr, -1,
+                                   splits, ta ? part * lda : part, tb ? part : part * ldb, m * n);
+            if (rc) return rc;
+            int64_t blocks = (m * n + 255) / 256;
+            if (blocks > 4096) blocks = 4096;
+            return launch(sizeof(S) == 8 ? "docc_splitk_combine_f64" : "docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s,
+                          (const S*) partials.ptr, C, (long) m, (long) n, (long) ldc, (int) splits, alpha, beta);
+        }
+    }
     size_t lds;
     if (cfg.stages > 0) {
         std::snprintf(name, sizeof(name), "docc_%sa_%dx%dx%d%c%d_%c%c", prefix, cfg.bm, cfg.bn, cfg.bk, cfg.small ? 'q' : cfg.spread ? 'p' : 's', cfg.stages,

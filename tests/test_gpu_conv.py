@@ -43,6 +43,10 @@ CASES = [
     (2, 32, 12, 12, 16, 1, 1, (1, 1), (0, 0), (1, 1), True),    # 1x1
     (1, 8, 3, 448, 8, 3, 3, (1, 1), (1, 1), (1, 1), False),     # one row per strip
     (2, 32, 14, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),    # 7 rows of 56: 13 column tiles, the last shared by two waves
+    (2, 16, 28, 28, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),    # small images: strips of 8 or 4 column tiles fill the device better
+    (3, 24, 14, 14, 96, 3, 3, (1, 1), (1, 1), (1, 1), False),
+    (2, 32, 7, 7, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),      # 49 pixels: one pixel group of the smallest strip works alone
+    (2, 32, 14, 14, 70, 1, 1, (1, 1), (0, 0), (1, 1), True),
 ]
 
 
@@ -146,13 +150,13 @@ def run_conv_ws(rt, X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1),
     return host(y), need
 
 
-@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-split-wide", "halo-whole", ""])
+@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-split-wide", "halo-whole", "halo-t4", "halo-t2", ""])
 @pytest.mark.parametrize("case", CASES)
 def test_conv_every_path_integer_exact(rt, monkeypatch, force, case):
     """Each way to run a layer (forced through DOCC_ROCM_CONV; a path that does not apply falls back; halo-split and
     halo-whole are the LDS-halo kernel with strips of 13 shared and 14 whole column tiles, halo-split-wide keeps the
-    shared tile 32 pixels wide where the 16-pixel form would apply) and the automatic choice
-    give the oracle's integers."""
+    shared tile 32 pixels wide where the 16-pixel form would apply, halo-t4 and halo-t2 are the strips of 8 and 4 column
+    tiles for small images) and the automatic choice give the oracle's integers."""
     N, C, H, W, OC, KH, KW, stride, pad, dil, use_bias = case
     if force:
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
@@ -166,7 +170,7 @@ def test_conv_every_path_integer_exact(rt, monkeypatch, force, case):
 
 GEMM_LAYERS = [  # small images with many channels: the shapes the choice sends to im2col + GEMM, and a 1x1 layer with C >= 128
     (8, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1), (1, 1), True), (8, 512, 7, 7, 512, 3, 3, (1, 1), (1, 1), (1, 1), True),
-    (1, 64, 56, 56, 64, 3, 3, (1, 1), (1, 1), (1, 1), False), (4, 256, 28, 28, 64, 1, 1, (1, 1), (0, 0), (1, 1), True),
+    (1, 256, 14, 14, 256, 3, 3, (1, 1), (1, 1), (1, 1), False), (4, 256, 28, 28, 64, 1, 1, (1, 1), (0, 0), (1, 1), True),
     (3, 128, 9, 9, 96, 3, 3, (2, 2), (1, 1), (1, 1), True),
 ]
 
