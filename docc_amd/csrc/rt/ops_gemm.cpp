@@ -273,22 +273,66 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         int cus = compute_units();
         if (cus <= 0) cus = 256;
         const char* env = std::getenv("DOCC_ROCM_GEMM_SPLITK");
-        const int64_t wanted = env ? std::atoll(env) : (2 * tiles <= cus ? 2 * (int64_t) cus / tiles : 1);
+        // the parts' products: in the stream's buffer of partial results where they fit, else in a block of the device
+        // block cache (taken and returned in stream order), up to 64 MiB
+        constexpr int64_t kMaxPartBytes = int64_t(64) << 20;
+        auto allowed = [&](int64_t parts) {
+            return parts <= 64 && k % parts == 0 && (k / parts) % 64 == 0 && k / parts >= 256 && parts * m * n * (int64_t) sizeof(S) <= kMaxPartBytes;
+        };
+        // Estimated seconds of the product in `parts` parts on the tile the picker gives that many matrices: the work of
+        // the padded tiles at what the tile sustains (relative to the 128 x 256 one) on the share of the CUs that get a
+        // work-group, plus writing and reading the parts at 5 TB/s and a second launch.
+        auto seconds = [&](const TileConfig& c, int64_t parts) {
+            const double tm = (double) ((m + c.bm - 1) / c.bm), tn = (double) ((n + c.bn - 1) / c.bn);
+            const double area = (double) c.bm * c.bn;
+            const double rel = area >= 65536 ? 1.03 : area >= 32768 ? 1.0 : area >= 16384 ? 0.97 : 0.75;
+            const double fill = tm * tn * (double) parts / cus;
+            const double rate = sizeof(T) == 8 ? 68e12 : sizeof(T) == 4 ? 141e12 : 1.25e15;
+            double t = 2.0 * tm * c.bm * tn * c.bn * (double) k / (rate * rel * (fill < 1.0 ? fill : 1.0));
+            if (parts > 1) t += 2.0 * (double) parts * (double) m * (double) n * sizeof(S) / 5e12 + 3e-6;
+            return t;
+        };
         int64_t splits = 1;
-        while (splits * 2 <= wanted && splits * 2 <= 64 && k % (splits * 2) == 0 && (k / (splits * 2)) % 64 == 0 && k / (splits * 2) >= 256 &&
-               splits * 2 * m * n * (int64_t) sizeof(S) <= (int64_t) kPartialsBytes)
-            splits *= 2;
+        if (env) {
+            const int64_t wanted = std::atoll(env);
+            while (splits * 2 <= wanted && allowed(splits * 2)) splits *= 2;
+        } else if (tiles < cus) {   // CUs without a work-group: the case parts are for
+            double best = seconds(cfg, 1);
+            for (int64_t parts = 2; allowed(parts); parts *= 2) {
+                const TileConfig c = pick(m, n, parts, true, 0);
+                if (c.stages == 0) break;
+                const double t = seconds(c, parts);
+                if (t < 0.9 * best) {   // only for a clear gain: the estimate is rough
+                    best = t;
+                    splits = parts;
+                }
+            }
+        }
         if (splits >= 2) {
-            PartialsLease partials;
-            if ((rc = partials_for(s, &partials))) return rc;
+            const int64_t bytes = splits * m * n * (int64_t) sizeof(S);
+            PartialsLease lease;
+            void* parts = nullptr;
+            const bool own_block = bytes > (int64_t) kPartialsBytes;
+            if (own_block) {
+                if ((rc = docc_rocm_malloc_async(&parts, (size_t) bytes, stream))) return rc;
+            } else {
+                if ((rc = partials_for(s, &lease))) return rc;
+                parts = lease.ptr;
+            }
             const int64_t part = k / splits;
-            rc = gemm_launch<T, S>(prefix, stream, trans_a, trans_b, m, n, part, (S) 1, A, lda, B, ldb, (S) 0, (S*) partials.ptr, n, pick, nullptr, -1,
-                                   splits, ta ? part * lda : part, tb ? part : part * ldb, m * n);
-            if (rc) return rc;
-            int64_t blocks = (m * n + 255) / 256;
-            if (blocks > 4096) blocks = 4096;
-            return launch(sizeof(S) == 8 ? "docc_splitk_combine_f64" : "docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s,
-                          (const S*) partials.ptr, C, (long) m, (long) n, (long) ldc, (int) splits, alpha, beta);
+            rc = gemm_launch<T, S>(prefix, stream, trans_a, trans_b, m, n, part, (S) 1, A, lda, B, ldb, (S) 0, (S*) parts, n, pick, nullptr, -1, splits,
+                                   ta ? part * lda : part, tb ? part : part * ldb, m * n);
+            if (!rc) {
+                int64_t blocks = (m * n + 255) / 256;
+                if (blocks > 4096) blocks = 4096;
+                rc = launch(sizeof(S) == 8 ? "docc_splitk_combine_f64" : "docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s, (const S*) parts, C,
+                            (long) m, (long) n, (long) ldc, (int) splits, alpha, beta);
+            }
+            if (own_block) {
+                const int rc2 = docc_rocm_free_async(parts, stream);
+                if (!rc) rc = rc2;
+            }
+            return rc;
         }
     }
     size_t lds;

@@ -55,6 +55,19 @@ def test_bgemm_with_k_in_parts(rt, ta, tb, m, n, k):
     assert np.array_equal(C, oracle.gemm_bf16(Ab, Bb, C=C0.copy(), alpha=0.5, beta=2.0, trans_a=ta, trans_b=tb))
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("m,n,k", [(512, 1568, 4608), (256, 4096, 4096)])
+def test_gemm_parts_larger_than_the_streams_buffer(rt, dt, m, n, k):
+    """More than 8 MiB of parts: they live in a block of the device block cache for the call. Integer-valued operands
+    against numpy's product in float64 (exact on both sides)."""
+    rng = np.random.default_rng(m + k)
+    A, B = int_matrix(rng, (m, k), dt, lim=3), int_matrix(rng, (k, n), dt, lim=3)
+    C0 = int_matrix(rng, (m, n), dt)
+    expect = (A.astype(np.float64) @ B.astype(np.float64) - 2.0 * C0).astype(dt)
+    for _ in range(2):      # the second call finds the block in the cache
+        assert np.array_equal(run_gemm(rt, A, B, C=C0.copy(), alpha=1.0, beta=-2.0), expect)
+
+
 def test_gemm_parts_on_two_streams_do_not_share_partial_results(rt):
     """The parts' products live in the stream's own buffer: the same shape on two streams at once."""
     rng = np.random.default_rng(3)
