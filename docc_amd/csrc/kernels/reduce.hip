@@ -7,7 +7,9 @@
 // `-INFINITY` and fmax, min_node.cpp `INFINITY` and fmin; Mean is Sum followed by a division by
 // the number of reduced elements, mean_node.cpp). Here the input is seen as [outer, reduce, inner]:
 //   inner == 1  one wavefront per output element: 128-bit loads strided over the wave, a tree
-//               over the lanes at the end (HBM-bound: one read of X)
+//               over the lanes at the end (HBM-bound: one read of X); long rows that are too few
+//               to give every CU its wavefronts are cut into pieces, a wavefront each, whose
+//               results a second launch reduces
 //   inner  > 1  one lane per output element, walking the reduced extent with stride `inner`, so
 //               that neighbouring lanes read neighbouring addresses; when there are too few
 //               output elements to fill the device the reduced extent is cut into slices, one
@@ -48,14 +50,12 @@ __device__ __forceinline__ T wave_combine(T v) {
     return v;
 }
 
-// Y[row] = reduce over X[row, 0..R); nvec = R / VEC when rows are 16-byte aligned, else 0
+// the wavefront's reduction over x[0..R), in every lane; nvec = R / VEC when x is 16-byte aligned, else 0
 template <typename T, int OP, int VEC>
-__device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, long nvec) {
+__device__ __forceinline__ T wave_row(const T* x, long R, long nvec) {
     typedef T V __attribute__((ext_vector_type(VEC)));
     const int lane = threadIdx.x & 63;
-    const long waves = (long) gridDim.x * (256 >> 6);
-    for (long row = (long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
-        const T* x = X + row * R;
+    {   // (a block of its own: the vector loop's index is declared again by the element loop below)
         T acc[VEC];
 #pragma unroll
         for (int e = 0; e < VEC; e++) acc[e] = reduce_identity<OP, T>();
@@ -80,7 +80,79 @@ __device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, 
 #pragma unroll
         for (int e = 1; e < VEC; e++) a = combine<OP>(a, acc[e]);
         for (long i = nvec * VEC + lane; i < R; i += kWave) a = combine<OP>(a, x[i]);
-        a = wave_combine<OP>(a);
+        return wave_combine<OP>(a);
+    }
+}
+
+// Y[row] = reduce over X[row, 0..R); nvec = R / VEC when rows are 16-byte aligned, else 0
+template <typename T, int OP, int VEC>
+__device__ __forceinline__ void row_reduce(const T* X, T* Y, long rows, long R, long nvec) {
+    const int lane = threadIdx.x & 63;
+    const long waves = (long) gridDim.x * (256 >> 6);
+    for (long row = (long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const T a = wave_row<T, OP, VEC>(X + row * R, R, nvec);
+        if (lane == 0) Y[row] = OP == kMean ? a / (T) R : a;
+    }
+}
+
+// Short rows (at most 32 vectors, 16-byte aligned): LPR lanes a row with one vector each, 64 / LPR rows per wavefront and
+// four such sets in turn, all loaded before the first is reduced; a wavefront per row would leave most lanes idle.
+template <typename T, int OP, int VEC, int LPR>
+__device__ __forceinline__ void row_reduce_short(const T* X, T* Y, long rows, long R) {
+    typedef T V __attribute__((ext_vector_type(VEC)));
+    constexpr int RPW = kWave / LPR, SETS = 4;
+    const int lane = threadIdx.x & 63, l = lane % LPR, g = lane / LPR;
+    const int nvec = (int) (R / VEC);
+    const long first = ((long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6)) * (RPW * SETS) + g;
+    const V* xv = reinterpret_cast<const V*>(X);
+    V v[SETS];
+    bool live[SETS];
+#pragma unroll
+    for (int i = 0; i < SETS; i++) {
+        const long row = first + (long) i * RPW;
+        live[i] = row < rows && l < nvec;
+        if (live[i]) v[i] = __builtin_nontemporal_load(xv + row * nvec + l);
+    }
+#pragma unroll
+    for (int i = 0; i < SETS; i++) {
+        T a = reduce_identity<OP, T>();
+        if (live[i]) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++) a = combine<OP>(a, v[i][e]);
+        }
+#pragma unroll
+        for (int off = LPR / 2; off >= 1; off >>= 1) a = combine<OP>(a, __shfl_xor(a, off, kWave));
+        const long row = first + (long) i * RPW;
+        if (l == 0 && row < rows) Y[row] = OP == kMean ? a / (T) R : a;
+    }
+}
+
+// Rows too few to give every CU its wavefronts: a row is cut into `slices` pieces of `chunk` elements (a multiple of
+// the vector; the last piece may be shorter), a wavefront reduces a piece into P[row, slice], and a second launch
+// reduces the rows of P (Mean: adds in both, and divides by the row length at the end). `vec`: rows start on
+// 16-byte boundaries.
+template <typename T, int OP, int VEC>
+__device__ __forceinline__ void row_reduce_pieces(void* partials, const T* X, long rows, long R, long chunk, long slices, int vec) {
+    constexpr int PART = OP == kMean ? kSum : OP;
+    T* P = reinterpret_cast<T*>(partials);
+    const int lane = threadIdx.x & 63;
+    const long waves = (long) gridDim.x * (256 >> 6), pieces = rows * slices;
+    for (long piece = (long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6); piece < pieces; piece += waves) {
+        const long row = piece / slices, c0 = (piece % slices) * chunk;
+        const long len = c0 + chunk < R ? chunk : R - c0;
+        const T a = wave_row<T, PART, VEC>(X + row * R + c0, len, vec ? len / VEC : 0);
+        if (lane == 0) P[piece] = a;
+    }
+}
+
+template <typename T, int OP>
+__device__ __forceinline__ void row_reduce_finish(const void* partials, T* Y, long rows, long R, long slices) {
+    constexpr int PART = OP == kMean ? kSum : OP;
+    const T* P = reinterpret_cast<const T*>(partials);
+    const int lane = threadIdx.x & 63;
+    const long waves = (long) gridDim.x * (256 >> 6);
+    for (long row = (long) blockIdx.x * (256 >> 6) + (threadIdx.x >> 6); row < rows; row += waves) {
+        const T a = wave_row<T, PART, 1>(P + row * slices, slices, 0);
         if (lane == 0) Y[row] = OP == kMean ? a / (T) R : a;
     }
 }
@@ -231,10 +303,41 @@ __device__ __forceinline__ void dot_final(void* partials, int groups) {
 DOCC_DOT(f32, float)
 DOCC_DOT(f64, double)
 
+#define DOCC_REDUCE_SHORT(NAME, OP, LPR)                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rows##LPR##_##NAME##_f32(const float* X, float* Y, long rows, long R) { \
+        docc_k::row_reduce_short<float, docc_k::OP, 4, LPR>(X, Y, rows, R);                                                    \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rows##LPR##_##NAME##_f64(const double* X, double* Y, long rows, long R) { \
+        docc_k::row_reduce_short<double, docc_k::OP, 2, LPR>(X, Y, rows, R);                                                   \
+    }
+#define DOCC_REDUCE_SHORT_ALL(NAME, OP) \
+    DOCC_REDUCE_SHORT(NAME, OP, 1) DOCC_REDUCE_SHORT(NAME, OP, 2) DOCC_REDUCE_SHORT(NAME, OP, 4) DOCC_REDUCE_SHORT(NAME, OP, 8) \
+    DOCC_REDUCE_SHORT(NAME, OP, 16) DOCC_REDUCE_SHORT(NAME, OP, 32)
+DOCC_REDUCE_SHORT_ALL(sum, kSum)
+DOCC_REDUCE_SHORT_ALL(max, kMax)
+DOCC_REDUCE_SHORT_ALL(min, kMin)
+DOCC_REDUCE_SHORT_ALL(mean, kMean)
+
 #define DOCC_REDUCE(NAME, OP)                                                                                                  \
     extern "C" __global__ __launch_bounds__(256) void docc_reduce_row_##NAME##_f32(const float* X, float* Y, long rows, long R,   \
                                                                                    long nvec) {                                \
         docc_k::row_reduce<float, docc_k::OP, 4>(X, Y, rows, R, nvec);                                                         \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rowp_##NAME##_f32(void* P, const float* X, long rows, long R,   \
+                                                                                    long chunk, long slices, int vec) {        \
+        docc_k::row_reduce_pieces<float, docc_k::OP, 4>(P, X, rows, R, chunk, slices, vec);                                    \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rowp_##NAME##_f64(void* P, const double* X, long rows, long R,  \
+                                                                                    long chunk, long slices, int vec) {        \
+        docc_k::row_reduce_pieces<double, docc_k::OP, 2>(P, X, rows, R, chunk, slices, vec);                                   \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rowf_##NAME##_f32(const void* P, float* Y, long rows, long R,   \
+                                                                                    long slices) {                             \
+        docc_k::row_reduce_finish<float, docc_k::OP>(P, Y, rows, R, slices);                                                   \
+    }                                                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_reduce_rowf_##NAME##_f64(const void* P, double* Y, long rows, long R,  \
+                                                                                    long slices) {                             \
+        docc_k::row_reduce_finish<double, docc_k::OP>(P, Y, rows, R, slices);                                                  \
     }                                                                                                                          \
     extern "C" __global__ __launch_bounds__(256) void docc_reduce_row_##NAME##_f64(const double* X, double* Y, long rows, long R, \
                                                                                    long nvec) {                                \

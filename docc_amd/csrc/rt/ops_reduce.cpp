@@ -28,6 +28,38 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
         // every row starts on a 16-byte boundary
         const bool aligned = (uintptr_t) X % 16 == 0 && (reduce * elem) % 16 == 0;
         const long nvec = aligned ? (long) (reduce / per_vec) : 0;
+        // short rows: several share a wavefront (1 to 32 lanes a row, four sets of rows per wavefront, four wavefronts)
+        if (aligned && nvec >= 1 && nvec <= 32 && outer >= 64) {
+            int lpr = 1;
+            while (lpr < nvec) lpr *= 2;
+            const int64_t per_group = 4 * 4 * (64 / lpr);
+            std::snprintf(name, sizeof(name), "docc_reduce_rows%d_%s_f%d", lpr, names[op], precision);
+            return launch(name, (uint32_t) ((outer + per_group - 1) / per_group), 1, 1, 256, 0, (hipStream_t) stream, X, Y, (long) outer, (long) reduce);
+        }
+        // Long rows, and too few of them for eight wavefronts per CU: each row in pieces of at least 4096 elements, one
+        // wavefront a piece, the pieces' results through the stream's buffer of partial results and a second launch
+        if (outer < (int64_t) cus * 8 && reduce >= 8192) {
+            int64_t slices = ((int64_t) cus * 8 + outer - 1) / outer;
+            if (slices > reduce / 4096) slices = reduce / 4096;
+            if (slices > 4096) slices = 4096;
+            const int64_t chunk = ((reduce + slices - 1) / slices + 1023) / 1024 * 1024;
+            slices = (reduce + chunk - 1) / chunk;
+            if (slices > 1 && outer * slices * (int64_t) elem <= (int64_t) kPartialsBytes) {
+                PartialsLease partials;
+                if (int rc = partials_for((hipStream_t) stream, &partials)) return rc;
+                const int64_t pieces = outer * slices;
+                int64_t groups = (pieces + 3) / 4;
+                if (groups > (int64_t) cus * 16) groups = (int64_t) cus * 16;
+                std::snprintf(name, sizeof(name), "docc_reduce_rowp_%s_f%d", names[op], precision);
+                if (int rc = launch(name, (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, partials.ptr, X, (long) outer, (long) reduce, (long) chunk,
+                                    (long) slices, aligned ? 1 : 0))
+                    return rc;
+                groups = (outer + 3) / 4;
+                std::snprintf(name, sizeof(name), "docc_reduce_rowf_%s_f%d", names[op], precision);
+                return launch(name, (uint32_t) groups, 1, 1, 256, 0, (hipStream_t) stream, (const void*) partials.ptr, Y, (long) outer, (long) reduce,
+                              (long) slices);
+            }
+        }
         int64_t blocks = (outer + 3) / 4;   // four wavefronts per work-group, one row each
         if (blocks > (int64_t) cus * 16) blocks = (int64_t) cus * 16;
         std::snprintf(name, sizeof(name), "docc_reduce_row_%s_f%d", names[op], precision);
@@ -42,10 +74,12 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
         const bool vec = inner % per_vec == 0 && (uintptr_t) X % 16 == 0;
         const int64_t pblocks = vec ? (total / per_vec + 255) / 256 : blocks;
         const int64_t scratch_elems = (int64_t) kPartialsBytes / (precision / 8);
-        int64_t slices = ((int64_t) cus * 8 + pblocks - 1) / pblocks;
+        // about three work-groups per CU: measured on [64, 1024, 512], [512, 512, 128], [8, 4096, 2048] and [1, 8192, 4096], twice as
+        // many slices cost 5-30 % (the second launch reads them all), half as many leave CUs without work
+        int64_t slices = ((int64_t) cus * 3 + pblocks - 1) / pblocks;
         if (slices > reduce / 16) slices = reduce / 16;
         if (slices > scratch_elems / total) slices = scratch_elems / total;
-        int64_t cap = 256;
+        int64_t cap = 1024;
         if (const char* e = std::getenv("DOCC_ROCM_REDUCE_SLICES")) cap = std::atoll(e) > 0 ? std::atoll(e) : cap;   // tuning
         if (slices > cap) slices = cap;
         if (slices > 1) {

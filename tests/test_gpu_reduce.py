@@ -16,7 +16,9 @@ pytestmark = pytest.mark.gpu
 # (shape, reduced axes)
 CASES = [((8192, 4096), (1,)), ((4096, 8192), (0,)), ((16, 16, 128, 128), (3,)), ((32, 64, 56, 56), (2, 3)), ((32, 64, 56, 56), (0,)),
          ((7, 33), (1,)), ((7, 33), (0,)), ((5, 1, 9), (1,)), ((3, 1000003), (1,)), ((1, 17), (0, 1)), ((2, 3, 4, 5), (1, 2)),
-         ((64, 4099), (1,)), ((6, 0, 4), (1,)), ((100000, 24), (0,)), ((3, 5000, 40), (1,))]      # the last two: sliced column reductions
+         ((64, 4099), (1,)), ((6, 0, 4), (1,)), ((100000, 24), (0,)), ((3, 5000, 40), (1,)),      # the last two: sliced column reductions
+         ((1, 1 << 22), (1,)), ((5, 40000), (1,)), ((2, 3, 8192), (1, 2)), ((300, 9000), (1,)),    # long rows, few of them: each row in pieces
+         ((1000, 4), (1,)), ((777, 8), (1,)), ((4099, 32), (1,)), ((65, 12, 5), (1, 2)), ((300, 100), (1,)), ((1025, 128), (1,))]   # short rows share a wavefront
 
 
 def run(rt, op, x, axes, offset=0):
@@ -47,6 +49,8 @@ def test_reduce_against_the_oracle(rt, dt, case):
         assert np.array_equal(run(rt, op, x, axes), oracle.reduce(op, x, axes)), op
     ints = rng.integers(-8, 9, shape).astype(dt)
     assert np.array_equal(run(rt, "sum", ints, axes), oracle.reduce("sum", ints, axes))
+    if extent:
+        assert np.array_equal(run(rt, "mean", ints, axes), oracle.reduce("mean", ints, axes))      # an exact sum, divided once
     eps = np.finfo(dt).eps
     scale = np.abs(x).sum(axis=tuple(axes)) + 1e-30
     got, ref = run(rt, "sum", x, axes), oracle.reduce("sum", x, axes)
