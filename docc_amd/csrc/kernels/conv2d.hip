@@ -195,7 +195,7 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, true, a)
 DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 
 // ---------------------------------------------------------------------------------------------
-// Stride-1, dilation-1 convolution with LDS-staged input halos.
+// Dilation-1 convolution with LDS-staged input halos (stride 1; strides of 2 with the small strips, whose patch still fits).
 //
 // One work-group computes 64 output channels x a strip of TH full output rows of one image
 // (TH*OW <= 448 pixels = 14 MFMA column tiles). Wave w takes output-channel tile (w & 1) and
@@ -255,7 +255,7 @@ struct ConvHaloKernel {
         const int l32 = lane & 31, g = lane >> 5;
         const int ocw = wave & 1, pg = wave >> 1;
 
-        const int WP = p.OW + KW - 1, PR = TH + KH - 1, PS = PR * WP;
+        const int WP = (p.OW - 1) * p.stride_w + KW, PR = (TH - 1) * p.stride_h + KH, PS = PR * WP;   // the patch a strip reads
         const int stage_elems = A_ELEMS + (PS + 1) * CI;    // [weights | patch | one spare pixel]
         const int strips = (p.OH + TH - 1) / TH;
         const int n = blockIdx.x / strips, oh0 = (blockIdx.x % strips) * TH;
@@ -273,7 +273,7 @@ struct ConvHaloKernel {
             for (int j = 0; j < TN; j++) {
                 int q = tile_pixel0(j) + l32;
                 q = q < npix ? q : 0;
-                boff[j] = ((q / p.OW) * WP + (q % p.OW)) * CI + 4 * g;
+                boff[j] = ((q / p.OW) * p.stride_h * WP + (q % p.OW) * p.stride_w) * CI + 4 * g;
             }
         };
 
@@ -286,7 +286,7 @@ struct ConvHaloKernel {
 #pragma unroll
         for (int r = 0; r < NR; r++) {
             const int e = tid + r * 256;
-            const int ih = oh0 - p.pad_h + e / WP, iw = e % WP - p.pad_w;
+            const int ih = oh0 * p.stride_h - p.pad_h + e / WP, iw = e % WP - p.pad_w;
             inside[r] = e < PS && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
             goff[r] = inside[r] ? 4u * (unsigned) (ih * p.W + iw) : 0u;
             slot[r] = (e < PS ? e : PS) * CI;
@@ -371,7 +371,7 @@ struct ConvHaloKernel {
             if constexpr (NARROW) {
                 int q = 2 * TOWN * 32 + (lane & 15);
                 q = q < npix ? q : 0;
-                boffn = ((q / p.OW) * WP + (q % p.OW)) * CI + (lane >> 4);
+                boffn = ((q / p.OW) * p.stride_h * WP + (q % p.OW) * p.stride_w) * CI + (lane >> 4);
             }
         };
         static_assert(!SPLIT || KHW % 2 == 1, "the shared tile is halved in the middle tap");

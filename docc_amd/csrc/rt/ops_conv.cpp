@@ -50,8 +50,17 @@ struct HaloPlan {
     double cost = 0;      // rounds x tiles per wave x overhead
 };
 
-HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int cus) {
+// whether a strip of `th` rows fits: at most three patch pixels per lane and chunk, three stages in 160 KB of LDS
+bool halo_strip_fits(int64_t th, int64_t OW, int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w) {
+    const int64_t PS = ((th - 1) * stride_h + KH) * ((OW - 1) * stride_w + KW);
+    const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);
+    return PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024;
+}
+
+// cost 0: no form of the kernel fits the layer
+HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int cus) {
     const int64_t ocb = (OC + 63) / 64;
+    auto fits = [&](int64_t th) { return th >= 1 && halo_strip_fits(th, OW, KH, KW, stride_h, stride_w); };
     auto rows_for = [&](int64_t pixels) {
         int64_t th = pixels / OW;
         if (th > OH) th = OH;
@@ -62,15 +71,15 @@ HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, in
     HaloPlan plan;
     plan.TH = 448 / OW < OH ? 448 / OW : OH;   // (not evened out: the strips of the whole form stay as high as they can be)
     if (plan.TH < 1) plan.TH = 1;
-    plan.cost = rounds(plan.TH) * 7.0;
+    plan.cost = fits(plan.TH) ? rounds(plan.TH) * 7.0 : 0.0;
     const char* force = std::getenv("DOCC_ROCM_CONV");
     const bool forced = force && std::strncmp(force, "halo-", 5) == 0;
     if (KH == 3) {
         int64_t ths = 416 / OW < OH ? 416 / OW : OH;
-        if (ths >= 1) {
+        if (fits(ths)) {
             const bool narrow = ths * OW <= 12 * 32 + 16;
             const double cost = rounds(ths) * (narrow ? 6.25 : 6.5) * 1.035;
-            bool split = cost < plan.cost;
+            bool split = cost < plan.cost || plan.cost == 0.0;
             bool narrow_form = narrow;
             if (forced) {
                 if (std::strncmp(force, "halo-split", 10) == 0) split = true;
@@ -87,10 +96,11 @@ HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, in
     }
     const struct { int tiles; double overhead; const char* name; } small[2] = {{4, 1.08, "halo-t4"}, {2, 1.20, "halo-t2"}};
     for (const auto& form : small) {
-        const int64_t th = rows_for(64 * form.tiles);
-        if (th < 1) continue;
+        int64_t th = rows_for(64 * form.tiles);
+        while (th > 1 && !fits(th)) th--;      // (a strided layer's patch grows with the rows)
+        if (!fits(th)) continue;
         const double cost = rounds(th) * form.tiles * form.overhead;
-        const bool take = forced ? std::strcmp(force, form.name) == 0 : cost < plan.cost;
+        const bool take = forced && plan.cost > 0.0 ? std::strcmp(force, form.name) == 0 : cost < plan.cost || plan.cost == 0.0;
         if (take) {
             plan.tiles = form.tiles;
             plan.TH = th;
@@ -106,8 +116,8 @@ HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, in
 // tiles fill the CUs evenly. The GEMM on a column matrix runs at
 // about 75 TFLOP/s on these shapes; the columns are written and read once at about 5 TB/s, and the extra launches
 // (columns, bias, transpose) cost about 15 us.
-double halo_time_us(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int64_t K, int cus) {
-    return plan_halo(N, OC, OH, OW, KH, cus).cost * (2.0 * 64 * 64 * (double) K) / 490e3;
+double halo_time_us(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, int64_t KW, int64_t stride_h, int64_t stride_w, int64_t K, int cus) {
+    return plan_halo(N, OC, OH, OW, KH, KW, stride_h, stride_w, cus).cost * (2.0 * 64 * 64 * (double) K) / 490e3;
 }
 
 double gather_time_us(int64_t N, int64_t OC, int64_t P, int64_t K, int cus) {
@@ -131,8 +141,8 @@ enum class ConvPath { Halo, Gather, Gemm1x1, GemmColumns };
 
 // shapes the LDS-halo kernel is built for (the launcher also wants 16-byte aligned weights)
 bool halo_shape_ok(int64_t C, int64_t KH, int64_t KW, int64_t OW, int64_t stride_h, int64_t stride_w, int64_t dil_h, int64_t dil_w) {
-    return stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && ((KH == 3 && KW == 3) || (KH == 1 && KW == 1)) && C % 8 == 0 &&
-           C > 0 && OW <= 448 && (C * KH * KW) % 4 == 0;
+    return stride_h >= 1 && stride_h <= 2 && stride_w >= 1 && stride_w <= 2 && dil_h == 1 && dil_w == 1 && ((KH == 3 && KW == 3) || (KH == 1 && KW == 1)) &&
+           C % 8 == 0 && C > 0 && OW <= 448 && (C * KH * KW) % 4 == 0 && halo_strip_fits(1, OW, KH, KW, stride_h, stride_w);
 }
 
 ConvPath choose_path(int64_t N, int64_t C, int64_t OC, int64_t KH, int64_t KW, int64_t OH, int64_t OW, int64_t stride_h, int64_t stride_w,
@@ -152,7 +162,7 @@ ConvPath choose_path(int64_t N, int64_t C, int64_t OC, int64_t KH, int64_t KW, i
     // 1x1 layers move more bytes than they compute, which the models above do not see: measured, the batched GEMM
     // wins from 128 input channels on (C 256 -> 64 on 56 x 56: 50 against 65 us; C 64 -> 256: 99 against 74)
     if (pointwise) return gemm_fast && C >= 128 ? gemm : halo_ok ? ConvPath::Halo : ConvPath::Gather;
-    const double direct = halo_ok ? halo_time_us(N, OC, OH, OW, KH, K, cus) : gather_time_us(N, OC, P, K, cus);
+    const double direct = halo_ok ? halo_time_us(N, OC, OH, OW, KH, KW, stride_h, stride_w, K, cus) : gather_time_us(N, OC, P, K, cus);
     if (gemm_fast && gemm_time_us(N, OC, P, K, true) < 0.75 * direct) return gemm;
     return halo_ok ? ConvPath::Halo : ConvPath::Gather;
 }
@@ -260,12 +270,12 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     if (path == ConvPath::Halo) {
         int cus = compute_units();
         if (cus <= 0) cus = 256;
-        const HaloPlan plan = plan_halo(N, OC, OH, OW, KH, cus);
+        const HaloPlan plan = plan_halo(N, OC, OH, OW, KH, KW, stride_h, stride_w, cus);
         const int64_t TH = plan.TH;
-        const int64_t PS = (TH + KH - 1) * (OW + KW - 1);           // patch pixels
+        const int64_t PS = ((TH - 1) * stride_h + KH) * ((OW - 1) * stride_w + KW);   // patch pixels
         const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
-        if (PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
+        if (plan.cost > 0.0 && halo_strip_fits(TH, OW, KH, KW, stride_h, stride_w) && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
             char name[64];
             std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s", KH == 3 ? "3x3" : "1x1",
                           plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "");

@@ -47,6 +47,10 @@ CASES = [
     (3, 24, 14, 14, 96, 3, 3, (1, 1), (1, 1), (1, 1), False),
     (2, 32, 7, 7, 64, 3, 3, (1, 1), (1, 1), (1, 1), True),      # 49 pixels: one pixel group of the smallest strip works alone
     (2, 32, 14, 14, 70, 1, 1, (1, 1), (0, 0), (1, 1), True),
+    (2, 16, 28, 28, 64, 3, 3, (2, 2), (1, 1), (1, 1), True),    # strides of 2 on the LDS-halo kernel: the patch of a strip covers the skipped pixels too
+    (2, 8, 15, 21, 40, 3, 3, (2, 1), (1, 1), (1, 1), False),    # mixed strides, odd image
+    (2, 32, 14, 14, 64, 1, 1, (2, 2), (0, 0), (1, 1), True),    # a 1x1 downsampling layer
+    (1, 8, 9, 120, 16, 3, 3, (2, 2), (0, 0), (1, 1), True),     # wide rows: one or two output rows per strip
 ]
 
 
