@@ -28,6 +28,18 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
+__device__ __forceinline__ double wave_max(double v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmax(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+
 // exp(t) for t <= 0 through the hardware exp2 with a compensated argument:
 // t*log2(e) is split into its rounded product and the rounding remainder, so
 // the result stays within ~2 ulp down to the underflow threshold.

@@ -6,7 +6,8 @@
 // Max -> Broadcast -> Sub -> Exp -> Sum -> Broadcast -> Div with six
 // temporaries) by one kernel that reads X once and writes Y once.
 //
-// HBM-bound: algorithmic traffic is 8 bytes per element. The shapes of the fp32 row kernels:
+// HBM-bound: algorithmic traffic is 8 bytes per element (16 in fp64). The shapes of the row kernels (one template over
+// the element type; the figures are those of fp32, whose 16-byte vector holds four columns - fp64 halves the widths):
 //   rows sharing a wavefront (cols <= 128, cols % 4 == 0): 1 to 32 lanes a row, 64 to 2 rows per
 //       wavefront and four such sets per wavefront, butterflies inside the lanes of a row;
 //   wave-per-row  (cols <= 1024, cols % 4 == 0; built up to 4096): a 64-lane wavefront
@@ -31,289 +32,284 @@ namespace {
 
 constexpr float kNegInf = -__builtin_huge_valf();
 
-template <int NV>
-__device__ __forceinline__ void softmax_row_wave(const float* __restrict__ x, float* __restrict__ y, int cols, int lane) {
-    const int nvec = cols >> 2;
-    const f32x4* xv = reinterpret_cast<const f32x4*>(x);
-    f32x4* yv = reinterpret_cast<f32x4*>(y);
-    f32x4 v[NV];
+// element type of a row kernel: its 16-byte vector, the exponential of a non-positive argument, the maximum that drops NaNs
+template <typename T> struct SoftmaxMath;
+template <> struct SoftmaxMath<float> {
+    static __device__ __forceinline__ float neg_inf() { return kNegInf; }
+    static __device__ __forceinline__ float exp_le0(float t) { return exp_neg(t); }
+    static __device__ __forceinline__ float max(float a, float b) { return fmaxf(a, b); }
+};
+template <> struct SoftmaxMath<double> {
+    static __device__ __forceinline__ double neg_inf() { return -__builtin_huge_val(); }
+    static __device__ __forceinline__ double exp_le0(double t) { return exp(t); }
+    static __device__ __forceinline__ double max(double a, double b) { return fmax(a, b); }
+};
+template <typename T> struct RowVec;
+template <> struct RowVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
+template <> struct RowVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
+
+template <typename T> __device__ __forceinline__ typename RowVec<T>::type all_neg_inf() {
+    typename RowVec<T>::type v;
+#pragma unroll
+    for (int e = 0; e < RowVec<T>::N; e++) v[e] = SoftmaxMath<T>::neg_inf();
+    return v;
+}
+template <typename T> __device__ __forceinline__ T vec_max(typename RowVec<T>::type v) {
+    T m = v[0];
+#pragma unroll
+    for (int e = 1; e < RowVec<T>::N; e++) m = SoftmaxMath<T>::max(m, v[e]);
+    return m;
+}
+// v = exp(v - m) in place; returns the sum of the results, added in pairs
+template <typename T> __device__ __forceinline__ T vec_exp(typename RowVec<T>::type& v, T m) {
+#pragma unroll
+    for (int e = 0; e < RowVec<T>::N; e++) v[e] = SoftmaxMath<T>::exp_le0(v[e] - m);
+    if constexpr (RowVec<T>::N == 4) return (v[0] + v[1]) + (v[2] + v[3]);
+    else return v[0] + v[1];
+}
+
+template <typename T, int NV>
+__device__ __forceinline__ void softmax_row_wave(const T* __restrict__ x, T* __restrict__ y, int cols, int lane) {
+    using V = typename RowVec<T>::type;
+    const int nvec = cols / RowVec<T>::N;
+    const V* xv = reinterpret_cast<const V*>(x);
+    V* yv = reinterpret_cast<V*>(y);
+    V v[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = lane + i * kWave;
         if (c < nvec) {
             v[i] = __builtin_nontemporal_load(xv + c);
         } else {
-            v[i] = f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+            v[i] = all_neg_inf<T>();
         }
     }
-    float m = kNegInf;
+    T m = SoftmaxMath<T>::neg_inf();
 #pragma unroll
-    for (int i = 0; i < NV; i++) m = fmaxf(fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)), m);
+    for (int i = 0; i < NV; i++) m = SoftmaxMath<T>::max(vec_max<T>(v[i]), m);
     m = wave_max(m);
-    float s = 0.f;
+    T s = (T) 0;
 #pragma unroll
-    for (int i = 0; i < NV; i++) {
-        v[i].x = exp_neg(v[i].x - m);
-        v[i].y = exp_neg(v[i].y - m);
-        v[i].z = exp_neg(v[i].z - m);
-        v[i].w = exp_neg(v[i].w - m);
-        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-    }
+    for (int i = 0; i < NV; i++) s += vec_exp<T>(v[i], m);
     s = wave_sum(s);
     // one IEEE division per row, then multiplies: within 1 ulp of the
     // element-wise division the reference's Div node performs
-    const float inv = 1.0f / s;
+    const T inv = (T) 1 / s;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = lane + i * kWave;
         if (c < nvec) {
-            f32x4 o = v[i] * inv;
+            V o = v[i] * inv;
             __builtin_nontemporal_store(o, yv + c);
         }
     }
 }
 
-template <int NV>
-__device__ __forceinline__ void softmax_wave_kernel(const float* X, float* Y, long rows, int cols) {
+template <typename T, int NV>
+__device__ __forceinline__ void softmax_wave_kernel(const T* X, T* Y, long rows, int cols) {
     const int lane = threadIdx.x & (kWave - 1);
     const long row = (long) blockIdx.x * (256 / kWave) + (threadIdx.x / kWave);   // launched with 256 lanes; blockDim.x would be a load to wait for
     if (row >= rows) return;
-    softmax_row_wave<NV>(X + row * (long) cols, Y + row * (long) cols, cols, lane);
+    softmax_row_wave<T, NV>(X + row * (long) cols, Y + row * (long) cols, cols, lane);
 }
 
 // block reductions across the NW waves of a work-group
-template <int NW = 4>
-__device__ __forceinline__ float block_max(float v, float* lds) {
+template <int NW = 4, typename T>
+__device__ __forceinline__ T block_max(T v, T* lds) {
     v = wave_max(v);
     const int w = threadIdx.x / kWave;
     if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
     __syncthreads();
-    float r = lds[0];
+    T r = lds[0];
 #pragma unroll
-    for (int i = 1; i < NW; i++) r = fmaxf(r, lds[i]);
+    for (int i = 1; i < NW; i++) r = SoftmaxMath<T>::max(r, lds[i]);
     __syncthreads();
     return r;
 }
 
-template <int NW = 4>
-__device__ __forceinline__ float block_sum(float v, float* lds) {
+template <int NW = 4, typename T>
+__device__ __forceinline__ T block_sum(T v, T* lds) {
     v = wave_sum(v);
     const int w = threadIdx.x / kWave;
     if ((threadIdx.x & (kWave - 1)) == 0) lds[w] = v;
     __syncthreads();
-    float r = lds[0];
+    T r = lds[0];
 #pragma unroll
     for (int i = 1; i < NW; i++) r += lds[i];
     __syncthreads();
     return r;
 }
 
-template <int NV, int NW = 4>
-__device__ __forceinline__ void softmax_block_kernel(const float* X, float* Y, long rows, int cols) {
+template <typename T, int NV, int NW = 4>
+__device__ __forceinline__ void softmax_block_kernel(const T* X, T* Y, long rows, int cols) {
+    using V = typename RowVec<T>::type;
     constexpr int NT = NW * kWave;
-    __shared__ float lds[NW];
+    __shared__ T lds[NW];
     const long row = blockIdx.x;
-    const int nvec = cols >> 2;
-    const f32x4* xv = reinterpret_cast<const f32x4*>(X + row * (long) cols);
-    f32x4* yv = reinterpret_cast<f32x4*>(Y + row * (long) cols);
-    f32x4 v[NV];
+    const int nvec = cols / RowVec<T>::N;
+    const V* xv = reinterpret_cast<const V*>(X + row * (long) cols);
+    V* yv = reinterpret_cast<V*>(Y + row * (long) cols);
+    V v[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = threadIdx.x + i * NT;
         if (c < nvec) {
             v[i] = __builtin_nontemporal_load(xv + c);
         } else {
-            v[i] = f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+            v[i] = all_neg_inf<T>();
         }
     }
-    float m = kNegInf;
+    T m = SoftmaxMath<T>::neg_inf();
 #pragma unroll
-    for (int i = 0; i < NV; i++) m = fmaxf(fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)), m);
+    for (int i = 0; i < NV; i++) m = SoftmaxMath<T>::max(vec_max<T>(v[i]), m);
     m = block_max<NW>(m, lds);
-    float s = 0.f;
+    T s = (T) 0;
 #pragma unroll
-    for (int i = 0; i < NV; i++) {
-        v[i].x = exp_neg(v[i].x - m);
-        v[i].y = exp_neg(v[i].y - m);
-        v[i].z = exp_neg(v[i].z - m);
-        v[i].w = exp_neg(v[i].w - m);
-        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
-    }
+    for (int i = 0; i < NV; i++) s += vec_exp<T>(v[i], m);
     s = block_sum<NW>(s, lds);
-    const float inv = 1.0f / s;
+    const T inv = (T) 1 / s;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = threadIdx.x + i * NT;
         if (c < nvec) {
-            f32x4 o = v[i] * inv;
+            V o = v[i] * inv;
             __builtin_nontemporal_store(o, yv + c);
         }
     }
 }
 
-// The work-group per row for rows that do not start on a 16-byte boundary (cols not a multiple of four, or operands
-// placed off it): up to three single elements, the vectors between the first and the last boundary, up to three single
-// elements; a lane holds NV vectors of the middle part and at most one of the single elements. X and Y must be placed
-// equally relative to 16 bytes, so that a row's boundaries are the same in both.
-template <int NV, int NW>
-__device__ __forceinline__ void softmax_block_any_kernel(const float* X, float* Y, long rows, int cols) {
+// The work-group per row for rows that do not start on a 16-byte boundary (cols not a multiple of the vector, or operands
+// placed off it): single elements up to the first boundary, the vectors between the first and the last boundary, single
+// elements after it; a lane holds NV vectors of the middle part and at most one of the single elements. X and Y must be
+// placed equally relative to 16 bytes, so that a row's boundaries are the same in both.
+template <typename T, int NV, int NW>
+__device__ __forceinline__ void softmax_block_any_kernel(const T* X, T* Y, long rows, int cols) {
+    using V = typename RowVec<T>::type;
+    using M = SoftmaxMath<T>;
+    constexpr int N = RowVec<T>::N;
     constexpr int NT = NW * kWave;
-    __shared__ float lds[NW];
+    __shared__ T lds[NW];
     const long row = blockIdx.x;
-    const float* x = X + row * (long) cols;
-    float* y = Y + row * (long) cols;
-    const int mis = (int) ((reinterpret_cast<uintptr_t>(x) >> 2) & 3);
-    int head = mis ? 4 - mis : 0;
+    const T* x = X + row * (long) cols;
+    T* y = Y + row * (long) cols;
+    const int mis = (int) ((reinterpret_cast<uintptr_t>(x) / sizeof(T)) & (N - 1));
+    int head = mis ? N - mis : 0;
     if (head > cols) head = cols;
-    const int nvec = (cols - head) >> 2;
-    const int tail0 = head + nvec * 4;
+    const int nvec = (cols - head) / N;
+    const int tail0 = head + nvec * N;
     const int t = threadIdx.x;
     const int edge = t < head ? t : (t - head < cols - tail0 ? tail0 + t - head : -1);   // this lane's single element, if any
-    float e = edge >= 0 ? x[edge] : kNegInf;
-    const f32x4* xv = reinterpret_cast<const f32x4*>(x + head);
-    f32x4* yv = reinterpret_cast<f32x4*>(y + head);
-    f32x4 v[NV];
+    T e = edge >= 0 ? x[edge] : M::neg_inf();
+    const V* xv = reinterpret_cast<const V*>(x + head);
+    V* yv = reinterpret_cast<V*>(y + head);
+    V v[NV];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = t + i * NT;
         if (c < nvec) {
             v[i] = __builtin_nontemporal_load(xv + c);
         } else {
-            v[i] = f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+            v[i] = all_neg_inf<T>();
         }
     }
-    float m = e;
+    T m = e;
 #pragma unroll
-    for (int i = 0; i < NV; i++) m = fmaxf(fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w)), m);
+    for (int i = 0; i < NV; i++) m = M::max(vec_max<T>(v[i]), m);
     m = block_max<NW>(m, lds);
-    e = exp_neg(e - m);
-    float s = edge >= 0 ? e : 0.f;
+    e = M::exp_le0(e - m);
+    T s = edge >= 0 ? e : (T) 0;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-        v[i].x = exp_neg(v[i].x - m);
-        v[i].y = exp_neg(v[i].y - m);
-        v[i].z = exp_neg(v[i].z - m);
-        v[i].w = exp_neg(v[i].w - m);
-        if (t + i * NT < nvec) s += (v[i].x + v[i].y) + (v[i].z + v[i].w);   // a vector past the row's end is NaN when the whole row is -inf
+        const T part = vec_exp<T>(v[i], m);
+        if (t + i * NT < nvec) s += part;   // a vector past the row's end is NaN when the whole row is -inf
     }
     s = block_sum<NW>(s, lds);
-    const float inv = 1.0f / s;
+    const T inv = (T) 1 / s;
     if (edge >= 0) y[edge] = e * inv;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int c = t + i * NT;
         if (c < nvec) {
-            f32x4 o = v[i] * inv;
+            V o = v[i] * inv;
             __builtin_nontemporal_store(o, yv + c);
         }
     }
 }
 
-} // namespace
-
-#define DOCC_SOFTMAX_BLOCK_ANY(NV, NW)                                                                                  \
-    extern "C" __global__ __launch_bounds__(NW * 64) void docc_softmax_f32_any##NW##_v##NV(const float* X, float* Y,    \
-                                                                                           long rows, int cols) {       \
-        softmax_block_any_kernel<NV, NW>(X, Y, rows, cols);                                                             \
-    }
-DOCC_SOFTMAX_BLOCK_ANY(1, 4)
-DOCC_SOFTMAX_BLOCK_ANY(4, 4)
-DOCC_SOFTMAX_BLOCK_ANY(16, 4)
-DOCC_SOFTMAX_BLOCK_ANY(8, 16)
-DOCC_SOFTMAX_BLOCK_ANY(16, 16)
-
-#define DOCC_SOFTMAX_WAVE(NV)                                                                             \
-    extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_wave_v##NV(const float* X, float* Y, \
-                                                                                  long rows, int cols) {  \
-        softmax_wave_kernel<NV>(X, Y, rows, cols);                                                        \
-    }
-DOCC_SOFTMAX_WAVE(1)
-DOCC_SOFTMAX_WAVE(2)
-DOCC_SOFTMAX_WAVE(4)
-DOCC_SOFTMAX_WAVE(8)
-DOCC_SOFTMAX_WAVE(16)
-
-#define DOCC_SOFTMAX_BLOCK(NV)                                                                             \
-    extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_block_v##NV(const float* X, float* Y, \
-                                                                                   long rows, int cols) {  \
-        softmax_block_kernel<NV>(X, Y, rows, cols);                                                        \
-    }
-// eight wavefronts per row
-#define DOCC_SOFTMAX_BLOCK8(NV)                                                                             \
-    extern "C" __global__ __launch_bounds__(512) void docc_softmax_f32_block8_v##NV(const float* X, float* Y, \
-                                                                                    long rows, int cols) {  \
-        softmax_block_kernel<NV, 8>(X, Y, rows, cols);                                                      \
-    }
-DOCC_SOFTMAX_BLOCK8(2)
-DOCC_SOFTMAX_BLOCK(1)
-DOCC_SOFTMAX_BLOCK(2)
-DOCC_SOFTMAX_BLOCK(4)
-DOCC_SOFTMAX_BLOCK(8)
-DOCC_SOFTMAX_BLOCK(16)
-// sixteen wavefronts per row: rows of up to 65536 columns stay in registers (one read, one write), for tensors with
-// enough rows to give every CU one
-#define DOCC_SOFTMAX_BLOCK16(NV)                                                                             \
-    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_f32_block16_v##NV(const float* X, float* Y, \
-                                                                                      long rows, int cols) {  \
-        softmax_block_kernel<NV, 16>(X, Y, rows, cols);                                                      \
-    }
-DOCC_SOFTMAX_BLOCK16(8)
-DOCC_SOFTMAX_BLOCK16(16)
-
-// Rows of at most 128 columns: LPR lanes of a wavefront share a row (one vector each, cols <= 4 * LPR), so a
-// wavefront holds 64 / LPR rows at a time and four such sets in turn, all loaded before the first is reduced; the
-// reductions are butterflies inside the LPR lanes. A wavefront per row would leave 32 of its 64 lanes (128 columns)
-// to 63 of them (4 columns) idle.
-namespace {
-template <int LPR>
-__device__ __forceinline__ void softmax_subwave_kernel(const float* X, float* Y, long rows, int cols) {
+// Rows of at most 32 vectors: LPR lanes of a wavefront share a row (one vector each), so a wavefront holds 64 / LPR rows
+// at a time and four such sets in turn, all loaded before the first is reduced; the reductions are butterflies inside
+// the LPR lanes. A wavefront per row would leave half to all but one of its lanes idle.
+template <typename T, int LPR>
+__device__ __forceinline__ void softmax_subwave_kernel(const T* X, T* Y, long rows, int cols) {
+    using V = typename RowVec<T>::type;
+    using M = SoftmaxMath<T>;
     constexpr int RPW = kWave / LPR;   // rows of a wavefront per set
     constexpr int SETS = 4;
     const int lane = threadIdx.x & (kWave - 1);
     const int l = lane % LPR, g = lane / LPR;
-    const int nvec = cols >> 2;
+    const int nvec = cols / RowVec<T>::N;
     const long first = ((long) blockIdx.x * (256 / kWave) + threadIdx.x / kWave) * (RPW * SETS) + g;
-    const f32x4* xv = reinterpret_cast<const f32x4*>(X);
-    f32x4* yv = reinterpret_cast<f32x4*>(Y);
-    f32x4 v[SETS];
+    const V* xv = reinterpret_cast<const V*>(X);
+    V* yv = reinterpret_cast<V*>(Y);
+    V v[SETS];
     bool live[SETS];
 #pragma unroll
     for (int i = 0; i < SETS; i++) {
         const long row = first + (long) i * RPW;
         live[i] = row < rows && l < nvec;
-        v[i] = live[i] ? __builtin_nontemporal_load(xv + row * nvec + l) : f32x4{kNegInf, kNegInf, kNegInf, kNegInf};
+        v[i] = live[i] ? __builtin_nontemporal_load(xv + row * nvec + l) : all_neg_inf<T>();
     }
 #pragma unroll
     for (int i = 0; i < SETS; i++) {
-        float m = fmaxf(fmaxf(v[i].x, v[i].y), fmaxf(v[i].z, v[i].w));
+        T m = vec_max<T>(v[i]);
 #pragma unroll
-        for (int o = LPR / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
-        v[i].x = exp_neg(v[i].x - m);
-        v[i].y = exp_neg(v[i].y - m);
-        v[i].z = exp_neg(v[i].z - m);
-        v[i].w = exp_neg(v[i].w - m);
-        float s = (v[i].x + v[i].y) + (v[i].z + v[i].w);
-        if (!(l < nvec)) s = 0.f;   // a lane past the row's end holds -inf, which is NaN after the subtraction when the whole row is -inf
+        for (int o = LPR / 2; o > 0; o >>= 1) m = M::max(m, __shfl_xor(m, o));
+        T s = vec_exp<T>(v[i], m);
+        if (!(l < nvec)) s = (T) 0;   // a lane past the row's end holds -inf, which is NaN after the subtraction when the whole row is -inf
 #pragma unroll
         for (int o = LPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o);
-        const float inv = 1.0f / s;
+        const T inv = (T) 1 / s;
         if (live[i]) {
-            f32x4 out = v[i] * inv;
+            V out = v[i] * inv;
             __builtin_nontemporal_store(out, yv + (first + (long) i * RPW) * nvec + l);
         }
     }
 }
+
 } // namespace
-#define DOCC_SOFTMAX_SUB(LPR)                                                                                                  \
-    extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_sub##LPR(const float* X, float* Y, long rows, int cols) { \
-        softmax_subwave_kernel<LPR>(X, Y, rows, cols);                                                                         \
-    }
-DOCC_SOFTMAX_SUB(1)
-DOCC_SOFTMAX_SUB(2)
-DOCC_SOFTMAX_SUB(4)
-DOCC_SOFTMAX_SUB(8)
-DOCC_SOFTMAX_SUB(16)
-DOCC_SOFTMAX_SUB(32)
+
+// T = float: docc_softmax_f32_<form>; T = double: docc_softmax_f64_<form>. A lane holds NV 16-byte vectors of its row.
+#define DOCC_SOFTMAX_ROW_FORMS(T, SFX)                                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_wave_v1(const T* X, T* Y, long rows, int cols) { softmax_wave_kernel<T, 1>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_wave_v2(const T* X, T* Y, long rows, int cols) { softmax_wave_kernel<T, 2>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_wave_v4(const T* X, T* Y, long rows, int cols) { softmax_wave_kernel<T, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_wave_v8(const T* X, T* Y, long rows, int cols) { softmax_wave_kernel<T, 8>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_wave_v16(const T* X, T* Y, long rows, int cols) { softmax_wave_kernel<T, 16>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_block_v1(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 1>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_block_v2(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 2>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_block_v4(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_block_v8(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 8>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_block_v16(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 16>(X, Y, rows, cols); } \
+    /* eight wavefronts per row */                                                                                                  \
+    extern "C" __global__ __launch_bounds__(512) void docc_softmax_##SFX##_block8_v2(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 2, 8>(X, Y, rows, cols); } \
+    /* sixteen wavefronts per row: long rows stay in registers (one read, one write), for tensors with rows enough to give every CU one */ \
+    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_##SFX##_block16_v8(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 8, 16>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_##SFX##_block16_v16(const T* X, T* Y, long rows, int cols) { softmax_block_kernel<T, 16, 16>(X, Y, rows, cols); } \
+    /* rows that start off a 16-byte boundary */                                                                                    \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_any4_v1(const T* X, T* Y, long rows, int cols) { softmax_block_any_kernel<T, 1, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_any4_v4(const T* X, T* Y, long rows, int cols) { softmax_block_any_kernel<T, 4, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_any4_v16(const T* X, T* Y, long rows, int cols) { softmax_block_any_kernel<T, 16, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_##SFX##_any16_v8(const T* X, T* Y, long rows, int cols) { softmax_block_any_kernel<T, 8, 16>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(1024) void docc_softmax_##SFX##_any16_v16(const T* X, T* Y, long rows, int cols) { softmax_block_any_kernel<T, 16, 16>(X, Y, rows, cols); } \
+    /* several rows per wavefront: 1 .. 32 lanes a row */                                                                           \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub1(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 1>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub2(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 2>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub4(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 4>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub8(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 8>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub16(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 16>(X, Y, rows, cols); } \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SFX##_sub32(const T* X, T* Y, long rows, int cols) { softmax_subwave_kernel<T, 32>(X, Y, rows, cols); }
+DOCC_SOFTMAX_ROW_FORMS(float, f32)
+DOCC_SOFTMAX_ROW_FORMS(double, f64)
 
 // Any cols, any alignment: one 256-thread block per row. Pass 1 keeps a
 // per-thread running (max, sum) pair that is rescaled whenever the max moves
@@ -351,17 +347,6 @@ extern "C" __global__ __launch_bounds__(256) void docc_softmax_f32_stream(const 
 
 namespace {
 
-template <typename T> struct SoftmaxMath;
-template <> struct SoftmaxMath<float> {
-    static __device__ __forceinline__ float neg_inf() { return kNegInf; }
-    static __device__ __forceinline__ float exp_le0(float t) { return exp_neg(t); }
-    static __device__ __forceinline__ float max(float a, float b) { return fmaxf(a, b); }
-};
-template <> struct SoftmaxMath<double> {
-    static __device__ __forceinline__ double neg_inf() { return -__builtin_huge_val(); }
-    static __device__ __forceinline__ double exp_le0(double t) { return exp(t); }
-    static __device__ __forceinline__ double max(double a, double b) { return fmax(a, b); }
-};
 
 // running (maximum, sum of exp(x - maximum)) of the elements seen so far; (-inf, 0) for none
 template <typename T>
@@ -559,9 +544,6 @@ __device__ __forceinline__ void softmax_sliced_finish(const void* partials, cons
 // so each slice is walked as a head of single elements up to the first 16-byte boundary, a body of vectors and a tail.
 // X and Y must be equally placed relative to 16 bytes for the vector form (`vec`), else every access is one element.
 
-template <typename T> struct RowVec;
-template <> struct RowVec<float> { typedef float type __attribute__((ext_vector_type(4))); static constexpr int N = 4; };
-template <> struct RowVec<double> { typedef double type __attribute__((ext_vector_type(2))); static constexpr int N = 2; };
 
 // the running pair after the elements of one vector: one rescaling per vector instead of one per element
 template <typename T>

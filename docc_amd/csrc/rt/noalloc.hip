@@ -9,6 +9,7 @@
 // code uses the address hipGetSymbolAddress returned, nothing else.
 #include <hip/hip_runtime.h>
 
+#include <cstdio>
 #include <mutex>
 
 #include "docc_rocm_ops.h"
@@ -44,22 +45,21 @@ int noalloc_setup_device(int dev) {
     if (err != hipSuccess || !ptr)
         return fail(err != hipSuccess ? (int) err : DOCC_ROCM_ERR_KERNEL_IMAGE, "address of the no-allocation scratch array on device %d: %s", dev,
                     hipGetErrorString(err));
-    static const char* const kernels[] = {
-        "docc_softmax_f64_stream",         "docc_softmax_f32_slab",          "docc_softmax_f64_slab",          "docc_softmax_f32_tile",
-        "docc_softmax_f64_tile",           "docc_softmax_f32_sliced_partial", "docc_softmax_f64_sliced_partial", "docc_softmax_f32_sliced_finish",
-        "docc_softmax_f64_sliced_finish",  "docc_softmax_f32_wave_v1",       "docc_softmax_f32_wave_v2",       "docc_softmax_f32_wave_v4",
-        "docc_softmax_f32_wave_v8",        "docc_softmax_f32_wave_v16",      "docc_softmax_f32_block8_v2",     "docc_softmax_f32_block_v1",
-        "docc_softmax_f32_block_v2",       "docc_softmax_f32_block_v4",      "docc_softmax_f32_block_v8",      "docc_softmax_f32_block_v16",
-        "docc_softmax_f32_stream",         "docc_softmax_f32_block16_v8",    "docc_softmax_f32_block16_v16",   "docc_softmax_f32_sub1",
-        "docc_softmax_f32_sub2",           "docc_softmax_f32_sub4",          "docc_softmax_f32_sub8",          "docc_softmax_f32_sub16",
-        "docc_softmax_f32_sub32",          "docc_softmax_f32_rowslice_partial", "docc_softmax_f64_rowslice_partial",
-        "docc_softmax_f32_rowslice_finish", "docc_softmax_f64_rowslice_finish", "docc_softmax_f32_any4_v1",      "docc_softmax_f32_any4_v4",
-        "docc_softmax_f32_any4_v16",       "docc_softmax_f32_any16_v8",      "docc_softmax_f32_any16_v16",
+    // every kernel docc_rocm_softmax may launch, in both precisions
+    static const char* const forms[] = {
+        "stream",     "slab",      "tile",      "sliced_partial", "sliced_finish", "rowslice_partial", "rowslice_finish",
+        "wave_v1",    "wave_v2",   "wave_v4",   "wave_v8",        "wave_v16",      "block8_v2",        "block_v1",
+        "block_v2",   "block_v4",  "block_v8",  "block_v16",      "block16_v8",    "block16_v16",      "any4_v1",
+        "any4_v4",    "any4_v16",  "any16_v8",  "any16_v16",      "sub1",          "sub2",             "sub4",
+        "sub8",       "sub16",     "sub32",
     };
-    for (const char* name : kernels) {
-        hipFunction_t fn;
-        if (int rc = kernel(name, &fn)) return rc;
-    }
+    for (const char* form : forms)
+        for (const char* type : {"f32", "f64"}) {
+            char name[64];
+            std::snprintf(name, sizeof(name), "docc_softmax_%s_%s", type, form);
+            hipFunction_t fn;
+            if (int rc = kernel(name, &fn)) return rc;
+        }
     g_scratch_ptr[dev] = ptr;
     return 0;
 }

@@ -11,17 +11,14 @@ namespace docc::rt::rocm {
 
 // Slices of the row-sliced form of a softmax over the rows of [rows, cols] (two launches around (maximum, sum) pairs,
 // rows * slices * 2 elements of them), 0 where a one-launch kernel serves; *per = columns of a slice. Rows that a
-// work-group's registers hold (16384 columns; 65536 with sixteen wavefronts, `in_registers`, where there are rows
+// work-group's registers hold (4096 16-byte vectors; 16384 with sixteen wavefronts, `in_registers`, where there are rows
 // enough to occupy half the CUs that way) stay with the one-launch kernels; longer rows, or rows too few to fill the
 // device one work-group each, are cut so that about eight work-groups per CU share the tensor, no slice shorter
 // than 4096 columns.
 int64_t softmax_row_slices(int precision, int64_t rows, int64_t cols, bool in_registers, int cus, int64_t capacity, int64_t* per) {
-    if (precision == 32) {
-        if (cols <= 16384) return 0;
-        if (in_registers && cols <= 65536 && rows >= cus / 2) return 0;
-    } else {
-        if (cols < 8192 || (rows >= 2 * (int64_t) cus && cols <= 65536)) return 0;
-    }
+    const int64_t per_vec = 128 / precision;
+    if (cols <= 4096 * per_vec) return 0;
+    if (in_registers && cols <= 16384 * per_vec && rows >= cus / 2) return 0;
     int64_t slices = (8 * (int64_t) cus + rows - 1) / rows;
     if (slices > cols / 4096) slices = cols / 4096;
     if (slices > 1024) slices = 1024;
@@ -52,65 +49,60 @@ int softmax_rowsliced(hipStream_t s, int precision, int64_t rows, int64_t cols, 
 }
 } // namespace
 
-// The fp32 row softmax; `partials` as for softmax_general.
-int softmax_rows_f32(hipStream_t s, int64_t rows, int64_t cols, const float* X, float* Y, void* partials) {
+// The row softmax (inner == 1) in either precision; `partials` as for softmax_general. The forms are chosen by the
+// number of 16-byte vectors in a row (four floats or two doubles each), which is what a lane holds.
+int softmax_rows(hipStream_t s, int precision, int64_t rows, int64_t cols, const void* X, void* Y, void* partials) {
     if (rows > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
-    const bool vec_ok = (cols % 4 == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
+    const int64_t per_vec = 128 / precision, elem = precision / 8;
+    const char* t = precision == 32 ? "f32" : "f64";
+    char name[64];
+    auto run = [&](const char* form, uint32_t groups, uint32_t threads) {
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_%s", t, form);
+        return launch(name, groups, 1, 1, threads, 0, s, X, Y, (long) rows, (int) cols);
+    };
+    auto stream_kernel = [&]() {
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_stream", t);
+        return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+    };
+    const bool vec_ok = (cols % per_vec == 0) && (((uintptr_t) X | (uintptr_t) Y) % 16 == 0);
     // rows that start off a 16-byte boundary are still read in vectors when they start equally far off it in X and Y
-    const bool same_place = (((uintptr_t) X | (uintptr_t) Y) % 4 == 0) && ((uintptr_t) X % 16 == (uintptr_t) Y % 16);
-    if (cols > 16384) {
+    const bool same_place = (((uintptr_t) X | (uintptr_t) Y) % elem == 0) && ((uintptr_t) X % 16 == (uintptr_t) Y % 16);
+    const int64_t nvec = (cols + per_vec - 1) / per_vec;
+    if (nvec > 4096) {
         int cus = compute_units();
         if (cus <= 0) cus = 256;
         int64_t per = 0;
-        const int64_t slices = softmax_row_slices(32, rows, cols, vec_ok || same_place, cus, (int64_t) kPartialsBytes, &per);
-        if (slices > 0) return softmax_rowsliced(s, 32, rows, cols, slices, per, X, Y, partials);
-        if (vec_ok && cols <= 65536)
-            return launch(cols <= 32768 ? "docc_softmax_f32_block16_v8" : "docc_softmax_f32_block16_v16", (uint32_t) rows, 1, 1, 1024, 0, s, X, Y,
-                          (long) rows, (int) cols);
-        if (same_place && cols <= 65536)
-            return launch(cols <= 32768 ? "docc_softmax_f32_any16_v8" : "docc_softmax_f32_any16_v16", (uint32_t) rows, 1, 1, 1024, 0, s, X, Y,
-                          (long) rows, (int) cols);
-        return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+        const int64_t slices = softmax_row_slices(precision, rows, cols, vec_ok || same_place, cus, (int64_t) kPartialsBytes, &per);
+        if (slices > 0) return softmax_rowsliced(s, precision, rows, cols, slices, per, X, Y, partials);
+        if (vec_ok && nvec <= 16384) return run(nvec <= 8192 ? "block16_v8" : "block16_v16", (uint32_t) rows, 1024);
+        if (same_place && nvec <= 16384) return run(nvec <= 8192 ? "any16_v8" : "any16_v16", (uint32_t) rows, 1024);
+        return stream_kernel();
     }
-    // Up to 1024 columns one wavefront per row moves the most bytes (6.1-6.4 TB/s measured against 2.6-5.6
-    // for a work-group per row); from 2048 columns on the work-group per row is ahead (6.1-6.3 against
+    // Up to 256 vectors (1024 floats) one wavefront per row moves the most bytes (6.1-6.4 TB/s measured against 2.6-5.6
+    // for a work-group per row); from 512 vectors on the work-group per row is ahead (6.1-6.3 against
     // 5.8-6.0 TB/s). DOCC_ROCM_SOFTMAX=wave|block overrides the choice (tuning; block = four wavefronts per row).
     const char* force = std::getenv("DOCC_ROCM_SOFTMAX");
-    const bool wave = force && force[0] == 'w' ? true : force && force[0] == 'b' ? false : cols <= 1024;
-    if (vec_ok && cols <= 128 && !force) {
+    const bool wave = force && force[0] == 'w' ? true : force && force[0] == 'b' ? false : nvec <= 256;
+    if (vec_ok && nvec <= 32 && !force) {
         // several rows per wavefront: LPR lanes a row, four sets of 64 / LPR rows per wavefront, four wavefronts
         int lpr = 1;
-        while (4 * lpr < cols) lpr *= 2;
-        char name[48];
-        std::snprintf(name, sizeof(name), "docc_softmax_f32_sub%d", lpr);
+        while (lpr < nvec) lpr *= 2;
+        char form[16];
+        std::snprintf(form, sizeof(form), "sub%d", lpr);
         const int64_t rows_per_group = 4 * 4 * (64 / lpr);
-        return launch(name, (uint32_t) ((rows + rows_per_group - 1) / rows_per_group), 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
+        return run(form, (uint32_t) ((rows + rows_per_group - 1) / rows_per_group), 256);
     }
-    if (vec_ok && cols <= 4096 && wave) {
-        // one wavefront per row, 4 rows per 256-thread block
-        const char* name = cols <= 256    ? "docc_softmax_f32_wave_v1"
-                           : cols <= 512  ? "docc_softmax_f32_wave_v2"
-                           : cols <= 1024 ? "docc_softmax_f32_wave_v4"
-                           : cols <= 2048 ? "docc_softmax_f32_wave_v8"
-                                          : "docc_softmax_f32_wave_v16";
-        uint32_t grid = (uint32_t) ((rows + 3) / 4);
-        return launch(name, grid, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
-    }
-    if (vec_ok && cols > 2048 && cols <= 4096 && !(force && force[0] == 'b'))
-        // eight wavefronts per row, two vectors per lane: 6.24 TB/s against 6.09 with four wavefronts at 4096 columns
-        return launch("docc_softmax_f32_block8_v2", (uint32_t) rows, 1, 1, 512, 0, s, X, Y, (long) rows, (int) cols);
-    if (vec_ok) {
-        const char* name = cols <= 1024   ? "docc_softmax_f32_block_v1"
-                           : cols <= 2048 ? "docc_softmax_f32_block_v2"
-                           : cols <= 4096 ? "docc_softmax_f32_block_v4"
-                           : cols <= 8192 ? "docc_softmax_f32_block_v8"
-                                          : "docc_softmax_f32_block_v16";
-        return launch(name, (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
-    }
-    if (same_place && cols >= 256 && !force)
-        return launch(cols <= 1024 ? "docc_softmax_f32_any4_v1" : cols <= 4096 ? "docc_softmax_f32_any4_v4" : "docc_softmax_f32_any4_v16", (uint32_t) rows,
-                      1, 1, 256, 0, s, X, Y, (long) rows, (int) cols);
-    return launch("docc_softmax_f32_stream", (uint32_t) rows, 1, 1, 256, 0, s, X, Y, (long) rows, (long) cols);
+    if (vec_ok && nvec <= 1024 && wave)   // one wavefront per row, 4 rows per 256-thread block
+        return run(nvec <= 64 ? "wave_v1" : nvec <= 128 ? "wave_v2" : nvec <= 256 ? "wave_v4" : nvec <= 512 ? "wave_v8" : "wave_v16",
+                   (uint32_t) ((rows + 3) / 4), 256);
+    if (vec_ok && nvec > 512 && nvec <= 1024 && !(force && force[0] == 'b'))
+        // eight wavefronts per row, two vectors per lane: 6.24 TB/s against 6.09 with four wavefronts at 4096 floats
+        return run("block8_v2", (uint32_t) rows, 512);
+    if (vec_ok)
+        return run(nvec <= 256 ? "block_v1" : nvec <= 512 ? "block_v2" : nvec <= 1024 ? "block_v4" : nvec <= 2048 ? "block_v8" : "block_v16",
+                   (uint32_t) rows, 256);
+    if (same_place && nvec >= 64 && !force) return run(nvec <= 256 ? "any4_v1" : nvec <= 1024 ? "any4_v4" : "any4_v16", (uint32_t) rows, 256);
+    return stream_kernel();
 }
 
 } // namespace docc::rt::rocm
@@ -122,7 +114,7 @@ int docc_rocm_softmax_f32(docc_rocm_stream_t stream, int64_t rows, int64_t cols,
     if (rows == 0 || cols == 0) return 0;
     if (!X || !Y) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "softmax: null pointer");
     if (int rc = ensure_device()) return rc;
-    return softmax_rows_f32((hipStream_t) stream, rows, cols, X, Y, nullptr);
+    return softmax_rows((hipStream_t) stream, 32, rows, cols, X, Y, nullptr);
 }
 
 } // extern "C"
@@ -149,16 +141,7 @@ int64_t softmax_slices(int precision, int64_t outer, int64_t reduce, int64_t inn
 int softmax_general(hipStream_t s, int precision, int64_t outer, int64_t reduce, int64_t inner, const void* X, void* Y, void* partials) {
     const char* t = precision == 32 ? "f32" : "f64";
     char name[64];
-    if (inner == 1) {
-        if (precision == 32) return softmax_rows_f32(s, outer, reduce, (const float*) X, (float*) Y, partials);
-        if (outer > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 rows");
-        int cus = compute_units();
-        if (cus <= 0) cus = 256;
-        int64_t per = 0;
-        const int64_t slices = softmax_row_slices(64, outer, reduce, false, cus, (int64_t) kPartialsBytes, &per);
-        if (slices > 0) return softmax_rowsliced(s, 64, outer, reduce, slices, per, X, Y, partials);
-        return launch("docc_softmax_f64_stream", (uint32_t) outer, 1, 1, 256, 0, s, X, Y, (long) outer, (long) reduce);
-    }
+    if (inner == 1) return softmax_rows(s, precision, outer, reduce, X, Y, partials);
     if (inner <= 32 && (inner & (inner - 1)) == 0) {
         // a few inner positions: one work-group per outer index walks its contiguous slab
         if (outer > 0x7fffffffLL) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "softmax: more than 2^31-1 outer indices");

@@ -105,6 +105,33 @@ def test_softmax_rows_that_start_off_a_vector_boundary(rt, cols):
         assert (got[:off_y] == 0).all() and (got[off_y + X.size:] == 0).all()
 
 
+F64_ROWS = [(1000, 2), (999, 4), (513, 16), (130, 28), (4099, 32), (1025, 64), (300, 100), (259, 128), (17, 512), (6, 514), (33, 1000), (9, 1024),
+            (9, 2048), (11, 3000), (5, 8192), (7, 4097), (13, 1001), (140, 8194), (129, 32768), (130, 20001), (3, 16388), (2, 40001)]
+
+
+@pytest.mark.parametrize("rows,cols", F64_ROWS)
+def test_softmax_fp64_rows_every_form(rt, rows, cols):
+    """The row kernels in fp64 (vectors of two): rows sharing a wavefront, a wavefront and a work-group per row, rows off
+    a 16-byte boundary, sixteen wavefronts per row, rows cut into slices. Against scipy in float64, -inf and NaN rows included."""
+    rng = np.random.default_rng(rows * 31 + cols)
+    X = rng.standard_normal((rows, cols)) * 8
+    X[rows // 2] = -np.inf
+    X[0, cols // 2] = -np.inf                      # (every case has at least two rows)
+    if rows > 4:
+        X[rows - 1, cols - 1] = np.nan
+    x = dev(X)
+    y = torch.empty_like(x)
+    rt.softmax(64, rows, cols, 1, x.data_ptr(), y.data_ptr())
+    torch.cuda.synchronize()
+    Y = host(y)
+    with np.errstate(invalid="ignore"):
+        ref = scipy.special.softmax(X, axis=-1)
+    assert np.array_equal(np.isnan(Y), np.isnan(ref))
+    ok = ~np.isnan(ref)
+    assert Y[0, cols // 2] == 0.0
+    np.testing.assert_allclose(Y[ok], ref[ok], rtol=1e-12, atol=1e-300)
+
+
 def test_softmax_long_rows_fp64_and_misplaced_operands(rt):
     """The sliced rows in fp64 (vectors of two), and fp32 operands that are not 16-byte aligned: equally misplaced
     operands keep the vector form (head and tail by single elements), unequally placed ones go element by element."""
