@@ -379,6 +379,13 @@ __device__ __forceinline__ void merge_pairs(const T* lm, const T* ls, int first,
     gs += gm - gm;   // an infinite maximum makes every result NaN, as inf - inf does in the node's Sub step
 }
 
+// what a result is multiplied or divided by: fp32 divides once per row and multiplies, fp64 divides every element
+template <typename T> __device__ __forceinline__ T softmax_scale(T gs);
+template <> __device__ __forceinline__ float softmax_scale<float>(float gs) { return 1.0f / gs; }   // one division per row, then multiplies
+template <> __device__ __forceinline__ double softmax_scale<double>(double gs) { return gs; }
+__device__ __forceinline__ float softmax_result(float e, float scale) { return e * scale; }
+__device__ __forceinline__ double softmax_result(double e, double scale) { return e / scale; }
+
 // inner == 1, any type: one 256-thread block per row, two reads of the row.
 template <typename T>
 __device__ __forceinline__ void softmax_row_stream(const T* X, T* Y, long cols) {
@@ -432,6 +439,76 @@ __device__ __forceinline__ void softmax_strided_tile(const T* X, T* Y, long redu
     merge_pairs(lm, ls, (int) (threadIdx.x & 63), 64, 4, gm, gs);
     if (live)
         for (long r = part; r < reduce; r += 4) y[r * inner] = M::exp_le0(x[r * inner] - gm) / gs;
+}
+
+// The same with 16-byte vectors (inner a multiple of the vector, operands 16-byte aligned): a lane owns the VN adjacent
+// columns of one vector, 256 / PARTS lanes cover the block's columns and the PARTS groups of lanes split the reduced
+// extent; four rows are loaded before the first is worked in. PARTS = 16 (256 bytes of a row per block) for long
+// extents, 4 (1 KB of a row) for short ones.
+template <typename T, int PARTS>
+__device__ __forceinline__ void softmax_strided_tile_vec(const T* X, T* Y, long reduce, long inner, long tiles) {
+    using M = SoftmaxMath<T>;
+    using V = typename RowVec<T>::type;
+    constexpr int VN = RowVec<T>::N;
+    constexpr int LANES = 256 / PARTS;       // lanes (vectors of columns) across the block
+    __shared__ T lm[VN][256];
+    __shared__ T ls[VN][256];
+    const long o = blockIdx.x / tiles;
+    const int cl = threadIdx.x % LANES, part = threadIdx.x / LANES;
+    const long col = ((blockIdx.x % tiles) * LANES + cl) * VN;
+    const bool live = col < inner;
+    const long nv = inner / VN;                                   // vectors per row
+    const V* x = reinterpret_cast<const V*>(X + o * reduce * inner + col);
+    V* y = reinterpret_cast<V*>(Y + o * reduce * inner + col);
+    T m[VN], s[VN];
+#pragma unroll
+    for (int e = 0; e < VN; e++) m[e] = M::neg_inf(), s[e] = (T) 0;
+    if (live) {
+        long r = part;
+        for (; r + 3 * PARTS < reduce; r += 4 * PARTS) {
+            V v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = x[(r + PARTS * u) * nv];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < VN; e++) online_step(v[u][e], m[e], s[e]);
+        }
+        for (; r < reduce; r += PARTS) {
+            const V v = x[r * nv];
+#pragma unroll
+            for (int e = 0; e < VN; e++) online_step(v[e], m[e], s[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VN; e++) lm[e][threadIdx.x] = m[e], ls[e][threadIdx.x] = s[e];
+    __syncthreads();
+    T gm[VN], scale[VN];
+#pragma unroll
+    for (int e = 0; e < VN; e++) {
+        T gs;
+        merge_pairs(lm[e], ls[e], cl, LANES, PARTS, gm[e], gs);
+        scale[e] = softmax_scale<T>(gs);
+    }
+    if (!live) return;
+    long r = part;
+    for (; r + 3 * PARTS < reduce; r += 4 * PARTS) {
+        V v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = __builtin_nontemporal_load(x + (r + PARTS * u) * nv);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int e = 0; e < VN; e++) v[u][e] = softmax_result(M::exp_le0(v[u][e] - gm[e]), scale[e]);
+            __builtin_nontemporal_store(v[u], y + (r + PARTS * u) * nv);
+        }
+    }
+    for (; r < reduce; r += PARTS) {
+        V v = __builtin_nontemporal_load(x + r * nv);
+#pragma unroll
+        for (int e = 0; e < VN; e++) v[e] = softmax_result(M::exp_le0(v[e] - gm[e]), scale[e]);
+        __builtin_nontemporal_store(v, y + r * nv);
+    }
 }
 
 // inner a power of two up to 32: a block owns one outer index, whose [reduce, inner] slab is contiguous;
@@ -537,6 +614,136 @@ __device__ __forceinline__ void softmax_sliced_finish(const void* partials, cons
     for (long r = w.r0 + part; r < w.r1; r += 4) y[r * inner] = M::exp_le0(x[r * inner] - gm) / gs;
 }
 
+// The sliced pair with 16-byte vectors (inner a multiple of the vector, operands 16-byte aligned): the layout of the
+// vector tile kernel - a lane owns the VN columns of one vector, sixteen lanes across, sixteen row groups - over the
+// rows of one slice. Same pairs in the same places of `partials` as the scalar pair.
+template <typename T>
+struct SlicedVecWork {
+    long o, slice, col, r0, r1;
+    int cl, part;
+    bool live;
+    __device__ __forceinline__ SlicedVecWork(long reduce, long inner, long vtiles, int slices) {
+        long b = blockIdx.x;
+        const long tile = b % vtiles;
+        b /= vtiles;
+        slice = b % slices;
+        o = b / slices;
+        cl = threadIdx.x & 15;
+        part = threadIdx.x >> 4;
+        col = (tile * 16 + cl) * RowVec<T>::N;
+        const long per = (reduce + slices - 1) / slices;
+        r0 = slice * per;
+        r1 = r0 + per < reduce ? r0 + per : reduce;
+        live = col < inner;
+    }
+};
+
+template <typename T>
+__device__ __forceinline__ void softmax_sliced_partial_vec(void* partials, const T* X, long reduce, long inner, long vtiles, int slices) {
+    using M = SoftmaxMath<T>;
+    using V = typename RowVec<T>::type;
+    constexpr int VN = RowVec<T>::N;
+    __shared__ T lm[VN][256];
+    __shared__ T ls[VN][256];
+    const SlicedVecWork<T> w(reduce, inner, vtiles, slices);
+    const long nv = inner / VN;
+    const V* x = reinterpret_cast<const V*>(X + w.o * reduce * inner + w.col);
+    T m[VN], s[VN];
+#pragma unroll
+    for (int e = 0; e < VN; e++) m[e] = M::neg_inf(), s[e] = (T) 0;
+    if (w.live) {
+        long r = w.r0 + w.part;
+        for (; r + 48 < w.r1; r += 64) {
+            V v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = x[(r + 16 * u) * nv];
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < VN; e++) online_step(v[u][e], m[e], s[e]);
+        }
+        for (; r < w.r1; r += 16) {
+            const V v = x[r * nv];
+#pragma unroll
+            for (int e = 0; e < VN; e++) online_step(v[e], m[e], s[e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VN; e++) lm[e][threadIdx.x] = m[e], ls[e][threadIdx.x] = s[e];
+    __syncthreads();
+    if (w.part == 0 && w.live) {
+        // the pairs of the slice, without the NaN marker for infinite maxima: that is applied once, at the end
+        T* P = reinterpret_cast<T*>(partials);
+#pragma unroll
+        for (int e = 0; e < VN; e++) {
+            T gm = M::neg_inf();
+            for (int i = 0; i < 16; i++) gm = M::max(gm, lm[e][w.cl + 16 * i]);
+            T gs = (T) 0;
+            for (int i = 0; i < 16; i++) gs += pair_weight(lm[e][w.cl + 16 * i], ls[e][w.cl + 16 * i], gm);
+            const long at = ((w.o * slices + w.slice) * inner + w.col + e) * 2;
+            P[at] = gm;
+            P[at + 1] = gs;
+        }
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ void softmax_sliced_finish_vec(const void* partials, const T* X, T* Y, long reduce, long inner, long vtiles, int slices) {
+    using M = SoftmaxMath<T>;
+    using V = typename RowVec<T>::type;
+    constexpr int VN = RowVec<T>::N;
+    __shared__ T lm[VN][256];
+    __shared__ T ls[VN][256];
+    const SlicedVecWork<T> w(reduce, inner, vtiles, slices);
+    const T* P = reinterpret_cast<const T*>(partials);
+    T m[VN], s[VN];
+#pragma unroll
+    for (int e = 0; e < VN; e++) m[e] = M::neg_inf(), s[e] = (T) 0;
+    if (w.live)
+        for (int sl = w.part; sl < slices; sl += 16) {
+#pragma unroll
+            for (int e = 0; e < VN; e++) {
+                const long at = ((w.o * slices + sl) * inner + w.col + e) * 2;
+                const T pm = P[at], ps = P[at + 1];
+                const T g = M::max(m[e], pm);
+                s[e] = pair_weight(m[e], s[e], g) + pair_weight(pm, ps, g);
+                m[e] = g;
+            }
+        }
+#pragma unroll
+    for (int e = 0; e < VN; e++) lm[e][threadIdx.x] = m[e], ls[e][threadIdx.x] = s[e];
+    __syncthreads();
+    T gm[VN], scale[VN];
+#pragma unroll
+    for (int e = 0; e < VN; e++) {
+        T gs;
+        merge_pairs(lm[e], ls[e], w.cl, 16, 16, gm[e], gs);
+        scale[e] = softmax_scale<T>(gs);
+    }
+    if (!w.live) return;
+    const long nv = inner / VN;
+    const V* x = reinterpret_cast<const V*>(X + w.o * reduce * inner + w.col);
+    V* y = reinterpret_cast<V*>(Y + w.o * reduce * inner + w.col);
+    long r = w.r0 + w.part;
+    for (; r + 48 < w.r1; r += 64) {
+        V v[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) v[u] = __builtin_nontemporal_load(x + (r + 16 * u) * nv);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+#pragma unroll
+            for (int e = 0; e < VN; e++) v[u][e] = softmax_result(M::exp_le0(v[u][e] - gm[e]), scale[e]);
+            __builtin_nontemporal_store(v[u], y + (r + 16 * u) * nv);
+        }
+    }
+    for (; r < w.r1; r += 16) {
+        V v = __builtin_nontemporal_load(x + r * nv);
+#pragma unroll
+        for (int e = 0; e < VN; e++) v[e] = softmax_result(M::exp_le0(v[e] - gm[e]), scale[e]);
+        __builtin_nontemporal_store(v, y + r * nv);
+    }
+}
+
 // Rows cut into slices (inner == 1): rows longer than a work-group's registers hold, or too few of them to give every
 // CU one. Work-group (row, slice) first leaves the (maximum, sum) pair of its `per` columns in the launcher's buffer,
 // then - in a second launch - merges the pairs of its row and writes its own columns. Both launches read with 16-byte
@@ -635,11 +842,6 @@ __device__ __forceinline__ void softmax_rowslice_partial(void* partials, const T
     }
 }
 
-template <typename T> __device__ __forceinline__ T softmax_scale(T gs);
-template <> __device__ __forceinline__ float softmax_scale<float>(float gs) { return 1.0f / gs; }   // one division per row, then multiplies
-template <> __device__ __forceinline__ double softmax_scale<double>(double gs) { return gs; }
-__device__ __forceinline__ float softmax_result(float e, float scale) { return e * scale; }
-__device__ __forceinline__ double softmax_result(double e, double scale) { return e / scale; }
 
 template <typename T>
 __device__ __forceinline__ void softmax_rowslice_finish(const void* partials, const T* X, T* Y, long cols, long per, int slices, int vec) {
@@ -701,6 +903,19 @@ __device__ __forceinline__ void softmax_rowslice_finish(const void* partials, co
 DOCC_SOFTMAX_ROWSLICE(float, f32)
 DOCC_SOFTMAX_ROWSLICE(double, f64)
 
+#define DOCC_SOFTMAX_SLICED_VEC(T, SUFFIX)                                                                                          \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_slicedv_partial(void* partials, const T* X, long reduce, \
+                                                                                             long inner, long tiles, int slices) { \
+        softmax_sliced_partial_vec<T>(partials, X, reduce, inner, tiles, slices);                                                  \
+    }                                                                                                                              \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_slicedv_finish(const void* partials, const T* X, T* Y, \
+                                                                                            long reduce, long inner, long tiles,  \
+                                                                                            int slices) {                         \
+        softmax_sliced_finish_vec<T>(partials, X, Y, reduce, inner, tiles, slices);                                                \
+    }
+DOCC_SOFTMAX_SLICED_VEC(float, f32)
+DOCC_SOFTMAX_SLICED_VEC(double, f64)
+
 #define DOCC_SOFTMAX_SLICED(T, SUFFIX)                                                                                        \
     extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_sliced_partial(void* partials, const T* X, long reduce, \
                                                                                             long inner, long tiles, int slices) { \
@@ -721,6 +936,14 @@ extern "C" __global__ __launch_bounds__(256) void docc_softmax_f64_stream(const 
     extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_tile(const T* X, T* Y, long reduce, long inner, \
                                                                                   long tiles) {                             \
         softmax_strided_tile<T>(X, Y, reduce, inner, tiles);                                                                \
+    }                                                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_tilev16(const T* X, T* Y, long reduce, long inner, \
+                                                                                     long tiles) {                          \
+        softmax_strided_tile_vec<T, 16>(X, Y, reduce, inner, tiles);                                                        \
+    }                                                                                                                       \
+    extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_tilev4(const T* X, T* Y, long reduce, long inner, \
+                                                                                    long tiles) {                           \
+        softmax_strided_tile_vec<T, 4>(X, Y, reduce, inner, tiles);                                                         \
     }                                                                                                                       \
     extern "C" __global__ __launch_bounds__(256) void docc_softmax_##SUFFIX##_slab(const T* X, T* Y, long reduce, int inner) { \
         softmax_strided_slab<T>(X, Y, reduce, inner);                                                                       \

@@ -47,7 +47,7 @@ int noalloc_setup_device(int dev) {
                     hipGetErrorString(err));
     // every kernel docc_rocm_softmax may launch, in both precisions
     static const char* const forms[] = {
-        "stream",     "slab",      "tile",      "sliced_partial", "sliced_finish", "rowslice_partial", "rowslice_finish",
+        "stream",     "slab",      "tile",      "tilev16",   "tilev4",    "sliced_partial", "sliced_finish", "slicedv_partial", "slicedv_finish", "rowslice_partial", "rowslice_finish",
         "wave_v1",    "wave_v2",   "wave_v4",   "wave_v8",        "wave_v16",      "block8_v2",        "block_v1",
         "block_v2",   "block_v4",  "block_v8",  "block_v16",      "block16_v8",    "block16_v16",      "any4_v1",
         "any4_v4",    "any4_v16",  "any16_v8",  "any16_v16",      "sub1",          "sub2",             "sub4",

@@ -160,12 +160,36 @@ int softmax_general(hipStream_t s, int precision, int64_t outer, int64_t reduce,
             if (int rc = partials_for(s, &lease)) return rc;
             partials = lease.ptr;
         }
-        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_partial", t);
-        int rc = launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, partials, X, (long) reduce, (long) inner, (long) tiles, (int) slices);
+        const int64_t vec = 128 / precision;
+        const char* form = std::getenv("DOCC_ROCM_SOFTMAX_TILE");
+        const int64_t vtiles = (inner / vec + 15) / 16;
+        // columns in 16-byte vectors where the tensor allows it: 16 vectors of columns per work-group
+        const bool vectors = inner % vec == 0 && (((uintptr_t) X | (uintptr_t) Y) % 16) == 0 && !(form && form[0] == 's') &&
+                             outer * vtiles <= 0x7fffffffLL / slices;
+        const int64_t launch_tiles = vectors ? vtiles : tiles;
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced%s_partial", t, vectors ? "v" : "");
+        int rc = launch(name, (uint32_t) (outer * launch_tiles * slices), 1, 1, 256, 0, s, partials, X, (long) reduce, (long) inner, (long) launch_tiles,
+                        (int) slices);
         if (rc) return rc;
-        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced_finish", t);
-        return launch(name, (uint32_t) (groups * slices), 1, 1, 256, 0, s, (const void*) partials, X, Y, (long) reduce, (long) inner, (long) tiles,
-                      (int) slices);
+        std::snprintf(name, sizeof(name), "docc_softmax_%s_sliced%s_finish", t, vectors ? "v" : "");
+        return launch(name, (uint32_t) (outer * launch_tiles * slices), 1, 1, 256, 0, s, (const void*) partials, X, Y, (long) reduce, (long) inner,
+                      (long) launch_tiles, (int) slices);
+    }
+    const int64_t per_vec = 128 / precision;
+    const char* tile_form = std::getenv("DOCC_ROCM_SOFTMAX_TILE");   // scalar | v16 | v4 (tests, tuning)
+    if (inner % per_vec == 0 && (((uintptr_t) X | (uintptr_t) Y) % 16) == 0 && !(tile_form && tile_form[0] == 's')) {
+        // 16-byte vectors: a work-group owns 16 vectors of columns and splits the extent sixteen ways, or 64 and four ways
+        // measured (us, sixteen / four ways / the scalar kernel): [64, 1024, 1024] fp32 124 / 189 / 343, [1024, 64, 1024] 144 / 127 / 198,
+        // [16, 21, 262144] 443 / 139 / 283, [256, 300, 256] 39 / 59 / 65, [4096, 128, 64] 62 / 115 / 68 (fp64: 179 / 202 / 159)
+        const int64_t row_vectors = inner / per_vec;
+        int parts = reduce >= 200 ? 16 : row_vectors >= 64 ? 4 : 0;
+        if (tile_form && tile_form[0] == 'v') parts = tile_form[1] == '4' ? 4 : 16;
+        const int64_t lanes = parts ? 256 / parts : 1;
+        const int64_t vtiles = (row_vectors + lanes - 1) / lanes;
+        if (parts && vtiles <= 0x7fffffffLL / outer) {
+            std::snprintf(name, sizeof(name), "docc_softmax_%s_tilev%d", t, parts);
+            return launch(name, (uint32_t) (outer * vtiles), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) vtiles);
+        }
     }
     std::snprintf(name, sizeof(name), "docc_softmax_%s_tile", t);
     return launch(name, (uint32_t) (outer * tiles), 1, 1, 256, 0, s, X, Y, (long) reduce, (long) inner, (long) tiles);

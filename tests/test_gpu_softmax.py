@@ -253,8 +253,11 @@ GENERAL = [  # shape, axes
     ((5, 7), (0,)), ((64, 300), (0,)), ((3, 1000, 8), (1,)), ((4, 257, 16), (1,)), ((2, 50, 33), (1,)), ((6, 31, 64), (1,)),
     ((2, 9, 200), (0, 1)), ((3, 4, 5, 6), (1, 2)), ((7, 129), (-1,)), ((1, 5000), (-1,)), ((4, 6, 2), (1,)), ((1, 4096, 1), (1,)),
     ((3, 3, 3), (0, 1, 2)), ((2, 2048, 4), (-2,)), ((5, 1, 70), (1,)),
+    # enough (outer index, column) pairs for one launch: columns in 16-byte vectors, sixteen row groups per work-group
+    ((40, 100, 68), (1,)), ((300, 7, 36), (1,)), ((9, 130, 1024), (1,)), ((64, 17, 130), (1,)), ((20, 64, 66), (1,)),
     # few columns, long extents: the rows are sliced over work-groups as well
     ((1000, 300), (0,)), ((3, 700, 130), (1,)), ((2, 4096, 65), (1,)), ((1, 257, 64), (1,)), ((5000, 40), (0,)),
+    ((2, 3000, 132), (1,)), ((1, 9000, 256), (1,)), ((3, 1024, 68), (1,)),      # the same with columns in 16-byte vectors
 ]
 
 
