@@ -281,6 +281,32 @@ def test_softmax_general_matches_oracle(rt, dt, tol, shape, axes):
     np.testing.assert_allclose(Y.sum(axis=tuple(norm)), 1.0, rtol=0, atol=max(tol, 1e-14) * 4)
 
 
+@pytest.mark.parametrize("form", ["scalar", "v16", "v4"])
+@pytest.mark.parametrize("dt,tol", [(np.float32, TOL_F32), (np.float64, 1e-12)], ids=["f32", "f64"])
+def test_softmax_over_inner_axes_every_kernel_form(rt, monkeypatch, form, dt, tol):
+    """One column per lane, or 16-byte vectors with the extent split sixteen or four ways: every form on every shape,
+    the one-launch and the sliced kernels, with a column of -inf, one with a NaN and one with +inf."""
+    monkeypatch.setenv("DOCC_ROCM_SOFTMAX_TILE", form)
+    rng = np.random.default_rng(8)
+    for shape in ((9, 70, 260), (300, 5, 36), (2, 700, 132), (1, 2100, 64), (40, 33, 1028)):
+        X = (rng.standard_normal(shape) * 6).astype(dt)
+        X[0, :, 3] = -np.inf
+        X[0, shape[1] // 2, 5] = np.nan
+        X[0, 1, 7] = np.inf
+        X[0, 2, 9] = -np.inf
+        x = dev(X)
+        y = torch.empty_like(x)
+        rt.softmax(64 if dt == np.float64 else 32, *shape, x.data_ptr(), y.data_ptr())
+        torch.cuda.synchronize()
+        Y = host(y)
+        with np.errstate(invalid="ignore"):
+            ref = oracle.softmax_axes(X, (1,))
+        assert np.array_equal(np.isnan(Y), np.isnan(ref)), shape
+        assert np.isnan(Y[0, :, 3]).all() and np.isnan(Y[0, :, 5]).all() and np.isnan(Y[0, :, 7]).all() and Y[0, 2, 9] == 0
+        ok = ~np.isnan(ref)
+        assert rel_err_max(Y[ok], ref[ok]) <= tol, shape
+
+
 def test_sliced_launch_pairs_on_two_streams_and_two_threads(rt):
     """The launchers that run as two launches with partial results in between (sliced softmax, column reduction,
     column matrix-vector product) keep those per stream: pairs issued to two streams, from two threads, many
