@@ -62,6 +62,7 @@ def parse_args():
     ap.add_argument("--no-e2e", action="store_true", help="skip the PCIe-inclusive calls through @native")
     ap.add_argument("--no-zero", action="store_true", help="skip the extra timing of the bf16 kernels on all-zero operands (profiling runs: "
                                                             "one kind of launch per kernel name)")
+    ap.add_argument("--no-graph", action="store_true", help="skip the recorded-call section (profiling runs)")
     return ap.parse_args()
 
 
@@ -475,7 +476,7 @@ def main():
     # few microseconds each. Wall time per call of the generated function (the host submits eight launches and the
     # cached allocations between them) against a replay of the same call recorded once (one submission).
     graph_replay = {}
-    if want("graph"):
+    if want("graph") and not args.no_graph:
         import docc_amd.torch as docc_torch
 
         os.environ.setdefault("DOCC_TMP", str(Path(tempfile.gettempdir()) / f"docc_bench_{os.getpid()}"))
