@@ -9,7 +9,9 @@ The reference goes FX -> torch-mlir -> linalg -> SDFG and supports only 2-d matm
 unpadded, bias-free convolution (mlir/lib/Target/SDFG/LinalgToSDFGTranslator.cpp:517-523,696-699);
 this front end lowers the FX graph directly and covers what the rocm kernels implement:
 
-    torch.matmul / @ / mm / bmm            -> GEMM (2-d, with transposed operands) or ml::MatMul (batched)
+    torch.matmul / @ / mm / bmm            -> GEMM (2-d, with transposed operands) or ml::MatMul (batched); bf16 operands:
+                                              the bf16 GEMM with float32 accumulation - its float32 result where the model
+                                              asks for it (`.float()`), else rounded once to bf16 (ml::Cast) as eager torch does
     softmax(x, dim=-1) on fp32             -> ml::Softmax
     F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
@@ -365,11 +367,21 @@ class _FxLowering:
             x, w = self.tensor(node, x), self.tensor(node, w)
         if not isinstance(x, _T) or not isinstance(w, _T) or len(w.shape) != 2 or len(x.shape) < 1 or x.shape[-1] != w.shape[1]:
             self.fail(node, "linear on these operands")
-        if x.dtype != w.dtype or (out_dtype is None and x.dtype not in (self.torch.float32, self.torch.float64)):
-            self.fail(node, "linear on dtypes other than float32 / float64 (bf16 operands: pass x.float(), w.float())")
+        bf16 = self.torch.bfloat16
+        if x.dtype != w.dtype or (out_dtype is None and x.dtype not in (self.torch.float32, self.torch.float64, bf16)):
+            self.fail(node, "linear on dtypes other than float32 / float64 / bfloat16")
         n, k = w.shape
         m = int(math.prod(x.shape[:-1]))
         shape = x.shape[:-1] + [n]
+        if out_dtype is None and x.dtype == bf16:
+            # bf16 throughout, as eager torch runs it: float32 accumulation, the bias added in float32, one rounding to bf16
+            wide = self.new_tensor(shape, self.torch.float32, None)
+            self.builder.add_gemm(x.name, w.name, wide.name, "1.0", "0.0", m, n, k, False, True, k, k, n)
+            if bias is not None:
+                wide = self.elementwise(node, "add", wide, self.cast(node, self.tensor(node, bias), self.torch.float32, None), None)
+            out = self.new_tensor(shape, bf16, dest)
+            self.builder.add_cast_op(wide.name, out.name, shape)
+            return out
         out = self.new_tensor(shape, out_dtype or x.dtype, dest if bias is None else None)
         self.builder.add_gemm(x.name, w.name, out.name, "1.0", "0.0", m, n, k, False, True, k, k, n)
         if bias is None:
@@ -407,10 +419,8 @@ class _FxLowering:
     def cast(self, node, x, dtype, dest=None):
         """ml::Cast; the same dtype passes the tensor on."""
         torch = self.torch
-        if isinstance(x, _Bf16Product):
-            if dtype != torch.float32:
-                self.fail(node, f"a bf16 product converted to {dtype} (only its float32 result is computed)")
-            return self.product(node, x.a, x.b, x.ta, x.tb, torch.float32, dest)
+        if isinstance(x, _Bf16Product) and dtype == torch.float32:
+            return self.product(node, x.a, x.b, x.ta, x.tb, torch.float32, dest)   # the GEMM's own result, not rounded in between
         if dtype == torch.float32 and dest is None:
             # bf16 -> float32 that may be an operand of a product: decided where it is used
             if isinstance(x, _T) and x.dtype == torch.bfloat16:
@@ -442,8 +452,11 @@ class _FxLowering:
             self.builder.add_cast_op(v.base.name, out.name, v.shape)
             return out
         if isinstance(v, _Bf16Product):
-            self.fail(node, "a bf16 product used without `.float()` (the target computes its float32 result; rounding it "
-                            "back to bf16 is not built)")
+            # a bf16 product used as the bf16 tensor eager torch makes of it: the float32 result of the GEMM, rounded once
+            wide = self.product(node, v.a, v.b, v.ta, v.tb, self.torch.float32, None)
+            out = self.new_tensor(wide.shape, self.torch.bfloat16, dest)
+            self.builder.add_cast_op(wide.name, out.name, wide.shape)
+            return out
         return v
 
     # ---- graph walk -------------------------------------------------------------------------

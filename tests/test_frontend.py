@@ -609,9 +609,22 @@ def test_bf16_products_lower_to_the_gemm_with_float32_accumulation():
     sdfg = docc_torch.TorchProgram(OneWidened(), target="rocm").to_sdfg(ta, tb)
     assert [n["code"] for n in sdfg.library_nodes()] == ["ml::Cast", "ml::ReLU", "ml::Cast", "GEMM"]
     assert sdfg.library_nodes()[-1]["precision"] == ord("s")
-    # the product rounded back to bf16 is not built
-    with pytest.raises(NotImplementedError, match="float"):
-        docc_torch.TorchProgram(Rounded(), target="rocm").to_sdfg(ta, tb)
+    # the product as the bf16 tensor eager torch makes of it: the float32 result of the bf16 GEMM, rounded once
+    sdfg = docc_torch.TorchProgram(Rounded(), target="rocm").to_sdfg(ta, tb)
+    assert [n["code"] for n in sdfg.library_nodes()] == ["GEMM", "ml::Cast"] and sdfg.library_nodes()[0]["precision"] == ord("b")
+    assert sdfg.containers["_docc_ret_0"]["element"] == "BFloat"
+
+    class Bf16Linear(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = torch.nn.Linear(32, 48).bfloat16()
+
+        def forward(self, x):
+            return self.fc(x)
+
+    sdfg = docc_torch.TorchProgram(Bf16Linear(), target="rocm").to_sdfg(ta)
+    codes = [n["code"] for n in sdfg.library_nodes()]
+    assert codes[0] == "GEMM" and codes[-1] == "ml::Cast" and "ml::Add" in codes and sdfg.containers["_docc_ret_0"]["element"] == "BFloat"
 
 
 def test_torch_lowering_of_composite_activations_and_layer_norm():

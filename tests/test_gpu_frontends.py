@@ -696,6 +696,33 @@ def test_torch_attention_with_other_head_dimensions(D):
         assert rel_err_max(out.float().cpu().numpy(), oracle.attention(bits(Q), bits(K), bits(V))) <= 2e-2
 
 
+def test_torch_bf16_products_and_linear_give_bf16_like_eager():
+    """A bf16 matmul and a bf16 nn.Linear return bf16 tensors as eager torch does: float32 accumulation, the bias added in
+    float32, one rounding at the end. Against the float64 product of the bf16 values rounded to bf16 (eager on the GPU
+    rounds the same way, so at most a last bit of bf16 differs), and against the oracle's bf16 GEMM before the rounding."""
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.fc = torch.nn.Linear(192, 96).bfloat16()
+
+        def forward(self, a, b):
+            return torch.matmul(a, b), self.fc(a)
+
+    torch.manual_seed(8)
+    model = Net().cuda()
+    a, b = torch.randn(130, 192).bfloat16().cuda(), torch.randn(192, 72).bfloat16().cuda()
+    program = docc_torch.compile_torch(model, (a, b), target="rocm")
+    p, l = program(a, b)
+    assert p.dtype == l.dtype == torch.bfloat16 and p.shape == (130, 72) and l.shape == (130, 96)
+    wide = oracle.gemm_bf16(bits(a.cpu()), bits(b.cpu()))
+    assert torch.equal(p.cpu(), torch.from_numpy(wide).bfloat16())                     # the fp32 result of the bf16 GEMM, rounded to nearest even
+    with torch.no_grad():
+        ref = (a.double() @ model.fc.weight.double().T + model.fc.bias.double())
+        eager = model.fc(a)
+    assert rel_err_max(l.float().cpu().numpy(), ref.cpu().numpy()) <= 2e-2
+    assert (l.float() - eager.float()).abs().max().item() <= 2.0 ** -7 * eager.float().abs().max().item()      # a last bit of bf16 at most
+
+
 def test_power_operator_through_both_front_ends():
     """x ** 2, x ** y and np.power lower to ml::Pow (array or scalar operand); torch.pow likewise."""
     @native(target="rocm")
