@@ -57,12 +57,13 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise,graph")
+    ap.add_argument("--only", type=str, default="", help="comma list of: softmax,dgemm,sgemm,bgemm,attention,conv,elementwise,shapes,graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines (profiling runs)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the PCIe-inclusive calls through @native")
     ap.add_argument("--no-zero", action="store_true", help="skip the extra timing of the bf16 kernels on all-zero operands (profiling runs: "
                                                             "one kind of launch per kernel name)")
     ap.add_argument("--no-graph", action="store_true", help="skip the recorded-call section (profiling runs)")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the section on shapes other than the benchmark configurations")
     return ap.parse_args()
 
 
@@ -471,6 +472,56 @@ def main():
                 "sample": "full tensor, the Map the reference's ElementWiseBinaryNode expands to (omp parallel for)"}
         del As, Bs, Ys
 
+    # ---- other shapes of the same nodes: the forms the launchers pick away from the benchmark configurations ----------
+    # (HBM-bound entries walk four input tensors in turn, like the elementwise section; `frac` is always relative to one
+    # read and one write of the tensor, so a form that reads twice shows it)
+    other = {}
+    if want("shapes") and not args.no_shapes:
+        def hbm(name, nbytes, fn, iters=48):
+            ms = time_kernel(fn, iters, 8)
+            other[name] = {"kernel_us": round(ms * 1e3, 2), "bound": "hbm", "achieved_GBps": round(nbytes / ms / 1e6, 1),
+                           "frac": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4), "algorithmic_bytes": nbytes}
+
+        def mfma(name, dtype, flops, fn, iters=48):
+            ms = time_kernel(fn, iters, 8)
+            other[name] = {"kernel_us": round(ms * 1e3, 2), "bound": "mfma", "achieved_TFLOPs": round(flops / ms / 1e9, 1),
+                           "frac": round(flops / ms / 1e9 / PEAK_TFLOPS[dtype], 4), "flop": flops}
+
+        n = 8192 * 4096
+        xs = [torch.randn(n, device="cuda") * 8 for _ in range(ROTATE)]
+        y = torch.empty(n, device="cuda")
+        x_ = lambda i: xs[i % ROTATE].data_ptr()
+        hbm("softmax_f32_1048576x32_rows_sharing_a_wavefront", 8 * n, lambda i: rt.softmax(32, 1 << 20, 32, 1, x_(i), y.data_ptr(), stream))
+        hbm("softmax_f32_512x65536_sixteen_wavefronts_a_row", 8 * n, lambda i: rt.softmax(32, 512, 65536, 1, x_(i), y.data_ptr(), stream))
+        hbm("softmax_f32_32x1048576_rows_in_slices", 8 * n, lambda i: rt.softmax(32, 32, 1 << 20, 1, x_(i), y.data_ptr(), stream))
+        hbm("softmax_f32_8190x4097_rows_off_the_vector_boundary", 8 * 8190 * 4097, lambda i: rt.softmax(32, 8190, 4097, 1, x_(i), y.data_ptr(), stream))
+        hbm("softmax_f32_32x1024x1024_over_axis_1", 8 * n, lambda i: rt.softmax(32, 32, 1024, 1024, x_(i), y.data_ptr(), stream))
+        hbm("softmax_f64_8192x2048", 8 * n, lambda i: rt.softmax(64, 8192, 2048, 1, x_(i), y.data_ptr(), stream))
+        hbm("reduce_sum_f32_1x33554432_row_in_pieces", 4 * n, lambda i: rt.reduce("sum", 32, 1, n, 1, x_(i), y.data_ptr(), stream))
+        hbm("reduce_sum_f32_1048576x32_rows_sharing_a_wavefront", 4 * n + 4 * (1 << 20), lambda i: rt.reduce("sum", 32, 1 << 20, 32, 1, x_(i), y.data_ptr(), stream))
+        # a few rows against a wide matrix: bound by reading the matrix (K in parts over two launches)
+        m_, n_, k_ = 32, 4096, 4096
+        hbm("sgemm_32x4096x4096_k_in_parts", 4 * (k_ * n_ + m_ * k_ + m_ * n_),
+            lambda i: rt.sgemm(m_, n_, k_, 1.0, y.data_ptr(), k_, x_(i), n_, 0.0, y.data_ptr() + 4 * (1 << 22), n_, stream=stream))
+        del xs, y
+        for D in (128, 32):
+            torch.manual_seed(3)
+            Q, K, V = (torch.randn(8, 16, 2048, D).bfloat16().cuda() for _ in range(3))
+            O = torch.empty(8, 16, 2048, D, device="cuda", dtype=torch.bfloat16)
+            mfma(f"attention_b8h16s2048d{D}", "bf16", 4 * 8 * 16 * 2048 * 2048 * D,
+                 lambda i: rt.attention_bf16(8, 16, 2048, 2048, D, D ** -0.5, Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), out_bf16=True, stream=stream))
+            del Q, K, V, O
+        torch.manual_seed(4)
+        for name, (C, H, OC, st) in (("conv2d_n32c128hw28k3", (128, 28, 128, 1)), ("conv2d_n32c256hw14k3", (256, 14, 256, 1)), ("conv2d_n32c128hw56k3s2", (128, 56, 128, 2))):
+            X = torch.randn(32, C, H, H).cuda()
+            W = (torch.randn(OC, C, 3, 3) * (2.0 / (9 * C)) ** 0.5).cuda()
+            b = (torch.randn(OC) * 0.1).cuda()
+            OH = (H + 2 - 3) // st + 1
+            Y = torch.empty(32, OC, OH, OH, device="cuda")
+            mfma(name, "f32", 2 * 32 * OC * OH * OH * C * 9,
+                 lambda i: rt.conv2d_f32(32, C, H, H, OC, 3, 3, (st, st), (1, 1), (1, 1), X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), stream=stream))
+            del X, W, b, Y
+
     # ---- a launch-bound function: kernel by kernel, and replayed as a HIP graph --------------------------
     # LayerNorm -> Linear -> GELU -> Linear + residual on [8, 128, 256] device tensors compiles to eight kernels of a
     # few microseconds each. Wall time per call of the generated function (the host submits eight launches and the
@@ -587,6 +638,8 @@ def main():
     if "cpu_baseline" in out:
         line["cpu_baseline"] = out["cpu_baseline"]
     line["kernels"] = kernels
+    if other:
+        line["other_shapes"] = other
     if graph_replay:
         line["graph_replay"] = graph_replay
     if end_to_end:

@@ -39,7 +39,9 @@ extern "C" int docc_rocm_reduce(docc_rocm_stream_t stream, int op, int precision
         // Long rows, and too few of them for eight wavefronts per CU: each row in pieces of at least 4096 elements, one
         // wavefront a piece, the pieces' results through the stream's buffer of partial results and a second launch
         if (outer < (int64_t) cus * 8 && reduce >= 8192) {
-            int64_t slices = ((int64_t) cus * 8 + outer - 1) / outer;
+            int64_t pieces_wanted = (int64_t) cus * 8;
+            if (const char* e = std::getenv("DOCC_ROCM_REDUCE_PIECES")) pieces_wanted = std::atoll(e) > 0 ? std::atoll(e) : pieces_wanted;   // tuning
+            int64_t slices = (pieces_wanted + outer - 1) / outer;
             if (slices > reduce / 4096) slices = reduce / 4096;
             if (slices > 4096) slices = 4096;
             const int64_t chunk = ((reduce + slices - 1) / slices + 1023) / 1024 * 1024;

@@ -138,6 +138,20 @@ extern "C" int docc_rocm_transpose(docc_rocm_stream_t stream, int element_bytes,
     bool quads = element_bytes == 4 && p.a_ext % 4 == 0 && p.b_ext % 4 == 0 && p.b_in_stride % 4 == 0 && p.a_out_stride % 4 == 0 &&
                  ((uintptr_t) X | (uintptr_t) Y) % 16 == 0 && !std::getenv("DOCC_ROCM_TRANSPOSE_SCALAR");
     for (int i = 0; i < p.rank; i++) quads = quads && p.in_stride[i] % 4 == 0 && p.out_stride[i] % 4 == 0;
+    if (quads) {
+        // tiles of 128 x 128 (rows of 512 bytes on both sides) where they still number four per CU: on tensors met for the
+        // first time [8192, 4096] takes 53.5 us against 56.5, [16384, 16384] 427 against 465, [2048, 2048] 9.6 against 7.9.
+        // DOCC_ROCM_TRANSPOSE_WIDE=1|0 forces the choice (tests, tuning).
+        TransposeParams w = p;
+        w.tiles_a = (p.a_ext + 127) / 128;
+        w.tiles_b = (p.b_ext + 127) / 128;
+        const int64_t wide_blocks = planes * w.tiles_a * w.tiles_b;
+        int cus = compute_units();
+        if (cus <= 0) cus = 256;
+        const char* force = std::getenv("DOCC_ROCM_TRANSPOSE_WIDE");
+        if (force ? force[0] == '1' : wide_blocks >= 4 * (int64_t) cus)
+            return launch("docc_transpose_tile4w_b32", (uint32_t) wide_blocks, 1, 1, 256, 0, st, X, Y, w);
+    }
     if (quads) return launch("docc_transpose_tile4_b32", (uint32_t) blocks, 1, 1, 256, 0, st, X, Y, p);
     std::snprintf(name, sizeof(name), "docc_transpose_tile_b%d", element_bytes * 8);
     return launch(name, (uint32_t) blocks, 1, 1, 256, 0, st, X, Y, p);

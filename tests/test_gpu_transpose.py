@@ -75,6 +75,16 @@ def test_tile_in_128_bit_units_equals_the_one_element_tile(rt, monkeypatch):
     assert np.array_equal(host(y).reshape(want.shape), want)
 
 
+@pytest.mark.parametrize("wide", ["1", "0"])
+def test_tiles_of_128_and_of_64_move_the_same_elements(rt, monkeypatch, wide):
+    """Large tensors take tiles of 128 x 128, small ones tiles of 64 x 64: either forced, on extents that end inside a
+    tile, and with batch axes in front and behind."""
+    monkeypatch.setenv("DOCC_ROCM_TRANSPOSE_WIDE", wide)
+    for shape, perm in (((260, 516), (1, 0)), ((3, 132, 200), (0, 2, 1)), ((128, 128), (1, 0)), ((4, 644), (1, 0)), ((2, 300, 8, 72), (0, 3, 2, 1))):
+        X = values(shape, np.float32, sum(shape))
+        assert np.array_equal(run_transpose(rt, X, perm), oracle.transpose(X, perm)), (shape, perm)
+
+
 def test_transpose_involution_at_full_size_and_errors(rt):
     """[8192, 4096] fp32: transposing twice gives the input back; row sums become column sums."""
     g = torch.Generator(device="cuda").manual_seed(4)
