@@ -234,8 +234,9 @@ DOCC_CONV_GATHER(64, 128, 16, 2, 2, false, u)
 
 namespace docc_k {
 
-template <int KH, int KW, bool SPLIT = false, bool NARROW = false, int TILES = 7>
+template <int KH, int KW, bool SPLIT = false, bool NARROW = false, int TILES = 7, bool MULTI = false>
 struct ConvHaloKernel {
+    static_assert(!MULTI || !SPLIT, "several images per work-group: the plain strips only");
     static_assert(!NARROW || SPLIT, "the narrow tile is the shared tile of a split strip");
     static_assert(TILES >= 2 && (!SPLIT || TILES == 7), "the last chunk goes in groups of at least two tiles; the split strip is 13 tiles");
     static constexpr int KHW = KH * KW;
@@ -248,7 +249,10 @@ struct ConvHaloKernel {
     static constexpr int NR = 3;                 // patch pixels per thread per chunk (upper bound)
     static constexpr int NWV = (64 * KC / 4 + 255) / 256;   // weight float4s per thread per chunk
 
-    static __device__ __forceinline__ void run(const ConvParams& p, int TH) {
+    // MULTI: a work-group takes G whole images (TH == OH; images of a few pixels, which alone would fill a fraction of
+    // the smallest strip): the patch buffer holds their G patches one after the other, pixel q of the strip is pixel
+    // q % (OH * OW) of image q / (OH * OW).
+    static __device__ __forceinline__ void run(const ConvParams& p, int TH, int G = 1) {
         extern __shared__ __attribute__((aligned(16))) unsigned char docc_conv_lds[];
         float* const lds = reinterpret_cast<float*>(docc_conv_lds);
         const int tid = threadIdx.x, lane = tid & 63, wave = SPLIT ? __builtin_amdgcn_readfirstlane(tid >> 6) : tid >> 6;   // SPLIT: the mirrored tap is a scalar
@@ -256,11 +260,13 @@ struct ConvHaloKernel {
         const int ocw = wave & 1, pg = wave >> 1;
 
         const int WP = (p.OW - 1) * p.stride_w + KW, PR = (TH - 1) * p.stride_h + KH, PS = PR * WP;   // the patch a strip reads
-        const int stage_elems = A_ELEMS + (PS + 1) * CI;    // [weights | patch | one spare pixel]
+        const int PST = MULTI ? G * PS : PS;                // patch pixels of the work-group
+        const int stage_elems = A_ELEMS + (PST + 1) * CI;   // [weights | patch | one spare pixel]
         const int strips = (p.OH + TH - 1) / TH;
-        const int n = blockIdx.x / strips, oh0 = (blockIdx.x % strips) * TH;
+        const int n = MULTI ? blockIdx.x * G : blockIdx.x / strips, oh0 = MULTI ? 0 : (blockIdx.x % strips) * TH;
         const int oc0 = blockIdx.y * 64;
-        const int npix = TH * p.OW;                    // pixels of a full strip
+        const int ipix = p.OH * p.OW;                  // MULTI: pixels of an image
+        const int npix = MULTI ? G * ipix : TH * p.OW; // pixels of a full strip
 
         // per-lane patch offsets (floats) of the 7 column tiles of this wave: pixel (r, c) of the
         // strip and the channel half of this lane
@@ -273,7 +279,12 @@ struct ConvHaloKernel {
             for (int j = 0; j < TN; j++) {
                 int q = tile_pixel0(j) + l32;
                 q = q < npix ? q : 0;
-                boff[j] = ((q / p.OW) * p.stride_h * WP + (q % p.OW) * p.stride_w) * CI + 4 * g;
+                int patch0 = 0;
+                if constexpr (MULTI) {
+                    patch0 = (q / ipix) * PS;
+                    q %= ipix;
+                }
+                boff[j] = (patch0 + (q / p.OW) * p.stride_h * WP + (q % p.OW) * p.stride_w) * CI + 4 * g;
             }
         };
 
@@ -286,10 +297,11 @@ struct ConvHaloKernel {
 #pragma unroll
         for (int r = 0; r < NR; r++) {
             const int e = tid + r * 256;
-            const int ih = oh0 * p.stride_h - p.pad_h + e / WP, iw = e % WP - p.pad_w;
-            inside[r] = e < PS && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-            goff[r] = inside[r] ? 4u * (unsigned) (ih * p.W + iw) : 0u;
-            slot[r] = (e < PS ? e : PS) * CI;
+            const int img = MULTI ? e / PS : 0, pe = MULTI ? e % PS : e;      // image of the group, pixel of its patch
+            const int ih = oh0 * p.stride_h - p.pad_h + pe / WP, iw = pe % WP - p.pad_w;
+            inside[r] = e < PST && n + img < p.N && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            goff[r] = inside[r] ? 4u * (unsigned) (img * p.C * p.H * p.W + ih * p.W + iw) : 0u;
+            slot[r] = (e < PST ? e : PST) * CI;
         }
         const long HW = (long) p.H * p.W;
         const char* xn = reinterpret_cast<const char*>(p.X + (long) n * p.C * HW);
@@ -305,7 +317,7 @@ struct ConvHaloKernel {
             const int row = idx / (KC / 4), rem = idx % (KC / 4);     // rem = 2*tap + channel half
             const int oc = oc0 + row < p.OC ? oc0 + row : p.OC - 1;
             woff[i] = 4u * (unsigned) (oc * K + (rem & 1) * 4 * KHW + (rem >> 1));
-            wdst[i] = idx < 64 * (KC / 4) ? row * LDA_S + rem * 4 : A_ELEMS + PS * CI;
+            wdst[i] = idx < 64 * (KC / 4) ? row * LDA_S + rem * 4 : A_ELEMS + PST * CI;
         }
 
         f32x16 acc[TN];
@@ -504,7 +516,7 @@ struct ConvHaloKernel {
         // leave at once and the kernel waits for memory to take them (25.7 MB: 3.4-4.3 us of 66.5 for N32 C64 56x56;
         // 1.3 us this way, against 1.1 us that the tile-by-tile order costs). Tap 0's operands are the ones the chunk
         // before has fetched.
-        const bool whole = oc0 + 64 <= p.OC && oh0 + TH <= p.OH && (pg + 1) * (TOWN * 32) <= npix;
+        const bool whole = !MULTI && oc0 + 64 <= p.OC && oh0 + TH <= p.OH && (pg + 1) * (TOWN * 32) <= npix;
         const bool early = DOCC_CONV_EARLY_STORE && KHW > 1 && whole && (long) p.OH * p.OW * 64 * 4 < (1L << 31);
         const long plane = (long) p.OH * p.OW;
         auto last_tiles = [&](auto par_c, int cur) {
@@ -680,10 +692,17 @@ struct ConvHaloKernel {
         // that lies wholly inside the output (the usual case) is stored by straight-line code; one
         // branch per element costs more in instruction fetch than the stores themselves.
         auto store_tile_checked = [&](int j, bool with_bias) {
-            const int q = tile_pixel0(j) + l32;
+            int q = tile_pixel0(j) + l32;
+            if (q >= npix) return;
+            int img = 0;
+            if constexpr (MULTI) {
+                img = q / ipix;
+                q %= ipix;
+                if (n + img >= p.N) return;
+            }
             const int oh = oh0 + q / p.OW, ow = q % p.OW;
-            if (q >= npix || oh >= p.OH) return;
-            float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+            if (oh >= p.OH) return;
+            float* ybase = p.Y + ((long) (n + img) * p.OC * p.OH + oh) * p.OW + ow;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
@@ -809,6 +828,23 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4(do
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2(docc_k::ConvParams p, int TH) {
     docc_k::ConvHaloKernel<1, 1, false, false, 2>::run(p, TH);
+}
+
+// several whole images per work-group (images of a few pixels)
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 4, true>::run(p, TH, G);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 2, true>::run(p, TH, G);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 4, true>::run(p, TH, G);
+}
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 2, true>::run(p, TH, G);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split(docc_k::ConvParams p, int TH) {

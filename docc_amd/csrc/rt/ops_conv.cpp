@@ -42,10 +42,12 @@ constexpr int64_t kConvWorkspaceCap = int64_t(2) << 30;   // images are processe
 // per-work-group set-up (measured on 32 x 64 x 56 x 56: 7 strips of 8 rows 68.4 us, 8 strips of 7 rows 70.9 us
 // with 7 tiles a wave, 67.0 us with 6.5); strips of 256 or 128 pixels (4 or 2 tiles per wave) for small images,
 // whose staging of weights per chunk is spread over fewer MFMAs (taken as 8 % and 20 %).
-// DOCC_ROCM_CONV=halo-split / halo-split-wide / halo-whole / halo-t4 / halo-t2 force a form (tests, tuning).
+// Images smaller than half the smallest strip go several to a work-group (`images`, the kernels with the suffix m).
+// DOCC_ROCM_CONV=halo-split / halo-split-wide / halo-whole / halo-t4 / halo-t2 / halo-t4m / halo-t2m force a form (tests, tuning).
 struct HaloPlan {
     int tiles = 7;        // column tiles per wave
     int64_t TH = 1;       // output rows per strip
+    int64_t images = 1;   // whole images per work-group (then TH == OH): images of a few pixels share a strip
     bool split = false, narrow = false;
     double cost = 0;      // rounds x tiles per wave x overhead
 };
@@ -104,6 +106,25 @@ HaloPlan plan_halo(int64_t N, int64_t OC, int64_t OH, int64_t OW, int64_t KH, in
         if (take) {
             plan.tiles = form.tiles;
             plan.TH = th;
+            plan.images = 1;
+            plan.split = plan.narrow = false;
+            plan.cost = cost;
+        }
+    }
+    // images of a few pixels (7 x 7: 49 of the 128 pixels of the smallest strip): several whole images per work-group
+    for (const auto& form : small) {
+        int64_t g = 64 * form.tiles / (OH * OW);
+        const int64_t patch = ((OH - 1) * stride_h + KH) * ((OW - 1) * stride_w + KW);
+        while (g >= 2 && !(g * patch <= 3 * 256 && 3 * (64 * (8 * KH * KW + 4) + 8 * (g * patch + 1)) * 4 <= 160 * 1024)) g--;
+        if (g < 2 || g > N) continue;
+        const double cost = (double) ((((N + g - 1) / g) * ocb + cus - 1) / cus) * form.tiles * form.overhead;
+        char name[16];
+        std::snprintf(name, sizeof(name), "%sm", form.name);
+        const bool take = forced && plan.cost > 0.0 ? std::strcmp(force, name) == 0 : cost < plan.cost || plan.cost == 0.0;
+        if (take) {
+            plan.tiles = form.tiles;
+            plan.TH = OH;
+            plan.images = g;
             plan.split = plan.narrow = false;
             plan.cost = cost;
         }
@@ -272,10 +293,17 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         if (cus <= 0) cus = 256;
         const HaloPlan plan = plan_halo(N, OC, OH, OW, KH, KW, stride_h, stride_w, cus);
         const int64_t TH = plan.TH;
-        const int64_t PS = ((TH - 1) * stride_h + KH) * ((OW - 1) * stride_w + KW);   // patch pixels
+        const int64_t PS = plan.images * ((TH - 1) * stride_h + KH) * ((OW - 1) * stride_w + KW);   // patch pixels
         const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
-        if (plan.cost > 0.0 && halo_strip_fits(TH, OW, KH, KW, stride_h, stride_w) && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
+        if (plan.images > 1 && plan.cost > 0.0 && PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) &&
+            plan.images * C * H * W < (int64_t(1) << 29) && (OC + 63) / 64 <= 65535) {
+            char name[64];
+            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s_t%dm", KH == 3 ? "3x3" : "1x1", plan.tiles);
+            return launch(name, (uint32_t) ((N + plan.images - 1) / plan.images), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4),
+                          (hipStream_t) stream, p, (int) TH, (int) plan.images);
+        }
+        if (plan.images == 1 && plan.cost > 0.0 && halo_strip_fits(TH, OW, KH, KW, stride_h, stride_w) && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
             char name[64];
             std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s", KH == 3 ? "3x3" : "1x1",
                           plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "");

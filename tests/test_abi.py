@@ -66,7 +66,7 @@ def test_kernels_the_launchers_name_are_in_the_images():
              "block16_v16", "any4_v1", "any4_v4", "any4_v16", "any16_v8", "any16_v16"]
     forms += [f"wave_v{v}" for v in (1, 2, 4, 8, 16)] + [f"block_v{v}" for v in (1, 2, 4, 8, 16)] + [f"sub{v}" for v in (1, 2, 4, 8, 16, 32)]
     named |= {f"docc_softmax_{t}_{form}" for t in ("f32", "f64") for form in forms}
-    named |= {f"docc_conv2d_f32_halo_{k}{form}" for k, fs in (("3x3", ("", "_split", "_split16", "_t4", "_t2")), ("1x1", ("", "_t4", "_t2"))) for form in fs}
+    named |= {f"docc_conv2d_f32_halo_{k}{form}" for k, fs in (("3x3", ("", "_split", "_split16", "_t4", "_t2", "_t4m", "_t2m")), ("1x1", ("", "_t4", "_t2", "_t4m", "_t2m"))) for form in fs}
     named |= {f"docc_attention_bf16_d{d}_q{q}_{o}" for d in (32, 64, 128) for q in (128, 256) for o in ("f32out", "bf16out")}
     # the entry point that may look nothing up at a call resolves every one of these forms at set-up
     listed = re.search(r"forms\[\] = \{(.*?)\};", (ROOT / "docc_amd" / "csrc" / "rt" / "noalloc.hip").read_text(), re.S).group(1)

@@ -51,6 +51,10 @@ CASES = [
     (2, 8, 15, 21, 40, 3, 3, (2, 1), (1, 1), (1, 1), False),    # mixed strides, odd image
     (2, 32, 14, 14, 64, 1, 1, (2, 2), (0, 0), (1, 1), True),    # a 1x1 downsampling layer
     (1, 8, 9, 120, 16, 3, 3, (2, 2), (0, 0), (1, 1), True),     # wide rows: one or two output rows per strip
+    (7, 16, 7, 7, 70, 3, 3, (1, 1), (1, 1), (1, 1), True),      # images of 49 pixels: several to a work-group, the last group not full
+    (5, 8, 4, 6, 64, 3, 3, (1, 1), (1, 1), (1, 1), False),
+    (9, 16, 9, 9, 32, 3, 3, (2, 2), (1, 1), (1, 1), True),      # 5 x 5 outputs of a strided layer
+    (6, 24, 5, 5, 40, 1, 1, (1, 1), (0, 0), (1, 1), True),
 ]
 
 
@@ -154,7 +158,7 @@ def run_conv_ws(rt, X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1),
     return host(y), need
 
 
-@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-split-wide", "halo-whole", "halo-t4", "halo-t2", ""])
+@pytest.mark.parametrize("force", ["gemm", "gather", "halo", "halo-split", "halo-split-wide", "halo-whole", "halo-t4", "halo-t2", "halo-t4m", "halo-t2m", ""])
 @pytest.mark.parametrize("case", CASES)
 def test_conv_every_path_integer_exact(rt, monkeypatch, force, case):
     """Each way to run a layer (forced through DOCC_ROCM_CONV; a path that does not apply falls back; halo-split and
