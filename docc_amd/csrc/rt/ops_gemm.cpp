@@ -225,6 +225,21 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                                            bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
     }
     const bool epilogue = bias || activation >= 0;
+    // A tall matrix times a few columns held as numpy holds them (B [k][n], n small): rows of B are a few elements long, so
+    // the kernels that read whole vectors along n do not apply (n = 2, 5, 9 ... went through the element-wise tiles at a
+    // ninth of the rate) and the matrix-vector kernels want the vectors contiguous along k. B is small: it is transposed
+    // into a block of the device block cache first (k x n elements), and the product runs as A B'^T.
+    if (!tb && batch == 1 && n >= 2 && n <= 64 && ldb == n && m >= 1024 && k >= 256 && k % (16 / (int64_t) sizeof(T)) == 0 &&
+        (n <= 4 || n % (16 / (int64_t) sizeof(T)) != 0) && !std::getenv("DOCC_ROCM_GEMV_OFF")) {
+        void* bt = nullptr;
+        if ((rc = docc_rocm_malloc_async(&bt, (size_t) (n * k) * sizeof(T), stream))) return rc;
+        const int64_t shape[2] = {k, n}, perm[2] = {1, 0};
+        rc = docc_rocm_transpose(stream, (int) sizeof(T), 2, shape, perm, B, bt);
+        if (!rc)
+            rc = gemm_launch<T, S>(prefix, stream, trans_a, DOCC_ROCM_TRANS, m, n, k, alpha, A, lda, (const T*) bt, k, beta, C, ldc, pick, bias, activation);
+        const int rc2 = docc_rocm_free_async(bt, stream);
+        return rc ? rc : rc2;
+    }
     if ((m <= 8 || n <= 8) && batch == 1 && (!epilogue || ldc == n)) {
         rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
         if (rc == 0 && epilogue) {

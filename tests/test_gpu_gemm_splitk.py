@@ -86,3 +86,18 @@ def test_gemm_parts_on_two_streams_do_not_share_partial_results(rt):
         assert np.array_equal(host(c[i]), oracle.gemm(A[i], B[i]))
     for s in streams:
         rt.stream_destroy(s)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("n", [2, 3, 5, 9, 17, 63])
+def test_tall_matrix_times_a_few_columns_stored_by_rows(rt, dt, n):
+    """A [m, k] times B [k, n] with a handful of columns: B's rows are too short for the kernels that read whole vectors,
+    so B is transposed into a temporary first and the product runs against its rows. Exact on integer-valued operands,
+    with alpha, beta and a padded C."""
+    rng = np.random.default_rng(n)
+    m, k = 1500, 512
+    A, B = int_matrix(rng, (m, k), dt, lim=4), int_matrix(rng, (k, n), dt, lim=4)
+    C0 = int_matrix(rng, (m, n), dt)
+    C = run_gemm(rt, A, B, C=C0.copy(), alpha=-1.0, beta=2.0, ldc=n + 3)
+    assert np.array_equal(C, oracle.gemm(A, B, C=C0.copy(), alpha=-1.0, beta=2.0))
+    assert np.array_equal(run_gemm(rt, A, B), oracle.gemm(A, B))
