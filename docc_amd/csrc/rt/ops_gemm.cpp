@@ -45,7 +45,9 @@ int gemv_launch(const char* prefix, hipStream_t s, bool ta, bool tb, int64_t m, 
         if (m > 8 && n > 8) return 1;
         int cusm = compute_units();
         if (cusm <= 0) cusm = 256;
-        const int64_t max_vectors = sizeof(T) == 4 ? 8 : 4;      // fp64 8 x 8192 x 8192: 296 us here, 172 through the tiles
+        // five to eight vectors would be two passes over the matrix: the tiles with K in parts are faster (fp32 8 x 4096 x 4096:
+        // 39 us here, 26 there; 8 x 8192 x 8192: 95 against 81; fp64 8 x 8192 x 8192: 296 against 172)
+        const int64_t max_vectors = 4;
         if (sizeof(T) != 2 && ((m <= max_vectors && !ta && !tb) || (n <= max_vectors && ta && !tb && m > 8))) {
             // the large operand is stored [k][columns] (y = x W with W as numpy holds it): columns form, sliced over k
             const bool small_a = m <= max_vectors && !ta;
