@@ -499,10 +499,11 @@ def main():
         hbm("softmax_f64_8192x2048", 8 * n, lambda i: rt.softmax(64, 8192, 2048, 1, x_(i), y.data_ptr(), stream))
         hbm("reduce_sum_f32_1x33554432_row_in_pieces", 4 * n, lambda i: rt.reduce("sum", 32, 1, n, 1, x_(i), y.data_ptr(), stream))
         hbm("reduce_sum_f32_1048576x32_rows_sharing_a_wavefront", 4 * n + 4 * (1 << 20), lambda i: rt.reduce("sum", 32, 1 << 20, 32, 1, x_(i), y.data_ptr(), stream))
-        # a few rows against a wide matrix: bound by reading the matrix (K in parts over two launches)
-        m_, n_, k_ = 32, 4096, 4096
-        hbm("sgemm_32x4096x4096_k_in_parts", 4 * (k_ * n_ + m_ * k_ + m_ * n_),
-            lambda i: rt.sgemm(m_, n_, k_, 1.0, y.data_ptr(), k_, x_(i), n_, 0.0, y.data_ptr() + 4 * (1 << 22), n_, stream=stream))
+        # a few rows against a wide matrix: bound by reading the matrix. Up to 32 rows B goes from global memory straight into
+        # the MFMA operands, above that through the tiles; both with K in parts over two launches
+        for m_, n_, k_, how in ((16, 8192, 4096, "b_straight_into_the_mfma"), (32, 4096, 4096, "b_straight_into_the_mfma"), (64, 4096, 4096, "tiles_k_in_parts")):
+            hbm(f"sgemm_{m_}x{n_}x{k_}_{how}", 4 * (k_ * n_ + m_ * k_ + m_ * n_),
+                lambda i: rt.sgemm(m_, n_, k_, 1.0, y.data_ptr(), k_, x_(i), n_, 0.0, y.data_ptr() + 4 * (1 << 22), n_, stream=stream))
         del xs, y
         for D in (128, 32):
             torch.manual_seed(3)

@@ -52,6 +52,7 @@ KERNEL_FAMILIES = {
     "reduce": "reduce.hip",
     "transpose": "transpose.hip",
     "gemv": "gemv.hip",
+    "gemm_skinny": "gemm_skinny.hip",
 }
 
 # Per-family extra device flags. "-amdgpu-mfma-vgpr-form" keeps MFMA accumulators in ordinary
@@ -68,6 +69,7 @@ FAMILY_FLAGS = {
     "gemm_bf16_async_epilogue": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "conv2d": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "attention": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "gemm_skinny": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
 }
 
 # packed fp32 VALU ops are switched off for every device compile

@@ -1,0 +1,219 @@
+// A few rows times a wide matrix for gfx950: C[m, n] = alpha * A[m, k] * op(B) + beta * C with 5 <= m <= 32 and n, k in the
+// thousands (a batch of vectors through a layer). The product reads B once (4 k n bytes) for 2 m k n flops, so it is bound by
+// HBM as long as the MFMA work stays small: the 32 x 32 x 2 instruction allows 9.8 TB/s of B at the device's fp32 rate, the
+// 16 x 16 x 4 one (m <= 16) twice that. The tiles of the GEMM kernels stage both operands through LDS in steps a work-group
+// waits out and pad m to 64; here B goes from global memory straight into the MFMA operand registers:
+//   * a work-group owns 128 columns of one part of K; its NW wavefronts cut that part among themselves, every wavefront
+//     keeps an MT x 128 block of sums in registers (MT = 16 or 32 rows);
+//   * K advances in chunks of CH: a lane holds CH / G consecutive k of its row of A (G = 64 / MT lane groups along k) and
+//     loads, for each of those k, the columns (B stored [k][n]: 128-bit loads along n) or, for its rows of B (B stored
+//     [n][k]), 128-bit loads along k that it feeds to the MFMA; the loads of the next chunks are issued before the products
+//     of this one;
+//   * the wavefronts' blocks are added pairwise through LDS (wave w + NW/2 into wave w, then halves again), and wave 0
+//     stores the part's product; the launcher adds the parts in order with docc_splitk_combine_f32, so the result does
+//     not depend on scheduling. With one part the store applies alpha and beta itself.
+// Sums run in fp32 (cblas_sgemm semantics, reference gemm_node.cpp:474-505).
+#include "common.h"
+
+namespace docc_k {
+
+typedef float skinny_f32x4 __attribute__((ext_vector_type(4)));
+typedef float skinny_f32x16 __attribute__((ext_vector_type(16)));
+
+template <int MT> struct SkinnyMfma;
+template <> struct SkinnyMfma<32> {
+    typedef skinny_f32x16 acc_t;
+    static constexpr int NACC = 16;
+    static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+    // row of register r of the block of sums for lane group g (the column is the lane's index within its group)
+    static __device__ __forceinline__ int row(int g, int r) { return 8 * (r / 4) + 4 * g + (r % 4); }
+};
+template <> struct SkinnyMfma<16> {
+    typedef skinny_f32x4 acc_t;
+    static constexpr int NACC = 4;
+    static __device__ __forceinline__ acc_t mfma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+    static __device__ __forceinline__ int row(int g, int r) { return 4 * g + r; }
+};
+
+// MT: rows of the MFMA (m <= MT). TB: B stored [n][k] (C = A B^T). NW: wavefronts per work-group. CH: k per chunk. NBUF: sets
+// of operand registers, NBUF - 1 chunks' loads are in flight during a chunk's products.
+// P: the part's product, [parts][m][ldp] when direct == 0, else C itself (one part).
+template <int MT, bool TB, int NW, int CH, int NBUF>
+__device__ __forceinline__ void gemm_skinny(const float* __restrict__ A, long lda, const float* __restrict__ B, long ldb, float* __restrict__ P,
+                                            long ldp, long m, long n, long k, long kpart, float alpha, float beta, int direct) {
+    typedef SkinnyMfma<MT> M;
+    typedef typename M::acc_t acc_t;
+    constexpr int G = 64 / MT;       // lane groups along k
+    constexpr int KL = CH / G;       // consecutive k of a lane in a chunk
+    constexpr int NJ = 128 / MT;     // MFMA blocks of sums across the 128 columns
+    constexpr int SETS = NJ / 4;     // NN: 128-bit loads of a lane per k (4 MT columns each over the wavefront)
+    constexpr int NLOAD = TB ? NJ * KL / 4 : KL * SETS;   // 128-bit loads of B per lane and chunk
+    constexpr int SLOT = NJ * M::NACC / 4 * 64;           // 128-bit words of a wavefront's block of sums
+    extern __shared__ __attribute__((aligned(16))) unsigned char skinny_lds[];
+    skinny_f32x4* lds = reinterpret_cast<skinny_f32x4*>(skinny_lds);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // wave: uniform, in a scalar register
+    const int c = lane % MT, g = lane / MT;
+    const long n0 = (long) blockIdx.x * 128;
+    const long part = blockIdx.y;
+    const long kw = kpart / NW;                       // a multiple of CH
+    const long k_begin = part * kpart + wave * kw;
+    long k_end = k_begin + kw;
+    if (k_end > k) k_end = k;
+
+    acc_t acc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int r = 0; r < M::NACC; r++) acc[j][r] = 0.0f;
+
+    // Addresses are a base every lane shares (the chunk's first k; the compiler keeps it in scalar registers) plus a 32-bit
+    // offset of the lane. NN: the lane's columns n0 + 4 MT s + 4c .. + 3 (s < SETS) at k + KL g; NT: its rows of B
+    // n0 + MT j + c at k + KL g
+    const unsigned b_lane = TB ? (unsigned) (c * ldb + KL * g) : (unsigned) (KL * g * ldb + 4 * c);
+    const unsigned a_lane = (unsigned) (c * lda + KL * g);
+    const skinny_f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+
+    auto load_b = [&](long kb, skinny_f32x4 (&bv)[NLOAD]) {
+        const long kl = kb + KL * g;   // the lane's k of this chunk
+        const bool whole = kb + CH <= k_end;
+        if (TB) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const bool ok = n0 + MT * j + c < n;
+                const float* base = B + (n0 + MT * j) * ldb + kb;
+#pragma unroll
+                for (int q = 0; q < KL / 4; q++)
+                    bv[j * (KL / 4) + q] = ok && (whole || kl + 4 * q < k_end) ? *reinterpret_cast<const skinny_f32x4*>(base + b_lane + 4 * q) : zero4;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < KL; i++)
+#pragma unroll
+                for (int s = 0; s < SETS; s++) {
+                    const bool ok = n0 + 4 * MT * s + 4 * c < n;
+                    const float* base = B + (kb + i) * ldb + n0 + 4 * MT * s;
+                    bv[i * SETS + s] =
+                        ok && (whole || kl + i < k_end) ? __builtin_nontemporal_load(reinterpret_cast<const skinny_f32x4*>(base + b_lane)) : zero4;
+                }
+        }
+    };
+    auto load_a = [&](long kb, skinny_f32x4 (&av)[KL / 4]) {
+        const long kl = kb + KL * g;
+        const bool whole = kb + CH <= k_end;
+        const float* base = A + kb;
+#pragma unroll
+        for (int q = 0; q < KL / 4; q++)
+            av[q] = c < m && (whole || kl + 4 * q < k_end) ? *reinterpret_cast<const skinny_f32x4*>(base + a_lane + 4 * q) : zero4;
+    };
+    auto products = [&](const skinny_f32x4 (&av)[KL / 4], const skinny_f32x4 (&bv)[NLOAD]) {
+#pragma unroll
+        for (int i = 0; i < KL; i++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const float a = av[i / 4][i % 4];
+                const float b = TB ? bv[j * (KL / 4) + i / 4][i % 4] : bv[i * SETS + j / 4][j % 4];
+                acc[j] = M::mfma(a, b, acc[j]);
+            }
+    };
+
+    {
+        skinny_f32x4 bq[NBUF][NLOAD], aq[NBUF][KL / 4];
+#pragma unroll
+        for (int u = 0; u < NBUF - 1; u++) {
+            load_b(k_begin + u * CH, bq[u]);   // past k_end: zeros, no access
+            load_a(k_begin + u * CH, aq[u]);
+        }
+        // NBUF chunks a turn, so that the sets of operand registers rotate by name
+        for (long kb = k_begin; kb < k_end; kb += NBUF * CH) {
+#pragma unroll
+            for (int u = 0; u < NBUF; u++) {
+                const long kc = kb + u * CH;
+                if (kc < k_end) {
+                    load_b(kc + (NBUF - 1) * CH, bq[(u + NBUF - 1) % NBUF]);
+                    load_a(kc + (NBUF - 1) * CH, aq[(u + NBUF - 1) % NBUF]);
+                    products(aq[u], bq[u]);
+                }
+            }
+        }
+    }
+
+    // The wavefronts' blocks meet in LDS, NW/2 places of SLOT words. Word (j / 4, r) of a lane holds register r of its blocks
+    // 4 (j / 4) .. + 3: for NN the four columns of one 128-bit store.
+#pragma unroll
+    for (int half = NW / 2; half >= 1; half /= 2) {
+        if (wave >= half && wave < 2 * half) {
+            skinny_f32x4* slot = lds + (long) (wave - half) * SLOT;
+#pragma unroll
+            for (int s = 0; s < NJ / 4; s++)
+#pragma unroll
+                for (int r = 0; r < M::NACC; r++) {
+                    skinny_f32x4 v = {acc[4 * s][r], acc[4 * s + 1][r], acc[4 * s + 2][r], acc[4 * s + 3][r]};
+                    slot[(s * M::NACC + r) * 64 + lane] = v;
+                }
+        }
+        __syncthreads();
+        if (wave < half) {
+            const skinny_f32x4* slot = lds + (long) wave * SLOT;
+#pragma unroll
+            for (int s = 0; s < NJ / 4; s++)
+#pragma unroll
+                for (int r = 0; r < M::NACC; r++) {
+                    const skinny_f32x4 v = slot[(s * M::NACC + r) * 64 + lane];
+                    acc[4 * s][r] += v[0];
+                    acc[4 * s + 1][r] += v[1];
+                    acc[4 * s + 2][r] += v[2];
+                    acc[4 * s + 3][r] += v[3];
+                }
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+    float* out = direct ? P : P + part * m * ldp;
+#pragma unroll
+    for (int r = 0; r < M::NACC; r++) {
+        const long row = M::row(g, r);
+        if (row >= m) continue;
+        if (TB) {
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const long col = n0 + MT * j + c;
+                if (col >= n) continue;
+                float* o = out + row * ldp + col;
+                const float v = acc[j][r];
+                *o = direct ? (beta == 0.0f ? alpha * v : alpha * v + beta * *o) : v;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < SETS; s++) {
+                const long col = n0 + 4 * MT * s + 4 * c;
+                if (col >= n) continue;
+                skinny_f32x4* o = reinterpret_cast<skinny_f32x4*>(out + row * ldp + col);
+                skinny_f32x4 v = {acc[4 * s][r], acc[4 * s + 1][r], acc[4 * s + 2][r], acc[4 * s + 3][r]};
+                if (direct) {
+                    if (beta == 0.0f) {
+                        v = alpha * v;
+                    } else {
+                        const skinny_f32x4 old = *o;
+                        v = alpha * v + beta * old;
+                    }
+                }
+                *o = v;
+            }
+        }
+    }
+}
+
+}  // namespace docc_k
+
+#define DOCC_GEMM_SKINNY(MT, TB, TBN, NW, CH, NBUF)                                                                                             \
+    extern "C" __global__ __launch_bounds__(64 * NW) void docc_sgemm_skinny##MT##_n##TBN##_w##NW##_c##CH##_b##NBUF(                             \
+        const float* A, long lda, const float* B, long ldb, float* P, long ldp, long m, long n, long k, long kpart, float alpha, float beta,      \
+        int direct) {                                                                                                                            \
+        docc_k::gemm_skinny<MT, TB, NW, CH, NBUF>(A, lda, B, ldb, P, ldp, m, n, k, kpart, alpha, beta, direct);                                  \
+    }
+
+// B stored [k][n]: 16 k per chunk, one spare set of operands (more sets cost wavefronts per SIMD and ran slower). B stored [n][k]:
+// 32 k per chunk, so that a row's 128-byte line is used up within the chunk; up to 16 rows of A.
+DOCC_GEMM_SKINNY(16, false, n, 4, 16, 2)
+DOCC_GEMM_SKINNY(32, false, n, 4, 16, 2)
+DOCC_GEMM_SKINNY(16, true, t, 4, 32, 2)

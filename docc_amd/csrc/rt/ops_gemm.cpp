@@ -242,7 +242,13 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         const int rc2 = docc_rocm_free_async(bt, stream);
         return rc ? rc : rc2;
     }
-    if ((m <= 8 || n <= 8) && batch == 1 && (!epilogue || ldc == n)) {
+    // Five to 32 rows of fp32 against a wide matrix go to the kernels of csrc/kernels/gemm_skinny.hip (below); measured against
+    // the tiles with K in parts and the matrix-vector forms, they pay from 8 M elements of B (16 M above 16 rows); DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests)
+    const char* skinny_env = std::getenv("DOCC_ROCM_GEMM_SKINNY");
+    const bool skinny = sizeof(T) == 4 && batch == 1 && !ta && m >= 5 && m <= (tb ? 16 : 32) && !epilogue && n >= 512 && k >= 512 &&
+                        (n * k >= (m <= 16 ? int64_t(8) << 20 : int64_t(16) << 20) || (skinny_env && skinny_env[0] == '1')) && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0 &&
+                        lda % 4 == 0 && ldb % 4 == 0 && k % 4 == 0 && (tb || n % 4 == 0) && !(skinny_env && skinny_env[0] == '0');
+    if ((m <= 8 || n <= 8) && !skinny && batch == 1 && (!epilogue || ldc == n)) {
         rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
         if (rc == 0 && epilogue) {
             // the few rows or columns of output are a small tensor: bias and activation as one elementwise pass over it,
@@ -261,6 +267,67 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     const bool aligned = ((uintptr_t) A % 16 == 0) && ((uintptr_t) B % 16 == 0) && (lda % vec == 0) && (ldb % vec == 0) &&
                          (a_contig % (int64_t) vec == 0) && (b_contig % (int64_t) vec == 0) &&
                          (batch == 1 || (batch_a % (int64_t) vec == 0 && batch_b % (int64_t) vec == 0));
+    // A few rows against a wide fp32 matrix: B goes from global memory straight into the MFMA operands, 128 columns of one part
+    // of K per work-group, the parts added in order by a second launch. With B stored [n][k] the lanes of a load walk different
+    // rows, which pays up to 16 rows only. DOCC_ROCM_GEMM_SKINNY=0 switches it off, DOCC_ROCM_GEMM_SPLITK forces the number of
+    // parts (tests, tuning).
+    if (skinny) {
+        {
+            int cus = compute_units();
+            if (cus <= 0) cus = 256;
+            const int nw = 4, nbuf = 2, ch = tb ? 32 : 16, mt = m <= 16 ? 16 : 32;
+            const int64_t col_blocks = (n + 127) / 128;
+            const int64_t unit = (int64_t) nw * ch;
+            auto part_length = [&](int64_t parts) { return ((k + parts - 1) / parts + unit - 1) / unit * unit; };
+            // The number of parts: measured on 4096 x 4096, 8192 x 8192, 11008 x 4096 and 4096 x 11008, what counts is that
+            // the work-groups come out as whole rounds over the CUs (8192 x 8192: 4, 8 and 12 parts 48-51 us, 6 parts 56 us),
+            // then few parts (their products are written and read again) and 128 and more k per wavefront.
+            int64_t parts = 1;
+            double best = -1.0;
+            for (int64_t p = 1; p <= 64 && part_length(p) >= nw * 64 && p * 16 * m <= k; p++) {
+                const int64_t kp = part_length(p);
+                if ((k + kp - 1) / kp != p) continue;   // rounding to whole chunks made it fewer parts
+                const double per_cu = (double) (col_blocks * p) / cus;
+                const double score = per_cu / (double) (int64_t) (per_cu + 0.999999) - 0.01 * (double) p - (kp < nw * 128 ? 0.15 : 0.0);
+                if (score > best) {
+                    best = score;
+                    parts = p;
+                }
+            }
+            if (const char* e = std::getenv("DOCC_ROCM_GEMM_SPLITK"))
+                if (std::atoll(e) > 0 && part_length(std::atoll(e)) >= unit) parts = std::atoll(e);
+            const int64_t kpart = part_length(parts);
+            parts = (k + kpart - 1) / kpart;
+            const int64_t bytes = parts * m * n * (int64_t) sizeof(S);
+            const bool direct = parts == 1 && (tb || ((uintptr_t) C % 16 == 0 && ldc % 4 == 0));
+            if (direct || bytes <= (int64_t(64) << 20)) {
+                PartialsLease lease;
+                void* buf = nullptr;
+                const bool own_block = !direct && bytes > (int64_t) kPartialsBytes;
+                if (own_block) {
+                    if ((rc = docc_rocm_malloc_async(&buf, (size_t) bytes, stream))) return rc;
+                } else if (!direct) {
+                    if ((rc = partials_for(s, &lease))) return rc;
+                    buf = lease.ptr;
+                }
+                std::snprintf(name, sizeof(name), "docc_sgemm_skinny%d_n%c_w%d_c%d_b%d", mt, tb ? 't' : 'n', nw, ch, nbuf);
+                rc = launch(name, (uint32_t) col_blocks, (uint32_t) parts, 1, 64 * nw, (uint32_t) (nw / 2) * (mt == 32 ? 16384 : 8192), s, A, (long) lda, B, (long) ldb,
+                            direct ? (void*) C : buf, (long) (direct ? ldc : n), (long) m, (long) n, (long) k, (long) kpart, (float) alpha, (float) beta,
+                            direct ? 1 : 0);
+                if (!rc && !direct) {
+                    int64_t blocks = (m * n + 255) / 256;
+                    if (blocks > 4096) blocks = 4096;
+                    rc = launch("docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s, (const S*) buf, C, (long) m, (long) n, (long) ldc,
+                                (int) parts, alpha, beta);
+                }
+                if (own_block) {
+                    const int rc2 = docc_rocm_free_async(buf, stream);
+                    if (!rc) rc = rc2;
+                }
+                return rc;
+            }
+        }
+    }
     // DOCC_ROCM_GEMM_TILE=big|small overrides the size heuristic (tests, tuning)
     const char* force = std::getenv("DOCC_ROCM_GEMM_TILE");
     TileConfig cfg = pick(m, n, batch, aligned, force && force[0] == 'b' ? 1 : force && force[0] == 's' ? -1 : 0);

@@ -47,6 +47,7 @@ const char* const kKernelImages[] = {
     "docc_rocm_reduce.hsaco",
     "docc_rocm_transpose.hsaco",
     "docc_rocm_gemv.hsaco",
+    "docc_rocm_gemm_skinny.hsaco",
 };
 
 struct DeviceState {
