@@ -203,6 +203,131 @@ __device__ __forceinline__ void gemm_skinny(const float* __restrict__ A, long ld
     }
 }
 
+// bf16 operands, B stored [n][k] (the layout of a layer's weights), fp32 sums and result: v_mfma_f32_16x16x32_bf16 takes eight
+// consecutive k of a row of B per lane - exactly a 128-bit load from that row, so B goes from global memory into the
+// instruction as it is. A work-group owns 64 columns of one part of K; K advances in chunks of 64 (two loads per lane and
+// group of 16 columns: a row's 128-byte line is used up within the chunk). RT blocks of 16 rows of A share the loads of B; the
+// matrix pipe is idle most of the time (a kilobyte of B per 16 cycles), the product is bound by reading B. Four blocks of rows
+// (230 registers) ran slower than the tiles.
+template <int RT, int NW, int NBUF>
+__device__ __forceinline__ void gemm_skinny_bf16_nt(const uint16_t* __restrict__ A, long lda, const uint16_t* __restrict__ B, long ldb,
+                                                    float* __restrict__ P, long ldp, long m, long n, long k, long kpart, float alpha, float beta,
+                                                    int direct) {
+    constexpr int CH = 64, NJ = 4;
+    constexpr int SLOT = RT * NJ * 64;   // 128-bit words of a wavefront's block of sums
+    extern __shared__ __attribute__((aligned(16))) unsigned char skinny_lds[];
+    f32x4* lds = reinterpret_cast<f32x4*>(skinny_lds);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const long n0 = (long) blockIdx.x * (16 * NJ);
+    const long part = blockIdx.y;
+    const long kw = kpart / NW;   // a multiple of CH
+    const long k_begin = part * kpart + wave * kw;
+    long k_end = k_begin + kw;
+    if (k_end > k) k_end = k;
+
+    f32x4 acc[RT][NJ];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int j = 0; j < NJ; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[rt][j][r] = 0.0f;
+
+    const unsigned b_lane = (unsigned) (c * ldb + 8 * g), a_lane = (unsigned) (c * lda + 8 * g);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    // half h of a chunk: the lane's k are kb + 32 h + 8 g .. + 7
+    auto load_b = [&](long kb, bf16x8 (&bv)[2 * NJ]) {
+        const bool whole = kb + CH <= k_end;
+#pragma unroll
+        for (int j = 0; j < NJ; j++) {
+            const bool ok = n0 + 16 * j + c < n;
+            const uint16_t* base = B + (n0 + 16 * j) * ldb + kb;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                bv[2 * j + h] = ok && (whole || kb + 32 * h + 8 * g < k_end) ? *reinterpret_cast<const bf16x8*>(base + b_lane + 32 * h) : zero8;
+        }
+    };
+    auto load_a = [&](long kb, bf16x8 (&av)[2 * RT]) {
+        const bool whole = kb + CH <= k_end;
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            const uint16_t* base = A + (long) (16 * rt) * lda + kb;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                av[2 * rt + h] = 16 * rt + c < m && (whole || kb + 32 * h + 8 * g < k_end) ? *reinterpret_cast<const bf16x8*>(base + a_lane + 32 * h) : zero8;
+        }
+    };
+    auto products = [&](const bf16x8 (&av)[2 * RT], const bf16x8 (&bv)[2 * NJ]) {
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) acc[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * rt + h], bv[2 * j + h], acc[rt][j], 0, 0, 0);
+    };
+
+    {
+        bf16x8 bq[NBUF][2 * NJ], aq[NBUF][2 * RT];
+#pragma unroll
+        for (int u = 0; u < NBUF - 1; u++) {
+            load_b(k_begin + u * CH, bq[u]);   // past k_end: zeros, no access
+            load_a(k_begin + u * CH, aq[u]);
+        }
+        for (long kb = k_begin; kb < k_end; kb += NBUF * CH) {
+#pragma unroll
+            for (int u = 0; u < NBUF; u++) {
+                const long kc = kb + u * CH;
+                if (kc < k_end) {
+                    load_b(kc + (NBUF - 1) * CH, bq[(u + NBUF - 1) % NBUF]);
+                    load_a(kc + (NBUF - 1) * CH, aq[(u + NBUF - 1) % NBUF]);
+                    products(aq[u], bq[u]);
+                }
+            }
+        }
+    }
+
+    // the wavefronts' blocks meet in LDS as above; a word is one block's four registers of a lane
+#pragma unroll
+    for (int half = NW / 2; half >= 1; half /= 2) {
+        if (wave >= half && wave < 2 * half) {
+            f32x4* slot = lds + (long) (wave - half) * SLOT;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++) slot[(rt * NJ + j) * 64 + lane] = acc[rt][j];
+        }
+        __syncthreads();
+        if (wave < half) {
+            const f32x4* slot = lds + (long) wave * SLOT;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+                for (int j = 0; j < NJ; j++) acc[rt][j] += slot[(rt * NJ + j) * 64 + lane];
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+    float* out = direct ? P : P + part * m * ldp;
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            // register r of a 16 x 16 block of sums: row 4 (lane / 16) + r, column lane % 16
+            const long row = 16 * rt + 4 * g + r;
+            if (row >= m) continue;
+#pragma unroll
+            for (int j = 0; j < NJ; j++) {
+                const long col = n0 + 16 * j + c;
+                if (col >= n) continue;
+                float* o = out + row * ldp + col;
+                const float v = acc[rt][j][r];
+                *o = direct ? (beta == 0.0f ? alpha * v : alpha * v + beta * *o) : v;
+            }
+        }
+}
+
 }  // namespace docc_k
 
 #define DOCC_GEMM_SKINNY(MT, TB, TBN, NW, CH, NBUF)                                                                                             \
@@ -217,3 +342,13 @@ __device__ __forceinline__ void gemm_skinny(const float* __restrict__ A, long ld
 DOCC_GEMM_SKINNY(16, false, n, 4, 16, 2)
 DOCC_GEMM_SKINNY(32, false, n, 4, 16, 2)
 DOCC_GEMM_SKINNY(16, true, t, 4, 32, 2)
+
+#define DOCC_GEMM_SKINNY_BF16(RT, NW, NBUF)                                                                                                     \
+    extern "C" __global__ __launch_bounds__(64 * NW) void docc_bgemm_skinny##RT##_nt_w##NW##_b##NBUF(                                           \
+        const uint16_t* A, long lda, const uint16_t* B, long ldb, float* P, long ldp, long m, long n, long k, long kpart, float alpha,           \
+        float beta, int direct) {                                                                                                                \
+        docc_k::gemm_skinny_bf16_nt<RT, NW, NBUF>(A, lda, B, ldb, P, ldp, m, n, k, kpart, alpha, beta, direct);                                  \
+    }
+
+DOCC_GEMM_SKINNY_BF16(1, 4, 2)
+DOCC_GEMM_SKINNY_BF16(2, 4, 2)

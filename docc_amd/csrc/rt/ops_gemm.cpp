@@ -245,9 +245,15 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // Five to 32 rows of fp32 against a wide matrix go to the kernels of csrc/kernels/gemm_skinny.hip (below); measured against
     // the tiles with K in parts and the matrix-vector forms, they pay from 8 M elements of B (16 M above 16 rows); DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests)
     const char* skinny_env = std::getenv("DOCC_ROCM_GEMM_SKINNY");
-    const bool skinny = sizeof(T) == 4 && batch == 1 && !ta && m >= 5 && m <= (tb ? 16 : 32) && !epilogue && n >= 512 && k >= 512 &&
-                        (n * k >= (m <= 16 ? int64_t(8) << 20 : int64_t(16) << 20) || (skinny_env && skinny_env[0] == '1')) && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0 &&
-                        lda % 4 == 0 && ldb % 4 == 0 && k % 4 == 0 && (tb || n % 4 == 0) && !(skinny_env && skinny_env[0] == '0');
+    const bool skinny_on = !(skinny_env && skinny_env[0] == '0'), skinny_any_size = skinny_env && skinny_env[0] == '1';
+    const bool skinny_base = batch == 1 && !ta && !epilogue && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0;
+    const bool skinny_f32 = sizeof(T) == 4 && skinny_base && m >= 5 && m <= (tb ? 16 : 32) &&
+                            (n * k >= (m <= 16 ? int64_t(8) << 20 : int64_t(16) << 20) || skinny_any_size) && lda % 4 == 0 && ldb % 4 == 0 &&
+                            k % 4 == 0 && (tb || n % 4 == 0);
+    // bf16 with B stored [n][k] (a layer's weights): 3 to 32 rows (two rows are faster as matrix-vector products, 64 on the tiles)
+    const bool skinny_bf16 = sizeof(T) == 2 && skinny_base && tb && m >= 3 && m <= 32 && (n * k >= (int64_t(8) << 20) || skinny_any_size) &&
+                             lda % 8 == 0 && ldb % 8 == 0 && k % 8 == 0;
+    const bool skinny = skinny_f32 || skinny_bf16;
     if ((m <= 8 || n <= 8) && !skinny && batch == 1 && (!epilogue || ldc == n)) {
         rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
         if (rc == 0 && epilogue) {
@@ -275,8 +281,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         {
             int cus = compute_units();
             if (cus <= 0) cus = 256;
-            const int nw = 4, nbuf = 2, ch = tb ? 32 : 16, mt = m <= 16 ? 16 : 32;
-            const int64_t col_blocks = (n + 127) / 128;
+            // fp32: 16 or 32 rows per MFMA, 128 columns per work-group; bf16: 1, 2 or 4 blocks of 16 rows, 64 columns
+            const int nw = 4, nbuf = 2;
+            const int ch = skinny_bf16 ? 64 : tb ? 32 : 16, mt = skinny_bf16 ? (m <= 16 ? 1 : 2) : m <= 16 ? 16 : 32;
+            const int64_t col_blocks = skinny_bf16 ? (n + 63) / 64 : (n + 127) / 128;
             const int64_t unit = (int64_t) nw * ch;
             auto part_length = [&](int64_t parts) { return ((k + parts - 1) / parts + unit - 1) / unit * unit; };
             // The number of parts: measured on 4096 x 4096, 8192 x 8192, 11008 x 4096 and 4096 x 11008, what counts is that
@@ -287,6 +295,9 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
             for (int64_t p = 1; p <= 64 && part_length(p) >= nw * 64 && p * 16 * m <= k; p++) {
                 const int64_t kp = part_length(p);
                 if ((k + kp - 1) / kp != p) continue;   // rounding to whole chunks made it fewer parts
+                // B stored [n][k]: a lane walks its row of B, and parts longer than 4096 ran a quarter slower (bf16 16384 x 16384
+                // in 1 or 2 parts 127 us, in 4 parts 97)
+                if (tb && kp > 4096 && part_length(p + 1) >= nw * 64) continue;
                 const double per_cu = (double) (col_blocks * p) / cus;
                 const double score = per_cu / (double) (int64_t) (per_cu + 0.999999) - 0.01 * (double) p - (kp < nw * 128 ? 0.15 : 0.0);
                 if (score > best) {
@@ -310,8 +321,12 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                     if ((rc = partials_for(s, &lease))) return rc;
                     buf = lease.ptr;
                 }
-                std::snprintf(name, sizeof(name), "docc_sgemm_skinny%d_n%c_w%d_c%d_b%d", mt, tb ? 't' : 'n', nw, ch, nbuf);
-                rc = launch(name, (uint32_t) col_blocks, (uint32_t) parts, 1, 64 * nw, (uint32_t) (nw / 2) * (mt == 32 ? 16384 : 8192), s, A, (long) lda, B, (long) ldb,
+                if (skinny_bf16)
+                    std::snprintf(name, sizeof(name), "docc_bgemm_skinny%d_nt_w%d_b%d", mt, nw, nbuf);
+                else
+                    std::snprintf(name, sizeof(name), "docc_sgemm_skinny%d_n%c_w%d_c%d_b%d", mt, tb ? 't' : 'n', nw, ch, nbuf);
+                const uint32_t slot_bytes = skinny_bf16 ? 4096u * mt : mt == 32 ? 16384u : 8192u;   // a wavefront's block of sums
+                rc = launch(name, (uint32_t) col_blocks, (uint32_t) parts, 1, 64 * nw, (uint32_t) (nw / 2) * slot_bytes, s, A, (long) lda, B, (long) ldb,
                             direct ? (void*) C : buf, (long) (direct ? ldc : n), (long) m, (long) n, (long) k, (long) kpart, (float) alpha, (float) beta,
                             direct ? 1 : 0);
                 if (!rc && !direct) {

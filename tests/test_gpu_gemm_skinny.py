@@ -1,6 +1,6 @@
 """Five to 32 rows of fp32 against a wide matrix: the kernels that feed B from global memory straight into the MFMA (16 rows per
-instruction up to m = 16, 32 above; B stored [k][n], and [n][k] up to 16 rows). Through the C-ABI against the oracle, bit for bit
-on integer-valued operands (every product and partial sum is exact, so neither the cut of K into parts nor the order of the
+instruction up to m = 16, 32 above; B stored [k][n], and [n][k] up to 16 rows), and 3 to 32 rows of bf16 against a matrix stored
+[n][k]. Through the C-ABI against the oracle, bit for bit on integer-valued operands (every product and partial sum is exact, so neither the cut of K into parts nor the order of the
 wavefronts' sums changes anything), at the fp32 bar against a float64 product otherwise."""
 import numpy as np
 import pytest
@@ -9,6 +9,7 @@ import torch
 import oracle
 from gpu_util import dev, host, rel_err_max
 from test_gpu_gemm import int_matrix, run_gemm
+from test_gpu_gemm_bf16 import run_bgemm
 
 pytestmark = pytest.mark.gpu
 
@@ -117,3 +118,48 @@ def test_skinny_on_two_streams(rt):
         assert np.array_equal(host(c[i]), oracle.gemm(A[i], B[i]))
     for st in streams:
         rt.stream_destroy(st)
+
+
+BF16_SHAPES = [(16, 1024, 1024), (9, 1000, 2056), (3, 520, 512), (32, 2048, 1032), (17, 640, 4104), (12, 4096, 4096), (31, 1288, 8192)]
+
+
+@pytest.mark.parametrize("m,n,k", BF16_SHAPES)
+def test_skinny_bf16_integer_exact(rt, m, n, k):
+    rng = np.random.default_rng(m + 3 * n + 5 * k)
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (n, k)).astype(np.float32)
+    Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+    C0 = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    C = run_bgemm(rt, Ab, Bb, C=C0.copy(), alpha=0.5, beta=2.0, tb=T)
+    assert np.array_equal(C, oracle.gemm_bf16(Ab, Bb, C=C0.copy(), alpha=0.5, beta=2.0, trans_b=T))
+    # beta == 0 must not read C (run_bgemm fills it with NaN)
+    assert np.array_equal(run_bgemm(rt, Ab, Bb, tb=T), A @ B.T)
+
+
+@pytest.mark.parametrize("parts", ["1", "3", "8", "64"])
+@pytest.mark.parametrize("m", [4, 16, 29])
+def test_skinny_bf16_any_number_of_parts(rt, monkeypatch, parts, m):
+    monkeypatch.setenv("DOCC_ROCM_GEMM_SPLITK", parts)
+    n, k = 1160, 3072
+    rng = np.random.default_rng(m + int(parts))
+    A = rng.integers(-4, 5, (m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, (n, k)).astype(np.float32)
+    Ab, Bb = oracle.f32_to_bf16(A), oracle.f32_to_bf16(B)
+    C0 = rng.integers(-8, 9, (m, n)).astype(np.float32)
+    assert np.array_equal(run_bgemm(rt, Ab, Bb, C=C0.copy(), alpha=-1.0, beta=2.0, tb=T), -(A @ B.T) + 2.0 * C0)
+    assert np.array_equal(run_bgemm(rt, Ab, Bb, tb=T), A @ B.T)
+
+
+@pytest.mark.parametrize("m,n,k", [(16, 4096, 4096), (32, 1024, 8192), (5, 11008, 2048)])
+def test_skinny_bf16_random_operands(rt, monkeypatch, m, n, k):
+    """bf16 products are exact in fp32; the sums differ from the oracle's by their order only."""
+    rng = np.random.default_rng(n + k)
+    Ab = oracle.f32_to_bf16(rng.standard_normal((m, k)).astype(np.float32))
+    Bb = oracle.f32_to_bf16(rng.standard_normal((n, k)).astype(np.float32))
+    ref = oracle.bf16_to_f32(Ab).astype(np.float64) @ oracle.bf16_to_f32(Bb).astype(np.float64).T
+    got = run_bgemm(rt, Ab, Bb, tb=T)
+    assert rel_err_max(got, ref) <= 1e-5
+    for _ in range(2):
+        assert np.array_equal(run_bgemm(rt, Ab, Bb, tb=T), got)     # parts are added in order
+    monkeypatch.setenv("DOCC_ROCM_GEMM_SKINNY", "0")
+    assert rel_err_max(run_bgemm(rt, Ab, Bb, tb=T), got.astype(np.float64)) <= 2e-5
