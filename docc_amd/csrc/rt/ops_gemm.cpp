@@ -246,7 +246,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // the tiles with K in parts and the matrix-vector forms, they pay from 8 M elements of B (16 M above 16 rows); DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests)
     const char* skinny_env = std::getenv("DOCC_ROCM_GEMM_SKINNY");
     const bool skinny_on = !(skinny_env && skinny_env[0] == '0'), skinny_any_size = skinny_env && skinny_env[0] == '1';
-    const bool skinny_base = batch == 1 && !ta && !epilogue && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0;
+    const bool skinny_base = batch == 1 && !ta && (!epilogue || ldc == n) && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0;
     const bool skinny_f32 = sizeof(T) == 4 && skinny_base && m >= 5 && m <= (tb ? 16 : 32) &&
                             (n * k >= (m <= 16 ? int64_t(8) << 20 : int64_t(16) << 20) || skinny_any_size) && lda % 4 == 0 && ldb % 4 == 0 &&
                             k % 4 == 0 && (tb || n % 4 == 0);
@@ -339,7 +339,13 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                     const int rc2 = docc_rocm_free_async(buf, stream);
                     if (!rc) rc = rc2;
                 }
-                return rc;
+                if (rc || !epilogue) return rc;
+                // the few rows of output are a small tensor: bias and activation as one elementwise pass over it, the same
+                // roundings as the fused store
+                const int64_t shape[2] = {m, n}, row[2] = {1, n};
+                const int post[1] = {activation};
+                return docc_rocm_elementwise_fused(stream, 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0, bias ? row : nullptr, bias, 0.0,
+                                                   activation >= 0 ? 1 : 0, post, C);
             }
         }
     }
@@ -368,7 +374,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // one entry of a batched launch into the stream's buffer of partial results, and a second launch adds the parts
     // (in order: the result does not depend on the device's scheduling). DOCC_ROCM_GEMM_SPLITK=0 switches it off,
     // another number forces that many parts where K allows it (tests, tuning).
-    if (batch == 1 && !epilogue && aligned && k >= 1024) {
+    if (batch == 1 && (!epilogue || ldc == n) && aligned && k >= 1024) {
         int cus = compute_units();
         if (cus <= 0) cus = 256;
         const char* env = std::getenv("DOCC_ROCM_GEMM_SPLITK");
@@ -431,7 +437,12 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                 const int rc2 = docc_rocm_free_async(parts, stream);
                 if (!rc) rc = rc2;
             }
-            return rc;
+            if (rc || !epilogue) return rc;
+            // bias and activation as one elementwise pass over the output, the same roundings as the fused store
+            const int64_t shape[2] = {m, n}, row[2] = {1, n};
+            const int post[1] = {activation};
+            return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
+                                               bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
         }
     }
     size_t lds;

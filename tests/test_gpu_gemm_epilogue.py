@@ -18,7 +18,9 @@ N, T = oracle.NO_TRANS, oracle.TRANS
 SHAPES = [(64, 64, 64, N, N), (100, 130, 70, N, T), (257, 129, 100, T, N), (33, 17, 5, T, T), (512, 384, 256, N, N),
           (1024, 1024, 128, N, T), (1, 300, 7, N, N), (40, 50, 0, N, N),
           # a small batch through a layer: the matrix-vector kernels, bias and activation as a pass over the few output rows
-          (4, 5000, 704, N, T), (3000, 1, 700, N, N), (4, 4200, 333, N, N), (1, 4096, 512, N, T)]
+          (4, 5000, 704, N, T), (3000, 1, 700, N, N), (4, 4200, 333, N, N), (1, 4096, 512, N, T),
+          # a dozen rows against a matrix of 8 M elements: the kernels that feed B straight into the MFMA, then the same pass
+          (12, 4096, 2048, N, N), (12, 4096, 2048, N, T)]
 ACTS = [None, "relu", "abs"]          # the activations built into the store
 
 
