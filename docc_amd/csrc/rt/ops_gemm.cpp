@@ -243,11 +243,16 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
         return rc ? rc : rc2;
     }
     // Five to 32 rows of fp32 against a wide matrix go to the kernels of csrc/kernels/gemm_skinny.hip (below); measured against
-    // the tiles with K in parts and the matrix-vector forms, they pay from 8 M elements of B (16 M above 16 rows); DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests)
+    // the tiles with K in parts and the matrix-vector forms, they pay from 8 M elements of B (16 M above 16 rows).
+    // DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests).
     const char* skinny_env = std::getenv("DOCC_ROCM_GEMM_SKINNY");
     const bool skinny_on = !(skinny_env && skinny_env[0] == '0'), skinny_any_size = skinny_env && skinny_env[0] == '1';
-    const bool skinny_base = batch == 1 && !ta && (!epilogue || ldc == n) && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 && (uintptr_t) B % 16 == 0;
-    const bool skinny_f32 = sizeof(T) == 4 && skinny_base && m >= 5 && m <= (tb ? 16 : 32) &&
+    const bool skinny_base = batch == 1 && !ta && (!epilogue || ldc == n) && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 &&
+                             (uintptr_t) B % 16 == 0;
+    // (B stored [n][k]: from 3 rows, where the matrix-vector form for several vectors falls behind - 4 x 8192 x 8192 67 -> 57 us,
+    // 4 x 4096 x 11008 62 -> 48 - but up to 8 rows not above 128 M elements, where that form is the faster one again)
+    const bool skinny_f32 = sizeof(T) == 4 && skinny_base && m >= (skinny_any_size ? 2 : tb ? 3 : 5) && m <= (tb ? 16 : 32) &&
+                            !(tb && m <= 8 && n * k > (int64_t(1) << 27)) &&
                             (n * k >= (m <= 16 ? int64_t(8) << 20 : int64_t(16) << 20) || skinny_any_size) && lda % 4 == 0 && ldb % 4 == 0 &&
                             k % 4 == 0 && (tb || n % 4 == 0);
     // bf16 with B stored [n][k] (a layer's weights): 3 to 32 rows (two rows are faster as matrix-vector products, 64 on the tiles)
