@@ -396,9 +396,12 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
             const double tm = (double) ((m + c.bm - 1) / c.bm), tn = (double) ((n + c.bn - 1) / c.bn);
             const double area = (double) c.bm * c.bn;
             const double rel = area >= 65536 ? 1.03 : area >= 32768 ? 1.0 : area >= 16384 ? 0.97 : 0.75;
-            const double fill = tm * tn * (double) parts / cus;
+            // the share of the CUs' time that does work: below one work-group per CU the CUs that get one, above it the
+            // whole rounds (344 work-groups on 256 CUs take as long as 512)
+            const double per_cu = tm * tn * (double) parts / cus;
+            const double fill = per_cu < 1.0 ? per_cu : per_cu / (double) (int64_t) (per_cu + 0.999999);
             const double rate = sizeof(T) == 8 ? 68e12 : sizeof(T) == 4 ? 141e12 : 1.25e15;
-            double t = 2.0 * tm * c.bm * tn * c.bn * (double) k / (rate * rel * (fill < 1.0 ? fill : 1.0));
+            double t = 2.0 * tm * c.bm * tn * c.bn * (double) k / (rate * rel * fill);
             if (parts > 1) t += 2.0 * (double) parts * (double) m * (double) n * sizeof(S) / 5e12 + 3e-6;
             return t;
         };
