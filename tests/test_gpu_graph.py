@@ -23,8 +23,12 @@ def chain(rt, m, n, k, a, b, bias, out, stream=0):
     return tmp
 
 
-def test_replays_give_the_bits_of_the_eager_calls(rt):
-    m, n, k = 384, 512, 256
+# the tiles; sixteen rows against a wide matrix (B straight into the MFMA, the parts' products in the stream's buffer); the same
+# kernels with 16 MiB of parts, which take a block of the block cache inside the record
+@pytest.mark.parametrize("m,n,k,parts,blocks", [(384, 512, 256, None, 1), (16, 4096, 2048, None, 1), (32, 8192, 4096, "16", 2)])
+def test_replays_give_the_bits_of_the_eager_calls(rt, monkeypatch, m, n, k, parts, blocks):
+    if parts:
+        monkeypatch.setenv("DOCC_ROCM_GEMM_SPLITK", parts)
     g = torch.Generator(device="cpu").manual_seed(11)
     a = torch.randn(m, k, generator=g).cuda()
     b = torch.randn(k, n, generator=g).cuda()
@@ -75,7 +79,7 @@ def test_replays_give_the_bits_of_the_eager_calls(rt):
 
     cached_before = rt.pool_stats()[1]
     graph.destroy()
-    assert rt.pool_stats()[1] == cached_before + 1          # the temporary is back in the cache
+    assert rt.pool_stats()[1] == cached_before + blocks     # the temporary (and the block of parts) are back in the cache
     rt.stream_destroy(stream)
 
 
