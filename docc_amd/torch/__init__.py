@@ -16,7 +16,9 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
                                            -> ml::Attention (bf16; head dims 32, 64, 128 fused)
-    + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number
+    + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number; on bf16
+                                              tensors in float32 with one rounding to bf16, as eager torch computes them
+                                              (likewise the unary operations, reductions, softmax, gelu, silu, layer_norm)
                                            -> ml::Add .. ml::Minimum, with ml::Broadcast where shapes differ
     relu, sigmoid, tanh, exp, abs, sqrt, erf (functions, methods, nn.ReLU / nn.Sigmoid / nn.Tanh),
     elu, leaky_relu, hardsigmoid (F.* and nn.ELU / nn.LeakyReLU / nn.Hardsigmoid)
@@ -235,6 +237,8 @@ class _FxLowering:
             self.fail(node, "softmax of this value")
         if not -len(x.shape) <= dim < len(x.shape):
             self.fail(node, "softmax dim out of range")
+        if self.is_bf16(x):
+            return self.narrowed(node, self.softmax(node, self.widened(node, x), dim, None), dest)
         if x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, "softmax on a dtype other than float32 / float64")
         out = self.new_tensor(x.shape, x.dtype, dest)
@@ -273,10 +277,27 @@ class _FxLowering:
         self.builder.add_broadcast(x.name, out.name, [1] * (len(shape) - len(x.shape)) + x.shape, shape)
         return out
 
+    # bf16 tensors outside products: eager torch computes elementwise operations, reductions and softmax on bf16 in float32 and
+    # rounds the result once; here the operands are widened (ml::Cast), the float32 nodes do the work and one ml::Cast rounds.
+    def is_bf16(self, v) -> bool:
+        return isinstance(v, _T) and v.dtype == self.torch.bfloat16
+
+    def widened(self, node, v):
+        return self.tensor(node, _Widened(v, self.torch.float32)) if self.is_bf16(v) else v
+
+    def narrowed(self, node, wide: _T, dest):
+        out = self.new_tensor(wide.shape, self.torch.bfloat16, dest)
+        self.builder.add_cast_op(wide.name, out.name, wide.shape)
+        return out
+
     def elementwise(self, node, op: str, a, b, dest):
         torch = self.torch
         a, b = self.tensor(node, a), self.tensor(node, b)
         tensors = [v for v in (a, b) if isinstance(v, _T)]
+        if any(self.is_bf16(v) for v in tensors) and all(v.dtype in (torch.bfloat16, torch.float32) for v in tensors):
+            narrow = all(self.is_bf16(v) for v in tensors)      # bf16 with float32 promotes to float32
+            wide = self.elementwise(node, op, self.widened(node, a), self.widened(node, b), None if narrow else dest)
+            return self.narrowed(node, wide, dest) if narrow else wide
         if not tensors or not all(isinstance(v, (_T, int, float)) and not isinstance(v, bool) for v in (a, b)):
             self.fail(node, f"elementwise {op} of these operands")
         dtype = tensors[0].dtype
@@ -297,6 +318,8 @@ class _FxLowering:
 
     def unary(self, node, op: str, x, dest, alpha=None, beta=None):
         x = self.tensor(node, x)
+        if self.is_bf16(x):
+            return self.narrowed(node, self.unary(node, op, self.widened(node, x), None, alpha, beta), dest)
         if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
         out = self.new_tensor(x.shape, x.dtype, dest)
@@ -308,6 +331,8 @@ class _FxLowering:
 
     def reduce(self, node, op: str, x, dim, keepdim: bool, dest):
         x = self.tensor(node, x)
+        if self.is_bf16(x):
+            return self.narrowed(node, self.reduce(node, op, self.widened(node, x), dim, keepdim, None), dest)
         if not isinstance(x, _T) or x.dtype not in (self.torch.float32, self.torch.float64):
             self.fail(node, f"{op} of a value that is not a float32 / float64 tensor")
         rank = len(x.shape)
@@ -322,6 +347,9 @@ class _FxLowering:
     # fusion pass of the target makes one generated kernel of each chain.
     def gelu(self, node, x, approximate: str, dest):
         """0.5 x (1 + erf(x / sqrt 2)), or with tanh(sqrt(2 / pi) (x + 0.044715 x^3)) in place of the erf."""
+        x = self.tensor(node, x)
+        if self.is_bf16(x):      # one rounding at the end, like eager torch's kernel
+            return self.narrowed(node, self.gelu(node, self.widened(node, x), approximate, None), dest)
         if approximate == "tanh":
             cube = self.elementwise(node, "mul", self.elementwise(node, "mul", x, x, None), x, None)
             inner = self.elementwise(node, "mul", self.elementwise(node, "add", x, self.elementwise(node, "mul", cube, 0.044715, None), None),
@@ -335,6 +363,9 @@ class _FxLowering:
         return self.elementwise(node, "mul", half, self.elementwise(node, "add", gate, 1.0, None), dest)
 
     def silu(self, node, x, dest):
+        x = self.tensor(node, x)
+        if self.is_bf16(x):
+            return self.narrowed(node, self.silu(node, self.widened(node, x), None), dest)
         return self.elementwise(node, "mul", x, self.unary(node, "sigmoid", x, None), dest)
 
     def layer_norm(self, node, x, normalized_shape, weight, bias, eps: float, dest):
@@ -343,6 +374,10 @@ class _FxLowering:
         x = self.tensor(node, x)
         if not isinstance(x, _T):
             self.fail(node, "layer_norm of this value")
+        if self.is_bf16(x):
+            wide = self.layer_norm(node, self.widened(node, x), normalized_shape, self.widened(node, self.tensor(node, weight)),
+                                   self.widened(node, self.tensor(node, bias)), eps, None)
+            return self.narrowed(node, wide, dest)
         shape = [int(v) for v in ([normalized_shape] if isinstance(normalized_shape, int) else normalized_shape)]
         if not shape or x.shape[-len(shape):] != shape:
             self.fail(node, "layer_norm whose normalized_shape is not the tensor's last axes")

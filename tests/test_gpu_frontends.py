@@ -723,6 +723,62 @@ def test_torch_bf16_products_and_linear_give_bf16_like_eager():
     assert (l.float() - eager.float()).abs().max().item() <= 2.0 ** -7 * eager.float().abs().max().item()      # a last bit of bf16 at most
 
 
+def test_torch_small_batch_through_wide_layers():
+    """Eight rows through nn.Linear layers of 8 M weights, bf16 and fp32 (the weights stored [out, in]): the products take the
+    kernels that feed the weights straight into the MFMA, the bias and the ReLU follow as a pass over the eight rows."""
+    class Net(torch.nn.Module):
+        def __init__(self, dtype):
+            super().__init__()
+            self.up = torch.nn.Linear(2048, 4096).to(dtype)
+            self.down = torch.nn.Linear(4096, 2048, bias=False).to(dtype)
+
+        def forward(self, x):
+            return self.down(torch.relu(self.up(x)))
+
+    for dtype, tol in ((torch.bfloat16, 2e-2), (torch.float32, 1e-5)):
+        torch.manual_seed(12)
+        model = Net(dtype).cuda()
+        x = torch.randn(8, 2048).to(dtype).cuda()
+        program = docc_torch.compile_torch(model, (x,), target="rocm")
+        out = program(x)
+        out = out[0] if isinstance(out, (tuple, list)) else out
+        assert out.dtype == dtype and out.shape == (8, 2048)
+        with torch.no_grad():
+            h = torch.relu(x.double() @ model.up.weight.double().T + model.up.bias.double())
+            if dtype == torch.bfloat16:
+                h = h.bfloat16().double()          # the layer's result is rounded to bf16 before the next one reads it
+            ref = h @ model.down.weight.double().T
+        assert rel_err_max(out.double().cpu().numpy(), ref.cpu().numpy()) <= tol, dtype
+
+
+def test_torch_bf16_elementwise_chain_like_eager():
+    """bf16 tensors outside products: elementwise operations, gelu, layer_norm, softmax and a sum run in float32 and round
+    once to bf16, as eager torch computes them. Against eager on the same device, a few last bits of bf16 over the chain."""
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.up = torch.nn.Linear(64, 128).bfloat16()
+            self.ln = torch.nn.LayerNorm(128).bfloat16()
+
+        def forward(self, x, y):
+            h = torch.nn.functional.gelu(self.up(x))
+            z = self.ln(h) * 0.5 + h
+            return torch.softmax(z, dim=-1), (z * y).sum(dim=0), torch.relu(z) + y.float()
+
+    torch.manual_seed(21)
+    model = Net().cuda()
+    x, y = torch.randn(24, 64).bfloat16().cuda(), torch.randn(24, 128).bfloat16().cuda()
+    program = docc_torch.compile_torch(model, (x, y), target="rocm")
+    got = program(x, y)
+    with torch.no_grad():
+        eager = model(x, y)
+    assert [g.dtype for g in got] == [torch.bfloat16, torch.bfloat16, torch.float32]      # bf16 with float32 promotes
+    for g, e in zip(got, eager):
+        assert g.shape == e.shape
+        scale = e.float().abs().max().item()
+        assert (g.float() - e.float()).abs().max().item() <= 4 * 2.0 ** -8 * scale
+
+
 def test_power_operator_through_both_front_ends():
     """x ** 2, x ** y and np.power lower to ml::Pow (array or scalar operand); torch.pow likewise."""
     @native(target="rocm")
