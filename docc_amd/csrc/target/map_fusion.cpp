@@ -226,9 +226,12 @@ private:
         return f;
     }
 
-    // between the two floating point types only: the conversion is the assignment's
+    // between float, double and bf16 (a bf16 tensor widened for the float32 nodes, their result rounded to bf16: the
+    // compiler's conversions, to nearest even): the conversion is the assignment's
     std::optional<MapForm> from_cast(const Block& blk, const tensor::CastNode& c) {
-        if (!floating(c.element()) || !floating(c.target_type()) || c.shape().empty()) return std::nullopt;
+        auto convertible = [](P t) { return floating(t) || t == P::BFloat; };
+        if (!convertible(c.element()) || !convertible(c.target_type()) || c.shape().empty()) return std::nullopt;
+        if (c.element() == P::BFloat && c.target_type() == P::BFloat) return std::nullopt;
         MapForm f;
         f.element = c.target_type();
         f.bounds = bounds_of(c.shape());

@@ -11,7 +11,10 @@ namespace sdfg::rocm {
 
 namespace {
 
-const char* c_type(types::PrimitiveType t) { return t == types::PrimitiveType::Double ? "double" : "float"; }
+// bf16 tensors are loaded, converted by an assignment (the compiler's conversions: exact to float, to nearest even back) and stored
+const char* c_type(types::PrimitiveType t) {
+    return t == types::PrimitiveType::Double ? "double" : t == types::PrimitiveType::BFloat ? "__bf16" : "float";
+}
 
 bool is_literal_stride(const Expression& s) { return s == "0" || s == "1"; }
 

@@ -967,7 +967,9 @@ void ROCMMapNode::validate() const {
     for (auto* list : {&reads_, &writes_})
         for (auto& a : *list) {
             if (a.strides.size() != indvars_.size()) throw InvalidSDFGException(code_ + ": operand " + a.connector + " needs one stride per induction variable");
-            if (!floating(a.element)) throw InvalidSDFGException(code_ + ": operand " + a.connector + " must be Float or Double");
+            // bf16 tensors are loaded and stored (converted by the assignments next to them), never computed on
+            if (!floating(a.element) && a.element != types::PrimitiveType::BFloat)
+                throw InvalidSDFGException(code_ + ": operand " + a.connector + " must be Float, Double or BFloat");
         }
     for (auto& r : reads_) define(r.connector);
     for (auto& s : scalars_) {
@@ -981,7 +983,8 @@ void ROCMMapNode::validate() const {
         const int n = arity(st.op);
         if (n < 0) throw InvalidSDFGException(code_ + ": unknown operation '" + st.op + "'");
         if ((int) st.args.size() != n) throw InvalidSDFGException(code_ + ": operation " + st.op + " takes " + std::to_string(n) + " arguments");
-        if (!floating(st.type)) throw InvalidSDFGException(code_ + ": statement " + st.out + " must be Float or Double");
+        if (!floating(st.type) && !(st.type == types::PrimitiveType::BFloat && st.op == "assign"))
+            throw InvalidSDFGException(code_ + ": statement " + st.out + " must be Float or Double (BFloat for an assignment)");
         for (auto& a : st.args)
             if (!known(a)) throw InvalidSDFGException(code_ + ": statement " + st.out + " uses '" + a + "' before it is defined");
         define(st.out);

@@ -1038,3 +1038,40 @@ def test_builder_map_nest_generates_a_kernel_and_its_launch(tmp_path):
     bad.add_map_nest([("i", 8)], [("a", "A", ["1"])], [("p", "fp_sqrt", ["a"])], [("A", ["1"], "p")])
     with pytest.raises(InvalidSDFGException, match="unknown operation 'fp_sqrt'"):
         bad.move().validate()
+
+
+def test_bf16_tensors_between_float32_nodes_join_the_generated_kernel(tmp_path):
+    """A bf16 tensor widened to float32, two float32 nodes and the rounding back to bf16 - what the torch front end makes of an
+    elementwise chain on bf16 tensors - become one generated kernel that loads and stores bf16: the conversions are the
+    assignments of the nest, the arithmetic stays in float32. A nest may not compute in bf16."""
+    b = StructuredSDFGBuilder("bf16_chain")
+    b.add_container("x", BF16, True)
+    b.add_container("y", BF16, True)
+    b.add_container("out", BF16, True)
+    for n in ("xw", "yw", "t0", "t1"):
+        b.add_container(n, F32, False, transient_bytes=64 * 48 * 4)
+    b.add_cast_op("x", "xw", [64, 48])
+    b.add_cast_op("y", "yw", [64, 48])
+    b.add_elementwise_op("mul", "xw", "yw", "t0", [64, 48])
+    b.add_elementwise_unary_op("tanh", "t0", "t1", [64, 48])
+    b.add_cast_op("t1", "out", [64, 48])
+    s = b.move()
+    s.schedule("rocm")
+    nodes = [n for n in s.library_nodes() if not n["code"].startswith("ROCMOff")]
+    assert [n["code"] for n in nodes] == ["ROCMMap"]
+    (nest,) = nodes
+    assert [r["element_type"] for r in nest["reads"]] == ["BFloat", "BFloat"] and [w["element_type"] for w in nest["writes"]] == ["BFloat"]
+    assert [(st["op"], st["type"]) for st in nest["statements"]] == [("assign", "Float"), ("assign", "Float"), ("fp_mul", "Float"),
+                                                                     ("tanh", "Float"), ("assign", "BFloat")]
+    assert not {"xw", "yw", "t0", "t1"} & set(s.containers)
+    s.generate(str(tmp_path))
+    (text,) = [p.read_text() for p in sorted(tmp_path.glob("kernel_*.hip"))]
+    assert "const __bf16* p__in0, const __bf16* p__in1, __bf16* p__out0" in text
+    assert "docc_load<__bf16, V, true>" in text and "docc_store<__bf16, V>" in text
+    assert "const float _v0 = (float) (_in0);" in text and "const __bf16 _v4 = (__bf16) (_v3);" in text
+    # arithmetic on bf16 values is not a nest
+    bad = StructuredSDFGBuilder("bad_bf16")
+    bad.add_container("A", BF16, True)
+    bad.add_map_nest([("i", 8)], [("a", "A", ["1"])], [("p", "fp_add", ["a", "a"])], [("A", ["1"], "p")])
+    with pytest.raises(InvalidSDFGException, match="must be Float or Double"):
+        bad.move().validate()
