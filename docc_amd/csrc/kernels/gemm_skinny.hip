@@ -1,5 +1,5 @@
-// A few rows times a wide matrix for gfx950: C[m, n] = alpha * A[m, k] * op(B) + beta * C with 5 <= m <= 32 and n, k in the
-// thousands (a batch of vectors through a layer). The product reads B once (4 k n bytes) for 2 m k n flops, so it is bound by
+// A few rows times a wide matrix for gfx950: C[m, n] = alpha * A[m, k] * op(B) + beta * C with m up to 32 and n, k in the
+// thousands (a batch of vectors through a layer); fp32 first, bf16 with B stored [n][k] further down. The product reads B once (4 k n bytes) for 2 m k n flops, so it is bound by
 // HBM as long as the MFMA work stays small: the 32 x 32 x 2 instruction allows 9.8 TB/s of B at the device's fp32 rate, the
 // 16 x 16 x 4 one (m <= 16) twice that. The tiles of the GEMM kernels stage both operands through LDS in steps a work-group
 // waits out and pad m to 64; here B goes from global memory straight into the MFMA operand registers:

@@ -45,7 +45,10 @@ extern "C" {
  * (reference opt/src/targets/cuda/blas/gemm.cpp:131-185).
  * Zero-sized m, n: nothing is done; k == 0: C = beta * C. Products with one output
  * column or row (bf16 ones too) run as matrix-vector kernels (HBM-bound); their partial sums may pass through
- * 8 MiB of device memory that the library keeps per stream (see docc_rocm_softmax).
+ * 8 MiB of device memory that the library keeps per stream (see docc_rocm_softmax). So may the products of a
+ * few rows or few output tiles with a long K extent, which are computed in parts of K and added in a fixed order
+ * (the result does not depend on scheduling); parts beyond 8 MiB take a block of the device block cache for the
+ * call, in stream order (up to 64 MiB).
  */
 int docc_rocm_dgemm(docc_rocm_stream_t stream, int trans_a, int trans_b, int64_t m, int64_t n, int64_t k,
                     double alpha, const double* A, int64_t lda, const double* B, int64_t ldb, double beta,
