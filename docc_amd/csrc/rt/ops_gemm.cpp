@@ -247,8 +247,9 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // DOCC_ROCM_GEMM_SKINNY=1 takes them for smaller ones too (tests).
     const char* skinny_env = std::getenv("DOCC_ROCM_GEMM_SKINNY");
     const bool skinny_on = !(skinny_env && skinny_env[0] == '0'), skinny_any_size = skinny_env && skinny_env[0] == '1';
+    // (a lane's offset from the chunk's base, up to 31 rows of either operand, is held in 32 bits)
     const bool skinny_base = batch == 1 && !ta && (!epilogue || ldc == n) && n >= 512 && k >= 512 && skinny_on && (uintptr_t) A % 16 == 0 &&
-                             (uintptr_t) B % 16 == 0;
+                             (uintptr_t) B % 16 == 0 && lda < (int64_t(1) << 26) && ldb < (int64_t(1) << 26);
     // (B stored [n][k]: from 3 rows, where the matrix-vector form for several vectors falls behind - 4 x 8192 x 8192 67 -> 57 us,
     // 4 x 4096 x 11008 62 -> 48 - but up to 8 rows not above 128 M elements, where that form is the faster one again)
     const bool skinny_f32 = sizeof(T) == 4 && skinny_base && m >= (skinny_any_size ? 2 : tb ? 3 : 5) && m <= (tb ? 16 : 32) &&
