@@ -27,6 +27,9 @@ struct ConvParams {
     float* Y;
     int N, C, H, W, OC, KH, KW, OH, OW;
     int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+    // channels of the tensors X and Y lie in: C and OC, or more when the call is one group of a grouped convolution (the
+    // images are then XC and YC channels apart)
+    int XC, YC;
 };
 
 template <int BM, int BN, int BK, int WM, int WN, bool ALIGNED>
@@ -69,7 +72,7 @@ struct ConvGatherKernel {
         const int gp = col_ok ? (int) (gcol % P) : 0;
         const int ih0 = (gp / p.OW) * p.stride_h - p.pad_h;
         const int iw0 = (gp % p.OW) * p.stride_w - p.pad_w;
-        const float* xbase = p.X + (gn * p.C * p.H + ih0) * (long) p.W + iw0;
+        const float* xbase = p.X + (gn * p.XC * p.H + ih0) * (long) p.W + iw0;
         const int kk0 = tid / BN;  // first k row of this thread inside a K-step
 
         auto build_table = [&](int kt, int buf) {
@@ -170,7 +173,7 @@ struct ConvGatherKernel {
             const long col = n0 + wn * WTN + j * MT + lrow;
             if (col >= ncols) continue;
             const long n = col / P, pp = col % P;
-            float* ybase = p.Y + n * p.OC * P + pp;
+            float* ybase = p.Y + n * p.YC * P + pp;
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -300,11 +303,11 @@ struct ConvHaloKernel {
             const int img = MULTI ? e / PS : 0, pe = MULTI ? e % PS : e;      // image of the group, pixel of its patch
             const int ih = oh0 * p.stride_h - p.pad_h + pe / WP, iw = pe % WP - p.pad_w;
             inside[r] = e < PST && n + img < p.N && ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
-            goff[r] = inside[r] ? 4u * (unsigned) (img * p.C * p.H * p.W + ih * p.W + iw) : 0u;
+            goff[r] = inside[r] ? 4u * (unsigned) (img * p.XC * p.H * p.W + ih * p.W + iw) : 0u;
             slot[r] = (e < PST ? e : PST) * CI;
         }
         const long HW = (long) p.H * p.W;
-        const char* xn = reinterpret_cast<const char*>(p.X + (long) n * p.C * HW);
+        const char* xn = reinterpret_cast<const char*>(p.X + (long) n * p.XC * HW);
         const int K = p.C * KHW;
         // weight slab: memory holds [oc][channel][tap], LDS wants [oc][tap][channel]. Each of this
         // thread's vectors is four channels of one (oc, tap): four loads KHW floats apart, one
@@ -536,7 +539,7 @@ struct ConvHaloKernel {
             auto bread = [&](int j, int t) { return *reinterpret_cast<const f32x4*>(bbase + ((t / KW) * WP + (t % KW)) * CI + boff[j]); };
             // full rows: pixel q of the strip is q floats behind the strip's first pixel in every channel plane. A wave-uniform
             // base and 32-bit lane offsets, one per accumulator row: a store is then an accumulator read, the bias and the store
-            char* const ybase = reinterpret_cast<char*>(p.Y + ((long) n * p.OC + oc0) * plane + (long) oh0 * p.OW);
+            char* const ybase = reinterpret_cast<char*>(p.Y + ((long) n * p.YC + oc0) * plane + (long) oh0 * p.OW);
             unsigned yoff[16];
 #pragma unroll
             for (int r = 0; r < 16; r++)
@@ -702,7 +705,7 @@ struct ConvHaloKernel {
             }
             const int oh = oh0 + q / p.OW, ow = q % p.OW;
             if (oh >= p.OH) return;
-            float* ybase = p.Y + ((long) (n + img) * p.OC * p.OH + oh) * p.OW + ow;
+            float* ybase = p.Y + ((long) (n + img) * p.YC * p.OH + oh) * p.OW + ow;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int oc = oc0 + ocw * 32 + Mfma<float>::acc_row(lane, r);
@@ -726,7 +729,7 @@ struct ConvHaloKernel {
 #pragma unroll
                 for (int j = 0; j < TOWN; j++) {
                     const int q = tile_pixel0(j) + l32;
-                    float* ybase = p.Y + ((long) n * p.OC * p.OH + oh0 + q / p.OW) * p.OW + q % p.OW +
+                    float* ybase = p.Y + ((long) n * p.YC * p.OH + oh0 + q / p.OW) * p.OW + q % p.OW +
                                    (long) (oc0 + ocw * 32 + 4 * g) * p.OH * p.OW;
 #pragma unroll
                     for (int r = 0; r < 16; r++)
@@ -779,7 +782,7 @@ struct ConvHaloKernel {
                 const int q = 2 * TOWN * 32 + (lane & 15);
                 const int oh = oh0 + q / p.OW, ow = q % p.OW;
                 if (q < npix && oh < p.OH) {
-                    float* ybase = p.Y + ((long) n * p.OC * p.OH + oh) * p.OW + ow;
+                    float* ybase = p.Y + ((long) n * p.YC * p.OH + oh) * p.OW + ow;
 #pragma unroll
                     for (int k = 0; k < 8; k++) {
                         const int oc = oc0 + ocw * 32 + (k / 4) * 16 + 4 * (lane >> 4) + k % 4;
@@ -867,7 +870,7 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_im2col_f32(docc_k:
     const int n = n0 + (int) (j / P), pix = (int) (j % P);
     const int oh = pix / p.OW, ow = pix % p.OW;
     const int ih0 = oh * p.stride_h - p.pad_h, iw0 = ow * p.stride_w - p.pad_w;
-    const float* x = p.X + (long) n * p.C * p.H * p.W;
+    const float* x = p.X + (long) n * p.XC * p.H * p.W;
     for (int kk = blockIdx.y; kk < K; kk += gridDim.y) {
         const int c = kk / (p.KH * p.KW), t = kk % (p.KH * p.KW);
         const int ih = ih0 + (t / p.KW) * p.dil_h, iw = iw0 + (t % p.KW) * p.dil_w;

@@ -19,6 +19,7 @@ struct ConvParams {
     float* Y;
     int N, C, H, W, OC, KH, KW, OH, OW;
     int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+    int XC, YC;   // channels of the tensors X and Y lie in (C and OC, or more for one group of a grouped convolution)
 };
 
 int64_t out_dim(int64_t d_in, int64_t pad_begin, int64_t pad_end, int64_t dil, int64_t kernel, int64_t stride) {
@@ -221,7 +222,13 @@ extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, in
 // enter through the output extents.
 static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
                       int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h,
-                      int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
+                      int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes,
+                      int64_t x_channels = -1, int64_t y_channels = -1) {
+    // x_channels, y_channels: the channels of the tensors X and Y point into, where this call is one group of a grouped
+    // convolution (the images are then that many channels apart); -1: C and OC
+    if (x_channels < 0) x_channels = C;
+    if (y_channels < 0) y_channels = OC;
+    const bool slice = x_channels != C || y_channels != OC;
     if (N < 0 || C < 0 || H < 0 || W < 0 || OC < 0 || KH <= 0 || KW <= 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
     if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0 || pad_h_end < 0 || pad_w_end < 0)
@@ -231,21 +238,24 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     if (N == 0 || OC == 0 || OH == 0 || OW == 0) return 0;
     if (!Y || !Wt || (C > 0 && !X)) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: null pointer");
     const int64_t lim = 0x7fffffffLL;
-    if (C * H * W >= lim || C * KH * KW >= lim || OH * OW >= lim || N >= lim || OC >= lim)
+    if (x_channels * H * W >= lim || C * KH * KW >= lim || OH * OW >= lim || N >= lim || y_channels >= lim)
         return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: per-image extents must fit in 31 bits");
     int rc = ensure_device();
     if (rc) return rc;
 
     ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
-                 (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w};
+                 (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) x_channels, (int) y_channels};
     // Stride-1, dilation-1 3x3 and 1x1 convolutions take the LDS-halo kernel: 64 output channels x a
     // strip of TH full output rows (at most 448 pixels) per work-group, 8 input channels per chunk.
     const bool halo_shape = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w) && ((uintptr_t) Wt % 16 == 0);
     const int64_t need = docc_rocm_conv2d_f32_pads_workspace_bytes(N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end,
                                                                    dil_h, dil_w);
     const bool have_workspace = workspace && workspace_bytes >= need && need > 0 && ((uintptr_t) workspace % 256) == 0;
-    const ConvPath path = C == 0 ? ConvPath::Gather
-                                 : choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, any_pad_h, any_pad_w, halo_shape, have_workspace);
+    ConvPath path = C == 0 ? ConvPath::Gather
+                           : choose_path(N, C, OC, KH, KW, OH, OW, stride_h, stride_w, any_pad_h, any_pad_w, halo_shape, have_workspace);
+    // one group of a grouped convolution: the direct kernels, which take the distance between the images as it is (the
+    // GEMM paths write whole [N, OC, P] tensors)
+    if (slice && (path == ConvPath::Gemm1x1 || path == ConvPath::GemmColumns)) path = halo_shape ? ConvPath::Halo : ConvPath::Gather;
     if (path == ConvPath::Gemm1x1) {
         // Y[n] (OC x P) = W (OC x C) X[n] (C x P): one batched GEMM on the tensors as they lie; the bias is
         // written first and accumulated onto
@@ -297,7 +307,7 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         const int64_t stage = 64 * (8 * KH * KW + 4) + 8 * (PS + 1);  // weights + patch + spare pixel, floats
         const int64_t strips = (OH + TH - 1) / TH;
         if (plan.images > 1 && plan.cost > 0.0 && PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) &&
-            plan.images * C * H * W < (int64_t(1) << 29) && (OC + 63) / 64 <= 65535) {
+            plan.images * x_channels * H * W < (int64_t(1) << 29) && (OC + 63) / 64 <= 65535) {
             char name[64];
             std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s_t%dm", KH == 3 ? "3x3" : "1x1", plan.tiles);
             return launch(name, (uint32_t) ((N + plan.images - 1) / plan.images), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4),
@@ -342,4 +352,30 @@ extern "C" int docc_rocm_conv2d_f32_pads(docc_rocm_stream_t stream, int64_t N, i
                                          const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
     return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w, X, Wt, bias, Y,
                       workspace, workspace_bytes);
+}
+
+// ONNX Conv with group > 1 (reference ConvNode: W [OC][C / group][KH][KW], conv_node.cpp:376-377; output channel oc belongs
+// to group oc / (OC / group) and reads that group's C / group input channels): one call of the kernels above per group, on
+// the group's channels of X and Y where they lie.
+extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH,
+                                            int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end,
+                                            int64_t pad_w_end, int64_t dil_h, int64_t dil_w, int64_t group, const float* X, const float* Wt,
+                                            const float* bias, float* Y, void* workspace, int64_t workspace_bytes) {
+    if (group <= 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: group must be positive");
+    if (group == 1)
+        return conv2d_run(stream, N, C, H, W, OC, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w, X, Wt, bias, Y,
+                          workspace, workspace_bytes);
+    if (C < 0 || OC < 0 || C % group != 0 || OC % group != 0)
+        return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: group %lld does not divide the channels (%lld in, %lld out)", (long long) group,
+                    (long long) C, (long long) OC);
+    if (KH <= 0 || KW <= 0 || H < 0 || W < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
+    const int64_t cg = C / group, og = OC / group;
+    const int64_t OH = out_dim(H, pad_h, pad_h_end, dil_h, KH, stride_h), OW = out_dim(W, pad_w, pad_w_end, dil_w, KW, stride_w);
+    for (int64_t g = 0; g < group; g++) {
+        const int rc = conv2d_run(stream, N, cg, H, W, og, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w,
+                                  X ? X + g * cg * H * W : nullptr, Wt ? Wt + g * og * cg * KH * KW : nullptr, bias ? bias + g * og : nullptr,
+                                  Y ? Y + g * og * OH * OW : nullptr, nullptr, 0, C, OC);
+        if (rc) return rc;
+    }
+    return 0;
 }

@@ -294,6 +294,15 @@ protected:
              << ", " << get(c.dilations(), 0, "1") << ", " << get(c.dilations(), 1, "1");   // pads: begins, then ends
         // layers that run as im2col + GEMM take their column matrix from a workspace that lives around the node;
         // for the others the size is 0 and nothing is allocated
+        int64_t group = 1;
+        if (!symbolic::is_integer(c.group(), &group) || group != 1) {
+            // the node's group (weights [C_out][C_in / group][kh][kw]): the direct kernels, once per group
+            s << "DOCC_ROCM_CHECK(docc_rocm_conv2d_f32_grouped(nullptr, " << dims.str() << ", (int64_t) (" << c.group() << "), (const float *) "
+              << name_of("X") << ", (const float *) " << name_of("W") << ", "
+              << (c.has_bias() ? "(const float *) " + name_of("B") : std::string("nullptr")) << ", (float *) " << name_of("Y")
+              << ", nullptr, 0));" << std::endl;
+            return;
+        }
         s << "{" << std::endl;
         s.setIndent(s.indent() + 4);
         s << "const int64_t __ws_bytes = docc_rocm_conv2d_f32_pads_workspace_bytes(" << dims.str() << ");" << std::endl;
@@ -950,8 +959,8 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!c) return decline("not a Conv node object");
         if (c->element() != P::Float) return decline("only Float is supported");
         if (c->kernel_shape().size() != 2) return decline("only 2-d convolution is supported");
-        int64_t group = 0;
-        if (!symbolic::is_integer(c->group(), &group) || group != 1) return decline("only group == 1 is supported");
+        int64_t group = 1;
+        if (symbolic::is_integer(c->group(), &group) && group < 1) return decline("group must be positive");
     } else if (node.code() == tensor::LibraryNodeType_Attention) {
         auto* a = dynamic_cast<tensor::AttentionNode*>(&node);
         if (!a) return decline("not an Attention node object");

@@ -451,6 +451,9 @@ Expression ConvNode::flop() const {
         out = symbolic::mul(out, output_dim(i));
         taps = symbolic::mul(taps, kernel_shape_[i]);
     }
+    int64_t g = 1;
+    if (!symbolic::is_integer(group_, &g)) return "2*(" + symbolic::mul(out, taps) + ") / (" + group_ + ")";
+    if (g > 1) return "2*(" + symbolic::mul(out, taps) + ") / " + std::to_string(g);
     return "2*" + symbolic::mul(out, taps);
 }
 
@@ -479,9 +482,12 @@ std::unique_ptr<ConvNode> ConvNode::from_json(const Value& j) {
 
 Expression ConvNode::connector_bytes(const std::string& connector) const {
     if (connector == "X") return bytes_of(product(shape_, 0, shape_.size()), element_);
-    if (connector == "W") {
+    if (connector == "W") {   // [C_out][C_in / group][k0][k1] (reference conv_node.cpp:376-377)
         Expression e = symbolic::mul(output_channels_, shape_[1]);
         for (auto& k : kernel_shape_) e = symbolic::mul(e, k);
+        int64_t g = 1;
+        if (!symbolic::is_integer(group_, &g)) e = "(" + e + ") / (" + group_ + ")";
+        else if (g > 1) e = "(" + e + ") / " + std::to_string(g);
         return bytes_of(e, element_);
     }
     if (connector == "B") return bytes_of(output_channels_, element_);

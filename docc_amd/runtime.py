@@ -88,6 +88,7 @@ _SIGNATURES = {
     "docc_rocm_conv2d_f32": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp],
     "docc_rocm_conv2d_f32_pads_workspace_bytes": [_i64] * 15,
     "docc_rocm_conv2d_f32_pads": [_vp] + [_i64] * 15 + [_vp, _vp, _vp, _vp, _vp, _i64],
+    "docc_rocm_conv2d_f32_grouped": [_vp] + [_i64] * 16 + [_vp, _vp, _vp, _vp, _vp, _i64],
     "docc_rocm_conv2d_f32_workspace_bytes": [_i64] * 13,
     "docc_rocm_conv2d_f32_ws": [_vp] + [_i64] * 13 + [_vp, _vp, _vp, _vp, _vp, _i64],
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
@@ -340,6 +341,12 @@ def conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, pads, dilation, X, Wt, bias,
     """The convolution with a begin and an end pad per axis: `pads` = (top, left, bottom, right)."""
     call("docc_rocm_conv2d_f32_pads", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pads[0], pads[1], pads[2], pads[3],
          dilation[0], dilation[1], X, Wt, bias or None, Y, workspace or None, workspace_bytes)
+
+
+def conv2d_f32_grouped(N, C, H, W, OC, KH, KW, stride, pads, dilation, group, X, Wt, bias, Y, workspace=0, workspace_bytes=0, stream=0) -> None:
+    """The convolution with the node's `group`: weights [OC, C / group, KH, KW]; `pads` = (top, left, bottom, right)."""
+    call("docc_rocm_conv2d_f32_grouped", stream, N, C, H, W, OC, KH, KW, stride[0], stride[1], pads[0], pads[1], pads[2], pads[3],
+         dilation[0], dilation[1], group, X, Wt, bias or None, Y, workspace or None, workspace_bytes)
 
 
 def attention_bf16(B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16=False, stream=0) -> None:

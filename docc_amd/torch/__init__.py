@@ -13,7 +13,7 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
                                               the bf16 GEMM with float32 accumulation - its float32 result where the model
                                               asks for it (`.float()`), else rounded once to bf16 (ml::Cast) as eager torch does
     softmax(x, dim=-1) on fp32             -> ml::Softmax
-    F.conv2d / nn.Conv2d (groups == 1)     -> ml::Conv with padding and bias
+    F.conv2d / nn.Conv2d                   -> ml::Conv with padding, bias and groups
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
                                            -> ml::Attention (bf16; head dims 32, 64, 128 fused)
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number; on bf16
@@ -249,8 +249,9 @@ class _FxLowering:
         pair = lambda v: [int(v), int(v)] if isinstance(v, int) else [int(e) for e in v]
         if not isinstance(x, _T) or not isinstance(w, _T) or len(x.shape) != 4 or len(w.shape) != 4:
             self.fail(node, "conv2d on these operands")
-        if groups != 1:
-            self.fail(node, "grouped convolution")
+        groups = int(groups)
+        if groups < 1 or x.shape[1] % groups or w.shape[0] % groups or w.shape[1] * groups != x.shape[1]:
+            self.fail(node, "a convolution whose groups do not divide the channels")
         if isinstance(padding, str):
             self.fail(node, "string padding modes")
         if x.dtype != self.torch.float32:
@@ -258,7 +259,7 @@ class _FxLowering:
         stride, padding, dilation = pair(stride), pair(padding), pair(dilation)
         oh, ow = ((x.shape[2 + i] + 2 * padding[i] - dilation[i] * (w.shape[2 + i] - 1) - 1) // stride[i] + 1 for i in range(2))
         out = self.new_tensor([x.shape[0], w.shape[0], oh, ow], x.dtype, dest)
-        self.builder.add_conv(x.name, w.name, out.name, x.shape, w.shape[2:], stride, padding + padding, dilation, w.shape[0], 1,
+        self.builder.add_conv(x.name, w.name, out.name, x.shape, w.shape[2:], stride, padding + padding, dilation, w.shape[0], groups,
                               bias.name if isinstance(bias, _T) else None)
         return out
 

@@ -208,15 +208,24 @@ def conv_out_dim(d_in, pad, dilation, kernel, stride) -> int:
     return int(load().oracle_conv_out_dim(d_in, pad, pad, dilation, kernel, stride))
 
 
-def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None) -> np.ndarray:
-    """`pad`: (height, width) on both sides, or (top, left, bottom, right) as the node orders them (begins, then ends)."""
+def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None, group=1) -> np.ndarray:
+    """`pad`: (height, width) on both sides, or (top, left, bottom, right) as the node orders them (begins, then ends).
+    `group` (reference conv_node.cpp:376-377: W [OC][C / group][KH][KW]; ONNX Conv): output channel oc belongs to group
+    oc / (OC / group) and reads that group's C / group input channels - the convolution below on each group's slices."""
     lib = lib or load()
     X = _c(X, np.float32)
     W = _c(W, np.float32)
     N, C, H, Wd = X.shape
     OC, C2, KH, KW = W.shape
+    if group != 1:
+        if group < 1 or C % group or OC % group or C2 * group != C:
+            raise ValueError("group must divide the channels, and W must hold C / group input channels")
+        cg, og = C // group, OC // group
+        parts = [conv2d(X[:, g * cg:(g + 1) * cg], W[g * og:(g + 1) * og], None if bias is None else np.asarray(bias)[g * og:(g + 1) * og],
+                        stride, pad, dilation, lib) for g in range(group)]
+        return np.concatenate(parts, axis=1)
     if C2 != C:
-        raise ValueError("group != 1 is not supported")
+        raise ValueError("W holds another number of input channels than X (pass group)")
     pad = tuple(pad) if len(pad) == 4 else (pad[0], pad[1], pad[0], pad[1])
     OH = int(lib.oracle_conv_out_dim(H, pad[0], pad[2], dilation[0], KH, stride[0]))
     OW = int(lib.oracle_conv_out_dim(Wd, pad[1], pad[3], dilation[1], KW, stride[1]))

@@ -259,3 +259,43 @@ def test_conv_with_different_pads_before_and_after(rt, monkeypatch, force, case)
         assert torch.equal(y1, y2)
     with pytest.raises(rt.RocmRuntimeError, match="padding non-negative"):
         rt.conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, (0, 0, -1, 0), dil, x.data_ptr(), w.data_ptr(), 0, y.data_ptr())
+
+
+GROUP_CASES = [
+    # N, C, H, W, OC, KH, KW, stride, pads, dilation, group, bias
+    (2, 32, 12, 12, 64, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 2, True),      # 16 channels a group: the LDS-halo kernel per group
+    (3, 64, 9, 11, 64, 3, 3, (2, 2), (1, 0, 0, 1), (1, 1), 4, False),      # strides of 2, a begin and an end pad, four groups
+    (2, 16, 10, 10, 16, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 16, True),     # depthwise: one channel a group, the gather kernel
+    (1, 12, 8, 7, 30, 2, 3, (1, 2), (0, 1, 1, 0), (2, 1), 6, True),        # two channels in, five out per group, dilation
+    (2, 256, 7, 7, 512, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 2, False),     # pointwise: a GEMM when whole, direct per group
+]
+
+
+@pytest.mark.parametrize("case", GROUP_CASES)
+def test_conv_with_groups(rt, case):
+    """The node's `group`: weights [OC, C / group, KH, KW], every group on its own channels of X and Y where they lie. Integer-
+    valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
+    N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
+    rng = np.random.default_rng(hash(case[:7]) & 0xffff)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, C // group, KH, KW)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    ref = oracle.conv2d(X, Wt, b, stride, pads, dil, group=group)
+    x, w = dev(X), dev(Wt)
+    bd = dev(b) if b is not None else None
+    y = torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, KH, KW, stride, pads, dil, group, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0,
+                          y.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    # one group is the entry point without groups
+    full = rng.integers(-4, 5, (OC, C, KH, KW)).astype(np.float32)
+    wf = dev(full)
+    y1, y2 = torch.full(ref.shape, float("nan"), device="cuda"), torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, KH, KW, stride, pads, dil, 1, x.data_ptr(), wf.data_ptr(), bd.data_ptr() if bd is not None else 0, y1.data_ptr())
+    rt.conv2d_f32_pads(N, C, H, W, OC, KH, KW, stride, pads, dil, x.data_ptr(), wf.data_ptr(), bd.data_ptr() if bd is not None else 0, y2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2)
+    for bad in (0, -2, 5 if C % 5 else 7):
+        with pytest.raises(rt.RocmRuntimeError, match="group"):
+            rt.conv2d_f32_grouped(N, C, H, W, OC, KH, KW, stride, pads, dil, bad, x.data_ptr(), w.data_ptr(), 0, y.data_ptr())

@@ -779,6 +779,33 @@ def test_torch_bf16_elementwise_chain_like_eager():
         assert (g.float() - e.float()).abs().max().item() <= 4 * 2.0 ** -8 * scale
 
 
+def test_torch_grouped_and_depthwise_convolutions():
+    """nn.Conv2d with groups: ml::Conv carries the group, the weights [out, in / groups, kh, kw] travel as they are. A grouped
+    3x3 layer and a depthwise one (as in a MobileNet block) against eager torch in float64."""
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.grouped = torch.nn.Conv2d(32, 64, 3, padding=1, groups=4)
+            self.depthwise = torch.nn.Conv2d(64, 64, 3, stride=2, padding=1, groups=64, bias=False)
+            self.pointwise = torch.nn.Conv2d(64, 48, 1)
+
+        def forward(self, x):
+            return self.pointwise(torch.relu(self.depthwise(torch.relu(self.grouped(x)))))
+
+    torch.manual_seed(31)
+    model = Net().cuda()
+    x = torch.randn(3, 32, 20, 20).cuda()
+    program = docc_torch.compile_torch(model, (x,), target="rocm")
+    out = program(x)
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    convs = [n for n in program.last_sdfg.library_nodes() if n["code"] == "ml::Conv"]
+    assert [n["group"] for n in convs] == ["4", "64", "1"]
+    with torch.no_grad():
+        ref = model.double()(x.double())
+    assert out.shape == ref.shape == (3, 48, 10, 10)
+    assert rel_err_max(out.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
+
+
 def test_power_operator_through_both_front_ends():
     """x ** 2, x ** y and np.power lower to ml::Pow (array or scalar operand); torch.pow likewise."""
     @native(target="rocm")

@@ -150,6 +150,25 @@ def test_conv_against_torch(stride, pad, dil):
     assert rel(oracle.conv2d(x.numpy(), w.numpy(), None, stride, pad, dil), ref - b.double().numpy()[None, :, None, None]) <= 1e-6
 
 
+@pytest.mark.parametrize("group,C,OC", [(2, 6, 4), (3, 3, 6), (4, 8, 8)])
+def test_conv_with_groups_two_other_statements(group, C, OC):
+    """The grouped form against two statements that share none of its code: torch's conv2d with groups in float64, and the
+    dense convolution with the weights laid out block-diagonally (a group's filters see zeros on the other groups' channels)."""
+    g = torch.Generator().manual_seed(group)
+    x, w, b = torch.randn(2, C, 9, 8, generator=g), torch.randn(OC, C // group, 3, 2, generator=g), torch.randn(OC, generator=g)
+    Y = oracle.conv2d(x.numpy(), w.numpy(), b.numpy(), (2, 1), (1, 0, 0, 2), (1, 2), group=group)
+    xp = torch.nn.functional.pad(x.double(), (0, 2, 1, 0))          # (left, right, top, bottom)
+    ref = torch.nn.functional.conv2d(xp, w.double(), b.double(), stride=(2, 1), dilation=(1, 2), groups=group).numpy()
+    assert Y.shape == ref.shape and rel(Y, ref) <= 1e-6
+    dense = np.zeros((OC, C, 3, 2), np.float32)
+    cg, og = C // group, OC // group
+    for j in range(group):
+        dense[j * og:(j + 1) * og, j * cg:(j + 1) * cg] = w.numpy()[j * og:(j + 1) * og]
+    assert np.array_equal(Y, oracle.conv2d(x.numpy(), dense, b.numpy(), (2, 1), (1, 0, 0, 2), (1, 2)))
+    with pytest.raises(ValueError):
+        oracle.conv2d(x.numpy(), w.numpy(), None, group=group + 5)
+
+
 def test_conv_closed_forms():
     # all-ones input and kernel: the output counts the taps inside the image (zero padding)
     Y = oracle.conv2d(np.ones((1, 2, 5, 5), np.float32), np.ones((1, 2, 3, 3), np.float32), pad=(1, 1))

@@ -143,9 +143,22 @@ def test_mapper_sets_implementation_types_and_declines_what_the_kernels_lack():
     b = StructuredSDFGBuilder("c")
     for n in ("X", "W", "Y"):
         b.add_container(n, F32, True)
-    b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 4, group=2)
+    b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 4, group=0)
     with pytest.raises(InvalidSDFGException, match="group"):
         b.move().schedule("rocm")
+    # the node's group is taken: the launcher for grouped convolutions, the weights [C_out, C_in / group, kh, kw] on the device
+    b = StructuredSDFGBuilder("cg")
+    for n in ("X", "W", "Y"):
+        b.add_container(n, F32, True)
+    b.add_conv("X", "W", "Y", [1, 4, 8, 8], [3, 3], [1, 1], [1, 1, 1, 1], [1, 1], 6, group=2)
+    s = b.move()
+    s.schedule("rocm")
+    import tempfile
+    with tempfile.TemporaryDirectory() as folder:
+        text = re.sub(r"\s+", " ", Path(s.generate(folder)["source"]).read_text())
+    assert "docc_rocm_conv2d_f32_grouped(nullptr, 1, 4, 8, 8, 6, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, (int64_t) (2), (const float *)" in text
+    assert "nullptr, 0));" in text and "docc_rocm_conv2d_f32_pads(" not in text
+    assert "docc_rocm_memcpy_h2d_async(_dst, _src, (size_t) (((216) / 2)*4), nullptr)" in text       # W: 6 x 4 / 2 x 3 x 3 floats
     # a convolution whose pads differ between begin and end is taken: the launcher gets all four (begins, then ends)
     b = StructuredSDFGBuilder("cp")
     for n in ("X", "W", "Y"):
