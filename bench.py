@@ -522,6 +522,17 @@ def main():
             mfma(name, "f32", 2 * 32 * OC * OH * OH * C * 9,
                  lambda i: rt.conv2d_f32(32, C, H, H, OC, 3, 3, (st, st), (1, 1), (1, 1), X.data_ptr(), W.data_ptr(), b.data_ptr(), Y.data_ptr(), stream=stream))
             del X, W, b, Y
+        # a depthwise layer (group == C): nine multiply-adds per element against eight bytes moved, bound by HBM; four
+        # input tensors of 103 MB in turn
+        C = 256
+        Xs = [torch.randn(32, C, 56, 56).cuda() for _ in range(ROTATE)]
+        W = torch.randn(C, 1, 3, 3).cuda()
+        b = torch.randn(C).cuda()
+        Y = torch.empty(32, C, 56, 56, device="cuda")
+        hbm("conv2d_depthwise_n32c256hw56k3", 2 * 4 * 32 * C * 56 * 56,
+            lambda i: rt.conv2d_f32_grouped(32, C, 56, 56, C, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), C, Xs[i % ROTATE].data_ptr(), W.data_ptr(),
+                                            b.data_ptr(), Y.data_ptr(), stream=stream))
+        del Xs, W, b, Y
 
     # ---- a launch-bound function: kernel by kernel, and replayed as a HIP graph --------------------------
     # LayerNorm -> Linear -> GELU -> Linear + residual on [8, 128, 256] device tensors compiles to eight kernels of a

@@ -371,6 +371,30 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
     if (KH <= 0 || KW <= 0 || H < 0 || W < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
     const int64_t cg = C / group, og = OC / group;
     const int64_t OH = out_dim(H, pad_h, pad_h_end, dil_h, KH, stride_h), OW = out_dim(W, pad_w, pad_w_end, dil_w, KW, stride_w);
+    // depthwise (one input channel a group): one launch of the kernel that is bound by moving X and Y; DOCC_ROCM_CONV=gather
+    // keeps the launch per group (tests)
+    const char* force = std::getenv("DOCC_ROCM_CONV");
+    if (cg == 1 && !(force && force[0] == 'g')) {
+        if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0 || pad_h_end < 0 || pad_w_end < 0 || N < 0)
+            return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: stride and dilation must be positive, padding non-negative");
+        if (N == 0 || OC == 0 || OH == 0 || OW == 0) return 0;
+        if (!Y || !Wt || !X) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: null pointer");
+        const int64_t lim = 0x7fffffffLL, P = OH * OW;
+        const int64_t blocks = N * OC * ((P + 255) / 256);
+        if (C * H * W >= lim || P >= lim || N >= lim || OC >= lim || KH * KW >= lim || blocks >= lim)
+            return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: per-image extents must fit in 31 bits");
+        if (int rc = ensure_device()) return rc;
+        ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
+                     (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) C, (int) OC};
+        // 3x3, stride 1, rows of whole aligned quads: four pixels a lane
+        if (KH == 3 && KW == 3 && stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && pad_w == 1 && OW == W && W % 4 == 0 &&
+            (uintptr_t) X % 16 == 0 && (uintptr_t) Y % 16 == 0 && !(force && force[0] == 's')) {   // DOCC_ROCM_CONV=scalar: a pixel a lane (tests)
+            const int64_t quads = N * OC * ((OH * (OW / 4) + 255) / 256);
+            return launch("docc_conv2d_depthwise_f32_3x3_v4", (uint32_t) quads, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
+        }
+        const char* name = KH == 3 && KW == 3 ? "docc_conv2d_depthwise_f32_3x3" : KH == 5 && KW == 5 ? "docc_conv2d_depthwise_f32_5x5" : "docc_conv2d_depthwise_f32";
+        return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
+    }
     for (int64_t g = 0; g < group; g++) {
         const int rc = conv2d_run(stream, N, cg, H, W, og, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w,
                                   X ? X + g * cg * H * W : nullptr, Wt ? Wt + g * og * cg * KH * KW : nullptr, bias ? bias + g * og : nullptr,

@@ -268,14 +268,24 @@ GROUP_CASES = [
     (2, 16, 10, 10, 16, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 16, True),     # depthwise: one channel a group, the gather kernel
     (1, 12, 8, 7, 30, 2, 3, (1, 2), (0, 1, 1, 0), (2, 1), 6, True),        # two channels in, five out per group, dilation
     (2, 256, 7, 7, 512, 1, 1, (1, 1), (0, 0, 0, 0), (1, 1), 2, False),     # pointwise: a GEMM when whole, direct per group
+    (3, 8, 13, 9, 24, 3, 3, (2, 1), (1, 1, 0, 2), (1, 1), 8, True),        # depthwise with three output channels per input channel
+    (2, 24, 17, 17, 24, 5, 5, (1, 1), (2, 2, 2, 2), (1, 1), 24, False),    # depthwise 5x5
+    (1, 6, 9, 20, 12, 2, 4, (1, 3), (0, 3, 1, 0), (2, 1), 6, True),        # depthwise, a 2x4 filter with dilation and a stride of 3
+    (2, 40, 28, 28, 40, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 40, True),     # depthwise on planes of more than one work-group
+    (3, 16, 9, 12, 32, 3, 3, (1, 1), (0, 1, 2, 1), (1, 1), 16, True),      # rows of three quads, no rows above, two below
 ]
 
 
+@pytest.mark.parametrize("force", ["", "scalar", "gather"])      # depthwise layers: four pixels a lane where rows allow, one, and a launch per group
 @pytest.mark.parametrize("case", GROUP_CASES)
-def test_conv_with_groups(rt, case):
+def test_conv_with_groups(rt, monkeypatch, force, case):
     """The node's `group`: weights [OC, C / group, KH, KW], every group on its own channels of X and Y where they lie. Integer-
     valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
     N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
+    if force:
+        if group != C:
+            pytest.skip("only depthwise layers have a second form")
+        monkeypatch.setenv("DOCC_ROCM_CONV", force)
     rng = np.random.default_rng(hash(case[:7]) & 0xffff)
     X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
     Wt = rng.integers(-4, 5, (OC, C // group, KH, KW)).astype(np.float32)
