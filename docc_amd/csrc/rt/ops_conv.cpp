@@ -19,7 +19,8 @@ struct ConvParams {
     float* Y;
     int N, C, H, W, OC, KH, KW, OH, OW;
     int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
-    int XC, YC;   // channels of the tensors X and Y lie in (C and OC, or more for one group of a grouped convolution)
+    int XC, YC;   // channels of the tensors X and Y lie in (C and OC, or more for the groups of a grouped convolution)
+    long GX, GW, GB, GY;   // grouped convolution in one launch: elements from one group's operands to the next's (grid z = groups)
 };
 
 int64_t out_dim(int64_t d_in, int64_t pad_begin, int64_t pad_end, int64_t dil, int64_t kernel, int64_t stride) {
@@ -223,12 +224,13 @@ extern "C" int64_t docc_rocm_conv2d_f32_workspace_bytes(int64_t N, int64_t C, in
 static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH, int64_t KW,
                       int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end, int64_t pad_w_end, int64_t dil_h,
                       int64_t dil_w, const float* X, const float* Wt, const float* bias, float* Y, void* workspace, int64_t workspace_bytes,
-                      int64_t x_channels = -1, int64_t y_channels = -1) {
-    // x_channels, y_channels: the channels of the tensors X and Y point into, where this call is one group of a grouped
-    // convolution (the images are then that many channels apart); -1: C and OC
+                      int64_t x_channels = -1, int64_t y_channels = -1, int64_t groups = 1) {
+    // x_channels, y_channels: the channels of the tensors X and Y point into, where this call is a grouped convolution (the
+    // images are then that many channels apart); -1: C and OC. groups: that many convolutions of these extents in one launch
+    // (grid z), group g on the channels g * C .. of X, g * OC .. of Y, filters and bias
     if (x_channels < 0) x_channels = C;
     if (y_channels < 0) y_channels = OC;
-    const bool slice = x_channels != C || y_channels != OC;
+    const bool slice = x_channels != C || y_channels != OC || groups > 1;
     if (N < 0 || C < 0 || H < 0 || W < 0 || OC < 0 || KH <= 0 || KW <= 0)
         return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "conv2d: bad shape");
     if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0 || pad_h_end < 0 || pad_w_end < 0)
@@ -244,7 +246,10 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     if (rc) return rc;
 
     ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
-                 (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) x_channels, (int) y_channels};
+                 (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) x_channels, (int) y_channels,
+                 groups > 1 ? (long) (C * H * W) : 0, groups > 1 ? (long) (OC * C * KH * KW) : 0, groups > 1 ? (long) OC : 0, groups > 1 ? (long) (OC * OH * OW) : 0};
+    if (groups < 1 || groups > 65535) return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: 1 to 65535 groups");
+    const uint32_t gz = (uint32_t) groups;
     // Stride-1, dilation-1 3x3 and 1x1 convolutions take the LDS-halo kernel: 64 output channels x a
     // strip of TH full output rows (at most 448 pixels) per work-group, 8 input channels per chunk.
     const bool halo_shape = halo_shape_ok(C, KH, KW, OW, stride_h, stride_w, dil_h, dil_w) && ((uintptr_t) Wt % 16 == 0);
@@ -310,14 +315,14 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
             plan.images * x_channels * H * W < (int64_t(1) << 29) && (OC + 63) / 64 <= 65535) {
             char name[64];
             std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s_t%dm", KH == 3 ? "3x3" : "1x1", plan.tiles);
-            return launch(name, (uint32_t) ((N + plan.images - 1) / plan.images), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4),
+            return launch(name, (uint32_t) ((N + plan.images - 1) / plan.images), (uint32_t) ((OC + 63) / 64), gz, 256, (uint32_t) (3 * stage * 4),
                           (hipStream_t) stream, p, (int) TH, (int) plan.images);
         }
         if (plan.images == 1 && plan.cost > 0.0 && halo_strip_fits(TH, OW, KH, KW, stride_h, stride_w) && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
             char name[64];
             std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s", KH == 3 ? "3x3" : "1x1",
                           plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "");
-            return launch(name, (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), 1, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
+            return launch(name, (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), gz, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
         }
     }
     constexpr int BM = 64, BN = 128, BK = 16;
@@ -328,7 +333,7 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     // LDS: 2 x (A tile [BM][BK+4] + B tile [BK][BN+8]) floats + 2 x BK table entries of 16 bytes
     const uint32_t lds = 2 * (BM * (BK + 4) + BK * (BN + 8)) * 4 + 2 * BK * 16;
     return launch(aligned ? "docc_conv2d_f32_gather_64x128_a" : "docc_conv2d_f32_gather_64x128_u", (uint32_t) tiles, 1,
-                  1, 256, lds, (hipStream_t) stream, p);
+                  gz, 256, lds, (hipStream_t) stream, p);
 }
 
 extern "C" int docc_rocm_conv2d_f32(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC,
@@ -385,7 +390,7 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
             return fail(DOCC_ROCM_ERR_UNSUPPORTED, "conv2d: per-image extents must fit in 31 bits");
         if (int rc = ensure_device()) return rc;
         ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
-                     (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) C, (int) OC};
+                     (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) C, (int) OC, 0, 0, 0, 0};
         // 3x3, stride 1, rows of whole aligned quads: four pixels a lane
         if (KH == 3 && KW == 3 && stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && pad_w == 1 && OW == W && W % 4 == 0 &&
             (uintptr_t) X % 16 == 0 && (uintptr_t) Y % 16 == 0 && !(force && force[0] == 's')) {   // DOCC_ROCM_CONV=scalar: a pixel a lane (tests)
@@ -395,6 +400,10 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
         const char* name = KH == 3 && KW == 3 ? "docc_conv2d_depthwise_f32_3x3" : KH == 5 && KW == 5 ? "docc_conv2d_depthwise_f32_5x5" : "docc_conv2d_depthwise_f32";
         return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
     }
+    // every group in one launch (grid z) where the groups fit it, else a launch per group
+    if (group <= 65535 && !(force && force[0] == 'l'))   // DOCC_ROCM_CONV=loop: a launch per group (tests)
+        return conv2d_run(stream, N, cg, H, W, og, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w, X, Wt, bias, Y,
+                          nullptr, 0, C, OC, group);
     for (int64_t g = 0; g < group; g++) {
         const int rc = conv2d_run(stream, N, cg, H, W, og, KH, KW, stride_h, stride_w, pad_h, pad_w, pad_h_end, pad_w_end, dil_h, dil_w,
                                   X ? X + g * cg * H * W : nullptr, Wt ? Wt + g * og * cg * KH * KW : nullptr, bias ? bias + g * og : nullptr,

@@ -205,9 +205,9 @@ int docc_rocm_conv2d_f32_pads(docc_rocm_stream_t stream, int64_t N, int64_t C, i
 /*
  * The node's `group` (reference conv_node.h / conv_node.cpp:27-40 constructor, :376-377 weights [OC][C / group][KH][KW],
  * :586 JSON field; ONNX Conv semantics: output channel oc belongs to group oc / (OC / group) and reads the C / group input
- * channels of that group). C and OC are the channels of the whole tensors; group must divide both. One launch of the
- * direct kernels per group on that group's channels where they lie (group == 1: docc_rocm_conv2d_f32_pads, `workspace`
- * as there; it is not used for group > 1).
+ * channels of that group). C and OC are the channels of the whole tensors; group must divide both. The direct kernels run
+ * every group in one launch on that group's channels where they lie, a depthwise layer (group == C) on kernels of its own
+ * (group == 1: docc_rocm_conv2d_f32_pads, `workspace` as there; it is not used for group > 1).
  */
 int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H, int64_t W, int64_t OC, int64_t KH,
                                  int64_t KW, int64_t stride_h, int64_t stride_w, int64_t pad_h, int64_t pad_w, int64_t pad_h_end,

@@ -276,15 +276,17 @@ GROUP_CASES = [
 ]
 
 
-@pytest.mark.parametrize("force", ["", "scalar", "gather"])      # depthwise layers: four pixels a lane where rows allow, one, and a launch per group
+# depthwise layers: four pixels a lane where rows allow, one pixel, and the kernels of the other groups; those: every group in one
+# launch, and a launch per group
+@pytest.mark.parametrize("force", ["", "scalar", "gather", "loop"])
 @pytest.mark.parametrize("case", GROUP_CASES)
 def test_conv_with_groups(rt, monkeypatch, force, case):
     """The node's `group`: weights [OC, C / group, KH, KW], every group on its own channels of X and Y where they lie. Integer-
     valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
     N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
     if force:
-        if group != C:
-            pytest.skip("only depthwise layers have a second form")
+        if (group == C) == (force == "loop"):
+            pytest.skip("a form of the other kind of layer")
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
     rng = np.random.default_rng(hash(case[:7]) & 0xffff)
     X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
