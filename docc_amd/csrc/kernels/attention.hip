@@ -1,4 +1,4 @@
-// ml::Attention forward (non-causal), bf16 inputs, head dim 32, 64 or 128, for gfx950:
+// ml::Attention forward (all keys, or causal), bf16 inputs, head dim 32, 64 or 128, for gfx950:
 //   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) V[b,h,j,:]
 // with fp32 scores, softmax statistics and accumulation.
 //
@@ -96,7 +96,10 @@ __device__ __forceinline__ float half_swap(float x, int which) {
     return __builtin_bit_cast(float, which ? sw[1] : sw[0]);
 }
 
-template <bool OUT_BF16, int QT, int HD, int NW>
+// CAUSAL: query i sees the keys j <= i (torch's is_causal: the mask is aligned at the top left whatever SQ and SKV are, so
+// every query sees key 0 and no row is empty). A work-group then walks the blocks up to its last query's only, and the
+// blocks that reach past a wavefront's first query have the scores of the later keys set to -inf.
+template <bool OUT_BF16, int QT, int HD, int NW, bool CAUSAL = false>
 __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, const uint16_t* __restrict__ K,
                                               const uint16_t* __restrict__ V, void* __restrict__ O, int SQ,
                                               int SKV, float scale_log2e) {
@@ -139,7 +142,10 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
             bq[qt][ks] = __builtin_bit_cast(bf16x8, v);
         }
 
-    const int nblocks = (SKV + kBlockKV - 1) / kBlockKV;
+    const int all_blocks = (SKV + kBlockKV - 1) / kBlockKV;
+    const int wg_last_query = qblk * kBlockQ + kBlockQ - 1 < SQ - 1 ? qblk * kBlockQ + kBlockQ - 1 : SQ - 1;
+    const int nblocks = CAUSAL && wg_last_query / kBlockKV + 1 < all_blocks ? wg_last_query / kBlockKV + 1 : all_blocks;
+    const int wave_first_query = qblk * kBlockQ + wave * (32 * QT);
     const int full_blocks = SKV / kBlockKV, keys_left = SKV - full_blocks * kBlockKV;
 
     // K/V copies: a block is 64 * GR granules of 16 bytes per tensor, PASSES per thread. LDS slot s (in copy
@@ -238,6 +244,17 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
 #pragma unroll
                         for (int qt = 0; qt < QT; qt++) s[qt][t][r] = ninf;
                     }
+        }
+        if (CAUSAL && (kb + 1) * kBlockKV - 1 > wave_first_query) {   // the block holds keys past this wavefront's first query
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int key = kb * kBlockKV + 32 * t + Mfma<float>::acc_row(lane, r);
+#pragma unroll
+                    for (int qt = 0; qt < QT; qt++)
+                        if (key > q0 + 32 * qt) s[qt][t][r] = ninf;
+                }
         }
     };
 
@@ -393,6 +410,10 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
     extern "C" __global__ __launch_bounds__(64 * nw) __attribute__((amdgpu_waves_per_eu(waves))) void name(                       \
         const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int SQ, int SKV, float scale_log2e) {                   \
         docc_k::attention_fwd<out_bf16, qt, hd, nw>(Q, K, V, O, SQ, SKV, scale_log2e);                                            \
+    }                                                                                                                             \
+    extern "C" __global__ __launch_bounds__(64 * nw) __attribute__((amdgpu_waves_per_eu(waves))) void name##_causal(              \
+        const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int SQ, int SKV, float scale_log2e) {                   \
+        docc_k::attention_fwd<out_bf16, qt, hd, nw, true>(Q, K, V, O, SQ, SKV, scale_log2e);                                      \
     }
 #define DOCC_ATTENTION_KERNEL(name, out_bf16, qt, waves) DOCC_ATTENTION_KERNEL_D(name, out_bf16, qt, waves, 64, 4)
 

@@ -8,9 +8,10 @@
 
 using namespace docc::rt::rocm;
 
-extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV,
-                                        int64_t D, float scale, const uint16_t* Q, const uint16_t* K,
-                                        const uint16_t* V, void* O, int out_bf16) {
+namespace {
+
+int attention_fused(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, float scale, const uint16_t* Q,
+                    const uint16_t* K, const uint16_t* V, void* O, int out_bf16, bool causal) {
     if (B < 0 || H < 0 || SQ < 0 || SKV < 0 || D < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: negative shape");
     if (D != 32 && D != 64 && D != 128)
         return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: head dim %lld (32, 64 and 128 are built; docc_rocm_attention_bf16_ws takes any)", (long long) D);
@@ -41,7 +42,8 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
     // head dim 128: the large form is eight wavefronts of 32 queries (one work-group per CU), the small one four
     if (D == 128 && !std::getenv("DOCC_ROCM_ATTENTION_Q")) per_group = ((SQ + 255) / 256) * BH >= compute_units() && no_extra_padding ? 256 : 128;
     char kernel[64];
-    std::snprintf(kernel, sizeof(kernel), "docc_attention_bf16_d%d_q%d_%s", (int) D, per_group, out_bf16 ? "bf16out" : "f32out");
+    std::snprintf(kernel, sizeof(kernel), "docc_attention_bf16_d%d_q%d_%s%s", (int) D, per_group, out_bf16 ? "bf16out" : "f32out",
+                  causal ? "_causal" : "");
     const uint32_t threads = D == 128 && per_group == 256 ? 512 : 256;
     // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
     for (int64_t h0 = 0; h0 < BH; h0 += 65535) {
@@ -52,6 +54,14 @@ extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, in
         if (rc) return rc;
     }
     return 0;
+}
+
+} // namespace
+
+extern "C" int docc_rocm_attention_bf16(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV,
+                                        int64_t D, float scale, const uint16_t* Q, const uint16_t* K,
+                                        const uint16_t* V, void* O, int out_bf16) {
+    return attention_fused(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16, false);
 }
 
 // ---- any head dimension, through a caller-provided workspace -----------------------------------
@@ -94,10 +104,12 @@ extern "C" int64_t docc_rocm_attention_bf16_workspace_bytes(int64_t B, int64_t H
     return attention_heads_per_chunk(B * H, per_head) * per_head;
 }
 
-extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
-                                           float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
-                                           int out_bf16, void* workspace, int64_t workspace_bytes) {
-    if (fused_head_dim(D)) return docc_rocm_attention_bf16(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16);
+static int attention_any_head_dim(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D, float scale,
+                                  const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int out_bf16, void* workspace,
+                                  int64_t workspace_bytes, bool causal) {
+    if (fused_head_dim(D)) return attention_fused(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16, causal);
+    if (causal && !widened_head_dim(D))
+        return fail(DOCC_ROCM_ERR_UNSUPPORTED, "attention: the causal form is built for head dims up to 128 (head dim %lld)", (long long) D);
     if (B < 0 || H < 0 || SQ < 0 || SKV < 0 || D < 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: negative shape");
     if (B == 0 || H == 0 || SQ == 0) return 0;
     if (SKV == 0) return fail(DOCC_ROCM_ERR_INVALID_ARGUMENT, "attention: no keys (softmax over an empty axis)");
@@ -129,7 +141,7 @@ extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B,
             for (const auto& part : parts)
                 if (int rc = launch("docc_pad_rows_b16", grid(part.rows * (Dp / 8)), 1, 1, 256, 0, s, part.from, part.to, (long) part.rows, (int) D, (int) Dp))
                     return rc;
-            if (int rc = docc_rocm_attention_bf16(stream, 1, nh, SQ, SKV, Dp, scale, Qp, Kp, Vp, Op, out_bf16)) return rc;
+            if (int rc = attention_fused(stream, 1, nh, SQ, SKV, Dp, scale, Qp, Kp, Vp, Op, out_bf16, causal)) return rc;
             const int64_t rows = nh * SQ;
             int rc = out_bf16 ? launch("docc_unpad_rows_b16", grid(rows * D), 1, 1, 256, 0, s, (const uint16_t*) Op, (uint16_t*) O + h0 * SQ * D, (long) rows,
                                        (int) D, (int) Dp)
@@ -167,4 +179,18 @@ extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B,
         }
     }
     return 0;
+}
+
+extern "C" int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                                           float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
+                                           int out_bf16, void* workspace, int64_t workspace_bytes) {
+    return attention_any_head_dim(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16, workspace, workspace_bytes, false);
+}
+
+// Query i attends to the keys j <= i (torch's is_causal: the mask is aligned at the top left). Head dims up to 128; the
+// workspace is the one of docc_rocm_attention_bf16_workspace_bytes (none for 32, 64 and 128).
+extern "C" int docc_rocm_attention_bf16_causal(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                                               float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
+                                               int out_bf16, void* workspace, int64_t workspace_bytes) {
+    return attention_any_head_dim(stream, B, H, SQ, SKV, D, scale, Q, K, V, O, out_bf16, workspace, workspace_bytes, true);
 }

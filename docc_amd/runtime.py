@@ -94,6 +94,7 @@ _SIGNATURES = {
     "docc_rocm_attention_bf16": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int],
     "docc_rocm_attention_bf16_workspace_bytes": [_i64] * 5 + [_int],
     "docc_rocm_attention_bf16_ws": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int, _vp, _i64],
+    "docc_rocm_attention_bf16_causal": [_vp] + [_i64] * 5 + [_f32, _vp, _vp, _vp, _vp, _int, _vp, _i64],
     "docc_rocm_convert_f32_to_bf16": [_vp, _i64, _vp, _vp],
     "docc_rocm_convert_bf16_to_f32": [_vp, _i64, _vp, _vp],
     "docc_rocm_elementwise_unary": [_vp, ctypes.c_int, ctypes.c_int, _i64, _vp, _vp],
@@ -360,6 +361,12 @@ def attention_bf16_workspace_bytes(B, H, SQ, SKV, D, out_bf16=False) -> int:
 def attention_bf16_ws(B, H, SQ, SKV, D, scale, Q, K, V, O, workspace, workspace_bytes, out_bf16=False, stream=0) -> None:
     """Attention for any head dimension; `workspace` is device memory of attention_bf16_workspace_bytes(...) bytes."""
     call("docc_rocm_attention_bf16_ws", stream, B, H, SQ, SKV, D, scale, Q, K, V, O, 1 if out_bf16 else 0, workspace or None,
+         workspace_bytes)
+
+
+def attention_bf16_causal(B, H, SQ, SKV, D, scale, Q, K, V, O, workspace=0, workspace_bytes=0, out_bf16=False, stream=0) -> None:
+    """Attention in which query i sees the keys j <= i; head dims up to 128 (`workspace` as for attention_bf16_ws)."""
+    call("docc_rocm_attention_bf16_causal", stream, B, H, SQ, SKV, D, scale, Q, K, V, O, 1 if out_bf16 else 0, workspace or None,
          workspace_bytes)
 
 

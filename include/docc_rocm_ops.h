@@ -241,6 +241,17 @@ int docc_rocm_attention_bf16_ws(docc_rocm_stream_t stream, int64_t B, int64_t H,
                                 float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O,
                                 int out_bf16, void* workspace, int64_t workspace_bytes);
 
+/*
+ * The same with a causal mask: query i attends to the keys j <= i (torch's is_causal: the mask is aligned at the top left
+ * whatever SQ and SKV are, so every query sees key 0). No counterpart in the reference (it has no attention node; a model
+ * reaches it as F.scaled_dot_product_attention(..., is_causal=True) through the torch entry, mlir/docc/torch/__init__.py).
+ * Head dims up to 128 (32, 64, 128 fused; others widened as in docc_rocm_attention_bf16_ws, with the workspace
+ * docc_rocm_attention_bf16_workspace_bytes asks for); a work-group walks the key blocks up to its last query only.
+ */
+int docc_rocm_attention_bf16_causal(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ, int64_t SKV, int64_t D,
+                                    float scale, const uint16_t* Q, const uint16_t* K, const uint16_t* V, void* O, int out_bf16,
+                                    void* workspace, int64_t workspace_bytes);
+
 /* fp32 -> bf16 (round to nearest even) and back, on the device; used by the
  * WithTransfers dispatchers when a node's inputs arrive as fp32. */
 int docc_rocm_convert_f32_to_bf16(docc_rocm_stream_t stream, int64_t count, const float* src, uint16_t* dst);

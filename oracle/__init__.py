@@ -236,8 +236,9 @@ def conv2d(X, W, bias=None, stride=(1, 1), pad=(0, 0), dilation=(1, 1), lib=None
     return Y
 
 
-def attention(Q_bits, K_bits, V_bits, scale=None, lib=None) -> np.ndarray:
-    """bf16 bits [B,H,S,D] in, fp32 [B,H,SQ,D] out."""
+def attention(Q_bits, K_bits, V_bits, scale=None, lib=None, causal=False) -> np.ndarray:
+    """bf16 bits [B,H,S,D] in, fp32 [B,H,SQ,D] out. `causal`: query i attends to the keys j <= i (torch's is_causal, the
+    mask aligned at the top left) - stated as what it means: row i is the attention of query i over the first i + 1 keys."""
     lib = lib or load()
     Q = _c(Q_bits, np.uint16)
     K = _c(K_bits, np.uint16)
@@ -246,6 +247,9 @@ def attention(Q_bits, K_bits, V_bits, scale=None, lib=None) -> np.ndarray:
     SKV = K.shape[2]
     if scale is None:
         scale = 1.0 / float(np.sqrt(D))
+    if causal:
+        rows = [attention(Q[:, :, i:i + 1], K[:, :, :min(i + 1, SKV)], V[:, :, :min(i + 1, SKV)], scale, lib) for i in range(SQ)]
+        return np.concatenate(rows, axis=2) if rows else np.empty((B, H, 0, D), np.float32)
     O = np.empty((B, H, SQ, D), np.float32)
     if lib.oracle_attention_bf16(B, H, SQ, SKV, D, scale, _p(Q, _u16p), _p(K, _u16p), _p(V, _u16p), _p(O, _f32p)) != 0:
         raise MemoryError("oracle attention could not allocate its scratch row")

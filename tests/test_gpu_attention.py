@@ -385,3 +385,74 @@ def test_many_heads_with_few_queries(rt, kernel_form):
 
         auto, small, large = timed(None), timed("128"), timed("256")
         assert abs(auto - small) <= 0.25 * small and small < large, (auto, small, large)
+
+
+# ---- causal: query i attends to the keys j <= i ------------------------------------------------------
+
+def run_attention_causal(rt, Qb, Kb, Vb, scale=None, out_bf16=False):
+    B, H, SQ, D = Qb.shape
+    SKV = Kb.shape[2]
+    scale = scale if scale is not None else 1.0 / np.sqrt(D)
+    q, k, v = dev(Qb), dev(Kb), dev(Vb)
+    o = torch.full((B, H, SQ, D), float("nan"), device="cuda", dtype=torch.bfloat16 if out_bf16 else torch.float32)
+    need = rt.attention_bf16_workspace_bytes(B, H, SQ, SKV, D, out_bf16)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device="cuda")
+    rt.attention_bf16_causal(B, H, SQ, SKV, D, scale, q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), ws.data_ptr() if need else 0, need,
+                             out_bf16=out_bf16)
+    torch.cuda.synchronize()
+    return o.float().cpu().numpy()
+
+
+# square, more keys than queries, fewer keys than queries (the later queries see every key), off the block and tile sizes
+@pytest.mark.parametrize("B,H,SQ,SKV", [(1, 2, 96, 96), (1, 1, 1, 1), (2, 2, 256, 256), (1, 2, 130, 200), (1, 1, 300, 65), (1, 3, 513, 513)])
+@pytest.mark.parametrize("out_bf16", [False, True])
+@pytest.mark.parametrize("D", [64, 32, 128, 80])
+def test_causal_attention_matches_oracle(rt, B, H, SQ, SKV, out_bf16, D):
+    g = torch.Generator().manual_seed(B * 7 + H * 5 + SQ * 3 + SKV + D)
+    Q, K, V = (torch.randn(B, H, s, D, generator=g).bfloat16() for s in (SQ, SKV, SKV))
+    O = run_attention_causal(rt, bits(Q), bits(K), bits(V), out_bf16=out_bf16)
+    ref = oracle.attention(bits(Q), bits(K), bits(V), causal=True)
+    assert np.isfinite(O).all()
+    assert rel_err_max(O, ref) <= TOL_BF16
+
+
+def test_causal_attention_closed_forms(rt):
+    """What the mask fixes whatever the values are: row 0 is V's row 0; a later key never reaches an earlier query (a NaN or
+    a huge value in key j and V's row j leaves the rows i < j as they were); with all keys equal row i is the mean of V's
+    rows 0 .. i; and one query against one key is the plain kernel."""
+    g = torch.Generator().manual_seed(5)
+    B, H, S, D = 1, 2, 200, 64
+    Q, K, V = (torch.randn(B, H, S, D, generator=g).bfloat16() for _ in range(3))
+    O = run_attention_causal(rt, bits(Q), bits(K), bits(V))
+    assert np.array_equal(O[:, :, 0], V[:, :, 0].float().numpy())
+    K2, V2 = K.clone(), V.clone()
+    K2[:, :, 150] = float("nan")
+    V2[:, :, 150] = 1e30
+    O2 = run_attention_causal(rt, bits(Q), bits(K2), bits(V2))
+    # bit for bit where no query of the wavefront sees key 150; the earlier queries of its wavefront (128 .. 149) move their
+    # reference point with it, so their probabilities round to bf16 at other points
+    assert np.array_equal(O2[:, :, :128], O[:, :, :128])
+    assert rel_err_max(O2[:, :, 128:150], O[:, :, 128:150]) <= 5e-3
+    assert not np.isfinite(O2[:, :, 150:]).all()
+    Ke = K[:, :, :1].expand(B, H, S, D).contiguous()
+    Oe = run_attention_causal(rt, bits(Q), bits(Ke), bits(V))
+    means = np.cumsum(V.float().numpy().astype(np.float64), axis=2) / np.arange(1, S + 1)[None, None, :, None]
+    assert rel_err_max(Oe, means) <= TOL_BF16
+    one = run_attention_causal(rt, bits(Q[:, :, :1]), bits(K[:, :, :1]), bits(V[:, :, :1]))
+    assert np.array_equal(one, run_attention(rt, bits(Q[:, :, :1]), bits(K[:, :, :1]), bits(V[:, :, :1])))
+
+
+def test_causal_attention_at_size_and_errors(rt):
+    """B2 H4 S2048 D64 against the plain kernel on the keys a query may see (rows 0, 63, 64, 1000 and 2047), and the head
+    dims the causal form is not built for."""
+    g = torch.Generator().manual_seed(9)
+    B, H, S, D = 2, 4, 2048, 64
+    Q, K, V = (torch.randn(B, H, S, D, generator=g).bfloat16() for _ in range(3))
+    O = run_attention_causal(rt, bits(Q), bits(K), bits(V), out_bf16=True)
+    assert np.isfinite(O).all()
+    for i in (0, 63, 64, 1000, 2047):
+        row = oracle.attention(bits(Q[:, :, i:i + 1]), bits(K[:, :, :i + 1]), bits(V[:, :, :i + 1]))
+        assert rel_err_max(O[:, :, i:i + 1], row) <= TOL_BF16, i
+    q = dev(bits(Q[:, :, :8, :1].expand(B, H, 8, 256).contiguous()))
+    with pytest.raises(rt.RocmRuntimeError, match="causal"):
+        rt.attention_bf16_causal(B, H, 8, 8, 256, 0.1, q.data_ptr(), q.data_ptr(), q.data_ptr(), q.data_ptr(), q.data_ptr(), 1 << 20)

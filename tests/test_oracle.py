@@ -134,6 +134,21 @@ def test_softmax_over_any_axes_against_scipy(dt, tol, axes):
 
 # ---- conv -----------------------------------------------------------------------------
 
+def test_causal_attention_against_torch_and_by_hand():
+    """The causal form of the oracle against torch's own (math path, float64, is_causal=True; for SQ != SKV the mask is the
+    lower triangle aligned at the top left) and against a mask added by hand to the scores."""
+    g = torch.Generator().manual_seed(3)
+    bits = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
+    for SQ, SKV in ((17, 17), (9, 30), (40, 12)):
+        Q, K, V = (torch.randn(2, 3, s, 16, generator=g).bfloat16() for s in (SQ, SKV, SKV))
+        got = oracle.attention(bits(Q), bits(K), bits(V), causal=True)
+        ref = torch.nn.functional.scaled_dot_product_attention(Q.double(), K.double(), V.double(), is_causal=True).numpy()
+        assert got.shape == ref.shape and rel(got, ref) <= 1e-5
+        scores = Q.double() @ K.double().transpose(-2, -1) / 4.0
+        scores = scores.masked_fill(torch.arange(SKV)[None, :] > torch.arange(SQ)[:, None], float("-inf"))
+        assert rel(got, (torch.softmax(scores, dim=-1) @ V.double()).numpy()) <= 1e-5
+
+
 def test_conv_golden():
     g = np.load(GOLDEN / "conv_2x3x7x7_k3_p1_bias_f32.npz")
     assert rel(oracle.conv2d(g["X"], g["W"], g["b"], pad=(1, 1)), g["Y"]) <= 1e-6
