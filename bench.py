@@ -505,6 +505,13 @@ def main():
             hbm(f"sgemm_{m_}x{n_}x{k_}_{how}", 4 * (k_ * n_ + m_ * k_ + m_ * n_),
                 lambda i: rt.sgemm(m_, n_, k_, 1.0, y.data_ptr(), k_, x_(i), n_, 0.0, y.data_ptr() + 4 * (1 << 22), n_, stream=stream))
         del xs, y
+        # causal: query i sees the keys j <= i; the flops are those of the pairs it computes on (S (S + 1) / 2 per head)
+        torch.manual_seed(3)
+        Q, K, V = (torch.randn(8, 16, 2048, 64).bfloat16().cuda() for _ in range(3))
+        O = torch.empty(8, 16, 2048, 64, device="cuda", dtype=torch.bfloat16)
+        mfma("attention_b8h16s2048d64_causal", "bf16", 4 * 8 * 16 * (2048 * 2049 // 2) * 64,
+             lambda i: rt.attention_bf16_causal(8, 16, 2048, 2048, 64, 0.125, Q.data_ptr(), K.data_ptr(), V.data_ptr(), O.data_ptr(), out_bf16=True, stream=stream))
+        del Q, K, V, O
         for D in (128, 32):
             torch.manual_seed(3)
             Q, K, V = (torch.randn(8, 16, 2048, D).bfloat16().cuda() for _ in range(3))

@@ -123,7 +123,14 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
     int lid = blockIdx.y * gridDim.x + blockIdx.x;
     if (total % 8 == 0) lid = (lid % 8) * (total / 8) + lid / 8;
     const long bh = lid / nqb;
-    const int qblk = lid % nqb;
+    // Causal: a work-group takes a pair of query blocks, the one with the most keys and the one with the fewest of what is
+    // left (blocks t and T - 1 - t of the T = ceil(SQ / kBlockQ) of a head), one after the other: every work-group then has
+    // the same number of key blocks to walk, and the launch does not end on a few long ones (the grid's x extent is the
+    // number of pairs; the middle block of an odd T is a pair of one)
+    const int tiles_q = (SQ + kBlockQ - 1) / kBlockQ;
+    const int first_of_pair = lid % nqb;
+    // one query block of the head, start to finish
+    auto run_block = [&](const int qblk) {
     const uint16_t* Qh = Q + bh * (long) SQ * kHeadDim;
     const char* Kh = reinterpret_cast<const char*>(K + bh * (long) SKV * kHeadDim);
     const char* Vh = reinterpret_cast<const char*>(V + bh * (long) SKV * kHeadDim);
@@ -246,15 +253,17 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
                     }
         }
         if (CAUSAL && (kb + 1) * kBlockKV - 1 > wave_first_query) {   // the block holds keys past this wavefront's first query
+            // key = 64 kb + 32 t + 8 (r / 4) + 4 g + r % 4 > query  <=>  32 t + 8 (r / 4) + r % 4 > query - 64 kb - 4 g: a constant of
+            // the instruction against one value per lane and query tile, no table of key numbers in registers
 #pragma unroll
-            for (int t = 0; t < 2; t++)
+            for (int qt = 0; qt < QT; qt++) {
+                const int lim = q0 + 32 * qt - kb * kBlockKV - 4 * g;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int key = kb * kBlockKV + 32 * t + Mfma<float>::acc_row(lane, r);
+                for (int t = 0; t < 2; t++)
 #pragma unroll
-                    for (int qt = 0; qt < QT; qt++)
-                        if (key > q0 + 32 * qt) s[qt][t][r] = ninf;
-                }
+                    for (int r = 0; r < 16; r++)
+                        s[qt][t][r] = 32 * t + 8 * (r / 4) + (r % 4) > lim ? ninf : s[qt][t][r];
+            }
         }
     };
 
@@ -400,6 +409,17 @@ __device__ __forceinline__ void attention_fwd(const uint16_t* __restrict__ Q, co
                     }
                 }
             }
+        }
+    }
+    };
+    if constexpr (!CAUSAL) {
+        run_block(first_of_pair);
+    } else {
+#pragma unroll 1
+        for (int pass = 0; pass < 2; pass++) {
+            if (pass == 1 && first_of_pair == tiles_q - 1 - first_of_pair) break;
+            run_block(pass == 0 ? tiles_q - 1 - first_of_pair : first_of_pair);
+            __syncthreads();   // every wave is done with the LDS ring before the next query block's copies land in it
         }
     }
 }

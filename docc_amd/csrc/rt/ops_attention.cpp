@@ -48,7 +48,9 @@ int attention_fused(docc_rocm_stream_t stream, int64_t B, int64_t H, int64_t SQ,
     // gridDim.y numbers the (batch, head) pairs: at most 65535 per launch
     for (int64_t h0 = 0; h0 < BH; h0 += 65535) {
         const int64_t nh = BH - h0 < 65535 ? BH - h0 : 65535;
-        rc = launch(kernel, (uint32_t) ((SQ + per_group - 1) / per_group), (uint32_t) nh, 1, threads, lds, (hipStream_t) stream,
+        // causal: a work-group takes a pair of query blocks (the longest and the shortest left), see the kernel
+        const int64_t query_blocks = (SQ + per_group - 1) / per_group;
+        rc = launch(kernel, (uint32_t) (causal ? (query_blocks + 1) / 2 : query_blocks), (uint32_t) nh, 1, threads, lds, (hipStream_t) stream,
                     Q + h0 * SQ * D, K + h0 * SKV * D, V + h0 * SKV * D, (void*) ((char*) O + h0 * SQ * D * out_bytes), (int) SQ,
                     (int) SKV, scale_log2e);
         if (rc) return rc;

@@ -334,6 +334,24 @@ protected:
         const auto& q = a.shape_q();
         const int out_bf16 = a.output_element() == types::PrimitiveType::BFloat ? 1 : 0;
         int64_t d = 0;
+        if (a.causal()) {
+            // query i attends to the keys j <= i: the entry point for every head dimension it is built for (a workspace for
+            // those that are widened, none for 32, 64 and 128)
+            std::ostringstream cd;
+            cd << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv() << ", " << q[3];
+            s << "{" << std::endl;
+            s.setIndent(s.indent() + 4);
+            s << "const int64_t __ws_bytes = docc_rocm_attention_bf16_workspace_bytes(" << cd.str() << ", " << out_bf16 << ");" << std::endl;
+            s << "void *__ws = nullptr;" << std::endl;
+            s << "if (__ws_bytes > 0) DOCC_ROCM_CHECK(docc_rocm_malloc_async(&__ws, (size_t) __ws_bytes, nullptr));" << std::endl;
+            s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16_causal(nullptr, " << cd.str() << ", (float) (" << a.scale()
+              << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) " << name_of("K") << ", (const uint16_t *) "
+              << name_of("V") << ", (void *) " << name_of("O") << ", " << out_bf16 << ", __ws, __ws_bytes));" << std::endl;
+            s << "if (__ws) DOCC_ROCM_CHECK(docc_rocm_free_async(__ws, nullptr));" << std::endl;
+            s.setIndent(s.indent() - 4);
+            s << "}" << std::endl;
+            return;
+        }
         if (symbolic::is_integer(q[3], &d) && (d == 32 || d == 64 || d == 128)) {   // the head dimensions of the fused kernel
             s << "DOCC_ROCM_CHECK(docc_rocm_attention_bf16(nullptr, " << q[0] << ", " << q[1] << ", " << q[2] << ", " << a.seq_kv()
               << ", " << q[3] << ", (float) (" << a.scale() << "), (const uint16_t *) " << name_of("Q") << ", (const uint16_t *) "
@@ -966,6 +984,9 @@ bool RocmLibNodeMapper::try_map(builder::StructuredSDFGBuilder&, analysis::Analy
         if (!a) return decline("not an Attention node object");
         if (a->element() != P::BFloat) return decline("inputs must be BFloat");
         if (a->output_element() != P::BFloat && a->output_element() != P::Float) return decline("output must be BFloat or Float");
+        int64_t head_dim = 0;
+        if (a->causal() && symbolic::is_integer(a->shape_q()[3], &head_dim) && head_dim > 128)
+            return decline("the causal form is built for head dimensions up to 128");
         // head dimensions 32, 64 and 128 run the fused kernel, any other the GEMM / softmax / GEMM sequence
     } else if (auto* act = dynamic_cast<tensor::ActivationNode*>(&node)) {
         if (act->element() != P::Float && act->element() != P::Double) return decline("element type must be Float or Double");

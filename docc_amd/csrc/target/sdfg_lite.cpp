@@ -535,10 +535,10 @@ Expression MatMulNode::connector_bytes(const std::string& connector) const {
 }
 
 AttentionNode::AttentionNode(std::string implementation_type, std::vector<Expression> shape_q, Expression seq_kv,
-                             std::string scale, types::PrimitiveType element, types::PrimitiveType output_element)
+                             std::string scale, types::PrimitiveType element, types::PrimitiveType output_element, bool causal)
     : LibraryNode(LibraryNodeType_Attention, {"O"}, {"Q", "K", "V"}, false, std::move(implementation_type)),
       shape_q_(std::move(shape_q)), seq_kv_(std::move(seq_kv)), scale_(std::move(scale)), element_(element),
-      output_element_(output_element) {}
+      output_element_(output_element), causal_(causal) {}
 
 void AttentionNode::validate() const {
     if (shape_q_.size() != 4) throw InvalidSDFGException("Attention: Q must be [B, H, S, D]");
@@ -556,13 +556,16 @@ void AttentionNode::to_json(Value& j) const {
     j.set("scale", scale_);
     j.set("element_type", types::primitive_type_to_string(element_));
     j.set("output_type", types::primitive_type_to_string(output_element_));
+    if (causal_) j.set("causal", true);
 }
 
 std::unique_ptr<AttentionNode> AttentionNode::from_json(const Value& j) {
+    const Value* causal = j.find("causal");
     return std::make_unique<AttentionNode>(impl_of(j), exprs_from_json(j.at("shape_q")), j.at("seq_kv").as_expression(),
                                            j.at("scale").as_expression(),
                                            types::primitive_type_from_string(j.at("element_type").as_string()),
-                                           types::primitive_type_from_string(j.at("output_type").as_string()));
+                                           types::primitive_type_from_string(j.at("output_type").as_string()),
+                                           causal ? causal->as_bool() : false);
 }
 
 Expression AttentionNode::connector_bytes(const std::string& connector) const {

@@ -302,12 +302,14 @@ private:
 class AttentionNode : public data_flow::LibraryNode {
 public:
     AttentionNode(std::string implementation_type, std::vector<Expression> shape_q, Expression seq_kv, std::string scale,
-                  types::PrimitiveType element, types::PrimitiveType output_element);
+                  types::PrimitiveType element, types::PrimitiveType output_element, bool causal = false);
     const std::vector<Expression>& shape_q() const { return shape_q_; }
     const Expression& seq_kv() const { return seq_kv_; }
     const std::string& scale() const { return scale_; }
     types::PrimitiveType element() const { return element_; }
     types::PrimitiveType output_element() const { return output_element_; }
+    // query i attends to the keys j <= i (torch's is_causal)
+    bool causal() const { return causal_; }
 
     void validate() const override;
     Expression flop() const override;
@@ -320,6 +322,7 @@ private:
     Expression seq_kv_;
     std::string scale_;
     types::PrimitiveType element_, output_element_;
+    bool causal_ = false;
 };
 
 // Reduce nodes over a set of axes, "X" -> "Y" (reference .../tensor/reduce_node.h, reduce_ops/

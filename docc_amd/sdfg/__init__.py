@@ -549,12 +549,15 @@ class StructuredSDFGBuilder:
                          "shape": [_expr(s) for s in shape], "perm": perm, "element_type": self._element(X).value},
                         [self._operand("X", X)], [self._operand("Y", Y)])
 
-    def add_attention(self, Q: str, K: str, V: str, O: str, shape_q: Sequence[Any], seq_kv: Any, scale: Any) -> None:
-        """ml::Attention: O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]."""
-        self._add_block({"code": "ml::Attention", "implementation_type": "NONE", "side_effect": False,
-                         "shape_q": [_expr(s) for s in shape_q], "seq_kv": _expr(seq_kv), "scale": repr(float(scale)),
-                         "element_type": self._element(Q).value, "output_type": self._element(O).value},
-                        [self._operand("Q", Q), self._operand("K", K), self._operand("V", V)], [self._operand("O", O)])
+    def add_attention(self, Q: str, K: str, V: str, O: str, shape_q: Sequence[Any], seq_kv: Any, scale: Any, causal: bool = False) -> None:
+        """ml::Attention: O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]; `causal`: query i attends to the
+        keys j <= i."""
+        block = {"code": "ml::Attention", "implementation_type": "NONE", "side_effect": False,
+                 "shape_q": [_expr(s) for s in shape_q], "seq_kv": _expr(seq_kv), "scale": repr(float(scale)),
+                 "element_type": self._element(Q).value, "output_type": self._element(O).value}
+        if causal:
+            block["causal"] = True
+        self._add_block(block, [self._operand("Q", Q), self._operand("K", K), self._operand("V", V)], [self._operand("O", O)])
 
     def add_return(self, container: str) -> None:
         self._data["return"] = container

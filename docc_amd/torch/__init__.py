@@ -14,8 +14,8 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
                                               asks for it (`.float()`), else rounded once to bf16 (ml::Cast) as eager torch does
     softmax(x, dim=-1) on fp32             -> ml::Softmax
     F.conv2d / nn.Conv2d                   -> ml::Conv with padding, bias and groups
-    softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v)
-                                           -> ml::Attention (bf16; head dims 32, 64, 128 fused)
+    softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v[, is_causal=True])
+                                           -> ml::Attention (bf16; head dims 32, 64, 128 fused; causal up to 128)
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number; on bf16
                                               tensors in float32 with one rounding to bf16, as eager torch computes them
                                               (likewise the unary operations, reductions, softmax, gelu, silu, layer_norm)
@@ -209,7 +209,7 @@ class _FxLowering:
         self.builder.add_matmul(a.name, b.name, out.name, a.shape, b.shape)
         return out
 
-    def attention(self, node, q: _T, k: _T, v, scale: float, dest):
+    def attention(self, node, q: _T, k: _T, v, scale: float, dest, causal: bool = False):
         torch = self.torch
         if not isinstance(v, _T):
             self.fail(node, "attention values of this form")
@@ -224,7 +224,9 @@ class _FxLowering:
         if k.shape != v.shape or k.shape[:-2] != q.shape[:-2] or k.shape[-1] != q.shape[-1]:
             self.fail(node, "attention with mismatched q/k/v shapes")
         out = self.new_tensor(q.shape, q.dtype, dest)
-        self.builder.add_attention(q.name, k.name, v.name, out.name, shape_q, k.shape[-2], scale)
+        if causal and q.shape[-1] > 128:
+            self.fail(node, "causal attention with a head dimension above 128")
+        self.builder.add_attention(q.name, k.name, v.name, out.name, shape_q, k.shape[-2], scale, causal)
         return out
 
     def softmax(self, node, x, dim, dest):
@@ -730,13 +732,13 @@ class _FxLowering:
         if t is F.scaled_dot_product_attention:
             names = ["query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale"]
             bound = {"attn_mask": None, "dropout_p": 0.0, "is_causal": False, "scale": None, **dict(zip(names, args)), **kwargs}
-            if bound["attn_mask"] is not None or bound["dropout_p"] not in (0, 0.0) or bound["is_causal"]:
-                self.fail(node, "masked, causal or dropout attention")
+            if bound["attn_mask"] is not None or bound["dropout_p"] not in (0, 0.0):
+                self.fail(node, "attention with a mask tensor or dropout")
             q = bound["query"]
             if not isinstance(q, _T):
                 self.fail(node, "attention on this query")
             scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
-            return self.attention(node, q, bound["key"], bound["value"], float(scale), dest)
+            return self.attention(node, q, bound["key"], bound["value"], float(scale), dest, bool(bound["is_causal"]))
         casts = {"float": torch.float32, "double": torch.float64, "bfloat16": torch.bfloat16, "half": torch.float16, "int": torch.int32,
                  "long": torch.int64}
         if method in casts and len(args) == 1:

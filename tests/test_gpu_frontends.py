@@ -806,6 +806,26 @@ def test_torch_grouped_and_depthwise_convolutions():
     assert rel_err_max(out.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
 
 
+def test_torch_causal_attention():
+    """F.scaled_dot_product_attention(..., is_causal=True): ml::Attention with the causal flag, on the fused kernel's causal
+    form (head dim 64) and through the widened operands (head dim 80). Against eager torch's math in float64."""
+    class Net(torch.nn.Module):
+        def forward(self, q, k, v):
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+
+    for D in (64, 80):
+        torch.manual_seed(D)
+        q, k, v = (torch.randn(2, 3, 300, D).bfloat16().cuda() for _ in range(3))
+        program = docc_torch.compile_torch(Net(), (q, k, v), target="rocm")
+        out = program(q, k, v)
+        out = out[0] if isinstance(out, (tuple, list)) else out
+        (node,) = [n for n in program.last_sdfg.library_nodes() if n["code"] == "ml::Attention"]
+        assert node["causal"] is True
+        ref = torch.nn.functional.scaled_dot_product_attention(q.double().cpu(), k.double().cpu(), v.double().cpu(), is_causal=True)
+        assert out.dtype == torch.bfloat16 and out.shape == (2, 3, 300, D)
+        assert rel_err_max(out.float().cpu().numpy(), ref.numpy()) <= 2e-2
+
+
 def test_power_operator_through_both_front_ends():
     """x ** 2, x ** y and np.power lower to ml::Pow (array or scalar operand); torch.pow likewise."""
     @native(target="rocm")

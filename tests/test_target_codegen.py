@@ -1088,3 +1088,31 @@ def test_bf16_tensors_between_float32_nodes_join_the_generated_kernel(tmp_path):
     bad.add_map_nest([("i", 8)], [("a", "A", ["1"])], [("p", "fp_add", ["a", "a"])], [("A", ["1"], "p")])
     with pytest.raises(InvalidSDFGException, match="must be Float or Double"):
         bad.move().validate()
+
+
+def test_causal_attention_binds_its_entry_point(tmp_path):
+    """The Attention node's causal flag serialises and selects docc_rocm_attention_bf16_causal with the workspace the widened
+    head dimensions need; a head dimension above 128 is declined."""
+    b = StructuredSDFGBuilder("ca")
+    for n in ("Q", "K", "V", "O"):
+        b.add_container(n, BF16, True)
+    b.add_attention("Q", "K", "V", "O", [2, 4, 128, 80], 128, 0.1, causal=True)
+    s = b.move()
+    assert StructuredSDFG.parse(s.to_json()).library_nodes()[0]["causal"] is True
+    s.schedule("rocm", options={"offload": "none"})
+    text = re.sub(r"\s+", " ", source_of(s, tmp_path)[0])
+    assert "docc_rocm_attention_bf16_workspace_bytes(2, 4, 128, 128, 80, 1)" in text
+    assert "docc_rocm_attention_bf16_causal(nullptr, 2, 4, 128, 128, 80, (float) (0.1), (const uint16_t *) Q" in text and "__ws, __ws_bytes));" in text
+    b = StructuredSDFGBuilder("cb")
+    for n in ("Q", "K", "V", "O"):
+        b.add_container(n, BF16, True)
+    b.add_attention("Q", "K", "V", "O", [1, 1, 64, 256], 64, 0.1, causal=True)
+    with pytest.raises(InvalidSDFGException, match="causal"):
+        b.move().schedule("rocm")
+    # without the flag nothing changes
+    b = StructuredSDFGBuilder("cc")
+    for n in ("Q", "K", "V", "O"):
+        b.add_container(n, BF16, True)
+    b.add_attention("Q", "K", "V", "O", [1, 1, 64, 64], 64, 0.1)
+    s = b.move()
+    assert "causal" not in s.library_nodes()[0]
