@@ -30,8 +30,8 @@ struct ConvParams {
     // channels of the tensors X and Y lie in: C and OC, or more when the call is one group of a grouped convolution (the
     // images are then XC and YC channels apart)
     int XC, YC;
-    // grouped convolution in one launch: blockIdx.z is the group, whose operands lie these many elements further on (0 each
-    // when the launch is one convolution)
+    // grouped convolution in one launch (the entry points with the suffix _g): blockIdx.z is the group, whose operands lie
+    // these many elements further on. The kernels of a single convolution do not look at them (their registers are full).
     long GX, GW, GB, GY;
 };
 
@@ -201,6 +201,10 @@ struct ConvGatherKernel {
 
 #define DOCC_CONV_GATHER(BM, BN, BK, WM, WN, AL, ALTAG)                                                         \
     extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_conv2d_f32_gather_##BM##x##BN##_##ALTAG(     \
+        docc_k::ConvParams p) {                                                                                 \
+        docc_k::ConvGatherKernel<BM, BN, BK, WM, WN, AL>::run(p);                                               \
+    }                                                                                                           \
+    extern "C" __global__ __launch_bounds__(64 * WM * WN) void docc_conv2d_f32_gather_##BM##x##BN##_##ALTAG##_g( \
         docc_k::ConvParams p) {                                                                                 \
         docc_k::conv_select_group(p);                                                                           \
         docc_k::ConvGatherKernel<BM, BN, BK, WM, WN, AL>::run(p);                                               \
@@ -822,62 +826,98 @@ struct ConvHaloKernel {
 } // namespace docc_k
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<1, 1>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 4>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, false, false, 4>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 2>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, false, false, 2>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 4>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<1, 1, false, false, 4>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 2>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<1, 1, false, false, 2>::run(p, TH);
 }
 
 // several whole images per work-group (images of a few pixels)
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 4, true>::run(p, TH, G);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t4m_g(docc_k::ConvParams p, int TH, int G) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, false, false, 4, true>::run(p, TH, G);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<3, 3, false, false, 2, true>::run(p, TH, G);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_t2m_g(docc_k::ConvParams p, int TH, int G) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, false, false, 2, true>::run(p, TH, G);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 4, true>::run(p, TH, G);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t4m_g(docc_k::ConvParams p, int TH, int G) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<1, 1, false, false, 4, true>::run(p, TH, G);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2m(docc_k::ConvParams p, int TH, int G) {
+    docc_k::ConvHaloKernel<1, 1, false, false, 2, true>::run(p, TH, G);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_1x1_t2m_g(docc_k::ConvParams p, int TH, int G) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<1, 1, false, false, 2, true>::run(p, TH, G);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, true>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, true>::run(p, TH);
 }
 
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split16(docc_k::ConvParams p, int TH) {
+    docc_k::ConvHaloKernel<3, 3, true, true>::run(p, TH);
+}
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_f32_halo_3x3_split16_g(docc_k::ConvParams p, int TH) {
     docc_k::conv_select_group(p);
     docc_k::ConvHaloKernel<3, 3, true, true>::run(p, TH);
 }

@@ -314,14 +314,15 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
         if (plan.images > 1 && plan.cost > 0.0 && PS <= 3 * 256 && 3 * stage * 4 <= 160 * 1024 && OC * C * KH * KW < (int64_t(1) << 29) &&
             plan.images * x_channels * H * W < (int64_t(1) << 29) && (OC + 63) / 64 <= 65535) {
             char name[64];
-            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s_t%dm", KH == 3 ? "3x3" : "1x1", plan.tiles);
+            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s_t%dm%s", KH == 3 ? "3x3" : "1x1", plan.tiles, groups > 1 ? "_g" : "");
             return launch(name, (uint32_t) ((N + plan.images - 1) / plan.images), (uint32_t) ((OC + 63) / 64), gz, 256, (uint32_t) (3 * stage * 4),
                           (hipStream_t) stream, p, (int) TH, (int) plan.images);
         }
         if (plan.images == 1 && plan.cost > 0.0 && halo_strip_fits(TH, OW, KH, KW, stride_h, stride_w) && OC * C * KH * KW < (int64_t(1) << 29) && C * H * W < (int64_t(1) << 29) && N * strips < lim && (OC + 63) / 64 <= 65535) {
             char name[64];
-            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s", KH == 3 ? "3x3" : "1x1",
-                          plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "");
+            std::snprintf(name, sizeof(name), "docc_conv2d_f32_halo_%s%s%s", KH == 3 ? "3x3" : "1x1",
+                          plan.tiles == 4 ? "_t4" : plan.tiles == 2 ? "_t2" : plan.split ? (plan.narrow ? "_split16" : "_split") : "",
+                          groups > 1 ? "_g" : "");
             return launch(name, (uint32_t) (N * strips), (uint32_t) ((OC + 63) / 64), gz, 256, (uint32_t) (3 * stage * 4), (hipStream_t) stream, p, (int) TH);
         }
     }
@@ -332,7 +333,9 @@ static int conv2d_run(docc_rocm_stream_t stream, int64_t N, int64_t C, int64_t H
     const bool aligned = ((uintptr_t) Wt % 16 == 0) && (K % 4 == 0);
     // LDS: 2 x (A tile [BM][BK+4] + B tile [BK][BN+8]) floats + 2 x BK table entries of 16 bytes
     const uint32_t lds = 2 * (BM * (BK + 4) + BK * (BN + 8)) * 4 + 2 * BK * 16;
-    return launch(aligned ? "docc_conv2d_f32_gather_64x128_a" : "docc_conv2d_f32_gather_64x128_u", (uint32_t) tiles, 1,
+    return launch(groups > 1 ? (aligned ? "docc_conv2d_f32_gather_64x128_a_g" : "docc_conv2d_f32_gather_64x128_u_g")
+                             : (aligned ? "docc_conv2d_f32_gather_64x128_a" : "docc_conv2d_f32_gather_64x128_u"),
+                  (uint32_t) tiles, 1,
                   gz, 256, lds, (hipStream_t) stream, p);
 }
 
