@@ -298,7 +298,7 @@ private:
 
 // Added by the rocm target; the reference's node set has no attention
 // (sdfg/include/sdfg/data_flow/library_nodes/math/math.h:5-42).
-// O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D], non-causal.
+// O = softmax(scale * Q K^T) V, Q [B,H,SQ,D], K/V [B,H,SKV,D]; with the `causal` flag query i attends to the keys j <= i.
 class AttentionNode : public data_flow::LibraryNode {
 public:
     AttentionNode(std::string implementation_type, std::vector<Expression> shape_q, Expression seq_kv, std::string scale,

@@ -218,7 +218,8 @@ int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N, int64_t C
  * ml::Attention (a node the rocm target adds; the reference has none):
  *   O[b,h,i,:] = sum_j softmax_j(scale * <Q[b,h,i,:], K[b,h,j,:]>) * V[b,h,j,:]
  * Q [B,H,SQ,D], K and V [B,H,SKV,D], all contiguous bf16 (raw bits); fp32
- * scores, softmax and accumulation; non-causal. O is [B,H,SQ,D], fp32 when
+ * scores, softmax and accumulation; every query attends to every key (docc_rocm_attention_bf16_causal below is the
+ * causal form). O is [B,H,SQ,D], fp32 when
  * out_bf16 == 0 and bf16 (round-to-nearest-even) otherwise. D must be 32, 64 or 128
  * (docc_rocm_attention_bf16_ws takes any D).
  */
