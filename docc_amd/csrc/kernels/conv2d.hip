@@ -1026,3 +1026,81 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_
     }
     __builtin_nontemporal_store(acc, reinterpret_cast<v4*>(p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + (long) oh * p.OW + ow));
 }
+
+// Groups of a few channels (a ResNeXt layer: 32 groups of 4 or 8 channels in, as many out): per output element the layer does
+// C/group * 9 multiply-adds against eight bytes moved, so it is bound by HBM like the depthwise one, and a 64-row MFMA tile
+// would hold 4 or 8 real output channels. 3x3, stride 1, no dilation, one column of padding, rows of whole aligned quads (as
+// the depthwise kernel above): a lane takes four output pixels of OGT output channels of one group, every input row segment it
+// loads (one 128-bit load and its two neighbours) serves the four pixels, the three taps of the row and the OGT channels; the
+// group's filters wait in LDS and are read by all lanes at once. Work-group = (image, group, OGT channels of it, 256 quads).
+namespace docc_k {
+template <int OGT>
+__device__ __forceinline__ void conv_small_groups_3x3_v4(const ConvParams& p, int cg, int og) {
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_sg_lds[];
+    float* wl = reinterpret_cast<float*>(conv_sg_lds);   // [OGT][cg][9]
+    const int Q = p.OH * (p.OW / 4);
+    const int blocks_per_plane = (Q + 255) / 256;
+    const int chunks = og / OGT;                           // OGT divides og
+    long b = blockIdx.x;
+    const int qblock = (int) (b % blocks_per_plane);
+    b /= blocks_per_plane;
+    const int chunk = (int) (b % chunks);
+    b /= chunks;
+    const int groups = p.OC / og;
+    const int grp = (int) (b % groups), n = (int) (b / groups);
+    const int oc0 = grp * og + chunk * OGT;
+    for (int i = threadIdx.x; i < OGT * cg * 9; i += 256) wl[i] = p.Wt[(long) oc0 * cg * 9 + i];
+    __syncthreads();
+    const int quad = qblock * 256 + threadIdx.x;
+    if (quad >= Q) return;
+    const int oh = quad / (p.OW / 4), ow = (quad % (p.OW / 4)) * 4;
+    v4 acc[OGT];
+#pragma unroll
+    for (int o = 0; o < OGT; o++) acc[o] = v4{0.f, 0.f, 0.f, 0.f};
+    const float* x = p.X + ((long) n * p.XC + (long) grp * cg) * p.H * p.W;
+    for (int ci = 0; ci < cg; ci++) {
+        const float* plane = x + (long) ci * p.H * p.W;
+#pragma unroll
+        for (int kh = 0; kh < 3; kh++) {
+            const int ih = oh - p.pad_h + kh;
+            v4 mid = {0.f, 0.f, 0.f, 0.f};
+            float left = 0.f, right = 0.f;
+            if ((unsigned) ih < (unsigned) p.H) {
+                const float* row = plane + (long) ih * p.W;
+                mid = *reinterpret_cast<const v4*>(row + ow);
+                if (ow > 0) left = row[ow - 1];
+                if (ow + 4 < p.W) right = row[ow + 4];
+            }
+            const float in[6] = {left, mid[0], mid[1], mid[2], mid[3], right};
+#pragma unroll
+            for (int kw = 0; kw < 3; kw++)
+#pragma unroll
+                for (int o = 0; o < OGT; o++) {
+                    const float wt = wl[(o * cg + ci) * 9 + kh * 3 + kw];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[o][e] = __builtin_fmaf(in[e + kw], wt, acc[o][e]);
+                }
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < OGT; o++) {
+        const int oc = oc0 + o;
+        if (p.bias) {
+            const float bv = p.bias[oc];
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[o][e] += bv;
+        }
+        __builtin_nontemporal_store(acc[o], reinterpret_cast<v4*>(p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + (long) oh * p.OW + ow));
+    }
+}
+}  // namespace docc_k
+
+#define DOCC_CONV_SMALL_GROUPS(OGT)                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void docc_conv2d_small_groups_f32_3x3_v4_o##OGT(docc_k::ConvParams p, int cg, int og) {     \
+        docc_k::conv_small_groups_3x3_v4<OGT>(p, cg, og);                                                                                  \
+    }
+DOCC_CONV_SMALL_GROUPS(1)
+DOCC_CONV_SMALL_GROUPS(2)
+DOCC_CONV_SMALL_GROUPS(4)
+DOCC_CONV_SMALL_GROUPS(8)

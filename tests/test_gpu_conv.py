@@ -273,6 +273,10 @@ GROUP_CASES = [
     (1, 6, 9, 20, 12, 2, 4, (1, 3), (0, 3, 1, 0), (2, 1), 6, True),        # depthwise, a 2x4 filter with dilation and a stride of 3
     (2, 40, 28, 28, 40, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 40, True),     # depthwise on planes of more than one work-group
     (3, 16, 9, 12, 32, 3, 3, (1, 1), (0, 1, 2, 1), (1, 1), 16, True),      # rows of three quads, no rows above, two below
+    (2, 32, 12, 16, 32, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 8, True),      # eight groups of four channels (a ResNeXt layer in small)
+    (2, 16, 9, 8, 48, 3, 3, (1, 1), (2, 1, 0, 1), (1, 1), 2, False),       # two groups of eight channels in, 24 out each
+    (1, 12, 10, 12, 18, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 6, True),      # two channels in, three out per group: one output channel a lane
+    (2, 10, 11, 20, 20, 3, 3, (1, 1), (1, 1, 1, 1), (1, 1), 2, True),      # five channels in, ten out per group: pairs of output channels
 ]
 
 
@@ -285,7 +289,7 @@ def test_conv_with_groups(rt, monkeypatch, force, case):
     valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
     N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
     if force:
-        if (group == C) == (force == "loop"):
+        if (group == C) == (force == "loop") or (force == "scalar" and group != C):
             pytest.skip("a form of the other kind of layer")
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
     rng = np.random.default_rng(hash(case[:7]) & 0xffff)
