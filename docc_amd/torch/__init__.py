@@ -15,7 +15,8 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     softmax(x, dim=-1) on fp32             -> ml::Softmax
     F.conv2d / nn.Conv2d                   -> ml::Conv with padding, bias and groups
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v[, is_causal=True])
-                                           -> ml::Attention (bf16; head dims 32, 64, 128 fused; causal up to 128)
+                                           -> ml::Attention (bf16; head dims 32, 64, 128 fused; causal up to 128);
+                                              float32 / float64 tensors: ml::Transpose, ml::MatMul, ml::Softmax, ml::MatMul
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number; on bf16
                                               tensors in float32 with one rounding to bf16, as eager torch computes them
                                               (likewise the unary operations, reductions, softmax, gelu, silu, layer_norm)
@@ -738,6 +739,16 @@ class _FxLowering:
             if not isinstance(q, _T):
                 self.fail(node, "attention on this query")
             scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
+            if q.dtype in (torch.float32, torch.float64):
+                # no fused kernel in these types: the nodes the expression is made of (batched products around a softmax)
+                k, v = self.tensor(node, bound["key"]), self.tensor(node, bound["value"])
+                if bound["is_causal"]:
+                    self.fail(node, "causal attention on float32 / float64 tensors")
+                if not isinstance(k, _T) or not isinstance(v, _T) or len(q.shape) < 3 or k.dtype != q.dtype or v.dtype != q.dtype:
+                    self.fail(node, "attention on these operands")
+                scores = self.product(node, q, self.tensor(node, _Transposed(k)), False, False, q.dtype, None)
+                probs = self.softmax(node, self.elementwise(node, "mul", scores, float(scale), None), len(q.shape) - 1, None)
+                return self.product(node, probs, v, False, False, q.dtype, dest)
             return self.attention(node, q, bound["key"], bound["value"], float(scale), dest, bool(bound["is_causal"]))
         casts = {"float": torch.float32, "double": torch.float64, "bfloat16": torch.bfloat16, "half": torch.float16, "int": torch.int32,
                  "long": torch.int64}

@@ -806,6 +806,23 @@ def test_torch_grouped_and_depthwise_convolutions():
     assert rel_err_max(out.cpu().numpy(), ref.cpu().numpy()) <= 1e-5
 
 
+def test_torch_attention_on_float32_tensors():
+    """F.scaled_dot_product_attention on float32 tensors has no fused kernel: it runs as the nodes it is made of."""
+    class Net(torch.nn.Module):
+        def forward(self, q, k, v):
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v)
+
+    torch.manual_seed(17)
+    q, k, v = torch.randn(2, 3, 70, 24).cuda(), torch.randn(2, 3, 90, 24).cuda(), torch.randn(2, 3, 90, 24).cuda()
+    program = docc_torch.compile_torch(Net(), (q, k, v), target="rocm")
+    out = program(q, k, v)
+    out = out[0] if isinstance(out, (tuple, list)) else out
+    codes = [n["code"] for n in program.last_sdfg.library_nodes()]
+    assert "ml::Attention" not in codes and "ml::Softmax" in codes and codes.count("ml::MatMul") == 2
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double().cpu(), k.double().cpu(), v.double().cpu())
+    assert out.dtype == torch.float32 and rel_err_max(out.cpu().numpy(), ref.numpy()) <= 1e-5
+
+
 def test_torch_causal_attention():
     """F.scaled_dot_product_attention(..., is_causal=True): ml::Attention with the causal flag, on the fused kernel's causal
     form (head dim 64) and through the widened operands (head dim 80). Against eager torch's math in float64."""
