@@ -16,7 +16,8 @@ this front end lowers the FX graph directly and covers what the rocm kernels imp
     F.conv2d / nn.Conv2d                   -> ml::Conv with padding, bias and groups
     softmax(q @ k.transpose(-2, -1) * c, dim=-1) @ v   and   F.scaled_dot_product_attention(q, k, v[, is_causal=True])
                                            -> ml::Attention (bf16; head dims 32, 64, 128 fused; causal up to 128);
-                                              float32 / float64 tensors: ml::Transpose, ml::MatMul, ml::Softmax, ml::MatMul
+                                              float32 / float64 tensors, or an additive attn_mask: ml::Transpose, ml::MatMul,
+                                              ml::Softmax, ml::MatMul
     + - * / ** torch.maximum / torch.minimum on fp32/fp64 tensors (broadcasting) or a tensor and a number; on bf16
                                               tensors in float32 with one rounding to bf16, as eager torch computes them
                                               (likewise the unary operations, reductions, softmax, gelu, silu, layer_norm)
@@ -229,6 +230,30 @@ class _FxLowering:
             self.fail(node, "causal attention with a head dimension above 128")
         self.builder.add_attention(q.name, k.name, v.name, out.name, shape_q, k.shape[-2], scale, causal)
         return out
+
+    def attention_unfused(self, node, q: _T, k, v, scale: float, mask, dest):
+        """softmax(scale * q k^T + mask) v as batched products around a softmax: float32 / float64 tensors, and bf16 tensors
+        with an additive mask (scores, mask and softmax in float32, the probabilities rounded to bf16 for the second product,
+        as eager torch's math path does)."""
+        torch = self.torch
+        k, v = self.tensor(node, k), self.tensor(node, v)
+        if not isinstance(k, _T) or not isinstance(v, _T) or len(q.shape) < 3 or k.dtype != q.dtype or v.dtype != q.dtype:
+            self.fail(node, "attention on these operands")
+        if q.dtype not in (torch.float32, torch.float64, torch.bfloat16):
+            self.fail(node, "attention on tensors other than float32 / float64 / bfloat16")
+        bf16 = q.dtype == torch.bfloat16
+        wide = torch.float32 if bf16 else q.dtype
+        scores = self.product(node, q, self.tensor(node, _Transposed(k)), False, False, wide, None)
+        scores = self.elementwise(node, "mul", scores, float(scale), None)
+        if mask is not None:
+            mask = self.widened(node, self.tensor(node, mask))
+            if not isinstance(mask, _T) or mask.dtype != wide:
+                self.fail(node, "a mask that is not a floating-point tensor of the scores' type (a boolean mask: add -inf where it is False)")
+            scores = self.elementwise(node, "add", scores, mask, None)
+        probs = self.softmax(node, scores, len(q.shape) - 1, None)
+        if not bf16:
+            return self.product(node, probs, v, False, False, q.dtype, dest)
+        return self.narrowed(node, self.product(node, self.narrowed(node, probs, None), v, False, False, wide, None), dest)
 
     def softmax(self, node, x, dim, dest):
         if isinstance(x, _Scores):
@@ -733,22 +758,18 @@ class _FxLowering:
         if t is F.scaled_dot_product_attention:
             names = ["query", "key", "value", "attn_mask", "dropout_p", "is_causal", "scale"]
             bound = {"attn_mask": None, "dropout_p": 0.0, "is_causal": False, "scale": None, **dict(zip(names, args)), **kwargs}
-            if bound["attn_mask"] is not None or bound["dropout_p"] not in (0, 0.0):
-                self.fail(node, "attention with a mask tensor or dropout")
+            if bound["dropout_p"] not in (0, 0.0):
+                self.fail(node, "attention with dropout")
             q = bound["query"]
             if not isinstance(q, _T):
                 self.fail(node, "attention on this query")
             scale = bound["scale"] if bound["scale"] is not None else 1.0 / math.sqrt(q.shape[-1])
-            if q.dtype in (torch.float32, torch.float64):
-                # no fused kernel in these types: the nodes the expression is made of (batched products around a softmax)
-                k, v = self.tensor(node, bound["key"]), self.tensor(node, bound["value"])
+            mask = bound["attn_mask"]
+            if mask is not None or q.dtype in (torch.float32, torch.float64):
+                # no fused kernel for a mask tensor or in these types: the nodes the expression is made of
                 if bound["is_causal"]:
-                    self.fail(node, "causal attention on float32 / float64 tensors")
-                if not isinstance(k, _T) or not isinstance(v, _T) or len(q.shape) < 3 or k.dtype != q.dtype or v.dtype != q.dtype:
-                    self.fail(node, "attention on these operands")
-                scores = self.product(node, q, self.tensor(node, _Transposed(k)), False, False, q.dtype, None)
-                probs = self.softmax(node, self.elementwise(node, "mul", scores, float(scale), None), len(q.shape) - 1, None)
-                return self.product(node, probs, v, False, False, q.dtype, dest)
+                    self.fail(node, "causal attention on float32 / float64 tensors, or together with a mask tensor,")
+                return self.attention_unfused(node, q, bound["key"], bound["value"], float(scale), mask, dest)
             return self.attention(node, q, bound["key"], bound["value"], float(scale), dest, bool(bound["is_causal"]))
         casts = {"float": torch.float32, "double": torch.float64, "bfloat16": torch.bfloat16, "half": torch.float16, "int": torch.int32,
                  "long": torch.int64}

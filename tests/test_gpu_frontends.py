@@ -823,6 +823,28 @@ def test_torch_attention_on_float32_tensors():
     assert out.dtype == torch.float32 and rel_err_max(out.cpu().numpy(), ref.numpy()) <= 1e-5
 
 
+def test_torch_attention_with_an_additive_mask():
+    """attn_mask as a float tensor: bf16 q, k, v with a [SQ, SK] mask that closes the later keys and adds a bias, and float32
+    q, k, v with a mask per batch entry. No fused kernel: products around a softmax, against eager's math in float64."""
+    class Net(torch.nn.Module):
+        def forward(self, q, k, v, mask):
+            return torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+
+    torch.manual_seed(23)
+    SQ, SK, D = 70, 90, 32
+    for dtype, mask_shape, tol in ((torch.bfloat16, (SQ, SK), 2e-2), (torch.float32, (2, 1, SQ, SK), 1e-5)):
+        q, k, v = torch.randn(2, 3, SQ, D).to(dtype).cuda(), torch.randn(2, 3, SK, D).to(dtype).cuda(), torch.randn(2, 3, SK, D).to(dtype).cuda()
+        mask = torch.randn(mask_shape) * 0.5
+        mask.masked_fill_(torch.arange(SK)[None, :] > torch.arange(SQ)[:, None] + 20, float("-inf"))
+        mask = mask.cuda()
+        program = docc_torch.compile_torch(Net(), (q, k, v, mask), target="rocm")
+        out = program(q, k, v, mask)
+        out = out[0] if isinstance(out, (tuple, list)) else out
+        assert "ml::Attention" not in [n["code"] for n in program.last_sdfg.library_nodes()]
+        ref = torch.nn.functional.scaled_dot_product_attention(q.double().cpu(), k.double().cpu(), v.double().cpu(), attn_mask=mask.double().cpu())
+        assert out.dtype == dtype and rel_err_max(out.float().cpu().numpy(), ref.numpy()) <= tol, dtype
+
+
 def test_torch_causal_attention():
     """F.scaled_dot_product_attention(..., is_causal=True): ml::Attention with the causal flag, on the fused kernel's causal
     form (head dim 64) and through the widened operands (head dim 80). Against eager torch's math in float64."""
