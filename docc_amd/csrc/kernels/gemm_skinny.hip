@@ -328,6 +328,130 @@ __device__ __forceinline__ void gemm_skinny_bf16_nt(const uint16_t* __restrict__
         }
 }
 
+// fp64, B stored [k][n], up to 16 rows: the same scheme on v_mfma_f64_16x16x4_f64 (a lane holds one k of its row of A and of
+// its column of B; 512 bytes of B per instruction and 64 cycles: 19.6 TB/s at the device's fp64 rate, so the product is bound by
+// reading B). A work-group owns 64 columns of one part of K; a lane's 128-bit load of B is two adjacent columns, K advances in
+// chunks of 16 (four consecutive k per lane group).
+template <int NW, int NBUF>
+__device__ __forceinline__ void gemm_skinny_f64_nn(const double* __restrict__ A, long lda, const double* __restrict__ B, long ldb,
+                                                   double* __restrict__ P, long ldp, long m, long n, long k, long kpart, double alpha,
+                                                   double beta, int direct) {
+    typedef double d2 __attribute__((ext_vector_type(2)));
+    constexpr int CH = 16, KL = 4, SETS = 2, NJ = 4;   // 64 columns: two loads of two columns a lane and k
+    constexpr int SLOT = NJ / 2 * 4 * 64;              // 128-bit words of a wavefront's block of sums
+    extern __shared__ __attribute__((aligned(16))) unsigned char skinny_lds[];
+    d2* lds = reinterpret_cast<d2*>(skinny_lds);
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int c = lane & 15, g = lane >> 4;
+    const long n0 = (long) blockIdx.x * 64;
+    const long part = blockIdx.y;
+    const long kw = kpart / NW;   // a multiple of CH
+    const long k_begin = part * kpart + wave * kw;
+    long k_end = k_begin + kw;
+    if (k_end > k) k_end = k;
+
+    f64x4 acc[NJ];
+#pragma unroll
+    for (int j = 0; j < NJ; j++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[j][r] = 0.0;
+
+    const unsigned b_lane = (unsigned) (KL * g * ldb + 2 * c), a_lane = (unsigned) (c * lda + KL * g);
+    const d2 zero2 = {0.0, 0.0};
+    auto load_b = [&](long kb, d2 (&bv)[KL * SETS]) {
+        const long kl = kb + KL * g;
+        const bool whole = kb + CH <= k_end;
+#pragma unroll
+        for (int i = 0; i < KL; i++)
+#pragma unroll
+            for (int s = 0; s < SETS; s++) {
+                const bool ok = n0 + 32 * s + 2 * c < n;
+                const double* base = B + (kb + i) * ldb + n0 + 32 * s;
+                bv[i * SETS + s] = ok && (whole || kl + i < k_end) ? __builtin_nontemporal_load(reinterpret_cast<const d2*>(base + b_lane)) : zero2;
+            }
+    };
+    auto load_a = [&](long kb, d2 (&av)[KL / 2]) {
+        const long kl = kb + KL * g;
+        const bool whole = kb + CH <= k_end;
+#pragma unroll
+        for (int q = 0; q < KL / 2; q++)
+            av[q] = c < m && (whole || kl + 2 * q < k_end) ? *reinterpret_cast<const d2*>(A + kb + a_lane + 2 * q) : zero2;
+    };
+    auto products = [&](const d2 (&av)[KL / 2], const d2 (&bv)[KL * SETS]) {
+#pragma unroll
+        for (int i = 0; i < KL; i++)
+#pragma unroll
+            for (int j = 0; j < NJ; j++)
+                acc[j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i / 2][i % 2], bv[i * SETS + j / 2][j % 2], acc[j], 0, 0, 0);
+    };
+    {
+        d2 bq[NBUF][KL * SETS], aq[NBUF][KL / 2];
+#pragma unroll
+        for (int u = 0; u < NBUF - 1; u++) {
+            load_b(k_begin + u * CH, bq[u]);   // past k_end: zeros, no access
+            load_a(k_begin + u * CH, aq[u]);
+        }
+        for (long kb = k_begin; kb < k_end; kb += NBUF * CH) {
+#pragma unroll
+            for (int u = 0; u < NBUF; u++) {
+                const long kc = kb + u * CH;
+                if (kc < k_end) {
+                    load_b(kc + (NBUF - 1) * CH, bq[(u + NBUF - 1) % NBUF]);
+                    load_a(kc + (NBUF - 1) * CH, aq[(u + NBUF - 1) % NBUF]);
+                    products(aq[u], bq[u]);
+                }
+            }
+        }
+    }
+    // the wavefronts' blocks meet in LDS; a word holds register r of the blocks 2 s and 2 s + 1: two adjacent columns
+#pragma unroll
+    for (int half = NW / 2; half >= 1; half /= 2) {
+        if (wave >= half && wave < 2 * half) {
+            d2* slot = lds + (long) (wave - half) * SLOT;
+#pragma unroll
+            for (int s = 0; s < SETS; s++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) slot[(s * 4 + r) * 64 + lane] = d2{acc[2 * s][r], acc[2 * s + 1][r]};
+        }
+        __syncthreads();
+        if (wave < half) {
+            const d2* slot = lds + (long) wave * SLOT;
+#pragma unroll
+            for (int s = 0; s < SETS; s++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const d2 v = slot[(s * 4 + r) * 64 + lane];
+                    acc[2 * s][r] += v[0];
+                    acc[2 * s + 1][r] += v[1];
+                }
+        }
+        __syncthreads();
+    }
+    if (wave != 0) return;
+    double* out = direct ? P : P + part * m * ldp;
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const long row = 4 * r + g;   // register r of a 16 x 16 block of fp64 sums: row 4 r + lane / 16, column lane % 16
+        if (row >= m) continue;
+#pragma unroll
+        for (int s = 0; s < SETS; s++) {
+            const long col = n0 + 32 * s + 2 * c;
+            if (col >= n) continue;
+            d2* o = reinterpret_cast<d2*>(out + row * ldp + col);
+            d2 v = {acc[2 * s][r], acc[2 * s + 1][r]};
+            if (direct) {
+                if (beta == 0.0) {
+                    v = alpha * v;
+                } else {
+                    const d2 old = *o;
+                    v = alpha * v + beta * old;
+                }
+            }
+            *o = v;
+        }
+    }
+}
+
 }  // namespace docc_k
 
 #define DOCC_GEMM_SKINNY(MT, TB, TBN, NW, CH, NBUF)                                                                                             \
@@ -352,3 +476,9 @@ DOCC_GEMM_SKINNY(16, true, t, 4, 32, 2)
 
 DOCC_GEMM_SKINNY_BF16(1, 4, 2)
 DOCC_GEMM_SKINNY_BF16(2, 4, 2)
+
+extern "C" __global__ __launch_bounds__(256) void docc_dgemm_skinny16_nn_w4_b2(const double* A, long lda, const double* B, long ldb, double* P,
+                                                                              long ldp, long m, long n, long k, long kpart, double alpha,
+                                                                              double beta, int direct) {
+    docc_k::gemm_skinny_f64_nn<4, 2>(A, lda, B, ldb, P, ldp, m, n, k, kpart, alpha, beta, direct);
+}

@@ -259,7 +259,10 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
     // bf16 with B stored [n][k] (a layer's weights): 3 to 32 rows (two rows are faster as matrix-vector products, 64 on the tiles)
     const bool skinny_bf16 = sizeof(T) == 2 && skinny_base && tb && m >= 3 && m <= 32 && (n * k >= (int64_t(8) << 20) || skinny_any_size) &&
                              lda % 8 == 0 && ldb % 8 == 0 && k % 8 == 0;
-    const bool skinny = skinny_f32 || skinny_bf16;
+    // fp64 with B stored [k][n]: 5 to 16 rows (up to four are matrix-vector products, above 16 the tiles)
+    const bool skinny_f64 = sizeof(T) == 8 && skinny_base && !tb && m >= 5 && m <= 16 && (n * k >= (int64_t(4) << 20) || skinny_any_size) &&
+                            lda % 2 == 0 && ldb % 2 == 0 && k % 2 == 0 && n % 2 == 0;
+    const bool skinny = skinny_f32 || skinny_bf16 || skinny_f64;
     if ((m <= 8 || n <= 8) && !skinny && batch == 1 && (!epilogue || ldc == n)) {
         rc = gemv_launch<T, S>(prefix, s, ta, tb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc);
         if (rc == 0 && epilogue) {
@@ -290,7 +293,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
             // fp32: 16 or 32 rows per MFMA, 128 columns per work-group; bf16: 1, 2 or 4 blocks of 16 rows, 64 columns
             const int nw = 4, nbuf = 2;
             const int ch = skinny_bf16 ? 64 : tb ? 32 : 16, mt = skinny_bf16 ? (m <= 16 ? 1 : 2) : m <= 16 ? 16 : 32;
-            const int64_t col_blocks = skinny_bf16 ? (n + 63) / 64 : (n + 127) / 128;
+            const int64_t col_blocks = skinny_bf16 || skinny_f64 ? (n + 63) / 64 : (n + 127) / 128;
             const int64_t unit = (int64_t) nw * ch;
             auto part_length = [&](int64_t parts) { return ((k + parts - 1) / parts + unit - 1) / unit * unit; };
             // The number of parts: measured on 4096 x 4096, 8192 x 8192, 11008 x 4096 and 4096 x 11008, what counts is that
@@ -316,7 +319,7 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
             const int64_t kpart = part_length(parts);
             parts = (k + kpart - 1) / kpart;
             const int64_t bytes = parts * m * n * (int64_t) sizeof(S);
-            const bool direct = parts == 1 && (tb || ((uintptr_t) C % 16 == 0 && ldc % 4 == 0));
+            const bool direct = parts == 1 && (tb || ((uintptr_t) C % 16 == 0 && ldc % (skinny_f64 ? 2 : 4) == 0));
             if (direct || bytes <= (int64_t(64) << 20)) {
                 PartialsLease lease;
                 void* buf = nullptr;
@@ -327,19 +330,21 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                     if ((rc = partials_for(s, &lease))) return rc;
                     buf = lease.ptr;
                 }
-                if (skinny_bf16)
+                if (skinny_f64)
+                    std::snprintf(name, sizeof(name), "docc_dgemm_skinny16_nn_w%d_b%d", nw, nbuf);
+                else if (skinny_bf16)
                     std::snprintf(name, sizeof(name), "docc_bgemm_skinny%d_nt_w%d_b%d", mt, nw, nbuf);
                 else
                     std::snprintf(name, sizeof(name), "docc_sgemm_skinny%d_n%c_w%d_c%d_b%d", mt, tb ? 't' : 'n', nw, ch, nbuf);
-                const uint32_t slot_bytes = skinny_bf16 ? 4096u * mt : mt == 32 ? 16384u : 8192u;   // a wavefront's block of sums
+                const uint32_t slot_bytes = skinny_bf16 ? 4096u * mt : mt == 32 && !skinny_f64 ? 16384u : 8192u;   // a wavefront's block of sums
                 rc = launch(name, (uint32_t) col_blocks, (uint32_t) parts, 1, 64 * nw, (uint32_t) (nw / 2) * slot_bytes, s, A, (long) lda, B, (long) ldb,
-                            direct ? (void*) C : buf, (long) (direct ? ldc : n), (long) m, (long) n, (long) k, (long) kpart, (float) alpha, (float) beta,
+                            direct ? (void*) C : buf, (long) (direct ? ldc : n), (long) m, (long) n, (long) k, (long) kpart, alpha, beta,
                             direct ? 1 : 0);
                 if (!rc && !direct) {
                     int64_t blocks = (m * n + 255) / 256;
                     if (blocks > 4096) blocks = 4096;
-                    rc = launch("docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s, (const S*) buf, C, (long) m, (long) n, (long) ldc,
-                                (int) parts, alpha, beta);
+                    rc = launch(sizeof(S) == 8 ? "docc_splitk_combine_f64" : "docc_splitk_combine_f32", (uint32_t) blocks, 1, 1, 256, 0, s, (const S*) buf, C,
+                                (long) m, (long) n, (long) ldc, (int) parts, alpha, beta);
                 }
                 if (own_block) {
                     const int rc2 = docc_rocm_free_async(buf, stream);
@@ -350,8 +355,8 @@ int gemm_launch(const char* prefix, docc_rocm_stream_t stream, int trans_a, int 
                 // roundings as the fused store
                 const int64_t shape[2] = {m, n}, row[2] = {1, n};
                 const int post[1] = {activation};
-                return docc_rocm_elementwise_fused(stream, 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0, bias ? row : nullptr, bias, 0.0,
-                                                   activation >= 0 ? 1 : 0, post, C);
+                return docc_rocm_elementwise_fused(stream, sizeof(S) == 8 ? 64 : 32, 2, shape, bias ? DOCC_ROCM_BINARY_ADD : -1, shape, C, 0.0,
+                                                   bias ? row : nullptr, bias, 0.0, activation >= 0 ? 1 : 0, post, C);
             }
         }
     }

@@ -163,3 +163,35 @@ def test_skinny_bf16_random_operands(rt, monkeypatch, m, n, k):
         assert np.array_equal(run_bgemm(rt, Ab, Bb, tb=T), got)     # parts are added in order
     monkeypatch.setenv("DOCC_ROCM_GEMM_SKINNY", "0")
     assert rel_err_max(run_bgemm(rt, Ab, Bb, tb=T), got.astype(np.float64)) <= 2e-5
+
+
+F64_SHAPES = [(16, 1024, 1024), (9, 1000, 2052), (5, 514, 512), (12, 4096, 4096), (13, 1286, 4098)]
+
+
+@pytest.mark.parametrize("m,n,k", F64_SHAPES)
+def test_skinny_f64_integer_exact(rt, m, n, k):
+    """fp64, B stored [k][n], 5 to 16 rows: the same scheme on the fp64 MFMA."""
+    rng = np.random.default_rng(m + 3 * n + 5 * k)
+    A, B = int_matrix(rng, (m, k), np.float64, lim=4), int_matrix(rng, (k, n), np.float64, lim=4)
+    C0 = int_matrix(rng, (m, n), np.float64)
+    C = run_gemm(rt, A, B, C=C0.copy(), alpha=2.0, beta=-3.0, ldc=n + 6)
+    assert np.array_equal(C, oracle.gemm(A, B, C=C0.copy(), alpha=2.0, beta=-3.0))
+    assert np.array_equal(run_gemm(rt, A, B), oracle.gemm(A, B))      # beta == 0 must not read C
+
+
+@pytest.mark.parametrize("parts", ["1", "3", "8", "64"])
+@pytest.mark.parametrize("m", [7, 16])
+def test_skinny_f64_any_number_of_parts_and_random_operands(rt, monkeypatch, parts, m):
+    monkeypatch.setenv("DOCC_ROCM_GEMM_SPLITK", parts)
+    n, k = 1154, 3072
+    rng = np.random.default_rng(m + int(parts))
+    A, B = int_matrix(rng, (m, k), np.float64, lim=4), int_matrix(rng, (k, n), np.float64, lim=4)
+    C0 = int_matrix(rng, (m, n), np.float64)
+    expect = oracle.gemm(A, B, C=C0.copy(), alpha=-1.0, beta=2.0)
+    for ldc in (n, n + 2, n + 1):           # the last: rows of C off the 16-byte boundary, no direct store
+        assert np.array_equal(run_gemm(rt, A, B, C=C0.copy(), alpha=-1.0, beta=2.0, ldc=ldc), expect), ldc
+    A, B = rng.standard_normal((m, k)), rng.standard_normal((k, n))
+    got = run_gemm(rt, A, B)
+    assert rel_err_max(got, A @ B) <= 1e-12
+    monkeypatch.setenv("DOCC_ROCM_GEMM_SKINNY", "0")
+    assert rel_err_max(run_gemm(rt, A, B), got) <= 1e-12
