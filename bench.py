@@ -504,7 +504,12 @@ def main():
         for m_, n_, k_, how in ((16, 8192, 4096, "b_straight_into_the_mfma"), (32, 4096, 4096, "b_straight_into_the_mfma"), (64, 4096, 4096, "tiles_k_in_parts")):
             hbm(f"sgemm_{m_}x{n_}x{k_}_{how}", 4 * (k_ * n_ + m_ * k_ + m_ * n_),
                 lambda i: rt.sgemm(m_, n_, k_, 1.0, y.data_ptr(), k_, x_(i), n_, 0.0, y.data_ptr() + 4 * (1 << 22), n_, stream=stream))
-        del xs, y
+        del xs
+        ds = [torch.randn(4096 * 4096, device="cuda", dtype=torch.float64) for _ in range(ROTATE)]
+        y.view(torch.float64)[: 8 * 4096].normal_()
+        hbm("dgemm_8x4096x4096_b_straight_into_the_mfma", 8 * (4096 * 4096 + 2 * 8 * 4096),
+            lambda i: rt.dgemm(8, 4096, 4096, 1.0, y.data_ptr(), 4096, ds[i % ROTATE].data_ptr(), 4096, 0.0, y.data_ptr() + (1 << 24), 4096, stream=stream))
+        del ds, y
         # causal: query i sees the keys j <= i; the flops are those of the pairs it computes on (S (S + 1) / 2 per head)
         torch.manual_seed(3)
         Q, K, V = (torch.randn(8, 16, 2048, 64).bfloat16().cuda() for _ in range(3))

@@ -1027,6 +1027,67 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_
     __builtin_nontemporal_store(acc, reinterpret_cast<v4*>(p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + (long) oh * p.OW + ow));
 }
 
+// The same layer with R output rows of the quad a lane: the R + 2 input row segments are loaded once (3 (R + 2) loads for 4 R
+// outputs instead of 9 R) and all before the first multiply-add, so a lane has that many loads in flight; the lanes count
+// through (plane, block of R rows, quad of the row), so a wavefront runs over plane borders and none of its lanes idles on a
+// plane that is no multiple of 256 quads (a 56 x 56 plane: 784). The filter differs between the lanes of a wavefront and
+// comes through vector loads, nine for 4 R outputs. Each output sums in the order of the kernel above.
+namespace docc_k {
+template <int R>
+__device__ __forceinline__ void conv_depthwise_3x3_v4_rows(const ConvParams& p, int mult) {
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    const unsigned qw = (unsigned) p.OW / 4, rbs = ((unsigned) p.OH + R - 1) / R;
+    const unsigned per_plane = qw * rbs;
+    const unsigned item = blockIdx.x * 256u + threadIdx.x;     // the host keeps the count of items below 2^31
+    const unsigned plane = item / per_plane;                   // n * OC + oc
+    if (plane >= (unsigned) p.N * (unsigned) p.OC) return;
+    const unsigned rest = item - plane * per_plane;
+    const int ow = (int) (rest % qw) * 4, oh0 = (int) (rest / qw) * R;
+    const int n = (int) (plane / (unsigned) p.OC), oc = (int) (plane % (unsigned) p.OC);
+    const float* x = p.X + ((long) n * p.XC + oc / mult) * p.H * p.W;
+    const float* w = p.Wt + (long) oc * 9;
+    float wt[9];
+#pragma unroll
+    for (int t = 0; t < 9; t++) wt[t] = w[t];
+    float in[R + 2][6];
+#pragma unroll
+    for (int j = 0; j < R + 2; j++) {
+        const int ih = oh0 - p.pad_h + j;
+        v4 mid = {0.f, 0.f, 0.f, 0.f};
+        float left = 0.f, right = 0.f;
+        if ((unsigned) ih < (unsigned) p.H) {
+            const float* row = x + (long) ih * p.W;
+            mid = *reinterpret_cast<const v4*>(row + ow);
+            if (ow > 0) left = row[ow - 1];
+            if (ow + 4 < p.W) right = row[ow + 4];
+        }
+        in[j][0] = left; in[j][1] = mid[0]; in[j][2] = mid[1]; in[j][3] = mid[2]; in[j][4] = mid[3]; in[j][5] = right;
+    }
+    const float b = p.bias ? p.bias[oc] : 0.f;
+    float* y = p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + ow;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (oh0 + r >= p.OH) break;
+        v4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kh = 0; kh < 3; kh++)
+#pragma unroll
+            for (int kw = 0; kw < 3; kw++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[e] = __builtin_fmaf(in[r + kh][e + kw], wt[kh * 3 + kw], acc[e]);
+        if (p.bias) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[e] += b;
+        }
+        __builtin_nontemporal_store(acc, reinterpret_cast<v4*>(y + (long) (oh0 + r) * p.OW));
+    }
+}
+}  // namespace docc_k
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<4>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<7>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r8(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<8>(p, mult); }
+
 // Groups of a few channels (a ResNeXt layer: 32 groups of 4 or 8 channels in, as many out): per output element the layer does
 // C/group * 9 multiply-adds against eight bytes moved, so it is bound by HBM like the depthwise one, and a 64-row MFMA tile
 // would hold 4 or 8 real output channels. 3x3, stride 1, no dilation, one column of padding, rows of whole aligned quads (as

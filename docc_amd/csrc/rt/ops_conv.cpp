@@ -397,6 +397,17 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
         // 3x3, stride 1, rows of whole aligned quads: four pixels a lane
         if (KH == 3 && KW == 3 && stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && pad_w == 1 && OW == W && W % 4 == 0 &&
             (uintptr_t) X % 16 == 0 && (uintptr_t) Y % 16 == 0 && !(force && force[0] == 's')) {   // DOCC_ROCM_CONV=scalar: a pixel a lane (tests)
+            // several output rows a lane (seven where that divides the plane's rows, as the 224 / 2^i planes of the image
+            // networks, else eight, four for low planes); DOCC_ROCM_CONV=quad keeps one row a lane, DOCC_ROCM_CONV_ROWS=4|7|8
+            // names the count (both for tests and measurements)
+            const char* rows_env = std::getenv("DOCC_ROCM_CONV_ROWS");
+            int rows = OH % 7 == 0 ? 7 : OH >= 16 ? 8 : 4;
+            if (rows_env && (rows_env[0] == '4' || rows_env[0] == '7' || rows_env[0] == '8') && !rows_env[1]) rows = rows_env[0] - '0';
+            const int64_t items = N * OC * (OW / 4) * ((OH + rows - 1) / rows);
+            if (!(force && force[0] == 'q') && items + 255 < lim) {
+                const char* name = rows == 7 ? "docc_conv2d_depthwise_f32_3x3_v4_r7" : rows == 8 ? "docc_conv2d_depthwise_f32_3x3_v4_r8" : "docc_conv2d_depthwise_f32_3x3_v4_r4";
+                return launch(name, (uint32_t) ((items + 255) / 256), 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
+            }
             const int64_t quads = N * OC * ((OH * (OW / 4) + 255) / 256);
             return launch("docc_conv2d_depthwise_f32_3x3_v4", (uint32_t) quads, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
         }

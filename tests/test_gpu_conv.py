@@ -280,16 +280,16 @@ GROUP_CASES = [
 ]
 
 
-# depthwise layers: four pixels a lane where rows allow, one pixel, and the kernels of the other groups; those: every group in one
+# depthwise layers: four pixels of several rows a lane where rows allow, of one row (quad), one pixel, and the kernels of the other groups; those: every group in one
 # launch, and a launch per group
-@pytest.mark.parametrize("force", ["", "scalar", "gather", "loop"])
+@pytest.mark.parametrize("force", ["", "quad", "scalar", "gather", "loop"])
 @pytest.mark.parametrize("case", GROUP_CASES)
 def test_conv_with_groups(rt, monkeypatch, force, case):
     """The node's `group`: weights [OC, C / group, KH, KW], every group on its own channels of X and Y where they lie. Integer-
     valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
     N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
     if force:
-        if (group == C) == (force == "loop") or (force == "scalar" and group != C):
+        if (group == C) == (force == "loop") or (force in ("scalar", "quad") and group != C):
             pytest.skip("a form of the other kind of layer")
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
     rng = np.random.default_rng(hash(case[:7]) & 0xffff)
@@ -315,3 +315,37 @@ def test_conv_with_groups(rt, monkeypatch, force, case):
     for bad in (0, -2, 5 if C % 5 else 7):
         with pytest.raises(rt.RocmRuntimeError, match="group"):
             rt.conv2d_f32_grouped(N, C, H, W, OC, KH, KW, stride, pads, dil, bad, x.data_ptr(), w.data_ptr(), 0, y.data_ptr())
+
+
+@pytest.mark.parametrize("rows", ["4", "7", "8"])
+@pytest.mark.parametrize("shape", [
+    # N, C, H, W, channels out per channel in, pads (h, w, h end, w end), bias
+    (2, 24, 19, 16, 2, (1, 1, 1, 1), True),     # 19 rows: the last block of rows is cut for every count
+    (1, 8, 5, 8, 1, (2, 1, 0, 1), False),       # fewer rows than a block, two rows of padding above and none below
+    (3, 5, 56, 56, 1, (1, 1, 1, 1), True),      # 15 planes of 784 quads: wavefronts run over plane borders
+    (1, 3, 33, 4, 3, (0, 1, 3, 1), True),       # one quad a row
+])
+def test_depthwise_rows_a_lane(rt, monkeypatch, rows, shape):
+    """The depthwise 3x3 kernel with 4, 7 and 8 output rows a lane (DOCC_ROCM_CONV_ROWS) against the oracle bit for bit, and equal
+    to the kernel with one row a lane on random operands (same order of the sums)."""
+    N, C, H, W, mult, pads, use_bias = shape
+    OC = C * mult
+    monkeypatch.setenv("DOCC_ROCM_CONV_ROWS", rows)
+    rng = np.random.default_rng(int(rows) * 131 + H)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, 1, 3, 3)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    ref = oracle.conv2d(X, Wt, b, (1, 1), pads, (1, 1), group=C)
+    x, w = dev(X), dev(Wt)
+    bd = dev(b) if b is not None else None
+    y = torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), C, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    xr, wr = torch.randn(N, C, H, W, device="cuda"), torch.randn(OC, 1, 3, 3, device="cuda")
+    ya, yb = torch.full(ref.shape, float("nan"), device="cuda"), torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
+    monkeypatch.setenv("DOCC_ROCM_CONV", "quad")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb)
