@@ -1088,6 +1088,58 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<7>(p, mult); }
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r8(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<8>(p, mult); }
 
+// 3x3 depthwise layers whose rows are no whole aligned quads (14 x 14 and 7 x 7 planes) or that step by two: a lane takes one
+// output column and R output rows, loads the (R - 1) S + 3 input rows of its three columns once and before the first
+// multiply-add, and the lanes count through (plane, block of rows, column) as above: a 7 x 7 plane fills 7 lanes instead of
+// 49 of a work-group's 256, and a lane loads 27 + 9 values for seven outputs instead of 18 for one. Sums in the same order.
+namespace docc_k {
+template <int R, int S>
+__device__ __forceinline__ void conv_depthwise_3x3_rows(const ConvParams& p, int mult) {
+    const unsigned ow_n = (unsigned) p.OW, rbs = ((unsigned) p.OH + R - 1) / R;
+    const unsigned per_plane = ow_n * rbs;
+    const unsigned item = blockIdx.x * 256u + threadIdx.x;     // the host keeps the count of items below 2^31
+    const unsigned plane = item / per_plane;                   // n * OC + oc
+    if (plane >= (unsigned) p.N * (unsigned) p.OC) return;
+    const unsigned rest = item - plane * per_plane;
+    const int ow = (int) (rest % ow_n), oh0 = (int) (rest / ow_n) * R;
+    const int n = (int) (plane / (unsigned) p.OC), oc = (int) (plane % (unsigned) p.OC);
+    const float* x = p.X + ((long) n * p.XC + oc / mult) * p.H * p.W;
+    const float* w = p.Wt + (long) oc * 9;
+    float wt[9];
+#pragma unroll
+    for (int t = 0; t < 9; t++) wt[t] = w[t];
+    constexpr int ROWS = (R - 1) * S + 3;
+    float in[ROWS][3];
+    const int iw0 = ow * S - p.pad_w, ih0 = oh0 * S - p.pad_h;
+#pragma unroll
+    for (int j = 0; j < ROWS; j++) {
+        const int ih = ih0 + j;
+        const bool row_in = (unsigned) ih < (unsigned) p.H;
+        const float* row = x + (long) ih * p.W;
+#pragma unroll
+        for (int kw = 0; kw < 3; kw++) in[j][kw] = row_in && (unsigned) (iw0 + kw) < (unsigned) p.W ? row[iw0 + kw] : 0.f;
+    }
+    const float b = p.bias ? p.bias[oc] : 0.f;
+    float* y = p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + ow;
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        if (oh0 + r >= p.OH) break;
+        float acc = 0.f;
+#pragma unroll
+        for (int kh = 0; kh < 3; kh++)
+#pragma unroll
+            for (int kw = 0; kw < 3; kw++) acc = __builtin_fmaf(in[r * S + kh][kw], wt[kh * 3 + kw], acc);
+        if (p.bias) acc += b;
+        __builtin_nontemporal_store(acc, y + (long) (oh0 + r) * p.OW);
+    }
+}
+}  // namespace docc_k
+
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<4, 1>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<7, 1>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<4, 2>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<7, 2>(p, mult); }
+
 // Groups of a few channels (a ResNeXt layer: 32 groups of 4 or 8 channels in, as many out): per output element the layer does
 // C/group * 9 multiply-adds against eight bytes moved, so it is bound by HBM like the depthwise one, and a 64-row MFMA tile
 // would hold 4 or 8 real output channels. 3x3, stride 1, no dilation, one column of padding, rows of whole aligned quads (as

@@ -349,3 +349,38 @@ def test_depthwise_rows_a_lane(rt, monkeypatch, rows, shape):
     rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
     torch.cuda.synchronize()
     assert torch.equal(ya, yb)
+
+
+@pytest.mark.parametrize("rows", ["4", "7"])
+@pytest.mark.parametrize("shape", [
+    # N, C, H, W, channels out per channel in, stride, pads (h, w, h end, w end), bias
+    (3, 20, 14, 14, 1, 1, (1, 1, 1, 1), True),     # 14 x 14 planes: rows of no whole quads
+    (2, 37, 7, 7, 2, 1, (1, 1, 1, 1), False),      # 7 x 7 planes, seven lanes a plane
+    (2, 6, 23, 17, 1, 2, (1, 1, 1, 1), True),      # steps of two on odd extents
+    (1, 5, 30, 9, 3, 2, (0, 2, 1, 0), True),       # steps of two, pads that differ, 15 output rows
+    (2, 4, 9, 13, 1, 1, (2, 0, 0, 2), False),      # no column of padding on the left, two on the right
+])
+def test_depthwise_column_and_rows_a_lane(rt, monkeypatch, rows, shape):
+    """The depthwise 3x3 kernel with one output column and 4 or 7 output rows a lane (stride 1 or 2) against the oracle bit for
+    bit, and equal to the kernel with a pixel a lane on random operands (same order of the sums)."""
+    N, C, H, W, mult, st, pads, use_bias = shape
+    OC = C * mult
+    monkeypatch.setenv("DOCC_ROCM_CONV_ROWS", rows)
+    rng = np.random.default_rng(int(rows) * 977 + H)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, 1, 3, 3)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    ref = oracle.conv2d(X, Wt, b, (st, st), pads, (1, 1), group=C)
+    x, w = dev(X), dev(Wt)
+    bd = dev(b) if b is not None else None
+    y = torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    xr, wr = torch.randn(N, C, H, W, device="cuda"), torch.randn(OC, 1, 3, 3, device="cuda")
+    ya, yb = torch.full(ref.shape, float("nan"), device="cuda"), torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
+    monkeypatch.setenv("DOCC_ROCM_CONV", "scalar")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb)
