@@ -1209,6 +1209,96 @@ __device__ __forceinline__ void conv_small_groups_3x3_v4(const ConvParams& p, in
 }
 }  // namespace docc_k
 
+// The same with R output rows of the quad a lane (OGT * R = 16 accumulator quads): an input channel's R + 2 row segments are
+// loaded once for the R rows, and a filter value read from LDS serves 4 R multiply-adds instead of 4 - with one row a lane the
+// kernel issued an LDS read for every four multiply-adds. The lanes of a work-group count through (image, block of rows, quad)
+// for one (group, OGT channels): only the last work-group of those has idle lanes (a 56 x 56 plane of 784 quads left 240 of
+// 1024 idle). Each output sums over (input channel, kh, kw) in the order of the kernel above.
+namespace docc_k {
+template <int OGT, int R>
+__device__ __forceinline__ void conv_small_groups_3x3_v4_rows(const ConvParams& p, int cg, int og) {
+    typedef float v4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) unsigned char conv_sg_lds[];
+    float* wl = reinterpret_cast<float*>(conv_sg_lds);   // [OGT][cg][9]
+    const unsigned qw = (unsigned) p.OW / 4, rbs = ((unsigned) p.OH + R - 1) / R;
+    const unsigned per_image = qw * rbs, total = (unsigned) p.N * per_image;   // the host keeps total + 255 below 2^31
+    const unsigned blocks_per = (total + 255) / 256;
+    const int chunks = og / OGT;                           // OGT divides og
+    unsigned b = blockIdx.x;
+    const unsigned iblock = b % blocks_per;
+    b /= blocks_per;
+    const int chunk = (int) (b % (unsigned) chunks), grp = (int) (b / (unsigned) chunks);
+    const int oc0 = grp * og + chunk * OGT;
+    for (int i = threadIdx.x; i < OGT * cg * 9; i += 256) wl[i] = p.Wt[(long) oc0 * cg * 9 + i];
+    __syncthreads();
+    const unsigned item = iblock * 256 + threadIdx.x;
+    if (item >= total) return;
+    const int n = (int) (item / per_image);
+    const unsigned rest = item - (unsigned) n * per_image;
+    const int ow = (int) (rest % qw) * 4, oh0 = (int) (rest / qw) * R;
+    v4 acc[OGT][R];
+#pragma unroll
+    for (int o = 0; o < OGT; o++)
+#pragma unroll
+        for (int r = 0; r < R; r++) acc[o][r] = v4{0.f, 0.f, 0.f, 0.f};
+    const float* x = p.X + ((long) n * p.XC + (long) grp * cg) * p.H * p.W;
+    for (int ci = 0; ci < cg; ci++) {
+        const float* plane = x + (long) ci * p.H * p.W;
+        float in[R + 2][6];
+#pragma unroll
+        for (int j = 0; j < R + 2; j++) {
+            const int ih = oh0 - p.pad_h + j;
+            v4 mid = {0.f, 0.f, 0.f, 0.f};
+            float left = 0.f, right = 0.f;
+            if ((unsigned) ih < (unsigned) p.H) {
+                const float* row = plane + (long) ih * p.W;
+                mid = *reinterpret_cast<const v4*>(row + ow);
+                if (ow > 0) left = row[ow - 1];
+                if (ow + 4 < p.W) right = row[ow + 4];
+            }
+            in[j][0] = left; in[j][1] = mid[0]; in[j][2] = mid[1]; in[j][3] = mid[2]; in[j][4] = mid[3]; in[j][5] = right;
+        }
+#pragma unroll
+        for (int kh = 0; kh < 3; kh++)
+#pragma unroll
+            for (int kw = 0; kw < 3; kw++)
+#pragma unroll
+                for (int o = 0; o < OGT; o++) {
+                    const float wt = wl[(o * cg + ci) * 9 + kh * 3 + kw];
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) acc[o][r][e] = __builtin_fmaf(in[r + kh][e + kw], wt, acc[o][r][e]);
+                }
+    }
+#pragma unroll
+    for (int o = 0; o < OGT; o++) {
+        const int oc = oc0 + o;
+        const float bv = p.bias ? p.bias[oc] : 0.f;
+        float* y = p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + ow;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            if (oh0 + r >= p.OH) break;
+            if (p.bias) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[o][r][e] += bv;
+            }
+            __builtin_nontemporal_store(acc[o][r], reinterpret_cast<v4*>(y + (long) (oh0 + r) * p.OW));
+        }
+    }
+}
+}  // namespace docc_k
+
+#define DOCC_CONV_SMALL_GROUPS_ROWS(OGT, R)                                                                                                      \
+    extern "C" __global__ __launch_bounds__(256) void docc_conv2d_small_groups_f32_3x3_v4_o##OGT##_r##R(docc_k::ConvParams p, int cg, int og) {   \
+        docc_k::conv_small_groups_3x3_v4_rows<OGT, R>(p, cg, og);                                                                                \
+    }
+DOCC_CONV_SMALL_GROUPS_ROWS(1, 8)
+DOCC_CONV_SMALL_GROUPS_ROWS(2, 8)
+DOCC_CONV_SMALL_GROUPS_ROWS(4, 4)
+DOCC_CONV_SMALL_GROUPS_ROWS(8, 2)
+DOCC_CONV_SMALL_GROUPS_ROWS(8, 4)
+
 #define DOCC_CONV_SMALL_GROUPS(OGT)                                                                                                        \
     extern "C" __global__ __launch_bounds__(256) void docc_conv2d_small_groups_f32_3x3_v4_o##OGT(docc_k::ConvParams p, int cg, int og) {     \
         docc_k::conv_small_groups_3x3_v4<OGT>(p, cg, og);                                                                                  \

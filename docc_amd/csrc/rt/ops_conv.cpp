@@ -440,6 +440,22 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
             ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
                          (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) C, (int) OC, 0, 0, 0, 0};
             char name[64];
+            // several output rows a lane, the lanes counting through the images; DOCC_ROCM_CONV=quad keeps one row a lane and
+            // DOCC_ROCM_CONV_ROWS=4 takes four rows for eight output channels instead of two (tests, measurements)
+            const char* rows_env = std::getenv("DOCC_ROCM_CONV_ROWS");
+            const int rows = ogt == 8 ? (rows_env && rows_env[0] == '4' && !rows_env[1] ? 4 : 2) : ogt == 4 ? 4 : 8;
+            const int64_t items = N * (OW / 4) * ((OH + rows - 1) / rows);
+            const int64_t row_blocks = group * (og / ogt) * ((items + 255) / 256);
+            // measured: the form pays once its work-groups fill the chip about three times over (768 of them on 256 CUs: C128
+            // 56x56 in 32 groups 38 -> 34 us, C256 56x56 87 -> 67), and always for one or two output channels a lane, where the
+            // LDS reads bound the other form (C64 56x56 19 -> 14); with fewer work-groups one row a lane has more waves to
+            // hide the loads behind (C256 28x28: 24 against 29)
+            const int cus = compute_units() > 0 ? compute_units() : 256;
+            const bool rows_pay = row_blocks >= 3 * (int64_t) cus || ogt <= 2 || (rows_env && rows_env[0]);
+            if (!(force && force[0] == 'q') && rows_pay && items + 255 < lim && row_blocks < lim) {
+                std::snprintf(name, sizeof(name), "docc_conv2d_small_groups_f32_3x3_v4_o%d_r%d", ogt, rows);
+                return launch(name, (uint32_t) row_blocks, 1, 1, 256, (uint32_t) (ogt * cg * 9 * 4), (hipStream_t) stream, p, (int) cg, (int) og);
+            }
             std::snprintf(name, sizeof(name), "docc_conv2d_small_groups_f32_3x3_v4_o%d", ogt);
             return launch(name, (uint32_t) blocks, 1, 1, 256, (uint32_t) (ogt * cg * 9 * 4), (hipStream_t) stream, p, (int) cg, (int) og);
         }

@@ -289,7 +289,7 @@ def test_conv_with_groups(rt, monkeypatch, force, case):
     valued operands against the oracle bit for bit; the oracle's grouped form is pinned in tests/test_oracle.py."""
     N, C, H, W, OC, KH, KW, stride, pads, dil, group, use_bias = case
     if force:
-        if (group == C) == (force == "loop") or (force in ("scalar", "quad") and group != C):
+        if (group == C) == (force == "loop") or (force == "scalar" and group != C):
             pytest.skip("a form of the other kind of layer")
         monkeypatch.setenv("DOCC_ROCM_CONV", force)
     rng = np.random.default_rng(hash(case[:7]) & 0xffff)
@@ -382,5 +382,38 @@ def test_depthwise_column_and_rows_a_lane(rt, monkeypatch, rows, shape):
     rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
     monkeypatch.setenv("DOCC_ROCM_CONV", "scalar")
     rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb)
+
+
+@pytest.mark.parametrize("rows", ["8", "4"])   # set, the variable keeps small layers on this form; 4: four rows for eight channels
+@pytest.mark.parametrize("shape", [
+    # N, C, H, W, OC, group, pads (h, w, h end, w end), bias
+    (3, 32, 19, 16, 32, 8, (1, 1, 1, 1), True),     # four in, four out per group: four rows a lane, 19 rows
+    (2, 32, 13, 8, 64, 4, (1, 1, 1, 1), True),      # eight in, 16 out: two chunks of eight channels, two (or four) rows a lane
+    (5, 12, 56, 56, 12, 6, (1, 1, 1, 1), False),    # two in, two out: eight rows a lane, lanes counting through the images
+    (2, 9, 11, 12, 15, 3, (2, 1, 0, 1), True),      # three in, five out: one output channel and eight rows a lane, pads that differ
+])
+def test_small_groups_rows_a_lane(rt, monkeypatch, rows, shape):
+    """Groups of a few channels with several output rows a lane against the oracle bit for bit, and equal to the kernel with one
+    row a lane on random operands (same order of the sums)."""
+    N, C, H, W, OC, group, pads, use_bias = shape
+    monkeypatch.setenv("DOCC_ROCM_CONV_ROWS", rows)
+    rng = np.random.default_rng(H * 31 + W)
+    X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, C // group, 3, 3)).astype(np.float32)
+    b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
+    ref = oracle.conv2d(X, Wt, b, (1, 1), pads, (1, 1), group=group)
+    x, w = dev(X), dev(Wt)
+    bd = dev(b) if b is not None else None
+    y = torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), group, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(host(y), ref)
+    xr, wr = torch.randn(N, C, H, W, device="cuda"), torch.randn(OC, C // group, 3, 3, device="cuda")
+    ya, yb = torch.full(ref.shape, float("nan"), device="cuda"), torch.full(ref.shape, float("nan"), device="cuda")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), group, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
+    monkeypatch.setenv("DOCC_ROCM_CONV", "quad")
+    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (1, 1), pads, (1, 1), group, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
     torch.cuda.synchronize()
     assert torch.equal(ya, yb)
