@@ -427,15 +427,26 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
         const char* name = KH == 3 && KW == 3 ? "docc_conv2d_depthwise_f32_3x3" : KH == 5 && KW == 5 ? "docc_conv2d_depthwise_f32_5x5" : "docc_conv2d_depthwise_f32";
         return launch(name, (uint32_t) blocks, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
     }
-    // groups of at most eight channels in, 3x3, stride 1, rows of whole aligned quads: the kernel that is bound by moving X and Y
+    // groups of at most 16 channels in, 3x3, stride 1, rows of whole aligned quads: the kernel that is bound by moving X and Y
+    // (DOCC_ROCM_CONV_SMALL_GROUP=<channels> moves the limit: measurements)
+    const char* sg_env = std::getenv("DOCC_ROCM_CONV_SMALL_GROUP");
+    const int64_t small_group_limit = sg_env && sg_env[0] ? std::atoll(sg_env) : 16;
     // (DOCC_ROCM_CONV=gather or loop keeps the kernels of the larger groups: tests)
-    if (cg <= 8 && og <= 64 && KH == 3 && KW == 3 && stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && pad_w == 1 && pad_h >= 0 &&
+    if (cg <= small_group_limit && og <= 64 && KH == 3 && KW == 3 && stride_h == 1 && stride_w == 1 && dil_h == 1 && dil_w == 1 && pad_w == 1 && pad_h >= 0 &&
         pad_h_end >= 0 && pad_w_end >= 0 && OW == W && W % 4 == 0 && (uintptr_t) X % 16 == 0 && (uintptr_t) Y % 16 == 0 && X && Y && Wt && N > 0 &&
         OH > 0 && !(force && (force[0] == 'g' || force[0] == 'l'))) {
         const int ogt = og % 8 == 0 ? 8 : og % 4 == 0 ? 4 : og % 2 == 0 ? 2 : 1;
         const int64_t lim = 0x7fffffffLL;
         const int64_t blocks = N * group * (og / ogt) * ((OH * (OW / 4) + 255) / 256);
-        if (C * H * W < lim && OH * OW < lim && OC < lim && blocks < lim) {
+        // nine to 16 channels in: the 64 output channels of an MFMA tile are a quarter or a half real up to 32 channels out
+        // (measured with 16 in and out: C512 28x28 in 32 groups 214 -> 69 us, C256 56x56 in 16 groups 352 -> 114, C64 56x56 in 4
+        // groups 91 -> 40); with 64 out the tiles win (40 against 64 us), and so they do on launches that leave CUs idle
+        bool pays = true;
+        if (cg > 8) {
+            if (int rc = ensure_device()) return rc;
+            pays = og <= 32 && blocks >= (compute_units() > 0 ? compute_units() : 256);
+        }
+        if (pays && C * H * W < lim && OH * OW < lim && OC < lim && blocks < lim) {
             if (int rc = ensure_device()) return rc;
             ConvParams p{X, Wt, bias, Y, (int) N, (int) C, (int) H, (int) W, (int) OC, (int) KH, (int) KW, (int) OH, (int) OW,
                          (int) stride_h, (int) stride_w, (int) pad_h, (int) pad_w, (int) dil_h, (int) dil_w, (int) C, (int) OC, 0, 0, 0, 0};

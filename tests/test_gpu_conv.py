@@ -393,6 +393,7 @@ def test_depthwise_column_and_rows_a_lane(rt, monkeypatch, rows, shape):
     (2, 32, 13, 8, 64, 4, (1, 1, 1, 1), True),      # eight in, 16 out: two chunks of eight channels, two (or four) rows a lane
     (5, 12, 56, 56, 12, 6, (1, 1, 1, 1), False),    # two in, two out: eight rows a lane, lanes counting through the images
     (2, 9, 11, 12, 15, 3, (2, 1, 0, 1), True),      # three in, five out: one output channel and eight rows a lane, pads that differ
+    (4, 512, 8, 8, 512, 32, (1, 1, 1, 1), True),    # 16 in, 16 out in 32 groups: enough work-groups for this kernel to be the choice
 ])
 def test_small_groups_rows_a_lane(rt, monkeypatch, rows, shape):
     """Groups of a few channels with several output rows a lane against the oracle bit for bit, and equal to the kernel with one
