@@ -1088,13 +1088,13 @@ extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<7>(p, mult); }
 extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_v4_r8(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_v4_rows<8>(p, mult); }
 
-// 3x3 depthwise layers whose rows are no whole aligned quads (14 x 14 and 7 x 7 planes) or that step by two: a lane takes one
-// output column and R output rows, loads the (R - 1) S + 3 input rows of its three columns once and before the first
+// 3x3 depthwise layers whose rows are no whole aligned quads (14 x 14 and 7 x 7 planes) or that step by two, and 5x5 ones: a lane
+// takes one output column and R output rows, loads the (R - 1) S + K input rows of its K columns once and before the first
 // multiply-add, and the lanes count through (plane, block of rows, column) as above: a 7 x 7 plane fills 7 lanes instead of
 // 49 of a work-group's 256, and a lane loads 27 + 9 values for seven outputs instead of 18 for one. Sums in the same order.
 namespace docc_k {
-template <int R, int S>
-__device__ __forceinline__ void conv_depthwise_3x3_rows(const ConvParams& p, int mult) {
+template <int R, int S, int K>   // K x K filter
+__device__ __forceinline__ void conv_depthwise_rows(const ConvParams& p, int mult) {
     const unsigned ow_n = (unsigned) p.OW, rbs = ((unsigned) p.OH + R - 1) / R;
     const unsigned per_plane = ow_n * rbs;
     const unsigned item = blockIdx.x * 256u + threadIdx.x;     // the host keeps the count of items below 2^31
@@ -1104,12 +1104,12 @@ __device__ __forceinline__ void conv_depthwise_3x3_rows(const ConvParams& p, int
     const int ow = (int) (rest % ow_n), oh0 = (int) (rest / ow_n) * R;
     const int n = (int) (plane / (unsigned) p.OC), oc = (int) (plane % (unsigned) p.OC);
     const float* x = p.X + ((long) n * p.XC + oc / mult) * p.H * p.W;
-    const float* w = p.Wt + (long) oc * 9;
-    float wt[9];
+    const float* w = p.Wt + (long) oc * (K * K);
+    float wt[K * K];
 #pragma unroll
-    for (int t = 0; t < 9; t++) wt[t] = w[t];
-    constexpr int ROWS = (R - 1) * S + 3;
-    float in[ROWS][3];
+    for (int t = 0; t < K * K; t++) wt[t] = w[t];
+    constexpr int ROWS = (R - 1) * S + K;
+    float in[ROWS][K];
     const int iw0 = ow * S - p.pad_w, ih0 = oh0 * S - p.pad_h;
 #pragma unroll
     for (int j = 0; j < ROWS; j++) {
@@ -1117,7 +1117,7 @@ __device__ __forceinline__ void conv_depthwise_3x3_rows(const ConvParams& p, int
         const bool row_in = (unsigned) ih < (unsigned) p.H;
         const float* row = x + (long) ih * p.W;
 #pragma unroll
-        for (int kw = 0; kw < 3; kw++) in[j][kw] = row_in && (unsigned) (iw0 + kw) < (unsigned) p.W ? row[iw0 + kw] : 0.f;
+        for (int kw = 0; kw < K; kw++) in[j][kw] = row_in && (unsigned) (iw0 + kw) < (unsigned) p.W ? row[iw0 + kw] : 0.f;
     }
     const float b = p.bias ? p.bias[oc] : 0.f;
     float* y = p.Y + ((long) n * p.YC + oc) * p.OH * p.OW + ow;
@@ -1126,19 +1126,23 @@ __device__ __forceinline__ void conv_depthwise_3x3_rows(const ConvParams& p, int
         if (oh0 + r >= p.OH) break;
         float acc = 0.f;
 #pragma unroll
-        for (int kh = 0; kh < 3; kh++)
+        for (int kh = 0; kh < K; kh++)
 #pragma unroll
-            for (int kw = 0; kw < 3; kw++) acc = __builtin_fmaf(in[r * S + kh][kw], wt[kh * 3 + kw], acc);
+            for (int kw = 0; kw < K; kw++) acc = __builtin_fmaf(in[r * S + kh][kw], wt[kh * K + kw], acc);
         if (p.bias) acc += b;
         __builtin_nontemporal_store(acc, y + (long) (oh0 + r) * p.OW);
     }
 }
 }  // namespace docc_k
 
-extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<4, 1>(p, mult); }
-extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<7, 1>(p, mult); }
-extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<4, 2>(p, mult); }
-extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_3x3_rows<7, 2>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<4, 1, 3>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s1_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<7, 1, 3>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<4, 2, 3>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_3x3_s2_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<7, 2, 3>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_5x5_s1_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<4, 1, 5>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_5x5_s1_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<7, 1, 5>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_5x5_s2_r4(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<4, 2, 5>(p, mult); }
+extern "C" __global__ __launch_bounds__(256) void docc_conv2d_depthwise_f32_5x5_s2_r7(docc_k::ConvParams p, int mult) { docc_k::conv_depthwise_rows<7, 2, 5>(p, mult); }
 
 // Groups of a few channels (a ResNeXt layer: 32 groups of 4 or 8 channels in, as many out): per output element the layer does
 // C/group * 9 multiply-adds against eight bytes moved, so it is bound by HBM like the depthwise one, and a 64-row MFMA tile

@@ -411,16 +411,16 @@ extern "C" int docc_rocm_conv2d_f32_grouped(docc_rocm_stream_t stream, int64_t N
             const int64_t quads = N * OC * ((OH * (OW / 4) + 255) / 256);
             return launch("docc_conv2d_depthwise_f32_3x3_v4", (uint32_t) quads, 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
         }
-        // other 3x3 layers without dilation that step by one or by two: a column and seven or four output rows a lane
-        if (KH == 3 && KW == 3 && stride_h == stride_w && (stride_h == 1 || stride_h == 2) && dil_h == 1 && dil_w == 1 &&
+        // other 3x3 layers and 5x5 ones without dilation that step by one or by two: a column and seven or four output rows a lane
+        if (((KH == 3 && KW == 3) || (KH == 5 && KW == 5)) && stride_h == stride_w && (stride_h == 1 || stride_h == 2) && dil_h == 1 && dil_w == 1 &&
             !(force && (force[0] == 's' || force[0] == 'q'))) {
             const char* rows_env = std::getenv("DOCC_ROCM_CONV_ROWS");
             int rows = OH % 7 == 0 && OH >= 28 ? 7 : 4;   // measured: planes of 14 and 7 rows run faster with four
             if (rows_env && (rows_env[0] == '4' || rows_env[0] == '7') && !rows_env[1]) rows = rows_env[0] - '0';
             const int64_t items = N * OC * OW * ((OH + rows - 1) / rows);
             if (items + 255 < lim) {
-                const char* name = stride_h == 1 ? (rows == 7 ? "docc_conv2d_depthwise_f32_3x3_s1_r7" : "docc_conv2d_depthwise_f32_3x3_s1_r4")
-                                                 : (rows == 7 ? "docc_conv2d_depthwise_f32_3x3_s2_r7" : "docc_conv2d_depthwise_f32_3x3_s2_r4");
+                char name[64];
+                std::snprintf(name, sizeof(name), "docc_conv2d_depthwise_f32_%dx%d_s%d_r%d", (int) KH, (int) KW, (int) stride_h, rows);
                 return launch(name, (uint32_t) ((items + 255) / 256), 1, 1, 256, 0, (hipStream_t) stream, p, (int) og);
             }
         }

@@ -359,29 +359,33 @@ def test_depthwise_rows_a_lane(rt, monkeypatch, rows, shape):
     (2, 6, 23, 17, 1, 2, (1, 1, 1, 1), True),      # steps of two on odd extents
     (1, 5, 30, 9, 3, 2, (0, 2, 1, 0), True),       # steps of two, pads that differ, 15 output rows
     (2, 4, 9, 13, 1, 1, (2, 0, 0, 2), False),      # no column of padding on the left, two on the right
+    (2, 18, 28, 28, 1, 1, (2, 2, 2, 2), True, 5),  # 5x5 filters
+    (3, 7, 17, 15, 2, 2, (2, 2, 2, 2), False, 5),  # 5x5, steps of two, odd extents
+    (1, 6, 6, 9, 1, 1, (0, 1, 3, 2), True, 5),     # 5x5 on planes lower than the filter without the pads
 ])
 def test_depthwise_column_and_rows_a_lane(rt, monkeypatch, rows, shape):
-    """The depthwise 3x3 kernel with one output column and 4 or 7 output rows a lane (stride 1 or 2) against the oracle bit for
+    """The depthwise 3x3 and 5x5 kernels with one output column and 4 or 7 output rows a lane (stride 1 or 2) against the oracle bit for
     bit, and equal to the kernel with a pixel a lane on random operands (same order of the sums)."""
-    N, C, H, W, mult, st, pads, use_bias = shape
+    N, C, H, W, mult, st, pads, use_bias = shape[:8]
+    K = shape[8] if len(shape) > 8 else 3
     OC = C * mult
     monkeypatch.setenv("DOCC_ROCM_CONV_ROWS", rows)
     rng = np.random.default_rng(int(rows) * 977 + H)
     X = rng.integers(-4, 5, (N, C, H, W)).astype(np.float32)
-    Wt = rng.integers(-4, 5, (OC, 1, 3, 3)).astype(np.float32)
+    Wt = rng.integers(-4, 5, (OC, 1, K, K)).astype(np.float32)
     b = rng.integers(-4, 5, OC).astype(np.float32) if use_bias else None
     ref = oracle.conv2d(X, Wt, b, (st, st), pads, (1, 1), group=C)
     x, w = dev(X), dev(Wt)
     bd = dev(b) if b is not None else None
     y = torch.full(ref.shape, float("nan"), device="cuda")
-    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y.data_ptr())
+    rt.conv2d_f32_grouped(N, C, H, W, OC, K, K, (st, st), pads, (1, 1), C, x.data_ptr(), w.data_ptr(), bd.data_ptr() if bd is not None else 0, y.data_ptr())
     torch.cuda.synchronize()
     assert np.array_equal(host(y), ref)
-    xr, wr = torch.randn(N, C, H, W, device="cuda"), torch.randn(OC, 1, 3, 3, device="cuda")
+    xr, wr = torch.randn(N, C, H, W, device="cuda"), torch.randn(OC, 1, K, K, device="cuda")
     ya, yb = torch.full(ref.shape, float("nan"), device="cuda"), torch.full(ref.shape, float("nan"), device="cuda")
-    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
+    rt.conv2d_f32_grouped(N, C, H, W, OC, K, K, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, ya.data_ptr())
     monkeypatch.setenv("DOCC_ROCM_CONV", "scalar")
-    rt.conv2d_f32_grouped(N, C, H, W, OC, 3, 3, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
+    rt.conv2d_f32_grouped(N, C, H, W, OC, K, K, (st, st), pads, (1, 1), C, xr.data_ptr(), wr.data_ptr(), bd.data_ptr() if bd is not None else 0, yb.data_ptr())
     torch.cuda.synchronize()
     assert torch.equal(ya, yb)
 
